@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Headline benchmark: 1-bit quantize + unquantize of a 2048 x 9304 fp32 gradient with in-place residual.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = QuantizeAsync (gradient + carried residual -> packed codes + new residual) followed by UnquantizeAsync
+(packed codes -> fp32), through the C ABI, inputs resident in device memory. Buffer sets are rotated so that no step
+finds its inputs in the 256 MB Infinity Cache. Prints ONE JSON line.
+
+  value     algorithmic GB/s of the whole step: (16 + nbits/4) bytes per element + 16 bytes per column
+            = 309,790,784 bytes for 2048 x 9304 at 1 bit, divided by the step time
+  roofline  the dominant kernel (quantize): algorithmic bytes per launch (12 + nbits/8 per element + 8 per column
+            = 231,116,664) over its average duration measured with HIP events on the launch stream, against
+            8 TB/s of HBM
+  cpu_baseline  the CPU oracle (a port of the reference's MatrixQuantizerCPU) timed on this host, single thread
+            like the reference, on the same matrix
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+ROWS, COLS, NBITS = 2048, 9304, 1
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(rows, cols, nbits):
+    elems = rows * cols
+    quant = elems * 12 + elems * nbits // 8 + cols * 8
+    unquant = elems * 4 + elems * nbits // 8 + cols * 8
+    return quant, unquant
+
+
+def cpu_baseline(budget_s=12.0):
+    """Times the CPU oracle on the full 2048 x 9304 matrix (single thread, like the reference CPU quantizer)."""
+    import numpy as np
+
+    import datagen
+    import oracle
+
+    g = datagen.normal(datagen.case_seed(0), ROWS, COLS, 0.01)
+    r = np.zeros_like(g, order="F")
+    out = np.zeros_like(g, order="F")
+    qb, ub = algorithmic_bytes(ROWS, COLS, NBITS)
+
+    def run(threads, budget):
+        best = float("inf")
+        passes = 0
+        t_end = time.perf_counter() + budget
+        while passes < 3 or (time.perf_counter() < t_end and passes < 40):
+            t0 = time.perf_counter()
+            q, _ = oracle.quantize(g, r, NBITS, False, r_out=r, threads=threads)
+            oracle.unquantize(q, ROWS, COLS, NBITS, out=out, threads=threads)
+            best = min(best, time.perf_counter() - t0)
+            passes += 1
+        return best, passes
+
+    t1, p1 = run(1, budget_s)
+    cores = min(16, os.cpu_count() or 1)
+    tn, pn = run(cores, budget_s / 3)
+    return {
+        "value": round((qb + ub) / t1 / 1e9, 4),
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": "%d passes of quantize+unquantize over the full %dx%d fp32 matrix, 1 bit, best pass" % (p1, ROWS, COLS),
+        "ms_per_step": round(t1 * 1e3, 2),
+        "elements_per_s": round(ROWS * COLS / t1, 1),
+        "all_cores": {"cores": cores, "value": round((qb + ub) / tn / 1e9, 4), "ms_per_step": round(tn * 1e3, 2),
+                      "passes": pn},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--zero-threshold", type=int, default=0, help="zeroThresholdFor1Bit (default off, as in config 1)")
+    ap.add_argument("--sets", type=int, default=6, help="rotating buffer sets (each 231 MB)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU only (K workers are simulated in one GPU's memory); "
+                 "--gpus %d is not supported" % args.gpus)
+
+    import torch
+
+    import cntk_amd
+    from cntk_amd import Matrix, MatrixQuantizerImpl, QuantizedMatrix
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = "cuda:0"
+    zt = bool(args.zero_threshold)
+    qz = MatrixQuantizerImpl.Create(0, False)  # issues on the main (null) stream = torch's current stream
+
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0x1B17)
+    sets = []
+    for _ in range(args.sets):
+        G = Matrix(ROWS, COLS, 0, torch.randn(ROWS * COLS, generator=gen, device=dev, dtype=torch.float32) * 0.01)
+        sets.append((G, Matrix(ROWS, COLS), QuantizedMatrix(ROWS, COLS, NBITS, 0), Matrix(ROWS, COLS)))
+    torch.cuda.synchronize()
+
+    def step(i, ev=None):
+        G, R, Q, Out = sets[i % len(sets)]
+        if ev is not None:
+            ev[0].record()
+        qz.QuantizeAsync(G, R, Q, R, zt)
+        if ev is not None:
+            ev[1].record()
+        qz.UnquantizeAsync(Q, Out, False)
+        if ev is not None:
+            ev[2].record()
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    # timed region: exactly `steps` steps, host clock around a synchronize on both sides
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(args.warmup + i, events[i])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    sec_per_step = (t1 - t0) / args.steps
+    q_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
+    u_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+    qb, ub = algorithmic_bytes(ROWS, COLS, NBITS)
+    total = qb + ub
+    achieved = qb / (q_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "1-bit quantize+unquantize GB/s & % HBM peak, 2048x9304 fp32 gradient",
+        "value": round(total / sec_per_step / 1e9, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec_per_step * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "quantize+unquantize 2048x9304 fp32, 1 bit, in-place residual carried across steps, "
+                        "zeroThresholdFor1Bit %s" % ("on" if zt else "off"),
+            "rows": ROWS, "cols": COLS, "nbits": NBITS, "zero_threshold_for_1bit": zt,
+            "buffer_sets": len(sets), "algorithmic_bytes_per_step": total,
+        },
+        "pct_hbm_peak": round(100.0 * total / sec_per_step / 1e9 / HBM_PEAK_GBS, 2),
+        "elements_per_s": round(ROWS * COLS / sec_per_step, 1),
+        "kernel_ms": {"quantize": round(q_ms, 5), "unquantize": round(u_ms, 5)},
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "quantize (gradient + residual -> codes + residual)",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+        },
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,316 @@
+"""cntk_amd -- MI355X (gfx950) implementation of CNTK's quantized-gradient hot path.
+
+Python mirror of the reference's quantizer interface on top of the C ABI in
+``include/cntk_amd_quantizer.h`` (``libcntk_amd_quantizer.so``):
+
+    MatrixQuantizerImpl  <->  Source/Math/MatrixQuantizerImpl.h:19-49
+    QuantizedMatrix      <->  Source/Math/QuantizedMatrix.h:54-124
+    MatrixQuantizer      <->  Source/1BitSGD/MatrixQuantizer.h:24-85
+    Matrix               <->  the little of Source/Math/Matrix.h the path needs (dense fp32, column-major)
+
+torch is used only as the owner of device memory. There is no CPU implementation and no fallback:
+if the HIP library is missing, importing the bindings raises.
+"""
+import ctypes
+import os
+
+import numpy as np
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libcntk_amd_quantizer.so")
+
+CPUDEVICE = -1
+
+_sz = ctypes.c_size_t
+_vp = ctypes.c_void_p
+_lib = None
+
+
+class QuantizerError(RuntimeError):
+    """RuntimeError of the reference (a failed device call)."""
+
+
+class QuantizerLogicError(ValueError):
+    """LogicError / InvalidArgument of the reference (bad nbits, mismatching sizes)."""
+
+
+def lib():
+    """The loaded C-ABI library. Raises if it has not been built (python -m cntk_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("%s is missing: build it with `python -m cntk_amd.build` "
+                              "(there is no CPU fallback)" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        L.cntkq_last_error.restype = ctypes.c_char_p
+        L.cntkq_qwords_per_col.argtypes = [_sz, _sz]
+        L.cntkq_qwords_per_col.restype = _sz
+        L.cntkq_qcol_bytes.argtypes = [_sz, _sz]
+        L.cntkq_qcol_bytes.restype = _sz
+        L.cntkq_qmatrix_bytes.argtypes = [_sz, _sz, _sz]
+        L.cntkq_qmatrix_bytes.restype = _sz
+        L.cntkq_stripe_range.argtypes = [_sz, _sz, _sz, ctypes.POINTER(_sz), ctypes.POINTER(_sz)]
+        L.cntkq_create.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(_vp)]
+        L.cntkq_destroy.argtypes = [_vp]
+        L.cntkq_device_id.argtypes = [_vp]
+        L.cntkq_stream.argtypes = [_vp]
+        L.cntkq_stream.restype = _vp
+        L.cntkq_set_main_stream.argtypes = [_vp, _vp]
+        L.cntkq_sync_with_main_stream.argtypes = [_vp]
+        L.cntkq_quantize_async.argtypes = [_vp, _vp, _vp, _sz, _sz, _vp, _sz, ctypes.c_int, _sz, _vp, ctypes.c_int]
+        L.cntkq_wait_quantize_done.argtypes = [_vp]
+        L.cntkq_unquantize_async.argtypes = [_vp, _vp, _sz, ctypes.c_int, _vp, _sz, _sz, _sz, ctypes.c_int]
+        L.cntkq_wait_unquantize_done.argtypes = [_vp]
+        L.cntkq_stripe_reduce_async.argtypes = [_vp, ctypes.POINTER(_vp), _sz, _sz, _sz, _sz, _sz, _vp, _vp, _vp,
+                                                ctypes.c_int]
+        L.cntkq_wait_stripe_reduce_done.argtypes = [_vp]
+        L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int]
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc == 0:
+        return
+    msg = lib().cntkq_last_error().decode("utf-8", "replace")
+    if rc == 3:
+        raise QuantizerError(msg)
+    raise QuantizerLogicError(msg)
+
+
+def qwords_per_col(rows, nbits):
+    return lib().cntkq_qwords_per_col(rows, nbits)
+
+
+def qcol_bytes(nbits, rows):
+    return lib().cntkq_qcol_bytes(nbits, rows)
+
+
+def stripe_range(cols, rank, workers):
+    """GetStripeForNode (Source/1BitSGD/AllReduceDistGradAggregator.h:56-65) -> (start_col, num_cols)."""
+    s, n = _sz(), _sz()
+    _check(lib().cntkq_stripe_range(cols, rank, workers, ctypes.byref(s), ctypes.byref(n)))
+    return s.value, n.value
+
+
+# ---------------------------------------------------------------------------------------------------
+
+
+class Matrix:
+    """Dense fp32 matrix in column-major storage on one device (Source/Math/Matrix.h, the part used here).
+
+    ``data`` is a flat torch tensor of rows * cols floats: element (i, j) is data[j * rows + i].
+    """
+
+    def __init__(self, rows, cols, device_id=0, data=None):
+        self.rows, self.cols, self.device_id = int(rows), int(cols), device_id
+        if data is None:
+            dev = "cpu" if device_id < 0 else "cuda:%d" % device_id
+            data = torch.zeros(self.rows * self.cols, dtype=torch.float32, device=dev)
+        if data.dtype != torch.float32 or data.dim() != 1 or data.numel() != self.rows * self.cols:
+            raise QuantizerLogicError("Matrix data must be a flat float32 tensor of rows * cols elements")
+        if not data.is_contiguous():
+            raise QuantizerLogicError("Matrix data must be contiguous")
+        self.data = data
+
+    @classmethod
+    def from_numpy(cls, a, device_id=0):
+        """From a (rows, cols) float32 numpy array; the values are laid out column-major on the device."""
+        a = np.asfortranarray(a, dtype=np.float32)
+        flat = torch.from_numpy(a.reshape(-1, order="F").copy())
+        if device_id >= 0:
+            flat = flat.to("cuda:%d" % device_id)
+        return cls(a.shape[0], a.shape[1], device_id, flat)
+
+    def to_numpy(self):
+        """(rows, cols) float32 numpy array in Fortran order."""
+        return np.asfortranarray(self.data.detach().cpu().numpy().reshape((self.rows, self.cols), order="F"))
+
+    def GetNumRows(self):
+        return self.rows
+
+    def GetNumCols(self):
+        return self.cols
+
+    def GetDeviceId(self):
+        return self.device_id
+
+    def Data(self):
+        return self.data.data_ptr()
+
+    def ColumnSlice(self, start_col, num_cols):
+        """Zero-copy view of columns [start_col, start_col + num_cols) (Source/Math/Matrix.h:194)."""
+        if start_col + num_cols > self.cols:
+            raise QuantizerLogicError("ColumnSlice out of range")
+        view = self.data[start_col * self.rows:(start_col + num_cols) * self.rows]
+        return Matrix(self.rows, num_cols, self.device_id, view)
+
+    def SetValue(self, v):
+        self.data.fill_(v)
+
+
+class QuantizedMatrix:
+    """Packed matrix: per column {f32 lower, f32 upper, u32 bits[nq]} (Source/Math/QuantizedMatrix.h:27-124).
+
+    device_id >= 0 keeps the buffer on that GPU; CPUDEVICE keeps it in pinned host memory, as the
+    reference's v1 aggregator does through its page-locked allocator
+    (Source/1BitSGD/AllReduceDistGradAggregator.h:76-77, 88).
+    """
+
+    def __init__(self, num_rows, num_cols, nbits, device_id=0, _buffer=None):
+        if nbits not in (1, 2, 4, 8, 16, 32):
+            # Source/Math/QuantizedMatrix.cpp:12-15
+            raise QuantizerLogicError("Quantization: 'nbits' must be a power of two that divides 32")
+        self.num_rows, self.num_cols, self.nbits, self.device_id = int(num_rows), int(num_cols), int(nbits), device_id
+        self.qcol_size = qcol_bytes(nbits, self.num_rows)
+        size = self.qcol_size * self.num_cols
+        if _buffer is None:
+            if device_id < 0:
+                _buffer = torch.zeros(size, dtype=torch.uint8, pin_memory=torch.cuda.is_available())
+            else:
+                _buffer = torch.zeros(size, dtype=torch.uint8, device="cuda:%d" % device_id)
+        self.buffer = _buffer
+
+    def GetNumRows(self):
+        return self.num_rows
+
+    def GetNumCols(self):
+        return self.num_cols
+
+    def GetNumBits(self):
+        return self.nbits
+
+    def GetDeviceId(self):
+        return self.device_id
+
+    def GetSize(self):
+        return self.buffer.numel()
+
+    def Buffer(self):
+        return self.buffer.data_ptr()
+
+    def ColumnSlice(self, start_col, num_cols):
+        """Non-owning view of a run of columns (Source/Math/QuantizedMatrix.cpp:102-107)."""
+        if start_col + num_cols > self.num_cols:
+            raise QuantizerLogicError("ColumnSlice out of range")
+        view = self.buffer[start_col * self.qcol_size:(start_col + num_cols) * self.qcol_size]
+        return QuantizedMatrix(self.num_rows, num_cols, self.nbits, self.device_id, view)
+
+    def to_numpy(self):
+        return self.buffer.detach().cpu().numpy().copy()
+
+    def from_numpy(self, a):
+        self.buffer.copy_(torch.from_numpy(np.ascontiguousarray(a, dtype=np.uint8)))
+
+
+class MatrixQuantizerImpl:
+    """The quantizer object (Source/Math/MatrixQuantizerImpl.h:19-49) for one GPU."""
+
+    def __init__(self, device_id, use_async):
+        if device_id < 0:
+            # the reference returns its CPU quantizer here; this library has none
+            raise QuantizerError("MatrixQuantizerImpl.Create: no CPU quantizer in this library (device %d)" % device_id)
+        h = _vp()
+        _check(lib().cntkq_create(device_id, int(bool(use_async)), ctypes.byref(h)))
+        self._h = h
+        self._device_id = device_id
+
+    @staticmethod
+    def Create(device_id, use_async):
+        return MatrixQuantizerImpl(device_id, use_async)
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h and _lib is not None:
+            _lib.cntkq_destroy(h)
+
+    def GetDeviceId(self):
+        return self._device_id
+
+    def stream(self):
+        return lib().cntkq_stream(self._h)
+
+    def SynchronizeWithMainStream(self):
+        """MatrixComputeStreamEvent::SynchronizeQuantizationComputeStreamWithEvent
+        (Source/Math/MatrixQuantizerGPU.cu:347-371)."""
+        _check(lib().cntkq_sync_with_main_stream(self._h))
+
+    def QuantizeAsync(self, in_matrix, in_residual, out_qmatrix, out_residual, zero_threshold_for_1bit):
+        rows, cols = in_matrix.GetNumRows(), in_matrix.GetNumCols()
+        # the reference asserts these (Source/Math/MatrixQuantizerGPU.cu:229-232)
+        for m in (in_residual, out_residual, out_qmatrix):
+            if m.GetNumRows() != rows or m.GetNumCols() != cols:
+                raise QuantizerLogicError("QuantizeAsync: matrix dimensions do not match")
+        _check(lib().cntkq_quantize_async(self._h, in_matrix.Data(), in_residual.Data(), rows, cols,
+                                          out_qmatrix.Buffer(), out_qmatrix.GetSize(),
+                                          int(out_qmatrix.GetDeviceId() < 0), out_qmatrix.GetNumBits(),
+                                          out_residual.Data(), int(bool(zero_threshold_for_1bit))))
+
+    def WaitQuantizeAsyncDone(self):
+        _check(lib().cntkq_wait_quantize_done(self._h))
+
+    def UnquantizeAsync(self, in_qmatrix, out_matrix, add=False):
+        rows, cols = out_matrix.GetNumRows(), out_matrix.GetNumCols()
+        _check(lib().cntkq_unquantize_async(self._h, in_qmatrix.Buffer(), in_qmatrix.GetSize(),
+                                            int(in_qmatrix.GetDeviceId() < 0), out_matrix.Data(), rows, cols,
+                                            in_qmatrix.GetNumBits(), int(bool(add))))
+
+    def WaitUnquantizeAsyncDone(self):
+        _check(lib().cntkq_wait_unquantize_done(self._h))
+
+    def StripeReduceAsync(self, stripes, owner, stripe_residual, out_qstripe, zero_threshold_for_1bit, agg_out=None):
+        """Fused stripe reduction of the quantized all-reduce (dataflow of
+        Source/1BitSGD/AllReduceDistGradAggregator.h:365-436): stripes[w] is worker w's packed stripe."""
+        k = len(stripes)
+        rows, cols, nbits = out_qstripe.GetNumRows(), out_qstripe.GetNumCols(), out_qstripe.GetNumBits()
+        for s in stripes:
+            if s.GetNumRows() != rows or s.GetNumCols() != cols or s.GetNumBits() != nbits or s.GetDeviceId() < 0:
+                raise QuantizerLogicError("StripeReduceAsync: stripes must be device-resident and of equal shape")
+        if stripe_residual.GetNumRows() != rows or stripe_residual.GetNumCols() != cols:
+            raise QuantizerLogicError("StripeReduceAsync: stripe residual has the wrong shape")
+        arr = (_vp * k)(*[s.Buffer() for s in stripes])
+        _check(lib().cntkq_stripe_reduce_async(self._h, arr, k, owner, rows, cols, nbits, stripe_residual.Data(),
+                                               out_qstripe.Buffer(), agg_out.Data() if agg_out is not None else None,
+                                               int(bool(zero_threshold_for_1bit))))
+
+    def WaitStripeReduceDone(self):
+        _check(lib().cntkq_wait_stripe_reduce_done(self._h))
+
+    def _set_tuning(self, quantize_path=0, tile_gs=0, unq_slots=0, unq_force_scalar=0):
+        _check(lib().cntkq_debug_set_tuning(self._h, quantize_path, tile_gs, unq_slots, unq_force_scalar))
+
+
+class MatrixQuantizer:
+    """Quantizer that owns its error-feedback residual (Source/1BitSGD/MatrixQuantizer.h:24-85)."""
+
+    def __init__(self, num_rows, num_cols, device_id, use_async):
+        self._impl = MatrixQuantizerImpl.Create(device_id, use_async)
+        self._residual = Matrix(num_rows, num_cols, device_id)
+
+    def QuantizeAsync(self, in_matrix, out_qmatrix, zero_threshold_for_1bit, in_residual=None, out_residual=None):
+        if in_residual is None:
+            in_residual = out_residual = self._residual
+        self._impl.QuantizeAsync(in_matrix, in_residual, out_qmatrix, out_residual, zero_threshold_for_1bit)
+
+    def WaitQuantizeAsyncDone(self):
+        self._impl.WaitQuantizeAsyncDone()
+
+    def UnquantizeAsync(self, in_qmatrix, out_matrix, add=False):
+        self._impl.UnquantizeAsync(in_qmatrix, out_matrix, add)
+
+    def WaitUnquantizeAsyncDone(self):
+        self._impl.WaitUnquantizeAsyncDone()
+
+    def GetDeviceId(self):
+        return self._impl.GetDeviceId()
+
+    def ResetResidue(self):
+        self._residual.SetValue(0.0)
+
+    def GetResidualMatrix(self):
+        return self._residual
+
+    @property
+    def impl(self):
+        return self._impl

@@ -1,0 +1,471 @@
+// C ABI of the MI355X gradient quantizer: handles, streams, events, argument checks.
+// Replaces the host side of the reference's GPU quantizer (Source/Math/MatrixQuantizerGPU.cu:83-341).
+#include "../../include/cntk_amd_quantizer.h"
+#include "quantizer_internal.h"
+#include "quantizer_launch.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+
+using namespace cntkq;
+
+namespace {
+
+thread_local char g_last_error[1024] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof g_last_error, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(call, what)                                                                                          \
+    do                                                                                                               \
+    {                                                                                                                \
+        hipError_t rc__ = (call);                                                                                    \
+        if (rc__ != hipSuccess)                                                                                      \
+            return fail(CNTKQ_RUNTIME_ERROR, "%s: %s (hip error %d)", what, hipGetErrorString(rc__), (int) rc__);    \
+    } while (0)
+
+// Process-wide streams per device, created on first use and never destroyed, like the reference's
+// static compute / fetch / assign streams (Source/Math/MatrixQuantizerGPU.cu:83-90, 197-206).
+constexpr int kMaxDevices = 64;
+struct DeviceStreams
+{
+    hipStream_t compute = nullptr;
+    hipStream_t fetch = nullptr;
+    hipStream_t assign = nullptr;
+};
+DeviceStreams g_streams[kMaxDevices];
+std::mutex g_streams_mutex;
+
+class DeviceGuard // PrepareDevice (Source/Math/MatrixQuantizerGPU.cu:186, 234): make the handle's device current
+{
+public:
+    explicit DeviceGuard(int device) : m_prev(-1), m_changed(false)
+    {
+        if (hipGetDevice(&m_prev) == hipSuccess && m_prev != device)
+            m_changed = (hipSetDevice(device) == hipSuccess);
+    }
+    ~DeviceGuard()
+    {
+        if (m_changed)
+            (void) hipSetDevice(m_prev);
+    }
+
+private:
+    int m_prev;
+    bool m_changed;
+};
+
+bool aligned4(const void* p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & 3u) == 0;
+}
+
+} // namespace
+
+struct cntkq_quantizer
+{
+    int device = 0;
+    bool dedicated = false;
+    hipStream_t main_stream = nullptr;
+    hipStream_t compute = nullptr; // == main_stream when !dedicated
+    hipStream_t fetch = nullptr;
+    hipStream_t assign = nullptr;
+    hipEvent_t ev_quantize = nullptr;
+    hipEvent_t ev_fetch = nullptr;
+    hipEvent_t ev_assign = nullptr;
+    hipEvent_t ev_unquantize = nullptr;
+    hipEvent_t ev_stripe = nullptr;
+    hipEvent_t ev_main = nullptr;
+    bool quantize_included_fetch = false;
+    bool fetch_pending = false;   // a device-to-host copy out of the staging buffer may still be running
+    bool staging_read_pending = false; // a kernel reading the staging buffer may still be running
+    char* staging = nullptr;      // device buffer used when the packed matrix lives in host memory
+    size_t staging_bytes = 0;
+    LaunchTuning tune;
+};
+
+namespace {
+
+hipStream_t work_stream(const cntkq_quantizer* h)
+{
+    return h->dedicated ? h->compute : h->main_stream;
+}
+
+// Temp device buffer for a host-resident packed matrix (GetTempGPUQuantizedMatrix,
+// Source/Math/MatrixQuantizerGPU.cu:158-179). Grows only; waits for everything that may still use the old one.
+int ensure_staging(cntkq_quantizer* h, size_t bytes)
+{
+    if (h->staging_bytes >= bytes)
+        return CNTKQ_OK;
+    if (h->staging != nullptr)
+    {
+        HIP_TRY(hipStreamSynchronize(work_stream(h)), "hipStreamSynchronize failed");
+        HIP_TRY(hipStreamSynchronize(h->fetch), "hipStreamSynchronize failed");
+        HIP_TRY(hipStreamSynchronize(h->assign), "hipStreamSynchronize failed");
+        HIP_TRY(hipFree(h->staging), "hipFree failed");
+        h->staging = nullptr;
+        h->staging_bytes = 0;
+        h->fetch_pending = false;
+        h->staging_read_pending = false;
+    }
+    void* p = nullptr;
+    HIP_TRY(hipMalloc(&p, bytes), "hipMalloc of the packed staging buffer failed");
+    h->staging = static_cast<char*>(p);
+    h->staging_bytes = bytes;
+    return CNTKQ_OK;
+}
+
+int sync_event(hipEvent_t ev) // SyncEvent (Source/Math/MatrixQuantizerGPU.cu:68-80)
+{
+    hipError_t rc = hipEventQuery(ev);
+    if (rc == hipSuccess)
+        return CNTKQ_OK;
+    if (rc != hipErrorNotReady)
+        return fail(CNTKQ_RUNTIME_ERROR, "hipEventQuery failed: %s (hip error %d)", hipGetErrorString(rc), (int) rc);
+    HIP_TRY(hipEventSynchronize(ev), "hipEventSynchronize failed");
+    return CNTKQ_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+const char* cntkq_last_error(void)
+{
+    return g_last_error;
+}
+
+size_t cntkq_qwords_per_col(size_t rows, size_t nbits)
+{
+    return valid_nbits(nbits) ? qwords_per_col(rows, nbits) : 0;
+}
+
+size_t cntkq_qcol_bytes(size_t nbits, size_t rows)
+{
+    return valid_nbits(nbits) ? qcol_bytes(nbits, rows) : 0;
+}
+
+size_t cntkq_qmatrix_bytes(size_t rows, size_t cols, size_t nbits)
+{
+    return valid_nbits(nbits) ? qcol_bytes(nbits, rows) * cols : 0;
+}
+
+int cntkq_stripe_range(size_t cols, size_t rank, size_t workers, size_t* start_col, size_t* num_cols)
+{
+    if (workers == 0 || rank >= workers || start_col == nullptr || num_cols == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_range: need 0 <= rank < workers and non-null outputs");
+    const size_t per = cols / workers;
+    const size_t extra = cols % workers;
+    *start_col = per * rank + (extra < rank ? extra : rank);
+    *num_cols = per + (rank < extra ? 1 : 0);
+    return CNTKQ_OK;
+}
+
+int cntkq_create(int device_id, int use_dedicated_stream, cntkq_quantizer** out)
+{
+    if (out == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_create: out is null");
+    *out = nullptr;
+    if (device_id < 0)
+        return fail(CNTKQ_RUNTIME_ERROR, "cntkq_create: device %d requested, but this library has no CPU quantizer", device_id);
+    int count = 0;
+    HIP_TRY(hipGetDeviceCount(&count), "hipGetDeviceCount failed");
+    if (device_id >= count || device_id >= kMaxDevices)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_create: device %d out of range (%d devices)", device_id, count);
+
+    DeviceGuard guard(device_id);
+    cntkq_quantizer* h = new (std::nothrow) cntkq_quantizer();
+    if (h == nullptr)
+        return fail(CNTKQ_RUNTIME_ERROR, "cntkq_create: out of host memory");
+    h->device = device_id;
+    h->dedicated = use_dedicated_stream != 0;
+    {
+        std::lock_guard<std::mutex> lock(g_streams_mutex);
+        DeviceStreams& ds = g_streams[device_id];
+        // all streams keep the default priority
+        if (h->dedicated && ds.compute == nullptr)
+        {
+            hipError_t rc = hipStreamCreateWithFlags(&ds.compute, hipStreamNonBlocking);
+            if (rc != hipSuccess)
+            {
+                delete h;
+                return fail(CNTKQ_RUNTIME_ERROR, "hipStreamCreateWithFlags failed: %s", hipGetErrorString(rc));
+            }
+        }
+        if (ds.fetch == nullptr)
+        {
+            hipError_t rc = hipStreamCreateWithFlags(&ds.fetch, hipStreamNonBlocking);
+            if (rc == hipSuccess)
+                rc = hipStreamCreateWithFlags(&ds.assign, hipStreamNonBlocking);
+            if (rc != hipSuccess)
+            {
+                delete h;
+                return fail(CNTKQ_RUNTIME_ERROR, "hipStreamCreateWithFlags failed: %s", hipGetErrorString(rc));
+            }
+        }
+        h->compute = ds.compute;
+        h->fetch = ds.fetch;
+        h->assign = ds.assign;
+    }
+    hipEvent_t* evs[] = {&h->ev_quantize, &h->ev_fetch, &h->ev_assign, &h->ev_unquantize, &h->ev_stripe, &h->ev_main};
+    for (hipEvent_t* e : evs)
+    {
+        // no blocking-sync flag: waiting spins, as the reference found blocking events to stall for tens of ms
+        hipError_t rc = hipEventCreateWithFlags(e, hipEventDisableTiming);
+        if (rc != hipSuccess)
+        {
+            cntkq_destroy(h);
+            return fail(CNTKQ_RUNTIME_ERROR, "hipEventCreateWithFlags failed: %s", hipGetErrorString(rc));
+        }
+    }
+    *out = h;
+    return CNTKQ_OK;
+}
+
+int cntkq_destroy(cntkq_quantizer* h)
+{
+    if (h == nullptr)
+        return CNTKQ_OK;
+    DeviceGuard guard(h->device);
+    if (h->ev_quantize) (void) hipEventSynchronize(h->ev_quantize);
+    if (h->ev_fetch) (void) hipEventSynchronize(h->ev_fetch);
+    if (h->ev_assign) (void) hipEventSynchronize(h->ev_assign);
+    if (h->ev_unquantize) (void) hipEventSynchronize(h->ev_unquantize);
+    if (h->ev_stripe) (void) hipEventSynchronize(h->ev_stripe);
+    if (h->staging != nullptr)
+        (void) hipFree(h->staging);
+    hipEvent_t evs[] = {h->ev_quantize, h->ev_fetch, h->ev_assign, h->ev_unquantize, h->ev_stripe, h->ev_main};
+    for (hipEvent_t e : evs)
+        if (e != nullptr)
+            (void) hipEventDestroy(e);
+    delete h;
+    return CNTKQ_OK;
+}
+
+int cntkq_device_id(const cntkq_quantizer* h)
+{
+    return h ? h->device : -1;
+}
+
+void* cntkq_stream(const cntkq_quantizer* h)
+{
+    return h ? static_cast<void*>(work_stream(h)) : nullptr;
+}
+
+int cntkq_set_main_stream(cntkq_quantizer* h, void* hip_stream)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_set_main_stream: null handle");
+    h->main_stream = static_cast<hipStream_t>(hip_stream);
+    return CNTKQ_OK;
+}
+
+int cntkq_sync_with_main_stream(cntkq_quantizer* h)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_sync_with_main_stream: null handle");
+    if (!h->dedicated)
+        return CNTKQ_OK; // the work stream is the main stream
+    DeviceGuard guard(h->device);
+    HIP_TRY(hipEventRecord(h->ev_main, h->main_stream), "hipEventRecord failed");
+    HIP_TRY(hipStreamWaitEvent(h->compute, h->ev_main, 0), "hipStreamWaitEvent failed");
+    return CNTKQ_OK;
+}
+
+int cntkq_quantize_async(cntkq_quantizer* h, const float* in, const float* res_in, size_t rows, size_t cols, void* qbuf,
+                         size_t qbuf_bytes, int qbuf_on_host, size_t nbits, float* res_out, int zero_threshold_for_1bit)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: null handle");
+    if (!valid_nbits(nbits))
+        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
+    if (rows >= (1ull << 31) || cols >= (1ull << 31))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: rows and cols must be below 2^31");
+    const size_t need = qcol_bytes(nbits, rows) * cols;
+    if (qbuf_bytes != need)
+        return fail(CNTKQ_LOGIC_ERROR,
+                    "quantize: packed buffer of %zu bytes does not match %zu x %zu at %zu bits (%zu bytes)", qbuf_bytes,
+                    rows, cols, nbits, need);
+    h->quantize_included_fetch = false;
+    if (rows == 0 || cols == 0)
+        return CNTKQ_OK;
+    if (in == nullptr || res_in == nullptr || res_out == nullptr || qbuf == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: null matrix pointer");
+    if (!aligned4(in) || !aligned4(res_in) || !aligned4(res_out) || !aligned4(qbuf))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: pointers must be 4-byte aligned");
+
+    DeviceGuard guard(h->device);
+    hipStream_t s = work_stream(h);
+    char* qdev = static_cast<char*>(qbuf);
+    if (qbuf_on_host)
+    {
+        int rc = ensure_staging(h, need);
+        if (rc != CNTKQ_OK)
+            return rc;
+        // a copy out of the staging buffer issued earlier must have drained before it is overwritten
+        if (h->fetch_pending)
+            HIP_TRY(hipStreamWaitEvent(s, h->ev_fetch, 0), "hipStreamWaitEvent failed");
+        qdev = h->staging;
+    }
+
+    hipError_t lrc = launch_quantize(s, in, res_in, res_out, qdev, rows, cols, nbits, zero_threshold_for_1bit != 0, h->tune);
+    if (lrc == hipErrorInvalidValue)
+        return fail(CNTKQ_INVALID_ARGUMENT, "quantize: the forced kernel path does not support %zu x %zu at %zu bits", rows, cols, nbits);
+    HIP_TRY(lrc, "quantize kernel launch failed");
+    HIP_TRY(hipEventRecord(h->ev_quantize, s), "hipEventRecord failed");
+
+    if (qbuf_on_host)
+    {
+        HIP_TRY(hipStreamWaitEvent(h->fetch, h->ev_quantize, 0), "hipStreamWaitEvent failed");
+        HIP_TRY(hipMemcpyAsync(qbuf, qdev, need, hipMemcpyDeviceToHost, h->fetch), "hipMemcpyAsync failed");
+        HIP_TRY(hipEventRecord(h->ev_fetch, h->fetch), "hipEventRecord failed");
+        h->quantize_included_fetch = true;
+        h->fetch_pending = true;
+    }
+    return CNTKQ_OK;
+}
+
+int cntkq_wait_quantize_done(cntkq_quantizer* h)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_wait_quantize_done: null handle");
+    DeviceGuard guard(h->device);
+    if (h->quantize_included_fetch)
+    {
+        int rc = sync_event(h->ev_fetch);
+        if (rc == CNTKQ_OK)
+            h->fetch_pending = false;
+        return rc;
+    }
+    return sync_event(h->ev_quantize);
+}
+
+int cntkq_unquantize_async(cntkq_quantizer* h, const void* qbuf, size_t qbuf_bytes, int qbuf_on_host, float* out,
+                           size_t rows, size_t cols, size_t nbits, int add)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: null handle");
+    if (!valid_nbits(nbits))
+        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
+    if (rows >= (1ull << 31) || cols >= (1ull << 31))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: rows and cols must be below 2^31");
+    const size_t need = qcol_bytes(nbits, rows) * cols;
+    if (qbuf_bytes != need)
+        return fail(CNTKQ_LOGIC_ERROR,
+                    "unquantizestripe: dimension of patch to be unquantized does not match size of quantized data "
+                    "(%zu bytes given, %zu x %zu at %zu bits needs %zu)", qbuf_bytes, rows, cols, nbits, need);
+    if (qbuf_bytes == 0 || rows == 0 || cols == 0)
+        return CNTKQ_OK; // empty buffer: empty matrix, nothing to do
+    if (qbuf == nullptr || out == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: null matrix pointer");
+    if (!aligned4(qbuf) || !aligned4(out))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: pointers must be 4-byte aligned");
+
+    DeviceGuard guard(h->device);
+    hipStream_t s = work_stream(h);
+    const char* qdev = static_cast<const char*>(qbuf);
+    if (qbuf_on_host)
+    {
+        int rc = ensure_staging(h, need);
+        if (rc != CNTKQ_OK)
+            return rc;
+        // the staging buffer may still be read by an earlier kernel or copied out by an earlier fetch
+        HIP_TRY(hipEventRecord(h->ev_assign, s), "hipEventRecord failed");
+        HIP_TRY(hipStreamWaitEvent(h->assign, h->ev_assign, 0), "hipStreamWaitEvent failed");
+        if (h->fetch_pending)
+            HIP_TRY(hipStreamWaitEvent(h->assign, h->ev_fetch, 0), "hipStreamWaitEvent failed");
+        HIP_TRY(hipMemcpyAsync(h->staging, qbuf, need, hipMemcpyHostToDevice, h->assign), "hipMemcpyAsync failed");
+        HIP_TRY(hipEventRecord(h->ev_assign, h->assign), "hipEventRecord failed");
+        HIP_TRY(hipStreamWaitEvent(s, h->ev_assign, 0), "hipStreamWaitEvent failed");
+        qdev = h->staging;
+    }
+    HIP_TRY(launch_unquantize(s, qdev, out, rows, cols, nbits, add != 0, h->tune), "unquantize kernel launch failed");
+    HIP_TRY(hipEventRecord(h->ev_unquantize, s), "hipEventRecord failed");
+    return CNTKQ_OK;
+}
+
+int cntkq_wait_unquantize_done(cntkq_quantizer* h)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_wait_unquantize_done: null handle");
+    DeviceGuard guard(h->device);
+    return sync_event(h->ev_unquantize);
+}
+
+int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows,
+                              size_t stripe_cols, size_t nbits, float* stripe_res, void* q_out, float* agg_out,
+                              int zero_threshold_for_1bit)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: null handle");
+    if (!valid_nbits(nbits))
+        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
+    if (workers == 0 || workers > CNTKQ_MAX_WORKERS || owner >= workers || stripes == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: need 1 <= workers <= %d and owner < workers",
+                    CNTKQ_MAX_WORKERS);
+    if (rows >= (1ull << 31) || stripe_cols >= (1ull << 31))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: rows and cols must be below 2^31");
+    if (rows == 0 || stripe_cols == 0)
+        return CNTKQ_OK;
+    if (rows > kTileMaxRows)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: columns taller than %u rows are not supported",
+                    kTileMaxRows);
+    if (stripe_res == nullptr || q_out == nullptr || !aligned4(stripe_res) || !aligned4(q_out) || !aligned4(agg_out))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: null or misaligned matrix pointer");
+    StripeSources src;
+    std::memset(&src, 0, sizeof src);
+    for (size_t w = 0; w < workers; ++w)
+    {
+        if (stripes[w] == nullptr || !aligned4(stripes[w]))
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: stripe %zu is null or misaligned", w);
+        src.q[w] = static_cast<const char*>(stripes[w]);
+    }
+    src.workers = (uint32_t) workers;
+    src.owner = (uint32_t) owner;
+
+    DeviceGuard guard(h->device);
+    hipStream_t s = work_stream(h);
+    HIP_TRY(launch_stripe_reduce(s, src, stripe_res, q_out, agg_out, rows, stripe_cols, nbits,
+                                 zero_threshold_for_1bit != 0, h->tune),
+            "stripe reduction kernel launch failed");
+    HIP_TRY(hipEventRecord(h->ev_stripe, s), "hipEventRecord failed");
+    return CNTKQ_OK;
+}
+
+int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_wait_stripe_reduce_done: null handle");
+    DeviceGuard guard(h->device);
+    return sync_event(h->ev_stripe);
+}
+
+// ---- hooks for tests and tuning runs (not part of the public header) --------------------------------
+
+int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_gs, unsigned unq_slots, int unq_force_scalar)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: null handle");
+    if (quantize_path < kPathAuto || quantize_path > kPathWaveCol)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: unknown quantize path %d", quantize_path);
+    if (tile_gs != 0 && (tile_gs < 8 || tile_gs > kTileThreads || (tile_gs & (tile_gs - 1)) != 0))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: tile_gs must be a power of two in [8, 256]");
+    h->tune.quantize_path = quantize_path;
+    h->tune.tile_gs = tile_gs;
+    h->tune.unq_slots = unq_slots;
+    h->tune.unq_force_scalar = unq_force_scalar;
+    return CNTKQ_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,22 @@
+// Entry points that the shared library exports for its own tests and tuning runs.
+// They are not part of the drop-in boundary and may change.
+#pragma once
+
+#include "../../include/cntk_amd_quantizer.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Forces kernel choices on a handle:
+ *   quantize_path    0 = automatic, 1 = LDS column tile, 2 = tall-column (global re-read),
+ *                    3 = one wavefront per column (1 bit, 2048 or 4096 rows only)
+ *   tile_gs          0 = automatic, else threads per column in the tile statistics phase (power of two, 8..256)
+ *   unq_slots        0 = automatic, else bit positions decoded per thread by unquantize
+ *   unq_force_scalar non-zero = never use the 16-byte store variant of unquantize */
+int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_gs, unsigned unq_slots,
+                           int unq_force_scalar);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,670 @@
+// gfx950 kernels of the per-column gradient quantizer.
+//
+// Work decomposition (fp32, QWord = uint32):
+//   * quantize_tile_kernel / stripe_reduce_tile_kernel: one workgroup owns a run of consecutive columns
+//     (a contiguous piece of the column-major matrix). It reads gradient and residual ONCE with
+//     coalesced 16-byte loads, keeps v = g + r in LDS, takes the column statistics from LDS
+//     (wavefront shuffles, LDS across wavefronts), then packs codes and writes the new residual.
+//   * quantize_wavecol_kernel: 1-bit columns whose QWord count is a multiple of 64; one wavefront
+//     owns a column, every lane owns whole QWords and keeps its share of the column in registers.
+//   * quantize_tall_kernel: columns too tall for LDS; statistics and packing re-read global memory.
+//   * unquantize_kernel: streams codes back to fp32 (optionally accumulating).
+//
+// Packed layout (Source/Math/QuantizedMatrix.h:27-48): column j = { f32 lower; f32 upper; u32 bits[nq] }
+// at byte j * qcol; element i of the column is in bits[i % nq] at bit (i / nq) * NBITS
+// (Source/Math/ColumnQuantizer.h:90-147).
+#pragma once
+
+#include "quantizer_math.h"
+
+namespace cntkq {
+
+constexpr uint32_t kTileThreads = 256;
+constexpr uint32_t kTallThreads = 1024;
+constexpr uint32_t kMaxWorkers = 64;
+
+// floats of LDS in front of the column tile: 8 reduction slots (4 float + 4 uint),
+// then (lower, upper) per tile column (at most 32 columns)
+constexpr uint32_t kTileScratchFloats = 8;
+constexpr uint32_t kTileMaxCols = 32;
+constexpr uint32_t kTilePrefixFloats = kTileScratchFloats + 2 * kTileMaxCols; // 72 floats = 288 B (16-B multiple)
+
+struct TileGeom
+{
+    uint32_t rows;
+    uint32_t cols;
+    uint32_t nq;            // QWords per column
+    uint32_t cols_per_tile; // kTileThreads / gs, <= kTileMaxCols
+    uint32_t gs;            // threads per column in the statistics phase: power of two in [8, 256]
+    uint32_t gs_log2;
+    uint64_t qcol;          // bytes per packed column
+};
+
+__host__ __device__ inline size_t tile_lds_bytes(const TileGeom& t, uint32_t workers)
+{
+    // prefix, tile (+3 floats of alignment slack, rounded up), per-(column, worker) decode constants
+    size_t tile_floats = (size_t) t.cols_per_tile * t.rows + 4;
+    tile_floats = (tile_floats + 3) & ~(size_t) 3;
+    return (kTilePrefixFloats + tile_floats + (size_t) 2 * workers * t.cols_per_tile) * sizeof(float);
+}
+
+// ---- statistics + packing of a tile that already sits in LDS --------------------------------------
+//
+// tile[c * rows + i] holds v(i, c) = value to quantize for tile column c. On return the column headers are
+// in global memory and in hdr[], codes are in global memory and the new residual v - unquantize(code) has
+// been written to res_out (dense, column-major, tile-relative).
+
+template <int NBITS, bool ZT>
+__device__ __forceinline__ void tile_stats(const float* tile, float* hdr, float* scratch_f, uint32_t* scratch_u,
+                                           const TileGeom& t, uint32_t nc, char* qtile)
+{
+    const uint32_t tid = threadIdx.x;
+    const uint32_t c = tid >> t.gs_log2;
+    const uint32_t lg = tid & (t.gs - 1);
+    const bool col_ok = c < nc;
+    const float* colv = tile + (size_t) c * t.rows;
+    float lo = 0.0f, hi = 0.0f;
+
+    if constexpr (NBITS == 1)
+    {
+        float mean = 0.0f;
+        if constexpr (!ZT)
+        {
+            float s = 0.0f;
+            if (col_ok)
+                for (uint32_t i = lg; i < t.rows; i += t.gs)
+                    s += colv[i];
+            s = group_sum(s, t.gs, scratch_f);
+            mean = s / (float) t.rows;
+        }
+        float s0 = 0.0f, s1 = 0.0f;
+        uint32_t n0 = 0, n1 = 0;
+        if (col_ok)
+        {
+            for (uint32_t i = lg; i < t.rows; i += t.gs)
+            {
+                const float v = colv[i];
+                if (v < mean)
+                {
+                    s0 += v;
+                    n0++;
+                }
+                else
+                {
+                    s1 += v;
+                    n1++;
+                }
+            }
+        }
+        s0 = group_sum(s0, t.gs, scratch_f);
+        s1 = group_sum(s1, t.gs, scratch_f);
+        n0 = group_sum(n0, t.gs, scratch_u);
+        n1 = group_sum(n1, t.gs, scratch_u);
+        finish_stats_1bit<ZT>(mean, s0, s1, n0, n1, t.rows, lo, hi);
+    }
+    else
+    {
+        float s = 0.0f;
+        if (col_ok)
+        {
+            for (uint32_t i = lg; i < t.rows; i += t.gs)
+            {
+                const float v = colv[i];
+                s += v * v;
+            }
+        }
+        s = group_sum(s, t.gs, scratch_f);
+        finish_stats_multibit(s, t.rows, lo, hi);
+    }
+
+    if (col_ok && lg == 0)
+    {
+        hdr[2 * c] = lo;
+        hdr[2 * c + 1] = hi;
+        // a record is only 4-byte aligned when the column has an odd number of QWords
+        float* gh = reinterpret_cast<float*>(qtile + (size_t) c * t.qcol);
+        gh[0] = lo;
+        gh[1] = hi;
+    }
+    __syncthreads();
+}
+
+template <int NBITS, bool ZT>
+__device__ __forceinline__ void tile_pack(const float* tile, const float* hdr, const TileGeom& t, uint32_t nc,
+                                          char* qtile, float* res_out)
+{
+    constexpr uint32_t VPW = 32 / NBITS;
+    constexpr uint32_t MASKBITS = NBITS & 31;
+    const uint32_t nwords = nc * t.nq;
+    for (uint32_t qi = threadIdx.x; qi < nwords; qi += kTileThreads)
+    {
+        const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
+        const uint32_t w = qi - c * t.nq;
+        const ValueQ vq = make_vq<NBITS>(hdr[2 * c], hdr[2 * c + 1]);
+        const float val0 = unquantize_value<NBITS>(vq, 0u);
+        const float val1 = unquantize_value<NBITS>(vq, 1u);
+        const float* colv = tile + (size_t) c * t.rows;
+        float* ro = res_out + (size_t) c * t.rows;
+        uint32_t word = 0;
+#pragma unroll
+        for (uint32_t k = 0; k < VPW; ++k)
+        {
+            const uint32_t i = w + k * t.nq;
+            if (i < t.rows)
+            {
+                const float v = colv[i];
+                const uint32_t code = quantize_value<NBITS, ZT>(vq, v);
+                float back;
+                if constexpr (NBITS == 1)
+                    back = code ? val1 : val0;
+                else
+                    back = unquantize_value<NBITS>(vq, code);
+                ro[i] = v - back;
+                word |= code << (k * MASKBITS);
+            }
+        }
+        reinterpret_cast<uint32_t*>(qtile + (size_t) c * t.qcol + 8)[w] = word;
+    }
+}
+
+// ---- quantize: gradient + residual -> packed codes + new residual -----------------------------------
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float* __restrict__ g, const float* r_in,
+                                                                     float* r_out, char* __restrict__ q, TileGeom t)
+{
+    extern __shared__ f32x4 smem_v4[];
+    float* smem = reinterpret_cast<float*>(smem_v4);
+    float* scratch_f = smem;
+    uint32_t* scratch_u = reinterpret_cast<uint32_t*>(smem + 4);
+    float* hdr = smem + kTileScratchFloats;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t j0 = blockIdx.x * t.cols_per_tile;
+    const uint32_t nc = min(t.cols_per_tile, t.cols - j0);
+    const size_t base = (size_t) j0 * t.rows;
+    const uint32_t total = nc * t.rows;
+    const float* gp = g + base;
+    const float* rp = r_in + base;
+
+    // The tile starts `mis` floats into its LDS area so that LDS and global addresses share 16-byte phase.
+    const uint32_t mis_g = (uint32_t) ((reinterpret_cast<uintptr_t>(gp) >> 2) & 3u);
+    const uint32_t mis_r = (uint32_t) ((reinterpret_cast<uintptr_t>(rp) >> 2) & 3u);
+    float* tile = smem + kTilePrefixFloats + mis_g;
+
+    if (mis_g == mis_r)
+    {
+        uint32_t head = (4u - mis_g) & 3u;
+        if (head > total)
+            head = total;
+        const uint32_t nvec = (total - head) >> 2;
+        const uint32_t tail0 = head + (nvec << 2);
+        if (tid < head)
+            tile[tid] = gp[tid] + rp[tid];
+        const f32x4* g4 = reinterpret_cast<const f32x4*>(gp + head);
+        const f32x4* r4 = reinterpret_cast<const f32x4*>(rp + head);
+        f32x4* t4 = reinterpret_cast<f32x4*>(tile + head);
+        for (uint32_t e0 = tid; e0 < nvec; e0 += 4 * kTileThreads)
+        {
+            f32x4 a[4], b[4];
+#pragma unroll
+            for (uint32_t u = 0; u < 4; ++u)
+            {
+                const uint32_t e = e0 + u * kTileThreads;
+                if (e < nvec)
+                {
+                    a[u] = __builtin_nontemporal_load(g4 + e);
+                    b[u] = __builtin_nontemporal_load(r4 + e);
+                }
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 4; ++u)
+            {
+                const uint32_t e = e0 + u * kTileThreads;
+                if (e < nvec)
+                    t4[e] = a[u] + b[u];
+            }
+        }
+        for (uint32_t e = tail0 + tid; e < total; e += kTileThreads)
+            tile[e] = gp[e] + rp[e];
+    }
+    else
+    {
+        for (uint32_t e = tid; e < total; e += kTileThreads)
+            tile[e] = gp[e] + rp[e];
+    }
+    __syncthreads();
+
+    char* qtile = q + (size_t) j0 * t.qcol;
+    tile_stats<NBITS, ZT>(tile, hdr, scratch_f, scratch_u, t, nc, qtile);
+    tile_pack<NBITS, ZT>(tile, hdr, t, nc, qtile, r_out + base);
+}
+
+// ---- stripe reduction: K packed stripes -> fp32 sum -> requantize with the stripe residual ----------
+
+struct StripeSources
+{
+    const char* q[kMaxWorkers]; // packed stripes, one per worker
+    uint32_t workers;
+    uint32_t owner;
+};
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(StripeSources src, float* stripe_res,
+                                                                          char* q_out, float* agg_out, TileGeom t)
+{
+    constexpr uint32_t VPW = 32 / NBITS;
+    constexpr uint32_t MASKBITS = NBITS & 31;
+    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << MASKBITS) - 1u);
+
+    extern __shared__ f32x4 smem_v4[];
+    float* smem = reinterpret_cast<float*>(smem_v4);
+    float* scratch_f = smem;
+    uint32_t* scratch_u = reinterpret_cast<uint32_t*>(smem + 4);
+    float* hdr = smem + kTileScratchFloats;
+    float* tile = smem + kTilePrefixFloats;
+    size_t tile_floats = ((size_t) t.cols_per_tile * t.rows + 4 + 3) & ~(size_t) 3;
+    float* dec = tile + tile_floats; // per (tile column, worker): two decode constants
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t j0 = blockIdx.x * t.cols_per_tile;
+    const uint32_t nc = min(t.cols_per_tile, t.cols - j0);
+    const size_t base = (size_t) j0 * t.rows;
+    const uint32_t K = src.workers;
+
+    // decode constants from every worker's column header: 1 bit -> the two levels, else (ufactor, lower)
+    for (uint32_t x = tid; x < nc * K; x += kTileThreads)
+    {
+        const uint32_t c = x / K;
+        const uint32_t wk = x - c * K;
+        const float* h = reinterpret_cast<const float*>(src.q[wk] + (size_t) (j0 + c) * t.qcol);
+        const ValueQ vq = make_vq<NBITS>(h[0], h[1]);
+        if constexpr (NBITS == 1)
+        {
+            dec[2 * x] = unquantize_value<NBITS>(vq, 0u);
+            dec[2 * x + 1] = unquantize_value<NBITS>(vq, 1u);
+        }
+        else
+        {
+            dec[2 * x] = vq.uf;
+            dec[2 * x + 1] = vq.lo;
+        }
+    }
+    __syncthreads();
+
+    const float* sp = stripe_res + base;
+    const uint32_t nwords = nc * t.nq;
+    for (uint32_t qi = tid; qi < nwords; qi += kTileThreads)
+    {
+        const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
+        const uint32_t w = qi - c * t.nq;
+        const size_t word_off = (size_t) (j0 + c) * t.qcol + 8 + (size_t) w * 4;
+        float acc[VPW];
+        {
+            // the owner's own stripe seeds the sum
+            const uint32_t word = *reinterpret_cast<const uint32_t*>(src.q[src.owner] + word_off);
+            const float a = dec[2 * (c * K + src.owner)];
+            const float b = dec[2 * (c * K + src.owner) + 1];
+#pragma unroll
+            for (uint32_t k = 0; k < VPW; ++k)
+            {
+                const uint32_t code = (word >> (k * MASKBITS)) & CODEMASK;
+                if constexpr (NBITS == 1)
+                    acc[k] = code ? b : a;
+                else
+                    acc[k] = unquantize_value<NBITS>(a, b, code);
+            }
+        }
+        for (uint32_t wk = 0; wk < K; ++wk)
+        {
+            if (wk == src.owner)
+                continue;
+            const uint32_t word = *reinterpret_cast<const uint32_t*>(src.q[wk] + word_off);
+            const float a = dec[2 * (c * K + wk)];
+            const float b = dec[2 * (c * K + wk) + 1];
+#pragma unroll
+            for (uint32_t k = 0; k < VPW; ++k)
+            {
+                const uint32_t code = (word >> (k * MASKBITS)) & CODEMASK;
+                float x;
+                if constexpr (NBITS == 1)
+                    x = code ? b : a;
+                else
+                    x = unquantize_value<NBITS>(a, b, code);
+                acc[k] = x + acc[k];
+            }
+        }
+        float* colv = tile + (size_t) c * t.rows;
+        const float* sc = sp + (size_t) c * t.rows;
+#pragma unroll
+        for (uint32_t k = 0; k < VPW; ++k)
+        {
+            const uint32_t i = w + k * t.nq;
+            if (i < t.rows)
+            {
+                if (agg_out != nullptr)
+                    agg_out[base + (size_t) c * t.rows + i] = acc[k];
+                colv[i] = acc[k] + sc[i];
+            }
+        }
+    }
+    __syncthreads();
+
+    char* qtile = q_out + (size_t) j0 * t.qcol;
+    tile_stats<NBITS, ZT>(tile, hdr, scratch_f, scratch_u, t, nc, qtile);
+    tile_pack<NBITS, ZT>(tile, hdr, t, nc, qtile, stripe_res + base);
+}
+
+// ---- quantize, 1 bit, one wavefront per column, column share in registers ---------------------------
+//
+// rows = 2048 * WPL, nq = 64 * WPL. Lane l owns QWords l, l + 64, ...; QWord w packs rows w + k * nq, so for
+// fixed k the 64 lanes read 64 consecutive floats, and each lane builds its QWords with shifts alone.
+
+template <bool ZT, int WPL>
+__global__ __launch_bounds__(kTileThreads) void quantize_wavecol_kernel(const float* __restrict__ g, const float* r_in,
+                                                                        float* r_out, char* __restrict__ q,
+                                                                        uint32_t cols, uint64_t qcol)
+{
+    constexpr uint32_t NQ = 64 * WPL;
+    constexpr uint32_t ROWS = 32 * NQ;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t j = blockIdx.x * (kTileThreads / 64) + (threadIdx.x >> 6);
+    if (j >= cols)
+        return; // whole wavefront leaves; no barriers below
+    const size_t base = (size_t) j * ROWS;
+    const float* gp = g + base + lane;
+    const float* rp = r_in + base + lane;
+
+    float v[WPL][32];
+#pragma unroll
+    for (int c = 0; c < WPL; ++c)
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+        {
+            const uint32_t i = 64u * c + NQ * k;
+            v[c][k] = __builtin_nontemporal_load(gp + i) + __builtin_nontemporal_load(rp + i);
+        }
+
+    float mean = 0.0f;
+    if constexpr (!ZT)
+    {
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < WPL; ++c)
+#pragma unroll
+            for (int k = 0; k < 32; ++k)
+                s += v[c][k];
+        s = wave_sum(s);
+        mean = s / (float) ROWS;
+    }
+    float s0 = 0.0f, s1 = 0.0f;
+    uint32_t n0 = 0;
+#pragma unroll
+    for (int c = 0; c < WPL; ++c)
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+        {
+            const float x = v[c][k];
+            const bool below = x < mean;
+            s0 += below ? x : 0.0f;
+            s1 += below ? 0.0f : x;
+            n0 += below ? 1u : 0u;
+        }
+    s0 = wave_sum(s0);
+    s1 = wave_sum(s1);
+    n0 = wave_sum(n0);
+    const uint32_t n1 = ROWS - n0;
+    float lo, hi;
+    finish_stats_1bit<ZT>(mean, s0, s1, n0, n1, ROWS, lo, hi);
+
+    char* qc = q + (size_t) j * qcol;
+    if (lane == 0)
+    {
+        f32x2 h;
+        h.x = lo;
+        h.y = hi;
+        *reinterpret_cast<f32x2*>(qc) = h;
+    }
+    const ValueQ vq = make_vq<1>(lo, hi);
+    const float val0 = unquantize_value<1>(vq, 0u);
+    const float val1 = unquantize_value<1>(vq, 1u);
+    float* op = r_out + base + lane;
+    uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
+#pragma unroll
+    for (int c = 0; c < WPL; ++c)
+    {
+        uint32_t word = 0;
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+        {
+            const float x = v[c][k];
+            const uint32_t code = quantize_value<1, ZT>(vq, x);
+            __builtin_nontemporal_store(x - (code ? val1 : val0), op + 64u * c + NQ * k);
+            word |= code << k;
+        }
+        bits[lane + 64u * c] = word;
+    }
+}
+
+// ---- quantize, columns too tall for LDS: one workgroup per column, global memory re-read -------------
+
+template <typename T>
+__device__ __forceinline__ T tall_block_sum(T v, T* scratch)
+{
+    v = wave_sum(v);
+    const uint32_t wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63u) == 0)
+        scratch[wave] = v;
+    __syncthreads();
+    T t = scratch[0];
+    for (uint32_t x = 1; x < kTallThreads / 64; ++x)
+        t += scratch[x];
+    __syncthreads();
+    return t;
+}
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTallThreads) void quantize_tall_kernel(const float* __restrict__ g, const float* r_in,
+                                                                     float* r_out, char* __restrict__ q, uint32_t rows,
+                                                                     uint32_t nq, uint64_t qcol)
+{
+    constexpr uint32_t VPW = 32 / NBITS;
+    constexpr uint32_t MASKBITS = NBITS & 31;
+    __shared__ float scratch_f[kTallThreads / 64];
+    __shared__ uint32_t scratch_u[kTallThreads / 64];
+
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * rows;
+    const float* gp = g + base;
+    const float* rp = r_in + base;
+    float lo, hi;
+
+    if constexpr (NBITS == 1)
+    {
+        float mean = 0.0f;
+        if constexpr (!ZT)
+        {
+            float s = 0.0f;
+            for (uint32_t i = tid; i < rows; i += kTallThreads)
+                s += gp[i] + rp[i];
+            s = tall_block_sum(s, scratch_f);
+            mean = s / (float) rows;
+        }
+        float s0 = 0.0f, s1 = 0.0f;
+        uint32_t n0 = 0, n1 = 0;
+        for (uint32_t i = tid; i < rows; i += kTallThreads)
+        {
+            const float v = gp[i] + rp[i];
+            if (v < mean)
+            {
+                s0 += v;
+                n0++;
+            }
+            else
+            {
+                s1 += v;
+                n1++;
+            }
+        }
+        s0 = tall_block_sum(s0, scratch_f);
+        s1 = tall_block_sum(s1, scratch_f);
+        n0 = tall_block_sum(n0, scratch_u);
+        n1 = tall_block_sum(n1, scratch_u);
+        finish_stats_1bit<ZT>(mean, s0, s1, n0, n1, rows, lo, hi);
+    }
+    else
+    {
+        float s = 0.0f;
+        for (uint32_t i = tid; i < rows; i += kTallThreads)
+        {
+            const float v = gp[i] + rp[i];
+            s += v * v;
+        }
+        s = tall_block_sum(s, scratch_f);
+        finish_stats_multibit(s, rows, lo, hi);
+    }
+    // every thread has passed the last barrier of tall_block_sum, so all statistics reads of r_in are done
+    // before any residual is written (r_out may be r_in)
+
+    char* qc = q + (size_t) blockIdx.x * qcol;
+    if (tid == 0)
+    {
+        float* gh = reinterpret_cast<float*>(qc);
+        gh[0] = lo;
+        gh[1] = hi;
+    }
+    const ValueQ vq = make_vq<NBITS>(lo, hi);
+    const float val0 = unquantize_value<NBITS>(vq, 0u);
+    const float val1 = unquantize_value<NBITS>(vq, 1u);
+    float* op = r_out + base;
+    uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
+    for (uint32_t w = tid; w < nq; w += kTallThreads)
+    {
+        uint32_t word = 0;
+#pragma unroll
+        for (uint32_t k = 0; k < VPW; ++k)
+        {
+            const uint32_t i = w + k * nq;
+            if (i < rows)
+            {
+                const float v = gp[i] + rp[i];
+                const uint32_t code = quantize_value<NBITS, ZT>(vq, v);
+                float back;
+                if constexpr (NBITS == 1)
+                    back = code ? val1 : val0;
+                else
+                    back = unquantize_value<NBITS>(vq, code);
+                op[i] = v - back;
+                word |= code << (k * MASKBITS);
+            }
+        }
+        bits[w] = word;
+    }
+}
+
+// ---- unquantize ---------------------------------------------------------------------------------------
+//
+// One thread decodes WV consecutive QWords of a column (WV = 4: 16-byte stores; WV = 1: any shape) for a
+// chunk of `slots` consecutive bit positions. For fixed bit position k the rows w + k * nq of
+// consecutive QWords are consecutive in memory, so stores coalesce.
+
+struct UnqGeom
+{
+    uint32_t rows;
+    uint32_t cols;
+    uint32_t nq;
+    uint32_t groups;  // ceil(nq / WV) word groups per column
+    uint32_t chunks;  // ceil(VPW / slots)
+    uint32_t slots;   // bit positions per thread
+    uint32_t per_col; // groups * chunks work items per column
+    uint32_t items;   // per_col * cols (the host refuses matrices that need more than 2^32 - 1)
+    uint64_t qcol;
+};
+
+template <int NBITS, int WV>
+__global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, float* out, UnqGeom t, int add)
+{
+    constexpr uint32_t VPW = 32 / NBITS;
+    constexpr uint32_t MASKBITS = NBITS & 31;
+    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << MASKBITS) - 1u);
+
+    const uint64_t id64 = (uint64_t) blockIdx.x * 256 + threadIdx.x;
+    if (id64 >= t.items)
+        return;
+    const uint32_t id = (uint32_t) id64;
+    const uint32_t c = id / t.per_col;
+    const uint32_t rem = id - c * t.per_col;
+    const uint32_t chunk = rem / t.groups;
+    const uint32_t grp = rem - chunk * t.groups;
+    const uint32_t w0 = grp * WV;
+
+    const char* qc = q + (size_t) c * t.qcol;
+    const float* gh = reinterpret_cast<const float*>(qc);
+    const ValueQ vq = make_vq<NBITS>(gh[0], gh[1]);
+    const float val0 = unquantize_value<NBITS>(vq, 0u);
+    const float val1 = unquantize_value<NBITS>(vq, 1u);
+    const uint32_t* bits = reinterpret_cast<const uint32_t*>(qc + 8);
+    float* oc = out + (size_t) c * t.rows;
+
+    uint32_t word[WV];
+    if constexpr (WV == 4)
+    {
+        // the word group starts 8 bytes past a 16-byte boundary or on one: two 8-byte loads are always aligned
+        const u32x2 a = *reinterpret_cast<const u32x2*>(bits + w0);
+        const u32x2 b = *reinterpret_cast<const u32x2*>(bits + w0 + 2);
+        word[0] = a.x;
+        word[1] = a.y;
+        word[2] = b.x;
+        word[3] = b.y;
+    }
+    else
+    {
+        word[0] = bits[w0];
+    }
+
+    const uint32_t k0 = chunk * t.slots;
+    const uint32_t k1 = min(k0 + t.slots, VPW);
+    for (uint32_t k = k0; k < k1; ++k)
+    {
+        const uint32_t i = w0 + k * t.nq;
+        if (i >= t.rows)
+            break; // rows only grow with k
+        const uint32_t sh = k * MASKBITS;
+        if constexpr (WV == 4)
+        {
+            // rows % 4 == 0 and i % 4 == 0: the four rows are all inside the column
+            f32x4 x;
+            if constexpr (NBITS == 1)
+            {
+                x.x = ((word[0] >> sh) & 1u) ? val1 : val0;
+                x.y = ((word[1] >> sh) & 1u) ? val1 : val0;
+                x.z = ((word[2] >> sh) & 1u) ? val1 : val0;
+                x.w = ((word[3] >> sh) & 1u) ? val1 : val0;
+            }
+            else
+            {
+                x.x = unquantize_value<NBITS>(vq, (word[0] >> sh) & CODEMASK);
+                x.y = unquantize_value<NBITS>(vq, (word[1] >> sh) & CODEMASK);
+                x.z = unquantize_value<NBITS>(vq, (word[2] >> sh) & CODEMASK);
+                x.w = unquantize_value<NBITS>(vq, (word[3] >> sh) & CODEMASK);
+            }
+            f32x4* dst = reinterpret_cast<f32x4*>(oc + i);
+            if (add)
+                x = x + *dst; // unquantized value + previous content
+            __builtin_nontemporal_store(x, dst);
+        }
+        else
+        {
+            float x;
+            if constexpr (NBITS == 1)
+                x = ((word[0] >> sh) & 1u) ? val1 : val0;
+            else
+                x = unquantize_value<NBITS>(vq, (word[0] >> sh) & CODEMASK);
+            if (add)
+                x = x + oc[i];
+            oc[i] = x;
+        }
+    }
+}
+
+} // namespace cntkq

@@ -1,0 +1,239 @@
+// Host-side kernel selection and launch for the per-column quantizer (gfx950).
+// Shared by the C-ABI library and by stand-alone timing programs; no allocation happens here.
+#pragma once
+
+#include "quantizer_kernels.h"
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace cntkq {
+
+// which quantize kernel to use
+enum QuantizePath
+{
+    kPathAuto = 0,
+    kPathTile = 1,    // LDS-staged column tile (rows <= kTileMaxRows)
+    kPathTall = 2,    // one workgroup per column, global re-read (any rows)
+    kPathWaveCol = 3  // 1 bit, rows in {2048, 4096}, one wavefront per column in registers
+};
+
+constexpr uint32_t kTileMaxRows = 15360; // 60 KB of LDS for a one-column tile
+
+struct LaunchTuning
+{
+    int quantize_path = kPathAuto;
+    uint32_t tile_gs = 0;   // 0 = pick from rows; else threads per column (power of two, 8..256)
+    uint32_t unq_slots = 0; // 0 = default; else bit positions per thread in unquantize
+    int unq_force_scalar = 0;
+};
+
+inline bool valid_nbits(size_t nbits)
+{
+    return nbits == 1 || nbits == 2 || nbits == 4 || nbits == 8 || nbits == 16 || nbits == 32;
+}
+
+inline size_t qwords_per_col(size_t rows, size_t nbits)
+{
+    const size_t per = 32 / nbits;
+    return (rows + per - 1) / per;
+}
+
+inline size_t qcol_bytes(size_t nbits, size_t rows)
+{
+    return 8 + ((rows * nbits + 31) / 32) * 4;
+}
+
+inline TileGeom make_tile_geom(size_t rows, size_t cols, size_t nbits, uint32_t gs_override)
+{
+    TileGeom t;
+    t.rows = (uint32_t) rows;
+    t.cols = (uint32_t) cols;
+    t.nq = (uint32_t) qwords_per_col(rows, nbits);
+    uint32_t gs = 8;
+    if (gs_override != 0)
+        gs = gs_override;
+    else
+        while (gs < kTileThreads && rows > (size_t) gs * 32)
+            gs <<= 1;
+    // a tile may not exceed 8192 floats unless it is a single column
+    while (gs < kTileThreads && (size_t) (kTileThreads / gs) * rows > 8192)
+        gs <<= 1;
+    t.gs = gs;
+    t.gs_log2 = 0;
+    while ((1u << t.gs_log2) < gs)
+        t.gs_log2++;
+    t.cols_per_tile = kTileThreads / gs;
+    t.qcol = qcol_bytes(nbits, rows);
+    return t;
+}
+
+template <template <int, bool> class Launcher, typename... Args>
+inline hipError_t dispatch_nbits(size_t nbits, bool zt, Args... args)
+{
+    switch (nbits)
+    {
+    case 1: return zt ? Launcher<1, true>::run(args...) : Launcher<1, false>::run(args...);
+    case 2: return Launcher<2, false>::run(args...);
+    case 4: return Launcher<4, false>::run(args...);
+    case 8: return Launcher<8, false>::run(args...);
+    case 16: return Launcher<16, false>::run(args...);
+    case 32: return Launcher<32, false>::run(args...);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <int NBITS, bool ZT>
+struct TileLauncher
+{
+    static hipError_t run(hipStream_t s, const float* g, const float* r_in, float* r_out, char* q, TileGeom t)
+    {
+        const uint32_t tiles = (t.cols + t.cols_per_tile - 1) / t.cols_per_tile;
+        const size_t lds = tile_lds_bytes(t, 0);
+        hipLaunchKernelGGL((quantize_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(kTileThreads), lds, s, g, r_in, r_out, q, t);
+        return hipGetLastError();
+    }
+};
+
+template <int NBITS, bool ZT>
+struct TallLauncher
+{
+    static hipError_t run(hipStream_t s, const float* g, const float* r_in, float* r_out, char* q, uint32_t rows,
+                          uint32_t cols, uint32_t nq, uint64_t qcol)
+    {
+        hipLaunchKernelGGL((quantize_tall_kernel<NBITS, ZT>), dim3(cols), dim3(kTallThreads), 0, s, g, r_in, r_out, q, rows,
+                           nq, qcol);
+        return hipGetLastError();
+    }
+};
+
+template <int NBITS, bool ZT>
+struct StripeLauncher
+{
+    static hipError_t run(hipStream_t s, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
+                          TileGeom t)
+    {
+        const uint32_t tiles = (t.cols + t.cols_per_tile - 1) / t.cols_per_tile;
+        const size_t lds = tile_lds_bytes(t, src.workers);
+        hipLaunchKernelGGL((stripe_reduce_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(kTileThreads), lds, s, src, stripe_res,
+                           q_out, agg_out, t);
+        return hipGetLastError();
+    }
+};
+
+inline bool wavecol_applicable(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows,
+                               size_t nbits)
+{
+    (void) g, (void) r_in, (void) r_out;
+    return nbits == 1 && (rows == 2048 || rows == 4096) && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
+}
+
+// Launches the quantize kernel(s) for one matrix. rows, cols > 0; pointers 4-byte aligned (checked by caller).
+inline hipError_t launch_quantize(hipStream_t s, const float* g, const float* r_in, float* r_out, void* q, size_t rows,
+                                  size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+{
+    zt = zt && (nbits == 1);
+    char* qc = static_cast<char*>(q);
+    int path = tune.quantize_path;
+    if (path == kPathAuto)
+    {
+        if (rows > kTileMaxRows)
+            path = kPathTall;
+        else
+            path = kPathTile;
+    }
+    if (path == kPathWaveCol)
+    {
+        if (!wavecol_applicable(g, r_in, r_out, q, rows, nbits))
+            return hipErrorInvalidValue;
+        const uint32_t blocks = (uint32_t) ((cols + 3) / 4);
+        const uint64_t qcol = qcol_bytes(nbits, rows);
+        if (rows == 2048)
+        {
+            if (zt)
+                hipLaunchKernelGGL((quantize_wavecol_kernel<true, 1>), dim3(blocks), dim3(kTileThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+            else
+                hipLaunchKernelGGL((quantize_wavecol_kernel<false, 1>), dim3(blocks), dim3(kTileThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+        }
+        else
+        {
+            if (zt)
+                hipLaunchKernelGGL((quantize_wavecol_kernel<true, 2>), dim3(blocks), dim3(kTileThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+            else
+                hipLaunchKernelGGL((quantize_wavecol_kernel<false, 2>), dim3(blocks), dim3(kTileThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+        }
+        return hipGetLastError();
+    }
+    if (path == kPathTile)
+    {
+        if (rows > kTileMaxRows)
+            return hipErrorInvalidValue;
+        const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs);
+        return dispatch_nbits<TileLauncher>(nbits, zt, s, g, r_in, r_out, qc, t);
+    }
+    return dispatch_nbits<TallLauncher>(nbits, zt, s, g, r_in, r_out, qc, (uint32_t) rows, (uint32_t) cols,
+                                        (uint32_t) qwords_per_col(rows, nbits), (uint64_t) qcol_bytes(nbits, rows));
+}
+
+inline hipError_t launch_stripe_reduce(hipStream_t s, const StripeSources& src, float* stripe_res, void* q_out,
+                                       float* agg_out, size_t rows, size_t cols, size_t nbits, bool zt,
+                                       const LaunchTuning& tune)
+{
+    zt = zt && (nbits == 1);
+    if (rows > kTileMaxRows)
+        return hipErrorInvalidValue;
+    const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs);
+    return dispatch_nbits<StripeLauncher>(nbits, zt, s, src, stripe_res, static_cast<char*>(q_out), agg_out, t);
+}
+
+template <int NBITS, int WV>
+inline hipError_t launch_unquantize_t(hipStream_t s, const char* q, float* out, size_t rows, size_t cols, uint32_t slots,
+                                      int add)
+{
+    constexpr uint32_t VPW = 32 / NBITS;
+    UnqGeom t;
+    t.rows = (uint32_t) rows;
+    t.cols = (uint32_t) cols;
+    t.nq = (uint32_t) qwords_per_col(rows, NBITS);
+    t.groups = (t.nq + WV - 1) / WV;
+    if (slots == 0)
+        slots = VPW < 8 ? VPW : 8;
+    if (slots > VPW)
+        slots = VPW;
+    t.slots = slots;
+    t.chunks = (VPW + slots - 1) / slots;
+    const uint64_t per_col = (uint64_t) t.groups * t.chunks;
+    const uint64_t items = per_col * cols;
+    if (items > 0xFFFFFFFFull)
+        return hipErrorInvalidValue;
+    t.per_col = (uint32_t) per_col;
+    t.items = (uint32_t) items;
+    t.qcol = qcol_bytes(NBITS, rows);
+    const uint32_t blocks = (uint32_t) ((items + 255) / 256);
+    hipLaunchKernelGGL((unquantize_kernel<NBITS, WV>), dim3(blocks), dim3(256), 0, s, q, out, t, add);
+    return hipGetLastError();
+}
+
+inline hipError_t launch_unquantize(hipStream_t s, const void* q, float* out, size_t rows, size_t cols, size_t nbits,
+                                    bool add, const LaunchTuning& tune)
+{
+    const char* qc = static_cast<const char*>(q);
+    const size_t nq = qwords_per_col(rows, nbits);
+    const bool vec = !tune.unq_force_scalar && (nq % 4 == 0) && (rows % 4 == 0) &&
+                     (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
+    const int a = add ? 1 : 0;
+    const uint32_t sl = tune.unq_slots;
+    switch (nbits)
+    {
+    case 1: return vec ? launch_unquantize_t<1, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<1, 1>(s, qc, out, rows, cols, sl, a);
+    case 2: return vec ? launch_unquantize_t<2, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<2, 1>(s, qc, out, rows, cols, sl, a);
+    case 4: return vec ? launch_unquantize_t<4, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<4, 1>(s, qc, out, rows, cols, sl, a);
+    case 8: return vec ? launch_unquantize_t<8, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<8, 1>(s, qc, out, rows, cols, sl, a);
+    case 16: return vec ? launch_unquantize_t<16, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<16, 1>(s, qc, out, rows, cols, sl, a);
+    case 32: return vec ? launch_unquantize_t<32, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<32, 1>(s, qc, out, rows, cols, sl, a);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+} // namespace cntkq

@@ -1,0 +1,144 @@
+/*
+ * cntk_amd_quantizer.h -- C ABI of the MI355X (gfx950) gradient quantizer.
+ *
+ * This is the boundary a CNTK build binds in place of MatrixQuantizerGPU: one opaque handle per
+ * MatrixQuantizerImpl<float> object, plain pointers and sizes, no C++ or torch types. Every call
+ * returns a status code; cntkq_last_error() gives the text the reference would have thrown.
+ *
+ * Data contracts (identical to the reference):
+ *   - gradients / residuals / outputs: dense fp32, column-major, rows x cols, leading dimension = rows
+ *     (Source/Math/ColumnQuantizer.h:10);
+ *   - packed matrix: cols records of cntkq_qcol_bytes(nbits, rows) bytes each, back to back:
+ *         { float lower; float upper; uint32_t bits[nq]; }      nq = cntkq_qwords_per_col(rows, nbits)
+ *     element i of a column is stored in bits[i % nq] at bit (i / nq) * nbits
+ *     (Source/Math/QuantizedMatrix.h:27-48, Source/Math/QuantizedMatrix.cpp:143-169).
+ *     A contiguous run of columns of a packed matrix is itself a packed matrix (ColumnSlice,
+ *     Source/Math/QuantizedMatrix.cpp:102-107): pass  buffer + first_col * qcol_bytes.
+ *   - nbits is one of 1, 2, 4, 8, 16, 32 (32 = pass-through, Source/Math/ValueQuantizer.h:104-107).
+ *
+ * Ordering: all work of a handle is issued on ONE HIP stream (cntkq_stream). Handles created with
+ * use_dedicated_stream != 0 on the same device share one process-wide non-blocking stream, exactly
+ * like the reference's static compute stream (Source/Math/MatrixQuantizerGPU.cu:83-90, 197-206), so
+ * work issued through different handles is implicitly sequenced. Handles created with
+ * use_dedicated_stream == 0 issue on the caller's main stream (the null stream unless
+ * cntkq_set_main_stream was called). A handle is not re-entrant; distinct handles may be used
+ * from distinct threads.
+ */
+#ifndef CNTK_AMD_QUANTIZER_H
+#define CNTK_AMD_QUANTIZER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct cntkq_quantizer cntkq_quantizer;
+
+enum
+{
+    CNTKQ_OK = 0,
+    CNTKQ_INVALID_ARGUMENT = 1, /* reference: InvalidArgument / failed assert on dimensions */
+    CNTKQ_LOGIC_ERROR = 2,      /* reference: LogicError (bad nbits, packed-size mismatch) */
+    CNTKQ_RUNTIME_ERROR = 3     /* reference: RuntimeError from a failed device call */
+};
+
+/* Text of the last failure on the calling thread ("" if none). */
+const char* cntkq_last_error(void);
+
+/* ---- layout helpers ------------------------------------------------------------------------ */
+
+/* ColumnQuantizer<float>::QWordsPerCol (Source/Math/ColumnQuantizer.h:36-45). 0 if nbits is invalid. */
+size_t cntkq_qwords_per_col(size_t rows, size_t nbits);
+
+/* QuantizedColumn<float>::QuantizedColumnSize (Source/Math/QuantizedMatrix.h:42-47). 0 if nbits is invalid. */
+size_t cntkq_qcol_bytes(size_t nbits, size_t rows);
+
+/* QuantizedMatrix<float>::GetSize (Source/Math/QuantizedMatrix.cpp:90-94): cols * qcol_bytes. */
+size_t cntkq_qmatrix_bytes(size_t rows, size_t cols, size_t nbits);
+
+/* AllReduceDistGradAggregator::GetStripeForNode (Source/1BitSGD/AllReduceDistGradAggregator.h:56-65). */
+int cntkq_stripe_range(size_t cols, size_t rank, size_t workers, size_t* start_col, size_t* num_cols);
+
+/* ---- the quantizer object -------------------------------------------------------------------- */
+
+/* MatrixQuantizerImpl<float>::Create(deviceId, useAsync) (Source/Math/MatrixQuantizerImpl.cpp:10-26) for
+ * deviceId >= 0, i.e. the MatrixQuantizerGPU constructor (Source/Math/MatrixQuantizerGPU.cu:183-207).
+ * device_id < 0 (the reference's CPU quantizer) is refused: this library has no CPU path. */
+int cntkq_create(int device_id, int use_dedicated_stream, cntkq_quantizer** out);
+
+/* ~MatrixQuantizerGPU (Source/Math/MatrixQuantizerGPU.cu:209-223). Waits for the handle's own work. */
+int cntkq_destroy(cntkq_quantizer* h);
+
+/* MatrixQuantizerImpl::GetDeviceId (Source/Math/MatrixQuantizerImpl.h:36-39). */
+int cntkq_device_id(const cntkq_quantizer* h);
+
+/* The hipStream_t the handle issues on (MatrixQuantizerGPU::GetComputeStream,
+ * Source/Math/MatrixQuantizerGPU.cu:92-96). */
+void* cntkq_stream(const cntkq_quantizer* h);
+
+/* Sets the main stream used by handles without a dedicated stream (the reference's GetStream(),
+ * Source/Math/MatrixQuantizerGPU.cu:248-252) and by cntkq_sync_with_main_stream. */
+int cntkq_set_main_stream(cntkq_quantizer* h, void* hip_stream);
+
+/* MatrixComputeStreamEvent::Create + SynchronizeQuantizationComputeStreamWithEvent
+ * (Source/Math/MatrixQuantizerImpl.h:53-72, Source/Math/MatrixQuantizerGPU.cu:347-371): work issued on the
+ * handle's stream after this call starts only after everything already issued on the main stream. */
+int cntkq_sync_with_main_stream(cntkq_quantizer* h);
+
+/* MatrixQuantizerImpl::QuantizeAsync (Source/Math/MatrixQuantizerImpl.h:30, Source/Math/MatrixQuantizerGPU.cu:226-269).
+ *   in, res_in, res_out : device, rows x cols fp32; res_out may be the same pointer as res_in (in place),
+ *                         no other overlap is allowed.
+ *   qbuf                : packed matrix, qbuf_bytes == cntkq_qmatrix_bytes(rows, cols, nbits);
+ *                         device memory, or (qbuf_on_host != 0) host memory, in which case the packed
+ *                         data is produced in a device staging buffer owned by the handle and copied
+ *                         out asynchronously (pinned host memory keeps that copy asynchronous).
+ *   zero_threshold_for_1bit : the reference's zeroThresholdFor1Bit; ignored unless nbits == 1.
+ * rows == 0 or cols == 0 is a no-op. */
+int cntkq_quantize_async(cntkq_quantizer* h, const float* in, const float* res_in, size_t rows, size_t cols,
+                         void* qbuf, size_t qbuf_bytes, int qbuf_on_host, size_t nbits, float* res_out,
+                         int zero_threshold_for_1bit);
+
+/* MatrixQuantizerImpl::WaitQuantizeAsyncDone (Source/Math/MatrixQuantizerGPU.cu:271-284): blocks the host
+ * until the last quantize of this handle (including its copy to the host, if any) has finished. */
+int cntkq_wait_quantize_done(cntkq_quantizer* h);
+
+/* MatrixQuantizerImpl::UnquantizeAsync (Source/Math/MatrixQuantizerImpl.h:33, Source/Math/MatrixQuantizerGPU.cu:286-334).
+ *   out = (add ? out : 0) + unquantize(qbuf).  qbuf_bytes must equal cntkq_qmatrix_bytes(rows, cols, nbits),
+ *   else CNTKQ_LOGIC_ERROR (Source/Math/MatrixQuantizer_kernel.cu:287-289); an empty buffer is a no-op (:290-291).
+ *   With qbuf_on_host != 0 the packed data is first copied to the handle's staging buffer. */
+int cntkq_unquantize_async(cntkq_quantizer* h, const void* qbuf, size_t qbuf_bytes, int qbuf_on_host, float* out,
+                           size_t rows, size_t cols, size_t nbits, int add);
+
+/* MatrixQuantizerImpl::WaitUnquantizeAsyncDone (Source/Math/MatrixQuantizerGPU.cu:336-341). */
+int cntkq_wait_unquantize_done(cntkq_quantizer* h);
+
+/* One owner's stripe reduction of the quantized all-reduce, fused into one pass
+ * (dataflow of Source/1BitSGD/AllReduceDistGradAggregator.h:365-375 and :385-436; v2:
+ * Source/1BitSGD/QuantizedDistributedCommunicator.h:423-471), replacing the reference's sequence
+ * UnquantizeAsync(own, add=false); (workers-1) x UnquantizeAsync(peer, add=true); QuantizeAsync(aggregate).
+ *   stripes      : host array of `workers` device pointers; stripes[w] is worker w's packed stripe
+ *                  (stripe_cols columns of height rows), all quantized with the same nbits.
+ *   owner        : index of the worker that owns this stripe. The fp32 sum is taken in the order
+ *                  owner first, then the other workers in ascending index (the reference adds them in
+ *                  message-arrival order).
+ *   stripe_res   : device, rows x stripe_cols fp32, the owner's aggregation residual; updated in place.
+ *   q_out        : device, packed stripe that receives the requantized aggregate; may be stripes[owner]
+ *                  (the reference overwrites the owner's own slice), must not overlap any other input.
+ *   agg_out      : optional (may be NULL) device rows x stripe_cols fp32 that receives the fp32 aggregate
+ *                  before requantization (the reference leaves it in the owner's slice of the gradient).
+ * Limits: 1 <= workers <= CNTKQ_MAX_WORKERS. */
+#define CNTKQ_MAX_WORKERS 64
+int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner,
+                              size_t rows, size_t stripe_cols, size_t nbits, float* stripe_res, void* q_out,
+                              float* agg_out, int zero_threshold_for_1bit);
+
+/* Blocks until the last stripe reduction of this handle has finished (the reference waits on the stripe
+ * quantizer's WaitQuantizeAsyncDone, Source/1BitSGD/AllReduceDistGradAggregator.h:494). */
+int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CNTK_AMD_QUANTIZER_H */

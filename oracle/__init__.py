@@ -54,6 +54,8 @@ def lib():
         L.oracle_quantize.argtypes = [ctypes.c_void_p, ctypes.c_void_p, _sz, _sz, ctypes.c_void_p, _sz,
                                       ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
         L.oracle_quantize.restype = ctypes.c_int
+        L.oracle_pack_with_headers.argtypes = L.oracle_quantize.argtypes
+        L.oracle_pack_with_headers.restype = ctypes.c_int
         L.oracle_unquantize.argtypes = [ctypes.c_void_p, _sz, _sz, _sz, ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
         L.oracle_unquantize.restype = ctypes.c_int
         L.oracle_stripe_range.argtypes = [_sz, _sz, _sz, ctypes.POINTER(_sz), ctypes.POINTER(_sz)]
@@ -139,6 +141,22 @@ def quantize(g, r_in, nbits, zero_threshold, r_out=None, threads=1, use_ref=Fals
     else:
         rc = lib().oracle_quantize(_ptr(g), _ptr(r_in), rows, cols, _ptr(q), nbits, _ptr(r_out),
                                    int(zero_threshold), threads)
+    if rc != 0:
+        raise ValueError("nbits must be one of 1, 2, 4, 8, 16, 32")
+    return q, r_out
+
+
+def pack_with_headers(g, r_in, q_with_headers, nbits, zero_threshold, threads=1):
+    """Codes and residual under the headers already stored in q_with_headers (not modified).
+    Returns (packed buffer, residual)."""
+    _colmajor(g, "g"), _colmajor(r_in, "r_in")
+    rows, cols = g.shape
+    q = np.array(q_with_headers, dtype=np.uint8, copy=True)
+    if q.size != cols * qcol_bytes(nbits, rows):
+        raise ValueError("packed buffer has the wrong size")
+    r_out = np.zeros_like(g, order="F")
+    rc = lib().oracle_pack_with_headers(_ptr(g), _ptr(r_in), rows, cols, _ptr(q), nbits, _ptr(r_out),
+                                        int(zero_threshold), threads)
     if rc != 0:
         raise ValueError("nbits must be one of 1, 2, 4, 8, 16, 32")
     return q, r_out

@@ -275,6 +275,25 @@ int oracle_quantize(const float* g, const float* r_in, size_t rows, size_t cols,
     return 0;
 }
 
+int oracle_pack_with_headers(const float* g, const float* r_in, size_t rows, size_t cols, void* qbuf,
+                             size_t nbits, float* r_out, int zero_threshold, int threads)
+{
+    /* second half of oracle_quantize alone: the (lower, upper) already stored in qbuf are kept */
+    if (oracle_check_nbits(nbits) != 0)
+        return -1;
+    const size_t qcol = oracle_qcol_bytes(nbits, rows);
+    char* q = (char*) qbuf;
+    long long n = (long long) cols;
+#pragma omp parallel for schedule(static) num_threads(threads) if (threads > 1)
+    for (long long jj = 0; jj < n; jj++)
+    {
+        size_t j = (size_t) jj;
+        float* hdr = (float*) (q + j * qcol);
+        quantize_column(g, r_in, rows, j, nbits, zero_threshold, hdr[0], hdr[1], (uint32_t*) (hdr + 2), r_out);
+    }
+    return 0;
+}
+
 int oracle_unquantize(const void* qbuf, size_t rows, size_t cols, size_t nbits, float* out, int add,
                       int threads)
 {

@@ -45,6 +45,12 @@ void oracle_column_stats(const float* g, const float* r, size_t rows, size_t j, 
 int oracle_quantize(const float* g, const float* r_in, size_t rows, size_t cols, void* qbuf,
                     size_t nbits, float* r_out, int zero_threshold, int threads);
 
+/* Packing step of oracle_quantize alone (Source/Math/ColumnQuantizer.h:50-65, 90-147): the column
+ * headers already present in qbuf are used as they are, only codes and residual are produced. Lets a
+ * test check codes and residuals bit for bit under headers that came from somewhere else. */
+int oracle_pack_with_headers(const float* g, const float* r_in, size_t rows, size_t cols, void* qbuf,
+                             size_t nbits, float* r_out, int zero_threshold, int threads);
+
 /* Inverse: out = (add ? out : 0) + unquantize(qbuf)
  * (Source/Math/MatrixQuantizerCPU.cpp:72-100, Source/Math/ColumnQuantizer.h:68-78, 149-203). */
 int oracle_unquantize(const void* qbuf, size_t rows, size_t cols, size_t nbits, float* out,

@@ -1,0 +1,69 @@
+"""Seeded synthetic gradients for the parity tests and the benchmark (column-major float32 numpy arrays).
+
+`exact_bell` uses integer arithmetic only, so its output is bit-identical on every machine and numpy
+version; the golden vectors whose inputs are not stored are generated from it. The other generators
+go through numpy's Generator and are used where both sides of a comparison see the same array.
+"""
+import numpy as np
+
+BASE_SEED = 0x1B17
+
+
+def case_seed(config, matrix=0, step=0, worker=0):
+    return BASE_SEED + 1000 * config + 100 * matrix + step + 10000 * worker
+
+
+def _f(a):
+    return np.asfortranarray(a.astype(np.float32))
+
+
+def _splitmix64(x):
+    x = (x + np.uint64(0x9E3779B97F4A7C15)) & np.uint64(0xFFFFFFFFFFFFFFFF)
+    z = x
+    z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+    z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+    return z ^ (z >> np.uint64(31))
+
+
+def exact_bell(seed, rows, cols, shift=22):
+    """Bell-shaped values (sum of four 16-bit uniforms, centred) times 2^-shift; exact in fp32.
+    Standard deviation = 2^-shift * 65536 / sqrt(3), e.g. about 0.009 for shift = 22."""
+    n = rows * cols
+    with np.errstate(over="ignore"):
+        idx = np.arange(n, dtype=np.uint64)
+        z = _splitmix64(idx * np.uint64(0x632BE59BD9B4E019) + np.uint64(seed) * np.uint64(0xD1342543DE82EF95))
+    parts = [(z >> np.uint64(16 * k)) & np.uint64(0xFFFF) for k in range(4)]
+    total = (parts[0] + parts[1] + parts[2] + parts[3]).astype(np.int64) - 2 * 65535
+    vals = np.ldexp(total.astype(np.float64), -shift)
+    return _f(vals.reshape((rows, cols), order="F"))
+
+
+def uniform(seed, rows, cols, lo, hi):
+    rng = np.random.default_rng(seed)
+    return _f(lo + (hi - lo) * rng.random((rows, cols)))
+
+
+def normal(seed, rows, cols, sigma=0.01):
+    rng = np.random.default_rng(seed)
+    return _f(rng.standard_normal((rows, cols)) * sigma)
+
+
+def student_t(seed, rows, cols, nu=3.0, scale=1e-3):
+    rng = np.random.default_rng(seed)
+    return _f(rng.standard_t(nu, (rows, cols)) * scale)
+
+
+def normal_with_outliers(seed, rows, cols, sigma=0.01, frac=0.01, mult=50.0):
+    rng = np.random.default_rng(seed)
+    a = rng.standard_normal((rows, cols)) * sigma
+    mask = rng.random((rows, cols)) < frac
+    a[mask] *= mult
+    return _f(a)
+
+
+def zero_columns(a, seed, frac=0.9):
+    """Zeroes a fixed (seed-dependent) subset of whole columns, in place; returns the mask of zeroed columns."""
+    rng = np.random.default_rng(seed)
+    mask = rng.random(a.shape[1]) < frac
+    a[:, mask] = 0.0
+    return mask

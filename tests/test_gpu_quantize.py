@@ -1,0 +1,275 @@
+"""Parity of the HIP quantizer against the CPU oracle, through the C ABI. Needs an MI355X.
+
+Mirrors the structure of the reference's own test (Tests/UnitTests/MathTests/MatrixQuantizerTests.cpp:239-402):
+for every bit width and, at 1 bit, both threshold modes, several iterations with the residual carried over and
+the output accumulated from the second iteration on; each iteration is checked against the oracle on the same
+(gradient, residual-in), which the oracle chain supplies (teacher forcing), and the free-running GPU chain is
+checked through the conservation law.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import cntk_amd
+import datagen
+import oracle
+import parity
+from cntk_amd import Matrix, MatrixQuantizerImpl, QuantizedMatrix
+
+pytestmark = pytest.mark.gpu
+
+VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False)]
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_WAVECOL = 0, 1, 2, 3
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def quantizer():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    q = MatrixQuantizerImpl.Create(0, False)
+    yield q
+    torch.cuda.synchronize()
+
+
+def gpu_quantize(qz, g, r_in, nbits, zt, in_place=True, host_q=False):
+    rows, cols = g.shape
+    G = Matrix.from_numpy(g)
+    R = Matrix.from_numpy(r_in)
+    Rout = R if in_place else Matrix(rows, cols)
+    Q = QuantizedMatrix(rows, cols, nbits, cntk_amd.CPUDEVICE if host_q else 0)
+    qz.QuantizeAsync(G, R, Q, Rout, zt)
+    qz.WaitQuantizeAsyncDone()
+    if not host_q:
+        torch.cuda.synchronize()
+    return Q, Rout.to_numpy()
+
+
+def run_chain(qz, rows, cols, nbits, zt, make_input, iterations, report, in_place=True, host_q=False):
+    """Teacher-forced chain: the oracle's residual feeds both sides at every step."""
+    res_o = np.zeros((rows, cols), np.float32, order="F")
+    out_o = np.zeros((rows, cols), np.float32, order="F")
+    Out = Matrix(rows, cols)
+    for it in range(iterations):
+        g = make_input(it)
+        Q, r_gpu = gpu_quantize(qz, g, res_o, nbits, zt, in_place=in_place, host_q=host_q)
+        q_gpu = Q.to_numpy()
+        parity.check_quantize(g, res_o, q_gpu, r_gpu, nbits, zt, report=report)
+        # unquantize what the GPU packed, accumulating like the reference test does
+        prev = Out.to_numpy()
+        qz.UnquantizeAsync(Q, Out, add=(it > 0))
+        qz.WaitUnquantizeAsyncDone()
+        parity.check_unquantize(q_gpu, rows, cols, nbits, Out.to_numpy(), prev_out=prev if it > 0 else None)
+        # carry the ORACLE's state forward so that both sides keep seeing identical inputs
+        q_or, _ = oracle.quantize(g, res_o, nbits, zt, r_out=res_o, threads=8)
+        oracle.unquantize(q_or, rows, cols, nbits, out=out_o, add=(it > 0), threads=8)
+        Out = Matrix.from_numpy(out_o)
+
+
+# ---- the reference unit test's shapes ------------------------------------------------------------------
+
+UNIT_SHAPES = [
+    (25, 13, -1.0, 1.0, 2015), (25, 13, -0.005, 0.005, 2115), (13, 25, -0.00001, 0.00001, 2215),
+    (13, 25, -10.0, 10.0, 2315), (25, 13, -1.0, 2.05, 2415), (489, 1, -0.5, 0.5, 2515), (1, 135, -0.5, 0.5, 2615),
+    (89, 23, -0.5, 0.5, 2715), (15, 35, -0.5, 0.5, 2815), (100, 50, -0.5, 0.5, 2915),
+    # the sizes the reference test was first written with (MatrixQuantizerTests.cpp:474-487)
+    (256, 135, -1.0, 2.05, 2415), (737, 373, -0.5, 0.5, 2915),
+]
+
+
+@pytest.mark.parametrize("shape", UNIT_SHAPES, ids=["%dx%d_%d" % (s[0], s[1], s[4]) for s in UNIT_SHAPES])
+def test_reference_unit_shapes(quantizer, shape):
+    rows, cols, lo, hi, seed = shape
+    rep = parity.Report()
+    for nbits, zt in VARIANTS:
+        say("unit shape", shape, "nbits", nbits, "zeroThr", zt)
+        run_chain(quantizer, rows, cols, nbits, zt, lambda it: datagen.uniform(seed + it, rows, cols, lo, hi), 5, rep)
+    say("  ", rep)
+
+
+def test_free_running_conservation(quantizer):
+    """GPU chain on its own state: g + r_in + prev_out == r_out + out (MatrixQuantizerTests.cpp:327-338)."""
+    rows, cols, lo, hi = 100, 50, -0.5, 0.5
+    for nbits, zt in VARIANTS:
+        say("conservation nbits", nbits, "zeroThr", zt)
+        R, Out = Matrix(rows, cols), Matrix(rows, cols)
+        for it in range(5):
+            g = datagen.uniform(2915 + it, rows, cols, lo, hi)
+            r_in, prev = R.to_numpy(), Out.to_numpy()
+            Q = QuantizedMatrix(rows, cols, nbits, 0)
+            quantizer.QuantizeAsync(Matrix.from_numpy(g), R, Q, R, zt)
+            quantizer.WaitQuantizeAsyncDone()
+            quantizer.UnquantizeAsync(Q, Out, add=(it > 0))
+            quantizer.WaitUnquantizeAsyncDone()
+            tol = (hi - lo) * 1e-4 if nbits != 32 else 1e-6
+            parity.conservation(g, r_in, prev, R.to_numpy(), Out.to_numpy(), tol)
+
+
+# ---- every kernel path on shapes that stress its indexing ------------------------------------------------
+
+PATH_CASES = [
+    # rows, cols, path, tile_gs
+    (1, 1, PATH_TILE, 0), (3, 70, PATH_TILE, 0), (31, 5, PATH_TILE, 8), (33, 67, PATH_TILE, 0), (64, 64, PATH_TILE, 16),
+    (147, 64, PATH_TILE, 0), (429, 37, PATH_TILE, 0), (429, 37, PATH_TILE, 64), (576, 64, PATH_TILE, 0),
+    (1023, 9, PATH_TILE, 0), (1024, 33, PATH_TILE, 0), (2048, 19, PATH_TILE, 0), (2048, 19, PATH_TILE, 256),
+    (2304, 5, PATH_TILE, 0), (4608, 3, PATH_TILE, 0), (9304, 2, PATH_TILE, 0), (15360, 1, PATH_TILE, 0),
+    (1, 5, PATH_TALL, 0), (70, 3, PATH_TALL, 0), (1025, 3, PATH_TALL, 0), (20001, 2, PATH_TALL, 0),
+    (33000, 2, PATH_AUTO, 0),
+]
+
+
+@pytest.mark.parametrize("case", PATH_CASES, ids=["%dx%d_p%d_g%d" % c for c in PATH_CASES])
+def test_kernel_paths(case):
+    rows, cols, path, gs = case
+    qz = MatrixQuantizerImpl.Create(0, False)
+    qz._set_tuning(quantize_path=path, tile_gs=gs)
+    rep = parity.Report()
+    for nbits, zt in VARIANTS:
+        say("path case", case, "nbits", nbits, "zeroThr", zt)
+        # a shifted mean, one all-zero column and outliers exercise every branch of the statistics
+        def make(it):
+            a = datagen.normal_with_outliers(1000 * rows + cols + it, rows, cols, 0.01) + np.float32(0.004 * (it % 2))
+            a = np.asfortranarray(a.astype(np.float32))
+            if cols > 1:
+                a[:, cols // 2] = 0.0
+            return a
+        run_chain(qz, rows, cols, nbits, zt, make, 2, rep)
+    say("  ", rep)
+
+
+@pytest.mark.parametrize("rows", [2048, 4096])
+def test_wavefront_per_column_path(rows):
+    qz = MatrixQuantizerImpl.Create(0, False)
+    qz._set_tuning(quantize_path=PATH_WAVECOL)
+    rep = parity.Report()
+    for cols in (1, 4, 7, 130):
+        for zt in (False, True):
+            say("wavecol", rows, cols, zt)
+            def make(it):
+                a = datagen.normal(rows + cols + it, rows, cols) + np.float32(0.003 * it)
+                a = np.asfortranarray(a.astype(np.float32))
+                if cols > 2:
+                    a[:, 1] = 0.0
+                return a
+            run_chain(qz, rows, cols, 1, zt, make, 3, rep)
+    say("  ", rep)
+    # shapes the path does not cover are refused, not mis-computed
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        gpu_quantize(qz, datagen.normal(1, 512, 4), np.zeros((512, 4), np.float32, order="F"), 1, False)
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        gpu_quantize(qz, datagen.normal(1, rows, 4), np.zeros((rows, 4), np.float32, order="F"), 2, False)
+
+
+def test_unquantize_variants(quantizer):
+    """Scalar and 16-byte-store decoders, every slot split, add and overwrite: all bit-exact."""
+    for rows, cols in [(5, 3), (37, 2), (128, 9), (429, 5), (2048, 6), (4100, 2)]:
+        for nbits, zt in VARIANTS:
+            g = datagen.normal(rows * 7 + nbits, rows, cols)
+            q, _ = oracle.quantize(g, np.zeros_like(g, order="F"), nbits, zt)
+            prev = datagen.normal(rows * 9 + nbits, rows, cols, 1.0)
+            for slots in (0, 1, 3, 32):
+                for scalar in (0, 1):
+                    say("unquantize", rows, cols, nbits, "slots", slots, "scalar", scalar)
+                    qz = MatrixQuantizerImpl.Create(0, False)
+                    qz._set_tuning(unq_slots=slots, unq_force_scalar=scalar)
+                    Q = QuantizedMatrix(rows, cols, nbits, 0)
+                    Q.from_numpy(q)
+                    for add in (False, True):
+                        Out = Matrix.from_numpy(prev)
+                        qz.UnquantizeAsync(Q, Out, add=add)
+                        qz.WaitUnquantizeAsyncDone()
+                        parity.check_unquantize(q, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
+
+
+# ---- boundary behaviour ------------------------------------------------------------------------------
+
+
+def test_out_of_place_residual_and_host_buffer(quantizer):
+    """Distinct in/out residual buffers (first call of the v2 communicator, QuantizedDistributedCommunicator.h:246-252)
+    and a host-resident packed matrix (the reference always stages through pinned host memory) give the same bytes."""
+    rows, cols = 429, 37
+    for nbits, zt in VARIANTS:
+        say("out-of-place / host", nbits, zt)
+        rep = parity.Report()
+        make = lambda it: datagen.student_t(50 + it, rows, cols)
+        run_chain(quantizer, rows, cols, nbits, zt, make, 2, rep, in_place=False)
+        run_chain(quantizer, rows, cols, nbits, zt, make, 2, rep, host_q=True)
+
+
+def test_column_slices_are_packed_matrices(quantizer):
+    """ColumnSlice of gradient, residual and packed matrix addresses the same bytes as the whole
+    (Source/Math/QuantizedMatrix.cpp:102-107) -- also exercises tiles that start at unaligned addresses."""
+    rows, cols, nbits = 429, 23, 1
+    g = datagen.normal(11, rows, cols)
+    r = datagen.normal(12, rows, cols, 0.002)
+    G, R, Q = Matrix.from_numpy(g), Matrix.from_numpy(r), QuantizedMatrix(rows, cols, nbits, 0)
+    for start, n in [(0, 5), (5, 1), (6, 17)]:
+        quantizer.QuantizeAsync(G.ColumnSlice(start, n), R.ColumnSlice(start, n), Q.ColumnSlice(start, n),
+                                R.ColumnSlice(start, n), False)
+    quantizer.WaitQuantizeAsyncDone()
+    parity.check_quantize(g, r, Q.to_numpy(), R.to_numpy(), nbits, False)
+    Out = Matrix(rows, cols)
+    quantizer.UnquantizeAsync(Q.ColumnSlice(3, 11), Out.ColumnSlice(3, 11))
+    quantizer.WaitUnquantizeAsyncDone()
+    ref = oracle.unquantize(Q.to_numpy(), rows, cols, nbits)
+    out = Out.to_numpy()
+    assert parity.bits_equal(np.asfortranarray(out[:, 3:14]), np.asfortranarray(ref[:, 3:14]))
+    assert not out[:, :3].any() and not out[:, 14:].any()
+
+
+def test_special_columns(quantizer):
+    """All-zero columns: lower = upper = 0, every valid bit 1, padding 0, residual 0 -- in both threshold modes."""
+    z = np.zeros((70, 3), np.float32, order="F")
+    for zt in (False, True):
+        Q, r = gpu_quantize(quantizer, z, z.copy(order="F"), 1, zt)
+        w = oracle.words(Q.to_numpy(), 70, 3, 1)
+        assert [hex(x) for x in w[0]] == ["0xffffff", "0x7fffff", "0x7fffff"]
+        lo, hi = oracle.headers(Q.to_numpy(), 70, 3, 1)
+        assert not lo.any() and not hi.any() and not r.any()
+    # the five-element column worked by hand
+    g = np.asfortranarray(np.array([[0.1], [-0.2], [0.3], [-0.4], [0.05]], np.float32))
+    Q, r = gpu_quantize(quantizer, g, np.zeros_like(g, order="F"), 1, False)
+    lo, hi = oracle.headers(Q.to_numpy(), 5, 1, 1)
+    assert abs(lo[0] + 0.462) < 1e-6 and abs(hi[0] - 0.402) < 1e-6
+    assert oracle.words(Q.to_numpy(), 5, 1, 1)[0, 0] == 0b10101
+
+
+def test_error_behaviour(quantizer):
+    g = Matrix(8, 4)
+    with pytest.raises(cntk_amd.QuantizerLogicError):  # dimension mismatch (asserts in the reference)
+        quantizer.QuantizeAsync(g, Matrix(8, 5), QuantizedMatrix(8, 4, 1, 0), g, False)
+    with pytest.raises(cntk_amd.QuantizerLogicError):  # packed size does not match the output matrix
+        quantizer.UnquantizeAsync(QuantizedMatrix(8, 4, 1, 0), Matrix(8, 5))
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        quantizer.UnquantizeAsync(QuantizedMatrix(8, 4, 2, 0), Matrix(16, 4))
+    # empty matrices are silent no-ops
+    quantizer.QuantizeAsync(Matrix(0, 4), Matrix(0, 4), QuantizedMatrix(0, 4, 1, 0), Matrix(0, 4), False)
+    quantizer.UnquantizeAsync(QuantizedMatrix(5, 0, 1, 0), Matrix(5, 0))
+    quantizer.WaitQuantizeAsyncDone()
+    quantizer.WaitUnquantizeAsyncDone()
+    assert quantizer.GetDeviceId() == 0
+
+
+def test_dedicated_stream_handles_share_one_stream():
+    """Handles created with useAsync share one process-wide stream, so work issued through different quantizer
+    objects is sequenced without waits -- callers rely on it (AllReduceDistGradAggregator.h:426-428)."""
+    a = MatrixQuantizerImpl.Create(0, True)
+    b = MatrixQuantizerImpl.Create(0, True)
+    c = MatrixQuantizerImpl.Create(0, False)
+    assert a.stream() == b.stream() and a.stream() is not None and a.stream() != c.stream()
+    rows, cols = 2048, 64
+    g = datagen.normal(3, rows, cols)
+    G = Matrix.from_numpy(g)
+    R, Out, Q = Matrix(rows, cols), Matrix(rows, cols), QuantizedMatrix(rows, cols, 1, 0)
+    torch.cuda.synchronize()
+    a.SynchronizeWithMainStream()
+    a.QuantizeAsync(G, R, Q, R, False)
+    b.UnquantizeAsync(Q, Out)  # no wait in between: same stream
+    b.WaitUnquantizeAsyncDone()
+    parity.check_quantize(g, np.zeros_like(g, order="F"), Q.to_numpy(), R.to_numpy(), 1, False)
+    parity.check_unquantize(Q.to_numpy(), rows, cols, 1, Out.to_numpy())

@@ -1,0 +1,219 @@
+"""Parity of the fused stripe reduction and of the whole simulated K-worker quantized all-reduce
+(Source/1BitSGD/AllReduceDistGradAggregator.h:268-531) against the CPU oracle. Needs an MI355X.
+
+All K workers live in one GPU's memory. The fp32 sum inside the stripe reduction has a fixed order (owner
+first, then ascending rank), so the fp32 aggregate must equal the oracle's bit for bit; the requantized
+stripe is then checked like any quantize result.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import cntk_amd
+import datagen
+import oracle
+import parity
+from cntk_amd import Matrix, MatrixQuantizer, MatrixQuantizerImpl, QuantizedMatrix
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def gpu_stripe_reduce(qz, q_workers, owner, rows, cols, nbits, stripe_res, zt, alias_out=True):
+    """q_workers: list of numpy packed FULL matrices; returns (new packed stripe, new stripe residual, aggregate)."""
+    k = len(q_workers)
+    start, n = cntk_amd.stripe_range(cols, owner, k)
+    Qs = []
+    for q in q_workers:
+        Q = QuantizedMatrix(rows, cols, nbits, 0)
+        Q.from_numpy(q)
+        Qs.append(Q)
+    stripes = [Q.ColumnSlice(start, n) for Q in Qs]
+    S = Matrix.from_numpy(stripe_res)
+    Agg = Matrix(rows, n)
+    out_q = stripes[owner] if alias_out else QuantizedMatrix(rows, n, nbits, 0)
+    qz.StripeReduceAsync(stripes, owner, S, out_q, zt, agg_out=Agg)
+    qz.WaitStripeReduceDone()
+    torch.cuda.synchronize()
+    return out_q.to_numpy(), S.to_numpy(), Agg.to_numpy()
+
+
+CASES = [
+    # rows, cols, workers, nbits, zeroThr
+    (5, 7, 2, 1, False), (37, 11, 3, 2, False), (70, 10, 4, 1, True), (429, 40, 8, 1, False), (429, 40, 8, 1, True),
+    (147, 64, 8, 4, False), (576, 24, 5, 8, False), (100, 9, 3, 16, False), (64, 12, 4, 32, False),
+    (2048, 48, 8, 1, False), (2048, 48, 8, 1, True), (2048, 16, 8, 2, False), (4608, 8, 2, 1, False),
+    (9304, 3, 3, 1, True), (33, 5, 8, 1, False), (512, 64, 64, 1, False),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=["%dx%d_k%d_b%d_z%d" % (c[0], c[1], c[2], c[3], int(c[4])) for c in CASES])
+def test_stripe_reduce(case):
+    rows, cols, k, nbits, zt = case
+    qz = MatrixQuantizerImpl.Create(0, False)
+    gs = [datagen.normal(datagen.case_seed(4, 0, 0, w) + rows, rows, cols) for w in range(k)]
+    zeros = np.zeros((rows, cols), np.float32, order="F")
+    qs = [oracle.quantize(g, zeros, nbits, zt, threads=8)[0] for g in gs]
+    rep = parity.Report()
+    for owner in sorted({0, k // 2, k - 1}):
+        start, n = oracle.stripe_range(cols, owner, k)
+        if n == 0:
+            continue
+        say("stripe reduce", case, "owner", owner, "cols", start, n)
+        sres = datagen.normal(900 + owner, rows, n, 0.003)
+        for alias in (True, False):
+            q_new, s_new, agg = gpu_stripe_reduce(qz, qs, owner, rows, cols, nbits, sres, zt, alias_out=alias)
+            # oracle on copies
+            qs_o = [q.copy() for q in qs]
+            s_o = sres.copy(order="F")
+            agg_o = oracle.stripe_reduce(qs_o, owner, rows, cols, nbits, s_o, zt, threads=8)
+            assert parity.bits_equal(agg, agg_o), "fp32 aggregate differs from the oracle (order: owner, then ascending)"
+            # the requantization sees (aggregate, stripe residual) as (gradient, residual)
+            parity.check_quantize(agg_o, sres, q_new, s_new, nbits, zt, report=rep)
+    say("  ", rep)
+
+
+def test_stripe_reduce_32bit_equals_plain_sum():
+    """The reference's own known-answer trick (32 bits: Tests/EndToEndTests/CNTKv2Library/EndToEndTests/FrameMode.cpp:112-116)."""
+    rows, cols, k = 129, 24, 4
+    qz = MatrixQuantizerImpl.Create(0, False)
+    gs = [datagen.normal(70 + w, rows, cols, 1.0) for w in range(k)]
+    zeros = np.zeros((rows, cols), np.float32, order="F")
+    qs = [oracle.quantize(g, zeros, 32, False)[0] for g in gs]
+    for owner in range(k):
+        start, n = oracle.stripe_range(cols, owner, k)
+        q_new, s_new, agg = gpu_stripe_reduce(qz, qs, owner, rows, cols, 32, np.zeros((rows, n), np.float32, order="F"), False)
+        acc = gs[owner][:, start:start + n].copy()
+        for w in range(k):
+            if w != owner:
+                acc = gs[w][:, start:start + n] + acc
+        assert parity.bits_equal(np.asfortranarray(acc), agg)
+        assert not s_new.any()
+        assert parity.bits_equal(oracle.unquantize(q_new, rows, n, 32), np.asfortranarray(acc))
+
+
+def simulated_allreduce_gpu(gs, res, sres, nbits, zt, use_async):
+    """The aggregator's dataflow on one GPU: per-worker MatrixQuantizer objects, stripes exchanged by pointer.
+    Returns (worker residuals, stripe residuals, packed matrices before the reduction, assembled packed
+    aggregate, output)."""
+    k = len(gs)
+    rows, cols = gs[0].shape
+    workers = [MatrixQuantizer(rows, cols, 0, use_async) for _ in range(k)]
+    G = [Matrix.from_numpy(g) for g in gs]
+    Q = [QuantizedMatrix(rows, cols, nbits, 0) for _ in range(k)]
+    S = [Matrix.from_numpy(s) for s in sres]
+    for w in range(k):
+        workers[w].GetResidualMatrix().data.copy_(Matrix.from_numpy(res[w]).data)
+    torch.cuda.synchronize()
+    for w in range(k):
+        workers[w].impl.SynchronizeWithMainStream()
+        workers[w].QuantizeAsync(G[w], Q[w], zt)
+    for w in range(k):
+        workers[w].WaitQuantizeAsyncDone()
+    torch.cuda.synchronize()
+    q_before = [q.to_numpy() for q in Q]
+    for s in range(k):
+        start, n = cntk_amd.stripe_range(cols, s, k)
+        if n == 0:
+            continue
+        stripes = [Q[w].ColumnSlice(start, n) for w in range(k)]
+        # the owner's requantized stripe overwrites its own slice, as in the reference
+        workers[s].impl.StripeReduceAsync(stripes, s, S[s], stripes[s], zt)
+    for s in range(k):
+        workers[s].impl.WaitStripeReduceDone()
+    torch.cuda.synchronize()
+    # "broadcast": assemble the requantized stripes; every worker would unquantize this same buffer
+    Qagg = QuantizedMatrix(rows, cols, nbits, 0)
+    for s in range(k):
+        start, n = cntk_amd.stripe_range(cols, s, k)
+        if n:
+            Qagg.ColumnSlice(start, n).buffer.copy_(Q[s].ColumnSlice(start, n).buffer)
+    torch.cuda.synchronize()
+    Out = Matrix(rows, cols)
+    workers[0].impl.SynchronizeWithMainStream()
+    workers[0].UnquantizeAsync(Qagg, Out)
+    workers[0].WaitUnquantizeAsyncDone()
+    torch.cuda.synchronize()
+    return ([w.GetResidualMatrix().to_numpy() for w in workers], [s.to_numpy() for s in S], q_before,
+            Qagg.to_numpy(), Out.to_numpy())
+
+
+ALLREDUCE_SHAPES = [(429, 37, 8, 1, True), (2048, 64, 8, 1, False), (576, 20, 3, 4, False), (64, 5, 8, 1, False)]
+
+
+@pytest.mark.parametrize("shape", ALLREDUCE_SHAPES, ids=lambda s: "%dx%d_k%d_b%d" % (s[0], s[1], s[2], s[3]))
+@pytest.mark.parametrize("use_async", [False, True], ids=["mainstream", "dedicated"])
+def test_simulated_allreduce(shape, use_async):
+    """Two carried steps of the whole all-reduce. Every stage is checked against the oracle applied to the
+    GPU's own previous stage (so each comparison sees identical inputs); the end-to-end aggregate is then
+    compared with the free-standing oracle run."""
+    rows, cols, k, nbits, zt = shape
+    res_o = [np.zeros((rows, cols), np.float32, order="F") for _ in range(k)]
+    sres_o = [np.zeros((rows, oracle.stripe_range(cols, s, k)[1]), np.float32, order="F") for s in range(k)]
+    qcol = oracle.qcol_bytes(nbits, rows)
+    rep = parity.Report()
+    for step in range(2):
+        say("all-reduce", shape, "async", use_async, "step", step)
+        gs = [datagen.normal(datagen.case_seed(4, 1, step, w), rows, cols) for w in range(k)]
+        res_in = [r.copy(order="F") for r in res_o]
+        sres_in = [s.copy(order="F") for s in sres_o]
+        res_g, sres_g, q1_g, qagg_g, out_g = simulated_allreduce_gpu(gs, res_in, sres_in, nbits, zt, use_async)
+        qs_o, qagg_o, out_o = oracle.allreduce(gs, res_o, sres_o, nbits, zt, threads=8)
+
+        # stage 1: every worker's own quantization
+        for w in range(k):
+            parity.check_quantize(gs[w], res_in[w], q1_g[w], res_g[w], nbits, zt, report=rep)
+        # stage 2: each owner's stripe reduction, given the GPU's stage-1 buffers
+        for s in range(k):
+            start, n = oracle.stripe_range(cols, s, k)
+            if n == 0:
+                continue
+            q_copy = [q.copy() for q in q1_g]
+            s_copy = sres_in[s].copy(order="F")
+            agg = oracle.stripe_reduce(q_copy, s, rows, cols, nbits, s_copy, zt, threads=8)
+            parity.check_quantize(agg, sres_in[s], qagg_g[start * qcol:(start + n) * qcol], sres_g[s], nbits, zt,
+                                  report=rep)
+        # stage 3: unquantize is exact given the packed buffer
+        parity.check_unquantize(qagg_g, rows, cols, nbits, out_g)
+
+        # end to end against the free-standing oracle: aggregated gradient within 1e-5 of the column scale
+        # wherever the packed codes agree (a first-stage code that flips at its threshold moves that element's
+        # aggregate by a whole level, which may in turn move second-stage codes)
+        lo, hi = oracle.headers(qagg_o, rows, cols, nbits)
+        scale = np.maximum(np.abs(hi.astype(np.float64) - lo), np.finfo(np.float32).tiny)
+        same = oracle.codes(qagg_g, rows, cols, nbits) == oracle.codes(qagg_o, rows, cols, nbits)
+        err = np.where(same, np.abs(out_g.astype(np.float64) - out_o) / scale[None, :], 0.0)
+        say("   aggregated gradient: max err %.3g of column scale, %d of %d codes differ"
+            % (err.max(), int((~same).sum()), same.size))
+        assert err.max() <= parity.VALUE_RTOL
+        assert int((~same).sum()) <= max(2, int(1e-3 * same.size))
+    say("  ", rep)
+
+
+def test_config4_shape_one_stripe():
+    """BASELINE config 4 at its real shape, one owner: 8 workers x 2048x9304, stripe 2048x1163."""
+    rows, cols, k, nbits = 2048, 9304, 8, 1
+    qz = MatrixQuantizerImpl.Create(0, False)
+    zeros = np.zeros((rows, cols), np.float32, order="F")
+    qs = []
+    for w in range(k):
+        g = datagen.normal(datagen.case_seed(4, 0, 0, w), rows, cols)
+        qs.append(oracle.quantize(g, zeros, nbits, False, threads=8)[0])
+    owner = 3
+    start, n = oracle.stripe_range(cols, owner, k)
+    assert (start, n) == (3 * 1163, 1163)
+    sres = datagen.normal(4242, rows, n, 0.004)
+    say("config 4 stripe", owner)
+    q_new, s_new, agg = gpu_stripe_reduce(qz, qs, owner, rows, cols, nbits, sres, False)
+    qs_o = [q.copy() for q in qs]
+    s_o = sres.copy(order="F")
+    agg_o = oracle.stripe_reduce(qs_o, owner, rows, cols, nbits, s_o, False, threads=8)
+    assert parity.bits_equal(agg, agg_o)
+    rep = parity.check_quantize(agg_o, sres, q_new, s_new, nbits, False)
+    say("  ", rep)
