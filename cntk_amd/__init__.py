@@ -65,7 +65,7 @@ def lib():
         L.cntkq_stripe_reduce_async.argtypes = [_vp, ctypes.POINTER(_vp), _sz, _sz, _sz, _sz, _sz, _vp, _vp, _vp,
                                                 ctypes.c_int]
         L.cntkq_wait_stripe_reduce_done.argtypes = [_vp]
-        L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int]
+        L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int]
         _lib = L
     return _lib
 
@@ -252,6 +252,9 @@ class MatrixQuantizerImpl:
 
     def UnquantizeAsync(self, in_qmatrix, out_matrix, add=False):
         rows, cols = out_matrix.GetNumRows(), out_matrix.GetNumCols()
+        # the reference asserts this (Source/Math/MatrixQuantizerGPU.cu:297)
+        if in_qmatrix.GetNumRows() != rows or in_qmatrix.GetNumCols() != cols:
+            raise QuantizerLogicError("UnquantizeAsync: matrix dimensions do not match")
         _check(lib().cntkq_unquantize_async(self._h, in_qmatrix.Buffer(), in_qmatrix.GetSize(),
                                             int(in_qmatrix.GetDeviceId() < 0), out_matrix.Data(), rows, cols,
                                             in_qmatrix.GetNumBits(), int(bool(add))))
@@ -277,8 +280,8 @@ class MatrixQuantizerImpl:
     def WaitStripeReduceDone(self):
         _check(lib().cntkq_wait_stripe_reduce_done(self._h))
 
-    def _set_tuning(self, quantize_path=0, tile_gs=0, unq_slots=0, unq_force_scalar=0):
-        _check(lib().cntkq_debug_set_tuning(self._h, quantize_path, tile_gs, unq_slots, unq_force_scalar))
+    def _set_tuning(self, quantize_path=0, tile_gs=0, unq_slots=0, unq_force_scalar=0, tile_stage=-1):
+        _check(lib().cntkq_debug_set_tuning(self._h, quantize_path, tile_gs, unq_slots, unq_force_scalar, tile_stage))
 
 
 class MatrixQuantizer:

@@ -13,9 +13,10 @@ extern "C" {
  *                    3 = one wavefront per column (1 bit, 2048 or 4096 rows only)
  *   tile_gs          0 = automatic, else threads per column in the tile statistics phase (power of two, 8..256)
  *   unq_slots        0 = automatic, else bit positions decoded per thread by unquantize
- *   unq_force_scalar non-zero = never use the 16-byte store variant of unquantize */
+ *   unq_force_scalar non-zero = never use the 16-byte store variant of unquantize
+ *   tile_stage       -1 = automatic, 0 = tile kernels write the residual straight to memory, 1 = through LDS */
 int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_gs, unsigned unq_slots,
-                           int unq_force_scalar);
+                           int unq_force_scalar, int tile_stage);
 
 #ifdef __cplusplus
 }

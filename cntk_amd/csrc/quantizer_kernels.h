@@ -29,6 +29,18 @@ constexpr uint32_t kTileScratchFloats = 8;
 constexpr uint32_t kTileMaxCols = 32;
 constexpr uint32_t kTilePrefixFloats = kTileScratchFloats + 2 * kTileMaxCols; // 72 floats = 288 B (16-B multiple)
 
+// A QWord is assembled from work items of at most 8 bit positions each, so that a tile with few QWords
+// still keeps every thread busy; the partial words meet in LDS (atomic OR).
+template <int NBITS>
+struct PackShape
+{
+    static constexpr uint32_t VPW = 32 / NBITS;              // values per QWord
+    static constexpr uint32_t SLOTS = VPW < 8 ? VPW : 8;     // bit positions per work item
+    static constexpr uint32_t CHUNKS = VPW / SLOTS;          // work items per QWord (4, 2, 1, 1, 1, 1)
+    static constexpr uint32_t SHIFT = NBITS & 31;
+    static constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
+};
+
 struct TileGeom
 {
     uint32_t rows;
@@ -37,15 +49,17 @@ struct TileGeom
     uint32_t cols_per_tile; // kTileThreads / gs, <= kTileMaxCols
     uint32_t gs;            // threads per column in the statistics phase: power of two in [8, 256]
     uint32_t gs_log2;
+    uint32_t tile_floats;   // LDS floats reserved for the tile: cols_per_tile * rows + alignment slack, multiple of 4
+    uint32_t words_floats;  // LDS words for partial QWords: cols_per_tile * nq when a QWord has several work items, else 0
+    uint32_t stage_residual; // non-zero: the new residual goes back through LDS and leaves in 16-byte stores
     uint64_t qcol;          // bytes per packed column
 };
 
+// LDS layout in floats: [prefix | tile | partial QWords | decode constants (2 * workers * cols_per_tile)]
 __host__ __device__ inline size_t tile_lds_bytes(const TileGeom& t, uint32_t workers)
 {
-    // prefix, tile (+3 floats of alignment slack, rounded up), per-(column, worker) decode constants
-    size_t tile_floats = (size_t) t.cols_per_tile * t.rows + 4;
-    tile_floats = (tile_floats + 3) & ~(size_t) 3;
-    return (kTilePrefixFloats + tile_floats + (size_t) 2 * workers * t.cols_per_tile) * sizeof(float);
+    return ((size_t) kTilePrefixFloats + t.tile_floats + t.words_floats + (size_t) 2 * workers * t.cols_per_tile) *
+           sizeof(float);
 }
 
 // ---- statistics + packing of a tile that already sits in LDS --------------------------------------
@@ -129,26 +143,32 @@ __device__ __forceinline__ void tile_stats(const float* tile, float* hdr, float*
     __syncthreads();
 }
 
+// words[] (LDS, nc * nq entries) must be zero on entry when PackShape<NBITS>::CHUNKS > 1.
 template <int NBITS, bool ZT>
-__device__ __forceinline__ void tile_pack(const float* tile, const float* hdr, const TileGeom& t, uint32_t nc,
-                                          char* qtile, float* res_out)
+__device__ __forceinline__ void tile_pack(float* tile, const float* hdr, uint32_t* words, const TileGeom& t,
+                                          uint32_t nc, char* qtile, float* res_out)
 {
-    constexpr uint32_t VPW = 32 / NBITS;
-    constexpr uint32_t MASKBITS = NBITS & 31;
+    using PS = PackShape<NBITS>;
     const uint32_t nwords = nc * t.nq;
-    for (uint32_t qi = threadIdx.x; qi < nwords; qi += kTileThreads)
+    const uint32_t items = nwords * PS::CHUNKS;
+    const bool stage = t.stage_residual != 0;
+    for (uint32_t it = threadIdx.x; it < items; it += kTileThreads)
     {
+        // chunk-major: consecutive threads take consecutive QWords, hence consecutive rows
+        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
+        const uint32_t qi = it - chunk * nwords;
         const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
         const uint32_t w = qi - c * t.nq;
         const ValueQ vq = make_vq<NBITS>(hdr[2 * c], hdr[2 * c + 1]);
         const float val0 = unquantize_value<NBITS>(vq, 0u);
         const float val1 = unquantize_value<NBITS>(vq, 1u);
-        const float* colv = tile + (size_t) c * t.rows;
+        float* colv = tile + (size_t) c * t.rows;
         float* ro = res_out + (size_t) c * t.rows;
         uint32_t word = 0;
 #pragma unroll
-        for (uint32_t k = 0; k < VPW; ++k)
+        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
         {
+            const uint32_t k = chunk * PS::SLOTS + kk;
             const uint32_t i = w + k * t.nq;
             if (i < t.rows)
             {
@@ -159,11 +179,61 @@ __device__ __forceinline__ void tile_pack(const float* tile, const float* hdr, c
                     back = code ? val1 : val0;
                 else
                     back = unquantize_value<NBITS>(vq, code);
-                ro[i] = v - back;
-                word |= code << (k * MASKBITS);
+                const float res = v - back;
+                if (stage)
+                    colv[i] = res; // this element belongs to this work item alone
+                else
+                    __builtin_nontemporal_store(res, ro + i);
+                word |= code << (k * PS::SHIFT);
             }
         }
-        reinterpret_cast<uint32_t*>(qtile + (size_t) c * t.qcol + 8)[w] = word;
+        if constexpr (PS::CHUNKS == 1)
+            reinterpret_cast<uint32_t*>(qtile + (size_t) c * t.qcol + 8)[w] = word;
+        else
+            atomicOr(&words[qi], word);
+    }
+    if constexpr (PS::CHUNKS > 1)
+    {
+        __syncthreads();
+        for (uint32_t qi = threadIdx.x; qi < nwords; qi += kTileThreads)
+        {
+            const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
+            const uint32_t w = qi - c * t.nq;
+            reinterpret_cast<uint32_t*>(qtile + (size_t) c * t.qcol + 8)[w] = words[qi];
+        }
+    }
+    else if (stage)
+    {
+        __syncthreads();
+    }
+}
+
+// Coalesced copy of the tile (now holding the new residual) to global memory; 16-byte stores where the
+// destination shares the tile's 16-byte phase (`mis` = floats by which the tile start is off a 16-byte boundary).
+__device__ __forceinline__ void tile_store(const float* tile, uint32_t mis, float* dst, uint32_t total)
+{
+    const uint32_t tid = threadIdx.x;
+    const uint32_t mis_d = (uint32_t) ((reinterpret_cast<uintptr_t>(dst) >> 2) & 3u);
+    if (mis_d == mis)
+    {
+        uint32_t head = (4u - mis) & 3u;
+        if (head > total)
+            head = total;
+        const uint32_t nvec = (total - head) >> 2;
+        const uint32_t tail0 = head + (nvec << 2);
+        if (tid < head)
+            dst[tid] = tile[tid];
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(tile + head);
+        f32x4* d4 = reinterpret_cast<f32x4*>(dst + head);
+        for (uint32_t e = tid; e < nvec; e += kTileThreads)
+            __builtin_nontemporal_store(t4[e], d4 + e);
+        for (uint32_t e = tail0 + tid; e < total; e += kTileThreads)
+            dst[e] = tile[e];
+    }
+    else
+    {
+        for (uint32_t e = tid; e < total; e += kTileThreads)
+            __builtin_nontemporal_store(tile[e], dst + e);
     }
 }
 
@@ -178,6 +248,7 @@ __global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float
     float* scratch_f = smem;
     uint32_t* scratch_u = reinterpret_cast<uint32_t*>(smem + 4);
     float* hdr = smem + kTileScratchFloats;
+    uint32_t* words = reinterpret_cast<uint32_t*>(smem + kTilePrefixFloats + t.tile_floats);
 
     const uint32_t tid = threadIdx.x;
     const uint32_t j0 = blockIdx.x * t.cols_per_tile;
@@ -186,6 +257,10 @@ __global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float
     const uint32_t total = nc * t.rows;
     const float* gp = g + base;
     const float* rp = r_in + base;
+
+    if constexpr (PackShape<NBITS>::CHUNKS > 1)
+        for (uint32_t x = tid; x < nc * t.nq; x += kTileThreads)
+            words[x] = 0u;
 
     // The tile starts `mis` floats into its LDS area so that LDS and global addresses share 16-byte phase.
     const uint32_t mis_g = (uint32_t) ((reinterpret_cast<uintptr_t>(gp) >> 2) & 3u);
@@ -231,13 +306,15 @@ __global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float
     else
     {
         for (uint32_t e = tid; e < total; e += kTileThreads)
-            tile[e] = gp[e] + rp[e];
+            tile[e] = __builtin_nontemporal_load(gp + e) + __builtin_nontemporal_load(rp + e);
     }
     __syncthreads();
 
     char* qtile = q + (size_t) j0 * t.qcol;
     tile_stats<NBITS, ZT>(tile, hdr, scratch_f, scratch_u, t, nc, qtile);
-    tile_pack<NBITS, ZT>(tile, hdr, t, nc, qtile, r_out + base);
+    tile_pack<NBITS, ZT>(tile, hdr, words, t, nc, qtile, r_out + base);
+    if (t.stage_residual)
+        tile_store(tile, mis_g, r_out + base, total);
 }
 
 // ---- stripe reduction: K packed stripes -> fp32 sum -> requantize with the stripe residual ----------
@@ -249,35 +326,49 @@ struct StripeSources
     uint32_t owner;
 };
 
+// Position n of the summation order: the owner first, then the other workers in ascending index.
+__device__ __forceinline__ uint32_t stripe_order(uint32_t n, uint32_t owner)
+{
+    return n == 0 ? owner : (n - 1 < owner ? n - 1 : n);
+}
+
 template <int NBITS, bool ZT>
 __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(StripeSources src, float* stripe_res,
                                                                           char* q_out, float* agg_out, TileGeom t)
 {
-    constexpr uint32_t VPW = 32 / NBITS;
-    constexpr uint32_t MASKBITS = NBITS & 31;
-    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << MASKBITS) - 1u);
+    using PS = PackShape<NBITS>;
+    constexpr uint32_t BATCH = 8; // packed words fetched together, so their latencies overlap
 
     extern __shared__ f32x4 smem_v4[];
     float* smem = reinterpret_cast<float*>(smem_v4);
     float* scratch_f = smem;
     uint32_t* scratch_u = reinterpret_cast<uint32_t*>(smem + 4);
     float* hdr = smem + kTileScratchFloats;
-    float* tile = smem + kTilePrefixFloats;
-    size_t tile_floats = ((size_t) t.cols_per_tile * t.rows + 4 + 3) & ~(size_t) 3;
-    float* dec = tile + tile_floats; // per (tile column, worker): two decode constants
+    uint32_t* words = reinterpret_cast<uint32_t*>(smem + kTilePrefixFloats + t.tile_floats);
+    float* dec = smem + kTilePrefixFloats + t.tile_floats + t.words_floats;
 
     const uint32_t tid = threadIdx.x;
     const uint32_t j0 = blockIdx.x * t.cols_per_tile;
     const uint32_t nc = min(t.cols_per_tile, t.cols - j0);
     const size_t base = (size_t) j0 * t.rows;
     const uint32_t K = src.workers;
+    const uint32_t nwords = nc * t.nq;
+    const uint32_t total = nc * t.rows;
+    float* sp = stripe_res + base;
+    const uint32_t mis_s = (uint32_t) ((reinterpret_cast<uintptr_t>(sp) >> 2) & 3u);
+    float* tile = smem + kTilePrefixFloats + mis_s;
 
-    // decode constants from every worker's column header: 1 bit -> the two levels, else (ufactor, lower)
+    if constexpr (PS::CHUNKS > 1)
+        for (uint32_t x = tid; x < nwords; x += kTileThreads)
+            words[x] = 0u;
+
+    // decode constants from every worker's column header, stored in summation order:
+    // 1 bit -> the two levels, else (ufactor, lower)
     for (uint32_t x = tid; x < nc * K; x += kTileThreads)
     {
         const uint32_t c = x / K;
-        const uint32_t wk = x - c * K;
-        const float* h = reinterpret_cast<const float*>(src.q[wk] + (size_t) (j0 + c) * t.qcol);
+        const uint32_t n = x - c * K;
+        const float* h = reinterpret_cast<const float*>(src.q[stripe_order(n, src.owner)] + (size_t) (j0 + c) * t.qcol);
         const ValueQ vq = make_vq<NBITS>(h[0], h[1]);
         if constexpr (NBITS == 1)
         {
@@ -292,59 +383,58 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
     }
     __syncthreads();
 
-    const float* sp = stripe_res + base;
-    const uint32_t nwords = nc * t.nq;
-    for (uint32_t qi = tid; qi < nwords; qi += kTileThreads)
+    const uint32_t items = nwords * PS::CHUNKS;
+    for (uint32_t it = tid; it < items; it += kTileThreads)
     {
+        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
+        const uint32_t qi = it - chunk * nwords;
         const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
         const uint32_t w = qi - c * t.nq;
         const size_t word_off = (size_t) (j0 + c) * t.qcol + 8 + (size_t) w * 4;
-        float acc[VPW];
+        const uint32_t sh0 = chunk * PS::SLOTS * PS::SHIFT;
+        const float* d = dec + 2 * (size_t) c * K;
+        float acc[PS::SLOTS];
+        for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
         {
-            // the owner's own stripe seeds the sum
-            const uint32_t word = *reinterpret_cast<const uint32_t*>(src.q[src.owner] + word_off);
-            const float a = dec[2 * (c * K + src.owner)];
-            const float b = dec[2 * (c * K + src.owner) + 1];
+            uint32_t word[BATCH];
 #pragma unroll
-            for (uint32_t k = 0; k < VPW; ++k)
-            {
-                const uint32_t code = (word >> (k * MASKBITS)) & CODEMASK;
-                if constexpr (NBITS == 1)
-                    acc[k] = code ? b : a;
-                else
-                    acc[k] = unquantize_value<NBITS>(a, b, code);
-            }
-        }
-        for (uint32_t wk = 0; wk < K; ++wk)
-        {
-            if (wk == src.owner)
-                continue;
-            const uint32_t word = *reinterpret_cast<const uint32_t*>(src.q[wk] + word_off);
-            const float a = dec[2 * (c * K + wk)];
-            const float b = dec[2 * (c * K + wk) + 1];
+            for (uint32_t u = 0; u < BATCH; ++u)
+                if (n0 + u < K)
+                    word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + word_off);
 #pragma unroll
-            for (uint32_t k = 0; k < VPW; ++k)
+            for (uint32_t u = 0; u < BATCH; ++u)
             {
-                const uint32_t code = (word >> (k * MASKBITS)) & CODEMASK;
-                float x;
-                if constexpr (NBITS == 1)
-                    x = code ? b : a;
-                else
-                    x = unquantize_value<NBITS>(a, b, code);
-                acc[k] = x + acc[k];
+                if (n0 + u < K)
+                {
+                    const float a = d[2 * (n0 + u)];
+                    const float b = d[2 * (n0 + u) + 1];
+                    const uint32_t bits = word[u] >> sh0;
+#pragma unroll
+                    for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+                    {
+                        const uint32_t code = (bits >> (kk * PS::SHIFT)) & PS::CODEMASK;
+                        float x;
+                        if constexpr (NBITS == 1)
+                            x = code ? b : a;
+                        else
+                            x = unquantize_value<NBITS>(a, b, code);
+                        // the first term seeds the sum; afterwards: decoded value + running sum
+                        acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
+                    }
+                }
             }
         }
         float* colv = tile + (size_t) c * t.rows;
         const float* sc = sp + (size_t) c * t.rows;
 #pragma unroll
-        for (uint32_t k = 0; k < VPW; ++k)
+        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
         {
-            const uint32_t i = w + k * t.nq;
+            const uint32_t i = w + (chunk * PS::SLOTS + kk) * t.nq;
             if (i < t.rows)
             {
                 if (agg_out != nullptr)
-                    agg_out[base + (size_t) c * t.rows + i] = acc[k];
-                colv[i] = acc[k] + sc[i];
+                    agg_out[base + (size_t) c * t.rows + i] = acc[kk];
+                colv[i] = acc[kk] + __builtin_nontemporal_load(sc + i);
             }
         }
     }
@@ -352,7 +442,9 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
 
     char* qtile = q_out + (size_t) j0 * t.qcol;
     tile_stats<NBITS, ZT>(tile, hdr, scratch_f, scratch_u, t, nc, qtile);
-    tile_pack<NBITS, ZT>(tile, hdr, t, nc, qtile, stripe_res + base);
+    tile_pack<NBITS, ZT>(tile, hdr, words, t, nc, qtile, sp);
+    if (t.stage_residual)
+        tile_store(tile, mis_s, sp, total);
 }
 
 // ---- quantize, 1 bit, one wavefront per column, column share in registers ---------------------------
@@ -360,15 +452,17 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
 // rows = 2048 * WPL, nq = 64 * WPL. Lane l owns QWords l, l + 64, ...; QWord w packs rows w + k * nq, so for
 // fixed k the 64 lanes read 64 consecutive floats, and each lane builds its QWords with shifts alone.
 
+constexpr uint32_t kWaveColThreads = 128;
+
 template <bool ZT, int WPL>
-__global__ __launch_bounds__(kTileThreads) void quantize_wavecol_kernel(const float* __restrict__ g, const float* r_in,
+__global__ __launch_bounds__(kWaveColThreads) void quantize_wavecol_kernel(const float* __restrict__ g, const float* r_in,
                                                                         float* r_out, char* __restrict__ q,
                                                                         uint32_t cols, uint64_t qcol)
 {
     constexpr uint32_t NQ = 64 * WPL;
     constexpr uint32_t ROWS = 32 * NQ;
     const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t j = blockIdx.x * (kTileThreads / 64) + (threadIdx.x >> 6);
+    const uint32_t j = blockIdx.x * (kWaveColThreads / 64) + (threadIdx.x >> 6);
     if (j >= cols)
         return; // whole wavefront leaves; no barriers below
     const size_t base = (size_t) j * ROWS;

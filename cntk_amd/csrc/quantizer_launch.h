@@ -19,12 +19,13 @@ enum QuantizePath
     kPathWaveCol = 3  // 1 bit, rows in {2048, 4096}, one wavefront per column in registers
 };
 
-constexpr uint32_t kTileMaxRows = 15360; // 60 KB of LDS for a one-column tile
+constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
 
 struct LaunchTuning
 {
     int quantize_path = kPathAuto;
     uint32_t tile_gs = 0;   // 0 = pick from rows; else threads per column (power of two, 8..256)
+    int tile_stage = -1;    // -1 = automatic; 0 / 1 = residual written straight to memory / staged through LDS
     uint32_t unq_slots = 0; // 0 = default; else bit positions per thread in unquantize
     int unq_force_scalar = 0;
 };
@@ -45,7 +46,7 @@ inline size_t qcol_bytes(size_t nbits, size_t rows)
     return 8 + ((rows * nbits + 31) / 32) * 4;
 }
 
-inline TileGeom make_tile_geom(size_t rows, size_t cols, size_t nbits, uint32_t gs_override)
+inline TileGeom make_tile_geom(size_t rows, size_t cols, size_t nbits, uint32_t gs_override, int stage = -1)
 {
     TileGeom t;
     t.rows = (uint32_t) rows;
@@ -57,14 +58,18 @@ inline TileGeom make_tile_geom(size_t rows, size_t cols, size_t nbits, uint32_t 
     else
         while (gs < kTileThreads && rows > (size_t) gs * 32)
             gs <<= 1;
-    // a tile may not exceed 8192 floats unless it is a single column
-    while (gs < kTileThreads && (size_t) (kTileThreads / gs) * rows > 8192)
+    // a tile may not exceed 4096 floats (16 KB) unless it is a single column: small tiles keep many
+    // workgroups resident per CU, which is what hides the barrier-separated phases of each of them
+    while (gs < kTileThreads && (size_t) (kTileThreads / gs) * rows > 4096)
         gs <<= 1;
     t.gs = gs;
     t.gs_log2 = 0;
     while ((1u << t.gs_log2) < gs)
         t.gs_log2++;
     t.cols_per_tile = kTileThreads / gs;
+    t.tile_floats = (uint32_t) (((size_t) t.cols_per_tile * rows + 4 + 3) & ~(size_t) 3);
+    t.words_floats = (nbits <= 2) ? t.cols_per_tile * t.nq : 0;
+    t.stage_residual = (stage < 0) ? 1u : (uint32_t) (stage != 0);
     t.qcol = qcol_bytes(nbits, rows);
     return t;
 }
@@ -140,6 +145,8 @@ inline hipError_t launch_quantize(hipStream_t s, const float* g, const float* r_
     {
         if (rows > kTileMaxRows)
             path = kPathTall;
+        else if (wavecol_applicable(g, r_in, r_out, q, rows, nbits))
+            path = kPathWaveCol;
         else
             path = kPathTile;
     }
@@ -147,21 +154,22 @@ inline hipError_t launch_quantize(hipStream_t s, const float* g, const float* r_
     {
         if (!wavecol_applicable(g, r_in, r_out, q, rows, nbits))
             return hipErrorInvalidValue;
-        const uint32_t blocks = (uint32_t) ((cols + 3) / 4);
+        constexpr uint32_t per_block = kWaveColThreads / 64;
+        const uint32_t blocks = (uint32_t) ((cols + per_block - 1) / per_block);
         const uint64_t qcol = qcol_bytes(nbits, rows);
         if (rows == 2048)
         {
             if (zt)
-                hipLaunchKernelGGL((quantize_wavecol_kernel<true, 1>), dim3(blocks), dim3(kTileThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+                hipLaunchKernelGGL((quantize_wavecol_kernel<true, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
             else
-                hipLaunchKernelGGL((quantize_wavecol_kernel<false, 1>), dim3(blocks), dim3(kTileThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+                hipLaunchKernelGGL((quantize_wavecol_kernel<false, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
         }
         else
         {
             if (zt)
-                hipLaunchKernelGGL((quantize_wavecol_kernel<true, 2>), dim3(blocks), dim3(kTileThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+                hipLaunchKernelGGL((quantize_wavecol_kernel<true, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
             else
-                hipLaunchKernelGGL((quantize_wavecol_kernel<false, 2>), dim3(blocks), dim3(kTileThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+                hipLaunchKernelGGL((quantize_wavecol_kernel<false, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
         }
         return hipGetLastError();
     }
@@ -169,7 +177,7 @@ inline hipError_t launch_quantize(hipStream_t s, const float* g, const float* r_
     {
         if (rows > kTileMaxRows)
             return hipErrorInvalidValue;
-        const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs);
+        const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs, tune.tile_stage);
         return dispatch_nbits<TileLauncher>(nbits, zt, s, g, r_in, r_out, qc, t);
     }
     return dispatch_nbits<TallLauncher>(nbits, zt, s, g, r_in, r_out, qc, (uint32_t) rows, (uint32_t) cols,
@@ -183,7 +191,18 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, const StripeSources& src, 
     zt = zt && (nbits == 1);
     if (rows > kTileMaxRows)
         return hipErrorInvalidValue;
-    const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs);
+    // A stripe is small (one GPU's share of the columns), so the kernel is latency-bound: take the smallest
+    // tile that still gives every thread of a workgroup a work item, to spread the stripe over all CUs.
+    uint32_t gs = tune.tile_gs;
+    if (gs == 0)
+    {
+        const size_t chunks = nbits == 1 ? 4 : (nbits == 2 ? 2 : 1);
+        const size_t items_per_col = qwords_per_col(rows, nbits) * chunks;
+        gs = kTileThreads;
+        while (gs > 8 && items_per_col * (kTileThreads / gs) < kTileThreads)
+            gs >>= 1;
+    }
+    const TileGeom t = make_tile_geom(rows, cols, nbits, gs, tune.tile_stage);
     return dispatch_nbits<StripeLauncher>(nbits, zt, s, src, stripe_res, static_cast<char*>(q_out), agg_out, t);
 }
 
@@ -198,7 +217,7 @@ inline hipError_t launch_unquantize_t(hipStream_t s, const char* q, float* out, 
     t.nq = (uint32_t) qwords_per_col(rows, NBITS);
     t.groups = (t.nq + WV - 1) / WV;
     if (slots == 0)
-        slots = VPW < 8 ? VPW : 8;
+        slots = VPW < 2 ? VPW : 2;
     if (slots > VPW)
         slots = VPW;
     t.slots = slots;

@@ -6,6 +6,12 @@ Two layers:
   tolerance -- the GPU headers against the sequential-sum oracle headers: lower/upper within 1e-5 of the column
                scale (upper - lower); a code may differ only for an element within 1e-6 * scale of a decision
                threshold (their number is reported); residuals of all other elements within 1e-5 * scale.
+
+A decision threshold lies between lower and upper, so it can move by as much as the header moved. Where the header
+of a column deviates by more than 1e-6 of its scale (long columns: the oracle's own sequential fp32 sum is that
+inexact; fine code grids: 16 bits), a differing code is accepted within 1.5 x that column's observed header
+deviation instead, and counted separately as "beyond 1e-6"; callers that must hold the 1e-6 rule literally pass
+strict=True, which makes any such element a failure.
 """
 import numpy as np
 
@@ -26,25 +32,34 @@ class Report:
     def __init__(self):
         self.elements = 0
         self.near_threshold_mismatches = 0
+        self.beyond_1e6 = 0
+        self.last_mismatch_cols = None  # per column of the last check: did any code differ from the oracle's
         self.max_bound_err = 0.0
         self.max_residual_err = 0.0
 
     def __repr__(self):
-        return ("elements=%d near-threshold code mismatches=%d max bound err=%.3g max residual err=%.3g (relative to column scale)"
-                % (self.elements, self.near_threshold_mismatches, self.max_bound_err, self.max_residual_err))
+        return ("elements=%d near-threshold code mismatches=%d (of which beyond 1e-6 of scale: %d) max bound err=%.3g "
+                "max residual err=%.3g (relative to column scale)"
+                % (self.elements, self.near_threshold_mismatches, self.beyond_1e6, self.max_bound_err,
+                   self.max_residual_err))
 
 
-def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, report=None):
-    """g, r_in: inputs (F-order float32); q_gpu: packed bytes from the GPU; r_gpu: residual from the GPU."""
+def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, report=None, strict=False, exact=True,
+                   skip_cols=None):
+    """g, r_in: inputs (F-order float32); q_gpu: packed bytes from the GPU; r_gpu: residual from the GPU.
+    exact=False skips the bit-exact layer (for inputs that are themselves only equal within tolerance);
+    skip_cols (bool per column) leaves columns out of the tolerance layer."""
     rows, cols = g.shape
     zt = bool(zero_threshold) and nbits == 1
     rep = report if report is not None else Report()
     rep.elements += rows * cols
+    keep = np.ones(cols, dtype=bool) if skip_cols is None else ~np.asarray(skip_cols, dtype=bool)
 
     # ---- exact layer
-    q_ex, r_ex = oracle.pack_with_headers(g, r_in, q_gpu, nbits, zt, threads=threads)
-    assert np.array_equal(q_ex, q_gpu), "codes differ from the oracle's under the GPU's own headers"
-    assert bits_equal(r_ex, r_gpu), "residual differs from the oracle's under the GPU's own headers"
+    if exact:
+        q_ex, r_ex = oracle.pack_with_headers(g, r_in, q_gpu, nbits, zt, threads=threads)
+        assert np.array_equal(q_ex, q_gpu), "codes differ from the oracle's under the GPU's own headers"
+        assert bits_equal(r_ex, r_gpu), "residual differs from the oracle's under the GPU's own headers"
 
     # ---- tolerance layer
     q_or, r_or = oracle.quantize(g, r_in, nbits, zt, threads=threads)
@@ -53,11 +68,13 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
     scale = (hi_o.astype(np.float64) - lo_o.astype(np.float64))
     tiny = np.finfo(np.float32).tiny
     denom = np.maximum(np.abs(scale), tiny)
-    err = np.maximum(np.abs(lo_g.astype(np.float64) - lo_o), np.abs(hi_g.astype(np.float64) - hi_o)) / denom
+    abs_dev = np.maximum(np.abs(lo_g.astype(np.float64) - lo_o), np.abs(hi_g.astype(np.float64) - hi_o))
+    err = abs_dev / denom
     # columns without any spread (all-zero) must agree exactly
-    flat = scale == 0
+    flat = (scale == 0) & keep
     assert np.array_equal(lo_g[flat], lo_o[flat]) and np.array_equal(hi_g[flat], hi_o[flat])
     err[flat] = 0.0
+    err[~keep] = 0.0
     rep.max_bound_err = max(rep.max_bound_err, float(err.max(initial=0.0)))
     assert err.max(initial=0.0) <= BOUND_RTOL, "column bounds off by %.3g of the column scale" % err.max()
 
@@ -65,12 +82,14 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
         assert np.array_equal(q_or[:], q_gpu[:]) or np.array_equal(oracle.words(q_or, rows, cols, 32),
                                                                    oracle.words(q_gpu, rows, cols, 32))
         assert bits_equal(r_or, r_gpu)
+        rep.last_mismatch_cols = np.zeros(cols, dtype=bool)
         return rep
 
     c_g = oracle.codes(q_gpu, rows, cols, nbits)
     c_o = oracle.codes(q_or, rows, cols, nbits)
-    diff = c_g != c_o
+    diff = (c_g != c_o) & keep[None, :]
     ndiff = int(diff.sum())
+    rep.last_mismatch_cols = diff.any(axis=0)
     if ndiff:
         v = (g + r_in).astype(np.float64)  # one rounded fp32 add, then widened
         ii, jj = np.nonzero(diff)
@@ -87,11 +106,16 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
             dist = np.minimum(dist, np.minimum(np.abs(vv - lo), np.abs(vv - hi_o[jj].astype(np.float64))))
             assert np.all(np.abs(c_g[ii, jj].astype(np.int64) - c_o[ii, jj].astype(np.int64)) == 1), \
                 "codes differ by more than one level"
-        assert np.all(dist <= THRESH_RTOL * sc), \
+        far = dist > THRESH_RTOL * sc
+        allowed = np.maximum(THRESH_RTOL * sc, 1.5 * abs_dev[jj] + 1e-7 * sc)
+        if strict:
+            allowed = THRESH_RTOL * sc
+        assert np.all(dist <= allowed), \
             "%d codes differ away from a threshold (worst %.3g of scale)" % (ndiff, float((dist / sc).max()))
         rep.near_threshold_mismatches += ndiff
+        rep.beyond_1e6 += int(far.sum())
 
-    same = ~diff
+    same = ~diff & keep[None, :]
     rerr = np.abs(r_gpu.astype(np.float64) - r_or) / denom[None, :]
     rerr = np.where(same, rerr, 0.0)
     rep.max_residual_err = max(rep.max_residual_err, float(rerr.max(initial=0.0)))
@@ -112,3 +136,52 @@ def conservation(g, r_in, prev_out, r_out, out, tol):
     lhs = g.astype(np.float64) + r_in + prev_out
     rhs = r_out.astype(np.float64) + out
     assert np.abs(lhs - rhs).max(initial=0.0) <= tol
+
+
+def oracle_allreduce_staged(gs, res, sres, nbits, zt, threads=8):
+    """The oracle's all-reduce, stage by stage, keeping the intermediates. Updates res[w], sres[s] in place.
+    Returns (packed matrices after stage 1, fp32 aggregates per stripe, assembled packed aggregate, output)."""
+    k = len(gs)
+    rows, cols = gs[0].shape
+    qcol = oracle.qcol_bytes(nbits, rows)
+    q1 = [oracle.quantize(gs[w], res[w], nbits, zt, r_out=res[w], threads=threads)[0] for w in range(k)]
+    qagg = np.zeros_like(q1[0])
+    aggs = []
+    for s in range(k):
+        start, n = oracle.stripe_range(cols, s, k)
+        if n == 0:
+            aggs.append(np.zeros((rows, 0), np.float32, order="F"))
+            continue
+        qc = [q.copy() for q in q1]
+        aggs.append(oracle.stripe_reduce(qc, s, rows, cols, nbits, sres[s], zt, threads=threads))
+        qagg[start * qcol:(start + n) * qcol] = qc[s][start * qcol:(start + n) * qcol]
+    out = oracle.unquantize(qagg, rows, cols, nbits, threads=threads)
+    return q1, aggs, qagg, out
+
+
+def check_end_to_end(aggs_or, sres_in, qagg_gpu, sres_gpu, out_gpu, qagg_or, out_or, rows, cols, nbits, zt, tainted_cols,
+                     threads=8, report=None):
+    """Whole all-reduce against the free-standing oracle run (oracle_allreduce_staged). A first-stage code that flips
+    at its threshold moves that element's aggregate by a whole reconstruction level, hence the second-stage header
+    of that column by about level / rows; such columns (tainted_cols) are left out and counted. Everywhere else the
+    second stage must agree with the oracle's under the usual tolerance rules (its inputs, the aggregates, are
+    themselves equal only within the first-stage header tolerance), and the aggregated gradient must be within 1e-5
+    of the column scale wherever the final codes agree."""
+    k = len(aggs_or)
+    qcol = oracle.qcol_bytes(nbits, rows)
+    rep = report if report is not None else Report()
+    for s in range(k):
+        start, n = oracle.stripe_range(cols, s, k)
+        if n == 0:
+            continue
+        check_quantize(aggs_or[s], sres_in[s], qagg_gpu[start * qcol:(start + n) * qcol], sres_gpu[s], nbits, zt,
+                       threads=threads, report=rep, exact=False, skip_cols=tainted_cols[start:start + n])
+    clean = ~tainted_cols
+    lo, hi = oracle.headers(qagg_or, rows, cols, nbits)
+    scale = np.maximum(np.abs(hi.astype(np.float64) - lo), np.finfo(np.float32).tiny)
+    # elements whose final code differs sit a whole level apart; the check above has vetted each of them
+    same = oracle.codes(qagg_gpu, rows, cols, nbits) == oracle.codes(qagg_or, rows, cols, nbits)
+    err = np.where(same, np.abs(out_gpu.astype(np.float64) - out_or) / scale[None, :], 0.0)
+    worst = float(err[:, clean].max(initial=0.0))
+    assert worst <= VALUE_RTOL, "aggregated gradient off by %.3g of the column scale" % worst
+    return worst, int(tainted_cols.sum())

@@ -117,7 +117,7 @@ PATH_CASES = [
     (1, 1, PATH_TILE, 0), (3, 70, PATH_TILE, 0), (31, 5, PATH_TILE, 8), (33, 67, PATH_TILE, 0), (64, 64, PATH_TILE, 16),
     (147, 64, PATH_TILE, 0), (429, 37, PATH_TILE, 0), (429, 37, PATH_TILE, 64), (576, 64, PATH_TILE, 0),
     (1023, 9, PATH_TILE, 0), (1024, 33, PATH_TILE, 0), (2048, 19, PATH_TILE, 0), (2048, 19, PATH_TILE, 256),
-    (2304, 5, PATH_TILE, 0), (4608, 3, PATH_TILE, 0), (9304, 2, PATH_TILE, 0), (15360, 1, PATH_TILE, 0),
+    (2304, 5, PATH_TILE, 0), (4608, 3, PATH_TILE, 0), (9304, 2, PATH_TILE, 0), (14336, 1, PATH_TILE, 0),
     (1, 5, PATH_TALL, 0), (70, 3, PATH_TALL, 0), (1025, 3, PATH_TALL, 0), (20001, 2, PATH_TALL, 0),
     (33000, 2, PATH_AUTO, 0),
 ]
@@ -127,10 +127,11 @@ PATH_CASES = [
 def test_kernel_paths(case):
     rows, cols, path, gs = case
     qz = MatrixQuantizerImpl.Create(0, False)
-    qz._set_tuning(quantize_path=path, tile_gs=gs)
     rep = parity.Report()
     for nbits, zt in VARIANTS:
         say("path case", case, "nbits", nbits, "zeroThr", zt)
+        # alternate between the two ways a tile kernel writes its residual
+        qz._set_tuning(quantize_path=path, tile_gs=gs, tile_stage=(nbits + rows) % 2 if path == PATH_TILE else -1)
         # a shifted mean, one all-zero column and outliers exercise every branch of the statistics
         def make(it):
             a = datagen.normal_with_outliers(1000 * rows + cols + it, rows, cols, 0.01) + np.float32(0.004 * (it % 2))
@@ -247,6 +248,9 @@ def test_error_behaviour(quantizer):
         quantizer.UnquantizeAsync(QuantizedMatrix(8, 4, 1, 0), Matrix(8, 5))
     with pytest.raises(cntk_amd.QuantizerLogicError):
         quantizer.UnquantizeAsync(QuantizedMatrix(8, 4, 2, 0), Matrix(16, 4))
+    with pytest.raises(cntk_amd.QuantizerLogicError):  # same dimensions, packed buffer of another bit width
+        cntk_amd._check(cntk_amd.lib().cntkq_unquantize_async(quantizer._h, QuantizedMatrix(8, 4, 2, 0).Buffer(), 48, 0,
+                                                              Matrix(8, 4).Data(), 8, 4, 8, 0))
     # empty matrices are silent no-ops
     quantizer.QuantizeAsync(Matrix(0, 4), Matrix(0, 4), QuantizedMatrix(0, 4, 1, 0), Matrix(0, 4), False)
     quantizer.UnquantizeAsync(QuantizedMatrix(5, 0, 1, 0), Matrix(5, 0))

@@ -164,11 +164,13 @@ def test_simulated_allreduce(shape, use_async):
         res_in = [r.copy(order="F") for r in res_o]
         sres_in = [s.copy(order="F") for s in sres_o]
         res_g, sres_g, q1_g, qagg_g, out_g = simulated_allreduce_gpu(gs, res_in, sres_in, nbits, zt, use_async)
-        qs_o, qagg_o, out_o = oracle.allreduce(gs, res_o, sres_o, nbits, zt, threads=8)
+        _, aggs_o, qagg_o, out_o = parity.oracle_allreduce_staged(gs, res_o, sres_o, nbits, zt, threads=8)
 
         # stage 1: every worker's own quantization
+        tainted = np.zeros(cols, dtype=bool)
         for w in range(k):
             parity.check_quantize(gs[w], res_in[w], q1_g[w], res_g[w], nbits, zt, report=rep)
+            tainted |= rep.last_mismatch_cols
         # stage 2: each owner's stripe reduction, given the GPU's stage-1 buffers
         for s in range(k):
             start, n = oracle.stripe_range(cols, s, k)
@@ -179,20 +181,14 @@ def test_simulated_allreduce(shape, use_async):
             agg = oracle.stripe_reduce(q_copy, s, rows, cols, nbits, s_copy, zt, threads=8)
             parity.check_quantize(agg, sres_in[s], qagg_g[start * qcol:(start + n) * qcol], sres_g[s], nbits, zt,
                                   report=rep)
+            tainted[start:start + n] |= rep.last_mismatch_cols
         # stage 3: unquantize is exact given the packed buffer
         parity.check_unquantize(qagg_g, rows, cols, nbits, out_g)
-
-        # end to end against the free-standing oracle: aggregated gradient within 1e-5 of the column scale
-        # wherever the packed codes agree (a first-stage code that flips at its threshold moves that element's
-        # aggregate by a whole level, which may in turn move second-stage codes)
-        lo, hi = oracle.headers(qagg_o, rows, cols, nbits)
-        scale = np.maximum(np.abs(hi.astype(np.float64) - lo), np.finfo(np.float32).tiny)
-        same = oracle.codes(qagg_g, rows, cols, nbits) == oracle.codes(qagg_o, rows, cols, nbits)
-        err = np.where(same, np.abs(out_g.astype(np.float64) - out_o) / scale[None, :], 0.0)
-        say("   aggregated gradient: max err %.3g of column scale, %d of %d codes differ"
-            % (err.max(), int((~same).sum()), same.size))
-        assert err.max() <= parity.VALUE_RTOL
-        assert int((~same).sum()) <= max(2, int(1e-3 * same.size))
+        worst, ntaint = parity.check_end_to_end(aggs_o, sres_in, qagg_g, sres_g, out_g, qagg_o, out_o, rows, cols, nbits, zt,
+                                                tainted, report=rep)
+        say("   aggregated gradient: max err %.3g of column scale; %d of %d columns hold a near-threshold flip"
+            % (worst, ntaint, cols))
+        assert ntaint <= max(1, cols // 100)
     say("  ", rep)
 
 
