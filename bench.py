@@ -84,6 +84,13 @@ def main():
     ap.add_argument("--zero-threshold", type=int, default=0, help="zeroThresholdFor1Bit (default off, as in config 1)")
     ap.add_argument("--sets", type=int, default=6, help="rotating buffer sets (each 231 MB)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-events", action="store_true", help="no per-kernel HIP events in the timed region")
+    ap.add_argument("--event-every", type=int, default=8,
+                    help="attach timing events to the kernels of every n-th step (creating a profiled dispatch costs "
+                         "the host ~25 us, so doing it on every step would leave the GPU waiting for the host)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="instead of the benchmark, run plain device copies of one 2048x9304 fp32 matrix "
+                         "(76,218,368 bytes read and as many written per copy), for scaling hardware counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU only (K workers are simulated in one GPU's memory); "
@@ -96,6 +103,16 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     dev = "cuda:0"
+    if args.copy_calibration:
+        src = [torch.randn(ROWS * COLS, device=dev, dtype=torch.float32) for _ in range(args.sets)]
+        dst = [torch.empty(ROWS * COLS, device=dev, dtype=torch.float32) for _ in range(args.sets)]
+        torch.cuda.synchronize()
+        for i in range(args.steps):
+            dst[i % args.sets].copy_(src[i % args.sets])
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": True, "copies": args.steps, "bytes_read_per_copy": ROWS * COLS * 4,
+                          "bytes_written_per_copy": ROWS * COLS * 4}), flush=True)
+        return
     zt = bool(args.zero_threshold)
     qz = MatrixQuantizerImpl.Create(0, False)  # issues on the main (null) stream = torch's current stream
 
@@ -107,33 +124,73 @@ def main():
         sets.append((G, Matrix(ROWS, COLS), QuantizedMatrix(ROWS, COLS, NBITS, 0), Matrix(ROWS, COLS)))
     torch.cuda.synchronize()
 
+    # The timed loop calls the C ABI directly with pre-computed pointers: two calls per step, so that the host
+    # stays well ahead of the GPU and the measured time is the GPU's.
+    L, h = cntk_amd.lib(), qz._h
+    qbytes = sets[0][2].GetSize()
+    ptrs = [(G.Data(), R.Data(), Q.Buffer(), Out.Data()) for G, R, Q, Out in sets]
+    izt = int(zt)
+
+    # HIP events with timing, tied to the kernel dispatches themselves (start when the kernel begins, stop when it
+    # has finished) on the stream the handle launches on: separate event records would idle the GPU for several
+    # microseconds per kernel and show up in the very time they measure.
+    import ctypes
+
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+    hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+
+    def new_event():
+        e = ctypes.c_void_p()
+        if hip.hipEventCreate(ctypes.byref(e)) != 0:
+            raise RuntimeError("hipEventCreate failed")
+        return e
+
+    def elapsed_ms(a, b):
+        ms = ctypes.c_float()
+        if hip.hipEventElapsedTime(ctypes.byref(ms), a, b) != 0:
+            raise RuntimeError("hipEventElapsedTime failed")
+        return ms.value
+
+    L.cntkq_debug_attach_events.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+
     def step(i, ev=None):
-        G, R, Q, Out = sets[i % len(sets)]
+        g, r, q, o = ptrs[i % len(ptrs)]
         if ev is not None:
-            ev[0].record()
-        qz.QuantizeAsync(G, R, Q, R, zt)
+            L.cntkq_debug_attach_events(h, ev[0], ev[1])
+        rc1 = L.cntkq_quantize_async(h, g, r, ROWS, COLS, q, qbytes, 0, NBITS, r, izt)
         if ev is not None:
-            ev[1].record()
-        qz.UnquantizeAsync(Q, Out, False)
-        if ev is not None:
-            ev[2].record()
+            L.cntkq_debug_attach_events(h, ev[2], ev[3])
+        rc2 = L.cntkq_unquantize_async(h, q, qbytes, 0, o, ROWS, COLS, NBITS, 0)
+        if rc1 or rc2:
+            raise RuntimeError(L.cntkq_last_error().decode())
 
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
 
     # timed region: exactly `steps` steps, host clock around a synchronize on both sides
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    events = {}
+    if not args.no_events:
+        events = {i: [new_event() for _ in range(4)] for i in range(0, args.steps, max(1, args.event_every))}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(args.warmup + i, events[i])
+        step(args.warmup + i, events.get(i))
+    t_enqueued = time.perf_counter()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
 
     sec_per_step = (t1 - t0) / args.steps
-    q_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
-    u_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+    if args.no_events:
+        q_ms = u_ms = float("nan")
+    else:
+        q_ms = sum(elapsed_ms(e[0], e[1]) for e in events.values()) / len(events)
+        u_ms = sum(elapsed_ms(e[2], e[3]) for e in events.values()) / len(events)
+        for e in events.values():
+            for x in e:
+                hip.hipEventDestroy(x)
     qb, ub = algorithmic_bytes(ROWS, COLS, NBITS)
     total = qb + ub
     achieved = qb / (q_ms * 1e-3) / 1e9
@@ -159,7 +216,8 @@ def main():
         },
         "pct_hbm_peak": round(100.0 * total / sec_per_step / 1e9 / HBM_PEAK_GBS, 2),
         "elements_per_s": round(ROWS * COLS / sec_per_step, 1),
-        "kernel_ms": {"quantize": round(q_ms, 5), "unquantize": round(u_ms, 5)},
+        "kernel_ms": {"quantize": round(q_ms, 5), "unquantize": round(u_ms, 5), "launches_timed": len(events)},
+        "host_enqueue_ms_per_step": round((t_enqueued - t0) / args.steps * 1e3, 5),
         "roofline": {
             "bound": "hbm",
             "kernel": "quantize (gradient + residual -> codes + residual)",

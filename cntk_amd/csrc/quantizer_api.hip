@@ -87,6 +87,12 @@ struct cntkq_quantizer
     hipEvent_t ev_unquantize = nullptr;
     hipEvent_t ev_stripe = nullptr;
     hipEvent_t ev_main = nullptr;
+    // the event each Wait call waits on: the handle's own, or one attached through the debug hook
+    hipEvent_t last_quantize = nullptr;
+    hipEvent_t last_unquantize = nullptr;
+    hipEvent_t last_stripe = nullptr;
+    hipEvent_t attach_start = nullptr; // one-shot: tied to the next kernel this handle launches
+    hipEvent_t attach_stop = nullptr;
     bool quantize_included_fetch = false;
     bool fetch_pending = false;   // a device-to-host copy out of the staging buffer may still be running
     bool staging_read_pending = false; // a kernel reading the staging buffer may still be running
@@ -100,6 +106,17 @@ namespace {
 hipStream_t work_stream(const cntkq_quantizer* h)
 {
     return h->dedicated ? h->compute : h->main_stream;
+}
+
+// Completion is signalled by the kernel dispatch itself (no separate event record in the stream).
+LaunchEvents take_events(cntkq_quantizer* h, hipEvent_t own)
+{
+    LaunchEvents ev;
+    ev.start = h->attach_start;
+    ev.stop = h->attach_stop != nullptr ? h->attach_stop : own;
+    h->attach_start = nullptr;
+    h->attach_stop = nullptr;
+    return ev;
 }
 
 // Temp device buffer for a host-resident packed matrix (GetTempGPUQuantizedMatrix,
@@ -319,15 +336,16 @@ int cntkq_quantize_async(cntkq_quantizer* h, const float* in, const float* res_i
         qdev = h->staging;
     }
 
-    hipError_t lrc = launch_quantize(s, in, res_in, res_out, qdev, rows, cols, nbits, zero_threshold_for_1bit != 0, h->tune);
+    const LaunchEvents ev = take_events(h, h->ev_quantize);
+    hipError_t lrc = launch_quantize(s, ev, in, res_in, res_out, qdev, rows, cols, nbits, zero_threshold_for_1bit != 0, h->tune);
     if (lrc == hipErrorInvalidValue)
         return fail(CNTKQ_INVALID_ARGUMENT, "quantize: the forced kernel path does not support %zu x %zu at %zu bits", rows, cols, nbits);
     HIP_TRY(lrc, "quantize kernel launch failed");
-    HIP_TRY(hipEventRecord(h->ev_quantize, s), "hipEventRecord failed");
+    h->last_quantize = ev.stop;
 
     if (qbuf_on_host)
     {
-        HIP_TRY(hipStreamWaitEvent(h->fetch, h->ev_quantize, 0), "hipStreamWaitEvent failed");
+        HIP_TRY(hipStreamWaitEvent(h->fetch, ev.stop, 0), "hipStreamWaitEvent failed");
         HIP_TRY(hipMemcpyAsync(qbuf, qdev, need, hipMemcpyDeviceToHost, h->fetch), "hipMemcpyAsync failed");
         HIP_TRY(hipEventRecord(h->ev_fetch, h->fetch), "hipEventRecord failed");
         h->quantize_included_fetch = true;
@@ -348,7 +366,7 @@ int cntkq_wait_quantize_done(cntkq_quantizer* h)
             h->fetch_pending = false;
         return rc;
     }
-    return sync_event(h->ev_quantize);
+    return h->last_quantize != nullptr ? sync_event(h->last_quantize) : CNTKQ_OK;
 }
 
 int cntkq_unquantize_async(cntkq_quantizer* h, const void* qbuf, size_t qbuf_bytes, int qbuf_on_host, float* out,
@@ -390,8 +408,9 @@ int cntkq_unquantize_async(cntkq_quantizer* h, const void* qbuf, size_t qbuf_byt
         HIP_TRY(hipStreamWaitEvent(s, h->ev_assign, 0), "hipStreamWaitEvent failed");
         qdev = h->staging;
     }
-    HIP_TRY(launch_unquantize(s, qdev, out, rows, cols, nbits, add != 0, h->tune), "unquantize kernel launch failed");
-    HIP_TRY(hipEventRecord(h->ev_unquantize, s), "hipEventRecord failed");
+    const LaunchEvents ev = take_events(h, h->ev_unquantize);
+    HIP_TRY(launch_unquantize(s, ev, qdev, out, rows, cols, nbits, add != 0, h->tune), "unquantize kernel launch failed");
+    h->last_unquantize = ev.stop;
     return CNTKQ_OK;
 }
 
@@ -400,7 +419,7 @@ int cntkq_wait_unquantize_done(cntkq_quantizer* h)
     if (h == nullptr)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_wait_unquantize_done: null handle");
     DeviceGuard guard(h->device);
-    return sync_event(h->ev_unquantize);
+    return h->last_unquantize != nullptr ? sync_event(h->last_unquantize) : CNTKQ_OK;
 }
 
 int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows,
@@ -436,10 +455,11 @@ int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, si
 
     DeviceGuard guard(h->device);
     hipStream_t s = work_stream(h);
-    HIP_TRY(launch_stripe_reduce(s, src, stripe_res, q_out, agg_out, rows, stripe_cols, nbits,
+    const LaunchEvents ev = take_events(h, h->ev_stripe);
+    HIP_TRY(launch_stripe_reduce(s, ev, src, stripe_res, q_out, agg_out, rows, stripe_cols, nbits,
                                  zero_threshold_for_1bit != 0, h->tune),
             "stripe reduction kernel launch failed");
-    HIP_TRY(hipEventRecord(h->ev_stripe, s), "hipEventRecord failed");
+    h->last_stripe = ev.stop;
     return CNTKQ_OK;
 }
 
@@ -448,7 +468,7 @@ int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h)
     if (h == nullptr)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_wait_stripe_reduce_done: null handle");
     DeviceGuard guard(h->device);
-    return sync_event(h->ev_stripe);
+    return h->last_stripe != nullptr ? sync_event(h->last_stripe) : CNTKQ_OK;
 }
 
 // ---- hooks for tests and tuning runs (not part of the public header) --------------------------------
@@ -467,6 +487,15 @@ int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_
     h->tune.unq_slots = unq_slots;
     h->tune.unq_force_scalar = unq_force_scalar;
     h->tune.tile_stage = tile_stage;
+    return CNTKQ_OK;
+}
+
+int cntkq_debug_attach_events(cntkq_quantizer* h, void* start_event, void* stop_event)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_attach_events: null handle");
+    h->attach_start = static_cast<hipEvent_t>(start_event);
+    h->attach_stop = static_cast<hipEvent_t>(stop_event);
     return CNTKQ_OK;
 }
 

@@ -18,6 +18,12 @@ extern "C" {
 int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_gs, unsigned unq_slots,
                            int unq_force_scalar, int tile_stage);
 
+/* Ties caller-owned hipEvent_t objects (either may be NULL) to the NEXT kernel this handle launches: start_event is
+ * set when that kernel begins, stop_event when it has finished, by the dispatch itself. Used to time single kernels
+ * without putting extra commands into the stream. The stop event also becomes what the matching Wait call waits on,
+ * so it must stay alive until then. */
+int cntkq_debug_attach_events(cntkq_quantizer* h, void* start_event, void* stop_event);
+
 #ifdef __cplusplus
 }
 #endif

@@ -4,6 +4,7 @@
 
 #include "quantizer_kernels.h"
 
+#include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
@@ -28,6 +29,14 @@ struct LaunchTuning
     int tile_stage = -1;    // -1 = automatic; 0 / 1 = residual written straight to memory / staged through LDS
     uint32_t unq_slots = 0; // 0 = default; else bit positions per thread in unquantize
     int unq_force_scalar = 0;
+};
+
+// Events tied to the kernel dispatch itself (its completion signal), not recorded as separate stream
+// commands: a separate record after every kernel costs about 3 us of idle GPU per launch on MI355X.
+struct LaunchEvents
+{
+    hipEvent_t start = nullptr; // optional: set when the kernel starts
+    hipEvent_t stop = nullptr;  // optional: set when the kernel has finished
 };
 
 inline bool valid_nbits(size_t nbits)
@@ -92,11 +101,11 @@ inline hipError_t dispatch_nbits(size_t nbits, bool zt, Args... args)
 template <int NBITS, bool ZT>
 struct TileLauncher
 {
-    static hipError_t run(hipStream_t s, const float* g, const float* r_in, float* r_out, char* q, TileGeom t)
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, TileGeom t)
     {
         const uint32_t tiles = (t.cols + t.cols_per_tile - 1) / t.cols_per_tile;
         const size_t lds = tile_lds_bytes(t, 0);
-        hipLaunchKernelGGL((quantize_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(kTileThreads), lds, s, g, r_in, r_out, q, t);
+        hipExtLaunchKernelGGL((quantize_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(kTileThreads), lds, s, ev.start, ev.stop, 0, g, r_in, r_out, q, t);
         return hipGetLastError();
     }
 };
@@ -104,10 +113,10 @@ struct TileLauncher
 template <int NBITS, bool ZT>
 struct TallLauncher
 {
-    static hipError_t run(hipStream_t s, const float* g, const float* r_in, float* r_out, char* q, uint32_t rows,
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t rows,
                           uint32_t cols, uint32_t nq, uint64_t qcol)
     {
-        hipLaunchKernelGGL((quantize_tall_kernel<NBITS, ZT>), dim3(cols), dim3(kTallThreads), 0, s, g, r_in, r_out, q, rows,
+        hipExtLaunchKernelGGL((quantize_tall_kernel<NBITS, ZT>), dim3(cols), dim3(kTallThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, q, rows,
                            nq, qcol);
         return hipGetLastError();
     }
@@ -116,12 +125,12 @@ struct TallLauncher
 template <int NBITS, bool ZT>
 struct StripeLauncher
 {
-    static hipError_t run(hipStream_t s, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
                           TileGeom t)
     {
         const uint32_t tiles = (t.cols + t.cols_per_tile - 1) / t.cols_per_tile;
         const size_t lds = tile_lds_bytes(t, src.workers);
-        hipLaunchKernelGGL((stripe_reduce_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(kTileThreads), lds, s, src, stripe_res,
+        hipExtLaunchKernelGGL((stripe_reduce_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(kTileThreads), lds, s, ev.start, ev.stop, 0, src, stripe_res,
                            q_out, agg_out, t);
         return hipGetLastError();
     }
@@ -135,7 +144,7 @@ inline bool wavecol_applicable(const float* g, const float* r_in, const float* r
 }
 
 // Launches the quantize kernel(s) for one matrix. rows, cols > 0; pointers 4-byte aligned (checked by caller).
-inline hipError_t launch_quantize(hipStream_t s, const float* g, const float* r_in, float* r_out, void* q, size_t rows,
+inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, void* q, size_t rows,
                                   size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
 {
     zt = zt && (nbits == 1);
@@ -160,16 +169,16 @@ inline hipError_t launch_quantize(hipStream_t s, const float* g, const float* r_
         if (rows == 2048)
         {
             if (zt)
-                hipLaunchKernelGGL((quantize_wavecol_kernel<true, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+                hipExtLaunchKernelGGL((quantize_wavecol_kernel<true, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, qc, (uint32_t) cols, qcol);
             else
-                hipLaunchKernelGGL((quantize_wavecol_kernel<false, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+                hipExtLaunchKernelGGL((quantize_wavecol_kernel<false, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, qc, (uint32_t) cols, qcol);
         }
         else
         {
             if (zt)
-                hipLaunchKernelGGL((quantize_wavecol_kernel<true, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+                hipExtLaunchKernelGGL((quantize_wavecol_kernel<true, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, qc, (uint32_t) cols, qcol);
             else
-                hipLaunchKernelGGL((quantize_wavecol_kernel<false, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, g, r_in, r_out, qc, (uint32_t) cols, qcol);
+                hipExtLaunchKernelGGL((quantize_wavecol_kernel<false, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, qc, (uint32_t) cols, qcol);
         }
         return hipGetLastError();
     }
@@ -178,13 +187,13 @@ inline hipError_t launch_quantize(hipStream_t s, const float* g, const float* r_
         if (rows > kTileMaxRows)
             return hipErrorInvalidValue;
         const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs, tune.tile_stage);
-        return dispatch_nbits<TileLauncher>(nbits, zt, s, g, r_in, r_out, qc, t);
+        return dispatch_nbits<TileLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, t);
     }
-    return dispatch_nbits<TallLauncher>(nbits, zt, s, g, r_in, r_out, qc, (uint32_t) rows, (uint32_t) cols,
+    return dispatch_nbits<TallLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) rows, (uint32_t) cols,
                                         (uint32_t) qwords_per_col(rows, nbits), (uint64_t) qcol_bytes(nbits, rows));
 }
 
-inline hipError_t launch_stripe_reduce(hipStream_t s, const StripeSources& src, float* stripe_res, void* q_out,
+inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, void* q_out,
                                        float* agg_out, size_t rows, size_t cols, size_t nbits, bool zt,
                                        const LaunchTuning& tune)
 {
@@ -203,11 +212,11 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, const StripeSources& src, 
             gs >>= 1;
     }
     const TileGeom t = make_tile_geom(rows, cols, nbits, gs, tune.tile_stage);
-    return dispatch_nbits<StripeLauncher>(nbits, zt, s, src, stripe_res, static_cast<char*>(q_out), agg_out, t);
+    return dispatch_nbits<StripeLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, t);
 }
 
 template <int NBITS, int WV>
-inline hipError_t launch_unquantize_t(hipStream_t s, const char* q, float* out, size_t rows, size_t cols, uint32_t slots,
+inline hipError_t launch_unquantize_t(hipStream_t s, LaunchEvents ev, const char* q, float* out, size_t rows, size_t cols, uint32_t slots,
                                       int add)
 {
     constexpr uint32_t VPW = 32 / NBITS;
@@ -230,11 +239,11 @@ inline hipError_t launch_unquantize_t(hipStream_t s, const char* q, float* out, 
     t.items = (uint32_t) items;
     t.qcol = qcol_bytes(NBITS, rows);
     const uint32_t blocks = (uint32_t) ((items + 255) / 256);
-    hipLaunchKernelGGL((unquantize_kernel<NBITS, WV>), dim3(blocks), dim3(256), 0, s, q, out, t, add);
+    hipExtLaunchKernelGGL((unquantize_kernel<NBITS, WV>), dim3(blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, t, add);
     return hipGetLastError();
 }
 
-inline hipError_t launch_unquantize(hipStream_t s, const void* q, float* out, size_t rows, size_t cols, size_t nbits,
+inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* q, float* out, size_t rows, size_t cols, size_t nbits,
                                     bool add, const LaunchTuning& tune)
 {
     const char* qc = static_cast<const char*>(q);
@@ -245,12 +254,12 @@ inline hipError_t launch_unquantize(hipStream_t s, const void* q, float* out, si
     const uint32_t sl = tune.unq_slots;
     switch (nbits)
     {
-    case 1: return vec ? launch_unquantize_t<1, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<1, 1>(s, qc, out, rows, cols, sl, a);
-    case 2: return vec ? launch_unquantize_t<2, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<2, 1>(s, qc, out, rows, cols, sl, a);
-    case 4: return vec ? launch_unquantize_t<4, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<4, 1>(s, qc, out, rows, cols, sl, a);
-    case 8: return vec ? launch_unquantize_t<8, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<8, 1>(s, qc, out, rows, cols, sl, a);
-    case 16: return vec ? launch_unquantize_t<16, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<16, 1>(s, qc, out, rows, cols, sl, a);
-    case 32: return vec ? launch_unquantize_t<32, 4>(s, qc, out, rows, cols, sl, a) : launch_unquantize_t<32, 1>(s, qc, out, rows, cols, sl, a);
+    case 1: return vec ? launch_unquantize_t<1, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<1, 1>(s, ev, qc, out, rows, cols, sl, a);
+    case 2: return vec ? launch_unquantize_t<2, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<2, 1>(s, ev, qc, out, rows, cols, sl, a);
+    case 4: return vec ? launch_unquantize_t<4, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<4, 1>(s, ev, qc, out, rows, cols, sl, a);
+    case 8: return vec ? launch_unquantize_t<8, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<8, 1>(s, ev, qc, out, rows, cols, sl, a);
+    case 16: return vec ? launch_unquantize_t<16, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<16, 1>(s, ev, qc, out, rows, cols, sl, a);
+    case 32: return vec ? launch_unquantize_t<32, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<32, 1>(s, ev, qc, out, rows, cols, sl, a);
     default: return hipErrorInvalidValue;
     }
 }
