@@ -1,0 +1,397 @@
+// C++ host side of the MI355X gradient quantizer: the reference's class shapes on top of the C ABI.
+//
+//   cntk_amd::MatrixQuantizerImpl<float>   <->  Source/Math/MatrixQuantizerImpl.h:19-49
+//   cntk_amd::QuantizedMatrix<float>       <->  Source/Math/QuantizedMatrix.h:54-124, Source/Math/QuantizedMatrix.cpp
+//   cntk_amd::QuantizedColumn<float>       <->  Source/Math/QuantizedMatrix.h:27-48
+//   cntk_amd::MatrixQuantizer<float>       <->  Source/1BitSGD/MatrixQuantizer.h:24-85
+//   cntk_amd::MatrixComputeStreamEvent     <->  Source/Math/MatrixQuantizerImpl.h:53-72
+//   cntk_amd::Matrix<float>                     the little of Source/Math/Matrix.h this path needs
+//
+// Same method names, argument meaning and error behaviour (LogicError / RuntimeError / InvalidArgument become
+// std::logic_error / std::runtime_error / std::invalid_argument). Only ElemType = float exists. Header-only; link with
+// libcntk_amd_quantizer.so and the HIP runtime. There is no CPU quantizer: Create(deviceId < 0) throws.
+#pragma once
+
+#include "../../include/cntk_amd_quantizer.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+#include <vector>
+
+namespace cntk_amd {
+
+constexpr int CPUDEVICE = -1;
+
+namespace detail {
+inline void Check(int rc)
+{
+    if (rc == CNTKQ_OK)
+        return;
+    const std::string msg = cntkq_last_error();
+    if (rc == CNTKQ_RUNTIME_ERROR)
+        throw std::runtime_error(msg);
+    if (rc == CNTKQ_INVALID_ARGUMENT)
+        throw std::invalid_argument(msg);
+    throw std::logic_error(msg);
+}
+
+inline void HipCheck(hipError_t rc, const char* what)
+{
+    if (rc != hipSuccess)
+        throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(rc));
+}
+} // namespace detail
+
+// Dense column-major matrix on one GPU: element (i, j) at Data()[j * GetNumRows() + i]. Owning, or a view of columns.
+template <class ElemType>
+class Matrix
+{
+    static_assert(std::is_same<ElemType, float>::value, "only float is instantiated");
+
+public:
+    Matrix(size_t numRows, size_t numCols, int deviceId) : m_rows(numRows), m_cols(numCols), m_device(deviceId), m_owner(true)
+    {
+        if (deviceId < 0)
+            throw std::invalid_argument("Matrix: this library keeps matrices on a GPU");
+        detail::HipCheck(hipSetDevice(deviceId), "hipSetDevice");
+        const size_t bytes = numRows * numCols * sizeof(ElemType);
+        if (bytes != 0)
+        {
+            detail::HipCheck(hipMalloc(reinterpret_cast<void**>(&m_data), bytes), "hipMalloc");
+            detail::HipCheck(hipMemset(m_data, 0, bytes), "hipMemset"); // matrices start as zeros, like the reference's
+        }
+    }
+    Matrix(Matrix&& o) noexcept : m_data(o.m_data), m_rows(o.m_rows), m_cols(o.m_cols), m_device(o.m_device), m_owner(o.m_owner)
+    {
+        o.m_data = nullptr;
+        o.m_owner = false;
+    }
+    Matrix(const Matrix&) = delete;
+    Matrix& operator=(const Matrix&) = delete;
+    ~Matrix()
+    {
+        if (m_owner && m_data != nullptr)
+            (void) hipFree(m_data);
+    }
+
+    size_t GetNumRows() const { return m_rows; }
+    size_t GetNumCols() const { return m_cols; }
+    size_t GetNumElements() const { return m_rows * m_cols; }
+    int GetDeviceId() const { return m_device; }
+    ElemType* Data() const { return m_data; }
+
+    // zero-copy view of columns [startColumn, startColumn + numCols) (Source/Math/Matrix.h:194)
+    Matrix ColumnSlice(size_t startColumn, size_t numCols) const
+    {
+        if (startColumn + numCols > m_cols)
+            throw std::logic_error("ColumnSlice: out of range");
+        return Matrix(m_data + startColumn * m_rows, m_rows, numCols, m_device);
+    }
+
+    void SetValue(ElemType v)
+    {
+        std::vector<ElemType> host(GetNumElements(), v);
+        SetValue(host.data());
+    }
+    void SetValue(const ElemType* hostColumnMajor)
+    {
+        if (GetNumElements() != 0)
+            detail::HipCheck(hipMemcpy(m_data, hostColumnMajor, GetNumElements() * sizeof(ElemType), hipMemcpyHostToDevice), "hipMemcpy");
+    }
+    // host copy in column-major order (Matrix::CopyToArray)
+    std::unique_ptr<ElemType[]> CopyToArray() const
+    {
+        std::unique_ptr<ElemType[]> host(new ElemType[GetNumElements() ? GetNumElements() : 1]);
+        if (GetNumElements() != 0)
+            detail::HipCheck(hipMemcpy(host.get(), m_data, GetNumElements() * sizeof(ElemType), hipMemcpyDeviceToHost), "hipMemcpy");
+        return host;
+    }
+
+private:
+    Matrix(ElemType* data, size_t rows, size_t cols, int device) : m_data(data), m_rows(rows), m_cols(cols), m_device(device), m_owner(false) {}
+
+    ElemType* m_data = nullptr;
+    size_t m_rows, m_cols;
+    int m_device;
+    bool m_owner;
+};
+
+// One packed column: { lower; upper; bits[nq] } (Source/Math/QuantizedMatrix.h:27-48)
+template <class ElemType>
+struct QuantizedColumn
+{
+    typedef uint32_t QWord;
+    static const size_t QWordNumBits = 8 * sizeof(QWord);
+    ElemType lower;
+    ElemType upper;
+    QWord bits[1];
+
+    static size_t QuantizedColumnSize(size_t bits, size_t rows) { return cntkq_qcol_bytes(bits, rows); }
+};
+
+// Packed matrix; on a GPU (deviceId >= 0) or in pinned host memory (CPUDEVICE), which is how the reference's v1
+// aggregator keeps it (Source/1BitSGD/AllReduceDistGradAggregator.h:76-77, 88). Move-only; ColumnSlice is a view.
+template <class ElemType>
+class QuantizedMatrix
+{
+    static_assert(std::is_same<ElemType, float>::value, "only float is instantiated");
+
+public:
+    QuantizedMatrix(size_t numRows, size_t numCols, size_t nbits, int deviceId)
+        : m_rows(numRows), m_cols(numCols), m_bits(nbits), m_device(deviceId), m_owner(true)
+    {
+        m_qColSize = cntkq_qcol_bytes(nbits, numRows);
+        if (m_qColSize == 0) // Source/Math/QuantizedMatrix.cpp:12-15
+            throw std::logic_error("Quantization: 'nbits' must be a power of two that divides 32");
+        const size_t bytes = m_qColSize * numCols;
+        if (bytes == 0)
+            return;
+        if (deviceId >= 0)
+        {
+            detail::HipCheck(hipSetDevice(deviceId), "hipSetDevice");
+            detail::HipCheck(hipMalloc(reinterpret_cast<void**>(&m_buffer), bytes), "hipMalloc");
+            detail::HipCheck(hipMemset(m_buffer, 0, bytes), "hipMemset");
+        }
+        else
+        {
+            detail::HipCheck(hipHostMalloc(reinterpret_cast<void**>(&m_buffer), bytes, hipHostMallocDefault), "hipHostMalloc");
+            std::memset(m_buffer, 0, bytes);
+        }
+    }
+    QuantizedMatrix(QuantizedMatrix&& o) noexcept
+        : m_buffer(o.m_buffer), m_rows(o.m_rows), m_cols(o.m_cols), m_bits(o.m_bits), m_qColSize(o.m_qColSize), m_device(o.m_device), m_owner(o.m_owner)
+    {
+        o.m_buffer = nullptr;
+        o.m_owner = false;
+    }
+    QuantizedMatrix(const QuantizedMatrix&) = delete;
+    QuantizedMatrix& operator=(const QuantizedMatrix&) = delete;
+    ~QuantizedMatrix()
+    {
+        if (m_owner && m_buffer != nullptr)
+        {
+            if (m_device >= 0)
+                (void) hipFree(m_buffer);
+            else
+                (void) hipHostFree(m_buffer);
+        }
+    }
+
+    int GetDeviceId() const { return m_device; }
+    size_t GetNumRows() const { return m_rows; }
+    size_t GetNumCols() const { return m_cols; }
+    size_t GetNumBits() const { return m_bits; }
+    size_t GetSize() const { return m_qColSize * m_cols; }
+    char* Buffer() const { return m_buffer; }
+
+    // valid to dereference only for a host-resident matrix
+    QuantizedColumn<ElemType>* GetQuantizedColumn(size_t colIdx)
+    {
+        return reinterpret_cast<QuantizedColumn<ElemType>*>(m_buffer + m_qColSize * colIdx);
+    }
+
+    QuantizedMatrix ColumnSlice(size_t startColumn, size_t numCols) const
+    {
+        if (startColumn + numCols > m_cols)
+            throw std::logic_error("ColumnSlice: out of range");
+        return QuantizedMatrix(m_buffer + startColumn * m_qColSize, m_rows, numCols, m_bits, m_qColSize, m_device);
+    }
+
+    // host copy of the packed bytes, wherever they live
+    std::vector<char> CopyToHost() const
+    {
+        std::vector<char> host(GetSize());
+        if (!host.empty())
+        {
+            if (m_device >= 0)
+                detail::HipCheck(hipMemcpy(host.data(), m_buffer, host.size(), hipMemcpyDeviceToHost), "hipMemcpy");
+            else
+                std::memcpy(host.data(), m_buffer, host.size());
+        }
+        return host;
+    }
+
+private:
+    QuantizedMatrix(char* buffer, size_t rows, size_t cols, size_t bits, size_t qColSize, int device)
+        : m_buffer(buffer), m_rows(rows), m_cols(cols), m_bits(bits), m_qColSize(qColSize), m_device(device), m_owner(false)
+    {
+    }
+
+    char* m_buffer = nullptr;
+    size_t m_rows, m_cols, m_bits;
+    size_t m_qColSize = 0;
+    int m_device;
+    bool m_owner;
+};
+
+// The quantizer boundary (Source/Math/MatrixQuantizerImpl.h:19-49)
+template <class ElemType>
+class MatrixQuantizerImpl
+{
+    static_assert(std::is_same<ElemType, float>::value, "only float is instantiated");
+
+public:
+    // deviceId >= 0: the GPU quantizer, useAsync = dedicated compute stream (Source/Math/MatrixQuantizerImpl.cpp:10-26)
+    static MatrixQuantizerImpl<ElemType>* Create(int deviceId, bool useAsync);
+    virtual ~MatrixQuantizerImpl() {}
+    MatrixQuantizerImpl(const MatrixQuantizerImpl&) = delete;
+    MatrixQuantizerImpl& operator=(const MatrixQuantizerImpl&) = delete;
+
+    virtual void QuantizeAsync(const Matrix<ElemType>& inMatrix, const Matrix<ElemType>& inResidual, QuantizedMatrix<ElemType>& outQMatrix,
+                               Matrix<ElemType>& outResidual, bool zeroThresholdFor1Bit) = 0;
+    virtual void WaitQuantizeAsyncDone() = 0;
+    virtual void UnquantizeAsync(QuantizedMatrix<ElemType>& inQMatrix, Matrix<ElemType>& outMatrix, bool add = false) = 0;
+    virtual void WaitUnquantizeAsyncDone() = 0;
+
+    int GetDeviceId() const { return m_deviceId; }
+
+protected:
+    explicit MatrixQuantizerImpl(int deviceId) : m_deviceId(deviceId) {}
+
+private:
+    int m_deviceId;
+};
+
+// Replaces MatrixQuantizerGPU (Source/Math/MatrixQuantizerGPU.h:17-95)
+template <class ElemType>
+class MatrixQuantizerGPU final : public MatrixQuantizerImpl<ElemType>
+{
+public:
+    MatrixQuantizerGPU(int deviceId, bool useDedicatedComputeStream) : MatrixQuantizerImpl<ElemType>(deviceId)
+    {
+        detail::Check(cntkq_create(deviceId, useDedicatedComputeStream ? 1 : 0, &m_handle));
+    }
+    ~MatrixQuantizerGPU() override { (void) cntkq_destroy(m_handle); }
+
+    void QuantizeAsync(const Matrix<ElemType>& inMatrix, const Matrix<ElemType>& inResidual, QuantizedMatrix<ElemType>& outQMatrix,
+                       Matrix<ElemType>& outResidual, bool zeroThresholdFor1Bit) override
+    {
+        const size_t rows = inMatrix.GetNumRows(), cols = inMatrix.GetNumCols();
+        // asserts in the reference (Source/Math/MatrixQuantizerGPU.cu:229-232)
+        if (outQMatrix.GetNumRows() != rows || outQMatrix.GetNumCols() != cols || inResidual.GetNumRows() != rows ||
+            inResidual.GetNumCols() != cols || outResidual.GetNumRows() != rows || outResidual.GetNumCols() != cols)
+            throw std::invalid_argument("QuantizeAsync: matrix dimensions do not match");
+        detail::Check(cntkq_quantize_async(m_handle, inMatrix.Data(), inResidual.Data(), rows, cols, outQMatrix.Buffer(), outQMatrix.GetSize(),
+                                           outQMatrix.GetDeviceId() == CPUDEVICE, outQMatrix.GetNumBits(), outResidual.Data(),
+                                           zeroThresholdFor1Bit ? 1 : 0));
+    }
+    void WaitQuantizeAsyncDone() override { detail::Check(cntkq_wait_quantize_done(m_handle)); }
+
+    void UnquantizeAsync(QuantizedMatrix<ElemType>& inQMatrix, Matrix<ElemType>& outMatrix, bool add = false) override
+    {
+        if (inQMatrix.GetNumRows() != outMatrix.GetNumRows() || inQMatrix.GetNumCols() != outMatrix.GetNumCols())
+            throw std::invalid_argument("UnquantizeAsync: matrix dimensions do not match");
+        detail::Check(cntkq_unquantize_async(m_handle, inQMatrix.Buffer(), inQMatrix.GetSize(), inQMatrix.GetDeviceId() == CPUDEVICE, outMatrix.Data(),
+                                             outMatrix.GetNumRows(), outMatrix.GetNumCols(), inQMatrix.GetNumBits(), add ? 1 : 0));
+    }
+    void WaitUnquantizeAsyncDone() override { detail::Check(cntkq_wait_unquantize_done(m_handle)); }
+
+    // Fused stripe reduction of the quantized all-reduce (dataflow of Source/1BitSGD/AllReduceDistGradAggregator.h:365-436):
+    // stripes[w] is worker w's packed stripe; the requantized aggregate goes to outQStripe (may be stripes[owner]).
+    void StripeReduceAsync(const std::vector<const QuantizedMatrix<ElemType>*>& stripes, size_t owner, Matrix<ElemType>& stripeResidual,
+                           QuantizedMatrix<ElemType>& outQStripe, bool zeroThresholdFor1Bit, Matrix<ElemType>* aggregate = nullptr)
+    {
+        std::vector<const void*> ptrs;
+        for (const auto* s : stripes)
+        {
+            if (s->GetNumRows() != outQStripe.GetNumRows() || s->GetNumCols() != outQStripe.GetNumCols() || s->GetNumBits() != outQStripe.GetNumBits() ||
+                s->GetDeviceId() < 0)
+                throw std::invalid_argument("StripeReduceAsync: stripes must be device-resident and of equal shape");
+            ptrs.push_back(s->Buffer());
+        }
+        detail::Check(cntkq_stripe_reduce_async(m_handle, ptrs.data(), ptrs.size(), owner, outQStripe.GetNumRows(), outQStripe.GetNumCols(),
+                                                outQStripe.GetNumBits(), stripeResidual.Data(), outQStripe.Buffer(),
+                                                aggregate ? aggregate->Data() : nullptr, zeroThresholdFor1Bit ? 1 : 0));
+    }
+    void WaitStripeReduceDone() { detail::Check(cntkq_wait_stripe_reduce_done(m_handle)); }
+
+    cntkq_quantizer* Handle() const { return m_handle; }
+
+private:
+    cntkq_quantizer* m_handle = nullptr;
+};
+
+template <class ElemType>
+MatrixQuantizerImpl<ElemType>* MatrixQuantizerImpl<ElemType>::Create(int deviceId, bool useAsync)
+{
+    if (deviceId >= 0)
+        return new MatrixQuantizerGPU<ElemType>(deviceId, useAsync);
+    // the reference returns its CPU quantizer here; a build without one throws, as CPUONLY builds do for GPUs
+    throw std::runtime_error("CreateMatrixQuantizer: this library has no CPU quantizer");
+}
+
+// Orders the quantizer's stream after everything already issued on the main stream
+// (Source/Math/MatrixQuantizerImpl.h:53-72, Source/Math/MatrixQuantizerGPU.cu:347-371)
+class MatrixComputeStreamEvent
+{
+public:
+    static MatrixComputeStreamEvent* Create(int deviceId) { return new MatrixComputeStreamEvent(deviceId); }
+    virtual ~MatrixComputeStreamEvent() {}
+    virtual void SynchronizeEvent() { detail::HipCheck(hipStreamSynchronize(nullptr), "hipStreamSynchronize"); }
+
+    template <typename ElemType>
+    void SynchronizeQuantizationComputeStreamWithEvent(MatrixQuantizerImpl<ElemType>& quantizer)
+    {
+        auto* gpu = dynamic_cast<MatrixQuantizerGPU<ElemType>*>(&quantizer);
+        if (gpu != nullptr)
+            detail::Check(cntkq_sync_with_main_stream(gpu->Handle()));
+    }
+
+protected:
+    explicit MatrixComputeStreamEvent(int deviceId) : m_deviceId(deviceId) {}
+    int m_deviceId;
+};
+
+// Quantizer that owns the error-feedback residual (Source/1BitSGD/MatrixQuantizer.h:24-85)
+class MatrixQuantizerBase
+{
+};
+
+template <class ElemType>
+class MatrixQuantizer final : public MatrixQuantizerBase
+{
+public:
+    MatrixQuantizer(size_t numRows, size_t numCols, int deviceId, bool useAsync) : MatrixQuantizer(deviceId, useAsync)
+    {
+        m_residual = std::make_shared<Matrix<ElemType>>(numRows, numCols, deviceId);
+    }
+    MatrixQuantizer(int deviceId, bool useAsync) : m_residual(nullptr)
+    {
+        m_quantizerImpl.reset(MatrixQuantizerImpl<ElemType>::Create(deviceId, useAsync));
+    }
+    MatrixQuantizer(const MatrixQuantizer&) = delete;
+    MatrixQuantizer& operator=(const MatrixQuantizer&) = delete;
+
+    void QuantizeAsync(const Matrix<ElemType>& inMatrix, QuantizedMatrix<ElemType>& outQMatrix, bool zeroThresholdFor1Bit)
+    {
+        m_quantizerImpl->QuantizeAsync(inMatrix, *m_residual, outQMatrix, *m_residual, zeroThresholdFor1Bit);
+    }
+    void QuantizeAsync(const Matrix<ElemType>& inMatrix, const Matrix<ElemType>& inResidual, QuantizedMatrix<ElemType>& outQMatrix,
+                       Matrix<ElemType>& outResidual, bool zeroThresholdFor1Bit)
+    {
+        m_quantizerImpl->QuantizeAsync(inMatrix, inResidual, outQMatrix, outResidual, zeroThresholdFor1Bit);
+    }
+    void WaitQuantizeAsyncDone() { m_quantizerImpl->WaitQuantizeAsyncDone(); }
+    void UnquantizeAsync(QuantizedMatrix<ElemType>& inQMatrix, Matrix<ElemType>& outMatrix, bool add = false)
+    {
+        m_quantizerImpl->UnquantizeAsync(inQMatrix, outMatrix, add);
+    }
+    void WaitUnquantizeAsyncDone() { m_quantizerImpl->WaitUnquantizeAsyncDone(); }
+    int GetDeviceId() const { return m_quantizerImpl->GetDeviceId(); }
+    void ResetResidue() { m_residual->SetValue(0.0f); }
+    const Matrix<ElemType>& GetResidualMatrix() const { return *m_residual; }
+    MatrixQuantizerImpl<ElemType>& Impl() { return *m_quantizerImpl; }
+
+private:
+    std::unique_ptr<MatrixQuantizerImpl<ElemType>> m_quantizerImpl;
+    std::shared_ptr<Matrix<ElemType>> m_residual;
+};
+
+} // namespace cntk_amd

@@ -46,8 +46,9 @@ struct TileGeom
     uint32_t rows;
     uint32_t cols;
     uint32_t nq;            // QWords per column
-    uint32_t cols_per_tile; // kTileThreads / gs, <= kTileMaxCols
-    uint32_t gs;            // threads per column in the statistics phase: power of two in [8, 256]
+    uint32_t threads;       // workgroup size: 64, 128 or 256
+    uint32_t cols_per_tile; // threads / gs, <= kTileMaxCols
+    uint32_t gs;            // threads per column in the statistics phase: power of two in [8, threads]
     uint32_t gs_log2;
     uint32_t tile_floats;   // LDS floats reserved for the tile: cols_per_tile * rows + alignment slack, multiple of 4
     uint32_t words_floats;  // LDS words for partial QWords: cols_per_tile * nq when a QWord has several work items, else 0
@@ -152,7 +153,7 @@ __device__ __forceinline__ void tile_pack(float* tile, const float* hdr, uint32_
     const uint32_t nwords = nc * t.nq;
     const uint32_t items = nwords * PS::CHUNKS;
     const bool stage = t.stage_residual != 0;
-    for (uint32_t it = threadIdx.x; it < items; it += kTileThreads)
+    for (uint32_t it = threadIdx.x; it < items; it += t.threads)
     {
         // chunk-major: consecutive threads take consecutive QWords, hence consecutive rows
         const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
@@ -195,7 +196,7 @@ __device__ __forceinline__ void tile_pack(float* tile, const float* hdr, uint32_
     if constexpr (PS::CHUNKS > 1)
     {
         __syncthreads();
-        for (uint32_t qi = threadIdx.x; qi < nwords; qi += kTileThreads)
+        for (uint32_t qi = threadIdx.x; qi < nwords; qi += t.threads)
         {
             const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
             const uint32_t w = qi - c * t.nq;
@@ -210,7 +211,8 @@ __device__ __forceinline__ void tile_pack(float* tile, const float* hdr, uint32_
 
 // Coalesced copy of the tile (now holding the new residual) to global memory; 16-byte stores where the
 // destination shares the tile's 16-byte phase (`mis` = floats by which the tile start is off a 16-byte boundary).
-__device__ __forceinline__ void tile_store(const float* tile, uint32_t mis, float* dst, uint32_t total)
+__device__ __forceinline__ void tile_store(const float* tile, uint32_t mis, float* dst, uint32_t total,
+                                           const TileGeom& t)
 {
     const uint32_t tid = threadIdx.x;
     const uint32_t mis_d = (uint32_t) ((reinterpret_cast<uintptr_t>(dst) >> 2) & 3u);
@@ -225,14 +227,14 @@ __device__ __forceinline__ void tile_store(const float* tile, uint32_t mis, floa
             dst[tid] = tile[tid];
         const f32x4* t4 = reinterpret_cast<const f32x4*>(tile + head);
         f32x4* d4 = reinterpret_cast<f32x4*>(dst + head);
-        for (uint32_t e = tid; e < nvec; e += kTileThreads)
+        for (uint32_t e = tid; e < nvec; e += t.threads)
             __builtin_nontemporal_store(t4[e], d4 + e);
-        for (uint32_t e = tail0 + tid; e < total; e += kTileThreads)
+        for (uint32_t e = tail0 + tid; e < total; e += t.threads)
             dst[e] = tile[e];
     }
     else
     {
-        for (uint32_t e = tid; e < total; e += kTileThreads)
+        for (uint32_t e = tid; e < total; e += t.threads)
             __builtin_nontemporal_store(tile[e], dst + e);
     }
 }
@@ -259,7 +261,7 @@ __global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float
     const float* rp = r_in + base;
 
     if constexpr (PackShape<NBITS>::CHUNKS > 1)
-        for (uint32_t x = tid; x < nc * t.nq; x += kTileThreads)
+        for (uint32_t x = tid; x < nc * t.nq; x += t.threads)
             words[x] = 0u;
 
     // The tile starts `mis` floats into its LDS area so that LDS and global addresses share 16-byte phase.
@@ -279,13 +281,13 @@ __global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float
         const f32x4* g4 = reinterpret_cast<const f32x4*>(gp + head);
         const f32x4* r4 = reinterpret_cast<const f32x4*>(rp + head);
         f32x4* t4 = reinterpret_cast<f32x4*>(tile + head);
-        for (uint32_t e0 = tid; e0 < nvec; e0 += 4 * kTileThreads)
+        for (uint32_t e0 = tid; e0 < nvec; e0 += 4 * t.threads)
         {
             f32x4 a[4], b[4];
 #pragma unroll
             for (uint32_t u = 0; u < 4; ++u)
             {
-                const uint32_t e = e0 + u * kTileThreads;
+                const uint32_t e = e0 + u * t.threads;
                 if (e < nvec)
                 {
                     a[u] = __builtin_nontemporal_load(g4 + e);
@@ -295,17 +297,17 @@ __global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float
 #pragma unroll
             for (uint32_t u = 0; u < 4; ++u)
             {
-                const uint32_t e = e0 + u * kTileThreads;
+                const uint32_t e = e0 + u * t.threads;
                 if (e < nvec)
                     t4[e] = a[u] + b[u];
             }
         }
-        for (uint32_t e = tail0 + tid; e < total; e += kTileThreads)
+        for (uint32_t e = tail0 + tid; e < total; e += t.threads)
             tile[e] = gp[e] + rp[e];
     }
     else
     {
-        for (uint32_t e = tid; e < total; e += kTileThreads)
+        for (uint32_t e = tid; e < total; e += t.threads)
             tile[e] = __builtin_nontemporal_load(gp + e) + __builtin_nontemporal_load(rp + e);
     }
     __syncthreads();
@@ -314,7 +316,7 @@ __global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float
     tile_stats<NBITS, ZT>(tile, hdr, scratch_f, scratch_u, t, nc, qtile);
     tile_pack<NBITS, ZT>(tile, hdr, words, t, nc, qtile, r_out + base);
     if (t.stage_residual)
-        tile_store(tile, mis_g, r_out + base, total);
+        tile_store(tile, mis_g, r_out + base, total, t);
 }
 
 // ---- stripe reduction: K packed stripes -> fp32 sum -> requantize with the stripe residual ----------
@@ -359,12 +361,12 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
     float* tile = smem + kTilePrefixFloats + mis_s;
 
     if constexpr (PS::CHUNKS > 1)
-        for (uint32_t x = tid; x < nwords; x += kTileThreads)
+        for (uint32_t x = tid; x < nwords; x += t.threads)
             words[x] = 0u;
 
     // decode constants from every worker's column header, stored in summation order:
     // 1 bit -> the two levels, else (ufactor, lower)
-    for (uint32_t x = tid; x < nc * K; x += kTileThreads)
+    for (uint32_t x = tid; x < nc * K; x += t.threads)
     {
         const uint32_t c = x / K;
         const uint32_t n = x - c * K;
@@ -384,7 +386,7 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
     __syncthreads();
 
     const uint32_t items = nwords * PS::CHUNKS;
-    for (uint32_t it = tid; it < items; it += kTileThreads)
+    for (uint32_t it = tid; it < items; it += t.threads)
     {
         const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
         const uint32_t qi = it - chunk * nwords;
@@ -444,7 +446,7 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
     tile_stats<NBITS, ZT>(tile, hdr, scratch_f, scratch_u, t, nc, qtile);
     tile_pack<NBITS, ZT>(tile, hdr, words, t, nc, qtile, sp);
     if (t.stage_residual)
-        tile_store(tile, mis_s, sp, total);
+        tile_store(tile, mis_s, sp, total, t);
 }
 
 // ---- quantize, 1 bit, one wavefront per column, column share in registers ---------------------------
@@ -454,31 +456,13 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
 
 constexpr uint32_t kWaveColThreads = 128;
 
+// Statistics, header, codes and residual for one column held in registers by one wavefront:
+// v[c][k] is row lane + 64 * c + NQ * k; op = residual column + lane; qc = packed column record.
 template <bool ZT, int WPL>
-__global__ __launch_bounds__(kWaveColThreads) void quantize_wavecol_kernel(const float* __restrict__ g, const float* r_in,
-                                                                        float* r_out, char* __restrict__ q,
-                                                                        uint32_t cols, uint64_t qcol)
+__device__ __forceinline__ void wavecol_stats_pack(const float (&v)[WPL][32], uint32_t lane, float* op, char* qc)
 {
     constexpr uint32_t NQ = 64 * WPL;
     constexpr uint32_t ROWS = 32 * NQ;
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t j = blockIdx.x * (kWaveColThreads / 64) + (threadIdx.x >> 6);
-    if (j >= cols)
-        return; // whole wavefront leaves; no barriers below
-    const size_t base = (size_t) j * ROWS;
-    const float* gp = g + base + lane;
-    const float* rp = r_in + base + lane;
-
-    float v[WPL][32];
-#pragma unroll
-    for (int c = 0; c < WPL; ++c)
-#pragma unroll
-        for (int k = 0; k < 32; ++k)
-        {
-            const uint32_t i = 64u * c + NQ * k;
-            v[c][k] = __builtin_nontemporal_load(gp + i) + __builtin_nontemporal_load(rp + i);
-        }
-
     float mean = 0.0f;
     if constexpr (!ZT)
     {
@@ -511,10 +495,9 @@ __global__ __launch_bounds__(kWaveColThreads) void quantize_wavecol_kernel(const
     float lo, hi;
     finish_stats_1bit<ZT>(mean, s0, s1, n0, n1, ROWS, lo, hi);
 
-    char* qc = q + (size_t) j * qcol;
     if (lane == 0)
     {
-        f32x2 h;
+        f32x2 h; // NQ is even and the buffer 8-byte aligned, so every record is
         h.x = lo;
         h.y = hi;
         *reinterpret_cast<f32x2*>(qc) = h;
@@ -522,7 +505,6 @@ __global__ __launch_bounds__(kWaveColThreads) void quantize_wavecol_kernel(const
     const ValueQ vq = make_vq<1>(lo, hi);
     const float val0 = unquantize_value<1>(vq, 0u);
     const float val1 = unquantize_value<1>(vq, 1u);
-    float* op = r_out + base + lane;
     uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
 #pragma unroll
     for (int c = 0; c < WPL; ++c)
@@ -538,6 +520,120 @@ __global__ __launch_bounds__(kWaveColThreads) void quantize_wavecol_kernel(const
         }
         bits[lane + 64u * c] = word;
     }
+}
+
+template <bool ZT, int WPL>
+__global__ __launch_bounds__(kWaveColThreads) void quantize_wavecol_kernel(const float* __restrict__ g, const float* r_in,
+                                                                           float* r_out, char* __restrict__ q,
+                                                                           uint32_t cols, uint64_t qcol)
+{
+    constexpr uint32_t NQ = 64 * WPL;
+    constexpr uint32_t ROWS = 32 * NQ;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t j = blockIdx.x * (kWaveColThreads / 64) + (threadIdx.x >> 6);
+    if (j >= cols)
+        return; // whole wavefront leaves; no barriers below
+    const size_t base = (size_t) j * ROWS;
+    const float* gp = g + base + lane;
+    const float* rp = r_in + base + lane;
+
+    float v[WPL][32];
+#pragma unroll
+    for (int c = 0; c < WPL; ++c)
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+        {
+            const uint32_t i = 64u * c + NQ * k;
+            v[c][k] = __builtin_nontemporal_load(gp + i) + __builtin_nontemporal_load(rp + i);
+        }
+    wavecol_stats_pack<ZT, WPL>(v, lane, r_out + base + lane, q + (size_t) j * qcol);
+}
+
+// ---- stripe reduction, 1 bit, one wavefront per column (rows = 2048 * WPL) ---------------------------
+//
+// Lane l owns QWords l, l + 64, ... of the column in EVERY worker's packed stripe: it decodes its 32 * WPL rows
+// from each worker in turn, sums them in registers, adds the stripe residual and requantizes, all without LDS.
+
+template <bool ZT, int WPL>
+__global__ __launch_bounds__(kWaveColThreads) void stripe_reduce_wavecol_kernel(StripeSources src, float* stripe_res,
+                                                                                char* q_out, float* agg_out,
+                                                                                uint32_t cols, uint64_t qcol)
+{
+    constexpr uint32_t NQ = 64 * WPL;
+    constexpr uint32_t ROWS = 32 * NQ;
+    constexpr uint32_t BATCH = 8;
+    const uint32_t lane = threadIdx.x & 63u;
+    // the column index is the same for the whole wavefront: keep it (and everything derived from it) scalar
+    const uint32_t j = __builtin_amdgcn_readfirstlane(blockIdx.x * (kWaveColThreads / 64) + (threadIdx.x >> 6));
+    if (j >= cols)
+        return;
+    const size_t base = (size_t) j * ROWS;
+    const size_t rec = (size_t) j * qcol;
+    const uint32_t K = src.workers;
+
+    float sres[WPL][32];
+    const float* sp = stripe_res + base + lane;
+#pragma unroll
+    for (int c = 0; c < WPL; ++c)
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+            sres[c][k] = __builtin_nontemporal_load(sp + 64u * c + NQ * k);
+
+    float acc[WPL][32];
+    for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
+    {
+        uint32_t word[BATCH][WPL];
+        float lo[BATCH], hi[BATCH];
+#pragma unroll
+        for (uint32_t u = 0; u < BATCH; ++u)
+        {
+            if (n0 + u < K)
+            {
+                const char* qc = src.q[stripe_order(n0 + u, src.owner)] + rec;
+                lo[u] = reinterpret_cast<const float*>(qc)[0];
+                hi[u] = reinterpret_cast<const float*>(qc)[1];
+#pragma unroll
+                for (int c = 0; c < WPL; ++c)
+                    word[u][c] = reinterpret_cast<const uint32_t*>(qc + 8)[lane + 64u * c];
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < BATCH; ++u)
+        {
+            if (n0 + u < K)
+            {
+                const ValueQ vq = make_vq<1>(lo[u], hi[u]);
+                const float val0 = unquantize_value<1>(vq, 0u);
+                const float val1 = unquantize_value<1>(vq, 1u);
+#pragma unroll
+                for (int c = 0; c < WPL; ++c)
+#pragma unroll
+                    for (int k = 0; k < 32; ++k)
+                    {
+                        const float x = ((word[u][c] >> k) & 1u) ? val1 : val0;
+                        // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
+                        acc[c][k] = (n0 + u == 0) ? x : x + acc[c][k];
+                    }
+            }
+        }
+    }
+
+    if (agg_out != nullptr)
+    {
+        float* ap = agg_out + base + lane;
+#pragma unroll
+        for (int c = 0; c < WPL; ++c)
+#pragma unroll
+            for (int k = 0; k < 32; ++k)
+                ap[64u * c + NQ * k] = acc[c][k];
+    }
+    float v[WPL][32];
+#pragma unroll
+    for (int c = 0; c < WPL; ++c)
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+            v[c][k] = acc[c][k] + sres[c][k];
+    wavecol_stats_pack<ZT, WPL>(v, lane, stripe_res + base + lane, q_out + rec);
 }
 
 // ---- quantize, columns too tall for LDS: one workgroup per column, global memory re-read -------------

@@ -27,6 +27,7 @@ struct LaunchTuning
     int quantize_path = kPathAuto;
     uint32_t tile_gs = 0;   // 0 = pick from rows; else threads per column (power of two, 8..256)
     int tile_stage = -1;    // -1 = automatic; 0 / 1 = residual written straight to memory / staged through LDS
+    uint32_t tile_threads = 0; // 0 = automatic; else workgroup size of the tile kernels (64, 128, 256)
     uint32_t unq_slots = 0; // 0 = default; else bit positions per thread in unquantize
     int unq_force_scalar = 0;
 };
@@ -55,27 +56,32 @@ inline size_t qcol_bytes(size_t nbits, size_t rows)
     return 8 + ((rows * nbits + 31) / 32) * 4;
 }
 
-inline TileGeom make_tile_geom(size_t rows, size_t cols, size_t nbits, uint32_t gs_override, int stage = -1)
+inline TileGeom make_tile_geom(size_t rows, size_t cols, size_t nbits, uint32_t gs_override, int stage = -1,
+                               uint32_t threads_override = 0)
 {
     TileGeom t;
     t.rows = (uint32_t) rows;
     t.cols = (uint32_t) cols;
     t.nq = (uint32_t) qwords_per_col(rows, nbits);
+    uint32_t threads = threads_override != 0 ? threads_override : kTileThreads;
     uint32_t gs = 8;
     if (gs_override != 0)
         gs = gs_override;
     else
-        while (gs < kTileThreads && rows > (size_t) gs * 32)
+        while (gs < threads && rows > (size_t) gs * 32)
             gs <<= 1;
+    if (gs > threads)
+        gs = threads;
     // a tile may not exceed 4096 floats (16 KB) unless it is a single column: small tiles keep many
     // workgroups resident per CU, which is what hides the barrier-separated phases of each of them
-    while (gs < kTileThreads && (size_t) (kTileThreads / gs) * rows > 4096)
+    while (gs < threads && (size_t) (threads / gs) * rows > 4096)
         gs <<= 1;
+    t.threads = threads;
     t.gs = gs;
     t.gs_log2 = 0;
     while ((1u << t.gs_log2) < gs)
         t.gs_log2++;
-    t.cols_per_tile = kTileThreads / gs;
+    t.cols_per_tile = threads / gs;
     t.tile_floats = (uint32_t) (((size_t) t.cols_per_tile * rows + 4 + 3) & ~(size_t) 3);
     t.words_floats = (nbits <= 2) ? t.cols_per_tile * t.nq : 0;
     t.stage_residual = (stage < 0) ? 1u : (uint32_t) (stage != 0);
@@ -105,7 +111,7 @@ struct TileLauncher
     {
         const uint32_t tiles = (t.cols + t.cols_per_tile - 1) / t.cols_per_tile;
         const size_t lds = tile_lds_bytes(t, 0);
-        hipExtLaunchKernelGGL((quantize_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(kTileThreads), lds, s, ev.start, ev.stop, 0, g, r_in, r_out, q, t);
+        hipExtLaunchKernelGGL((quantize_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(t.threads), lds, s, ev.start, ev.stop, 0, g, r_in, r_out, q, t);
         return hipGetLastError();
     }
 };
@@ -130,7 +136,7 @@ struct StripeLauncher
     {
         const uint32_t tiles = (t.cols + t.cols_per_tile - 1) / t.cols_per_tile;
         const size_t lds = tile_lds_bytes(t, src.workers);
-        hipExtLaunchKernelGGL((stripe_reduce_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(kTileThreads), lds, s, ev.start, ev.stop, 0, src, stripe_res,
+        hipExtLaunchKernelGGL((stripe_reduce_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(t.threads), lds, s, ev.start, ev.stop, 0, src, stripe_res,
                            q_out, agg_out, t);
         return hipGetLastError();
     }
@@ -186,7 +192,7 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     {
         if (rows > kTileMaxRows)
             return hipErrorInvalidValue;
-        const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs, tune.tile_stage);
+        const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs, tune.tile_stage, tune.tile_threads);
         return dispatch_nbits<TileLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, t);
     }
     return dispatch_nbits<TallLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) rows, (uint32_t) cols,
@@ -200,6 +206,31 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
     zt = zt && (nbits == 1);
     if (rows > kTileMaxRows)
         return hipErrorInvalidValue;
+    bool aligned8 = (reinterpret_cast<uintptr_t>(q_out) & 7u) == 0;
+    for (uint32_t w = 0; w < src.workers; ++w)
+        aligned8 = aligned8 && (reinterpret_cast<uintptr_t>(src.q[w]) & 7u) == 0;
+    if (tune.quantize_path != kPathTile && nbits == 1 && (rows == 2048 || rows == 4096) && aligned8)
+    {
+        constexpr uint32_t per_block = kWaveColThreads / 64;
+        const uint32_t blocks = (uint32_t) ((cols + per_block - 1) / per_block);
+        const uint64_t qcol = qcol_bytes(nbits, rows);
+        char* qo = static_cast<char*>(q_out);
+        if (rows == 2048)
+        {
+            if (zt)
+                hipExtLaunchKernelGGL((stripe_reduce_wavecol_kernel<true, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, src, stripe_res, qo, agg_out, (uint32_t) cols, qcol);
+            else
+                hipExtLaunchKernelGGL((stripe_reduce_wavecol_kernel<false, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, src, stripe_res, qo, agg_out, (uint32_t) cols, qcol);
+        }
+        else
+        {
+            if (zt)
+                hipExtLaunchKernelGGL((stripe_reduce_wavecol_kernel<true, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, src, stripe_res, qo, agg_out, (uint32_t) cols, qcol);
+            else
+                hipExtLaunchKernelGGL((stripe_reduce_wavecol_kernel<false, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, src, stripe_res, qo, agg_out, (uint32_t) cols, qcol);
+        }
+        return hipGetLastError();
+    }
     // A stripe is small (one GPU's share of the columns), so the kernel is latency-bound: take the smallest
     // tile that still gives every thread of a workgroup a work item, to spread the stripe over all CUs.
     uint32_t gs = tune.tile_gs;
@@ -211,7 +242,7 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
         while (gs > 8 && items_per_col * (kTileThreads / gs) < kTileThreads)
             gs >>= 1;
     }
-    const TileGeom t = make_tile_geom(rows, cols, nbits, gs, tune.tile_stage);
+    const TileGeom t = make_tile_geom(rows, cols, nbits, gs, tune.tile_stage, tune.tile_threads);
     return dispatch_nbits<StripeLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, t);
 }
 

@@ -1,0 +1,203 @@
+// C++ test of the drop-in boundary through the host mirror classes, after the reference's own unit test
+// (Tests/UnitTests/MathTests/MatrixQuantizerTests.cpp:239-472): for every bit width and, at 1 bit, both threshold
+// modes, ten shapes x five iterations with the residual carried over and the output accumulated from the second
+// iteration on. The checker is the CPU oracle (oracle/liboracle.so), fed the very inputs the device saw.
+//
+// Checks per iteration, as in the reference test:
+//   * conservation:  in + prevResidual + prevOut == newResidual + newOut   within (hi - lo) * 1e-4       (:327-338)
+//   * output and residual against the CPU checker within the same tolerance, with at most
+//     max(1, 0.1 % of the elements) outliers ("may quantize to different integers")                     (:340-377)
+// and, stricter than the reference: under the headers the device produced, codes and residual must equal the
+// oracle's bit for bit, and unquantize must be bit-exact.
+#include "../../cntk_amd/cpp/MatrixQuantizer.h"
+#include "../../oracle/quantizer_oracle.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <random>
+#include <vector>
+
+using namespace cntk_amd;
+
+static int g_failures = 0;
+#define CHECK(cond, ...)                                                                                               \
+    do                                                                                                                 \
+    {                                                                                                                  \
+        if (!(cond))                                                                                                   \
+        {                                                                                                              \
+            if (g_failures < 20)                                                                                       \
+            {                                                                                                          \
+                std::fprintf(stderr, "CHECK failed %s:%d: %s  ", __FILE__, __LINE__, #cond);                         \
+                std::fprintf(stderr, __VA_ARGS__);                                                                     \
+                std::fprintf(stderr, "\n");                                                                            \
+            }                                                                                                          \
+            g_failures++;                                                                                              \
+        }                                                                                                              \
+    } while (0)
+
+static const float c_SinglePrecisionTolerance = 1e-4f;
+static const float c_SinglePrecisionGpuQuantizationTolerance = 1e-3f;
+
+static std::vector<float> RandomUniform(size_t rows, size_t cols, float lo, float hi, unsigned long seed)
+{
+    std::mt19937_64 rng(seed);
+    std::vector<float> a(rows * cols);
+    for (auto& x : a)
+        x = (float) (lo + (hi - lo) * ((rng() >> 11) * (1.0 / 9007199254740992.0)));
+    return a;
+}
+
+static void TestRunQuantization(size_t numBits, size_t numRows, size_t numCols, float rangeLow, float rangeHigh, int seed,
+                                int numIterations, int deviceId, bool zeroThresholdFor1Bit, bool hostQuantizedMatrix)
+{
+    Matrix<float> inMatrix(numRows, numCols, deviceId);
+    std::unique_ptr<MatrixQuantizerImpl<float>> quantizer(MatrixQuantizerImpl<float>::Create(deviceId, false /*useAsync*/));
+    Matrix<float> residueMatrix(numRows, numCols, deviceId);
+    Matrix<float> outMatrix(numRows, numCols, deviceId);
+    const size_t numMatrixElems = inMatrix.GetNumElements();
+
+    {
+        // the initial residue and output are all zeros
+        auto r = residueMatrix.CopyToArray(), o = outMatrix.CopyToArray();
+        for (size_t i = 0; i < numMatrixElems; ++i)
+            CHECK(r[i] == 0.0f && o[i] == 0.0f, "fresh matrices must be zero");
+    }
+
+    for (int iterNum = 0; iterNum < numIterations; ++iterNum)
+    {
+        std::vector<float> in = RandomUniform(numRows, numCols, rangeLow, rangeHigh, (unsigned long) (seed + iterNum));
+        inMatrix.SetValue(in.data());
+        auto prevResidual = residueMatrix.CopyToArray();
+        auto prevOut = outMatrix.CopyToArray();
+
+        QuantizedMatrix<float> tempQuantizationBuffer(numRows, numCols, numBits, hostQuantizedMatrix ? CPUDEVICE : deviceId);
+        quantizer->QuantizeAsync(inMatrix, residueMatrix, tempQuantizationBuffer, residueMatrix, zeroThresholdFor1Bit);
+        quantizer->WaitQuantizeAsyncDone();
+        quantizer->UnquantizeAsync(tempQuantizationBuffer, outMatrix, (iterNum > 0));
+        quantizer->WaitUnquantizeAsyncDone();
+
+        auto newResidual = residueMatrix.CopyToArray();
+        auto newOut = outMatrix.CopyToArray();
+        std::vector<char> packed = tempQuantizationBuffer.CopyToHost();
+
+        float tolerance = 0.0f;
+        if (numBits != 8 * sizeof(float))
+            tolerance = (rangeHigh - rangeLow) * c_SinglePrecisionTolerance;
+
+        for (size_t i = 0; i < numMatrixElems; ++i)
+            CHECK(std::fabs((in[i] + prevResidual[i] + prevOut[i]) - (newResidual[i] + newOut[i])) <= tolerance + 1e-6f * (rangeHigh - rangeLow),
+                  "conservation, element %zu", i);
+
+        const size_t numIncorrectAllowed = std::max<size_t>(1, (size_t) (numMatrixElems * c_SinglePrecisionGpuQuantizationTolerance));
+
+        // the CPU checker on the same inputs
+        std::vector<float> refResidual(numMatrixElems), refOut(prevOut.get(), prevOut.get() + numMatrixElems);
+        std::vector<char> refPacked(packed.size());
+        oracle_quantize(in.data(), prevResidual.get(), numRows, numCols, refPacked.data(), numBits, refResidual.data(), zeroThresholdFor1Bit, 1);
+        oracle_unquantize(refPacked.data(), numRows, numCols, numBits, refOut.data(), iterNum > 0, 1);
+        size_t numIncorrectOut = 0, numIncorrectResidual = 0;
+        for (size_t i = 0; i < numMatrixElems; ++i)
+        {
+            if (std::fabs(newOut[i] - refOut[i]) > tolerance && ++numIncorrectOut > numIncorrectAllowed)
+                CHECK(false, "output differs from the CPU checker at %zu: %g vs %g", i, newOut[i], refOut[i]);
+            if (std::fabs(newResidual[i] - refResidual[i]) > tolerance && ++numIncorrectResidual > numIncorrectAllowed)
+                CHECK(false, "residual differs from the CPU checker at %zu: %g vs %g", i, newResidual[i], refResidual[i]);
+        }
+
+        // stricter: bit-exact codes / residual under the device's own headers, bit-exact unquantize
+        std::vector<char> exactPacked(packed);
+        std::vector<float> exactResidual(numMatrixElems), exactOut(prevOut.get(), prevOut.get() + numMatrixElems);
+        oracle_pack_with_headers(in.data(), prevResidual.get(), numRows, numCols, exactPacked.data(), numBits, exactResidual.data(), zeroThresholdFor1Bit, 1);
+        CHECK(std::memcmp(exactPacked.data(), packed.data(), packed.size()) == 0, "codes under the device's headers");
+        CHECK(std::memcmp(exactResidual.data(), newResidual.get(), numMatrixElems * sizeof(float)) == 0, "residual under the device's headers");
+        oracle_unquantize(packed.data(), numRows, numCols, numBits, exactOut.data(), iterNum > 0, 1);
+        CHECK(std::memcmp(exactOut.data(), newOut.get(), numMatrixElems * sizeof(float)) == 0, "unquantize");
+    }
+}
+
+static void TestQuantization(int deviceId, size_t numRows, size_t numCols, float rangeLow, float rangeHigh, int seed, int numIterations)
+{
+    // all power-of-two bit widths; 1 bit with and without zeroThresholdFor1Bit
+    const size_t maxNumBits = 8 * sizeof(float);
+    for (size_t numBits = 1; numBits <= maxNumBits; numBits *= 2)
+        for (int i = 0; i < 2; ++i)
+        {
+            const bool zeroThresholdFor1Bit = (i == 1);
+            if (numBits != 1 && zeroThresholdFor1Bit)
+                continue;
+            for (int host = 0; host < 2; ++host)
+                TestRunQuantization(numBits, numRows, numCols, rangeLow, rangeHigh, seed, numIterations, deviceId, zeroThresholdFor1Bit, host != 0);
+        }
+}
+
+static void GPUMatrix1BitQuantizeFloat()
+{
+    const int dev = 0;
+    TestQuantization(dev, 25, 13, -1.0f, +1.0f, 2015, 5);
+    TestQuantization(dev, 25, 13, -0.005f, +0.005f, 2115, 5);
+    TestQuantization(dev, 13, 25, -0.00001f, +0.00001f, 2215, 5);
+    TestQuantization(dev, 13, 25, -10.0f, +10.0f, 2315, 5);
+    TestQuantization(dev, 25, 13, -1.0f, +2.05f, 2415, 5);
+    TestQuantization(dev, 489, 1, -0.5f, +0.5f, 2515, 5);
+    TestQuantization(dev, 1, 135, -0.5f, +0.5f, 2615, 5);
+    TestQuantization(dev, 89, 23, -0.5f, +0.5f, 2715, 5);
+    TestQuantization(dev, 15, 35, -0.5f, +0.5f, 2815, 5);
+    TestQuantization(dev, 100, 50, -0.5f, +0.5f, 2915, 5);
+    // the sizes the reference test was first written with (:474-487)
+    TestQuantization(dev, 256, 135, -1.0f, +2.05f, 2415, 5);
+    TestQuantization(dev, 737, 373, -0.5f, +0.5f, 2915, 5);
+    // the headline column height
+    TestQuantization(dev, 2048, 33, -0.02f, +0.03f, 3015, 3);
+}
+
+static void ErrorBehaviour()
+{
+    bool threw = false;
+    try { QuantizedMatrix<float> q(8, 8, 3, 0); } catch (const std::logic_error&) { threw = true; }
+    CHECK(threw, "nbits = 3 must be a logic error");
+    threw = false;
+    try { std::unique_ptr<MatrixQuantizerImpl<float>> q(MatrixQuantizerImpl<float>::Create(CPUDEVICE, false)); } catch (const std::runtime_error&) { threw = true; }
+    CHECK(threw, "no CPU quantizer");
+    std::unique_ptr<MatrixQuantizerImpl<float>> q(MatrixQuantizerImpl<float>::Create(0, true));
+    Matrix<float> a(8, 4, 0), b(8, 5, 0);
+    QuantizedMatrix<float> qa(8, 4, 1, 0);
+    threw = false;
+    try { q->QuantizeAsync(a, b, qa, a, false); } catch (const std::invalid_argument&) { threw = true; }
+    CHECK(threw, "dimension mismatch");
+    threw = false;
+    try { q->UnquantizeAsync(qa, b); } catch (const std::invalid_argument&) { threw = true; }
+    CHECK(threw, "dimension mismatch on unquantize");
+    CHECK(q->GetDeviceId() == 0, "device id");
+    // residual-owning wrapper: ResetResidue really clears
+    MatrixQuantizer<float> mq(64, 8, 0, true);
+    Matrix<float> g(64, 8, 0);
+    g.SetValue(0.25f);
+    QuantizedMatrix<float> qm(64, 8, 1, 0);
+    mq.QuantizeAsync(g, qm, true);
+    mq.WaitQuantizeAsyncDone();
+    mq.ResetResidue();
+    auto r = mq.GetResidualMatrix().CopyToArray();
+    for (size_t i = 0; i < 64 * 8; ++i)
+        CHECK(r[i] == 0.0f, "ResetResidue");
+}
+
+int main()
+{
+    try
+    {
+        GPUMatrix1BitQuantizeFloat();
+        std::printf("Test case GPUMatrixSuite/GPUMatrix1BitQuantizeFloat %s\n", g_failures ? "has FAILED" : "has passed");
+        const int before = g_failures;
+        ErrorBehaviour();
+        std::printf("Test case GPUMatrixSuite/QuantizerErrorBehaviour %s\n", g_failures != before ? "has FAILED" : "has passed");
+    }
+    catch (const std::exception& e)
+    {
+        std::fprintf(stderr, "unexpected exception: %s\n", e.what());
+        return 2;
+    }
+    std::fflush(stdout);
+    return g_failures ? 1 : 0;
+}
