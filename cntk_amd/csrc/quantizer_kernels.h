@@ -790,7 +790,9 @@ __global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict_
 
     const char* qc = q + (size_t) c * t.qcol;
     const float* gh = reinterpret_cast<const float*>(qc);
-    const ValueQ vq = make_vq<NBITS>(gh[0], gh[1]);
+    ValueQ vq; // decoding needs only the code -> value factor and the lower bound
+    vq.lo = gh[0];
+    vq.uf = make_ufactor<NBITS>(gh[0], gh[1]);
     const float val0 = unquantize_value<NBITS>(vq, 0u);
     const float val1 = unquantize_value<NBITS>(vq, 1u);
     const uint32_t* bits = reinterpret_cast<const uint32_t*>(qc + 8);
@@ -853,6 +855,74 @@ __global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict_
             if (add)
                 x = x + oc[i];
             oc[i] = x;
+        }
+    }
+}
+
+// Decoder with 16-byte stores for shapes the QWord-major decoder above can only serve with 4-byte stores
+// (nq or rows not a multiple of 4, e.g. 100000 rows -> 3125 QWords). For one column and one bit position k the
+// rows k * nq ... (k + 1) * nq - 1 are consecutive in memory: such a segment is cut into groups of four elements
+// aligned to 16 bytes in the OUTPUT (the first and last group of a segment may be partial and use 4-byte stores).
+struct UnqSegGeom
+{
+    uint32_t rows;
+    uint32_t nq;
+    uint32_t segs;    // bit positions in use per column: ceil(rows / nq)
+    uint32_t gps;     // groups per segment
+    uint32_t items;   // cols * segs * gps (the host refuses more than 2^32 - 1)
+    double inv_gps;
+    double inv_segs;
+    uint64_t qcol;
+};
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_segment_kernel(const char* __restrict__ q, float* out, UnqSegGeom t, int add)
+{
+    constexpr uint32_t SHIFT = NBITS & 31;
+    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
+    const uint64_t id64 = (uint64_t) blockIdx.x * 256 + threadIdx.x;
+    if (id64 >= t.items)
+        return;
+    uint32_t seg, g, c, k;
+    divmod_u32((uint32_t) id64, t.gps, t.inv_gps, seg, g);
+    divmod_u32(seg, t.segs, t.inv_segs, c, k);
+    const uint32_t row0 = k * t.nq;
+    const uint32_t seg_len = min(t.nq, t.rows - row0);
+    const size_t obase = (size_t) c * t.rows + row0;       // out is 16-byte aligned (checked by the host)
+    const int32_t first = (int32_t) (4u * g) - (int32_t) (obase & 3u); // QWord index of this group's first element
+    if (first >= (int32_t) seg_len)
+        return;
+
+    const char* qc = q + (size_t) c * t.qcol;
+    const float* gh = reinterpret_cast<const float*>(qc);
+    const float lo = gh[0];
+    const float uf = make_ufactor<NBITS>(lo, gh[1]);
+    const uint32_t* bits = reinterpret_cast<const uint32_t*>(qc + 8);
+    const uint32_t sh = k * SHIFT;
+    float* dst = out + obase;
+
+    if (first >= 0 && first + 3 < (int32_t) seg_len)
+    {
+        f32x4 v;
+        v.x = unquantize_value<NBITS>(uf, lo, (bits[first] >> sh) & CODEMASK);
+        v.y = unquantize_value<NBITS>(uf, lo, (bits[first + 1] >> sh) & CODEMASK);
+        v.z = unquantize_value<NBITS>(uf, lo, (bits[first + 2] >> sh) & CODEMASK);
+        v.w = unquantize_value<NBITS>(uf, lo, (bits[first + 3] >> sh) & CODEMASK);
+        f32x4* d4 = reinterpret_cast<f32x4*>(dst + first);
+        if (add)
+            v = v + *d4;
+        __builtin_nontemporal_store(v, d4);
+    }
+    else
+    {
+        for (int32_t e = 0; e < 4; ++e)
+        {
+            const int32_t w = first + e;
+            if (w >= 0 && w < (int32_t) seg_len)
+            {
+                const float x = unquantize_value<NBITS>(uf, lo, (bits[w] >> sh) & CODEMASK);
+                dst[w] = add ? x + dst[w] : x;
+            }
         }
     }
 }

@@ -274,6 +274,26 @@ inline hipError_t launch_unquantize_t(hipStream_t s, LaunchEvents ev, const char
     return hipGetLastError();
 }
 
+template <int NBITS>
+inline hipError_t launch_unquantize_segment_t(hipStream_t s, LaunchEvents ev, const char* q, float* out, size_t rows, size_t cols, int add)
+{
+    UnqSegGeom t;
+    t.rows = (uint32_t) rows;
+    t.nq = (uint32_t) qwords_per_col(rows, NBITS);
+    t.segs = (uint32_t) ((rows + t.nq - 1) / t.nq);
+    t.gps = (t.nq + 3 + 3) / 4;
+    const uint64_t items = (uint64_t) cols * t.segs * t.gps;
+    if (items > 0xFFFFFFFFull)
+        return hipErrorInvalidValue;
+    t.items = (uint32_t) items;
+    t.inv_gps = 1.0 / (double) t.gps;
+    t.inv_segs = 1.0 / (double) t.segs;
+    t.qcol = qcol_bytes(NBITS, rows);
+    const uint32_t blocks = (uint32_t) ((items + 255) / 256);
+    hipExtLaunchKernelGGL((unquantize_segment_kernel<NBITS>), dim3(blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, t, add);
+    return hipGetLastError();
+}
+
 inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* q, float* out, size_t rows, size_t cols, size_t nbits,
                                     bool add, const LaunchTuning& tune)
 {
@@ -283,6 +303,22 @@ inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* 
                      (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
     const int a = add ? 1 : 0;
     const uint32_t sl = tune.unq_slots;
+    // long columns that the QWord-major decoder could only serve with 4-byte stores go to the segment decoder
+    const bool seg = !vec && !tune.unq_force_scalar && (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && nq >= 32 &&
+                     (uint64_t) cols * (32 / nbits) * ((nq + 6) / 4) <= 0xFFFFFFFFull;
+    if (seg)
+    {
+        switch (nbits)
+        {
+        case 1: return launch_unquantize_segment_t<1>(s, ev, qc, out, rows, cols, a);
+        case 2: return launch_unquantize_segment_t<2>(s, ev, qc, out, rows, cols, a);
+        case 4: return launch_unquantize_segment_t<4>(s, ev, qc, out, rows, cols, a);
+        case 8: return launch_unquantize_segment_t<8>(s, ev, qc, out, rows, cols, a);
+        case 16: return launch_unquantize_segment_t<16>(s, ev, qc, out, rows, cols, a);
+        case 32: return launch_unquantize_segment_t<32>(s, ev, qc, out, rows, cols, a);
+        default: return hipErrorInvalidValue;
+        }
+    }
     switch (nbits)
     {
     case 1: return vec ? launch_unquantize_t<1, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<1, 1>(s, ev, qc, out, rows, cols, sl, a);

@@ -51,6 +51,38 @@ __device__ __forceinline__ ValueQ make_vq(float lo, float hi)
     return v;
 }
 
+// Only what decoding needs: the code -> value step of the same quantizer state (identical arithmetic to make_vq).
+template <int NBITS>
+__device__ __forceinline__ float make_ufactor(float lo, float hi)
+{
+    constexpr uint32_t rangeend = (NBITS >= 32) ? 0u : (1u << (NBITS & 31));
+    const float span = hi - lo;
+    if ((span < 1e-36f) || (rangeend == 0))
+        return 0.0f;
+    constexpr float used = (float) (rangeend - (NBITS > 1 ? 1u : 0u));
+    return span / used;
+}
+
+// x / d and x % d for 32-bit operands through one double-precision multiply by a host-computed reciprocal
+// (exact after the single correction step: the product is off by less than 2^-20).
+__device__ __forceinline__ void divmod_u32(uint32_t x, uint32_t d, double inv_d, uint32_t& quot, uint32_t& rem)
+{
+    uint32_t qv = (uint32_t) ((double) x * inv_d);
+    uint32_t r = x - qv * d;
+    if ((int32_t) r < 0)
+    {
+        qv--;
+        r += d;
+    }
+    else if (r >= d)
+    {
+        qv++;
+        r -= d;
+    }
+    quot = qv;
+    rem = r;
+}
+
 // Source/Math/ValueQuantizer.h:101-128, 144-156
 template <int NBITS, bool ZT>
 __device__ __forceinline__ uint32_t quantize_value(const ValueQ& v, float u)

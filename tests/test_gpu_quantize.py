@@ -168,7 +168,8 @@ def test_wavefront_per_column_path(rows):
 
 def test_unquantize_variants(quantizer):
     """Scalar and 16-byte-store decoders, every slot split, add and overwrite: all bit-exact."""
-    for rows, cols in [(5, 3), (37, 2), (128, 9), (429, 5), (2048, 6), (4100, 2)]:
+    # QWord-major decoder with 16-byte stores, its 4-byte variant, and the segment decoder for long odd columns
+    for rows, cols in [(5, 3), (37, 2), (128, 9), (429, 5), (2048, 6), (4100, 2), (1001, 5), (3003, 3), (100000, 2)]:
         for nbits, zt in VARIANTS:
             g = datagen.normal(rows * 7 + nbits, rows, cols)
             q, _ = oracle.quantize(g, np.zeros_like(g, order="F"), nbits, zt)
