@@ -35,6 +35,14 @@ class QuantizerLogicError(ValueError):
     """LogicError / InvalidArgument of the reference (bad nbits, mismatching sizes)."""
 
 
+class _QuantizeItem(ctypes.Structure):
+    _fields_ = [("in_", _vp), ("res_in", _vp), ("res_out", _vp), ("qbuf", _vp), ("rows", _sz), ("cols", _sz)]
+
+
+class _UnquantizeItem(ctypes.Structure):
+    _fields_ = [("qbuf", _vp), ("out", _vp), ("rows", _sz), ("cols", _sz)]
+
+
 def lib():
     """The loaded C-ABI library. Raises if it has not been built (python -m cntk_amd.build)."""
     global _lib
@@ -65,6 +73,8 @@ def lib():
         L.cntkq_stripe_reduce_async.argtypes = [_vp, ctypes.POINTER(_vp), _sz, _sz, _sz, _sz, _sz, _vp, _vp, _vp,
                                                 ctypes.c_int]
         L.cntkq_wait_stripe_reduce_done.argtypes = [_vp]
+        L.cntkq_quantize_batch_async.argtypes = [_vp, ctypes.POINTER(_QuantizeItem), _sz, _sz, ctypes.c_int]
+        L.cntkq_unquantize_batch_async.argtypes = [_vp, ctypes.POINTER(_UnquantizeItem), _sz, _sz, ctypes.c_int]
         L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int]
         _lib = L
     return _lib
@@ -261,6 +271,39 @@ class MatrixQuantizerImpl:
 
     def WaitUnquantizeAsyncDone(self):
         _check(lib().cntkq_wait_unquantize_done(self._h))
+
+    def QuantizeBatchAsync(self, items, zero_threshold_for_1bit):
+        """The aggregator's loop over its gradient matrices as one call (Source/1BitSGD/AllReduceDistGradAggregator.h:288-300).
+        items: sequence of (in_matrix, in_residual, out_qmatrix, out_residual); all packed matrices on the device and of
+        one bit width."""
+        if not items:
+            return
+        nbits = items[0][2].GetNumBits()
+        arr = (_QuantizeItem * len(items))()
+        for k, (g, r_in, q, r_out) in enumerate(items):
+            rows, cols = g.GetNumRows(), g.GetNumCols()
+            for m in (r_in, r_out, q):
+                if m.GetNumRows() != rows or m.GetNumCols() != cols:
+                    raise QuantizerLogicError("QuantizeBatchAsync: matrix dimensions do not match")
+            if q.GetNumBits() != nbits or q.GetDeviceId() < 0:
+                raise QuantizerLogicError("QuantizeBatchAsync: packed matrices must share one bit width and live on the device")
+            arr[k] = _QuantizeItem(g.Data(), r_in.Data(), r_out.Data(), q.Buffer(), rows, cols)
+        _check(lib().cntkq_quantize_batch_async(self._h, arr, len(items), nbits, int(bool(zero_threshold_for_1bit))))
+
+    def UnquantizeBatchAsync(self, items, add=False):
+        """The aggregator's final loop (Source/1BitSGD/AllReduceDistGradAggregator.h:517-522) as one call.
+        items: sequence of (in_qmatrix, out_matrix)."""
+        if not items:
+            return
+        nbits = items[0][0].GetNumBits()
+        arr = (_UnquantizeItem * len(items))()
+        for k, (q, out) in enumerate(items):
+            if q.GetNumRows() != out.GetNumRows() or q.GetNumCols() != out.GetNumCols():
+                raise QuantizerLogicError("UnquantizeBatchAsync: matrix dimensions do not match")
+            if q.GetNumBits() != nbits or q.GetDeviceId() < 0:
+                raise QuantizerLogicError("UnquantizeBatchAsync: packed matrices must share one bit width and live on the device")
+            arr[k] = _UnquantizeItem(q.Buffer(), out.Data(), out.GetNumRows(), out.GetNumCols())
+        _check(lib().cntkq_unquantize_batch_async(self._h, arr, len(items), nbits, int(bool(add))))
 
     def StripeReduceAsync(self, stripes, owner, stripe_residual, out_qstripe, zero_threshold_for_1bit, agg_out=None):
         """Fused stripe reduction of the quantized all-reduce (dataflow of

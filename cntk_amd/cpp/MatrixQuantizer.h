@@ -293,6 +293,55 @@ public:
     }
     void WaitUnquantizeAsyncDone() override { detail::Check(cntkq_wait_unquantize_done(m_handle)); }
 
+    // A whole gradient set per call: the aggregator's loops over its matrices
+    // (Source/1BitSGD/AllReduceDistGradAggregator.h:288-300 and :517-522) as one launch each.
+    struct QuantizeItem
+    {
+        const Matrix<ElemType>* inMatrix;
+        const Matrix<ElemType>* inResidual;
+        QuantizedMatrix<ElemType>* outQMatrix;
+        Matrix<ElemType>* outResidual;
+    };
+    void QuantizeBatchAsync(const std::vector<QuantizeItem>& items, bool zeroThresholdFor1Bit)
+    {
+        if (items.empty())
+            return;
+        const size_t nbits = items[0].outQMatrix->GetNumBits();
+        std::vector<cntkq_quantize_item> raw;
+        for (const auto& it : items)
+        {
+            const size_t rows = it.inMatrix->GetNumRows(), cols = it.inMatrix->GetNumCols();
+            if (it.outQMatrix->GetNumRows() != rows || it.outQMatrix->GetNumCols() != cols || it.inResidual->GetNumRows() != rows ||
+                it.inResidual->GetNumCols() != cols || it.outResidual->GetNumRows() != rows || it.outResidual->GetNumCols() != cols)
+                throw std::invalid_argument("QuantizeBatchAsync: matrix dimensions do not match");
+            if (it.outQMatrix->GetNumBits() != nbits || it.outQMatrix->GetDeviceId() < 0)
+                throw std::invalid_argument("QuantizeBatchAsync: packed matrices must share one bit width and live on the device");
+            raw.push_back(cntkq_quantize_item{it.inMatrix->Data(), it.inResidual->Data(), it.outResidual->Data(), it.outQMatrix->Buffer(), rows, cols});
+        }
+        detail::Check(cntkq_quantize_batch_async(m_handle, raw.data(), raw.size(), nbits, zeroThresholdFor1Bit ? 1 : 0));
+    }
+    struct UnquantizeItem
+    {
+        const QuantizedMatrix<ElemType>* inQMatrix;
+        Matrix<ElemType>* outMatrix;
+    };
+    void UnquantizeBatchAsync(const std::vector<UnquantizeItem>& items, bool add = false)
+    {
+        if (items.empty())
+            return;
+        const size_t nbits = items[0].inQMatrix->GetNumBits();
+        std::vector<cntkq_unquantize_item> raw;
+        for (const auto& it : items)
+        {
+            if (it.inQMatrix->GetNumRows() != it.outMatrix->GetNumRows() || it.inQMatrix->GetNumCols() != it.outMatrix->GetNumCols())
+                throw std::invalid_argument("UnquantizeBatchAsync: matrix dimensions do not match");
+            if (it.inQMatrix->GetNumBits() != nbits || it.inQMatrix->GetDeviceId() < 0)
+                throw std::invalid_argument("UnquantizeBatchAsync: packed matrices must share one bit width and live on the device");
+            raw.push_back(cntkq_unquantize_item{it.inQMatrix->Buffer(), it.outMatrix->Data(), it.outMatrix->GetNumRows(), it.outMatrix->GetNumCols()});
+        }
+        detail::Check(cntkq_unquantize_batch_async(m_handle, raw.data(), raw.size(), nbits, add ? 1 : 0));
+    }
+
     // Fused stripe reduction of the quantized all-reduce (dataflow of Source/1BitSGD/AllReduceDistGradAggregator.h:365-436):
     // stripes[w] is worker w's packed stripe; the requantized aggregate goes to outQStripe (may be stripes[owner]).
     void StripeReduceAsync(const std::vector<const QuantizedMatrix<ElemType>*>& stripes, size_t owner, Matrix<ElemType>& stripeResidual,

@@ -98,6 +98,15 @@ struct cntkq_quantizer
     bool staging_read_pending = false; // a kernel reading the staging buffer may still be running
     char* staging = nullptr;      // device buffer used when the packed matrix lives in host memory
     size_t staging_bytes = 0;
+    // entry tables of batched launches: a ring of slots, each with a pinned host copy and a device copy; a slot is
+    // reused only after the last kernel that read it has finished (its event)
+    static constexpr int kBatchSlots = 4;
+    char* batch_host = nullptr;
+    char* batch_dev = nullptr;
+    size_t batch_slot_bytes = 0;
+    int batch_next = 0;
+    hipEvent_t batch_event[kBatchSlots] = {nullptr, nullptr, nullptr, nullptr};
+    bool batch_used[kBatchSlots] = {false, false, false, false};
     LaunchTuning tune;
 };
 
@@ -140,6 +149,40 @@ int ensure_staging(cntkq_quantizer* h, size_t bytes)
     HIP_TRY(hipMalloc(&p, bytes), "hipMalloc of the packed staging buffer failed");
     h->staging = static_cast<char*>(p);
     h->staging_bytes = bytes;
+    return CNTKQ_OK;
+}
+
+// Makes a table slot of at least `bytes` available for writing; returns its index.
+int acquire_batch_slot(cntkq_quantizer* h, size_t bytes, int* slot_out)
+{
+    if (bytes > h->batch_slot_bytes)
+    {
+        for (int i = 0; i < cntkq_quantizer::kBatchSlots; ++i)
+            if (h->batch_used[i])
+                HIP_TRY(hipEventSynchronize(h->batch_event[i]), "hipEventSynchronize failed");
+        if (h->batch_host != nullptr)
+            HIP_TRY(hipHostFree(h->batch_host), "hipHostFree failed");
+        if (h->batch_dev != nullptr)
+            HIP_TRY(hipFree(h->batch_dev), "hipFree failed");
+        h->batch_host = h->batch_dev = nullptr;
+        const size_t slot = (bytes * 2 + 4095) & ~(size_t) 4095;
+        void* p = nullptr;
+        HIP_TRY(hipHostMalloc(&p, slot * cntkq_quantizer::kBatchSlots, hipHostMallocDefault), "hipHostMalloc of the batch table failed");
+        h->batch_host = static_cast<char*>(p);
+        HIP_TRY(hipMalloc(&p, slot * cntkq_quantizer::kBatchSlots), "hipMalloc of the batch table failed");
+        h->batch_dev = static_cast<char*>(p);
+        h->batch_slot_bytes = slot;
+        for (int i = 0; i < cntkq_quantizer::kBatchSlots; ++i)
+            h->batch_used[i] = false;
+    }
+    const int slot = h->batch_next;
+    h->batch_next = (slot + 1) % cntkq_quantizer::kBatchSlots;
+    if (h->batch_event[slot] == nullptr)
+        HIP_TRY(hipEventCreateWithFlags(&h->batch_event[slot], hipEventDisableTiming), "hipEventCreateWithFlags failed");
+    if (h->batch_used[slot])
+        HIP_TRY(hipEventSynchronize(h->batch_event[slot]), "hipEventSynchronize failed");
+    h->batch_used[slot] = true;
+    *slot_out = slot;
     return CNTKQ_OK;
 }
 
@@ -262,6 +305,19 @@ int cntkq_destroy(cntkq_quantizer* h)
     if (h->ev_stripe) (void) hipEventSynchronize(h->ev_stripe);
     if (h->staging != nullptr)
         (void) hipFree(h->staging);
+    for (int i = 0; i < cntkq_quantizer::kBatchSlots; ++i)
+    {
+        if (h->batch_event[i] != nullptr)
+        {
+            if (h->batch_used[i])
+                (void) hipEventSynchronize(h->batch_event[i]);
+            (void) hipEventDestroy(h->batch_event[i]);
+        }
+    }
+    if (h->batch_host != nullptr)
+        (void) hipHostFree(h->batch_host);
+    if (h->batch_dev != nullptr)
+        (void) hipFree(h->batch_dev);
     hipEvent_t evs[] = {h->ev_quantize, h->ev_fetch, h->ev_assign, h->ev_unquantize, h->ev_stripe, h->ev_main};
     for (hipEvent_t e : evs)
         if (e != nullptr)
@@ -420,6 +476,207 @@ int cntkq_wait_unquantize_done(cntkq_quantizer* h)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_wait_unquantize_done: null handle");
     DeviceGuard guard(h->device);
     return h->last_unquantize != nullptr ? sync_event(h->last_unquantize) : CNTKQ_OK;
+}
+
+int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* items, size_t count, size_t nbits,
+                               int zero_threshold_for_1bit)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: null handle");
+    if (!valid_nbits(nbits))
+        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
+    if (count == 0)
+        return CNTKQ_OK;
+    if (items == nullptr || count > 0xFFFFFF)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: bad item list");
+    for (size_t i = 0; i < count; ++i)
+    {
+        const cntkq_quantize_item& it = items[i];
+        if (it.rows >= (1ull << 31) || it.cols >= (1ull << 31))
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: item %zu: rows and cols must be below 2^31", i);
+        if (it.rows == 0 || it.cols == 0)
+            continue;
+        if (it.in == nullptr || it.res_in == nullptr || it.res_out == nullptr || it.qbuf == nullptr || !aligned4(it.in) ||
+            !aligned4(it.res_in) || !aligned4(it.res_out) || !aligned4(it.qbuf))
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: item %zu: null or misaligned pointer", i);
+    }
+    const bool zt = zero_threshold_for_1bit != 0;
+    DeviceGuard guard(h->device);
+    hipStream_t s = work_stream(h);
+
+    // small-LDS tiles, large-LDS tiles (one launch each), and matrices that get a launch of their own
+    constexpr size_t kSmallLds = 20 * 1024;
+    size_t n_tile[2] = {0, 0};
+    for (size_t i = 0; i < count; ++i)
+    {
+        const cntkq_quantize_item& it = items[i];
+        if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.qbuf, it.rows, nbits) != kPathTile)
+            continue;
+        const TileGeom t = make_tile_geom(it.rows, it.cols, nbits, 0, -1, 0);
+        n_tile[tile_lds_bytes(t, 0) <= kSmallLds ? 0 : 1]++;
+    }
+    const size_t n_tiles_total = n_tile[0] + n_tile[1];
+    hipEvent_t done = h->ev_quantize;
+    size_t launches_left = (n_tile[0] ? 1 : 0) + (n_tile[1] ? 1 : 0);
+    for (size_t i = 0; i < count; ++i)
+        if (items[i].rows != 0 && items[i].cols != 0 && quantize_auto_path(items[i].qbuf, items[i].rows, nbits) != kPathTile)
+            launches_left++;
+    if (launches_left == 0)
+        return CNTKQ_OK;
+
+    if (n_tiles_total != 0)
+    {
+        const size_t entries_bytes = n_tiles_total * sizeof(QuantizeBatchEntry);
+        const size_t begins_bytes = (n_tiles_total + 2) * sizeof(uint32_t);
+        int slot = 0;
+        int rc = acquire_batch_slot(h, entries_bytes + begins_bytes + 64, &slot);
+        if (rc != CNTKQ_OK)
+            return rc;
+        done = h->batch_event[slot];
+        char* host = h->batch_host + (size_t) slot * h->batch_slot_bytes;
+        char* dev = h->batch_dev + (size_t) slot * h->batch_slot_bytes;
+        QuantizeBatchEntry* he = reinterpret_cast<QuantizeBatchEntry*>(host);
+        uint32_t* hb = reinterpret_cast<uint32_t*>(host + entries_bytes);
+        size_t lds[2] = {0, 0};
+        uint32_t total_tiles[2] = {0, 0};
+        size_t e = 0, bpos = 0;
+        size_t first_entry[2] = {0, 0}, first_begin[2] = {0, 0};
+        for (int cls = 0; cls < 2; ++cls)
+        {
+            first_entry[cls] = e;
+            first_begin[cls] = bpos;
+            uint64_t tiles_acc = 0;
+            for (size_t i = 0; i < count; ++i)
+            {
+                const cntkq_quantize_item& it = items[i];
+                if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.qbuf, it.rows, nbits) != kPathTile)
+                    continue;
+                const TileGeom t = make_tile_geom(it.rows, it.cols, nbits, 0, -1, 0);
+                const size_t l = tile_lds_bytes(t, 0);
+                if ((l <= kSmallLds ? 0 : 1) != cls)
+                    continue;
+                he[e].g = it.in;
+                he[e].r_in = it.res_in;
+                he[e].r_out = it.res_out;
+                he[e].q = static_cast<char*>(it.qbuf);
+                he[e].t = t;
+                hb[bpos++] = (uint32_t) tiles_acc;
+                tiles_acc += (t.cols + t.cols_per_tile - 1) / t.cols_per_tile;
+                if (tiles_acc > 0x7FFFFFFFull)
+                    return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: too many tiles in one batch");
+                if (l > lds[cls])
+                    lds[cls] = l;
+                e++;
+            }
+            if (n_tile[cls] != 0)
+                hb[bpos++] = (uint32_t) tiles_acc; // sentinel
+            total_tiles[cls] = (uint32_t) tiles_acc;
+        }
+        HIP_TRY(hipMemcpyAsync(dev, host, entries_bytes + bpos * sizeof(uint32_t), hipMemcpyHostToDevice, s), "hipMemcpyAsync of the batch table failed");
+        for (int cls = 0; cls < 2; ++cls)
+        {
+            if (n_tile[cls] == 0)
+                continue;
+            LaunchEvents ev;
+            launches_left--;
+            ev.stop = launches_left == 0 ? done : nullptr;
+            const QuantizeBatchEntry* de = reinterpret_cast<const QuantizeBatchEntry*>(dev) + first_entry[cls];
+            const uint32_t* db = reinterpret_cast<const uint32_t*>(dev + entries_bytes) + first_begin[cls];
+            HIP_TRY(launch_quantize_tile_batch(s, ev, de, db, (uint32_t) n_tile[cls], total_tiles[cls], lds[cls], nbits, zt),
+                    "batched quantize kernel launch failed");
+        }
+        if (launches_left != 0)
+        {
+            // the table slot is guarded by its own event, which the LAST kernel of the batch will carry; the kernels
+            // in between run on the same stream, so they are finished by then as well
+        }
+    }
+    LaunchTuning autotune;
+    for (size_t i = 0; i < count; ++i)
+    {
+        const cntkq_quantize_item& it = items[i];
+        if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.qbuf, it.rows, nbits) == kPathTile)
+            continue;
+        LaunchEvents ev;
+        launches_left--;
+        ev.stop = launches_left == 0 ? done : nullptr;
+        HIP_TRY(launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune),
+                "quantize kernel launch failed");
+    }
+    h->last_quantize = done;
+    h->quantize_included_fetch = false;
+    return CNTKQ_OK;
+}
+
+int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item* items, size_t count, size_t nbits, int add)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: null handle");
+    if (!valid_nbits(nbits))
+        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
+    if (count == 0)
+        return CNTKQ_OK;
+    if (items == nullptr || count > 0xFFFFFF)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: bad item list");
+    size_t n = 0;
+    for (size_t i = 0; i < count; ++i)
+    {
+        const cntkq_unquantize_item& it = items[i];
+        if (it.rows >= (1ull << 31) || it.cols >= (1ull << 31))
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: item %zu: rows and cols must be below 2^31", i);
+        if (it.rows == 0 || it.cols == 0)
+            continue;
+        if (it.qbuf == nullptr || it.out == nullptr || !aligned4(it.qbuf) || !aligned4(it.out))
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: item %zu: null or misaligned pointer", i);
+        n++;
+    }
+    if (n == 0)
+        return CNTKQ_OK;
+    DeviceGuard guard(h->device);
+    hipStream_t s = work_stream(h);
+    const size_t entries_bytes = n * sizeof(UnquantizeBatchEntry);
+    int slot = 0;
+    int rc = acquire_batch_slot(h, entries_bytes + (n + 1) * sizeof(uint32_t) + 64, &slot);
+    if (rc != CNTKQ_OK)
+        return rc;
+    char* host = h->batch_host + (size_t) slot * h->batch_slot_bytes;
+    char* dev = h->batch_dev + (size_t) slot * h->batch_slot_bytes;
+    UnquantizeBatchEntry* he = reinterpret_cast<UnquantizeBatchEntry*>(host);
+    uint32_t* hb = reinterpret_cast<uint32_t*>(host + entries_bytes);
+    LaunchTuning autotune;
+    uint64_t blocks = 0;
+    size_t e = 0;
+    for (size_t i = 0; i < count; ++i)
+    {
+        const cntkq_unquantize_item& it = items[i];
+        if (it.rows == 0 || it.cols == 0)
+            continue;
+        const UnquantizePlan p = plan_unquantize(it.qbuf, it.out, it.rows, it.cols, nbits, autotune);
+        if (!p.ok)
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: item %zu is too large", i);
+        he[e].q = static_cast<const char*>(it.qbuf);
+        he[e].out = it.out;
+        he[e].kind = p.kind;
+        he[e].pad = 0;
+        he[e].qw = p.qw;
+        he[e].seg = p.seg;
+        hb[e] = (uint32_t) blocks;
+        blocks += p.blocks;
+        if (blocks > 0x7FFFFFFFull)
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: too much work in one batch");
+        e++;
+    }
+    hb[e] = (uint32_t) blocks;
+    HIP_TRY(hipMemcpyAsync(dev, host, entries_bytes + (n + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, s),
+            "hipMemcpyAsync of the batch table failed");
+    LaunchEvents ev;
+    ev.stop = h->batch_event[slot];
+    HIP_TRY(launch_unquantize_batch(s, ev, reinterpret_cast<const UnquantizeBatchEntry*>(dev),
+                                    reinterpret_cast<const uint32_t*>(dev + entries_bytes), (uint32_t) n, (uint32_t) blocks, nbits,
+                                    add != 0),
+            "batched unquantize kernel launch failed");
+    h->last_unquantize = ev.stop;
+    return CNTKQ_OK;
 }
 
 int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows,

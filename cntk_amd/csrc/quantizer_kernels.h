@@ -242,8 +242,8 @@ __device__ __forceinline__ void tile_store(const float* tile, uint32_t mis, floa
 // ---- quantize: gradient + residual -> packed codes + new residual -----------------------------------
 
 template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float* __restrict__ g, const float* r_in,
-                                                                     float* r_out, char* __restrict__ q, TileGeom t)
+__device__ __forceinline__ void quantize_tile_body(const float* __restrict__ g, const float* r_in, float* r_out,
+                                                   char* __restrict__ q, const TileGeom& t, uint32_t tile_index)
 {
     extern __shared__ f32x4 smem_v4[];
     float* smem = reinterpret_cast<float*>(smem_v4);
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float
     uint32_t* words = reinterpret_cast<uint32_t*>(smem + kTilePrefixFloats + t.tile_floats);
 
     const uint32_t tid = threadIdx.x;
-    const uint32_t j0 = blockIdx.x * t.cols_per_tile;
+    const uint32_t j0 = tile_index * t.cols_per_tile;
     const uint32_t nc = min(t.cols_per_tile, t.cols - j0);
     const size_t base = (size_t) j0 * t.rows;
     const uint32_t total = nc * t.rows;
@@ -317,6 +317,49 @@ __global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float
     tile_pack<NBITS, ZT>(tile, hdr, words, t, nc, qtile, r_out + base);
     if (t.stage_residual)
         tile_store(tile, mis_g, r_out + base, total, t);
+}
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float* __restrict__ g, const float* r_in,
+                                                                     float* r_out, char* __restrict__ q, TileGeom t)
+{
+    quantize_tile_body<NBITS, ZT>(g, r_in, r_out, q, t, blockIdx.x);
+}
+
+// Many matrices in one launch: the tiles of all matrices form one grid; `begins` (count + 1 entries, ascending)
+// gives the first tile of every matrix. Removes the per-launch floor (several microseconds) that dominates
+// gradient sets made of many small matrices.
+struct QuantizeBatchEntry
+{
+    const float* g;
+    const float* r_in;
+    float* r_out;
+    char* q;
+    TileGeom t;
+};
+
+// largest e with begins[e] <= b; b and everything derived from it is uniform over the workgroup
+__device__ __forceinline__ uint32_t batch_find(const uint32_t* __restrict__ begins, uint32_t count, uint32_t b)
+{
+    uint32_t lo = 0, hi = count;
+    while (hi - lo > 1)
+    {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (begins[mid] <= b)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    return lo;
+}
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTileThreads) void quantize_tile_batch_kernel(const QuantizeBatchEntry* __restrict__ entries,
+                                                                           const uint32_t* __restrict__ begins, uint32_t count)
+{
+    const uint32_t e = batch_find(begins, count, blockIdx.x);
+    const QuantizeBatchEntry en = entries[e];
+    quantize_tile_body<NBITS, ZT>(en.g, en.r_in, en.r_out, en.q, en.t, blockIdx.x - begins[e]);
 }
 
 // ---- stripe reduction: K packed stripes -> fp32 sum -> requantize with the stripe residual ----------
@@ -772,13 +815,13 @@ struct UnqGeom
 };
 
 template <int NBITS, int WV>
-__global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, float* out, UnqGeom t, int add)
+__device__ __forceinline__ void unquantize_body(const char* __restrict__ q, float* out, const UnqGeom& t, int add, uint32_t block)
 {
     constexpr uint32_t VPW = 32 / NBITS;
     constexpr uint32_t MASKBITS = NBITS & 31;
     constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << MASKBITS) - 1u);
 
-    const uint64_t id64 = (uint64_t) blockIdx.x * 256 + threadIdx.x;
+    const uint64_t id64 = (uint64_t) block * 256 + threadIdx.x;
     if (id64 >= t.items)
         return;
     const uint32_t id = (uint32_t) id64;
@@ -859,6 +902,12 @@ __global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict_
     }
 }
 
+template <int NBITS, int WV>
+__global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, float* out, UnqGeom t, int add)
+{
+    unquantize_body<NBITS, WV>(q, out, t, add, blockIdx.x);
+}
+
 // Decoder with 16-byte stores for shapes the QWord-major decoder above can only serve with 4-byte stores
 // (nq or rows not a multiple of 4, e.g. 100000 rows -> 3125 QWords). For one column and one bit position k the
 // rows k * nq ... (k + 1) * nq - 1 are consecutive in memory: such a segment is cut into groups of four elements
@@ -876,11 +925,12 @@ struct UnqSegGeom
 };
 
 template <int NBITS>
-__global__ __launch_bounds__(256) void unquantize_segment_kernel(const char* __restrict__ q, float* out, UnqSegGeom t, int add)
+__device__ __forceinline__ void unquantize_segment_body(const char* __restrict__ q, float* out, const UnqSegGeom& t, int add,
+                                                        uint32_t block)
 {
     constexpr uint32_t SHIFT = NBITS & 31;
     constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
-    const uint64_t id64 = (uint64_t) blockIdx.x * 256 + threadIdx.x;
+    const uint64_t id64 = (uint64_t) block * 256 + threadIdx.x;
     if (id64 >= t.items)
         return;
     uint32_t seg, g, c, k;
@@ -925,6 +975,45 @@ __global__ __launch_bounds__(256) void unquantize_segment_kernel(const char* __r
             }
         }
     }
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_segment_kernel(const char* __restrict__ q, float* out, UnqSegGeom t, int add)
+{
+    unquantize_segment_body<NBITS>(q, out, t, add, blockIdx.x);
+}
+
+// Many matrices in one launch (see quantize_tile_batch_kernel): the 256-thread blocks of all matrices form one grid.
+enum UnqKind : uint32_t
+{
+    kUnqVec4 = 0,   // QWord-major, 16-byte stores
+    kUnqScalar = 1, // QWord-major, 4-byte stores
+    kUnqSegment = 2 // segment decoder
+};
+
+struct UnquantizeBatchEntry
+{
+    const char* q;
+    float* out;
+    uint32_t kind;
+    uint32_t pad;
+    UnqGeom qw;     // valid for kUnqVec4 / kUnqScalar
+    UnqSegGeom seg; // valid for kUnqSegment
+};
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_batch_kernel(const UnquantizeBatchEntry* __restrict__ entries,
+                                                               const uint32_t* __restrict__ begins, uint32_t count, int add)
+{
+    const uint32_t e = batch_find(begins, count, blockIdx.x);
+    const UnquantizeBatchEntry& en = entries[e];
+    const uint32_t block = blockIdx.x - begins[e];
+    if (en.kind == kUnqVec4)
+        unquantize_body<NBITS, 4>(en.q, en.out, en.qw, add, block);
+    else if (en.kind == kUnqScalar)
+        unquantize_body<NBITS, 1>(en.q, en.out, en.qw, add, block);
+    else
+        unquantize_segment_body<NBITS>(en.q, en.out, en.seg, add, block);
 }
 
 } // namespace cntkq

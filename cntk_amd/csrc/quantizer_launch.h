@@ -8,6 +8,8 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <string.h>
+#include <cstring>
 
 namespace cntkq {
 
@@ -246,89 +248,156 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
     return dispatch_nbits<StripeLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, t);
 }
 
-template <int NBITS, int WV>
-inline hipError_t launch_unquantize_t(hipStream_t s, LaunchEvents ev, const char* q, float* out, size_t rows, size_t cols, uint32_t slots,
-                                      int add)
+// ---- unquantize: which decoder, with which geometry ---------------------------------------------------
+
+struct UnquantizePlan
 {
-    constexpr uint32_t VPW = 32 / NBITS;
-    UnqGeom t;
+    uint32_t kind = kUnqScalar;
+    UnqGeom qw;
+    UnqSegGeom seg;
+    uint32_t blocks = 0; // 256-thread blocks
+    bool ok = false;
+};
+
+inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t rows, size_t cols, size_t nbits,
+                                      const LaunchTuning& tune)
+{
+    UnquantizePlan p;
+    std::memset(&p.qw, 0, sizeof p.qw);
+    std::memset(&p.seg, 0, sizeof p.seg);
+    const size_t vpw = 32 / nbits;
+    const size_t nq = qwords_per_col(rows, nbits);
+    const bool out16 = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    const bool vec = !tune.unq_force_scalar && (nq % 4 == 0) && (rows % 4 == 0) && out16 &&
+                     (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
+    // long columns that the QWord-major decoder could only serve with 4-byte stores go to the segment decoder
+    const bool seg = !vec && !tune.unq_force_scalar && out16 && nq >= 32;
+    if (seg)
+    {
+        UnqSegGeom& t = p.seg;
+        t.rows = (uint32_t) rows;
+        t.nq = (uint32_t) nq;
+        t.segs = (uint32_t) ((rows + nq - 1) / nq);
+        t.gps = (uint32_t) ((nq + 3 + 3) / 4);
+        const uint64_t items = (uint64_t) cols * t.segs * t.gps;
+        if (items <= 0xFFFFFFFFull)
+        {
+            t.items = (uint32_t) items;
+            t.inv_gps = 1.0 / (double) t.gps;
+            t.inv_segs = 1.0 / (double) t.segs;
+            t.qcol = qcol_bytes(nbits, rows);
+            p.kind = kUnqSegment;
+            p.blocks = (uint32_t) ((items + 255) / 256);
+            p.ok = true;
+            return p;
+        }
+    }
+    const uint32_t wv = vec ? 4 : 1;
+    UnqGeom& t = p.qw;
     t.rows = (uint32_t) rows;
     t.cols = (uint32_t) cols;
-    t.nq = (uint32_t) qwords_per_col(rows, NBITS);
-    t.groups = (t.nq + WV - 1) / WV;
+    t.nq = (uint32_t) nq;
+    t.groups = (uint32_t) ((nq + wv - 1) / wv);
+    uint32_t slots = tune.unq_slots;
     if (slots == 0)
-        slots = VPW < 2 ? VPW : 2;
-    if (slots > VPW)
-        slots = VPW;
+        slots = vpw < 2 ? (uint32_t) vpw : 2;
+    if (slots > vpw)
+        slots = (uint32_t) vpw;
     t.slots = slots;
-    t.chunks = (VPW + slots - 1) / slots;
+    t.chunks = (uint32_t) ((vpw + slots - 1) / slots);
     const uint64_t per_col = (uint64_t) t.groups * t.chunks;
     const uint64_t items = per_col * cols;
     if (items > 0xFFFFFFFFull)
-        return hipErrorInvalidValue;
+        return p; // not ok
     t.per_col = (uint32_t) per_col;
     t.items = (uint32_t) items;
-    t.qcol = qcol_bytes(NBITS, rows);
-    const uint32_t blocks = (uint32_t) ((items + 255) / 256);
-    hipExtLaunchKernelGGL((unquantize_kernel<NBITS, WV>), dim3(blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, t, add);
-    return hipGetLastError();
+    t.qcol = qcol_bytes(nbits, rows);
+    p.kind = vec ? kUnqVec4 : kUnqScalar;
+    p.blocks = (uint32_t) ((items + 255) / 256);
+    p.ok = true;
+    return p;
 }
 
 template <int NBITS>
-inline hipError_t launch_unquantize_segment_t(hipStream_t s, LaunchEvents ev, const char* q, float* out, size_t rows, size_t cols, int add)
+inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const char* q, float* out, const UnquantizePlan& p, int add)
 {
-    UnqSegGeom t;
-    t.rows = (uint32_t) rows;
-    t.nq = (uint32_t) qwords_per_col(rows, NBITS);
-    t.segs = (uint32_t) ((rows + t.nq - 1) / t.nq);
-    t.gps = (t.nq + 3 + 3) / 4;
-    const uint64_t items = (uint64_t) cols * t.segs * t.gps;
-    if (items > 0xFFFFFFFFull)
-        return hipErrorInvalidValue;
-    t.items = (uint32_t) items;
-    t.inv_gps = 1.0 / (double) t.gps;
-    t.inv_segs = 1.0 / (double) t.segs;
-    t.qcol = qcol_bytes(NBITS, rows);
-    const uint32_t blocks = (uint32_t) ((items + 255) / 256);
-    hipExtLaunchKernelGGL((unquantize_segment_kernel<NBITS>), dim3(blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, t, add);
+    if (p.kind == kUnqSegment)
+        hipExtLaunchKernelGGL((unquantize_segment_kernel<NBITS>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.seg, add);
+    else if (p.kind == kUnqVec4)
+        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 4>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.qw, add);
+    else
+        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 1>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.qw, add);
     return hipGetLastError();
 }
 
 inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* q, float* out, size_t rows, size_t cols, size_t nbits,
                                     bool add, const LaunchTuning& tune)
 {
+    const UnquantizePlan p = plan_unquantize(q, out, rows, cols, nbits, tune);
+    if (!p.ok)
+        return hipErrorInvalidValue;
     const char* qc = static_cast<const char*>(q);
-    const size_t nq = qwords_per_col(rows, nbits);
-    const bool vec = !tune.unq_force_scalar && (nq % 4 == 0) && (rows % 4 == 0) &&
-                     (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
     const int a = add ? 1 : 0;
-    const uint32_t sl = tune.unq_slots;
-    // long columns that the QWord-major decoder could only serve with 4-byte stores go to the segment decoder
-    const bool seg = !vec && !tune.unq_force_scalar && (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && nq >= 32 &&
-                     (uint64_t) cols * (32 / nbits) * ((nq + 6) / 4) <= 0xFFFFFFFFull;
-    if (seg)
-    {
-        switch (nbits)
-        {
-        case 1: return launch_unquantize_segment_t<1>(s, ev, qc, out, rows, cols, a);
-        case 2: return launch_unquantize_segment_t<2>(s, ev, qc, out, rows, cols, a);
-        case 4: return launch_unquantize_segment_t<4>(s, ev, qc, out, rows, cols, a);
-        case 8: return launch_unquantize_segment_t<8>(s, ev, qc, out, rows, cols, a);
-        case 16: return launch_unquantize_segment_t<16>(s, ev, qc, out, rows, cols, a);
-        case 32: return launch_unquantize_segment_t<32>(s, ev, qc, out, rows, cols, a);
-        default: return hipErrorInvalidValue;
-        }
-    }
     switch (nbits)
     {
-    case 1: return vec ? launch_unquantize_t<1, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<1, 1>(s, ev, qc, out, rows, cols, sl, a);
-    case 2: return vec ? launch_unquantize_t<2, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<2, 1>(s, ev, qc, out, rows, cols, sl, a);
-    case 4: return vec ? launch_unquantize_t<4, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<4, 1>(s, ev, qc, out, rows, cols, sl, a);
-    case 8: return vec ? launch_unquantize_t<8, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<8, 1>(s, ev, qc, out, rows, cols, sl, a);
-    case 16: return vec ? launch_unquantize_t<16, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<16, 1>(s, ev, qc, out, rows, cols, sl, a);
-    case 32: return vec ? launch_unquantize_t<32, 4>(s, ev, qc, out, rows, cols, sl, a) : launch_unquantize_t<32, 1>(s, ev, qc, out, rows, cols, sl, a);
+    case 1: return launch_unquantize_plan<1>(s, ev, qc, out, p, a);
+    case 2: return launch_unquantize_plan<2>(s, ev, qc, out, p, a);
+    case 4: return launch_unquantize_plan<4>(s, ev, qc, out, p, a);
+    case 8: return launch_unquantize_plan<8>(s, ev, qc, out, p, a);
+    case 16: return launch_unquantize_plan<16>(s, ev, qc, out, p, a);
+    case 32: return launch_unquantize_plan<32>(s, ev, qc, out, p, a);
     default: return hipErrorInvalidValue;
     }
+}
+
+// ---- many matrices per launch -----------------------------------------------------------------------
+// The entry tables live in device memory; the caller (the C-ABI layer) owns them and keeps them alive until the
+// kernel has finished.
+
+template <int NBITS, bool ZT>
+struct TileBatchLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const QuantizeBatchEntry* entries, const uint32_t* begins, uint32_t count,
+                          uint32_t total_tiles, size_t lds)
+    {
+        hipExtLaunchKernelGGL((quantize_tile_batch_kernel<NBITS, ZT>), dim3(total_tiles), dim3(kTileThreads), lds, s, ev.start, ev.stop,
+                              0, entries, begins, count);
+        return hipGetLastError();
+    }
+};
+
+inline hipError_t launch_quantize_tile_batch(hipStream_t s, LaunchEvents ev, const QuantizeBatchEntry* entries, const uint32_t* begins,
+                                             uint32_t count, uint32_t total_tiles, size_t lds, size_t nbits, bool zt)
+{
+    zt = zt && (nbits == 1);
+    return dispatch_nbits<TileBatchLauncher>(nbits, zt, s, ev, entries, begins, count, total_tiles, lds);
+}
+
+inline hipError_t launch_unquantize_batch(hipStream_t s, LaunchEvents ev, const UnquantizeBatchEntry* entries, const uint32_t* begins,
+                                          uint32_t count, uint32_t total_blocks, size_t nbits, bool add)
+{
+    const int a = add ? 1 : 0;
+    switch (nbits)
+    {
+    case 1: hipExtLaunchKernelGGL((unquantize_batch_kernel<1>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 2: hipExtLaunchKernelGGL((unquantize_batch_kernel<2>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 4: hipExtLaunchKernelGGL((unquantize_batch_kernel<4>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 8: hipExtLaunchKernelGGL((unquantize_batch_kernel<8>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 16: hipExtLaunchKernelGGL((unquantize_batch_kernel<16>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 32: hipExtLaunchKernelGGL((unquantize_batch_kernel<32>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// which path launch_quantize would take for this matrix
+inline int quantize_auto_path(const void* q, size_t rows, size_t nbits)
+{
+    if (rows > kTileMaxRows)
+        return kPathTall;
+    if (wavecol_applicable(nullptr, nullptr, nullptr, q, rows, nbits))
+        return kPathWaveCol;
+    return kPathTile;
 }
 
 } // namespace cntkq

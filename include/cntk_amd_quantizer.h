@@ -114,6 +114,38 @@ int cntkq_unquantize_async(cntkq_quantizer* h, const void* qbuf, size_t qbuf_byt
 /* MatrixQuantizerImpl::WaitUnquantizeAsyncDone (Source/Math/MatrixQuantizerGPU.cu:336-341). */
 int cntkq_wait_unquantize_done(cntkq_quantizer* h);
 
+/* A whole gradient set in one piece of stream work.
+ *
+ * The reference's aggregator quantizes (and later unquantizes) its gradient matrices one call each, in a loop
+ * (Source/1BitSGD/AllReduceDistGradAggregator.h:288-300 and :517-522; v2: Source/1BitSGD/QuantizedDistributedCommunicator.h:356-366
+ * and :516-521), all with the same bit width and threshold mode. On MI355X each launch has a floor of several
+ * microseconds, which dominates sets of many small matrices (ResNet-50: 161 matrices); these two calls take the whole
+ * loop at once and run it as one launch (plus one per very large matrix). Results are identical to the per-matrix calls.
+ *   items : host array, read during the call only. All buffers device-resident, same alignment rules as the
+ *           per-matrix calls; res_out may equal res_in; the matrices must not overlap one another.
+ *   cntkq_wait_quantize_done / cntkq_wait_unquantize_done wait for the whole batch. */
+typedef struct cntkq_quantize_item
+{
+    const float* in;
+    const float* res_in;
+    float* res_out;
+    void* qbuf; /* cntkq_qmatrix_bytes(rows, cols, nbits) bytes */
+    size_t rows;
+    size_t cols;
+} cntkq_quantize_item;
+
+typedef struct cntkq_unquantize_item
+{
+    const void* qbuf; /* cntkq_qmatrix_bytes(rows, cols, nbits) bytes */
+    float* out;
+    size_t rows;
+    size_t cols;
+} cntkq_unquantize_item;
+
+int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* items, size_t count, size_t nbits,
+                               int zero_threshold_for_1bit);
+int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item* items, size_t count, size_t nbits, int add);
+
 /* One owner's stripe reduction of the quantized all-reduce, fused into one pass
  * (dataflow of Source/1BitSGD/AllReduceDistGradAggregator.h:365-375 and :385-436; v2:
  * Source/1BitSGD/QuantizedDistributedCommunicator.h:423-471), replacing the reference's sequence

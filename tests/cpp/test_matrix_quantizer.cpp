@@ -152,6 +152,53 @@ static void GPUMatrix1BitQuantizeFloat()
     TestQuantization(dev, 2048, 33, -0.02f, +0.03f, 3015, 3);
 }
 
+// A gradient set through the batched calls gives the bytes of the per-matrix calls.
+static void BatchEqualsPerMatrix()
+{
+    const size_t shapes[][2] = {{147, 64}, {64, 64}, {576, 64}, {1, 5}, {429, 37}, {2048, 33}, {2304, 5}, {9304, 1}, {1000, 1}, {512, 100}};
+    const size_t numBits[] = {1, 4};
+    for (size_t nb : numBits)
+    {
+        auto* gpu = new MatrixQuantizerGPU<float>(0, true);
+        std::unique_ptr<MatrixQuantizerImpl<float>> owner(gpu);
+        std::vector<std::unique_ptr<Matrix<float>>> in, res1, res2, out1, out2;
+        std::vector<std::unique_ptr<QuantizedMatrix<float>>> q1, q2;
+        for (const auto& s : shapes)
+        {
+            in.emplace_back(new Matrix<float>(s[0], s[1], 0));
+            std::vector<float> host = RandomUniform(s[0], s[1], -0.01f, 0.02f, 77 + s[0]);
+            in.back()->SetValue(host.data());
+            res1.emplace_back(new Matrix<float>(s[0], s[1], 0));
+            res2.emplace_back(new Matrix<float>(s[0], s[1], 0));
+            out1.emplace_back(new Matrix<float>(s[0], s[1], 0));
+            out2.emplace_back(new Matrix<float>(s[0], s[1], 0));
+            q1.emplace_back(new QuantizedMatrix<float>(s[0], s[1], nb, 0));
+            q2.emplace_back(new QuantizedMatrix<float>(s[0], s[1], nb, 0));
+        }
+        std::vector<MatrixQuantizerGPU<float>::QuantizeItem> qi;
+        std::vector<MatrixQuantizerGPU<float>::UnquantizeItem> ui;
+        for (size_t i = 0; i < in.size(); ++i)
+        {
+            gpu->QuantizeAsync(*in[i], *res1[i], *q1[i], *res1[i], nb == 1);
+            qi.push_back({in[i].get(), res2[i].get(), q2[i].get(), res2[i].get()});
+            ui.push_back({q2[i].get(), out2[i].get()});
+        }
+        gpu->QuantizeBatchAsync(qi, nb == 1);
+        gpu->WaitQuantizeAsyncDone();
+        for (size_t i = 0; i < in.size(); ++i)
+            gpu->UnquantizeAsync(*q1[i], *out1[i]);
+        gpu->UnquantizeBatchAsync(ui);
+        gpu->WaitUnquantizeAsyncDone();
+        for (size_t i = 0; i < in.size(); ++i)
+        {
+            const size_t n = in[i]->GetNumElements();
+            CHECK(q1[i]->CopyToHost() == q2[i]->CopyToHost(), "batched codes, matrix %zu", i);
+            CHECK(std::memcmp(res1[i]->CopyToArray().get(), res2[i]->CopyToArray().get(), n * sizeof(float)) == 0, "batched residual, matrix %zu", i);
+            CHECK(std::memcmp(out1[i]->CopyToArray().get(), out2[i]->CopyToArray().get(), n * sizeof(float)) == 0, "batched output, matrix %zu", i);
+        }
+    }
+}
+
 static void ErrorBehaviour()
 {
     bool threw = false;
@@ -189,7 +236,10 @@ int main()
     {
         GPUMatrix1BitQuantizeFloat();
         std::printf("Test case GPUMatrixSuite/GPUMatrix1BitQuantizeFloat %s\n", g_failures ? "has FAILED" : "has passed");
-        const int before = g_failures;
+        int before = g_failures;
+        BatchEqualsPerMatrix();
+        std::printf("Test case GPUMatrixSuite/QuantizerBatchEqualsPerMatrix %s\n", g_failures != before ? "has FAILED" : "has passed");
+        before = g_failures;
         ErrorBehaviour();
         std::printf("Test case GPUMatrixSuite/QuantizerErrorBehaviour %s\n", g_failures != before ? "has FAILED" : "has passed");
     }

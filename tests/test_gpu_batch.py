@@ -1,0 +1,96 @@
+"""The batched entry points (a whole gradient set per call) give exactly the bytes of the per-matrix calls, and so
+inherit their parity with the oracle. Needs an MI355X."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import cntk_amd
+import datagen
+import oracle
+import parity
+from cntk_amd import Matrix, MatrixQuantizerImpl, QuantizedMatrix
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+MIXED = [(147, 64), (64, 64), (576, 64), (64, 256), (1, 5), (5, 1), (429, 37), (2048, 33), (2304, 5), (4608, 3), (9304, 1),
+         (2048, 1), (0, 4), (1000, 1), (1152, 128), (4096, 6), (20000, 2), (512, 100), (33, 67), (14336, 1)]
+
+
+@pytest.mark.parametrize("nbits,zt", [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False)])
+def test_batch_equals_per_matrix_calls(nbits, zt):
+    qz = MatrixQuantizerImpl.Create(0, False)
+    gs = [datagen.normal_with_outliers(100 * i + nbits, r, c) for i, (r, c) in enumerate(MIXED)]
+    rs = [datagen.normal(300 * i + nbits, r, c, 0.003) for i, (r, c) in enumerate(MIXED)]
+    for step in range(2):
+        say("batch", nbits, zt, "step", step)
+        # per-matrix calls
+        G = [Matrix.from_numpy(g) for g in gs]
+        R1 = [Matrix.from_numpy(r) for r in rs]
+        Q1 = [QuantizedMatrix(r, c, nbits, 0) for r, c in MIXED]
+        O1 = [Matrix.from_numpy(r) for r in rs]
+        for g, r, q in zip(G, R1, Q1):
+            qz.QuantizeAsync(g, r, q, r, zt)
+        qz.WaitQuantizeAsyncDone()
+        for q, o in zip(Q1, O1):
+            qz.UnquantizeAsync(q, o, add=(step == 1))
+        qz.WaitUnquantizeAsyncDone()
+        # one call each
+        R2 = [Matrix.from_numpy(r) for r in rs]
+        Q2 = [QuantizedMatrix(r, c, nbits, 0) for r, c in MIXED]
+        O2 = [Matrix.from_numpy(r) for r in rs]
+        qz.QuantizeBatchAsync([(g, r, q, r) for g, r, q in zip(G, R2, Q2)], zt)
+        qz.WaitQuantizeAsyncDone()
+        qz.UnquantizeBatchAsync(list(zip(Q2, O2)), add=(step == 1))
+        qz.WaitUnquantizeAsyncDone()
+        torch.cuda.synchronize()
+        for i, (r, c) in enumerate(MIXED):
+            assert np.array_equal(Q1[i].to_numpy(), Q2[i].to_numpy()), ("packed", MIXED[i])
+            assert parity.bits_equal(R1[i].to_numpy(), R2[i].to_numpy()), ("residual", MIXED[i])
+            assert parity.bits_equal(O1[i].to_numpy(), O2[i].to_numpy()), ("output", MIXED[i])
+            if r and c:
+                parity.check_quantize(gs[i], rs[i], Q2[i].to_numpy(), R2[i].to_numpy(), nbits, zt)
+        rs = [m.to_numpy() for m in R2]
+
+
+def test_batch_many_calls_reuse_tables():
+    """More batches in flight than the handle has table slots, with growing item counts."""
+    qz = MatrixQuantizerImpl.Create(0, True)
+    for n in (3, 40, 7, 161, 5, 5, 5, 5, 5, 300):
+        shapes = [(64 + 8 * (i % 13), 3 + (i % 5)) for i in range(n)]
+        gs = [datagen.normal(1000 + i, r, c) for i, (r, c) in enumerate(shapes)]
+        G = [Matrix.from_numpy(g) for g in gs]
+        R = [Matrix(r, c) for r, c in shapes]
+        Q = [QuantizedMatrix(r, c, 4, 0) for r, c in shapes]
+        O = [Matrix(r, c) for r, c in shapes]
+        torch.cuda.synchronize()
+        qz.SynchronizeWithMainStream()
+        for _ in range(6):
+            qz.QuantizeBatchAsync([(g, r, q, r) for g, r, q in zip(G, R, Q)], False)
+            qz.UnquantizeBatchAsync(list(zip(Q, O)))
+        qz.WaitUnquantizeAsyncDone()
+        torch.cuda.synchronize()
+        for i, (r, c) in enumerate(shapes):
+            parity.check_unquantize(Q[i].to_numpy(), r, c, 4, O[i].to_numpy())
+            # six steps of error feedback on a constant gradient: g * 6 == sum of outputs + residual, approximately
+        say("batch of", n, "ok")
+
+
+def test_batch_argument_checks():
+    qz = MatrixQuantizerImpl.Create(0, False)
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        qz.QuantizeBatchAsync([(Matrix(8, 4), Matrix(8, 5), QuantizedMatrix(8, 4, 1, 0), Matrix(8, 4))], False)
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        qz.QuantizeBatchAsync([(Matrix(8, 4), Matrix(8, 4), QuantizedMatrix(8, 4, 1, 0), Matrix(8, 4)),
+                               (Matrix(8, 4), Matrix(8, 4), QuantizedMatrix(8, 4, 2, 0), Matrix(8, 4))], False)
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        qz.UnquantizeBatchAsync([(QuantizedMatrix(8, 4, 1, cntk_amd.CPUDEVICE), Matrix(8, 4))])
+    qz.QuantizeBatchAsync([], False)
+    qz.UnquantizeBatchAsync([])

@@ -18,6 +18,7 @@ def test_cpp_matrix_quantizer_suite():
     assert res.returncode == 0, "C++ quantizer tests failed"
     assert "GPUMatrix1BitQuantizeFloat has passed" in res.stdout
     assert "QuantizerErrorBehaviour has passed" in res.stdout
+    assert "QuantizerBatchEqualsPerMatrix has passed" in res.stdout
 
 
 def test_cpp_mirror_header_is_self_contained():
