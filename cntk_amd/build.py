@@ -37,28 +37,37 @@ def build_library(verbose=False):
     return LIB_PATH
 
 
+CPP_TESTS = ["test_matrix_quantizer", "test_allreduce_aggregator", "bench_allreduce"]
+
+
 def build_cpp_tests(verbose=False):
-    """Compiles the C++ test program of the host mirror classes (tests/cpp) against the library and the CPU oracle."""
+    """Compiles the C++ programs under tests/cpp (host mirror classes, aggregator, all-reduce timing) against the
+    library and the CPU oracle."""
     root = os.path.dirname(HERE)
     out_dir = os.path.join(root, "tests", "cpp", "bin")
     os.makedirs(out_dir, exist_ok=True)
-    exe = os.path.join(out_dir, "test_matrix_quantizer")
     oracle_dir = os.path.join(root, "oracle")
     subprocess.run(["make", "-C", oracle_dir, "all"], check=True, capture_output=True)
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
-    # plain host C++ (no device code): the mirror classes only call the C ABI and the HIP runtime API
-    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-Wall",
-           os.path.join(root, "tests", "cpp", "test_matrix_quantizer.cpp"),
-           "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(rocm, "include"), "-o", exe,
-           "-L" + HERE, "-lcntk_amd_quantizer", "-L" + oracle_dir, "-loracle",
-           "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(rocm, "lib"),
-           "-Wl,-rpath,$ORIGIN/../../../cntk_amd", "-Wl,-rpath,$ORIGIN/../../../oracle"]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError("building the C++ tests failed:\n" + res.stderr)
-    return exe
+    exes = []
+    for name in CPP_TESTS:
+        src = os.path.join(root, "tests", "cpp", name + ".cpp")
+        if not os.path.exists(src):
+            continue
+        exe = os.path.join(out_dir, name)
+        # plain host C++ (no device code): the mirror classes only call the C ABI and the HIP runtime API
+        cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-Wall", src,
+               "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(rocm, "include"), "-o", exe,
+               "-L" + HERE, "-lcntk_amd_quantizer", "-L" + oracle_dir, "-loracle",
+               "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(rocm, "lib"),
+               "-Wl,-rpath,$ORIGIN/../../../cntk_amd", "-Wl,-rpath,$ORIGIN/../../../oracle"]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("building %s failed:\n%s" % (name, res.stderr))
+        exes.append(exe)
+    return exes
 
 
 if __name__ == "__main__":

@@ -1,0 +1,502 @@
+// Quantized all-reduce of gradient matrices: the reference's 1-bit-SGD aggregator restated over the MI355X quantizer,
+// with the message transport factored out.
+//
+//   cntk_amd::AllReduceDistGradAggregator<float>  <->  Source/1BitSGD/AllReduceDistGradAggregator.h:20-631
+//   cntk_amd::DistGradHeader                      <->  Source/SGDLib/DistGradHeader.h:5-100
+//   cntk_amd::StripeTransport                          what the reference does with MPI point-to-point messages
+//   cntk_amd::InProcessCluster                         K workers of one process sharing one GPU's memory
+//
+// Dataflow per worker r of K (Source/1BitSGD/AllReduceDistGradAggregator.h:237-566):
+//   1. quantize every gradient with its carried residual                                   (:288-300)
+//   2. hand stripe j of every packed gradient to worker j                                  (:303-378)
+//   3. sum the K packed versions of the own stripe in fp32, requantize the sum with the
+//      stripe residual, over the own slice of the own packed gradient                      (:365-375, 385-436)
+//   4. hand the requantized stripe to every other worker                                   (:459-502)
+//   5. unquantize the assembled packed gradient into the gradient matrix                   (:517-531)
+//   The header (sample counts, criterion, evaluation errors) is summed on the main node and sent back (:380-383, 440-457).
+//
+// The reference runs one aggregator per MPI rank and interleaves the steps with blocking waits. Here the steps are three
+// methods per worker (QuantizeAndPost, ReduceOwnStripes, FetchAndUnquantize) so that a single thread can drive K workers
+// (InProcessCluster); a transport over real links would call the same methods around its own waits.
+//
+// Differences from the reference, all deliberate: packed gradients stay in device memory (the reference stages every
+// stripe through pinned host memory); step 3 is one fused kernel when useFusedStripeReduce is set (bit-identical to the
+// reference's sequence of calls, which remains available and is what useQuantizationForSelfStripe = false needs); the
+// other workers' stripes are added in ascending rank order (the reference: message arrival order); the loops of steps 1
+// and 5 can run as one launch each (useBatchedCalls).
+#pragma once
+
+#include "MatrixQuantizer.h"
+
+#include <algorithm>
+#include <map>
+#include <tuple>
+#include <utility>
+
+namespace cntk_amd {
+
+// Source/SGDLib/DistGradHeader.h:5-100
+struct DistGradHeader
+{
+    size_t numSamples = 0;
+    size_t numSamplesWithLabel = 0; // denominator of 'criterion'
+    double criterion = 0.0;
+    std::vector<std::pair<double, size_t>> evalErrors; // (numerator, denominator) per evaluation node
+
+    explicit DistGradHeader(int numEvalNode) : evalErrors((size_t) numEvalNode) {}
+    int numEvalNode() const { return (int) evalErrors.size(); }
+
+    void Aggregate(const DistGradHeader& other, bool add = false)
+    {
+        if (other.numEvalNode() != numEvalNode())
+            throw std::runtime_error("mismatched size");
+        if (!add)
+        {
+            *this = other;
+            return;
+        }
+        numSamples += other.numSamples;
+        numSamplesWithLabel += other.numSamplesWithLabel;
+        criterion += other.criterion;
+        for (size_t i = 0; i < evalErrors.size(); i++)
+        {
+            evalErrors[i].first += other.evalErrors[i].first;
+            evalErrors[i].second += other.evalErrors[i].second;
+        }
+    }
+
+    void Clear()
+    {
+        numSamples = numSamplesWithLabel = 0;
+        criterion = 0;
+        for (auto& e : evalErrors)
+            e = {0.0, 0};
+    }
+};
+
+// The messages of the quantized all-reduce. `from`, `to`, `owner` are worker ranks; a stripe is always the column range
+// GetStripeForNode(cols, owner, K) of gradient matrix `matrixIdx`, as a packed matrix.
+class StripeTransport
+{
+public:
+    virtual ~StripeTransport() {}
+    virtual size_t NumProc() const = 0;
+    // True when every message is device work on the quantizers' own stream, so that stream order alone keeps the steps
+    // in sequence and the host waits the reference needs before handing buffers to MPI (:339, :494) can be skipped.
+    virtual bool StreamOrdered() const { return false; }
+    // Isend of a pre-aggregation stripe (Source/1BitSGD/AllReduceDistGradAggregator.h:339-365)
+    virtual void PostStripe(size_t from, size_t to, size_t matrixIdx, QuantizedMatrix<float>&& stripe) = 0;
+    // what the matching Irecv delivered (:303-320)
+    virtual const QuantizedMatrix<float>& ReceivedStripe(size_t owner, size_t from, size_t matrixIdx) = 0;
+    // Isend of the requantized stripe to everybody (:484-497) and its reception into the receiver's own packed gradient (:463-476)
+    virtual void PostAggregatedStripe(size_t owner, size_t matrixIdx, QuantizedMatrix<float>&& stripe) = 0;
+    virtual void FetchAggregatedStripe(size_t to, size_t owner, size_t matrixIdx, QuantizedMatrix<float>& dst, void* hipStream) = 0;
+    // Where the receiver can read the owner's requantized stripe in place (same memory, or peer-accessible memory),
+    // a view of it; nullptr where it has to be fetched into the receiver's own buffer first.
+    virtual const QuantizedMatrix<float>* AggregatedStripeView(size_t /*to*/, size_t /*owner*/, size_t /*matrixIdx*/) { return nullptr; }
+    // headers to the main node and back (:323-333, 380-383, 440-457, 478-514)
+    virtual void PostHeader(size_t from, const DistGradHeader& header) = 0;
+    virtual DistGradHeader AggregatedHeader() = 0;
+};
+
+// All workers live in one process and their buffers in one GPU's memory: a stripe "message" is a view of the sender's
+// buffer, the broadcast is a device-to-device copy on the quantizers' stream.
+class InProcessTransport final : public StripeTransport
+{
+public:
+    explicit InProcessTransport(size_t numWorkers, bool streamOrdered = true) : m_numWorkers(numWorkers), m_streamOrdered(streamOrdered) {}
+    size_t NumProc() const override { return m_numWorkers; }
+    bool StreamOrdered() const override { return m_streamOrdered; }
+
+    void PostStripe(size_t from, size_t to, size_t matrixIdx, QuantizedMatrix<float>&& stripe) override
+    {
+        m_stripes.erase({to, from, matrixIdx});
+        m_stripes.emplace(Key{to, from, matrixIdx}, std::move(stripe));
+    }
+    const QuantizedMatrix<float>& ReceivedStripe(size_t owner, size_t from, size_t matrixIdx) override
+    {
+        auto it = m_stripes.find({owner, from, matrixIdx});
+        if (it == m_stripes.end())
+            throw std::logic_error("InProcessTransport: stripe was never posted");
+        return it->second;
+    }
+    void PostAggregatedStripe(size_t owner, size_t matrixIdx, QuantizedMatrix<float>&& stripe) override
+    {
+        m_aggregated.erase({owner, 0, matrixIdx});
+        m_aggregated.emplace(Key{owner, 0, matrixIdx}, std::move(stripe));
+    }
+    void FetchAggregatedStripe(size_t /*to*/, size_t owner, size_t matrixIdx, QuantizedMatrix<float>& dst, void* hipStream) override
+    {
+        auto it = m_aggregated.find({owner, 0, matrixIdx});
+        if (it == m_aggregated.end())
+            throw std::logic_error("InProcessTransport: aggregated stripe was never posted");
+        if (it->second.GetSize() != dst.GetSize())
+            throw std::logic_error("InProcessTransport: stripe size mismatch");
+        if (dst.GetSize() != 0)
+            detail::HipCheck(hipMemcpyAsync(dst.Buffer(), it->second.Buffer(), dst.GetSize(), hipMemcpyDeviceToDevice,
+                                            static_cast<hipStream_t>(hipStream)),
+                             "hipMemcpyAsync");
+    }
+    const QuantizedMatrix<float>* AggregatedStripeView(size_t /*to*/, size_t owner, size_t matrixIdx) override
+    {
+        auto it = m_aggregated.find({owner, 0, matrixIdx});
+        return it == m_aggregated.end() ? nullptr : &it->second;
+    }
+    void PostHeader(size_t from, const DistGradHeader& header) override
+    {
+        m_headers.erase(from);
+        m_headers.emplace(from, header);
+    }
+    DistGradHeader AggregatedHeader() override
+    {
+        // the main node starts from its own header and adds the others as they arrive (:440-457)
+        if (m_headers.size() != m_numWorkers)
+            throw std::logic_error("InProcessTransport: not every worker posted its header");
+        DistGradHeader sum = m_headers.at(0);
+        for (size_t r = 1; r < m_numWorkers; ++r)
+            sum.Aggregate(m_headers.at(r), true);
+        return sum;
+    }
+
+private:
+    struct Key
+    {
+        size_t a, b, c;
+        bool operator<(const Key& o) const { return std::tie(a, b, c) < std::tie(o.a, o.b, o.c); }
+    };
+    size_t m_numWorkers;
+    bool m_streamOrdered;
+    std::map<Key, QuantizedMatrix<float>> m_stripes;
+    std::map<Key, QuantizedMatrix<float>> m_aggregated;
+    std::map<size_t, DistGradHeader> m_headers;
+};
+
+template <class ElemType>
+class AllReduceDistGradAggregator
+{
+public:
+    struct Stripe
+    {
+        size_t m_startCol;
+        size_t m_numCols;
+    };
+
+    struct Options
+    {
+        bool useFusedStripeReduce = true; // one kernel for "unquantize all stripes, sum, requantize"
+        bool useBatchedCalls = true;      // one launch for all gradients in steps 1 and 5
+    };
+
+    AllReduceDistGradAggregator(StripeTransport& transport, size_t myRank, int deviceId, int nBits, bool zeroThresholdFor1Bit,
+                                bool useQuantizationForSelfStripe, bool useAsyncAggregation, Options options = Options())
+        : m_transport(transport), m_rank(myRank), m_deviceId(deviceId), m_numQuantizationBits((size_t) nBits),
+          m_zeroThresholdFor1Bit(zeroThresholdFor1Bit), m_useQuantizationForSelfStripe(useQuantizationForSelfStripe),
+          m_useAsyncAggregation(useAsyncAggregation), m_options(options), m_initialized(false)
+    {
+        if (myRank >= transport.NumProc())
+            throw std::invalid_argument("AllReduceDistGradAggregator: rank out of range");
+    }
+
+    size_t MyRank() const { return m_rank; }
+    size_t NumProc() const { return m_transport.NumProc(); }
+    bool IsMainNode() const { return m_rank == 0; }
+
+    // Source/1BitSGD/AllReduceDistGradAggregator.h:56-65
+    static Stripe GetStripeForNode(size_t numCols, size_t nodeRank, size_t numNodes)
+    {
+        size_t start = 0, len = 0;
+        detail::Check(cntkq_stripe_range(numCols, nodeRank, numNodes, &start, &len));
+        return Stripe{start, len};
+    }
+
+    // First call: quantizers (with residuals) and packed buffers for every gradient and for the own stripe of every
+    // gradient; later calls with resetState: all residuals back to zero (:67-147).
+    void ResetState(const std::vector<Matrix<ElemType>*>& gradients, bool resetState)
+    {
+        if (!m_initialized)
+        {
+            m_initialized = true;
+            for (size_t i = 0; i < gradients.size(); i++)
+            {
+                const size_t nRow = gradients[i]->GetNumRows(), nCol = gradients[i]->GetNumCols();
+                m_preAggGradQuantizers.emplace_back(new MatrixQuantizer<ElemType>(nRow, nCol, m_deviceId, m_useAsyncAggregation));
+                m_gradQuantized.emplace_back(new QuantizedMatrix<ElemType>(nRow, nCol, m_numQuantizationBits, m_deviceId));
+                const Stripe stripe = GetStripeForNode(nCol, MyRank(), NumProc());
+                MatrixQuantizer<ElemType>* stripeQuantizer = nullptr;
+                if (stripe.m_numCols > 0)
+                    stripeQuantizer = new MatrixQuantizer<ElemType>(nRow, stripe.m_numCols, m_deviceId, m_useAsyncAggregation);
+                m_aggGradStripeQuantizers.emplace_back(stripeQuantizer);
+            }
+        }
+        else if (resetState)
+        {
+            for (auto& q : m_preAggGradQuantizers)
+                q->ResetResidue();
+            for (auto& q : m_aggGradStripeQuantizers)
+                if (q)
+                    q->ResetResidue();
+        }
+        if (gradients.size() != m_preAggGradQuantizers.size())
+            throw std::logic_error("AggregateGradients: the set of gradient matrices changed");
+    }
+
+    // Steps 1 and 2.
+    void QuantizeAndPost(const std::vector<Matrix<ElemType>*>& gradients, DistGradHeader& headerCPU, bool resetState)
+    {
+        ResetState(gradients, resetState);
+        const size_t numGradMatrices = gradients.size();
+        // a worker that saw no samples contributes zero gradients (:250-266)
+        if (headerCPU.numSamples == 0)
+            for (auto* g : gradients)
+                g->SetValue(0.0f);
+        // the gradients were produced on the main stream
+        if (m_useAsyncAggregation && numGradMatrices > 0)
+            SyncWithMainStream(*m_preAggGradQuantizers[0]);
+
+        if (m_options.useBatchedCalls)
+        {
+            std::vector<typename MatrixQuantizerGPU<ElemType>::QuantizeItem> items;
+            for (size_t i = 0; i < numGradMatrices; ++i)
+                items.push_back({gradients[i], &m_preAggGradQuantizers[i]->GetResidualMatrix(), m_gradQuantized[i].get(),
+                                 const_cast<Matrix<ElemType>*>(&m_preAggGradQuantizers[i]->GetResidualMatrix())});
+            if (numGradMatrices > 0)
+                Gpu(*m_preAggGradQuantizers[0]).QuantizeBatchAsync(items, m_zeroThresholdFor1Bit);
+        }
+        else
+        {
+            for (size_t i = 0; i < numGradMatrices; ++i)
+                m_preAggGradQuantizers[i]->QuantizeAsync(*gradients[i], *m_gradQuantized[i], m_zeroThresholdFor1Bit);
+        }
+
+        const bool hostWaits = !m_transport.StreamOrdered();
+        for (size_t i = 0; i < numGradMatrices; ++i)
+        {
+            if (hostWaits && !m_options.useBatchedCalls)
+                m_preAggGradQuantizers[i]->WaitQuantizeAsyncDone(); // (:339)
+            else if (hostWaits && i == 0)
+                m_preAggGradQuantizers[0]->WaitQuantizeAsyncDone();
+            for (size_t j = 0; j < NumProc(); ++j)
+            {
+                const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), j, NumProc());
+                if (stripe.m_numCols == 0)
+                    continue;
+                // the owner's own stripe travels the same way: the fused reduction reads it like any other
+                m_transport.PostStripe(MyRank(), j, i, m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+            }
+        }
+        m_transport.PostHeader(MyRank(), headerCPU);
+    }
+
+    // Steps 3 and 4.
+    void ReduceOwnStripes(const std::vector<Matrix<ElemType>*>& gradients)
+    {
+        const size_t K = NumProc();
+        const bool fused = m_options.useFusedStripeReduce && m_useQuantizationForSelfStripe;
+        for (size_t i = 0; i < gradients.size(); ++i)
+        {
+            const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K);
+            if (stripe.m_numCols == 0)
+                continue;
+            MatrixQuantizer<ElemType>& stripeQuantizer = *m_aggGradStripeQuantizers[i];
+            QuantizedMatrix<ElemType> ownSlice = m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols);
+            Matrix<ElemType>& stripeResidual = const_cast<Matrix<ElemType>&>(stripeQuantizer.GetResidualMatrix());
+            if (fused)
+            {
+                std::vector<const QuantizedMatrix<ElemType>*> stripes;
+                for (size_t w = 0; w < K; ++w)
+                    stripes.push_back(&m_transport.ReceivedStripe(MyRank(), w, i));
+                Gpu(stripeQuantizer).StripeReduceAsync(stripes, MyRank(), stripeResidual, ownSlice, m_zeroThresholdFor1Bit);
+            }
+            else
+            {
+                // the reference's sequence: the aggregate lives in the own slice of the gradient matrix (:268-286)
+                Matrix<ElemType> aggGradStripe = gradients[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols);
+                if (m_useQuantizationForSelfStripe)
+                    stripeQuantizer.UnquantizeAsync(ownSlice, aggGradStripe, false); // (:365-375)
+                for (size_t w = 0; w < K; ++w)
+                {
+                    if (w == MyRank())
+                        continue;
+                    QuantizedMatrix<ElemType>& received = const_cast<QuantizedMatrix<ElemType>&>(m_transport.ReceivedStripe(MyRank(), w, i));
+                    stripeQuantizer.UnquantizeAsync(received, aggGradStripe, true); // (:421)
+                }
+                // same stream: no wait needed between the last unquantize and the quantize (:426-434)
+                stripeQuantizer.QuantizeAsync(aggGradStripe, ownSlice, m_zeroThresholdFor1Bit);
+            }
+        }
+        const bool hostWaits = !m_transport.StreamOrdered();
+        for (size_t i = 0; i < gradients.size(); ++i)
+        {
+            const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K);
+            if (stripe.m_numCols == 0)
+                continue;
+            if (hostWaits && fused)
+                Gpu(*m_aggGradStripeQuantizers[i]).WaitStripeReduceDone();
+            else if (hostWaits)
+                m_aggGradStripeQuantizers[i]->WaitQuantizeAsyncDone(); // (:494)
+            m_transport.PostAggregatedStripe(MyRank(), i, m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+        }
+    }
+
+    // Step 5. Returns whether any worker processed samples (the reference's return value of AggregateGradients).
+    bool FetchAndUnquantize(const std::vector<Matrix<ElemType>*>& gradients, DistGradHeader& headerCPU)
+    {
+        const size_t K = NumProc();
+        // Stripes that can be read where their owner left them are unquantized straight from there, stripe by stripe;
+        // the others are first gathered into the own packed gradient (:459-476), which is then unquantized whole (:517-522).
+        std::vector<Matrix<ElemType>> outSlices;            // keep the views alive until the call below
+        std::vector<QuantizedMatrix<ElemType>> ownSlices;
+        std::vector<std::pair<const QuantizedMatrix<ElemType>*, size_t>> viewItems; // (packed stripe, index into outSlices)
+        std::vector<bool> whole(gradients.size(), true);
+        if (m_options.useBatchedCalls)
+        {
+            size_t slices = 0;
+            for (size_t i = 0; i < gradients.size(); ++i)
+                for (size_t j = 0; j < K; ++j)
+                    slices += GetStripeForNode(gradients[i]->GetNumCols(), j, K).m_numCols > 0 ? 1 : 0;
+            outSlices.reserve(slices);
+            ownSlices.reserve(slices);
+            for (size_t i = 0; i < gradients.size(); ++i)
+            {
+                bool allViews = true;
+                for (size_t j = 0; j < K && allViews; ++j)
+                    if (j != MyRank() && GetStripeForNode(gradients[i]->GetNumCols(), j, K).m_numCols > 0)
+                        allViews = m_transport.AggregatedStripeView(MyRank(), j, i) != nullptr;
+                if (!allViews)
+                    continue;
+                whole[i] = false;
+                for (size_t j = 0; j < K; ++j)
+                {
+                    const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), j, K);
+                    if (stripe.m_numCols == 0)
+                        continue;
+                    outSlices.push_back(gradients[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+                    if (j == MyRank())
+                    {
+                        ownSlices.push_back(m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+                        viewItems.push_back({&ownSlices.back(), outSlices.size() - 1});
+                    }
+                    else
+                        viewItems.push_back({m_transport.AggregatedStripeView(MyRank(), j, i), outSlices.size() - 1});
+                }
+            }
+        }
+        for (size_t i = 0; i < gradients.size(); ++i)
+        {
+            if (!whole[i])
+                continue;
+            for (size_t j = 0; j < K; ++j)
+            {
+                if (j == MyRank())
+                    continue;
+                const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), j, K);
+                if (stripe.m_numCols == 0)
+                    continue;
+                QuantizedMatrix<ElemType> dst = m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols);
+                m_transport.FetchAggregatedStripe(MyRank(), j, i, dst, cntkq_stream(Gpu(*m_preAggGradQuantizers[i]).Handle()));
+            }
+        }
+        if (m_options.useBatchedCalls)
+        {
+            std::vector<typename MatrixQuantizerGPU<ElemType>::UnquantizeItem> items;
+            for (size_t i = 0; i < gradients.size(); ++i)
+                if (whole[i])
+                    items.push_back({m_gradQuantized[i].get(), gradients[i]});
+            for (const auto& v : viewItems)
+                items.push_back({v.first, &outSlices[v.second]});
+            if (!items.empty())
+            {
+                Gpu(*m_preAggGradQuantizers[0]).UnquantizeBatchAsync(items, false);
+                m_preAggGradQuantizers[0]->WaitUnquantizeAsyncDone();
+            }
+        }
+        else
+        {
+            for (size_t i = 0; i < gradients.size(); ++i)
+                m_preAggGradQuantizers[i]->UnquantizeAsync(*m_gradQuantized[i], *gradients[i], false); // (:521)
+            for (size_t i = 0; i < gradients.size(); ++i)
+                m_preAggGradQuantizers[i]->WaitUnquantizeAsyncDone();                                   // (:531)
+        }
+        headerCPU.Aggregate(m_transport.AggregatedHeader(), false);
+        return headerCPU.numSamples != 0;
+    }
+
+    const Matrix<ElemType>& GradientResidual(size_t i) const { return m_preAggGradQuantizers[i]->GetResidualMatrix(); }
+    const Matrix<ElemType>* StripeResidual(size_t i) const
+    {
+        return m_aggGradStripeQuantizers[i] ? &m_aggGradStripeQuantizers[i]->GetResidualMatrix() : nullptr;
+    }
+    const QuantizedMatrix<ElemType>& QuantizedGradient(size_t i) const { return *m_gradQuantized[i]; }
+
+private:
+    static MatrixQuantizerGPU<ElemType>& Gpu(MatrixQuantizer<ElemType>& q)
+    {
+        return dynamic_cast<MatrixQuantizerGPU<ElemType>&>(q.Impl());
+    }
+    void SyncWithMainStream(MatrixQuantizer<ElemType>& q)
+    {
+        std::unique_ptr<MatrixComputeStreamEvent> ev(MatrixComputeStreamEvent::Create(m_deviceId));
+        ev->SynchronizeQuantizationComputeStreamWithEvent<ElemType>(q.Impl());
+    }
+
+    StripeTransport& m_transport;
+    size_t m_rank;
+    int m_deviceId;
+    size_t m_numQuantizationBits;
+    bool m_zeroThresholdFor1Bit;
+    bool m_useQuantizationForSelfStripe;
+    bool m_useAsyncAggregation;
+    Options m_options;
+    bool m_initialized;
+
+    std::vector<std::unique_ptr<MatrixQuantizer<ElemType>>> m_preAggGradQuantizers;
+    std::vector<std::unique_ptr<QuantizedMatrix<ElemType>>> m_gradQuantized;
+    std::vector<std::unique_ptr<MatrixQuantizer<ElemType>>> m_aggGradStripeQuantizers;
+};
+
+// K workers of one process on one GPU: drives the three steps of every worker in turn. This is the arrangement of the
+// "K simulated workers in one GPU's memory" workload; a deployment has one worker per GPU and a transport over links.
+template <class ElemType>
+class InProcessCluster
+{
+public:
+    typedef typename AllReduceDistGradAggregator<ElemType>::Options Options;
+
+    // All quantizers of the cluster issue on one stream (the shared dedicated stream, or the main stream) and the transport is
+    // stream-ordered: the K workers' steps are queued back to back and the host waits only at the very end.
+    InProcessCluster(size_t numWorkers, int deviceId, int nBits, bool zeroThresholdFor1Bit, bool useQuantizationForSelfStripe = true,
+                     bool useAsyncAggregation = true, Options options = Options())
+        : m_transport(numWorkers, true)
+    {
+        for (size_t r = 0; r < numWorkers; ++r)
+            m_workers.emplace_back(new AllReduceDistGradAggregator<ElemType>(m_transport, r, deviceId, nBits, zeroThresholdFor1Bit,
+                                                                             useQuantizationForSelfStripe, useAsyncAggregation, options));
+    }
+
+    size_t NumWorkers() const { return m_workers.size(); }
+    AllReduceDistGradAggregator<ElemType>& Worker(size_t r) { return *m_workers[r]; }
+
+    // gradients[r] / headers[r] belong to worker r. With unquantizeOnAllWorkers = false only worker 0 ends up with the
+    // aggregated gradients (the others would hold the same bytes); the packed aggregate is assembled on every worker.
+    bool AggregateGradients(const std::vector<std::vector<Matrix<ElemType>*>>& gradients, std::vector<DistGradHeader>& headers,
+                            bool resetState, bool unquantizeOnAllWorkers = true)
+    {
+        const size_t K = m_workers.size();
+        if (gradients.size() != K || headers.size() != K)
+            throw std::invalid_argument("InProcessCluster: one gradient set and one header per worker");
+        for (size_t r = 0; r < K; ++r)
+            m_workers[r]->QuantizeAndPost(gradients[r], headers[r], resetState);
+        for (size_t r = 0; r < K; ++r)
+            m_workers[r]->ReduceOwnStripes(gradients[r]);
+        bool any = false;
+        for (size_t r = 0; r < (unquantizeOnAllWorkers ? K : 1); ++r)
+            any = m_workers[r]->FetchAndUnquantize(gradients[r], headers[r]) || any;
+        return any;
+    }
+
+private:
+    InProcessTransport m_transport;
+    std::vector<std::unique_ptr<AllReduceDistGradAggregator<ElemType>>> m_workers;
+};
+
+} // namespace cntk_amd

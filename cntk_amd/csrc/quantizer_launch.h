@@ -233,18 +233,9 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
         }
         return hipGetLastError();
     }
-    // A stripe is small (one GPU's share of the columns), so the kernel is latency-bound: take the smallest
-    // tile that still gives every thread of a workgroup a work item, to spread the stripe over all CUs.
-    uint32_t gs = tune.tile_gs;
-    if (gs == 0)
-    {
-        const size_t chunks = nbits == 1 ? 4 : (nbits == 2 ? 2 : 1);
-        const size_t items_per_col = qwords_per_col(rows, nbits) * chunks;
-        gs = kTileThreads;
-        while (gs > 8 && items_per_col * (kTileThreads / gs) < kTileThreads)
-            gs >>= 1;
-    }
-    const TileGeom t = make_tile_geom(rows, cols, nbits, gs, tune.tile_stage, tune.tile_threads);
+    // Same tile geometry as launch_quantize would use for a matrix of this height, so that the statistics are summed in
+    // the same order and the fused call gives the bytes of the reference's unquantize ... quantize call sequence.
+    const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs, tune.tile_stage, tune.tile_threads);
     return dispatch_nbits<StripeLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, t);
 }
 

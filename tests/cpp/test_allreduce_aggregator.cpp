@@ -1,0 +1,304 @@
+// Tests of the quantized all-reduce aggregator (cntk_amd/cpp/AllReduceDistGradAggregator.h) with K workers in one
+// process on one GPU. The checker is the CPU oracle's restatement of the same dataflow (oracle_allreduce).
+//
+//   * every worker ends with the same aggregated gradients (what the reference's distributed tests assert:
+//     bindings/python/cntk/learners/tests/distributed_learner_test.py:101-128);
+//   * the fused stripe reduction, the batched calls and the dedicated stream change nothing: bit-identical gradients,
+//     residuals and stripe residuals against the reference's sequence of per-matrix calls on the main stream;
+//   * 32 bits: the aggregate equals the plain fp32 sum in the documented order (the reference's own known answer,
+//     Tests/EndToEndTests/CNTKv2Library/EndToEndTests/FrameMode.cpp:112-116);
+//   * 1, 2, 4 bits over several carried steps: aggregated gradients against the oracle within 1e-4 of the value range
+//     with at most 0.1 % outliers (the reference unit test's GPU tolerance), residuals carried on both sides;
+//   * headers are summed; a worker without samples contributes zeros; resetState clears all residuals.
+#include "../../cntk_amd/cpp/AllReduceDistGradAggregator.h"
+#include "../../oracle/quantizer_oracle.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <random>
+
+using namespace cntk_amd;
+
+static int g_failures = 0;
+#define CHECK(cond, ...)                                                                                               \
+    do                                                                                                                 \
+    {                                                                                                                  \
+        if (!(cond))                                                                                                   \
+        {                                                                                                              \
+            if (g_failures < 20)                                                                                       \
+            {                                                                                                          \
+                std::fprintf(stderr, "CHECK failed %s:%d: %s  ", __FILE__, __LINE__, #cond);                         \
+                std::fprintf(stderr, __VA_ARGS__);                                                                     \
+                std::fprintf(stderr, "\n");                                                                            \
+            }                                                                                                          \
+            g_failures++;                                                                                              \
+        }                                                                                                              \
+    } while (0)
+
+typedef std::vector<std::pair<size_t, size_t>> Shapes;
+
+static std::vector<float> Gaussian(size_t n, float sigma, unsigned long seed)
+{
+    std::mt19937_64 rng(seed);
+    std::normal_distribution<float> d(0.0f, sigma);
+    std::vector<float> a(n);
+    for (auto& x : a)
+        x = d(rng);
+    return a;
+}
+
+struct WorkerSet
+{
+    std::vector<std::unique_ptr<Matrix<float>>> owned;
+    std::vector<Matrix<float>*> ptrs;
+};
+
+static std::vector<WorkerSet> MakeGradients(const Shapes& shapes, size_t K, const std::vector<std::vector<std::vector<float>>>& host)
+{
+    std::vector<WorkerSet> sets(K);
+    for (size_t r = 0; r < K; ++r)
+        for (size_t i = 0; i < shapes.size(); ++i)
+        {
+            sets[r].owned.emplace_back(new Matrix<float>(shapes[i].first, shapes[i].second, 0));
+            sets[r].owned.back()->SetValue(host[r][i].data());
+            sets[r].ptrs.push_back(sets[r].owned.back().get());
+        }
+    return sets;
+}
+
+static bool SameBits(const Matrix<float>& a, const Matrix<float>& b)
+{
+    if (a.GetNumElements() != b.GetNumElements())
+        return false;
+    auto x = a.CopyToArray(), y = b.CopyToArray();
+    return std::memcmp(x.get(), y.get(), a.GetNumElements() * sizeof(float)) == 0;
+}
+
+// Runs `steps` aggregations with the given options; returns the clusters' final state for comparison.
+struct RunResult
+{
+    std::vector<std::vector<std::vector<float>>> gradients; // [step][matrix] of worker 0
+    std::unique_ptr<InProcessCluster<float>> cluster;
+    std::vector<WorkerSet> last;
+};
+
+static RunResult Run(const Shapes& shapes, size_t K, int nBits, bool zeroThr, bool selfStripeQuantized, bool useAsync, bool fused, bool batched,
+                     int steps, unsigned long seed, bool checkAllWorkersEqual)
+{
+    RunResult out;
+    InProcessCluster<float>::Options opt;
+    opt.useFusedStripeReduce = fused;
+    opt.useBatchedCalls = batched;
+    out.cluster.reset(new InProcessCluster<float>(K, 0, nBits, zeroThr, selfStripeQuantized, useAsync, opt));
+    for (int step = 0; step < steps; ++step)
+    {
+        std::vector<std::vector<std::vector<float>>> host(K);
+        for (size_t r = 0; r < K; ++r)
+            for (size_t i = 0; i < shapes.size(); ++i)
+                host[r].push_back(Gaussian(shapes[i].first * shapes[i].second, 0.01f, seed + 1000 * step + 10 * r + i));
+        std::vector<WorkerSet> sets = MakeGradients(shapes, K, host);
+        std::vector<std::vector<Matrix<float>*>> grads;
+        std::vector<DistGradHeader> headers;
+        for (size_t r = 0; r < K; ++r)
+        {
+            grads.push_back(sets[r].ptrs);
+            headers.emplace_back(2);
+            headers.back().numSamples = 10 + r;
+            headers.back().numSamplesWithLabel = 9 + r;
+            headers.back().criterion = 1.5 * (double) (r + 1);
+            headers.back().evalErrors[0] = {0.25 * (double) r, 10 + r};
+            headers.back().evalErrors[1] = {1.0, 1};
+        }
+        const bool any = out.cluster->AggregateGradients(grads, headers, step == 0, true);
+        CHECK(any, "samples were processed");
+        detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize");
+        // headers: every worker holds the sum
+        size_t ns = 0;
+        double crit = 0;
+        for (size_t r = 0; r < K; ++r)
+        {
+            ns += 10 + r;
+            crit += 1.5 * (double) (r + 1);
+        }
+        for (size_t r = 0; r < K; ++r)
+        {
+            CHECK(headers[r].numSamples == ns && std::fabs(headers[r].criterion - crit) < 1e-12, "header sum on worker %zu", r);
+            CHECK(headers[r].evalErrors[1].second == K, "eval error denominators");
+        }
+        if (checkAllWorkersEqual)
+            for (size_t r = 1; r < K; ++r)
+                for (size_t i = 0; i < shapes.size(); ++i)
+                    CHECK(SameBits(*sets[0].ptrs[i], *sets[r].ptrs[i]), "worker %zu, matrix %zu differs from worker 0", r, i);
+        out.gradients.emplace_back();
+        for (size_t i = 0; i < shapes.size(); ++i)
+        {
+            auto a = sets[0].ptrs[i]->CopyToArray();
+            out.gradients.back().emplace_back(a.get(), a.get() + sets[0].ptrs[i]->GetNumElements());
+        }
+        out.last = std::move(sets);
+    }
+    return out;
+}
+
+static void VariantsAreBitIdentical()
+{
+    const Shapes shapes = {{2048, 40}, {429, 37}, {64, 5}, {576, 24}, {1, 9}, {33, 3}};
+    const size_t K = 4;
+    for (int nBits : {1, 4})
+        for (bool zeroThr : {false, true})
+        {
+            if (nBits != 1 && zeroThr)
+                continue;
+            // the reference's arrangement: per-matrix calls, unfused stripe reduction, main stream
+            RunResult ref = Run(shapes, K, nBits, zeroThr, true, false, false, false, 3, 4242, true);
+            for (int variant = 1; variant < 8; ++variant)
+            {
+                const bool useAsync = variant & 1, fused = variant & 2, batched = variant & 4;
+                RunResult v = Run(shapes, K, nBits, zeroThr, true, useAsync, fused, batched, 3, 4242, false);
+                for (size_t step = 0; step < ref.gradients.size(); ++step)
+                    for (size_t i = 0; i < shapes.size(); ++i)
+                        CHECK(ref.gradients[step][i].size() == v.gradients[step][i].size() &&
+                                  std::memcmp(ref.gradients[step][i].data(), v.gradients[step][i].data(), ref.gradients[step][i].size() * 4) == 0,
+                              "bits=%d zeroThr=%d variant=%d step=%zu matrix=%zu", nBits, (int) zeroThr, variant, step, i);
+                for (size_t r = 0; r < K; ++r)
+                    for (size_t i = 0; i < shapes.size(); ++i)
+                    {
+                        CHECK(SameBits(ref.cluster->Worker(r).GradientResidual(i), v.cluster->Worker(r).GradientResidual(i)), "gradient residual");
+                        const Matrix<float>* a = ref.cluster->Worker(r).StripeResidual(i);
+                        const Matrix<float>* b = v.cluster->Worker(r).StripeResidual(i);
+                        CHECK((a == nullptr) == (b == nullptr) && (a == nullptr || SameBits(*a, *b)), "stripe residual");
+                    }
+            }
+        }
+}
+
+static void AgainstOracle()
+{
+    const Shapes shapes = {{2048, 24}, {429, 37}, {100, 50}, {64, 3}};
+    const size_t K = 8;
+    const int steps = 3;
+    struct Case { int nBits; bool zeroThr; };
+    for (Case c : {Case{1, false}, Case{1, true}, Case{2, false}, Case{4, false}, Case{32, false}})
+    {
+        RunResult gpu = Run(shapes, K, c.nBits, c.zeroThr, true, true, true, true, steps, 99, true);
+        // oracle: one all-reduce per matrix and step, residuals carried
+        for (size_t i = 0; i < shapes.size(); ++i)
+        {
+            const size_t rows = shapes[i].first, cols = shapes[i].second, n = rows * cols;
+            const size_t qbytes = oracle_qcol_bytes(c.nBits, rows) * cols;
+            std::vector<std::vector<float>> res(K, std::vector<float>(n, 0.0f)), sres(K);
+            for (size_t s = 0; s < K; ++s)
+            {
+                size_t start, len;
+                oracle_stripe_range(cols, s, K, &start, &len);
+                sres[s].assign(rows * len + 1, 0.0f);
+            }
+            for (int step = 0; step < steps; ++step)
+            {
+                std::vector<std::vector<float>> g(K);
+                std::vector<std::vector<char>> q(K, std::vector<char>(qbytes));
+                std::vector<const float*> gp;
+                std::vector<float*> rp, sp;
+                std::vector<void*> qp;
+                for (size_t r = 0; r < K; ++r)
+                {
+                    g[r] = Gaussian(n, 0.01f, 99 + 1000 * step + 10 * r + i);
+                    gp.push_back(g[r].data());
+                    rp.push_back(res[r].data());
+                    sp.push_back(sres[r].data());
+                    qp.push_back(q[r].data());
+                }
+                std::vector<char> qagg(qbytes);
+                std::vector<float> out(n);
+                oracle_allreduce(gp.data(), rp.data(), qp.data(), sp.data(), K, rows, cols, c.nBits, c.zeroThr, qagg.data(), out.data(), 4);
+                const std::vector<float>& got = gpu.gradients[step][i];
+                if (c.nBits == 32)
+                {
+                    CHECK(std::memcmp(got.data(), out.data(), n * 4) == 0, "32 bits must reproduce the ordered fp32 sum exactly (matrix %zu)", i);
+                    continue;
+                }
+                // the reference unit test's GPU tolerance: 1e-4 of the value range, at most 0.1 % outliers
+                const float tolerance = 0.08f * 8 * 1e-4f;
+                size_t bad = 0;
+                for (size_t e = 0; e < n; ++e)
+                    if (std::fabs(got[e] - out[e]) > tolerance)
+                        bad++;
+                CHECK(bad <= std::max<size_t>(1, n / 1000), "bits=%d zeroThr=%d matrix %zu step %d: %zu of %zu elements off", c.nBits, (int) c.zeroThr, i, step, bad, n);
+            }
+        }
+    }
+}
+
+static void UnquantizedSelfStripe()
+{
+    // useQuantizationForSelfStripe = false: the owner's own contribution enters the sum unquantized
+    // (Source/1BitSGD/AllReduceDistGradAggregator.h:366-375); with 32 bits both settings give the plain sum
+    const Shapes shapes = {{128, 16}, {33, 5}};
+    RunResult a = Run(shapes, 3, 32, false, false, false, true, false, 2, 7, true);
+    RunResult b = Run(shapes, 3, 32, false, true, false, true, false, 2, 7, true);
+    for (size_t step = 0; step < a.gradients.size(); ++step)
+        for (size_t i = 0; i < shapes.size(); ++i)
+            CHECK(a.gradients[step][i] == b.gradients[step][i], "32-bit aggregate independent of self-stripe setting");
+    // at 1 bit the two settings differ, and every worker still ends with identical gradients
+    RunResult c = Run(shapes, 3, 1, true, false, true, true, true, 2, 7, true);
+    RunResult d = Run(shapes, 3, 1, true, true, true, true, true, 2, 7, true);
+    CHECK(c.gradients[1][0] != d.gradients[1][0], "self-stripe setting must matter at 1 bit");
+}
+
+static void EmptyMinibatchAndReset()
+{
+    const Shapes shapes = {{256, 12}, {64, 7}};
+    const size_t K = 3;
+    InProcessCluster<float> cluster(K, 0, 1, true);
+    auto step = [&](bool reset, size_t silent, std::vector<WorkerSet>& sets, std::vector<DistGradHeader>& headers) {
+        std::vector<std::vector<std::vector<float>>> host(K);
+        for (size_t r = 0; r < K; ++r)
+            for (size_t i = 0; i < shapes.size(); ++i)
+                host[r].push_back(Gaussian(shapes[i].first * shapes[i].second, 0.01f, 5 + 10 * r + i));
+        sets = MakeGradients(shapes, K, host);
+        std::vector<std::vector<Matrix<float>*>> grads;
+        headers.clear();
+        for (size_t r = 0; r < K; ++r)
+        {
+            grads.push_back(sets[r].ptrs);
+            headers.emplace_back(1);
+            headers.back().numSamples = (r == silent) ? 0 : 4;
+        }
+        cluster.AggregateGradients(grads, headers, reset);
+        detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    };
+    std::vector<WorkerSet> s1, s2, s3;
+    std::vector<DistGradHeader> h1, h2, h3;
+    step(true, K, s1, h1);  // everybody has samples
+    step(true, K, s2, h2);  // same inputs after a reset: identical result, i.e. no residual survived the reset
+    for (size_t i = 0; i < shapes.size(); ++i)
+        CHECK(SameBits(*s1[0].ptrs[i], *s2[0].ptrs[i]), "resetState must clear every residual");
+    step(true, 1, s3, h3);  // worker 1 saw no samples: its gradients are zeroed before quantization
+    CHECK(h3[0].numSamples == 8, "header sum with a silent worker");
+    for (size_t i = 0; i < shapes.size(); ++i)
+        CHECK(!SameBits(*s1[0].ptrs[i], *s3[0].ptrs[i]), "a silent worker changes the aggregate");
+}
+
+int main()
+{
+    try
+    {
+        struct T { const char* name; void (*fn)(); };
+        const T tests[] = {{"QuantizedAllReduceVariantsBitIdentical", VariantsAreBitIdentical}, {"QuantizedAllReduceAgainstOracle", AgainstOracle},
+                           {"QuantizedAllReduceUnquantizedSelfStripe", UnquantizedSelfStripe}, {"QuantizedAllReduceEmptyMinibatchAndReset", EmptyMinibatchAndReset}};
+        for (const T& t : tests)
+        {
+            const int before = g_failures;
+            t.fn();
+            std::printf("Test case AggregatorSuite/%s %s\n", t.name, g_failures != before ? "has FAILED" : "has passed");
+            std::fflush(stdout);
+        }
+    }
+    catch (const std::exception& e)
+    {
+        std::fprintf(stderr, "unexpected exception: %s\n", e.what());
+        return 2;
+    }
+    return g_failures ? 1 : 0;
+}

@@ -21,11 +21,34 @@ def test_cpp_matrix_quantizer_suite():
     assert "QuantizerBatchEqualsPerMatrix has passed" in res.stdout
 
 
+@pytest.mark.gpu
+def test_cpp_allreduce_aggregator_suite():
+    """The aggregator restatement (cntk_amd/cpp/AllReduceDistGradAggregator.h) with K in-process workers."""
+    exe = os.path.join(ROOT, "tests", "cpp", "bin", "test_allreduce_aggregator")
+    assert os.path.exists(exe), "build it first: python -m cntk_amd.build"
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=900)
+    print(res.stdout)
+    print(res.stderr[-4000:])
+    assert res.returncode == 0, "C++ aggregator tests failed"
+    for name in ("VariantsBitIdentical", "AgainstOracle", "UnquantizedSelfStripe", "EmptyMinibatchAndReset"):
+        assert "QuantizedAllReduce%s has passed" % name in res.stdout
+
+
+@pytest.mark.gpu
+def test_cpp_allreduce_timing_program_runs():
+    """The all-reduce timing program on a small shape (its full-size numbers are quoted in the design notes)."""
+    exe = os.path.join(ROOT, "tests", "cpp", "bin", "bench_allreduce")
+    assert os.path.exists(exe), "build it first: python -m cntk_amd.build"
+    res = subprocess.run([exe, "4", "2048", "256", "1", "3"], capture_output=True, text=True, timeout=300)
+    print(res.stdout, res.stderr[-2000:])
+    assert res.returncode == 0 and res.stdout.count("GB/s") == 3
+
+
 def test_cpp_mirror_header_is_self_contained():
     """The mirror header compiles as plain host C++ (no device code, no torch)."""
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     src = '#include "%s"\nint main() { return sizeof(cntk_amd::QuantizedColumn<float>) == 12 ? 0 : 1; }\n' % os.path.join(
-        ROOT, "cntk_amd", "cpp", "MatrixQuantizer.h")
+        ROOT, "cntk_amd", "cpp", "AllReduceDistGradAggregator.h")
     res = subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(rocm, "include"),
                           "-x", "c++", "-"], input=src, capture_output=True, text=True)
     assert res.returncode == 0, res.stderr[-3000:]
