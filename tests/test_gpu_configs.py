@@ -1,4 +1,4 @@
-"""The five workloads BASELINE.json names, at their real shapes, through the C ABI. Needs an MI355X.
+"""The five benchmark workloads of this path (speech DNN, ResNet-50, LSTM LM gradient sets, simulated 8-worker all-reduce), at their real shapes, through the C ABI. Needs an MI355X.
 
 At full size the GPU chain runs freely on its own residual (gradients are generated on the device), every step is
 checked through size-independent properties (conservation of the error feedback, codes consistent with the

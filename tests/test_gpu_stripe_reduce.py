@@ -197,7 +197,7 @@ def test_simulated_allreduce(shape, use_async):
 
 
 def test_config4_shape_one_stripe():
-    """BASELINE config 4 at its real shape, one owner: 8 workers x 2048x9304, stripe 2048x1163."""
+    """The 8-worker all-reduce workload at its real shape, one owner: 8 workers x 2048x9304, stripe 2048x1163."""
     rows, cols, k, nbits = 2048, 9304, 8, 1
     qz = MatrixQuantizerImpl.Create(0, False)
     zeros = np.zeros((rows, cols), np.float32, order="F")
