@@ -80,6 +80,28 @@ int oracle_allreduce(const float* const* g, float* const* res, void* const* q, f
                      size_t workers, size_t rows, size_t cols, size_t nbits, int zero_threshold,
                      void* qagg, float* out, int threads);
 
+/* ---- MatrixQuantizerImpl<double> (QWord = uint64_t, nbits in 1..64, record {f64 lower; f64 upper; u64 bits[nq]}) ----
+ * Same functions, same citations; only the element and QWord types differ. */
+int oracle_check_nbits_f64(size_t nbits);
+size_t oracle_qwords_per_col_f64(size_t rows, size_t nbits);
+size_t oracle_qcol_bytes_f64(size_t nbits, size_t rows);
+uint64_t oracle_quantize_value_f64(double u, size_t nbits, double lower, double upper, int zero_threshold);
+double oracle_unquantize_value_f64(uint64_t q, size_t nbits, double lower, double upper);
+void oracle_column_stats_f64(const double* g, const double* r, size_t rows, size_t j, size_t nbits,
+                             int zero_threshold, double* lower, double* upper);
+int oracle_quantize_f64(const double* g, const double* r_in, size_t rows, size_t cols, void* qbuf,
+                        size_t nbits, double* r_out, int zero_threshold, int threads);
+int oracle_pack_with_headers_f64(const double* g, const double* r_in, size_t rows, size_t cols, void* qbuf,
+                                 size_t nbits, double* r_out, int zero_threshold, int threads);
+int oracle_unquantize_f64(const void* qbuf, size_t rows, size_t cols, size_t nbits, double* out,
+                          int add, int threads);
+int oracle_stripe_reduce_f64(void* const* q, size_t workers, size_t owner, size_t rows, size_t cols,
+                             size_t nbits, double* stripe_res, double* agg_scratch,
+                             int zero_threshold, int threads);
+int oracle_allreduce_f64(const double* const* g, double* const* res, void* const* q, double* const* stripe_res,
+                         size_t workers, size_t rows, size_t cols, size_t nbits, int zero_threshold,
+                         void* qagg, double* out, int threads);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,4 +1,5 @@
-"""Seeded synthetic gradients for the parity tests and the benchmark (column-major float32 numpy arrays).
+"""Seeded synthetic gradients for the parity tests and the benchmark (column-major numpy arrays, float32 unless
+`dtype=np.float64` is asked for).
 
 `exact_bell` uses integer arithmetic only, so its output is bit-identical on every machine and numpy
 version; the golden vectors whose inputs are not stored are generated from it. The other generators
@@ -13,8 +14,8 @@ def case_seed(config, matrix=0, step=0, worker=0):
     return BASE_SEED + 1000 * config + 100 * matrix + step + 10000 * worker
 
 
-def _f(a):
-    return np.asfortranarray(a.astype(np.float32))
+def _f(a, dtype=np.float32):
+    return np.asfortranarray(a.astype(dtype))
 
 
 def _splitmix64(x):
@@ -25,9 +26,11 @@ def _splitmix64(x):
     return z ^ (z >> np.uint64(31))
 
 
-def exact_bell(seed, rows, cols, shift=22):
+def exact_bell(seed, rows, cols, shift=22, dtype=np.float32):
     """Bell-shaped values (sum of four 16-bit uniforms, centred) times 2^-shift; exact in fp32.
-    Standard deviation = 2^-shift * 65536 / sqrt(3), e.g. about 0.009 for shift = 22."""
+    Standard deviation = 2^-shift * 65536 / sqrt(3), e.g. about 0.009 for shift = 22.
+    With dtype=float64 a second 16-bit uniform times 2^-52 is added (still exact), so that the values
+    use mantissa bits a float32 does not have."""
     n = rows * cols
     with np.errstate(over="ignore"):
         idx = np.arange(n, dtype=np.uint64)
@@ -35,30 +38,34 @@ def exact_bell(seed, rows, cols, shift=22):
     parts = [(z >> np.uint64(16 * k)) & np.uint64(0xFFFF) for k in range(4)]
     total = (parts[0] + parts[1] + parts[2] + parts[3]).astype(np.int64) - 2 * 65535
     vals = np.ldexp(total.astype(np.float64), -shift)
-    return _f(vals.reshape((rows, cols), order="F"))
+    if np.dtype(dtype) == np.float64:
+        with np.errstate(over="ignore"):
+            z2 = _splitmix64(z + np.uint64(0x2545F4914F6CDD1D))
+        vals = vals + np.ldexp((z2 & np.uint64(0xFFFF)).astype(np.float64), -52)
+    return _f(vals.reshape((rows, cols), order="F"), dtype)
 
 
-def uniform(seed, rows, cols, lo, hi):
+def uniform(seed, rows, cols, lo, hi, dtype=np.float32):
     rng = np.random.default_rng(seed)
-    return _f(lo + (hi - lo) * rng.random((rows, cols)))
+    return _f(lo + (hi - lo) * rng.random((rows, cols)), dtype)
 
 
-def normal(seed, rows, cols, sigma=0.01):
+def normal(seed, rows, cols, sigma=0.01, dtype=np.float32):
     rng = np.random.default_rng(seed)
-    return _f(rng.standard_normal((rows, cols)) * sigma)
+    return _f(rng.standard_normal((rows, cols)) * sigma, dtype)
 
 
-def student_t(seed, rows, cols, nu=3.0, scale=1e-3):
+def student_t(seed, rows, cols, nu=3.0, scale=1e-3, dtype=np.float32):
     rng = np.random.default_rng(seed)
-    return _f(rng.standard_t(nu, (rows, cols)) * scale)
+    return _f(rng.standard_t(nu, (rows, cols)) * scale, dtype)
 
 
-def normal_with_outliers(seed, rows, cols, sigma=0.01, frac=0.01, mult=50.0):
+def normal_with_outliers(seed, rows, cols, sigma=0.01, frac=0.01, mult=50.0, dtype=np.float32):
     rng = np.random.default_rng(seed)
     a = rng.standard_normal((rows, cols)) * sigma
     mask = rng.random((rows, cols)) < frac
     a[mask] *= mult
-    return _f(a)
+    return _f(a, dtype)
 
 
 def zero_columns(a, seed, frac=0.9):

@@ -208,15 +208,15 @@ def test_brute_force_placement(nbits):
                 assert [int(x) for x in w[j]] == expect
 
 
-def _inline_checker(nbits, g, prev_res, prev_out, zt):
+def _inline_checker(nbits, g, prev_res, prev_out, zt, passthrough_bits=32):
     """Independent float64 restatement after the reference unit test's ReferenceCPUQuantizer: row-major loops,
-    `val < mean` decisions for 1 bit, no packing at all."""
+    `val < mean` decisions for 1 bit, no packing at all. passthrough_bits = width of the QWord."""
     rows, cols = g.shape
     out = np.zeros((rows, cols))
     res = np.zeros((rows, cols))
     for j in range(cols):
         v = g[:, j].astype(np.float64) + prev_res[:, j]
-        if nbits == 32:
+        if nbits == passthrough_bits:
             out[:, j] = prev_out[:, j] + v
             continue
         mean = v.sum() / rows if (not zt and nbits == 1) else 0.0
