@@ -6,7 +6,10 @@ Python mirror of the reference's quantizer interface on top of the C ABI in
     MatrixQuantizerImpl  <->  Source/Math/MatrixQuantizerImpl.h:19-49
     QuantizedMatrix      <->  Source/Math/QuantizedMatrix.h:54-124
     MatrixQuantizer      <->  Source/1BitSGD/MatrixQuantizer.h:24-85
-    Matrix               <->  the little of Source/Math/Matrix.h the path needs (dense fp32, column-major)
+    Matrix               <->  the little of Source/Math/Matrix.h the path needs (dense, column-major)
+
+Both instantiations of the reference are served: float32 matrices with 32-bit QWords and float64 matrices with
+64-bit QWords (Source/Math/ValueQuantizer.h:36-57); the element type of the matrices selects the entry points.
 
 torch is used only as the owner of device memory. There is no CPU implementation and no fallback:
 if the HIP library is missing, importing the bindings raises.
@@ -75,6 +78,15 @@ def lib():
         L.cntkq_wait_stripe_reduce_done.argtypes = [_vp]
         L.cntkq_quantize_batch_async.argtypes = [_vp, ctypes.POINTER(_QuantizeItem), _sz, _sz, ctypes.c_int]
         L.cntkq_unquantize_batch_async.argtypes = [_vp, ctypes.POINTER(_UnquantizeItem), _sz, _sz, ctypes.c_int]
+        L.cntkq_qwords_per_col_f64.argtypes = [_sz, _sz]
+        L.cntkq_qwords_per_col_f64.restype = _sz
+        L.cntkq_qcol_bytes_f64.argtypes = [_sz, _sz]
+        L.cntkq_qcol_bytes_f64.restype = _sz
+        L.cntkq_qmatrix_bytes_f64.argtypes = [_sz, _sz, _sz]
+        L.cntkq_qmatrix_bytes_f64.restype = _sz
+        L.cntkq_quantize_async_f64.argtypes = L.cntkq_quantize_async.argtypes
+        L.cntkq_unquantize_async_f64.argtypes = L.cntkq_unquantize_async.argtypes
+        L.cntkq_stripe_reduce_async_f64.argtypes = L.cntkq_stripe_reduce_async.argtypes
         L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int]
         _lib = L
     return _lib
@@ -89,12 +101,25 @@ def _check(rc):
     raise QuantizerLogicError(msg)
 
 
-def qwords_per_col(rows, nbits):
-    return lib().cntkq_qwords_per_col(rows, nbits)
+def _is64(dtype):
+    """True for float64, False for float32 (numpy or torch dtype); anything else is refused."""
+    if dtype in (np.float32, torch.float32) or dtype == np.dtype(np.float32):
+        return False
+    if dtype in (np.float64, torch.float64) or dtype == np.dtype(np.float64):
+        return True
+    raise QuantizerLogicError("element type must be float32 or float64")
 
 
-def qcol_bytes(nbits, rows):
-    return lib().cntkq_qcol_bytes(nbits, rows)
+def _fn(name, dtype):
+    return getattr(lib(), name + ("_f64" if _is64(dtype) else ""))
+
+
+def qwords_per_col(rows, nbits, dtype=np.float32):
+    return _fn("cntkq_qwords_per_col", dtype)(rows, nbits)
+
+
+def qcol_bytes(nbits, rows, dtype=np.float32):
+    return _fn("cntkq_qcol_bytes", dtype)(nbits, rows)
 
 
 def stripe_range(cols, rank, workers):
@@ -108,33 +133,40 @@ def stripe_range(cols, rank, workers):
 
 
 class Matrix:
-    """Dense fp32 matrix in column-major storage on one device (Source/Math/Matrix.h, the part used here).
+    """Dense float32 or float64 matrix in column-major storage on one device (Source/Math/Matrix.h, the part used
+    here: Matrix<float> / Matrix<double>).
 
-    ``data`` is a flat torch tensor of rows * cols floats: element (i, j) is data[j * rows + i].
+    ``data`` is a flat torch tensor of rows * cols elements: element (i, j) is data[j * rows + i].
     """
 
-    def __init__(self, rows, cols, device_id=0, data=None):
+    def __init__(self, rows, cols, device_id=0, data=None, dtype=torch.float32):
         self.rows, self.cols, self.device_id = int(rows), int(cols), device_id
         if data is None:
             dev = "cpu" if device_id < 0 else "cuda:%d" % device_id
-            data = torch.zeros(self.rows * self.cols, dtype=torch.float32, device=dev)
-        if data.dtype != torch.float32 or data.dim() != 1 or data.numel() != self.rows * self.cols:
-            raise QuantizerLogicError("Matrix data must be a flat float32 tensor of rows * cols elements")
+            data = torch.zeros(self.rows * self.cols, dtype=torch.float64 if _is64(dtype) else torch.float32, device=dev)
+        if data.dtype not in (torch.float32, torch.float64) or data.dim() != 1 or data.numel() != self.rows * self.cols:
+            raise QuantizerLogicError("Matrix data must be a flat float32 or float64 tensor of rows * cols elements")
         if not data.is_contiguous():
             raise QuantizerLogicError("Matrix data must be contiguous")
         self.data = data
 
+    @property
+    def dtype(self):
+        return self.data.dtype
+
     @classmethod
     def from_numpy(cls, a, device_id=0):
-        """From a (rows, cols) float32 numpy array; the values are laid out column-major on the device."""
-        a = np.asfortranarray(a, dtype=np.float32)
+        """From a (rows, cols) float32 / float64 numpy array (anything else becomes float32); the values are laid
+        out column-major on the device."""
+        a = np.asarray(a)
+        a = np.asfortranarray(a, dtype=a.dtype if a.dtype == np.float64 else np.float32)
         flat = torch.from_numpy(a.reshape(-1, order="F").copy())
         if device_id >= 0:
             flat = flat.to("cuda:%d" % device_id)
         return cls(a.shape[0], a.shape[1], device_id, flat)
 
     def to_numpy(self):
-        """(rows, cols) float32 numpy array in Fortran order."""
+        """(rows, cols) numpy array in Fortran order."""
         return np.asfortranarray(self.data.detach().cpu().numpy().reshape((self.rows, self.cols), order="F"))
 
     def GetNumRows(self):
@@ -161,19 +193,23 @@ class Matrix:
 
 
 class QuantizedMatrix:
-    """Packed matrix: per column {f32 lower, f32 upper, u32 bits[nq]} (Source/Math/QuantizedMatrix.h:27-124).
+    """Packed matrix: per column {lower, upper, bits[nq]} (Source/Math/QuantizedMatrix.h:27-124); float and 32-bit
+    QWords for dtype float32, double and 64-bit QWords for float64.
 
     device_id >= 0 keeps the buffer on that GPU; CPUDEVICE keeps it in pinned host memory, as the
     reference's v1 aggregator does through its page-locked allocator
     (Source/1BitSGD/AllReduceDistGradAggregator.h:76-77, 88).
     """
 
-    def __init__(self, num_rows, num_cols, nbits, device_id=0, _buffer=None):
-        if nbits not in (1, 2, 4, 8, 16, 32):
+    def __init__(self, num_rows, num_cols, nbits, device_id=0, _buffer=None, dtype=torch.float32):
+        self.is64 = _is64(dtype)
+        word_bits = 64 if self.is64 else 32
+        if nbits not in (1, 2, 4, 8, 16, 32, 64) or nbits > word_bits:
             # Source/Math/QuantizedMatrix.cpp:12-15
-            raise QuantizerLogicError("Quantization: 'nbits' must be a power of two that divides 32")
+            raise QuantizerLogicError("Quantization: 'nbits' must be a power of two that divides %d" % word_bits)
         self.num_rows, self.num_cols, self.nbits, self.device_id = int(num_rows), int(num_cols), int(nbits), device_id
-        self.qcol_size = qcol_bytes(nbits, self.num_rows)
+        self.dtype = torch.float64 if self.is64 else torch.float32
+        self.qcol_size = qcol_bytes(nbits, self.num_rows, self.dtype)
         size = self.qcol_size * self.num_cols
         if _buffer is None:
             if device_id < 0:
@@ -205,7 +241,7 @@ class QuantizedMatrix:
         if start_col + num_cols > self.num_cols:
             raise QuantizerLogicError("ColumnSlice out of range")
         view = self.buffer[start_col * self.qcol_size:(start_col + num_cols) * self.qcol_size]
-        return QuantizedMatrix(self.num_rows, num_cols, self.nbits, self.device_id, view)
+        return QuantizedMatrix(self.num_rows, num_cols, self.nbits, self.device_id, view, dtype=self.dtype)
 
     def to_numpy(self):
         return self.buffer.detach().cpu().numpy().copy()
@@ -252,7 +288,9 @@ class MatrixQuantizerImpl:
         for m in (in_residual, out_residual, out_qmatrix):
             if m.GetNumRows() != rows or m.GetNumCols() != cols:
                 raise QuantizerLogicError("QuantizeAsync: matrix dimensions do not match")
-        _check(lib().cntkq_quantize_async(self._h, in_matrix.Data(), in_residual.Data(), rows, cols,
+            if m.dtype != in_matrix.dtype:
+                raise QuantizerLogicError("QuantizeAsync: element types do not match")
+        _check(_fn("cntkq_quantize_async", in_matrix.dtype)(self._h, in_matrix.Data(), in_residual.Data(), rows, cols,
                                           out_qmatrix.Buffer(), out_qmatrix.GetSize(),
                                           int(out_qmatrix.GetDeviceId() < 0), out_qmatrix.GetNumBits(),
                                           out_residual.Data(), int(bool(zero_threshold_for_1bit))))
@@ -265,7 +303,9 @@ class MatrixQuantizerImpl:
         # the reference asserts this (Source/Math/MatrixQuantizerGPU.cu:297)
         if in_qmatrix.GetNumRows() != rows or in_qmatrix.GetNumCols() != cols:
             raise QuantizerLogicError("UnquantizeAsync: matrix dimensions do not match")
-        _check(lib().cntkq_unquantize_async(self._h, in_qmatrix.Buffer(), in_qmatrix.GetSize(),
+        if in_qmatrix.dtype != out_matrix.dtype:
+            raise QuantizerLogicError("UnquantizeAsync: element types do not match")
+        _check(_fn("cntkq_unquantize_async", out_matrix.dtype)(self._h, in_qmatrix.Buffer(), in_qmatrix.GetSize(),
                                             int(in_qmatrix.GetDeviceId() < 0), out_matrix.Data(), rows, cols,
                                             in_qmatrix.GetNumBits(), int(bool(add))))
 
@@ -287,6 +327,8 @@ class MatrixQuantizerImpl:
                     raise QuantizerLogicError("QuantizeBatchAsync: matrix dimensions do not match")
             if q.GetNumBits() != nbits or q.GetDeviceId() < 0:
                 raise QuantizerLogicError("QuantizeBatchAsync: packed matrices must share one bit width and live on the device")
+            if any(m.dtype != torch.float32 for m in (g, r_in, r_out, q)):
+                raise QuantizerLogicError("QuantizeBatchAsync: the batched calls exist for float32 only")
             arr[k] = _QuantizeItem(g.Data(), r_in.Data(), r_out.Data(), q.Buffer(), rows, cols)
         _check(lib().cntkq_quantize_batch_async(self._h, arr, len(items), nbits, int(bool(zero_threshold_for_1bit))))
 
@@ -302,6 +344,8 @@ class MatrixQuantizerImpl:
                 raise QuantizerLogicError("UnquantizeBatchAsync: matrix dimensions do not match")
             if q.GetNumBits() != nbits or q.GetDeviceId() < 0:
                 raise QuantizerLogicError("UnquantizeBatchAsync: packed matrices must share one bit width and live on the device")
+            if q.dtype != torch.float32 or out.dtype != torch.float32:
+                raise QuantizerLogicError("UnquantizeBatchAsync: the batched calls exist for float32 only")
             arr[k] = _UnquantizeItem(q.Buffer(), out.Data(), out.GetNumRows(), out.GetNumCols())
         _check(lib().cntkq_unquantize_batch_async(self._h, arr, len(items), nbits, int(bool(add))))
 
@@ -313,10 +357,14 @@ class MatrixQuantizerImpl:
         for s in stripes:
             if s.GetNumRows() != rows or s.GetNumCols() != cols or s.GetNumBits() != nbits or s.GetDeviceId() < 0:
                 raise QuantizerLogicError("StripeReduceAsync: stripes must be device-resident and of equal shape")
+            if s.dtype != out_qstripe.dtype:
+                raise QuantizerLogicError("StripeReduceAsync: element types do not match")
         if stripe_residual.GetNumRows() != rows or stripe_residual.GetNumCols() != cols:
             raise QuantizerLogicError("StripeReduceAsync: stripe residual has the wrong shape")
+        if stripe_residual.dtype != out_qstripe.dtype or (agg_out is not None and agg_out.dtype != out_qstripe.dtype):
+            raise QuantizerLogicError("StripeReduceAsync: element types do not match")
         arr = (_vp * k)(*[s.Buffer() for s in stripes])
-        _check(lib().cntkq_stripe_reduce_async(self._h, arr, k, owner, rows, cols, nbits, stripe_residual.Data(),
+        _check(_fn("cntkq_stripe_reduce_async", out_qstripe.dtype)(self._h, arr, k, owner, rows, cols, nbits, stripe_residual.Data(),
                                                out_qstripe.Buffer(), agg_out.Data() if agg_out is not None else None,
                                                int(bool(zero_threshold_for_1bit))))
 
@@ -330,9 +378,9 @@ class MatrixQuantizerImpl:
 class MatrixQuantizer:
     """Quantizer that owns its error-feedback residual (Source/1BitSGD/MatrixQuantizer.h:24-85)."""
 
-    def __init__(self, num_rows, num_cols, device_id, use_async):
+    def __init__(self, num_rows, num_cols, device_id, use_async, dtype=torch.float32):
         self._impl = MatrixQuantizerImpl.Create(device_id, use_async)
-        self._residual = Matrix(num_rows, num_cols, device_id)
+        self._residual = Matrix(num_rows, num_cols, device_id, dtype=dtype)
 
     def QuantizeAsync(self, in_matrix, out_qmatrix, zero_threshold_for_1bit, in_residual=None, out_residual=None):
         if in_residual is None:

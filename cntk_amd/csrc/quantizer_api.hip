@@ -3,6 +3,7 @@
 #include "../../include/cntk_amd_quantizer.h"
 #include "quantizer_internal.h"
 #include "quantizer_launch.h"
+#include "quantizer_launch_f64.h"
 
 #include <hip/hip_runtime.h>
 
@@ -69,6 +70,66 @@ private:
 bool aligned4(const void* p)
 {
     return (reinterpret_cast<uintptr_t>(p) & 3u) == 0;
+}
+
+// What differs between the two instantiations of the boundary (MatrixQuantizerImpl<float> / <double>).
+template <typename E>
+struct Elem;
+
+template <>
+struct Elem<float>
+{
+    static constexpr size_t kAlign = 4;
+    static constexpr size_t kWordBits = 32;
+    static constexpr uint32_t kStripeMaxRows = cntkq::kTileMaxRows;
+    static bool valid_nbits(size_t nbits) { return cntkq::valid_nbits(nbits); }
+    static size_t qcol_bytes(size_t nbits, size_t rows) { return cntkq::qcol_bytes(nbits, rows); }
+    static hipError_t quantize(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, void* q, size_t rows,
+                               size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+    {
+        return cntkq::launch_quantize(s, ev, g, r_in, r_out, q, rows, cols, nbits, zt, tune);
+    }
+    static hipError_t unquantize(hipStream_t s, LaunchEvents ev, const void* q, float* out, size_t rows, size_t cols, size_t nbits,
+                                 bool add, const LaunchTuning& tune)
+    {
+        return cntkq::launch_unquantize(s, ev, q, out, rows, cols, nbits, add, tune);
+    }
+    static hipError_t stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, void* q_out,
+                                    float* agg_out, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+    {
+        return cntkq::launch_stripe_reduce(s, ev, src, stripe_res, q_out, agg_out, rows, cols, nbits, zt, tune);
+    }
+};
+
+template <>
+struct Elem<double>
+{
+    static constexpr size_t kAlign = 8;
+    static constexpr size_t kWordBits = 64;
+    static constexpr uint32_t kStripeMaxRows = cntkq::f64::kTileMaxRows;
+    static bool valid_nbits(size_t nbits) { return cntkq::f64::valid_nbits(nbits); }
+    static size_t qcol_bytes(size_t nbits, size_t rows) { return cntkq::f64::qcol_bytes(nbits, rows); }
+    static hipError_t quantize(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, void* q, size_t rows,
+                               size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+    {
+        return cntkq::f64::launch_quantize(s, ev, g, r_in, r_out, q, rows, cols, nbits, zt, tune);
+    }
+    static hipError_t unquantize(hipStream_t s, LaunchEvents ev, const void* q, double* out, size_t rows, size_t cols, size_t nbits,
+                                 bool add, const LaunchTuning& tune)
+    {
+        return cntkq::f64::launch_unquantize(s, ev, q, out, rows, cols, nbits, add, tune);
+    }
+    static hipError_t stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, double* stripe_res, void* q_out,
+                                    double* agg_out, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+    {
+        return cntkq::f64::launch_stripe_reduce(s, ev, src, stripe_res, q_out, agg_out, rows, cols, nbits, zt, tune);
+    }
+};
+
+template <typename E>
+bool aligned_for(const void* p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & (Elem<E>::kAlign - 1)) == 0;
 }
 
 } // namespace
@@ -197,6 +258,157 @@ int sync_event(hipEvent_t ev) // SyncEvent (Source/Math/MatrixQuantizerGPU.cu:68
     return CNTKQ_OK;
 }
 
+
+// ---- the three asynchronous calls, written once for both element types ----------------------------------
+
+template <typename E>
+int quantize_async_impl(cntkq_quantizer* h, const E* in, const E* res_in, size_t rows, size_t cols, void* qbuf, size_t qbuf_bytes,
+                        int qbuf_on_host, size_t nbits, E* res_out, int zero_threshold_for_1bit)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: null handle");
+    if (!Elem<E>::valid_nbits(nbits))
+        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides %zu (got %zu)", Elem<E>::kWordBits, nbits);
+    if (rows >= (1ull << 31) || cols >= (1ull << 31))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: rows and cols must be below 2^31");
+    const size_t need = Elem<E>::qcol_bytes(nbits, rows) * cols;
+    if (qbuf_bytes != need)
+        return fail(CNTKQ_LOGIC_ERROR,
+                    "quantize: packed buffer of %zu bytes does not match %zu x %zu at %zu bits (%zu bytes)", qbuf_bytes,
+                    rows, cols, nbits, need);
+    h->quantize_included_fetch = false;
+    if (rows == 0 || cols == 0)
+        return CNTKQ_OK;
+    if (in == nullptr || res_in == nullptr || res_out == nullptr || qbuf == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: null matrix pointer");
+    if (!aligned_for<E>(in) || !aligned_for<E>(res_in) || !aligned_for<E>(res_out) || !aligned_for<E>(qbuf))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: pointers must be %zu-byte aligned", Elem<E>::kAlign);
+
+    DeviceGuard guard(h->device);
+    hipStream_t s = work_stream(h);
+    char* qdev = static_cast<char*>(qbuf);
+    if (qbuf_on_host)
+    {
+        int rc = ensure_staging(h, need);
+        if (rc != CNTKQ_OK)
+            return rc;
+        // a copy out of the staging buffer issued earlier must have drained before it is overwritten
+        if (h->fetch_pending)
+            HIP_TRY(hipStreamWaitEvent(s, h->ev_fetch, 0), "hipStreamWaitEvent failed");
+        qdev = h->staging;
+    }
+
+    const LaunchEvents ev = take_events(h, h->ev_quantize);
+    hipError_t lrc = Elem<E>::quantize(s, ev, in, res_in, res_out, qdev, rows, cols, nbits, zero_threshold_for_1bit != 0, h->tune);
+    if (lrc == hipErrorInvalidValue)
+        return fail(CNTKQ_INVALID_ARGUMENT, "quantize: the forced kernel path does not support %zu x %zu at %zu bits", rows, cols, nbits);
+    HIP_TRY(lrc, "quantize kernel launch failed");
+    h->last_quantize = ev.stop;
+
+    if (qbuf_on_host)
+    {
+        HIP_TRY(hipStreamWaitEvent(h->fetch, ev.stop, 0), "hipStreamWaitEvent failed");
+        HIP_TRY(hipMemcpyAsync(qbuf, qdev, need, hipMemcpyDeviceToHost, h->fetch), "hipMemcpyAsync failed");
+        HIP_TRY(hipEventRecord(h->ev_fetch, h->fetch), "hipEventRecord failed");
+        h->quantize_included_fetch = true;
+        h->fetch_pending = true;
+    }
+    return CNTKQ_OK;
+}
+
+template <typename E>
+int unquantize_async_impl(cntkq_quantizer* h, const void* qbuf, size_t qbuf_bytes, int qbuf_on_host, E* out, size_t rows, size_t cols,
+                          size_t nbits, int add)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: null handle");
+    if (!Elem<E>::valid_nbits(nbits))
+        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides %zu (got %zu)", Elem<E>::kWordBits, nbits);
+    if (rows >= (1ull << 31) || cols >= (1ull << 31))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: rows and cols must be below 2^31");
+    const size_t need = Elem<E>::qcol_bytes(nbits, rows) * cols;
+    if (qbuf_bytes != need)
+        return fail(CNTKQ_LOGIC_ERROR,
+                    "unquantizestripe: dimension of patch to be unquantized does not match size of quantized data "
+                    "(%zu bytes given, %zu x %zu at %zu bits needs %zu)", qbuf_bytes, rows, cols, nbits, need);
+    if (qbuf_bytes == 0 || rows == 0 || cols == 0)
+        return CNTKQ_OK; // empty buffer: empty matrix, nothing to do
+    if (qbuf == nullptr || out == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: null matrix pointer");
+    if (!aligned_for<E>(qbuf) || !aligned_for<E>(out))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: pointers must be %zu-byte aligned", Elem<E>::kAlign);
+
+    DeviceGuard guard(h->device);
+    hipStream_t s = work_stream(h);
+    const char* qdev = static_cast<const char*>(qbuf);
+    if (qbuf_on_host)
+    {
+        int rc = ensure_staging(h, need);
+        if (rc != CNTKQ_OK)
+            return rc;
+        // the staging buffer may still be read by an earlier kernel or copied out by an earlier fetch
+        HIP_TRY(hipEventRecord(h->ev_assign, s), "hipEventRecord failed");
+        HIP_TRY(hipStreamWaitEvent(h->assign, h->ev_assign, 0), "hipStreamWaitEvent failed");
+        if (h->fetch_pending)
+            HIP_TRY(hipStreamWaitEvent(h->assign, h->ev_fetch, 0), "hipStreamWaitEvent failed");
+        HIP_TRY(hipMemcpyAsync(h->staging, qbuf, need, hipMemcpyHostToDevice, h->assign), "hipMemcpyAsync failed");
+        HIP_TRY(hipEventRecord(h->ev_assign, h->assign), "hipEventRecord failed");
+        HIP_TRY(hipStreamWaitEvent(s, h->ev_assign, 0), "hipStreamWaitEvent failed");
+        qdev = h->staging;
+    }
+    const LaunchEvents ev = take_events(h, h->ev_unquantize);
+    hipError_t lrc = Elem<E>::unquantize(s, ev, qdev, out, rows, cols, nbits, add != 0, h->tune);
+    if (lrc == hipErrorInvalidValue)
+        return fail(CNTKQ_INVALID_ARGUMENT, "unquantize: %zu x %zu at %zu bits is too large for one launch", rows, cols, nbits);
+    HIP_TRY(lrc, "unquantize kernel launch failed");
+    h->last_unquantize = ev.stop;
+    return CNTKQ_OK;
+}
+
+template <typename E>
+int stripe_reduce_async_impl(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows,
+                             size_t stripe_cols, size_t nbits, E* stripe_res, void* q_out, E* agg_out, int zero_threshold_for_1bit)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: null handle");
+    if (!Elem<E>::valid_nbits(nbits))
+        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides %zu (got %zu)", Elem<E>::kWordBits, nbits);
+    if (workers == 0 || workers > CNTKQ_MAX_WORKERS || owner >= workers || stripes == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: need 1 <= workers <= %d and owner < workers",
+                    CNTKQ_MAX_WORKERS);
+    if (rows >= (1ull << 31) || stripe_cols >= (1ull << 31))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: rows and cols must be below 2^31");
+    if (rows == 0 || stripe_cols == 0)
+        return CNTKQ_OK;
+    if (rows > Elem<E>::kStripeMaxRows)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: columns taller than %u rows are not supported",
+                    Elem<E>::kStripeMaxRows);
+    if (stripe_res == nullptr || q_out == nullptr || !aligned_for<E>(stripe_res) || !aligned_for<E>(q_out) || !aligned_for<E>(agg_out))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: null or misaligned matrix pointer");
+    StripeSources src;
+    std::memset(&src, 0, sizeof src);
+    for (size_t w = 0; w < workers; ++w)
+    {
+        if (stripes[w] == nullptr || !aligned_for<E>(stripes[w]))
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: stripe %zu is null or misaligned", w);
+        src.q[w] = static_cast<const char*>(stripes[w]);
+    }
+    src.workers = (uint32_t) workers;
+    src.owner = (uint32_t) owner;
+
+    DeviceGuard guard(h->device);
+    hipStream_t s = work_stream(h);
+    const LaunchEvents ev = take_events(h, h->ev_stripe);
+    hipError_t lrc = Elem<E>::stripe_reduce(s, ev, src, stripe_res, q_out, agg_out, rows, stripe_cols, nbits,
+                                            zero_threshold_for_1bit != 0, h->tune);
+    if (lrc == hipErrorInvalidValue)
+        return fail(CNTKQ_INVALID_ARGUMENT, "stripe reduction: %zu rows with %zu workers at %zu bits does not fit the kernel", rows, workers,
+                    nbits);
+    HIP_TRY(lrc, "stripe reduction kernel launch failed");
+    h->last_stripe = ev.stop;
+    return CNTKQ_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -219,6 +431,21 @@ size_t cntkq_qcol_bytes(size_t nbits, size_t rows)
 size_t cntkq_qmatrix_bytes(size_t rows, size_t cols, size_t nbits)
 {
     return valid_nbits(nbits) ? qcol_bytes(nbits, rows) * cols : 0;
+}
+
+size_t cntkq_qwords_per_col_f64(size_t rows, size_t nbits)
+{
+    return f64::valid_nbits(nbits) ? f64::qwords_per_col(rows, nbits) : 0;
+}
+
+size_t cntkq_qcol_bytes_f64(size_t nbits, size_t rows)
+{
+    return f64::valid_nbits(nbits) ? f64::qcol_bytes(nbits, rows) : 0;
+}
+
+size_t cntkq_qmatrix_bytes_f64(size_t rows, size_t cols, size_t nbits)
+{
+    return f64::valid_nbits(nbits) ? f64::qcol_bytes(nbits, rows) * cols : 0;
 }
 
 int cntkq_stripe_range(size_t cols, size_t rank, size_t workers, size_t* start_col, size_t* num_cols)
@@ -359,55 +586,13 @@ int cntkq_sync_with_main_stream(cntkq_quantizer* h)
 int cntkq_quantize_async(cntkq_quantizer* h, const float* in, const float* res_in, size_t rows, size_t cols, void* qbuf,
                          size_t qbuf_bytes, int qbuf_on_host, size_t nbits, float* res_out, int zero_threshold_for_1bit)
 {
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: null handle");
-    if (!valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
-    if (rows >= (1ull << 31) || cols >= (1ull << 31))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: rows and cols must be below 2^31");
-    const size_t need = qcol_bytes(nbits, rows) * cols;
-    if (qbuf_bytes != need)
-        return fail(CNTKQ_LOGIC_ERROR,
-                    "quantize: packed buffer of %zu bytes does not match %zu x %zu at %zu bits (%zu bytes)", qbuf_bytes,
-                    rows, cols, nbits, need);
-    h->quantize_included_fetch = false;
-    if (rows == 0 || cols == 0)
-        return CNTKQ_OK;
-    if (in == nullptr || res_in == nullptr || res_out == nullptr || qbuf == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: null matrix pointer");
-    if (!aligned4(in) || !aligned4(res_in) || !aligned4(res_out) || !aligned4(qbuf))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: pointers must be 4-byte aligned");
+    return quantize_async_impl<float>(h, in, res_in, rows, cols, qbuf, qbuf_bytes, qbuf_on_host, nbits, res_out, zero_threshold_for_1bit);
+}
 
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    char* qdev = static_cast<char*>(qbuf);
-    if (qbuf_on_host)
-    {
-        int rc = ensure_staging(h, need);
-        if (rc != CNTKQ_OK)
-            return rc;
-        // a copy out of the staging buffer issued earlier must have drained before it is overwritten
-        if (h->fetch_pending)
-            HIP_TRY(hipStreamWaitEvent(s, h->ev_fetch, 0), "hipStreamWaitEvent failed");
-        qdev = h->staging;
-    }
-
-    const LaunchEvents ev = take_events(h, h->ev_quantize);
-    hipError_t lrc = launch_quantize(s, ev, in, res_in, res_out, qdev, rows, cols, nbits, zero_threshold_for_1bit != 0, h->tune);
-    if (lrc == hipErrorInvalidValue)
-        return fail(CNTKQ_INVALID_ARGUMENT, "quantize: the forced kernel path does not support %zu x %zu at %zu bits", rows, cols, nbits);
-    HIP_TRY(lrc, "quantize kernel launch failed");
-    h->last_quantize = ev.stop;
-
-    if (qbuf_on_host)
-    {
-        HIP_TRY(hipStreamWaitEvent(h->fetch, ev.stop, 0), "hipStreamWaitEvent failed");
-        HIP_TRY(hipMemcpyAsync(qbuf, qdev, need, hipMemcpyDeviceToHost, h->fetch), "hipMemcpyAsync failed");
-        HIP_TRY(hipEventRecord(h->ev_fetch, h->fetch), "hipEventRecord failed");
-        h->quantize_included_fetch = true;
-        h->fetch_pending = true;
-    }
-    return CNTKQ_OK;
+int cntkq_quantize_async_f64(cntkq_quantizer* h, const double* in, const double* res_in, size_t rows, size_t cols, void* qbuf,
+                             size_t qbuf_bytes, int qbuf_on_host, size_t nbits, double* res_out, int zero_threshold_for_1bit)
+{
+    return quantize_async_impl<double>(h, in, res_in, rows, cols, qbuf, qbuf_bytes, qbuf_on_host, nbits, res_out, zero_threshold_for_1bit);
 }
 
 int cntkq_wait_quantize_done(cntkq_quantizer* h)
@@ -428,46 +613,13 @@ int cntkq_wait_quantize_done(cntkq_quantizer* h)
 int cntkq_unquantize_async(cntkq_quantizer* h, const void* qbuf, size_t qbuf_bytes, int qbuf_on_host, float* out,
                            size_t rows, size_t cols, size_t nbits, int add)
 {
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: null handle");
-    if (!valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
-    if (rows >= (1ull << 31) || cols >= (1ull << 31))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: rows and cols must be below 2^31");
-    const size_t need = qcol_bytes(nbits, rows) * cols;
-    if (qbuf_bytes != need)
-        return fail(CNTKQ_LOGIC_ERROR,
-                    "unquantizestripe: dimension of patch to be unquantized does not match size of quantized data "
-                    "(%zu bytes given, %zu x %zu at %zu bits needs %zu)", qbuf_bytes, rows, cols, nbits, need);
-    if (qbuf_bytes == 0 || rows == 0 || cols == 0)
-        return CNTKQ_OK; // empty buffer: empty matrix, nothing to do
-    if (qbuf == nullptr || out == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: null matrix pointer");
-    if (!aligned4(qbuf) || !aligned4(out))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: pointers must be 4-byte aligned");
+    return unquantize_async_impl<float>(h, qbuf, qbuf_bytes, qbuf_on_host, out, rows, cols, nbits, add);
+}
 
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    const char* qdev = static_cast<const char*>(qbuf);
-    if (qbuf_on_host)
-    {
-        int rc = ensure_staging(h, need);
-        if (rc != CNTKQ_OK)
-            return rc;
-        // the staging buffer may still be read by an earlier kernel or copied out by an earlier fetch
-        HIP_TRY(hipEventRecord(h->ev_assign, s), "hipEventRecord failed");
-        HIP_TRY(hipStreamWaitEvent(h->assign, h->ev_assign, 0), "hipStreamWaitEvent failed");
-        if (h->fetch_pending)
-            HIP_TRY(hipStreamWaitEvent(h->assign, h->ev_fetch, 0), "hipStreamWaitEvent failed");
-        HIP_TRY(hipMemcpyAsync(h->staging, qbuf, need, hipMemcpyHostToDevice, h->assign), "hipMemcpyAsync failed");
-        HIP_TRY(hipEventRecord(h->ev_assign, h->assign), "hipEventRecord failed");
-        HIP_TRY(hipStreamWaitEvent(s, h->ev_assign, 0), "hipStreamWaitEvent failed");
-        qdev = h->staging;
-    }
-    const LaunchEvents ev = take_events(h, h->ev_unquantize);
-    HIP_TRY(launch_unquantize(s, ev, qdev, out, rows, cols, nbits, add != 0, h->tune), "unquantize kernel launch failed");
-    h->last_unquantize = ev.stop;
-    return CNTKQ_OK;
+int cntkq_unquantize_async_f64(cntkq_quantizer* h, const void* qbuf, size_t qbuf_bytes, int qbuf_on_host, double* out,
+                               size_t rows, size_t cols, size_t nbits, int add)
+{
+    return unquantize_async_impl<double>(h, qbuf, qbuf_bytes, qbuf_on_host, out, rows, cols, nbits, add);
 }
 
 int cntkq_wait_unquantize_done(cntkq_quantizer* h)
@@ -683,41 +835,16 @@ int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, si
                               size_t stripe_cols, size_t nbits, float* stripe_res, void* q_out, float* agg_out,
                               int zero_threshold_for_1bit)
 {
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: null handle");
-    if (!valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
-    if (workers == 0 || workers > CNTKQ_MAX_WORKERS || owner >= workers || stripes == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: need 1 <= workers <= %d and owner < workers",
-                    CNTKQ_MAX_WORKERS);
-    if (rows >= (1ull << 31) || stripe_cols >= (1ull << 31))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: rows and cols must be below 2^31");
-    if (rows == 0 || stripe_cols == 0)
-        return CNTKQ_OK;
-    if (rows > kTileMaxRows)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: columns taller than %u rows are not supported",
-                    kTileMaxRows);
-    if (stripe_res == nullptr || q_out == nullptr || !aligned4(stripe_res) || !aligned4(q_out) || !aligned4(agg_out))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: null or misaligned matrix pointer");
-    StripeSources src;
-    std::memset(&src, 0, sizeof src);
-    for (size_t w = 0; w < workers; ++w)
-    {
-        if (stripes[w] == nullptr || !aligned4(stripes[w]))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: stripe %zu is null or misaligned", w);
-        src.q[w] = static_cast<const char*>(stripes[w]);
-    }
-    src.workers = (uint32_t) workers;
-    src.owner = (uint32_t) owner;
+    return stripe_reduce_async_impl<float>(h, stripes, workers, owner, rows, stripe_cols, nbits, stripe_res, q_out, agg_out,
+                                           zero_threshold_for_1bit);
+}
 
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    const LaunchEvents ev = take_events(h, h->ev_stripe);
-    HIP_TRY(launch_stripe_reduce(s, ev, src, stripe_res, q_out, agg_out, rows, stripe_cols, nbits,
-                                 zero_threshold_for_1bit != 0, h->tune),
-            "stripe reduction kernel launch failed");
-    h->last_stripe = ev.stop;
-    return CNTKQ_OK;
+int cntkq_stripe_reduce_async_f64(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows,
+                                  size_t stripe_cols, size_t nbits, double* stripe_res, void* q_out, double* agg_out,
+                                  int zero_threshold_for_1bit)
+{
+    return stripe_reduce_async_impl<double>(h, stripes, workers, owner, rows, stripe_cols, nbits, stripe_res, q_out, agg_out,
+                                            zero_threshold_for_1bit);
 }
 
 int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h)

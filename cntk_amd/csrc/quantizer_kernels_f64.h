@@ -1,0 +1,657 @@
+// gfx950 kernels of the per-column gradient quantizer, double-precision instantiation
+// (MatrixQuantizerImpl<double>: QWord = 64-bit, Source/Math/ValueQuantizer.h:50-57).
+//
+// Packed layout (Source/Math/QuantizedMatrix.h:27-48 with ElemType = double):
+//   column j = { f64 lower; f64 upper; u64 bits[nq] } at byte j * qcol,  nq = ceil(rows / (64 / NBITS));
+//   element i of the column is in bits[i % nq] at bit (i / nq) * NBITS. NBITS is 1, 2, 4, ..., 64 (64 = pass-through).
+// Every record is a multiple of 8 bytes, so all headers and QWords are naturally aligned.
+//
+// Work decomposition mirrors the fp32 tile kernels: a workgroup owns a run of consecutive columns, reads gradient and
+// residual once, keeps v = g + r in LDS as doubles, takes the statistics from LDS, packs, writes the residual.
+// Columns too tall for LDS take the one-workgroup-per-column kernel that re-reads global memory.
+// All arithmetic is separately rounded IEEE fp64 (compile with -ffp-contract=off).
+#pragma once
+
+#include "quantizer_kernels.h"
+
+namespace cntkq {
+namespace f64 {
+
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+
+constexpr uint32_t kThreads = 256;
+constexpr uint32_t kMaxTileCols = 32;
+// LDS prefix in 8-byte units: 4 double + 4 slots holding one uint32 each for the reductions, then (lower, upper) per column
+constexpr uint32_t kPrefixWords = 8 + 2 * kMaxTileCols;
+
+// ---- per-value quantizer (Source/Math/ValueQuantizer.h:68-156 with ElemType = double) ----------------
+
+struct ValueQ
+{
+    double lo, hi, mid, qf, uf;
+};
+
+template <int NBITS>
+__device__ __forceinline__ ValueQ make_vq(double lo, double hi)
+{
+    constexpr uint64_t rangeend = (NBITS >= 64) ? 0ull : (1ull << (NBITS & 63));
+    ValueQ v;
+    v.lo = lo;
+    v.hi = hi;
+    const double span = hi - lo;
+    // the reference compares with the float literal 1e-36f, converted to double
+    if ((span < (double) 1e-36f) || (rangeend == 0))
+    {
+        v.qf = 0.0;
+        v.uf = 0.0;
+    }
+    else
+    {
+        constexpr double used = (double) (rangeend - (NBITS > 1 ? 1ull : 0ull)); // exact: at most 2^32 - 1
+        v.qf = used / span;
+        v.uf = span / used;
+    }
+    v.mid = 0.5 * (hi + lo);
+    return v;
+}
+
+template <int NBITS, bool ZT>
+__device__ __forceinline__ uint64_t quantize_value(const ValueQ& v, double u)
+{
+    if constexpr (NBITS == 64)
+    {
+        return (uint64_t) __double_as_longlong(u);
+    }
+    else if constexpr (NBITS == 1)
+    {
+        return ZT ? (u >= 0.0 ? 1ull : 0ull) : (u >= v.mid ? 1ull : 0ull);
+    }
+    else
+    {
+        constexpr uint64_t top = (1ull << (NBITS & 63)) - 1ull;
+        if (u <= v.lo)
+            return 0ull;
+        if (u >= v.hi)
+            return top;
+        return (uint64_t) (int64_t) ((u - v.lo) * v.qf);
+    }
+}
+
+// (q + 0.5) * uf + lo, multiply and add rounded separately
+template <int NBITS>
+__device__ __forceinline__ double unquantize_value(double uf, double lo, uint64_t q)
+{
+    if constexpr (NBITS == 64)
+    {
+        return __longlong_as_double((long long) q);
+    }
+    else
+    {
+        // codes are below 2^32 here, so the conversion is exact whichever way it is done
+        double t = (double) (uint32_t) q + 0.5;
+        t = t * uf;
+        return t + lo;
+    }
+}
+
+// ---- column header from reduced sums (Source/Math/ColumnQuantizer.h:265-340) --------------------------
+
+template <bool ZT>
+__device__ __forceinline__ void finish_stats_1bit(double mean, double s0, double s1, uint32_t n0, uint32_t n1,
+                                                  uint32_t rows, double& lo, double& hi)
+{
+    double radius, centre;
+    if constexpr (!ZT)
+    {
+        const double dev0 = ((double) n0 * mean) - s0;
+        const double dev1 = s1 - ((double) n1 * mean);
+        const double dev = (dev0 + dev1) / (double) rows;
+        radius = 2.0 * dev;
+        centre = mean;
+    }
+    else
+    {
+        if (n0 == 0)
+            n0 = 1;
+        if (n1 == 0)
+            n1 = 1;
+        const double m0 = s0 / (double) n0;
+        const double m1 = s1 / (double) n1;
+        centre = 0.5 * (m0 + m1);
+        radius = 2.0 * (m1 - centre);
+    }
+    lo = centre - radius;
+    hi = centre + radius;
+}
+
+__device__ __forceinline__ void finish_stats_multibit(double sumsq, uint32_t rows, double& lo, double& hi)
+{
+    const double mean = 0.0;
+    const double sd = sqrt(sumsq / (double) rows);
+    const double half = 4.0 * sd;
+    lo = mean - half;
+    hi = mean + half;
+}
+
+// ---- geometry -------------------------------------------------------------------------------------------
+
+template <int NBITS>
+struct PackShape
+{
+    static constexpr uint32_t VPW = 64 / NBITS;          // values per QWord
+    static constexpr uint32_t SLOTS = VPW < 8 ? VPW : 8; // bit positions per work item
+    static constexpr uint32_t CHUNKS = VPW / SLOTS;      // work items per QWord (8, 4, 2, 1, 1, 1, 1)
+    static constexpr uint32_t SHIFT = NBITS & 63;
+    static constexpr uint64_t CODEMASK = (NBITS >= 64) ? ~0ull : ((1ull << SHIFT) - 1ull);
+};
+
+struct TileGeom
+{
+    uint32_t rows;
+    uint32_t cols;
+    uint32_t nq;
+    uint32_t cols_per_tile; // kThreads / gs
+    uint32_t gs;            // threads per column in the statistics phase: power of two in [8, kThreads]
+    uint32_t gs_log2;
+    uint32_t tile_words;    // LDS doubles reserved for the tile
+    uint32_t words_words;   // LDS QWords for partial words (cols_per_tile * nq when a QWord has several work items)
+    uint64_t qcol;
+};
+
+// LDS layout in 8-byte units: [prefix | tile | partial QWords | decode constants (2 * workers * cols_per_tile)]
+__host__ __device__ inline size_t tile_lds_bytes(const TileGeom& t, uint32_t workers)
+{
+    return ((size_t) kPrefixWords + t.tile_words + t.words_words + (size_t) 2 * workers * t.cols_per_tile) * 8;
+}
+
+// ---- statistics + packing of a tile in LDS (same contract as the fp32 tile_stats / tile_pack) ----------
+
+template <int NBITS, bool ZT>
+__device__ __forceinline__ void tile_stats(const double* tile, double* hdr, double* scratch_f, uint32_t* scratch_u,
+                                           const TileGeom& t, uint32_t nc, char* qtile)
+{
+    const uint32_t tid = threadIdx.x;
+    const uint32_t c = tid >> t.gs_log2;
+    const uint32_t lg = tid & (t.gs - 1);
+    const bool col_ok = c < nc;
+    const double* colv = tile + (size_t) c * t.rows;
+    double lo = 0.0, hi = 0.0;
+
+    if constexpr (NBITS == 1)
+    {
+        double mean = 0.0;
+        if constexpr (!ZT)
+        {
+            double s = 0.0;
+            if (col_ok)
+                for (uint32_t i = lg; i < t.rows; i += t.gs)
+                    s += colv[i];
+            s = group_sum(s, t.gs, scratch_f);
+            mean = s / (double) t.rows;
+        }
+        double s0 = 0.0, s1 = 0.0;
+        uint32_t n0 = 0, n1 = 0;
+        if (col_ok)
+        {
+            for (uint32_t i = lg; i < t.rows; i += t.gs)
+            {
+                const double v = colv[i];
+                if (v < mean)
+                {
+                    s0 += v;
+                    n0++;
+                }
+                else
+                {
+                    s1 += v;
+                    n1++;
+                }
+            }
+        }
+        s0 = group_sum(s0, t.gs, scratch_f);
+        s1 = group_sum(s1, t.gs, scratch_f);
+        n0 = group_sum(n0, t.gs, scratch_u);
+        n1 = group_sum(n1, t.gs, scratch_u);
+        finish_stats_1bit<ZT>(mean, s0, s1, n0, n1, t.rows, lo, hi);
+    }
+    else
+    {
+        double s = 0.0;
+        if (col_ok)
+        {
+            for (uint32_t i = lg; i < t.rows; i += t.gs)
+            {
+                const double v = colv[i];
+                s += v * v;
+            }
+        }
+        s = group_sum(s, t.gs, scratch_f);
+        finish_stats_multibit(s, t.rows, lo, hi);
+    }
+
+    if (col_ok && lg == 0)
+    {
+        hdr[2 * c] = lo;
+        hdr[2 * c + 1] = hi;
+        double* gh = reinterpret_cast<double*>(qtile + (size_t) c * t.qcol);
+        gh[0] = lo;
+        gh[1] = hi;
+    }
+    __syncthreads();
+}
+
+// words[] (LDS, nc * nq entries) must be zero on entry when PackShape<NBITS>::CHUNKS > 1.
+// The new residual goes straight to global memory: for a fixed bit position consecutive threads hold consecutive rows.
+template <int NBITS, bool ZT>
+__device__ __forceinline__ void tile_pack(const double* tile, const double* hdr, unsigned long long* words, const TileGeom& t,
+                                          uint32_t nc, char* qtile, double* res_out)
+{
+    using PS = PackShape<NBITS>;
+    const uint32_t nwords = nc * t.nq;
+    const uint32_t items = nwords * PS::CHUNKS;
+    for (uint32_t it = threadIdx.x; it < items; it += kThreads)
+    {
+        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
+        const uint32_t qi = it - chunk * nwords;
+        const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
+        const uint32_t w = qi - c * t.nq;
+        const ValueQ vq = make_vq<NBITS>(hdr[2 * c], hdr[2 * c + 1]);
+        const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
+        const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
+        const double* colv = tile + (size_t) c * t.rows;
+        double* ro = res_out + (size_t) c * t.rows;
+        uint64_t word = 0;
+#pragma unroll
+        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+        {
+            const uint32_t k = chunk * PS::SLOTS + kk;
+            const uint32_t i = w + k * t.nq;
+            if (i < t.rows)
+            {
+                const double v = colv[i];
+                const uint64_t code = quantize_value<NBITS, ZT>(vq, v);
+                double back;
+                if constexpr (NBITS == 1)
+                    back = code ? val1 : val0;
+                else
+                    back = unquantize_value<NBITS>(vq.uf, vq.lo, code);
+                __builtin_nontemporal_store(v - back, ro + i);
+                word |= code << (k * PS::SHIFT);
+            }
+        }
+        if constexpr (PS::CHUNKS == 1)
+            reinterpret_cast<uint64_t*>(qtile + (size_t) c * t.qcol + 16)[w] = word;
+        else
+            atomicOr(&words[qi], (unsigned long long) word);
+    }
+    if constexpr (PS::CHUNKS > 1)
+    {
+        __syncthreads();
+        for (uint32_t qi = threadIdx.x; qi < nwords; qi += kThreads)
+        {
+            const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
+            const uint32_t w = qi - c * t.nq;
+            reinterpret_cast<uint64_t*>(qtile + (size_t) c * t.qcol + 16)[w] = words[qi];
+        }
+    }
+}
+
+struct TileLds
+{
+    double* scratch_f;
+    uint32_t* scratch_u;
+    double* hdr;
+    double* tile;
+    unsigned long long* words;
+    double* dec;
+};
+
+__device__ __forceinline__ TileLds tile_lds(double* smem, const TileGeom& t)
+{
+    TileLds l;
+    l.scratch_f = smem;
+    l.scratch_u = reinterpret_cast<uint32_t*>(smem + 4);
+    l.hdr = smem + 8;
+    l.tile = smem + kPrefixWords;
+    l.words = reinterpret_cast<unsigned long long*>(smem + kPrefixWords + t.tile_words);
+    l.dec = smem + kPrefixWords + t.tile_words + t.words_words;
+    return l;
+}
+
+// ---- quantize ---------------------------------------------------------------------------------------------
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kThreads) void quantize_tile_kernel(const double* __restrict__ g, const double* r_in, double* r_out,
+                                                                 char* __restrict__ q, TileGeom t)
+{
+    extern __shared__ f64x2 smem_f64[];
+    const TileLds l = tile_lds(reinterpret_cast<double*>(smem_f64), t);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t j0 = blockIdx.x * t.cols_per_tile;
+    const uint32_t nc = min(t.cols_per_tile, t.cols - j0);
+    const size_t base = (size_t) j0 * t.rows;
+    const uint32_t total = nc * t.rows;
+    const double* gp = g + base;
+    const double* rp = r_in + base;
+
+    if constexpr (PackShape<NBITS>::CHUNKS > 1)
+        for (uint32_t x = tid; x < nc * t.nq; x += kThreads)
+            l.words[x] = 0ull;
+
+    // four loads of each operand in flight per thread
+    for (uint32_t e0 = tid; e0 < total; e0 += 4 * kThreads)
+    {
+        double a[4], b[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+        {
+            const uint32_t e = e0 + u * kThreads;
+            if (e < total)
+            {
+                a[u] = __builtin_nontemporal_load(gp + e);
+                b[u] = __builtin_nontemporal_load(rp + e);
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+        {
+            const uint32_t e = e0 + u * kThreads;
+            if (e < total)
+                l.tile[e] = a[u] + b[u];
+        }
+    }
+    __syncthreads(); // from here on r_in is no longer read by this workgroup, so r_out may be r_in
+
+    char* qtile = q + (size_t) j0 * t.qcol;
+    tile_stats<NBITS, ZT>(l.tile, l.hdr, l.scratch_f, l.scratch_u, t, nc, qtile);
+    tile_pack<NBITS, ZT>(l.tile, l.hdr, l.words, t, nc, qtile, r_out + base);
+}
+
+// one workgroup of 1024 threads per column, statistics and packing re-read global memory
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTallThreads) void quantize_tall_kernel(const double* __restrict__ g, const double* r_in, double* r_out,
+                                                                     char* __restrict__ q, uint32_t rows, uint32_t nq, uint64_t qcol)
+{
+    using PS = PackShape<NBITS>;
+    __shared__ double scratch_f[kTallThreads / 64];
+    __shared__ uint32_t scratch_u[kTallThreads / 64];
+
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * rows;
+    const double* gp = g + base;
+    const double* rp = r_in + base;
+    double lo, hi;
+
+    if constexpr (NBITS == 1)
+    {
+        double mean = 0.0;
+        if constexpr (!ZT)
+        {
+            double s = 0.0;
+            for (uint32_t i = tid; i < rows; i += kTallThreads)
+                s += gp[i] + rp[i];
+            s = tall_block_sum(s, scratch_f);
+            mean = s / (double) rows;
+        }
+        double s0 = 0.0, s1 = 0.0;
+        uint32_t n0 = 0, n1 = 0;
+        for (uint32_t i = tid; i < rows; i += kTallThreads)
+        {
+            const double v = gp[i] + rp[i];
+            if (v < mean)
+            {
+                s0 += v;
+                n0++;
+            }
+            else
+            {
+                s1 += v;
+                n1++;
+            }
+        }
+        s0 = tall_block_sum(s0, scratch_f);
+        s1 = tall_block_sum(s1, scratch_f);
+        n0 = tall_block_sum(n0, scratch_u);
+        n1 = tall_block_sum(n1, scratch_u);
+        finish_stats_1bit<ZT>(mean, s0, s1, n0, n1, rows, lo, hi);
+    }
+    else
+    {
+        double s = 0.0;
+        for (uint32_t i = tid; i < rows; i += kTallThreads)
+        {
+            const double v = gp[i] + rp[i];
+            s += v * v;
+        }
+        s = tall_block_sum(s, scratch_f);
+        finish_stats_multibit(s, rows, lo, hi);
+    }
+    // every thread has passed the last barrier of tall_block_sum: all statistics reads of r_in are done
+    // before any residual is written (r_out may be r_in)
+
+    char* qc = q + (size_t) blockIdx.x * qcol;
+    if (tid == 0)
+    {
+        double* gh = reinterpret_cast<double*>(qc);
+        gh[0] = lo;
+        gh[1] = hi;
+    }
+    const ValueQ vq = make_vq<NBITS>(lo, hi);
+    const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
+    const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
+    double* op = r_out + base;
+    uint64_t* bits = reinterpret_cast<uint64_t*>(qc + 16);
+    for (uint32_t w = tid; w < nq; w += kTallThreads)
+    {
+        uint64_t word = 0;
+        for (uint32_t k = 0; k < PS::VPW; ++k)
+        {
+            const uint32_t i = w + k * nq;
+            if (i >= rows)
+                break;
+            const double v = gp[i] + rp[i];
+            const uint64_t code = quantize_value<NBITS, ZT>(vq, v);
+            double back;
+            if constexpr (NBITS == 1)
+                back = code ? val1 : val0;
+            else
+                back = unquantize_value<NBITS>(vq.uf, vq.lo, code);
+            op[i] = v - back;
+            word |= code << (k * PS::SHIFT);
+        }
+        bits[w] = word;
+    }
+}
+
+// ---- stripe reduction: K packed stripes -> fp64 sum (owner first, then ascending) -> requantize ------------
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kThreads) void stripe_reduce_tile_kernel(StripeSources src, double* stripe_res, char* q_out,
+                                                                      double* agg_out, TileGeom t)
+{
+    using PS = PackShape<NBITS>;
+    constexpr uint32_t BATCH = 8; // packed words fetched together, so their latencies overlap
+
+    extern __shared__ f64x2 smem_f64[];
+    const TileLds l = tile_lds(reinterpret_cast<double*>(smem_f64), t);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t j0 = blockIdx.x * t.cols_per_tile;
+    const uint32_t nc = min(t.cols_per_tile, t.cols - j0);
+    const size_t base = (size_t) j0 * t.rows;
+    const uint32_t K = src.workers;
+    const uint32_t nwords = nc * t.nq;
+    double* sp = stripe_res + base;
+
+    if constexpr (PS::CHUNKS > 1)
+        for (uint32_t x = tid; x < nwords; x += kThreads)
+            l.words[x] = 0ull;
+
+    // decode constants from every worker's column header, in summation order: 1 bit -> the two levels, else (ufactor, lower)
+    for (uint32_t x = tid; x < nc * K; x += kThreads)
+    {
+        const uint32_t c = x / K;
+        const uint32_t n = x - c * K;
+        const double* h = reinterpret_cast<const double*>(src.q[stripe_order(n, src.owner)] + (size_t) (j0 + c) * t.qcol);
+        const ValueQ vq = make_vq<NBITS>(h[0], h[1]);
+        if constexpr (NBITS == 1)
+        {
+            l.dec[2 * x] = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
+            l.dec[2 * x + 1] = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
+        }
+        else
+        {
+            l.dec[2 * x] = vq.uf;
+            l.dec[2 * x + 1] = vq.lo;
+        }
+    }
+    __syncthreads();
+
+    const uint32_t items = nwords * PS::CHUNKS;
+    for (uint32_t it = tid; it < items; it += kThreads)
+    {
+        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
+        const uint32_t qi = it - chunk * nwords;
+        const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
+        const uint32_t w = qi - c * t.nq;
+        const size_t word_off = (size_t) (j0 + c) * t.qcol + 16 + (size_t) w * 8;
+        const uint32_t sh0 = chunk * PS::SLOTS * PS::SHIFT;
+        const double* d = l.dec + 2 * (size_t) c * K;
+        double acc[PS::SLOTS];
+        for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
+        {
+            uint64_t word[BATCH];
+#pragma unroll
+            for (uint32_t u = 0; u < BATCH; ++u)
+                if (n0 + u < K)
+                    word[u] = *reinterpret_cast<const uint64_t*>(src.q[stripe_order(n0 + u, src.owner)] + word_off);
+#pragma unroll
+            for (uint32_t u = 0; u < BATCH; ++u)
+            {
+                if (n0 + u < K)
+                {
+                    const double a = d[2 * (n0 + u)];
+                    const double b = d[2 * (n0 + u) + 1];
+                    const uint64_t bits = word[u] >> sh0;
+#pragma unroll
+                    for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+                    {
+                        const uint64_t code = (bits >> (kk * PS::SHIFT)) & PS::CODEMASK;
+                        double x;
+                        if constexpr (NBITS == 1)
+                            x = code ? b : a;
+                        else
+                            x = unquantize_value<NBITS>(a, b, code);
+                        // the first term seeds the sum; afterwards: decoded value + running sum
+                        acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
+                    }
+                }
+            }
+        }
+        double* colv = l.tile + (size_t) c * t.rows;
+        const double* sc = sp + (size_t) c * t.rows;
+#pragma unroll
+        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+        {
+            const uint32_t i = w + (chunk * PS::SLOTS + kk) * t.nq;
+            if (i < t.rows)
+            {
+                if (agg_out != nullptr)
+                    agg_out[base + (size_t) c * t.rows + i] = acc[kk];
+                colv[i] = acc[kk] + __builtin_nontemporal_load(sc + i);
+            }
+        }
+    }
+    __syncthreads();
+
+    char* qtile = q_out + (size_t) j0 * t.qcol;
+    tile_stats<NBITS, ZT>(l.tile, l.hdr, l.scratch_f, l.scratch_u, t, nc, qtile);
+    tile_pack<NBITS, ZT>(l.tile, l.hdr, l.words, t, nc, qtile, sp);
+}
+
+// ---- unquantize ----------------------------------------------------------------------------------------------
+// One thread decodes WV consecutive QWords of a column (WV = 2: 16-byte stores; WV = 1: any shape) for a chunk of
+// `slots` consecutive bit positions; for a fixed bit position consecutive QWords are consecutive rows.
+
+struct UnqGeom
+{
+    uint32_t rows;
+    uint32_t cols;
+    uint32_t nq;
+    uint32_t groups;  // ceil(nq / WV)
+    uint32_t chunks;  // ceil(VPW / slots)
+    uint32_t slots;
+    uint32_t per_col; // groups * chunks
+    uint32_t items;   // per_col * cols
+    uint64_t qcol;
+};
+
+template <int NBITS, int WV>
+__global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, double* out, UnqGeom t, int add)
+{
+    using PS = PackShape<NBITS>;
+    const uint64_t id64 = (uint64_t) blockIdx.x * 256 + threadIdx.x;
+    if (id64 >= t.items)
+        return;
+    const uint32_t id = (uint32_t) id64;
+    const uint32_t c = id / t.per_col;
+    const uint32_t rem = id - c * t.per_col;
+    const uint32_t chunk = rem / t.groups;
+    const uint32_t grp = rem - chunk * t.groups;
+    const uint32_t w0 = grp * WV;
+
+    const char* qc = q + (size_t) c * t.qcol;
+    const double* gh = reinterpret_cast<const double*>(qc);
+    const ValueQ vq = make_vq<NBITS>(gh[0], gh[1]);
+    const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
+    const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
+    const uint64_t* bits = reinterpret_cast<const uint64_t*>(qc + 16);
+    double* oc = out + (size_t) c * t.rows;
+
+    uint64_t word[WV];
+#pragma unroll
+    for (int u = 0; u < WV; ++u)
+        word[u] = bits[w0 + u]; // WV == 2 only when nq is even
+
+    const uint32_t k0 = chunk * t.slots;
+    const uint32_t k1 = min(k0 + t.slots, PS::VPW);
+    for (uint32_t k = k0; k < k1; ++k)
+    {
+        const uint32_t i = w0 + k * t.nq;
+        if (i >= t.rows)
+            break; // rows only grow with k
+        const uint32_t sh = k * PS::SHIFT;
+        if constexpr (WV == 2)
+        {
+            // rows and nq even, i even: both rows are inside the column and the store is 16-byte aligned
+            f64x2 x;
+            if constexpr (NBITS == 1)
+            {
+                x.x = ((word[0] >> sh) & 1ull) ? val1 : val0;
+                x.y = ((word[1] >> sh) & 1ull) ? val1 : val0;
+            }
+            else
+            {
+                x.x = unquantize_value<NBITS>(vq.uf, vq.lo, (word[0] >> sh) & PS::CODEMASK);
+                x.y = unquantize_value<NBITS>(vq.uf, vq.lo, (word[1] >> sh) & PS::CODEMASK);
+            }
+            f64x2* dst = reinterpret_cast<f64x2*>(oc + i);
+            if (add)
+                x = x + *dst; // unquantized value + previous content
+            __builtin_nontemporal_store(x, dst);
+        }
+        else
+        {
+            double x;
+            if constexpr (NBITS == 1)
+                x = ((word[0] >> sh) & 1ull) ? val1 : val0;
+            else
+                x = unquantize_value<NBITS>(vq.uf, vq.lo, (word[0] >> sh) & PS::CODEMASK);
+            if (add)
+                x = x + oc[i];
+            oc[i] = x;
+        }
+    }
+}
+
+} // namespace f64
+} // namespace cntkq

@@ -2,7 +2,7 @@
  * cntk_amd_quantizer.h -- C ABI of the MI355X (gfx950) gradient quantizer.
  *
  * This is the boundary a CNTK build binds in place of MatrixQuantizerGPU: one opaque handle per
- * MatrixQuantizerImpl<float> object, plain pointers and sizes, no C++ or torch types. Every call
+ * MatrixQuantizerImpl<float> (or <double>, see the _f64 calls at the end) object, plain pointers and sizes, no C++ or torch types. Every call
  * returns a status code; cntkq_last_error() gives the text the reference would have thrown.
  *
  * Data contracts (identical to the reference):
@@ -169,6 +169,38 @@ int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, si
 /* Blocks until the last stripe reduction of this handle has finished (the reference waits on the stripe
  * quantizer's WaitQuantizeAsyncDone, Source/1BitSGD/AllReduceDistGradAggregator.h:494). */
 int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h);
+
+/* ---- the double instantiation: MatrixQuantizerImpl<double> -----------------------------------------------
+ *
+ * The reference instantiates the whole path for ElemType = double as well (Source/Math/MatrixQuantizerImpl.cpp:28-29,
+ * Source/Math/MatrixQuantizerGPU.cu:344-345, Source/Math/QuantizedMatrix.cpp:183-184); its QWord is then the 64-bit
+ * unsigned integer (Source/Math/ValueQuantizer.h:50-57). Same handle type, same streams, same waits
+ * (cntkq_wait_quantize_done etc.), same semantics as the float calls above, with
+ *   - matrices: dense fp64, column-major, 8-byte aligned;
+ *   - packed matrix: cols records { double lower; double upper; uint64_t bits[nq]; }, nq = ceil(rows / (64 / nbits)),
+ *     element i in bits[i % nq] at bit (i / nq) * nbits; the buffer must be 8-byte aligned;
+ *   - nbits one of 1, 2, 4, 8, 16, 32, 64 (64 = pass-through; 32 is a real quantizer with 2^32 - 1 steps);
+ *   - stripe reduction: rows <= 7168.
+ * The gradient-set (batch) calls exist for float only. */
+
+/* ColumnQuantizer<double>::QWordsPerCol, QuantizedColumn<double>::QuantizedColumnSize, QuantizedMatrix<double>::GetSize. */
+size_t cntkq_qwords_per_col_f64(size_t rows, size_t nbits);
+size_t cntkq_qcol_bytes_f64(size_t nbits, size_t rows);
+size_t cntkq_qmatrix_bytes_f64(size_t rows, size_t cols, size_t nbits);
+
+/* MatrixQuantizerImpl<double>::QuantizeAsync (Source/Math/MatrixQuantizerImpl.h:30, Source/Math/MatrixQuantizerGPU.cu:226-269). */
+int cntkq_quantize_async_f64(cntkq_quantizer* h, const double* in, const double* res_in, size_t rows, size_t cols,
+                             void* qbuf, size_t qbuf_bytes, int qbuf_on_host, size_t nbits, double* res_out,
+                             int zero_threshold_for_1bit);
+
+/* MatrixQuantizerImpl<double>::UnquantizeAsync (Source/Math/MatrixQuantizerImpl.h:33, Source/Math/MatrixQuantizerGPU.cu:286-334). */
+int cntkq_unquantize_async_f64(cntkq_quantizer* h, const void* qbuf, size_t qbuf_bytes, int qbuf_on_host, double* out,
+                               size_t rows, size_t cols, size_t nbits, int add);
+
+/* cntkq_stripe_reduce_async for double stripes (same dataflow and summation order). */
+int cntkq_stripe_reduce_async_f64(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner,
+                                  size_t rows, size_t stripe_cols, size_t nbits, double* stripe_res, void* q_out,
+                                  double* agg_out, int zero_threshold_for_1bit);
 
 #ifdef __cplusplus
 }

@@ -12,6 +12,9 @@ of a column deviates by more than 1e-6 of its scale (long columns: the oracle's 
 inexact; fine code grids: 16 bits), a differing code is accepted within 1.5 x that column's observed header
 deviation instead, and counted separately as "beyond 1e-6"; callers that must hold the 1e-6 rule literally pass
 strict=True, which makes any such element a failure.
+
+The figures above are for float32 matrices. For float64 matrices (64-bit QWords) the same rules apply with 1e-12 /
+1e-13 / 1e-12: both sides sum in double and differ in the order of the additions only.
 """
 import numpy as np
 
@@ -20,6 +23,13 @@ import oracle
 BOUND_RTOL = 1e-5
 THRESH_RTOL = 1e-6
 VALUE_RTOL = 1e-5
+
+
+def tolerances(dtype):
+    """(bound, threshold, value, floor of the relaxed rule), relative to the column scale."""
+    if np.dtype(dtype) == np.float64:
+        return 1e-12, 1e-13, 1e-12, 1e-14
+    return BOUND_RTOL, THRESH_RTOL, VALUE_RTOL, 1e-7
 
 
 def bits_equal(a, b):
@@ -50,6 +60,9 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
     exact=False skips the bit-exact layer (for inputs that are themselves only equal within tolerance);
     skip_cols (bool per column) leaves columns out of the tolerance layer."""
     rows, cols = g.shape
+    dt = g.dtype
+    bound_rtol, thresh_rtol, value_rtol, relaxed_floor = tolerances(dt)
+    word_bits = 8 * dt.itemsize
     zt = bool(zero_threshold) and nbits == 1
     rep = report if report is not None else Report()
     rep.elements += rows * cols
@@ -63,10 +76,10 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
 
     # ---- tolerance layer
     q_or, r_or = oracle.quantize(g, r_in, nbits, zt, threads=threads)
-    lo_g, hi_g = oracle.headers(q_gpu, rows, cols, nbits)
-    lo_o, hi_o = oracle.headers(q_or, rows, cols, nbits)
+    lo_g, hi_g = oracle.headers(q_gpu, rows, cols, nbits, dtype=dt)
+    lo_o, hi_o = oracle.headers(q_or, rows, cols, nbits, dtype=dt)
     scale = (hi_o.astype(np.float64) - lo_o.astype(np.float64))
-    tiny = np.finfo(np.float32).tiny
+    tiny = np.finfo(dt).tiny
     denom = np.maximum(np.abs(scale), tiny)
     abs_dev = np.maximum(np.abs(lo_g.astype(np.float64) - lo_o), np.abs(hi_g.astype(np.float64) - hi_o))
     err = abs_dev / denom
@@ -76,22 +89,22 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
     err[flat] = 0.0
     err[~keep] = 0.0
     rep.max_bound_err = max(rep.max_bound_err, float(err.max(initial=0.0)))
-    assert err.max(initial=0.0) <= BOUND_RTOL, "column bounds off by %.3g of the column scale" % err.max()
+    assert err.max(initial=0.0) <= bound_rtol, "column bounds off by %.3g of the column scale" % err.max()
 
-    if nbits == 32:
-        assert np.array_equal(q_or[:], q_gpu[:]) or np.array_equal(oracle.words(q_or, rows, cols, 32),
-                                                                   oracle.words(q_gpu, rows, cols, 32))
+    if nbits == word_bits:
+        assert np.array_equal(q_or[:], q_gpu[:]) or np.array_equal(oracle.words(q_or, rows, cols, nbits, dtype=dt),
+                                                                   oracle.words(q_gpu, rows, cols, nbits, dtype=dt))
         assert bits_equal(r_or, r_gpu)
         rep.last_mismatch_cols = np.zeros(cols, dtype=bool)
         return rep
 
-    c_g = oracle.codes(q_gpu, rows, cols, nbits)
-    c_o = oracle.codes(q_or, rows, cols, nbits)
+    c_g = oracle.codes(q_gpu, rows, cols, nbits, dtype=dt)
+    c_o = oracle.codes(q_or, rows, cols, nbits, dtype=dt)
     diff = (c_g != c_o) & keep[None, :]
     ndiff = int(diff.sum())
     rep.last_mismatch_cols = diff.any(axis=0)
     if ndiff:
-        v = (g + r_in).astype(np.float64)  # one rounded fp32 add, then widened
+        v = (g + r_in).astype(np.float64)  # one add rounded in the element type, then widened
         ii, jj = np.nonzero(diff)
         vv = v[ii, jj]
         sc = denom[jj]
@@ -106,10 +119,10 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
             dist = np.minimum(dist, np.minimum(np.abs(vv - lo), np.abs(vv - hi_o[jj].astype(np.float64))))
             assert np.all(np.abs(c_g[ii, jj].astype(np.int64) - c_o[ii, jj].astype(np.int64)) == 1), \
                 "codes differ by more than one level"
-        far = dist > THRESH_RTOL * sc
-        allowed = np.maximum(THRESH_RTOL * sc, 1.5 * abs_dev[jj] + 1e-7 * sc)
+        far = dist > thresh_rtol * sc
+        allowed = np.maximum(thresh_rtol * sc, 1.5 * abs_dev[jj] + relaxed_floor * sc)
         if strict:
-            allowed = THRESH_RTOL * sc
+            allowed = thresh_rtol * sc
         assert np.all(dist <= allowed), \
             "%d codes differ away from a threshold (worst %.3g of scale)" % (ndiff, float((dist / sc).max()))
         rep.near_threshold_mismatches += ndiff
@@ -119,15 +132,15 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
     rerr = np.abs(r_gpu.astype(np.float64) - r_or) / denom[None, :]
     rerr = np.where(same, rerr, 0.0)
     rep.max_residual_err = max(rep.max_residual_err, float(rerr.max(initial=0.0)))
-    assert rerr.max(initial=0.0) <= VALUE_RTOL, "residual off by %.3g of the column scale" % rerr.max()
+    assert rerr.max(initial=0.0) <= value_rtol, "residual off by %.3g of the column scale" % rerr.max()
     return rep
 
 
 def check_unquantize(q, rows, cols, nbits, out_gpu, prev_out=None, threads=8):
     """Unquantize has no reductions: bit-exact against the oracle."""
     add = prev_out is not None
-    out = np.array(prev_out, dtype=np.float32, order="F", copy=True) if add else None
-    ref = oracle.unquantize(q, rows, cols, nbits, out=out, add=add, threads=threads)
+    out = np.array(prev_out, dtype=out_gpu.dtype, order="F", copy=True) if add else None
+    ref = oracle.unquantize(q, rows, cols, nbits, out=out, add=add, threads=threads, dtype=out_gpu.dtype)
     assert bits_equal(ref, out_gpu), "unquantized output differs from the oracle"
 
 
@@ -143,19 +156,20 @@ def oracle_allreduce_staged(gs, res, sres, nbits, zt, threads=8):
     Returns (packed matrices after stage 1, fp32 aggregates per stripe, assembled packed aggregate, output)."""
     k = len(gs)
     rows, cols = gs[0].shape
-    qcol = oracle.qcol_bytes(nbits, rows)
+    dt = gs[0].dtype
+    qcol = oracle.qcol_bytes(nbits, rows, dt)
     q1 = [oracle.quantize(gs[w], res[w], nbits, zt, r_out=res[w], threads=threads)[0] for w in range(k)]
     qagg = np.zeros_like(q1[0])
     aggs = []
     for s in range(k):
         start, n = oracle.stripe_range(cols, s, k)
         if n == 0:
-            aggs.append(np.zeros((rows, 0), np.float32, order="F"))
+            aggs.append(np.zeros((rows, 0), dt, order="F"))
             continue
         qc = [q.copy() for q in q1]
         aggs.append(oracle.stripe_reduce(qc, s, rows, cols, nbits, sres[s], zt, threads=threads))
         qagg[start * qcol:(start + n) * qcol] = qc[s][start * qcol:(start + n) * qcol]
-    out = oracle.unquantize(qagg, rows, cols, nbits, threads=threads)
+    out = oracle.unquantize(qagg, rows, cols, nbits, threads=threads, dtype=dt)
     return q1, aggs, qagg, out
 
 
@@ -168,7 +182,8 @@ def check_end_to_end(aggs_or, sres_in, qagg_gpu, sres_gpu, out_gpu, qagg_or, out
     themselves equal only within the first-stage header tolerance), and the aggregated gradient must be within 1e-5
     of the column scale wherever the final codes agree."""
     k = len(aggs_or)
-    qcol = oracle.qcol_bytes(nbits, rows)
+    dt = out_or.dtype
+    qcol = oracle.qcol_bytes(nbits, rows, dt)
     rep = report if report is not None else Report()
     for s in range(k):
         start, n = oracle.stripe_range(cols, s, k)
@@ -177,11 +192,11 @@ def check_end_to_end(aggs_or, sres_in, qagg_gpu, sres_gpu, out_gpu, qagg_or, out
         check_quantize(aggs_or[s], sres_in[s], qagg_gpu[start * qcol:(start + n) * qcol], sres_gpu[s], nbits, zt,
                        threads=threads, report=rep, exact=False, skip_cols=tainted_cols[start:start + n])
     clean = ~tainted_cols
-    lo, hi = oracle.headers(qagg_or, rows, cols, nbits)
-    scale = np.maximum(np.abs(hi.astype(np.float64) - lo), np.finfo(np.float32).tiny)
+    lo, hi = oracle.headers(qagg_or, rows, cols, nbits, dtype=dt)
+    scale = np.maximum(np.abs(hi.astype(np.float64) - lo), np.finfo(dt).tiny)
     # elements whose final code differs sit a whole level apart; the check above has vetted each of them
-    same = oracle.codes(qagg_gpu, rows, cols, nbits) == oracle.codes(qagg_or, rows, cols, nbits)
+    same = oracle.codes(qagg_gpu, rows, cols, nbits, dtype=dt) == oracle.codes(qagg_or, rows, cols, nbits, dtype=dt)
     err = np.where(same, np.abs(out_gpu.astype(np.float64) - out_or) / scale[None, :], 0.0)
     worst = float(err[:, clean].max(initial=0.0))
-    assert worst <= VALUE_RTOL, "aggregated gradient off by %.3g of the column scale" % worst
+    assert worst <= tolerances(dt)[2], "aggregated gradient off by %.3g of the column scale" % worst
     return worst, int(tainted_cols.sum())

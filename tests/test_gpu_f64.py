@@ -1,0 +1,325 @@
+"""Parity of the double-precision instantiation (MatrixQuantizerImpl<double>, 64-bit QWords) against the CPU oracle,
+through the C ABI (the _f64 entry points). Needs an MI355X.
+
+Same structure as the float tests: the reference unit test's shapes (Tests/UnitTests/MathTests/MatrixQuantizerTests.cpp
+runs every case for double as well, :420-431), every bit width 1..64, both 1-bit threshold modes, teacher-forced
+chains with carried residual, every kernel path, the unquantize variants, the fused stripe reduction.
+Tolerances: bit-exact under the GPU's own headers; headers within 1e-12 of the column scale, codes different only
+within 1e-13 of a threshold, other residuals within 1e-12 (both sides sum in double).
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import cntk_amd
+import datagen
+import oracle
+import parity
+from cntk_amd import Matrix, MatrixQuantizerImpl, QuantizedMatrix
+
+pytestmark = pytest.mark.gpu
+
+F64 = np.float64
+VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False), (64, False)]
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_WAVECOL = 0, 1, 2, 3
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def zeros(rows, cols):
+    return np.zeros((rows, cols), F64, order="F")
+
+
+@pytest.fixture(scope="module")
+def quantizer():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    q = MatrixQuantizerImpl.Create(0, False)
+    yield q
+    torch.cuda.synchronize()
+
+
+def gpu_quantize(qz, g, r_in, nbits, zt, in_place=True, host_q=False):
+    rows, cols = g.shape
+    G = Matrix.from_numpy(g)
+    R = Matrix.from_numpy(r_in)
+    assert G.dtype == torch.float64
+    Rout = R if in_place else Matrix(rows, cols, dtype=torch.float64)
+    Q = QuantizedMatrix(rows, cols, nbits, cntk_amd.CPUDEVICE if host_q else 0, dtype=torch.float64)
+    qz.QuantizeAsync(G, R, Q, Rout, zt)
+    qz.WaitQuantizeAsyncDone()
+    if not host_q:
+        torch.cuda.synchronize()
+    return Q, Rout.to_numpy()
+
+
+def run_chain(qz, rows, cols, nbits, zt, make_input, iterations, report, in_place=True, host_q=False):
+    """Teacher-forced chain: the oracle's residual feeds both sides at every step."""
+    res_o, out_o = zeros(rows, cols), zeros(rows, cols)
+    Out = Matrix(rows, cols, dtype=torch.float64)
+    for it in range(iterations):
+        g = make_input(it)
+        assert g.dtype == F64
+        Q, r_gpu = gpu_quantize(qz, g, res_o, nbits, zt, in_place=in_place, host_q=host_q)
+        q_gpu = Q.to_numpy()
+        parity.check_quantize(g, res_o, q_gpu, r_gpu, nbits, zt, report=report)
+        prev = Out.to_numpy()
+        qz.UnquantizeAsync(Q, Out, add=(it > 0))
+        qz.WaitUnquantizeAsyncDone()
+        parity.check_unquantize(q_gpu, rows, cols, nbits, Out.to_numpy(), prev_out=prev if it > 0 else None)
+        q_or, _ = oracle.quantize(g, res_o, nbits, zt, r_out=res_o, threads=8)
+        oracle.unquantize(q_or, rows, cols, nbits, out=out_o, add=(it > 0), threads=8)
+        Out = Matrix.from_numpy(out_o)
+
+
+UNIT_SHAPES = [
+    (25, 13, -1.0, 1.0, 2015), (25, 13, -0.005, 0.005, 2115), (13, 25, -0.00001, 0.00001, 2215),
+    (13, 25, -10.0, 10.0, 2315), (25, 13, -1.0, 2.05, 2415), (489, 1, -0.5, 0.5, 2515), (1, 135, -0.5, 0.5, 2615),
+    (89, 23, -0.5, 0.5, 2715), (15, 35, -0.5, 0.5, 2815), (100, 50, -0.5, 0.5, 2915), (737, 373, -0.5, 0.5, 2915),
+]
+
+
+@pytest.mark.parametrize("shape", UNIT_SHAPES, ids=["%dx%d_%d" % (s[0], s[1], s[4]) for s in UNIT_SHAPES])
+def test_reference_unit_shapes_f64(quantizer, shape):
+    rows, cols, lo, hi, seed = shape
+    rep = parity.Report()
+    for nbits, zt in VARIANTS:
+        say("f64 unit shape", shape, "nbits", nbits, "zeroThr", zt)
+        run_chain(quantizer, rows, cols, nbits, zt, lambda it: datagen.uniform(seed + it, rows, cols, lo, hi, dtype=F64), 3, rep)
+    say("  ", rep)
+
+
+def test_golden_vectors_f64(quantizer):
+    """Against the packed bytes the reference's own headers wrote for double (tests/golden/unit_shapes_f64.npz): the
+    oracle reproduces them byte for byte, and the GPU result is held to the parity rules against that same result.
+    Byte-identical GPU output is counted, not required: the sums behind a header are taken in another order."""
+    import os
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "unit_shapes_f64.npz"))
+    from golden.make_golden import UNIT_SHAPES as GOLD_SHAPES
+    same = total = 0
+    for si, (rows, cols, lo, hi, seed) in enumerate(GOLD_SHAPES):
+        g = np.asfortranarray(gold["s%d_inputs" % si][0].reshape((rows, cols), order="F"))
+        for nbits, zt in VARIANTS:
+            Q, r = gpu_quantize(quantizer, g, zeros(rows, cols), nbits, zt)
+            ref_q = gold["s%d_b%d_z%d_q" % (si, nbits, int(zt))][0]
+            assert np.array_equal(oracle.quantize(g, zeros(rows, cols), nbits, zt)[0], ref_q)
+            parity.check_quantize(g, zeros(rows, cols), Q.to_numpy(), r, nbits, zt)
+            total += 1
+            same += int(np.array_equal(Q.to_numpy(), ref_q))
+    say("f64 golden: %d of %d packed matrices byte-identical to the reference's" % (same, total))
+    assert same > 0
+
+
+def test_free_running_conservation_f64(quantizer):
+    rows, cols, lo, hi = 100, 50, -0.5, 0.5
+    for nbits, zt in VARIANTS:
+        R, Out = Matrix(rows, cols, dtype=torch.float64), Matrix(rows, cols, dtype=torch.float64)
+        for it in range(4):
+            g = datagen.uniform(2915 + it, rows, cols, lo, hi, dtype=F64)
+            r_in, prev = R.to_numpy(), Out.to_numpy()
+            Q = QuantizedMatrix(rows, cols, nbits, 0, dtype=torch.float64)
+            quantizer.QuantizeAsync(Matrix.from_numpy(g), R, Q, R, zt)
+            quantizer.WaitQuantizeAsyncDone()
+            quantizer.UnquantizeAsync(Q, Out, add=(it > 0))
+            quantizer.WaitUnquantizeAsyncDone()
+            parity.conservation(g, r_in, prev, R.to_numpy(), Out.to_numpy(), 1e-14)
+
+
+PATH_CASES = [
+    # rows, cols, path, tile_gs
+    (1, 1, PATH_TILE, 0), (3, 70, PATH_TILE, 0), (31, 5, PATH_TILE, 8), (65, 67, PATH_TILE, 0), (64, 64, PATH_TILE, 16),
+    (147, 64, PATH_TILE, 0), (429, 37, PATH_TILE, 0), (429, 37, PATH_TILE, 64), (1023, 9, PATH_TILE, 0),
+    (2048, 19, PATH_TILE, 0), (2048, 19, PATH_TILE, 256), (4608, 3, PATH_TILE, 0), (7168, 2, PATH_TILE, 0),
+    (1, 5, PATH_TALL, 0), (70, 3, PATH_TALL, 0), (1025, 3, PATH_TALL, 0), (20001, 2, PATH_TALL, 0), (9304, 2, PATH_AUTO, 0),
+]
+
+
+@pytest.mark.parametrize("case", PATH_CASES, ids=["%dx%d_p%d_g%d" % c for c in PATH_CASES])
+def test_kernel_paths_f64(case):
+    rows, cols, path, gs = case
+    qz = MatrixQuantizerImpl.Create(0, False)
+    qz._set_tuning(quantize_path=path, tile_gs=gs)
+    rep = parity.Report()
+    for nbits, zt in VARIANTS:
+        say("f64 path case", case, "nbits", nbits, "zeroThr", zt)
+
+        def make(it):
+            a = datagen.normal_with_outliers(1000 * rows + cols + it, rows, cols, 0.01, dtype=F64) + 0.004 * (it % 2)
+            a = np.asfortranarray(a)
+            if cols > 1:
+                a[:, cols // 2] = 0.0
+            return a
+        run_chain(qz, rows, cols, nbits, zt, make, 2, rep)
+    say("  ", rep)
+
+
+def test_unsupported_paths_are_refused_f64():
+    qz = MatrixQuantizerImpl.Create(0, False)
+    qz._set_tuning(quantize_path=PATH_WAVECOL)
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        gpu_quantize(qz, datagen.normal(1, 2048, 4, dtype=F64), zeros(2048, 4), 1, False)
+    qz._set_tuning(quantize_path=PATH_TILE)
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        gpu_quantize(qz, datagen.normal(1, 7169, 2, dtype=F64), zeros(7169, 2), 1, False)
+
+
+def test_unquantize_variants_f64(quantizer):
+    for rows, cols in [(5, 3), (37, 2), (128, 9), (429, 5), (2048, 6), (4100, 2), (1001, 5), (100000, 2)]:
+        for nbits, zt in VARIANTS:
+            g = datagen.normal(rows * 7 + nbits, rows, cols, dtype=F64)
+            q, _ = oracle.quantize(g, zeros(rows, cols), nbits, zt)
+            prev = datagen.normal(rows * 9 + nbits, rows, cols, 1.0, dtype=F64)
+            for slots in (0, 1, 3, 64):
+                for scalar in (0, 1):
+                    say("f64 unquantize", rows, cols, nbits, "slots", slots, "scalar", scalar)
+                    qz = MatrixQuantizerImpl.Create(0, False)
+                    qz._set_tuning(unq_slots=slots, unq_force_scalar=scalar)
+                    Q = QuantizedMatrix(rows, cols, nbits, 0, dtype=torch.float64)
+                    Q.from_numpy(q)
+                    for add in (False, True):
+                        Out = Matrix.from_numpy(prev)
+                        qz.UnquantizeAsync(Q, Out, add=add)
+                        qz.WaitUnquantizeAsyncDone()
+                        parity.check_unquantize(q, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
+
+
+def test_out_of_place_host_buffer_and_slices_f64(quantizer):
+    rows, cols = 429, 37
+    for nbits, zt in VARIANTS:
+        rep = parity.Report()
+        make = lambda it: datagen.student_t(50 + it, rows, cols, dtype=F64)
+        run_chain(quantizer, rows, cols, nbits, zt, make, 2, rep, in_place=False)
+        run_chain(quantizer, rows, cols, nbits, zt, make, 2, rep, host_q=True)
+    # column slices of gradient, residual and packed matrix
+    rows, cols, nbits = 429, 23, 1
+    g, r = datagen.normal(11, rows, cols, dtype=F64), datagen.normal(12, rows, cols, 0.002, dtype=F64)
+    G, R, Q = Matrix.from_numpy(g), Matrix.from_numpy(r), QuantizedMatrix(rows, cols, nbits, 0, dtype=torch.float64)
+    for start, n in [(0, 5), (5, 1), (6, 17)]:
+        quantizer.QuantizeAsync(G.ColumnSlice(start, n), R.ColumnSlice(start, n), Q.ColumnSlice(start, n),
+                                R.ColumnSlice(start, n), False)
+    quantizer.WaitQuantizeAsyncDone()
+    parity.check_quantize(g, r, Q.to_numpy(), R.to_numpy(), nbits, False)
+    Out = Matrix(rows, cols, dtype=torch.float64)
+    quantizer.UnquantizeAsync(Q.ColumnSlice(3, 11), Out.ColumnSlice(3, 11))
+    quantizer.WaitUnquantizeAsyncDone()
+    ref = oracle.unquantize(Q.to_numpy(), rows, cols, nbits, dtype=F64)
+    out = Out.to_numpy()
+    assert parity.bits_equal(np.asfortranarray(out[:, 3:14]), np.asfortranarray(ref[:, 3:14]))
+    assert not out[:, :3].any() and not out[:, 14:].any()
+
+
+def test_special_columns_and_errors_f64(quantizer):
+    z = zeros(70, 3)
+    for zt in (False, True):
+        Q, r = gpu_quantize(quantizer, z, z.copy(order="F"), 1, zt)
+        w = oracle.words(Q.to_numpy(), 70, 3, 1, dtype=F64)  # 70 rows -> 2 QWords: 35 valid bits each
+        assert [hex(int(x)) for x in w[0]] == ["0x7ffffffff", "0x7ffffffff"]
+        lo, hi = oracle.headers(Q.to_numpy(), 70, 3, 1, dtype=F64)
+        assert not lo.any() and not hi.any() and not r.any()
+    g = np.asfortranarray(np.array([[0.1], [-0.2], [0.3], [-0.4], [0.05]], F64))
+    Q, r = gpu_quantize(quantizer, g, zeros(5, 1), 1, False)
+    lo, hi = oracle.headers(Q.to_numpy(), 5, 1, 1, dtype=F64)
+    assert abs(lo[0] + 0.462) < 1e-15 and abs(hi[0] - 0.402) < 1e-15
+    assert int(oracle.words(Q.to_numpy(), 5, 1, 1, dtype=F64)[0, 0]) == 0b10101
+    # element types may not be mixed; 64 bits does not exist for float
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        quantizer.QuantizeAsync(Matrix(8, 4, dtype=torch.float64), Matrix(8, 4), QuantizedMatrix(8, 4, 1, 0, dtype=torch.float64),
+                                Matrix(8, 4, dtype=torch.float64), False)
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        quantizer.UnquantizeAsync(QuantizedMatrix(8, 4, 1, 0), Matrix(8, 4, dtype=torch.float64))
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        QuantizedMatrix(8, 4, 64, 0)
+    with pytest.raises(cntk_amd.QuantizerLogicError):  # packed size of the float layout handed to the double call
+        cntk_amd._check(cntk_amd.lib().cntkq_unquantize_async_f64(quantizer._h, QuantizedMatrix(8, 4, 1, 0).Buffer(), 48, 0,
+                                                                  Matrix(8, 4, dtype=torch.float64).Data(), 8, 4, 1, 0))
+    quantizer.QuantizeAsync(Matrix(0, 4, dtype=torch.float64), Matrix(0, 4, dtype=torch.float64),
+                            QuantizedMatrix(0, 4, 1, 0, dtype=torch.float64), Matrix(0, 4, dtype=torch.float64), False)
+    quantizer.WaitQuantizeAsyncDone()
+
+
+# ---- fused stripe reduction ---------------------------------------------------------------------------------
+
+
+def unfused_reference(qz, stripes_np, owner, rows, n, nbits, sres, zt):
+    """The reference's call sequence on the GPU: unquantize own stripe, add the others in ascending order, requantize."""
+    Agg = Matrix(rows, n, dtype=torch.float64)
+    order = [owner] + [w for w in range(len(stripes_np)) if w != owner]
+    for pos, w in enumerate(order):
+        Q = QuantizedMatrix(rows, n, nbits, 0, dtype=torch.float64)
+        Q.from_numpy(stripes_np[w])
+        qz.UnquantizeAsync(Q, Agg, add=(pos > 0))
+    S = Matrix.from_numpy(sres)
+    Qo = QuantizedMatrix(rows, n, nbits, 0, dtype=torch.float64)
+    qz.QuantizeAsync(Agg, S, Qo, S, zt)
+    qz.WaitQuantizeAsyncDone()
+    return Agg.to_numpy(), Qo.to_numpy(), S.to_numpy()
+
+
+@pytest.mark.parametrize("rows,n,k", [(70, 9, 3), (429, 12, 4), (2048, 20, 8), (4096, 3, 2), (7168, 2, 5), (64, 40, 64)])
+def test_stripe_reduce_f64(quantizer, rows, n, k):
+    for nbits, zt in VARIANTS:
+        say("f64 stripe reduce", rows, n, k, nbits, zt)
+        stripes = [oracle.quantize(datagen.normal(31 * w + rows + nbits, rows, n, dtype=F64), zeros(rows, n), nbits, zt, threads=8)[0]
+                   for w in range(k)]
+        sres = datagen.normal(977 + rows, rows, n, 0.002, dtype=F64)
+        for owner in sorted({0, k - 1, k // 2}):
+            # the oracle's aggregate: owner first, then ascending
+            agg_o = oracle.unquantize(stripes[owner], rows, n, nbits, dtype=F64, threads=8)
+            for w in range(k):
+                if w != owner:
+                    oracle.unquantize(stripes[w], rows, n, nbits, out=agg_o, add=True, threads=8)
+            Qs = []
+            for w in range(k):
+                Q = QuantizedMatrix(rows, n, nbits, 0, dtype=torch.float64)
+                Q.from_numpy(stripes[w])
+                Qs.append(Q)
+            S = Matrix.from_numpy(sres)
+            Agg = Matrix(rows, n, dtype=torch.float64)
+            quantizer.StripeReduceAsync(Qs, owner, S, Qs[owner], zt, agg_out=Agg)  # in place over the owner's stripe
+            quantizer.WaitStripeReduceDone()
+            assert parity.bits_equal(Agg.to_numpy(), agg_o), "aggregate differs from the ordered sum"
+            parity.check_quantize(agg_o, sres, Qs[owner].to_numpy(), S.to_numpy(), nbits, zt)
+            # the fused call gives the very bytes of the reference's unquantize ... quantize call sequence
+            agg_u, q_u, s_u = unfused_reference(quantizer, stripes, owner, rows, n, nbits, sres, zt)
+            assert parity.bits_equal(agg_u, agg_o)
+            assert np.array_equal(q_u, Qs[owner].to_numpy()) and parity.bits_equal(s_u, S.to_numpy())
+
+
+def test_end_to_end_allreduce_f64(quantizer):
+    """K = 4 workers through quantize -> fused stripe reduction -> unquantize against the staged oracle."""
+    k, rows, cols = 4, 512, 37
+    for nbits, zt in [(1, False), (1, True), (4, False)]:
+        gs = [datagen.normal(700 + w, rows, cols, dtype=F64) for w in range(k)]
+        res = [datagen.normal(750 + w, rows, cols, 0.002, dtype=F64) for w in range(k)]
+        sres = [datagen.normal(770 + s, rows, oracle.stripe_range(cols, s, k)[1], 0.002, dtype=F64) for s in range(k)]
+        res_o = [r.copy(order="F") for r in res]
+        sres_o = [s.copy(order="F") for s in sres]
+        q1_o, aggs_o, qagg_o, out_o = parity.oracle_allreduce_staged(gs, res_o, sres_o, nbits, zt)
+        rep = parity.Report()
+        Qw, tainted = [], np.zeros(cols, dtype=bool)
+        for w in range(k):
+            Q = QuantizedMatrix(rows, cols, nbits, 0, dtype=torch.float64)
+            R = Matrix.from_numpy(res[w])
+            quantizer.QuantizeAsync(Matrix.from_numpy(gs[w]), R, Q, R, zt)
+            quantizer.WaitQuantizeAsyncDone()
+            parity.check_quantize(gs[w], res[w], Q.to_numpy(), R.to_numpy(), nbits, zt, report=rep)
+            tainted |= rep.last_mismatch_cols
+            Qw.append(Q)
+        Qagg = QuantizedMatrix(rows, cols, nbits, 0, dtype=torch.float64)
+        sres_gpu = []
+        for s in range(k):
+            st, n = oracle.stripe_range(cols, s, k)
+            S = Matrix.from_numpy(sres[s])
+            quantizer.StripeReduceAsync([Q.ColumnSlice(st, n) for Q in Qw], s, S, Qagg.ColumnSlice(st, n), zt)
+            quantizer.WaitStripeReduceDone()
+            sres_gpu.append(S.to_numpy())
+        Out = Matrix(rows, cols, dtype=torch.float64)
+        quantizer.UnquantizeAsync(Qagg, Out)
+        quantizer.WaitUnquantizeAsyncDone()
+        worst, ntaint = parity.check_end_to_end(aggs_o, sres, Qagg.to_numpy(), sres_gpu, Out.to_numpy(), qagg_o, out_o, rows, cols,
+                                                nbits, zt, tainted, report=rep)
+        say("f64 all-reduce nbits", nbits, "zt", zt, "worst", worst, "tainted columns", ntaint, rep)
