@@ -662,7 +662,7 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
     for (size_t i = 0; i < count; ++i)
     {
         const cntkq_quantize_item& it = items[i];
-        if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.qbuf, it.rows, nbits) != kPathTile)
+        if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.in, it.res_in, it.res_out, it.qbuf, it.rows, nbits) != kPathTile)
             continue;
         const TileGeom t = make_tile_geom(it.rows, it.cols, nbits, 0, -1, 0);
         n_tile[tile_lds_bytes(t, 0) <= kSmallLds ? 0 : 1]++;
@@ -671,7 +671,7 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
     hipEvent_t done = h->ev_quantize;
     size_t launches_left = (n_tile[0] ? 1 : 0) + (n_tile[1] ? 1 : 0);
     for (size_t i = 0; i < count; ++i)
-        if (items[i].rows != 0 && items[i].cols != 0 && quantize_auto_path(items[i].qbuf, items[i].rows, nbits) != kPathTile)
+        if (items[i].rows != 0 && items[i].cols != 0 && quantize_auto_path(items[i].in, items[i].res_in, items[i].res_out, items[i].qbuf, items[i].rows, nbits) != kPathTile)
             launches_left++;
     if (launches_left == 0)
         return CNTKQ_OK;
@@ -701,7 +701,7 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
             for (size_t i = 0; i < count; ++i)
             {
                 const cntkq_quantize_item& it = items[i];
-                if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.qbuf, it.rows, nbits) != kPathTile)
+                if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.in, it.res_in, it.res_out, it.qbuf, it.rows, nbits) != kPathTile)
                     continue;
                 const TileGeom t = make_tile_geom(it.rows, it.cols, nbits, 0, -1, 0);
                 const size_t l = tile_lds_bytes(t, 0);
@@ -747,7 +747,7 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
     for (size_t i = 0; i < count; ++i)
     {
         const cntkq_quantize_item& it = items[i];
-        if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.qbuf, it.rows, nbits) == kPathTile)
+        if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.in, it.res_in, it.res_out, it.qbuf, it.rows, nbits) == kPathTile)
             continue;
         LaunchEvents ev;
         launches_left--;
@@ -862,7 +862,7 @@ int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_
 {
     if (h == nullptr)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: null handle");
-    if (quantize_path < kPathAuto || quantize_path > kPathWaveCol)
+    if (quantize_path < kPathAuto || quantize_path > kPathCol)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: unknown quantize path %d", quantize_path);
     if (tile_gs != 0 && (tile_gs < 8 || tile_gs > kTileThreads || (tile_gs & (tile_gs - 1)) != 0))
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: tile_gs must be a power of two in [8, 256]");

@@ -5,8 +5,8 @@
 //     (a contiguous piece of the column-major matrix). It reads gradient and residual ONCE with
 //     coalesced 16-byte loads, keeps v = g + r in LDS, takes the column statistics from LDS
 //     (wavefront shuffles, LDS across wavefronts), then packs codes and writes the new residual.
-//   * quantize_wavecol_kernel: 1-bit columns whose QWord count is a multiple of 64; one wavefront
-//     owns a column, every lane owns whole QWords and keeps its share of the column in registers.
+//   * quantize_col_kernel / stripe_reduce_col_kernel: 1-bit columns of 1024, 2048 or 4096 rows; one workgroup
+//     owns one column, 16-byte loads, column sum taken while loading.
 //   * quantize_tall_kernel: columns too tall for LDS; statistics and packing re-read global memory.
 //   * unquantize_kernel: streams codes back to fp32 (optionally accumulating).
 //
@@ -492,55 +492,120 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
         tile_store(tile, mis_s, sp, total, t);
 }
 
-// ---- quantize, 1 bit, one wavefront per column, column share in registers ---------------------------
+// ---- quantize, 1 bit, one workgroup per column, rows = 1024 * PER (PER = 1, 2, 4) ---------------------------
 //
-// rows = 2048 * WPL, nq = 64 * WPL. Lane l owns QWords l, l + 64, ...; QWord w packs rows w + k * nq, so for
-// fixed k the 64 lanes read 64 consecutive floats, and each lane builds its QWords with shifts alone.
+// 256 threads own one column: each loads PER 16-byte pieces of gradient and residual, adds them into an LDS copy
+// of the column and sums its own values on the way, so the column mean needs no second pass. The split sums are
+// then taken from LDS (thread t takes rows t, t + 256, ...), and the codes are packed from LDS by work items of
+// (QWord, run of 4 * PER bit positions), whose partial words meet in LDS. Few registers and 4..16 KB of LDS per
+// workgroup keep 8 workgroups resident per CU; that, not wider stores, is what brings this kernel to the rate of a
+// plain read-read-write stream.
 
-constexpr uint32_t kWaveColThreads = 128;
+constexpr uint32_t kColThreads = 256;
 
-// Statistics, header, codes and residual for one column held in registers by one wavefront:
-// v[c][k] is row lane + 64 * c + NQ * k; op = residual column + lane; qc = packed column record.
-template <bool ZT, int WPL>
-__device__ __forceinline__ void wavecol_stats_pack(const float (&v)[WPL][32], uint32_t lane, float* op, char* qc)
+struct ColLds
 {
-    constexpr uint32_t NQ = 64 * WPL;
-    constexpr uint32_t ROWS = 32 * NQ;
+    float* tile;      // 1024 * PER floats, 16-byte aligned
+    uint32_t* words;  // 32 * PER partial QWords
+    float* red_f;     // 2 * 4 floats
+    uint32_t* red_u;  // 4
+};
+
+template <int PER>
+__device__ __forceinline__ ColLds col_lds(f32x4* smem)
+{
+    ColLds l;
+    l.tile = reinterpret_cast<float*>(smem);
+    l.words = reinterpret_cast<uint32_t*>(l.tile + 1024 * PER);
+    l.red_f = reinterpret_cast<float*>(l.words + 32 * PER);
+    l.red_u = reinterpret_cast<uint32_t*>(l.red_f + 8);
+    return l;
+}
+
+template <int PER>
+constexpr size_t col_lds_bytes()
+{
+    return (size_t) (1024 * PER + 32 * PER + 8 + 4) * 4;
+}
+
+// Sum of the values thread tid holds when the column is cut into 16-byte pieces tid, tid + 256, ...: in that order,
+// x y z w within a piece. Both the quantize and the stripe-reduction kernel take the column mean from these
+// per-thread sums, so they produce identical headers for identical columns.
+template <int PER>
+__device__ __forceinline__ float col_thread_sum(const f32x4 (&v)[PER])
+{
+    float s = 0.0f;
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+    {
+        s += v[u].x;
+        s += v[u].y;
+        s += v[u].z;
+        s += v[u].w;
+    }
+    return s;
+}
+
+// Statistics, header, codes and residual of the column held in l.tile. csum: this thread's col_thread_sum
+// (ignored when ZT). l.words[0 .. 32 * PER) must be zero; no barrier is needed between writing l.tile / l.words
+// and calling this. res_col: the column of the residual output; qc: the packed column record (8-byte aligned).
+template <bool ZT, int PER>
+__device__ __forceinline__ void col_stats_pack(const ColLds& l, float csum, float* res_col, char* qc)
+{
+    constexpr uint32_t ROWS = 1024 * PER, NQ = 32 * PER, T = kColThreads, NW = T / 64;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     float mean = 0.0f;
     if constexpr (!ZT)
     {
-        float s = 0.0f;
+        const float s = wave_sum(csum);
+        if (lane == 0)
+            l.red_f[wave] = s;
+    }
+    __syncthreads(); // the column and the wave sums are visible
+    if constexpr (!ZT)
+    {
+        float s = l.red_f[0];
 #pragma unroll
-        for (int c = 0; c < WPL; ++c)
-#pragma unroll
-            for (int k = 0; k < 32; ++k)
-                s += v[c][k];
-        s = wave_sum(s);
+        for (uint32_t x = 1; x < NW; ++x)
+            s += l.red_f[x];
         mean = s / (float) ROWS;
     }
     float s0 = 0.0f, s1 = 0.0f;
     uint32_t n0 = 0;
 #pragma unroll
-    for (int c = 0; c < WPL; ++c)
-#pragma unroll
-        for (int k = 0; k < 32; ++k)
-        {
-            const float x = v[c][k];
-            const bool below = x < mean;
-            s0 += below ? x : 0.0f;
-            s1 += below ? 0.0f : x;
-            n0 += below ? 1u : 0u;
-        }
+    for (uint32_t i = 0; i < ROWS / T; ++i)
+    {
+        const float x = l.tile[tid + T * i];
+        const bool below = x < mean;
+        s0 += below ? x : 0.0f;
+        s1 += below ? 0.0f : x;
+        n0 += below ? 1u : 0u;
+    }
     s0 = wave_sum(s0);
     s1 = wave_sum(s1);
     n0 = wave_sum(n0);
-    const uint32_t n1 = ROWS - n0;
-    float lo, hi;
-    finish_stats_1bit<ZT>(mean, s0, s1, n0, n1, ROWS, lo, hi);
-
+    __syncthreads(); // everyone has read the wave sums of the mean
     if (lane == 0)
     {
-        f32x2 h; // NQ is even and the buffer 8-byte aligned, so every record is
+        l.red_f[wave] = s0;
+        l.red_f[4 + wave] = s1;
+        l.red_u[wave] = n0;
+    }
+    __syncthreads();
+    float S0 = l.red_f[0], S1 = l.red_f[4];
+    uint32_t N0 = l.red_u[0];
+#pragma unroll
+    for (uint32_t x = 1; x < NW; ++x)
+    {
+        S0 += l.red_f[x];
+        S1 += l.red_f[4 + x];
+        N0 += l.red_u[x];
+    }
+    float lo, hi;
+    finish_stats_1bit<ZT>(mean, S0, S1, N0, ROWS - N0, ROWS, lo, hi);
+    if (tid == 0)
+    {
+        f32x2 h;
         h.x = lo;
         h.y = hi;
         *reinterpret_cast<f32x2*>(qc) = h;
@@ -548,135 +613,130 @@ __device__ __forceinline__ void wavecol_stats_pack(const float (&v)[WPL][32], ui
     const ValueQ vq = make_vq<1>(lo, hi);
     const float val0 = unquantize_value<1>(vq, 0u);
     const float val1 = unquantize_value<1>(vq, 1u);
-    uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
+    // work item = (QWord p, chunk of KS bit positions); NQ * (32 / KS) = 256 items
+    constexpr uint32_t KS = 4 * PER;
+    const uint32_t p = tid % NQ, chunk = tid / NQ;
+    uint32_t word = 0;
 #pragma unroll
-    for (int c = 0; c < WPL; ++c)
+    for (uint32_t kk = 0; kk < KS; ++kk)
     {
-        uint32_t word = 0;
-#pragma unroll
-        for (int k = 0; k < 32; ++k)
-        {
-            const float x = v[c][k];
-            const uint32_t code = quantize_value<1, ZT>(vq, x);
-            __builtin_nontemporal_store(x - (code ? val1 : val0), op + 64u * c + NQ * k);
-            word |= code << k;
-        }
-        bits[lane + 64u * c] = word;
+        const uint32_t k = chunk * KS + kk;
+        const uint32_t i = p + NQ * k;
+        const float x = l.tile[i];
+        const uint32_t code = quantize_value<1, ZT>(vq, x);
+        __builtin_nontemporal_store(x - (code ? val1 : val0), res_col + i);
+        word |= code << k;
     }
+    atomicOr(&l.words[p], word);
+    __syncthreads();
+    if (tid < NQ)
+        reinterpret_cast<uint32_t*>(qc + 8)[tid] = l.words[tid];
 }
 
-template <bool ZT, int WPL>
-__global__ __launch_bounds__(kWaveColThreads) void quantize_wavecol_kernel(const float* __restrict__ g, const float* r_in,
-                                                                           float* r_out, char* __restrict__ q,
-                                                                           uint32_t cols, uint64_t qcol)
+template <bool ZT, int PER>
+__global__ __launch_bounds__(kColThreads) void quantize_col_kernel(const float* __restrict__ g, const float* r_in, float* r_out,
+                                                                   char* __restrict__ q, uint64_t qcol)
 {
-    constexpr uint32_t NQ = 64 * WPL;
-    constexpr uint32_t ROWS = 32 * NQ;
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t j = blockIdx.x * (kWaveColThreads / 64) + (threadIdx.x >> 6);
-    if (j >= cols)
-        return; // whole wavefront leaves; no barriers below
-    const size_t base = (size_t) j * ROWS;
-    const float* gp = g + base + lane;
-    const float* rp = r_in + base + lane;
-
-    float v[WPL][32];
+    constexpr uint32_t ROWS = 1024 * PER, T = kColThreads;
+    extern __shared__ f32x4 smem_v4[];
+    const ColLds l = col_lds<PER>(smem_v4);
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * ROWS;
+    if (tid < 32 * PER)
+        l.words[tid] = 0u;
+    const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base);
+    const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base);
+    f32x4* t4 = reinterpret_cast<f32x4*>(l.tile);
+    f32x4 a[PER], b[PER];
 #pragma unroll
-    for (int c = 0; c < WPL; ++c)
+    for (int u = 0; u < PER; ++u)
+    {
+        a[u] = __builtin_nontemporal_load(g4 + tid + T * u);
+        b[u] = __builtin_nontemporal_load(r4 + tid + T * u);
+    }
 #pragma unroll
-        for (int k = 0; k < 32; ++k)
-        {
-            const uint32_t i = 64u * c + NQ * k;
-            v[c][k] = __builtin_nontemporal_load(gp + i) + __builtin_nontemporal_load(rp + i);
-        }
-    wavecol_stats_pack<ZT, WPL>(v, lane, r_out + base + lane, q + (size_t) j * qcol);
+    for (int u = 0; u < PER; ++u)
+    {
+        a[u] = a[u] + b[u];
+        t4[tid + T * u] = a[u];
+    }
+    // the whole column has been read before col_stats_pack's first barrier, so r_out may be r_in
+    col_stats_pack<ZT, PER>(l, col_thread_sum<PER>(a), r_out + base, q + (size_t) blockIdx.x * qcol);
 }
 
-// ---- stripe reduction, 1 bit, one wavefront per column (rows = 2048 * WPL) ---------------------------
-//
-// Lane l owns QWords l, l + 64, ... of the column in EVERY worker's packed stripe: it decodes its 32 * WPL rows
-// from each worker in turn, sums them in registers, adds the stripe residual and requantizes, all without LDS.
-
-template <bool ZT, int WPL>
-__global__ __launch_bounds__(kWaveColThreads) void stripe_reduce_wavecol_kernel(StripeSources src, float* stripe_res,
-                                                                                char* q_out, float* agg_out,
-                                                                                uint32_t cols, uint64_t qcol)
+// Stripe reduction in the same shape: the work item that will pack (QWord p, chunk) first decodes those bit positions
+// from every worker's packed stripe, sums them (owner first, then ascending) and adds the stripe residual.
+template <bool ZT, int PER>
+__global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSources src, float* stripe_res, char* q_out,
+                                                                        float* agg_out, uint64_t qcol)
 {
-    constexpr uint32_t NQ = 64 * WPL;
-    constexpr uint32_t ROWS = 32 * NQ;
-    constexpr uint32_t BATCH = 8;
-    const uint32_t lane = threadIdx.x & 63u;
-    // the column index is the same for the whole wavefront: keep it (and everything derived from it) scalar
-    const uint32_t j = __builtin_amdgcn_readfirstlane(blockIdx.x * (kWaveColThreads / 64) + (threadIdx.x >> 6));
-    if (j >= cols)
-        return;
-    const size_t base = (size_t) j * ROWS;
-    const size_t rec = (size_t) j * qcol;
+    constexpr uint32_t ROWS = 1024 * PER, NQ = 32 * PER, T = kColThreads, KS = 4 * PER, BATCH = 8;
+    extern __shared__ f32x4 smem_v4[];
+    const ColLds l = col_lds<PER>(smem_v4);
+    float* dec = reinterpret_cast<float*>(l.red_u + 4); // two reconstruction levels per worker, in summation order
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * ROWS;
+    const size_t rec = (size_t) blockIdx.x * qcol;
     const uint32_t K = src.workers;
+    if (tid < NQ)
+        l.words[tid] = 0u;
+    if (tid < K)
+    {
+        const float* h = reinterpret_cast<const float*>(src.q[stripe_order(tid, src.owner)] + rec);
+        const ValueQ vq = make_vq<1>(h[0], h[1]);
+        dec[2 * tid] = unquantize_value<1>(vq, 0u);
+        dec[2 * tid + 1] = unquantize_value<1>(vq, 1u);
+    }
+    __syncthreads();
 
-    float sres[WPL][32];
-    const float* sp = stripe_res + base + lane;
-#pragma unroll
-    for (int c = 0; c < WPL; ++c)
-#pragma unroll
-        for (int k = 0; k < 32; ++k)
-            sres[c][k] = __builtin_nontemporal_load(sp + 64u * c + NQ * k);
-
-    float acc[WPL][32];
+    const uint32_t p = tid % NQ, chunk = tid / NQ;
+    const uint32_t sh0 = chunk * KS;
+    float acc[KS];
     for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
     {
-        uint32_t word[BATCH][WPL];
-        float lo[BATCH], hi[BATCH];
+        uint32_t word[BATCH];
+#pragma unroll
+        for (uint32_t u = 0; u < BATCH; ++u)
+            if (n0 + u < K)
+                word[u] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + rec + 8)[p];
 #pragma unroll
         for (uint32_t u = 0; u < BATCH; ++u)
         {
             if (n0 + u < K)
             {
-                const char* qc = src.q[stripe_order(n0 + u, src.owner)] + rec;
-                lo[u] = reinterpret_cast<const float*>(qc)[0];
-                hi[u] = reinterpret_cast<const float*>(qc)[1];
+                const float val0 = dec[2 * (n0 + u)], val1 = dec[2 * (n0 + u) + 1];
+                const uint32_t bits = word[u] >> sh0;
 #pragma unroll
-                for (int c = 0; c < WPL; ++c)
-                    word[u][c] = reinterpret_cast<const uint32_t*>(qc + 8)[lane + 64u * c];
-            }
-        }
-#pragma unroll
-        for (uint32_t u = 0; u < BATCH; ++u)
-        {
-            if (n0 + u < K)
-            {
-                const ValueQ vq = make_vq<1>(lo[u], hi[u]);
-                const float val0 = unquantize_value<1>(vq, 0u);
-                const float val1 = unquantize_value<1>(vq, 1u);
-#pragma unroll
-                for (int c = 0; c < WPL; ++c)
-#pragma unroll
-                    for (int k = 0; k < 32; ++k)
-                    {
-                        const float x = ((word[u][c] >> k) & 1u) ? val1 : val0;
-                        // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
-                        acc[c][k] = (n0 + u == 0) ? x : x + acc[c][k];
-                    }
+                for (uint32_t kk = 0; kk < KS; ++kk)
+                {
+                    const float x = ((bits >> kk) & 1u) ? val1 : val0;
+                    // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
+                    acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
+                }
             }
         }
     }
-
-    if (agg_out != nullptr)
+    const float* sp = stripe_res + base;
+#pragma unroll
+    for (uint32_t kk = 0; kk < KS; ++kk)
     {
-        float* ap = agg_out + base + lane;
-#pragma unroll
-        for (int c = 0; c < WPL; ++c)
-#pragma unroll
-            for (int k = 0; k < 32; ++k)
-                ap[64u * c + NQ * k] = acc[c][k];
+        const uint32_t i = p + NQ * (sh0 + kk);
+        if (agg_out != nullptr)
+            agg_out[base + i] = acc[kk];
+        l.tile[i] = acc[kk] + __builtin_nontemporal_load(sp + i);
     }
-    float v[WPL][32];
+    float csum = 0.0f;
+    if constexpr (!ZT)
+    {
+        __syncthreads();
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(l.tile);
+        f32x4 v[PER];
 #pragma unroll
-    for (int c = 0; c < WPL; ++c)
-#pragma unroll
-        for (int k = 0; k < 32; ++k)
-            v[c][k] = acc[c][k] + sres[c][k];
-    wavecol_stats_pack<ZT, WPL>(v, lane, stripe_res + base + lane, q_out + rec);
+        for (int u = 0; u < PER; ++u)
+            v[u] = t4[tid + T * u];
+        csum = col_thread_sum<PER>(v);
+    }
+    col_stats_pack<ZT, PER>(l, csum, stripe_res + base, q_out + rec);
 }
 
 // ---- quantize, columns too tall for LDS: one workgroup per column, global memory re-read -------------

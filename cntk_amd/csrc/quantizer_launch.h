@@ -19,7 +19,7 @@ enum QuantizePath
     kPathAuto = 0,
     kPathTile = 1,    // LDS-staged column tile (rows <= kTileMaxRows)
     kPathTall = 2,    // one workgroup per column, global re-read (any rows)
-    kPathWaveCol = 3  // 1 bit, rows in {2048, 4096}, one wavefront per column in registers
+    kPathCol = 3      // 1 bit, rows in {1024, 2048, 4096}, one workgroup per column, column in LDS
 };
 
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
@@ -144,11 +144,27 @@ struct StripeLauncher
     }
 };
 
-inline bool wavecol_applicable(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows,
-                               size_t nbits)
+inline bool col_applicable(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
 {
-    (void) g, (void) r_in, (void) r_out;
-    return nbits == 1 && (rows == 2048 || rows == 4096) && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
+    const uintptr_t m = reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(r_in) | reinterpret_cast<uintptr_t>(r_out);
+    return nbits == 1 && (rows == 1024 || rows == 2048 || rows == 4096) && (m & 15u) == 0 &&
+           (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
+}
+
+template <bool ZT, int PER>
+inline void launch_quantize_col(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
+                                uint64_t qcol)
+{
+    hipExtLaunchKernelGGL((quantize_col_kernel<ZT, PER>), dim3(cols), dim3(kColThreads), col_lds_bytes<PER>(), s, ev.start, ev.stop, 0, g,
+                          r_in, r_out, q, qcol);
+}
+
+template <bool ZT, int PER>
+inline void launch_stripe_col(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
+                              uint32_t cols, uint64_t qcol)
+{
+    hipExtLaunchKernelGGL((stripe_reduce_col_kernel<ZT, PER>), dim3(cols), dim3(kColThreads), col_lds_bytes<PER>() + 2 * kMaxWorkers * 4, s,
+                          ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, qcol);
 }
 
 // Launches the quantize kernel(s) for one matrix. rows, cols > 0; pointers 4-byte aligned (checked by caller).
@@ -162,32 +178,23 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     {
         if (rows > kTileMaxRows)
             path = kPathTall;
-        else if (wavecol_applicable(g, r_in, r_out, q, rows, nbits))
-            path = kPathWaveCol;
+        else if (col_applicable(g, r_in, r_out, q, rows, nbits))
+            path = kPathCol;
         else
             path = kPathTile;
     }
-    if (path == kPathWaveCol)
+    if (path == kPathCol)
     {
-        if (!wavecol_applicable(g, r_in, r_out, q, rows, nbits))
+        if (!col_applicable(g, r_in, r_out, q, rows, nbits))
             return hipErrorInvalidValue;
-        constexpr uint32_t per_block = kWaveColThreads / 64;
-        const uint32_t blocks = (uint32_t) ((cols + per_block - 1) / per_block);
         const uint64_t qcol = qcol_bytes(nbits, rows);
-        if (rows == 2048)
-        {
-            if (zt)
-                hipExtLaunchKernelGGL((quantize_wavecol_kernel<true, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, qc, (uint32_t) cols, qcol);
-            else
-                hipExtLaunchKernelGGL((quantize_wavecol_kernel<false, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, qc, (uint32_t) cols, qcol);
-        }
+        const uint32_t c = (uint32_t) cols;
+        if (rows == 1024)
+            zt ? launch_quantize_col<true, 1>(s, ev, g, r_in, r_out, qc, c, qcol) : launch_quantize_col<false, 1>(s, ev, g, r_in, r_out, qc, c, qcol);
+        else if (rows == 2048)
+            zt ? launch_quantize_col<true, 2>(s, ev, g, r_in, r_out, qc, c, qcol) : launch_quantize_col<false, 2>(s, ev, g, r_in, r_out, qc, c, qcol);
         else
-        {
-            if (zt)
-                hipExtLaunchKernelGGL((quantize_wavecol_kernel<true, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, qc, (uint32_t) cols, qcol);
-            else
-                hipExtLaunchKernelGGL((quantize_wavecol_kernel<false, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, qc, (uint32_t) cols, qcol);
-        }
+            zt ? launch_quantize_col<true, 4>(s, ev, g, r_in, r_out, qc, c, qcol) : launch_quantize_col<false, 4>(s, ev, g, r_in, r_out, qc, c, qcol);
         return hipGetLastError();
     }
     if (path == kPathTile)
@@ -211,26 +218,19 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
     bool aligned8 = (reinterpret_cast<uintptr_t>(q_out) & 7u) == 0;
     for (uint32_t w = 0; w < src.workers; ++w)
         aligned8 = aligned8 && (reinterpret_cast<uintptr_t>(src.q[w]) & 7u) == 0;
-    if (tune.quantize_path != kPathTile && nbits == 1 && (rows == 2048 || rows == 4096) && aligned8)
+    if ((tune.quantize_path == kPathAuto || tune.quantize_path == kPathCol) && nbits == 1 &&
+        (rows == 1024 || rows == 2048 || rows == 4096) && aligned8)
     {
-        constexpr uint32_t per_block = kWaveColThreads / 64;
-        const uint32_t blocks = (uint32_t) ((cols + per_block - 1) / per_block);
+        // same column statistics, in the same order, as quantize_col_kernel
         const uint64_t qcol = qcol_bytes(nbits, rows);
+        const uint32_t c = (uint32_t) cols;
         char* qo = static_cast<char*>(q_out);
-        if (rows == 2048)
-        {
-            if (zt)
-                hipExtLaunchKernelGGL((stripe_reduce_wavecol_kernel<true, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, src, stripe_res, qo, agg_out, (uint32_t) cols, qcol);
-            else
-                hipExtLaunchKernelGGL((stripe_reduce_wavecol_kernel<false, 1>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, src, stripe_res, qo, agg_out, (uint32_t) cols, qcol);
-        }
+        if (rows == 1024)
+            zt ? launch_stripe_col<true, 1>(s, ev, src, stripe_res, qo, agg_out, c, qcol) : launch_stripe_col<false, 1>(s, ev, src, stripe_res, qo, agg_out, c, qcol);
+        else if (rows == 2048)
+            zt ? launch_stripe_col<true, 2>(s, ev, src, stripe_res, qo, agg_out, c, qcol) : launch_stripe_col<false, 2>(s, ev, src, stripe_res, qo, agg_out, c, qcol);
         else
-        {
-            if (zt)
-                hipExtLaunchKernelGGL((stripe_reduce_wavecol_kernel<true, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, src, stripe_res, qo, agg_out, (uint32_t) cols, qcol);
-            else
-                hipExtLaunchKernelGGL((stripe_reduce_wavecol_kernel<false, 2>), dim3(blocks), dim3(kWaveColThreads), 0, s, ev.start, ev.stop, 0, src, stripe_res, qo, agg_out, (uint32_t) cols, qcol);
-        }
+            zt ? launch_stripe_col<true, 4>(s, ev, src, stripe_res, qo, agg_out, c, qcol) : launch_stripe_col<false, 4>(s, ev, src, stripe_res, qo, agg_out, c, qcol);
         return hipGetLastError();
     }
     // Same tile geometry as launch_quantize would use for a matrix of this height, so that the statistics are summed in
@@ -382,12 +382,12 @@ inline hipError_t launch_unquantize_batch(hipStream_t s, LaunchEvents ev, const 
 }
 
 // which path launch_quantize would take for this matrix
-inline int quantize_auto_path(const void* q, size_t rows, size_t nbits)
+inline int quantize_auto_path(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
 {
     if (rows > kTileMaxRows)
         return kPathTall;
-    if (wavecol_applicable(nullptr, nullptr, nullptr, q, rows, nbits))
-        return kPathWaveCol;
+    if (col_applicable(g, r_in, r_out, q, rows, nbits))
+        return kPathCol;
     return kPathTile;
 }
 

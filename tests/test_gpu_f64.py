@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 
 F64 = np.float64
 VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False), (64, False)]
-PATH_AUTO, PATH_TILE, PATH_TALL, PATH_WAVECOL = 0, 1, 2, 3
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL = 0, 1, 2, 3
 
 
 def say(*a):
@@ -159,7 +159,7 @@ def test_kernel_paths_f64(case):
 
 def test_unsupported_paths_are_refused_f64():
     qz = MatrixQuantizerImpl.Create(0, False)
-    qz._set_tuning(quantize_path=PATH_WAVECOL)
+    qz._set_tuning(quantize_path=PATH_COL)  # exists for float only
     with pytest.raises(cntk_amd.QuantizerLogicError):
         gpu_quantize(qz, datagen.normal(1, 2048, 4, dtype=F64), zeros(2048, 4), 1, False)
     qz._set_tuning(quantize_path=PATH_TILE)

@@ -21,7 +21,7 @@ from cntk_amd import Matrix, MatrixQuantizerImpl, QuantizedMatrix
 pytestmark = pytest.mark.gpu
 
 VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False)]
-PATH_AUTO, PATH_TILE, PATH_TALL, PATH_WAVECOL = 0, 1, 2, 3
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL = 0, 1, 2, 3
 
 
 def say(*a):
@@ -143,27 +143,44 @@ def test_kernel_paths(case):
     say("  ", rep)
 
 
-@pytest.mark.parametrize("rows", [2048, 4096])
-def test_wavefront_per_column_path(rows):
+@pytest.mark.parametrize("rows", [1024, 2048, 4096])
+def test_workgroup_per_column_path(rows):
+    """The 1-bit kernel that keeps one column per workgroup in LDS: the path the automatic choice takes for these
+    heights, here also forced, against the oracle and against the general tile kernel's codes."""
     qz = MatrixQuantizerImpl.Create(0, False)
-    qz._set_tuning(quantize_path=PATH_WAVECOL)
     rep = parity.Report()
-    for cols in (1, 4, 7, 130):
-        for zt in (False, True):
-            say("wavecol", rows, cols, zt)
-            def make(it):
-                a = datagen.normal(rows + cols + it, rows, cols) + np.float32(0.003 * it)
-                a = np.asfortranarray(a.astype(np.float32))
-                if cols > 2:
-                    a[:, 1] = 0.0
-                return a
-            run_chain(qz, rows, cols, 1, zt, make, 3, rep)
+    for path in (PATH_COL, PATH_AUTO):
+        qz._set_tuning(quantize_path=path)
+        for cols in (1, 4, 7, 130):
+            for zt in (False, True):
+                say("column kernel", rows, cols, zt, "path", path)
+                def make(it):
+                    a = datagen.normal(rows + cols + it, rows, cols) + np.float32(0.003 * it)
+                    a = np.asfortranarray(a.astype(np.float32))
+                    if cols > 2:
+                        a[:, 1] = 0.0
+                    return a
+                run_chain(qz, rows, cols, 1, zt, make, 3, rep)
     say("  ", rep)
-    # shapes the path does not cover are refused, not mis-computed
+    qz._set_tuning(quantize_path=PATH_COL)
+    # shapes and alignments the path does not cover are refused when forced, not mis-computed
     with pytest.raises(cntk_amd.QuantizerLogicError):
         gpu_quantize(qz, datagen.normal(1, 512, 4), np.zeros((512, 4), np.float32, order="F"), 1, False)
     with pytest.raises(cntk_amd.QuantizerLogicError):
         gpu_quantize(qz, datagen.normal(1, rows, 4), np.zeros((rows, 4), np.float32, order="F"), 2, False)
+    # a gradient that starts 4 bytes off a 16-byte boundary: refused when forced, served by the tile kernel otherwise
+    cols = 5
+    g = datagen.normal(5, rows, cols)
+    big = torch.zeros(rows * cols + 4, dtype=torch.float32, device="cuda:0")
+    big[1:1 + rows * cols] = torch.from_numpy(g.reshape(-1, order="F").copy()).cuda()
+    G = Matrix(rows, cols, 0, big[1:1 + rows * cols])
+    R, Q = Matrix(rows, cols), QuantizedMatrix(rows, cols, 1, 0)
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        qz.QuantizeAsync(G, R, Q, R, False)
+    qz._set_tuning(quantize_path=PATH_AUTO)
+    qz.QuantizeAsync(G, R, Q, R, False)
+    qz.WaitQuantizeAsyncDone()
+    parity.check_quantize(g, np.zeros_like(g, order="F"), Q.to_numpy(), R.to_numpy(), 1, False, report=rep)
 
 
 def test_unquantize_variants(quantizer):

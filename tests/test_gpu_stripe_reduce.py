@@ -50,7 +50,7 @@ CASES = [
     (147, 64, 8, 4, False), (576, 24, 5, 8, False), (100, 9, 3, 16, False), (64, 12, 4, 32, False),
     (2048, 48, 8, 1, False), (2048, 48, 8, 1, True), (2048, 16, 8, 2, False), (4608, 8, 2, 1, False),
     (9304, 3, 3, 1, True), (33, 5, 8, 1, False), (512, 64, 64, 1, False), (4096, 7, 3, 1, False), (4096, 4, 12, 1, True),
-    (2048, 20, 11, 1, False),
+    (2048, 20, 11, 1, False), (1024, 24, 4, 1, False), (1024, 9, 64, 1, True), (4096, 5, 64, 1, False),
 ]
 
 
@@ -68,8 +68,9 @@ def test_stripe_reduce(case):
             continue
         say("stripe reduce", case, "owner", owner, "cols", start, n)
         sres = datagen.normal(900 + owner, rows, n, 0.003)
-        # 1-bit stripes of 2048 or 4096 rows have a register-resident kernel; run the general tile kernel on them too
-        variants = [(True, 0), (False, 0)] + ([(True, 1)] if (nbits == 1 and rows in (2048, 4096)) else [])
+        # 1-bit stripes of 1024, 2048 or 4096 rows have a kernel of their own (one workgroup per column); run the
+        # general tile kernel (path 1) on them too
+        variants = [(True, 0), (False, 0)] + ([(True, 1)] if (nbits == 1 and rows in (1024, 2048, 4096)) else [])
         for alias, path in variants:
             qz._set_tuning(quantize_path=path)
             q_new, s_new, agg = gpu_stripe_reduce(qz, qs, owner, rows, cols, nbits, sres, zt, alias_out=alias)
