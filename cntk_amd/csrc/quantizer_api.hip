@@ -12,6 +12,7 @@
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <vector>
 
 using namespace cntkq;
 
@@ -134,6 +135,24 @@ bool aligned_for(const void* p)
 
 } // namespace
 
+struct BatchTable
+{
+    std::vector<char> key;   // the item list and parameters the table was built for
+    char* host = nullptr;    // pinned
+    char* dev = nullptr;
+    size_t capacity = 0;
+    hipEvent_t event = nullptr; // set when the last kernel that reads the table has finished
+    bool in_flight = false;
+    // launch parameters of the two LDS classes and the matrices that get a launch of their own
+    size_t members[2] = {0, 0};
+    uint32_t blocks[2] = {0, 0};
+    size_t lds[2] = {0, 0};
+    size_t first_entry[2] = {0, 0};
+    size_t first_begin[2] = {0, 0};
+    size_t entries_bytes = 0;
+    std::vector<size_t> own;
+};
+
 struct cntkq_quantizer
 {
     int device = 0;
@@ -159,15 +178,12 @@ struct cntkq_quantizer
     bool staging_read_pending = false; // a kernel reading the staging buffer may still be running
     char* staging = nullptr;      // device buffer used when the packed matrix lives in host memory
     size_t staging_bytes = 0;
-    // entry tables of batched launches: a ring of slots, each with a pinned host copy and a device copy; a slot is
-    // reused only after the last kernel that read it has finished (its event)
-    static constexpr int kBatchSlots = 4;
-    char* batch_host = nullptr;
-    char* batch_dev = nullptr;
-    size_t batch_slot_bytes = 0;
-    int batch_next = 0;
-    hipEvent_t batch_event[kBatchSlots] = {nullptr, nullptr, nullptr, nullptr};
-    bool batch_used[kBatchSlots] = {false, false, false, false};
+    // entry tables of the batched calls, one for quantize and one for unquantize. A gradient set is the same list of
+    // matrices step after step, so the table built for a list is kept (host key, pinned host copy, device copy, launch
+    // parameters) and a call with the same list only launches. A table is rebuilt only after the last kernel that
+    // reads it has finished (its event).
+    BatchTable quantize_table;
+    BatchTable unquantize_table;
     LaunchTuning tune;
 };
 
@@ -213,38 +229,63 @@ int ensure_staging(cntkq_quantizer* h, size_t bytes)
     return CNTKQ_OK;
 }
 
-// Makes a table slot of at least `bytes` available for writing; returns its index.
-int acquire_batch_slot(cntkq_quantizer* h, size_t bytes, int* slot_out)
+// True when `t` was built for exactly this item list and parameters.
+bool table_matches(const BatchTable& t, const void* items, size_t items_bytes, const size_t (&params)[3])
 {
-    if (bytes > h->batch_slot_bytes)
+    if (t.key.size() != items_bytes + sizeof params)
+        return false;
+    return std::memcmp(t.key.data(), params, sizeof params) == 0 && std::memcmp(t.key.data() + sizeof params, items, items_bytes) == 0;
+}
+
+// Makes `t` writable with room for `bytes`: waits for the kernels that still read it, grows the buffers.
+int table_begin_rebuild(BatchTable& t, size_t bytes)
+{
+    t.key.clear();
+    if (t.event == nullptr)
+        HIP_TRY(hipEventCreateWithFlags(&t.event, hipEventDisableTiming), "hipEventCreateWithFlags failed");
+    if (t.in_flight)
     {
-        for (int i = 0; i < cntkq_quantizer::kBatchSlots; ++i)
-            if (h->batch_used[i])
-                HIP_TRY(hipEventSynchronize(h->batch_event[i]), "hipEventSynchronize failed");
-        if (h->batch_host != nullptr)
-            HIP_TRY(hipHostFree(h->batch_host), "hipHostFree failed");
-        if (h->batch_dev != nullptr)
-            HIP_TRY(hipFree(h->batch_dev), "hipFree failed");
-        h->batch_host = h->batch_dev = nullptr;
-        const size_t slot = (bytes * 2 + 4095) & ~(size_t) 4095;
-        void* p = nullptr;
-        HIP_TRY(hipHostMalloc(&p, slot * cntkq_quantizer::kBatchSlots, hipHostMallocDefault), "hipHostMalloc of the batch table failed");
-        h->batch_host = static_cast<char*>(p);
-        HIP_TRY(hipMalloc(&p, slot * cntkq_quantizer::kBatchSlots), "hipMalloc of the batch table failed");
-        h->batch_dev = static_cast<char*>(p);
-        h->batch_slot_bytes = slot;
-        for (int i = 0; i < cntkq_quantizer::kBatchSlots; ++i)
-            h->batch_used[i] = false;
+        HIP_TRY(hipEventSynchronize(t.event), "hipEventSynchronize failed");
+        t.in_flight = false;
     }
-    const int slot = h->batch_next;
-    h->batch_next = (slot + 1) % cntkq_quantizer::kBatchSlots;
-    if (h->batch_event[slot] == nullptr)
-        HIP_TRY(hipEventCreateWithFlags(&h->batch_event[slot], hipEventDisableTiming), "hipEventCreateWithFlags failed");
-    if (h->batch_used[slot])
-        HIP_TRY(hipEventSynchronize(h->batch_event[slot]), "hipEventSynchronize failed");
-    h->batch_used[slot] = true;
-    *slot_out = slot;
+    if (bytes > t.capacity)
+    {
+        if (t.host != nullptr)
+            HIP_TRY(hipHostFree(t.host), "hipHostFree failed");
+        if (t.dev != nullptr)
+            HIP_TRY(hipFree(t.dev), "hipFree failed");
+        t.host = t.dev = nullptr;
+        t.capacity = 0;
+        const size_t cap = (bytes * 2 + 4095) & ~(size_t) 4095;
+        void* p = nullptr;
+        HIP_TRY(hipHostMalloc(&p, cap, hipHostMallocDefault), "hipHostMalloc of the batch table failed");
+        t.host = static_cast<char*>(p);
+        HIP_TRY(hipMalloc(&p, cap), "hipMalloc of the batch table failed");
+        t.dev = static_cast<char*>(p);
+        t.capacity = cap;
+    }
     return CNTKQ_OK;
+}
+
+void table_set_key(BatchTable& t, const void* items, size_t items_bytes, const size_t (&params)[3])
+{
+    t.key.resize(items_bytes + sizeof params);
+    std::memcpy(t.key.data(), params, sizeof params);
+    std::memcpy(t.key.data() + sizeof params, items, items_bytes);
+}
+
+void table_destroy(BatchTable& t)
+{
+    if (t.event != nullptr)
+    {
+        if (t.in_flight)
+            (void) hipEventSynchronize(t.event);
+        (void) hipEventDestroy(t.event);
+    }
+    if (t.host != nullptr)
+        (void) hipHostFree(t.host);
+    if (t.dev != nullptr)
+        (void) hipFree(t.dev);
 }
 
 int sync_event(hipEvent_t ev) // SyncEvent (Source/Math/MatrixQuantizerGPU.cu:68-80)
@@ -532,19 +573,8 @@ int cntkq_destroy(cntkq_quantizer* h)
     if (h->ev_stripe) (void) hipEventSynchronize(h->ev_stripe);
     if (h->staging != nullptr)
         (void) hipFree(h->staging);
-    for (int i = 0; i < cntkq_quantizer::kBatchSlots; ++i)
-    {
-        if (h->batch_event[i] != nullptr)
-        {
-            if (h->batch_used[i])
-                (void) hipEventSynchronize(h->batch_event[i]);
-            (void) hipEventDestroy(h->batch_event[i]);
-        }
-    }
-    if (h->batch_host != nullptr)
-        (void) hipHostFree(h->batch_host);
-    if (h->batch_dev != nullptr)
-        (void) hipFree(h->batch_dev);
+    table_destroy(h->quantize_table);
+    table_destroy(h->unquantize_table);
     hipEvent_t evs[] = {h->ev_quantize, h->ev_fetch, h->ev_assign, h->ev_unquantize, h->ev_stripe, h->ev_main};
     for (hipEvent_t e : evs)
         if (e != nullptr)
@@ -655,105 +685,137 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
     const bool zt = zero_threshold_for_1bit != 0;
     DeviceGuard guard(h->device);
     hipStream_t s = work_stream(h);
+    BatchTable& tb = h->quantize_table;
+    const size_t params[3] = {count, nbits, (size_t) (zt ? 1 : 0)};
+    const size_t items_bytes = count * sizeof(cntkq_quantize_item);
 
-    // small-LDS tiles, large-LDS tiles (one launch each), and matrices that get a launch of their own
-    constexpr size_t kSmallLds = 20 * 1024;
-    size_t n_tile[2] = {0, 0};
-    for (size_t i = 0; i < count; ++i)
+    if (!table_matches(tb, items, items_bytes, params))
     {
-        const cntkq_quantize_item& it = items[i];
-        if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.in, it.res_in, it.res_out, it.qbuf, it.rows, nbits) != kPathTile)
-            continue;
-        const TileGeom t = make_tile_geom(it.rows, it.cols, nbits, 0, -1, 0);
-        n_tile[tile_lds_bytes(t, 0) <= kSmallLds ? 0 : 1]++;
-    }
-    const size_t n_tiles_total = n_tile[0] + n_tile[1];
-    hipEvent_t done = h->ev_quantize;
-    size_t launches_left = (n_tile[0] ? 1 : 0) + (n_tile[1] ? 1 : 0);
-    for (size_t i = 0; i < count; ++i)
-        if (items[i].rows != 0 && items[i].cols != 0 && quantize_auto_path(items[i].in, items[i].res_in, items[i].res_out, items[i].qbuf, items[i].rows, nbits) != kPathTile)
-            launches_left++;
-    if (launches_left == 0)
-        return CNTKQ_OK;
-
-    if (n_tiles_total != 0)
-    {
-        const size_t entries_bytes = n_tiles_total * sizeof(QuantizeBatchEntry);
-        const size_t begins_bytes = (n_tiles_total + 2) * sizeof(uint32_t);
-        int slot = 0;
-        int rc = acquire_batch_slot(h, entries_bytes + begins_bytes + 64, &slot);
+        // Every matrix is a member of one of two grid-wide launches (small / large LDS need), as a run of column
+        // tiles or of single columns; only columns too tall for LDS get a launch of their own. Large matrices gain
+        // from sharing a grid too: their workgroups fill the gaps the others leave.
+        constexpr size_t kSmallLds = 20 * 1024;
+        struct Plan
+        {
+            int kind; // -1 skip, 0 tiles in a batch, 1 columns in a batch, 2 own launch
+            int cls;  // LDS class of a batch member
+            size_t lds;
+            uint64_t blocks;
+            TileGeom t;
+            ColGeom c;
+        };
+        std::vector<Plan> plans(count);
+        size_t members[2] = {0, 0};
+        for (size_t i = 0; i < count; ++i)
+        {
+            const cntkq_quantize_item& it = items[i];
+            Plan& p = plans[i];
+            std::memset(&p, 0, sizeof p);
+            p.kind = -1;
+            if (it.rows == 0 || it.cols == 0)
+                continue;
+            const int path = quantize_auto_path(it.in, it.res_in, it.res_out, it.qbuf, it.rows, nbits);
+            if (path == kPathTile)
+            {
+                p.kind = 0;
+                p.t = make_tile_geom(it.rows, it.cols, nbits, 0, -1, 0);
+                p.lds = tile_lds_bytes(p.t, 0);
+                p.blocks = (p.t.cols + p.t.cols_per_tile - 1) / p.t.cols_per_tile;
+            }
+            else if (path == kPathCol)
+            {
+                p.kind = 1;
+                p.c = make_col_geom(it.rows, nbits);
+                p.lds = colg_lds_bytes_rt(p.c, nbits);
+                p.blocks = it.cols;
+            }
+            else
+            {
+                p.kind = 2;
+                continue;
+            }
+            p.cls = p.lds <= kSmallLds ? 0 : 1;
+            members[p.cls]++;
+        }
+        const size_t total = members[0] + members[1];
+        const size_t entries_bytes = total * sizeof(QuantizeBatchEntry);
+        int rc = table_begin_rebuild(tb, entries_bytes + (total + 2) * sizeof(uint32_t) + 64);
         if (rc != CNTKQ_OK)
             return rc;
-        done = h->batch_event[slot];
-        char* host = h->batch_host + (size_t) slot * h->batch_slot_bytes;
-        char* dev = h->batch_dev + (size_t) slot * h->batch_slot_bytes;
-        QuantizeBatchEntry* he = reinterpret_cast<QuantizeBatchEntry*>(host);
-        uint32_t* hb = reinterpret_cast<uint32_t*>(host + entries_bytes);
-        size_t lds[2] = {0, 0};
-        uint32_t total_tiles[2] = {0, 0};
+        QuantizeBatchEntry* he = reinterpret_cast<QuantizeBatchEntry*>(tb.host);
+        uint32_t* hb = reinterpret_cast<uint32_t*>(tb.host + entries_bytes);
         size_t e = 0, bpos = 0;
-        size_t first_entry[2] = {0, 0}, first_begin[2] = {0, 0};
+        tb.own.clear();
         for (int cls = 0; cls < 2; ++cls)
         {
-            first_entry[cls] = e;
-            first_begin[cls] = bpos;
-            uint64_t tiles_acc = 0;
+            tb.first_entry[cls] = e;
+            tb.first_begin[cls] = bpos;
+            tb.lds[cls] = 0;
+            uint64_t acc = 0;
             for (size_t i = 0; i < count; ++i)
             {
-                const cntkq_quantize_item& it = items[i];
-                if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.in, it.res_in, it.res_out, it.qbuf, it.rows, nbits) != kPathTile)
+                const Plan& p = plans[i];
+                if ((p.kind != 0 && p.kind != 1) || p.cls != cls)
                     continue;
-                const TileGeom t = make_tile_geom(it.rows, it.cols, nbits, 0, -1, 0);
-                const size_t l = tile_lds_bytes(t, 0);
-                if ((l <= kSmallLds ? 0 : 1) != cls)
-                    continue;
-                he[e].g = it.in;
-                he[e].r_in = it.res_in;
-                he[e].r_out = it.res_out;
-                he[e].q = static_cast<char*>(it.qbuf);
-                he[e].t = t;
-                hb[bpos++] = (uint32_t) tiles_acc;
-                tiles_acc += (t.cols + t.cols_per_tile - 1) / t.cols_per_tile;
-                if (tiles_acc > 0x7FFFFFFFull)
-                    return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: too many tiles in one batch");
-                if (l > lds[cls])
-                    lds[cls] = l;
+                he[e].g = items[i].in;
+                he[e].r_in = items[i].res_in;
+                he[e].r_out = items[i].res_out;
+                he[e].q = static_cast<char*>(items[i].qbuf);
+                he[e].kind = (uint32_t) p.kind;
+                he[e].pad = 0;
+                he[e].t = p.t;
+                he[e].c = p.c;
+                hb[bpos++] = (uint32_t) acc;
+                acc += p.blocks;
+                if (acc > 0x7FFFFFFFull)
+                    return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: too many workgroups in one batch");
+                if (p.lds > tb.lds[cls])
+                    tb.lds[cls] = p.lds;
                 e++;
             }
-            if (n_tile[cls] != 0)
-                hb[bpos++] = (uint32_t) tiles_acc; // sentinel
-            total_tiles[cls] = (uint32_t) tiles_acc;
+            if (members[cls] != 0)
+                hb[bpos++] = (uint32_t) acc; // sentinel
+            tb.members[cls] = members[cls];
+            tb.blocks[cls] = (uint32_t) acc;
         }
-        HIP_TRY(hipMemcpyAsync(dev, host, entries_bytes + bpos * sizeof(uint32_t), hipMemcpyHostToDevice, s), "hipMemcpyAsync of the batch table failed");
-        for (int cls = 0; cls < 2; ++cls)
-        {
-            if (n_tile[cls] == 0)
-                continue;
-            LaunchEvents ev;
-            launches_left--;
-            ev.stop = launches_left == 0 ? done : nullptr;
-            const QuantizeBatchEntry* de = reinterpret_cast<const QuantizeBatchEntry*>(dev) + first_entry[cls];
-            const uint32_t* db = reinterpret_cast<const uint32_t*>(dev + entries_bytes) + first_begin[cls];
-            HIP_TRY(launch_quantize_tile_batch(s, ev, de, db, (uint32_t) n_tile[cls], total_tiles[cls], lds[cls], nbits, zt),
-                    "batched quantize kernel launch failed");
-        }
-        if (launches_left != 0)
-        {
-            // the table slot is guarded by its own event, which the LAST kernel of the batch will carry; the kernels
-            // in between run on the same stream, so they are finished by then as well
-        }
+        for (size_t i = 0; i < count; ++i)
+            if (plans[i].kind == 2)
+                tb.own.push_back(i);
+        tb.entries_bytes = entries_bytes;
+        if (total != 0)
+            HIP_TRY(hipMemcpyAsync(tb.dev, tb.host, entries_bytes + bpos * sizeof(uint32_t), hipMemcpyHostToDevice, s),
+                    "hipMemcpyAsync of the batch table failed");
+        table_set_key(tb, items, items_bytes, params);
+    }
+
+    size_t launches_left = (tb.members[0] ? 1 : 0) + (tb.members[1] ? 1 : 0) + tb.own.size();
+    if (launches_left == 0)
+        return CNTKQ_OK;
+    // the last kernel of the call carries the table's event: the kernels before it run on the same stream
+    hipEvent_t done = tb.event;
+    for (int cls = 0; cls < 2; ++cls)
+    {
+        if (tb.members[cls] == 0)
+            continue;
+        LaunchEvents ev;
+        launches_left--;
+        ev.stop = launches_left == 0 ? done : nullptr;
+        const QuantizeBatchEntry* de = reinterpret_cast<const QuantizeBatchEntry*>(tb.dev) + tb.first_entry[cls];
+        const uint32_t* db = reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes) + tb.first_begin[cls];
+        HIP_TRY(launch_quantize_batch(s, ev, de, db, (uint32_t) tb.members[cls], tb.blocks[cls], tb.lds[cls], nbits, zt),
+                "batched quantize kernel launch failed");
+        tb.in_flight = true;
     }
     LaunchTuning autotune;
-    for (size_t i = 0; i < count; ++i)
+    for (size_t i : tb.own)
     {
         const cntkq_quantize_item& it = items[i];
-        if (it.rows == 0 || it.cols == 0 || quantize_auto_path(it.in, it.res_in, it.res_out, it.qbuf, it.rows, nbits) == kPathTile)
-            continue;
         LaunchEvents ev;
         launches_left--;
         ev.stop = launches_left == 0 ? done : nullptr;
         HIP_TRY(launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune),
                 "quantize kernel launch failed");
+        tb.in_flight = true;
     }
     h->last_quantize = done;
     h->quantize_included_fetch = false;
@@ -786,47 +848,55 @@ int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item
         return CNTKQ_OK;
     DeviceGuard guard(h->device);
     hipStream_t s = work_stream(h);
-    const size_t entries_bytes = n * sizeof(UnquantizeBatchEntry);
-    int slot = 0;
-    int rc = acquire_batch_slot(h, entries_bytes + (n + 1) * sizeof(uint32_t) + 64, &slot);
-    if (rc != CNTKQ_OK)
-        return rc;
-    char* host = h->batch_host + (size_t) slot * h->batch_slot_bytes;
-    char* dev = h->batch_dev + (size_t) slot * h->batch_slot_bytes;
-    UnquantizeBatchEntry* he = reinterpret_cast<UnquantizeBatchEntry*>(host);
-    uint32_t* hb = reinterpret_cast<uint32_t*>(host + entries_bytes);
-    LaunchTuning autotune;
-    uint64_t blocks = 0;
-    size_t e = 0;
-    for (size_t i = 0; i < count; ++i)
+    BatchTable& tb = h->unquantize_table;
+    const size_t params[3] = {count, nbits, 0};
+    const size_t items_bytes = count * sizeof(cntkq_unquantize_item);
+    if (!table_matches(tb, items, items_bytes, params))
     {
-        const cntkq_unquantize_item& it = items[i];
-        if (it.rows == 0 || it.cols == 0)
-            continue;
-        const UnquantizePlan p = plan_unquantize(it.qbuf, it.out, it.rows, it.cols, nbits, autotune);
-        if (!p.ok)
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: item %zu is too large", i);
-        he[e].q = static_cast<const char*>(it.qbuf);
-        he[e].out = it.out;
-        he[e].kind = p.kind;
-        he[e].pad = 0;
-        he[e].qw = p.qw;
-        he[e].seg = p.seg;
+        const size_t entries_bytes = n * sizeof(UnquantizeBatchEntry);
+        int rc = table_begin_rebuild(tb, entries_bytes + (n + 1) * sizeof(uint32_t) + 64);
+        if (rc != CNTKQ_OK)
+            return rc;
+        UnquantizeBatchEntry* he = reinterpret_cast<UnquantizeBatchEntry*>(tb.host);
+        uint32_t* hb = reinterpret_cast<uint32_t*>(tb.host + entries_bytes);
+        LaunchTuning autotune;
+        uint64_t blocks = 0;
+        size_t e = 0;
+        for (size_t i = 0; i < count; ++i)
+        {
+            const cntkq_unquantize_item& it = items[i];
+            if (it.rows == 0 || it.cols == 0)
+                continue;
+            const UnquantizePlan p = plan_unquantize(it.qbuf, it.out, it.rows, it.cols, nbits, autotune);
+            if (!p.ok)
+                return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: item %zu is too large", i);
+            he[e].q = static_cast<const char*>(it.qbuf);
+            he[e].out = it.out;
+            he[e].kind = p.kind;
+            he[e].pad = 0;
+            he[e].qw = p.qw;
+            he[e].seg = p.seg;
+            hb[e] = (uint32_t) blocks;
+            blocks += p.blocks;
+            if (blocks > 0x7FFFFFFFull)
+                return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: too much work in one batch");
+            e++;
+        }
         hb[e] = (uint32_t) blocks;
-        blocks += p.blocks;
-        if (blocks > 0x7FFFFFFFull)
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: too much work in one batch");
-        e++;
+        tb.members[0] = n;
+        tb.blocks[0] = (uint32_t) blocks;
+        tb.entries_bytes = entries_bytes;
+        HIP_TRY(hipMemcpyAsync(tb.dev, tb.host, entries_bytes + (n + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, s),
+                "hipMemcpyAsync of the batch table failed");
+        table_set_key(tb, items, items_bytes, params);
     }
-    hb[e] = (uint32_t) blocks;
-    HIP_TRY(hipMemcpyAsync(dev, host, entries_bytes + (n + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, s),
-            "hipMemcpyAsync of the batch table failed");
     LaunchEvents ev;
-    ev.stop = h->batch_event[slot];
-    HIP_TRY(launch_unquantize_batch(s, ev, reinterpret_cast<const UnquantizeBatchEntry*>(dev),
-                                    reinterpret_cast<const uint32_t*>(dev + entries_bytes), (uint32_t) n, (uint32_t) blocks, nbits,
-                                    add != 0),
+    ev.stop = tb.event;
+    HIP_TRY(launch_unquantize_batch(s, ev, reinterpret_cast<const UnquantizeBatchEntry*>(tb.dev),
+                                    reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes), (uint32_t) tb.members[0], tb.blocks[0],
+                                    nbits, add != 0),
             "batched unquantize kernel launch failed");
+    tb.in_flight = true;
     h->last_unquantize = ev.stop;
     return CNTKQ_OK;
 }

@@ -23,11 +23,11 @@ constexpr uint32_t kTileThreads = 256;
 constexpr uint32_t kTallThreads = 1024;
 constexpr uint32_t kMaxWorkers = 64;
 
-// floats of LDS in front of the column tile: 8 reduction slots (4 float + 4 uint),
+// floats of LDS in front of the column tile: 12 reduction slots (8 float + 4 uint: up to 4 wavefronts),
 // then (lower, upper) per tile column (at most 32 columns)
-constexpr uint32_t kTileScratchFloats = 8;
+constexpr uint32_t kTileScratchFloats = 12;
 constexpr uint32_t kTileMaxCols = 32;
-constexpr uint32_t kTilePrefixFloats = kTileScratchFloats + 2 * kTileMaxCols; // 72 floats = 288 B (16-B multiple)
+constexpr uint32_t kTilePrefixFloats = kTileScratchFloats + 2 * kTileMaxCols; // 76 floats = 304 B (16-B multiple)
 
 // A QWord is assembled from work items of at most 8 bit positions each, so that a tile with few QWords
 // still keeps every thread busy; the partial words meet in LDS (atomic OR).
@@ -93,7 +93,7 @@ __device__ __forceinline__ void tile_stats(const float* tile, float* hdr, float*
             mean = s / (float) t.rows;
         }
         float s0 = 0.0f, s1 = 0.0f;
-        uint32_t n0 = 0, n1 = 0;
+        uint32_t n0 = 0;
         if (col_ok)
         {
             for (uint32_t i = lg; i < t.rows; i += t.gs)
@@ -107,15 +107,11 @@ __device__ __forceinline__ void tile_stats(const float* tile, float* hdr, float*
                 else
                 {
                     s1 += v;
-                    n1++;
                 }
             }
         }
-        s0 = group_sum(s0, t.gs, scratch_f);
-        s1 = group_sum(s1, t.gs, scratch_f);
-        n0 = group_sum(n0, t.gs, scratch_u);
-        n1 = group_sum(n1, t.gs, scratch_u);
-        finish_stats_1bit<ZT>(mean, s0, s1, n0, n1, t.rows, lo, hi);
+        group_sum3(s0, s1, n0, t.gs, scratch_f, scratch_u);
+        finish_stats_1bit<ZT>(mean, s0, s1, n0, t.rows - n0, t.rows, lo, hi);
     }
     else
     {
@@ -248,7 +244,7 @@ __device__ __forceinline__ void quantize_tile_body(const float* __restrict__ g, 
     extern __shared__ f32x4 smem_v4[];
     float* smem = reinterpret_cast<float*>(smem_v4);
     float* scratch_f = smem;
-    uint32_t* scratch_u = reinterpret_cast<uint32_t*>(smem + 4);
+    uint32_t* scratch_u = reinterpret_cast<uint32_t*>(smem + 8);
     float* hdr = smem + kTileScratchFloats;
     uint32_t* words = reinterpret_cast<uint32_t*>(smem + kTilePrefixFloats + t.tile_floats);
 
@@ -326,18 +322,6 @@ __global__ __launch_bounds__(kTileThreads) void quantize_tile_kernel(const float
     quantize_tile_body<NBITS, ZT>(g, r_in, r_out, q, t, blockIdx.x);
 }
 
-// Many matrices in one launch: the tiles of all matrices form one grid; `begins` (count + 1 entries, ascending)
-// gives the first tile of every matrix. Removes the per-launch floor (several microseconds) that dominates
-// gradient sets made of many small matrices.
-struct QuantizeBatchEntry
-{
-    const float* g;
-    const float* r_in;
-    float* r_out;
-    char* q;
-    TileGeom t;
-};
-
 // largest e with begins[e] <= b; b and everything derived from it is uniform over the workgroup
 __device__ __forceinline__ uint32_t batch_find(const uint32_t* __restrict__ begins, uint32_t count, uint32_t b)
 {
@@ -351,15 +335,6 @@ __device__ __forceinline__ uint32_t batch_find(const uint32_t* __restrict__ begi
             hi = mid;
     }
     return lo;
-}
-
-template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kTileThreads) void quantize_tile_batch_kernel(const QuantizeBatchEntry* __restrict__ entries,
-                                                                           const uint32_t* __restrict__ begins, uint32_t count)
-{
-    const uint32_t e = batch_find(begins, count, blockIdx.x);
-    const QuantizeBatchEntry en = entries[e];
-    quantize_tile_body<NBITS, ZT>(en.g, en.r_in, en.r_out, en.q, en.t, blockIdx.x - begins[e]);
 }
 
 // ---- stripe reduction: K packed stripes -> fp32 sum -> requantize with the stripe residual ----------
@@ -387,7 +362,7 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
     extern __shared__ f32x4 smem_v4[];
     float* smem = reinterpret_cast<float*>(smem_v4);
     float* scratch_f = smem;
-    uint32_t* scratch_u = reinterpret_cast<uint32_t*>(smem + 4);
+    uint32_t* scratch_u = reinterpret_cast<uint32_t*>(smem + 8);
     float* hdr = smem + kTileScratchFloats;
     uint32_t* words = reinterpret_cast<uint32_t*>(smem + kTilePrefixFloats + t.tile_floats);
     float* dec = smem + kTilePrefixFloats + t.tile_floats + t.words_floats;
@@ -737,6 +712,350 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSo
         csum = col_thread_sum<PER>(v);
     }
     col_stats_pack<ZT, PER>(l, csum, stripe_res + base, q_out + rec);
+}
+
+// ---- the same decomposition for any bit width and any column height that is a multiple of 4 ----------------
+//
+// One workgroup of 256 threads per column, the column in LDS. The running statistic (sum for 1 bit, sum of squares
+// otherwise) is taken piece by piece while loading, in the order col_thread_sum defines, so for 1 bit and 1024 * PER
+// rows these kernels give the very bytes of the unrolled ones above.
+
+struct ColGeom
+{
+    uint32_t rows;   // multiple of 4
+    uint32_t nq;
+    uint32_t pieces; // rows / 4
+    uint64_t qcol;
+};
+
+// LDS in floats: [column | partial QWords (nq when a QWord has several work items) | 12 reduction slots | decode constants]
+template <int NBITS>
+__host__ __device__ inline size_t colg_lds_bytes(const ColGeom& c, uint32_t workers)
+{
+    return ((size_t) c.rows + (PackShape<NBITS>::CHUNKS > 1 ? c.nq : 0) + 12 + (size_t) 2 * workers) * sizeof(float);
+}
+
+template <int NBITS>
+__device__ __forceinline__ float colg_add_piece(float s, const f32x4& v)
+{
+    if constexpr (NBITS == 1)
+    {
+        s += v.x;
+        s += v.y;
+        s += v.z;
+        s += v.w;
+    }
+    else
+    {
+        s += v.x * v.x;
+        s += v.y * v.y;
+        s += v.z * v.z;
+        s += v.w * v.w;
+    }
+    return s;
+}
+
+// stat: this thread's running statistic over its pieces (unused for 1 bit with ZT). tile = the column, words = zeroed
+// partial QWords, red = 12 reduction slots. No barrier is needed between writing the column and calling this.
+template <int NBITS, bool ZT>
+__device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, float* red, const ColGeom& c, float stat,
+                                                float* res_col, char* qc)
+{
+    using PS = PackShape<NBITS>;
+    constexpr uint32_t T = kColThreads, NW = T / 64;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 8);
+    constexpr bool need_stat = (NBITS != 1) || !ZT;
+    float total = 0.0f;
+    if constexpr (need_stat)
+    {
+        const float s = wave_sum(stat);
+        if (lane == 0)
+            red[wave] = s;
+    }
+    __syncthreads(); // the column and the wave sums are visible
+    if constexpr (need_stat)
+    {
+        total = red[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+            total += red[x];
+    }
+    float lo, hi;
+    if constexpr (NBITS == 1)
+    {
+        const float mean = ZT ? 0.0f : total / (float) c.rows;
+        float s0 = 0.0f, s1 = 0.0f;
+        uint32_t n0 = 0;
+        for (uint32_t i = tid; i < c.rows; i += T)
+        {
+            const float x = tile[i];
+            const bool below = x < mean;
+            s0 += below ? x : 0.0f;
+            s1 += below ? 0.0f : x;
+            n0 += below ? 1u : 0u;
+        }
+        s0 = wave_sum(s0);
+        s1 = wave_sum(s1);
+        n0 = wave_sum(n0);
+        __syncthreads(); // everyone has read the wave sums of the mean
+        if (lane == 0)
+        {
+            red[wave] = s0;
+            red[4 + wave] = s1;
+            red_u[wave] = n0;
+        }
+        __syncthreads();
+        float S0 = red[0], S1 = red[4];
+        uint32_t N0 = red_u[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+        {
+            S0 += red[x];
+            S1 += red[4 + x];
+            N0 += red_u[x];
+        }
+        finish_stats_1bit<ZT>(mean, S0, S1, N0, c.rows - N0, c.rows, lo, hi);
+    }
+    else
+    {
+        finish_stats_multibit(total, c.rows, lo, hi);
+    }
+    if (tid == 0)
+    {
+        // a record is only 4-byte aligned when the column has an odd number of QWords
+        float* gh = reinterpret_cast<float*>(qc);
+        gh[0] = lo;
+        gh[1] = hi;
+    }
+    const ValueQ vq = make_vq<NBITS>(lo, hi);
+    const float val0 = unquantize_value<NBITS>(vq, 0u);
+    const float val1 = unquantize_value<NBITS>(vq, 1u);
+    uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
+    const uint32_t items = c.nq * PS::CHUNKS;
+    for (uint32_t it = tid; it < items; it += T)
+    {
+        // chunk-major: consecutive threads take consecutive QWords, hence consecutive rows
+        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / c.nq;
+        const uint32_t w = it - chunk * c.nq;
+        uint32_t word = 0;
+#pragma unroll
+        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+        {
+            const uint32_t k = chunk * PS::SLOTS + kk;
+            const uint32_t i = w + k * c.nq;
+            if (i < c.rows)
+            {
+                const float v = tile[i];
+                const uint32_t code = quantize_value<NBITS, ZT>(vq, v);
+                float back;
+                if constexpr (NBITS == 1)
+                    back = code ? val1 : val0;
+                else
+                    back = unquantize_value<NBITS>(vq, code);
+                __builtin_nontemporal_store(v - back, res_col + i);
+                word |= code << (k * PS::SHIFT);
+            }
+        }
+        if constexpr (PS::CHUNKS == 1)
+            bits[w] = word;
+        else
+            atomicOr(&words[w], word);
+    }
+    if constexpr (PS::CHUNKS > 1)
+    {
+        __syncthreads();
+        for (uint32_t w = tid; w < c.nq; w += T)
+            bits[w] = words[w];
+    }
+}
+
+template <int NBITS, bool ZT>
+__device__ __forceinline__ void quantize_colg_body(const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q,
+                                                   const ColGeom& c, uint32_t column, f32x4* smem)
+{
+    using PS = PackShape<NBITS>;
+    constexpr uint32_t T = kColThreads;
+    float* tile = reinterpret_cast<float*>(smem);
+    uint32_t* words = reinterpret_cast<uint32_t*>(tile + c.rows);
+    float* red = tile + c.rows + (PS::CHUNKS > 1 ? c.nq : 0);
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) column * c.rows;
+    if constexpr (PS::CHUNKS > 1)
+        for (uint32_t x = tid; x < c.nq; x += T)
+            words[x] = 0u;
+    const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base);
+    const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base);
+    f32x4* t4 = reinterpret_cast<f32x4*>(tile);
+    float stat = 0.0f;
+    for (uint32_t p0 = tid; p0 < c.pieces; p0 += 4 * T)
+    {
+        f32x4 a[4], b[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+        {
+            const uint32_t p = p0 + u * T;
+            if (p < c.pieces)
+            {
+                a[u] = __builtin_nontemporal_load(g4 + p);
+                b[u] = __builtin_nontemporal_load(r4 + p);
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+        {
+            const uint32_t p = p0 + u * T;
+            if (p < c.pieces)
+            {
+                const f32x4 v = a[u] + b[u];
+                t4[p] = v;
+                stat = colg_add_piece<NBITS>(stat, v);
+            }
+        }
+    }
+    // the whole column has been read before the first barrier of colg_stats_pack, so r_out may be r_in
+    colg_stats_pack<NBITS, ZT>(tile, words, red, c, stat, r_out + base, q + (size_t) column * c.qcol);
+}
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kColThreads) void quantize_colg_kernel(const float* __restrict__ g, const float* r_in, float* r_out,
+                                                                    char* __restrict__ q, ColGeom c)
+{
+    extern __shared__ f32x4 smem_v4[];
+    quantize_colg_body<NBITS, ZT>(g, r_in, r_out, q, c, blockIdx.x, smem_v4);
+}
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kColThreads) void stripe_reduce_colg_kernel(StripeSources src, float* stripe_res, char* q_out,
+                                                                         float* agg_out, ColGeom c)
+{
+    using PS = PackShape<NBITS>;
+    constexpr uint32_t T = kColThreads, BATCH = 8;
+    extern __shared__ f32x4 smem_v4[];
+    float* tile = reinterpret_cast<float*>(smem_v4);
+    uint32_t* words = reinterpret_cast<uint32_t*>(tile + c.rows);
+    float* red = tile + c.rows + (PS::CHUNKS > 1 ? c.nq : 0);
+    float* dec = red + 12; // per worker, in summation order: 1 bit -> the two levels, else (ufactor, lower)
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * c.rows;
+    const size_t rec = (size_t) blockIdx.x * c.qcol;
+    const uint32_t K = src.workers;
+    if constexpr (PS::CHUNKS > 1)
+        for (uint32_t x = tid; x < c.nq; x += T)
+            words[x] = 0u;
+    if (tid < K)
+    {
+        const float* h = reinterpret_cast<const float*>(src.q[stripe_order(tid, src.owner)] + rec);
+        const ValueQ vq = make_vq<NBITS>(h[0], h[1]);
+        if constexpr (NBITS == 1)
+        {
+            dec[2 * tid] = unquantize_value<NBITS>(vq, 0u);
+            dec[2 * tid + 1] = unquantize_value<NBITS>(vq, 1u);
+        }
+        else
+        {
+            dec[2 * tid] = vq.uf;
+            dec[2 * tid + 1] = vq.lo;
+        }
+    }
+    __syncthreads();
+
+    const float* sp = stripe_res + base;
+    const uint32_t items = c.nq * PS::CHUNKS;
+    for (uint32_t it = tid; it < items; it += T)
+    {
+        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / c.nq;
+        const uint32_t w = it - chunk * c.nq;
+        const size_t word_off = rec + 8 + (size_t) w * 4;
+        const uint32_t sh0 = chunk * PS::SLOTS * PS::SHIFT;
+        float acc[PS::SLOTS];
+        for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
+        {
+            uint32_t word[BATCH];
+#pragma unroll
+            for (uint32_t u = 0; u < BATCH; ++u)
+                if (n0 + u < K)
+                    word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + word_off);
+#pragma unroll
+            for (uint32_t u = 0; u < BATCH; ++u)
+            {
+                if (n0 + u < K)
+                {
+                    const float a = dec[2 * (n0 + u)];
+                    const float b = dec[2 * (n0 + u) + 1];
+                    const uint32_t bits = word[u] >> sh0;
+#pragma unroll
+                    for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+                    {
+                        const uint32_t code = (bits >> (kk * PS::SHIFT)) & PS::CODEMASK;
+                        float x;
+                        if constexpr (NBITS == 1)
+                            x = code ? b : a;
+                        else
+                            x = unquantize_value<NBITS>(a, b, code);
+                        // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
+                        acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+        {
+            const uint32_t i = w + (chunk * PS::SLOTS + kk) * c.nq;
+            if (i < c.rows)
+            {
+                if (agg_out != nullptr)
+                    agg_out[base + i] = acc[kk];
+                tile[i] = acc[kk] + __builtin_nontemporal_load(sp + i);
+            }
+        }
+    }
+    float stat = 0.0f;
+    if constexpr ((NBITS != 1) || !ZT)
+    {
+        __syncthreads();
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
+        for (uint32_t p = tid; p < c.pieces; p += T)
+            stat = colg_add_piece<NBITS>(stat, t4[p]);
+    }
+    colg_stats_pack<NBITS, ZT>(tile, words, red, c, stat, stripe_res + base, q_out + rec);
+}
+
+// Many matrices in one launch: the workgroups of all matrices form one grid; `begins` (count + 1 entries, ascending)
+// gives the first workgroup of every matrix. A matrix is a run of column tiles (quantize_tile_body) or of single columns
+// (quantize_colg_body). Removes the per-launch floor (several microseconds) that dominates gradient sets made of many
+// small matrices.
+struct QuantizeBatchEntry
+{
+    const float* g;
+    const float* r_in;
+    float* r_out;
+    char* q;
+    uint32_t kind; // 0: tiles (t), 1: columns (c)
+    uint32_t pad;
+    TileGeom t;
+    ColGeom c;
+};
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTileThreads) void quantize_batch_kernel(const QuantizeBatchEntry* __restrict__ entries,
+                                                                      const uint32_t* __restrict__ begins, uint32_t count)
+{
+    extern __shared__ f32x4 smem_v4[];
+    const uint32_t e = batch_find(begins, count, blockIdx.x);
+    const uint32_t index = blockIdx.x - begins[e];
+    // geometry by value: read once, then held in registers whatever the kernel stores
+    if (entries[e].kind == 0)
+    {
+        const TileGeom t = entries[e].t;
+        quantize_tile_body<NBITS, ZT>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, t, index);
+    }
+    else
+    {
+        const ColGeom c = entries[e].c;
+        quantize_colg_body<NBITS, ZT>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, c, index, smem_v4);
+    }
 }
 
 // ---- quantize, columns too tall for LDS: one workgroup per column, global memory re-read -------------

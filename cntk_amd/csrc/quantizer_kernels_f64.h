@@ -21,8 +21,8 @@ typedef double f64x2 __attribute__((ext_vector_type(2)));
 
 constexpr uint32_t kThreads = 256;
 constexpr uint32_t kMaxTileCols = 32;
-// LDS prefix in 8-byte units: 4 double + 4 slots holding one uint32 each for the reductions, then (lower, upper) per column
-constexpr uint32_t kPrefixWords = 8 + 2 * kMaxTileCols;
+// LDS prefix in 8-byte units: 8 double + 2 (four uint32) for the reductions of up to 4 wavefronts, then (lower, upper) per column
+constexpr uint32_t kPrefixWords = 10 + 2 * kMaxTileCols;
 
 // ---- per-value quantizer (Source/Math/ValueQuantizer.h:68-156 with ElemType = double) ----------------
 
@@ -190,7 +190,7 @@ __device__ __forceinline__ void tile_stats(const double* tile, double* hdr, doub
             mean = s / (double) t.rows;
         }
         double s0 = 0.0, s1 = 0.0;
-        uint32_t n0 = 0, n1 = 0;
+        uint32_t n0 = 0;
         if (col_ok)
         {
             for (uint32_t i = lg; i < t.rows; i += t.gs)
@@ -204,15 +204,11 @@ __device__ __forceinline__ void tile_stats(const double* tile, double* hdr, doub
                 else
                 {
                     s1 += v;
-                    n1++;
                 }
             }
         }
-        s0 = group_sum(s0, t.gs, scratch_f);
-        s1 = group_sum(s1, t.gs, scratch_f);
-        n0 = group_sum(n0, t.gs, scratch_u);
-        n1 = group_sum(n1, t.gs, scratch_u);
-        finish_stats_1bit<ZT>(mean, s0, s1, n0, n1, t.rows, lo, hi);
+        group_sum3(s0, s1, n0, t.gs, scratch_f, scratch_u);
+        finish_stats_1bit<ZT>(mean, s0, s1, n0, t.rows - n0, t.rows, lo, hi);
     }
     else
     {
@@ -310,8 +306,8 @@ __device__ __forceinline__ TileLds tile_lds(double* smem, const TileGeom& t)
 {
     TileLds l;
     l.scratch_f = smem;
-    l.scratch_u = reinterpret_cast<uint32_t*>(smem + 4);
-    l.hdr = smem + 8;
+    l.scratch_u = reinterpret_cast<uint32_t*>(smem + 8);
+    l.hdr = smem + 10;
     l.tile = smem + kPrefixWords;
     l.words = reinterpret_cast<unsigned long long*>(smem + kPrefixWords + t.tile_words);
     l.dec = smem + kPrefixWords + t.tile_words + t.words_words;

@@ -19,10 +19,11 @@ enum QuantizePath
     kPathAuto = 0,
     kPathTile = 1,    // LDS-staged column tile (rows <= kTileMaxRows)
     kPathTall = 2,    // one workgroup per column, global re-read (any rows)
-    kPathCol = 3      // 1 bit, rows in {1024, 2048, 4096}, one workgroup per column, column in LDS
+    kPathCol = 3      // one workgroup per column, column in LDS: rows a multiple of 4, matrices 16-byte aligned
 };
 
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
+constexpr uint32_t kColMinRows = 1024;   // shorter columns are better served several to a workgroup (tile kernels)
 
 struct LaunchTuning
 {
@@ -144,12 +145,54 @@ struct StripeLauncher
     }
 };
 
-inline bool col_applicable(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
+// forced = the caller insists on the column kernels: any height they can handle; otherwise only where they pay
+inline bool col_applicable(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits,
+                           bool forced = false)
 {
+    (void) nbits;
     const uintptr_t m = reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(r_in) | reinterpret_cast<uintptr_t>(r_out);
-    return nbits == 1 && (rows == 1024 || rows == 2048 || rows == 4096) && (m & 15u) == 0 &&
-           (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
+    return rows % 4 == 0 && rows <= kTileMaxRows && (forced ? rows >= 4 : rows >= kColMinRows) && (m & 15u) == 0 &&
+           (reinterpret_cast<uintptr_t>(q) & 3u) == 0;
 }
+
+// the unrolled 1-bit kernels: 1024, 2048 or 4096 rows and 8-byte aligned packed buffers
+inline bool col_unrolled(const void* q, size_t rows, size_t nbits)
+{
+    return nbits == 1 && (rows == 1024 || rows == 2048 || rows == 4096) && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
+}
+
+inline ColGeom make_col_geom(size_t rows, size_t nbits)
+{
+    ColGeom c;
+    c.rows = (uint32_t) rows;
+    c.nq = (uint32_t) qwords_per_col(rows, nbits);
+    c.pieces = (uint32_t) (rows / 4);
+    c.qcol = qcol_bytes(nbits, rows);
+    return c;
+}
+
+template <int NBITS, bool ZT>
+struct ColLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, ColGeom c)
+    {
+        hipExtLaunchKernelGGL((quantize_colg_kernel<NBITS, ZT>), dim3(cols), dim3(kColThreads), colg_lds_bytes<NBITS>(c, 0), s, ev.start,
+                              ev.stop, 0, g, r_in, r_out, q, c);
+        return hipGetLastError();
+    }
+};
+
+template <int NBITS, bool ZT>
+struct StripeColLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
+                          uint32_t cols, ColGeom c)
+    {
+        hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT>), dim3(cols), dim3(kColThreads), colg_lds_bytes<NBITS>(c, src.workers),
+                              s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
+        return hipGetLastError();
+    }
+};
 
 template <bool ZT, int PER>
 inline void launch_quantize_col(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
@@ -185,8 +228,10 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     }
     if (path == kPathCol)
     {
-        if (!col_applicable(g, r_in, r_out, q, rows, nbits))
+        if (!col_applicable(g, r_in, r_out, q, rows, nbits, true))
             return hipErrorInvalidValue;
+        if (!col_unrolled(q, rows, nbits))
+            return dispatch_nbits<ColLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, make_col_geom(rows, nbits));
         const uint64_t qcol = qcol_bytes(nbits, rows);
         const uint32_t c = (uint32_t) cols;
         if (rows == 1024)
@@ -218,8 +263,12 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
     bool aligned8 = (reinterpret_cast<uintptr_t>(q_out) & 7u) == 0;
     for (uint32_t w = 0; w < src.workers; ++w)
         aligned8 = aligned8 && (reinterpret_cast<uintptr_t>(src.q[w]) & 7u) == 0;
-    if ((tune.quantize_path == kPathAuto || tune.quantize_path == kPathCol) && nbits == 1 &&
-        (rows == 1024 || rows == 2048 || rows == 4096) && aligned8)
+    const bool col_forced = tune.quantize_path == kPathCol;
+    const bool col = (tune.quantize_path == kPathAuto || col_forced) && rows % 4 == 0 && (col_forced || rows >= kColMinRows);
+    if (col && !(aligned8 && col_unrolled(q_out, rows, nbits)))
+        return dispatch_nbits<StripeColLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols,
+                                                 make_col_geom(rows, nbits));
+    if (col)
     {
         // same column statistics, in the same order, as quantize_col_kernel
         const uint64_t qcol = qcol_bytes(nbits, rows);
@@ -346,22 +395,29 @@ inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* 
 // kernel has finished.
 
 template <int NBITS, bool ZT>
-struct TileBatchLauncher
+struct BatchLauncher
 {
     static hipError_t run(hipStream_t s, LaunchEvents ev, const QuantizeBatchEntry* entries, const uint32_t* begins, uint32_t count,
-                          uint32_t total_tiles, size_t lds)
+                          uint32_t total_blocks, size_t lds)
     {
-        hipExtLaunchKernelGGL((quantize_tile_batch_kernel<NBITS, ZT>), dim3(total_tiles), dim3(kTileThreads), lds, s, ev.start, ev.stop,
-                              0, entries, begins, count);
+        static_assert(kTileThreads == kColThreads, "tiles and columns share one workgroup size in a batch");
+        hipExtLaunchKernelGGL((quantize_batch_kernel<NBITS, ZT>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start, ev.stop, 0,
+                              entries, begins, count);
         return hipGetLastError();
     }
 };
 
-inline hipError_t launch_quantize_tile_batch(hipStream_t s, LaunchEvents ev, const QuantizeBatchEntry* entries, const uint32_t* begins,
-                                             uint32_t count, uint32_t total_tiles, size_t lds, size_t nbits, bool zt)
+inline hipError_t launch_quantize_batch(hipStream_t s, LaunchEvents ev, const QuantizeBatchEntry* entries, const uint32_t* begins,
+                                        uint32_t count, uint32_t total_blocks, size_t lds, size_t nbits, bool zt)
 {
     zt = zt && (nbits == 1);
-    return dispatch_nbits<TileBatchLauncher>(nbits, zt, s, ev, entries, begins, count, total_tiles, lds);
+    return dispatch_nbits<BatchLauncher>(nbits, zt, s, ev, entries, begins, count, total_blocks, lds);
+}
+
+// colg_lds_bytes for a bit width known only at run time
+inline size_t colg_lds_bytes_rt(const ColGeom& c, size_t nbits)
+{
+    return ((size_t) c.rows + (nbits <= 2 ? c.nq : 0) + 12) * sizeof(float);
 }
 
 inline hipError_t launch_unquantize_batch(hipStream_t s, LaunchEvents ev, const UnquantizeBatchEntry* entries, const uint32_t* begins,

@@ -214,4 +214,42 @@ __device__ __forceinline__ T group_sum(T v, uint32_t gs, T* scratch)
     return v;
 }
 
+// The three sums of the 1-bit split (sum below, sum not below, count below) over aligned groups of `gs` threads in
+// one exchange: same order of additions as three group_sum calls, one pair of barriers instead of three.
+// scratch_f holds two T per wave (a of every wave, then b of every wave), scratch_u one uint32 per wave.
+template <typename T>
+__device__ __forceinline__ void group_sum3(T& a, T& b, uint32_t& c, uint32_t gs, T* scratch_f, uint32_t* scratch_u)
+{
+    const uint32_t width = gs < (uint32_t) kWave ? gs : (uint32_t) kWave;
+    a = lanes_sum(a, width);
+    b = lanes_sum(b, width);
+    c = lanes_sum(c, width);
+    if (gs > (uint32_t) kWave)
+    {
+        const uint32_t wave = threadIdx.x >> 6;
+        const uint32_t waves = blockDim.x >> 6;
+        if ((threadIdx.x & 63u) == 0)
+        {
+            scratch_f[wave] = a;
+            scratch_f[waves + wave] = b;
+            scratch_u[wave] = c;
+        }
+        __syncthreads();
+        const uint32_t per = gs >> 6;
+        const uint32_t first = (threadIdx.x / gs) * per;
+        T ta = scratch_f[first], tb = scratch_f[waves + first];
+        uint32_t tc = scratch_u[first];
+        for (uint32_t x = 1; x < per; ++x)
+        {
+            ta += scratch_f[first + x];
+            tb += scratch_f[waves + first + x];
+            tc += scratch_u[first + x];
+        }
+        __syncthreads();
+        a = ta;
+        b = tb;
+        c = tc;
+    }
+}
+
 } // namespace cntkq

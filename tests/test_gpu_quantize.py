@@ -120,6 +120,10 @@ PATH_CASES = [
     (2304, 5, PATH_TILE, 0), (4608, 3, PATH_TILE, 0), (9304, 2, PATH_TILE, 0), (14336, 1, PATH_TILE, 0),
     (1, 5, PATH_TALL, 0), (70, 3, PATH_TALL, 0), (1025, 3, PATH_TALL, 0), (20001, 2, PATH_TALL, 0),
     (33000, 2, PATH_AUTO, 0),
+    # one workgroup per column: any height that is a multiple of 4
+    (4, 3, PATH_COL, 0), (36, 70, PATH_COL, 0), (128, 9, PATH_COL, 0), (1000, 5, PATH_COL, 0), (1028, 7, PATH_COL, 0),
+    (2048, 19, PATH_COL, 0), (2304, 5, PATH_COL, 0), (4100, 3, PATH_COL, 0), (9304, 2, PATH_COL, 0), (14336, 2, PATH_COL, 0),
+    (9304, 3, PATH_AUTO, 0), (1152, 40, PATH_AUTO, 0),
 ]
 
 
@@ -165,9 +169,19 @@ def test_workgroup_per_column_path(rows):
     qz._set_tuning(quantize_path=PATH_COL)
     # shapes and alignments the path does not cover are refused when forced, not mis-computed
     with pytest.raises(cntk_amd.QuantizerLogicError):
-        gpu_quantize(qz, datagen.normal(1, 512, 4), np.zeros((512, 4), np.float32, order="F"), 1, False)
-    with pytest.raises(cntk_amd.QuantizerLogicError):
-        gpu_quantize(qz, datagen.normal(1, rows, 4), np.zeros((rows, 4), np.float32, order="F"), 2, False)
+        gpu_quantize(qz, datagen.normal(1, 513, 4), np.zeros((513, 4), np.float32, order="F"), 1, False)
+    # a packed buffer that is only 4-byte aligned takes the general (not unrolled) column kernel: same bytes
+    cols = 6
+    g, r = datagen.normal(8, rows, cols), datagen.normal(9, rows, cols, 0.002)
+    for zt in (False, True):
+        Qa, ra = gpu_quantize(qz, g, r, 1, zt)
+        raw = torch.zeros(Qa.GetSize() + 4, dtype=torch.uint8, device="cuda:0")
+        Qb = QuantizedMatrix(rows, cols, 1, 0, raw[4:])
+        assert Qb.Buffer() % 8 == 4
+        G, R = Matrix.from_numpy(g), Matrix.from_numpy(r)
+        qz.QuantizeAsync(G, R, Qb, R, zt)
+        qz.WaitQuantizeAsyncDone()
+        assert np.array_equal(Qa.to_numpy(), Qb.to_numpy()) and parity.bits_equal(ra, R.to_numpy())
     # a gradient that starts 4 bytes off a 16-byte boundary: refused when forced, served by the tile kernel otherwise
     cols = 5
     g = datagen.normal(5, rows, cols)

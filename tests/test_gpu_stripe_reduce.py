@@ -68,9 +68,9 @@ def test_stripe_reduce(case):
             continue
         say("stripe reduce", case, "owner", owner, "cols", start, n)
         sres = datagen.normal(900 + owner, rows, n, 0.003)
-        # 1-bit stripes of 1024, 2048 or 4096 rows have a kernel of their own (one workgroup per column); run the
-        # general tile kernel (path 1) on them too
-        variants = [(True, 0), (False, 0)] + ([(True, 1)] if (nbits == 1 and rows in (1024, 2048, 4096)) else [])
+        # heights that are a multiple of 4 can take the kernels with one workgroup per column (path 3; the automatic
+        # choice from 1024 rows on) as well as the tile kernels (path 1)
+        variants = [(True, 0), (False, 0)] + ([(True, 1), (True, 3)] if rows % 4 == 0 else [])
         for alias, path in variants:
             qz._set_tuning(quantize_path=path)
             q_new, s_new, agg = gpu_stripe_reduce(qz, qs, owner, rows, cols, nbits, sres, zt, alias_out=alias)
@@ -81,6 +81,23 @@ def test_stripe_reduce(case):
             assert parity.bits_equal(agg, agg_o), "fp32 aggregate differs from the oracle (order: owner, then ascending)"
             # the requantization sees (aggregate, stripe residual) as (gradient, residual)
             parity.check_quantize(agg_o, sres, q_new, s_new, nbits, zt, report=rep)
+            # and the fused call gives the very bytes of the reference's call sequence on the same handle:
+            # unquantize own stripe, add the others in ascending order, quantize the aggregate
+            if alias:
+                Agg = Matrix(rows, n)
+                order = [owner] + [w for w in range(k) if w != owner]
+                qcol = oracle.qcol_bytes(nbits, rows)
+                for pos, w in enumerate(order):
+                    Qw = QuantizedMatrix(rows, n, nbits, 0)
+                    Qw.from_numpy(qs[w][start * qcol:(start + n) * qcol])
+                    qz.UnquantizeAsync(Qw, Agg, add=(pos > 0))
+                S = Matrix.from_numpy(sres)
+                Qo = QuantizedMatrix(rows, n, nbits, 0)
+                qz.QuantizeAsync(Agg, S, Qo, S, zt)
+                qz.WaitQuantizeAsyncDone()
+                assert parity.bits_equal(Agg.to_numpy(), agg)
+                assert np.array_equal(Qo.to_numpy(), q_new), "fused != call sequence (codes)"
+                assert parity.bits_equal(S.to_numpy(), s_new), "fused != call sequence (residual)"
     say("  ", rep)
 
 
