@@ -859,6 +859,7 @@ int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item
             return rc;
         UnquantizeBatchEntry* he = reinterpret_cast<UnquantizeBatchEntry*>(tb.host);
         uint32_t* hb = reinterpret_cast<uint32_t*>(tb.host + entries_bytes);
+        tb.lds[0] = 0;
         LaunchTuning autotune;
         uint64_t blocks = 0;
         size_t e = 0;
@@ -876,6 +877,9 @@ int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item
             he[e].pad = 0;
             he[e].qw = p.qw;
             he[e].seg = p.seg;
+            he[e].rowg = p.rowg;
+            if (p.lds > tb.lds[0])
+                tb.lds[0] = p.lds;
             hb[e] = (uint32_t) blocks;
             blocks += p.blocks;
             if (blocks > 0x7FFFFFFFull)
@@ -894,7 +898,7 @@ int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item
     ev.stop = tb.event;
     HIP_TRY(launch_unquantize_batch(s, ev, reinterpret_cast<const UnquantizeBatchEntry*>(tb.dev),
                                     reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes), (uint32_t) tb.members[0], tb.blocks[0],
-                                    nbits, add != 0),
+                                    nbits, add != 0, tb.lds[0]),
             "batched unquantize kernel launch failed");
     tb.in_flight = true;
     h->last_unquantize = ev.stop;

@@ -1159,14 +1159,15 @@ __global__ __launch_bounds__(kTallThreads) void quantize_tall_kernel(const float
             const uint32_t i = w + k * nq;
             if (i < rows)
             {
-                const float v = gp[i] + rp[i];
+                // last use of these values: streaming loads and stores
+                const float v = __builtin_nontemporal_load(gp + i) + __builtin_nontemporal_load(rp + i);
                 const uint32_t code = quantize_value<NBITS, ZT>(vq, v);
                 float back;
                 if constexpr (NBITS == 1)
                     back = code ? val1 : val0;
                 else
                     back = unquantize_value<NBITS>(vq, code);
-                op[i] = v - back;
+                __builtin_nontemporal_store(v - back, op + i);
                 word |= code << (k * MASKBITS);
             }
         }
@@ -1362,12 +1363,77 @@ __global__ __launch_bounds__(256) void unquantize_segment_kernel(const char* __r
     unquantize_segment_body<NBITS>(q, out, t, add, blockIdx.x);
 }
 
-// Many matrices in one launch (see quantize_tile_batch_kernel): the 256-thread blocks of all matrices form one grid.
+// Row-major decoder for columns whose height is a multiple of 4 but whose QWord count is not (9304 rows -> 291 QWords,
+// 100000 -> 3125): a workgroup copies the packed column into LDS once (every QWord is used by up to 32 rows) and then
+// walks a chunk of consecutive rows, four per thread and store, so that all stores are aligned 16-byte stores whatever
+// the QWord count.
+struct UnqRowGeom
+{
+    uint32_t rows;
+    uint32_t nq;
+    uint32_t chunk;  // rows per workgroup, multiple of 4
+    uint32_t chunks; // workgroups per column
+    uint32_t blocks; // cols * chunks
+    uint32_t pad;
+    uint64_t qcol;
+};
+
+template <int NBITS>
+__device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q, float* out, const UnqRowGeom& t, int add, uint32_t block,
+                                                     uint32_t* words)
+{
+    constexpr uint32_t SHIFT = NBITS & 31;
+    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t c = block / t.chunks;
+    const uint32_t ch = block - c * t.chunks;
+    const char* qc = q + (size_t) c * t.qcol;
+    const float* gh = reinterpret_cast<const float*>(qc);
+    const float lo = gh[0];
+    const float uf = make_ufactor<NBITS>(lo, gh[1]);
+    const uint32_t* bits = reinterpret_cast<const uint32_t*>(qc + 8);
+    for (uint32_t w = tid; w < t.nq; w += 256)
+        words[w] = bits[w];
+    __syncthreads();
+    const uint32_t r0 = ch * t.chunk;
+    const uint32_t pieces = (min(t.rows, r0 + t.chunk) - r0) >> 2;
+    f32x4* o4 = reinterpret_cast<f32x4*>(out + (size_t) c * t.rows + r0);
+    for (uint32_t p = tid; p < pieces; p += 256)
+    {
+        const uint32_t i = r0 + 4 * p;
+        uint32_t k = i / t.nq;
+        uint32_t w = i - k * t.nq;
+        f32x4 x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            x[e] = unquantize_value<NBITS>(uf, lo, (words[w] >> (k * SHIFT)) & CODEMASK);
+            if (++w == t.nq)
+            {
+                w = 0;
+                ++k;
+            }
+        }
+        if (add)
+            x = x + o4[p]; // unquantized value + previous content
+        __builtin_nontemporal_store(x, o4 + p);
+    }
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __restrict__ q, float* out, UnqRowGeom t, int add)
+{
+    extern __shared__ f32x4 smem_v4[];
+    unquantize_rows_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint32_t*>(smem_v4));
+}
+
+// Many matrices in one launch (see quantize_batch_kernel): the 256-thread blocks of all matrices form one grid.
 enum UnqKind : uint32_t
 {
-    kUnqVec4 = 0,   // QWord-major, 16-byte stores
-    kUnqScalar = 1, // QWord-major, 4-byte stores
-    kUnqSegment = 2 // segment decoder
+    kUnqVec4 = 0,    // QWord-major, 16-byte stores
+    kUnqScalar = 1,  // QWord-major, 4-byte stores
+    kUnqSegment = 2, // segment decoder
+    kUnqRows = 3     // row-major decoder, packed column in LDS
 };
 
 struct UnquantizeBatchEntry
@@ -1376,14 +1442,16 @@ struct UnquantizeBatchEntry
     float* out;
     uint32_t kind;
     uint32_t pad;
-    UnqGeom qw;     // valid for kUnqVec4 / kUnqScalar
-    UnqSegGeom seg; // valid for kUnqSegment
+    UnqGeom qw;      // valid for kUnqVec4 / kUnqScalar
+    UnqSegGeom seg;  // valid for kUnqSegment
+    UnqRowGeom rowg; // valid for kUnqRows
 };
 
 template <int NBITS>
 __global__ __launch_bounds__(256) void unquantize_batch_kernel(const UnquantizeBatchEntry* __restrict__ entries,
                                                                const uint32_t* __restrict__ begins, uint32_t count, int add)
 {
+    extern __shared__ f32x4 smem_v4[];
     const uint32_t e = batch_find(begins, count, blockIdx.x);
     const UnquantizeBatchEntry& en = entries[e];
     const uint32_t block = blockIdx.x - begins[e];
@@ -1391,8 +1459,13 @@ __global__ __launch_bounds__(256) void unquantize_batch_kernel(const UnquantizeB
         unquantize_body<NBITS, 4>(en.q, en.out, en.qw, add, block);
     else if (en.kind == kUnqScalar)
         unquantize_body<NBITS, 1>(en.q, en.out, en.qw, add, block);
-    else
+    else if (en.kind == kUnqSegment)
         unquantize_segment_body<NBITS>(en.q, en.out, en.seg, add, block);
+    else
+    {
+        const UnqRowGeom t = en.rowg; // by value: the loop below stores between its uses
+        unquantize_rows_body<NBITS>(en.q, en.out, t, add, block, reinterpret_cast<uint32_t*>(smem_v4));
+    }
 }
 
 } // namespace cntkq

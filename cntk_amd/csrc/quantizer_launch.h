@@ -295,9 +295,14 @@ struct UnquantizePlan
     uint32_t kind = kUnqScalar;
     UnqGeom qw;
     UnqSegGeom seg;
+    UnqRowGeom rowg;
     uint32_t blocks = 0; // 256-thread blocks
+    size_t lds = 0;      // dynamic LDS (kUnqRows only)
     bool ok = false;
 };
+
+constexpr size_t kUnqRowsMaxLds = 48 * 1024;
+constexpr uint32_t kUnqRowsChunk = 8192;
 
 inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t rows, size_t cols, size_t nbits,
                                       const LaunchTuning& tune)
@@ -305,12 +310,35 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
     UnquantizePlan p;
     std::memset(&p.qw, 0, sizeof p.qw);
     std::memset(&p.seg, 0, sizeof p.seg);
+    std::memset(&p.rowg, 0, sizeof p.rowg);
     const size_t vpw = 32 / nbits;
     const size_t nq = qwords_per_col(rows, nbits);
     const bool out16 = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
     const bool vec = !tune.unq_force_scalar && (nq % 4 == 0) && (rows % 4 == 0) && out16 &&
                      (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
-    // long columns that the QWord-major decoder could only serve with 4-byte stores go to the segment decoder
+    // columns of aligned height that the QWord-major decoder could only serve with 4-byte stores: row-major decoder
+    const bool rowmajor = !vec && !tune.unq_force_scalar && tune.unq_slots == 0 && out16 && rows % 4 == 0 && nq >= 32 &&
+                          nq * 4 <= kUnqRowsMaxLds;
+    if (rowmajor)
+    {
+        UnqRowGeom& t = p.rowg;
+        t.rows = (uint32_t) rows;
+        t.nq = (uint32_t) nq;
+        t.chunk = rows <= 2 * kUnqRowsChunk ? (uint32_t) rows : kUnqRowsChunk;
+        t.chunks = (uint32_t) ((rows + t.chunk - 1) / t.chunk);
+        const uint64_t blocks = (uint64_t) cols * t.chunks;
+        if (blocks <= 0x7FFFFFFFull)
+        {
+            t.blocks = (uint32_t) blocks;
+            t.qcol = qcol_bytes(nbits, rows);
+            p.kind = kUnqRows;
+            p.blocks = t.blocks;
+            p.lds = nq * 4;
+            p.ok = true;
+            return p;
+        }
+    }
+    // other long columns that the QWord-major decoder could only serve with 4-byte stores go to the segment decoder
     const bool seg = !vec && !tune.unq_force_scalar && out16 && nq >= 32;
     if (seg)
     {
@@ -361,7 +389,9 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
 template <int NBITS>
 inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const char* q, float* out, const UnquantizePlan& p, int add)
 {
-    if (p.kind == kUnqSegment)
+    if (p.kind == kUnqRows)
+        hipExtLaunchKernelGGL((unquantize_rows_kernel<NBITS>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.rowg, add);
+    else if (p.kind == kUnqSegment)
         hipExtLaunchKernelGGL((unquantize_segment_kernel<NBITS>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.seg, add);
     else if (p.kind == kUnqVec4)
         hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 4>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.qw, add);
@@ -421,17 +451,17 @@ inline size_t colg_lds_bytes_rt(const ColGeom& c, size_t nbits)
 }
 
 inline hipError_t launch_unquantize_batch(hipStream_t s, LaunchEvents ev, const UnquantizeBatchEntry* entries, const uint32_t* begins,
-                                          uint32_t count, uint32_t total_blocks, size_t nbits, bool add)
+                                          uint32_t count, uint32_t total_blocks, size_t nbits, bool add, size_t lds)
 {
     const int a = add ? 1 : 0;
     switch (nbits)
     {
-    case 1: hipExtLaunchKernelGGL((unquantize_batch_kernel<1>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    case 2: hipExtLaunchKernelGGL((unquantize_batch_kernel<2>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    case 4: hipExtLaunchKernelGGL((unquantize_batch_kernel<4>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    case 8: hipExtLaunchKernelGGL((unquantize_batch_kernel<8>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    case 16: hipExtLaunchKernelGGL((unquantize_batch_kernel<16>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    case 32: hipExtLaunchKernelGGL((unquantize_batch_kernel<32>), dim3(total_blocks), dim3(256), 0, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 1: hipExtLaunchKernelGGL((unquantize_batch_kernel<1>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 2: hipExtLaunchKernelGGL((unquantize_batch_kernel<2>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 4: hipExtLaunchKernelGGL((unquantize_batch_kernel<4>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 8: hipExtLaunchKernelGGL((unquantize_batch_kernel<8>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 16: hipExtLaunchKernelGGL((unquantize_batch_kernel<16>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
+    case 32: hipExtLaunchKernelGGL((unquantize_batch_kernel<32>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -13,6 +13,11 @@ inexact; fine code grids: 16 bits), a differing code is accepted within 1.5 x th
 deviation instead, and counted separately as "beyond 1e-6"; callers that must hold the 1e-6 rule literally pass
 strict=True, which makes any such element a failure.
 
+Columns of more than 16384 rows: the oracle adds such a column term by term in fp32, which is itself off by about
+sqrt(rows) * 2^-24 of the sum (2e-5 at 100000 rows). A column whose bounds miss the oracle's by more than 1e-5 is
+accepted if it is within 1e-5 of the bounds computed from the same values in float64 (exact_headers); its residuals
+may then differ from the oracle's by 1.5 x the observed deviation of the bounds.
+
 The figures above are for float32 matrices. For float64 matrices (64-bit QWords) the same rules apply with 1e-12 /
 1e-13 / 1e-12: both sides sum in double and differ in the order of the additions only.
 """
@@ -54,6 +59,30 @@ class Report:
                    self.max_residual_err))
 
 
+def exact_headers(g, r_in, nbits, zt):
+    """(lower, upper) per column from the statistics of Source/Math/ColumnQuantizer.h:209-341 evaluated in float64 on
+    v = g + r_in (the sum itself rounded in the element type, as every implementation does)."""
+    v = (g + r_in).astype(np.float64)
+    rows = v.shape[0]
+    if nbits > 1:
+        half = 4.0 * np.sqrt((v * v).sum(axis=0) / rows)
+        return -half, half
+    mean = np.zeros(v.shape[1]) if zt else v.sum(axis=0) / rows
+    below = v < mean[None, :]
+    s0 = np.where(below, v, 0.0).sum(axis=0)
+    s1 = np.where(below, 0.0, v).sum(axis=0)
+    n0 = below.sum(axis=0)
+    n1 = rows - n0
+    if zt:
+        m0, m1 = s0 / np.maximum(n0, 1), s1 / np.maximum(n1, 1)
+        centre = 0.5 * (m0 + m1)
+        radius = 2.0 * (m1 - centre)
+    else:
+        radius = 2.0 * ((n0 * mean - s0) + (s1 - n1 * mean)) / rows
+        centre = mean
+    return centre - radius, centre + radius
+
+
 def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, report=None, strict=False, exact=True,
                    skip_cols=None):
     """g, r_in: inputs (F-order float32); q_gpu: packed bytes from the GPU; r_gpu: residual from the GPU.
@@ -88,6 +117,18 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
     assert np.array_equal(lo_g[flat], lo_o[flat]) and np.array_equal(hi_g[flat], hi_o[flat])
     err[flat] = 0.0
     err[~keep] = 0.0
+    res_allow = np.full(cols, value_rtol)
+    if err.max(initial=0.0) > bound_rtol and rows > 16384:
+        # The oracle adds a long column term by term in the element type, which is itself inexact (about
+        # sqrt(rows) * 2^-24 of the sum for fp32: 2e-5 at 100000 rows). A column that misses the oracle's bounds may
+        # instead be within the tolerance of the bounds computed from the same values in float64.
+        lo_x, hi_x = exact_headers(g, r_in, nbits, zt)
+        err_x = np.maximum(np.abs(lo_g.astype(np.float64) - lo_x), np.abs(hi_g.astype(np.float64) - hi_x)) / denom
+        # a residual is value - reconstruction, so in such a column it differs from the oracle's by as much as the bounds do
+        res_allow = np.where(err > bound_rtol, np.maximum(value_rtol, 1.5 * err), value_rtol)
+        err = np.where(err > bound_rtol, np.minimum(err, err_x), err)
+        err[flat] = 0.0
+        err[~keep] = 0.0
     rep.max_bound_err = max(rep.max_bound_err, float(err.max(initial=0.0)))
     assert err.max(initial=0.0) <= bound_rtol, "column bounds off by %.3g of the column scale" % err.max()
 
@@ -117,8 +158,10 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
             pos = (vv - lo) * (used / sc)
             dist = np.abs(pos - np.round(pos)) * (sc / used)
             dist = np.minimum(dist, np.minimum(np.abs(vv - lo), np.abs(vv - hi_o[jj].astype(np.float64))))
-            assert np.all(np.abs(c_g[ii, jj].astype(np.int64) - c_o[ii, jj].astype(np.int64)) == 1), \
-                "codes differ by more than one level"
+            # one level, plus however many levels the bounds themselves moved (fine grids under long columns)
+            levels = 1 + np.floor(1.5 * abs_dev[jj] * used / sc)
+            assert np.all(np.abs(c_g[ii, jj].astype(np.int64) - c_o[ii, jj].astype(np.int64)) <= levels), \
+                "codes differ by more levels than the bounds moved"
         far = dist > thresh_rtol * sc
         allowed = np.maximum(thresh_rtol * sc, 1.5 * abs_dev[jj] + relaxed_floor * sc)
         if strict:
@@ -132,7 +175,7 @@ def check_quantize(g, r_in, q_gpu, r_gpu, nbits, zero_threshold, threads=8, repo
     rerr = np.abs(r_gpu.astype(np.float64) - r_or) / denom[None, :]
     rerr = np.where(same, rerr, 0.0)
     rep.max_residual_err = max(rep.max_residual_err, float(rerr.max(initial=0.0)))
-    assert rerr.max(initial=0.0) <= value_rtol, "residual off by %.3g of the column scale" % rerr.max()
+    assert np.all(rerr <= res_allow[None, :]), "residual off by %.3g of the column scale" % rerr.max()
     return rep
 
 

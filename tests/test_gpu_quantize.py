@@ -123,7 +123,7 @@ PATH_CASES = [
     # one workgroup per column: any height that is a multiple of 4
     (4, 3, PATH_COL, 0), (36, 70, PATH_COL, 0), (128, 9, PATH_COL, 0), (1000, 5, PATH_COL, 0), (1028, 7, PATH_COL, 0),
     (2048, 19, PATH_COL, 0), (2304, 5, PATH_COL, 0), (4100, 3, PATH_COL, 0), (9304, 2, PATH_COL, 0), (14336, 2, PATH_COL, 0),
-    (9304, 3, PATH_AUTO, 0), (1152, 40, PATH_AUTO, 0),
+    (9304, 3, PATH_AUTO, 0), (1152, 40, PATH_AUTO, 0), (100000, 2, PATH_AUTO, 0), (14340, 3, PATH_AUTO, 0),
 ]
 
 
