@@ -1371,7 +1371,7 @@ struct UnqRowGeom
 {
     uint32_t rows;
     uint32_t nq;
-    uint32_t chunk;  // rows per workgroup, multiple of 4
+    uint32_t chunk;  // rows per workgroup, multiple of 4 (the last workgroup of a column also takes the remainder)
     uint32_t chunks; // workgroups per column
     uint32_t blocks; // cols * chunks
     uint32_t pad;
@@ -1396,18 +1396,28 @@ __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q,
         words[w] = bits[w];
     __syncthreads();
     const uint32_t r0 = ch * t.chunk;
-    const uint32_t pieces = (min(t.rows, r0 + t.chunk) - r0) >> 2;
+    const uint32_t pieces = ((ch + 1 == t.chunks ? t.rows : r0 + t.chunk) - r0) >> 2; // the last chunk runs to the end
     f32x4* o4 = reinterpret_cast<f32x4*>(out + (size_t) c * t.rows + r0);
+    const float val0 = unquantize_value<NBITS>(uf, lo, 0u);
+    const float val1 = unquantize_value<NBITS>(uf, lo, 1u);
+    // row i sits in QWord i % nq at bit position i / nq; a thread's pieces are 1024 rows apart
+    const uint32_t i0 = r0 + 4 * tid;
+    uint32_t k0 = i0 / t.nq;
+    uint32_t w0 = i0 - k0 * t.nq;
+    const uint32_t dk = 1024u / t.nq;
+    const uint32_t dw = 1024u - dk * t.nq;
     for (uint32_t p = tid; p < pieces; p += 256)
     {
-        const uint32_t i = r0 + 4 * p;
-        uint32_t k = i / t.nq;
-        uint32_t w = i - k * t.nq;
+        uint32_t k = k0, w = w0;
         f32x4 x;
 #pragma unroll
         for (int e = 0; e < 4; ++e)
         {
-            x[e] = unquantize_value<NBITS>(uf, lo, (words[w] >> (k * SHIFT)) & CODEMASK);
+            const uint32_t code = (words[w] >> (k * SHIFT)) & CODEMASK;
+            if constexpr (NBITS == 1)
+                x[e] = code ? val1 : val0;
+            else
+                x[e] = unquantize_value<NBITS>(uf, lo, code);
             if (++w == t.nq)
             {
                 w = 0;
@@ -1417,6 +1427,13 @@ __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q,
         if (add)
             x = x + o4[p]; // unquantized value + previous content
         __builtin_nontemporal_store(x, o4 + p);
+        k0 += dk;
+        w0 += dw;
+        if (w0 >= t.nq)
+        {
+            w0 -= t.nq;
+            ++k0;
+        }
     }
 }
 

@@ -302,7 +302,7 @@ struct UnquantizePlan
 };
 
 constexpr size_t kUnqRowsMaxLds = 48 * 1024;
-constexpr uint32_t kUnqRowsChunk = 8192;
+constexpr uint32_t kUnqRowsChunk = 2048;
 
 inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t rows, size_t cols, size_t nbits,
                                       const LaunchTuning& tune)
@@ -324,8 +324,14 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
         UnqRowGeom& t = p.rowg;
         t.rows = (uint32_t) rows;
         t.nq = (uint32_t) nq;
-        t.chunk = rows <= 2 * kUnqRowsChunk ? (uint32_t) rows : kUnqRowsChunk;
-        t.chunks = (uint32_t) ((rows + t.chunk - 1) / t.chunk);
+        // small chunks keep many workgroups in flight; a chunk still spans at least four bit positions so that copying
+        // the packed column into LDS stays a small part of the work
+        size_t chunk = ((4 * nq + 1023) / 1024) * 1024;
+        if (chunk < kUnqRowsChunk)
+            chunk = kUnqRowsChunk;
+        t.chunk = (uint32_t) chunk;
+        // the last chunk is the remainder, or takes the remainder along when that is less than half a chunk
+        t.chunks = rows >= chunk ? (uint32_t) ((rows + chunk / 2) / chunk) : 1u;
         const uint64_t blocks = (uint64_t) cols * t.chunks;
         if (blocks <= 0x7FFFFFFFull)
         {
