@@ -226,9 +226,9 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             # HBM bytes per launch of the quantize kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE (two runs), each scaled
-            # by what the same counter reads for a plain 76,218,368-byte device copy (x1.99924 and x1.00000):
-            # 152.45 MB read + 78.75 MB written
-            "traffic": 231.21e6,
+            # by what the same counter reads for a plain 76,218,368-byte device copy (x1.99923 and x1.00000):
+            # 152.42 MB read + 78.90 MB written
+            "traffic": 231.32e6,
         },
     }
     if not args.no_cpu:

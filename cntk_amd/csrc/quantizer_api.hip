@@ -737,6 +737,14 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
             p.cls = p.lds <= kSmallLds ? 0 : 1;
             members[p.cls]++;
         }
+        if (members[0] + members[1] == 1)
+        {
+            // a grid of its own is nothing to share: the plain launch picks the best kernel for the matrix
+            for (size_t i = 0; i < count; ++i)
+                if (plans[i].kind == 0 || plans[i].kind == 1)
+                    plans[i].kind = 2;
+            members[0] = members[1] = 0;
+        }
         const size_t total = members[0] + members[1];
         const size_t entries_bytes = total * sizeof(QuantizeBatchEntry);
         int rc = table_begin_rebuild(tb, entries_bytes + (total + 2) * sizeof(uint32_t) + 64);
@@ -846,6 +854,13 @@ int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item
     }
     if (n == 0)
         return CNTKQ_OK;
+    if (n == 1)
+    {
+        for (size_t i = 0; i < count; ++i)
+            if (items[i].rows != 0 && items[i].cols != 0)
+                return cntkq_unquantize_async(h, items[i].qbuf, qcol_bytes(nbits, items[i].rows) * items[i].cols, 0, items[i].out,
+                                              items[i].rows, items[i].cols, nbits, add);
+    }
     DeviceGuard guard(h->device);
     hipStream_t s = work_stream(h);
     BatchTable& tb = h->unquantize_table;
