@@ -1,14 +1,15 @@
 // C++ host side of the MI355X gradient quantizer: the reference's class shapes on top of the C ABI.
 //
-//   cntk_amd::MatrixQuantizerImpl<float>   <->  Source/Math/MatrixQuantizerImpl.h:19-49
-//   cntk_amd::QuantizedMatrix<float>       <->  Source/Math/QuantizedMatrix.h:54-124, Source/Math/QuantizedMatrix.cpp
-//   cntk_amd::QuantizedColumn<float>       <->  Source/Math/QuantizedMatrix.h:27-48
-//   cntk_amd::MatrixQuantizer<float>       <->  Source/1BitSGD/MatrixQuantizer.h:24-85
+//   cntk_amd::MatrixQuantizerImpl<E>       <->  Source/Math/MatrixQuantizerImpl.h:19-49
+//   cntk_amd::QuantizedMatrix<E>           <->  Source/Math/QuantizedMatrix.h:54-124, Source/Math/QuantizedMatrix.cpp
+//   cntk_amd::QuantizedColumn<E>           <->  Source/Math/QuantizedMatrix.h:27-48
+//   cntk_amd::MatrixQuantizer<E>           <->  Source/1BitSGD/MatrixQuantizer.h:24-85
 //   cntk_amd::MatrixComputeStreamEvent     <->  Source/Math/MatrixQuantizerImpl.h:53-72
-//   cntk_amd::Matrix<float>                     the little of Source/Math/Matrix.h this path needs
+//   cntk_amd::Matrix<E>                         the little of Source/Math/Matrix.h this path needs
 //
 // Same method names, argument meaning and error behaviour (LogicError / RuntimeError / InvalidArgument become
-// std::logic_error / std::runtime_error / std::invalid_argument). Only ElemType = float exists. Header-only; link with
+// std::logic_error / std::runtime_error / std::invalid_argument). ElemType is float or double (the batched calls: float
+// only). Header-only; link with
 // libcntk_amd_quantizer.so and the HIP runtime. There is no CPU quantizer: Create(deviceId < 0) throws.
 #pragma once
 
@@ -47,13 +48,61 @@ inline void HipCheck(hipError_t rc, const char* what)
     if (rc != hipSuccess)
         throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(rc));
 }
+
+// What differs between the two instantiations the reference has (Source/Math/MatrixQuantizerImpl.cpp:28-29): the QWord
+// (Source/Math/ValueQuantizer.h:36-57) and the entry points of the C ABI.
+template <class ElemType>
+struct Abi;
+
+template <>
+struct Abi<float>
+{
+    typedef uint32_t QWord;
+    static size_t QColBytes(size_t bits, size_t rows) { return cntkq_qcol_bytes(bits, rows); }
+    static int Quantize(cntkq_quantizer* h, const float* in, const float* resIn, size_t rows, size_t cols, void* q, size_t qBytes, int onHost,
+                        size_t bits, float* resOut, int zt)
+    {
+        return cntkq_quantize_async(h, in, resIn, rows, cols, q, qBytes, onHost, bits, resOut, zt);
+    }
+    static int Unquantize(cntkq_quantizer* h, const void* q, size_t qBytes, int onHost, float* out, size_t rows, size_t cols, size_t bits, int add)
+    {
+        return cntkq_unquantize_async(h, q, qBytes, onHost, out, rows, cols, bits, add);
+    }
+    static int StripeReduce(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows, size_t cols,
+                            size_t bits, float* stripeRes, void* qOut, float* agg, int zt)
+    {
+        return cntkq_stripe_reduce_async(h, stripes, workers, owner, rows, cols, bits, stripeRes, qOut, agg, zt);
+    }
+};
+
+template <>
+struct Abi<double>
+{
+    typedef uint64_t QWord;
+    static size_t QColBytes(size_t bits, size_t rows) { return cntkq_qcol_bytes_f64(bits, rows); }
+    static int Quantize(cntkq_quantizer* h, const double* in, const double* resIn, size_t rows, size_t cols, void* q, size_t qBytes,
+                        int onHost, size_t bits, double* resOut, int zt)
+    {
+        return cntkq_quantize_async_f64(h, in, resIn, rows, cols, q, qBytes, onHost, bits, resOut, zt);
+    }
+    static int Unquantize(cntkq_quantizer* h, const void* q, size_t qBytes, int onHost, double* out, size_t rows, size_t cols, size_t bits,
+                          int add)
+    {
+        return cntkq_unquantize_async_f64(h, q, qBytes, onHost, out, rows, cols, bits, add);
+    }
+    static int StripeReduce(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows, size_t cols,
+                            size_t bits, double* stripeRes, void* qOut, double* agg, int zt)
+    {
+        return cntkq_stripe_reduce_async_f64(h, stripes, workers, owner, rows, cols, bits, stripeRes, qOut, agg, zt);
+    }
+};
 } // namespace detail
 
 // Dense column-major matrix on one GPU: element (i, j) at Data()[j * GetNumRows() + i]. Owning, or a view of columns.
 template <class ElemType>
 class Matrix
 {
-    static_assert(std::is_same<ElemType, float>::value, "only float is instantiated");
+    static_assert(std::is_same<ElemType, float>::value || std::is_same<ElemType, double>::value, "float or double");
 
 public:
     Matrix(size_t numRows, size_t numCols, int deviceId) : m_rows(numRows), m_cols(numCols), m_device(deviceId), m_owner(true)
@@ -127,13 +176,13 @@ private:
 template <class ElemType>
 struct QuantizedColumn
 {
-    typedef uint32_t QWord;
+    typedef typename detail::Abi<ElemType>::QWord QWord;
     static const size_t QWordNumBits = 8 * sizeof(QWord);
     ElemType lower;
     ElemType upper;
     QWord bits[1];
 
-    static size_t QuantizedColumnSize(size_t bits, size_t rows) { return cntkq_qcol_bytes(bits, rows); }
+    static size_t QuantizedColumnSize(size_t bits, size_t rows) { return detail::Abi<ElemType>::QColBytes(bits, rows); }
 };
 
 // Packed matrix; on a GPU (deviceId >= 0) or in pinned host memory (CPUDEVICE), which is how the reference's v1
@@ -141,15 +190,15 @@ struct QuantizedColumn
 template <class ElemType>
 class QuantizedMatrix
 {
-    static_assert(std::is_same<ElemType, float>::value, "only float is instantiated");
+    static_assert(std::is_same<ElemType, float>::value || std::is_same<ElemType, double>::value, "float or double");
 
 public:
     QuantizedMatrix(size_t numRows, size_t numCols, size_t nbits, int deviceId)
         : m_rows(numRows), m_cols(numCols), m_bits(nbits), m_device(deviceId), m_owner(true)
     {
-        m_qColSize = cntkq_qcol_bytes(nbits, numRows);
+        m_qColSize = detail::Abi<ElemType>::QColBytes(nbits, numRows);
         if (m_qColSize == 0) // Source/Math/QuantizedMatrix.cpp:12-15
-            throw std::logic_error("Quantization: 'nbits' must be a power of two that divides 32");
+            throw std::logic_error("Quantization: 'nbits' must be a power of two that divides the QWord width");
         const size_t bytes = m_qColSize * numCols;
         if (bytes == 0)
             return;
@@ -235,7 +284,7 @@ private:
 template <class ElemType>
 class MatrixQuantizerImpl
 {
-    static_assert(std::is_same<ElemType, float>::value, "only float is instantiated");
+    static_assert(std::is_same<ElemType, float>::value || std::is_same<ElemType, double>::value, "float or double");
 
 public:
     // deviceId >= 0: the GPU quantizer, useAsync = dedicated compute stream (Source/Math/MatrixQuantizerImpl.cpp:10-26)
@@ -278,9 +327,9 @@ public:
         if (outQMatrix.GetNumRows() != rows || outQMatrix.GetNumCols() != cols || inResidual.GetNumRows() != rows ||
             inResidual.GetNumCols() != cols || outResidual.GetNumRows() != rows || outResidual.GetNumCols() != cols)
             throw std::invalid_argument("QuantizeAsync: matrix dimensions do not match");
-        detail::Check(cntkq_quantize_async(m_handle, inMatrix.Data(), inResidual.Data(), rows, cols, outQMatrix.Buffer(), outQMatrix.GetSize(),
-                                           outQMatrix.GetDeviceId() == CPUDEVICE, outQMatrix.GetNumBits(), outResidual.Data(),
-                                           zeroThresholdFor1Bit ? 1 : 0));
+        detail::Check(detail::Abi<ElemType>::Quantize(m_handle, inMatrix.Data(), inResidual.Data(), rows, cols, outQMatrix.Buffer(),
+                                                      outQMatrix.GetSize(), outQMatrix.GetDeviceId() == CPUDEVICE, outQMatrix.GetNumBits(),
+                                                      outResidual.Data(), zeroThresholdFor1Bit ? 1 : 0));
     }
     void WaitQuantizeAsyncDone() override { detail::Check(cntkq_wait_quantize_done(m_handle)); }
 
@@ -288,8 +337,9 @@ public:
     {
         if (inQMatrix.GetNumRows() != outMatrix.GetNumRows() || inQMatrix.GetNumCols() != outMatrix.GetNumCols())
             throw std::invalid_argument("UnquantizeAsync: matrix dimensions do not match");
-        detail::Check(cntkq_unquantize_async(m_handle, inQMatrix.Buffer(), inQMatrix.GetSize(), inQMatrix.GetDeviceId() == CPUDEVICE, outMatrix.Data(),
-                                             outMatrix.GetNumRows(), outMatrix.GetNumCols(), inQMatrix.GetNumBits(), add ? 1 : 0));
+        detail::Check(detail::Abi<ElemType>::Unquantize(m_handle, inQMatrix.Buffer(), inQMatrix.GetSize(), inQMatrix.GetDeviceId() == CPUDEVICE,
+                                                        outMatrix.Data(), outMatrix.GetNumRows(), outMatrix.GetNumCols(), inQMatrix.GetNumBits(),
+                                                        add ? 1 : 0));
     }
     void WaitUnquantizeAsyncDone() override { detail::Check(cntkq_wait_unquantize_done(m_handle)); }
 
@@ -304,6 +354,7 @@ public:
     };
     void QuantizeBatchAsync(const std::vector<QuantizeItem>& items, bool zeroThresholdFor1Bit)
     {
+        static_assert(std::is_same<ElemType, float>::value, "the batched calls exist for float only");
         if (items.empty())
             return;
         const size_t nbits = items[0].outQMatrix->GetNumBits();
@@ -327,6 +378,7 @@ public:
     };
     void UnquantizeBatchAsync(const std::vector<UnquantizeItem>& items, bool add = false)
     {
+        static_assert(std::is_same<ElemType, float>::value, "the batched calls exist for float only");
         if (items.empty())
             return;
         const size_t nbits = items[0].inQMatrix->GetNumBits();
@@ -355,9 +407,10 @@ public:
                 throw std::invalid_argument("StripeReduceAsync: stripes must be device-resident and of equal shape");
             ptrs.push_back(s->Buffer());
         }
-        detail::Check(cntkq_stripe_reduce_async(m_handle, ptrs.data(), ptrs.size(), owner, outQStripe.GetNumRows(), outQStripe.GetNumCols(),
-                                                outQStripe.GetNumBits(), stripeResidual.Data(), outQStripe.Buffer(),
-                                                aggregate ? aggregate->Data() : nullptr, zeroThresholdFor1Bit ? 1 : 0));
+        detail::Check(detail::Abi<ElemType>::StripeReduce(m_handle, ptrs.data(), ptrs.size(), owner, outQStripe.GetNumRows(),
+                                                          outQStripe.GetNumCols(), outQStripe.GetNumBits(), stripeResidual.Data(),
+                                                          outQStripe.Buffer(), aggregate ? aggregate->Data() : nullptr,
+                                                          zeroThresholdFor1Bit ? 1 : 0));
     }
     void WaitStripeReduceDone() { detail::Check(cntkq_wait_stripe_reduce_done(m_handle)); }
 
@@ -434,7 +487,7 @@ public:
     }
     void WaitUnquantizeAsyncDone() { m_quantizerImpl->WaitUnquantizeAsyncDone(); }
     int GetDeviceId() const { return m_quantizerImpl->GetDeviceId(); }
-    void ResetResidue() { m_residual->SetValue(0.0f); }
+    void ResetResidue() { m_residual->SetValue((ElemType) 0); }
     const Matrix<ElemType>& GetResidualMatrix() const { return *m_residual; }
     MatrixQuantizerImpl<ElemType>& Impl() { return *m_quantizerImpl; }
 

@@ -37,42 +37,71 @@ static int g_failures = 0;
         }                                                                                                              \
     } while (0)
 
+// tolerances of the reference test (MatrixQuantizerTests.cpp:24-29)
 static const float c_SinglePrecisionTolerance = 1e-4f;
+static const double c_DoublePrecisionTolerance = 1e-8;
 static const float c_SinglePrecisionGpuQuantizationTolerance = 1e-3f;
+static const double c_DoublePrecisionGpuQuantizationTolerance = 1e-4;
 
-static std::vector<float> RandomUniform(size_t rows, size_t cols, float lo, float hi, unsigned long seed)
+// the CPU checker for either element type
+template <class E> struct Oracle;
+template <> struct Oracle<float>
+{
+    static int Quantize(const float* g, const float* r, size_t rows, size_t cols, void* q, size_t bits, float* rOut, int zt) { return oracle_quantize(g, r, rows, cols, q, bits, rOut, zt, 1); }
+    static int Pack(const float* g, const float* r, size_t rows, size_t cols, void* q, size_t bits, float* rOut, int zt) { return oracle_pack_with_headers(g, r, rows, cols, q, bits, rOut, zt, 1); }
+    static int Unquantize(const void* q, size_t rows, size_t cols, size_t bits, float* out, int add) { return oracle_unquantize(q, rows, cols, bits, out, add, 1); }
+    static double Tolerance() { return c_SinglePrecisionTolerance; }
+    static double OutlierShare() { return c_SinglePrecisionGpuQuantizationTolerance; }
+};
+template <> struct Oracle<double>
+{
+    static int Quantize(const double* g, const double* r, size_t rows, size_t cols, void* q, size_t bits, double* rOut, int zt) { return oracle_quantize_f64(g, r, rows, cols, q, bits, rOut, zt, 1); }
+    static int Pack(const double* g, const double* r, size_t rows, size_t cols, void* q, size_t bits, double* rOut, int zt) { return oracle_pack_with_headers_f64(g, r, rows, cols, q, bits, rOut, zt, 1); }
+    static int Unquantize(const void* q, size_t rows, size_t cols, size_t bits, double* out, int add) { return oracle_unquantize_f64(q, rows, cols, bits, out, add, 1); }
+    static double Tolerance() { return c_DoublePrecisionTolerance; }
+    static double OutlierShare() { return c_DoublePrecisionGpuQuantizationTolerance; }
+};
+
+template <class E>
+static std::vector<E> RandomUniformT(size_t rows, size_t cols, E lo, E hi, unsigned long seed)
 {
     std::mt19937_64 rng(seed);
-    std::vector<float> a(rows * cols);
+    std::vector<E> a(rows * cols);
     for (auto& x : a)
-        x = (float) (lo + (hi - lo) * ((rng() >> 11) * (1.0 / 9007199254740992.0)));
+        x = (E) (lo + (hi - lo) * ((rng() >> 11) * (1.0 / 9007199254740992.0)));
     return a;
 }
 
-static void TestRunQuantization(size_t numBits, size_t numRows, size_t numCols, float rangeLow, float rangeHigh, int seed,
+static std::vector<float> RandomUniform(size_t rows, size_t cols, float lo, float hi, unsigned long seed)
+{
+    return RandomUniformT<float>(rows, cols, lo, hi, seed);
+}
+
+template <class E>
+static void TestRunQuantization(size_t numBits, size_t numRows, size_t numCols, E rangeLow, E rangeHigh, int seed,
                                 int numIterations, int deviceId, bool zeroThresholdFor1Bit, bool hostQuantizedMatrix)
 {
-    Matrix<float> inMatrix(numRows, numCols, deviceId);
-    std::unique_ptr<MatrixQuantizerImpl<float>> quantizer(MatrixQuantizerImpl<float>::Create(deviceId, false /*useAsync*/));
-    Matrix<float> residueMatrix(numRows, numCols, deviceId);
-    Matrix<float> outMatrix(numRows, numCols, deviceId);
+    Matrix<E> inMatrix(numRows, numCols, deviceId);
+    std::unique_ptr<MatrixQuantizerImpl<E>> quantizer(MatrixQuantizerImpl<E>::Create(deviceId, false /*useAsync*/));
+    Matrix<E> residueMatrix(numRows, numCols, deviceId);
+    Matrix<E> outMatrix(numRows, numCols, deviceId);
     const size_t numMatrixElems = inMatrix.GetNumElements();
 
     {
         // the initial residue and output are all zeros
         auto r = residueMatrix.CopyToArray(), o = outMatrix.CopyToArray();
         for (size_t i = 0; i < numMatrixElems; ++i)
-            CHECK(r[i] == 0.0f && o[i] == 0.0f, "fresh matrices must be zero");
+            CHECK(r[i] == (E) 0 && o[i] == (E) 0, "fresh matrices must be zero");
     }
 
     for (int iterNum = 0; iterNum < numIterations; ++iterNum)
     {
-        std::vector<float> in = RandomUniform(numRows, numCols, rangeLow, rangeHigh, (unsigned long) (seed + iterNum));
+        std::vector<E> in = RandomUniformT<E>(numRows, numCols, rangeLow, rangeHigh, (unsigned long) (seed + iterNum));
         inMatrix.SetValue(in.data());
         auto prevResidual = residueMatrix.CopyToArray();
         auto prevOut = outMatrix.CopyToArray();
 
-        QuantizedMatrix<float> tempQuantizationBuffer(numRows, numCols, numBits, hostQuantizedMatrix ? CPUDEVICE : deviceId);
+        QuantizedMatrix<E> tempQuantizationBuffer(numRows, numCols, numBits, hostQuantizedMatrix ? CPUDEVICE : deviceId);
         quantizer->QuantizeAsync(inMatrix, residueMatrix, tempQuantizationBuffer, residueMatrix, zeroThresholdFor1Bit);
         quantizer->WaitQuantizeAsyncDone();
         quantizer->UnquantizeAsync(tempQuantizationBuffer, outMatrix, (iterNum > 0));
@@ -82,45 +111,50 @@ static void TestRunQuantization(size_t numBits, size_t numRows, size_t numCols, 
         auto newOut = outMatrix.CopyToArray();
         std::vector<char> packed = tempQuantizationBuffer.CopyToHost();
 
-        float tolerance = 0.0f;
-        if (numBits != 8 * sizeof(float))
-            tolerance = (rangeHigh - rangeLow) * c_SinglePrecisionTolerance;
+        double tolerance = 0.0;
+        if (numBits != 8 * sizeof(E))
+            tolerance = (double) (rangeHigh - rangeLow) * Oracle<E>::Tolerance();
+        // a last-bit difference of the bounds moves a value by one code: 2^-32 of the range at 32 bits (double only)
+        if (sizeof(E) == 8 && numBits == 32)
+            tolerance = (double) (rangeHigh - rangeLow) * 1e-7;
 
         for (size_t i = 0; i < numMatrixElems; ++i)
-            CHECK(std::fabs((in[i] + prevResidual[i] + prevOut[i]) - (newResidual[i] + newOut[i])) <= tolerance + 1e-6f * (rangeHigh - rangeLow),
+            CHECK(std::fabs((double) (in[i] + prevResidual[i] + prevOut[i]) - (double) (newResidual[i] + newOut[i])) <=
+                      tolerance + (sizeof(E) == 4 ? 1e-6 : 1e-14) * (double) (rangeHigh - rangeLow),
                   "conservation, element %zu", i);
 
-        const size_t numIncorrectAllowed = std::max<size_t>(1, (size_t) (numMatrixElems * c_SinglePrecisionGpuQuantizationTolerance));
+        const size_t numIncorrectAllowed = std::max<size_t>(1, (size_t) (numMatrixElems * Oracle<E>::OutlierShare()));
 
         // the CPU checker on the same inputs
-        std::vector<float> refResidual(numMatrixElems), refOut(prevOut.get(), prevOut.get() + numMatrixElems);
+        std::vector<E> refResidual(numMatrixElems), refOut(prevOut.get(), prevOut.get() + numMatrixElems);
         std::vector<char> refPacked(packed.size());
-        oracle_quantize(in.data(), prevResidual.get(), numRows, numCols, refPacked.data(), numBits, refResidual.data(), zeroThresholdFor1Bit, 1);
-        oracle_unquantize(refPacked.data(), numRows, numCols, numBits, refOut.data(), iterNum > 0, 1);
+        Oracle<E>::Quantize(in.data(), prevResidual.get(), numRows, numCols, refPacked.data(), numBits, refResidual.data(), zeroThresholdFor1Bit);
+        Oracle<E>::Unquantize(refPacked.data(), numRows, numCols, numBits, refOut.data(), iterNum > 0);
         size_t numIncorrectOut = 0, numIncorrectResidual = 0;
         for (size_t i = 0; i < numMatrixElems; ++i)
         {
-            if (std::fabs(newOut[i] - refOut[i]) > tolerance && ++numIncorrectOut > numIncorrectAllowed)
-                CHECK(false, "output differs from the CPU checker at %zu: %g vs %g", i, newOut[i], refOut[i]);
-            if (std::fabs(newResidual[i] - refResidual[i]) > tolerance && ++numIncorrectResidual > numIncorrectAllowed)
-                CHECK(false, "residual differs from the CPU checker at %zu: %g vs %g", i, newResidual[i], refResidual[i]);
+            if (std::fabs((double) newOut[i] - (double) refOut[i]) > tolerance && ++numIncorrectOut > numIncorrectAllowed)
+                CHECK(false, "output differs from the CPU checker at %zu: %g vs %g", i, (double) newOut[i], (double) refOut[i]);
+            if (std::fabs((double) newResidual[i] - (double) refResidual[i]) > tolerance && ++numIncorrectResidual > numIncorrectAllowed)
+                CHECK(false, "residual differs from the CPU checker at %zu: %g vs %g", i, (double) newResidual[i], (double) refResidual[i]);
         }
 
         // stricter: bit-exact codes / residual under the device's own headers, bit-exact unquantize
         std::vector<char> exactPacked(packed);
-        std::vector<float> exactResidual(numMatrixElems), exactOut(prevOut.get(), prevOut.get() + numMatrixElems);
-        oracle_pack_with_headers(in.data(), prevResidual.get(), numRows, numCols, exactPacked.data(), numBits, exactResidual.data(), zeroThresholdFor1Bit, 1);
+        std::vector<E> exactResidual(numMatrixElems), exactOut(prevOut.get(), prevOut.get() + numMatrixElems);
+        Oracle<E>::Pack(in.data(), prevResidual.get(), numRows, numCols, exactPacked.data(), numBits, exactResidual.data(), zeroThresholdFor1Bit);
         CHECK(std::memcmp(exactPacked.data(), packed.data(), packed.size()) == 0, "codes under the device's headers");
-        CHECK(std::memcmp(exactResidual.data(), newResidual.get(), numMatrixElems * sizeof(float)) == 0, "residual under the device's headers");
-        oracle_unquantize(packed.data(), numRows, numCols, numBits, exactOut.data(), iterNum > 0, 1);
-        CHECK(std::memcmp(exactOut.data(), newOut.get(), numMatrixElems * sizeof(float)) == 0, "unquantize");
+        CHECK(std::memcmp(exactResidual.data(), newResidual.get(), numMatrixElems * sizeof(E)) == 0, "residual under the device's headers");
+        Oracle<E>::Unquantize(packed.data(), numRows, numCols, numBits, exactOut.data(), iterNum > 0);
+        CHECK(std::memcmp(exactOut.data(), newOut.get(), numMatrixElems * sizeof(E)) == 0, "unquantize");
     }
 }
 
-static void TestQuantization(int deviceId, size_t numRows, size_t numCols, float rangeLow, float rangeHigh, int seed, int numIterations)
+template <class E>
+static void TestQuantization(int deviceId, size_t numRows, size_t numCols, E rangeLow, E rangeHigh, int seed, int numIterations)
 {
     // all power-of-two bit widths; 1 bit with and without zeroThresholdFor1Bit
-    const size_t maxNumBits = 8 * sizeof(float);
+    const size_t maxNumBits = 8 * sizeof(E);
     for (size_t numBits = 1; numBits <= maxNumBits; numBits *= 2)
         for (int i = 0; i < 2; ++i)
         {
@@ -128,28 +162,40 @@ static void TestQuantization(int deviceId, size_t numRows, size_t numCols, float
             if (numBits != 1 && zeroThresholdFor1Bit)
                 continue;
             for (int host = 0; host < 2; ++host)
-                TestRunQuantization(numBits, numRows, numCols, rangeLow, rangeHigh, seed, numIterations, deviceId, zeroThresholdFor1Bit, host != 0);
+                TestRunQuantization<E>(numBits, numRows, numCols, rangeLow, rangeHigh, seed, numIterations, deviceId, zeroThresholdFor1Bit, host != 0);
         }
+}
+
+// the reference runs its ten cases for float and for double (MatrixQuantizerTests.cpp:406-431)
+template <class E>
+static void GPUMatrix1BitQuantize()
+{
+    const int dev = 0;
+    TestQuantization<E>(dev, 25, 13, (E) -1.0, (E) +1.0, 2015, 5);
+    TestQuantization<E>(dev, 25, 13, (E) -0.005, (E) +0.005, 2115, 5);
+    TestQuantization<E>(dev, 13, 25, (E) -0.00001, (E) +0.00001, 2215, 5);
+    TestQuantization<E>(dev, 13, 25, (E) -10.0, (E) +10.0, 2315, 5);
+    TestQuantization<E>(dev, 25, 13, (E) -1.0, (E) +2.05, 2415, 5);
+    TestQuantization<E>(dev, 489, 1, (E) -0.5, (E) +0.5, 2515, 5);
+    TestQuantization<E>(dev, 1, 135, (E) -0.5, (E) +0.5, 2615, 5);
+    TestQuantization<E>(dev, 89, 23, (E) -0.5, (E) +0.5, 2715, 5);
+    TestQuantization<E>(dev, 15, 35, (E) -0.5, (E) +0.5, 2815, 5);
+    TestQuantization<E>(dev, 100, 50, (E) -0.5, (E) +0.5, 2915, 5);
+    // the sizes the reference test was first written with (:474-487)
+    TestQuantization<E>(dev, 256, 135, (E) -1.0, (E) +2.05, 2415, 5);
+    TestQuantization<E>(dev, 737, 373, (E) -0.5, (E) +0.5, 2915, 5);
+    // the headline column height
+    TestQuantization<E>(dev, 2048, 33, (E) -0.02, (E) +0.03, 3015, 3);
 }
 
 static void GPUMatrix1BitQuantizeFloat()
 {
-    const int dev = 0;
-    TestQuantization(dev, 25, 13, -1.0f, +1.0f, 2015, 5);
-    TestQuantization(dev, 25, 13, -0.005f, +0.005f, 2115, 5);
-    TestQuantization(dev, 13, 25, -0.00001f, +0.00001f, 2215, 5);
-    TestQuantization(dev, 13, 25, -10.0f, +10.0f, 2315, 5);
-    TestQuantization(dev, 25, 13, -1.0f, +2.05f, 2415, 5);
-    TestQuantization(dev, 489, 1, -0.5f, +0.5f, 2515, 5);
-    TestQuantization(dev, 1, 135, -0.5f, +0.5f, 2615, 5);
-    TestQuantization(dev, 89, 23, -0.5f, +0.5f, 2715, 5);
-    TestQuantization(dev, 15, 35, -0.5f, +0.5f, 2815, 5);
-    TestQuantization(dev, 100, 50, -0.5f, +0.5f, 2915, 5);
-    // the sizes the reference test was first written with (:474-487)
-    TestQuantization(dev, 256, 135, -1.0f, +2.05f, 2415, 5);
-    TestQuantization(dev, 737, 373, -0.5f, +0.5f, 2915, 5);
-    // the headline column height
-    TestQuantization(dev, 2048, 33, -0.02f, +0.03f, 3015, 3);
+    GPUMatrix1BitQuantize<float>();
+}
+
+static void GPUMatrix1BitQuantizeDouble()
+{
+    GPUMatrix1BitQuantize<double>();
 }
 
 // A gradient set through the batched calls gives the bytes of the per-matrix calls.
@@ -237,6 +283,9 @@ int main()
         GPUMatrix1BitQuantizeFloat();
         std::printf("Test case GPUMatrixSuite/GPUMatrix1BitQuantizeFloat %s\n", g_failures ? "has FAILED" : "has passed");
         int before = g_failures;
+        GPUMatrix1BitQuantizeDouble();
+        std::printf("Test case GPUMatrixSuite/GPUMatrix1BitQuantizeDouble %s\n", g_failures != before ? "has FAILED" : "has passed");
+        before = g_failures;
         BatchEqualsPerMatrix();
         std::printf("Test case GPUMatrixSuite/QuantizerBatchEqualsPerMatrix %s\n", g_failures != before ? "has FAILED" : "has passed");
         before = g_failures;

@@ -17,6 +17,7 @@ def test_cpp_matrix_quantizer_suite():
     print(res.stderr[-4000:])
     assert res.returncode == 0, "C++ quantizer tests failed"
     assert "GPUMatrix1BitQuantizeFloat has passed" in res.stdout
+    assert "GPUMatrix1BitQuantizeDouble has passed" in res.stdout
     assert "QuantizerErrorBehaviour has passed" in res.stdout
     assert "QuantizerBatchEqualsPerMatrix has passed" in res.stdout
 
