@@ -272,6 +272,38 @@ def test_special_columns(quantizer):
     assert oracle.words(Q.to_numpy(), 5, 1, 1)[0, 0] == 0b10101
 
 
+@pytest.mark.parametrize("rows,cols", [(70, 9), (429, 8), (2048, 12), (1152, 10), (20000, 6)])
+def test_non_finite_columns_stay_in_their_columns(rows, cols):
+    """A NaN or an infinity in one column must not disturb any other column (columns are independent in the reference,
+    Source/Math/MatrixQuantizerCPU.cpp:28-59), and the call must complete. What the poisoned column itself holds is
+    not compared: the reference converts a NaN to an integer there, which C leaves undefined."""
+    qz = MatrixQuantizerImpl.Create(0, False)
+    g = datagen.normal(4242 + rows, rows, cols)
+    r = datagen.normal(4243 + rows, rows, cols, 0.002)
+    bad = [1, cols - 2, cols - 1]
+    g[rows // 2, bad[0]] = np.nan
+    g[0, bad[1]] = np.inf
+    r[rows - 1, bad[2]] = -np.inf
+    good = [j for j in range(cols) if j not in bad]
+    for nbits, zt in VARIANTS:
+        say("non-finite", rows, cols, nbits, zt)
+        Q, r_out = gpu_quantize(qz, g, r, nbits, zt)
+        q = Q.to_numpy()
+        qcol = oracle.qcol_bytes(nbits, rows)
+        q_good = np.concatenate([q[j * qcol:(j + 1) * qcol] for j in good])
+        parity.check_quantize(np.asfortranarray(g[:, good]), np.asfortranarray(r[:, good]), q_good,
+                              np.asfortranarray(r_out[:, good]), nbits, zt)
+        Out = Matrix(rows, cols)
+        qz.UnquantizeAsync(Q, Out)
+        qz.WaitUnquantizeAsyncDone()
+        out = Out.to_numpy()
+        ref = oracle.unquantize(q_good, rows, len(good), nbits)
+        assert parity.bits_equal(np.asfortranarray(out[:, good]), ref)
+        if nbits < 32:
+            # the poisoned values do not come back as ordinary numbers in the error feedback
+            assert not np.isfinite(r_out[rows // 2, bad[0]]) and not np.isfinite(r_out[0, bad[1]])
+
+
 def test_error_behaviour(quantizer):
     g = Matrix(8, 4)
     with pytest.raises(cntk_amd.QuantizerLogicError):  # dimension mismatch (asserts in the reference)
