@@ -46,6 +46,11 @@ class _UnquantizeItem(ctypes.Structure):
     _fields_ = [("qbuf", _vp), ("out", _vp), ("rows", _sz), ("cols", _sz)]
 
 
+class _StripeReduceItem(ctypes.Structure):
+    _fields_ = [("stripes", ctypes.POINTER(_vp)), ("stripe_res", _vp), ("q_out", _vp), ("agg_out", _vp), ("rows", _sz),
+                ("stripe_cols", _sz)]
+
+
 def lib():
     """The loaded C-ABI library. Raises if it has not been built (python -m cntk_amd.build)."""
     global _lib
@@ -87,6 +92,7 @@ def lib():
         L.cntkq_quantize_async_f64.argtypes = L.cntkq_quantize_async.argtypes
         L.cntkq_unquantize_async_f64.argtypes = L.cntkq_unquantize_async.argtypes
         L.cntkq_stripe_reduce_async_f64.argtypes = L.cntkq_stripe_reduce_async.argtypes
+        L.cntkq_stripe_reduce_batch_async.argtypes = [_vp, ctypes.POINTER(_StripeReduceItem), _sz, _sz, _sz, _sz, ctypes.c_int]
         L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int]
         _lib = L
     return _lib
@@ -367,6 +373,34 @@ class MatrixQuantizerImpl:
         _check(_fn("cntkq_stripe_reduce_async", out_qstripe.dtype)(self._h, arr, k, owner, rows, cols, nbits, stripe_residual.Data(),
                                                out_qstripe.Buffer(), agg_out.Data() if agg_out is not None else None,
                                                int(bool(zero_threshold_for_1bit))))
+
+    def StripeReduceBatchAsync(self, items, owner, zero_threshold_for_1bit):
+        """The owner's stripe reductions of a whole gradient set as one call. items: sequence of
+        (stripes, stripe_residual, out_qstripe, agg_out or None), one per gradient matrix, float32 only."""
+        if not items:
+            return
+        k = len(items[0][0])
+        nbits = items[0][2].GetNumBits()
+        arr = (_StripeReduceItem * len(items))()
+        keep = []
+        for n, (stripes, stripe_residual, out_qstripe, agg_out) in enumerate(items):
+            rows, cols = out_qstripe.GetNumRows(), out_qstripe.GetNumCols()
+            if len(stripes) != k or out_qstripe.GetNumBits() != nbits:
+                raise QuantizerLogicError("StripeReduceBatchAsync: items must share the worker count and the bit width")
+            for s in stripes:
+                if s.GetNumRows() != rows or s.GetNumCols() != cols or s.GetNumBits() != nbits or s.GetDeviceId() < 0:
+                    raise QuantizerLogicError("StripeReduceBatchAsync: stripes must be device-resident and of equal shape")
+            if stripe_residual.GetNumRows() != rows or stripe_residual.GetNumCols() != cols:
+                raise QuantizerLogicError("StripeReduceBatchAsync: stripe residual has the wrong shape")
+            mats = list(stripes) + [stripe_residual, out_qstripe] + ([agg_out] if agg_out is not None else [])
+            if any(m.dtype != torch.float32 for m in mats):
+                raise QuantizerLogicError("StripeReduceBatchAsync: the batched calls exist for float32 only")
+            ptrs = (_vp * k)(*[s.Buffer() for s in stripes])
+            keep.append(ptrs)
+            arr[n] = _StripeReduceItem(ptrs, stripe_residual.Data(), out_qstripe.Buffer(),
+                                       agg_out.Data() if agg_out is not None else None, rows, cols)
+        _check(lib().cntkq_stripe_reduce_batch_async(self._h, arr, len(items), k, owner, nbits,
+                                                     int(bool(zero_threshold_for_1bit))))
 
     def WaitStripeReduceDone(self):
         _check(lib().cntkq_wait_stripe_reduce_done(self._h))

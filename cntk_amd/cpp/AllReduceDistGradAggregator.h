@@ -110,37 +110,34 @@ public:
 
     void PostStripe(size_t from, size_t to, size_t matrixIdx, QuantizedMatrix<float>&& stripe) override
     {
-        m_stripes.erase({to, from, matrixIdx});
-        m_stripes.emplace(Key{to, from, matrixIdx}, std::move(stripe));
+        Store(m_stripes, to * m_numWorkers + from, matrixIdx, std::move(stripe));
     }
     const QuantizedMatrix<float>& ReceivedStripe(size_t owner, size_t from, size_t matrixIdx) override
     {
-        auto it = m_stripes.find({owner, from, matrixIdx});
-        if (it == m_stripes.end())
+        const QuantizedMatrix<float>* s = Find(m_stripes, owner * m_numWorkers + from, matrixIdx);
+        if (s == nullptr)
             throw std::logic_error("InProcessTransport: stripe was never posted");
-        return it->second;
+        return *s;
     }
     void PostAggregatedStripe(size_t owner, size_t matrixIdx, QuantizedMatrix<float>&& stripe) override
     {
-        m_aggregated.erase({owner, 0, matrixIdx});
-        m_aggregated.emplace(Key{owner, 0, matrixIdx}, std::move(stripe));
+        Store(m_aggregated, owner, matrixIdx, std::move(stripe));
     }
     void FetchAggregatedStripe(size_t /*to*/, size_t owner, size_t matrixIdx, QuantizedMatrix<float>& dst, void* hipStream) override
     {
-        auto it = m_aggregated.find({owner, 0, matrixIdx});
-        if (it == m_aggregated.end())
+        const QuantizedMatrix<float>* s = Find(m_aggregated, owner, matrixIdx);
+        if (s == nullptr)
             throw std::logic_error("InProcessTransport: aggregated stripe was never posted");
-        if (it->second.GetSize() != dst.GetSize())
+        if (s->GetSize() != dst.GetSize())
             throw std::logic_error("InProcessTransport: stripe size mismatch");
         if (dst.GetSize() != 0)
-            detail::HipCheck(hipMemcpyAsync(dst.Buffer(), it->second.Buffer(), dst.GetSize(), hipMemcpyDeviceToDevice,
+            detail::HipCheck(hipMemcpyAsync(dst.Buffer(), s->Buffer(), dst.GetSize(), hipMemcpyDeviceToDevice,
                                             static_cast<hipStream_t>(hipStream)),
                              "hipMemcpyAsync");
     }
     const QuantizedMatrix<float>* AggregatedStripeView(size_t /*to*/, size_t owner, size_t matrixIdx) override
     {
-        auto it = m_aggregated.find({owner, 0, matrixIdx});
-        return it == m_aggregated.end() ? nullptr : &it->second;
+        return Find(m_aggregated, owner, matrixIdx);
     }
     void PostHeader(size_t from, const DistGradHeader& header) override
     {
@@ -159,15 +156,31 @@ public:
     }
 
 private:
-    struct Key
+    // messages by (channel, matrix); a message that names the very buffer of the previous step's is kept as it is,
+    // so a steady training loop allocates nothing here
+    typedef std::vector<std::vector<std::unique_ptr<QuantizedMatrix<float>>>> Slots;
+    static void Store(Slots& slots, size_t channel, size_t matrixIdx, QuantizedMatrix<float>&& stripe)
     {
-        size_t a, b, c;
-        bool operator<(const Key& o) const { return std::tie(a, b, c) < std::tie(o.a, o.b, o.c); }
-    };
+        if (slots.size() <= channel)
+            slots.resize(channel + 1);
+        if (slots[channel].size() <= matrixIdx)
+            slots[channel].resize(matrixIdx + 1);
+        std::unique_ptr<QuantizedMatrix<float>>& slot = slots[channel][matrixIdx];
+        if (slot && slot->Buffer() == stripe.Buffer() && slot->GetNumRows() == stripe.GetNumRows() &&
+            slot->GetNumCols() == stripe.GetNumCols() && slot->GetNumBits() == stripe.GetNumBits())
+            return;
+        slot.reset(new QuantizedMatrix<float>(std::move(stripe)));
+    }
+    static const QuantizedMatrix<float>* Find(const Slots& slots, size_t channel, size_t matrixIdx)
+    {
+        if (channel >= slots.size() || matrixIdx >= slots[channel].size())
+            return nullptr;
+        return slots[channel][matrixIdx].get();
+    }
     size_t m_numWorkers;
     bool m_streamOrdered;
-    std::map<Key, QuantizedMatrix<float>> m_stripes;
-    std::map<Key, QuantizedMatrix<float>> m_aggregated;
+    Slots m_stripes;
+    Slots m_aggregated;
     std::map<size_t, DistGradHeader> m_headers;
 };
 
@@ -292,7 +305,37 @@ public:
     {
         const size_t K = NumProc();
         const bool fused = m_options.useFusedStripeReduce && m_useQuantizationForSelfStripe;
-        for (size_t i = 0; i < gradients.size(); ++i)
+        // every matrix's stripe in one call: the stripe quantizers share one stream, so any of their handles will do
+        const bool batched = fused && m_options.useBatchedCalls && gradients.size() > 1;
+        if (batched)
+        {
+            typedef typename MatrixQuantizerGPU<ElemType>::StripeReduceItem Item;
+            std::vector<Item> items;
+            std::vector<QuantizedMatrix<ElemType>> ownSlices; // keep the views alive until the call
+            ownSlices.reserve(gradients.size());
+            for (size_t i = 0; i < gradients.size(); ++i)
+            {
+                const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K);
+                if (stripe.m_numCols == 0)
+                    continue;
+                ownSlices.push_back(m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+                Item it;
+                for (size_t w = 0; w < K; ++w)
+                    it.stripes.push_back(&m_transport.ReceivedStripe(MyRank(), w, i));
+                it.stripeResidual = &const_cast<Matrix<ElemType>&>(m_aggGradStripeQuantizers[i]->GetResidualMatrix());
+                it.outQStripe = &ownSlices.back();
+                it.aggregate = nullptr;
+                items.push_back(std::move(it));
+            }
+            if (!items.empty())
+            {
+                m_stripeBatchQuantizer = 0;
+                while (GetStripeForNode(gradients[m_stripeBatchQuantizer]->GetNumCols(), MyRank(), K).m_numCols == 0)
+                    m_stripeBatchQuantizer++;
+                Gpu(*m_aggGradStripeQuantizers[m_stripeBatchQuantizer]).StripeReduceBatchAsync(items, MyRank(), m_zeroThresholdFor1Bit);
+            }
+        }
+        for (size_t i = 0; i < gradients.size() && !batched; ++i)
         {
             const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K);
             if (stripe.m_numCols == 0)
@@ -330,7 +373,9 @@ public:
             const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K);
             if (stripe.m_numCols == 0)
                 continue;
-            if (hostWaits && fused)
+            if (hostWaits && batched)
+                Gpu(*m_aggGradStripeQuantizers[m_stripeBatchQuantizer]).WaitStripeReduceDone();
+            else if (hostWaits && fused)
                 Gpu(*m_aggGradStripeQuantizers[i]).WaitStripeReduceDone();
             else if (hostWaits)
                 m_aggGradStripeQuantizers[i]->WaitQuantizeAsyncDone(); // (:494)
@@ -452,6 +497,7 @@ private:
     std::vector<std::unique_ptr<MatrixQuantizer<ElemType>>> m_preAggGradQuantizers;
     std::vector<std::unique_ptr<QuantizedMatrix<ElemType>>> m_gradQuantized;
     std::vector<std::unique_ptr<MatrixQuantizer<ElemType>>> m_aggGradStripeQuantizers;
+    size_t m_stripeBatchQuantizer = 0; // which of them carried the last batched stripe reduction
 };
 
 // K workers of one process on one GPU: drives the three steps of every worker in turn. This is the arrangement of the

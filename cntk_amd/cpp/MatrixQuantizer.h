@@ -412,6 +412,41 @@ public:
                                                           outQStripe.Buffer(), aggregate ? aggregate->Data() : nullptr,
                                                           zeroThresholdFor1Bit ? 1 : 0));
     }
+    // The owner's stripe reductions of a whole gradient set as one call (one item per gradient matrix).
+    struct StripeReduceItem
+    {
+        std::vector<const QuantizedMatrix<ElemType>*> stripes;
+        Matrix<ElemType>* stripeResidual;
+        QuantizedMatrix<ElemType>* outQStripe;
+        Matrix<ElemType>* aggregate; // may be null
+    };
+    void StripeReduceBatchAsync(const std::vector<StripeReduceItem>& items, size_t owner, bool zeroThresholdFor1Bit)
+    {
+        static_assert(std::is_same<ElemType, float>::value, "the batched calls exist for float only");
+        if (items.empty())
+            return;
+        const size_t workers = items[0].stripes.size();
+        const size_t nbits = items[0].outQStripe->GetNumBits();
+        std::vector<std::vector<const void*>> ptrs(items.size());
+        std::vector<cntkq_stripe_reduce_item> raw;
+        for (size_t i = 0; i < items.size(); ++i)
+        {
+            const auto& it = items[i];
+            if (it.stripes.size() != workers || it.outQStripe->GetNumBits() != nbits)
+                throw std::invalid_argument("StripeReduceBatchAsync: items must share the worker count and the bit width");
+            for (const auto* s : it.stripes)
+            {
+                if (s->GetNumRows() != it.outQStripe->GetNumRows() || s->GetNumCols() != it.outQStripe->GetNumCols() ||
+                    s->GetNumBits() != nbits || s->GetDeviceId() < 0)
+                    throw std::invalid_argument("StripeReduceBatchAsync: stripes must be device-resident and of equal shape");
+                ptrs[i].push_back(s->Buffer());
+            }
+            raw.push_back(cntkq_stripe_reduce_item{ptrs[i].data(), it.stripeResidual->Data(), it.outQStripe->Buffer(),
+                                                   it.aggregate ? it.aggregate->Data() : nullptr, it.outQStripe->GetNumRows(),
+                                                   it.outQStripe->GetNumCols()});
+        }
+        detail::Check(cntkq_stripe_reduce_batch_async(m_handle, raw.data(), raw.size(), workers, owner, nbits, zeroThresholdFor1Bit ? 1 : 0));
+    }
     void WaitStripeReduceDone() { detail::Check(cntkq_wait_stripe_reduce_done(m_handle)); }
 
     cntkq_quantizer* Handle() const { return m_handle; }

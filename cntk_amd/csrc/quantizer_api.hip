@@ -184,6 +184,7 @@ struct cntkq_quantizer
     // reads it has finished (its event).
     BatchTable quantize_table;
     BatchTable unquantize_table;
+    BatchTable stripe_table;
     LaunchTuning tune;
 };
 
@@ -575,6 +576,7 @@ int cntkq_destroy(cntkq_quantizer* h)
         (void) hipFree(h->staging);
     table_destroy(h->quantize_table);
     table_destroy(h->unquantize_table);
+    table_destroy(h->stripe_table);
     hipEvent_t evs[] = {h->ev_quantize, h->ev_fetch, h->ev_assign, h->ev_unquantize, h->ev_stripe, h->ev_main};
     for (hipEvent_t e : evs)
         if (e != nullptr)
@@ -934,6 +936,155 @@ int cntkq_stripe_reduce_async_f64(cntkq_quantizer* h, const void* const* stripes
 {
     return stripe_reduce_async_impl<double>(h, stripes, workers, owner, rows, stripe_cols, nbits, stripe_res, q_out, agg_out,
                                             zero_threshold_for_1bit);
+}
+
+int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduce_item* items, size_t count, size_t workers,
+                                    size_t owner, size_t nbits, int zero_threshold_for_1bit)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: null handle");
+    if (!valid_nbits(nbits))
+        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
+    if (workers == 0 || workers > CNTKQ_MAX_WORKERS || owner >= workers)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: need 1 <= workers <= %d and owner < workers",
+                    CNTKQ_MAX_WORKERS);
+    if (count == 0)
+        return CNTKQ_OK;
+    if (items == nullptr || count > 0xFFFFFF)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: bad item list");
+    size_t n = 0, only = 0;
+    for (size_t i = 0; i < count; ++i)
+    {
+        const cntkq_stripe_reduce_item& it = items[i];
+        if (it.rows >= (1ull << 31) || it.stripe_cols >= (1ull << 31))
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: rows and cols must be below 2^31", i);
+        if (it.rows == 0 || it.stripe_cols == 0)
+            continue;
+        if (it.rows > kTileMaxRows)
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: columns taller than %u rows are not supported", i,
+                        kTileMaxRows);
+        if (it.stripes == nullptr || it.stripe_res == nullptr || it.q_out == nullptr || !aligned4(it.stripe_res) || !aligned4(it.q_out) ||
+            !aligned4(it.agg_out))
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: null or misaligned pointer", i);
+        for (size_t w = 0; w < workers; ++w)
+            if (it.stripes[w] == nullptr || !aligned4(it.stripes[w]))
+                return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: stripe %zu is null or misaligned", i, w);
+        only = i;
+        n++;
+    }
+    if (n == 0)
+        return CNTKQ_OK;
+    if (n == 1) // a grid of its own is nothing to share: the plain call picks the best kernel for the stripe
+        return cntkq_stripe_reduce_async(h, items[only].stripes, workers, owner, items[only].rows, items[only].stripe_cols, nbits,
+                                         items[only].stripe_res, items[only].q_out, items[only].agg_out, zero_threshold_for_1bit);
+    const bool zt = zero_threshold_for_1bit != 0;
+    DeviceGuard guard(h->device);
+    hipStream_t s = work_stream(h);
+    BatchTable& tb = h->stripe_table;
+
+    // the key is the item list with the workers' stripe pointers written out
+    const size_t params[3] = {count, nbits | (workers << 8) | (owner << 16), (size_t) (zt ? 1 : 0)};
+    std::vector<size_t> flat;
+    flat.reserve(count * (5 + workers));
+    for (size_t i = 0; i < count; ++i)
+    {
+        const cntkq_stripe_reduce_item& it = items[i];
+        flat.push_back(reinterpret_cast<size_t>(it.stripe_res));
+        flat.push_back(reinterpret_cast<size_t>(it.q_out));
+        flat.push_back(reinterpret_cast<size_t>(it.agg_out));
+        flat.push_back(it.rows);
+        flat.push_back(it.stripe_cols);
+        if (it.rows != 0 && it.stripe_cols != 0)
+            for (size_t w = 0; w < workers; ++w)
+                flat.push_back(reinterpret_cast<size_t>(it.stripes[w]));
+    }
+    const size_t flat_bytes = flat.size() * sizeof(size_t);
+
+    if (!table_matches(tb, flat.data(), flat_bytes, params))
+    {
+        constexpr size_t kSmallLds = 20 * 1024;
+        const size_t entries_bytes = n * sizeof(StripeBatchEntry);
+        int rc = table_begin_rebuild(tb, entries_bytes + (n + 2) * sizeof(uint32_t) + 64);
+        if (rc != CNTKQ_OK)
+            return rc;
+        StripeBatchEntry* he = reinterpret_cast<StripeBatchEntry*>(tb.host);
+        uint32_t* hb = reinterpret_cast<uint32_t*>(tb.host + entries_bytes);
+        size_t e = 0, bpos = 0;
+        for (int cls = 0; cls < 2; ++cls)
+        {
+            tb.first_entry[cls] = e;
+            tb.first_begin[cls] = bpos;
+            tb.lds[cls] = 0;
+            tb.members[cls] = 0;
+            uint64_t acc = 0;
+            for (size_t i = 0; i < count; ++i)
+            {
+                const cntkq_stripe_reduce_item& it = items[i];
+                if (it.rows == 0 || it.stripe_cols == 0)
+                    continue;
+                // the kernel family the plain call would take, so that both give the same bytes
+                const bool col = stripe_auto_col(it.rows);
+                StripeBatchEntry en;
+                std::memset(&en, 0, sizeof en);
+                size_t lds, blocks;
+                if (col)
+                {
+                    en.kind = 1;
+                    en.c = make_col_geom(it.rows, nbits);
+                    lds = colg_lds_bytes_rt(en.c, nbits) + 2 * workers * sizeof(float);
+                    blocks = it.stripe_cols;
+                }
+                else
+                {
+                    en.kind = 0;
+                    en.t = make_tile_geom(it.rows, it.stripe_cols, nbits, 0, -1, 0);
+                    lds = tile_lds_bytes(en.t, (uint32_t) workers);
+                    blocks = (en.t.cols + en.t.cols_per_tile - 1) / en.t.cols_per_tile;
+                }
+                if ((lds <= kSmallLds ? 0 : 1) != cls)
+                    continue;
+                for (size_t w = 0; w < workers; ++w)
+                    en.src.q[w] = static_cast<const char*>(it.stripes[w]);
+                en.src.workers = (uint32_t) workers;
+                en.src.owner = (uint32_t) owner;
+                en.stripe_res = it.stripe_res;
+                en.q_out = static_cast<char*>(it.q_out);
+                en.agg_out = it.agg_out;
+                he[e] = en;
+                hb[bpos++] = (uint32_t) acc;
+                acc += blocks;
+                if (acc > 0x7FFFFFFFull)
+                    return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: too many workgroups in one batch");
+                if (lds > tb.lds[cls])
+                    tb.lds[cls] = lds;
+                tb.members[cls]++;
+                e++;
+            }
+            if (tb.members[cls] != 0)
+                hb[bpos++] = (uint32_t) acc; // sentinel
+            tb.blocks[cls] = (uint32_t) acc;
+        }
+        tb.entries_bytes = entries_bytes;
+        HIP_TRY(hipMemcpyAsync(tb.dev, tb.host, entries_bytes + bpos * sizeof(uint32_t), hipMemcpyHostToDevice, s),
+                "hipMemcpyAsync of the batch table failed");
+        table_set_key(tb, flat.data(), flat_bytes, params);
+    }
+    size_t launches_left = (tb.members[0] ? 1 : 0) + (tb.members[1] ? 1 : 0);
+    for (int cls = 0; cls < 2; ++cls)
+    {
+        if (tb.members[cls] == 0)
+            continue;
+        LaunchEvents ev;
+        launches_left--;
+        ev.stop = launches_left == 0 ? tb.event : nullptr;
+        const StripeBatchEntry* de = reinterpret_cast<const StripeBatchEntry*>(tb.dev) + tb.first_entry[cls];
+        const uint32_t* db = reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes) + tb.first_begin[cls];
+        HIP_TRY(launch_stripe_reduce_batch(s, ev, de, db, (uint32_t) tb.members[cls], tb.blocks[cls], tb.lds[cls], nbits, zt),
+                "batched stripe reduction kernel launch failed");
+        tb.in_flight = true;
+    }
+    h->last_stripe = tb.event;
+    return CNTKQ_OK;
 }
 
 int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h)

@@ -353,8 +353,8 @@ __device__ __forceinline__ uint32_t stripe_order(uint32_t n, uint32_t owner)
 }
 
 template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(StripeSources src, float* stripe_res,
-                                                                          char* q_out, float* agg_out, TileGeom t)
+__device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
+                                                        const TileGeom& t, uint32_t tile_index)
 {
     using PS = PackShape<NBITS>;
     constexpr uint32_t BATCH = 8; // packed words fetched together, so their latencies overlap
@@ -368,7 +368,7 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
     float* dec = smem + kTilePrefixFloats + t.tile_floats + t.words_floats;
 
     const uint32_t tid = threadIdx.x;
-    const uint32_t j0 = blockIdx.x * t.cols_per_tile;
+    const uint32_t j0 = tile_index * t.cols_per_tile;
     const uint32_t nc = min(t.cols_per_tile, t.cols - j0);
     const size_t base = (size_t) j0 * t.rows;
     const uint32_t K = src.workers;
@@ -465,6 +465,13 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(Stripe
     tile_pack<NBITS, ZT>(tile, hdr, words, t, nc, qtile, sp);
     if (t.stage_residual)
         tile_store(tile, mis_s, sp, total, t);
+}
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(StripeSources src, float* stripe_res,
+                                                                          char* q_out, float* agg_out, TileGeom t)
+{
+    stripe_reduce_tile_body<NBITS, ZT>(src, stripe_res, q_out, agg_out, t, blockIdx.x);
 }
 
 // ---- quantize, 1 bit, one workgroup per column, rows = 1024 * PER (PER = 1, 2, 4) ---------------------------
@@ -926,19 +933,18 @@ __global__ __launch_bounds__(kColThreads) void quantize_colg_kernel(const float*
 }
 
 template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kColThreads) void stripe_reduce_colg_kernel(StripeSources src, float* stripe_res, char* q_out,
-                                                                         float* agg_out, ColGeom c)
+__device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
+                                                        const ColGeom& c, uint32_t column, f32x4* smem)
 {
     using PS = PackShape<NBITS>;
     constexpr uint32_t T = kColThreads, BATCH = 8;
-    extern __shared__ f32x4 smem_v4[];
-    float* tile = reinterpret_cast<float*>(smem_v4);
+    float* tile = reinterpret_cast<float*>(smem);
     uint32_t* words = reinterpret_cast<uint32_t*>(tile + c.rows);
     float* red = tile + c.rows + (PS::CHUNKS > 1 ? c.nq : 0);
     float* dec = red + 12; // per worker, in summation order: 1 bit -> the two levels, else (ufactor, lower)
     const uint32_t tid = threadIdx.x;
-    const size_t base = (size_t) blockIdx.x * c.rows;
-    const size_t rec = (size_t) blockIdx.x * c.qcol;
+    const size_t base = (size_t) column * c.rows;
+    const size_t rec = (size_t) column * c.qcol;
     const uint32_t K = src.workers;
     if constexpr (PS::CHUNKS > 1)
         for (uint32_t x = tid; x < c.nq; x += T)
@@ -1022,6 +1028,14 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_colg_kernel(StripeS
     colg_stats_pack<NBITS, ZT>(tile, words, red, c, stat, stripe_res + base, q_out + rec);
 }
 
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kColThreads) void stripe_reduce_colg_kernel(StripeSources src, float* stripe_res, char* q_out,
+                                                                         float* agg_out, ColGeom c)
+{
+    extern __shared__ f32x4 smem_v4[];
+    stripe_reduce_colg_body<NBITS, ZT>(src, stripe_res, q_out, agg_out, c, blockIdx.x, smem_v4);
+}
+
 // Many matrices in one launch: the workgroups of all matrices form one grid; `begins` (count + 1 entries, ascending)
 // gives the first workgroup of every matrix. A matrix is a run of column tiles (quantize_tile_body) or of single columns
 // (quantize_colg_body). Removes the per-launch floor (several microseconds) that dominates gradient sets made of many
@@ -1055,6 +1069,39 @@ __global__ __launch_bounds__(kTileThreads) void quantize_batch_kernel(const Quan
     {
         const ColGeom c = entries[e].c;
         quantize_colg_body<NBITS, ZT>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, c, index, smem_v4);
+    }
+}
+
+// The owner's stripe reductions of a whole gradient set in one launch: same grid construction as quantize_batch_kernel.
+struct StripeBatchEntry
+{
+    StripeSources src;
+    float* stripe_res;
+    char* q_out;
+    float* agg_out;
+    uint32_t kind; // 0: tiles (t), 1: columns (c)
+    uint32_t pad;
+    TileGeom t;
+    ColGeom c;
+};
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTileThreads) void stripe_reduce_batch_kernel(const StripeBatchEntry* __restrict__ entries,
+                                                                           const uint32_t* __restrict__ begins, uint32_t count)
+{
+    extern __shared__ f32x4 smem_v4[];
+    const uint32_t e = batch_find(begins, count, blockIdx.x);
+    const uint32_t index = blockIdx.x - begins[e];
+    const StripeBatchEntry& en = entries[e]; // the table is read-only while the kernel runs
+    if (en.kind == 0)
+    {
+        const TileGeom t = en.t;
+        stripe_reduce_tile_body<NBITS, ZT>(en.src, en.stripe_res, en.q_out, en.agg_out, t, index);
+    }
+    else
+    {
+        const ColGeom c = en.c;
+        stripe_reduce_colg_body<NBITS, ZT>(en.src, en.stripe_res, en.q_out, en.agg_out, c, index, smem_v4);
     }
 }
 

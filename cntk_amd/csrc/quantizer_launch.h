@@ -450,6 +450,31 @@ inline hipError_t launch_quantize_batch(hipStream_t s, LaunchEvents ev, const Qu
     return dispatch_nbits<BatchLauncher>(nbits, zt, s, ev, entries, begins, count, total_blocks, lds);
 }
 
+template <int NBITS, bool ZT>
+struct StripeBatchLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeBatchEntry* entries, const uint32_t* begins, uint32_t count,
+                          uint32_t total_blocks, size_t lds)
+    {
+        hipExtLaunchKernelGGL((stripe_reduce_batch_kernel<NBITS, ZT>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start, ev.stop, 0,
+                              entries, begins, count);
+        return hipGetLastError();
+    }
+};
+
+inline hipError_t launch_stripe_reduce_batch(hipStream_t s, LaunchEvents ev, const StripeBatchEntry* entries, const uint32_t* begins,
+                                             uint32_t count, uint32_t total_blocks, size_t lds, size_t nbits, bool zt)
+{
+    zt = zt && (nbits == 1);
+    return dispatch_nbits<StripeBatchLauncher>(nbits, zt, s, ev, entries, begins, count, total_blocks, lds);
+}
+
+// which kernel family launch_stripe_reduce takes by itself for a stripe of this height: columns (true) or tiles
+inline bool stripe_auto_col(size_t rows)
+{
+    return rows % 4 == 0 && rows >= kColMinRows;
+}
+
 // colg_lds_bytes for a bit width known only at run time
 inline size_t colg_lds_bytes_rt(const ColGeom& c, size_t nbits)
 {

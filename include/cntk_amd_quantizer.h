@@ -166,6 +166,24 @@ int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, si
                               size_t rows, size_t stripe_cols, size_t nbits, float* stripe_res, void* q_out,
                               float* agg_out, int zero_threshold_for_1bit);
 
+/* The owner's stripe reductions for a whole gradient set (one item per gradient matrix) as one piece of stream work:
+ * the loop over the gradient matrices around the calls above (Source/1BitSGD/AllReduceDistGradAggregator.h:339-436 runs
+ * per matrix i). Same workers, owner, bit width and threshold mode for all items; results identical to
+ * cntkq_stripe_reduce_async item by item. items and the stripes arrays are host memory, read during the call only.
+ * cntkq_wait_stripe_reduce_done waits for the whole batch. */
+typedef struct cntkq_stripe_reduce_item
+{
+    const void* const* stripes; /* `workers` device pointers: worker w's packed stripe of this matrix */
+    float* stripe_res;          /* rows x stripe_cols, updated in place */
+    void* q_out;                /* packed stripe receiving the requantized aggregate; may be stripes[owner] */
+    float* agg_out;             /* optional (may be NULL) */
+    size_t rows;
+    size_t stripe_cols;
+} cntkq_stripe_reduce_item;
+
+int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduce_item* items, size_t count, size_t workers,
+                                    size_t owner, size_t nbits, int zero_threshold_for_1bit);
+
 /* Blocks until the last stripe reduction of this handle has finished (the reference waits on the stripe
  * quantizer's WaitQuantizeAsyncDone, Source/1BitSGD/AllReduceDistGradAggregator.h:494). */
 int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h);
