@@ -62,12 +62,23 @@ def cpu_baseline(budget_s=12.0):
 
     t1, p1 = run(1, budget_s)
     cores = min(16, os.cpu_count() or 1)
+    cpu_model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    cpu_model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
     tn, pn = run(cores, budget_s / 3)
     return {
         "value": round((qb + ub) / t1 / 1e9, 4),
         "unit": "GB/s",
         "cores": 1,
         "kind": "port",
+        "cpu_model": cpu_model,
+        "host_cpus": os.cpu_count(),
         "sample": "%d passes of quantize+unquantize over the full %dx%d fp32 matrix, 1 bit, best pass" % (p1, ROWS, COLS),
         "ms_per_step": round(t1 * 1e3, 2),
         "elements_per_s": round(ROWS * COLS / t1, 1),

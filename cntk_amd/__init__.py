@@ -74,6 +74,7 @@ def lib():
         L.cntkq_stream.restype = _vp
         L.cntkq_set_main_stream.argtypes = [_vp, _vp]
         L.cntkq_sync_with_main_stream.argtypes = [_vp]
+        L.cntkq_stream_wait_event.argtypes = [_vp, _vp]
         L.cntkq_quantize_async.argtypes = [_vp, _vp, _vp, _sz, _sz, _vp, _sz, ctypes.c_int, _sz, _vp, ctypes.c_int]
         L.cntkq_wait_quantize_done.argtypes = [_vp]
         L.cntkq_unquantize_async.argtypes = [_vp, _vp, _sz, ctypes.c_int, _vp, _sz, _sz, _sz, ctypes.c_int]
@@ -287,6 +288,11 @@ class MatrixQuantizerImpl:
         """MatrixComputeStreamEvent::SynchronizeQuantizationComputeStreamWithEvent
         (Source/Math/MatrixQuantizerGPU.cu:347-371)."""
         _check(lib().cntkq_sync_with_main_stream(self._h))
+
+    def WaitEvent(self, hip_event):
+        """Work issued through this quantizer from now on starts only after `hip_event` (a hipEvent_t as an integer,
+        e.g. torch.cuda.Event(...).cuda_event after record()) has completed."""
+        _check(lib().cntkq_stream_wait_event(self._h, hip_event))
 
     def QuantizeAsync(self, in_matrix, in_residual, out_qmatrix, out_residual, zero_threshold_for_1bit):
         rows, cols = in_matrix.GetNumRows(), in_matrix.GetNumCols()

@@ -615,6 +615,15 @@ int cntkq_sync_with_main_stream(cntkq_quantizer* h)
     return CNTKQ_OK;
 }
 
+int cntkq_stream_wait_event(cntkq_quantizer* h, void* hip_event)
+{
+    if (h == nullptr || hip_event == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stream_wait_event: null handle or event");
+    DeviceGuard guard(h->device);
+    HIP_TRY(hipStreamWaitEvent(work_stream(h), static_cast<hipEvent_t>(hip_event), 0), "hipStreamWaitEvent failed");
+    return CNTKQ_OK;
+}
+
 int cntkq_quantize_async(cntkq_quantizer* h, const float* in, const float* res_in, size_t rows, size_t cols, void* qbuf,
                          size_t qbuf_bytes, int qbuf_on_host, size_t nbits, float* res_out, int zero_threshold_for_1bit)
 {

@@ -87,6 +87,11 @@ int cntkq_set_main_stream(cntkq_quantizer* h, void* hip_stream);
  * handle's stream after this call starts only after everything already issued on the main stream. */
 int cntkq_sync_with_main_stream(cntkq_quantizer* h);
 
+/* The same hand-over for a caller that has its own event: work issued on the handle's stream after this call starts
+ * only after `hip_event` (a hipEvent_t recorded by the caller, on any stream of the device) has completed. This is what
+ * MatrixComputeStreamEvent does with its event (Source/Math/MatrixQuantizerGPU.cu:353-371). */
+int cntkq_stream_wait_event(cntkq_quantizer* h, void* hip_event);
+
 /* MatrixQuantizerImpl::QuantizeAsync (Source/Math/MatrixQuantizerImpl.h:30, Source/Math/MatrixQuantizerGPU.cu:226-269).
  *   in, res_in, res_out : device, rows x cols fp32; res_out may be the same pointer as res_in (in place),
  *                         no other overlap is allowed.

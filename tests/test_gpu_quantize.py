@@ -323,6 +323,30 @@ def test_error_behaviour(quantizer):
     assert quantizer.GetDeviceId() == 0
 
 
+def test_wait_event_orders_the_quantizer_stream():
+    """A dedicated-stream quantizer that is told to wait for the caller's event sees the data written before it."""
+    rows, cols = 2048, 256
+    q = MatrixQuantizerImpl.Create(0, True)
+    side = torch.cuda.Stream()
+    G, R, Q = Matrix(rows, cols), Matrix(rows, cols), QuantizedMatrix(rows, cols, 1, 0)
+    g = datagen.normal(21, rows, cols)
+    src = torch.from_numpy(g.reshape(-1, order="F").copy()).cuda()
+    torch.cuda.synchronize()
+    ev = torch.cuda.Event()
+    with torch.cuda.stream(side):
+        for _ in range(20):  # keep the side stream busy so that the copy really is pending when the quantizer is called
+            G.data.mul_(1.0)
+        G.data.copy_(src)
+        ev.record(side)
+    q.WaitEvent(ev.cuda_event)
+    q.QuantizeAsync(G, R, Q, R, False)
+    q.WaitQuantizeAsyncDone()
+    torch.cuda.synchronize()
+    parity.check_quantize(g, np.zeros_like(g, order="F"), Q.to_numpy(), R.to_numpy(), 1, False)
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        q.WaitEvent(None)
+
+
 def test_dedicated_stream_handles_share_one_stream():
     """Handles created with useAsync share one process-wide stream, so work issued through different quantizer
     objects is sequenced without waits -- callers rely on it (AllReduceDistGradAggregator.h:426-428)."""
