@@ -510,6 +510,22 @@ constexpr size_t col_lds_bytes()
     return (size_t) (1024 * PER + 32 * PER + 8 + 4) * 4;
 }
 
+// The 1-bit split sums of one 16-byte piece (x y z w in order): values below the mean go to s0 / n0, the others to s1.
+// Like the column sum, the split sums are taken piece by piece by every column kernel, whether it keeps the column in
+// LDS or in registers, so that all of them give the same header for the same column.
+__device__ __forceinline__ void split_add_piece(const f32x4& v, float mean, float& s0, float& s1, uint32_t& n0)
+{
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+    {
+        const float x = v[c];
+        const bool below = x < mean;
+        s0 += below ? x : 0.0f;
+        s1 += below ? 0.0f : x;
+        n0 += below ? 1u : 0u;
+    }
+}
+
 // Sum of the values thread tid holds when the column is cut into 16-byte pieces tid, tid + 256, ...: in that order,
 // x y z w within a piece. Both the quantize and the stripe-reduction kernel take the column mean from these
 // per-thread sums, so they produce identical headers for identical columns.
@@ -554,14 +570,11 @@ __device__ __forceinline__ void col_stats_pack(const ColLds& l, float csum, floa
     }
     float s0 = 0.0f, s1 = 0.0f;
     uint32_t n0 = 0;
-#pragma unroll
-    for (uint32_t i = 0; i < ROWS / T; ++i)
     {
-        const float x = l.tile[tid + T * i];
-        const bool below = x < mean;
-        s0 += below ? x : 0.0f;
-        s1 += below ? 0.0f : x;
-        n0 += below ? 1u : 0u;
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(l.tile);
+#pragma unroll
+        for (uint32_t u = 0; u < PER; ++u)
+            split_add_piece(t4[tid + T * u], mean, s0, s1, n0);
     }
     s0 = wave_sum(s0);
     s1 = wave_sum(s1);
@@ -794,14 +807,9 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
         const float mean = ZT ? 0.0f : total / (float) c.rows;
         float s0 = 0.0f, s1 = 0.0f;
         uint32_t n0 = 0;
-        for (uint32_t i = tid; i < c.rows; i += T)
-        {
-            const float x = tile[i];
-            const bool below = x < mean;
-            s0 += below ? x : 0.0f;
-            s1 += below ? 0.0f : x;
-            n0 += below ? 1u : 0u;
-        }
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
+        for (uint32_t p = tid; p < c.pieces; p += T)
+            split_add_piece(t4[p], mean, s0, s1, n0);
         s0 = wave_sum(s0);
         s1 = wave_sum(s1);
         n0 = wave_sum(n0);
@@ -1034,6 +1042,192 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_colg_kernel(StripeS
 {
     extern __shared__ f32x4 smem_v4[];
     stripe_reduce_colg_body<NBITS, ZT>(src, stripe_res, q_out, agg_out, c, blockIdx.x, smem_v4);
+}
+
+// ---- one workgroup per column, the column in registers ------------------------------------------------------
+//
+// Thread tid of T loads the 16-byte pieces tid, tid + T, ... (at most PER of them) of gradient and residual and keeps
+// their sum in registers through statistics, coding and the residual store; LDS holds only the column's QWords, which
+// the threads assemble with atomic OR (element i is bit position i / nq of QWord i % nq). With no column in LDS the
+// number of resident workgroups no longer falls with the column height. Statistics are summed in the piece order of
+// the LDS kernels above, so with T = 256 the bytes are theirs.
+
+struct RegGeom
+{
+    uint32_t rows;   // multiple of 4, at most 4 * T * PER
+    uint32_t nq;
+    uint32_t pieces; // rows / 4
+    uint32_t step_k; // (4 * T) / nq: a thread's next piece lies this many bit positions ...
+    uint32_t step_w; // (4 * T) % nq: ... and this many QWords further on
+    uint32_t pad;
+    uint64_t qcol;
+};
+
+constexpr uint32_t kRegRedSlots = 48; // three partial results for each of up to 16 waves
+
+__host__ __device__ inline size_t reg_lds_bytes(const RegGeom& c)
+{
+    return ((size_t) kRegRedSlots + c.nq) * 4;
+}
+
+// Waves per SIMD the register allocator is asked to keep possible: the column's 4 * PER registers, one batch of
+// residual pieces and about 40 more for addresses, statistics and coding.
+template <int T, int PER>
+constexpr int reg_waves()
+{
+    if (T == 1024)
+        return PER <= 4 ? 8 : 4; // a workgroup is 4 waves on every SIMD
+    int w = 512 / (4 * PER + 16 + 40);
+    return w > 8 ? 8 : w;
+}
+
+template <int NBITS, bool ZT, int T, int PER>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, PER>(), reg_waves<T, PER>()))) void quantize_reg_kernel(const float* __restrict__ g, const float* r_in, float* r_out,
+                                                         char* __restrict__ q, RegGeom c)
+{
+    using PS = PackShape<NBITS>;
+    static_assert(NBITS < 32, "32-bit codes are whole QWords: nothing to assemble");
+    constexpr uint32_t NW = T / 64;
+    extern __shared__ f32x4 smem_v4[];
+    float* red = reinterpret_cast<float*>(smem_v4);
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
+    uint32_t* words = reinterpret_cast<uint32_t*>(red + kRegRedSlots);
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const size_t base = (size_t) blockIdx.x * c.rows;
+    char* qc = q + (size_t) blockIdx.x * c.qcol;
+    for (uint32_t x = tid; x < c.nq; x += T)
+        words[x] = 0u;
+    const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base);
+    const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base);
+    f32x4 a[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+        if (tid + T * u < c.pieces)
+            a[u] = __builtin_nontemporal_load(g4 + tid + T * u);
+#pragma unroll
+    for (int u0 = 0; u0 < PER; u0 += 4)
+    {
+        f32x4 b[4];
+#pragma unroll
+        for (int u = u0; u < u0 + 4 && u < PER; ++u)
+            if (tid + T * u < c.pieces)
+                b[u - u0] = __builtin_nontemporal_load(r4 + tid + T * u);
+#pragma unroll
+        for (int u = u0; u < u0 + 4 && u < PER; ++u)
+            if (tid + T * u < c.pieces)
+                a[u] = a[u] + b[u - u0];
+    }
+    constexpr bool need_stat = (NBITS != 1) || !ZT;
+    float total = 0.0f;
+    if constexpr (need_stat)
+    {
+        float stat = 0.0f;
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            if (tid + T * u < c.pieces)
+                stat = colg_add_piece<NBITS>(stat, a[u]);
+        stat = wave_sum(stat);
+        if (lane == 0)
+            red[wave] = stat;
+    }
+    // the whole column has been read before this barrier, so r_out may be r_in
+    __syncthreads();
+    if constexpr (need_stat)
+    {
+        total = red[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+            total += red[x];
+    }
+    float lo, hi;
+    if constexpr (NBITS == 1)
+    {
+        const float mean = ZT ? 0.0f : total / (float) c.rows;
+        float s0 = 0.0f, s1 = 0.0f;
+        uint32_t n0 = 0;
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            if (tid + T * u < c.pieces)
+                split_add_piece(a[u], mean, s0, s1, n0);
+        s0 = wave_sum(s0);
+        s1 = wave_sum(s1);
+        n0 = wave_sum(n0);
+        __syncthreads(); // everyone has read the wave sums of the mean
+        if (lane == 0)
+        {
+            red[wave] = s0;
+            red[NW + wave] = s1;
+            red_u[wave] = n0;
+        }
+        __syncthreads();
+        float S0 = red[0], S1 = red[NW];
+        uint32_t N0 = red_u[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+        {
+            S0 += red[x];
+            S1 += red[NW + x];
+            N0 += red_u[x];
+        }
+        finish_stats_1bit<ZT>(mean, S0, S1, N0, c.rows - N0, c.rows, lo, hi);
+    }
+    else
+    {
+        finish_stats_multibit(total, c.rows, lo, hi);
+    }
+    if (tid == 0)
+    {
+        float* gh = reinterpret_cast<float*>(qc);
+        gh[0] = lo;
+        gh[1] = hi;
+    }
+    const ValueQ vq = make_vq<NBITS>(lo, hi);
+    const float val0 = unquantize_value<NBITS>(vq, 0u);
+    const float val1 = unquantize_value<NBITS>(vq, 1u);
+    f32x4* o4 = reinterpret_cast<f32x4*>(r_out + base);
+    // element 4 * tid is bit position k of QWord w; the following elements are the following QWords
+    uint32_t k = (4 * tid) / c.nq;
+    uint32_t w = 4 * tid - k * c.nq;
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+    {
+        const uint32_t p = tid + T * u;
+        if (p < c.pieces)
+        {
+            f32x4 res;
+            uint32_t kk = k, ww = w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+            {
+                const float v = a[u][e];
+                const uint32_t code = quantize_value<NBITS, ZT>(vq, v);
+                float back;
+                if constexpr (NBITS == 1)
+                    back = code ? val1 : val0;
+                else
+                    back = unquantize_value<NBITS>(vq, code);
+                res[e] = v - back;
+                atomicOr(&words[ww], code << (kk * PS::SHIFT));
+                if (++ww == c.nq)
+                {
+                    ww = 0;
+                    ++kk;
+                }
+            }
+            __builtin_nontemporal_store(res, o4 + p);
+        }
+        w += c.step_w;
+        k += c.step_k;
+        if (w >= c.nq)
+        {
+            w -= c.nq;
+            ++k;
+        }
+    }
+    __syncthreads();
+    uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
+    for (uint32_t x = tid; x < c.nq; x += T)
+        bits[x] = words[x];
 }
 
 // Many matrices in one launch: the workgroups of all matrices form one grid; `begins` (count + 1 entries, ascending)

@@ -19,7 +19,8 @@ enum QuantizePath
     kPathAuto = 0,
     kPathTile = 1,    // LDS-staged column tile (rows <= kTileMaxRows)
     kPathTall = 2,    // one workgroup per column, global re-read (any rows)
-    kPathCol = 3      // one workgroup per column, column in LDS: rows a multiple of 4, matrices 16-byte aligned
+    kPathCol = 3,     // one workgroup per column, column in LDS: rows a multiple of 4, matrices 16-byte aligned
+    kPathReg = 4      // one workgroup per column, column in registers: same conditions, 1 to 16 bits
 };
 
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
@@ -194,6 +195,59 @@ struct StripeColLauncher
     }
 };
 
+inline RegGeom make_reg_geom(size_t rows, size_t nbits, uint32_t threads)
+{
+    RegGeom c;
+    c.rows = (uint32_t) rows;
+    c.nq = (uint32_t) qwords_per_col(rows, nbits);
+    c.pieces = (uint32_t) (rows / 4);
+    c.step_k = (4 * threads) / c.nq;
+    c.step_w = (4 * threads) % c.nq;
+    c.pad = 0;
+    c.qcol = qcol_bytes(nbits, rows);
+    return c;
+}
+
+template <int NBITS, bool ZT, int T, int PER>
+inline hipError_t launch_reg_one(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
+                                 const RegGeom& c)
+{
+    hipExtLaunchKernelGGL((quantize_reg_kernel<NBITS, ZT, T, PER>), dim3(cols), dim3(T), reg_lds_bytes(c), s, ev.start, ev.stop, 0, g, r_in,
+                          r_out, q, c);
+    return hipGetLastError();
+}
+
+template <int NBITS, bool ZT>
+struct RegLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, RegGeom c,
+                          uint32_t threads)
+    {
+        if constexpr (NBITS >= 32)
+            return hipErrorInvalidValue;
+        else
+        {
+            const uint32_t per = (c.pieces + threads - 1) / threads;
+#define CNTKQ_REG(T, P) if (threads == T && per <= P) return launch_reg_one<NBITS, ZT, T, P>(s, ev, g, r_in, r_out, q, cols, c)
+            CNTKQ_REG(256, 6);
+            CNTKQ_REG(256, 8);
+            CNTKQ_REG(256, 10);
+            CNTKQ_REG(256, 12);
+            CNTKQ_REG(256, 14);
+            CNTKQ_REG(1024, 4);
+            CNTKQ_REG(1024, 6);
+            CNTKQ_REG(1024, 8);
+            CNTKQ_REG(1024, 10);
+            CNTKQ_REG(1024, 13);
+            CNTKQ_REG(1024, 16);
+            CNTKQ_REG(1024, 20);
+            CNTKQ_REG(1024, 25);
+#undef CNTKQ_REG
+            return hipErrorInvalidValue;
+        }
+    }
+};
+
 template <bool ZT, int PER>
 inline void launch_quantize_col(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
                                 uint64_t qcol)
@@ -210,6 +264,40 @@ inline void launch_stripe_col(hipStream_t s, LaunchEvents ev, const StripeSource
                           ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, qcol);
 }
 
+// The register kernels: taller than the unrolled LDS kernels' 4096 rows (unless forced), up to 25 pieces for each of
+// 1024 threads, the column's QWords within 64 KB of LDS. 256 threads up to the height the stripe reduction handles (whose
+// LDS kernels then sum in the same order), 1024 above.
+constexpr uint32_t kRegMinRows = 4096;
+constexpr uint32_t kRegMaxRows = 4 * 1024 * 25;
+
+inline uint32_t reg_threads(size_t rows)
+{
+    return rows <= kTileMaxRows ? 256u : 1024u;
+}
+
+inline bool reg_applicable(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits,
+                           bool forced = false)
+{
+    const uintptr_t m = reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(r_in) | reinterpret_cast<uintptr_t>(r_out);
+    if (rows % 4 != 0 || rows < 4 || rows > kRegMaxRows || nbits >= 32 || (m & 15u) != 0 || (reinterpret_cast<uintptr_t>(q) & 3u) != 0)
+        return false;
+    if (!forced && rows <= kRegMinRows)
+        return false;
+    return (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
+}
+
+// which path launch_quantize takes for this matrix when nothing is forced
+inline int quantize_auto_path(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
+{
+    if (reg_applicable(g, r_in, r_out, q, rows, nbits))
+        return kPathReg;
+    if (rows > kTileMaxRows)
+        return kPathTall;
+    if (col_applicable(g, r_in, r_out, q, rows, nbits))
+        return kPathCol;
+    return kPathTile;
+}
+
 // Launches the quantize kernel(s) for one matrix. rows, cols > 0; pointers 4-byte aligned (checked by caller).
 inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, void* q, size_t rows,
                                   size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
@@ -219,12 +307,14 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     int path = tune.quantize_path;
     if (path == kPathAuto)
     {
-        if (rows > kTileMaxRows)
-            path = kPathTall;
-        else if (col_applicable(g, r_in, r_out, q, rows, nbits))
-            path = kPathCol;
-        else
-            path = kPathTile;
+        path = quantize_auto_path(g, r_in, r_out, q, rows, nbits);
+    }
+    if (path == kPathReg)
+    {
+        if (!reg_applicable(g, r_in, r_out, q, rows, nbits, true))
+            return hipErrorInvalidValue;
+        const uint32_t threads = reg_threads(rows);
+        return dispatch_nbits<RegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, make_reg_geom(rows, nbits, threads), threads);
     }
     if (path == kPathCol)
     {
@@ -498,14 +588,5 @@ inline hipError_t launch_unquantize_batch(hipStream_t s, LaunchEvents ev, const 
     return hipGetLastError();
 }
 
-// which path launch_quantize would take for this matrix
-inline int quantize_auto_path(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
-{
-    if (rows > kTileMaxRows)
-        return kPathTall;
-    if (col_applicable(g, r_in, r_out, q, rows, nbits))
-        return kPathCol;
-    return kPathTile;
-}
 
 } // namespace cntkq

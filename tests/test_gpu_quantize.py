@@ -21,7 +21,7 @@ from cntk_amd import Matrix, MatrixQuantizerImpl, QuantizedMatrix
 pytestmark = pytest.mark.gpu
 
 VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False)]
-PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL = 0, 1, 2, 3
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG = 0, 1, 2, 3, 4
 
 
 def say(*a):
@@ -124,6 +124,10 @@ PATH_CASES = [
     (4, 3, PATH_COL, 0), (36, 70, PATH_COL, 0), (128, 9, PATH_COL, 0), (1000, 5, PATH_COL, 0), (1028, 7, PATH_COL, 0),
     (2048, 19, PATH_COL, 0), (2304, 5, PATH_COL, 0), (4100, 3, PATH_COL, 0), (9304, 2, PATH_COL, 0), (14336, 2, PATH_COL, 0),
     (9304, 3, PATH_AUTO, 0), (1152, 40, PATH_AUTO, 0), (100000, 2, PATH_AUTO, 0), (14340, 3, PATH_AUTO, 0),
+    # one workgroup per column, the column in registers: 256 threads up to 14336 rows, 1024 above
+    (4, 3, PATH_REG, 0), (36, 70, PATH_REG, 0), (1000, 5, PATH_REG, 0), (4100, 3, PATH_REG, 0), (6148, 5, PATH_REG, 0),
+    (9304, 2, PATH_REG, 0), (12292, 3, PATH_REG, 0), (14336, 2, PATH_REG, 0), (14340, 3, PATH_REG, 0), (20000, 3, PATH_REG, 0),
+    (40964, 2, PATH_REG, 0), (65540, 2, PATH_REG, 0), (102400, 1, PATH_REG, 0), (102404, 2, PATH_AUTO, 0),
 ]
 
 
@@ -134,6 +138,12 @@ def test_kernel_paths(case):
     rep = parity.Report()
     for nbits, zt in VARIANTS:
         say("path case", case, "nbits", nbits, "zeroThr", zt)
+        if path == PATH_REG and (nbits == 32 or (48 + oracle.qwords_per_col(rows, nbits)) * 4 > 65536):
+            # whole-QWord codes and columns whose QWords exceed 64 KB of LDS are not the register kernels' business
+            qz._set_tuning(quantize_path=path)
+            with pytest.raises(cntk_amd.QuantizerLogicError):
+                gpu_quantize(qz, datagen.normal(1, rows, cols), np.zeros((rows, cols), np.float32, order="F"), nbits, zt)
+            continue
         # alternate between the two ways a tile kernel writes its residual
         qz._set_tuning(quantize_path=path, tile_gs=gs, tile_stage=(nbits + rows) % 2 if path == PATH_TILE else -1)
         # a shifted mean, one all-zero column and outliers exercise every branch of the statistics
@@ -145,6 +155,27 @@ def test_kernel_paths(case):
             return a
         run_chain(qz, rows, cols, nbits, zt, make, 2, rep)
     say("  ", rep)
+
+
+@pytest.mark.parametrize("rows", [2048, 4100, 9304, 14336])
+def test_register_and_lds_column_kernels_give_the_same_bytes(rows):
+    """Up to 14336 rows the register kernels sum the column statistics in the order of the LDS kernels (which the
+    stripe reduction uses at these heights): packed bytes and residuals are identical for every bit width."""
+    qz = MatrixQuantizerImpl.Create(0, False)
+    cols = 5
+    g, r = datagen.normal_with_outliers(rows, rows, cols, 0.01), datagen.normal(rows + 1, rows, cols, 0.002)
+    for nbits, zt in VARIANTS:
+        if nbits == 32:
+            continue
+        say("register vs LDS column kernel", rows, nbits, zt)
+        qz._set_tuning(quantize_path=PATH_COL)
+        Qa, ra = gpu_quantize(qz, g, r, nbits, zt)
+        qz._set_tuning(quantize_path=PATH_REG)
+        Qb, rb = gpu_quantize(qz, g, r, nbits, zt)
+        assert np.array_equal(Qa.to_numpy(), Qb.to_numpy()) and parity.bits_equal(ra, rb)
+    # beyond 25 pieces for each of 1024 threads the forced path refuses
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        gpu_quantize(qz, datagen.normal(1, 102404, 1), np.zeros((102404, 1), np.float32, order="F"), 1, False)
 
 
 @pytest.mark.parametrize("rows", [1024, 2048, 4096])
