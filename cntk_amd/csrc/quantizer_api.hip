@@ -706,6 +706,7 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
         // tiles or of single columns; only columns too tall for LDS get a launch of their own. Large matrices gain
         // from sharing a grid too: their workgroups fill the gaps the others leave.
         constexpr size_t kSmallLds = 20 * 1024;
+        constexpr size_t kOwnLaunchElements = (size_t) 8 << 20;
         struct Plan
         {
             int kind; // -1 skip, 0 tiles in a batch, 1 columns in a batch, 2 own launch
@@ -733,8 +734,9 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
                 p.lds = tile_lds_bytes(p.t, 0);
                 p.blocks = (p.t.cols + p.t.cols_per_tile - 1) / p.t.cols_per_tile;
             }
-            else if (path == kPathCol)
+            else if (path == kPathCol || (path == kPathReg && it.rows <= kTileMaxRows && it.rows * it.cols < kOwnLaunchElements))
             {
+                // (a register-kernel matrix of modest size gives the same bytes as a member: a launch costs more than it gains)
                 p.kind = 1;
                 p.c = make_col_geom(it.rows, nbits);
                 p.lds = colg_lds_bytes_rt(p.c, nbits);

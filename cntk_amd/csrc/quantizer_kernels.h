@@ -1075,10 +1075,11 @@ __host__ __device__ inline size_t reg_lds_bytes(const RegGeom& c)
 template <int T, int PER>
 constexpr int reg_waves()
 {
-    if (T == 1024)
-        return PER <= 4 ? 8 : 4; // a workgroup is 4 waves on every SIMD
-    int w = 512 / (4 * PER + 16 + 40);
-    return w > 8 ? 8 : w;
+    // (a looser budget does not help: given 128 registers the compiler hoists work until it spills)
+    if (T == 1024 && PER <= 4)
+        return 8; // a workgroup is 4 waves on every SIMD: two of them fit
+    int w = 512 / (4 * PER + 40);
+    return w > 8 ? 8 : (w < T / 256 ? T / 256 : w);
 }
 
 template <int NBITS, bool ZT, int T, int PER>
@@ -1099,23 +1100,29 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
         words[x] = 0u;
     const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base);
     const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base);
+    // Branch-free loads: a thread whose piece lies beyond the column reads the column's last piece instead (and leaves
+    // it out of every sum and store), so that all loads are in flight together.
+    const uint32_t last = c.pieces - 1;
     f32x4 a[PER];
 #pragma unroll
     for (int u = 0; u < PER; ++u)
-        if (tid + T * u < c.pieces)
-            a[u] = __builtin_nontemporal_load(g4 + tid + T * u);
+    {
+        const uint32_t p = tid + T * u;
+        a[u] = __builtin_nontemporal_load(g4 + (p < c.pieces ? p : last));
+    }
 #pragma unroll
     for (int u0 = 0; u0 < PER; u0 += 4)
     {
         f32x4 b[4];
 #pragma unroll
         for (int u = u0; u < u0 + 4 && u < PER; ++u)
-            if (tid + T * u < c.pieces)
-                b[u - u0] = __builtin_nontemporal_load(r4 + tid + T * u);
+        {
+            const uint32_t p = tid + T * u;
+            b[u - u0] = __builtin_nontemporal_load(r4 + (p < c.pieces ? p : last));
+        }
 #pragma unroll
         for (int u = u0; u < u0 + 4 && u < PER; ++u)
-            if (tid + T * u < c.pieces)
-                a[u] = a[u] + b[u - u0];
+            a[u] = a[u] + b[u - u0];
     }
     constexpr bool need_stat = (NBITS != 1) || !ZT;
     float total = 0.0f;
@@ -1124,8 +1131,10 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
         float stat = 0.0f;
 #pragma unroll
         for (int u = 0; u < PER; ++u)
-            if (tid + T * u < c.pieces)
-                stat = colg_add_piece<NBITS>(stat, a[u]);
+        {
+            const float with = colg_add_piece<NBITS>(stat, a[u]);
+            stat = (tid + T * u < c.pieces) ? with : stat;
+        }
         stat = wave_sum(stat);
         if (lane == 0)
             red[wave] = stat;
@@ -1147,8 +1156,15 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
         uint32_t n0 = 0;
 #pragma unroll
         for (int u = 0; u < PER; ++u)
-            if (tid + T * u < c.pieces)
-                split_add_piece(a[u], mean, s0, s1, n0);
+        {
+            float t0 = s0, t1 = s1;
+            uint32_t tn = n0;
+            split_add_piece(a[u], mean, t0, t1, tn);
+            const bool valid = tid + T * u < c.pieces;
+            s0 = valid ? t0 : s0;
+            s1 = valid ? t1 : s1;
+            n0 = valid ? tn : n0;
+        }
         s0 = wave_sum(s0);
         s1 = wave_sum(s1);
         n0 = wave_sum(n0);
