@@ -906,6 +906,7 @@ int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item
             he[e].qw = p.qw;
             he[e].seg = p.seg;
             he[e].rowg = p.rowg;
+            he[e].tile = p.tile;
             if (p.lds > tb.lds[0])
                 tb.lds[0] = p.lds;
             hb[e] = (uint32_t) blocks;

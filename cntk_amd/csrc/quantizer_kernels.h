@@ -1701,13 +1701,134 @@ __global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __rest
     unquantize_rows_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint32_t*>(smem_v4));
 }
 
+// Tile decoder for short columns. Consecutive columns are adjacent in the packed matrix and in the output, so a
+// workgroup takes `cpt` columns at once: their packed records (one contiguous run) go to LDS in coalesced loads, each
+// column's decoding constants are computed once, and the cpt * rows values (one contiguous run) leave in aligned
+// 16-byte stores, four consecutive elements per thread and store, whatever the column height: a group of four may
+// straddle columns. cpt is a multiple of 4, so every tile starts on a 16-byte boundary of an aligned output.
+struct UnqTileGeom
+{
+    uint32_t rows;
+    uint32_t cols;
+    uint32_t nq;
+    uint32_t cpt;        // columns per workgroup
+    uint32_t rec_words;  // nq + 2: 32-bit words per packed record
+    uint32_t rows_magic; // ceil(2^32 / rows) (unused when rows == 1)
+    uint32_t nq_magic;   // ceil(2^32 / nq) (unused when nq == 1)
+    uint32_t blocks;
+};
+
+__host__ __device__ inline size_t unq_tile_lds_bytes(const UnqTileGeom& t)
+{
+    return (size_t) t.cpt * (t.rec_words + 2) * 4;
+}
+
+// x / d for x * d < 2^32 with magic = ceil(2^32 / d)
+__device__ __forceinline__ uint32_t small_div(uint32_t x, uint32_t d, uint32_t magic)
+{
+    return d == 1 ? x : __umulhi(x, magic);
+}
+
+template <int NBITS>
+__device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q, float* out, const UnqTileGeom& t, int add, uint32_t block,
+                                                     uint32_t* smem)
+{
+    constexpr uint32_t SHIFT = NBITS & 31;
+    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t col0 = block * t.cpt;
+    const uint32_t ncols = (t.cols - col0 < t.cpt) ? t.cols - col0 : t.cpt;
+    uint32_t* words = smem;                                          // ncols packed records
+    float* dec = reinterpret_cast<float*>(smem + t.cpt * t.rec_words); // per column: the two levels (1 bit) or (ufactor, lower)
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(q + (size_t) col0 * t.rec_words * 4);
+    const uint32_t total_words = ncols * t.rec_words;
+    for (uint32_t x = tid; x < total_words; x += 256)
+        words[x] = __builtin_nontemporal_load(src + x);
+    __syncthreads();
+    for (uint32_t c = tid; c < ncols; c += 256)
+    {
+        const float lo = __uint_as_float(words[c * t.rec_words]);
+        const float hi = __uint_as_float(words[c * t.rec_words + 1]);
+        const float uf = make_ufactor<NBITS>(lo, hi);
+        if constexpr (NBITS == 1)
+        {
+            dec[2 * c] = unquantize_value<NBITS>(uf, lo, 0u);
+            dec[2 * c + 1] = unquantize_value<NBITS>(uf, lo, 1u);
+        }
+        else
+        {
+            dec[2 * c] = uf;
+            dec[2 * c + 1] = lo;
+        }
+    }
+    __syncthreads();
+    const uint32_t elems = ncols * t.rows;
+    float* o = out + (size_t) col0 * t.rows;
+    for (uint32_t i = 4 * tid; i < elems; i += 1024)
+    {
+        uint32_t c = small_div(i, t.rows, t.rows_magic);
+        uint32_t r = i - c * t.rows;
+        uint32_t k = small_div(r, t.nq, t.nq_magic);
+        uint32_t w = r - k * t.nq;
+        const uint32_t* cw = words + c * t.rec_words + 2;
+        float d0 = dec[2 * c], d1 = dec[2 * c + 1];
+        f32x4 x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            // (past the end of the matrix c == ncols: the reads stay inside the LDS block and the value is not stored)
+            const uint32_t code = (cw[w] >> (k * SHIFT)) & CODEMASK;
+            if constexpr (NBITS == 1)
+                x[e] = code ? d1 : d0;
+            else
+                x[e] = unquantize_value<NBITS>(d0, d1, code);
+            ++r;
+            if (++w == t.nq)
+            {
+                w = 0;
+                ++k;
+            }
+            if (r == t.rows)
+            {
+                r = 0;
+                k = 0;
+                w = 0;
+                c = (c + 1 < t.cpt) ? c + 1 : c;
+                cw = words + c * t.rec_words + 2;
+                d0 = dec[2 * c];
+                d1 = dec[2 * c + 1];
+            }
+        }
+        if (i + 4 <= elems)
+        {
+            f32x4* o4 = reinterpret_cast<f32x4*>(o + i);
+            if (add)
+                x = x + *o4; // unquantized value + previous content
+            __builtin_nontemporal_store(x, o4);
+        }
+        else
+        {
+            for (uint32_t e = 0; i + e < elems; ++e)
+                o[i + e] = add ? x[e] + o[i + e] : x[e];
+        }
+    }
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_tile_kernel(const char* __restrict__ q, float* out, UnqTileGeom t, int add)
+{
+    extern __shared__ f32x4 smem_v4[];
+    unquantize_tile_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint32_t*>(smem_v4));
+}
+
 // Many matrices in one launch (see quantize_batch_kernel): the 256-thread blocks of all matrices form one grid.
 enum UnqKind : uint32_t
 {
     kUnqVec4 = 0,    // QWord-major, 16-byte stores
     kUnqScalar = 1,  // QWord-major, 4-byte stores
     kUnqSegment = 2, // segment decoder
-    kUnqRows = 3     // row-major decoder, packed column in LDS
+    kUnqRows = 3,    // row-major decoder, packed column in LDS
+    kUnqTile = 4     // several short columns per workgroup, packed records in LDS
 };
 
 struct UnquantizeBatchEntry
@@ -1719,6 +1840,7 @@ struct UnquantizeBatchEntry
     UnqGeom qw;      // valid for kUnqVec4 / kUnqScalar
     UnqSegGeom seg;  // valid for kUnqSegment
     UnqRowGeom rowg; // valid for kUnqRows
+    UnqTileGeom tile; // valid for kUnqTile
 };
 
 template <int NBITS>
@@ -1735,10 +1857,15 @@ __global__ __launch_bounds__(256) void unquantize_batch_kernel(const UnquantizeB
         unquantize_body<NBITS, 1>(en.q, en.out, en.qw, add, block);
     else if (en.kind == kUnqSegment)
         unquantize_segment_body<NBITS>(en.q, en.out, en.seg, add, block);
-    else
+    else if (en.kind == kUnqRows)
     {
         const UnqRowGeom t = en.rowg; // by value: the loop below stores between its uses
         unquantize_rows_body<NBITS>(en.q, en.out, t, add, block, reinterpret_cast<uint32_t*>(smem_v4));
+    }
+    else
+    {
+        const UnqTileGeom t = en.tile;
+        unquantize_tile_body<NBITS>(en.q, en.out, t, add, block, reinterpret_cast<uint32_t*>(smem_v4));
     }
 }
 

@@ -33,7 +33,7 @@ struct LaunchTuning
     int tile_stage = -1;    // -1 = automatic; 0 / 1 = residual written straight to memory / staged through LDS
     uint32_t tile_threads = 0; // 0 = automatic; else workgroup size of the tile kernels (64, 128, 256)
     uint32_t unq_slots = 0; // 0 = default; else bit positions per thread in unquantize
-    int unq_force_scalar = 0;
+    int unq_force_scalar = 0; // 0 automatic, 1 QWord-major with 4-byte stores, 2 / 4 tile / row-major decoder wherever it can run, 3 automatic without the tile decoder
 };
 
 // Events tied to the kernel dispatch itself (its completion signal), not recorded as separate stream
@@ -386,13 +386,17 @@ struct UnquantizePlan
     UnqGeom qw;
     UnqSegGeom seg;
     UnqRowGeom rowg;
+    UnqTileGeom tile;
     uint32_t blocks = 0; // 256-thread blocks
-    size_t lds = 0;      // dynamic LDS (kUnqRows only)
+    size_t lds = 0;      // dynamic LDS (kUnqRows, kUnqTile)
     bool ok = false;
 };
 
 constexpr size_t kUnqRowsMaxLds = 48 * 1024;
 constexpr uint32_t kUnqRowsChunk = 2048;
+constexpr size_t kUnqTileMaxRows = 4096;  // 4 columns of that height: 16384 elements, small enough for the magic divisions
+constexpr size_t kUnqTileElems = 4096;    // values per workgroup the tile decoder aims for
+constexpr size_t kUnqRowsMinRows = 1024;  // from this height on a column keeps the 256 threads of the row-major decoder busy
 
 inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t rows, size_t cols, size_t nbits,
                                       const LaunchTuning& tune)
@@ -403,12 +407,64 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
     std::memset(&p.rowg, 0, sizeof p.rowg);
     const size_t vpw = 32 / nbits;
     const size_t nq = qwords_per_col(rows, nbits);
+    std::memset(&p.tile, 0, sizeof p.tile);
+    const int mode = tune.unq_force_scalar;
     const bool out16 = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
-    const bool vec = !tune.unq_force_scalar && (nq % 4 == 0) && (rows % 4 == 0) && out16 &&
-                     (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
-    // columns of aligned height that the QWord-major decoder could only serve with 4-byte stores: row-major decoder
-    const bool rowmajor = !vec && !tune.unq_force_scalar && tune.unq_slots == 0 && out16 && rows % 4 == 0 && nq >= 32 &&
-                          nq * 4 <= kUnqRowsMaxLds;
+    const bool slots_free = tune.unq_slots == 0;
+    // QWord-major decoder with 16-byte stores. It is at its best when every bit position of a column is a run of whole
+    // 128-byte lines: QWords a multiple of 32, all of them full, columns starting on a line.
+    const bool vec_can = (nq % 4 == 0) && (rows % 4 == 0) && out16 && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
+    const bool vec_ideal = vec_can && nq % 32 == 0 && rows % 32 == 0 && rows * nbits == nq * 32;
+    const bool rows_can = slots_free && out16 && rows % 4 == 0 && nq >= 32 && nq * 4 <= kUnqRowsMaxLds;
+    const bool tile_can = slots_free && out16 && rows <= kUnqTileMaxRows;
+    bool vec = false, rowmajor = false, tile = false, seg_allowed = true;
+    if (mode == 1)
+        seg_allowed = false; // QWord-major, 4-byte stores
+    else if (mode == 2 && tile_can)
+        tile = true;
+    else if (mode == 4 && rows_can)
+        rowmajor = true;
+    else if (mode == 3 || !slots_free)
+    {
+        // the choice without the tile decoder
+        vec = vec_can;
+        rowmajor = !vec && rows_can;
+    }
+    else if (vec_ideal)
+        vec = true;
+    else if (rows_can && rows >= kUnqRowsMinRows)
+        rowmajor = true; // a column fills a workgroup
+    else if (tile_can)
+        tile = true;
+    else if (rows_can)
+        rowmajor = true;
+    else
+        vec = vec_can;
+    if (tile)
+    {
+        UnqTileGeom& t = p.tile;
+        t.rows = (uint32_t) rows;
+        t.cols = (uint32_t) cols;
+        t.nq = (uint32_t) nq;
+        size_t cpt = (kUnqTileElems / rows) & ~(size_t) 3;
+        if (cpt < 4)
+            cpt = 4;
+        t.cpt = (uint32_t) cpt;
+        t.rec_words = (uint32_t) nq + 2;
+        t.rows_magic = rows > 1 ? (uint32_t) ((((uint64_t) 1 << 32) + rows - 1) / rows) : 0u;
+        t.nq_magic = nq > 1 ? (uint32_t) ((((uint64_t) 1 << 32) + nq - 1) / nq) : 0u;
+        const uint64_t blocks = (cols + cpt - 1) / cpt;
+        if (blocks <= 0x7FFFFFFFull)
+        {
+            t.blocks = (uint32_t) blocks;
+            p.kind = kUnqTile;
+            p.blocks = t.blocks;
+            p.lds = unq_tile_lds_bytes(t);
+            p.ok = true;
+            return p;
+        }
+        vec = vec_can;
+    }
     if (rowmajor)
     {
         UnqRowGeom& t = p.rowg;
@@ -435,7 +491,7 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
         }
     }
     // other long columns that the QWord-major decoder could only serve with 4-byte stores go to the segment decoder
-    const bool seg = !vec && !tune.unq_force_scalar && out16 && nq >= 32;
+    const bool seg = !vec && seg_allowed && out16 && nq >= 32;
     if (seg)
     {
         UnqSegGeom& t = p.seg;
@@ -485,7 +541,9 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
 template <int NBITS>
 inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const char* q, float* out, const UnquantizePlan& p, int add)
 {
-    if (p.kind == kUnqRows)
+    if (p.kind == kUnqTile)
+        hipExtLaunchKernelGGL((unquantize_tile_kernel<NBITS>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.tile, add);
+    else if (p.kind == kUnqRows)
         hipExtLaunchKernelGGL((unquantize_rows_kernel<NBITS>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.rowg, add);
     else if (p.kind == kUnqSegment)
         hipExtLaunchKernelGGL((unquantize_segment_kernel<NBITS>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.seg, add);

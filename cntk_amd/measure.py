@@ -33,6 +33,7 @@ def main():
     ap.add_argument("--steps", type=int, default=40)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--path", type=int, default=0, help="force a quantize kernel: 1 tile, 2 tall, 3 workgroup-per-column")
+    ap.add_argument("--unq-mode", type=int, default=0, help="decoder choice: 0 automatic, 1 scalar, 2 tile decoder, 3 automatic without it")
     ap.add_argument("--budget-mb", type=int, default=1600, help="device memory for the rotating buffer sets")
     args = ap.parse_args()
 
@@ -43,7 +44,7 @@ def main():
     sfx = "_f64" if args.dtype == "f64" else ""
     L = cntk_amd.lib()
     qz = MatrixQuantizerImpl.Create(0, False)
-    qz._set_tuning(quantize_path=args.path)
+    qz._set_tuning(quantize_path=args.path, unq_force_scalar=args.unq_mode)
     h = qz._h
 
     elems = rows * cols

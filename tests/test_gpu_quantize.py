@@ -250,6 +250,40 @@ def test_unquantize_variants(quantizer):
                         parity.check_unquantize(q, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
 
 
+TILE_DECODER_SHAPES = [(1, 1), (1, 9), (2, 7), (3, 5), (5, 3), (31, 13), (32, 8), (33, 41), (64, 100), (147, 64), (256, 1031),
+                       (429, 37), (512, 24), (1000, 9), (1001, 5), (1024, 3), (2047, 2), (2048, 7), (4096, 5), (4095, 3)]
+
+
+@pytest.mark.parametrize("shape", TILE_DECODER_SHAPES, ids=["%dx%d" % s for s in TILE_DECODER_SHAPES])
+def test_tile_decoder(shape):
+    """The decoder that takes several short columns per workgroup: forced on every height it accepts (groups of four
+    values that straddle columns, matrices whose size is not a multiple of four, a last tile with fewer columns), and
+    as the automatic choice; add and overwrite; bit-exact. A misaligned output falls back to another decoder."""
+    rows, cols = shape
+    for nbits, zt in VARIANTS:
+        g = datagen.normal_with_outliers(rows * 11 + nbits, rows, cols, 0.01)
+        q, _ = oracle.quantize(g, np.zeros_like(g, order="F"), nbits, zt)
+        prev = datagen.normal(rows * 13 + nbits, rows, cols, 1.0)
+        for mode in (2, 0, 3):
+            say("tile decoder", rows, cols, nbits, "mode", mode)
+            qz = MatrixQuantizerImpl.Create(0, False)
+            qz._set_tuning(unq_force_scalar=mode)
+            Q = QuantizedMatrix(rows, cols, nbits, 0)
+            Q.from_numpy(q)
+            for add in (False, True):
+                Out = Matrix.from_numpy(prev)
+                qz.UnquantizeAsync(Q, Out, add=add)
+                qz.WaitUnquantizeAsyncDone()
+                parity.check_unquantize(q, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
+        # output 4 bytes off a 16-byte boundary
+        big = torch.zeros(rows * cols + 4, dtype=torch.float32, device="cuda:0")
+        Out = Matrix(rows, cols, 0, big[1:1 + rows * cols])
+        qz.UnquantizeAsync(Q, Out)
+        qz.WaitUnquantizeAsyncDone()
+        parity.check_unquantize(q, rows, cols, nbits, Out.to_numpy())
+        assert float(big[0]) == 0.0 and float(big[-1]) == 0.0 and float(big[-2]) == 0.0 and float(big[-3]) == 0.0
+
+
 # ---- boundary behaviour ------------------------------------------------------------------------------
 
 
