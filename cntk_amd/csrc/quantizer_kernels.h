@@ -1649,8 +1649,27 @@ __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q,
     const float lo = gh[0];
     const float uf = make_ufactor<NBITS>(lo, gh[1]);
     const uint32_t* bits = reinterpret_cast<const uint32_t*>(qc + 8);
-    for (uint32_t w = tid; w < t.nq; w += 256)
-        words[w] = bits[w];
+    if (t.nq <= 1024)
+    {
+        for (uint32_t w = tid; w < t.nq; w += 256)
+            words[w] = bits[w];
+    }
+    else
+    {
+        // eight loads in flight per thread: a tall column has thousands of QWords, and one round trip for every 256 of
+        // them would cost more than the decoding
+        for (uint32_t w = tid; w < t.nq; w += 8 * 256)
+        {
+            uint32_t v[8];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u)
+                v[u] = bits[(w + 256 * u < t.nq) ? w + 256 * u : w];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u)
+                if (w + 256 * u < t.nq)
+                    words[w + 256 * u] = v[u];
+        }
+    }
     __syncthreads();
     const uint32_t r0 = ch * t.chunk;
     const uint32_t pieces = ((ch + 1 == t.chunks ? t.rows : r0 + t.chunk) - r0) >> 2; // the last chunk runs to the end

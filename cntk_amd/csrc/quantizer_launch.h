@@ -470,9 +470,11 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
         UnqRowGeom& t = p.rowg;
         t.rows = (uint32_t) rows;
         t.nq = (uint32_t) nq;
-        // small chunks keep many workgroups in flight; a chunk still spans at least four bit positions so that copying
-        // the packed column into LDS stays a small part of the work
-        size_t chunk = ((4 * nq + 1023) / 1024) * 1024;
+        // small chunks keep many workgroups in flight; a chunk still spans several bit positions so that copying the
+        // packed column into LDS stays a small part of the work
+        // (columns of more than 1024 QWords did best with two bit positions, shorter ones with four)
+        const size_t mult = nq > 1024 ? 2 : 4;
+        size_t chunk = ((mult * nq + 1023) / 1024) * 1024;
         if (chunk < kUnqRowsChunk)
             chunk = kUnqRowsChunk;
         t.chunk = (uint32_t) chunk;
