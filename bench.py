@@ -48,19 +48,23 @@ def cpu_baseline(budget_s=12.0):
     out = np.zeros_like(g, order="F")
     qb, ub = algorithmic_bytes(ROWS, COLS, NBITS)
 
-    def run(threads, budget):
+    def run(threads, budget, use_ref=False):
         best = float("inf")
         passes = 0
         t_end = time.perf_counter() + budget
         while passes < 3 or (time.perf_counter() < t_end and passes < 40):
             t0 = time.perf_counter()
-            q, _ = oracle.quantize(g, r, NBITS, False, r_out=r, threads=threads)
-            oracle.unquantize(q, ROWS, COLS, NBITS, out=out, threads=threads)
+            q, _ = oracle.quantize(g, r, NBITS, False, r_out=r, threads=threads, use_ref=use_ref)
+            oracle.unquantize(q, ROWS, COLS, NBITS, out=out, threads=threads, use_ref=use_ref)
             best = min(best, time.perf_counter() - t0)
             passes += 1
         return best, passes
 
-    t1, p1 = run(1, budget_s)
+    # the reference's own CPU quantizer (its headers, compiled under oracle/_ref) where that build is present; it is
+    # single-threaded, like the reference's CPU path
+    have_ref = oracle.ref_available()
+    t1, p1 = run(1, budget_s if not have_ref else budget_s / 2)
+    tr, pr = run(1, budget_s / 2, use_ref=True) if have_ref else (None, 0)
     cores = min(16, os.cpu_count() or 1)
     cpu_model = ""
     try:
@@ -72,17 +76,19 @@ def cpu_baseline(budget_s=12.0):
     except OSError:
         pass
     tn, pn = run(cores, budget_s / 3)
+    tb = tr if have_ref else t1
     return {
-        "value": round((qb + ub) / t1 / 1e9, 4),
+        "value": round((qb + ub) / tb / 1e9, 4),
         "unit": "GB/s",
         "cores": 1,
-        "kind": "port",
+        "kind": "reference" if have_ref else "port",
+        "port": {"cores": 1, "value": round((qb + ub) / t1 / 1e9, 4), "ms_per_step": round(t1 * 1e3, 2), "passes": p1},
         "cpu_model": cpu_model,
         "host_cpus": os.cpu_count(),
-        "sample": "%d passes of quantize+unquantize over the full %dx%d fp32 matrix, 1 bit, best pass" % (p1, ROWS, COLS),
-        "ms_per_step": round(t1 * 1e3, 2),
-        "elements_per_s": round(ROWS * COLS / t1, 1),
-        "all_cores": {"cores": cores, "value": round((qb + ub) / tn / 1e9, 4), "ms_per_step": round(tn * 1e3, 2),
+        "sample": "%d passes of quantize+unquantize over the full %dx%d fp32 matrix, 1 bit, best pass" % (pr if have_ref else p1, ROWS, COLS),
+        "ms_per_step": round(tb * 1e3, 2),
+        "elements_per_s": round(ROWS * COLS / tb, 1),
+        "port_all_cores": {"cores": cores, "value": round((qb + ub) / tn / 1e9, 4), "ms_per_step": round(tn * 1e3, 2),
                       "passes": pn},
     }
 
