@@ -37,7 +37,7 @@ def build_library(verbose=False):
     return LIB_PATH
 
 
-CPP_TESTS = ["test_matrix_quantizer", "test_allreduce_aggregator", "bench_allreduce"]
+CPP_TESTS = ["test_matrix_quantizer", "test_allreduce_aggregator", "test_distributed_learner", "bench_allreduce"]
 
 
 def build_cpp_tests(verbose=False):

@@ -36,6 +36,19 @@ def test_cpp_allreduce_aggregator_suite():
 
 
 @pytest.mark.gpu
+def test_cpp_distributed_learner_suite():
+    """The learner glue (cntk_amd/cpp/QuantizedDataParallelDistributedLearner.h) with K in-process ranks."""
+    exe = os.path.join(ROOT, "tests", "cpp", "bin", "test_distributed_learner")
+    assert os.path.exists(exe), "build it first: python -m cntk_amd.build"
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    print(res.stdout)
+    print(res.stderr[-4000:])
+    assert res.returncode == 0, "C++ distributed learner tests failed"
+    for name in ("WarmStartThenExactSum", "OneBitUidOrderEmptyAndCheckpoint"):
+        assert "DistributedLearner%s has passed" % name in res.stdout
+
+
+@pytest.mark.gpu
 def test_cpp_allreduce_timing_program_runs():
     """The all-reduce timing program on a small shape (its full-size numbers are quoted in the design notes)."""
     exe = os.path.join(ROOT, "tests", "cpp", "bin", "bench_allreduce")
