@@ -738,7 +738,7 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
             {
                 // (a register-kernel matrix of modest size gives the same bytes as a member: a launch costs more than it gains)
                 p.kind = 1;
-                p.c = make_col_geom(it.rows, nbits);
+                p.c = make_col_geom(it.rows, nbits, quantize_line_shift(it.in, it.res_in, it.res_out, it.rows));
                 p.lds = colg_lds_bytes_rt(p.c, nbits);
                 p.blocks = it.cols;
             }
@@ -1042,7 +1042,7 @@ int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduc
                 if (col)
                 {
                     en.kind = 1;
-                    en.c = make_col_geom(it.rows, nbits);
+                    en.c = make_col_geom(it.rows, nbits, !columns_start_on_lines(it.stripe_res, it.rows));
                     lds = colg_lds_bytes_rt(en.c, nbits) + 2 * workers * sizeof(float);
                     blocks = it.stripe_cols;
                 }

@@ -740,11 +740,32 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSo
 // otherwise) is taken piece by piece while loading, in the order col_thread_sum defines, so for 1 bit and 1024 * PER
 // rows these kernels give the very bytes of the unrolled ones above.
 
+// How a column's 16-byte pieces are dealt to the slots of a workgroup (slot v = thread + T * u). With line_shift set,
+// slot v holds piece v - shift, shift = the column's offset into its 128-byte line in pieces (the residual input's
+// address decides; the launch sets line_shift only when gradient and residual output share that offset).
+__device__ __forceinline__ uint32_t column_shift(const float* column, uint32_t line_shift)
+{
+    return line_shift ? (uint32_t) ((reinterpret_cast<uintptr_t>(column) >> 4) & 7u) : 0u;
+}
+
+__device__ __forceinline__ bool slot_valid(uint32_t v, uint32_t shift, uint32_t pieces)
+{
+    return v >= shift && v - shift < pieces;
+}
+
+// the piece a slot loads: its own, or (outside the column) the column's first or last
+__device__ __forceinline__ uint32_t slot_piece(uint32_t v, uint32_t shift, uint32_t last)
+{
+    const uint32_t p = v < shift ? 0u : v - shift;
+    return p < last ? p : last;
+}
+
 struct ColGeom
 {
     uint32_t rows;   // multiple of 4
     uint32_t nq;
     uint32_t pieces; // rows / 4
+    uint32_t line_shift; // non-zero: statistics are summed in the order of line-aligned slots (see column_shift)
     uint64_t qcol;
 };
 
@@ -779,7 +800,7 @@ __device__ __forceinline__ float colg_add_piece(float s, const f32x4& v)
 // partial QWords, red = 12 reduction slots. No barrier is needed between writing the column and calling this.
 template <int NBITS, bool ZT>
 __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, float* red, const ColGeom& c, float stat,
-                                                float* res_col, char* qc)
+                                                uint32_t shift, float* res_col, char* qc)
 {
     using PS = PackShape<NBITS>;
     constexpr uint32_t T = kColThreads, NW = T / 64;
@@ -808,8 +829,9 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
         float s0 = 0.0f, s1 = 0.0f;
         uint32_t n0 = 0;
         const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
-        for (uint32_t p = tid; p < c.pieces; p += T)
-            split_add_piece(t4[p], mean, s0, s1, n0);
+        for (uint32_t v = tid; v < c.pieces + shift; v += T)
+            if (v >= shift)
+                split_add_piece(t4[v - shift], mean, s0, s1, n0);
         s0 = wave_sum(s0);
         s1 = wave_sum(s1);
         n0 = wave_sum(n0);
@@ -903,33 +925,36 @@ __device__ __forceinline__ void quantize_colg_body(const float* __restrict__ g, 
     const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base);
     f32x4* t4 = reinterpret_cast<f32x4*>(tile);
     float stat = 0.0f;
-    for (uint32_t p0 = tid; p0 < c.pieces; p0 += 4 * T)
+    // slot v holds piece v - shift (see column_shift): the order the register kernels sum in, and whole lines per wavefront
+    const uint32_t shift = column_shift(r_in + base, c.line_shift);
+    const uint32_t slots = c.pieces + shift;
+    for (uint32_t v0 = tid; v0 < slots; v0 += 4 * T)
     {
         f32x4 a[4], b[4];
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u)
         {
-            const uint32_t p = p0 + u * T;
-            if (p < c.pieces)
+            const uint32_t v = v0 + u * T;
+            if (v >= shift && v < slots)
             {
-                a[u] = __builtin_nontemporal_load(g4 + p);
-                b[u] = __builtin_nontemporal_load(r4 + p);
+                a[u] = __builtin_nontemporal_load(g4 + (v - shift));
+                b[u] = __builtin_nontemporal_load(r4 + (v - shift));
             }
         }
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u)
         {
-            const uint32_t p = p0 + u * T;
-            if (p < c.pieces)
+            const uint32_t v = v0 + u * T;
+            if (v >= shift && v < slots)
             {
-                const f32x4 v = a[u] + b[u];
-                t4[p] = v;
-                stat = colg_add_piece<NBITS>(stat, v);
+                const f32x4 x = a[u] + b[u];
+                t4[v - shift] = x;
+                stat = colg_add_piece<NBITS>(stat, x);
             }
         }
     }
     // the whole column has been read before the first barrier of colg_stats_pack, so r_out may be r_in
-    colg_stats_pack<NBITS, ZT>(tile, words, red, c, stat, r_out + base, q + (size_t) column * c.qcol);
+    colg_stats_pack<NBITS, ZT>(tile, words, red, c, stat, shift, r_out + base, q + (size_t) column * c.qcol);
 }
 
 template <int NBITS, bool ZT>
@@ -1026,14 +1051,17 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
         }
     }
     float stat = 0.0f;
+    // the quantize kernels' summation order for a residual at this address
+    const uint32_t shift = column_shift(stripe_res + base, c.line_shift);
     if constexpr ((NBITS != 1) || !ZT)
     {
         __syncthreads();
         const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
-        for (uint32_t p = tid; p < c.pieces; p += T)
-            stat = colg_add_piece<NBITS>(stat, t4[p]);
+        for (uint32_t v = tid; v < c.pieces + shift; v += T)
+            if (v >= shift)
+                stat = colg_add_piece<NBITS>(stat, t4[v - shift]);
     }
-    colg_stats_pack<NBITS, ZT>(tile, words, red, c, stat, stripe_res + base, q_out + rec);
+    colg_stats_pack<NBITS, ZT>(tile, words, red, c, stat, shift, stripe_res + base, q_out + rec);
 }
 
 template <int NBITS, bool ZT>
@@ -1059,11 +1087,12 @@ struct RegGeom
     uint32_t pieces; // rows / 4
     uint32_t step_k; // (4 * T) / nq: a thread's next piece lies this many bit positions ...
     uint32_t step_w; // (4 * T) % nq: ... and this many QWords further on
-    uint32_t pad;
+    uint32_t line_shift; // non-zero: slots are dealt so that wavefronts cover whole 128-byte lines (see column_shift)
     uint64_t qcol;
 };
 
-constexpr uint32_t kRegRedSlots = 48; // three partial results for each of up to 16 waves
+constexpr uint32_t kRegRedSlots = 48;
+constexpr int kRegMaxShiftPer = 16; // most pieces per thread of a register kernel that deals its slots by lines // three partial results for each of up to 16 waves
 
 __host__ __device__ inline size_t reg_lds_bytes(const RegGeom& c)
 {
@@ -1076,15 +1105,15 @@ template <int T, int PER>
 constexpr int reg_waves()
 {
     // (a looser budget does not help: given 128 registers the compiler hoists work until it spills)
-    if (T == 1024 && PER <= 4)
-        return 8; // a workgroup is 4 waves on every SIMD: two of them fit
-    int w = 512 / (4 * PER + 40);
+    if (T == 1024)
+        return PER <= 6 ? 8 : 4; // a workgroup is 4 waves on every SIMD: two of them fit, or one
+    int w = 512 / (4 * PER + (PER >= 10 ? 48 : 40));
     return w > 8 ? 8 : (w < T / 256 ? T / 256 : w);
 }
 
 template <int NBITS, bool ZT, int T, int PER>
-__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, PER>(), reg_waves<T, PER>()))) void quantize_reg_kernel(const float* __restrict__ g, const float* r_in, float* r_out,
-                                                         char* __restrict__ q, RegGeom c)
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, PER>(), reg_waves<T, PER>()))) void quantize_reg_kernel(
+    const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q, RegGeom c)
 {
     using PS = PackShape<NBITS>;
     static_assert(NBITS < 32, "32-bit codes are whole QWords: nothing to assemble");
@@ -1100,26 +1129,24 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
         words[x] = 0u;
     const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base);
     const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base);
-    // Branch-free loads: a thread whose piece lies beyond the column reads the column's last piece instead (and leaves
-    // it out of every sum and store), so that all loads are in flight together.
+    // Slot v = tid + T * u holds piece v - shift, where shift (0..7) is the column's offset into its 128-byte line in
+    // pieces: every wavefront's 64 slots then cover whole lines, also in columns that start inside a line (9304 rows: every
+    // column but each fourth). Slots before the column or past its end read a piece of the column all the same (no
+    // branch, all loads in flight together) and are left out of every sum and store.
+    // (not with more than 16 pieces per thread: there the registers are needed for the column itself)
+    const uint32_t shift = PER <= kRegMaxShiftPer ? column_shift(r_in + base, c.line_shift) : 0u;
     const uint32_t last = c.pieces - 1;
     f32x4 a[PER];
 #pragma unroll
     for (int u = 0; u < PER; ++u)
-    {
-        const uint32_t p = tid + T * u;
-        a[u] = __builtin_nontemporal_load(g4 + (p < c.pieces ? p : last));
-    }
+        a[u] = __builtin_nontemporal_load(g4 + slot_piece(tid + T * u, shift, last));
 #pragma unroll
     for (int u0 = 0; u0 < PER; u0 += 4)
     {
         f32x4 b[4];
 #pragma unroll
         for (int u = u0; u < u0 + 4 && u < PER; ++u)
-        {
-            const uint32_t p = tid + T * u;
-            b[u - u0] = __builtin_nontemporal_load(r4 + (p < c.pieces ? p : last));
-        }
+            b[u - u0] = __builtin_nontemporal_load(r4 + slot_piece(tid + T * u, shift, last));
 #pragma unroll
         for (int u = u0; u < u0 + 4 && u < PER; ++u)
             a[u] = a[u] + b[u - u0];
@@ -1133,7 +1160,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
         for (int u = 0; u < PER; ++u)
         {
             const float with = colg_add_piece<NBITS>(stat, a[u]);
-            stat = (tid + T * u < c.pieces) ? with : stat;
+            stat = slot_valid(tid + T * u, shift, c.pieces) ? with : stat;
         }
         stat = wave_sum(stat);
         if (lane == 0)
@@ -1160,7 +1187,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
             float t0 = s0, t1 = s1;
             uint32_t tn = n0;
             split_add_piece(a[u], mean, t0, t1, tn);
-            const bool valid = tid + T * u < c.pieces;
+            const bool valid = slot_valid(tid + T * u, shift, c.pieces);
             s0 = valid ? t0 : s0;
             s1 = valid ? t1 : s1;
             n0 = valid ? tn : n0;
@@ -1201,14 +1228,17 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     const float val0 = unquantize_value<NBITS>(vq, 0u);
     const float val1 = unquantize_value<NBITS>(vq, 1u);
     f32x4* o4 = reinterpret_cast<f32x4*>(r_out + base);
-    // element 4 * tid is bit position k of QWord w; the following elements are the following QWords
-    uint32_t k = (4 * tid) / c.nq;
-    uint32_t w = 4 * tid - k * c.nq;
+    // the first element of this thread's first slot inside the column is bit position k of QWord w; the elements after it
+    // are the following QWords, the slots after it lie 4 * T elements further on
+    const uint32_t ufirst = tid < shift ? 1u : 0u;
+    const uint32_t e0 = 4 * (tid + T * ufirst - shift);
+    uint32_t k = e0 / c.nq;
+    uint32_t w = e0 - k * c.nq;
 #pragma unroll
     for (int u = 0; u < PER; ++u)
     {
-        const uint32_t p = tid + T * u;
-        if (p < c.pieces)
+        const uint32_t p = tid + T * u - shift;
+        if (slot_valid(tid + T * u, shift, c.pieces))
         {
             f32x4 res;
             uint32_t kk = k, ww = w;
@@ -1232,12 +1262,15 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
             }
             __builtin_nontemporal_store(res, o4 + p);
         }
-        w += c.step_w;
-        k += c.step_k;
-        if (w >= c.nq)
+        if ((uint32_t) u >= ufirst)
         {
-            w -= c.nq;
-            ++k;
+            w += c.step_w;
+            k += c.step_k;
+            if (w >= c.nq)
+            {
+                w -= c.nq;
+                ++k;
+            }
         }
     }
     __syncthreads();
@@ -1676,13 +1709,17 @@ __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q,
     f32x4* o4 = reinterpret_cast<f32x4*>(out + (size_t) c * t.rows + r0);
     const float val0 = unquantize_value<NBITS>(uf, lo, 0u);
     const float val1 = unquantize_value<NBITS>(uf, lo, 1u);
+    // Slot v = tid, tid + 256, ... holds piece v - shift, shift = the chunk's offset into its 128-byte line in pieces, so
+    // that every wavefront's 64 stores cover whole lines also where columns do not start on one (9304 rows).
+    const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o4) >> 4) & 7u);
+    const uint32_t vfirst = tid < shift ? tid + 256 : tid;
     // row i sits in QWord i % nq at bit position i / nq; a thread's pieces are 1024 rows apart
-    const uint32_t i0 = r0 + 4 * tid;
+    const uint32_t i0 = r0 + 4 * (vfirst - shift);
     uint32_t k0 = i0 / t.nq;
     uint32_t w0 = i0 - k0 * t.nq;
     const uint32_t dk = 1024u / t.nq;
     const uint32_t dw = 1024u - dk * t.nq;
-    for (uint32_t p = tid; p < pieces; p += 256)
+    for (uint32_t p = vfirst - shift; p < pieces; p += 256)
     {
         uint32_t k = k0, w = w0;
         f32x4 x;

@@ -156,18 +156,40 @@ inline bool col_applicable(const float* g, const float* r_in, const float* r_out
            (reinterpret_cast<uintptr_t>(q) & 3u) == 0;
 }
 
+// Whether the three matrices sit at the same offset within a 128-byte line (then so do their columns), and whether any
+// column can start inside a line at all.
+inline bool same_line_offset(const float* g, const float* r_in, const float* r_out)
+{
+    const uintptr_t a = reinterpret_cast<uintptr_t>(g) & 127u, b = reinterpret_cast<uintptr_t>(r_in) & 127u,
+                    c = reinterpret_cast<uintptr_t>(r_out) & 127u;
+    return a == b && b == c;
+}
+
+inline bool columns_start_on_lines(const float* r_in, size_t rows)
+{
+    return (reinterpret_cast<uintptr_t>(r_in) & 127u) == 0 && rows % 32 == 0;
+}
+
+// Column kernels sum their statistics in the order of line-aligned slots when the three matrices share their offset
+// within a line and some column starts inside one.
+inline bool quantize_line_shift(const float* g, const float* r_in, const float* r_out, size_t rows)
+{
+    return same_line_offset(g, r_in, r_out) && !columns_start_on_lines(r_in, rows);
+}
+
 // the unrolled 1-bit kernels: 1024, 2048 or 4096 rows and 8-byte aligned packed buffers
 inline bool col_unrolled(const void* q, size_t rows, size_t nbits)
 {
     return nbits == 1 && (rows == 1024 || rows == 2048 || rows == 4096) && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
 }
 
-inline ColGeom make_col_geom(size_t rows, size_t nbits)
+inline ColGeom make_col_geom(size_t rows, size_t nbits, bool line_shift)
 {
     ColGeom c;
     c.rows = (uint32_t) rows;
     c.nq = (uint32_t) qwords_per_col(rows, nbits);
     c.pieces = (uint32_t) (rows / 4);
+    c.line_shift = line_shift ? 1u : 0u;
     c.qcol = qcol_bytes(nbits, rows);
     return c;
 }
@@ -195,7 +217,7 @@ struct StripeColLauncher
     }
 };
 
-inline RegGeom make_reg_geom(size_t rows, size_t nbits, uint32_t threads)
+inline RegGeom make_reg_geom(size_t rows, size_t nbits, uint32_t threads, bool line_shift)
 {
     RegGeom c;
     c.rows = (uint32_t) rows;
@@ -203,7 +225,7 @@ inline RegGeom make_reg_geom(size_t rows, size_t nbits, uint32_t threads)
     c.pieces = (uint32_t) (rows / 4);
     c.step_k = (4 * threads) / c.nq;
     c.step_w = (4 * threads) % c.nq;
-    c.pad = 0;
+    c.line_shift = line_shift ? 1u : 0u;
     c.qcol = qcol_bytes(nbits, rows);
     return c;
 }
@@ -227,13 +249,14 @@ struct RegLauncher
             return hipErrorInvalidValue;
         else
         {
-            const uint32_t per = (c.pieces + threads - 1) / threads;
+            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + threads - 1) / threads; // up to 7 slots lie before the column
 #define CNTKQ_REG(T, P) if (threads == T && per <= P) return launch_reg_one<NBITS, ZT, T, P>(s, ev, g, r_in, r_out, q, cols, c)
             CNTKQ_REG(256, 6);
             CNTKQ_REG(256, 8);
             CNTKQ_REG(256, 10);
             CNTKQ_REG(256, 12);
             CNTKQ_REG(256, 14);
+            CNTKQ_REG(256, 16);
             CNTKQ_REG(1024, 4);
             CNTKQ_REG(1024, 6);
             CNTKQ_REG(1024, 8);
@@ -314,14 +337,20 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
         if (!reg_applicable(g, r_in, r_out, q, rows, nbits, true))
             return hipErrorInvalidValue;
         const uint32_t threads = reg_threads(rows);
-        return dispatch_nbits<RegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, make_reg_geom(rows, nbits, threads), threads);
+        // up to 14336 rows the shift is part of the summation order all column kernels share; above, it is used where
+        // the registers allow
+        const bool line_shift = quantize_line_shift(g, r_in, r_out, rows) && (threads == 256 || rows / 4 + 7 <= 1024 * (size_t) kRegMaxShiftPer);
+        return dispatch_nbits<RegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols,
+                                           make_reg_geom(rows, nbits, threads, line_shift), threads);
     }
     if (path == kPathCol)
     {
         if (!col_applicable(g, r_in, r_out, q, rows, nbits, true))
             return hipErrorInvalidValue;
-        if (!col_unrolled(q, rows, nbits))
-            return dispatch_nbits<ColLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, make_col_geom(rows, nbits));
+        // (the unrolled kernels deal pieces without a shift: only for columns that start on lines)
+        const bool line_shift = quantize_line_shift(g, r_in, r_out, rows);
+        if (line_shift || !col_unrolled(q, rows, nbits))
+            return dispatch_nbits<ColLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, make_col_geom(rows, nbits, line_shift));
         const uint64_t qcol = qcol_bytes(nbits, rows);
         const uint32_t c = (uint32_t) cols;
         if (rows == 1024)
@@ -355,9 +384,11 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
         aligned8 = aligned8 && (reinterpret_cast<uintptr_t>(src.q[w]) & 7u) == 0;
     const bool col_forced = tune.quantize_path == kPathCol;
     const bool col = (tune.quantize_path == kPathAuto || col_forced) && rows % 4 == 0 && (col_forced || rows >= kColMinRows);
-    if (col && !(aligned8 && col_unrolled(q_out, rows, nbits)))
+    // the summation order a quantize call on (aggregate, stripe residual) would use, given the residual's address
+    const bool line_shift = !columns_start_on_lines(stripe_res, rows);
+    if (col && (line_shift || !(aligned8 && col_unrolled(q_out, rows, nbits))))
         return dispatch_nbits<StripeColLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols,
-                                                 make_col_geom(rows, nbits));
+                                                 make_col_geom(rows, nbits, line_shift));
     if (col)
     {
         // same column statistics, in the same order, as quantize_col_kernel

@@ -173,6 +173,23 @@ def test_register_and_lds_column_kernels_give_the_same_bytes(rows):
         qz._set_tuning(quantize_path=PATH_REG)
         Qb, rb = gpu_quantize(qz, g, r, nbits, zt)
         assert np.array_equal(Qa.to_numpy(), Qb.to_numpy()) and parity.bits_equal(ra, rb)
+    # matrices that all start 16, 48 or 112 bytes into a 128-byte line (and once at different offsets, where no shift
+    # is used): still the same bytes from both kernels, and right by the oracle
+    for og, orr in ((4, 4), (12, 12), (28, 28), (4, 8)):
+        def place(a, off):
+            buf = torch.zeros(rows * cols + 64, dtype=torch.float32, device="cuda:0")
+            buf[off:off + rows * cols] = torch.from_numpy(a.reshape(-1, order="F").copy()).cuda()
+            return Matrix(rows, cols, 0, buf[off:off + rows * cols])
+        outs = []
+        for path in (PATH_COL, PATH_REG):
+            qz._set_tuning(quantize_path=path)
+            G, R, Q = place(g, og), place(r, orr), QuantizedMatrix(rows, cols, 1, 0)
+            assert G.Data() % 128 == 4 * og and R.Data() % 128 == 4 * orr
+            qz.QuantizeAsync(G, R, Q, R, False)
+            qz.WaitQuantizeAsyncDone()
+            outs.append((Q.to_numpy(), R.to_numpy()))
+        assert np.array_equal(outs[0][0], outs[1][0]) and parity.bits_equal(outs[0][1], outs[1][1])
+        parity.check_quantize(g, r, outs[1][0], outs[1][1], 1, False)
     # beyond 25 pieces for each of 1024 threads the forced path refuses
     with pytest.raises(cntk_amd.QuantizerLogicError):
         gpu_quantize(qz, datagen.normal(1, 102404, 1), np.zeros((102404, 1), np.float32, order="F"), 1, False)
