@@ -675,6 +675,21 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSo
     const uint32_t K = src.workers;
     if (tid < NQ)
         l.words[tid] = 0u;
+    // Everything this thread will need from memory is requested before the first barrier, so that the headers, the
+    // first eight workers' QWords and the stripe residual cost one round trip, not three: a stripe is one GPU's share
+    // of a matrix, a single round of workgroups, and its time is the length of this dependent chain.
+    const uint32_t p = tid % NQ, chunk = tid / NQ;
+    const uint32_t sh0 = chunk * KS;
+    uint32_t word[BATCH];
+#pragma unroll
+    for (uint32_t u = 0; u < BATCH; ++u)
+        if (u < K)
+            word[u] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(u, src.owner)] + rec + 8)[p];
+    const float* sp = stripe_res + base;
+    float resid[KS];
+#pragma unroll
+    for (uint32_t kk = 0; kk < KS; ++kk)
+        resid[kk] = __builtin_nontemporal_load(sp + p + NQ * (sh0 + kk));
     if (tid < K)
     {
         const float* h = reinterpret_cast<const float*>(src.q[stripe_order(tid, src.owner)] + rec);
@@ -684,16 +699,16 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSo
     }
     __syncthreads();
 
-    const uint32_t p = tid % NQ, chunk = tid / NQ;
-    const uint32_t sh0 = chunk * KS;
     float acc[KS];
     for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
     {
-        uint32_t word[BATCH];
+        if (n0 != 0)
+        {
 #pragma unroll
-        for (uint32_t u = 0; u < BATCH; ++u)
-            if (n0 + u < K)
-                word[u] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + rec + 8)[p];
+            for (uint32_t u = 0; u < BATCH; ++u)
+                if (n0 + u < K)
+                    word[u] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + rec + 8)[p];
+        }
 #pragma unroll
         for (uint32_t u = 0; u < BATCH; ++u)
         {
@@ -711,14 +726,13 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSo
             }
         }
     }
-    const float* sp = stripe_res + base;
 #pragma unroll
     for (uint32_t kk = 0; kk < KS; ++kk)
     {
         const uint32_t i = p + NQ * (sh0 + kk);
         if (agg_out != nullptr)
             agg_out[base + i] = acc[kk];
-        l.tile[i] = acc[kk] + __builtin_nontemporal_load(sp + i);
+        l.tile[i] = acc[kk] + resid[kk];
     }
     float csum = 0.0f;
     if constexpr (!ZT)
@@ -798,12 +812,15 @@ __device__ __forceinline__ float colg_add_piece(float s, const f32x4& v)
 
 // stat: this thread's running statistic over its pieces (unused for 1 bit with ZT). tile = the column, words = zeroed
 // partial QWords, red = 12 reduction slots. No barrier is needed between writing the column and calling this.
-template <int NBITS, bool ZT>
+// WG: threads in the workgroup. The sums are always taken by the first 256 threads (their order is part of the result);
+// coding and packing use all of them.
+template <int NBITS, bool ZT, int WG = kColThreads>
 __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, float* red, const ColGeom& c, float stat,
                                                 uint32_t shift, float* res_col, char* qc)
 {
     using PS = PackShape<NBITS>;
     constexpr uint32_t T = kColThreads, NW = T / 64;
+    static_assert(WG >= (int) T && WG % 64 == 0, "workgroup size");
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 8);
     constexpr bool need_stat = (NBITS != 1) || !ZT;
@@ -811,7 +828,7 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
     if constexpr (need_stat)
     {
         const float s = wave_sum(stat);
-        if (lane == 0)
+        if (lane == 0 && wave < NW)
             red[wave] = s;
     }
     __syncthreads(); // the column and the wave sums are visible
@@ -829,14 +846,15 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
         float s0 = 0.0f, s1 = 0.0f;
         uint32_t n0 = 0;
         const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
-        for (uint32_t v = tid; v < c.pieces + shift; v += T)
-            if (v >= shift)
-                split_add_piece(t4[v - shift], mean, s0, s1, n0);
+        if (WG == T || tid < T)
+            for (uint32_t v = tid; v < c.pieces + shift; v += T)
+                if (v >= shift)
+                    split_add_piece(t4[v - shift], mean, s0, s1, n0);
         s0 = wave_sum(s0);
         s1 = wave_sum(s1);
         n0 = wave_sum(n0);
         __syncthreads(); // everyone has read the wave sums of the mean
-        if (lane == 0)
+        if (lane == 0 && wave < NW)
         {
             red[wave] = s0;
             red[4 + wave] = s1;
@@ -870,7 +888,7 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
     const float val1 = unquantize_value<NBITS>(vq, 1u);
     uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
     const uint32_t items = c.nq * PS::CHUNKS;
-    for (uint32_t it = tid; it < items; it += T)
+    for (uint32_t it = tid; it < items; it += WG)
     {
         // chunk-major: consecutive threads take consecutive QWords, hence consecutive rows
         const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / c.nq;
@@ -902,7 +920,7 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
     if constexpr (PS::CHUNKS > 1)
     {
         __syncthreads();
-        for (uint32_t w = tid; w < c.nq; w += T)
+        for (uint32_t w = tid; w < c.nq; w += WG)
             bits[w] = words[w];
     }
 }
@@ -965,12 +983,15 @@ __global__ __launch_bounds__(kColThreads) void quantize_colg_kernel(const float*
     quantize_colg_body<NBITS, ZT>(g, r_in, r_out, q, c, blockIdx.x, smem_v4);
 }
 
-template <int NBITS, bool ZT>
+// WG: threads in the workgroup (256, or 1024 for tall columns, whose many work items would otherwise be a long chain of
+// dependent loads for each of few threads)
+template <int NBITS, bool ZT, int WG = kColThreads>
 __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
                                                         const ColGeom& c, uint32_t column, f32x4* smem)
 {
     using PS = PackShape<NBITS>;
     constexpr uint32_t T = kColThreads, BATCH = 8;
+    static_assert(WG >= (int) T, "workgroup size");
     float* tile = reinterpret_cast<float*>(smem);
     uint32_t* words = reinterpret_cast<uint32_t*>(tile + c.rows);
     float* red = tile + c.rows + (PS::CHUNKS > 1 ? c.nq : 0);
@@ -980,8 +1001,30 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
     const size_t rec = (size_t) column * c.qcol;
     const uint32_t K = src.workers;
     if constexpr (PS::CHUNKS > 1)
-        for (uint32_t x = tid; x < c.nq; x += T)
+        for (uint32_t x = tid; x < c.nq; x += WG)
             words[x] = 0u;
+    // what this thread's first work item needs from memory is requested before the first barrier: one round trip for
+    // headers, QWords and stripe residual instead of three (see stripe_reduce_col_kernel)
+    const float* sp = stripe_res + base;
+    const uint32_t items = c.nq * PS::CHUNKS;
+    uint32_t word[BATCH];
+    float resid[PS::SLOTS];
+    if (tid < items)
+    {
+        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : tid / c.nq;
+        const uint32_t w = tid - chunk * c.nq;
+#pragma unroll
+        for (uint32_t u = 0; u < BATCH; ++u)
+            if (u < K)
+                word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(u, src.owner)] + rec + 8 + (size_t) w * 4);
+#pragma unroll
+        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+        {
+            const uint32_t i = w + (chunk * PS::SLOTS + kk) * c.nq;
+            if (i < c.rows)
+                resid[kk] = __builtin_nontemporal_load(sp + i);
+        }
+    }
     if (tid < K)
     {
         const float* h = reinterpret_cast<const float*>(src.q[stripe_order(tid, src.owner)] + rec);
@@ -999,22 +1042,32 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
     }
     __syncthreads();
 
-    const float* sp = stripe_res + base;
-    const uint32_t items = c.nq * PS::CHUNKS;
-    for (uint32_t it = tid; it < items; it += T)
+    for (uint32_t it = tid; it < items; it += WG)
     {
         const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / c.nq;
         const uint32_t w = it - chunk * c.nq;
         const size_t word_off = rec + 8 + (size_t) w * 4;
         const uint32_t sh0 = chunk * PS::SLOTS * PS::SHIFT;
+        if (it != tid)
+        {
+#pragma unroll
+            for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+            {
+                const uint32_t i = w + (chunk * PS::SLOTS + kk) * c.nq;
+                if (i < c.rows)
+                    resid[kk] = __builtin_nontemporal_load(sp + i);
+            }
+        }
         float acc[PS::SLOTS];
         for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
         {
-            uint32_t word[BATCH];
+            if (it != tid || n0 != 0)
+            {
 #pragma unroll
-            for (uint32_t u = 0; u < BATCH; ++u)
-                if (n0 + u < K)
-                    word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + word_off);
+                for (uint32_t u = 0; u < BATCH; ++u)
+                    if (n0 + u < K)
+                        word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + word_off);
+            }
 #pragma unroll
             for (uint32_t u = 0; u < BATCH; ++u)
             {
@@ -1046,7 +1099,7 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
             {
                 if (agg_out != nullptr)
                     agg_out[base + i] = acc[kk];
-                tile[i] = acc[kk] + __builtin_nontemporal_load(sp + i);
+                tile[i] = acc[kk] + resid[kk];
             }
         }
     }
@@ -1057,19 +1110,20 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
     {
         __syncthreads();
         const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
-        for (uint32_t v = tid; v < c.pieces + shift; v += T)
-            if (v >= shift)
-                stat = colg_add_piece<NBITS>(stat, t4[v - shift]);
+        if (WG == T || tid < T)
+            for (uint32_t v = tid; v < c.pieces + shift; v += T)
+                if (v >= shift)
+                    stat = colg_add_piece<NBITS>(stat, t4[v - shift]);
     }
-    colg_stats_pack<NBITS, ZT>(tile, words, red, c, stat, shift, stripe_res + base, q_out + rec);
+    colg_stats_pack<NBITS, ZT, WG>(tile, words, red, c, stat, shift, stripe_res + base, q_out + rec);
 }
 
-template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kColThreads) void stripe_reduce_colg_kernel(StripeSources src, float* stripe_res, char* q_out,
-                                                                         float* agg_out, ColGeom c)
+template <int NBITS, bool ZT, int WG>
+__global__ __launch_bounds__(WG) void stripe_reduce_colg_kernel(StripeSources src, float* stripe_res, char* q_out, float* agg_out,
+                                                                ColGeom c)
 {
     extern __shared__ f32x4 smem_v4[];
-    stripe_reduce_colg_body<NBITS, ZT>(src, stripe_res, q_out, agg_out, c, blockIdx.x, smem_v4);
+    stripe_reduce_colg_body<NBITS, ZT, WG>(src, stripe_res, q_out, agg_out, c, blockIdx.x, smem_v4);
 }
 
 // ---- one workgroup per column, the column in registers ------------------------------------------------------

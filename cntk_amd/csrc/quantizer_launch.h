@@ -24,6 +24,7 @@ enum QuantizePath
 };
 
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
+constexpr uint32_t kStripeWideItems = 768; // work items per column from which the stripe reduction uses 1024 threads
 constexpr uint32_t kColMinRows = 1024;   // shorter columns are better served several to a workgroup (tile kernels)
 
 struct LaunchTuning
@@ -211,8 +212,14 @@ struct StripeColLauncher
     static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
                           uint32_t cols, ColGeom c)
     {
-        hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT>), dim3(cols), dim3(kColThreads), colg_lds_bytes<NBITS>(c, src.workers),
-                              s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
+        // columns with many work items (QWords x chunks of bit positions) get 1024 threads: each item is a chain of
+        // dependent loads, and few columns of a tall stripe would leave a CU with four wavefronts
+        if (c.nq * PackShape<NBITS>::CHUNKS >= kStripeWideItems)
+            hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, 1024>), dim3(cols), dim3(1024), colg_lds_bytes<NBITS>(c, src.workers),
+                                  s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
+        else
+            hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, kColThreads>), dim3(cols), dim3(kColThreads),
+                                  colg_lds_bytes<NBITS>(c, src.workers), s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
         return hipGetLastError();
     }
 };

@@ -51,6 +51,8 @@ CASES = [
     (2048, 48, 8, 1, False), (2048, 48, 8, 1, True), (2048, 16, 8, 2, False), (4608, 8, 2, 1, False),
     (9304, 3, 3, 1, True), (33, 5, 8, 1, False), (512, 64, 64, 1, False), (4096, 7, 3, 1, False), (4096, 4, 12, 1, True),
     (2048, 20, 11, 1, False), (1024, 24, 4, 1, False), (1024, 9, 64, 1, True), (4096, 5, 64, 1, False),
+    # tall columns: 1024 threads per column in the stripe reduction, register kernels in the call sequence
+    (9304, 6, 4, 1, False), (8192, 4, 3, 4, False), (12000, 4, 5, 2, False), (14336, 2, 2, 8, False),
 ]
 
 
