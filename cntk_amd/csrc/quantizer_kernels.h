@@ -757,7 +757,7 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSo
 // How a column's 16-byte pieces are dealt to the slots of a workgroup (slot v = thread + T * u). With line_shift set,
 // slot v holds piece v - shift, shift = the column's offset into its 128-byte line in pieces (the residual input's
 // address decides; the launch sets line_shift only when gradient and residual output share that offset).
-__device__ __forceinline__ uint32_t column_shift(const float* column, uint32_t line_shift)
+__device__ __forceinline__ uint32_t column_shift(const void* column, uint32_t line_shift)
 {
     return line_shift ? (uint32_t) ((reinterpret_cast<uintptr_t>(column) >> 4) & 7u) : 0u;
 }

@@ -649,5 +649,358 @@ __global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict_
     }
 }
 
+// ---- row-major and tile decoders (the fp32 unquantize_rows_kernel / unquantize_tile_kernel on doubles) ---------
+//
+// A 16-byte store holds two doubles; QWords are 64-bit; a packed record is nq + 2 QWords (lower, upper, bits).
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __restrict__ q, double* out, UnqRowGeom t, int add)
+{
+    using PS = PackShape<NBITS>;
+    extern __shared__ f32x4 smem_v4[];
+    uint64_t* words = reinterpret_cast<uint64_t*>(smem_v4);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t c = blockIdx.x / t.chunks;
+    const uint32_t ch = blockIdx.x - c * t.chunks;
+    const char* qc = q + (size_t) c * t.qcol;
+    const double* gh = reinterpret_cast<const double*>(qc);
+    const ValueQ vq = make_vq<NBITS>(gh[0], gh[1]);
+    const uint64_t* bits = reinterpret_cast<const uint64_t*>(qc + 16);
+    for (uint32_t w = tid; w < t.nq; w += 4 * 256)
+    {
+        uint64_t v[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+            v[u] = bits[(w + 256 * u < t.nq) ? w + 256 * u : w];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+            if (w + 256 * u < t.nq)
+                words[w + 256 * u] = v[u];
+    }
+    __syncthreads();
+    const uint32_t r0 = ch * t.chunk;
+    const uint32_t pieces = ((ch + 1 == t.chunks ? t.rows : r0 + t.chunk) - r0) >> 1; // the last chunk runs to the end
+    f64x2* o2 = reinterpret_cast<f64x2*>(out + (size_t) c * t.rows + r0);
+    const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
+    const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
+    // slots dealt by 128-byte lines, as in the fp32 decoder
+    const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o2) >> 4) & 7u);
+    const uint32_t vfirst = tid < shift ? tid + 256 : tid;
+    // row i sits in QWord i % nq at bit position i / nq; a thread's pieces are 512 rows apart
+    const uint32_t i0 = r0 + 2 * (vfirst - shift);
+    uint32_t k0 = i0 / t.nq;
+    uint32_t w0 = i0 - k0 * t.nq;
+    const uint32_t dk = 512u / t.nq;
+    const uint32_t dw = 512u - dk * t.nq;
+    for (uint32_t p = vfirst - shift; p < pieces; p += 256)
+    {
+        uint32_t k = k0, w = w0;
+        f64x2 x;
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+        {
+            const uint64_t code = (words[w] >> (k * PS::SHIFT)) & PS::CODEMASK;
+            if constexpr (NBITS == 1)
+                x[e] = code ? val1 : val0;
+            else
+                x[e] = unquantize_value<NBITS>(vq.uf, vq.lo, code);
+            if (++w == t.nq)
+            {
+                w = 0;
+                ++k;
+            }
+        }
+        if (add)
+            x = x + o2[p]; // unquantized value + previous content
+        __builtin_nontemporal_store(x, o2 + p);
+        k0 += dk;
+        w0 += dw;
+        if (w0 >= t.nq)
+        {
+            w0 -= t.nq;
+            ++k0;
+        }
+    }
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_tile_kernel(const char* __restrict__ q, double* out, UnqTileGeom t, int add)
+{
+    using PS = PackShape<NBITS>;
+    extern __shared__ f32x4 smem_v4[];
+    uint64_t* words = reinterpret_cast<uint64_t*>(smem_v4);            // ncols packed records
+    double* dec = reinterpret_cast<double*>(words + t.cpt * t.rec_words); // per column: the two levels (1 bit) or (ufactor, lower)
+    const uint32_t tid = threadIdx.x;
+    const uint32_t col0 = blockIdx.x * t.cpt;
+    const uint32_t ncols = (t.cols - col0 < t.cpt) ? t.cols - col0 : t.cpt;
+    const uint64_t* src = reinterpret_cast<const uint64_t*>(q + (size_t) col0 * t.rec_words * 8);
+    const uint32_t total_words = ncols * t.rec_words;
+    for (uint32_t x = tid; x < total_words; x += 256)
+        words[x] = __builtin_nontemporal_load(src + x);
+    __syncthreads();
+    for (uint32_t c = tid; c < ncols; c += 256)
+    {
+        const double lo = __longlong_as_double((long long) words[c * t.rec_words]);
+        const double hi = __longlong_as_double((long long) words[c * t.rec_words + 1]);
+        const ValueQ vq = make_vq<NBITS>(lo, hi);
+        if constexpr (NBITS == 1)
+        {
+            dec[2 * c] = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
+            dec[2 * c + 1] = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
+        }
+        else
+        {
+            dec[2 * c] = vq.uf;
+            dec[2 * c + 1] = vq.lo;
+        }
+    }
+    __syncthreads();
+    const uint32_t elems = ncols * t.rows;
+    double* o = out + (size_t) col0 * t.rows;
+    for (uint32_t i = 2 * tid; i < elems; i += 512)
+    {
+        uint32_t c = small_div(i, t.rows, t.rows_magic);
+        uint32_t r = i - c * t.rows;
+        uint32_t k = small_div(r, t.nq, t.nq_magic);
+        uint32_t w = r - k * t.nq;
+        const uint64_t* cw = words + c * t.rec_words + 2;
+        double d0 = dec[2 * c], d1 = dec[2 * c + 1];
+        f64x2 x;
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+        {
+            // (past the end of the matrix the reads stay inside the LDS block and the value is not stored)
+            const uint64_t code = (cw[w] >> (k * PS::SHIFT)) & PS::CODEMASK;
+            if constexpr (NBITS == 1)
+                x[e] = code ? d1 : d0;
+            else
+                x[e] = unquantize_value<NBITS>(d0, d1, code);
+            ++r;
+            if (++w == t.nq)
+            {
+                w = 0;
+                ++k;
+            }
+            if (r == t.rows)
+            {
+                r = 0;
+                k = 0;
+                w = 0;
+                c = (c + 1 < t.cpt) ? c + 1 : c;
+                cw = words + c * t.rec_words + 2;
+                d0 = dec[2 * c];
+                d1 = dec[2 * c + 1];
+            }
+        }
+        if (i + 2 <= elems)
+        {
+            f64x2* o2 = reinterpret_cast<f64x2*>(o + i);
+            if (add)
+                x = x + *o2; // unquantized value + previous content
+            __builtin_nontemporal_store(x, o2);
+        }
+        else
+            o[i] = add ? x[0] + o[i] : x[0];
+    }
+}
+
+// ---- one workgroup per column, the column in registers (the fp32 quantize_reg_kernel on doubles) ------------
+//
+// Thread tid of T keeps the 16-byte pieces (two doubles) of its slots tid, tid + T, ... through statistics, coding and
+// the residual store; LDS holds only the column's 64-bit QWords, assembled by atomic OR. Slots are dealt by 128-byte
+// lines (column_shift). For columns too tall for the tile kernels: up to 25 pieces for each of 1024 threads.
+
+template <int NBITS>
+__device__ __forceinline__ double reg_add_piece(double s, const f64x2& v)
+{
+    if constexpr (NBITS == 1)
+    {
+        s += v.x;
+        s += v.y;
+    }
+    else
+    {
+        s += v.x * v.x;
+        s += v.y * v.y;
+    }
+    return s;
+}
+
+__host__ __device__ inline size_t reg_lds_bytes64(const RegGeom& c)
+{
+    return ((size_t) kRegRedSlots + c.nq) * 8;
+}
+
+template <int NBITS, bool ZT, int T, int PER>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, PER>(), reg_waves<T, PER>()))) void quantize_reg_kernel(
+    const double* __restrict__ g, const double* r_in, double* r_out, char* __restrict__ q, RegGeom c)
+{
+    using PS = PackShape<NBITS>;
+    static_assert(NBITS < 64, "64-bit codes are whole QWords: nothing to assemble");
+    constexpr uint32_t NW = T / 64;
+    extern __shared__ f32x4 smem_v4[];
+    double* red = reinterpret_cast<double*>(smem_v4);
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
+    unsigned long long* words = reinterpret_cast<unsigned long long*>(red + kRegRedSlots);
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const size_t base = (size_t) blockIdx.x * c.rows;
+    char* qc = q + (size_t) blockIdx.x * c.qcol;
+    for (uint32_t x = tid; x < c.nq; x += T)
+        words[x] = 0ull;
+    const f64x2* g2 = reinterpret_cast<const f64x2*>(g + base);
+    const f64x2* r2 = reinterpret_cast<const f64x2*>(r_in + base);
+    const uint32_t shift = PER <= kRegMaxShiftPer ? column_shift(r_in + base, c.line_shift) : 0u;
+    const uint32_t last = c.pieces - 1;
+    f64x2 a[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+        a[u] = __builtin_nontemporal_load(g2 + slot_piece(tid + T * u, shift, last));
+#pragma unroll
+    for (int u0 = 0; u0 < PER; u0 += 4)
+    {
+        f64x2 b[4];
+#pragma unroll
+        for (int u = u0; u < u0 + 4 && u < PER; ++u)
+            b[u - u0] = __builtin_nontemporal_load(r2 + slot_piece(tid + T * u, shift, last));
+#pragma unroll
+        for (int u = u0; u < u0 + 4 && u < PER; ++u)
+            a[u] = a[u] + b[u - u0];
+    }
+    constexpr bool need_stat = (NBITS != 1) || !ZT;
+    double total = 0.0;
+    if constexpr (need_stat)
+    {
+        double stat = 0.0;
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+        {
+            const double with = reg_add_piece<NBITS>(stat, a[u]);
+            stat = slot_valid(tid + T * u, shift, c.pieces) ? with : stat;
+        }
+        stat = wave_sum(stat);
+        if (lane == 0)
+            red[wave] = stat;
+    }
+    // the whole column has been read before this barrier, so r_out may be r_in
+    __syncthreads();
+    if constexpr (need_stat)
+    {
+        total = red[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+            total += red[x];
+    }
+    double lo, hi;
+    if constexpr (NBITS == 1)
+    {
+        const double mean = ZT ? 0.0 : total / (double) c.rows;
+        double s0 = 0.0, s1 = 0.0;
+        uint32_t n0 = 0;
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+        {
+            double t0 = s0, t1 = s1;
+            uint32_t tn = n0;
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+            {
+                const double x = a[u][e];
+                const bool below = x < mean;
+                t0 += below ? x : 0.0;
+                t1 += below ? 0.0 : x;
+                tn += below ? 1u : 0u;
+            }
+            const bool valid = slot_valid(tid + T * u, shift, c.pieces);
+            s0 = valid ? t0 : s0;
+            s1 = valid ? t1 : s1;
+            n0 = valid ? tn : n0;
+        }
+        s0 = wave_sum(s0);
+        s1 = wave_sum(s1);
+        n0 = wave_sum(n0);
+        __syncthreads(); // everyone has read the wave sums of the mean
+        if (lane == 0)
+        {
+            red[wave] = s0;
+            red[NW + wave] = s1;
+            red_u[wave] = n0;
+        }
+        __syncthreads();
+        double S0 = red[0], S1 = red[NW];
+        uint32_t N0 = red_u[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+        {
+            S0 += red[x];
+            S1 += red[NW + x];
+            N0 += red_u[x];
+        }
+        finish_stats_1bit<ZT>(mean, S0, S1, N0, c.rows - N0, c.rows, lo, hi);
+    }
+    else
+    {
+        finish_stats_multibit(total, c.rows, lo, hi);
+    }
+    if (tid == 0)
+    {
+        double* gh = reinterpret_cast<double*>(qc);
+        gh[0] = lo;
+        gh[1] = hi;
+    }
+    const ValueQ vq = make_vq<NBITS>(lo, hi);
+    const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
+    const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
+    f64x2* o2 = reinterpret_cast<f64x2*>(r_out + base);
+    // the first element of this thread's first slot inside the column is bit position k of QWord w; the element after it
+    // is the following QWord, the slots after it lie 2 * T elements further on (step_k, step_w)
+    const uint32_t ufirst = tid < shift ? 1u : 0u;
+    const uint32_t e0 = 2 * (tid + T * ufirst - shift);
+    uint32_t k = e0 / c.nq;
+    uint32_t w = e0 - k * c.nq;
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+    {
+        const uint32_t p = tid + T * u - shift;
+        if (slot_valid(tid + T * u, shift, c.pieces))
+        {
+            f64x2 res;
+            uint32_t kk = k, ww = w;
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+            {
+                const double v = a[u][e];
+                const uint64_t code = quantize_value<NBITS, ZT>(vq, v);
+                double back;
+                if constexpr (NBITS == 1)
+                    back = code ? val1 : val0;
+                else
+                    back = unquantize_value<NBITS>(vq.uf, vq.lo, code);
+                res[e] = v - back;
+                atomicOr(&words[ww], (unsigned long long) (code << (kk * PS::SHIFT)));
+                if (++ww == c.nq)
+                {
+                    ww = 0;
+                    ++kk;
+                }
+            }
+            __builtin_nontemporal_store(res, o2 + p);
+        }
+        if ((uint32_t) u >= ufirst)
+        {
+            w += c.step_w;
+            k += c.step_k;
+            if (w >= c.nq)
+            {
+                w -= c.nq;
+                ++k;
+            }
+        }
+    }
+    __syncthreads();
+    unsigned long long* bits = reinterpret_cast<unsigned long long*>(qc + 16);
+    for (uint32_t x = tid; x < c.nq; x += T)
+        bits[x] = words[x];
+}
+
 } // namespace f64
 } // namespace cntkq

@@ -159,16 +159,16 @@ inline bool col_applicable(const float* g, const float* r_in, const float* r_out
 
 // Whether the three matrices sit at the same offset within a 128-byte line (then so do their columns), and whether any
 // column can start inside a line at all.
-inline bool same_line_offset(const float* g, const float* r_in, const float* r_out)
+inline bool same_line_offset(const void* g, const void* r_in, const void* r_out)
 {
     const uintptr_t a = reinterpret_cast<uintptr_t>(g) & 127u, b = reinterpret_cast<uintptr_t>(r_in) & 127u,
                     c = reinterpret_cast<uintptr_t>(r_out) & 127u;
     return a == b && b == c;
 }
 
-inline bool columns_start_on_lines(const float* r_in, size_t rows)
+inline bool columns_start_on_lines(const void* r_in, size_t rows, size_t rows_per_line = 32)
 {
-    return (reinterpret_cast<uintptr_t>(r_in) & 127u) == 0 && rows % 32 == 0;
+    return (reinterpret_cast<uintptr_t>(r_in) & 127u) == 0 && rows % rows_per_line == 0;
 }
 
 // Column kernels sum their statistics in the order of line-aligned slots when the three matrices share their offset

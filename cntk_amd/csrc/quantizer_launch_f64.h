@@ -109,6 +109,66 @@ struct StripeLauncher
     }
 };
 
+// The register kernel: for columns the tile kernel cannot hold, of even height, 16-byte aligned matrices, below 64 bits,
+// at most 25 pieces of two doubles for each of 1024 threads, QWords within 64 KB of LDS.
+constexpr uint32_t kRegThreads = 1024;
+constexpr size_t kRegMaxRows = 2 * 1024 * 25;
+
+inline bool reg_applicable(const double* g, const double* r_in, const double* r_out, size_t rows, size_t nbits)
+{
+    const uintptr_t m = reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(r_in) | reinterpret_cast<uintptr_t>(r_out);
+    if (rows % 2 != 0 || rows < 2 || rows > kRegMaxRows || nbits >= 64 || (m & 15u) != 0)
+        return false;
+    return (kRegRedSlots + qwords_per_col(rows, nbits)) * 8 <= kMaxLdsBytes;
+}
+
+inline RegGeom make_reg_geom(size_t rows, size_t nbits, bool line_shift)
+{
+    RegGeom c;
+    c.rows = (uint32_t) rows;
+    c.nq = (uint32_t) qwords_per_col(rows, nbits);
+    c.pieces = (uint32_t) (rows / 2);
+    c.step_k = (2 * kRegThreads) / c.nq;
+    c.step_w = (2 * kRegThreads) % c.nq;
+    c.line_shift = line_shift ? 1u : 0u;
+    c.qcol = qcol_bytes(nbits, rows);
+    return c;
+}
+
+template <int NBITS, bool ZT, int PER>
+inline hipError_t launch_reg_one(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, char* q, uint32_t cols,
+                                 const RegGeom& c)
+{
+    hipExtLaunchKernelGGL((quantize_reg_kernel<NBITS, ZT, (int) kRegThreads, PER>), dim3(cols), dim3(kRegThreads), reg_lds_bytes64(c), s,
+                          ev.start, ev.stop, 0, g, r_in, r_out, q, c);
+    return hipGetLastError();
+}
+
+template <int NBITS, bool ZT>
+struct RegLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, char* q, uint32_t cols, RegGeom c)
+    {
+        if constexpr (NBITS >= 64)
+            return hipErrorInvalidValue;
+        else
+        {
+            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + kRegThreads - 1) / kRegThreads;
+#define CNTKQ_REG64(P) if (per <= P) return launch_reg_one<NBITS, ZT, P>(s, ev, g, r_in, r_out, q, cols, c)
+            CNTKQ_REG64(4);
+            CNTKQ_REG64(6);
+            CNTKQ_REG64(8);
+            CNTKQ_REG64(10);
+            CNTKQ_REG64(13);
+            CNTKQ_REG64(16);
+            CNTKQ_REG64(20);
+            CNTKQ_REG64(25);
+#undef CNTKQ_REG64
+            return hipErrorInvalidValue;
+        }
+    }
+};
+
 // rows, cols > 0; pointers 8-byte aligned (checked by the caller). tune.quantize_path may force the tile or tall kernel.
 inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, void* q, size_t rows,
                                   size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
@@ -117,7 +177,15 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* 
     char* qc = static_cast<char*>(q);
     int path = tune.quantize_path;
     if (path == kPathAuto)
-        path = rows > kTileMaxRows ? kPathTall : kPathTile;
+        path = rows <= kTileMaxRows ? kPathTile : (reg_applicable(g, r_in, r_out, rows, nbits) ? kPathReg : kPathTall);
+    if (path == kPathReg)
+    {
+        if (!reg_applicable(g, r_in, r_out, rows, nbits))
+            return hipErrorInvalidValue;
+        const bool line_shift = same_line_offset(g, r_in, r_out) && !columns_start_on_lines(r_in, rows, 16) &&
+                                rows / 2 + 7 <= (size_t) kRegThreads * kRegMaxShiftPer;
+        return dispatch_nbits64<RegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, make_reg_geom(rows, nbits, line_shift));
+    }
     if (path == kPathTile)
     {
         if (rows > kTileMaxRows)
@@ -157,12 +225,108 @@ inline hipError_t launch_unquantize_n(hipStream_t s, LaunchEvents ev, const char
     return hipGetLastError();
 }
 
+constexpr size_t kUnqRowsMinRows64 = 512;  // from this height on a column keeps the 256 threads of the row-major decoder busy
+constexpr size_t kUnqTileMaxRows64 = 4096;
+constexpr size_t kUnqTileElems64 = 2048;   // values per workgroup the tile decoder aims for
+
+template <int NBITS>
+inline hipError_t launch_unquantize_rows(hipStream_t s, LaunchEvents ev, const char* q, double* out, const UnqRowGeom& t, int add)
+{
+    hipExtLaunchKernelGGL((unquantize_rows_kernel<NBITS>), dim3(t.blocks), dim3(256), (size_t) t.nq * 8, s, ev.start, ev.stop, 0, q, out, t, add);
+    return hipGetLastError();
+}
+
+template <int NBITS>
+inline hipError_t launch_unquantize_tile(hipStream_t s, LaunchEvents ev, const char* q, double* out, const UnqTileGeom& t, int add)
+{
+    hipExtLaunchKernelGGL((unquantize_tile_kernel<NBITS>), dim3(t.blocks), dim3(256), (size_t) t.cpt * (t.rec_words + 2) * 8, s, ev.start,
+                          ev.stop, 0, q, out, t, add);
+    return hipGetLastError();
+}
+
+#define CNTKQ_NBITS64_SWITCH(FN, ...)                                                                                  \
+    switch (nbits)                                                                                                     \
+    {                                                                                                                  \
+    case 1: return FN<1>(__VA_ARGS__);                                                                                 \
+    case 2: return FN<2>(__VA_ARGS__);                                                                                 \
+    case 4: return FN<4>(__VA_ARGS__);                                                                                 \
+    case 8: return FN<8>(__VA_ARGS__);                                                                                 \
+    case 16: return FN<16>(__VA_ARGS__);                                                                               \
+    case 32: return FN<32>(__VA_ARGS__);                                                                               \
+    case 64: return FN<64>(__VA_ARGS__);                                                                               \
+    default: return hipErrorInvalidValue;                                                                              \
+    }
+
 inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* q, double* out, size_t rows, size_t cols, size_t nbits,
                                     bool add, const LaunchTuning& tune)
 {
     const size_t vpw = 64 / nbits;
     const size_t nq = qwords_per_col(rows, nbits);
-    const bool vec = !tune.unq_force_scalar && (nq % 2 == 0) && (rows % 2 == 0) && (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    const bool out16 = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    const int mode = tune.unq_force_scalar; // 0 automatic, 1 QWord-major 8-byte stores, 2 / 4 tile / row-major decoder wherever it can run, 3 QWord-major
+    // The QWord-major decoder is at its best when every bit position of a column is a run of whole 128-byte lines. Other
+    // columns: row-major decoder from 512 rows on, tile decoder for shorter ones (the choices of the fp32 side).
+    const bool vec_ideal = nq % 16 == 0 && rows % 16 == 0 && rows * nbits == nq * 64 && out16;
+    const bool rows_can = tune.unq_slots == 0 && out16 && rows % 2 == 0 && nq >= 16 && nq * 8 <= 48 * 1024;
+    const bool tile_can = tune.unq_slots == 0 && out16 && rows <= kUnqTileMaxRows64;
+    bool use_rows = false, use_tile = false;
+    if (mode == 2 && tile_can)
+        use_tile = true;
+    else if (mode == 4 && rows_can)
+        use_rows = true;
+    else if (mode == 0 && tune.unq_slots == 0 && !vec_ideal)
+    {
+        if (rows_can && rows >= kUnqRowsMinRows64)
+            use_rows = true;
+        else if (tile_can)
+            use_tile = true;
+        else if (rows_can)
+            use_rows = true;
+    }
+    const char* qc0 = static_cast<const char*>(q);
+    if (use_rows)
+    {
+        UnqRowGeom t;
+        t.rows = (uint32_t) rows;
+        t.nq = (uint32_t) nq;
+        const size_t mult = nq > 512 ? 2 : 4;
+        size_t chunk = ((mult * nq + 511) / 512) * 512;
+        if (chunk < 1024)
+            chunk = 1024;
+        t.chunk = (uint32_t) chunk;
+        t.chunks = rows >= chunk ? (uint32_t) ((rows + chunk / 2) / chunk) : 1u;
+        t.pad = 0;
+        t.qcol = qcol_bytes(nbits, rows);
+        const uint64_t blocks = (uint64_t) cols * t.chunks;
+        if (blocks <= 0x7FFFFFFFull)
+        {
+            t.blocks = (uint32_t) blocks;
+            const int a = add ? 1 : 0;
+            CNTKQ_NBITS64_SWITCH(launch_unquantize_rows, s, ev, qc0, out, t, a)
+        }
+    }
+    if (use_tile)
+    {
+        UnqTileGeom t;
+        t.rows = (uint32_t) rows;
+        t.cols = (uint32_t) cols;
+        t.nq = (uint32_t) nq;
+        size_t cpt = (kUnqTileElems64 / rows) & ~(size_t) 1;
+        if (cpt < 2)
+            cpt = 2;
+        t.cpt = (uint32_t) cpt;
+        t.rec_words = (uint32_t) nq + 2;
+        t.rows_magic = rows > 1 ? (uint32_t) ((((uint64_t) 1 << 32) + rows - 1) / rows) : 0u;
+        t.nq_magic = nq > 1 ? (uint32_t) ((((uint64_t) 1 << 32) + nq - 1) / nq) : 0u;
+        const uint64_t blocks = (cols + cpt - 1) / cpt;
+        if (blocks <= 0x7FFFFFFFull && (size_t) t.cpt * (t.rec_words + 2) * 8 <= kMaxLdsBytes)
+        {
+            t.blocks = (uint32_t) blocks;
+            const int a = add ? 1 : 0;
+            CNTKQ_NBITS64_SWITCH(launch_unquantize_tile, s, ev, qc0, out, t, a)
+        }
+    }
+    const bool vec = mode != 1 && (nq % 2 == 0) && (rows % 2 == 0) && out16;
     const uint32_t wv = vec ? 2 : 1;
     UnqGeom t;
     t.rows = (uint32_t) rows;

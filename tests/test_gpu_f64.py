@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 
 F64 = np.float64
 VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False), (64, False)]
-PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL = 0, 1, 2, 3
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG = 0, 1, 2, 3, 4
 
 
 def say(*a):
@@ -135,6 +135,9 @@ PATH_CASES = [
     (147, 64, PATH_TILE, 0), (429, 37, PATH_TILE, 0), (429, 37, PATH_TILE, 64), (1023, 9, PATH_TILE, 0),
     (2048, 19, PATH_TILE, 0), (2048, 19, PATH_TILE, 256), (4608, 3, PATH_TILE, 0), (7168, 2, PATH_TILE, 0),
     (1, 5, PATH_TALL, 0), (70, 3, PATH_TALL, 0), (1025, 3, PATH_TALL, 0), (20001, 2, PATH_TALL, 0), (9304, 2, PATH_AUTO, 0),
+    # one workgroup of 1024 threads per column, the column in registers: even heights; the automatic choice above 7168 rows
+    (2, 3, PATH_REG, 0), (70, 3, PATH_REG, 0), (1000, 5, PATH_REG, 0), (7170, 3, PATH_REG, 0), (9304, 3, PATH_REG, 0),
+    (20000, 3, PATH_AUTO, 0), (32770, 2, PATH_REG, 0), (51200, 1, PATH_AUTO, 0), (51202, 1, PATH_AUTO, 0),
 ]
 
 
@@ -146,6 +149,11 @@ def test_kernel_paths_f64(case):
     rep = parity.Report()
     for nbits, zt in VARIANTS:
         say("f64 path case", case, "nbits", nbits, "zeroThr", zt)
+        if path == PATH_REG and (nbits == 64 or (48 + oracle.qwords_per_col(rows, nbits, F64)) * 8 > 65536):
+            # whole-QWord codes and columns whose QWords exceed 64 KB of LDS are refused when forced
+            with pytest.raises(cntk_amd.QuantizerLogicError):
+                gpu_quantize(qz, datagen.normal(1, rows, cols, dtype=F64), zeros(rows, cols), nbits, zt)
+            continue
 
         def make(it):
             a = datagen.normal_with_outliers(1000 * rows + cols + it, rows, cols, 0.01, dtype=F64) + 0.004 * (it % 2)
@@ -185,6 +193,39 @@ def test_unquantize_variants_f64(quantizer):
                         qz.UnquantizeAsync(Q, Out, add=add)
                         qz.WaitUnquantizeAsyncDone()
                         parity.check_unquantize(q, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
+
+
+DECODER_SHAPES_F64 = [(1, 1), (1, 9), (3, 5), (31, 13), (64, 100), (147, 64), (429, 37), (512, 24), (1000, 9), (1001, 5), (2048, 7),
+                      (4095, 3), (4096, 2), (9304, 3), (20000, 2), (100000, 2)]
+
+
+@pytest.mark.parametrize("shape", DECODER_SHAPES_F64, ids=["%dx%d" % s for s in DECODER_SHAPES_F64])
+def test_tile_and_row_major_decoders_f64(shape):
+    """The decoders for columns whose QWord-major stores would not be whole lines: several short columns per workgroup
+    (mode 2), row-major with the packed column in LDS (mode 4), and the automatic choice; add and overwrite; bit-exact."""
+    rows, cols = shape
+    for nbits, zt in VARIANTS:
+        g = datagen.normal_with_outliers(rows * 11 + nbits, rows, cols, 0.01, dtype=F64)
+        q, _ = oracle.quantize(g, zeros(rows, cols), nbits, zt)
+        prev = datagen.normal(rows * 13 + nbits, rows, cols, 1.0, dtype=F64)
+        for mode in (2, 4, 0):
+            say("f64 decoder", rows, cols, nbits, "mode", mode)
+            qz = MatrixQuantizerImpl.Create(0, False)
+            qz._set_tuning(unq_force_scalar=mode)
+            Q = QuantizedMatrix(rows, cols, nbits, 0, dtype=torch.float64)
+            Q.from_numpy(q)
+            for add in (False, True):
+                Out = Matrix.from_numpy(prev)
+                qz.UnquantizeAsync(Q, Out, add=add)
+                qz.WaitUnquantizeAsyncDone()
+                parity.check_unquantize(q, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
+        # output 8 bytes off a 16-byte boundary: another decoder serves it
+        big = torch.zeros(rows * cols + 2, dtype=torch.float64, device="cuda:0")
+        Out = Matrix(rows, cols, 0, big[1:1 + rows * cols], dtype=torch.float64)
+        qz.UnquantizeAsync(Q, Out)
+        qz.WaitUnquantizeAsyncDone()
+        parity.check_unquantize(q, rows, cols, nbits, Out.to_numpy())
+        assert float(big[0]) == 0.0 and float(big[-1]) == 0.0
 
 
 def test_out_of_place_host_buffer_and_slices_f64(quantizer):
