@@ -1,0 +1,91 @@
+"""Seeded random shapes through the automatic kernel choice, fp32 and fp64: heights drawn around every boundary of the
+kernel selection (multiples of 4 and 32 and their neighbours, 1024, 4096, 7168, 14336, 51200, 102400), few columns, every
+bit width, matrices at random offsets inside their allocations, residual in place or not. Every case: quantize against the
+oracle (codes under the GPU's own headers bit-exact, bounds and residuals within tolerance), unquantize bit-exact."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import datagen
+import oracle
+import parity
+from cntk_amd import Matrix, MatrixQuantizerImpl, QuantizedMatrix
+
+pytestmark = pytest.mark.gpu
+
+BOUNDARIES = [1, 4, 31, 32, 33, 64, 128, 255, 256, 1000, 1023, 1024, 1028, 2048, 2304, 4095, 4096, 4100, 4128, 6148, 7168, 7170, 9304,
+              12288, 14332, 14336, 14340, 16384, 20000, 32768, 51198, 51200, 51204, 65540, 102396, 102400, 102404]
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def draw_case(rng, is64):
+    r = rng.random()
+    if r < 0.5:
+        rows = int(rng.choice(BOUNDARIES))
+    elif r < 0.8:
+        rows = int(rng.integers(1, 3000))
+    else:
+        rows = int(rng.integers(1, 26000)) * 4
+    rows = max(1, rows + int(rng.choice([0, 0, 0, -1, 1, 2])))
+    max_cols = max(1, min(40, 400000 // rows))
+    cols = int(rng.integers(1, max_cols + 1))
+    nbits = int(rng.choice([1, 1, 1, 2, 4, 8, 16, 32] + ([64] if is64 else [])))
+    zt = bool(rng.integers(0, 2)) and nbits == 1
+    # element offsets of gradient, residual and output inside their allocations: mostly equal (then the kernels may
+    # align their accesses to cache lines), sometimes not
+    unit = 2 if is64 else 4
+    off = int(rng.integers(0, 8)) * unit if rng.random() < 0.5 else 0
+    offs = (off, off, off) if rng.random() < 0.7 else tuple(int(rng.integers(0, 9)) for _ in range(3))
+    in_place = bool(rng.integers(0, 2))
+    return rows, cols, nbits, zt, offs, in_place
+
+
+def place(a, off, tdt):
+    n = a.size
+    buf = torch.zeros(n + 64, dtype=tdt, device="cuda:0")
+    buf[off:off + n] = torch.from_numpy(a.reshape(-1, order="F").copy()).cuda()
+    return Matrix(a.shape[0], a.shape[1], 0, buf[off:off + n], dtype=tdt), buf
+
+
+@pytest.mark.parametrize("dtype,seed,count", [("f32", 11, 150), ("f32", 12, 150), ("f64", 13, 120), ("f64", 14, 120)])
+def test_random_shapes(dtype, seed, count):
+    is64 = dtype == "f64"
+    ndt, tdt = (np.float64, torch.float64) if is64 else (np.float32, torch.float32)
+    rng = np.random.default_rng(seed)
+    qz = MatrixQuantizerImpl.Create(0, False)
+    rep = parity.Report()
+    for n in range(count):
+        rows, cols, nbits, zt, offs, in_place = draw_case(rng, is64)
+        say("random case", dtype, seed, n, "rows", rows, "cols", cols, "nbits", nbits, "zeroThr", zt, "offsets", offs, "in place", in_place)
+        g = datagen.normal_with_outliers(seed * 1000 + n, rows, cols, 0.01, dtype=ndt)
+        r = datagen.normal(seed * 2000 + n, rows, cols, 0.002, dtype=ndt)
+        G, _g = place(g, offs[0], tdt)
+        R, rbuf = place(r, offs[1], tdt)
+        if in_place:
+            Rout, obuf = R, rbuf
+        else:
+            Rout, obuf = place(np.zeros_like(g, order="F"), offs[2], tdt)
+        Q = QuantizedMatrix(rows, cols, nbits, 0, dtype=tdt)
+        qz.QuantizeAsync(G, R, Q, Rout, zt)
+        qz.WaitQuantizeAsyncDone()
+        torch.cuda.synchronize()
+        q_gpu = Q.to_numpy()
+        parity.check_quantize(g, r, q_gpu, Rout.to_numpy(), nbits, zt, report=rep)
+        # nothing written outside the residual
+        off_o = offs[1] if in_place else offs[2]
+        assert float(obuf[:off_o].abs().sum()) == 0.0 and float(obuf[off_o + rows * cols:].abs().sum()) == 0.0
+        prev = datagen.normal(seed * 3000 + n, rows, cols, 1.0, dtype=ndt)
+        add = bool(n % 2)
+        Out, outbuf = place(prev, offs[2], tdt)
+        qz.UnquantizeAsync(Q, Out, add=add)
+        qz.WaitUnquantizeAsyncDone()
+        torch.cuda.synchronize()
+        parity.check_unquantize(q_gpu, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
+        assert float(outbuf[:offs[2]].abs().sum()) == 0.0 and float(outbuf[offs[2] + rows * cols:].abs().sum()) == 0.0
+    say("  ", rep)
