@@ -89,3 +89,51 @@ def test_random_shapes(dtype, seed, count):
         parity.check_unquantize(q_gpu, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
         assert float(outbuf[:offs[2]].abs().sum()) == 0.0 and float(outbuf[offs[2] + rows * cols:].abs().sum()) == 0.0
     say("  ", rep)
+
+
+@pytest.mark.parametrize("seed,count", [(21, 60), (22, 60)])
+def test_random_stripe_reductions(seed, count):
+    """Random stripes through the fused reduction: the fp32 aggregate bit-exact against the oracle (owner first, then
+    ascending rank), the requantized stripe like any quantize result, and the bytes of the reference's call sequence
+    (unquantize own stripe, add the others, quantize the aggregate) on the same handle."""
+    from test_gpu_stripe_reduce import gpu_stripe_reduce
+
+    rng = np.random.default_rng(seed)
+    qz = MatrixQuantizerImpl.Create(0, False)
+    rep = parity.Report()
+    heights = [h for h in BOUNDARIES if h <= 14336]
+    for n in range(count):
+        rows = int(rng.choice(heights)) if rng.random() < 0.6 else int(rng.integers(1, 3600)) * 4
+        rows = max(1, min(14336, rows + int(rng.choice([0, 0, 0, -1, 1]))))
+        k = int(rng.choice([1, 2, 3, 5, 8, 8, 13, 64]))
+        cols = int(rng.integers(1, max(2, min(48, 120000 // rows)) + 1))
+        nbits = int(rng.choice([1, 1, 1, 2, 4, 8, 16, 32]))
+        zt = bool(rng.integers(0, 2)) and nbits == 1
+        owner = int(rng.integers(0, k))
+        start, ncols = oracle.stripe_range(cols, owner, k)
+        say("random stripe", seed, n, "rows", rows, "cols", cols, "workers", k, "owner", owner, "stripe", start, ncols, "nbits", nbits, "zeroThr", zt)
+        if ncols == 0:
+            continue
+        gs = [datagen.normal(seed * 5000 + 70 * n + w, rows, cols) for w in range(k)]
+        zeros = np.zeros((rows, cols), np.float32, order="F")
+        qs = [oracle.quantize(g, zeros, nbits, zt, threads=8)[0] for g in gs]
+        sres = datagen.normal(seed * 7000 + n, rows, ncols, 0.003)
+        q_new, s_new, agg = gpu_stripe_reduce(qz, qs, owner, rows, cols, nbits, sres, zt, alias_out=bool(n % 2))
+        s_o = sres.copy(order="F")
+        agg_o = oracle.stripe_reduce([q.copy() for q in qs], owner, rows, cols, nbits, s_o, zt, threads=8)
+        assert parity.bits_equal(agg, agg_o), "fp32 aggregate differs from the oracle"
+        parity.check_quantize(agg_o, sres, q_new, s_new, nbits, zt, report=rep)
+        Agg = Matrix(rows, ncols)
+        qcol = oracle.qcol_bytes(nbits, rows)
+        for pos, w in enumerate([owner] + [w for w in range(k) if w != owner]):
+            Qw = QuantizedMatrix(rows, ncols, nbits, 0)
+            Qw.from_numpy(qs[w][start * qcol:(start + ncols) * qcol])
+            qz.UnquantizeAsync(Qw, Agg, add=(pos > 0))
+        S = Matrix.from_numpy(sres)
+        Qo = QuantizedMatrix(rows, ncols, nbits, 0)
+        qz.QuantizeAsync(Agg, S, Qo, S, zt)
+        qz.WaitQuantizeAsyncDone()
+        torch.cuda.synchronize()
+        assert np.array_equal(Qo.to_numpy(), q_new), "fused != call sequence (codes)"
+        assert parity.bits_equal(S.to_numpy(), s_new), "fused != call sequence (residual)"
+    say("  ", rep)
