@@ -56,7 +56,7 @@ def build_cpp_tests(verbose=False):
             continue
         exe = os.path.join(out_dir, name)
         # plain host C++ (no device code): the mirror classes only call the C ABI and the HIP runtime API
-        cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-Wall", src,
+        cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-Wall", "-pthread", src,
                "-D__HIP_PLATFORM_AMD__", "-I" + os.path.join(rocm, "include"), "-o", exe,
                "-L" + HERE, "-lcntk_amd_quantizer", "-L" + oracle_dir, "-loracle",
                "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(rocm, "lib"),

@@ -29,6 +29,7 @@
 #include "MatrixQuantizer.h"
 
 #include <algorithm>
+#include <future>
 #include <map>
 #include <tuple>
 #include <utility>
@@ -466,6 +467,14 @@ public:
         return headerCPU.numSamples != 0;
     }
 
+    // Work this worker issues from now on starts only after `event` (a hipEvent_t recorded by the caller) has completed.
+    // Needs the quantizers, i.e. a ResetState call before it.
+    void WaitForEvent(void* event)
+    {
+        if (!m_preAggGradQuantizers.empty())
+            detail::Check(cntkq_stream_wait_event(Gpu(*m_preAggGradQuantizers[0]).Handle(), event));
+    }
+
     const Matrix<ElemType>& GradientResidual(size_t i) const { return m_preAggGradQuantizers[i]->GetResidualMatrix(); }
     const Matrix<ElemType>* StripeResidual(size_t i) const
     {
@@ -540,9 +549,86 @@ public:
         return any;
     }
 
+    // The double-buffered aggregation of the reference (Source/1BitSGD/AllReduceDistGradAggregator.h:155-225, every
+    // worker at once): waits for the aggregation started by the previous call, exchanges the contents of the gradient
+    // matrices and headers with the buffered ones - the caller gets the gradients aggregated from the PREVIOUS call's
+    // input (zeros the first time) - and starts aggregating what it was just given on another host thread, ordered after
+    // everything already issued on the main (null) stream. As in the reference, aggregation starts only when state is
+    // reset or the header coming back (the previous aggregate's) saw samples; the return value says whether it started.
+    bool AggregateGradientsBuffered(const std::vector<std::vector<Matrix<ElemType>*>>& gradients, std::vector<DistGradHeader>& headers,
+                                    bool resetState)
+    {
+        const size_t K = m_workers.size();
+        if (gradients.size() != K || headers.size() != K)
+            throw std::invalid_argument("InProcessCluster: one gradient set and one header per worker");
+        WaitForPendingAggregation();
+        if (m_buffered.empty())
+        {
+            m_buffered.resize(K);
+            for (size_t r = 0; r < K; ++r)
+            {
+                for (auto* g : gradients[r])
+                    m_buffered[r].emplace_back(new Matrix<ElemType>(g->GetNumRows(), g->GetNumCols(), g->GetDeviceId()));
+                m_bufferedHeaders.emplace_back(headers[r].numEvalNode());
+            }
+        }
+        std::vector<std::vector<Matrix<ElemType>*>> fresh(K);
+        for (size_t r = 0; r < K; ++r)
+        {
+            if (gradients[r].size() != m_buffered[r].size())
+                throw std::logic_error("No buffered gradient matrix found corresponding to a gradient matrix to be aggregated!");
+            for (size_t i = 0; i < gradients[r].size(); ++i)
+            {
+                Matrix<ElemType>& b = *m_buffered[r][i];
+                if (b.GetNumRows() != gradients[r][i]->GetNumRows() || b.GetNumCols() != gradients[r][i]->GetNumCols() ||
+                    b.GetDeviceId() != gradients[r][i]->GetDeviceId())
+                    throw std::logic_error("No buffered gradient matrix found corresponding to a gradient matrix to be aggregated!");
+                gradients[r][i]->Swap(b);
+                fresh[r].push_back(&b);
+            }
+            std::swap(headers[r], m_bufferedHeaders[r]);
+        }
+        if (!(resetState || headers[0].numSamples != 0))
+            return false;
+        int device = 0;
+        detail::HipCheck(hipGetDevice(&device), "hipGetDevice");
+        hipEvent_t computed = nullptr;
+        detail::HipCheck(hipEventCreateWithFlags(&computed, hipEventDisableTiming), "hipEventCreate");
+        detail::HipCheck(hipEventRecord(computed, nullptr), "hipEventRecord");
+        for (size_t r = 0; r < K; ++r)
+            m_workers[r]->ResetState(fresh[r], false); // the quantizers exist before the other thread needs their stream
+        m_pending = std::async(std::launch::async, [this, fresh, device, computed, resetState]() {
+            detail::HipCheck(hipSetDevice(device), "hipSetDevice");
+            m_workers[0]->WaitForEvent(computed);
+            AggregateGradients(fresh, m_bufferedHeaders, resetState, true);
+            detail::HipCheck(hipEventDestroy(computed), "hipEventDestroy");
+        });
+        return true;
+    }
+
+    void WaitForPendingAggregation()
+    {
+        if (m_pending.valid())
+            m_pending.get();
+    }
+
+    ~InProcessCluster()
+    {
+        try
+        {
+            WaitForPendingAggregation();
+        }
+        catch (...)
+        {
+        }
+    }
+
 private:
     InProcessTransport m_transport;
     std::vector<std::unique_ptr<AllReduceDistGradAggregator<ElemType>>> m_workers;
+    std::vector<std::vector<std::unique_ptr<Matrix<ElemType>>>> m_buffered;
+    std::vector<DistGradHeader> m_bufferedHeaders;
+    std::future<void> m_pending;
 };
 
 } // namespace cntk_amd

@@ -144,6 +144,16 @@ public:
         return Matrix(m_data + startColumn * m_rows, m_rows, numCols, m_device);
     }
 
+    // exchange of contents (std::swap of two matrices in the reference's double-buffered aggregation)
+    void Swap(Matrix& o) noexcept
+    {
+        std::swap(m_data, o.m_data);
+        std::swap(m_rows, o.m_rows);
+        std::swap(m_cols, o.m_cols);
+        std::swap(m_device, o.m_device);
+        std::swap(m_owner, o.m_owner);
+    }
+
     void SetValue(ElemType v)
     {
         std::vector<ElemType> host(GetNumElements(), v);

@@ -280,13 +280,101 @@ static void EmptyMinibatchAndReset()
         CHECK(!SameBits(*s1[0].ptrs[i], *s3[0].ptrs[i]), "a silent worker changes the aggregate");
 }
 
+// The double-buffered aggregation (Source/1BitSGD/AllReduceDistGradAggregator.h:155-225): call t hands back what a
+// synchronous aggregator produced for the input of call t - 1, bit for bit, and zeros the first time; without resetState
+// and with no samples in the header that comes back, nothing is started.
+static void BufferedAggregation()
+{
+    const Shapes shapes = {{2048, 24}, {429, 37}, {64, 5}};
+    const size_t K = 4;
+    const int steps = 4;
+    InProcessCluster<float> sync(K, 0, 1, false), buffered(K, 0, 1, false);
+    std::vector<std::vector<std::vector<float>>> expected; // [step][matrix] of worker 0 from the synchronous cluster
+    std::vector<size_t> expectedSamples;
+    for (int step = 0; step <= steps; ++step)
+    {
+        std::vector<std::vector<std::vector<float>>> host(K);
+        for (size_t r = 0; r < K; ++r)
+            for (size_t i = 0; i < shapes.size(); ++i)
+                host[r].push_back(Gaussian(shapes[i].first * shapes[i].second, 0.01f, 5150 + 1000 * step + 10 * r + i));
+        std::vector<WorkerSet> a = MakeGradients(shapes, K, host), b = MakeGradients(shapes, K, host);
+        std::vector<std::vector<Matrix<float>*>> ga, gb;
+        std::vector<DistGradHeader> ha, hb;
+        for (size_t r = 0; r < K; ++r)
+        {
+            ga.push_back(a[r].ptrs);
+            gb.push_back(b[r].ptrs);
+            ha.emplace_back(1);
+            ha.back().numSamples = 7 + r + step;
+            hb.push_back(ha.back());
+        }
+        if (step < steps)
+        {
+            sync.AggregateGradients(ga, ha, step == 0, true);
+            detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize");
+            expected.emplace_back();
+            for (size_t i = 0; i < shapes.size(); ++i)
+            {
+                auto x = a[0].ptrs[i]->CopyToArray();
+                expected.back().emplace_back(x.get(), x.get() + a[0].ptrs[i]->GetNumElements());
+            }
+            expectedSamples.push_back(ha[0].numSamples);
+        }
+        const bool started = buffered.AggregateGradientsBuffered(gb, hb, step == 0);
+        CHECK(started, "step %d: aggregation started", step);
+        for (size_t r = 0; r < K; ++r)
+            for (size_t i = 0; i < shapes.size(); ++i)
+            {
+                auto x = b[r].ptrs[i]->CopyToArray();
+                const size_t n = b[r].ptrs[i]->GetNumElements();
+                if (step == 0)
+                {
+                    bool zero = true;
+                    for (size_t e = 0; e < n; ++e)
+                        zero = zero && x[e] == 0.0f;
+                    CHECK(zero && hb[r].numSamples == 0, "the first call hands back zeros");
+                }
+                else
+                    CHECK(std::memcmp(x.get(), expected[step - 1][i].data(), n * 4) == 0 && hb[r].numSamples == expectedSamples[step - 1],
+                          "step %d worker %zu matrix %zu: the previous call's aggregate", step, r, i);
+            }
+    }
+    buffered.WaitForPendingAggregation();
+
+    // nothing starts without resetState while the header that comes back has no samples; the gradients are exchanged all the same
+    InProcessCluster<float> idle(K, 0, 1, false);
+    std::vector<std::vector<std::vector<float>>> host(K);
+    for (size_t r = 0; r < K; ++r)
+        for (size_t i = 0; i < shapes.size(); ++i)
+            host[r].push_back(Gaussian(shapes[i].first * shapes[i].second, 0.01f, 77 + 10 * r + i));
+    std::vector<WorkerSet> first = MakeGradients(shapes, K, host), second = MakeGradients(shapes, K, host);
+    std::vector<std::vector<Matrix<float>*>> g1, g2;
+    std::vector<DistGradHeader> h1, h2;
+    for (size_t r = 0; r < K; ++r)
+    {
+        g1.push_back(first[r].ptrs);
+        g2.push_back(second[r].ptrs);
+        h1.emplace_back(1);
+        h1.back().numSamples = 3;
+        h2.emplace_back(1);
+        h2.back().numSamples = 4;
+    }
+    CHECK(!idle.AggregateGradientsBuffered(g1, h1, false), "no aggregation without reset and without samples coming back");
+    CHECK(idle.AggregateGradientsBuffered(g2, h2, false), "the header coming back now has samples");
+    CHECK(h2[0].numSamples == 3, "the header handed back is the first call's own");
+    auto x = second[0].ptrs[0]->CopyToArray();
+    CHECK(std::memcmp(x.get(), host[0][0].data(), host[0][0].size() * 4) == 0, "and so are the gradients: never aggregated");
+    idle.WaitForPendingAggregation();
+}
+
 int main()
 {
     try
     {
         struct T { const char* name; void (*fn)(); };
         const T tests[] = {{"QuantizedAllReduceVariantsBitIdentical", VariantsAreBitIdentical}, {"QuantizedAllReduceAgainstOracle", AgainstOracle},
-                           {"QuantizedAllReduceUnquantizedSelfStripe", UnquantizedSelfStripe}, {"QuantizedAllReduceEmptyMinibatchAndReset", EmptyMinibatchAndReset}};
+                           {"QuantizedAllReduceUnquantizedSelfStripe", UnquantizedSelfStripe}, {"QuantizedAllReduceEmptyMinibatchAndReset", EmptyMinibatchAndReset},
+                           {"QuantizedAllReduceBufferedAggregation", BufferedAggregation}};
         for (const T& t : tests)
         {
             const int before = g_failures;

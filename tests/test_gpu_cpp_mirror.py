@@ -31,7 +31,7 @@ def test_cpp_allreduce_aggregator_suite():
     print(res.stdout)
     print(res.stderr[-4000:])
     assert res.returncode == 0, "C++ aggregator tests failed"
-    for name in ("VariantsBitIdentical", "AgainstOracle", "UnquantizedSelfStripe", "EmptyMinibatchAndReset"):
+    for name in ("VariantsBitIdentical", "AgainstOracle", "UnquantizedSelfStripe", "EmptyMinibatchAndReset", "BufferedAggregation"):
         assert "QuantizedAllReduce%s has passed" % name in res.stdout
 
 
