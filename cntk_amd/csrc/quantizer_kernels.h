@@ -1874,7 +1874,10 @@ __device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q,
     __syncthreads();
     const uint32_t elems = ncols * t.rows;
     float* o = out + (size_t) col0 * t.rows;
-    for (uint32_t i = 4 * tid; i < elems; i += 1024)
+    // slots dealt by 128-byte lines: slot v = tid, tid + 256, ... holds the group of four that starts at element
+    // 4 * (v - shift), shift = the tile's offset into its line in 16-byte pieces
+    const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o) >> 4) & 7u);
+    for (uint32_t i = 4 * ((tid < shift ? tid + 256 : tid) - shift); i < elems; i += 1024)
     {
         uint32_t c = small_div(i, t.rows, t.rows_magic);
         uint32_t r = i - c * t.rows;

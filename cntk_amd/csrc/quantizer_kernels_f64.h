@@ -757,7 +757,9 @@ __global__ __launch_bounds__(256) void unquantize_tile_kernel(const char* __rest
     __syncthreads();
     const uint32_t elems = ncols * t.rows;
     double* o = out + (size_t) col0 * t.rows;
-    for (uint32_t i = 2 * tid; i < elems; i += 512)
+    // slots dealt by 128-byte lines, as in the fp32 decoder
+    const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o) >> 4) & 7u);
+    for (uint32_t i = 2 * ((tid < shift ? tid + 256 : tid) - shift); i < elems; i += 512)
     {
         uint32_t c = small_div(i, t.rows, t.rows_magic);
         uint32_t r = i - c * t.rows;

@@ -432,7 +432,7 @@ struct UnquantizePlan
 
 constexpr size_t kUnqRowsMaxLds = 48 * 1024;
 constexpr uint32_t kUnqRowsChunk = 2048;
-constexpr size_t kUnqTileMaxRows = 4096;  // 4 columns of that height: 16384 elements, small enough for the magic divisions
+constexpr size_t kUnqTileMaxRows = 16384; // 4 columns of that height: 65536 elements, small enough for the magic divisions
 constexpr size_t kUnqTileElems = 4096;    // values per workgroup the tile decoder aims for
 constexpr size_t kUnqRowsMinRows = 1024;  // from this height on a column keeps the 256 threads of the row-major decoder busy
 
@@ -492,7 +492,7 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
         t.rows_magic = rows > 1 ? (uint32_t) ((((uint64_t) 1 << 32) + rows - 1) / rows) : 0u;
         t.nq_magic = nq > 1 ? (uint32_t) ((((uint64_t) 1 << 32) + nq - 1) / nq) : 0u;
         const uint64_t blocks = (cols + cpt - 1) / cpt;
-        if (blocks <= 0x7FFFFFFFull)
+        if (blocks <= 0x7FFFFFFFull && unq_tile_lds_bytes(t) <= 64 * 1024)
         {
             t.blocks = (uint32_t) blocks;
             p.kind = kUnqTile;

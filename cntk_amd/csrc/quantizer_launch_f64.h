@@ -226,7 +226,7 @@ inline hipError_t launch_unquantize_n(hipStream_t s, LaunchEvents ev, const char
 }
 
 constexpr size_t kUnqRowsMinRows64 = 512;  // from this height on a column keeps the 256 threads of the row-major decoder busy
-constexpr size_t kUnqTileMaxRows64 = 4096;
+constexpr size_t kUnqTileMaxRows64 = 16384;
 constexpr size_t kUnqTileElems64 = 2048;   // values per workgroup the tile decoder aims for
 
 template <int NBITS>

@@ -196,7 +196,7 @@ def test_unquantize_variants_f64(quantizer):
 
 
 DECODER_SHAPES_F64 = [(1, 1), (1, 9), (3, 5), (31, 13), (64, 100), (147, 64), (429, 37), (512, 24), (1000, 9), (1001, 5), (2048, 7),
-                      (4095, 3), (4096, 2), (9304, 3), (20000, 2), (100000, 2)]
+                      (4095, 3), (4096, 2), (4097, 3), (9304, 3), (9305, 2), (16383, 2), (20000, 2), (100000, 2)]
 
 
 @pytest.mark.parametrize("shape", DECODER_SHAPES_F64, ids=["%dx%d" % s for s in DECODER_SHAPES_F64])

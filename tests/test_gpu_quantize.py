@@ -268,7 +268,7 @@ def test_unquantize_variants(quantizer):
 
 
 TILE_DECODER_SHAPES = [(1, 1), (1, 9), (2, 7), (3, 5), (5, 3), (31, 13), (32, 8), (33, 41), (64, 100), (147, 64), (256, 1031),
-                       (429, 37), (512, 24), (1000, 9), (1001, 5), (1024, 3), (2047, 2), (2048, 7), (4096, 5), (4095, 3)]
+                       (429, 37), (512, 24), (1000, 9), (1001, 5), (1024, 3), (2047, 2), (2048, 7), (4096, 5), (4095, 3), (4097, 3), (9305, 2), (16383, 2), (16385, 2)]
 
 
 @pytest.mark.parametrize("shape", TILE_DECODER_SHAPES, ids=["%dx%d" % s for s in TILE_DECODER_SHAPES])
