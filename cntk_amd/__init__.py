@@ -411,8 +411,8 @@ class MatrixQuantizerImpl:
     def WaitStripeReduceDone(self):
         _check(lib().cntkq_wait_stripe_reduce_done(self._h))
 
-    def _set_tuning(self, quantize_path=0, tile_gs=0, unq_slots=0, unq_force_scalar=0, tile_stage=-1):
-        _check(lib().cntkq_debug_set_tuning(self._h, quantize_path, tile_gs, unq_slots, unq_force_scalar, tile_stage))
+    def _set_tuning(self, quantize_path=0, tile_gs=0, unq_slots=0, unq_mode=0, tile_stage=-1):
+        _check(lib().cntkq_debug_set_tuning(self._h, quantize_path, tile_gs, unq_slots, unq_mode, tile_stage))
 
 
 class MatrixQuantizer:

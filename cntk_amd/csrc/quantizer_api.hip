@@ -1109,7 +1109,7 @@ int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h)
 
 // ---- hooks for tests and tuning runs (not part of the public header) --------------------------------
 
-int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_gs, unsigned unq_slots, int unq_force_scalar,
+int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_gs, unsigned unq_slots, int unq_mode,
                            int tile_stage)
 {
     if (h == nullptr)
@@ -1121,7 +1121,7 @@ int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_
     h->tune.quantize_path = quantize_path;
     h->tune.tile_gs = tile_gs;
     h->tune.unq_slots = unq_slots;
-    h->tune.unq_force_scalar = unq_force_scalar;
+    h->tune.unq_mode = unq_mode;
     h->tune.tile_stage = tile_stage;
     return CNTKQ_OK;
 }

@@ -10,13 +10,15 @@ extern "C" {
 
 /* Forces kernel choices on a handle:
  *   quantize_path    0 = automatic, 1 = LDS column tile, 2 = tall-column (global re-read),
- *                    3 = one wavefront per column (1 bit, 2048 or 4096 rows only)
+ *                    3 = one workgroup per column, column in LDS (fp32, rows a multiple of 4 up to 14336),
+ *                    4 = one workgroup per column, column in registers (rows a multiple of 4 (fp64: even), below 32 (64) bits)
  *   tile_gs          0 = automatic, else threads per column in the tile statistics phase (power of two, 8..256)
- *   unq_slots        0 = automatic, else bit positions decoded per thread by unquantize
- *   unq_force_scalar non-zero = never use the 16-byte store variant of unquantize
+ *   unq_slots        0 = automatic, else bit positions decoded per thread by the QWord-major unquantize
+ *   unq_mode         0 = automatic, 1 = QWord-major decoder with one store per value, 2 = tile decoder wherever it can run,
+ *                    3 = automatic without the tile decoder, 4 = row-major decoder wherever it can run
  *   tile_stage       -1 = automatic, 0 = tile kernels write the residual straight to memory, 1 = through LDS */
 int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_gs, unsigned unq_slots,
-                           int unq_force_scalar, int tile_stage);
+                           int unq_mode, int tile_stage);
 
 /* Ties caller-owned hipEvent_t objects (either may be NULL) to the NEXT kernel this handle launches: start_event is
  * set when that kernel begins, stop_event when it has finished, by the dispatch itself. Used to time single kernels

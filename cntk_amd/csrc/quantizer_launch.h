@@ -34,7 +34,7 @@ struct LaunchTuning
     int tile_stage = -1;    // -1 = automatic; 0 / 1 = residual written straight to memory / staged through LDS
     uint32_t tile_threads = 0; // 0 = automatic; else workgroup size of the tile kernels (64, 128, 256)
     uint32_t unq_slots = 0; // 0 = default; else bit positions per thread in unquantize
-    int unq_force_scalar = 0; // 0 automatic, 1 QWord-major with 4-byte stores, 2 / 4 tile / row-major decoder wherever it can run, 3 automatic without the tile decoder
+    int unq_mode = 0; // 0 automatic, 1 QWord-major with 4-byte stores, 2 / 4 tile / row-major decoder wherever it can run, 3 automatic without the tile decoder
 };
 
 // Events tied to the kernel dispatch itself (its completion signal), not recorded as separate stream
@@ -446,7 +446,7 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
     const size_t vpw = 32 / nbits;
     const size_t nq = qwords_per_col(rows, nbits);
     std::memset(&p.tile, 0, sizeof p.tile);
-    const int mode = tune.unq_force_scalar;
+    const int mode = tune.unq_mode;
     const bool out16 = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
     const bool slots_free = tune.unq_slots == 0;
     // QWord-major decoder with 16-byte stores. It is at its best when every bit position of a column is a run of whole

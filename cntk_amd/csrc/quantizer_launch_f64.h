@@ -263,7 +263,7 @@ inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* 
     const size_t vpw = 64 / nbits;
     const size_t nq = qwords_per_col(rows, nbits);
     const bool out16 = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
-    const int mode = tune.unq_force_scalar; // 0 automatic, 1 QWord-major 8-byte stores, 2 / 4 tile / row-major decoder wherever it can run, 3 QWord-major
+    const int mode = tune.unq_mode; // 0 automatic, 1 QWord-major 8-byte stores, 2 / 4 tile / row-major decoder wherever it can run, 3 QWord-major
     // The QWord-major decoder is at its best when every bit position of a column is a run of whole 128-byte lines. Other
     // columns: row-major decoder from 512 rows on, tile decoder for shorter ones (the choices of the fp32 side).
     const bool vec_ideal = nq % 16 == 0 && rows % 16 == 0 && rows * nbits == nq * 64 && out16;

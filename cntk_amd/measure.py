@@ -44,7 +44,7 @@ def main():
     sfx = "_f64" if args.dtype == "f64" else ""
     L = cntk_amd.lib()
     qz = MatrixQuantizerImpl.Create(0, False)
-    qz._set_tuning(quantize_path=args.path, unq_force_scalar=args.unq_mode)
+    qz._set_tuning(quantize_path=args.path, unq_mode=args.unq_mode)
     h = qz._h
 
     elems = rows * cols

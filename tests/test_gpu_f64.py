@@ -185,7 +185,7 @@ def test_unquantize_variants_f64(quantizer):
                 for scalar in (0, 1):
                     say("f64 unquantize", rows, cols, nbits, "slots", slots, "scalar", scalar)
                     qz = MatrixQuantizerImpl.Create(0, False)
-                    qz._set_tuning(unq_slots=slots, unq_force_scalar=scalar)
+                    qz._set_tuning(unq_slots=slots, unq_mode=scalar)
                     Q = QuantizedMatrix(rows, cols, nbits, 0, dtype=torch.float64)
                     Q.from_numpy(q)
                     for add in (False, True):
@@ -211,7 +211,7 @@ def test_tile_and_row_major_decoders_f64(shape):
         for mode in (2, 4, 0):
             say("f64 decoder", rows, cols, nbits, "mode", mode)
             qz = MatrixQuantizerImpl.Create(0, False)
-            qz._set_tuning(unq_force_scalar=mode)
+            qz._set_tuning(unq_mode=mode)
             Q = QuantizedMatrix(rows, cols, nbits, 0, dtype=torch.float64)
             Q.from_numpy(q)
             for add in (False, True):

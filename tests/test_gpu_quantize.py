@@ -257,7 +257,7 @@ def test_unquantize_variants(quantizer):
                 for scalar in (0, 1):
                     say("unquantize", rows, cols, nbits, "slots", slots, "scalar", scalar)
                     qz = MatrixQuantizerImpl.Create(0, False)
-                    qz._set_tuning(unq_slots=slots, unq_force_scalar=scalar)
+                    qz._set_tuning(unq_slots=slots, unq_mode=scalar)
                     Q = QuantizedMatrix(rows, cols, nbits, 0)
                     Q.from_numpy(q)
                     for add in (False, True):
@@ -284,7 +284,7 @@ def test_tile_decoder(shape):
         for mode in (2, 0, 3):
             say("tile decoder", rows, cols, nbits, "mode", mode)
             qz = MatrixQuantizerImpl.Create(0, False)
-            qz._set_tuning(unq_force_scalar=mode)
+            qz._set_tuning(unq_mode=mode)
             Q = QuantizedMatrix(rows, cols, nbits, 0)
             Q.from_numpy(q)
             for add in (False, True):
