@@ -1722,6 +1722,30 @@ struct UnqRowGeom
     uint64_t qcol;
 };
 
+// Which (column, chunk) a workgroup of the row-major decoder takes. Consecutive workgroups go to the 8 XCDs in turn and
+// every XCD has its own L2, so the chunks of one column are given to workgroups 8 apart: they then read the column's
+// packed record through one L2 instead of fetching it once per XCD. Columns are taken in groups of 8; what is left over
+// at the end is dealt column by column.
+__device__ __forceinline__ void unq_rows_block_to_chunk(uint32_t block, uint32_t chunks, uint32_t blocks, uint32_t& c, uint32_t& ch)
+{
+    const uint32_t per_group = 8 * chunks;
+    const uint32_t grouped = (blocks / per_group) * per_group;
+    if (block < grouped)
+    {
+        const uint32_t grp = block / per_group;
+        const uint32_t rem = block - grp * per_group;
+        ch = rem >> 3;
+        c = grp * 8 + (rem & 7u);
+    }
+    else
+    {
+        const uint32_t b = block - grouped;
+        const uint32_t cc = b / chunks;
+        ch = b - cc * chunks;
+        c = grouped / chunks + cc;
+    }
+}
+
 template <int NBITS>
 __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q, float* out, const UnqRowGeom& t, int add, uint32_t block,
                                                      uint32_t* words)
@@ -1729,8 +1753,8 @@ __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q,
     constexpr uint32_t SHIFT = NBITS & 31;
     constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
     const uint32_t tid = threadIdx.x;
-    const uint32_t c = block / t.chunks;
-    const uint32_t ch = block - c * t.chunks;
+    uint32_t c, ch;
+    unq_rows_block_to_chunk(block, t.chunks, t.blocks, c, ch);
     const char* qc = q + (size_t) c * t.qcol;
     const float* gh = reinterpret_cast<const float*>(qc);
     const float lo = gh[0];

@@ -660,8 +660,8 @@ __global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __rest
     extern __shared__ f32x4 smem_v4[];
     uint64_t* words = reinterpret_cast<uint64_t*>(smem_v4);
     const uint32_t tid = threadIdx.x;
-    const uint32_t c = blockIdx.x / t.chunks;
-    const uint32_t ch = blockIdx.x - c * t.chunks;
+    uint32_t c, ch;
+    unq_rows_block_to_chunk(blockIdx.x, t.chunks, t.blocks, c, ch);
     const char* qc = q + (size_t) c * t.qcol;
     const double* gh = reinterpret_cast<const double*>(qc);
     const ValueQ vq = make_vq<NBITS>(gh[0], gh[1]);
