@@ -578,6 +578,8 @@ struct UnqGeom
     uint32_t slots;
     uint32_t per_col; // groups * chunks
     uint32_t items;   // per_col * cols
+    uint32_t swz_members; // > 1: workgroups regrouped by XCD (unq_xcd_block)
+    uint32_t swz_gw;
     uint64_t qcol;
 };
 
@@ -585,7 +587,8 @@ template <int NBITS, int WV>
 __global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, double* out, UnqGeom t, int add)
 {
     using PS = PackShape<NBITS>;
-    const uint64_t id64 = (uint64_t) blockIdx.x * 256 + threadIdx.x;
+    const uint32_t block = t.swz_members > 1 ? unq_xcd_block(blockIdx.x, t.items / 256, t.swz_members, t.swz_gw) : blockIdx.x;
+    const uint64_t id64 = (uint64_t) block * 256 + threadIdx.x;
     if (id64 >= t.items)
         return;
     const uint32_t id = (uint32_t) id64;

@@ -571,6 +571,19 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
         return p; // not ok
     t.per_col = (uint32_t) per_col;
     t.items = (uint32_t) items;
+    // several workgroups per column that read the same QWords: regroup them by XCD (whole workgroups per column only)
+    t.swz_members = 0;
+    t.swz_gw = 1;
+    if (per_col % 256 == 0 && per_col > 256)
+    {
+        if (t.groups <= 256)
+            t.swz_members = (uint32_t) (per_col / 256); // every workgroup of the column spans all its QWords
+        else if (t.groups % 256 == 0)
+        {
+            t.swz_members = t.chunks;
+            t.swz_gw = t.groups / 256;
+        }
+    }
     t.qcol = qcol_bytes(nbits, rows);
     p.kind = vec ? kUnqVec4 : kUnqScalar;
     p.blocks = (uint32_t) ((items + 255) / 256);

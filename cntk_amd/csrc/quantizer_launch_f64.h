@@ -346,6 +346,19 @@ inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* 
         return hipErrorInvalidValue;
     t.per_col = (uint32_t) per_col;
     t.items = (uint32_t) items;
+    // several workgroups per column that read the same QWords: regroup them by XCD (whole workgroups per column only)
+    t.swz_members = 0;
+    t.swz_gw = 1;
+    if (per_col % 256 == 0 && per_col > 256)
+    {
+        if (t.groups <= 256)
+            t.swz_members = (uint32_t) (per_col / 256);
+        else if (t.groups % 256 == 0)
+        {
+            t.swz_members = t.chunks;
+            t.swz_gw = t.groups / 256;
+        }
+    }
     t.qcol = qcol_bytes(nbits, rows);
     const char* qc = static_cast<const char*>(q);
     const int a = add ? 1 : 0;
