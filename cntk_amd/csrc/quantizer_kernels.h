@@ -1145,8 +1145,18 @@ struct RegGeom
     uint64_t qcol;
 };
 
-constexpr uint32_t kRegRedSlots = 48;
-constexpr int kRegMaxShiftPer = 16; // most pieces per thread of a register kernel that deals its slots by lines // three partial results for each of up to 16 waves
+// The value of x, but unknown to the compiler. The register kernels use the same indices and bounds checks in every
+// phase (loads of the gradient, loads of the residual, sums, stores); recognised as common subexpressions they would
+// all be kept in registers from the first phase to the last (a 64-bit address pair for every piece), which costs more
+// registers than the column itself. Recomputing them from an opaque copy of the thread index is a few instructions.
+__device__ __forceinline__ uint32_t opaque(uint32_t x)
+{
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
+constexpr uint32_t kRegRedSlots = 48; // three partial results for each of up to 16 waves
+constexpr int kRegMaxShiftPer = 25;   // most pieces per thread of a register kernel that deals its slots by lines (all of them)
 
 __host__ __device__ inline size_t reg_lds_bytes(const RegGeom& c)
 {
@@ -1161,11 +1171,14 @@ constexpr int reg_waves()
     // (a looser budget does not help: given 128 registers the compiler hoists work until it spills)
     if (T == 1024)
         return PER <= 6 ? 8 : 4; // a workgroup is 4 waves on every SIMD: two of them fit, or one
-    int w = 512 / (4 * PER + (PER >= 10 ? 48 : 40));
+    int w = 512 / (4 * PER + 40);
     return w > 8 ? 8 : (w < T / 256 ? T / 256 : w);
 }
 
-template <int NBITS, bool ZT, int T, int PER>
+// EDGE: the column need not start on a 16-byte boundary nor hold a multiple of 4 elements: up to 3 elements before the
+// first aligned piece and up to 3 after the last are held, one each, by threads 0..5 and take part in every phase after
+// the thread's pieces. (c.pieces then only bounds the pieces; the count is taken from the column's address.)
+template <int NBITS, bool ZT, int T, int PER, bool EDGE = false>
 __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, PER>(), reg_waves<T, PER>()))) void quantize_reg_kernel(
     const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q, RegGeom c)
 {
@@ -1181,26 +1194,42 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     char* qc = q + (size_t) blockIdx.x * c.qcol;
     for (uint32_t x = tid; x < c.nq; x += T)
         words[x] = 0u;
-    const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base);
-    const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base);
+    uint32_t head = 0, tail = 0, pieces = c.pieces;
+    if constexpr (EDGE)
+    {
+        head = (4u - (uint32_t) ((reinterpret_cast<uintptr_t>(r_in + base) >> 2) & 3u)) & 3u; // elements before the first aligned piece
+        pieces = (c.rows - head) >> 2;
+        tail = c.rows - head - 4 * pieces;
+    }
+    const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base + head);
+    const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base + head);
+    // the edge element of this thread, if it has one
+    const bool has_edge = EDGE && tid < head + tail;
+    const uint32_t edge_at = tid < head ? tid : c.rows - tail + (tid - head);
+    float edge = 0.0f;
+    if (has_edge)
+        edge = g[base + edge_at] + r_in[base + edge_at];
     // Slot v = tid + T * u holds piece v - shift, where shift (0..7) is the column's offset into its 128-byte line in
     // pieces: every wavefront's 64 slots then cover whole lines, also in columns that start inside a line (9304 rows: every
     // column but each fourth). Slots before the column or past its end read a piece of the column all the same (no
     // branch, all loads in flight together) and are left out of every sum and store.
-    // (not with more than 16 pieces per thread: there the registers are needed for the column itself)
-    const uint32_t shift = PER <= kRegMaxShiftPer ? column_shift(r_in + base, c.line_shift) : 0u;
-    const uint32_t last = c.pieces - 1;
+    const uint32_t shift = PER <= kRegMaxShiftPer ? column_shift(r_in + base + head, c.line_shift) : 0u;
+    const uint32_t last = pieces - 1;
     f32x4 a[PER];
+    {
+        const uint32_t t = opaque(tid);
 #pragma unroll
-    for (int u = 0; u < PER; ++u)
-        a[u] = __builtin_nontemporal_load(g4 + slot_piece(tid + T * u, shift, last));
+        for (int u = 0; u < PER; ++u)
+            a[u] = __builtin_nontemporal_load(g4 + slot_piece(t + T * u, shift, last));
+    }
 #pragma unroll
     for (int u0 = 0; u0 < PER; u0 += 4)
     {
+        const uint32_t t = opaque(tid);
         f32x4 b[4];
 #pragma unroll
         for (int u = u0; u < u0 + 4 && u < PER; ++u)
-            b[u - u0] = __builtin_nontemporal_load(r4 + slot_piece(tid + T * u, shift, last));
+            b[u - u0] = __builtin_nontemporal_load(r4 + slot_piece(t + T * u, shift, last));
 #pragma unroll
         for (int u = u0; u < u0 + 4 && u < PER; ++u)
             a[u] = a[u] + b[u - u0];
@@ -1210,12 +1239,15 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     if constexpr (need_stat)
     {
         float stat = 0.0f;
+        const uint32_t t = opaque(tid);
 #pragma unroll
         for (int u = 0; u < PER; ++u)
         {
             const float with = colg_add_piece<NBITS>(stat, a[u]);
-            stat = slot_valid(tid + T * u, shift, c.pieces) ? with : stat;
+            stat = slot_valid(t + T * u, shift, pieces) ? with : stat;
         }
+        if (has_edge)
+            stat += NBITS == 1 ? edge : edge * edge;
         stat = wave_sum(stat);
         if (lane == 0)
             red[wave] = stat;
@@ -1235,16 +1267,24 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
         const float mean = ZT ? 0.0f : total / (float) c.rows;
         float s0 = 0.0f, s1 = 0.0f;
         uint32_t n0 = 0;
+        const uint32_t t = opaque(tid);
 #pragma unroll
         for (int u = 0; u < PER; ++u)
         {
             float t0 = s0, t1 = s1;
             uint32_t tn = n0;
             split_add_piece(a[u], mean, t0, t1, tn);
-            const bool valid = slot_valid(tid + T * u, shift, c.pieces);
+            const bool valid = slot_valid(t + T * u, shift, pieces);
             s0 = valid ? t0 : s0;
             s1 = valid ? t1 : s1;
             n0 = valid ? tn : n0;
+        }
+        if (has_edge)
+        {
+            const bool below = edge < mean;
+            s0 += below ? edge : 0.0f;
+            s1 += below ? 0.0f : edge;
+            n0 += below ? 1u : 0u;
         }
         s0 = wave_sum(s0);
         s1 = wave_sum(s1);
@@ -1281,18 +1321,19 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     const ValueQ vq = make_vq<NBITS>(lo, hi);
     const float val0 = unquantize_value<NBITS>(vq, 0u);
     const float val1 = unquantize_value<NBITS>(vq, 1u);
-    f32x4* o4 = reinterpret_cast<f32x4*>(r_out + base);
+    f32x4* o4 = reinterpret_cast<f32x4*>(r_out + base + head);
     // the first element of this thread's first slot inside the column is bit position k of QWord w; the elements after it
     // are the following QWords, the slots after it lie 4 * T elements further on
     const uint32_t ufirst = tid < shift ? 1u : 0u;
-    const uint32_t e0 = 4 * (tid + T * ufirst - shift);
+    const uint32_t e0 = head + 4 * (tid + T * ufirst - shift);
     uint32_t k = e0 / c.nq;
     uint32_t w = e0 - k * c.nq;
+    const uint32_t to = opaque(tid);
 #pragma unroll
     for (int u = 0; u < PER; ++u)
     {
-        const uint32_t p = tid + T * u - shift;
-        if (slot_valid(tid + T * u, shift, c.pieces))
+        const uint32_t p = to + T * u - shift;
+        if (slot_valid(to + T * u, shift, pieces))
         {
             f32x4 res;
             uint32_t kk = k, ww = w;
@@ -1325,6 +1366,190 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
                 w -= c.nq;
                 ++k;
             }
+        }
+    }
+    if (has_edge)
+    {
+        const uint32_t code = quantize_value<NBITS, ZT>(vq, edge);
+        float back;
+        if constexpr (NBITS == 1)
+            back = code ? val1 : val0;
+        else
+            back = unquantize_value<NBITS>(vq, code);
+        r_out[base + edge_at] = edge - back;
+        const uint32_t ek = edge_at / c.nq;
+        atomicOr(&words[edge_at - ek * c.nq], code << (ek * PS::SHIFT));
+    }
+    __syncthreads();
+    uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
+    for (uint32_t x = tid; x < c.nq; x += T)
+        bits[x] = words[x];
+}
+
+// ---- the same for tall columns of any height and alignment: elements instead of pieces ----------------------
+//
+// Thread tid of 1024 keeps elements tid, tid + 1024, ... (at most EPT) of the column in registers, loaded and stored one
+// float at a time: consecutive lanes touch consecutive floats, so nothing depends on the height being a multiple of 4
+// or on the matrices being 16-byte aligned (columns of 50257 or 100001 rows, unaligned slices). One read of the
+// inputs, like the piece-wise kernel above; step_k / step_w describe a stride of 1024 elements.
+
+constexpr int kRegsThreads = 1024;
+
+template <int EPT>
+constexpr int regs_waves()
+{
+    return EPT <= 24 ? 8 : 4; // two workgroups per CU where 64 registers are enough, else one
+}
+
+template <int NBITS, bool ZT, int EPT>
+__global__ __launch_bounds__(kRegsThreads) __attribute__((amdgpu_waves_per_eu(regs_waves<EPT>(), regs_waves<EPT>()))) void quantize_regs_kernel(
+    const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q, RegGeom c)
+{
+    using PS = PackShape<NBITS>;
+    static_assert(NBITS < 32, "32-bit codes are whole QWords: nothing to assemble");
+    constexpr uint32_t T = kRegsThreads, NW = T / 64;
+    extern __shared__ f32x4 smem_v4[];
+    float* red = reinterpret_cast<float*>(smem_v4);
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
+    uint32_t* words = reinterpret_cast<uint32_t*>(red + kRegRedSlots);
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const size_t base = (size_t) blockIdx.x * c.rows;
+    char* qc = q + (size_t) blockIdx.x * c.qcol;
+    for (uint32_t x = tid; x < c.nq; x += T)
+        words[x] = 0u;
+    const float* gc = g + base;
+    const float* rc = r_in + base;
+    // branch-free loads: an element beyond the column is replaced by the column's last one and left out of every sum and store
+    const uint32_t last = c.rows - 1;
+    float a[EPT];
+    {
+        const uint32_t t = opaque(tid);
+#pragma unroll
+        for (int j = 0; j < EPT; ++j)
+        {
+            const uint32_t e = t + T * j;
+            a[j] = gc[e < c.rows ? e : last];
+        }
+    }
+#pragma unroll
+    for (int j0 = 0; j0 < EPT; j0 += 8)
+    {
+        const uint32_t t = opaque(tid);
+        float b[8];
+#pragma unroll
+        for (int j = j0; j < j0 + 8 && j < EPT; ++j)
+        {
+            const uint32_t e = t + T * j;
+            b[j - j0] = rc[e < c.rows ? e : last];
+        }
+#pragma unroll
+        for (int j = j0; j < j0 + 8 && j < EPT; ++j)
+            a[j] = a[j] + b[j - j0];
+    }
+    constexpr bool need_stat = (NBITS != 1) || !ZT;
+    float total = 0.0f;
+    if constexpr (need_stat)
+    {
+        float stat = 0.0f;
+        const uint32_t t = opaque(tid);
+#pragma unroll
+        for (int j = 0; j < EPT; ++j)
+        {
+            const float with = stat + (NBITS == 1 ? a[j] : a[j] * a[j]);
+            stat = (t + T * j < c.rows) ? with : stat;
+        }
+        stat = wave_sum(stat);
+        if (lane == 0)
+            red[wave] = stat;
+    }
+    // the whole column has been read before this barrier, so r_out may be r_in
+    __syncthreads();
+    if constexpr (need_stat)
+    {
+        total = red[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+            total += red[x];
+    }
+    float lo, hi;
+    if constexpr (NBITS == 1)
+    {
+        const float mean = ZT ? 0.0f : total / (float) c.rows;
+        float s0 = 0.0f, s1 = 0.0f;
+        uint32_t n0 = 0;
+        const uint32_t t = opaque(tid);
+#pragma unroll
+        for (int j = 0; j < EPT; ++j)
+        {
+            const float x = a[j];
+            const bool below = x < mean;
+            const bool valid = t + T * j < c.rows;
+            s0 = valid ? s0 + (below ? x : 0.0f) : s0;
+            s1 = valid ? s1 + (below ? 0.0f : x) : s1;
+            n0 += (valid && below) ? 1u : 0u;
+        }
+        s0 = wave_sum(s0);
+        s1 = wave_sum(s1);
+        n0 = wave_sum(n0);
+        __syncthreads(); // everyone has read the wave sums of the mean
+        if (lane == 0)
+        {
+            red[wave] = s0;
+            red[NW + wave] = s1;
+            red_u[wave] = n0;
+        }
+        __syncthreads();
+        float S0 = red[0], S1 = red[NW];
+        uint32_t N0 = red_u[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+        {
+            S0 += red[x];
+            S1 += red[NW + x];
+            N0 += red_u[x];
+        }
+        finish_stats_1bit<ZT>(mean, S0, S1, N0, c.rows - N0, c.rows, lo, hi);
+    }
+    else
+    {
+        finish_stats_multibit(total, c.rows, lo, hi);
+    }
+    if (tid == 0)
+    {
+        float* gh = reinterpret_cast<float*>(qc);
+        gh[0] = lo;
+        gh[1] = hi;
+    }
+    const ValueQ vq = make_vq<NBITS>(lo, hi);
+    const float val0 = unquantize_value<NBITS>(vq, 0u);
+    const float val1 = unquantize_value<NBITS>(vq, 1u);
+    float* oc = r_out + base;
+    // element tid is bit position k of QWord w; this thread's next element lies 1024 elements further on
+    uint32_t k = tid / c.nq;
+    uint32_t w = tid - k * c.nq;
+    const uint32_t to = opaque(tid);
+#pragma unroll
+    for (int j = 0; j < EPT; ++j)
+    {
+        const uint32_t e = to + T * j;
+        if (e < c.rows)
+        {
+            const float v = a[j];
+            const uint32_t code = quantize_value<NBITS, ZT>(vq, v);
+            float back;
+            if constexpr (NBITS == 1)
+                back = code ? val1 : val0;
+            else
+                back = unquantize_value<NBITS>(vq, code);
+            oc[e] = v - back;
+            atomicOr(&words[w], code << (k * PS::SHIFT));
+        }
+        w += c.step_w;
+        k += c.step_k;
+        if (w >= c.nq)
+        {
+            w -= c.nq;
+            ++k;
         }
     }
     __syncthreads();
@@ -1740,10 +1965,10 @@ __global__ __launch_bounds__(256) void unquantize_segment_kernel(const char* __r
     unquantize_segment_body<NBITS>(q, out, t, add, blockIdx.x);
 }
 
-// Row-major decoder for columns whose height is a multiple of 4 but whose QWord count is not (9304 rows -> 291 QWords,
-// 100000 -> 3125): a workgroup copies the packed column into LDS once (every QWord is used by up to 32 rows) and then
-// walks a chunk of consecutive rows, four per thread and store, so that all stores are aligned 16-byte stores whatever
-// the QWord count.
+// Row-major decoder for columns of 1024 rows and more whose QWord-major stores would not be whole lines (9304 rows -> 291
+// QWords, 100000 -> 3125, 50257 -> 1571): a workgroup copies the packed column into LDS once (every QWord is used by
+// up to 32 rows) and then walks a chunk of consecutive rows, four per thread and store, so that all stores are aligned
+// 16-byte stores whatever the QWord count, the height and the alignment of the output.
 struct UnqRowGeom
 {
     uint32_t rows;
@@ -1815,17 +2040,42 @@ __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q,
         }
     }
     __syncthreads();
+    // The column need not start on a 16-byte boundary nor hold a multiple of 4 rows: `head` rows (0..3) lie before its
+    // first aligned group of four and `tail` rows (0..3) after the last; chunks are counted from the first aligned row,
+    // the first chunk's workgroup also writes the head rows, the last one's the tail rows, one row per thread.
+    float* oc = out + (size_t) c * t.rows;
+    const uint32_t head = (4u - (uint32_t) ((reinterpret_cast<uintptr_t>(oc) >> 2) & 3u)) & 3u;
+    const uint32_t body = (t.rows - head) & ~3u; // rows in aligned groups of four
+    const uint32_t tail = t.rows - head - body;
     const uint32_t r0 = ch * t.chunk;
-    const uint32_t pieces = ((ch + 1 == t.chunks ? t.rows : r0 + t.chunk) - r0) >> 2; // the last chunk runs to the end
-    f32x4* o4 = reinterpret_cast<f32x4*>(out + (size_t) c * t.rows + r0);
+    const uint32_t pieces = ((ch + 1 == t.chunks ? body : r0 + t.chunk) - r0) >> 2; // the last chunk runs to the end
+    f32x4* o4 = reinterpret_cast<f32x4*>(oc + head + r0);
     const float val0 = unquantize_value<NBITS>(uf, lo, 0u);
     const float val1 = unquantize_value<NBITS>(uf, lo, 1u);
+    {
+        uint32_t row = t.rows; // none
+        if (ch == 0 && tid < head)
+            row = tid;
+        else if (ch + 1 == t.chunks && tid >= 4 && tid < 4 + tail)
+            row = head + body + (tid - 4);
+        if (row < t.rows)
+        {
+            const uint32_t k = row / t.nq;
+            const uint32_t code = (words[row - k * t.nq] >> (k * SHIFT)) & CODEMASK;
+            float x;
+            if constexpr (NBITS == 1)
+                x = code ? val1 : val0;
+            else
+                x = unquantize_value<NBITS>(uf, lo, code);
+            oc[row] = add ? x + oc[row] : x;
+        }
+    }
     // Slot v = tid, tid + 256, ... holds piece v - shift, shift = the chunk's offset into its 128-byte line in pieces, so
     // that every wavefront's 64 stores cover whole lines also where columns do not start on one (9304 rows).
     const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o4) >> 4) & 7u);
     const uint32_t vfirst = tid < shift ? tid + 256 : tid;
     // row i sits in QWord i % nq at bit position i / nq; a thread's pieces are 1024 rows apart
-    const uint32_t i0 = r0 + 4 * (vfirst - shift);
+    const uint32_t i0 = head + r0 + 4 * (vfirst - shift);
     uint32_t k0 = i0 / t.nq;
     uint32_t w0 = i0 - k0 * t.nq;
     const uint32_t dk = 1024u / t.nq;

@@ -857,16 +857,20 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     const uint32_t shift = PER <= kRegMaxShiftPer ? column_shift(r_in + base, c.line_shift) : 0u;
     const uint32_t last = c.pieces - 1;
     f64x2 a[PER];
+    {
+        const uint32_t t = opaque(tid);
 #pragma unroll
-    for (int u = 0; u < PER; ++u)
-        a[u] = __builtin_nontemporal_load(g2 + slot_piece(tid + T * u, shift, last));
+        for (int u = 0; u < PER; ++u)
+            a[u] = __builtin_nontemporal_load(g2 + slot_piece(t + T * u, shift, last));
+    }
 #pragma unroll
     for (int u0 = 0; u0 < PER; u0 += 4)
     {
+        const uint32_t t = opaque(tid);
         f64x2 b[4];
 #pragma unroll
         for (int u = u0; u < u0 + 4 && u < PER; ++u)
-            b[u - u0] = __builtin_nontemporal_load(r2 + slot_piece(tid + T * u, shift, last));
+            b[u - u0] = __builtin_nontemporal_load(r2 + slot_piece(t + T * u, shift, last));
 #pragma unroll
         for (int u = u0; u < u0 + 4 && u < PER; ++u)
             a[u] = a[u] + b[u - u0];
@@ -876,11 +880,12 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     if constexpr (need_stat)
     {
         double stat = 0.0;
+        const uint32_t t = opaque(tid);
 #pragma unroll
         for (int u = 0; u < PER; ++u)
         {
             const double with = reg_add_piece<NBITS>(stat, a[u]);
-            stat = slot_valid(tid + T * u, shift, c.pieces) ? with : stat;
+            stat = slot_valid(t + T * u, shift, c.pieces) ? with : stat;
         }
         stat = wave_sum(stat);
         if (lane == 0)
@@ -901,6 +906,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
         const double mean = ZT ? 0.0 : total / (double) c.rows;
         double s0 = 0.0, s1 = 0.0;
         uint32_t n0 = 0;
+        const uint32_t t = opaque(tid);
 #pragma unroll
         for (int u = 0; u < PER; ++u)
         {
@@ -915,7 +921,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
                 t1 += below ? 0.0 : x;
                 tn += below ? 1u : 0u;
             }
-            const bool valid = slot_valid(tid + T * u, shift, c.pieces);
+            const bool valid = slot_valid(t + T * u, shift, c.pieces);
             s0 = valid ? t0 : s0;
             s1 = valid ? t1 : s1;
             n0 = valid ? tn : n0;
@@ -962,11 +968,12 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     const uint32_t e0 = 2 * (tid + T * ufirst - shift);
     uint32_t k = e0 / c.nq;
     uint32_t w = e0 - k * c.nq;
+    const uint32_t to = opaque(tid);
 #pragma unroll
     for (int u = 0; u < PER; ++u)
     {
-        const uint32_t p = tid + T * u - shift;
-        if (slot_valid(tid + T * u, shift, c.pieces))
+        const uint32_t p = to + T * u - shift;
+        if (slot_valid(to + T * u, shift, c.pieces))
         {
             f64x2 res;
             uint32_t kk = k, ww = w;

@@ -20,7 +20,8 @@ enum QuantizePath
     kPathTile = 1,    // LDS-staged column tile (rows <= kTileMaxRows)
     kPathTall = 2,    // one workgroup per column, global re-read (any rows)
     kPathCol = 3,     // one workgroup per column, column in LDS: rows a multiple of 4, matrices 16-byte aligned
-    kPathReg = 4      // one workgroup per column, column in registers: same conditions, 1 to 16 bits
+    kPathReg = 4,     // one workgroup per column, column in registers: same conditions, 1 to 16 bits
+    kPathRegScalar = 5 // the same with one float per load and store: any height up to 98304 rows, any alignment, 1 to 16 bits
 };
 
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
@@ -246,6 +247,41 @@ inline hipError_t launch_reg_one(hipStream_t s, LaunchEvents ev, const float* g,
     return hipGetLastError();
 }
 
+template <int NBITS, bool ZT, int PER>
+inline hipError_t launch_reg_edge_one(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
+                                      const RegGeom& c)
+{
+    hipExtLaunchKernelGGL((quantize_reg_kernel<NBITS, ZT, 1024, PER, true>), dim3(cols), dim3(1024), reg_lds_bytes(c), s, ev.start, ev.stop, 0,
+                          g, r_in, r_out, q, c);
+    return hipGetLastError();
+}
+
+// The variant for columns that start anywhere and have any height (1024 threads only): c.pieces is an upper bound.
+template <int NBITS, bool ZT>
+struct RegEdgeLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, RegGeom c)
+    {
+        if constexpr (NBITS >= 32)
+            return hipErrorInvalidValue;
+        else
+        {
+            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + 1023u) / 1024u;
+#define CNTKQ_REGE(P) if (per <= P) return launch_reg_edge_one<NBITS, ZT, P>(s, ev, g, r_in, r_out, q, cols, c)
+            CNTKQ_REGE(4);
+            CNTKQ_REGE(6);
+            CNTKQ_REGE(8);
+            CNTKQ_REGE(10);
+            CNTKQ_REGE(13);
+            CNTKQ_REGE(16);
+            CNTKQ_REGE(20);
+            CNTKQ_REGE(25);
+#undef CNTKQ_REGE
+            return hipErrorInvalidValue;
+        }
+    }
+};
+
 template <int NBITS, bool ZT>
 struct RegLauncher
 {
@@ -316,13 +352,68 @@ inline bool reg_applicable(const float* g, const float* r_in, const float* r_out
     return (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
 }
 
+// The piece-wise register kernel with edge elements: matrices only 4-byte aligned but at the same offset within 16
+// bytes (then every column of all three starts at the same offset), any height from 8 rows on.
+inline bool reg_edge_applicable(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
+{
+    const uintptr_t a = reinterpret_cast<uintptr_t>(g) & 15u, b = reinterpret_cast<uintptr_t>(r_in) & 15u,
+                    c = reinterpret_cast<uintptr_t>(r_out) & 15u;
+    if (a != b || b != c || rows < 8 || rows > kRegMaxRows - 32 || nbits >= 32 || (reinterpret_cast<uintptr_t>(q) & 3u) != 0)
+        return false;
+    return (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
+}
+
+constexpr uint32_t kRegsMaxRows = 1024 * 96;
+
+inline bool regs_applicable(size_t rows, size_t nbits)
+{
+    return rows >= 1 && rows <= kRegsMaxRows && nbits < 32 && (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
+}
+
+template <int NBITS, bool ZT, int EPT>
+inline hipError_t launch_regs_one(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
+                                  const RegGeom& c)
+{
+    hipExtLaunchKernelGGL((quantize_regs_kernel<NBITS, ZT, EPT>), dim3(cols), dim3(kRegsThreads), reg_lds_bytes(c), s, ev.start, ev.stop, 0, g,
+                          r_in, r_out, q, c);
+    return hipGetLastError();
+}
+
+template <int NBITS, bool ZT>
+struct RegsLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, RegGeom c)
+    {
+        if constexpr (NBITS >= 32)
+            return hipErrorInvalidValue;
+        else
+        {
+            const uint32_t ept = (c.rows + kRegsThreads - 1) / kRegsThreads;
+#define CNTKQ_REGS(E) if (ept <= E) return launch_regs_one<NBITS, ZT, E>(s, ev, g, r_in, r_out, q, cols, c)
+            CNTKQ_REGS(16);
+            CNTKQ_REGS(24);
+            CNTKQ_REGS(32);
+            CNTKQ_REGS(48);
+            CNTKQ_REGS(64);
+            CNTKQ_REGS(80);
+            CNTKQ_REGS(96);
+#undef CNTKQ_REGS
+            return hipErrorInvalidValue;
+        }
+    }
+};
+
 // which path launch_quantize takes for this matrix when nothing is forced
 inline int quantize_auto_path(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
 {
     if (reg_applicable(g, r_in, r_out, q, rows, nbits))
         return kPathReg;
     if (rows > kTileMaxRows)
-        return kPathTall;
+    {
+        if (reg_edge_applicable(g, r_in, r_out, q, rows, nbits))
+            return kPathReg;
+        return regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
+    }
     if (col_applicable(g, r_in, r_out, q, rows, nbits))
         return kPathCol;
     return kPathTile;
@@ -342,13 +433,28 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     if (path == kPathReg)
     {
         if (!reg_applicable(g, r_in, r_out, q, rows, nbits, true))
-            return hipErrorInvalidValue;
+        {
+            // not whole aligned pieces: the variant with edge elements, where the three matrices allow it
+            if (!reg_edge_applicable(g, r_in, r_out, q, rows, nbits))
+                return hipErrorInvalidValue;
+            RegGeom c = make_reg_geom(rows, nbits, 1024, same_line_offset(g, r_in, r_out));
+            return dispatch_nbits<RegEdgeLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c);
+        }
         const uint32_t threads = reg_threads(rows);
         // up to 14336 rows the shift is part of the summation order all column kernels share; above, it is used where
         // the registers allow
         const bool line_shift = quantize_line_shift(g, r_in, r_out, rows) && (threads == 256 || rows / 4 + 7 <= 1024 * (size_t) kRegMaxShiftPer);
         return dispatch_nbits<RegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols,
                                            make_reg_geom(rows, nbits, threads, line_shift), threads);
+    }
+    if (path == kPathRegScalar)
+    {
+        if (!regs_applicable(rows, nbits))
+            return hipErrorInvalidValue;
+        RegGeom c = make_reg_geom(rows, nbits, kRegsThreads, false);
+        c.step_k = kRegsThreads / c.nq; // a thread's next element lies 1024 elements further on
+        c.step_w = kRegsThreads % c.nq;
+        return dispatch_nbits<RegsLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c);
     }
     if (path == kPathCol)
     {
@@ -453,7 +559,7 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
     // 128-byte lines: QWords a multiple of 32, all of them full, columns starting on a line.
     const bool vec_can = (nq % 4 == 0) && (rows % 4 == 0) && out16 && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
     const bool vec_ideal = vec_can && nq % 32 == 0 && rows % 32 == 0 && rows * nbits == nq * 32;
-    const bool rows_can = slots_free && out16 && rows % 4 == 0 && nq >= 32 && nq * 4 <= kUnqRowsMaxLds;
+    const bool rows_can = slots_free && rows >= 16 && nq >= 32 && nq * 4 <= kUnqRowsMaxLds; // any height, any (4-byte) alignment
     const bool tile_can = slots_free && out16 && rows <= kUnqTileMaxRows;
     bool vec = false, rowmajor = false, tile = false, seg_allowed = true;
     if (mode == 1)

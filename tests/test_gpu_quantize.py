@@ -21,7 +21,7 @@ from cntk_amd import Matrix, MatrixQuantizerImpl, QuantizedMatrix
 pytestmark = pytest.mark.gpu
 
 VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False)]
-PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG = 0, 1, 2, 3, 4
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG, PATH_REG_SCALAR = 0, 1, 2, 3, 4, 5
 
 
 def say(*a):
@@ -128,6 +128,15 @@ PATH_CASES = [
     (4, 3, PATH_REG, 0), (36, 70, PATH_REG, 0), (1000, 5, PATH_REG, 0), (4100, 3, PATH_REG, 0), (6148, 5, PATH_REG, 0),
     (9304, 2, PATH_REG, 0), (12292, 3, PATH_REG, 0), (14336, 2, PATH_REG, 0), (14340, 3, PATH_REG, 0), (20000, 3, PATH_REG, 0),
     (40964, 2, PATH_REG, 0), (65540, 2, PATH_REG, 0), (102400, 1, PATH_REG, 0), (102404, 2, PATH_AUTO, 0),
+    # the same one float at a time: any height up to 98304 rows (the automatic choice for tall columns the piece-wise
+    # kernel cannot take)
+    (1, 3, PATH_REG_SCALAR, 0), (37, 5, PATH_REG_SCALAR, 0), (1001, 3, PATH_REG_SCALAR, 0), (14337, 3, PATH_AUTO, 0),
+    (20001, 2, PATH_AUTO, 0), (32769, 2, PATH_REG_SCALAR, 0), (50257, 2, PATH_AUTO, 0), (65537, 1, PATH_AUTO, 0), (98303, 1, PATH_AUTO, 0),
+    (98304, 1, PATH_REG_SCALAR, 0), (98305, 1, PATH_AUTO, 0),
+    # the piece-wise kernel with edge elements (heights that are not a multiple of 4; the automatic choice for them above
+    # 14336 rows when the three matrices share their alignment)
+    (9, 5, PATH_REG, 0), (37, 5, PATH_REG, 0), (1001, 3, PATH_REG, 0), (4099, 2, PATH_REG, 0), (14338, 3, PATH_REG, 0),
+    (50257, 2, PATH_REG, 0), (102365, 1, PATH_REG, 0),
 ]
 
 
@@ -138,7 +147,7 @@ def test_kernel_paths(case):
     rep = parity.Report()
     for nbits, zt in VARIANTS:
         say("path case", case, "nbits", nbits, "zeroThr", zt)
-        if path == PATH_REG and (nbits == 32 or (48 + oracle.qwords_per_col(rows, nbits)) * 4 > 65536):
+        if path in (PATH_REG, PATH_REG_SCALAR) and (nbits == 32 or (48 + oracle.qwords_per_col(rows, nbits)) * 4 > 65536):
             # whole-QWord codes and columns whose QWords exceed 64 KB of LDS are not the register kernels' business
             qz._set_tuning(quantize_path=path)
             with pytest.raises(cntk_amd.QuantizerLogicError):
@@ -268,7 +277,7 @@ def test_unquantize_variants(quantizer):
 
 
 TILE_DECODER_SHAPES = [(1, 1), (1, 9), (2, 7), (3, 5), (5, 3), (31, 13), (32, 8), (33, 41), (64, 100), (147, 64), (256, 1031),
-                       (429, 37), (512, 24), (1000, 9), (1001, 5), (1024, 3), (2047, 2), (2048, 7), (4096, 5), (4095, 3), (4097, 3), (9305, 2), (16383, 2), (16385, 2)]
+                       (429, 37), (512, 24), (1000, 9), (1001, 5), (1024, 3), (2047, 2), (2048, 7), (4096, 5), (4095, 3), (4097, 3), (9305, 2), (16383, 2), (16385, 2), (1025, 7), (1026, 5), (1027, 3), (50257, 2), (100001, 2)]
 
 
 @pytest.mark.parametrize("shape", TILE_DECODER_SHAPES, ids=["%dx%d" % s for s in TILE_DECODER_SHAPES])
