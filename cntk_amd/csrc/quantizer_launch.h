@@ -294,6 +294,8 @@ struct RegLauncher
         {
             const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + threads - 1) / threads; // up to 7 slots lie before the column
 #define CNTKQ_REG(T, P) if (threads == T && per <= P) return launch_reg_one<NBITS, ZT, T, P>(s, ev, g, r_in, r_out, q, cols, c)
+            CNTKQ_REG(256, 3);
+            CNTKQ_REG(256, 4);
             CNTKQ_REG(256, 6);
             CNTKQ_REG(256, 8);
             CNTKQ_REG(256, 10);
@@ -330,10 +332,10 @@ inline void launch_stripe_col(hipStream_t s, LaunchEvents ev, const StripeSource
                           ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, qcol);
 }
 
-// The register kernels: taller than the unrolled LDS kernels' 4096 rows (unless forced), up to 25 pieces for each of
+// The register kernels: taller than 2048 rows (unless forced), up to 25 pieces for each of
 // 1024 threads, the column's QWords within 64 KB of LDS. 256 threads up to the height the stripe reduction handles (whose
 // LDS kernels then sum in the same order), 1024 above.
-constexpr uint32_t kRegMinRows = 4096;
+constexpr uint32_t kRegMinRows = 2048;
 constexpr uint32_t kRegMaxRows = 4 * 1024 * 25;
 
 inline uint32_t reg_threads(size_t rows)
@@ -406,7 +408,10 @@ struct RegsLauncher
 // which path launch_quantize takes for this matrix when nothing is forced
 inline int quantize_auto_path(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
 {
-    if (reg_applicable(g, r_in, r_out, q, rows, nbits))
+    // (4096 rows at 1 bit: the unrolled LDS kernel, where its conditions hold, is as fast)
+    const bool unrolled = col_applicable(g, r_in, r_out, q, rows, nbits) && col_unrolled(q, rows, nbits) &&
+                          !quantize_line_shift(g, r_in, r_out, rows);
+    if (!unrolled && reg_applicable(g, r_in, r_out, q, rows, nbits))
         return kPathReg;
     if (rows > kTileMaxRows)
     {
