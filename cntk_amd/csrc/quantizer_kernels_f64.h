@@ -681,16 +681,40 @@ __global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __rest
                 words[w + 256 * u] = v[u];
     }
     __syncthreads();
+    // any height, any (8-byte) alignment: one row may lie before the column's first aligned pair and one after its last;
+    // the first chunk's workgroup writes the former, the last one's the latter
+    double* oc = out + (size_t) c * t.rows;
+    const uint32_t head = (uint32_t) ((reinterpret_cast<uintptr_t>(oc) >> 3) & 1u);
+    const uint32_t body = (t.rows - head) & ~1u;
+    const uint32_t tail = t.rows - head - body;
     const uint32_t r0 = ch * t.chunk;
-    const uint32_t pieces = ((ch + 1 == t.chunks ? t.rows : r0 + t.chunk) - r0) >> 1; // the last chunk runs to the end
-    f64x2* o2 = reinterpret_cast<f64x2*>(out + (size_t) c * t.rows + r0);
+    const uint32_t pieces = ((ch + 1 == t.chunks ? body : r0 + t.chunk) - r0) >> 1; // the last chunk runs to the end
+    f64x2* o2 = reinterpret_cast<f64x2*>(oc + head + r0);
     const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
     const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
+    {
+        uint32_t row = t.rows; // none
+        if (ch == 0 && tid < head)
+            row = 0;
+        else if (ch + 1 == t.chunks && tid == 1 && tail != 0)
+            row = t.rows - 1;
+        if (row < t.rows)
+        {
+            const uint32_t k = row / t.nq;
+            const uint64_t code = (words[row - k * t.nq] >> (k * PS::SHIFT)) & PS::CODEMASK;
+            double x;
+            if constexpr (NBITS == 1)
+                x = code ? val1 : val0;
+            else
+                x = unquantize_value<NBITS>(vq.uf, vq.lo, code);
+            oc[row] = add ? x + oc[row] : x;
+        }
+    }
     // slots dealt by 128-byte lines, as in the fp32 decoder
     const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o2) >> 4) & 7u);
     const uint32_t vfirst = tid < shift ? tid + 256 : tid;
     // row i sits in QWord i % nq at bit position i / nq; a thread's pieces are 512 rows apart
-    const uint32_t i0 = r0 + 2 * (vfirst - shift);
+    const uint32_t i0 = head + r0 + 2 * (vfirst - shift);
     uint32_t k0 = i0 / t.nq;
     uint32_t w0 = i0 - k0 * t.nq;
     const uint32_t dk = 512u / t.nq;
@@ -852,10 +876,20 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     char* qc = q + (size_t) blockIdx.x * c.qcol;
     for (uint32_t x = tid; x < c.nq; x += T)
         words[x] = 0ull;
-    const f64x2* g2 = reinterpret_cast<const f64x2*>(g + base);
-    const f64x2* r2 = reinterpret_cast<const f64x2*>(r_in + base);
-    const uint32_t shift = PER <= kRegMaxShiftPer ? column_shift(r_in + base, c.line_shift) : 0u;
-    const uint32_t last = c.pieces - 1;
+    // the column may start 8 bytes off a 16-byte boundary and have an odd height: one element before the first aligned
+    // pair (held by thread 0) and one after the last (thread 1) then take part in every phase after the thread's pieces
+    const uint32_t head = (uint32_t) ((reinterpret_cast<uintptr_t>(r_in + base) >> 3) & 1u);
+    const uint32_t pieces = (c.rows - head) >> 1;
+    const uint32_t tail = c.rows - head - 2 * pieces;
+    const f64x2* g2 = reinterpret_cast<const f64x2*>(g + base + head);
+    const f64x2* r2 = reinterpret_cast<const f64x2*>(r_in + base + head);
+    const bool has_edge = (tid == 0 && head != 0) || (tid == 1 && tail != 0);
+    const uint32_t edge_at = tid == 0 ? 0u : c.rows - 1;
+    double edge = 0.0;
+    if (has_edge)
+        edge = g[base + edge_at] + r_in[base + edge_at];
+    const uint32_t shift = PER <= kRegMaxShiftPer ? column_shift(r_in + base + head, c.line_shift) : 0u;
+    const uint32_t last = pieces - 1;
     f64x2 a[PER];
     {
         const uint32_t t = opaque(tid);
@@ -885,8 +919,10 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
         for (int u = 0; u < PER; ++u)
         {
             const double with = reg_add_piece<NBITS>(stat, a[u]);
-            stat = slot_valid(t + T * u, shift, c.pieces) ? with : stat;
+            stat = slot_valid(t + T * u, shift, pieces) ? with : stat;
         }
+        if (has_edge)
+            stat += NBITS == 1 ? edge : edge * edge;
         stat = wave_sum(stat);
         if (lane == 0)
             red[wave] = stat;
@@ -921,10 +957,17 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
                 t1 += below ? 0.0 : x;
                 tn += below ? 1u : 0u;
             }
-            const bool valid = slot_valid(t + T * u, shift, c.pieces);
+            const bool valid = slot_valid(t + T * u, shift, pieces);
             s0 = valid ? t0 : s0;
             s1 = valid ? t1 : s1;
             n0 = valid ? tn : n0;
+        }
+        if (has_edge)
+        {
+            const bool below = edge < mean;
+            s0 += below ? edge : 0.0;
+            s1 += below ? 0.0 : edge;
+            n0 += below ? 1u : 0u;
         }
         s0 = wave_sum(s0);
         s1 = wave_sum(s1);
@@ -961,11 +1004,11 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     const ValueQ vq = make_vq<NBITS>(lo, hi);
     const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
     const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
-    f64x2* o2 = reinterpret_cast<f64x2*>(r_out + base);
+    f64x2* o2 = reinterpret_cast<f64x2*>(r_out + base + head);
     // the first element of this thread's first slot inside the column is bit position k of QWord w; the element after it
     // is the following QWord, the slots after it lie 2 * T elements further on (step_k, step_w)
     const uint32_t ufirst = tid < shift ? 1u : 0u;
-    const uint32_t e0 = 2 * (tid + T * ufirst - shift);
+    const uint32_t e0 = head + 2 * (tid + T * ufirst - shift);
     uint32_t k = e0 / c.nq;
     uint32_t w = e0 - k * c.nq;
     const uint32_t to = opaque(tid);
@@ -973,7 +1016,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     for (int u = 0; u < PER; ++u)
     {
         const uint32_t p = to + T * u - shift;
-        if (slot_valid(to + T * u, shift, c.pieces))
+        if (slot_valid(to + T * u, shift, pieces))
         {
             f64x2 res;
             uint32_t kk = k, ww = w;
@@ -1007,6 +1050,18 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
                 ++k;
             }
         }
+    }
+    if (has_edge)
+    {
+        const uint64_t code = quantize_value<NBITS, ZT>(vq, edge);
+        double back;
+        if constexpr (NBITS == 1)
+            back = code ? val1 : val0;
+        else
+            back = unquantize_value<NBITS>(vq.uf, vq.lo, code);
+        r_out[base + edge_at] = edge - back;
+        const uint32_t ek = edge_at / c.nq;
+        atomicOr(&words[edge_at - ek * c.nq], (unsigned long long) (code << (ek * PS::SHIFT)));
     }
     __syncthreads();
     unsigned long long* bits = reinterpret_cast<unsigned long long*>(qc + 16);

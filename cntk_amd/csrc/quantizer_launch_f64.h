@@ -109,15 +109,17 @@ struct StripeLauncher
     }
 };
 
-// The register kernel: for columns the tile kernel cannot hold, of even height, 16-byte aligned matrices, below 64 bits,
+// The register kernel: for columns the tile kernel cannot hold, below 64 bits,
 // at most 25 pieces of two doubles for each of 1024 threads, QWords within 64 KB of LDS.
 constexpr uint32_t kRegThreads = 1024;
 constexpr size_t kRegMaxRows = 2 * 1024 * 25;
 
 inline bool reg_applicable(const double* g, const double* r_in, const double* r_out, size_t rows, size_t nbits)
 {
-    const uintptr_t m = reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(r_in) | reinterpret_cast<uintptr_t>(r_out);
-    if (rows % 2 != 0 || rows < 2 || rows > kRegMaxRows || nbits >= 64 || (m & 15u) != 0)
+    // any height from 4 rows on; the three matrices at the same offset within 16 bytes (then so are all their columns)
+    const uintptr_t a = reinterpret_cast<uintptr_t>(g) & 15u, b = reinterpret_cast<uintptr_t>(r_in) & 15u,
+                    c = reinterpret_cast<uintptr_t>(r_out) & 15u;
+    if (a != b || b != c || rows < 4 || rows > kRegMaxRows - 16 || nbits >= 64)
         return false;
     return (kRegRedSlots + qwords_per_col(rows, nbits)) * 8 <= kMaxLdsBytes;
 }
@@ -267,7 +269,7 @@ inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* 
     // The QWord-major decoder is at its best when every bit position of a column is a run of whole 128-byte lines. Other
     // columns: row-major decoder from 512 rows on, tile decoder for shorter ones (the choices of the fp32 side).
     const bool vec_ideal = nq % 16 == 0 && rows % 16 == 0 && rows * nbits == nq * 64 && out16;
-    const bool rows_can = tune.unq_slots == 0 && out16 && rows % 2 == 0 && nq >= 16 && nq * 8 <= 48 * 1024;
+    const bool rows_can = tune.unq_slots == 0 && rows >= 16 && nq >= 16 && nq * 8 <= 48 * 1024; // any height, any alignment
     const bool tile_can = tune.unq_slots == 0 && out16 && rows <= kUnqTileMaxRows64;
     bool use_rows = false, use_tile = false;
     if (mode == 2 && tile_can)

@@ -136,8 +136,9 @@ PATH_CASES = [
     (2048, 19, PATH_TILE, 0), (2048, 19, PATH_TILE, 256), (4608, 3, PATH_TILE, 0), (7168, 2, PATH_TILE, 0),
     (1, 5, PATH_TALL, 0), (70, 3, PATH_TALL, 0), (1025, 3, PATH_TALL, 0), (20001, 2, PATH_TALL, 0), (9304, 2, PATH_AUTO, 0),
     # one workgroup of 1024 threads per column, the column in registers: even heights; the automatic choice above 7168 rows
-    (2, 3, PATH_REG, 0), (70, 3, PATH_REG, 0), (1000, 5, PATH_REG, 0), (7170, 3, PATH_REG, 0), (9304, 3, PATH_REG, 0),
+    (4, 3, PATH_REG, 0), (70, 3, PATH_REG, 0), (1000, 5, PATH_REG, 0), (7170, 3, PATH_REG, 0), (9304, 3, PATH_REG, 0),
     (20000, 3, PATH_AUTO, 0), (32770, 2, PATH_REG, 0), (51200, 1, PATH_AUTO, 0), (51202, 1, PATH_AUTO, 0),
+    (5, 3, PATH_REG, 0), (1001, 3, PATH_REG, 0), (9305, 3, PATH_AUTO, 0), (20001, 2, PATH_AUTO, 0), (50257, 1, PATH_AUTO, 0),
 ]
 
 
@@ -196,7 +197,7 @@ def test_unquantize_variants_f64(quantizer):
 
 
 DECODER_SHAPES_F64 = [(1, 1), (1, 9), (3, 5), (31, 13), (64, 100), (147, 64), (429, 37), (512, 24), (1000, 9), (1001, 5), (2048, 7),
-                      (4095, 3), (4096, 2), (4097, 3), (9304, 3), (9305, 2), (16383, 2), (20000, 2), (100000, 2)]
+                      (4095, 3), (4096, 2), (4097, 3), (9304, 3), (9305, 2), (16383, 2), (20000, 2), (20001, 3), (50257, 2), (100000, 2)]
 
 
 @pytest.mark.parametrize("shape", DECODER_SHAPES_F64, ids=["%dx%d" % s for s in DECODER_SHAPES_F64])
