@@ -332,10 +332,10 @@ inline void launch_stripe_col(hipStream_t s, LaunchEvents ev, const StripeSource
                           ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, qcol);
 }
 
-// The register kernels: taller than 2048 rows (unless forced), up to 25 pieces for each of
+// The register kernels: from 2048 rows on (unless forced), up to 25 pieces for each of
 // 1024 threads, the column's QWords within 64 KB of LDS. 256 threads up to the height the stripe reduction handles (whose
 // LDS kernels then sum in the same order), 1024 above.
-constexpr uint32_t kRegMinRows = 2048;
+constexpr uint32_t kRegMinRows = 2047;
 constexpr uint32_t kRegMaxRows = 4 * 1024 * 25;
 
 inline uint32_t reg_threads(size_t rows)
@@ -408,8 +408,8 @@ struct RegsLauncher
 // which path launch_quantize takes for this matrix when nothing is forced
 inline int quantize_auto_path(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
 {
-    // (4096 rows at 1 bit: the unrolled LDS kernel, where its conditions hold, is as fast)
-    const bool unrolled = col_applicable(g, r_in, r_out, q, rows, nbits) && col_unrolled(q, rows, nbits) &&
+    // (2048 rows at 1 bit: the unrolled LDS kernel, where its conditions hold, is as fast)
+    const bool unrolled = rows <= 2048 && col_applicable(g, r_in, r_out, q, rows, nbits) && col_unrolled(q, rows, nbits) &&
                           !quantize_line_shift(g, r_in, r_out, rows);
     if (!unrolled && reg_applicable(g, r_in, r_out, q, rows, nbits))
         return kPathReg;
