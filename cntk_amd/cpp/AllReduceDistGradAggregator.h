@@ -306,6 +306,9 @@ public:
     {
         const size_t K = NumProc();
         const bool fused = m_options.useFusedStripeReduce && m_useQuantizationForSelfStripe;
+        // stripes too tall for the fused call keep the reference's sequence of calls
+        const size_t fusedMaxRows = detail::Abi<ElemType>::StripeReduceMaxRows();
+        auto fusable = [&](size_t i) { return fused && gradients[i]->GetNumRows() <= fusedMaxRows; };
         // every matrix's stripe in one call: the stripe quantizers share one stream, so any of their handles will do
         const bool batched = fused && m_options.useBatchedCalls && gradients.size() > 1;
         if (batched)
@@ -317,7 +320,7 @@ public:
             for (size_t i = 0; i < gradients.size(); ++i)
             {
                 const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K);
-                if (stripe.m_numCols == 0)
+                if (stripe.m_numCols == 0 || !fusable(i))
                     continue;
                 ownSlices.push_back(m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
                 Item it;
@@ -331,20 +334,21 @@ public:
             if (!items.empty())
             {
                 m_stripeBatchQuantizer = 0;
-                while (GetStripeForNode(gradients[m_stripeBatchQuantizer]->GetNumCols(), MyRank(), K).m_numCols == 0)
+                while (GetStripeForNode(gradients[m_stripeBatchQuantizer]->GetNumCols(), MyRank(), K).m_numCols == 0 ||
+                       !fusable(m_stripeBatchQuantizer))
                     m_stripeBatchQuantizer++;
                 Gpu(*m_aggGradStripeQuantizers[m_stripeBatchQuantizer]).StripeReduceBatchAsync(items, MyRank(), m_zeroThresholdFor1Bit);
             }
         }
-        for (size_t i = 0; i < gradients.size() && !batched; ++i)
+        for (size_t i = 0; i < gradients.size(); ++i)
         {
             const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K);
-            if (stripe.m_numCols == 0)
+            if (stripe.m_numCols == 0 || (batched && fusable(i)))
                 continue;
             MatrixQuantizer<ElemType>& stripeQuantizer = *m_aggGradStripeQuantizers[i];
             QuantizedMatrix<ElemType> ownSlice = m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols);
             Matrix<ElemType>& stripeResidual = const_cast<Matrix<ElemType>&>(stripeQuantizer.GetResidualMatrix());
-            if (fused)
+            if (fusable(i))
             {
                 std::vector<const QuantizedMatrix<ElemType>*> stripes;
                 for (size_t w = 0; w < K; ++w)
@@ -374,9 +378,9 @@ public:
             const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K);
             if (stripe.m_numCols == 0)
                 continue;
-            if (hostWaits && batched)
+            if (hostWaits && batched && fusable(i))
                 Gpu(*m_aggGradStripeQuantizers[m_stripeBatchQuantizer]).WaitStripeReduceDone();
-            else if (hostWaits && fused)
+            else if (hostWaits && fusable(i))
                 Gpu(*m_aggGradStripeQuantizers[i]).WaitStripeReduceDone();
             else if (hostWaits)
                 m_aggGradStripeQuantizers[i]->WaitQuantizeAsyncDone(); // (:494)

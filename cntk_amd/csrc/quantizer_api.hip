@@ -490,6 +490,16 @@ size_t cntkq_qmatrix_bytes_f64(size_t rows, size_t cols, size_t nbits)
     return f64::valid_nbits(nbits) ? f64::qcol_bytes(nbits, rows) * cols : 0;
 }
 
+size_t cntkq_stripe_reduce_max_rows(void)
+{
+    return Elem<float>::kStripeMaxRows;
+}
+
+size_t cntkq_stripe_reduce_max_rows_f64(void)
+{
+    return Elem<double>::kStripeMaxRows;
+}
+
 int cntkq_stripe_range(size_t cols, size_t rank, size_t workers, size_t* start_col, size_t* num_cols)
 {
     if (workers == 0 || rank >= workers || start_col == nullptr || num_cols == nullptr)

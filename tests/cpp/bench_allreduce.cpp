@@ -70,6 +70,8 @@ int main(int argc, char** argv)
         shapes = ResNet50();
     else if (what == "speech")
         shapes = Speech();
+    else if (what == "lstm") // language model: embedding, four LSTM weight matrices, softmax
+        shapes = {{100000, 512}, {1024, 4096}, {1024, 4096}, {1024, 4096}, {1024, 4096}, {512, 100000}};
     else
         shapes = {{std::strtoul(what.c_str(), nullptr, 10), argc > 3 ? std::strtoul(argv[3], nullptr, 10) : 9304}};
     try

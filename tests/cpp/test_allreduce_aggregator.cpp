@@ -143,7 +143,8 @@ static RunResult Run(const Shapes& shapes, size_t K, int nBits, bool zeroThr, bo
 
 static void VariantsAreBitIdentical()
 {
-    const Shapes shapes = {{2048, 40}, {429, 37}, {64, 5}, {576, 24}, {1, 9}, {33, 3}};
+    // (14340 rows: too tall for the fused stripe reduction, which then keeps the reference's call sequence for that matrix)
+    const Shapes shapes = {{2048, 40}, {429, 37}, {64, 5}, {576, 24}, {1, 9}, {33, 3}, {14340, 6}};
     const size_t K = 4;
     for (int nBits : {1, 4})
         for (bool zeroThr : {false, true})
