@@ -307,7 +307,7 @@ public:
         const size_t K = NumProc();
         const bool fused = m_options.useFusedStripeReduce && m_useQuantizationForSelfStripe;
         // stripes too tall for the fused call keep the reference's sequence of calls
-        const size_t fusedMaxRows = detail::Abi<ElemType>::StripeReduceMaxRows();
+        const size_t fusedMaxRows = detail::Abi<ElemType>::StripeReduceMaxRows(m_numQuantizationBits);
         auto fusable = [&](size_t i) { return fused && gradients[i]->GetNumRows() <= fusedMaxRows; };
         // every matrix's stripe in one call: the stripe quantizers share one stream, so any of their handles will do
         const bool batched = fused && m_options.useBatchedCalls && gradients.size() > 1;

@@ -59,7 +59,7 @@ struct Abi<float>
 {
     typedef uint32_t QWord;
     static size_t QColBytes(size_t bits, size_t rows) { return cntkq_qcol_bytes(bits, rows); }
-    static size_t StripeReduceMaxRows() { return cntkq_stripe_reduce_max_rows(); }
+    static size_t StripeReduceMaxRows(size_t bits) { return cntkq_stripe_reduce_max_rows(bits); }
     static int Quantize(cntkq_quantizer* h, const float* in, const float* resIn, size_t rows, size_t cols, void* q, size_t qBytes, int onHost,
                         size_t bits, float* resOut, int zt)
     {
@@ -81,7 +81,7 @@ struct Abi<double>
 {
     typedef uint64_t QWord;
     static size_t QColBytes(size_t bits, size_t rows) { return cntkq_qcol_bytes_f64(bits, rows); }
-    static size_t StripeReduceMaxRows() { return cntkq_stripe_reduce_max_rows_f64(); }
+    static size_t StripeReduceMaxRows(size_t bits) { return cntkq_stripe_reduce_max_rows_f64(bits); }
     static int Quantize(cntkq_quantizer* h, const double* in, const double* resIn, size_t rows, size_t cols, void* q, size_t qBytes,
                         int onHost, size_t bits, double* resOut, int zt)
     {

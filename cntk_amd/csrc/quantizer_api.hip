@@ -82,7 +82,7 @@ struct Elem<float>
 {
     static constexpr size_t kAlign = 4;
     static constexpr size_t kWordBits = 32;
-    static constexpr uint32_t kStripeMaxRows = cntkq::kTileMaxRows;
+    static size_t stripe_max_rows(size_t nbits) { return cntkq::stripe_reduce_max_rows(nbits); }
     static bool valid_nbits(size_t nbits) { return cntkq::valid_nbits(nbits); }
     static size_t qcol_bytes(size_t nbits, size_t rows) { return cntkq::qcol_bytes(nbits, rows); }
     static hipError_t quantize(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, void* q, size_t rows,
@@ -107,7 +107,7 @@ struct Elem<double>
 {
     static constexpr size_t kAlign = 8;
     static constexpr size_t kWordBits = 64;
-    static constexpr uint32_t kStripeMaxRows = cntkq::f64::kTileMaxRows;
+    static size_t stripe_max_rows(size_t) { return cntkq::f64::kTileMaxRows; }
     static bool valid_nbits(size_t nbits) { return cntkq::f64::valid_nbits(nbits); }
     static size_t qcol_bytes(size_t nbits, size_t rows) { return cntkq::f64::qcol_bytes(nbits, rows); }
     static hipError_t quantize(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, void* q, size_t rows,
@@ -422,9 +422,9 @@ int stripe_reduce_async_impl(cntkq_quantizer* h, const void* const* stripes, siz
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: rows and cols must be below 2^31");
     if (rows == 0 || stripe_cols == 0)
         return CNTKQ_OK;
-    if (rows > Elem<E>::kStripeMaxRows)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: columns taller than %u rows are not supported",
-                    Elem<E>::kStripeMaxRows);
+    if (rows > Elem<E>::stripe_max_rows(nbits))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: columns taller than %zu rows are not supported at %zu bits",
+                    Elem<E>::stripe_max_rows(nbits), nbits);
     if (stripe_res == nullptr || q_out == nullptr || !aligned_for<E>(stripe_res) || !aligned_for<E>(q_out) || !aligned_for<E>(agg_out))
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: null or misaligned matrix pointer");
     StripeSources src;
@@ -490,14 +490,14 @@ size_t cntkq_qmatrix_bytes_f64(size_t rows, size_t cols, size_t nbits)
     return f64::valid_nbits(nbits) ? f64::qcol_bytes(nbits, rows) * cols : 0;
 }
 
-size_t cntkq_stripe_reduce_max_rows(void)
+size_t cntkq_stripe_reduce_max_rows(size_t nbits)
 {
-    return Elem<float>::kStripeMaxRows;
+    return valid_nbits(nbits) ? Elem<float>::stripe_max_rows(nbits) : 0;
 }
 
-size_t cntkq_stripe_reduce_max_rows_f64(void)
+size_t cntkq_stripe_reduce_max_rows_f64(size_t nbits)
 {
-    return Elem<double>::kStripeMaxRows;
+    return cntkq::f64::valid_nbits(nbits) ? Elem<double>::stripe_max_rows(nbits) : 0;
 }
 
 int cntkq_stripe_range(size_t cols, size_t rank, size_t workers, size_t* start_col, size_t* num_cols)
@@ -974,7 +974,7 @@ int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduc
         return CNTKQ_OK;
     if (items == nullptr || count > 0xFFFFFF)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: bad item list");
-    size_t n = 0, only = 0;
+    size_t n = 0, only = 0, tall = 0;
     for (size_t i = 0; i < count; ++i)
     {
         const cntkq_stripe_reduce_item& it = items[i];
@@ -982,17 +982,34 @@ int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduc
             return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: rows and cols must be below 2^31", i);
         if (it.rows == 0 || it.stripe_cols == 0)
             continue;
-        if (it.rows > kTileMaxRows)
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: columns taller than %u rows are not supported", i,
-                        kTileMaxRows);
+        if (it.rows > stripe_reduce_max_rows(nbits))
+            return fail(CNTKQ_INVALID_ARGUMENT,
+                        "cntkq_stripe_reduce_batch_async: item %zu: columns taller than %zu rows are not supported at %zu bits", i,
+                        stripe_reduce_max_rows(nbits), nbits);
         if (it.stripes == nullptr || it.stripe_res == nullptr || it.q_out == nullptr || !aligned4(it.stripe_res) || !aligned4(it.q_out) ||
             !aligned4(it.agg_out))
             return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: null or misaligned pointer", i);
         for (size_t w = 0; w < workers; ++w)
             if (it.stripes[w] == nullptr || !aligned4(it.stripes[w]))
                 return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: stripe %zu is null or misaligned", i, w);
+        if (it.rows > kTileMaxRows)
+        {
+            tall++; // a launch of its own, below
+            continue;
+        }
         only = i;
         n++;
+    }
+    // tall stripes (1024 threads per column, registers) do not fit the shared grid: each is a plain call on the same stream
+    for (size_t i = 0; i < count && tall != 0; ++i)
+    {
+        const cntkq_stripe_reduce_item& it = items[i];
+        if (it.rows <= kTileMaxRows || it.stripe_cols == 0)
+            continue;
+        const int rc = cntkq_stripe_reduce_async(h, it.stripes, workers, owner, it.rows, it.stripe_cols, nbits, it.stripe_res, it.q_out,
+                                                 it.agg_out, zero_threshold_for_1bit);
+        if (rc != CNTKQ_OK)
+            return rc;
     }
     if (n == 0)
         return CNTKQ_OK;
@@ -1042,7 +1059,7 @@ int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduc
             for (size_t i = 0; i < count; ++i)
             {
                 const cntkq_stripe_reduce_item& it = items[i];
-                if (it.rows == 0 || it.stripe_cols == 0)
+                if (it.rows == 0 || it.stripe_cols == 0 || it.rows > kTileMaxRows)
                     continue;
                 // the kernel family the plain call would take, so that both give the same bytes
                 const bool col = stripe_auto_col(it.rows);

@@ -172,11 +172,16 @@ inline bool columns_start_on_lines(const void* r_in, size_t rows, size_t rows_pe
     return (reinterpret_cast<uintptr_t>(r_in) & 127u) == 0 && rows % rows_per_line == 0;
 }
 
-// Column kernels sum their statistics in the order of line-aligned slots when the three matrices share their offset
-// within a line and some column starts inside one.
+// Column kernels sum their statistics in the order of line-aligned slots when some column of the residual starts
+// inside a 128-byte line.
 inline bool quantize_line_shift(const float* g, const float* r_in, const float* r_out, size_t rows)
 {
-    return same_line_offset(g, r_in, r_out) && !columns_start_on_lines(r_in, rows);
+    // The residual's address alone decides (the slot dealing is part of the summation order, and the stripe reduction,
+    // which must reproduce it, knows only the stripe residual); a gradient at another offset within a line is then
+    // simply read across line boundaries.
+    (void) g;
+    (void) r_out;
+    return !columns_start_on_lines(r_in, rows);
 }
 
 // the unrolled 1-bit kernels: 1024, 2048 or 4096 rows and 8-byte aligned packed buffers
@@ -442,7 +447,7 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
             // not whole aligned pieces: the variant with edge elements, where the three matrices allow it
             if (!reg_edge_applicable(g, r_in, r_out, q, rows, nbits))
                 return hipErrorInvalidValue;
-            RegGeom c = make_reg_geom(rows, nbits, 1024, same_line_offset(g, r_in, r_out));
+            RegGeom c = make_reg_geom(rows, nbits, 1024, true); // always dealt by the residual's lines
             return dispatch_nbits<RegEdgeLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c);
         }
         const uint32_t threads = reg_threads(rows);
@@ -490,13 +495,73 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
                                         (uint32_t) qwords_per_col(rows, nbits), (uint64_t) qcol_bytes(nbits, rows));
 }
 
+// Tallest column the fused stripe reduction takes at this bit width: up to kTileMaxRows with the LDS kernels, above it
+// with the register kernel, whose LDS holds the output QWords and one worker's packed record.
+inline size_t stripe_reduce_max_rows(size_t nbits)
+{
+    if (nbits >= 32)
+        return kTileMaxRows;
+    const size_t max_nq = (64 * 1024 / 4 - kRegRedSlots - 2) / 2;
+    const size_t by_lds = max_nq * (32 / nbits);
+    const size_t by_regs = kRegMaxRows - 32;
+    const size_t tall = by_lds < by_regs ? by_lds : by_regs;
+    return tall > kTileMaxRows ? tall : kTileMaxRows;
+}
+
+template <int NBITS, bool ZT, int PER>
+inline hipError_t launch_stripe_reg_one(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
+                                        uint32_t cols, const RegGeom& c)
+{
+    hipExtLaunchKernelGGL((stripe_reduce_reg_kernel<NBITS, ZT, PER>), dim3(cols), dim3(1024), stripe_reg_lds_bytes(c), s, ev.start, ev.stop, 0,
+                          src, stripe_res, q_out, agg_out, c);
+    return hipGetLastError();
+}
+
+template <int NBITS, bool ZT>
+struct StripeRegLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out, uint32_t cols,
+                          RegGeom c)
+    {
+        if constexpr (NBITS >= 32)
+            return hipErrorInvalidValue;
+        else
+        {
+            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + 1023u) / 1024u;
+#define CNTKQ_SREG(P) if (per <= P) return launch_stripe_reg_one<NBITS, ZT, P>(s, ev, src, stripe_res, q_out, agg_out, cols, c)
+            CNTKQ_SREG(4);
+            CNTKQ_SREG(6);
+            CNTKQ_SREG(8);
+            CNTKQ_SREG(10);
+            CNTKQ_SREG(13);
+            CNTKQ_SREG(16);
+            CNTKQ_SREG(20);
+            CNTKQ_SREG(25);
+#undef CNTKQ_SREG
+            return hipErrorInvalidValue;
+        }
+    }
+};
+
 inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, void* q_out,
                                        float* agg_out, size_t rows, size_t cols, size_t nbits, bool zt,
                                        const LaunchTuning& tune)
 {
     zt = zt && (nbits == 1);
     if (rows > kTileMaxRows)
-        return hipErrorInvalidValue;
+    {
+        if (rows > stripe_reduce_max_rows(nbits) || (reinterpret_cast<uintptr_t>(q_out) & 3u) != 0)
+            return hipErrorInvalidValue;
+        // The slots are dealt as a quantize call on (aggregate, stripe residual) deals them, given the residual's address:
+        // whole aligned pieces and a line shift where columns start inside a line, or the variant with edge elements
+        // (always shifted); a shift that would need a 26th piece per thread is dropped there as here.
+        const bool whole = rows % 4 == 0 && (reinterpret_cast<uintptr_t>(stripe_res) & 15u) == 0;
+        bool line_shift = whole ? !columns_start_on_lines(stripe_res, rows) : true;
+        if (whole && rows / 4 + 7 > 1024 * (size_t) kRegMaxShiftPer)
+            line_shift = false;
+        const RegGeom c = make_reg_geom(rows, nbits, 1024, line_shift);
+        return dispatch_nbits<StripeRegLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols, c);
+    }
     bool aligned8 = (reinterpret_cast<uintptr_t>(q_out) & 7u) == 0;
     for (uint32_t w = 0; w < src.workers; ++w)
         aligned8 = aligned8 && (reinterpret_cast<uintptr_t>(src.q[w]) & 7u) == 0;

@@ -62,9 +62,9 @@ size_t cntkq_qmatrix_bytes(size_t rows, size_t cols, size_t nbits);
 int cntkq_stripe_range(size_t cols, size_t rank, size_t workers, size_t* start_col, size_t* num_cols);
 
 /* Tallest column the fused stripe reduction (cntkq_stripe_reduce_async / _batch_async, an optional fast path without a
- * counterpart in the reference) accepts; for taller stripes the caller keeps the reference's sequence of
+ * counterpart in the reference) accepts at this bit width (0 for an invalid width); for taller stripes the caller keeps the reference's sequence of
  * UnquantizeAsync ... QuantizeAsync calls (Source/1BitSGD/AllReduceDistGradAggregator.h:365-436). */
-size_t cntkq_stripe_reduce_max_rows(void);
+size_t cntkq_stripe_reduce_max_rows(size_t nbits);
 
 /* ---- the quantizer object -------------------------------------------------------------------- */
 
@@ -229,7 +229,7 @@ int cntkq_unquantize_async_f64(cntkq_quantizer* h, const void* qbuf, size_t qbuf
 int cntkq_stripe_reduce_async_f64(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner,
                                   size_t rows, size_t stripe_cols, size_t nbits, double* stripe_res, void* q_out,
                                   double* agg_out, int zero_threshold_for_1bit);
-size_t cntkq_stripe_reduce_max_rows_f64(void);
+size_t cntkq_stripe_reduce_max_rows_f64(size_t nbits);
 
 #ifdef __cplusplus
 }

@@ -5,6 +5,7 @@ All K workers live in one GPU's memory. The fp32 sum inside the stripe reduction
 first, then ascending rank), so the fp32 aggregate must equal the oracle's bit for bit; the requantized
 stripe is then checked like any quantize result.
 """
+import ctypes
 import sys
 
 import numpy as np
@@ -53,6 +54,9 @@ CASES = [
     (2048, 20, 11, 1, False), (1024, 24, 4, 1, False), (1024, 9, 64, 1, True), (4096, 5, 64, 1, False),
     # tall columns: 1024 threads per column in the stripe reduction, register kernels in the call sequence
     (9304, 6, 4, 1, False), (8192, 4, 3, 4, False), (12000, 4, 5, 2, False), (14336, 2, 2, 8, False),
+    # above 14336 rows: the register kernel's shape (the running sum in registers, one worker's record at a time in LDS)
+    (14340, 6, 4, 1, False), (14337, 3, 2, 2, False), (20000, 5, 3, 1, True), (32768, 4, 5, 4, False), (50257, 3, 8, 1, False),
+    (100000, 2, 2, 1, False), (102365, 2, 3, 2, False), (16332, 2, 2, 16, False),
 ]
 
 
@@ -72,7 +76,7 @@ def test_stripe_reduce(case):
         sres = datagen.normal(900 + owner, rows, n, 0.003)
         # heights that are a multiple of 4 can take the kernels with one workgroup per column (path 3; the automatic
         # choice from 1024 rows on) as well as the tile kernels (path 1)
-        variants = [(True, 0), (False, 0)] + ([(True, 1), (True, 3)] if rows % 4 == 0 else [])
+        variants = [(True, 0), (False, 0)] + ([(True, 1), (True, 3)] if rows % 4 == 0 and rows <= 14336 else [])
         for alias, path in variants:
             qz._set_tuning(quantize_path=path)
             q_new, s_new, agg = gpu_stripe_reduce(qz, qs, owner, rows, cols, nbits, sres, zt, alias_out=alias)
@@ -101,6 +105,22 @@ def test_stripe_reduce(case):
                 assert np.array_equal(Qo.to_numpy(), q_new), "fused != call sequence (codes)"
                 assert parity.bits_equal(S.to_numpy(), s_new), "fused != call sequence (residual)"
     say("  ", rep)
+
+
+def test_stripe_reduce_height_limit():
+    """The tallest stripe the fused call takes depends on the bit width (its LDS holds the output QWords and one worker's
+    record); taller ones are refused, and the limit can be asked for."""
+    L = cntk_amd.lib()
+    L.cntkq_stripe_reduce_max_rows.restype = ctypes.c_size_t
+    L.cntkq_stripe_reduce_max_rows.argtypes = [ctypes.c_size_t]
+    assert L.cntkq_stripe_reduce_max_rows(1) == 102368 and L.cntkq_stripe_reduce_max_rows(32) == 14336
+    assert L.cntkq_stripe_reduce_max_rows(16) == 16334 and L.cntkq_stripe_reduce_max_rows(3) == 0
+    qz = MatrixQuantizerImpl.Create(0, False)
+    rows, cols, k = 16336, 2, 2
+    zeros = np.zeros((rows, cols), np.float32, order="F")
+    qs = [oracle.quantize(datagen.normal(5 + w, rows, cols), zeros, 16, False)[0] for w in range(k)]
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        gpu_stripe_reduce(qz, qs, 0, rows, cols, 16, np.zeros((rows, 1), np.float32, order="F"), False)
 
 
 def test_stripe_reduce_32bit_equals_plain_sum():
