@@ -94,6 +94,9 @@ def lib():
         L.cntkq_unquantize_async_f64.argtypes = L.cntkq_unquantize_async.argtypes
         L.cntkq_stripe_reduce_async_f64.argtypes = L.cntkq_stripe_reduce_async.argtypes
         L.cntkq_stripe_reduce_batch_async.argtypes = [_vp, ctypes.POINTER(_StripeReduceItem), _sz, _sz, _sz, _sz, ctypes.c_int]
+        for name in ("cntkq_stripe_reduce_max_rows", "cntkq_stripe_reduce_max_rows_f64"):
+            getattr(L, name).argtypes = [_sz]
+            getattr(L, name).restype = _sz
         L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int]
         _lib = L
     return _lib
@@ -257,6 +260,14 @@ class QuantizedMatrix:
         self.buffer.copy_(torch.from_numpy(np.ascontiguousarray(a, dtype=np.uint8)))
 
 
+class PreparedBatch:
+    """The argument block of one batched call, built once by MatrixQuantizerImpl.Prepare...Batch. It holds addresses,
+    not matrices: the caller keeps the matrices alive and in place for as long as it uses the block."""
+
+    def __init__(self, kind, array, count, nbits, keep, workers=0):
+        self.kind, self.array, self.count, self.nbits, self.keep, self.workers = kind, array, count, nbits, keep, workers
+
+
 class MatrixQuantizerImpl:
     """The quantizer object (Source/Math/MatrixQuantizerImpl.h:19-49) for one GPU."""
 
@@ -283,6 +294,12 @@ class MatrixQuantizerImpl:
 
     def stream(self):
         return lib().cntkq_stream(self._h)
+
+    def SetMainStream(self, hip_stream):
+        """The stream a quantizer without a dedicated stream issues on, and the one SynchronizeWithMainStream orders
+        against (the reference's GetStream(), Source/Math/MatrixQuantizerGPU.cu:248-252); a hipStream_t as an integer,
+        e.g. torch.cuda.current_stream().cuda_stream."""
+        _check(lib().cntkq_set_main_stream(self._h, hip_stream))
 
     def SynchronizeWithMainStream(self):
         """MatrixComputeStreamEvent::SynchronizeQuantizationComputeStreamWithEvent
@@ -328,8 +345,21 @@ class MatrixQuantizerImpl:
         """The aggregator's loop over its gradient matrices as one call (Source/1BitSGD/AllReduceDistGradAggregator.h:288-300).
         items: sequence of (in_matrix, in_residual, out_qmatrix, out_residual); all packed matrices on the device and of
         one bit width."""
-        if not items:
+        if isinstance(items, PreparedBatch):
+            if items.kind != "quantize":
+                raise QuantizerLogicError("QuantizeBatchAsync: prepared for another call")
+            if items.count:
+                _check(lib().cntkq_quantize_batch_async(self._h, items.array, items.count, items.nbits,
+                                                        int(bool(zero_threshold_for_1bit))))
             return
+        self.QuantizeBatchAsync(self.PrepareQuantizeBatch(items), zero_threshold_for_1bit)
+
+    @staticmethod
+    def PrepareQuantizeBatch(items):
+        """Checks the items of QuantizeBatchAsync and lays them out for the call once; the result can be passed to
+        QuantizeBatchAsync in place of the item list for as long as the matrices stay where they are."""
+        if not items:
+            return PreparedBatch("quantize", None, 0, 0, ())
         nbits = items[0][2].GetNumBits()
         arr = (_QuantizeItem * len(items))()
         for k, (g, r_in, q, r_out) in enumerate(items):
@@ -342,13 +372,24 @@ class MatrixQuantizerImpl:
             if any(m.dtype != torch.float32 for m in (g, r_in, r_out, q)):
                 raise QuantizerLogicError("QuantizeBatchAsync: the batched calls exist for float32 only")
             arr[k] = _QuantizeItem(g.Data(), r_in.Data(), r_out.Data(), q.Buffer(), rows, cols)
-        _check(lib().cntkq_quantize_batch_async(self._h, arr, len(items), nbits, int(bool(zero_threshold_for_1bit))))
+        return PreparedBatch("quantize", arr, len(items), nbits, ())
 
     def UnquantizeBatchAsync(self, items, add=False):
         """The aggregator's final loop (Source/1BitSGD/AllReduceDistGradAggregator.h:517-522) as one call.
         items: sequence of (in_qmatrix, out_matrix)."""
-        if not items:
+        if isinstance(items, PreparedBatch):
+            if items.kind != "unquantize":
+                raise QuantizerLogicError("UnquantizeBatchAsync: prepared for another call")
+            if items.count:
+                _check(lib().cntkq_unquantize_batch_async(self._h, items.array, items.count, items.nbits, int(bool(add))))
             return
+        self.UnquantizeBatchAsync(self.PrepareUnquantizeBatch(items), add)
+
+    @staticmethod
+    def PrepareUnquantizeBatch(items):
+        """The items of UnquantizeBatchAsync, checked and laid out once (see PrepareQuantizeBatch)."""
+        if not items:
+            return PreparedBatch("unquantize", None, 0, 0, ())
         nbits = items[0][0].GetNumBits()
         arr = (_UnquantizeItem * len(items))()
         for k, (q, out) in enumerate(items):
@@ -359,7 +400,7 @@ class MatrixQuantizerImpl:
             if q.dtype != torch.float32 or out.dtype != torch.float32:
                 raise QuantizerLogicError("UnquantizeBatchAsync: the batched calls exist for float32 only")
             arr[k] = _UnquantizeItem(q.Buffer(), out.Data(), out.GetNumRows(), out.GetNumCols())
-        _check(lib().cntkq_unquantize_batch_async(self._h, arr, len(items), nbits, int(bool(add))))
+        return PreparedBatch("unquantize", arr, len(items), nbits, ())
 
     def StripeReduceAsync(self, stripes, owner, stripe_residual, out_qstripe, zero_threshold_for_1bit, agg_out=None):
         """Fused stripe reduction of the quantized all-reduce (dataflow of
@@ -383,8 +424,20 @@ class MatrixQuantizerImpl:
     def StripeReduceBatchAsync(self, items, owner, zero_threshold_for_1bit):
         """The owner's stripe reductions of a whole gradient set as one call. items: sequence of
         (stripes, stripe_residual, out_qstripe, agg_out or None), one per gradient matrix, float32 only."""
-        if not items:
+        if isinstance(items, PreparedBatch):
+            if items.kind != "stripe_reduce":
+                raise QuantizerLogicError("StripeReduceBatchAsync: prepared for another call")
+            if items.count:
+                _check(lib().cntkq_stripe_reduce_batch_async(self._h, items.array, items.count, items.workers, owner, items.nbits,
+                                                             int(bool(zero_threshold_for_1bit))))
             return
+        self.StripeReduceBatchAsync(self.PrepareStripeReduceBatch(items), owner, zero_threshold_for_1bit)
+
+    @staticmethod
+    def PrepareStripeReduceBatch(items):
+        """The items of StripeReduceBatchAsync, checked and laid out once (see PrepareQuantizeBatch)."""
+        if not items:
+            return PreparedBatch("stripe_reduce", None, 0, 0, ())
         k = len(items[0][0])
         nbits = items[0][2].GetNumBits()
         arr = (_StripeReduceItem * len(items))()
@@ -405,8 +458,7 @@ class MatrixQuantizerImpl:
             keep.append(ptrs)
             arr[n] = _StripeReduceItem(ptrs, stripe_residual.Data(), out_qstripe.Buffer(),
                                        agg_out.Data() if agg_out is not None else None, rows, cols)
-        _check(lib().cntkq_stripe_reduce_batch_async(self._h, arr, len(items), k, owner, nbits,
-                                                     int(bool(zero_threshold_for_1bit))))
+        return PreparedBatch("stripe_reduce", arr, len(items), nbits, keep, workers=k)
 
     def WaitStripeReduceDone(self):
         _check(lib().cntkq_wait_stripe_reduce_done(self._h))
