@@ -113,6 +113,7 @@ struct StripeLauncher
 // at most 25 pieces of two doubles for each of 1024 threads, QWords within 64 KB of LDS.
 constexpr uint32_t kRegThreads = 1024;
 constexpr size_t kRegMaxRows = 2 * 1024 * 25;
+constexpr size_t kRegMinRows = 4992; // below, the tile kernel is faster
 
 inline bool reg_applicable(const double* g, const double* r_in, const double* r_out, size_t rows, size_t nbits)
 {
@@ -179,7 +180,15 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* 
     char* qc = static_cast<char*>(q);
     int path = tune.quantize_path;
     if (path == kPathAuto)
-        path = rows <= kTileMaxRows ? kPathTile : (reg_applicable(g, r_in, r_out, rows, nbits) ? kPathReg : kPathTall);
+    {
+        // one column of doubles per tile fills LDS from about 5000 rows on (two workgroups per CU at 5120 rows, one at
+        // 7168); the register kernel overtakes the tile kernel there: 5120 rows 88 us against 94 us on 19 M elements,
+        // 6144: 85 against 99, 7168: 81 against 112 (4096: 104 against 85)
+        if (rows >= kRegMinRows && reg_applicable(g, r_in, r_out, rows, nbits))
+            path = kPathReg;
+        else
+            path = rows <= kTileMaxRows ? kPathTile : kPathTall;
+    }
     if (path == kPathReg)
     {
         if (!reg_applicable(g, r_in, r_out, rows, nbits))
@@ -203,7 +212,9 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* 
                                         (uint32_t) qwords_per_col(rows, nbits), (uint64_t) qcol_bytes(nbits, rows));
 }
 
-// Same tile geometry as launch_quantize, so that the fused call gives the bytes of the unquantize ... quantize call sequence.
+// Same tile geometry as launch_quantize, so that the fused call gives the bytes of the unquantize ... quantize call sequence
+// wherever that sequence's quantize runs the tile kernel (below kRegMinRows rows); above, the two agree within the
+// tolerance of the column bounds.
 inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, double* stripe_res, void* q_out,
                                        double* agg_out, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
 {

@@ -301,7 +301,7 @@ def unfused_reference(qz, stripes_np, owner, rows, n, nbits, sres, zt):
     return Agg.to_numpy(), Qo.to_numpy(), S.to_numpy()
 
 
-@pytest.mark.parametrize("rows,n,k", [(70, 9, 3), (429, 12, 4), (2048, 20, 8), (4096, 3, 2), (7168, 2, 5), (64, 40, 64)])
+@pytest.mark.parametrize("rows,n,k", [(70, 9, 3), (429, 12, 4), (2048, 20, 8), (4096, 3, 2), (4988, 3, 3), (7168, 2, 5), (64, 40, 64)])
 def test_stripe_reduce_f64(quantizer, rows, n, k):
     for nbits, zt in VARIANTS:
         say("f64 stripe reduce", rows, n, k, nbits, zt)
@@ -326,9 +326,13 @@ def test_stripe_reduce_f64(quantizer, rows, n, k):
             assert parity.bits_equal(Agg.to_numpy(), agg_o), "aggregate differs from the ordered sum"
             parity.check_quantize(agg_o, sres, Qs[owner].to_numpy(), S.to_numpy(), nbits, zt)
             # the fused call gives the very bytes of the reference's unquantize ... quantize call sequence
+            # (up to 4991 rows, where the sequence's quantize is the tile kernel the fused call shares its order with)
             agg_u, q_u, s_u = unfused_reference(quantizer, stripes, owner, rows, n, nbits, sres, zt)
             assert parity.bits_equal(agg_u, agg_o)
-            assert np.array_equal(q_u, Qs[owner].to_numpy()) and parity.bits_equal(s_u, S.to_numpy())
+            if rows < 4992:
+                assert np.array_equal(q_u, Qs[owner].to_numpy()) and parity.bits_equal(s_u, S.to_numpy())
+            else:
+                parity.check_quantize(agg_o, sres, q_u, s_u, nbits, zt)
 
 
 def test_end_to_end_allreduce_f64(quantizer):

@@ -56,7 +56,7 @@ CASES = [
     (9304, 6, 4, 1, False), (8192, 4, 3, 4, False), (12000, 4, 5, 2, False), (14336, 2, 2, 8, False),
     # above 14336 rows: the register kernel's shape (the running sum in registers, one worker's record at a time in LDS)
     (14340, 6, 4, 1, False), (14337, 3, 2, 2, False), (20000, 5, 3, 1, True), (32768, 4, 5, 4, False), (50257, 3, 8, 1, False),
-    (100000, 2, 2, 1, False), (102365, 2, 3, 2, False), (16332, 2, 2, 16, False),
+    (100000, 2, 2, 1, False), (102365, 2, 3, 2, False), (16332, 2, 2, 16, False), (32668, 2, 2, 8, False),
 ]
 
 
