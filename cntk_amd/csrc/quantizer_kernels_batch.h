@@ -1,0 +1,142 @@
+// gfx950 kernels of the per-column gradient quantizer: whole gradient sets in one launch.
+#pragma once
+
+#include "quantizer_kernels_column.h"
+#include "quantizer_kernels_unquantize.h"
+
+namespace cntkq {
+
+// largest e with begins[e] <= b; b and everything derived from it is uniform over the workgroup
+__device__ __forceinline__ uint32_t batch_find(const uint32_t* __restrict__ begins, uint32_t count, uint32_t b)
+{
+    uint32_t lo = 0, hi = count;
+    while (hi - lo > 1)
+    {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (begins[mid] <= b)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    return lo;
+}
+
+// Many matrices in one launch: the workgroups of all matrices form one grid; `begins` (count + 1 entries, ascending)
+// gives the first workgroup of every matrix. A matrix is a run of column tiles (quantize_tile_body) or of single columns
+// (quantize_colg_body). Removes the per-launch floor (several microseconds) that dominates gradient sets made of many
+// small matrices.
+struct QuantizeBatchEntry
+{
+    const float* g;
+    const float* r_in;
+    float* r_out;
+    char* q;
+    uint32_t kind; // 0: tiles (t), 1: columns (c)
+    uint32_t pad;
+    TileGeom t;
+    ColGeom c;
+};
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTileThreads) void quantize_batch_kernel(const QuantizeBatchEntry* __restrict__ entries,
+                                                                      const uint32_t* __restrict__ begins, uint32_t count)
+{
+    extern __shared__ f32x4 smem_v4[];
+    const uint32_t e = batch_find(begins, count, blockIdx.x);
+    const uint32_t index = blockIdx.x - begins[e];
+    // geometry by value: read once, then held in registers whatever the kernel stores
+    if (entries[e].kind == 0)
+    {
+        const TileGeom t = entries[e].t;
+        quantize_tile_body<NBITS, ZT>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, t, index);
+    }
+    else
+    {
+        const ColGeom c = entries[e].c;
+        quantize_colg_body<NBITS, ZT>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, c, index, smem_v4);
+    }
+}
+
+// The owner's stripe reductions of a whole gradient set in one launch: same grid construction as quantize_batch_kernel.
+struct StripeBatchEntry
+{
+    StripeSources src;
+    float* stripe_res;
+    char* q_out;
+    float* agg_out;
+    uint32_t kind; // 0: tiles (t), 1: columns (c)
+    uint32_t pad;
+    TileGeom t;
+    ColGeom c;
+};
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTileThreads) void stripe_reduce_batch_kernel(const StripeBatchEntry* __restrict__ entries,
+                                                                           const uint32_t* __restrict__ begins, uint32_t count)
+{
+    extern __shared__ f32x4 smem_v4[];
+    const uint32_t e = batch_find(begins, count, blockIdx.x);
+    const uint32_t index = blockIdx.x - begins[e];
+    const StripeBatchEntry& en = entries[e]; // the table is read-only while the kernel runs
+    if (en.kind == 0)
+    {
+        const TileGeom t = en.t;
+        stripe_reduce_tile_body<NBITS, ZT>(en.src, en.stripe_res, en.q_out, en.agg_out, t, index);
+    }
+    else
+    {
+        const ColGeom c = en.c;
+        stripe_reduce_colg_body<NBITS, ZT>(en.src, en.stripe_res, en.q_out, en.agg_out, c, index, smem_v4);
+    }
+}
+
+
+// Many matrices in one launch (see quantize_batch_kernel): the 256-thread blocks of all matrices form one grid.
+enum UnqKind : uint32_t
+{
+    kUnqVec4 = 0,    // QWord-major, 16-byte stores
+    kUnqScalar = 1,  // QWord-major, 4-byte stores
+    kUnqSegment = 2, // segment decoder
+    kUnqRows = 3,    // row-major decoder, packed column in LDS
+    kUnqTile = 4     // several short columns per workgroup, packed records in LDS
+};
+
+struct UnquantizeBatchEntry
+{
+    const char* q;
+    float* out;
+    uint32_t kind;
+    uint32_t pad;
+    UnqGeom qw;      // valid for kUnqVec4 / kUnqScalar
+    UnqSegGeom seg;  // valid for kUnqSegment
+    UnqRowGeom rowg; // valid for kUnqRows
+    UnqTileGeom tile; // valid for kUnqTile
+};
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_batch_kernel(const UnquantizeBatchEntry* __restrict__ entries,
+                                                               const uint32_t* __restrict__ begins, uint32_t count, int add)
+{
+    extern __shared__ f32x4 smem_v4[];
+    const uint32_t e = batch_find(begins, count, blockIdx.x);
+    const UnquantizeBatchEntry& en = entries[e];
+    const uint32_t block = blockIdx.x - begins[e];
+    if (en.kind == kUnqVec4)
+        unquantize_body<NBITS, 4>(en.q, en.out, en.qw, add, block);
+    else if (en.kind == kUnqScalar)
+        unquantize_body<NBITS, 1>(en.q, en.out, en.qw, add, block);
+    else if (en.kind == kUnqSegment)
+        unquantize_segment_body<NBITS>(en.q, en.out, en.seg, add, block);
+    else if (en.kind == kUnqRows)
+    {
+        const UnqRowGeom t = en.rowg; // by value: the loop below stores between its uses
+        unquantize_rows_body<NBITS>(en.q, en.out, t, add, block, reinterpret_cast<uint32_t*>(smem_v4));
+    }
+    else
+    {
+        const UnqTileGeom t = en.tile;
+        unquantize_tile_body<NBITS>(en.q, en.out, t, add, block, reinterpret_cast<uint32_t*>(smem_v4));
+    }
+}
+
+} // namespace cntkq

@@ -1,0 +1,661 @@
+// gfx950 kernels of the per-column gradient quantizer: one workgroup per column, the column in LDS,
+// for quantize and for the stripe reduction.
+#pragma once
+
+#include "quantizer_kernels_tile.h"
+
+namespace cntkq {
+
+// ---- quantize, 1 bit, one workgroup per column, rows = 1024 * PER (PER = 1, 2, 4) ---------------------------
+//
+// 256 threads own one column: each loads PER 16-byte pieces of gradient and residual, adds them into an LDS copy
+// of the column and sums its own values on the way, so the column mean needs no second pass. The split sums are
+// then taken from LDS (thread t takes rows t, t + 256, ...), and the codes are packed from LDS by work items of
+// (QWord, run of 4 * PER bit positions), whose partial words meet in LDS. Few registers and 4..16 KB of LDS per
+// workgroup keep 8 workgroups resident per CU; that, not wider stores, is what brings this kernel to the rate of a
+// plain read-read-write stream.
+
+constexpr uint32_t kColThreads = 256;
+
+struct ColLds
+{
+    float* tile;      // 1024 * PER floats, 16-byte aligned
+    uint32_t* words;  // 32 * PER partial QWords
+    float* red_f;     // 2 * 4 floats
+    uint32_t* red_u;  // 4
+};
+
+template <int PER>
+__device__ __forceinline__ ColLds col_lds(f32x4* smem)
+{
+    ColLds l;
+    l.tile = reinterpret_cast<float*>(smem);
+    l.words = reinterpret_cast<uint32_t*>(l.tile + 1024 * PER);
+    l.red_f = reinterpret_cast<float*>(l.words + 32 * PER);
+    l.red_u = reinterpret_cast<uint32_t*>(l.red_f + 8);
+    return l;
+}
+
+template <int PER>
+constexpr size_t col_lds_bytes()
+{
+    return (size_t) (1024 * PER + 32 * PER + 8 + 4) * 4;
+}
+
+// The 1-bit split sums of one 16-byte piece (x y z w in order): values below the mean go to s0 / n0, the others to s1.
+// Like the column sum, the split sums are taken piece by piece by every column kernel, whether it keeps the column in
+// LDS or in registers, so that all of them give the same header for the same column.
+__device__ __forceinline__ void split_add_piece(const f32x4& v, float mean, float& s0, float& s1, uint32_t& n0)
+{
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+    {
+        const float x = v[c];
+        const bool below = x < mean;
+        s0 += below ? x : 0.0f;
+        s1 += below ? 0.0f : x;
+        n0 += below ? 1u : 0u;
+    }
+}
+
+// Sum of the values thread tid holds when the column is cut into 16-byte pieces tid, tid + 256, ...: in that order,
+// x y z w within a piece. Both the quantize and the stripe-reduction kernel take the column mean from these
+// per-thread sums, so they produce identical headers for identical columns.
+template <int PER>
+__device__ __forceinline__ float col_thread_sum(const f32x4 (&v)[PER])
+{
+    float s = 0.0f;
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+    {
+        s += v[u].x;
+        s += v[u].y;
+        s += v[u].z;
+        s += v[u].w;
+    }
+    return s;
+}
+
+// Statistics, header, codes and residual of the column held in l.tile. csum: this thread's col_thread_sum
+// (ignored when ZT). l.words[0 .. 32 * PER) must be zero; no barrier is needed between writing l.tile / l.words
+// and calling this. res_col: the column of the residual output; qc: the packed column record (8-byte aligned).
+template <bool ZT, int PER>
+__device__ __forceinline__ void col_stats_pack(const ColLds& l, float csum, float* res_col, char* qc)
+{
+    constexpr uint32_t ROWS = 1024 * PER, NQ = 32 * PER, T = kColThreads, NW = T / 64;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    float mean = 0.0f;
+    if constexpr (!ZT)
+    {
+        const float s = wave_sum(csum);
+        if (lane == 0)
+            l.red_f[wave] = s;
+    }
+    __syncthreads(); // the column and the wave sums are visible
+    if constexpr (!ZT)
+    {
+        float s = l.red_f[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+            s += l.red_f[x];
+        mean = s / (float) ROWS;
+    }
+    float s0 = 0.0f, s1 = 0.0f;
+    uint32_t n0 = 0;
+    {
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(l.tile);
+#pragma unroll
+        for (uint32_t u = 0; u < PER; ++u)
+            split_add_piece(t4[tid + T * u], mean, s0, s1, n0);
+    }
+    s0 = wave_sum(s0);
+    s1 = wave_sum(s1);
+    n0 = wave_sum(n0);
+    __syncthreads(); // everyone has read the wave sums of the mean
+    if (lane == 0)
+    {
+        l.red_f[wave] = s0;
+        l.red_f[4 + wave] = s1;
+        l.red_u[wave] = n0;
+    }
+    __syncthreads();
+    float S0 = l.red_f[0], S1 = l.red_f[4];
+    uint32_t N0 = l.red_u[0];
+#pragma unroll
+    for (uint32_t x = 1; x < NW; ++x)
+    {
+        S0 += l.red_f[x];
+        S1 += l.red_f[4 + x];
+        N0 += l.red_u[x];
+    }
+    float lo, hi;
+    finish_stats_1bit<ZT>(mean, S0, S1, N0, ROWS - N0, ROWS, lo, hi);
+    if (tid == 0)
+    {
+        f32x2 h;
+        h.x = lo;
+        h.y = hi;
+        *reinterpret_cast<f32x2*>(qc) = h;
+    }
+    const ValueQ vq = make_vq<1>(lo, hi);
+    const float val0 = unquantize_value<1>(vq, 0u);
+    const float val1 = unquantize_value<1>(vq, 1u);
+    // work item = (QWord p, chunk of KS bit positions); NQ * (32 / KS) = 256 items
+    constexpr uint32_t KS = 4 * PER;
+    const uint32_t p = tid % NQ, chunk = tid / NQ;
+    uint32_t word = 0;
+#pragma unroll
+    for (uint32_t kk = 0; kk < KS; ++kk)
+    {
+        const uint32_t k = chunk * KS + kk;
+        const uint32_t i = p + NQ * k;
+        const float x = l.tile[i];
+        const uint32_t code = quantize_value<1, ZT>(vq, x);
+        __builtin_nontemporal_store(x - (code ? val1 : val0), res_col + i);
+        word |= code << k;
+    }
+    atomicOr(&l.words[p], word);
+    __syncthreads();
+    if (tid < NQ)
+        reinterpret_cast<uint32_t*>(qc + 8)[tid] = l.words[tid];
+}
+
+template <bool ZT, int PER>
+__global__ __launch_bounds__(kColThreads) void quantize_col_kernel(const float* __restrict__ g, const float* r_in, float* r_out,
+                                                                   char* __restrict__ q, uint64_t qcol)
+{
+    constexpr uint32_t ROWS = 1024 * PER, T = kColThreads;
+    extern __shared__ f32x4 smem_v4[];
+    const ColLds l = col_lds<PER>(smem_v4);
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * ROWS;
+    if (tid < 32 * PER)
+        l.words[tid] = 0u;
+    const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base);
+    const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base);
+    f32x4* t4 = reinterpret_cast<f32x4*>(l.tile);
+    f32x4 a[PER], b[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+    {
+        a[u] = __builtin_nontemporal_load(g4 + tid + T * u);
+        b[u] = __builtin_nontemporal_load(r4 + tid + T * u);
+    }
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+    {
+        a[u] = a[u] + b[u];
+        t4[tid + T * u] = a[u];
+    }
+    // the whole column has been read before col_stats_pack's first barrier, so r_out may be r_in
+    col_stats_pack<ZT, PER>(l, col_thread_sum<PER>(a), r_out + base, q + (size_t) blockIdx.x * qcol);
+}
+
+// Stripe reduction in the same shape: the work item that will pack (QWord p, chunk) first decodes those bit positions
+// from every worker's packed stripe, sums them (owner first, then ascending) and adds the stripe residual.
+template <bool ZT, int PER>
+__global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSources src, float* stripe_res, char* q_out,
+                                                                        float* agg_out, uint64_t qcol)
+{
+    constexpr uint32_t ROWS = 1024 * PER, NQ = 32 * PER, T = kColThreads, KS = 4 * PER, BATCH = 8;
+    extern __shared__ f32x4 smem_v4[];
+    const ColLds l = col_lds<PER>(smem_v4);
+    float* dec = reinterpret_cast<float*>(l.red_u + 4); // two reconstruction levels per worker, in summation order
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * ROWS;
+    const size_t rec = (size_t) blockIdx.x * qcol;
+    const uint32_t K = src.workers;
+    if (tid < NQ)
+        l.words[tid] = 0u;
+    // Everything this thread will need from memory is requested before the first barrier, so that the headers, the
+    // first eight workers' QWords and the stripe residual cost one round trip, not three: a stripe is one GPU's share
+    // of a matrix, a single round of workgroups, and its time is the length of this dependent chain.
+    const uint32_t p = tid % NQ, chunk = tid / NQ;
+    const uint32_t sh0 = chunk * KS;
+    uint32_t word[BATCH];
+#pragma unroll
+    for (uint32_t u = 0; u < BATCH; ++u)
+        if (u < K)
+            word[u] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(u, src.owner)] + rec + 8)[p];
+    const float* sp = stripe_res + base;
+    float resid[KS];
+#pragma unroll
+    for (uint32_t kk = 0; kk < KS; ++kk)
+        resid[kk] = __builtin_nontemporal_load(sp + p + NQ * (sh0 + kk));
+    if (tid < K)
+    {
+        const float* h = reinterpret_cast<const float*>(src.q[stripe_order(tid, src.owner)] + rec);
+        const ValueQ vq = make_vq<1>(h[0], h[1]);
+        dec[2 * tid] = unquantize_value<1>(vq, 0u);
+        dec[2 * tid + 1] = unquantize_value<1>(vq, 1u);
+    }
+    __syncthreads();
+
+    float acc[KS];
+    for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
+    {
+        if (n0 != 0)
+        {
+#pragma unroll
+            for (uint32_t u = 0; u < BATCH; ++u)
+                if (n0 + u < K)
+                    word[u] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + rec + 8)[p];
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < BATCH; ++u)
+        {
+            if (n0 + u < K)
+            {
+                const float val0 = dec[2 * (n0 + u)], val1 = dec[2 * (n0 + u) + 1];
+                const uint32_t bits = word[u] >> sh0;
+#pragma unroll
+                for (uint32_t kk = 0; kk < KS; ++kk)
+                {
+                    const float x = ((bits >> kk) & 1u) ? val1 : val0;
+                    // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
+                    acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (uint32_t kk = 0; kk < KS; ++kk)
+    {
+        const uint32_t i = p + NQ * (sh0 + kk);
+        if (agg_out != nullptr)
+            agg_out[base + i] = acc[kk];
+        l.tile[i] = acc[kk] + resid[kk];
+    }
+    float csum = 0.0f;
+    if constexpr (!ZT)
+    {
+        __syncthreads();
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(l.tile);
+        f32x4 v[PER];
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            v[u] = t4[tid + T * u];
+        csum = col_thread_sum<PER>(v);
+    }
+    col_stats_pack<ZT, PER>(l, csum, stripe_res + base, q_out + rec);
+}
+
+// ---- the same decomposition for any bit width and any column height that is a multiple of 4 ----------------
+//
+// One workgroup of 256 threads per column, the column in LDS. The running statistic (sum for 1 bit, sum of squares
+// otherwise) is taken piece by piece while loading, in the order col_thread_sum defines, so for 1 bit and 1024 * PER
+// rows these kernels give the very bytes of the unrolled ones above.
+
+// How a column's 16-byte pieces are dealt to the slots of a workgroup (slot v = thread + T * u). With line_shift set,
+// slot v holds piece v - shift, shift = the column's offset into its 128-byte line in pieces (the residual input's
+// address decides; the launch sets line_shift only when gradient and residual output share that offset).
+__device__ __forceinline__ uint32_t column_shift(const void* column, uint32_t line_shift)
+{
+    return line_shift ? (uint32_t) ((reinterpret_cast<uintptr_t>(column) >> 4) & 7u) : 0u;
+}
+
+__device__ __forceinline__ bool slot_valid(uint32_t v, uint32_t shift, uint32_t pieces)
+{
+    return v >= shift && v - shift < pieces;
+}
+
+// the piece a slot loads: its own, or (outside the column) the column's first or last
+__device__ __forceinline__ uint32_t slot_piece(uint32_t v, uint32_t shift, uint32_t last)
+{
+    const uint32_t p = v < shift ? 0u : v - shift;
+    return p < last ? p : last;
+}
+
+struct ColGeom
+{
+    uint32_t rows;   // multiple of 4
+    uint32_t nq;
+    uint32_t pieces; // rows / 4
+    uint32_t line_shift; // non-zero: statistics are summed in the order of line-aligned slots (see column_shift)
+    uint64_t qcol;
+};
+
+// LDS in floats: [column | partial QWords (nq when a QWord has several work items) | 12 reduction slots | decode constants]
+template <int NBITS>
+__host__ __device__ inline size_t colg_lds_bytes(const ColGeom& c, uint32_t workers)
+{
+    return ((size_t) c.rows + (PackShape<NBITS>::CHUNKS > 1 ? c.nq : 0) + 12 + (size_t) 2 * workers) * sizeof(float);
+}
+
+template <int NBITS>
+__device__ __forceinline__ float colg_add_piece(float s, const f32x4& v)
+{
+    if constexpr (NBITS == 1)
+    {
+        s += v.x;
+        s += v.y;
+        s += v.z;
+        s += v.w;
+    }
+    else
+    {
+        s += v.x * v.x;
+        s += v.y * v.y;
+        s += v.z * v.z;
+        s += v.w * v.w;
+    }
+    return s;
+}
+
+// stat: this thread's running statistic over its pieces (unused for 1 bit with ZT). tile = the column, words = zeroed
+// partial QWords, red = 12 reduction slots. No barrier is needed between writing the column and calling this.
+// WG: threads in the workgroup. The sums are always taken by the first 256 threads (their order is part of the result);
+// coding and packing use all of them.
+template <int NBITS, bool ZT, int WG = kColThreads>
+__device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, float* red, const ColGeom& c, float stat,
+                                                uint32_t shift, float* res_col, char* qc)
+{
+    using PS = PackShape<NBITS>;
+    constexpr uint32_t T = kColThreads, NW = T / 64;
+    static_assert(WG >= (int) T && WG % 64 == 0, "workgroup size");
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 8);
+    constexpr bool need_stat = (NBITS != 1) || !ZT;
+    float total = 0.0f;
+    if constexpr (need_stat)
+    {
+        const float s = wave_sum(stat);
+        if (lane == 0 && wave < NW)
+            red[wave] = s;
+    }
+    __syncthreads(); // the column and the wave sums are visible
+    if constexpr (need_stat)
+    {
+        total = red[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+            total += red[x];
+    }
+    float lo, hi;
+    if constexpr (NBITS == 1)
+    {
+        const float mean = ZT ? 0.0f : total / (float) c.rows;
+        float s0 = 0.0f, s1 = 0.0f;
+        uint32_t n0 = 0;
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
+        if (WG == T || tid < T)
+            for (uint32_t v = tid; v < c.pieces + shift; v += T)
+                if (v >= shift)
+                    split_add_piece(t4[v - shift], mean, s0, s1, n0);
+        s0 = wave_sum(s0);
+        s1 = wave_sum(s1);
+        n0 = wave_sum(n0);
+        __syncthreads(); // everyone has read the wave sums of the mean
+        if (lane == 0 && wave < NW)
+        {
+            red[wave] = s0;
+            red[4 + wave] = s1;
+            red_u[wave] = n0;
+        }
+        __syncthreads();
+        float S0 = red[0], S1 = red[4];
+        uint32_t N0 = red_u[0];
+#pragma unroll
+        for (uint32_t x = 1; x < NW; ++x)
+        {
+            S0 += red[x];
+            S1 += red[4 + x];
+            N0 += red_u[x];
+        }
+        finish_stats_1bit<ZT>(mean, S0, S1, N0, c.rows - N0, c.rows, lo, hi);
+    }
+    else
+    {
+        finish_stats_multibit(total, c.rows, lo, hi);
+    }
+    if (tid == 0)
+    {
+        // a record is only 4-byte aligned when the column has an odd number of QWords
+        float* gh = reinterpret_cast<float*>(qc);
+        gh[0] = lo;
+        gh[1] = hi;
+    }
+    const ValueQ vq = make_vq<NBITS>(lo, hi);
+    const float val0 = unquantize_value<NBITS>(vq, 0u);
+    const float val1 = unquantize_value<NBITS>(vq, 1u);
+    uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
+    const uint32_t items = c.nq * PS::CHUNKS;
+    for (uint32_t it = tid; it < items; it += WG)
+    {
+        // chunk-major: consecutive threads take consecutive QWords, hence consecutive rows
+        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / c.nq;
+        const uint32_t w = it - chunk * c.nq;
+        uint32_t word = 0;
+#pragma unroll
+        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+        {
+            const uint32_t k = chunk * PS::SLOTS + kk;
+            const uint32_t i = w + k * c.nq;
+            if (i < c.rows)
+            {
+                const float v = tile[i];
+                const uint32_t code = quantize_value<NBITS, ZT>(vq, v);
+                float back;
+                if constexpr (NBITS == 1)
+                    back = code ? val1 : val0;
+                else
+                    back = unquantize_value<NBITS>(vq, code);
+                __builtin_nontemporal_store(v - back, res_col + i);
+                word |= code << (k * PS::SHIFT);
+            }
+        }
+        if constexpr (PS::CHUNKS == 1)
+            bits[w] = word;
+        else
+            atomicOr(&words[w], word);
+    }
+    if constexpr (PS::CHUNKS > 1)
+    {
+        __syncthreads();
+        for (uint32_t w = tid; w < c.nq; w += WG)
+            bits[w] = words[w];
+    }
+}
+
+template <int NBITS, bool ZT>
+__device__ __forceinline__ void quantize_colg_body(const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q,
+                                                   const ColGeom& c, uint32_t column, f32x4* smem)
+{
+    using PS = PackShape<NBITS>;
+    constexpr uint32_t T = kColThreads;
+    float* tile = reinterpret_cast<float*>(smem);
+    uint32_t* words = reinterpret_cast<uint32_t*>(tile + c.rows);
+    float* red = tile + c.rows + (PS::CHUNKS > 1 ? c.nq : 0);
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) column * c.rows;
+    if constexpr (PS::CHUNKS > 1)
+        for (uint32_t x = tid; x < c.nq; x += T)
+            words[x] = 0u;
+    const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base);
+    const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base);
+    f32x4* t4 = reinterpret_cast<f32x4*>(tile);
+    float stat = 0.0f;
+    // slot v holds piece v - shift (see column_shift): the order the register kernels sum in, and whole lines per wavefront
+    const uint32_t shift = column_shift(r_in + base, c.line_shift);
+    const uint32_t slots = c.pieces + shift;
+    for (uint32_t v0 = tid; v0 < slots; v0 += 4 * T)
+    {
+        f32x4 a[4], b[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+        {
+            const uint32_t v = v0 + u * T;
+            if (v >= shift && v < slots)
+            {
+                a[u] = __builtin_nontemporal_load(g4 + (v - shift));
+                b[u] = __builtin_nontemporal_load(r4 + (v - shift));
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+        {
+            const uint32_t v = v0 + u * T;
+            if (v >= shift && v < slots)
+            {
+                const f32x4 x = a[u] + b[u];
+                t4[v - shift] = x;
+                stat = colg_add_piece<NBITS>(stat, x);
+            }
+        }
+    }
+    // the whole column has been read before the first barrier of colg_stats_pack, so r_out may be r_in
+    colg_stats_pack<NBITS, ZT>(tile, words, red, c, stat, shift, r_out + base, q + (size_t) column * c.qcol);
+}
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kColThreads) void quantize_colg_kernel(const float* __restrict__ g, const float* r_in, float* r_out,
+                                                                    char* __restrict__ q, ColGeom c)
+{
+    extern __shared__ f32x4 smem_v4[];
+    quantize_colg_body<NBITS, ZT>(g, r_in, r_out, q, c, blockIdx.x, smem_v4);
+}
+
+// WG: threads in the workgroup (256, or 1024 for tall columns, whose many work items would otherwise be a long chain of
+// dependent loads for each of few threads)
+template <int NBITS, bool ZT, int WG = kColThreads>
+__device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
+                                                        const ColGeom& c, uint32_t column, f32x4* smem)
+{
+    using PS = PackShape<NBITS>;
+    constexpr uint32_t T = kColThreads, BATCH = 8;
+    static_assert(WG >= (int) T, "workgroup size");
+    float* tile = reinterpret_cast<float*>(smem);
+    uint32_t* words = reinterpret_cast<uint32_t*>(tile + c.rows);
+    float* red = tile + c.rows + (PS::CHUNKS > 1 ? c.nq : 0);
+    float* dec = red + 12; // per worker, in summation order: 1 bit -> the two levels, else (ufactor, lower)
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) column * c.rows;
+    const size_t rec = (size_t) column * c.qcol;
+    const uint32_t K = src.workers;
+    if constexpr (PS::CHUNKS > 1)
+        for (uint32_t x = tid; x < c.nq; x += WG)
+            words[x] = 0u;
+    // what this thread's first work item needs from memory is requested before the first barrier: one round trip for
+    // headers, QWords and stripe residual instead of three (see stripe_reduce_col_kernel)
+    const float* sp = stripe_res + base;
+    const uint32_t items = c.nq * PS::CHUNKS;
+    uint32_t word[BATCH];
+    float resid[PS::SLOTS];
+    if (tid < items)
+    {
+        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : tid / c.nq;
+        const uint32_t w = tid - chunk * c.nq;
+#pragma unroll
+        for (uint32_t u = 0; u < BATCH; ++u)
+            if (u < K)
+                word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(u, src.owner)] + rec + 8 + (size_t) w * 4);
+#pragma unroll
+        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+        {
+            const uint32_t i = w + (chunk * PS::SLOTS + kk) * c.nq;
+            if (i < c.rows)
+                resid[kk] = __builtin_nontemporal_load(sp + i);
+        }
+    }
+    if (tid < K)
+    {
+        const float* h = reinterpret_cast<const float*>(src.q[stripe_order(tid, src.owner)] + rec);
+        const ValueQ vq = make_vq<NBITS>(h[0], h[1]);
+        if constexpr (NBITS == 1)
+        {
+            dec[2 * tid] = unquantize_value<NBITS>(vq, 0u);
+            dec[2 * tid + 1] = unquantize_value<NBITS>(vq, 1u);
+        }
+        else
+        {
+            dec[2 * tid] = vq.uf;
+            dec[2 * tid + 1] = vq.lo;
+        }
+    }
+    __syncthreads();
+
+    for (uint32_t it = tid; it < items; it += WG)
+    {
+        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / c.nq;
+        const uint32_t w = it - chunk * c.nq;
+        const size_t word_off = rec + 8 + (size_t) w * 4;
+        const uint32_t sh0 = chunk * PS::SLOTS * PS::SHIFT;
+        if (it != tid)
+        {
+#pragma unroll
+            for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+            {
+                const uint32_t i = w + (chunk * PS::SLOTS + kk) * c.nq;
+                if (i < c.rows)
+                    resid[kk] = __builtin_nontemporal_load(sp + i);
+            }
+        }
+        float acc[PS::SLOTS];
+        for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
+        {
+            if (it != tid || n0 != 0)
+            {
+#pragma unroll
+                for (uint32_t u = 0; u < BATCH; ++u)
+                    if (n0 + u < K)
+                        word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + word_off);
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < BATCH; ++u)
+            {
+                if (n0 + u < K)
+                {
+                    const float a = dec[2 * (n0 + u)];
+                    const float b = dec[2 * (n0 + u) + 1];
+                    const uint32_t bits = word[u] >> sh0;
+#pragma unroll
+                    for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+                    {
+                        const uint32_t code = (bits >> (kk * PS::SHIFT)) & PS::CODEMASK;
+                        float x;
+                        if constexpr (NBITS == 1)
+                            x = code ? b : a;
+                        else
+                            x = unquantize_value<NBITS>(a, b, code);
+                        // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
+                        acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+        {
+            const uint32_t i = w + (chunk * PS::SLOTS + kk) * c.nq;
+            if (i < c.rows)
+            {
+                if (agg_out != nullptr)
+                    agg_out[base + i] = acc[kk];
+                tile[i] = acc[kk] + resid[kk];
+            }
+        }
+    }
+    float stat = 0.0f;
+    // the quantize kernels' summation order for a residual at this address
+    const uint32_t shift = column_shift(stripe_res + base, c.line_shift);
+    if constexpr ((NBITS != 1) || !ZT)
+    {
+        __syncthreads();
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
+        if (WG == T || tid < T)
+            for (uint32_t v = tid; v < c.pieces + shift; v += T)
+                if (v >= shift)
+                    stat = colg_add_piece<NBITS>(stat, t4[v - shift]);
+    }
+    colg_stats_pack<NBITS, ZT, WG>(tile, words, red, c, stat, shift, stripe_res + base, q_out + rec);
+}
+
+template <int NBITS, bool ZT, int WG>
+__global__ __launch_bounds__(WG) void stripe_reduce_colg_kernel(StripeSources src, float* stripe_res, char* q_out, float* agg_out,
+                                                                ColGeom c)
+{
+    extern __shared__ f32x4 smem_v4[];
+    stripe_reduce_colg_body<NBITS, ZT, WG>(src, stripe_res, q_out, agg_out, c, blockIdx.x, smem_v4);
+}
+
+} // namespace cntkq

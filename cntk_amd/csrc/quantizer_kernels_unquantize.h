@@ -1,0 +1,505 @@
+// gfx950 kernels of the per-column gradient quantizer: the decoders (packed codes -> values).
+#pragma once
+
+#include "quantizer_kernels_common.h"
+
+namespace cntkq {
+
+// ---- unquantize ---------------------------------------------------------------------------------------
+//
+// One thread decodes WV consecutive QWords of a column (WV = 4: 16-byte stores; WV = 1: any shape) for a
+// chunk of `slots` consecutive bit positions. For fixed bit position k the rows w + k * nq of
+// consecutive QWords are consecutive in memory, so stores coalesce.
+
+struct UnqGeom
+{
+    uint32_t rows;
+    uint32_t cols;
+    uint32_t nq;
+    uint32_t groups;  // ceil(nq / WV) word groups per column
+    uint32_t chunks;  // ceil(VPW / slots)
+    uint32_t slots;   // bit positions per thread
+    uint32_t per_col; // groups * chunks work items per column
+    uint32_t items;   // per_col * cols (the host refuses matrices that need more than 2^32 - 1)
+    uint32_t swz_members; // > 1: workgroups are regrouped by XCD, this many share the same QWords (see unq_xcd_block)
+    uint32_t swz_gw;      // workgroups side by side along the QWords of one column (1 when one workgroup spans them all)
+    uint64_t qcol;
+};
+
+// The workgroups of a column that decode different bit positions of the same QWords read the same packed bytes.
+// Consecutive workgroups go to the 8 XCDs in turn, each with its own L2; this permutation of the workgroup index puts
+// the `members` workgroups of such a set 8 apart, i.e. on one XCD, so that the QWords are fetched once (measured
+// without it: 4 to 4.5 times the packed bytes at 8192 and 65536 rows). Sets are taken in groups of 8; the remainder at
+// the end keeps its order. Returns the logical workgroup index (column-major, then chunk of bit positions, then QWords).
+__device__ __forceinline__ uint32_t unq_xcd_block(uint32_t b, uint32_t blocks, uint32_t members, uint32_t gw)
+{
+    const uint32_t per_group = 8 * members;
+    const uint32_t grouped = (blocks / per_group) * per_group;
+    uint32_t set, m;
+    if (b < grouped)
+    {
+        const uint32_t grp = b / per_group;
+        const uint32_t rem = b - grp * per_group;
+        m = rem >> 3;
+        set = grp * 8 + (rem & 7u);
+    }
+    else
+    {
+        const uint32_t r = b - grouped;
+        const uint32_t ss = r / members;
+        m = r - ss * members;
+        set = grouped / members + ss;
+    }
+    const uint32_t c = set / gw;
+    const uint32_t g = set - c * gw;
+    return (c * members + m) * gw + g;
+}
+
+template <int NBITS, int WV>
+__device__ __forceinline__ void unquantize_body(const char* __restrict__ q, float* out, const UnqGeom& t, int add, uint32_t block)
+{
+    constexpr uint32_t VPW = 32 / NBITS;
+    constexpr uint32_t MASKBITS = NBITS & 31;
+    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << MASKBITS) - 1u);
+
+    if (t.swz_members > 1)
+        block = unq_xcd_block(block, t.items / 256, t.swz_members, t.swz_gw);
+    const uint64_t id64 = (uint64_t) block * 256 + threadIdx.x;
+    if (id64 >= t.items)
+        return;
+    const uint32_t id = (uint32_t) id64;
+    const uint32_t c = id / t.per_col;
+    const uint32_t rem = id - c * t.per_col;
+    const uint32_t chunk = rem / t.groups;
+    const uint32_t grp = rem - chunk * t.groups;
+    const uint32_t w0 = grp * WV;
+
+    const char* qc = q + (size_t) c * t.qcol;
+    const float* gh = reinterpret_cast<const float*>(qc);
+    ValueQ vq; // decoding needs only the code -> value factor and the lower bound
+    vq.lo = gh[0];
+    vq.uf = make_ufactor<NBITS>(gh[0], gh[1]);
+    const float val0 = unquantize_value<NBITS>(vq, 0u);
+    const float val1 = unquantize_value<NBITS>(vq, 1u);
+    const uint32_t* bits = reinterpret_cast<const uint32_t*>(qc + 8);
+    float* oc = out + (size_t) c * t.rows;
+
+    uint32_t word[WV];
+    if constexpr (WV == 4)
+    {
+        // the word group starts 8 bytes past a 16-byte boundary or on one: two 8-byte loads are always aligned
+        const u32x2 a = *reinterpret_cast<const u32x2*>(bits + w0);
+        const u32x2 b = *reinterpret_cast<const u32x2*>(bits + w0 + 2);
+        word[0] = a.x;
+        word[1] = a.y;
+        word[2] = b.x;
+        word[3] = b.y;
+    }
+    else
+    {
+        word[0] = bits[w0];
+    }
+
+    const uint32_t k0 = chunk * t.slots;
+    const uint32_t k1 = min(k0 + t.slots, VPW);
+    for (uint32_t k = k0; k < k1; ++k)
+    {
+        const uint32_t i = w0 + k * t.nq;
+        if (i >= t.rows)
+            break; // rows only grow with k
+        const uint32_t sh = k * MASKBITS;
+        if constexpr (WV == 4)
+        {
+            // rows % 4 == 0 and i % 4 == 0: the four rows are all inside the column
+            f32x4 x;
+            if constexpr (NBITS == 1)
+            {
+                x.x = ((word[0] >> sh) & 1u) ? val1 : val0;
+                x.y = ((word[1] >> sh) & 1u) ? val1 : val0;
+                x.z = ((word[2] >> sh) & 1u) ? val1 : val0;
+                x.w = ((word[3] >> sh) & 1u) ? val1 : val0;
+            }
+            else
+            {
+                x.x = unquantize_value<NBITS>(vq, (word[0] >> sh) & CODEMASK);
+                x.y = unquantize_value<NBITS>(vq, (word[1] >> sh) & CODEMASK);
+                x.z = unquantize_value<NBITS>(vq, (word[2] >> sh) & CODEMASK);
+                x.w = unquantize_value<NBITS>(vq, (word[3] >> sh) & CODEMASK);
+            }
+            f32x4* dst = reinterpret_cast<f32x4*>(oc + i);
+            if (add)
+                x = x + *dst; // unquantized value + previous content
+            __builtin_nontemporal_store(x, dst);
+        }
+        else
+        {
+            float x;
+            if constexpr (NBITS == 1)
+                x = ((word[0] >> sh) & 1u) ? val1 : val0;
+            else
+                x = unquantize_value<NBITS>(vq, (word[0] >> sh) & CODEMASK);
+            if (add)
+                x = x + oc[i];
+            oc[i] = x;
+        }
+    }
+}
+
+template <int NBITS, int WV>
+__global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, float* out, UnqGeom t, int add)
+{
+    unquantize_body<NBITS, WV>(q, out, t, add, blockIdx.x);
+}
+
+// Decoder with 16-byte stores for shapes the QWord-major decoder above can only serve with 4-byte stores
+// (nq or rows not a multiple of 4, e.g. 100000 rows -> 3125 QWords). For one column and one bit position k the
+// rows k * nq ... (k + 1) * nq - 1 are consecutive in memory: such a segment is cut into groups of four elements
+// aligned to 16 bytes in the OUTPUT (the first and last group of a segment may be partial and use 4-byte stores).
+struct UnqSegGeom
+{
+    uint32_t rows;
+    uint32_t nq;
+    uint32_t segs;    // bit positions in use per column: ceil(rows / nq)
+    uint32_t gps;     // groups per segment
+    uint32_t items;   // cols * segs * gps (the host refuses more than 2^32 - 1)
+    double inv_gps;
+    double inv_segs;
+    uint64_t qcol;
+};
+
+template <int NBITS>
+__device__ __forceinline__ void unquantize_segment_body(const char* __restrict__ q, float* out, const UnqSegGeom& t, int add,
+                                                        uint32_t block)
+{
+    constexpr uint32_t SHIFT = NBITS & 31;
+    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
+    const uint64_t id64 = (uint64_t) block * 256 + threadIdx.x;
+    if (id64 >= t.items)
+        return;
+    uint32_t seg, g, c, k;
+    divmod_u32((uint32_t) id64, t.gps, t.inv_gps, seg, g);
+    divmod_u32(seg, t.segs, t.inv_segs, c, k);
+    const uint32_t row0 = k * t.nq;
+    const uint32_t seg_len = min(t.nq, t.rows - row0);
+    const size_t obase = (size_t) c * t.rows + row0;       // out is 16-byte aligned (checked by the host)
+    const int32_t first = (int32_t) (4u * g) - (int32_t) (obase & 3u); // QWord index of this group's first element
+    if (first >= (int32_t) seg_len)
+        return;
+
+    const char* qc = q + (size_t) c * t.qcol;
+    const float* gh = reinterpret_cast<const float*>(qc);
+    const float lo = gh[0];
+    const float uf = make_ufactor<NBITS>(lo, gh[1]);
+    const uint32_t* bits = reinterpret_cast<const uint32_t*>(qc + 8);
+    const uint32_t sh = k * SHIFT;
+    float* dst = out + obase;
+
+    if (first >= 0 && first + 3 < (int32_t) seg_len)
+    {
+        f32x4 v;
+        v.x = unquantize_value<NBITS>(uf, lo, (bits[first] >> sh) & CODEMASK);
+        v.y = unquantize_value<NBITS>(uf, lo, (bits[first + 1] >> sh) & CODEMASK);
+        v.z = unquantize_value<NBITS>(uf, lo, (bits[first + 2] >> sh) & CODEMASK);
+        v.w = unquantize_value<NBITS>(uf, lo, (bits[first + 3] >> sh) & CODEMASK);
+        f32x4* d4 = reinterpret_cast<f32x4*>(dst + first);
+        if (add)
+            v = v + *d4;
+        __builtin_nontemporal_store(v, d4);
+    }
+    else
+    {
+        for (int32_t e = 0; e < 4; ++e)
+        {
+            const int32_t w = first + e;
+            if (w >= 0 && w < (int32_t) seg_len)
+            {
+                const float x = unquantize_value<NBITS>(uf, lo, (bits[w] >> sh) & CODEMASK);
+                dst[w] = add ? x + dst[w] : x;
+            }
+        }
+    }
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_segment_kernel(const char* __restrict__ q, float* out, UnqSegGeom t, int add)
+{
+    unquantize_segment_body<NBITS>(q, out, t, add, blockIdx.x);
+}
+
+// Row-major decoder for columns of 1024 rows and more whose QWord-major stores would not be whole lines (9304 rows -> 291
+// QWords, 100000 -> 3125, 50257 -> 1571): a workgroup copies the packed column into LDS once (every QWord is used by
+// up to 32 rows) and then walks a chunk of consecutive rows, four per thread and store, so that all stores are aligned
+// 16-byte stores whatever the QWord count, the height and the alignment of the output.
+struct UnqRowGeom
+{
+    uint32_t rows;
+    uint32_t nq;
+    uint32_t chunk;  // rows per workgroup, multiple of 4 (the last workgroup of a column also takes the remainder)
+    uint32_t chunks; // workgroups per column
+    uint32_t blocks; // cols * chunks
+    uint32_t pad;
+    uint64_t qcol;
+};
+
+// Which (column, chunk) a workgroup of the row-major decoder takes. Consecutive workgroups go to the 8 XCDs in turn and
+// every XCD has its own L2, so the chunks of one column are given to workgroups 8 apart: they then read the column's
+// packed record through one L2 instead of fetching it once per XCD. Columns are taken in groups of 8; what is left over
+// at the end is dealt column by column.
+__device__ __forceinline__ void unq_rows_block_to_chunk(uint32_t block, uint32_t chunks, uint32_t blocks, uint32_t& c, uint32_t& ch)
+{
+    const uint32_t per_group = 8 * chunks;
+    const uint32_t grouped = (blocks / per_group) * per_group;
+    if (block < grouped)
+    {
+        const uint32_t grp = block / per_group;
+        const uint32_t rem = block - grp * per_group;
+        ch = rem >> 3;
+        c = grp * 8 + (rem & 7u);
+    }
+    else
+    {
+        const uint32_t b = block - grouped;
+        const uint32_t cc = b / chunks;
+        ch = b - cc * chunks;
+        c = grouped / chunks + cc;
+    }
+}
+
+template <int NBITS>
+__device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q, float* out, const UnqRowGeom& t, int add, uint32_t block,
+                                                     uint32_t* words)
+{
+    constexpr uint32_t SHIFT = NBITS & 31;
+    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
+    const uint32_t tid = threadIdx.x;
+    uint32_t c, ch;
+    unq_rows_block_to_chunk(block, t.chunks, t.blocks, c, ch);
+    const char* qc = q + (size_t) c * t.qcol;
+    const float* gh = reinterpret_cast<const float*>(qc);
+    const float lo = gh[0];
+    const float uf = make_ufactor<NBITS>(lo, gh[1]);
+    const uint32_t* bits = reinterpret_cast<const uint32_t*>(qc + 8);
+    if (t.nq <= 1024)
+    {
+        for (uint32_t w = tid; w < t.nq; w += 256)
+            words[w] = bits[w];
+    }
+    else
+    {
+        // eight loads in flight per thread: a tall column has thousands of QWords, and one round trip for every 256 of
+        // them would cost more than the decoding
+        for (uint32_t w = tid; w < t.nq; w += 8 * 256)
+        {
+            uint32_t v[8];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u)
+                v[u] = bits[(w + 256 * u < t.nq) ? w + 256 * u : w];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u)
+                if (w + 256 * u < t.nq)
+                    words[w + 256 * u] = v[u];
+        }
+    }
+    __syncthreads();
+    // The column need not start on a 16-byte boundary nor hold a multiple of 4 rows: `head` rows (0..3) lie before its
+    // first aligned group of four and `tail` rows (0..3) after the last; chunks are counted from the first aligned row,
+    // the first chunk's workgroup also writes the head rows, the last one's the tail rows, one row per thread.
+    float* oc = out + (size_t) c * t.rows;
+    const uint32_t head = (4u - (uint32_t) ((reinterpret_cast<uintptr_t>(oc) >> 2) & 3u)) & 3u;
+    const uint32_t body = (t.rows - head) & ~3u; // rows in aligned groups of four
+    const uint32_t tail = t.rows - head - body;
+    const uint32_t r0 = ch * t.chunk;
+    const uint32_t pieces = ((ch + 1 == t.chunks ? body : r0 + t.chunk) - r0) >> 2; // the last chunk runs to the end
+    f32x4* o4 = reinterpret_cast<f32x4*>(oc + head + r0);
+    const float val0 = unquantize_value<NBITS>(uf, lo, 0u);
+    const float val1 = unquantize_value<NBITS>(uf, lo, 1u);
+    {
+        uint32_t row = t.rows; // none
+        if (ch == 0 && tid < head)
+            row = tid;
+        else if (ch + 1 == t.chunks && tid >= 4 && tid < 4 + tail)
+            row = head + body + (tid - 4);
+        if (row < t.rows)
+        {
+            const uint32_t k = row / t.nq;
+            const uint32_t code = (words[row - k * t.nq] >> (k * SHIFT)) & CODEMASK;
+            float x;
+            if constexpr (NBITS == 1)
+                x = code ? val1 : val0;
+            else
+                x = unquantize_value<NBITS>(uf, lo, code);
+            oc[row] = add ? x + oc[row] : x;
+        }
+    }
+    // Slot v = tid, tid + 256, ... holds piece v - shift, shift = the chunk's offset into its 128-byte line in pieces, so
+    // that every wavefront's 64 stores cover whole lines also where columns do not start on one (9304 rows).
+    const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o4) >> 4) & 7u);
+    const uint32_t vfirst = tid < shift ? tid + 256 : tid;
+    // row i sits in QWord i % nq at bit position i / nq; a thread's pieces are 1024 rows apart
+    const uint32_t i0 = head + r0 + 4 * (vfirst - shift);
+    uint32_t k0 = i0 / t.nq;
+    uint32_t w0 = i0 - k0 * t.nq;
+    const uint32_t dk = 1024u / t.nq;
+    const uint32_t dw = 1024u - dk * t.nq;
+    for (uint32_t p = vfirst - shift; p < pieces; p += 256)
+    {
+        uint32_t k = k0, w = w0;
+        f32x4 x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            const uint32_t code = (words[w] >> (k * SHIFT)) & CODEMASK;
+            if constexpr (NBITS == 1)
+                x[e] = code ? val1 : val0;
+            else
+                x[e] = unquantize_value<NBITS>(uf, lo, code);
+            if (++w == t.nq)
+            {
+                w = 0;
+                ++k;
+            }
+        }
+        if (add)
+            x = x + o4[p]; // unquantized value + previous content
+        __builtin_nontemporal_store(x, o4 + p);
+        k0 += dk;
+        w0 += dw;
+        if (w0 >= t.nq)
+        {
+            w0 -= t.nq;
+            ++k0;
+        }
+    }
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __restrict__ q, float* out, UnqRowGeom t, int add)
+{
+    extern __shared__ f32x4 smem_v4[];
+    unquantize_rows_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint32_t*>(smem_v4));
+}
+
+// Tile decoder for short columns. Consecutive columns are adjacent in the packed matrix and in the output, so a
+// workgroup takes `cpt` columns at once: their packed records (one contiguous run) go to LDS in coalesced loads, each
+// column's decoding constants are computed once, and the cpt * rows values (one contiguous run) leave in aligned
+// 16-byte stores, four consecutive elements per thread and store, whatever the column height: a group of four may
+// straddle columns. cpt is a multiple of 4, so every tile starts on a 16-byte boundary of an aligned output.
+struct UnqTileGeom
+{
+    uint32_t rows;
+    uint32_t cols;
+    uint32_t nq;
+    uint32_t cpt;        // columns per workgroup
+    uint32_t rec_words;  // nq + 2: 32-bit words per packed record
+    uint32_t rows_magic; // ceil(2^32 / rows) (unused when rows == 1)
+    uint32_t nq_magic;   // ceil(2^32 / nq) (unused when nq == 1)
+    uint32_t blocks;
+};
+
+__host__ __device__ inline size_t unq_tile_lds_bytes(const UnqTileGeom& t)
+{
+    return (size_t) t.cpt * (t.rec_words + 2) * 4;
+}
+
+// x / d for x * d < 2^32 with magic = ceil(2^32 / d)
+__device__ __forceinline__ uint32_t small_div(uint32_t x, uint32_t d, uint32_t magic)
+{
+    return d == 1 ? x : __umulhi(x, magic);
+}
+
+template <int NBITS>
+__device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q, float* out, const UnqTileGeom& t, int add, uint32_t block,
+                                                     uint32_t* smem)
+{
+    constexpr uint32_t SHIFT = NBITS & 31;
+    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t col0 = block * t.cpt;
+    const uint32_t ncols = (t.cols - col0 < t.cpt) ? t.cols - col0 : t.cpt;
+    uint32_t* words = smem;                                          // ncols packed records
+    float* dec = reinterpret_cast<float*>(smem + t.cpt * t.rec_words); // per column: the two levels (1 bit) or (ufactor, lower)
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(q + (size_t) col0 * t.rec_words * 4);
+    const uint32_t total_words = ncols * t.rec_words;
+    for (uint32_t x = tid; x < total_words; x += 256)
+        words[x] = __builtin_nontemporal_load(src + x);
+    __syncthreads();
+    for (uint32_t c = tid; c < ncols; c += 256)
+    {
+        const float lo = __uint_as_float(words[c * t.rec_words]);
+        const float hi = __uint_as_float(words[c * t.rec_words + 1]);
+        const float uf = make_ufactor<NBITS>(lo, hi);
+        if constexpr (NBITS == 1)
+        {
+            dec[2 * c] = unquantize_value<NBITS>(uf, lo, 0u);
+            dec[2 * c + 1] = unquantize_value<NBITS>(uf, lo, 1u);
+        }
+        else
+        {
+            dec[2 * c] = uf;
+            dec[2 * c + 1] = lo;
+        }
+    }
+    __syncthreads();
+    const uint32_t elems = ncols * t.rows;
+    float* o = out + (size_t) col0 * t.rows;
+    // slots dealt by 128-byte lines: slot v = tid, tid + 256, ... holds the group of four that starts at element
+    // 4 * (v - shift), shift = the tile's offset into its line in 16-byte pieces
+    const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o) >> 4) & 7u);
+    for (uint32_t i = 4 * ((tid < shift ? tid + 256 : tid) - shift); i < elems; i += 1024)
+    {
+        uint32_t c = small_div(i, t.rows, t.rows_magic);
+        uint32_t r = i - c * t.rows;
+        uint32_t k = small_div(r, t.nq, t.nq_magic);
+        uint32_t w = r - k * t.nq;
+        const uint32_t* cw = words + c * t.rec_words + 2;
+        float d0 = dec[2 * c], d1 = dec[2 * c + 1];
+        f32x4 x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            // (past the end of the matrix c == ncols: the reads stay inside the LDS block and the value is not stored)
+            const uint32_t code = (cw[w] >> (k * SHIFT)) & CODEMASK;
+            if constexpr (NBITS == 1)
+                x[e] = code ? d1 : d0;
+            else
+                x[e] = unquantize_value<NBITS>(d0, d1, code);
+            ++r;
+            if (++w == t.nq)
+            {
+                w = 0;
+                ++k;
+            }
+            if (r == t.rows)
+            {
+                r = 0;
+                k = 0;
+                w = 0;
+                c = (c + 1 < t.cpt) ? c + 1 : c;
+                cw = words + c * t.rec_words + 2;
+                d0 = dec[2 * c];
+                d1 = dec[2 * c + 1];
+            }
+        }
+        if (i + 4 <= elems)
+        {
+            f32x4* o4 = reinterpret_cast<f32x4*>(o + i);
+            if (add)
+                x = x + *o4; // unquantized value + previous content
+            __builtin_nontemporal_store(x, o4);
+        }
+        else
+        {
+            for (uint32_t e = 0; i + e < elems; ++e)
+                o[i + e] = add ? x[e] + o[i + e] : x[e];
+        }
+    }
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_tile_kernel(const char* __restrict__ q, float* out, UnqTileGeom t, int add)
+{
+    extern __shared__ f32x4 smem_v4[];
+    unquantize_tile_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint32_t*>(smem_v4));
+}
+
+} // namespace cntkq
