@@ -337,10 +337,11 @@ inline void launch_stripe_col(hipStream_t s, LaunchEvents ev, const StripeSource
                           ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, qcol);
 }
 
-// The register kernels: from 2048 rows on (unless forced), up to 25 pieces for each of
+// The register kernels: above 1024 rows (unless forced; 37.7 M elements at 1152 / 1536 / 2000 rows: 95 / 76 / 72 us against
+// 102 / 81 / 80 us with the LDS column kernels, the same bytes), up to 25 pieces for each of
 // 1024 threads, the column's QWords within 64 KB of LDS. 256 threads up to the height the stripe reduction handles (whose
 // LDS kernels then sum in the same order), 1024 above.
-constexpr uint32_t kRegMinRows = 2047;
+constexpr uint32_t kRegMinRows = 1024;
 constexpr uint32_t kRegMaxRows = 4 * 1024 * 25;
 
 inline uint32_t reg_threads(size_t rows)
