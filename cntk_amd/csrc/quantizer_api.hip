@@ -143,6 +143,11 @@ struct BatchTable
     size_t capacity = 0;
     hipEvent_t event = nullptr; // set when the last kernel that reads the table has finished
     bool in_flight = false;
+    // A launch that reads the table was recorded into a graph (stream capture): the graph may be replayed at any time
+    // from then on, so the buffers are never written again; a rebuild retires them (freed with the handle) and takes
+    // fresh ones.
+    bool captured = false;
+    std::vector<std::pair<char*, char*>> retired;
     // launch parameters of the two LDS classes and the matrices that get a launch of their own
     size_t members[2] = {0, 0};
     uint32_t blocks[2] = {0, 0};
@@ -230,6 +235,18 @@ int ensure_staging(cntkq_quantizer* h, size_t bytes)
     return CNTKQ_OK;
 }
 
+// Whether work issued on `s` is being recorded into a graph instead of executed.
+bool stream_capturing(hipStream_t s)
+{
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) != hipSuccess)
+    {
+        (void) hipGetLastError();
+        return false;
+    }
+    return st == hipStreamCaptureStatusActive;
+}
+
 // True when `t` was built for exactly this item list and parameters.
 bool table_matches(const BatchTable& t, const void* items, size_t items_bytes, const size_t (&params)[3])
 {
@@ -244,6 +261,13 @@ int table_begin_rebuild(BatchTable& t, size_t bytes)
     t.key.clear();
     if (t.event == nullptr)
         HIP_TRY(hipEventCreateWithFlags(&t.event, hipEventDisableTiming), "hipEventCreateWithFlags failed");
+    if (t.captured)
+    {
+        t.retired.emplace_back(t.host, t.dev);
+        t.host = t.dev = nullptr;
+        t.capacity = 0;
+        t.captured = false;
+    }
     if (t.in_flight)
     {
         HIP_TRY(hipEventSynchronize(t.event), "hipEventSynchronize failed");
@@ -287,6 +311,11 @@ void table_destroy(BatchTable& t)
         (void) hipHostFree(t.host);
     if (t.dev != nullptr)
         (void) hipFree(t.dev);
+    for (auto& r : t.retired)
+    {
+        (void) hipHostFree(r.first);
+        (void) hipFree(r.second);
+    }
 }
 
 int sync_event(hipEvent_t ev) // SyncEvent (Source/Math/MatrixQuantizerGPU.cu:68-80)
@@ -329,6 +358,10 @@ int quantize_async_impl(cntkq_quantizer* h, const E* in, const E* res_in, size_t
     DeviceGuard guard(h->device);
     hipStream_t s = work_stream(h);
     char* qdev = static_cast<char*>(qbuf);
+    const bool capturing = stream_capturing(s);
+    if (capturing && qbuf_on_host)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: a host-resident packed matrix needs copies on other streams and cannot "
+                                            "be recorded into a graph");
     if (qbuf_on_host)
     {
         int rc = ensure_staging(h, need);
@@ -340,7 +373,9 @@ int quantize_async_impl(cntkq_quantizer* h, const E* in, const E* res_in, size_t
         qdev = h->staging;
     }
 
-    const LaunchEvents ev = take_events(h, h->ev_quantize);
+    LaunchEvents ev = take_events(h, h->ev_quantize);
+    if (capturing)
+        ev.stop = nullptr; // recorded, not executed: nothing to wait for
     hipError_t lrc = Elem<E>::quantize(s, ev, in, res_in, res_out, qdev, rows, cols, nbits, zero_threshold_for_1bit != 0, h->tune);
     if (lrc == hipErrorInvalidValue)
         return fail(CNTKQ_INVALID_ARGUMENT, "quantize: the forced kernel path does not support %zu x %zu at %zu bits", rows, cols, nbits);
@@ -383,6 +418,9 @@ int unquantize_async_impl(cntkq_quantizer* h, const void* qbuf, size_t qbuf_byte
     DeviceGuard guard(h->device);
     hipStream_t s = work_stream(h);
     const char* qdev = static_cast<const char*>(qbuf);
+    if (qbuf_on_host && stream_capturing(s))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: a host-resident packed matrix needs copies on other streams and "
+                                            "cannot be recorded into a graph");
     if (qbuf_on_host)
     {
         int rc = ensure_staging(h, need);
@@ -398,7 +436,9 @@ int unquantize_async_impl(cntkq_quantizer* h, const void* qbuf, size_t qbuf_byte
         HIP_TRY(hipStreamWaitEvent(s, h->ev_assign, 0), "hipStreamWaitEvent failed");
         qdev = h->staging;
     }
-    const LaunchEvents ev = take_events(h, h->ev_unquantize);
+    LaunchEvents ev = take_events(h, h->ev_unquantize);
+    if (stream_capturing(s))
+        ev.stop = nullptr; // recorded, not executed: nothing to wait for
     hipError_t lrc = Elem<E>::unquantize(s, ev, qdev, out, rows, cols, nbits, add != 0, h->tune);
     if (lrc == hipErrorInvalidValue)
         return fail(CNTKQ_INVALID_ARGUMENT, "unquantize: %zu x %zu at %zu bits is too large for one launch", rows, cols, nbits);
@@ -440,7 +480,9 @@ int stripe_reduce_async_impl(cntkq_quantizer* h, const void* const* stripes, siz
 
     DeviceGuard guard(h->device);
     hipStream_t s = work_stream(h);
-    const LaunchEvents ev = take_events(h, h->ev_stripe);
+    LaunchEvents ev = take_events(h, h->ev_stripe);
+    if (stream_capturing(s))
+        ev.stop = nullptr; // recorded, not executed: nothing to wait for
     hipError_t lrc = Elem<E>::stripe_reduce(s, ev, src, stripe_res, q_out, agg_out, rows, stripe_cols, nbits,
                                             zero_threshold_for_1bit != 0, h->tune);
     if (lrc == hipErrorInvalidValue)
@@ -710,6 +752,10 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
     const size_t params[3] = {count, nbits, (size_t) (zt ? 1 : 0)};
     const size_t items_bytes = count * sizeof(cntkq_quantize_item);
 
+    const bool capturing = stream_capturing(s);
+    if (capturing && !table_matches(tb, items, items_bytes, params))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: the stream is being captured into a graph and this item list "
+                                            "has not been seen: call once outside the capture first (the argument table is built and uploaded then)");
     if (!table_matches(tb, items, items_bytes, params))
     {
         // Every matrix is a member of one of two grid-wide launches (small / large LDS need), as a run of column
@@ -823,7 +869,10 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
     if (launches_left == 0)
         return CNTKQ_OK;
     // the last kernel of the call carries the table's event: the kernels before it run on the same stream
-    hipEvent_t done = tb.event;
+    // (none when the call is recorded into a graph: there is nothing to wait for, and the table is frozen instead)
+    hipEvent_t done = capturing ? nullptr : tb.event;
+    if (capturing)
+        tb.captured = true;
     for (int cls = 0; cls < 2; ++cls)
     {
         if (tb.members[cls] == 0)
@@ -835,7 +884,7 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
         const uint32_t* db = reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes) + tb.first_begin[cls];
         HIP_TRY(launch_quantize_batch(s, ev, de, db, (uint32_t) tb.members[cls], tb.blocks[cls], tb.lds[cls], nbits, zt),
                 "batched quantize kernel launch failed");
-        tb.in_flight = true;
+        tb.in_flight = tb.in_flight || !capturing;
     }
     LaunchTuning autotune;
     for (size_t i : tb.own)
@@ -846,7 +895,7 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
         ev.stop = launches_left == 0 ? done : nullptr;
         HIP_TRY(launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune),
                 "quantize kernel launch failed");
-        tb.in_flight = true;
+        tb.in_flight = tb.in_flight || !capturing;
     }
     h->last_quantize = done;
     h->quantize_included_fetch = false;
@@ -889,6 +938,10 @@ int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item
     BatchTable& tb = h->unquantize_table;
     const size_t params[3] = {count, nbits, 0};
     const size_t items_bytes = count * sizeof(cntkq_unquantize_item);
+    const bool capturing = stream_capturing(s);
+    if (capturing && !table_matches(tb, items, items_bytes, params))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: the stream is being captured into a graph and this item "
+                                            "list has not been seen: call once outside the capture first");
     if (!table_matches(tb, items, items_bytes, params))
     {
         const size_t entries_bytes = n * sizeof(UnquantizeBatchEntry);
@@ -934,12 +987,15 @@ int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item
         table_set_key(tb, items, items_bytes, params);
     }
     LaunchEvents ev;
-    ev.stop = tb.event;
+    ev.stop = capturing ? nullptr : tb.event;
     HIP_TRY(launch_unquantize_batch(s, ev, reinterpret_cast<const UnquantizeBatchEntry*>(tb.dev),
                                     reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes), (uint32_t) tb.members[0], tb.blocks[0],
                                     nbits, add != 0, tb.lds[0]),
             "batched unquantize kernel launch failed");
-    tb.in_flight = true;
+    if (capturing)
+        tb.captured = true;
+    else
+        tb.in_flight = true;
     h->last_unquantize = ev.stop;
     return CNTKQ_OK;
 }
@@ -1039,6 +1095,10 @@ int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduc
     }
     const size_t flat_bytes = flat.size() * sizeof(size_t);
 
+    const bool capturing = stream_capturing(s);
+    if (capturing && !table_matches(tb, flat.data(), flat_bytes, params))
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: the stream is being captured into a graph and this item "
+                                            "list has not been seen: call once outside the capture first");
     if (!table_matches(tb, flat.data(), flat_bytes, params))
     {
         constexpr size_t kSmallLds = 20 * 1024;
@@ -1115,14 +1175,17 @@ int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduc
             continue;
         LaunchEvents ev;
         launches_left--;
-        ev.stop = launches_left == 0 ? tb.event : nullptr;
+        ev.stop = launches_left == 0 && !capturing ? tb.event : nullptr;
         const StripeBatchEntry* de = reinterpret_cast<const StripeBatchEntry*>(tb.dev) + tb.first_entry[cls];
         const uint32_t* db = reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes) + tb.first_begin[cls];
         HIP_TRY(launch_stripe_reduce_batch(s, ev, de, db, (uint32_t) tb.members[cls], tb.blocks[cls], tb.lds[cls], nbits, zt),
                 "batched stripe reduction kernel launch failed");
-        tb.in_flight = true;
+        if (capturing)
+            tb.captured = true;
+        else
+            tb.in_flight = true;
     }
-    h->last_stripe = tb.event;
+    h->last_stripe = capturing ? nullptr : tb.event;
     return CNTKQ_OK;
 }
 

@@ -225,14 +225,13 @@ template <int NBITS, bool ZT, int T, int PER, bool EDGE = false>
 __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, PER>(), reg_waves<T, PER>()))) void quantize_reg_kernel(
     const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q, RegGeom c)
 {
-    using PS = PackShape<NBITS>;
     static_assert(NBITS < 32, "32-bit codes are whole QWords: nothing to assemble");
     constexpr uint32_t NW = T / 64;
     extern __shared__ f32x4 smem_v4[];
     float* red = reinterpret_cast<float*>(smem_v4);
     uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
     uint32_t* words = reinterpret_cast<uint32_t*>(red + kRegRedSlots);
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x;
     const size_t base = (size_t) blockIdx.x * c.rows;
     char* qc = q + (size_t) blockIdx.x * c.qcol;
     for (uint32_t x = tid; x < c.nq; x += T)

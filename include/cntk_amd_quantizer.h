@@ -23,6 +23,14 @@
  * use_dedicated_stream == 0 issue on the caller's main stream (the null stream unless
  * cntkq_set_main_stream was called). A handle is not re-entrant; distinct handles may be used
  * from distinct threads.
+ *
+ * HIP graphs: the quantize, unquantize and stripe-reduction calls (plain and batched) may be issued while the handle's
+ * stream is being captured; each becomes kernel nodes only (no allocation, no copy, no memset, no host wait). The
+ * matching cntkq_wait_* call then has nothing to wait for and returns at once: order against a replay with the graph's
+ * own launch stream. A batched call must have run once outside the capture with the same item list (its argument
+ * table is built and uploaded then); after a capture that table is never written again -- a later call with another
+ * list builds a new one -- so graphs stay valid until the handle is destroyed. Packed matrices in host memory
+ * (qbuf_on_host) are refused during capture.
  */
 #ifndef CNTK_AMD_QUANTIZER_H
 #define CNTK_AMD_QUANTIZER_H

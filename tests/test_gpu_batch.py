@@ -142,3 +142,61 @@ def test_batch_argument_checks():
         qz.UnquantizeBatchAsync([(QuantizedMatrix(8, 4, 1, cntk_amd.CPUDEVICE), Matrix(8, 4))])
     qz.QuantizeBatchAsync([], False)
     qz.UnquantizeBatchAsync([])
+
+
+@pytest.mark.filterwarnings("ignore:The CUDA Graph is empty")  # the refused capture below leaves one
+def test_batched_calls_and_hip_graphs():
+    """A batched call recorded into a graph: refused for an item list the handle has not seen (its table would have to
+    be built during the capture); once recorded, the table is frozen, so the graph still gives the right bytes after the
+    same handle has served other lists in between."""
+    qz = MatrixQuantizerImpl.Create(0, False)
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(datagen.case_seed(81))
+
+    def make(shapes):
+        return [(Matrix(r, c, 0, torch.randn(r * c, generator=gen, device="cuda:0") * 0.01), Matrix(r, c), QuantizedMatrix(r, c, 1, 0),
+                 Matrix(r, c)) for r, c in shapes]
+
+    first = make([(429, 64), (2048, 32), (64, 64)])
+    other = make([(147, 64), (1024, 16)])
+    items = lambda ms: [(g, r, q, r) for g, r, q, _ in ms]
+    unq = lambda ms: [(q, out) for _, _, q, out in ms]
+    side = torch.cuda.Stream()
+    qz.SetMainStream(side.cuda_stream)
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(cntk_amd.QuantizerLogicError, match="has not been seen"):
+        with torch.cuda.graph(graph, stream=side):
+            qz.QuantizeBatchAsync(items(first), False)
+    torch.cuda.synchronize()
+    # seen once, then recorded
+    qz.QuantizeBatchAsync(items(first), False)
+    qz.UnquantizeBatchAsync(unq(first))
+    qz.WaitUnquantizeAsyncDone()
+    torch.cuda.synchronize()
+    for _, r, _, _ in first:
+        r.data.zero_()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        qz.QuantizeBatchAsync(items(first), False)
+        qz.UnquantizeBatchAsync(unq(first))
+    qz.WaitQuantizeAsyncDone()  # nothing to wait for: returns at once
+    # the handle serves another gradient set (new tables), eagerly
+    qz.SetMainStream(torch.cuda.current_stream().cuda_stream)
+    qz.QuantizeBatchAsync(items(other), False)
+    qz.UnquantizeBatchAsync(unq(other))
+    qz.WaitUnquantizeAsyncDone()
+    torch.cuda.synchronize()
+    for step in range(3):
+        gs = [torch.randn(g.rows * g.cols, generator=gen, device="cuda:0") * 0.01 for g, _, _, _ in first]
+        r_in = [r.to_numpy() for _, r, _, _ in first]
+        for (g, _, _, _), x in zip(first, gs):
+            g.data.copy_(x)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for (g, r, q, out), r0 in zip(first, r_in):
+            parity.check_quantize(g.to_numpy(), r0, q.to_numpy(), r.to_numpy(), 1, False)
+            parity.check_unquantize(q.to_numpy(), g.rows, g.cols, 1, out.to_numpy())
+        # eager work on the other list between the replays
+        qz.QuantizeBatchAsync(items(other), False)
+        qz.WaitQuantizeAsyncDone()

@@ -456,3 +456,63 @@ def test_dedicated_stream_handles_share_one_stream():
     b.WaitUnquantizeAsyncDone()
     parity.check_quantize(g, np.zeros_like(g, order="F"), Q.to_numpy(), R.to_numpy(), 1, False)
     parity.check_unquantize(Q.to_numpy(), rows, cols, 1, Out.to_numpy())
+
+
+@pytest.mark.parametrize("rows,cols,nbits", [(2048, 96, 1), (429, 40, 4), (20000, 8, 1)])
+def test_calls_replayed_from_a_hip_graph(rows, cols, nbits):
+    """QuantizeAsync, UnquantizeAsync and the fused stripe reduction issued on a capturing stream become graph nodes
+    (no allocation, no host wait, no memset in them); every replay, with eager work and synchronisations in between,
+    must give the bytes of the same calls issued eagerly on the same inputs, residuals carried."""
+    k, owner = 3, 1
+    qz = MatrixQuantizerImpl.Create(0, False)
+
+    class Set:
+        def __init__(self):
+            self.G, self.R, self.Out = Matrix(rows, cols), Matrix(rows, cols), Matrix(rows, cols)
+            self.Q = QuantizedMatrix(rows, cols, nbits, 0)
+            self.S, self.Agg = Matrix(rows, cols), Matrix(rows, cols)
+            self.stripes = [QuantizedMatrix(rows, cols, nbits, 0) for _ in range(k)]
+
+        def run(self):
+            qz.QuantizeAsync(self.G, self.R, self.Q, self.R, False)
+            qz.UnquantizeAsync(self.Q, self.Out)
+            qz.StripeReduceAsync(self.stripes, owner, self.S, self.stripes[owner], False, agg_out=self.Agg)
+
+        def load(self, g, packed):
+            self.G.data.copy_(g)
+            for q, p in zip(self.stripes, packed):
+                q.buffer.copy_(p)
+
+    graphed, eager = Set(), Set()
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(datagen.case_seed(80, nbits) + rows)
+
+    def inputs():
+        g = torch.randn(rows * cols, generator=gen, device="cuda:0") * 0.01
+        packed = []
+        for w in range(k):  # valid packed stripes: quantize random matrices
+            T, Tr, Tq = Matrix(rows, cols, 0, torch.randn(rows * cols, generator=gen, device="cuda:0") * 0.01), Matrix(rows, cols), \
+                QuantizedMatrix(rows, cols, nbits, 0)
+            qz.QuantizeAsync(T, Tr, Tq, Tr, False)
+            packed.append(Tq.buffer)
+        torch.cuda.synchronize()
+        return g, packed
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        qz.SetMainStream(torch.cuda.current_stream().cuda_stream)
+        graphed.run()
+    qz.SetMainStream(torch.cuda.current_stream().cuda_stream)
+    for step in range(4):
+        g, packed = inputs()
+        graphed.load(g, packed)
+        eager.load(g, packed)
+        eager.run()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name in ("R", "Out", "S", "Agg"):
+            assert torch.equal(getattr(graphed, name).data, getattr(eager, name).data), "replay %d: %s differs" % (step, name)
+        assert torch.equal(graphed.Q.buffer, eager.Q.buffer), "replay %d: packed matrix differs" % step
+        assert torch.equal(graphed.stripes[owner].buffer, eager.stripes[owner].buffer), "replay %d: reduced stripe differs" % step

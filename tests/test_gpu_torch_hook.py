@@ -198,3 +198,36 @@ def test_hook_under_distributed_data_parallel():
         pytest.skip(out["skipped"])
     assert p.returncode == 0
     assert out["steps"] == 3 and out["max_err"] <= 1e-5 and out["aggregators"] >= 1
+
+
+def test_aggregate_replayed_from_a_hip_graph():
+    """The three batched launches of a step captured once (after a warm-up step has built the argument tables) and
+    replayed: every replay, with eager work and synchronisations in between, must give the bytes of an eager twin
+    that sees the same gradients, residuals carried from replay to replay."""
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(datagen.case_seed(79))
+    shapes = [s for s, dt in SHAPES if dt == torch.float32] + [(2048, 512), (9304, 64)]
+    fresh = lambda: [torch.randn(s, generator=gen, device="cuda:0") * 0.01 for s in shapes]
+    graphed, twin = QuantizedGradientAggregator(1, True), QuantizedGradientAggregator(1, True)
+    g = fresh()
+    graphed.aggregate(g)  # warm-up: buffers, residuals and the cached tables of the batched calls come into being
+    torch.cuda.synchronize()
+    graphed.reset_state()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        graphed.aggregate(g)
+    graphed.reset_state()
+    torch.cuda.synchronize()
+    for step in range(5):
+        new = fresh()
+        ref = [x.clone() for x in new]
+        twin.aggregate(ref)
+        for a, b in zip(g, new):
+            a.copy_(b)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(g, ref)):
+            assert torch.equal(a, b), "replay %d, gradient %d differs from the eager step" % (step, i)
+        for a, b in zip(graphed._residual + graphed._stripe_residual, twin._residual + twin._stripe_residual):
+            assert torch.equal(a, b), "replay %d: residuals differ from the eager step's" % step
