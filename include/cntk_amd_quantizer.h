@@ -92,7 +92,8 @@ int cntkq_device_id(const cntkq_quantizer* h);
 void* cntkq_stream(const cntkq_quantizer* h);
 
 /* Sets the main stream used by handles without a dedicated stream (the reference's GetStream(),
- * Source/Math/MatrixQuantizerGPU.cu:248-252) and by cntkq_sync_with_main_stream. */
+ * Source/Math/MatrixQuantizerGPU.cu:248-252) and by cntkq_sync_with_main_stream. Work already issued on the previous
+ * main stream is not ordered against work issued on the new one: that is the caller's to arrange. */
 int cntkq_set_main_stream(cntkq_quantizer* h, void* hip_stream);
 
 /* MatrixComputeStreamEvent::Create + SynchronizeQuantizationComputeStreamWithEvent
