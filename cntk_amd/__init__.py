@@ -94,6 +94,9 @@ def lib():
         L.cntkq_unquantize_async_f64.argtypes = L.cntkq_unquantize_async.argtypes
         L.cntkq_stripe_reduce_async_f64.argtypes = L.cntkq_stripe_reduce_async.argtypes
         L.cntkq_stripe_reduce_batch_async.argtypes = [_vp, ctypes.POINTER(_StripeReduceItem), _sz, _sz, _sz, _sz, ctypes.c_int]
+        L.cntkq_quantize_batch_async_f64.argtypes = L.cntkq_quantize_batch_async.argtypes
+        L.cntkq_unquantize_batch_async_f64.argtypes = L.cntkq_unquantize_batch_async.argtypes
+        L.cntkq_stripe_reduce_batch_async_f64.argtypes = L.cntkq_stripe_reduce_batch_async.argtypes
         for name in ("cntkq_stripe_reduce_max_rows", "cntkq_stripe_reduce_max_rows_f64"):
             getattr(L, name).argtypes = [_sz]
             getattr(L, name).restype = _sz
@@ -264,8 +267,9 @@ class PreparedBatch:
     """The argument block of one batched call, built once by MatrixQuantizerImpl.Prepare...Batch. It holds addresses,
     not matrices: the caller keeps the matrices alive and in place for as long as it uses the block."""
 
-    def __init__(self, kind, array, count, nbits, keep, workers=0):
+    def __init__(self, kind, array, count, nbits, keep, workers=0, dtype=torch.float32):
         self.kind, self.array, self.count, self.nbits, self.keep, self.workers = kind, array, count, nbits, keep, workers
+        self.dtype = dtype
 
 
 class MatrixQuantizerImpl:
@@ -343,14 +347,14 @@ class MatrixQuantizerImpl:
 
     def QuantizeBatchAsync(self, items, zero_threshold_for_1bit):
         """The aggregator's loop over its gradient matrices as one call (Source/1BitSGD/AllReduceDistGradAggregator.h:288-300).
-        items: sequence of (in_matrix, in_residual, out_qmatrix, out_residual); all packed matrices on the device and of
-        one bit width."""
+        items: sequence of (in_matrix, in_residual, out_qmatrix, out_residual); all packed matrices on the device, of
+        one bit width and one element type."""
         if isinstance(items, PreparedBatch):
             if items.kind != "quantize":
                 raise QuantizerLogicError("QuantizeBatchAsync: prepared for another call")
             if items.count:
-                _check(lib().cntkq_quantize_batch_async(self._h, items.array, items.count, items.nbits,
-                                                        int(bool(zero_threshold_for_1bit))))
+                _check(_fn("cntkq_quantize_batch_async", items.dtype)(self._h, items.array, items.count, items.nbits,
+                                                                      int(bool(zero_threshold_for_1bit))))
             return
         self.QuantizeBatchAsync(self.PrepareQuantizeBatch(items), zero_threshold_for_1bit)
 
@@ -369,10 +373,10 @@ class MatrixQuantizerImpl:
                     raise QuantizerLogicError("QuantizeBatchAsync: matrix dimensions do not match")
             if q.GetNumBits() != nbits or q.GetDeviceId() < 0:
                 raise QuantizerLogicError("QuantizeBatchAsync: packed matrices must share one bit width and live on the device")
-            if any(m.dtype != torch.float32 for m in (g, r_in, r_out, q)):
-                raise QuantizerLogicError("QuantizeBatchAsync: the batched calls exist for float32 only")
+            if any(m.dtype != items[0][0].dtype for m in (g, r_in, r_out, q)):
+                raise QuantizerLogicError("QuantizeBatchAsync: all matrices of a call must have one element type")
             arr[k] = _QuantizeItem(g.Data(), r_in.Data(), r_out.Data(), q.Buffer(), rows, cols)
-        return PreparedBatch("quantize", arr, len(items), nbits, ())
+        return PreparedBatch("quantize", arr, len(items), nbits, (), dtype=items[0][0].dtype)
 
     def UnquantizeBatchAsync(self, items, add=False):
         """The aggregator's final loop (Source/1BitSGD/AllReduceDistGradAggregator.h:517-522) as one call.
@@ -381,7 +385,7 @@ class MatrixQuantizerImpl:
             if items.kind != "unquantize":
                 raise QuantizerLogicError("UnquantizeBatchAsync: prepared for another call")
             if items.count:
-                _check(lib().cntkq_unquantize_batch_async(self._h, items.array, items.count, items.nbits, int(bool(add))))
+                _check(_fn("cntkq_unquantize_batch_async", items.dtype)(self._h, items.array, items.count, items.nbits, int(bool(add))))
             return
         self.UnquantizeBatchAsync(self.PrepareUnquantizeBatch(items), add)
 
@@ -397,10 +401,10 @@ class MatrixQuantizerImpl:
                 raise QuantizerLogicError("UnquantizeBatchAsync: matrix dimensions do not match")
             if q.GetNumBits() != nbits or q.GetDeviceId() < 0:
                 raise QuantizerLogicError("UnquantizeBatchAsync: packed matrices must share one bit width and live on the device")
-            if q.dtype != torch.float32 or out.dtype != torch.float32:
-                raise QuantizerLogicError("UnquantizeBatchAsync: the batched calls exist for float32 only")
+            if q.dtype != items[0][1].dtype or out.dtype != items[0][1].dtype:
+                raise QuantizerLogicError("UnquantizeBatchAsync: all matrices of a call must have one element type")
             arr[k] = _UnquantizeItem(q.Buffer(), out.Data(), out.GetNumRows(), out.GetNumCols())
-        return PreparedBatch("unquantize", arr, len(items), nbits, ())
+        return PreparedBatch("unquantize", arr, len(items), nbits, (), dtype=items[0][1].dtype)
 
     def StripeReduceAsync(self, stripes, owner, stripe_residual, out_qstripe, zero_threshold_for_1bit, agg_out=None):
         """Fused stripe reduction of the quantized all-reduce (dataflow of
@@ -423,13 +427,13 @@ class MatrixQuantizerImpl:
 
     def StripeReduceBatchAsync(self, items, owner, zero_threshold_for_1bit):
         """The owner's stripe reductions of a whole gradient set as one call. items: sequence of
-        (stripes, stripe_residual, out_qstripe, agg_out or None), one per gradient matrix, float32 only."""
+        (stripes, stripe_residual, out_qstripe, agg_out or None), one per gradient matrix, one element type."""
         if isinstance(items, PreparedBatch):
             if items.kind != "stripe_reduce":
                 raise QuantizerLogicError("StripeReduceBatchAsync: prepared for another call")
             if items.count:
-                _check(lib().cntkq_stripe_reduce_batch_async(self._h, items.array, items.count, items.workers, owner, items.nbits,
-                                                             int(bool(zero_threshold_for_1bit))))
+                _check(_fn("cntkq_stripe_reduce_batch_async", items.dtype)(self._h, items.array, items.count, items.workers, owner,
+                                                                           items.nbits, int(bool(zero_threshold_for_1bit))))
             return
         self.StripeReduceBatchAsync(self.PrepareStripeReduceBatch(items), owner, zero_threshold_for_1bit)
 
@@ -452,13 +456,13 @@ class MatrixQuantizerImpl:
             if stripe_residual.GetNumRows() != rows or stripe_residual.GetNumCols() != cols:
                 raise QuantizerLogicError("StripeReduceBatchAsync: stripe residual has the wrong shape")
             mats = list(stripes) + [stripe_residual, out_qstripe] + ([agg_out] if agg_out is not None else [])
-            if any(m.dtype != torch.float32 for m in mats):
-                raise QuantizerLogicError("StripeReduceBatchAsync: the batched calls exist for float32 only")
+            if any(m.dtype != items[0][1].dtype for m in mats):
+                raise QuantizerLogicError("StripeReduceBatchAsync: all matrices of a call must have one element type")
             ptrs = (_vp * k)(*[s.Buffer() for s in stripes])
             keep.append(ptrs)
             arr[n] = _StripeReduceItem(ptrs, stripe_residual.Data(), out_qstripe.Buffer(),
                                        agg_out.Data() if agg_out is not None else None, rows, cols)
-        return PreparedBatch("stripe_reduce", arr, len(items), nbits, keep, workers=k)
+        return PreparedBatch("stripe_reduce", arr, len(items), nbits, keep, workers=k, dtype=items[0][1].dtype)
 
     def WaitStripeReduceDone(self):
         _check(lib().cntkq_wait_stripe_reduce_done(self._h))

@@ -77,24 +77,25 @@ struct DistGradHeader
 
 // The messages of the quantized all-reduce. `from`, `to`, `owner` are worker ranks; a stripe is always the column range
 // GetStripeForNode(cols, owner, K) of gradient matrix `matrixIdx`, as a packed matrix.
-class StripeTransport
+template <class ElemType>
+class StripeTransportT
 {
 public:
-    virtual ~StripeTransport() {}
+    virtual ~StripeTransportT() {}
     virtual size_t NumProc() const = 0;
     // True when every message is device work on the quantizers' own stream, so that stream order alone keeps the steps
     // in sequence and the host waits the reference needs before handing buffers to MPI (:339, :494) can be skipped.
     virtual bool StreamOrdered() const { return false; }
     // Isend of a pre-aggregation stripe (Source/1BitSGD/AllReduceDistGradAggregator.h:339-365)
-    virtual void PostStripe(size_t from, size_t to, size_t matrixIdx, QuantizedMatrix<float>&& stripe) = 0;
+    virtual void PostStripe(size_t from, size_t to, size_t matrixIdx, QuantizedMatrix<ElemType>&& stripe) = 0;
     // what the matching Irecv delivered (:303-320)
-    virtual const QuantizedMatrix<float>& ReceivedStripe(size_t owner, size_t from, size_t matrixIdx) = 0;
+    virtual const QuantizedMatrix<ElemType>& ReceivedStripe(size_t owner, size_t from, size_t matrixIdx) = 0;
     // Isend of the requantized stripe to everybody (:484-497) and its reception into the receiver's own packed gradient (:463-476)
-    virtual void PostAggregatedStripe(size_t owner, size_t matrixIdx, QuantizedMatrix<float>&& stripe) = 0;
-    virtual void FetchAggregatedStripe(size_t to, size_t owner, size_t matrixIdx, QuantizedMatrix<float>& dst, void* hipStream) = 0;
+    virtual void PostAggregatedStripe(size_t owner, size_t matrixIdx, QuantizedMatrix<ElemType>&& stripe) = 0;
+    virtual void FetchAggregatedStripe(size_t to, size_t owner, size_t matrixIdx, QuantizedMatrix<ElemType>& dst, void* hipStream) = 0;
     // Where the receiver can read the owner's requantized stripe in place (same memory, or peer-accessible memory),
     // a view of it; nullptr where it has to be fetched into the receiver's own buffer first.
-    virtual const QuantizedMatrix<float>* AggregatedStripeView(size_t /*to*/, size_t /*owner*/, size_t /*matrixIdx*/) { return nullptr; }
+    virtual const QuantizedMatrix<ElemType>* AggregatedStripeView(size_t /*to*/, size_t /*owner*/, size_t /*matrixIdx*/) { return nullptr; }
     // headers to the main node and back (:323-333, 380-383, 440-457, 478-514)
     virtual void PostHeader(size_t from, const DistGradHeader& header) = 0;
     virtual DistGradHeader AggregatedHeader() = 0;
@@ -102,31 +103,32 @@ public:
 
 // All workers live in one process and their buffers in one GPU's memory: a stripe "message" is a view of the sender's
 // buffer, the broadcast is a device-to-device copy on the quantizers' stream.
-class InProcessTransport final : public StripeTransport
+template <class ElemType>
+class InProcessTransportT final : public StripeTransportT<ElemType>
 {
 public:
-    explicit InProcessTransport(size_t numWorkers, bool streamOrdered = true) : m_numWorkers(numWorkers), m_streamOrdered(streamOrdered) {}
+    explicit InProcessTransportT(size_t numWorkers, bool streamOrdered = true) : m_numWorkers(numWorkers), m_streamOrdered(streamOrdered) {}
     size_t NumProc() const override { return m_numWorkers; }
     bool StreamOrdered() const override { return m_streamOrdered; }
 
-    void PostStripe(size_t from, size_t to, size_t matrixIdx, QuantizedMatrix<float>&& stripe) override
+    void PostStripe(size_t from, size_t to, size_t matrixIdx, QuantizedMatrix<ElemType>&& stripe) override
     {
         Store(m_stripes, to * m_numWorkers + from, matrixIdx, std::move(stripe));
     }
-    const QuantizedMatrix<float>& ReceivedStripe(size_t owner, size_t from, size_t matrixIdx) override
+    const QuantizedMatrix<ElemType>& ReceivedStripe(size_t owner, size_t from, size_t matrixIdx) override
     {
-        const QuantizedMatrix<float>* s = Find(m_stripes, owner * m_numWorkers + from, matrixIdx);
+        const QuantizedMatrix<ElemType>* s = Find(m_stripes, owner * m_numWorkers + from, matrixIdx);
         if (s == nullptr)
             throw std::logic_error("InProcessTransport: stripe was never posted");
         return *s;
     }
-    void PostAggregatedStripe(size_t owner, size_t matrixIdx, QuantizedMatrix<float>&& stripe) override
+    void PostAggregatedStripe(size_t owner, size_t matrixIdx, QuantizedMatrix<ElemType>&& stripe) override
     {
         Store(m_aggregated, owner, matrixIdx, std::move(stripe));
     }
-    void FetchAggregatedStripe(size_t /*to*/, size_t owner, size_t matrixIdx, QuantizedMatrix<float>& dst, void* hipStream) override
+    void FetchAggregatedStripe(size_t /*to*/, size_t owner, size_t matrixIdx, QuantizedMatrix<ElemType>& dst, void* hipStream) override
     {
-        const QuantizedMatrix<float>* s = Find(m_aggregated, owner, matrixIdx);
+        const QuantizedMatrix<ElemType>* s = Find(m_aggregated, owner, matrixIdx);
         if (s == nullptr)
             throw std::logic_error("InProcessTransport: aggregated stripe was never posted");
         if (s->GetSize() != dst.GetSize())
@@ -136,7 +138,7 @@ public:
                                             static_cast<hipStream_t>(hipStream)),
                              "hipMemcpyAsync");
     }
-    const QuantizedMatrix<float>* AggregatedStripeView(size_t /*to*/, size_t owner, size_t matrixIdx) override
+    const QuantizedMatrix<ElemType>* AggregatedStripeView(size_t /*to*/, size_t owner, size_t matrixIdx) override
     {
         return Find(m_aggregated, owner, matrixIdx);
     }
@@ -159,20 +161,20 @@ public:
 private:
     // messages by (channel, matrix); a message that names the very buffer of the previous step's is kept as it is,
     // so a steady training loop allocates nothing here
-    typedef std::vector<std::vector<std::unique_ptr<QuantizedMatrix<float>>>> Slots;
-    static void Store(Slots& slots, size_t channel, size_t matrixIdx, QuantizedMatrix<float>&& stripe)
+    typedef std::vector<std::vector<std::unique_ptr<QuantizedMatrix<ElemType>>>> Slots;
+    static void Store(Slots& slots, size_t channel, size_t matrixIdx, QuantizedMatrix<ElemType>&& stripe)
     {
         if (slots.size() <= channel)
             slots.resize(channel + 1);
         if (slots[channel].size() <= matrixIdx)
             slots[channel].resize(matrixIdx + 1);
-        std::unique_ptr<QuantizedMatrix<float>>& slot = slots[channel][matrixIdx];
+        std::unique_ptr<QuantizedMatrix<ElemType>>& slot = slots[channel][matrixIdx];
         if (slot && slot->Buffer() == stripe.Buffer() && slot->GetNumRows() == stripe.GetNumRows() &&
             slot->GetNumCols() == stripe.GetNumCols() && slot->GetNumBits() == stripe.GetNumBits())
             return;
-        slot.reset(new QuantizedMatrix<float>(std::move(stripe)));
+        slot.reset(new QuantizedMatrix<ElemType>(std::move(stripe)));
     }
-    static const QuantizedMatrix<float>* Find(const Slots& slots, size_t channel, size_t matrixIdx)
+    static const QuantizedMatrix<ElemType>* Find(const Slots& slots, size_t channel, size_t matrixIdx)
     {
         if (channel >= slots.size() || matrixIdx >= slots[channel].size())
             return nullptr;
@@ -184,6 +186,10 @@ private:
     Slots m_aggregated;
     std::map<size_t, DistGradHeader> m_headers;
 };
+
+// the float instantiation under the names of the message interface
+typedef StripeTransportT<float> StripeTransport;
+typedef InProcessTransportT<float> InProcessTransport;
 
 template <class ElemType>
 class AllReduceDistGradAggregator
@@ -201,7 +207,7 @@ public:
         bool useBatchedCalls = true;      // one launch for all gradients in steps 1 and 5
     };
 
-    AllReduceDistGradAggregator(StripeTransport& transport, size_t myRank, int deviceId, int nBits, bool zeroThresholdFor1Bit,
+    AllReduceDistGradAggregator(StripeTransportT<ElemType>& transport, size_t myRank, int deviceId, int nBits, bool zeroThresholdFor1Bit,
                                 bool useQuantizationForSelfStripe, bool useAsyncAggregation, Options options = Options())
         : m_transport(transport), m_rank(myRank), m_deviceId(deviceId), m_numQuantizationBits((size_t) nBits),
           m_zeroThresholdFor1Bit(zeroThresholdFor1Bit), m_useQuantizationForSelfStripe(useQuantizationForSelfStripe),
@@ -497,7 +503,7 @@ private:
         ev->SynchronizeQuantizationComputeStreamWithEvent<ElemType>(q.Impl());
     }
 
-    StripeTransport& m_transport;
+    StripeTransportT<ElemType>& m_transport;
     size_t m_rank;
     int m_deviceId;
     size_t m_numQuantizationBits;
@@ -628,7 +634,7 @@ public:
     }
 
 private:
-    InProcessTransport m_transport;
+    InProcessTransportT<ElemType> m_transport;
     std::vector<std::unique_ptr<AllReduceDistGradAggregator<ElemType>>> m_workers;
     std::vector<std::vector<std::unique_ptr<Matrix<ElemType>>>> m_buffered;
     std::vector<DistGradHeader> m_bufferedHeaders;

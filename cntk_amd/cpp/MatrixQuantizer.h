@@ -74,6 +74,21 @@ struct Abi<float>
     {
         return cntkq_stripe_reduce_async(h, stripes, workers, owner, rows, cols, bits, stripeRes, qOut, agg, zt);
     }
+    typedef cntkq_quantize_item QuantizeItem;
+    typedef cntkq_unquantize_item UnquantizeItem;
+    typedef cntkq_stripe_reduce_item StripeReduceItem;
+    static int QuantizeBatch(cntkq_quantizer* h, const QuantizeItem* items, size_t n, size_t bits, int zt)
+    {
+        return cntkq_quantize_batch_async(h, items, n, bits, zt);
+    }
+    static int UnquantizeBatch(cntkq_quantizer* h, const UnquantizeItem* items, size_t n, size_t bits, int add)
+    {
+        return cntkq_unquantize_batch_async(h, items, n, bits, add);
+    }
+    static int StripeReduceBatch(cntkq_quantizer* h, const StripeReduceItem* items, size_t n, size_t workers, size_t owner, size_t bits, int zt)
+    {
+        return cntkq_stripe_reduce_batch_async(h, items, n, workers, owner, bits, zt);
+    }
 };
 
 template <>
@@ -96,6 +111,21 @@ struct Abi<double>
                             size_t bits, double* stripeRes, void* qOut, double* agg, int zt)
     {
         return cntkq_stripe_reduce_async_f64(h, stripes, workers, owner, rows, cols, bits, stripeRes, qOut, agg, zt);
+    }
+    typedef cntkq_quantize_item_f64 QuantizeItem;
+    typedef cntkq_unquantize_item_f64 UnquantizeItem;
+    typedef cntkq_stripe_reduce_item_f64 StripeReduceItem;
+    static int QuantizeBatch(cntkq_quantizer* h, const QuantizeItem* items, size_t n, size_t bits, int zt)
+    {
+        return cntkq_quantize_batch_async_f64(h, items, n, bits, zt);
+    }
+    static int UnquantizeBatch(cntkq_quantizer* h, const UnquantizeItem* items, size_t n, size_t bits, int add)
+    {
+        return cntkq_unquantize_batch_async_f64(h, items, n, bits, add);
+    }
+    static int StripeReduceBatch(cntkq_quantizer* h, const StripeReduceItem* items, size_t n, size_t workers, size_t owner, size_t bits, int zt)
+    {
+        return cntkq_stripe_reduce_batch_async_f64(h, items, n, workers, owner, bits, zt);
     }
 };
 } // namespace detail
@@ -366,11 +396,10 @@ public:
     };
     void QuantizeBatchAsync(const std::vector<QuantizeItem>& items, bool zeroThresholdFor1Bit)
     {
-        static_assert(std::is_same<ElemType, float>::value, "the batched calls exist for float only");
         if (items.empty())
             return;
         const size_t nbits = items[0].outQMatrix->GetNumBits();
-        std::vector<cntkq_quantize_item> raw;
+        std::vector<typename detail::Abi<ElemType>::QuantizeItem> raw;
         for (const auto& it : items)
         {
             const size_t rows = it.inMatrix->GetNumRows(), cols = it.inMatrix->GetNumCols();
@@ -379,9 +408,9 @@ public:
                 throw std::invalid_argument("QuantizeBatchAsync: matrix dimensions do not match");
             if (it.outQMatrix->GetNumBits() != nbits || it.outQMatrix->GetDeviceId() < 0)
                 throw std::invalid_argument("QuantizeBatchAsync: packed matrices must share one bit width and live on the device");
-            raw.push_back(cntkq_quantize_item{it.inMatrix->Data(), it.inResidual->Data(), it.outResidual->Data(), it.outQMatrix->Buffer(), rows, cols});
+            raw.push_back(typename detail::Abi<ElemType>::QuantizeItem{it.inMatrix->Data(), it.inResidual->Data(), it.outResidual->Data(), it.outQMatrix->Buffer(), rows, cols});
         }
-        detail::Check(cntkq_quantize_batch_async(m_handle, raw.data(), raw.size(), nbits, zeroThresholdFor1Bit ? 1 : 0));
+        detail::Check(detail::Abi<ElemType>::QuantizeBatch(m_handle, raw.data(), raw.size(), nbits, zeroThresholdFor1Bit ? 1 : 0));
     }
     struct UnquantizeItem
     {
@@ -390,20 +419,19 @@ public:
     };
     void UnquantizeBatchAsync(const std::vector<UnquantizeItem>& items, bool add = false)
     {
-        static_assert(std::is_same<ElemType, float>::value, "the batched calls exist for float only");
         if (items.empty())
             return;
         const size_t nbits = items[0].inQMatrix->GetNumBits();
-        std::vector<cntkq_unquantize_item> raw;
+        std::vector<typename detail::Abi<ElemType>::UnquantizeItem> raw;
         for (const auto& it : items)
         {
             if (it.inQMatrix->GetNumRows() != it.outMatrix->GetNumRows() || it.inQMatrix->GetNumCols() != it.outMatrix->GetNumCols())
                 throw std::invalid_argument("UnquantizeBatchAsync: matrix dimensions do not match");
             if (it.inQMatrix->GetNumBits() != nbits || it.inQMatrix->GetDeviceId() < 0)
                 throw std::invalid_argument("UnquantizeBatchAsync: packed matrices must share one bit width and live on the device");
-            raw.push_back(cntkq_unquantize_item{it.inQMatrix->Buffer(), it.outMatrix->Data(), it.outMatrix->GetNumRows(), it.outMatrix->GetNumCols()});
+            raw.push_back(typename detail::Abi<ElemType>::UnquantizeItem{it.inQMatrix->Buffer(), it.outMatrix->Data(), it.outMatrix->GetNumRows(), it.outMatrix->GetNumCols()});
         }
-        detail::Check(cntkq_unquantize_batch_async(m_handle, raw.data(), raw.size(), nbits, add ? 1 : 0));
+        detail::Check(detail::Abi<ElemType>::UnquantizeBatch(m_handle, raw.data(), raw.size(), nbits, add ? 1 : 0));
     }
 
     // Fused stripe reduction of the quantized all-reduce (dataflow of Source/1BitSGD/AllReduceDistGradAggregator.h:365-436):
@@ -434,13 +462,12 @@ public:
     };
     void StripeReduceBatchAsync(const std::vector<StripeReduceItem>& items, size_t owner, bool zeroThresholdFor1Bit)
     {
-        static_assert(std::is_same<ElemType, float>::value, "the batched calls exist for float only");
         if (items.empty())
             return;
         const size_t workers = items[0].stripes.size();
         const size_t nbits = items[0].outQStripe->GetNumBits();
         std::vector<std::vector<const void*>> ptrs(items.size());
-        std::vector<cntkq_stripe_reduce_item> raw;
+        std::vector<typename detail::Abi<ElemType>::StripeReduceItem> raw;
         for (size_t i = 0; i < items.size(); ++i)
         {
             const auto& it = items[i];
@@ -453,11 +480,11 @@ public:
                     throw std::invalid_argument("StripeReduceBatchAsync: stripes must be device-resident and of equal shape");
                 ptrs[i].push_back(s->Buffer());
             }
-            raw.push_back(cntkq_stripe_reduce_item{ptrs[i].data(), it.stripeResidual->Data(), it.outQStripe->Buffer(),
+            raw.push_back(typename detail::Abi<ElemType>::StripeReduceItem{ptrs[i].data(), it.stripeResidual->Data(), it.outQStripe->Buffer(),
                                                    it.aggregate ? it.aggregate->Data() : nullptr, it.outQStripe->GetNumRows(),
                                                    it.outQStripe->GetNumCols()});
         }
-        detail::Check(cntkq_stripe_reduce_batch_async(m_handle, raw.data(), raw.size(), workers, owner, nbits, zeroThresholdFor1Bit ? 1 : 0));
+        detail::Check(detail::Abi<ElemType>::StripeReduceBatch(m_handle, raw.data(), raw.size(), workers, owner, nbits, zeroThresholdFor1Bit ? 1 : 0));
     }
     void WaitStripeReduceDone() { detail::Check(cntkq_wait_stripe_reduce_done(m_handle)); }
 

@@ -316,14 +316,15 @@ __device__ __forceinline__ TileLds tile_lds(double* smem, const TileGeom& t)
 
 // ---- quantize ---------------------------------------------------------------------------------------------
 
+// (block: the tile's index within the matrix; smem: the workgroup's dynamic LDS -- a kernel of its own below, and a member
+// of the batched launch)
 template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kThreads) void quantize_tile_kernel(const double* __restrict__ g, const double* r_in, double* r_out,
-                                                                 char* __restrict__ q, TileGeom t)
+__device__ __forceinline__ void quantize_tile_body(const double* __restrict__ g, const double* r_in, double* r_out, char* __restrict__ q,
+                                                   const TileGeom& t, uint32_t block, double* smem)
 {
-    extern __shared__ f64x2 smem_f64[];
-    const TileLds l = tile_lds(reinterpret_cast<double*>(smem_f64), t);
+    const TileLds l = tile_lds(smem, t);
     const uint32_t tid = threadIdx.x;
-    const uint32_t j0 = blockIdx.x * t.cols_per_tile;
+    const uint32_t j0 = block * t.cols_per_tile;
     const uint32_t nc = min(t.cols_per_tile, t.cols - j0);
     const size_t base = (size_t) j0 * t.rows;
     const uint32_t total = nc * t.rows;
@@ -361,6 +362,14 @@ __global__ __launch_bounds__(kThreads) void quantize_tile_kernel(const double* _
     char* qtile = q + (size_t) j0 * t.qcol;
     tile_stats<NBITS, ZT>(l.tile, l.hdr, l.scratch_f, l.scratch_u, t, nc, qtile);
     tile_pack<NBITS, ZT>(l.tile, l.hdr, l.words, t, nc, qtile, r_out + base);
+}
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kThreads) void quantize_tile_kernel(const double* __restrict__ g, const double* r_in, double* r_out,
+                                                                 char* __restrict__ q, TileGeom t)
+{
+    extern __shared__ f64x2 smem_f64[];
+    quantize_tile_body<NBITS, ZT>(g, r_in, r_out, q, t, blockIdx.x, reinterpret_cast<double*>(smem_f64));
 }
 
 // one workgroup of 1024 threads per column, statistics and packing re-read global memory
@@ -462,16 +471,15 @@ __global__ __launch_bounds__(kTallThreads) void quantize_tall_kernel(const doubl
 // ---- stripe reduction: K packed stripes -> fp64 sum (owner first, then ascending) -> requantize ------------
 
 template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kThreads) void stripe_reduce_tile_kernel(StripeSources src, double* stripe_res, char* q_out,
-                                                                      double* agg_out, TileGeom t)
+__device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src, double* stripe_res, char* q_out, double* agg_out,
+                                                        const TileGeom& t, uint32_t block, double* smem)
 {
     using PS = PackShape<NBITS>;
     constexpr uint32_t BATCH = 8; // packed words fetched together, so their latencies overlap
 
-    extern __shared__ f64x2 smem_f64[];
-    const TileLds l = tile_lds(reinterpret_cast<double*>(smem_f64), t);
+    const TileLds l = tile_lds(smem, t);
     const uint32_t tid = threadIdx.x;
-    const uint32_t j0 = blockIdx.x * t.cols_per_tile;
+    const uint32_t j0 = block * t.cols_per_tile;
     const uint32_t nc = min(t.cols_per_tile, t.cols - j0);
     const size_t base = (size_t) j0 * t.rows;
     const uint32_t K = src.workers;
@@ -564,6 +572,14 @@ __global__ __launch_bounds__(kThreads) void stripe_reduce_tile_kernel(StripeSour
     tile_pack<NBITS, ZT>(l.tile, l.hdr, l.words, t, nc, qtile, sp);
 }
 
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kThreads) void stripe_reduce_tile_kernel(StripeSources src, double* stripe_res, char* q_out,
+                                                                      double* agg_out, TileGeom t)
+{
+    extern __shared__ f64x2 smem_f64[];
+    stripe_reduce_tile_body<NBITS, ZT>(src, stripe_res, q_out, agg_out, t, blockIdx.x, reinterpret_cast<double*>(smem_f64));
+}
+
 // ---- unquantize ----------------------------------------------------------------------------------------------
 // One thread decodes WV consecutive QWords of a column (WV = 2: 16-byte stores; WV = 1: any shape) for a chunk of
 // `slots` consecutive bit positions; for a fixed bit position consecutive QWords are consecutive rows.
@@ -584,10 +600,10 @@ struct UnqGeom
 };
 
 template <int NBITS, int WV>
-__global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, double* out, UnqGeom t, int add)
+__device__ __forceinline__ void unquantize_body(const char* __restrict__ q, double* out, const UnqGeom& t, int add, uint32_t block_in)
 {
     using PS = PackShape<NBITS>;
-    const uint32_t block = t.swz_members > 1 ? unq_xcd_block(blockIdx.x, t.items / 256, t.swz_members, t.swz_gw) : blockIdx.x;
+    const uint32_t block = t.swz_members > 1 ? unq_xcd_block(block_in, t.items / 256, t.swz_members, t.swz_gw) : block_in;
     const uint64_t id64 = (uint64_t) block * 256 + threadIdx.x;
     if (id64 >= t.items)
         return;
@@ -652,19 +668,24 @@ __global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict_
     }
 }
 
+template <int NBITS, int WV>
+__global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, double* out, UnqGeom t, int add)
+{
+    unquantize_body<NBITS, WV>(q, out, t, add, blockIdx.x);
+}
+
 // ---- row-major and tile decoders (the fp32 unquantize_rows_kernel / unquantize_tile_kernel on doubles) ---------
 //
 // A 16-byte store holds two doubles; QWords are 64-bit; a packed record is nq + 2 QWords (lower, upper, bits).
 
 template <int NBITS>
-__global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __restrict__ q, double* out, UnqRowGeom t, int add)
+__device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q, double* out, const UnqRowGeom& t, int add, uint32_t block,
+                                                     uint64_t* words)
 {
     using PS = PackShape<NBITS>;
-    extern __shared__ f32x4 smem_v4[];
-    uint64_t* words = reinterpret_cast<uint64_t*>(smem_v4);
     const uint32_t tid = threadIdx.x;
     uint32_t c, ch;
-    unq_rows_block_to_chunk(blockIdx.x, t.chunks, t.blocks, c, ch);
+    unq_rows_block_to_chunk(block, t.chunks, t.blocks, c, ch);
     const char* qc = q + (size_t) c * t.qcol;
     const double* gh = reinterpret_cast<const double*>(qc);
     const ValueQ vq = make_vq<NBITS>(gh[0], gh[1]);
@@ -751,14 +772,20 @@ __global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __rest
 }
 
 template <int NBITS>
-__global__ __launch_bounds__(256) void unquantize_tile_kernel(const char* __restrict__ q, double* out, UnqTileGeom t, int add)
+__global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __restrict__ q, double* out, UnqRowGeom t, int add)
+{
+    extern __shared__ f32x4 smem_v4[];
+    unquantize_rows_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint64_t*>(smem_v4));
+}
+
+template <int NBITS>
+__device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q, double* out, const UnqTileGeom& t, int add, uint32_t block,
+                                                     uint64_t* words)
 {
     using PS = PackShape<NBITS>;
-    extern __shared__ f32x4 smem_v4[];
-    uint64_t* words = reinterpret_cast<uint64_t*>(smem_v4);            // ncols packed records
     double* dec = reinterpret_cast<double*>(words + t.cpt * t.rec_words); // per column: the two levels (1 bit) or (ufactor, lower)
     const uint32_t tid = threadIdx.x;
-    const uint32_t col0 = blockIdx.x * t.cpt;
+    const uint32_t col0 = block * t.cpt;
     const uint32_t ncols = (t.cols - col0 < t.cpt) ? t.cols - col0 : t.cpt;
     const uint64_t* src = reinterpret_cast<const uint64_t*>(q + (size_t) col0 * t.rec_words * 8);
     const uint32_t total_words = ncols * t.rec_words;
@@ -831,6 +858,13 @@ __global__ __launch_bounds__(256) void unquantize_tile_kernel(const char* __rest
         else
             o[i] = add ? x[0] + o[i] : x[0];
     }
+}
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_tile_kernel(const char* __restrict__ q, double* out, UnqTileGeom t, int add)
+{
+    extern __shared__ f32x4 smem_v4[];
+    unquantize_tile_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint64_t*>(smem_v4));
 }
 
 // ---- one workgroup per column, the column in registers (the fp32 quantize_reg_kernel on doubles) ------------
@@ -1067,6 +1101,88 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     unsigned long long* bits = reinterpret_cast<unsigned long long*>(qc + 16);
     for (uint32_t x = tid; x < c.nq; x += T)
         bits[x] = words[x];
+}
+
+// ---- whole gradient sets in one launch (the fp32 batch kernels on doubles) ------------------------------------------
+//
+// The workgroups of all member matrices form one grid; `begins` (count + 1 entries, ascending) gives the first workgroup
+// of every matrix. Members of the quantize and stripe-reduction launches are runs of column tiles; members of the
+// unquantize launch keep the decoder the plain call would choose.
+
+struct QuantizeBatchEntry64
+{
+    const double* g;
+    const double* r_in;
+    double* r_out;
+    char* q;
+    TileGeom t;
+};
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kThreads) void quantize_batch_kernel64(const QuantizeBatchEntry64* __restrict__ entries,
+                                                                    const uint32_t* __restrict__ begins, uint32_t count)
+{
+    extern __shared__ f64x2 smem_f64[];
+    const uint32_t e = batch_find(begins, count, blockIdx.x);
+    const TileGeom t = entries[e].t; // by value: read once, then held in registers whatever the kernel stores
+    quantize_tile_body<NBITS, ZT>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, t, blockIdx.x - begins[e],
+                                  reinterpret_cast<double*>(smem_f64));
+}
+
+struct StripeBatchEntry64
+{
+    StripeSources src;
+    double* stripe_res;
+    char* q_out;
+    double* agg_out;
+    TileGeom t;
+};
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kThreads) void stripe_reduce_batch_kernel64(const StripeBatchEntry64* __restrict__ entries,
+                                                                         const uint32_t* __restrict__ begins, uint32_t count)
+{
+    extern __shared__ f64x2 smem_f64[];
+    const uint32_t e = batch_find(begins, count, blockIdx.x);
+    const StripeBatchEntry64& en = entries[e]; // the table is read-only while the kernel runs
+    const TileGeom t = en.t;
+    stripe_reduce_tile_body<NBITS, ZT>(en.src, en.stripe_res, en.q_out, en.agg_out, t, blockIdx.x - begins[e],
+                                       reinterpret_cast<double*>(smem_f64));
+}
+
+struct UnquantizeBatchEntry64
+{
+    const char* q;
+    double* out;
+    uint32_t kind; // kUnqVec4 (here: 16-byte stores of two doubles), kUnqScalar, kUnqRows or kUnqTile
+    uint32_t pad;
+    UnqGeom qw;
+    UnqRowGeom rowg;
+    UnqTileGeom tile;
+};
+
+template <int NBITS>
+__global__ __launch_bounds__(256) void unquantize_batch_kernel64(const UnquantizeBatchEntry64* __restrict__ entries,
+                                                                 const uint32_t* __restrict__ begins, uint32_t count, int add)
+{
+    extern __shared__ f32x4 smem_v4[];
+    const uint32_t e = batch_find(begins, count, blockIdx.x);
+    const UnquantizeBatchEntry64& en = entries[e];
+    const uint32_t block = blockIdx.x - begins[e];
+    if (en.kind == kUnqVec4)
+        unquantize_body<NBITS, 2>(en.q, en.out, en.qw, add, block);
+    else if (en.kind == kUnqScalar)
+        unquantize_body<NBITS, 1>(en.q, en.out, en.qw, add, block);
+    else if (en.kind == kUnqRows)
+    {
+        const UnqRowGeom t = en.rowg; // by value: the loop below stores between its uses
+        unquantize_rows_body<NBITS>(en.q, en.out, t, add, block, reinterpret_cast<uint64_t*>(smem_v4));
+    }
+    else
+    {
+        const UnqTileGeom t = en.tile;
+        unquantize_tile_body<NBITS>(en.q, en.out, t, add, block, reinterpret_cast<uint64_t*>(smem_v4));
+    }
 }
 
 } // namespace f64

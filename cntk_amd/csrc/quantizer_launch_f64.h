@@ -172,6 +172,17 @@ struct RegLauncher
     }
 };
 
+// The kernel family a matrix gets when nothing is forced.
+inline int quantize_auto_path(const double* g, const double* r_in, const double* r_out, size_t rows, size_t nbits)
+{
+    // one column of doubles per tile fills LDS from about 5000 rows on (two workgroups per CU at 5120 rows, one at
+    // 7168); the register kernel overtakes the tile kernel there: 5120 rows 88 us against 94 us on 19 M elements,
+    // 6144: 85 against 99, 7168: 81 against 112 (4096: 104 against 85)
+    if (rows >= kRegMinRows && reg_applicable(g, r_in, r_out, rows, nbits))
+        return kPathReg;
+    return rows <= kTileMaxRows ? kPathTile : kPathTall;
+}
+
 // rows, cols > 0; pointers 8-byte aligned (checked by the caller). tune.quantize_path may force the tile or tall kernel.
 inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, void* q, size_t rows,
                                   size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
@@ -180,15 +191,7 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* 
     char* qc = static_cast<char*>(q);
     int path = tune.quantize_path;
     if (path == kPathAuto)
-    {
-        // one column of doubles per tile fills LDS from about 5000 rows on (two workgroups per CU at 5120 rows, one at
-        // 7168); the register kernel overtakes the tile kernel there: 5120 rows 88 us against 94 us on 19 M elements,
-        // 6144: 85 against 99, 7168: 81 against 112 (4096: 104 against 85)
-        if (rows >= kRegMinRows && reg_applicable(g, r_in, r_out, rows, nbits))
-            path = kPathReg;
-        else
-            path = rows <= kTileMaxRows ? kPathTile : kPathTall;
-    }
+        path = quantize_auto_path(g, r_in, r_out, rows, nbits);
     if (path == kPathReg)
     {
         if (!reg_applicable(g, r_in, r_out, rows, nbits))
@@ -270,9 +273,24 @@ inline hipError_t launch_unquantize_tile(hipStream_t s, LaunchEvents ev, const c
     default: return hipErrorInvalidValue;                                                                              \
     }
 
-inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* q, double* out, size_t rows, size_t cols, size_t nbits,
-                                    bool add, const LaunchTuning& tune)
+// Which decoder unquantizes a matrix, and its geometry; shared by the plain call and the batched one.
+struct UnquantizePlan64
 {
+    uint32_t kind = kUnqScalar; // kUnqVec4 (16-byte stores of two doubles), kUnqScalar, kUnqRows, kUnqTile
+    UnqGeom qw;
+    UnqRowGeom rowg;
+    UnqTileGeom tile;
+    uint32_t blocks = 0; // 256-thread blocks
+    size_t lds = 0;      // dynamic LDS (kUnqRows, kUnqTile)
+    bool ok = false;
+};
+
+inline UnquantizePlan64 plan_unquantize(const double* out, size_t rows, size_t cols, size_t nbits, const LaunchTuning& tune)
+{
+    UnquantizePlan64 p;
+    std::memset(&p.qw, 0, sizeof p.qw);
+    std::memset(&p.rowg, 0, sizeof p.rowg);
+    std::memset(&p.tile, 0, sizeof p.tile);
     const size_t vpw = 64 / nbits;
     const size_t nq = qwords_per_col(rows, nbits);
     const bool out16 = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
@@ -296,10 +314,9 @@ inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* 
         else if (rows_can)
             use_rows = true;
     }
-    const char* qc0 = static_cast<const char*>(q);
     if (use_rows)
     {
-        UnqRowGeom t;
+        UnqRowGeom& t = p.rowg;
         t.rows = (uint32_t) rows;
         t.nq = (uint32_t) nq;
         const size_t mult = nq > 512 ? 2 : 4;
@@ -314,13 +331,16 @@ inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* 
         if (blocks <= 0x7FFFFFFFull)
         {
             t.blocks = (uint32_t) blocks;
-            const int a = add ? 1 : 0;
-            CNTKQ_NBITS64_SWITCH(launch_unquantize_rows, s, ev, qc0, out, t, a)
+            p.kind = kUnqRows;
+            p.blocks = t.blocks;
+            p.lds = (size_t) t.nq * 8;
+            p.ok = true;
+            return p;
         }
     }
     if (use_tile)
     {
-        UnqTileGeom t;
+        UnqTileGeom& t = p.tile;
         t.rows = (uint32_t) rows;
         t.cols = (uint32_t) cols;
         t.nq = (uint32_t) nq;
@@ -335,13 +355,16 @@ inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* 
         if (blocks <= 0x7FFFFFFFull && (size_t) t.cpt * (t.rec_words + 2) * 8 <= kMaxLdsBytes)
         {
             t.blocks = (uint32_t) blocks;
-            const int a = add ? 1 : 0;
-            CNTKQ_NBITS64_SWITCH(launch_unquantize_tile, s, ev, qc0, out, t, a)
+            p.kind = kUnqTile;
+            p.blocks = t.blocks;
+            p.lds = (size_t) t.cpt * (t.rec_words + 2) * 8;
+            p.ok = true;
+            return p;
         }
     }
     const bool vec = mode != 1 && (nq % 2 == 0) && (rows % 2 == 0) && out16;
     const uint32_t wv = vec ? 2 : 1;
-    UnqGeom t;
+    UnqGeom& t = p.qw;
     t.rows = (uint32_t) rows;
     t.cols = (uint32_t) cols;
     t.nq = (uint32_t) nq;
@@ -356,7 +379,7 @@ inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* 
     const uint64_t per_col = (uint64_t) t.groups * t.chunks;
     const uint64_t items = per_col * cols;
     if (items > 0xFFFFFFFFull)
-        return hipErrorInvalidValue;
+        return p; // not ok
     t.per_col = (uint32_t) per_col;
     t.items = (uint32_t) items;
     // several workgroups per column that read the same QWords: regroup them by XCD (whole workgroups per column only)
@@ -373,19 +396,71 @@ inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* 
         }
     }
     t.qcol = qcol_bytes(nbits, rows);
+    p.kind = vec ? kUnqVec4 : kUnqScalar;
+    p.blocks = (uint32_t) (((uint64_t) t.items + 255) / 256);
+    p.ok = true;
+    return p;
+}
+
+template <int NBITS>
+inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const char* q, double* out, const UnquantizePlan64& p, int add)
+{
+    if (p.kind == kUnqRows)
+        return launch_unquantize_rows<NBITS>(s, ev, q, out, p.rowg, add);
+    if (p.kind == kUnqTile)
+        return launch_unquantize_tile<NBITS>(s, ev, q, out, p.tile, add);
+    return launch_unquantize_n<NBITS>(s, ev, q, out, p.qw, p.kind == kUnqVec4, add);
+}
+
+inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* q, double* out, size_t rows, size_t cols, size_t nbits,
+                                    bool add, const LaunchTuning& tune)
+{
+    const UnquantizePlan64 p = plan_unquantize(out, rows, cols, nbits, tune);
+    if (!p.ok)
+        return hipErrorInvalidValue;
     const char* qc = static_cast<const char*>(q);
     const int a = add ? 1 : 0;
-    switch (nbits)
+    CNTKQ_NBITS64_SWITCH(launch_unquantize_plan, s, ev, qc, out, p, a)
+}
+
+template <int NBITS, bool ZT>
+struct QuantizeBatchLauncher64
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const QuantizeBatchEntry64* entries, const uint32_t* begins, uint32_t count,
+                          uint32_t blocks, size_t lds)
     {
-    case 1: return launch_unquantize_n<1>(s, ev, qc, out, t, vec, a);
-    case 2: return launch_unquantize_n<2>(s, ev, qc, out, t, vec, a);
-    case 4: return launch_unquantize_n<4>(s, ev, qc, out, t, vec, a);
-    case 8: return launch_unquantize_n<8>(s, ev, qc, out, t, vec, a);
-    case 16: return launch_unquantize_n<16>(s, ev, qc, out, t, vec, a);
-    case 32: return launch_unquantize_n<32>(s, ev, qc, out, t, vec, a);
-    case 64: return launch_unquantize_n<64>(s, ev, qc, out, t, vec, a);
-    default: return hipErrorInvalidValue;
+        hipExtLaunchKernelGGL((quantize_batch_kernel64<NBITS, ZT>), dim3(blocks), dim3(kThreads), lds, s, ev.start, ev.stop, 0, entries, begins,
+                              count);
+        return hipGetLastError();
     }
+};
+
+template <int NBITS, bool ZT>
+struct StripeBatchLauncher64
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeBatchEntry64* entries, const uint32_t* begins, uint32_t count,
+                          uint32_t blocks, size_t lds)
+    {
+        hipExtLaunchKernelGGL((stripe_reduce_batch_kernel64<NBITS, ZT>), dim3(blocks), dim3(kThreads), lds, s, ev.start, ev.stop, 0, entries,
+                              begins, count);
+        return hipGetLastError();
+    }
+};
+
+template <int NBITS>
+inline hipError_t launch_unquantize_batch_n(hipStream_t s, LaunchEvents ev, const UnquantizeBatchEntry64* entries, const uint32_t* begins,
+                                            uint32_t count, uint32_t blocks, int add, size_t lds)
+{
+    hipExtLaunchKernelGGL((unquantize_batch_kernel64<NBITS>), dim3(blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count,
+                          add);
+    return hipGetLastError();
+}
+
+inline hipError_t launch_unquantize_batch(hipStream_t s, LaunchEvents ev, const UnquantizeBatchEntry64* entries, const uint32_t* begins,
+                                          uint32_t count, uint32_t blocks, size_t nbits, bool add, size_t lds)
+{
+    const int a = add ? 1 : 0;
+    CNTKQ_NBITS64_SWITCH(launch_unquantize_batch_n, s, ev, entries, begins, count, blocks, a, lds)
 }
 
 } // namespace f64

@@ -5,7 +5,7 @@ and of the v2 QuantizedDistributedCommunicator (QuantizedAggregate, Source/1BitS
 on a set of torch gradient tensors, with every packed buffer resident on the device:
 
   1. every gradient is quantized with its error-feedback residual, stripe by stripe, straight into the send buffer
-     (one batched launch for the whole set),
+     (one batched launch for the whole set, one per element type),
   2. the packed stripes change hands (all-to-all: worker r's stripe s goes to worker s),
   3. the owner of a stripe decodes and sums the K packed stripes and requantizes the sum with its stripe residual
      (one batched launch),
@@ -163,9 +163,11 @@ class QuantizedGradientAggregator:
         where = tuple(g.data_ptr() for g in grads)
         if self._plan is not None and self._plan["where"] == where:
             return self._plan
-        q32, u32 = self._items(grads, False)
         P = MatrixQuantizerImpl
-        self._plan = dict(where=where, q32=P.PrepareQuantizeBatch(q32), u32=P.PrepareUnquantizeBatch(u32))
+        q32, u32 = self._items(grads, False)
+        q64, u64 = self._items(grads, True) if self._any64 else ([], [])
+        self._plan = dict(where=where, q=[P.PrepareQuantizeBatch(q32), P.PrepareQuantizeBatch(q64)],
+                          u=[P.PrepareUnquantizeBatch(u32), P.PrepareUnquantizeBatch(u64)])
         return self._plan
 
     def _plan_stripes(self):
@@ -174,7 +176,7 @@ class QuantizedGradientAggregator:
         arrived = self._send if W == 1 else self._recv
         max32 = _fn("cntkq_stripe_reduce_max_rows", torch.float32)(self.nbits)
         max64 = _fn("cntkq_stripe_reduce_max_rows", torch.float64)(self.nbits)
-        fused, plain, tall = [], [], []
+        fused, fused64, tall = [], [], []
         for i, (rows, _, dt, _) in enumerate(self._shapes):
             n = self._stripe[me][i][1]
             if n == 0:
@@ -188,8 +190,9 @@ class QuantizedGradientAggregator:
             elif dt == torch.float32:
                 fused.append(item)
             else:
-                plain.append(item)
-        self._s32, self._s_plain, self._s_tall = MatrixQuantizerImpl.PrepareStripeReduceBatch(fused), plain, tall
+                fused64.append(item)
+        P = MatrixQuantizerImpl
+        self._s_fused, self._s_tall = [P.PrepareStripeReduceBatch(fused), P.PrepareStripeReduceBatch(fused64)], tall
 
     def quantize(self, grads):
         """Phase 1 (AllReduceDistGradAggregator.h:288-300)."""
@@ -199,10 +202,9 @@ class QuantizedGradientAggregator:
         if [(tuple(g.shape), g.dtype) for g in grads] != self._geom:
             raise QuantizerLogicError("the gradient list differs from the one this aggregator was set up for")
         self._impl.SetMainStream(torch.cuda.current_stream(grads[0].device).cuda_stream)
-        self._current = (self._plan_for(grads), grads, self._items(grads, True) if self._any64 else ([], []))
-        self._impl.QuantizeBatchAsync(self._current[0]["q32"], self.zt)
-        for g, r_in, q, r_out in self._current[2][0]:
-            self._impl.QuantizeAsync(g, r_in, q, r_out, self.zt)
+        self._current = (self._plan_for(grads), grads)
+        for prepared in self._current[0]["q"]:
+            self._impl.QuantizeBatchAsync(prepared, self.zt)
 
     def exchange_stripes(self):
         """Phase 2 (AllReduceDistGradAggregator.h:302-384: the stripes' sends and receives): fills the receive buffer."""
@@ -213,9 +215,8 @@ class QuantizedGradientAggregator:
     def reduce(self):
         """Phase 3 (AllReduceDistGradAggregator.h:365-436, 494)."""
         W, me = self.transport.world_size, self.transport.rank
-        self._impl.StripeReduceBatchAsync(self._s32, me, self.zt)
-        for stripes, sres, out, _ in self._s_plain:
-            self._impl.StripeReduceAsync(stripes, me, sres, out, self.zt)
+        for prepared in self._s_fused:
+            self._impl.StripeReduceBatchAsync(prepared, me, self.zt)
         for stripes, sres, out, _ in self._s_tall:
             # columns too tall for the fused kernel: the reference's own sequence of calls
             agg = Matrix(sres.rows, sres.cols, sres.device_id, dtype=sres.dtype)
@@ -234,10 +235,9 @@ class QuantizedGradientAggregator:
     def unquantize(self):
         """Phase 5 (AllReduceDistGradAggregator.h:517-522)."""
         W = self.transport.world_size
-        plan, grads, items64 = self._current
-        self._impl.UnquantizeBatchAsync(plan["u32"], add=False)
-        for q, out in items64[1]:
-            self._impl.UnquantizeAsync(q, out, add=False)
+        plan, grads = self._current
+        for prepared in plan["u"]:
+            self._impl.UnquantizeBatchAsync(prepared, add=False)
         if self.average and W > 1:
             torch._foreach_div_(list(grads), W)
         self._current = None

@@ -240,6 +240,43 @@ int cntkq_stripe_reduce_async_f64(cntkq_quantizer* h, const void* const* stripes
                                   double* agg_out, int zero_threshold_for_1bit);
 size_t cntkq_stripe_reduce_max_rows_f64(size_t nbits);
 
+/* The gradient-set calls (cntkq_quantize_batch_async, cntkq_unquantize_batch_async, cntkq_stripe_reduce_batch_async) for
+ * double matrices: the same loops of the aggregator (Source/1BitSGD/AllReduceDistGradAggregator.h:288-300, 339-436,
+ * 517-522) as one call each; results identical to the _f64 plain calls item by item. Pointers 8-byte aligned. */
+typedef struct cntkq_quantize_item_f64
+{
+    const double* in;
+    const double* res_in;
+    double* res_out; /* may be res_in */
+    void* qbuf;      /* device memory, cols * cntkq_qcol_bytes_f64(nbits, rows) bytes */
+    size_t rows;
+    size_t cols;
+} cntkq_quantize_item_f64;
+
+typedef struct cntkq_unquantize_item_f64
+{
+    const void* qbuf;
+    double* out;
+    size_t rows;
+    size_t cols;
+} cntkq_unquantize_item_f64;
+
+typedef struct cntkq_stripe_reduce_item_f64
+{
+    const void* const* stripes; /* `workers` device pointers: worker w's packed stripe of this matrix */
+    double* stripe_res;         /* rows x stripe_cols, updated in place */
+    void* q_out;                /* packed stripe receiving the requantized aggregate; may be stripes[owner] */
+    double* agg_out;            /* optional (may be NULL) */
+    size_t rows;                /* at most cntkq_stripe_reduce_max_rows_f64(nbits) */
+    size_t stripe_cols;
+} cntkq_stripe_reduce_item_f64;
+
+int cntkq_quantize_batch_async_f64(cntkq_quantizer* h, const cntkq_quantize_item_f64* items, size_t count, size_t nbits,
+                                   int zero_threshold_for_1bit);
+int cntkq_unquantize_batch_async_f64(cntkq_quantizer* h, const cntkq_unquantize_item_f64* items, size_t count, size_t nbits, int add);
+int cntkq_stripe_reduce_batch_async_f64(cntkq_quantizer* h, const cntkq_stripe_reduce_item_f64* items, size_t count, size_t workers,
+                                        size_t owner, size_t nbits, int zero_threshold_for_1bit);
+
 #ifdef __cplusplus
 }
 #endif

@@ -368,6 +368,63 @@ static void BufferedAggregation()
     idle.WaitForPendingAggregation();
 }
 
+// The double instantiation (the reference's end-to-end 1-bit tests run in double precision): the reference's arrangement
+// of calls against fused stripe reduction + batched calls, bit for bit, over carried steps. Heights stay below 4992 rows,
+// up to where the fused double stripe reduction shares its summation order with the call sequence's quantize kernel.
+static void DoublePrecisionVariantsAreBitIdentical()
+{
+    const Shapes shapes = {{2048, 12}, {429, 17}, {64, 5}, {1, 9}, {4096, 4}, {147, 3}};
+    const size_t K = 3;
+    for (int nBits : {1, 8})
+    {
+        std::vector<std::vector<std::vector<double>>> results[2]; // [arrangement][step][matrix] of worker 0
+        for (int arrangement = 0; arrangement < 2; ++arrangement)
+        {
+            InProcessCluster<double>::Options opt;
+            opt.useFusedStripeReduce = arrangement == 1;
+            opt.useBatchedCalls = arrangement == 1;
+            InProcessCluster<double> cluster(K, 0, nBits, false, true, arrangement == 1, opt);
+            for (int step = 0; step < 3; ++step)
+            {
+                std::vector<std::vector<std::unique_ptr<Matrix<double>>>> owned(K);
+                std::vector<std::vector<Matrix<double>*>> grads(K);
+                std::vector<DistGradHeader> headers;
+                for (size_t r = 0; r < K; ++r)
+                {
+                    for (size_t i = 0; i < shapes.size(); ++i)
+                    {
+                        const std::vector<float> f = Gaussian(shapes[i].first * shapes[i].second, 0.01f, 777 + 1000 * step + 10 * r + i);
+                        const std::vector<double> d(f.begin(), f.end());
+                        owned[r].emplace_back(new Matrix<double>(shapes[i].first, shapes[i].second, 0));
+                        owned[r].back()->SetValue(d.data());
+                        grads[r].push_back(owned[r].back().get());
+                    }
+                    headers.emplace_back(1);
+                    headers.back().numSamples = 5 + r;
+                }
+                cluster.AggregateGradients(grads, headers, step == 0, true);
+                detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize");
+                results[arrangement].emplace_back();
+                for (size_t i = 0; i < shapes.size(); ++i)
+                {
+                    auto a = grads[0][i]->CopyToArray();
+                    results[arrangement].back().emplace_back(a.get(), a.get() + grads[0][i]->GetNumElements());
+                    for (size_t r = 1; r < K; ++r)
+                    {
+                        auto b = grads[r][i]->CopyToArray();
+                        CHECK(std::memcmp(a.get(), b.get(), grads[0][i]->GetNumElements() * sizeof(double)) == 0,
+                              "double: worker %zu, matrix %zu differs from worker 0", r, i);
+                    }
+                }
+            }
+        }
+        for (size_t step = 0; step < results[0].size(); ++step)
+            for (size_t i = 0; i < shapes.size(); ++i)
+                CHECK(std::memcmp(results[0][step][i].data(), results[1][step][i].data(), results[0][step][i].size() * sizeof(double)) == 0,
+                      "double: bits=%d step=%zu matrix=%zu: fused + batched differs from the reference's arrangement", nBits, step, i);
+    }
+}
+
 int main()
 {
     try
@@ -375,7 +432,8 @@ int main()
         struct T { const char* name; void (*fn)(); };
         const T tests[] = {{"QuantizedAllReduceVariantsBitIdentical", VariantsAreBitIdentical}, {"QuantizedAllReduceAgainstOracle", AgainstOracle},
                            {"QuantizedAllReduceUnquantizedSelfStripe", UnquantizedSelfStripe}, {"QuantizedAllReduceEmptyMinibatchAndReset", EmptyMinibatchAndReset},
-                           {"QuantizedAllReduceBufferedAggregation", BufferedAggregation}};
+                           {"QuantizedAllReduceBufferedAggregation", BufferedAggregation},
+                           {"QuantizedAllReduceDoublePrecision", DoublePrecisionVariantsAreBitIdentical}};
         for (const T& t : tests)
         {
             const int before = g_failures;

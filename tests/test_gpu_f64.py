@@ -369,3 +369,90 @@ def test_end_to_end_allreduce_f64(quantizer):
         worst, ntaint = parity.check_end_to_end(aggs_o, sres, Qagg.to_numpy(), sres_gpu, Out.to_numpy(), qagg_o, out_o, rows, cols,
                                                 nbits, zt, tainted, report=rep)
         say("f64 all-reduce nbits", nbits, "zt", zt, "worst", worst, "tainted columns", ntaint, rep)
+
+
+# ---- the batched calls on doubles ---------------------------------------------------------------------------------------
+
+MIXED64 = [(147, 64), (64, 64), (576, 33), (1, 5), (5, 1), (429, 37), (2048, 33), (2304, 5), (4608, 3), (0, 4), (1000, 1), (1152, 40),
+           (4096, 6), (5120, 3), (7168, 2), (8000, 2), (20001, 2), (512, 100), (33, 67)]
+
+
+@pytest.mark.parametrize("nbits,zt", [(1, False), (1, True), (4, False), (16, False), (64, False)])
+def test_batch_equals_per_matrix_calls_f64(quantizer, nbits, zt):
+    """One call for a whole set of double matrices (tile members, register-kernel and tall matrices with launches of
+    their own, an empty one) gives the bytes of one call per matrix; the oracle checks the result as well."""
+    qz = quantizer
+    gs = [datagen.normal_with_outliers(100 * i + nbits, r, c, dtype=F64) for i, (r, c) in enumerate(MIXED64)]
+    rs = [datagen.normal(300 * i + nbits, r, c, 0.003, dtype=F64) for i, (r, c) in enumerate(MIXED64)]
+    new = lambda: [QuantizedMatrix(r, c, nbits, 0, dtype=torch.float64) for r, c in MIXED64]
+    for step in range(2):
+        say("f64 batch", nbits, zt, "step", step)
+        G = [Matrix.from_numpy(g) for g in gs]
+        R1, Q1, O1 = [Matrix.from_numpy(r) for r in rs], new(), [Matrix.from_numpy(r) for r in rs]
+        for g, r, q in zip(G, R1, Q1):
+            qz.QuantizeAsync(g, r, q, r, zt)
+        for q, o in zip(Q1, O1):
+            qz.UnquantizeAsync(q, o, add=(step == 1))
+        qz.WaitUnquantizeAsyncDone()
+        R2, Q2, O2 = [Matrix.from_numpy(r) for r in rs], new(), [Matrix.from_numpy(r) for r in rs]
+        qz.QuantizeBatchAsync([(g, r, q, r) for g, r, q in zip(G, R2, Q2)], zt)
+        qz.WaitQuantizeAsyncDone()
+        qz.UnquantizeBatchAsync(list(zip(Q2, O2)), add=(step == 1))
+        qz.WaitUnquantizeAsyncDone()
+        torch.cuda.synchronize()
+        for i, (r, c) in enumerate(MIXED64):
+            assert np.array_equal(Q1[i].to_numpy(), Q2[i].to_numpy()), ("packed", MIXED64[i])
+            assert parity.bits_equal(R1[i].to_numpy(), R2[i].to_numpy()), ("residual", MIXED64[i])
+            assert parity.bits_equal(O1[i].to_numpy(), O2[i].to_numpy()), ("output", MIXED64[i])
+            if r and c:
+                parity.check_quantize(gs[i], rs[i], Q2[i].to_numpy(), R2[i].to_numpy(), nbits, zt)
+        rs = [m.to_numpy() for m in R2]
+    with pytest.raises(cntk_amd.QuantizerLogicError):  # element types may not be mixed within a call
+        qz.QuantizeBatchAsync([(G[0], R2[0], Q2[0], R2[0]), (Matrix(4, 4), Matrix(4, 4), QuantizedMatrix(4, 4, nbits if nbits <= 32 else 32, 0),
+                                                             Matrix(4, 4))], zt)
+
+
+STRIPE_SETS64 = [(147, 8), (64, 16), (576, 9), (1, 5), (429, 7), (2048, 12), (4608, 3), (1000, 4), (4096, 6), (7168, 2), (0, 3), (33, 9)]
+
+
+@pytest.mark.parametrize("nbits,zt,k", [(1, False, 8), (1, True, 3), (4, False, 4), (64, False, 2)])
+def test_stripe_batch_equals_per_matrix_calls_f64(quantizer, nbits, zt, k):
+    qz = quantizer
+    owner = k // 2
+    packed = [[oracle.quantize(datagen.normal(50 * i + 7 * w + nbits, r, c, dtype=F64), zeros(r, c), nbits, zt, threads=8)[0] if r and c
+               else np.zeros(0, np.uint8) for w in range(k)] for i, (r, c) in enumerate(STRIPE_SETS64)]
+    sres = [datagen.normal(900 + i, r, c, 0.003, dtype=F64) for i, (r, c) in enumerate(STRIPE_SETS64)]
+
+    def device_state():
+        Qs = []
+        for i, (r, c) in enumerate(STRIPE_SETS64):
+            row = []
+            for w in range(k):
+                Q = QuantizedMatrix(r, c, nbits, 0, dtype=torch.float64)
+                if r and c:
+                    Q.from_numpy(packed[i][w])
+                row.append(Q)
+            Qs.append(row)
+        return Qs, [Matrix.from_numpy(s) for s in sres], [Matrix(r, c, dtype=torch.float64) for r, c in STRIPE_SETS64]
+
+    Q1, S1, A1 = device_state()
+    for i in range(len(STRIPE_SETS64)):
+        if STRIPE_SETS64[i][0]:
+            qz.StripeReduceAsync(Q1[i], owner, S1[i], Q1[i][owner], zt, agg_out=A1[i])
+    qz.WaitStripeReduceDone()
+    Q2, S2, A2 = device_state()
+    for rep in range(2):  # the second call finds the cached table
+        if rep == 1:
+            for i, (r, c) in enumerate(STRIPE_SETS64):
+                S2[i].data.copy_(Matrix.from_numpy(sres[i]).data)
+                if r and c:
+                    Q2[i][owner].from_numpy(packed[i][owner])
+        qz.StripeReduceBatchAsync([(Q2[i], S2[i], Q2[i][owner], A2[i]) for i in range(len(STRIPE_SETS64))], owner, zt)
+        qz.WaitStripeReduceDone()
+        torch.cuda.synchronize()
+        for i, (r, c) in enumerate(STRIPE_SETS64):
+            if r == 0:
+                continue
+            assert np.array_equal(Q1[i][owner].to_numpy(), Q2[i][owner].to_numpy()), ("packed", STRIPE_SETS64[i])
+            assert parity.bits_equal(S1[i].to_numpy(), S2[i].to_numpy()), ("stripe residual", STRIPE_SETS64[i])
+            assert parity.bits_equal(A1[i].to_numpy(), A2[i].to_numpy()), ("aggregate", STRIPE_SETS64[i])
