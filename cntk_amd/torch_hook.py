@@ -35,6 +35,26 @@ def matrix_view(t):
     return Matrix(t.numel() // max(cols, 1), cols, t.device.index, t.detach().view(-1))
 
 
+def stripe_layout(shapes, world_size, nbits):
+    """Where every packed stripe sits in a per-worker slot of the exchange buffers.
+
+    shapes: (rows, cols, torch dtype) per gradient matrix. Returns (stripes, rel, slot): stripes[s][i] = (first column,
+    columns) of matrix i that worker s owns (GetStripeForNode, Source/1BitSGD/AllReduceDistGradAggregator.h:56-65);
+    rel[s][i] = byte offset of that packed stripe inside worker s's slot, 8-byte aligned (a packed column of doubles
+    starts with two doubles); slot = bytes per slot, the largest worker's need, the same for all so that one size serves
+    the all-to-all and the all-gather."""
+    stripes = [[stripe_range(cols, s, world_size) for (_, cols, _) in shapes] for s in range(world_size)]
+    rel, need = [], []
+    for s in range(world_size):
+        off, row = 0, []
+        for i, (rows, _, dt) in enumerate(shapes):
+            row.append(off)
+            off += (stripes[s][i][1] * qcol_bytes(nbits, rows, dt) + 7) // 8 * 8
+        rel.append(row)
+        need.append(off)
+    return stripes, rel, max(max(need), 8)
+
+
 class LocalTransport:
     """One worker: nothing changes hands (the aggregator never calls a transport of one worker)."""
     rank, world_size = 0, 1
@@ -98,20 +118,7 @@ class QuantizedGradientAggregator:
         for g in grads:
             m = matrix_view(g)
             shapes.append((m.rows, m.cols, g.dtype, qcol_bytes(self.nbits, m.rows, g.dtype)))
-        # send buffer: for every destination, its stripe of every gradient; offsets are kept 8-byte aligned (the
-        # packed column of a double matrix starts with two doubles)
-        self._send_off = [[0] * len(grads) for _ in range(W)]
-        self._stripe = [[stripe_range(cols, s, W) for (_, cols, _, _) in shapes] for s in range(W)]
-        splits, off = [], 0
-        for s in range(W):
-            begin = off
-            for i, (rows, cols, dt, qcol) in enumerate(shapes):
-                self._send_off[s][i] = off
-                off += (self._stripe[s][i][1] * qcol + 7) // 8 * 8
-            splits.append(off - begin)
-        # equal-sized slots (the largest destination's) keep every slot's start aligned and let the gather use one size
-        self._slot = max(max(splits), 8)
-        self._rel = [[self._send_off[s][i] - self._send_off[s][0] for i in range(len(grads))] for s in range(W)]
+        self._stripe, self._rel, self._slot = stripe_layout([(r, c, dt) for (r, c, dt, _) in shapes], W, self.nbits)
         u8 = dict(dtype=torch.uint8, device=dev)
         self._send = torch.zeros(W * self._slot, **u8)
         self._recv = torch.zeros(W * self._slot, **u8) if W > 1 else None
