@@ -105,18 +105,19 @@ int main(int argc, char** argv)
             std::printf("K=%zu %s (%zu matrices, %zu parameters) nbits=%d: algorithmic bytes per step %.1f MB\n", K, what.c_str(),
                         shapes.size(), params, nbits, bytes / 1e6);
 
-        struct Arrangement { const char* name; bool fused, batched, allWorkers; };
+        struct Arrangement { const char* name; bool fused, batched, allWorkers, dedicatedStream; };
         const Arrangement arrangements[] = {
-            {"fused stripe reduction, unquantize on worker 0", true, true, false},
-            {"fused stripe reduction, unquantize on all workers", true, true, true},
-            {"reference call sequence (unfused), unquantize on worker 0", false, false, false},
+            {"fused stripe reduction, unquantize on worker 0", true, true, false, true},
+            {"the same on the main stream (no hand-over event)", true, true, false, false},
+            {"fused stripe reduction, unquantize on all workers", true, true, true, true},
+            {"reference call sequence (unfused), unquantize on worker 0", false, false, false, true},
         };
         for (const Arrangement& a : arrangements)
         {
             InProcessCluster<float>::Options opt;
             opt.useFusedStripeReduce = a.fused;
             opt.useBatchedCalls = a.batched;
-            InProcessCluster<float> cluster(K, 0, nbits, false, true, true, opt);
+            InProcessCluster<float> cluster(K, 0, nbits, false, true, a.dedicatedStream, opt);
             std::vector<std::vector<Matrix<float>*>> grads(K);
             std::vector<DistGradHeader> headers;
             for (size_t r = 0; r < K; ++r)
