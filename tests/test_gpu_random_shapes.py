@@ -91,8 +91,8 @@ def test_random_shapes(dtype, seed, count):
     say("  ", rep)
 
 
-@pytest.mark.parametrize("seed,count", [(21, 60), (22, 60)])
-def test_random_stripe_reductions(seed, count):
+@pytest.mark.parametrize("seed,count,tall", [(21, 60, False), (22, 60, False), (23, 40, True)])
+def test_random_stripe_reductions(seed, count, tall):
     """Random stripes through the fused reduction: the fp32 aggregate bit-exact against the oracle (owner first, then
     ascending rank), the requantized stripe like any quantize result, and the bytes of the reference's call sequence
     (unquantize own stripe, add the others, quantize the aggregate) on the same handle."""
@@ -103,11 +103,20 @@ def test_random_stripe_reductions(seed, count):
     rep = parity.Report()
     heights = [h for h in BOUNDARIES if h <= 14336]
     for n in range(count):
-        rows = int(rng.choice(heights)) if rng.random() < 0.6 else int(rng.integers(1, 3600)) * 4
-        rows = max(1, min(14336, rows + int(rng.choice([0, 0, 0, -1, 1]))))
-        k = int(rng.choice([1, 2, 3, 5, 8, 8, 13, 64]))
-        cols = int(rng.integers(1, max(2, min(48, 120000 // rows)) + 1))
         nbits = int(rng.choice([1, 1, 1, 2, 4, 8, 16, 32]))
+        if tall:
+            # above the LDS kernels' heights: the register kernel of the stripe reduction, up to its limit per bit width
+            nbits = int(rng.choice([1, 1, 2, 4, 8, 16]))
+            limit = {1: 102368, 2: 102368, 4: 65336, 8: 32668, 16: 16334}[nbits]
+            rows = int(rng.choice([14337, 14340, 16334, 20000, 32668, 50257, 65536, 102368, int(rng.integers(14337, 102369))]))
+            rows = max(14337, min(limit, rows + int(rng.choice([0, 0, -1, 1, 2]))))
+            k = int(rng.choice([1, 2, 3, 5, 8]))
+            cols = int(rng.integers(1, max(2, min(8, 240000 // rows)) + 1))
+        else:
+            rows = int(rng.choice(heights)) if rng.random() < 0.6 else int(rng.integers(1, 3600)) * 4
+            rows = max(1, min(14336, rows + int(rng.choice([0, 0, 0, -1, 1]))))
+            k = int(rng.choice([1, 2, 3, 5, 8, 8, 13, 64]))
+            cols = int(rng.integers(1, max(2, min(48, 120000 // rows)) + 1))
         zt = bool(rng.integers(0, 2)) and nbits == 1
         owner = int(rng.integers(0, k))
         start, ncols = oracle.stripe_range(cols, owner, k)

@@ -115,6 +115,7 @@ def test_stripe_reduce_height_limit():
     L.cntkq_stripe_reduce_max_rows.argtypes = [ctypes.c_size_t]
     assert L.cntkq_stripe_reduce_max_rows(1) == 102368 and L.cntkq_stripe_reduce_max_rows(32) == 14336
     assert L.cntkq_stripe_reduce_max_rows(16) == 16334 and L.cntkq_stripe_reduce_max_rows(8) == 32668 and L.cntkq_stripe_reduce_max_rows(3) == 0
+    assert L.cntkq_stripe_reduce_max_rows(4) == 65336 and L.cntkq_stripe_reduce_max_rows(2) == 102368
     qz = MatrixQuantizerImpl.Create(0, False)
     rows, cols, k = 16336, 2, 2
     zeros = np.zeros((rows, cols), np.float32, order="F")
