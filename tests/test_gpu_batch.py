@@ -145,7 +145,8 @@ def test_batch_argument_checks():
 
 
 @pytest.mark.filterwarnings("ignore:The CUDA Graph is empty")  # the refused capture below leaves one
-def test_batched_calls_and_hip_graphs():
+@pytest.mark.parametrize("tdt", [torch.float32, torch.float64], ids=["f32", "f64"])
+def test_batched_calls_and_hip_graphs(tdt):
     """A batched call recorded into a graph: refused for an item list the handle has not seen (its table would have to
     be built during the capture); once recorded, the table is frozen, so the graph still gives the right bytes after the
     same handle has served other lists in between."""
@@ -154,8 +155,8 @@ def test_batched_calls_and_hip_graphs():
     gen.manual_seed(datagen.case_seed(81))
 
     def make(shapes):
-        return [(Matrix(r, c, 0, torch.randn(r * c, generator=gen, device="cuda:0") * 0.01), Matrix(r, c), QuantizedMatrix(r, c, 1, 0),
-                 Matrix(r, c)) for r, c in shapes]
+        return [(Matrix(r, c, 0, (torch.randn(r * c, generator=gen, device="cuda:0") * 0.01).to(tdt)), Matrix(r, c, dtype=tdt),
+                 QuantizedMatrix(r, c, 1, 0, dtype=tdt), Matrix(r, c, dtype=tdt)) for r, c in shapes]
 
     first = make([(429, 64), (2048, 32), (64, 64)])
     other = make([(147, 64), (1024, 16)])
@@ -187,7 +188,7 @@ def test_batched_calls_and_hip_graphs():
     qz.WaitUnquantizeAsyncDone()
     torch.cuda.synchronize()
     for step in range(3):
-        gs = [torch.randn(g.rows * g.cols, generator=gen, device="cuda:0") * 0.01 for g, _, _, _ in first]
+        gs = [(torch.randn(g.rows * g.cols, generator=gen, device="cuda:0") * 0.01).to(tdt) for g, _, _, _ in first]
         r_in = [r.to_numpy() for _, r, _, _ in first]
         for (g, _, _, _), x in zip(first, gs):
             g.data.copy_(x)
