@@ -96,8 +96,8 @@ def cpu_baseline(budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)  # 53 ms of GPU time
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--zero-threshold", type=int, default=0, help="zeroThresholdFor1Bit (default off, as in config 1)")
     ap.add_argument("--sets", type=int, default=6, help="rotating buffer sets (each 231 MB)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
