@@ -55,7 +55,7 @@ def test_cpp_allreduce_timing_program_runs():
     assert os.path.exists(exe), "build it first: python -m cntk_amd.build"
     res = subprocess.run([exe, "4", "2048", "256", "1", "3"], capture_output=True, text=True, timeout=300)
     print(res.stdout, res.stderr[-2000:])
-    assert res.returncode == 0 and res.stdout.count("GB/s") == 3
+    assert res.returncode == 0 and res.stdout.count("GB/s") == 4  # one line per arrangement
 
 
 def test_cpp_mirror_header_is_self_contained():
