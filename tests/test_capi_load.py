@@ -62,3 +62,20 @@ def test_bad_arguments_are_reported_not_crashed():
     assert L.cntkq_quantize_async(None, None, None, 1, 1, None, 0, 0, 1, None, 0) == 1
     with pytest.raises(cntk_amd.QuantizerLogicError):
         cntk_amd.QuantizedMatrix(8, 8, 3, cntk_amd.CPUDEVICE)
+
+
+def test_public_header_is_plain_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 (no C++ types or keywords), warnings included."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc on this machine")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "cntk_amd_quantizer.h"\n'
+                   "int main(void) { cntkq_quantize_item a; cntkq_stripe_reduce_item_f64 b; (void) a; (void) b;\n"
+                   "    return cntkq_qcol_bytes(1, 2048) == 264 ? 0 : 1; }\n")
+    res = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", str(src),
+                          "-o", str(tmp_path / "use_header.o")], capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
