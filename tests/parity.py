@@ -242,6 +242,14 @@ def check_end_to_end(aggs_or, sres_in, qagg_gpu, sres_gpu, out_gpu, qagg_or, out
     # elements whose final code differs sit a whole level apart; the check above has vetted each of them
     same = oracle.codes(qagg_gpu, rows, cols, nbits, dtype=dt) == oracle.codes(qagg_or, rows, cols, nbits, dtype=dt)
     err = np.where(same, np.abs(out_gpu.astype(np.float64) - out_or) / scale[None, :], 0.0)
+    allow = np.full(cols, tolerances(dt)[2])
+    if rows > 16384:
+        # long columns: the oracle's own sequential sums move its bounds (see the module text); a value reconstructed
+        # from equal codes moves with the bounds, which check_quantize above has vetted against the float64 statistics
+        lo_g, hi_g = oracle.headers(qagg_gpu, rows, cols, nbits, dtype=dt)
+        moved = np.maximum(np.abs(lo_g.astype(np.float64) - lo), np.abs(hi_g.astype(np.float64) - hi)) / scale
+        allow = np.maximum(allow, 1.5 * moved)
+    over = err - allow[None, :]
     worst = float(err[:, clean].max(initial=0.0))
-    assert worst <= tolerances(dt)[2], "aggregated gradient off by %.3g of the column scale" % worst
+    assert float(over[:, clean].max(initial=-1.0)) <= 0.0, "aggregated gradient off by %.3g of the column scale" % worst
     return worst, int(tainted_cols.sum())

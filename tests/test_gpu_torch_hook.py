@@ -49,7 +49,9 @@ SHAPES = [((96, 300), torch.float32),       # Linear weight: 96 columns of 300 r
           ((40, 16, 3, 3), torch.float32),  # convolution: 40 columns of 144 rows
           ((96,), torch.float32),           # bias: one column
           ((3, 2048), torch.float32),       # fewer columns than workers: some stripes are empty
-          ((24, 130), torch.float64)]
+          ((24, 130), torch.float64),
+          ((2, 110000), torch.float32),     # columns too tall for the fused stripe reduction: the reference's call sequence
+          ((3, 9000), torch.float64)]       # the same for doubles (limit 7168 rows)
 
 
 @pytest.mark.parametrize("K,nbits,zt", [(1, 1, True), (4, 1, False), (4, 1, True), (3, 4, False), (8, 2, False)])
@@ -97,7 +99,7 @@ def test_in_process_workers_against_the_oracle(K, nbits, zt):
             _, aggs_o, qagg_o, out_o = parity.oracle_allreduce_staged([gs[w][i] for w in range(K)], ro, so, nbits, zt, threads=8)
             tainted = np.zeros(cols, dtype=bool)
             for w in range(K):
-                parity.check_quantize(gs[w][i], res_in[w][i], q1[w][i], res_out[w][i], nbits, zt, threads=8, report=rep, strict=True)
+                parity.check_quantize(gs[w][i], res_in[w][i], q1[w][i], res_out[w][i], nbits, zt, threads=8, report=rep, strict=rows <= 16384)
                 tainted |= rep.last_mismatch_cols
             for s in range(K):
                 start, n = oracle.stripe_range(cols, s, K)
@@ -107,12 +109,13 @@ def test_in_process_workers_against_the_oracle(K, nbits, zt):
                 s_copy = sres_in[s][i].copy(order="F")
                 agg = oracle.stripe_reduce(q_copy, s, rows, cols, nbits, s_copy, zt, threads=8)
                 parity.check_quantize(agg, sres_in[s][i], qagg_g[start * qcol:(start + n) * qcol], sres_out[s], nbits, zt,
-                                      threads=8, report=rep, strict=True)
+                                      threads=8, report=rep, strict=rows <= 16384)
                 tainted[start:start + n] |= rep.last_mismatch_cols
             parity.check_unquantize(qagg_g, rows, cols, nbits, outs[0], threads=8)
             parity.check_end_to_end(aggs_o, [sres_in[s][i] for s in range(K)], qagg_g, sres_out, outs[0], qagg_o, out_o, rows, cols,
                                     nbits, zt, tainted, threads=8, report=rep)
-            assert tainted.sum() <= max(1, cols // 50)
+            if rows <= 16384:  # (a column of 100000 elements is likelier than not to hold one element at a threshold)
+                assert tainted.sum() <= max(1, cols // 50)
     say("torch hook K=%d nbits=%d:" % (K, nbits), rep)
 
 
