@@ -496,6 +496,8 @@ int stripe_reduce_async_impl(cntkq_quantizer* h, const void* const* stripes, siz
     return CNTKQ_OK;
 }
 
+#include "quantizer_api_batch.inc"
+
 } // namespace
 
 extern "C" {
@@ -732,278 +734,12 @@ int cntkq_wait_unquantize_done(cntkq_quantizer* h)
 int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* items, size_t count, size_t nbits,
                                int zero_threshold_for_1bit)
 {
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: null handle");
-    if (!valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
-    if (count == 0)
-        return CNTKQ_OK;
-    if (items == nullptr || count > 0xFFFFFF)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: bad item list");
-    for (size_t i = 0; i < count; ++i)
-    {
-        const cntkq_quantize_item& it = items[i];
-        if (it.rows >= (1ull << 31) || it.cols >= (1ull << 31))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: item %zu: rows and cols must be below 2^31", i);
-        if (it.rows == 0 || it.cols == 0)
-            continue;
-        if (it.in == nullptr || it.res_in == nullptr || it.res_out == nullptr || it.qbuf == nullptr || !aligned4(it.in) ||
-            !aligned4(it.res_in) || !aligned4(it.res_out) || !aligned4(it.qbuf))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: item %zu: null or misaligned pointer", i);
-    }
-    const bool zt = zero_threshold_for_1bit != 0;
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    BatchTable& tb = h->quantize_table;
-    const size_t params[3] = {count, nbits, (size_t) (zt ? 1 : 0)};
-    const size_t items_bytes = count * sizeof(cntkq_quantize_item);
-
-    const bool capturing = stream_capturing(s);
-    if (capturing && !table_matches(tb, items, items_bytes, params))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: the stream is being captured into a graph and this item list "
-                                            "has not been seen: call once outside the capture first (the argument table is built and uploaded then)");
-    if (!table_matches(tb, items, items_bytes, params))
-    {
-        // Every matrix is a member of one of two grid-wide launches (small / large LDS need), as a run of column
-        // tiles or of single columns; only columns too tall for LDS get a launch of their own. Large matrices gain
-        // from sharing a grid too: their workgroups fill the gaps the others leave.
-        constexpr size_t kSmallLds = 20 * 1024;
-        constexpr size_t kOwnLaunchElements = (size_t) 8 << 20;
-        struct Plan
-        {
-            int kind; // -1 skip, 0 tiles in a batch, 1 columns in a batch, 2 own launch
-            int cls;  // LDS class of a batch member
-            size_t lds;
-            uint64_t blocks;
-            TileGeom t;
-            ColGeom c;
-        };
-        std::vector<Plan> plans(count);
-        size_t members[2] = {0, 0};
-        for (size_t i = 0; i < count; ++i)
-        {
-            const cntkq_quantize_item& it = items[i];
-            Plan& p = plans[i];
-            std::memset(&p, 0, sizeof p);
-            p.kind = -1;
-            if (it.rows == 0 || it.cols == 0)
-                continue;
-            const int path = quantize_auto_path(it.in, it.res_in, it.res_out, it.qbuf, it.rows, nbits);
-            if (path == kPathTile)
-            {
-                p.kind = 0;
-                p.t = make_tile_geom(it.rows, it.cols, nbits, 0, -1, 0);
-                p.lds = tile_lds_bytes(p.t, 0);
-                p.blocks = (p.t.cols + p.t.cols_per_tile - 1) / p.t.cols_per_tile;
-            }
-            else if (path == kPathCol || (path == kPathReg && it.rows <= kTileMaxRows && it.rows * it.cols < kOwnLaunchElements))
-            {
-                // (a register-kernel matrix of modest size gives the same bytes as a member: a launch costs more than it gains)
-                p.kind = 1;
-                p.c = make_col_geom(it.rows, nbits, quantize_line_shift(it.in, it.res_in, it.res_out, it.rows));
-                p.lds = colg_lds_bytes_rt(p.c, nbits);
-                p.blocks = it.cols;
-            }
-            else
-            {
-                p.kind = 2;
-                continue;
-            }
-            p.cls = p.lds <= kSmallLds ? 0 : 1;
-            members[p.cls]++;
-        }
-        if (members[0] + members[1] == 1)
-        {
-            // a grid of its own is nothing to share: the plain launch picks the best kernel for the matrix
-            for (size_t i = 0; i < count; ++i)
-                if (plans[i].kind == 0 || plans[i].kind == 1)
-                    plans[i].kind = 2;
-            members[0] = members[1] = 0;
-        }
-        const size_t total = members[0] + members[1];
-        const size_t entries_bytes = total * sizeof(QuantizeBatchEntry);
-        int rc = table_begin_rebuild(tb, entries_bytes + (total + 2) * sizeof(uint32_t) + 64);
-        if (rc != CNTKQ_OK)
-            return rc;
-        QuantizeBatchEntry* he = reinterpret_cast<QuantizeBatchEntry*>(tb.host);
-        uint32_t* hb = reinterpret_cast<uint32_t*>(tb.host + entries_bytes);
-        size_t e = 0, bpos = 0;
-        tb.own.clear();
-        for (int cls = 0; cls < 2; ++cls)
-        {
-            tb.first_entry[cls] = e;
-            tb.first_begin[cls] = bpos;
-            tb.lds[cls] = 0;
-            uint64_t acc = 0;
-            for (size_t i = 0; i < count; ++i)
-            {
-                const Plan& p = plans[i];
-                if ((p.kind != 0 && p.kind != 1) || p.cls != cls)
-                    continue;
-                he[e].g = items[i].in;
-                he[e].r_in = items[i].res_in;
-                he[e].r_out = items[i].res_out;
-                he[e].q = static_cast<char*>(items[i].qbuf);
-                he[e].kind = (uint32_t) p.kind;
-                he[e].pad = 0;
-                he[e].t = p.t;
-                he[e].c = p.c;
-                hb[bpos++] = (uint32_t) acc;
-                acc += p.blocks;
-                if (acc > 0x7FFFFFFFull)
-                    return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async: too many workgroups in one batch");
-                if (p.lds > tb.lds[cls])
-                    tb.lds[cls] = p.lds;
-                e++;
-            }
-            if (members[cls] != 0)
-                hb[bpos++] = (uint32_t) acc; // sentinel
-            tb.members[cls] = members[cls];
-            tb.blocks[cls] = (uint32_t) acc;
-        }
-        for (size_t i = 0; i < count; ++i)
-            if (plans[i].kind == 2)
-                tb.own.push_back(i);
-        tb.entries_bytes = entries_bytes;
-        if (total != 0)
-            HIP_TRY(hipMemcpyAsync(tb.dev, tb.host, entries_bytes + bpos * sizeof(uint32_t), hipMemcpyHostToDevice, s),
-                    "hipMemcpyAsync of the batch table failed");
-        table_set_key(tb, items, items_bytes, params);
-    }
-
-    size_t launches_left = (tb.members[0] ? 1 : 0) + (tb.members[1] ? 1 : 0) + tb.own.size();
-    if (launches_left == 0)
-        return CNTKQ_OK;
-    // the last kernel of the call carries the table's event: the kernels before it run on the same stream
-    // (none when the call is recorded into a graph: there is nothing to wait for, and the table is frozen instead)
-    hipEvent_t done = capturing ? nullptr : tb.event;
-    if (capturing)
-        tb.captured = true;
-    for (int cls = 0; cls < 2; ++cls)
-    {
-        if (tb.members[cls] == 0)
-            continue;
-        LaunchEvents ev;
-        launches_left--;
-        ev.stop = launches_left == 0 ? done : nullptr;
-        const QuantizeBatchEntry* de = reinterpret_cast<const QuantizeBatchEntry*>(tb.dev) + tb.first_entry[cls];
-        const uint32_t* db = reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes) + tb.first_begin[cls];
-        HIP_TRY(launch_quantize_batch(s, ev, de, db, (uint32_t) tb.members[cls], tb.blocks[cls], tb.lds[cls], nbits, zt),
-                "batched quantize kernel launch failed");
-        tb.in_flight = tb.in_flight || !capturing;
-    }
-    LaunchTuning autotune;
-    for (size_t i : tb.own)
-    {
-        const cntkq_quantize_item& it = items[i];
-        LaunchEvents ev;
-        launches_left--;
-        ev.stop = launches_left == 0 ? done : nullptr;
-        HIP_TRY(launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune),
-                "quantize kernel launch failed");
-        tb.in_flight = tb.in_flight || !capturing;
-    }
-    h->last_quantize = done;
-    h->quantize_included_fetch = false;
-    return CNTKQ_OK;
+    return quantize_batch_impl<float>(h, items, count, nbits, zero_threshold_for_1bit);
 }
 
 int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item* items, size_t count, size_t nbits, int add)
 {
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: null handle");
-    if (!valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
-    if (count == 0)
-        return CNTKQ_OK;
-    if (items == nullptr || count > 0xFFFFFF)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: bad item list");
-    size_t n = 0;
-    for (size_t i = 0; i < count; ++i)
-    {
-        const cntkq_unquantize_item& it = items[i];
-        if (it.rows >= (1ull << 31) || it.cols >= (1ull << 31))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: item %zu: rows and cols must be below 2^31", i);
-        if (it.rows == 0 || it.cols == 0)
-            continue;
-        if (it.qbuf == nullptr || it.out == nullptr || !aligned4(it.qbuf) || !aligned4(it.out))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: item %zu: null or misaligned pointer", i);
-        n++;
-    }
-    if (n == 0)
-        return CNTKQ_OK;
-    if (n == 1)
-    {
-        for (size_t i = 0; i < count; ++i)
-            if (items[i].rows != 0 && items[i].cols != 0)
-                return cntkq_unquantize_async(h, items[i].qbuf, qcol_bytes(nbits, items[i].rows) * items[i].cols, 0, items[i].out,
-                                              items[i].rows, items[i].cols, nbits, add);
-    }
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    BatchTable& tb = h->unquantize_table;
-    const size_t params[3] = {count, nbits, 0};
-    const size_t items_bytes = count * sizeof(cntkq_unquantize_item);
-    const bool capturing = stream_capturing(s);
-    if (capturing && !table_matches(tb, items, items_bytes, params))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: the stream is being captured into a graph and this item "
-                                            "list has not been seen: call once outside the capture first");
-    if (!table_matches(tb, items, items_bytes, params))
-    {
-        const size_t entries_bytes = n * sizeof(UnquantizeBatchEntry);
-        int rc = table_begin_rebuild(tb, entries_bytes + (n + 1) * sizeof(uint32_t) + 64);
-        if (rc != CNTKQ_OK)
-            return rc;
-        UnquantizeBatchEntry* he = reinterpret_cast<UnquantizeBatchEntry*>(tb.host);
-        uint32_t* hb = reinterpret_cast<uint32_t*>(tb.host + entries_bytes);
-        tb.lds[0] = 0;
-        LaunchTuning autotune;
-        uint64_t blocks = 0;
-        size_t e = 0;
-        for (size_t i = 0; i < count; ++i)
-        {
-            const cntkq_unquantize_item& it = items[i];
-            if (it.rows == 0 || it.cols == 0)
-                continue;
-            const UnquantizePlan p = plan_unquantize(it.qbuf, it.out, it.rows, it.cols, nbits, autotune);
-            if (!p.ok)
-                return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: item %zu is too large", i);
-            he[e].q = static_cast<const char*>(it.qbuf);
-            he[e].out = it.out;
-            he[e].kind = p.kind;
-            he[e].pad = 0;
-            he[e].qw = p.qw;
-            he[e].seg = p.seg;
-            he[e].rowg = p.rowg;
-            he[e].tile = p.tile;
-            if (p.lds > tb.lds[0])
-                tb.lds[0] = p.lds;
-            hb[e] = (uint32_t) blocks;
-            blocks += p.blocks;
-            if (blocks > 0x7FFFFFFFull)
-                return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async: too much work in one batch");
-            e++;
-        }
-        hb[e] = (uint32_t) blocks;
-        tb.members[0] = n;
-        tb.blocks[0] = (uint32_t) blocks;
-        tb.entries_bytes = entries_bytes;
-        HIP_TRY(hipMemcpyAsync(tb.dev, tb.host, entries_bytes + (n + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, s),
-                "hipMemcpyAsync of the batch table failed");
-        table_set_key(tb, items, items_bytes, params);
-    }
-    LaunchEvents ev;
-    ev.stop = capturing ? nullptr : tb.event;
-    HIP_TRY(launch_unquantize_batch(s, ev, reinterpret_cast<const UnquantizeBatchEntry*>(tb.dev),
-                                    reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes), (uint32_t) tb.members[0], tb.blocks[0],
-                                    nbits, add != 0, tb.lds[0]),
-            "batched unquantize kernel launch failed");
-    if (capturing)
-        tb.captured = true;
-    else
-        tb.in_flight = true;
-    h->last_unquantize = ev.stop;
-    return CNTKQ_OK;
+    return unquantize_batch_impl<float>(h, items, count, nbits, add);
 }
 
 int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows,
@@ -1025,174 +761,7 @@ int cntkq_stripe_reduce_async_f64(cntkq_quantizer* h, const void* const* stripes
 int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduce_item* items, size_t count, size_t workers,
                                     size_t owner, size_t nbits, int zero_threshold_for_1bit)
 {
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: null handle");
-    if (!valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
-    if (workers == 0 || workers > CNTKQ_MAX_WORKERS || owner >= workers)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: need 1 <= workers <= %d and owner < workers",
-                    CNTKQ_MAX_WORKERS);
-    if (count == 0)
-        return CNTKQ_OK;
-    if (items == nullptr || count > 0xFFFFFF)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: bad item list");
-    size_t n = 0, only = 0, tall = 0;
-    for (size_t i = 0; i < count; ++i)
-    {
-        const cntkq_stripe_reduce_item& it = items[i];
-        if (it.rows >= (1ull << 31) || it.stripe_cols >= (1ull << 31))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: rows and cols must be below 2^31", i);
-        if (it.rows == 0 || it.stripe_cols == 0)
-            continue;
-        if (it.rows > stripe_reduce_max_rows(nbits))
-            return fail(CNTKQ_INVALID_ARGUMENT,
-                        "cntkq_stripe_reduce_batch_async: item %zu: columns taller than %zu rows are not supported at %zu bits", i,
-                        stripe_reduce_max_rows(nbits), nbits);
-        if (it.stripes == nullptr || it.stripe_res == nullptr || it.q_out == nullptr || !aligned4(it.stripe_res) || !aligned4(it.q_out) ||
-            !aligned4(it.agg_out))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: null or misaligned pointer", i);
-        for (size_t w = 0; w < workers; ++w)
-            if (it.stripes[w] == nullptr || !aligned4(it.stripes[w]))
-                return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: item %zu: stripe %zu is null or misaligned", i, w);
-        if (it.rows > kTileMaxRows)
-        {
-            tall++; // a launch of its own, below
-            continue;
-        }
-        only = i;
-        n++;
-    }
-    // tall stripes (1024 threads per column, registers) do not fit the shared grid: each is a plain call on the same stream
-    for (size_t i = 0; i < count && tall != 0; ++i)
-    {
-        const cntkq_stripe_reduce_item& it = items[i];
-        if (it.rows <= kTileMaxRows || it.stripe_cols == 0)
-            continue;
-        const int rc = cntkq_stripe_reduce_async(h, it.stripes, workers, owner, it.rows, it.stripe_cols, nbits, it.stripe_res, it.q_out,
-                                                 it.agg_out, zero_threshold_for_1bit);
-        if (rc != CNTKQ_OK)
-            return rc;
-    }
-    if (n == 0)
-        return CNTKQ_OK;
-    if (n == 1) // a grid of its own is nothing to share: the plain call picks the best kernel for the stripe
-        return cntkq_stripe_reduce_async(h, items[only].stripes, workers, owner, items[only].rows, items[only].stripe_cols, nbits,
-                                         items[only].stripe_res, items[only].q_out, items[only].agg_out, zero_threshold_for_1bit);
-    const bool zt = zero_threshold_for_1bit != 0;
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    BatchTable& tb = h->stripe_table;
-
-    // the key is the item list with the workers' stripe pointers written out
-    const size_t params[3] = {count, nbits | (workers << 8) | (owner << 16), (size_t) (zt ? 1 : 0)};
-    std::vector<size_t> flat;
-    flat.reserve(count * (5 + workers));
-    for (size_t i = 0; i < count; ++i)
-    {
-        const cntkq_stripe_reduce_item& it = items[i];
-        flat.push_back(reinterpret_cast<size_t>(it.stripe_res));
-        flat.push_back(reinterpret_cast<size_t>(it.q_out));
-        flat.push_back(reinterpret_cast<size_t>(it.agg_out));
-        flat.push_back(it.rows);
-        flat.push_back(it.stripe_cols);
-        if (it.rows != 0 && it.stripe_cols != 0)
-            for (size_t w = 0; w < workers; ++w)
-                flat.push_back(reinterpret_cast<size_t>(it.stripes[w]));
-    }
-    const size_t flat_bytes = flat.size() * sizeof(size_t);
-
-    const bool capturing = stream_capturing(s);
-    if (capturing && !table_matches(tb, flat.data(), flat_bytes, params))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: the stream is being captured into a graph and this item "
-                                            "list has not been seen: call once outside the capture first");
-    if (!table_matches(tb, flat.data(), flat_bytes, params))
-    {
-        constexpr size_t kSmallLds = 20 * 1024;
-        const size_t entries_bytes = n * sizeof(StripeBatchEntry);
-        int rc = table_begin_rebuild(tb, entries_bytes + (n + 2) * sizeof(uint32_t) + 64);
-        if (rc != CNTKQ_OK)
-            return rc;
-        StripeBatchEntry* he = reinterpret_cast<StripeBatchEntry*>(tb.host);
-        uint32_t* hb = reinterpret_cast<uint32_t*>(tb.host + entries_bytes);
-        size_t e = 0, bpos = 0;
-        for (int cls = 0; cls < 2; ++cls)
-        {
-            tb.first_entry[cls] = e;
-            tb.first_begin[cls] = bpos;
-            tb.lds[cls] = 0;
-            tb.members[cls] = 0;
-            uint64_t acc = 0;
-            for (size_t i = 0; i < count; ++i)
-            {
-                const cntkq_stripe_reduce_item& it = items[i];
-                if (it.rows == 0 || it.stripe_cols == 0 || it.rows > kTileMaxRows)
-                    continue;
-                // the kernel family the plain call would take, so that both give the same bytes
-                const bool col = stripe_auto_col(it.rows);
-                StripeBatchEntry en;
-                std::memset(&en, 0, sizeof en);
-                size_t lds, blocks;
-                if (col)
-                {
-                    en.kind = 1;
-                    en.c = make_col_geom(it.rows, nbits, !columns_start_on_lines(it.stripe_res, it.rows));
-                    lds = colg_lds_bytes_rt(en.c, nbits) + 2 * workers * sizeof(float);
-                    blocks = it.stripe_cols;
-                }
-                else
-                {
-                    en.kind = 0;
-                    en.t = make_tile_geom(it.rows, it.stripe_cols, nbits, 0, -1, 0);
-                    lds = tile_lds_bytes(en.t, (uint32_t) workers);
-                    blocks = (en.t.cols + en.t.cols_per_tile - 1) / en.t.cols_per_tile;
-                }
-                if ((lds <= kSmallLds ? 0 : 1) != cls)
-                    continue;
-                for (size_t w = 0; w < workers; ++w)
-                    en.src.q[w] = static_cast<const char*>(it.stripes[w]);
-                en.src.workers = (uint32_t) workers;
-                en.src.owner = (uint32_t) owner;
-                en.stripe_res = it.stripe_res;
-                en.q_out = static_cast<char*>(it.q_out);
-                en.agg_out = it.agg_out;
-                he[e] = en;
-                hb[bpos++] = (uint32_t) acc;
-                acc += blocks;
-                if (acc > 0x7FFFFFFFull)
-                    return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async: too many workgroups in one batch");
-                if (lds > tb.lds[cls])
-                    tb.lds[cls] = lds;
-                tb.members[cls]++;
-                e++;
-            }
-            if (tb.members[cls] != 0)
-                hb[bpos++] = (uint32_t) acc; // sentinel
-            tb.blocks[cls] = (uint32_t) acc;
-        }
-        tb.entries_bytes = entries_bytes;
-        HIP_TRY(hipMemcpyAsync(tb.dev, tb.host, entries_bytes + bpos * sizeof(uint32_t), hipMemcpyHostToDevice, s),
-                "hipMemcpyAsync of the batch table failed");
-        table_set_key(tb, flat.data(), flat_bytes, params);
-    }
-    size_t launches_left = (tb.members[0] ? 1 : 0) + (tb.members[1] ? 1 : 0);
-    for (int cls = 0; cls < 2; ++cls)
-    {
-        if (tb.members[cls] == 0)
-            continue;
-        LaunchEvents ev;
-        launches_left--;
-        ev.stop = launches_left == 0 && !capturing ? tb.event : nullptr;
-        const StripeBatchEntry* de = reinterpret_cast<const StripeBatchEntry*>(tb.dev) + tb.first_entry[cls];
-        const uint32_t* db = reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes) + tb.first_begin[cls];
-        HIP_TRY(launch_stripe_reduce_batch(s, ev, de, db, (uint32_t) tb.members[cls], tb.blocks[cls], tb.lds[cls], nbits, zt),
-                "batched stripe reduction kernel launch failed");
-        if (capturing)
-            tb.captured = true;
-        else
-            tb.in_flight = true;
-    }
-    h->last_stripe = capturing ? nullptr : tb.event;
-    return CNTKQ_OK;
+    return stripe_reduce_batch_impl<float>(h, items, count, workers, owner, nbits, zero_threshold_for_1bit);
 }
 
 int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h)
@@ -1203,413 +772,23 @@ int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h)
     return h->last_stripe != nullptr ? sync_event(h->last_stripe) : CNTKQ_OK;
 }
 
-// ---- the batched calls on doubles ----------------------------------------------------------------------------------
-//
-// Same construction as the float calls: members of the quantize and stripe-reduction grids are runs of column tiles
-// (every double matrix the tile kernel serves; the register / tall kernels' matrices get launches of their own), members
-// of the unquantize grid keep their decoder. Two LDS classes per call, tables cached per handle, frozen once captured.
-
-namespace {
-
-bool aligned8(const void* p)
-{
-    return (reinterpret_cast<uintptr_t>(p) & 7u) == 0;
-}
-
-constexpr size_t kSmallLds64 = 20 * 1024;
-
-} // namespace
+// ---- the gradient-set calls on doubles (same implementation, see quantizer_api_batch.inc) ----------------------------
 
 int cntkq_quantize_batch_async_f64(cntkq_quantizer* h, const cntkq_quantize_item_f64* items, size_t count, size_t nbits,
                                    int zero_threshold_for_1bit)
 {
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async_f64: null handle");
-    if (!f64::valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 64 (got %zu)", nbits);
-    if (count == 0)
-        return CNTKQ_OK;
-    if (items == nullptr || count > 0xFFFFFF)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async_f64: bad item list");
-    for (size_t i = 0; i < count; ++i)
-    {
-        const cntkq_quantize_item_f64& it = items[i];
-        if (it.rows >= (1ull << 31) || it.cols >= (1ull << 31))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async_f64: item %zu: rows and cols must be below 2^31", i);
-        if (it.rows == 0 || it.cols == 0)
-            continue;
-        if (it.in == nullptr || it.res_in == nullptr || it.res_out == nullptr || it.qbuf == nullptr || !aligned8(it.in) ||
-            !aligned8(it.res_in) || !aligned8(it.res_out) || !aligned8(it.qbuf))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async_f64: item %zu: null or misaligned pointer", i);
-    }
-    const bool zt = zero_threshold_for_1bit != 0;
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    BatchTable& tb = h->quantize_table64;
-    const size_t params[3] = {count, nbits, (size_t) (zt ? 1 : 0)};
-    const size_t items_bytes = count * sizeof(cntkq_quantize_item_f64);
-    const bool capturing = stream_capturing(s);
-    if (capturing && !table_matches(tb, items, items_bytes, params))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async_f64: the stream is being captured into a graph and this item "
-                                            "list has not been seen: call once outside the capture first");
-    LaunchTuning autotune;
-    if (!table_matches(tb, items, items_bytes, params))
-    {
-        struct Plan
-        {
-            int cls; // -1 skip, 0 / 1 member of that LDS class, 2 own launch
-            size_t lds;
-            uint64_t blocks;
-            f64::TileGeom t;
-        };
-        std::vector<Plan> plans(count);
-        size_t members[2] = {0, 0};
-        for (size_t i = 0; i < count; ++i)
-        {
-            const cntkq_quantize_item_f64& it = items[i];
-            Plan& p = plans[i];
-            std::memset(&p, 0, sizeof p);
-            p.cls = -1;
-            if (it.rows == 0 || it.cols == 0)
-                continue;
-            p.cls = 2;
-            if (f64::quantize_auto_path(it.in, it.res_in, it.res_out, it.rows, nbits) != kPathTile)
-                continue;
-            p.t = f64::make_tile_geom(it.rows, it.cols, nbits, 0);
-            p.lds = f64::tile_lds_bytes(p.t, 0);
-            if (p.lds > f64::kMaxLdsBytes)
-                continue;
-            p.blocks = (p.t.cols + p.t.cols_per_tile - 1) / p.t.cols_per_tile;
-            p.cls = p.lds <= kSmallLds64 ? 0 : 1;
-            members[p.cls]++;
-        }
-        if (members[0] + members[1] == 1)
-        {
-            for (size_t i = 0; i < count; ++i)
-                if (plans[i].cls == 0 || plans[i].cls == 1)
-                    plans[i].cls = 2;
-            members[0] = members[1] = 0;
-        }
-        const size_t total = members[0] + members[1];
-        const size_t entries_bytes = total * sizeof(f64::QuantizeBatchEntry64);
-        int rc = table_begin_rebuild(tb, entries_bytes + (total + 2) * sizeof(uint32_t) + 64);
-        if (rc != CNTKQ_OK)
-            return rc;
-        f64::QuantizeBatchEntry64* he = reinterpret_cast<f64::QuantizeBatchEntry64*>(tb.host);
-        uint32_t* hb = reinterpret_cast<uint32_t*>(tb.host + entries_bytes);
-        size_t e = 0, bpos = 0;
-        tb.own.clear();
-        for (int cls = 0; cls < 2; ++cls)
-        {
-            tb.first_entry[cls] = e;
-            tb.first_begin[cls] = bpos;
-            tb.lds[cls] = 0;
-            uint64_t acc = 0;
-            for (size_t i = 0; i < count; ++i)
-            {
-                const Plan& p = plans[i];
-                if (p.cls != cls)
-                    continue;
-                he[e].g = items[i].in;
-                he[e].r_in = items[i].res_in;
-                he[e].r_out = items[i].res_out;
-                he[e].q = static_cast<char*>(items[i].qbuf);
-                he[e].t = p.t;
-                hb[bpos++] = (uint32_t) acc;
-                acc += p.blocks;
-                if (acc > 0x7FFFFFFFull)
-                    return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_async_f64: too many workgroups in one batch");
-                if (p.lds > tb.lds[cls])
-                    tb.lds[cls] = p.lds;
-                e++;
-            }
-            if (members[cls] != 0)
-                hb[bpos++] = (uint32_t) acc; // sentinel
-            tb.members[cls] = members[cls];
-            tb.blocks[cls] = (uint32_t) acc;
-        }
-        for (size_t i = 0; i < count; ++i)
-            if (plans[i].cls == 2)
-                tb.own.push_back(i);
-        tb.entries_bytes = entries_bytes;
-        if (total != 0)
-            HIP_TRY(hipMemcpyAsync(tb.dev, tb.host, entries_bytes + bpos * sizeof(uint32_t), hipMemcpyHostToDevice, s),
-                    "hipMemcpyAsync of the batch table failed");
-        table_set_key(tb, items, items_bytes, params);
-    }
-    size_t launches_left = (tb.members[0] ? 1 : 0) + (tb.members[1] ? 1 : 0) + tb.own.size();
-    if (launches_left == 0)
-        return CNTKQ_OK;
-    hipEvent_t done = capturing ? nullptr : tb.event;
-    if (capturing)
-        tb.captured = true;
-    for (int cls = 0; cls < 2; ++cls)
-    {
-        if (tb.members[cls] == 0)
-            continue;
-        LaunchEvents ev;
-        launches_left--;
-        ev.stop = launches_left == 0 ? done : nullptr;
-        const f64::QuantizeBatchEntry64* de = reinterpret_cast<const f64::QuantizeBatchEntry64*>(tb.dev) + tb.first_entry[cls];
-        const uint32_t* db = reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes) + tb.first_begin[cls];
-        HIP_TRY(f64::dispatch_nbits64<f64::QuantizeBatchLauncher64>(nbits, zt && nbits == 1, s, ev, de, db, (uint32_t) tb.members[cls],
-                                                                     tb.blocks[cls], tb.lds[cls]),
-                "batched quantize kernel launch failed");
-        tb.in_flight = tb.in_flight || !capturing;
-    }
-    for (size_t i : tb.own)
-    {
-        const cntkq_quantize_item_f64& it = items[i];
-        LaunchEvents ev;
-        launches_left--;
-        ev.stop = launches_left == 0 ? done : nullptr;
-        HIP_TRY(f64::launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune),
-                "quantize kernel launch failed");
-        tb.in_flight = tb.in_flight || !capturing;
-    }
-    h->last_quantize = done;
-    h->quantize_included_fetch = false;
-    return CNTKQ_OK;
+    return quantize_batch_impl<double>(h, items, count, nbits, zero_threshold_for_1bit);
 }
 
 int cntkq_unquantize_batch_async_f64(cntkq_quantizer* h, const cntkq_unquantize_item_f64* items, size_t count, size_t nbits, int add)
 {
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async_f64: null handle");
-    if (!f64::valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 64 (got %zu)", nbits);
-    if (count == 0)
-        return CNTKQ_OK;
-    if (items == nullptr || count > 0xFFFFFF)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async_f64: bad item list");
-    size_t n = 0;
-    for (size_t i = 0; i < count; ++i)
-    {
-        const cntkq_unquantize_item_f64& it = items[i];
-        if (it.rows >= (1ull << 31) || it.cols >= (1ull << 31))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async_f64: item %zu: rows and cols must be below 2^31", i);
-        if (it.rows == 0 || it.cols == 0)
-            continue;
-        if (it.qbuf == nullptr || it.out == nullptr || !aligned8(it.qbuf) || !aligned8(it.out))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async_f64: item %zu: null or misaligned pointer", i);
-        n++;
-    }
-    if (n == 0)
-        return CNTKQ_OK;
-    if (n == 1)
-    {
-        for (size_t i = 0; i < count; ++i)
-            if (items[i].rows != 0 && items[i].cols != 0)
-                return cntkq_unquantize_async_f64(h, items[i].qbuf, f64::qcol_bytes(nbits, items[i].rows) * items[i].cols, 0, items[i].out,
-                                                  items[i].rows, items[i].cols, nbits, add);
-    }
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    BatchTable& tb = h->unquantize_table64;
-    const size_t params[3] = {count, nbits, 0};
-    const size_t items_bytes = count * sizeof(cntkq_unquantize_item_f64);
-    const bool capturing = stream_capturing(s);
-    if (capturing && !table_matches(tb, items, items_bytes, params))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async_f64: the stream is being captured into a graph and this item "
-                                            "list has not been seen: call once outside the capture first");
-    if (!table_matches(tb, items, items_bytes, params))
-    {
-        const size_t entries_bytes = n * sizeof(f64::UnquantizeBatchEntry64);
-        int rc = table_begin_rebuild(tb, entries_bytes + (n + 1) * sizeof(uint32_t) + 64);
-        if (rc != CNTKQ_OK)
-            return rc;
-        f64::UnquantizeBatchEntry64* he = reinterpret_cast<f64::UnquantizeBatchEntry64*>(tb.host);
-        uint32_t* hb = reinterpret_cast<uint32_t*>(tb.host + entries_bytes);
-        tb.lds[0] = 0;
-        LaunchTuning autotune;
-        uint64_t blocks = 0;
-        size_t e = 0;
-        for (size_t i = 0; i < count; ++i)
-        {
-            const cntkq_unquantize_item_f64& it = items[i];
-            if (it.rows == 0 || it.cols == 0)
-                continue;
-            const f64::UnquantizePlan64 p = f64::plan_unquantize(it.out, it.rows, it.cols, nbits, autotune);
-            if (!p.ok)
-                return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async_f64: item %zu is too large", i);
-            he[e].q = static_cast<const char*>(it.qbuf);
-            he[e].out = it.out;
-            he[e].kind = p.kind;
-            he[e].pad = 0;
-            he[e].qw = p.qw;
-            he[e].rowg = p.rowg;
-            he[e].tile = p.tile;
-            if (p.lds > tb.lds[0])
-                tb.lds[0] = p.lds;
-            hb[e] = (uint32_t) blocks;
-            blocks += p.blocks;
-            if (blocks > 0x7FFFFFFFull)
-                return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_batch_async_f64: too much work in one batch");
-            e++;
-        }
-        hb[e] = (uint32_t) blocks;
-        tb.members[0] = n;
-        tb.blocks[0] = (uint32_t) blocks;
-        tb.entries_bytes = entries_bytes;
-        HIP_TRY(hipMemcpyAsync(tb.dev, tb.host, entries_bytes + (n + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, s),
-                "hipMemcpyAsync of the batch table failed");
-        table_set_key(tb, items, items_bytes, params);
-    }
-    LaunchEvents ev;
-    ev.stop = capturing ? nullptr : tb.event;
-    HIP_TRY(f64::launch_unquantize_batch(s, ev, reinterpret_cast<const f64::UnquantizeBatchEntry64*>(tb.dev),
-                                         reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes), (uint32_t) tb.members[0], tb.blocks[0],
-                                         nbits, add != 0, tb.lds[0]),
-            "batched unquantize kernel launch failed");
-    if (capturing)
-        tb.captured = true;
-    else
-        tb.in_flight = true;
-    h->last_unquantize = ev.stop;
-    return CNTKQ_OK;
+    return unquantize_batch_impl<double>(h, items, count, nbits, add);
 }
 
 int cntkq_stripe_reduce_batch_async_f64(cntkq_quantizer* h, const cntkq_stripe_reduce_item_f64* items, size_t count, size_t workers,
                                         size_t owner, size_t nbits, int zero_threshold_for_1bit)
 {
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async_f64: null handle");
-    if (!f64::valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 64 (got %zu)", nbits);
-    if (workers == 0 || workers > CNTKQ_MAX_WORKERS || owner >= workers)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async_f64: need 1 <= workers <= %d and owner < workers",
-                    CNTKQ_MAX_WORKERS);
-    if (count == 0)
-        return CNTKQ_OK;
-    if (items == nullptr || count > 0xFFFFFF)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async_f64: bad item list");
-    size_t n = 0, only = 0;
-    for (size_t i = 0; i < count; ++i)
-    {
-        const cntkq_stripe_reduce_item_f64& it = items[i];
-        if (it.rows >= (1ull << 31) || it.stripe_cols >= (1ull << 31))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async_f64: item %zu: rows and cols must be below 2^31", i);
-        if (it.rows == 0 || it.stripe_cols == 0)
-            continue;
-        if (it.rows > f64::kTileMaxRows)
-            return fail(CNTKQ_INVALID_ARGUMENT,
-                        "cntkq_stripe_reduce_batch_async_f64: item %zu: columns taller than %zu rows are not supported", i,
-                        (size_t) f64::kTileMaxRows);
-        if (it.stripes == nullptr || it.stripe_res == nullptr || it.q_out == nullptr || !aligned8(it.stripe_res) || !aligned8(it.q_out) ||
-            !aligned8(it.agg_out))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async_f64: item %zu: null or misaligned pointer", i);
-        for (size_t w = 0; w < workers; ++w)
-            if (it.stripes[w] == nullptr || !aligned8(it.stripes[w]))
-                return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async_f64: item %zu: stripe %zu is null or misaligned", i, w);
-        only = i;
-        n++;
-    }
-    if (n == 0)
-        return CNTKQ_OK;
-    if (n == 1)
-        return cntkq_stripe_reduce_async_f64(h, items[only].stripes, workers, owner, items[only].rows, items[only].stripe_cols, nbits,
-                                             items[only].stripe_res, items[only].q_out, items[only].agg_out, zero_threshold_for_1bit);
-    const bool zt = zero_threshold_for_1bit != 0;
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    BatchTable& tb = h->stripe_table64;
-    const size_t params[3] = {count, nbits | (workers << 8) | (owner << 16), (size_t) (zt ? 1 : 0)};
-    std::vector<size_t> flat;
-    flat.reserve(count * (5 + workers));
-    for (size_t i = 0; i < count; ++i)
-    {
-        const cntkq_stripe_reduce_item_f64& it = items[i];
-        flat.push_back(reinterpret_cast<size_t>(it.stripe_res));
-        flat.push_back(reinterpret_cast<size_t>(it.q_out));
-        flat.push_back(reinterpret_cast<size_t>(it.agg_out));
-        flat.push_back(it.rows);
-        flat.push_back(it.stripe_cols);
-        if (it.rows != 0 && it.stripe_cols != 0)
-            for (size_t w = 0; w < workers; ++w)
-                flat.push_back(reinterpret_cast<size_t>(it.stripes[w]));
-    }
-    const size_t flat_bytes = flat.size() * sizeof(size_t);
-    const bool capturing = stream_capturing(s);
-    if (capturing && !table_matches(tb, flat.data(), flat_bytes, params))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async_f64: the stream is being captured into a graph and this "
-                                            "item list has not been seen: call once outside the capture first");
-    if (!table_matches(tb, flat.data(), flat_bytes, params))
-    {
-        const size_t entries_bytes = n * sizeof(f64::StripeBatchEntry64);
-        int rc = table_begin_rebuild(tb, entries_bytes + (n + 2) * sizeof(uint32_t) + 64);
-        if (rc != CNTKQ_OK)
-            return rc;
-        f64::StripeBatchEntry64* he = reinterpret_cast<f64::StripeBatchEntry64*>(tb.host);
-        uint32_t* hb = reinterpret_cast<uint32_t*>(tb.host + entries_bytes);
-        size_t e = 0, bpos = 0;
-        for (int cls = 0; cls < 2; ++cls)
-        {
-            tb.first_entry[cls] = e;
-            tb.first_begin[cls] = bpos;
-            tb.lds[cls] = 0;
-            tb.members[cls] = 0;
-            uint64_t acc = 0;
-            for (size_t i = 0; i < count; ++i)
-            {
-                const cntkq_stripe_reduce_item_f64& it = items[i];
-                if (it.rows == 0 || it.stripe_cols == 0)
-                    continue;
-                f64::StripeBatchEntry64 en;
-                std::memset(&en, 0, sizeof en);
-                en.t = f64::make_tile_geom(it.rows, it.stripe_cols, nbits, 0); // the plain call's geometry: same bytes
-                const size_t lds = f64::tile_lds_bytes(en.t, (uint32_t) workers);
-                if (lds > f64::kMaxLdsBytes)
-                    return fail(CNTKQ_INVALID_ARGUMENT,
-                                "cntkq_stripe_reduce_batch_async_f64: item %zu: %zu rows with %zu workers at %zu bits does not fit the kernel", i,
-                                it.rows, workers, nbits);
-                if ((lds <= kSmallLds64 ? 0 : 1) != cls)
-                    continue;
-                for (size_t w = 0; w < workers; ++w)
-                    en.src.q[w] = static_cast<const char*>(it.stripes[w]);
-                en.src.workers = (uint32_t) workers;
-                en.src.owner = (uint32_t) owner;
-                en.stripe_res = it.stripe_res;
-                en.q_out = static_cast<char*>(it.q_out);
-                en.agg_out = it.agg_out;
-                he[e] = en;
-                hb[bpos++] = (uint32_t) acc;
-                acc += (en.t.cols + en.t.cols_per_tile - 1) / en.t.cols_per_tile;
-                if (acc > 0x7FFFFFFFull)
-                    return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_async_f64: too many workgroups in one batch");
-                if (lds > tb.lds[cls])
-                    tb.lds[cls] = lds;
-                tb.members[cls]++;
-                e++;
-            }
-            if (tb.members[cls] != 0)
-                hb[bpos++] = (uint32_t) acc; // sentinel
-            tb.blocks[cls] = (uint32_t) acc;
-        }
-        tb.entries_bytes = entries_bytes;
-        HIP_TRY(hipMemcpyAsync(tb.dev, tb.host, entries_bytes + bpos * sizeof(uint32_t), hipMemcpyHostToDevice, s),
-                "hipMemcpyAsync of the batch table failed");
-        table_set_key(tb, flat.data(), flat_bytes, params);
-    }
-    size_t launches_left = (tb.members[0] ? 1 : 0) + (tb.members[1] ? 1 : 0);
-    for (int cls = 0; cls < 2; ++cls)
-    {
-        if (tb.members[cls] == 0)
-            continue;
-        LaunchEvents ev;
-        launches_left--;
-        ev.stop = launches_left == 0 && !capturing ? tb.event : nullptr;
-        const f64::StripeBatchEntry64* de = reinterpret_cast<const f64::StripeBatchEntry64*>(tb.dev) + tb.first_entry[cls];
-        const uint32_t* db = reinterpret_cast<const uint32_t*>(tb.dev + tb.entries_bytes) + tb.first_begin[cls];
-        HIP_TRY(f64::dispatch_nbits64<f64::StripeBatchLauncher64>(nbits, zt && nbits == 1, s, ev, de, db, (uint32_t) tb.members[cls],
-                                                                   tb.blocks[cls], tb.lds[cls]),
-                "batched stripe reduction kernel launch failed");
-        if (capturing)
-            tb.captured = true;
-        else
-            tb.in_flight = true;
-    }
-    h->last_stripe = capturing ? nullptr : tb.event;
-    return CNTKQ_OK;
+    return stripe_reduce_batch_impl<double>(h, items, count, workers, owner, nbits, zero_threshold_for_1bit);
 }
 
 // ---- hooks for tests and tuning runs (not part of the public header) --------------------------------
