@@ -50,7 +50,7 @@ def test_cpp_distributed_learner_suite():
 
 @pytest.mark.gpu
 def test_cpp_allreduce_timing_program_runs():
-    """The all-reduce timing program on a small shape (its full-size numbers are quoted in the design notes)."""
+    """The all-reduce timing program runs through on a small shape and prints one line per arrangement."""
     exe = os.path.join(ROOT, "tests", "cpp", "bin", "bench_allreduce")
     assert os.path.exists(exe), "build it first: python -m cntk_amd.build"
     res = subprocess.run([exe, "4", "2048", "256", "1", "3"], capture_output=True, text=True, timeout=300)
