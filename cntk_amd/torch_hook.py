@@ -246,7 +246,8 @@ class QuantizedGradientAggregator:
         for prepared in plan["u"]:
             self._impl.UnquantizeBatchAsync(prepared, add=False)
         if self.average and W > 1:
-            torch._foreach_div_(list(grads), W)
+            for g in grads:
+                g.div_(W)
         self._current = None
 
     def aggregate(self, grads):
