@@ -234,3 +234,18 @@ def test_aggregate_replayed_from_a_hip_graph():
             assert torch.equal(a, b), "replay %d, gradient %d differs from the eager step" % (step, i)
         for a, b in zip(graphed._residual + graphed._stripe_residual, twin._residual + twin._stripe_residual):
             assert torch.equal(a, b), "replay %d: residuals differ from the eager step's" % step
+
+
+def test_average_divides_the_sum_by_the_number_of_workers():
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(datagen.case_seed(82))
+    shapes = [(96, 300), (96,), (24, 130)]
+    src = [[torch.randn(s, generator=gen, device="cuda:0") * 0.01 for s in shapes] for _ in range(4)]
+    summed = [[x.clone() for x in w] for w in src]
+    averaged = [[x.clone() for x in w] for w in src]
+    InProcessGroup(4, 1, True, average=False).aggregate(summed)
+    InProcessGroup(4, 1, True, average=True).aggregate(averaged)
+    torch.cuda.synchronize()
+    for w in range(4):
+        for a, b in zip(summed[w], averaged[w]):
+            assert torch.equal(a / 4, b)
