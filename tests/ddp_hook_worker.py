@@ -52,7 +52,17 @@ def main():
             worst = max(worst, float((p.grad - q.grad).abs().max()) / max(scale, 1e-30))
         steps += 1
         print("step", step, "worst relative difference", worst, flush=True)
-    print(json.dumps({"steps": steps, "max_err": worst, "aggregators": len(state.aggregators)}), flush=True)
+    # the transport's two collectives as the aggregator calls them (one rank: every byte comes back to its sender)
+    from cntk_amd.torch_hook import TorchDistributedTransport
+
+    t = TorchDistributedTransport(None)
+    send = torch.arange(4096, device="cuda", dtype=torch.int32).to(torch.uint8)
+    recv, gathered = torch.zeros_like(send), torch.zeros_like(send)
+    t.all_to_all(send, [send.numel()] * t.world_size, recv)
+    t.all_gather(send, gathered)
+    torch.cuda.synchronize()
+    transport_ok = bool(torch.equal(recv, send) and torch.equal(gathered, send)) and t.world_size == 1 and t.rank == 0
+    print(json.dumps({"steps": steps, "max_err": worst, "aggregators": len(state.aggregators), "transport_ok": transport_ok}), flush=True)
     dist.destroy_process_group()
     return 0
 

@@ -200,7 +200,7 @@ def test_hook_under_distributed_data_parallel():
     if out.get("skipped"):
         pytest.skip(out["skipped"])
     assert p.returncode == 0
-    assert out["steps"] == 3 and out["max_err"] <= 1e-5 and out["aggregators"] >= 1
+    assert out["steps"] == 3 and out["max_err"] <= 1e-5 and out["aggregators"] >= 1 and out["transport_ok"]
 
 
 def test_aggregate_replayed_from_a_hip_graph():
