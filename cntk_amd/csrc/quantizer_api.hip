@@ -107,7 +107,7 @@ struct Elem<double>
 {
     static constexpr size_t kAlign = 8;
     static constexpr size_t kWordBits = 64;
-    static size_t stripe_max_rows(size_t) { return cntkq::f64::kTileMaxRows; }
+    static size_t stripe_max_rows(size_t nbits) { return cntkq::f64::stripe_reduce_max_rows(nbits); }
     static bool valid_nbits(size_t nbits) { return cntkq::f64::valid_nbits(nbits); }
     static size_t qcol_bytes(size_t nbits, size_t rows) { return cntkq::f64::qcol_bytes(nbits, rows); }
     static hipError_t quantize(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, void* q, size_t rows,

@@ -894,55 +894,17 @@ __host__ __device__ inline size_t reg_lds_bytes64(const RegGeom& c)
     return ((size_t) kRegRedSlots + c.nq) * 8;
 }
 
+// Second half of the register kernel: statistics, header, codes, residual and packed QWords of the column a workgroup
+// holds in registers (a: the slots' pieces; edge: this thread's edge element if has_edge). words[0 .. nq) must be zero;
+// the first barrier inside also orders everything the caller did before it. Shared with the stripe reduction below.
 template <int NBITS, bool ZT, int T, int PER>
-__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, PER>(), reg_waves<T, PER>()))) void quantize_reg_kernel(
-    const double* __restrict__ g, const double* r_in, double* r_out, char* __restrict__ q, RegGeom c)
+__device__ __forceinline__ void reg_stats_pack(f64x2 (&a)[PER], double edge, bool has_edge, uint32_t edge_at, uint32_t head, uint32_t pieces,
+                                               uint32_t shift, const RegGeom& c, double* red, uint32_t* red_u, unsigned long long* words,
+                                               double* r_out_col, char* qc)
 {
     using PS = PackShape<NBITS>;
-    static_assert(NBITS < 64, "64-bit codes are whole QWords: nothing to assemble");
     constexpr uint32_t NW = T / 64;
-    extern __shared__ f32x4 smem_v4[];
-    double* red = reinterpret_cast<double*>(smem_v4);
-    uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
-    unsigned long long* words = reinterpret_cast<unsigned long long*>(red + kRegRedSlots);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const size_t base = (size_t) blockIdx.x * c.rows;
-    char* qc = q + (size_t) blockIdx.x * c.qcol;
-    for (uint32_t x = tid; x < c.nq; x += T)
-        words[x] = 0ull;
-    // the column may start 8 bytes off a 16-byte boundary and have an odd height: one element before the first aligned
-    // pair (held by thread 0) and one after the last (thread 1) then take part in every phase after the thread's pieces
-    const uint32_t head = (uint32_t) ((reinterpret_cast<uintptr_t>(r_in + base) >> 3) & 1u);
-    const uint32_t pieces = (c.rows - head) >> 1;
-    const uint32_t tail = c.rows - head - 2 * pieces;
-    const f64x2* g2 = reinterpret_cast<const f64x2*>(g + base + head);
-    const f64x2* r2 = reinterpret_cast<const f64x2*>(r_in + base + head);
-    const bool has_edge = (tid == 0 && head != 0) || (tid == 1 && tail != 0);
-    const uint32_t edge_at = tid == 0 ? 0u : c.rows - 1;
-    double edge = 0.0;
-    if (has_edge)
-        edge = g[base + edge_at] + r_in[base + edge_at];
-    const uint32_t shift = PER <= kRegMaxShiftPer ? column_shift(r_in + base + head, c.line_shift) : 0u;
-    const uint32_t last = pieces - 1;
-    f64x2 a[PER];
-    {
-        const uint32_t t = opaque(tid);
-#pragma unroll
-        for (int u = 0; u < PER; ++u)
-            a[u] = __builtin_nontemporal_load(g2 + slot_piece(t + T * u, shift, last));
-    }
-#pragma unroll
-    for (int u0 = 0; u0 < PER; u0 += 4)
-    {
-        const uint32_t t = opaque(tid);
-        f64x2 b[4];
-#pragma unroll
-        for (int u = u0; u < u0 + 4 && u < PER; ++u)
-            b[u - u0] = __builtin_nontemporal_load(r2 + slot_piece(t + T * u, shift, last));
-#pragma unroll
-        for (int u = u0; u < u0 + 4 && u < PER; ++u)
-            a[u] = a[u] + b[u - u0];
-    }
     constexpr bool need_stat = (NBITS != 1) || !ZT;
     double total = 0.0;
     if constexpr (need_stat)
@@ -1038,7 +1000,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     const ValueQ vq = make_vq<NBITS>(lo, hi);
     const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
     const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
-    f64x2* o2 = reinterpret_cast<f64x2*>(r_out + base + head);
+    f64x2* o2 = reinterpret_cast<f64x2*>(r_out_col + head);
     // the first element of this thread's first slot inside the column is bit position k of QWord w; the element after it
     // is the following QWord, the slots after it lie 2 * T elements further on (step_k, step_w)
     const uint32_t ufirst = tid < shift ? 1u : 0u;
@@ -1093,7 +1055,7 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
             back = code ? val1 : val0;
         else
             back = unquantize_value<NBITS>(vq.uf, vq.lo, code);
-        r_out[base + edge_at] = edge - back;
+        r_out_col[edge_at] = edge - back;
         const uint32_t ek = edge_at / c.nq;
         atomicOr(&words[edge_at - ek * c.nq], (unsigned long long) (code << (ek * PS::SHIFT)));
     }
@@ -1101,6 +1063,205 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     unsigned long long* bits = reinterpret_cast<unsigned long long*>(qc + 16);
     for (uint32_t x = tid; x < c.nq; x += T)
         bits[x] = words[x];
+}
+
+template <int NBITS, bool ZT, int T, int PER>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, PER>(), reg_waves<T, PER>()))) void quantize_reg_kernel(
+    const double* __restrict__ g, const double* r_in, double* r_out, char* __restrict__ q, RegGeom c)
+{
+    static_assert(NBITS < 64, "64-bit codes are whole QWords: nothing to assemble");
+    constexpr uint32_t NW = T / 64;
+    extern __shared__ f32x4 smem_v4[];
+    double* red = reinterpret_cast<double*>(smem_v4);
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
+    unsigned long long* words = reinterpret_cast<unsigned long long*>(red + kRegRedSlots);
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * c.rows;
+    char* qc = q + (size_t) blockIdx.x * c.qcol;
+    for (uint32_t x = tid; x < c.nq; x += T)
+        words[x] = 0ull;
+    // the column may start 8 bytes off a 16-byte boundary and have an odd height: one element before the first aligned
+    // pair (held by thread 0) and one after the last (thread 1) then take part in every phase after the thread's pieces
+    const uint32_t head = (uint32_t) ((reinterpret_cast<uintptr_t>(r_in + base) >> 3) & 1u);
+    const uint32_t pieces = (c.rows - head) >> 1;
+    const uint32_t tail = c.rows - head - 2 * pieces;
+    const f64x2* g2 = reinterpret_cast<const f64x2*>(g + base + head);
+    const f64x2* r2 = reinterpret_cast<const f64x2*>(r_in + base + head);
+    const bool has_edge = (tid == 0 && head != 0) || (tid == 1 && tail != 0);
+    const uint32_t edge_at = tid == 0 ? 0u : c.rows - 1;
+    double edge = 0.0;
+    if (has_edge)
+        edge = g[base + edge_at] + r_in[base + edge_at];
+    const uint32_t shift = PER <= kRegMaxShiftPer ? column_shift(r_in + base + head, c.line_shift) : 0u;
+    const uint32_t last = pieces - 1;
+    f64x2 a[PER];
+    {
+        const uint32_t t = opaque(tid);
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            a[u] = __builtin_nontemporal_load(g2 + slot_piece(t + T * u, shift, last));
+    }
+#pragma unroll
+    for (int u0 = 0; u0 < PER; u0 += 4)
+    {
+        const uint32_t t = opaque(tid);
+        f64x2 b[4];
+#pragma unroll
+        for (int u = u0; u < u0 + 4 && u < PER; ++u)
+            b[u - u0] = __builtin_nontemporal_load(r2 + slot_piece(t + T * u, shift, last));
+#pragma unroll
+        for (int u = u0; u < u0 + 4 && u < PER; ++u)
+            a[u] = a[u] + b[u - u0];
+    }
+    reg_stats_pack<NBITS, ZT, T, PER>(a, edge, has_edge, edge_at, head, pieces, shift, c, red, red_u, words, r_out + base, qc);
+}
+
+// Stripe reduction in the register kernel's shape (the fp32 stripe_reduce_reg_kernel on doubles): 1024 threads per owned
+// column, the running sum of the decoded stripes in registers. The workers are taken one at a time in the fixed order
+// (owner first, then ascending rank): the worker's packed record goes to LDS in one coalesced copy, each thread decodes
+// its slots' elements from it and adds them to its sums. Then the stripe residual is added and reg_stats_pack
+// requantizes: byte for byte what "unquantize own stripe, add the others, quantize_reg_kernel on (aggregate, stripe
+// residual)" gives. LDS: [reduction slots | nq output QWords | lower, upper and nq QWords of one worker's record].
+__host__ __device__ inline size_t stripe_reg_lds_bytes64(const RegGeom& c)
+{
+    return ((size_t) kRegRedSlots + 2 * (size_t) c.nq + 2) * 8;
+}
+
+template <int NBITS, bool ZT, int PER>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<1024, PER>(), reg_waves<1024, PER>()))) void stripe_reduce_reg_kernel(
+    StripeSources src, double* stripe_res, char* q_out, double* agg_out, RegGeom c)
+{
+    using PS = PackShape<NBITS>;
+    static_assert(NBITS < 64, "64-bit codes are whole QWords: nothing to assemble");
+    constexpr uint32_t T = 1024, NW = T / 64;
+    extern __shared__ f32x4 smem_v4[];
+    double* red = reinterpret_cast<double*>(smem_v4);
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
+    unsigned long long* words = reinterpret_cast<unsigned long long*>(red + kRegRedSlots);
+    unsigned long long* pw = words + c.nq; // one worker's record: lower, upper, QWords
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * c.rows;
+    const size_t rec = (size_t) blockIdx.x * c.qcol;
+    for (uint32_t x = tid; x < c.nq; x += T)
+        words[x] = 0ull;
+    // the column as the quantize kernel would see it: an element before the first aligned pair, pairs, an element after
+    double* sres = stripe_res + base;
+    const uint32_t head = (uint32_t) ((reinterpret_cast<uintptr_t>(sres) >> 3) & 1u);
+    const uint32_t pieces = (c.rows - head) >> 1;
+    const uint32_t tail = c.rows - head - 2 * pieces;
+    const bool has_edge = (tid == 0 && head != 0) || (tid == 1 && tail != 0);
+    const uint32_t edge_at = tid == 0 ? 0u : c.rows - 1;
+    const uint32_t shift = PER <= kRegMaxShiftPer ? column_shift(sres + head, c.line_shift) : 0u;
+    const uint32_t ufirst = tid < shift ? 1u : 0u;
+    const uint32_t e0 = head + 2 * (tid + T * ufirst - shift);
+    const uint32_t k_first = e0 / c.nq;
+    const uint32_t w_first = e0 - k_first * c.nq;
+    const uint32_t edge_k = edge_at / c.nq;
+    const uint32_t edge_w = edge_at - edge_k * c.nq;
+
+    f64x2 a[PER];
+    double edge = 0.0;
+    const uint32_t K = src.workers;
+    const uint32_t rec_words = c.nq + 2;
+    for (uint32_t n = 0; n < K; ++n)
+    {
+        const unsigned long long* from = reinterpret_cast<const unsigned long long*>(src.q[stripe_order(n, src.owner)] + rec);
+        if (n != 0)
+            __syncthreads(); // everyone has decoded the previous worker's record
+        for (uint32_t x = tid; x < rec_words; x += 8 * T)
+        {
+            unsigned long long v[8];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u)
+                v[u] = from[(x + T * u < rec_words) ? x + T * u : x];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u)
+                if (x + T * u < rec_words)
+                    pw[x + T * u] = v[u];
+        }
+        __syncthreads();
+        const ValueQ vq = make_vq<NBITS>(__longlong_as_double((long long) pw[0]), __longlong_as_double((long long) pw[1]));
+        const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
+        const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
+        const unsigned long long* bits = pw + 2;
+        // (opaque: the positions of all slots do not depend on the worker, and hoisted out of this loop they would be held
+        // in registers for its whole duration)
+        uint32_t k = opaque(k_first), w = opaque(w_first);
+        const uint32_t t = opaque(tid);
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+        {
+            if (slot_valid(t + T * u, shift, pieces))
+            {
+                uint32_t kk = k, ww = w;
+#pragma unroll
+                for (int e = 0; e < 2; ++e)
+                {
+                    const uint64_t code = (bits[ww] >> (kk * PS::SHIFT)) & PS::CODEMASK;
+                    double x;
+                    if constexpr (NBITS == 1)
+                        x = code ? val1 : val0;
+                    else
+                        x = unquantize_value<NBITS>(vq.uf, vq.lo, code);
+                    // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
+                    a[u][e] = (n == 0) ? x : x + a[u][e];
+                    if (++ww == c.nq)
+                    {
+                        ww = 0;
+                        ++kk;
+                    }
+                }
+            }
+            if ((uint32_t) u >= ufirst)
+            {
+                w += c.step_w;
+                k += c.step_k;
+                if (w >= c.nq)
+                {
+                    w -= c.nq;
+                    ++k;
+                }
+            }
+        }
+        if (has_edge)
+        {
+            const uint64_t code = (bits[edge_w] >> (edge_k * PS::SHIFT)) & PS::CODEMASK;
+            double x;
+            if constexpr (NBITS == 1)
+                x = code ? val1 : val0;
+            else
+                x = unquantize_value<NBITS>(vq.uf, vq.lo, code);
+            edge = (n == 0) ? x : x + edge;
+        }
+    }
+    // aggregate out (optional), then the stripe residual in
+    {
+        const f64x2* r2 = reinterpret_cast<const f64x2*>(sres + head);
+        double* ag = agg_out != nullptr ? agg_out + base : nullptr;
+        const uint32_t t = opaque(tid);
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+        {
+            const uint32_t v = t + T * u;
+            if (slot_valid(v, shift, pieces))
+            {
+                const uint32_t p = v - shift;
+                if (ag != nullptr)
+                {
+                    ag[head + 2 * p] = a[u][0];
+                    ag[head + 2 * p + 1] = a[u][1];
+                }
+                a[u] = a[u] + __builtin_nontemporal_load(r2 + p);
+            }
+        }
+        if (has_edge)
+        {
+            if (ag != nullptr)
+                ag[edge_at] = edge;
+            edge = edge + sres[edge_at];
+        }
+    }
+    reg_stats_pack<NBITS, ZT, T, PER>(a, edge, has_edge, edge_at, head, pieces, shift, c, red, red_u, words, sres, q_out + rec);
 }
 
 // ---- whole gradient sets in one launch (the fp32 batch kernels on doubles) ------------------------------------------

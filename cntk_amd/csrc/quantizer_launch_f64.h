@@ -125,6 +125,14 @@ inline bool reg_applicable(const double* g, const double* r_in, const double* r_
     return (kRegRedSlots + qwords_per_col(rows, nbits)) * 8 <= kMaxLdsBytes;
 }
 
+// Slots are dealt by 128-byte lines where some column of the residual starts inside one and the registers allow it. Only
+// the residual's address enters (the slot dealing is part of the summation order, and the stripe reduction, which must
+// reproduce it, knows only the stripe residual).
+inline bool reg_line_shift(const double* r_in, size_t rows)
+{
+    return !columns_start_on_lines(r_in, rows, 16) && rows / 2 + 7 <= (size_t) kRegThreads * kRegMaxShiftPer;
+}
+
 inline RegGeom make_reg_geom(size_t rows, size_t nbits, bool line_shift)
 {
     RegGeom c;
@@ -196,9 +204,8 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* 
     {
         if (!reg_applicable(g, r_in, r_out, rows, nbits))
             return hipErrorInvalidValue;
-        const bool line_shift = same_line_offset(g, r_in, r_out) && !columns_start_on_lines(r_in, rows, 16) &&
-                                rows / 2 + 7 <= (size_t) kRegThreads * kRegMaxShiftPer;
-        return dispatch_nbits64<RegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, make_reg_geom(rows, nbits, line_shift));
+        return dispatch_nbits64<RegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols,
+                                             make_reg_geom(rows, nbits, reg_line_shift(r_in, rows)));
     }
     if (path == kPathTile)
     {
@@ -215,13 +222,72 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* 
                                         (uint32_t) qwords_per_col(rows, nbits), (uint64_t) qcol_bytes(nbits, rows));
 }
 
-// Same tile geometry as launch_quantize, so that the fused call gives the bytes of the unquantize ... quantize call sequence
-// wherever that sequence's quantize runs the tile kernel (below kRegMinRows rows); above, the two agree within the
-// tolerance of the column bounds.
+template <int NBITS, bool ZT, int PER>
+inline hipError_t launch_stripe_reg_one(hipStream_t s, LaunchEvents ev, const StripeSources& src, double* stripe_res, char* q_out,
+                                        double* agg_out, uint32_t cols, const RegGeom& c)
+{
+    hipExtLaunchKernelGGL((stripe_reduce_reg_kernel<NBITS, ZT, PER>), dim3(cols), dim3(kRegThreads), stripe_reg_lds_bytes64(c), s, ev.start,
+                          ev.stop, 0, src, stripe_res, q_out, agg_out, c);
+    return hipGetLastError();
+}
+
+template <int NBITS, bool ZT>
+struct StripeRegLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, double* stripe_res, char* q_out, double* agg_out,
+                          uint32_t cols, RegGeom c)
+    {
+        if constexpr (NBITS >= 64)
+            return hipErrorInvalidValue;
+        else
+        {
+            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + kRegThreads - 1) / kRegThreads;
+#define CNTKQ_SREG64(P) if (per <= P) return launch_stripe_reg_one<NBITS, ZT, P>(s, ev, src, stripe_res, q_out, agg_out, cols, c)
+            CNTKQ_SREG64(4);
+            CNTKQ_SREG64(6);
+            CNTKQ_SREG64(8);
+            CNTKQ_SREG64(10);
+            CNTKQ_SREG64(13);
+            CNTKQ_SREG64(16);
+            CNTKQ_SREG64(20);
+            CNTKQ_SREG64(25);
+#undef CNTKQ_SREG64
+            return hipErrorInvalidValue;
+        }
+    }
+};
+
+// Whether the stripe reduction of such a stripe runs in the register kernel's shape: the heights where a quantize call on
+// (aggregate, stripe residual) takes the register kernel, as far as two packed columns fit LDS.
+inline bool stripe_uses_reg(size_t rows, size_t nbits)
+{
+    if (rows < kRegMinRows || rows > kRegMaxRows - 16 || nbits >= 64)
+        return false;
+    return ((size_t) kRegRedSlots + 2 * qwords_per_col(rows, nbits) + 2) * 8 <= kMaxLdsBytes;
+}
+
+// Tallest column the fused stripe reduction takes at this bit width.
+inline size_t stripe_reduce_max_rows(size_t nbits)
+{
+    if (nbits >= 64)
+        return kTileMaxRows;
+    const size_t max_nq = (kMaxLdsBytes / 8 - kRegRedSlots - 2) / 2;
+    const size_t by_lds = max_nq * (64 / nbits);
+    const size_t by_regs = kRegMaxRows - 16;
+    const size_t tall = by_lds < by_regs ? by_lds : by_regs;
+    return tall > kTileMaxRows ? tall : kTileMaxRows;
+}
+
+// The kernel family, and within it the geometry, that a quantize call on (aggregate, stripe residual) would take, so that the
+// fused call gives the bytes of the unquantize ... quantize call sequence (the sequence's aggregate must sit at the stripe
+// residual's offset within 16 bytes for that, as whole allocations do).
 inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, double* stripe_res, void* q_out,
                                        double* agg_out, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
 {
     zt = zt && (nbits == 1);
+    if (stripe_uses_reg(rows, nbits))
+        return dispatch_nbits64<StripeRegLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols,
+                                                   make_reg_geom(rows, nbits, reg_line_shift(stripe_res, rows)));
     if (rows > kTileMaxRows)
         return hipErrorInvalidValue;
     const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs);

@@ -301,9 +301,17 @@ def unfused_reference(qz, stripes_np, owner, rows, n, nbits, sres, zt):
     return Agg.to_numpy(), Qo.to_numpy(), S.to_numpy()
 
 
-@pytest.mark.parametrize("rows,n,k", [(70, 9, 3), (429, 12, 4), (2048, 20, 8), (4096, 3, 2), (4988, 3, 3), (7168, 2, 5), (64, 40, 64)])
+def stripe_max_rows_f64(nbits):
+    L = cntk_amd.lib()
+    return L.cntkq_stripe_reduce_max_rows_f64(nbits)
+
+
+@pytest.mark.parametrize("rows,n,k", [(70, 9, 3), (429, 12, 4), (2048, 20, 8), (4096, 3, 2), (4988, 3, 3), (4992, 3, 3), (5003, 2, 2),
+                                      (7168, 2, 5), (64, 40, 64), (8000, 2, 3), (20001, 2, 2), (51184, 1, 2)])
 def test_stripe_reduce_f64(quantizer, rows, n, k):
     for nbits, zt in VARIANTS:
+        if rows > stripe_max_rows_f64(nbits):
+            continue
         say("f64 stripe reduce", rows, n, k, nbits, zt)
         stripes = [oracle.quantize(datagen.normal(31 * w + rows + nbits, rows, n, dtype=F64), zeros(rows, n), nbits, zt, threads=8)[0]
                    for w in range(k)]
@@ -326,13 +334,9 @@ def test_stripe_reduce_f64(quantizer, rows, n, k):
             assert parity.bits_equal(Agg.to_numpy(), agg_o), "aggregate differs from the ordered sum"
             parity.check_quantize(agg_o, sres, Qs[owner].to_numpy(), S.to_numpy(), nbits, zt)
             # the fused call gives the very bytes of the reference's unquantize ... quantize call sequence
-            # (up to 4991 rows, where the sequence's quantize is the tile kernel the fused call shares its order with)
             agg_u, q_u, s_u = unfused_reference(quantizer, stripes, owner, rows, n, nbits, sres, zt)
             assert parity.bits_equal(agg_u, agg_o)
-            if rows < 4992:
-                assert np.array_equal(q_u, Qs[owner].to_numpy()) and parity.bits_equal(s_u, S.to_numpy())
-            else:
-                parity.check_quantize(agg_o, sres, q_u, s_u, nbits, zt)
+            assert np.array_equal(q_u, Qs[owner].to_numpy()) and parity.bits_equal(s_u, S.to_numpy())
 
 
 def test_end_to_end_allreduce_f64(quantizer):
@@ -456,3 +460,14 @@ def test_stripe_batch_equals_per_matrix_calls_f64(quantizer, nbits, zt, k):
             assert np.array_equal(Q1[i][owner].to_numpy(), Q2[i][owner].to_numpy()), ("packed", STRIPE_SETS64[i])
             assert parity.bits_equal(S1[i].to_numpy(), S2[i].to_numpy()), ("stripe residual", STRIPE_SETS64[i])
             assert parity.bits_equal(A1[i].to_numpy(), A2[i].to_numpy()), ("aggregate", STRIPE_SETS64[i])
+
+
+def test_stripe_reduce_height_limit_f64(quantizer):
+    """The limit the library reports per bit width is the tallest column the fused call takes."""
+    assert stripe_max_rows_f64(64) == 7168 and stripe_max_rows_f64(1) == 51184 and stripe_max_rows_f64(3) == 0
+    assert stripe_max_rows_f64(16) == 16284 and stripe_max_rows_f64(32) == 8142 and stripe_max_rows_f64(8) == 32568
+    rows, n, k = 16286, 2, 2
+    Qs = [QuantizedMatrix(rows, n, 16, 0, dtype=torch.float64) for _ in range(k)]
+    S = Matrix(rows, n, dtype=torch.float64)
+    with pytest.raises(cntk_amd.QuantizerLogicError, match="taller than 16284 rows"):
+        quantizer.StripeReduceAsync(Qs, 0, S, Qs[0], False)

@@ -51,7 +51,7 @@ SHAPES = [((96, 300), torch.float32),       # Linear weight: 96 columns of 300 r
           ((3, 2048), torch.float32),       # fewer columns than workers: some stripes are empty
           ((24, 130), torch.float64),
           ((2, 110000), torch.float32),     # columns too tall for the fused stripe reduction: the reference's call sequence
-          ((3, 9000), torch.float64)]       # the same for doubles (limit 7168 rows)
+          ((3, 52000), torch.float64)]      # the same for doubles (limit 51184 rows)
 
 
 @pytest.mark.parametrize("K,nbits,zt", [(1, 1, True), (4, 1, False), (4, 1, True), (3, 4, False), (8, 2, False)])
