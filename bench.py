@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 ROWS, COLS, NBITS = 2048, 9304, 1
+SETUP_STEPS = 50  # untimed steps before the warm-up steps the caller asks for (handle, streams, clocks)
 HBM_PEAK_GBS = 8000.0
 
 
@@ -183,6 +184,10 @@ def main():
         if rc1 or rc2:
             raise RuntimeError(L.cntkq_last_error().decode())
 
+    # set-up, outside warm-up and timing: first calls create streams and events, and the clocks need some work to come up
+    for i in range(SETUP_STEPS):
+        step(i)
+    torch.cuda.synchronize()
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -219,6 +224,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "setup_steps": SETUP_STEPS,
         "ms_per_step": round(sec_per_step * 1e3, 5),
         "higher_is_better": True,
         "scaling": "weak",
