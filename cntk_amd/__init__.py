@@ -259,6 +259,55 @@ class QuantizedMatrix:
     def to_numpy(self):
         return self.buffer.detach().cpu().numpy().copy()
 
+    def Decode(self, row_start, row_end, col_start, col_end):
+        """Host-side reading of a range of the packed matrix, by the layout alone (the index arithmetic of
+        QuantizedMatrix::Print, Source/Math/QuantizedMatrix.cpp:143-169): returns (lower, upper, codes, values) with
+        lower / upper per column and codes / values of shape (rows, cols) of the inclusive range. A debugging aid: the
+        values are reconstructed on the host in the element type, value = (code + 0.5) * ufactor + lower
+        (Source/Math/ValueQuantizer.h:68-97, 131-141)."""
+        if not (row_start <= row_end < self.num_rows and col_start <= col_end < self.num_cols):
+            raise QuantizerLogicError("Index out of range.")  # Source/Math/QuantizedMatrix.cpp:116-120
+        ft, wt = (np.float64, np.uint64) if self.is64 else (np.float32, np.uint32)
+        word_bits, hdr = (64, 16) if self.is64 else (32, 8)
+        raw = self.to_numpy()
+        nq = qwords_per_col(self.num_rows, self.nbits, self.dtype)
+        ncols, nrows = col_end - col_start + 1, row_end - row_start + 1
+        lower, upper = np.empty(ncols, ft), np.empty(ncols, ft)
+        codes, values = np.empty((nrows, ncols), wt), np.empty((nrows, ncols), ft)
+        rows = np.arange(row_start, row_end + 1)
+        word_idx, slot = rows % nq, (rows // nq).astype(wt)
+        for jj, j in enumerate(range(col_start, col_end + 1)):
+            col = raw[j * self.qcol_size:(j + 1) * self.qcol_size]
+            lo, hi = col[:hdr].view(ft)
+            bits = col[hdr:].view(wt)
+            lower[jj], upper[jj] = lo, hi
+            if self.nbits == word_bits:  # pass-through: the code is the value's bit pattern
+                codes[:, jj] = bits[word_idx]
+                values[:, jj] = bits[word_idx].view(ft)
+                continue
+            mask = wt((1 << self.nbits) - 1)
+            c = (bits[word_idx] >> (slot * wt(self.nbits))) & mask
+            used = ft((1 << self.nbits) - (1 if self.nbits > 1 else 0))
+            with np.errstate(invalid="ignore", over="ignore"):
+                spread = ft(hi - lo)
+                ufactor = ft(0) if not (spread >= ft(1e-36)) else ft(spread / used)
+                values[:, jj] = (c.astype(ft) + ft(0.5)) * ufactor + lo
+            codes[:, jj] = c
+        return lower, upper, codes, values
+
+    def Print(self, matrix_name, row_start, row_end, col_start, col_end, file=None):
+        """QuantizedMatrix::Print (Source/Math/QuantizedMatrix.cpp:109-171): the column bounds, then code and
+        reconstructed value of every element of the range, to stderr."""
+        import sys
+        out = file if file is not None else sys.stderr
+        lower, upper, codes, values = self.Decode(row_start, row_end, col_start, col_end)
+        name = matrix_name if matrix_name is not None else "Unnamed Matrix"
+        print("\n###### %s (%d, %d) ######" % (name, self.num_rows, self.num_cols), file=out)
+        print("\n------ Print Range (%d:%d, %d:%d) ------" % (row_start, row_end, col_start, col_end), file=out)
+        print("".join("Lower=%.10f,Upper=%.10f\t" % (lo, hi) for lo, hi in zip(lower, upper)), file=out)
+        for i in range(codes.shape[0]):
+            print("".join("%10d (%.10f)          \t" % (int(codes[i, j]), values[i, j]) for j in range(codes.shape[1])), file=out)
+
     def from_numpy(self, a):
         self.buffer.copy_(torch.from_numpy(np.ascontiguousarray(a, dtype=np.uint8)))
 

@@ -19,6 +19,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <cstdio>
 #include <cstring>
 #include <memory>
 #include <stdexcept>
@@ -307,6 +308,59 @@ public:
                 std::memcpy(host.data(), m_buffer, host.size());
         }
         return host;
+    }
+
+    // QuantizedMatrix::Print (Source/Math/QuantizedMatrix.cpp:109-171): the column bounds, then code and reconstructed
+    // value of every element of the inclusive range, to stderr (or `out`). Reads a host copy; element i of a column is in
+    // QWord i % nq at bit (i / nq) * nbits; value = (code + 0.5) * ufactor + lower (Source/Math/ValueQuantizer.h:68-97, 131-141).
+    void Print(const char* matrixName, size_t rowStart, size_t rowEnd, size_t colStart, size_t colEnd, FILE* out = stderr) const
+    {
+        typedef typename detail::Abi<ElemType>::QWord QWord;
+        if (rowStart > rowEnd || rowEnd >= m_rows || colStart > colEnd || colEnd >= m_cols)
+            throw std::invalid_argument("Index out of range.");
+        const std::vector<char> host = CopyToHost();
+        const size_t wordBits = 8 * sizeof(QWord);
+        const size_t nq = (m_qColSize - 2 * sizeof(ElemType)) / sizeof(QWord);
+        if (matrixName != nullptr)
+            std::fprintf(out, "\n###### %s (%lu, %lu) ######\n", matrixName, (unsigned long) m_rows, (unsigned long) m_cols);
+        else
+            std::fprintf(out, "\n###### Unnamed Matrix (%lu, %lu) ######\n", (unsigned long) m_rows, (unsigned long) m_cols);
+        std::fprintf(out, "\n------ Print Range (%lu:%lu, %lu:%lu) ------\n", (unsigned long) rowStart, (unsigned long) rowEnd,
+                     (unsigned long) colStart, (unsigned long) colEnd);
+        auto header = [&](size_t j, int which) {
+            ElemType v;
+            std::memcpy(&v, host.data() + j * m_qColSize + which * sizeof(ElemType), sizeof v);
+            return v;
+        };
+        for (size_t j = colStart; j <= colEnd; ++j)
+            std::fprintf(out, "Lower=%.10f,Upper=%.10f\t", (double) header(j, 0), (double) header(j, 1));
+        std::fprintf(out, "\n");
+        for (size_t i = rowStart; i <= rowEnd; ++i)
+        {
+            for (size_t j = colStart; j <= colEnd; ++j)
+            {
+                const ElemType lower = header(j, 0), upper = header(j, 1);
+                QWord word;
+                std::memcpy(&word, host.data() + j * m_qColSize + 2 * sizeof(ElemType) + (i % nq) * sizeof(QWord), sizeof word);
+                QWord code;
+                ElemType value;
+                if (m_bits == wordBits)
+                {
+                    code = word; // pass-through: the code is the value's bit pattern
+                    std::memcpy(&value, &word, sizeof value);
+                }
+                else
+                {
+                    code = (word >> ((i / nq) * m_bits)) & ((QWord(1) << m_bits) - 1);
+                    const ElemType spread = upper - lower;
+                    const ElemType used = (ElemType) ((QWord(1) << m_bits) - (m_bits > 1 ? 1 : 0));
+                    const ElemType ufactor = spread >= (ElemType) 1e-36f ? spread / used : (ElemType) 0;
+                    value = ((ElemType) code + (ElemType) 0.5) * ufactor + lower;
+                }
+                std::fprintf(out, "%10d (%.10f)          \t", (int) code, (double) value);
+            }
+            std::fprintf(out, "\n");
+        }
     }
 
 private:

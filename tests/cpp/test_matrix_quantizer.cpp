@@ -17,6 +17,7 @@
 #include <cstring>
 #include <memory>
 #include <random>
+#include <string>
 #include <vector>
 
 using namespace cntk_amd;
@@ -276,6 +277,54 @@ static void ErrorBehaviour()
         CHECK(r[i] == 0.0f, "ResetResidue");
 }
 
+// QuantizedMatrix::Print on the hand example {0.1, -0.2, 0.3, -0.4, 0.05} (1 bit, mean threshold): bounds -0.462 / 0.402,
+// codes 1 0 1 0 1, reconstructed values lower + (code + 0.5) * (upper - lower) / 2 ... written to a temporary file.
+template <class E>
+static void PrintOne()
+{
+    const E host[5] = {(E) 0.1, (E) -0.2, (E) 0.3, (E) -0.4, (E) 0.05};
+    Matrix<E> g(5, 1, 0);
+    g.SetValue(host);
+    MatrixQuantizer<E> mq(5, 1, 0, false);
+    QuantizedMatrix<E> q(5, 1, 1, 0);
+    mq.QuantizeAsync(g, q, false);
+    mq.WaitQuantizeAsyncDone();
+    FILE* f = std::tmpfile();
+    CHECK(f != nullptr, "tmpfile");
+    if (f == nullptr)
+        return;
+    q.Print("grad", 0, 4, 0, 0, f);
+    std::rewind(f);
+    std::string text;
+    char buf[256];
+    while (std::fgets(buf, sizeof buf, f) != nullptr)
+        text += buf;
+    std::fclose(f);
+    CHECK(text.find("###### grad (5, 1) ######") != std::string::npos, "title: %s", text.c_str());
+    CHECK(text.find("Print Range (0:4, 0:0)") != std::string::npos, "range");
+    CHECK(text.find("Lower=-0.462") != std::string::npos && text.find("Upper=0.402") != std::string::npos, "bounds: %s", text.c_str());
+    // five element lines: code then value in parentheses; low level -0.246, high level 0.186
+    const char* expect[5] = {"1 (0.18", "0 (-0.24", "1 (0.18", "0 (-0.24", "1 (0.18"};
+    size_t pos = text.find("Upper=");
+    for (int i = 0; i < 5; ++i)
+    {
+        const size_t at = text.find(expect[i], pos);
+        CHECK(at != std::string::npos, "element %d: %s", i, text.c_str());
+        if (at == std::string::npos)
+            break;
+        pos = at + 1;
+    }
+    bool threw = false;
+    try { q.Print(nullptr, 0, 5, 0, 0, stderr); } catch (const std::invalid_argument&) { threw = true; }
+    CHECK(threw, "Print: index out of range");
+}
+
+static void PrintPackedMatrix()
+{
+    PrintOne<float>();
+    PrintOne<double>();
+}
+
 int main()
 {
     try
@@ -291,6 +340,9 @@ int main()
         before = g_failures;
         ErrorBehaviour();
         std::printf("Test case GPUMatrixSuite/QuantizerErrorBehaviour %s\n", g_failures != before ? "has FAILED" : "has passed");
+        before = g_failures;
+        PrintPackedMatrix();
+        std::printf("Test case GPUMatrixSuite/QuantizedMatrixPrint %s\n", g_failures != before ? "has FAILED" : "has passed");
     }
     catch (const std::exception& e)
     {
