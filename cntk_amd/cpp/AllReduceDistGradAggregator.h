@@ -29,6 +29,8 @@
 #include "MatrixQuantizer.h"
 
 #include <algorithm>
+#include <chrono>
+#include <cstdio>
 #include <future>
 #include <map>
 #include <tuple>
@@ -205,6 +207,10 @@ public:
     {
         bool useFusedStripeReduce = true; // one kernel for "unquantize all stripes, sum, requantize"
         bool useBatchedCalls = true;      // one launch for all gradients in steps 1 and 5
+        // every syncStatsTrace-th aggregation is timed between two device synchronisations and reported on stderr as the
+        // reference does ("Actual gradient aggregation time", Source/1BitSGD/AllReduceDistGradAggregator.h:153, 241-246,
+        // 560-565); 0 = never
+        int syncStatsTrace = 0;
     };
 
     AllReduceDistGradAggregator(StripeTransportT<ElemType>& transport, size_t myRank, int deviceId, int nBits, bool zeroThresholdFor1Bit,
@@ -531,7 +537,7 @@ public:
     // stream-ordered: the K workers' steps are queued back to back and the host waits only at the very end.
     InProcessCluster(size_t numWorkers, int deviceId, int nBits, bool zeroThresholdFor1Bit, bool useQuantizationForSelfStripe = true,
                      bool useAsyncAggregation = true, Options options = Options())
-        : m_transport(numWorkers, true)
+        : m_transport(numWorkers, true), m_syncStatsTrace(options.syncStatsTrace)
     {
         for (size_t r = 0; r < numWorkers; ++r)
             m_workers.emplace_back(new AllReduceDistGradAggregator<ElemType>(m_transport, r, deviceId, nBits, zeroThresholdFor1Bit,
@@ -549,6 +555,14 @@ public:
         const size_t K = m_workers.size();
         if (gradients.size() != K || headers.size() != K)
             throw std::invalid_argument("InProcessCluster: one gradient set and one header per worker");
+        const bool showSyncPerfStats = m_syncStatsTrace > 0 && (m_iterationCount % (size_t) m_syncStatsTrace) == 0;
+        m_iterationCount++;
+        std::chrono::steady_clock::time_point t0;
+        if (showSyncPerfStats)
+        {
+            detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize"); // the gradients have been computed (:241-246)
+            t0 = std::chrono::steady_clock::now();
+        }
         for (size_t r = 0; r < K; ++r)
             m_workers[r]->QuantizeAndPost(gradients[r], headers[r], resetState);
         for (size_t r = 0; r < K; ++r)
@@ -556,6 +570,12 @@ public:
         bool any = false;
         for (size_t r = 0; r < (unquantizeOnAllWorkers ? K : 1); ++r)
             any = m_workers[r]->FetchAndUnquantize(gradients[r], headers[r]) || any;
+        if (showSyncPerfStats)
+        {
+            detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize");
+            const double seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+            std::fprintf(stderr, "Actual gradient aggregation time: %.6g\n", seconds);
+        }
         return any;
     }
 
@@ -639,6 +659,8 @@ private:
     std::vector<std::vector<std::unique_ptr<Matrix<ElemType>>>> m_buffered;
     std::vector<DistGradHeader> m_bufferedHeaders;
     std::future<void> m_pending;
+    int m_syncStatsTrace = 0;
+    size_t m_iterationCount = 0;
 };
 
 } // namespace cntk_amd

@@ -425,6 +425,44 @@ static void DoublePrecisionVariantsAreBitIdentical()
     }
 }
 
+// syncStatsTrace = 2: every second aggregation reports its time on stderr (the reference's wording).
+static void SyncStatsTrace()
+{
+    InProcessCluster<float>::Options opt;
+    opt.syncStatsTrace = 2;
+    InProcessCluster<float> cluster(2, 0, 1, false, true, false, opt);
+    FILE* saved = stderr;
+    FILE* f = std::tmpfile();
+    CHECK(f != nullptr, "tmpfile");
+    if (f == nullptr)
+        return;
+    stderr = f;
+    for (int step = 0; step < 5; ++step)
+    {
+        std::vector<std::unique_ptr<Matrix<float>>> owned;
+        std::vector<std::vector<Matrix<float>*>> grads(2);
+        std::vector<DistGradHeader> headers;
+        for (size_t r = 0; r < 2; ++r)
+        {
+            owned.emplace_back(new Matrix<float>(64, 8, 0));
+            owned.back()->SetValue(0.01f * (float) (r + 1));
+            grads[r].push_back(owned.back().get());
+            headers.emplace_back(1);
+            headers.back().numSamples = 4;
+        }
+        cluster.AggregateGradients(grads, headers, step == 0, true);
+    }
+    stderr = saved;
+    std::rewind(f);
+    int lines = 0;
+    char buf[256];
+    while (std::fgets(buf, sizeof buf, f) != nullptr)
+        if (std::strstr(buf, "Actual gradient aggregation time: ") != nullptr)
+            lines++;
+    std::fclose(f);
+    CHECK(lines == 3, "aggregations 0, 2 and 4 are reported, got %d lines", lines);
+}
+
 int main()
 {
     try
@@ -433,7 +471,8 @@ int main()
         const T tests[] = {{"QuantizedAllReduceVariantsBitIdentical", VariantsAreBitIdentical}, {"QuantizedAllReduceAgainstOracle", AgainstOracle},
                            {"QuantizedAllReduceUnquantizedSelfStripe", UnquantizedSelfStripe}, {"QuantizedAllReduceEmptyMinibatchAndReset", EmptyMinibatchAndReset},
                            {"QuantizedAllReduceBufferedAggregation", BufferedAggregation},
-                           {"QuantizedAllReduceDoublePrecision", DoublePrecisionVariantsAreBitIdentical}};
+                           {"QuantizedAllReduceDoublePrecision", DoublePrecisionVariantsAreBitIdentical},
+                           {"QuantizedAllReduceSyncStatsTrace", SyncStatsTrace}};
         for (const T& t : tests)
         {
             const int before = g_failures;
