@@ -55,6 +55,12 @@ def stripe_layout(shapes, world_size, nbits):
     return stripes, rel, max(max(need), 8)
 
 
+def stripe_residue_numel(t, rank, world_size):
+    """Elements of the stripe residual that worker `rank` keeps for gradient tensor t (rows times its stripe's columns)."""
+    cols = t.shape[0] if t.dim() >= 2 else 1
+    return (t.numel() // max(cols, 1)) * stripe_range(cols, rank, world_size)[1]
+
+
 class LocalTransport:
     """One worker: nothing changes hands (the aggregator never calls a transport of one worker)."""
     rank, world_size = 0, 1
@@ -99,11 +105,27 @@ class QuantizedGradientAggregator:
     DistributedDataParallel convention).
     """
 
-    def __init__(self, nbits=1, zero_threshold_for_1bit=True, transport=None, average=False):
+    def __init__(self, nbits=1, zero_threshold_for_1bit=True, transport=None, average=False, residues=None, stripe_residues=None):
+        """residues / stripe_residues: caller-owned residual tensors, as the v2 communicator takes them from its learner
+        (QuantizedAggregateInPlace, Source/1BitSGD/QuantizedDistributedCommunicator.h:51-62): one per gradient, of the
+        gradient's size, and one per gradient of the size of this worker's stripe (stripe_residue_numel). They are updated in
+        place; without them the aggregator creates its own, zeroed."""
         self.nbits, self.zt, self.average = int(nbits), bool(zero_threshold_for_1bit), bool(average)
         self.transport = transport if transport is not None else LocalTransport()
+        self._given = (residues, stripe_residues)
         self._geom = None
         self._plan = None
+
+    def _adopt(self, given, grads, numels, what):
+        """The caller's residual tensors as flat views, checked against what the gradients need."""
+        if len(given) != len(grads):
+            raise QuantizerLogicError("%s: one tensor per gradient" % what)
+        out = []
+        for t, g, n in zip(given, grads, numels):
+            if t.device != g.device or t.dtype != g.dtype or t.numel() != n or not t.is_contiguous():
+                raise QuantizerLogicError("%s: a contiguous tensor of %d elements of %s on %s is needed" % (what, n, g.dtype, g.device))
+            out.append(t.detach().view(-1))
+        return out
 
     # ---- set-up -------------------------------------------------------------------------------------
 
@@ -124,9 +146,15 @@ class QuantizedGradientAggregator:
         self._recv = torch.zeros(W * self._slot, **u8) if W > 1 else None
         self._mine = torch.zeros(self._slot, **u8)
         self._gathered = torch.zeros(W * self._slot, **u8) if W > 1 else None
-        self._residual = [torch.zeros(g.numel(), dtype=g.dtype, device=dev) for g in grads]
-        self._stripe_residual = [torch.zeros(shapes[i][0] * self._stripe[me][i][1], dtype=grads[i].dtype, device=dev)
-                                 for i in range(len(grads))]
+        stripe_numels = [shapes[i][0] * self._stripe[me][i][1] for i in range(len(grads))]
+        if self._given[0] is not None:
+            self._residual = self._adopt(self._given[0], grads, [g.numel() for g in grads], "residues")
+        else:
+            self._residual = [torch.zeros(g.numel(), dtype=g.dtype, device=dev) for g in grads]
+        if self._given[1] is not None:
+            self._stripe_residual = self._adopt(self._given[1], grads, stripe_numels, "stripe_residues")
+        else:
+            self._stripe_residual = [torch.zeros(n, dtype=g.dtype, device=dev) for n, g in zip(stripe_numels, grads)]
         self._shapes = shapes
         self._geom = [(tuple(g.shape), g.dtype) for g in grads]
         self._any64 = any(g.dtype == torch.float64 for g in grads)

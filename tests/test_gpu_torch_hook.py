@@ -249,3 +249,28 @@ def test_average_divides_the_sum_by_the_number_of_workers():
     for w in range(4):
         for a, b in zip(summed[w], averaged[w]):
             assert torch.equal(a / 4, b)
+
+
+def test_caller_owned_residues():
+    """The v2 communicator's shape of the call: the learner owns the residual tensors and hands them in; the result and
+    the residues are those of an aggregator that keeps its own."""
+    from cntk_amd.torch_hook import stripe_residue_numel
+
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(datagen.case_seed(83))
+    shapes = [(96, 300), (96,), (24, 130)]
+    res = [torch.zeros(int(np.prod(s)), device="cuda:0") for s in shapes]
+    sres = [torch.zeros(stripe_residue_numel(torch.empty(s), 0, 1), device="cuda:0") for s in shapes]
+    mine, own = QuantizedGradientAggregator(1, True, residues=res, stripe_residues=sres), QuantizedGradientAggregator(1, True)
+    for step in range(3):
+        g = [torch.randn(s, generator=gen, device="cuda:0") * 0.01 for s in shapes]
+        h = [x.clone() for x in g]
+        mine.aggregate(g)
+        own.aggregate(h)
+        torch.cuda.synchronize()
+        for a, b in zip(g, h):
+            assert torch.equal(a, b)
+    for a, b in zip(res + sres, own._residual + own._stripe_residual):
+        assert torch.equal(a, b) and float(a.abs().max()) > 0
+    with pytest.raises(QuantizerLogicError):
+        QuantizedGradientAggregator(1, True, residues=res[:2]).aggregate(g)
