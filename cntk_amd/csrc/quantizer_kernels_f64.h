@@ -236,15 +236,22 @@ __device__ __forceinline__ void tile_stats(const double* tile, double* hdr, doub
     __syncthreads();
 }
 
+// Columns of fewer QWords than this hand their new residual back through the LDS tile.
+constexpr uint32_t kStagedResidualBelowQWords = 16;
+
 // words[] (LDS, nc * nq entries) must be zero on entry when PackShape<NBITS>::CHUNKS > 1.
-// The new residual goes straight to global memory: for a fixed bit position consecutive threads hold consecutive rows.
+// For a fixed bit position consecutive threads hold consecutive rows of a column, nq of them: where that run is at least a
+// 128-byte line the new residual goes straight to global memory; shorter runs (a 147-row column at 1 bit: 3 doubles) would
+// reach memory as fragments, so there the residual replaces the value in the tile (every value is read by exactly one work
+// item) and the tile leaves in consecutive stores.
 template <int NBITS, bool ZT>
-__device__ __forceinline__ void tile_pack(const double* tile, const double* hdr, unsigned long long* words, const TileGeom& t,
+__device__ __forceinline__ void tile_pack(double* tile, const double* hdr, unsigned long long* words, const TileGeom& t,
                                           uint32_t nc, char* qtile, double* res_out)
 {
     using PS = PackShape<NBITS>;
     const uint32_t nwords = nc * t.nq;
     const uint32_t items = nwords * PS::CHUNKS;
+    const bool staged = t.nq < kStagedResidualBelowQWords;
     for (uint32_t it = threadIdx.x; it < items; it += kThreads)
     {
         const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
@@ -254,7 +261,7 @@ __device__ __forceinline__ void tile_pack(const double* tile, const double* hdr,
         const ValueQ vq = make_vq<NBITS>(hdr[2 * c], hdr[2 * c + 1]);
         const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
         const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
-        const double* colv = tile + (size_t) c * t.rows;
+        double* colv = tile + (size_t) c * t.rows;
         double* ro = res_out + (size_t) c * t.rows;
         uint64_t word = 0;
 #pragma unroll
@@ -271,7 +278,10 @@ __device__ __forceinline__ void tile_pack(const double* tile, const double* hdr,
                     back = code ? val1 : val0;
                 else
                     back = unquantize_value<NBITS>(vq.uf, vq.lo, code);
-                __builtin_nontemporal_store(v - back, ro + i);
+                if (staged)
+                    colv[i] = v - back;
+                else
+                    __builtin_nontemporal_store(v - back, ro + i);
                 word |= code << (k * PS::SHIFT);
             }
         }
@@ -280,15 +290,22 @@ __device__ __forceinline__ void tile_pack(const double* tile, const double* hdr,
         else
             atomicOr(&words[qi], (unsigned long long) word);
     }
+    if (PS::CHUNKS > 1 || staged) // uniform over the workgroup
+        __syncthreads();
     if constexpr (PS::CHUNKS > 1)
     {
-        __syncthreads();
         for (uint32_t qi = threadIdx.x; qi < nwords; qi += kThreads)
         {
             const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
             const uint32_t w = qi - c * t.nq;
             reinterpret_cast<uint64_t*>(qtile + (size_t) c * t.qcol + 16)[w] = words[qi];
         }
+    }
+    if (staged)
+    {
+        const uint32_t total = nc * t.rows;
+        for (uint32_t e = threadIdx.x; e < total; e += kThreads)
+            __builtin_nontemporal_store(tile[e], res_out + e);
     }
 }
 
@@ -490,6 +507,12 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
         for (uint32_t x = tid; x < nwords; x += kThreads)
             l.words[x] = 0ull;
 
+    // short columns: the stripe residual comes in as one consecutive run (see tile_pack), not as runs of nq rows
+    const bool staged = t.nq < kStagedResidualBelowQWords;
+    if (staged)
+        for (uint32_t e = tid; e < nc * t.rows; e += kThreads)
+            l.tile[e] = __builtin_nontemporal_load(sp + e);
+
     // decode constants from every worker's column header, in summation order: 1 bit -> the two levels, else (ufactor, lower)
     for (uint32_t x = tid; x < nc * K; x += kThreads)
     {
@@ -561,7 +584,7 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
             {
                 if (agg_out != nullptr)
                     agg_out[base + (size_t) c * t.rows + i] = acc[kk];
-                colv[i] = acc[kk] + __builtin_nontemporal_load(sc + i);
+                colv[i] = acc[kk] + (staged ? colv[i] : __builtin_nontemporal_load(sc + i));
             }
         }
     }
