@@ -389,6 +389,156 @@ __global__ __launch_bounds__(kThreads) void quantize_tile_kernel(const double* _
     quantize_tile_body<NBITS, ZT>(g, r_in, r_out, q, t, blockIdx.x, reinterpret_cast<double*>(smem_f64));
 }
 
+// ---- one 256-thread workgroup per column, the column in registers element by element ------------------------
+//
+// For the heights at which the tile kernel holds a single column per tile (more than 1024 rows) and that column starts to
+// crowd LDS (16 KB at 2048 rows, 39 KB at 4991): thread t keeps rows t, t + 256, ... (at most EPT of them) from the loads
+// to the residual store, LDS holds only the reduction slots and the column's QWords (assembled by atomic OR), and the
+// occupancy no longer falls with the height. Nothing depends on alignment: every access is one double, consecutive
+// threads on consecutive rows. The sums are taken exactly as tile_stats takes them for a one-column tile -- a thread adds
+// its rows in ascending order, then group_sum over the 256 threads -- so the bytes are those of the tile kernel, and the
+// tile stripe reduction still reproduces the call sequence. A row beyond the column is replaced by the last row on
+// loading and masked out of every sum and store, so the load and statistics phases have no branches.
+template <int EPT>
+constexpr int colreg_waves()
+{
+    int w = 512 / (2 * EPT + 40); // (with 8 registers fewer one instantiation spills)
+    return w > 8 ? 8 : w;
+}
+
+constexpr uint32_t kColRegPrefixWords = 10; // 8 doubles + four uint32 for the reductions, as in the tile kernels
+
+__host__ __device__ inline size_t colreg_lds_bytes(uint32_t nq)
+{
+    return ((size_t) kColRegPrefixWords + nq) * 8;
+}
+
+template <int NBITS, bool ZT, int EPT>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(colreg_waves<EPT>(), colreg_waves<EPT>()))) void quantize_colreg_kernel(
+    const double* __restrict__ g, const double* r_in, double* r_out, char* __restrict__ q, uint32_t rows, uint32_t nq, uint64_t qcol)
+{
+    static_assert(NBITS < 64, "64-bit codes are whole QWords: nothing to assemble");
+    using PS = PackShape<NBITS>;
+    extern __shared__ f64x2 smem_f64[];
+    double* scratch_f = reinterpret_cast<double*>(smem_f64);
+    uint32_t* scratch_u = reinterpret_cast<uint32_t*>(scratch_f + 8);
+    unsigned long long* words = reinterpret_cast<unsigned long long*>(scratch_f + kColRegPrefixWords);
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * rows;
+    char* qc = q + (size_t) blockIdx.x * qcol;
+    for (uint32_t x = tid; x < nq; x += kThreads)
+        words[x] = 0ull;
+    const double* gp = g + base;
+    const double* rp = r_in + base;
+    const uint32_t last = rows - 1;
+    double a[EPT];
+    {
+        const uint32_t t = opaque(tid);
+#pragma unroll
+        for (int u = 0; u < EPT; ++u)
+            a[u] = __builtin_nontemporal_load(gp + min(t + kThreads * u, last));
+    }
+#pragma unroll
+    for (int u0 = 0; u0 < EPT; u0 += 4)
+    {
+        const uint32_t t = opaque(tid);
+        double b[4];
+#pragma unroll
+        for (int u = u0; u < u0 + 4 && u < EPT; ++u)
+            b[u - u0] = __builtin_nontemporal_load(rp + min(t + kThreads * u, last));
+#pragma unroll
+        for (int u = u0; u < u0 + 4 && u < EPT; ++u)
+            a[u] = a[u] + b[u - u0];
+    }
+    // a thread stores only rows it has loaded itself, so r_out may be r_in without a barrier in between
+
+    double lo, hi;
+    if constexpr (NBITS == 1)
+    {
+        double mean = 0.0;
+        if constexpr (!ZT)
+        {
+            double sum = 0.0;
+            const uint32_t t = opaque(tid);
+#pragma unroll
+            for (int u = 0; u < EPT; ++u)
+                sum = (t + kThreads * u < rows) ? sum + a[u] : sum;
+            sum = group_sum(sum, kThreads, scratch_f);
+            mean = sum / (double) rows;
+        }
+        double s0 = 0.0, s1 = 0.0;
+        uint32_t n0 = 0;
+        const uint32_t t = opaque(tid);
+#pragma unroll
+        for (int u = 0; u < EPT; ++u)
+        {
+            const bool valid = t + kThreads * u < rows;
+            const bool below = a[u] < mean;
+            s0 = (valid && below) ? s0 + a[u] : s0;
+            s1 = (valid && !below) ? s1 + a[u] : s1;
+            n0 += (valid && below) ? 1u : 0u;
+        }
+        group_sum3(s0, s1, n0, kThreads, scratch_f, scratch_u);
+        finish_stats_1bit<ZT>(mean, s0, s1, n0, rows - n0, rows, lo, hi);
+    }
+    else
+    {
+        double sum = 0.0;
+        const uint32_t t = opaque(tid);
+#pragma unroll
+        for (int u = 0; u < EPT; ++u)
+        {
+            const double sq = a[u] * a[u];
+            sum = (t + kThreads * u < rows) ? sum + sq : sum;
+        }
+        sum = group_sum(sum, kThreads, scratch_f);
+        finish_stats_multibit(sum, rows, lo, hi);
+    }
+    if (tid == 0)
+    {
+        double* gh = reinterpret_cast<double*>(qc);
+        gh[0] = lo;
+        gh[1] = hi;
+    }
+    const ValueQ vq = make_vq<NBITS>(lo, hi);
+    const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
+    const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
+    double* ro = r_out + base;
+    // row i is bit position i / nq of QWord i % nq; a thread's rows lie 256 apart
+    const uint32_t step_k = kThreads / nq, step_w = kThreads - step_k * nq;
+    uint32_t k = tid / nq;
+    uint32_t w = tid - k * nq;
+    const uint32_t to = opaque(tid);
+#pragma unroll
+    for (int u = 0; u < EPT; ++u)
+    {
+        const uint32_t i = to + kThreads * u;
+        if (i < rows)
+        {
+            const double v = a[u];
+            const uint64_t code = quantize_value<NBITS, ZT>(vq, v);
+            double back;
+            if constexpr (NBITS == 1)
+                back = code ? val1 : val0;
+            else
+                back = unquantize_value<NBITS>(vq.uf, vq.lo, code);
+            __builtin_nontemporal_store(v - back, ro + i);
+            atomicOr(&words[w], (unsigned long long) (code << (k * PS::SHIFT)));
+        }
+        w += step_w;
+        k += step_k;
+        if (w >= nq)
+        {
+            w -= nq;
+            ++k;
+        }
+    }
+    __syncthreads();
+    unsigned long long* bits = reinterpret_cast<unsigned long long*>(qc + 16);
+    for (uint32_t x = tid; x < nq; x += kThreads)
+        bits[x] = words[x];
+}
+
 // one workgroup of 1024 threads per column, statistics and packing re-read global memory
 template <int NBITS, bool ZT>
 __global__ __launch_bounds__(kTallThreads) void quantize_tall_kernel(const double* __restrict__ g, const double* r_in, double* r_out,

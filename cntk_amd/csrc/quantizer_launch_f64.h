@@ -180,6 +180,44 @@ struct RegLauncher
     }
 };
 
+// The element-wise register kernel (256 threads, up to 20 rows each): the heights at which the tile kernel holds one column
+// per tile, any alignment, below 64 bits. Same bytes as the tile kernel in its default geometry.
+constexpr size_t kColRegMaxRows = 256 * 20;
+constexpr size_t kColRegMinRows = 1025; // the whole range: 1028 rows 87 us against 108 us on 18.5 M elements, 4096: 76 against 86
+
+inline bool colreg_applicable(size_t rows, size_t nbits)
+{
+    return rows > 1024 && rows <= kColRegMaxRows && nbits < 64;
+}
+
+template <int NBITS, bool ZT>
+struct ColRegLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, char* q, uint32_t rows,
+                          uint32_t cols, uint32_t nq, uint64_t qcol)
+    {
+        if constexpr (NBITS >= 64)
+            return hipErrorInvalidValue;
+        else
+        {
+            const uint32_t ept = (rows + kThreads - 1) / kThreads;
+#define CNTKQ_COLREG64(E)                                                                                                              \
+    if (ept <= E)                                                                                                                      \
+    {                                                                                                                                  \
+        hipExtLaunchKernelGGL((quantize_colreg_kernel<NBITS, ZT, E>), dim3(cols), dim3(kThreads), colreg_lds_bytes(nq), s, ev.start,   \
+                              ev.stop, 0, g, r_in, r_out, q, rows, nq, qcol);                                                          \
+        return hipGetLastError();                                                                                                      \
+    }
+            CNTKQ_COLREG64(8)
+            CNTKQ_COLREG64(12)
+            CNTKQ_COLREG64(16)
+            CNTKQ_COLREG64(20)
+#undef CNTKQ_COLREG64
+            return hipErrorInvalidValue;
+        }
+    }
+};
+
 // The kernel family a matrix gets when nothing is forced.
 inline int quantize_auto_path(const double* g, const double* r_in, const double* r_out, size_t rows, size_t nbits)
 {
@@ -188,6 +226,10 @@ inline int quantize_auto_path(const double* g, const double* r_in, const double*
     // 6144: 85 against 99, 7168: 81 against 112 (4096: 104 against 85)
     if (rows >= kRegMinRows && reg_applicable(g, r_in, r_out, rows, nbits))
         return kPathReg;
+    // from 1025 rows up to there, and where the register kernel's alignment conditions fail up to 5120 rows, the column
+    // stays in registers element by element
+    if (rows >= kColRegMinRows && colreg_applicable(rows, nbits))
+        return kPathRegScalar;
     return rows <= kTileMaxRows ? kPathTile : kPathTall;
 }
 
@@ -206,6 +248,13 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* 
             return hipErrorInvalidValue;
         return dispatch_nbits64<RegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols,
                                              make_reg_geom(rows, nbits, reg_line_shift(r_in, rows)));
+    }
+    if (path == kPathRegScalar)
+    {
+        if (!colreg_applicable(rows, nbits))
+            return hipErrorInvalidValue;
+        return dispatch_nbits64<ColRegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) rows, (uint32_t) cols,
+                                                (uint32_t) qwords_per_col(rows, nbits), (uint64_t) qcol_bytes(nbits, rows));
     }
     if (path == kPathTile)
     {

@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 
 F64 = np.float64
 VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False), (64, False)]
-PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG = 0, 1, 2, 3, 4
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG, PATH_REGS = 0, 1, 2, 3, 4, 5
 
 
 def say(*a):
@@ -139,6 +139,9 @@ PATH_CASES = [
     (4, 3, PATH_REG, 0), (70, 3, PATH_REG, 0), (1000, 5, PATH_REG, 0), (7170, 3, PATH_REG, 0), (9304, 3, PATH_REG, 0),
     (20000, 3, PATH_AUTO, 0), (32770, 2, PATH_REG, 0), (51200, 1, PATH_AUTO, 0), (51202, 1, PATH_AUTO, 0),
     (5, 3, PATH_REG, 0), (1001, 3, PATH_REG, 0), (9305, 3, PATH_AUTO, 0), (20001, 2, PATH_AUTO, 0), (50257, 1, PATH_AUTO, 0),
+    # one workgroup of 256 threads per column, the column in registers element by element: 1025 to 5120 rows
+    (1025, 3, PATH_REGS, 0), (2048, 5, PATH_REGS, 0), (2049, 3, PATH_AUTO, 0), (3073, 3, PATH_REGS, 0), (4096, 3, PATH_AUTO, 0),
+    (4991, 2, PATH_AUTO, 0), (5120, 2, PATH_REGS, 0), (4099, 2, PATH_REGS, 0),
 ]
 
 
@@ -150,7 +153,8 @@ def test_kernel_paths_f64(case):
     rep = parity.Report()
     for nbits, zt in VARIANTS:
         say("f64 path case", case, "nbits", nbits, "zeroThr", zt)
-        if path == PATH_REG and (nbits == 64 or (48 + oracle.qwords_per_col(rows, nbits, F64)) * 8 > 65536):
+        if (path == PATH_REGS and nbits == 64) or \
+                (path == PATH_REG and (nbits == 64 or (48 + oracle.qwords_per_col(rows, nbits, F64)) * 8 > 65536)):
             # whole-QWord codes and columns whose QWords exceed 64 KB of LDS are refused when forced
             with pytest.raises(cntk_amd.QuantizerLogicError):
                 gpu_quantize(qz, datagen.normal(1, rows, cols, dtype=F64), zeros(rows, cols), nbits, zt)
@@ -166,6 +170,38 @@ def test_kernel_paths_f64(case):
     say("  ", rep)
 
 
+@pytest.mark.parametrize("rows,cols", [(1025, 7), (2048, 9), (3000, 5), (4097, 4), (4990, 3), (5120, 3)])
+def test_element_register_kernel_gives_the_tile_kernels_bytes_f64(rows, cols):
+    """The 256-thread register kernel adds in the order of the one-column tile, so both give the same bytes (which is what
+    lets the tile stripe reduction reproduce a call sequence that quantizes with either); matrices 8 bytes off a 16-byte
+    boundary included."""
+    qa, qb = MatrixQuantizerImpl.Create(0, False), MatrixQuantizerImpl.Create(0, False)
+    qa._set_tuning(quantize_path=PATH_TILE)
+    qb._set_tuning(quantize_path=PATH_REGS)
+    for nbits, zt in VARIANTS:
+        if nbits == 64:
+            continue
+        for off in (0, 1):
+            say("tile against element registers", rows, cols, nbits, zt, "offset", off)
+            g = datagen.normal_with_outliers(17 * rows + nbits + off, rows, cols, 0.01, dtype=F64)
+            r = datagen.normal(19 * rows + nbits + off, rows, cols, 0.003, dtype=F64)
+            outs = []
+            for qz in (qa, qb):
+                n = rows * cols
+                gbuf = torch.zeros(n + 2, dtype=torch.float64, device="cuda:0")
+                rbuf = torch.zeros(n + 2, dtype=torch.float64, device="cuda:0")
+                gbuf[off:off + n].copy_(torch.from_numpy(np.ascontiguousarray(g.T).reshape(-1)))
+                rbuf[off:off + n].copy_(torch.from_numpy(np.ascontiguousarray(r.T).reshape(-1)))
+                G, R = Matrix(rows, cols, 0, gbuf[off:off + n]), Matrix(rows, cols, 0, rbuf[off:off + n])
+                Q = QuantizedMatrix(rows, cols, nbits, 0, dtype=torch.float64)
+                qz.QuantizeAsync(G, R, Q, R, zt)
+                qz.WaitQuantizeAsyncDone()
+                torch.cuda.synchronize()
+                outs.append((Q.to_numpy(), R.to_numpy()))
+            assert np.array_equal(outs[0][0], outs[1][0]), ("packed", rows, cols, nbits, zt, off)
+            assert parity.bits_equal(outs[0][1], outs[1][1]), ("residual", rows, cols, nbits, zt, off)
+
+
 def test_unsupported_paths_are_refused_f64():
     qz = MatrixQuantizerImpl.Create(0, False)
     qz._set_tuning(quantize_path=PATH_COL)  # exists for float only
@@ -174,6 +210,10 @@ def test_unsupported_paths_are_refused_f64():
     qz._set_tuning(quantize_path=PATH_TILE)
     with pytest.raises(cntk_amd.QuantizerLogicError):
         gpu_quantize(qz, datagen.normal(1, 7169, 2, dtype=F64), zeros(7169, 2), 1, False)
+    qz._set_tuning(quantize_path=PATH_REGS)  # 1025 to 5120 rows
+    for rows in (1024, 5121):
+        with pytest.raises(cntk_amd.QuantizerLogicError):
+            gpu_quantize(qz, datagen.normal(1, rows, 2, dtype=F64), zeros(rows, 2), 1, False)
 
 
 def test_unquantize_variants_f64(quantizer):
