@@ -33,7 +33,7 @@ def main():
     ap.add_argument("--steps", type=int, default=40)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--path", type=int, default=0, help="force a quantize kernel: 1 tile, 2 tall (re-reading), 3 column in LDS, 4 column in registers (16-byte accesses), "
-                    "5 column in registers (4-byte accesses)")
+                    "5 column in registers (one element per access)")
     ap.add_argument("--unq-mode", type=int, default=0, help="decoder choice: 0 automatic, 1 QWord-major with one store per value, 2 tile decoder, 3 automatic without the tile "
                     "decoder, 4 row-major decoder")
     ap.add_argument("--budget-mb", type=int, default=1600, help="device memory for the rotating buffer sets")
