@@ -14,7 +14,7 @@ extern "C" {
  *                    4 = one workgroup per column, column in registers, 16-byte accesses (below 32 (fp64: 64) bits; the
  *                        three matrices at the same offset within 16 bytes),
  *                    5 = the same with one element per access: fp32 any alignment, up to 98304 rows; fp64 256 threads per
- *                        column, 1025 to 5120 rows, below 64 bits, the bytes of path 1
+ *                        column, 1025 to 6144 rows, below 64 bits, the bytes of path 1
  *   tile_gs          0 = automatic, else threads per column in the tile statistics phase (power of two, 8..256)
  *   unq_slots        0 = automatic, else bit positions decoded per thread by the QWord-major unquantize
  *   unq_mode         0 = automatic, 1 = QWord-major decoder with one store per value, 2 = tile decoder wherever it can run,

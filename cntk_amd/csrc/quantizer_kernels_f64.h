@@ -392,7 +392,7 @@ __global__ __launch_bounds__(kThreads) void quantize_tile_kernel(const double* _
 // ---- one 256-thread workgroup per column, the column in registers element by element ------------------------
 //
 // For the heights at which the tile kernel holds a single column per tile (more than 1024 rows) and that column starts to
-// crowd LDS (16 KB at 2048 rows, 39 KB at 4991): thread t keeps rows t, t + 256, ... (at most EPT of them) from the loads
+// crowd LDS (16 KB at 2048 rows, 48 KB at 6144): thread t keeps rows t, t + 256, ... (at most EPT of them) from the loads
 // to the residual store, LDS holds only the reduction slots and the column's QWords (assembled by atomic OR), and the
 // occupancy no longer falls with the height. Nothing depends on alignment: every access is one double, consecutive
 // threads on consecutive rows. The sums are taken exactly as tile_stats takes them for a one-column tile -- a thread adds

@@ -113,7 +113,7 @@ struct StripeLauncher
 // at most 25 pieces of two doubles for each of 1024 threads, QWords within 64 KB of LDS.
 constexpr uint32_t kRegThreads = 1024;
 constexpr size_t kRegMaxRows = 2 * 1024 * 25;
-constexpr size_t kRegMinRows = 4992; // below, the tile kernel is faster
+constexpr size_t kRegMinRows = 6145; // up to 6144 rows the element-wise register kernel and the tile stripe reduction are faster
 
 inline bool reg_applicable(const double* g, const double* r_in, const double* r_out, size_t rows, size_t nbits)
 {
@@ -180,9 +180,9 @@ struct RegLauncher
     }
 };
 
-// The element-wise register kernel (256 threads, up to 20 rows each): the heights at which the tile kernel holds one column
+// The element-wise register kernel (256 threads, up to 24 rows each): the heights at which the tile kernel holds one column
 // per tile, any alignment, below 64 bits. Same bytes as the tile kernel in its default geometry.
-constexpr size_t kColRegMaxRows = 256 * 20;
+constexpr size_t kColRegMaxRows = 256 * 24;
 constexpr size_t kColRegMinRows = 1025; // the whole range: 1028 rows 87 us against 108 us on 18.5 M elements, 4096: 76 against 86
 
 inline bool colreg_applicable(size_t rows, size_t nbits)
@@ -212,6 +212,7 @@ struct ColRegLauncher
             CNTKQ_COLREG64(12)
             CNTKQ_COLREG64(16)
             CNTKQ_COLREG64(20)
+            CNTKQ_COLREG64(24)
 #undef CNTKQ_COLREG64
             return hipErrorInvalidValue;
         }
@@ -221,13 +222,11 @@ struct ColRegLauncher
 // The kernel family a matrix gets when nothing is forced.
 inline int quantize_auto_path(const double* g, const double* r_in, const double* r_out, size_t rows, size_t nbits)
 {
-    // one column of doubles per tile fills LDS from about 5000 rows on (two workgroups per CU at 5120 rows, one at
-    // 7168); the register kernel overtakes the tile kernel there: 5120 rows 88 us against 94 us on 19 M elements,
-    // 6144: 85 against 99, 7168: 81 against 112 (4096: 104 against 85)
+    // from 1025 to 6144 rows the column stays in registers element by element (256 threads); above, the 1024-thread
+    // register kernel is faster (7168 rows on 19 M elements: 78 us against 81 us, and the stripe reduction that has to
+    // follow the quantize kernel's order of additions 161 us against 202 us; at 6144 rows 77 against 75 and 164 against 126)
     if (rows >= kRegMinRows && reg_applicable(g, r_in, r_out, rows, nbits))
         return kPathReg;
-    // from 1025 rows up to there, and where the register kernel's alignment conditions fail up to 5120 rows, the column
-    // stays in registers element by element
     if (rows >= kColRegMinRows && colreg_applicable(rows, nbits))
         return kPathRegScalar;
     return rows <= kTileMaxRows ? kPathTile : kPathTall;

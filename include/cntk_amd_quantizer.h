@@ -217,8 +217,8 @@ int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h);
  *   - packed matrix: cols records { double lower; double upper; uint64_t bits[nq]; }, nq = ceil(rows / (64 / nbits)),
  *     element i in bits[i % nq] at bit (i / nq) * nbits; the buffer must be 8-byte aligned;
  *   - nbits one of 1, 2, 4, 8, 16, 32, 64 (64 = pass-through; 32 is a real quantizer with 2^32 - 1 steps);
- *   - stripe reduction: rows <= 7168.
- * The gradient-set (batch) calls exist for float only. */
+ *   - stripe reduction: rows <= cntkq_stripe_reduce_max_rows_f64(nbits).
+ * The gradient-set (batch) calls have their _f64 forms further down. */
 
 /* ColumnQuantizer<double>::QWordsPerCol, QuantizedColumn<double>::QuantizedColumnSize, QuantizedMatrix<double>::GetSize. */
 size_t cntkq_qwords_per_col_f64(size_t rows, size_t nbits);

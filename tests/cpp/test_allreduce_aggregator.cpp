@@ -369,11 +369,11 @@ static void BufferedAggregation()
 }
 
 // The double instantiation (the reference's end-to-end 1-bit tests run in double precision): the reference's arrangement
-// of calls against fused stripe reduction + batched calls, bit for bit, over carried steps (tile kernels up to 4991 rows,
-// register kernels above; 52000 rows are too tall for the fused reduction and keep the call sequence).
+// of calls against fused stripe reduction + batched calls, bit for bit, over carried steps (tile and 256-thread register kernels up to 6144 rows,
+// 1024-thread register kernels above; 52000 rows are too tall for the fused reduction and keep the call sequence).
 static void DoublePrecisionVariantsAreBitIdentical()
 {
-    const Shapes shapes = {{2048, 12}, {429, 17}, {64, 5}, {1, 9}, {4096, 4}, {147, 3}, {6000, 6}, {52000, 3}};
+    const Shapes shapes = {{2048, 12}, {429, 17}, {64, 5}, {1, 9}, {4096, 4}, {147, 3}, {6000, 6}, {7000, 4}, {52000, 3}};
     const size_t K = 3;
     for (int nBits : {1, 8})
     {

@@ -139,9 +139,10 @@ PATH_CASES = [
     (4, 3, PATH_REG, 0), (70, 3, PATH_REG, 0), (1000, 5, PATH_REG, 0), (7170, 3, PATH_REG, 0), (9304, 3, PATH_REG, 0),
     (20000, 3, PATH_AUTO, 0), (32770, 2, PATH_REG, 0), (51200, 1, PATH_AUTO, 0), (51202, 1, PATH_AUTO, 0),
     (5, 3, PATH_REG, 0), (1001, 3, PATH_REG, 0), (9305, 3, PATH_AUTO, 0), (20001, 2, PATH_AUTO, 0), (50257, 1, PATH_AUTO, 0),
-    # one workgroup of 256 threads per column, the column in registers element by element: 1025 to 5120 rows
+    # one workgroup of 256 threads per column, the column in registers element by element: 1025 to 6144 rows
     (1025, 3, PATH_REGS, 0), (2048, 5, PATH_REGS, 0), (2049, 3, PATH_AUTO, 0), (3073, 3, PATH_REGS, 0), (4096, 3, PATH_AUTO, 0),
-    (4991, 2, PATH_AUTO, 0), (5120, 2, PATH_REGS, 0), (4099, 2, PATH_REGS, 0),
+    (4991, 2, PATH_AUTO, 0), (5120, 2, PATH_REGS, 0), (4099, 2, PATH_REGS, 0), (6144, 2, PATH_AUTO, 0), (6143, 2, PATH_AUTO, 0),
+    (6146, 2, PATH_AUTO, 0),
 ]
 
 
@@ -170,7 +171,7 @@ def test_kernel_paths_f64(case):
     say("  ", rep)
 
 
-@pytest.mark.parametrize("rows,cols", [(1025, 7), (2048, 9), (3000, 5), (4097, 4), (4990, 3), (5120, 3)])
+@pytest.mark.parametrize("rows,cols", [(1025, 7), (2048, 9), (3000, 5), (4097, 4), (4990, 3), (5120, 3), (6144, 2)])
 def test_element_register_kernel_gives_the_tile_kernels_bytes_f64(rows, cols):
     """The 256-thread register kernel adds in the order of the one-column tile, so both give the same bytes (which is what
     lets the tile stripe reduction reproduce a call sequence that quantizes with either); matrices 8 bytes off a 16-byte
@@ -210,8 +211,8 @@ def test_unsupported_paths_are_refused_f64():
     qz._set_tuning(quantize_path=PATH_TILE)
     with pytest.raises(cntk_amd.QuantizerLogicError):
         gpu_quantize(qz, datagen.normal(1, 7169, 2, dtype=F64), zeros(7169, 2), 1, False)
-    qz._set_tuning(quantize_path=PATH_REGS)  # 1025 to 5120 rows
-    for rows in (1024, 5121):
+    qz._set_tuning(quantize_path=PATH_REGS)  # 1025 to 6144 rows
+    for rows in (1024, 6145):
         with pytest.raises(cntk_amd.QuantizerLogicError):
             gpu_quantize(qz, datagen.normal(1, rows, 2, dtype=F64), zeros(rows, 2), 1, False)
 
@@ -347,7 +348,7 @@ def stripe_max_rows_f64(nbits):
 
 
 @pytest.mark.parametrize("rows,n,k", [(70, 9, 3), (429, 12, 4), (2048, 20, 8), (4096, 3, 2), (4988, 3, 3), (4992, 3, 3), (5003, 2, 2),
-                                      (7168, 2, 5), (64, 40, 64), (8000, 2, 3), (20001, 2, 2), (51184, 1, 2)])
+                                      (6144, 2, 3), (6145, 2, 2), (6148, 3, 3), (7168, 2, 5), (64, 40, 64), (8000, 2, 3), (20001, 2, 2), (51184, 1, 2)])
 def test_stripe_reduce_f64(quantizer, rows, n, k):
     for nbits, zt in VARIANTS:
         if rows > stripe_max_rows_f64(nbits):
