@@ -178,6 +178,34 @@ __device__ __forceinline__ void tile_store(const float* tile, uint32_t mis, floa
     }
 }
 
+// The reverse: a coalesced copy of `total` floats into the tile (same phase rule).
+__device__ __forceinline__ void tile_load(float* tile, uint32_t mis, const float* src, uint32_t total, const TileGeom& t)
+{
+    const uint32_t tid = threadIdx.x;
+    const uint32_t mis_s = (uint32_t) ((reinterpret_cast<uintptr_t>(src) >> 2) & 3u);
+    if (mis_s == mis)
+    {
+        uint32_t head = (4u - mis) & 3u;
+        if (head > total)
+            head = total;
+        const uint32_t nvec = (total - head) >> 2;
+        const uint32_t tail0 = head + (nvec << 2);
+        if (tid < head)
+            tile[tid] = src[tid];
+        f32x4* t4 = reinterpret_cast<f32x4*>(tile + head);
+        const f32x4* s4 = reinterpret_cast<const f32x4*>(src + head);
+        for (uint32_t e = tid; e < nvec; e += t.threads)
+            t4[e] = __builtin_nontemporal_load(s4 + e);
+        for (uint32_t e = tail0 + tid; e < total; e += t.threads)
+            tile[e] = src[e];
+    }
+    else
+    {
+        for (uint32_t e = tid; e < total; e += t.threads)
+            tile[e] = __builtin_nontemporal_load(src + e);
+    }
+}
+
 // ---- quantize: gradient + residual -> packed codes + new residual -----------------------------------
 
 template <int NBITS, bool ZT>
@@ -310,6 +338,12 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
         for (uint32_t x = tid; x < nwords; x += t.threads)
             words[x] = 0u;
 
+    // the stripe residual comes in as one consecutive run where it also leaves as one: a work item's rows lie nq apart, and
+    // short columns (few QWords) would otherwise be read in fragments
+    const bool staged = t.stage_residual != 0;
+    if (staged)
+        tile_load(tile, mis_s, sp, total, t);
+
     // decode constants from every worker's column header, stored in summation order:
     // 1 bit -> the two levels, else (ufactor, lower)
     for (uint32_t x = tid; x < nc * K; x += t.threads)
@@ -382,7 +416,7 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
             {
                 if (agg_out != nullptr)
                     agg_out[base + (size_t) c * t.rows + i] = acc[kk];
-                colv[i] = acc[kk] + __builtin_nontemporal_load(sc + i);
+                colv[i] = acc[kk] + (staged ? colv[i] : __builtin_nontemporal_load(sc + i));
             }
         }
     }
