@@ -8,10 +8,14 @@ One step = QuantizeAsync (gradient + carried residual -> packed codes + new resi
 finds its inputs in the 256 MB Infinity Cache. Prints ONE JSON line.
 
   value     algorithmic GB/s of the whole step: (16 + nbits/4) bytes per element + 16 bytes per column
-            = 309,790,784 bytes for 2048 x 9304 at 1 bit, divided by the step time
+            = 309,785,984 bytes for 2048 x 9304 at 1 bit, divided by the step time. The step time is the host clock
+            around exactly K steps between two device synchronisations; nothing but the 2 K calls is issued in
+            between, so with few steps the launch latency of the first kernel and the return of the closing wait
+            are part of it (a 20-step run is about 1 ms long). gpu_timeline_ms_per_step, from a second pass of the
+            same K steps, is first kernel start -> last kernel end by dispatch-attached events.
   roofline  the dominant kernel (quantize): algorithmic bytes per launch (12 + nbits/8 per element + 8 per column
-            = 231,116,664) over its average duration measured with HIP events on the launch stream, against
-            8 TB/s of HBM
+            = 231,116,664) over its average duration measured with HIP events on the launch stream in a third,
+            untimed pass of the same steps, against 8 TB/s of HBM
   cpu_baseline  the CPU oracle (a port of the reference's MatrixQuantizerCPU) timed on this host, single thread
             like the reference, on the same matrix
 """
@@ -26,7 +30,10 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 ROWS, COLS, NBITS = 2048, 9304, 1
-SETUP_STEPS = 50  # untimed steps before the warm-up steps the caller asks for (handle, streams, clocks)
+# untimed set-up before the warm-up steps the caller asks for (handle, streams, clocks): at least this many steps and
+# this much time
+SETUP_STEPS = 50
+SETUP_SECONDS = 0.5
 HBM_PEAK_GBS = 8000.0
 
 
@@ -94,6 +101,28 @@ def cpu_baseline(budget_s=12.0):
     }
 
 
+TRAFFIC_PROFILE = os.path.join("profiles", "quantize_unquantize_2048x9304_1bit.md")
+
+
+def profiled_traffic():
+    """HBM bytes per launch of the quantize kernel from the committed counter summary (a line
+    `traffic_bytes_per_launch quantize = N` in it), with the file it came from; (None, None) if there is none."""
+    import re
+
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
+            m = re.search(r"^traffic_bytes_per_launch quantize = (\d+)", f.read(), re.M)
+    except OSError:
+        return None, None
+    if not m:
+        return None, None
+    return int(m.group(1)), TRAFFIC_PROFILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a plain copy of known size)"
+
+
+def rnd(x, n):
+    return None if x is None else round(x, n)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -102,10 +131,10 @@ def main():
     ap.add_argument("--zero-threshold", type=int, default=0, help="zeroThresholdFor1Bit (default off, as in config 1)")
     ap.add_argument("--sets", type=int, default=6, help="rotating buffer sets (each 231 MB)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-events", action="store_true", help="no per-kernel HIP events in the timed region")
-    ap.add_argument("--event-every", type=int, default=8,
-                    help="attach timing events to the kernels of every n-th step (creating a profiled dispatch costs "
-                         "the host ~25 us, so doing it on every step would leave the GPU waiting for the host)")
+    ap.add_argument("--no-events", action="store_true",
+                    help="skip the two untimed passes that carry HIP events (GPU timeline, kernel durations)")
+    ap.add_argument("--event-every", type=int, default=2,
+                    help="kernel-duration pass: attach timing events to the kernels of every n-th step")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="instead of the benchmark, run plain device copies of one 2048x9304 fp32 matrix "
                          "(76,218,368 bytes read and as many written per copy), for scaling hardware counters")
@@ -184,38 +213,70 @@ def main():
         if rc1 or rc2:
             raise RuntimeError(L.cntkq_last_error().decode())
 
-    # set-up, outside warm-up and timing: first calls create streams and events, and the clocks need some work to come up
-    for i in range(SETUP_STEPS):
-        step(i)
-    torch.cuda.synchronize()
+    # set-up, outside warm-up and timing: first calls create streams and events, and the GPU needs some tenths of a
+    # second of steady work before its clocks and memory system reach the state a training job runs in (measured: the
+    # same kernels take 38.9 + 13.4 us in the first milliseconds after start-up and 37.7 + 12.6 us from then on)
+    setup_steps = 0
+    t_setup = time.perf_counter()
+    while setup_steps < SETUP_STEPS or time.perf_counter() - t_setup < SETUP_SECONDS:
+        for i in range(50):
+            step(setup_steps + i)
+        setup_steps += 50
+        torch.cuda.synchronize()
+    setup_s = time.perf_counter() - t_setup
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
 
-    # timed region: exactly `steps` steps, host clock around a synchronize on both sides
-    events = {}
-    if not args.no_events:
-        events = {i: [new_event() for _ in range(4)] for i in range(0, args.steps, max(1, args.event_every))}
-    torch.cuda.synchronize()
+    # Timed region: exactly `steps` steps and nothing else, host clock around a device synchronisation on both sides.
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(args.warmup + i, events.get(i))
+        step(args.warmup + i)
     t_enqueued = time.perf_counter()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-
     sec_per_step = (t1 - t0) / args.steps
-    if args.no_events:
-        q_ms = u_ms = float("nan")
-    else:
+
+    # Second pass, not part of `value`: the same steps again with a start event tied to the first dispatch and a stop
+    # event to the last one, i.e. the GPU's own time for the K steps including the gaps between dependent launches but
+    # without the launch latency of the first kernel and the return of the closing wait.
+    # Third pass: start/stop events on the two kernels of every n-th step, for the kernel durations of `roofline`.
+    # Creating a profiled dispatch costs the host about 25 us, which is why neither is done inside the timed region.
+    timeline_ms = q_ms = u_ms = None
+    n_timed = 0
+    if not args.no_events:
+        first, last = new_event(), new_event()
+        none = ctypes.c_void_p()
+        for i in range(args.steps):
+            g, r, q, o = ptrs[(args.warmup + i) % len(ptrs)]
+            if i == 0:
+                L.cntkq_debug_attach_events(h, first, none)
+            rc1 = L.cntkq_quantize_async(h, g, r, ROWS, COLS, q, qbytes, 0, NBITS, r, izt)
+            if i == args.steps - 1:
+                L.cntkq_debug_attach_events(h, none, last)
+            rc2 = L.cntkq_unquantize_async(h, q, qbytes, 0, o, ROWS, COLS, NBITS, 0)
+            if rc1 or rc2:
+                raise RuntimeError(L.cntkq_last_error().decode())
+        torch.cuda.synchronize()
+        timeline_ms = elapsed_ms(first, last) / args.steps
+        hip.hipEventDestroy(first)
+        hip.hipEventDestroy(last)
+
+        every = max(1, args.event_every)
+        events = {i: [new_event() for _ in range(4)] for i in range(0, args.steps, every)}
+        for i in range(args.steps):
+            step(args.warmup + i, events.get(i))
+        torch.cuda.synchronize()
         q_ms = sum(elapsed_ms(e[0], e[1]) for e in events.values()) / len(events)
         u_ms = sum(elapsed_ms(e[2], e[3]) for e in events.values()) / len(events)
+        n_timed = len(events)
         for e in events.values():
             for x in e:
                 hip.hipEventDestroy(x)
     qb, ub = algorithmic_bytes(ROWS, COLS, NBITS)
     total = qb + ub
-    achieved = qb / (q_ms * 1e-3) / 1e9
+    achieved = qb / (q_ms * 1e-3) / 1e9 if q_ms else None
+    traffic, traffic_source = profiled_traffic()
 
     result = {
         "metric": "1-bit quantize+unquantize GB/s & % HBM peak, 2048x9304 fp32 gradient",
@@ -224,7 +285,8 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "setup_steps": SETUP_STEPS,
+        "setup_steps": setup_steps,
+        "setup_s": round(setup_s, 3),
         "ms_per_step": round(sec_per_step * 1e3, 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -239,19 +301,22 @@ def main():
         },
         "pct_hbm_peak": round(100.0 * total / sec_per_step / 1e9 / HBM_PEAK_GBS, 2),
         "elements_per_s": round(ROWS * COLS / sec_per_step, 1),
-        "kernel_ms": {"quantize": round(q_ms, 5), "unquantize": round(u_ms, 5), "launches_timed": len(events)},
+        "gpu_timeline_ms_per_step": rnd(timeline_ms, 5),
+        "kernel_ms": {"quantize": rnd(q_ms, 5), "unquantize": rnd(u_ms, 5), "launches_timed": n_timed},
         "host_enqueue_ms_per_step": round((t_enqueued - t0) / args.steps * 1e3, 5),
         "roofline": {
             "bound": "hbm",
             "kernel": "quantize (gradient + residual -> codes + residual)",
-            "achieved": round(achieved, 2),
+            "achieved": rnd(achieved, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            # HBM bytes per launch of the quantize kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE (two runs), each scaled
-            # by what the same counter reads for a plain 76,218,368-byte device copy (x1.99923 and x1.00000):
-            # 152.42 MB read + 78.90 MB written
-            "traffic": 231.32e6,
+            "frac": rnd(achieved / HBM_PEAK_GBS, 4) if achieved else None,
+            "algorithmic_bytes_per_launch": qb,
+            # not observed by this run: HBM bytes per launch of the quantize kernel as recorded in the committed
+            # rocprofv3 counter summary (FETCH_SIZE + WRITE_SIZE, two runs, each scaled by what the same counter
+            # reads for a plain device copy of known size); null when that file is absent
+            "traffic": traffic,
+            "traffic_source": traffic_source,
         },
     }
     if not args.no_cpu:
