@@ -84,6 +84,7 @@ def lib():
         L.cntkq_wait_stripe_reduce_done.argtypes = [_vp]
         L.cntkq_quantize_batch_async.argtypes = [_vp, ctypes.POINTER(_QuantizeItem), _sz, _sz, ctypes.c_int]
         L.cntkq_unquantize_batch_async.argtypes = [_vp, ctypes.POINTER(_UnquantizeItem), _sz, _sz, ctypes.c_int]
+        L.cntkq_quantize_batch_noalloc.argtypes = L.cntkq_quantize_batch_async.argtypes
         L.cntkq_qwords_per_col_f64.argtypes = [_sz, _sz]
         L.cntkq_qwords_per_col_f64.restype = _sz
         L.cntkq_qcol_bytes_f64.argtypes = [_sz, _sz]
@@ -406,6 +407,15 @@ class MatrixQuantizerImpl:
                                                                       int(bool(zero_threshold_for_1bit))))
             return
         self.QuantizeBatchAsync(self.PrepareQuantizeBatch(items), zero_threshold_for_1bit)
+
+    def QuantizeBatchNoAlloc(self, items, zero_threshold_for_1bit):
+        """QuantizeBatchAsync through the entry point that allocates nothing (float32 only): the argument table lives in
+        a fixed array in the library's device image; at most 256 items. No counterpart in the reference."""
+        prep = items if isinstance(items, PreparedBatch) else self.PrepareQuantizeBatch(items)
+        if prep.kind != "quantize" or _is64(prep.dtype):
+            raise QuantizerLogicError("QuantizeBatchNoAlloc: needs a float32 quantize item list")
+        if prep.count:
+            _check(lib().cntkq_quantize_batch_noalloc(self._h, prep.array, prep.count, prep.nbits, int(bool(zero_threshold_for_1bit))))
 
     @staticmethod
     def PrepareQuantizeBatch(items):

@@ -49,6 +49,53 @@ struct DeviceStreams
 DeviceStreams g_streams[kMaxDevices];
 std::mutex g_streams_mutex;
 
+// ---- the argument table of cntkq_quantize_batch_noalloc ----------------------------------------------------------
+//
+// That entry point must not allocate, so its table (entries, then the first workgroup of every member) lives in this
+// fixed array in the library's device image: every GPU the library runs on holds its own copy, at its own address,
+// until the process ends. Host code never uses the array's name as an address (in host code it is only a stand-in for
+// the symbol): scratch_for_device() asks the runtime for the copy's address on the current device, once per device, and
+// everything -- kernel arguments included -- goes through that pointer.
+constexpr size_t kNoAllocScratchBytes = 32 * 1024;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+struct DeviceScratch
+{
+    unsigned char* ptr = nullptr;        // address of `scratch` on this device
+    const void* writer = nullptr;        // the handle whose table the array holds (host-side bookkeeping)
+    uint64_t generation = 0;             // bumped on every upload
+};
+DeviceScratch g_scratch[kMaxDevices];
+
+// Call with `device` current. Returns hipSuccess once the device's address of `scratch` is known.
+hipError_t scratch_for_device(int device)
+{
+    std::lock_guard<std::mutex> lock(g_streams_mutex);
+    if (g_scratch[device].ptr != nullptr)
+        return hipSuccess;
+    void* p = nullptr;
+    hipError_t rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (rc != hipSuccess)
+        return rc;
+    if (p == nullptr)
+        return hipErrorInvalidSymbol;
+    g_scratch[device].ptr = static_cast<unsigned char*>(p);
+    return hipSuccess;
+}
+
+// The table travels to the device as kernel arguments, 2 KB per launch: no copy engine, no staging memory.
+constexpr uint32_t kChunkWords = 512;
+struct TableChunk
+{
+    uint32_t w[kChunkWords];
+};
+
+__global__ __launch_bounds__(256) void table_store_kernel(TableChunk chunk, uint32_t* dst, uint32_t words)
+{
+    for (uint32_t i = threadIdx.x; i < words; i += 256)
+        dst[i] = chunk.w[i];
+}
+
 class DeviceGuard // PrepareDevice (Source/Math/MatrixQuantizerGPU.cu:186, 234): make the handle's device current
 {
 public:
@@ -158,6 +205,32 @@ struct BatchTable
     std::vector<size_t> own;
 };
 
+// Host-side state of cntkq_quantize_batch_noalloc: everything the call needs besides the device array, at fixed size,
+// so that the call itself touches no allocator (host or device).
+struct NoAllocState
+{
+    static constexpr size_t kMaxItems = CNTKQ_NOALLOC_MAX_ITEMS;
+    static constexpr size_t kTableWords = kNoAllocScratchBytes / sizeof(uint32_t);
+    // the table as uploaded: entries of the two LDS classes, then the first-workgroup lists (with sentinels)
+    alignas(16) uint32_t table[kTableWords];
+    size_t table_words = 0;
+    // launch parameters
+    size_t members[2] = {0, 0};
+    uint32_t blocks[2] = {0, 0};
+    size_t lds[2] = {0, 0};
+    size_t first_entry[2] = {0, 0};
+    size_t first_begin[2] = {0, 0};
+    size_t entries_bytes = 0;
+    size_t own[kMaxItems];
+    size_t own_count = 0;
+    // what the table was built for, and the upload of it that the device array last received from this handle
+    cntkq_quantize_item key_items[kMaxItems];
+    size_t key_count = 0, key_nbits = 0, key_zt = 0;
+    bool key_valid = false;
+    uint64_t uploaded_generation = 0;
+    hipStream_t uploaded_stream = nullptr; // later launches on another stream would not be ordered after that upload
+};
+
 struct cntkq_quantizer
 {
     int device = 0;
@@ -194,6 +267,7 @@ struct cntkq_quantizer
     BatchTable unquantize_table64;
     BatchTable stripe_table64;
     LaunchTuning tune;
+    struct NoAllocState* noalloc = nullptr; // fixed-size host state of cntkq_quantize_batch_noalloc (created with the handle)
 };
 
 namespace {
@@ -498,6 +572,195 @@ int stripe_reduce_async_impl(cntkq_quantizer* h, const void* const* stripes, siz
 
 #include "quantizer_api_batch.inc"
 
+// ---- the gradient-set quantize that allocates nothing -----------------------------------------------------------------
+//
+// Same planning, same kernels and hence the same bytes as quantize_batch_impl<float>; what differs is where the argument
+// table lives (the fixed device array `scratch`, reached through the per-device pointer) and how it gets there (as kernel
+// arguments of table_store_kernel). Nothing on this path calls an allocator: no hipMalloc / hipHostMalloc / hipFree, no
+// host heap (the plan is built in the handle's NoAllocState), no copy that would need staging memory.
+int quantize_batch_noalloc_impl(cntkq_quantizer* h, const cntkq_quantize_item* items, size_t count, size_t nbits, int zero_threshold_for_1bit)
+{
+    typedef BatchAbi<float> A;
+    typedef QuantizeBatchEntry Entry;
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_noalloc: null handle");
+    if (!cntkq::valid_nbits(nbits))
+        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides 32 (got %zu)", nbits);
+    if (count == 0)
+        return CNTKQ_OK;
+    if (items == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_noalloc: bad item list");
+    if (count > NoAllocState::kMaxItems)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_noalloc: %zu items exceed the limit of %zu (CNTKQ_NOALLOC_MAX_ITEMS)", count,
+                    NoAllocState::kMaxItems);
+    for (size_t i = 0; i < count; ++i)
+    {
+        const cntkq_quantize_item& it = items[i];
+        if (it.rows >= (1ull << 31) || it.cols >= (1ull << 31))
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_noalloc: item %zu: rows and cols must be below 2^31", i);
+        if (it.rows == 0 || it.cols == 0)
+            continue;
+        if (it.in == nullptr || it.res_in == nullptr || it.res_out == nullptr || it.qbuf == nullptr || !aligned4(it.in) || !aligned4(it.res_in) ||
+            !aligned4(it.res_out) || !aligned4(it.qbuf))
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_noalloc: item %zu: null or misaligned pointer", i);
+    }
+    const bool zt = zero_threshold_for_1bit != 0;
+    DeviceGuard guard(h->device);
+    DeviceScratch& ds = g_scratch[h->device];
+    if (ds.ptr == nullptr || h->noalloc == nullptr)
+        return fail(CNTKQ_RUNTIME_ERROR, "cntkq_quantize_batch_noalloc: the device array was not set up when the handle was created");
+    NoAllocState& st = *h->noalloc;
+    hipStream_t s = work_stream(h);
+    const bool capturing = stream_capturing(s);
+
+    const bool same_list = st.key_valid && st.key_count == count && st.key_nbits == nbits && st.key_zt == (size_t) zt &&
+                           std::memcmp(st.key_items, items, count * sizeof(cntkq_quantize_item)) == 0;
+    if (!same_list)
+    {
+        st.key_valid = false;
+        // plan: the class of every item (-1 skip, 0 / 1 member of that LDS class, 2 a launch of its own), kept in `own`
+        // until the table is laid out
+        Entry* he = reinterpret_cast<Entry*>(st.table);
+        static_assert(sizeof(Entry) % sizeof(uint32_t) == 0 && alignof(Entry) <= 16, "table layout");
+        static_assert(sizeof(Entry) == CNTKQ_NOALLOC_ENTRY_BYTES, "the public header states the size of a table entry");
+        static_assert(CNTKQ_NOALLOC_MAX_ITEMS * (sizeof(Entry) + sizeof(uint32_t)) + 2 * sizeof(uint32_t) <= kNoAllocScratchBytes,
+                      "a list of the largest permitted size fits the fixed array");
+        // pass 1: count the members, so that the two classes can be laid out one after the other
+        size_t members[2] = {0, 0};
+        for (size_t i = 0; i < count; ++i)
+        {
+            const cntkq_quantize_item& it = items[i];
+            if (it.rows == 0 || it.cols == 0)
+                continue;
+            Entry e;
+            std::memset(&e, 0, sizeof e);
+            size_t lds = 0;
+            uint64_t blocks = 0;
+            if (A::quantize_member(it, nbits, e, lds, blocks))
+                members[lds <= kBatchSmallLds ? 0 : 1]++;
+        }
+        const bool single = members[0] + members[1] == 1; // a grid of its own is nothing to share: plain launch
+        if (single)
+            members[0] = members[1] = 0;
+        const size_t total = members[0] + members[1];
+        const size_t entries_bytes = total * sizeof(Entry);
+        const size_t need = entries_bytes + (total + 2) * sizeof(uint32_t);
+        if (need > kNoAllocScratchBytes)
+            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_noalloc: the argument table of %zu matrices (%zu bytes) exceeds the fixed "
+                                                "device array of %zu bytes", total, need, kNoAllocScratchBytes);
+        uint32_t* hb = st.table + entries_bytes / sizeof(uint32_t);
+        size_t e = 0, bpos = 0;
+        st.own_count = 0;
+        for (int cls = 0; cls < 2; ++cls)
+        {
+            st.first_entry[cls] = e;
+            st.first_begin[cls] = bpos;
+            st.lds[cls] = 0;
+            uint64_t acc = 0;
+            for (size_t i = 0; i < count && !single; ++i)
+            {
+                const cntkq_quantize_item& it = items[i];
+                if (it.rows == 0 || it.cols == 0)
+                    continue;
+                Entry en;
+                std::memset(&en, 0, sizeof en);
+                size_t lds = 0;
+                uint64_t blocks = 0;
+                if (!A::quantize_member(it, nbits, en, lds, blocks) || (lds <= kBatchSmallLds ? 0 : 1) != cls)
+                    continue;
+                en.g = it.in;
+                en.r_in = it.res_in;
+                en.r_out = it.res_out;
+                en.q = static_cast<char*>(it.qbuf);
+                he[e++] = en;
+                hb[bpos++] = (uint32_t) acc;
+                acc += blocks;
+                if (acc > 0x7FFFFFFFull)
+                    return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_noalloc: too many workgroups in one batch");
+                if (lds > st.lds[cls])
+                    st.lds[cls] = lds;
+            }
+            if (members[cls] != 0)
+                hb[bpos++] = (uint32_t) acc; // sentinel
+            st.members[cls] = members[cls];
+            st.blocks[cls] = (uint32_t) acc;
+        }
+        for (size_t i = 0; i < count; ++i)
+        {
+            const cntkq_quantize_item& it = items[i];
+            if (it.rows == 0 || it.cols == 0)
+                continue;
+            Entry en;
+            size_t lds = 0;
+            uint64_t blocks = 0;
+            if (single || !A::quantize_member(it, nbits, en, lds, blocks))
+                st.own[st.own_count++] = i;
+        }
+        st.entries_bytes = entries_bytes;
+        st.table_words = total != 0 ? entries_bytes / sizeof(uint32_t) + bpos : 0;
+        std::memcpy(st.key_items, items, count * sizeof(cntkq_quantize_item));
+        st.key_count = count;
+        st.key_nbits = nbits;
+        st.key_zt = (size_t) zt;
+        st.key_valid = true;
+        st.uploaded_generation = 0; // whatever the device array holds, it is not this table
+    }
+
+    // The device array is shared by every handle on this GPU and keeps the last call's contents: upload unless this very
+    // table is what it received last. (A recorded call always uploads: a replay must not depend on what ran before it.)
+    bool upload = st.table_words != 0;
+    {
+        std::lock_guard<std::mutex> lock(g_streams_mutex);
+        if (upload && !capturing && ds.writer == h && st.uploaded_generation != 0 && ds.generation == st.uploaded_generation &&
+            st.uploaded_stream == s)
+            upload = false;
+        if (upload)
+        {
+            ds.writer = h;
+            st.uploaded_generation = ++ds.generation;
+            st.uploaded_stream = s;
+        }
+    }
+    if (upload)
+    {
+        for (size_t w0 = 0; w0 < st.table_words; w0 += kChunkWords)
+        {
+            const uint32_t words = (uint32_t) (st.table_words - w0 < kChunkWords ? st.table_words - w0 : kChunkWords);
+            TableChunk chunk;
+            std::memcpy(chunk.w, st.table + w0, words * sizeof(uint32_t));
+            hipLaunchKernelGGL(table_store_kernel, dim3(1), dim3(256), 0, s, chunk, reinterpret_cast<uint32_t*>(ds.ptr) + w0, words);
+            HIP_TRY(hipGetLastError(), "table_store_kernel launch failed");
+        }
+    }
+
+    size_t launches_left = (st.members[0] ? 1 : 0) + (st.members[1] ? 1 : 0) + st.own_count;
+    if (launches_left == 0)
+        return CNTKQ_OK;
+    hipEvent_t done = capturing ? nullptr : h->ev_quantize;
+    for (int cls = 0; cls < 2; ++cls)
+    {
+        if (st.members[cls] == 0)
+            continue;
+        LaunchEvents ev;
+        launches_left--;
+        ev.stop = launches_left == 0 ? done : nullptr;
+        const Entry* de = reinterpret_cast<const Entry*>(ds.ptr) + st.first_entry[cls];
+        const uint32_t* db = reinterpret_cast<const uint32_t*>(ds.ptr + st.entries_bytes) + st.first_begin[cls];
+        HIP_TRY(A::launch_quantize_members(s, ev, de, db, (uint32_t) st.members[cls], st.blocks[cls], st.lds[cls], nbits, zt),
+                "batched quantize kernel launch failed");
+    }
+    for (size_t k = 0; k < st.own_count; ++k)
+    {
+        LaunchEvents ev;
+        launches_left--;
+        ev.stop = launches_left == 0 ? done : nullptr;
+        HIP_TRY(A::launch_quantize_own(s, ev, items[st.own[k]], nbits, zt), "quantize kernel launch failed");
+    }
+    h->last_quantize = done;
+    h->quantize_included_fetch = false;
+    return CNTKQ_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -604,6 +867,23 @@ int cntkq_create(int device_id, int use_dedicated_stream, cntkq_quantizer** out)
         h->fetch = ds.fetch;
         h->assign = ds.assign;
     }
+    {
+        // the no-allocation entry point's fixed state: the address of the device array on this GPU (looked up once per
+        // device, with the device current) and the handle's host-side plan space
+        hipError_t rc = scratch_for_device(device_id);
+        if (rc != hipSuccess)
+        {
+            delete h;
+            return fail(CNTKQ_RUNTIME_ERROR, "hipGetSymbolAddress of the fixed device array failed: %s (hip error %d)", hipGetErrorString(rc),
+                        (int) rc);
+        }
+        h->noalloc = new (std::nothrow) NoAllocState();
+        if (h->noalloc == nullptr)
+        {
+            delete h;
+            return fail(CNTKQ_RUNTIME_ERROR, "cntkq_create: out of host memory");
+        }
+    }
     hipEvent_t* evs[] = {&h->ev_quantize, &h->ev_fetch, &h->ev_assign, &h->ev_unquantize, &h->ev_stripe, &h->ev_main};
     for (hipEvent_t* e : evs)
     {
@@ -641,6 +921,12 @@ int cntkq_destroy(cntkq_quantizer* h)
     for (hipEvent_t e : evs)
         if (e != nullptr)
             (void) hipEventDestroy(e);
+    {
+        std::lock_guard<std::mutex> lock(g_streams_mutex);
+        if (g_scratch[h->device].writer == h)
+            g_scratch[h->device].writer = nullptr; // a later handle at the same address must upload again
+    }
+    delete h->noalloc;
     delete h;
     return CNTKQ_OK;
 }
@@ -740,6 +1026,12 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
 int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item* items, size_t count, size_t nbits, int add)
 {
     return unquantize_batch_impl<float>(h, items, count, nbits, add);
+}
+
+int cntkq_quantize_batch_noalloc(cntkq_quantizer* h, const cntkq_quantize_item* items, size_t count, size_t nbits,
+                                 int zero_threshold_for_1bit)
+{
+    return quantize_batch_noalloc_impl(h, items, count, nbits, zero_threshold_for_1bit);
 }
 
 int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows,

@@ -165,6 +165,24 @@ int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* it
                                int zero_threshold_for_1bit);
 int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item* items, size_t count, size_t nbits, int add);
 
+/* cntkq_quantize_batch_async for callers that cannot allocate. It has no counterpart in the reference; it is for code
+ * under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc. Same arguments, same kernels and the
+ * same bytes as cntkq_quantize_batch_async, but the call touches no allocator, device or host: the argument table that
+ * the batched kernels read (the only memory of that call beyond its inputs and outputs) lives in a fixed array in the
+ * library's device image -- 32 KB, held by every GPU the library runs on until the process ends -- and reaches it as
+ * kernel arguments of a small store kernel, not through a copy.
+ *   Limits: count <= CNTKQ_NOALLOC_MAX_ITEMS, and the table (CNTKQ_NOALLOC_ENTRY_BYTES + 4 bytes per matrix that shares
+ *   the grid, + 8) must fit the array -- it always does within that count; beyond the limit the call fails with
+ *   CNTKQ_INVALID_ARGUMENT and does nothing.
+ *   The array is shared by every call on that GPU and keeps the last call's contents. Calls on one stream are ordered
+ *   like any other stream work; calls that can overlap on one GPU (other streams, other handles on other streams) race
+ *   for the array and must be ordered by the caller.
+ *   cntkq_wait_quantize_done waits for the whole batch. */
+#define CNTKQ_NOALLOC_MAX_ITEMS 256
+#define CNTKQ_NOALLOC_ENTRY_BYTES 112
+int cntkq_quantize_batch_noalloc(cntkq_quantizer* h, const cntkq_quantize_item* items, size_t count, size_t nbits,
+                                 int zero_threshold_for_1bit);
+
 /* One owner's stripe reduction of the quantized all-reduce, fused into one pass
  * (dataflow of Source/1BitSGD/AllReduceDistGradAggregator.h:365-375 and :385-436; v2:
  * Source/1BitSGD/QuantizedDistributedCommunicator.h:423-471), replacing the reference's sequence
