@@ -11,7 +11,6 @@ HIPCC_FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     # the CPU reference never fuses multiply-add; bit-exact codes and residuals need the same here
     "-ffp-contract=off",
     # no packed fp32 instructions
@@ -21,19 +20,45 @@ HIPCC_FLAGS = [
 ]
 
 
-def build_library(verbose=False):
+# The library's two source files (float matrices + everything independent of the element type; double matrices) share
+# no device code and are compiled side by side.
+SOURCES = ["quantizer_api.hip", "quantizer_api_f64.hip"]
+
+
+def build_library(verbose=False, only=None):
+    """Compiles the sources (or, with `only`, just the named ones, keeping the other object files) and links the
+    library."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    src = os.path.join(HERE, "csrc", "quantizer_api.hip")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-o", LIB_PATH, src]
+    obj_dir = os.path.join(HERE, "csrc", "build")
+    os.makedirs(obj_dir, exist_ok=True)
+    procs = []
+    objs = []
+    for name in SOURCES:
+        obj = os.path.join(obj_dir, os.path.splitext(name)[0] + ".o")
+        objs.append(obj)
+        if only is not None and name not in only and os.path.exists(obj):
+            continue
+        cmd = [hipcc] + HIPCC_FLAGS + ["-c", "-o", obj, os.path.join(HERE, "csrc", name)]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((name, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
+    errors = []
+    for name, proc in procs:
+        _, stderr = proc.communicate()
+        # the host pass does not know the packed-fp32 feature and says so; that warning is harmless
+        err = "\n".join(l for l in stderr.splitlines() if "packed-fp32-ops" not in l)
+        if proc.returncode != 0:
+            errors.append("%s:\n%s" % (name, err))
+        elif verbose and err.strip():
+            print(err, file=sys.stderr)
+    if errors:
+        raise RuntimeError("hipcc failed:\n" + "\n".join(errors))
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
-    # the host pass does not know the packed-fp32 feature and says so; that warning is harmless
-    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + err)
-    if verbose and err.strip():
-        print(err, file=sys.stderr)
+        raise RuntimeError("linking the library failed:\n" + res.stderr)
     return LIB_PATH
 
 
@@ -71,5 +96,6 @@ def build_cpp_tests(verbose=False):
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    # python -m cntk_amd.build [source file names ...]: recompile only those (a development shortcut)
+    print(build_library(verbose=True, only=sys.argv[1:] or None))
     print(build_cpp_tests(verbose=True))

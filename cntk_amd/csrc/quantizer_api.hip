@@ -1,53 +1,151 @@
-// C ABI of the MI355X gradient quantizer: handles, streams, events, argument checks.
+// C ABI of the MI355X gradient quantizer: handles, streams, events, argument checks; the calls on float matrices.
 // Replaces the host side of the reference's GPU quantizer (Source/Math/MatrixQuantizerGPU.cu:83-341).
-#include "../../include/cntk_amd_quantizer.h"
-#include "quantizer_internal.h"
-#include "quantizer_launch.h"
-#include "quantizer_launch_f64.h"
-
-#include <hip/hip_runtime.h>
-
-#include <cstdarg>
-#include <cstdio>
-#include <cstring>
-#include <mutex>
-#include <new>
-#include <vector>
+#include "quantizer_api_shared.h"
 
 using namespace cntkq;
+using namespace cntkq_api;
+
+namespace cntkq_api {
+
+template <>
+struct Elem<float>
+{
+    static constexpr size_t kAlign = 4;
+    static constexpr size_t kWordBits = 32;
+    static size_t stripe_max_rows(size_t nbits) { return cntkq::stripe_reduce_max_rows(nbits); }
+    static bool valid_nbits(size_t nbits) { return cntkq::valid_nbits(nbits); }
+    static size_t qcol_bytes(size_t nbits, size_t rows) { return cntkq::qcol_bytes(nbits, rows); }
+    static hipError_t quantize(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, void* q, size_t rows,
+                               size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+    {
+        return cntkq::launch_quantize(s, ev, g, r_in, r_out, q, rows, cols, nbits, zt, tune);
+    }
+    static hipError_t unquantize(hipStream_t s, LaunchEvents ev, const void* q, float* out, size_t rows, size_t cols, size_t nbits,
+                                 bool add, const LaunchTuning& tune)
+    {
+        return cntkq::launch_unquantize(s, ev, q, out, rows, cols, nbits, add, tune);
+    }
+    static hipError_t stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, void* q_out,
+                                    float* agg_out, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+    {
+        return cntkq::launch_stripe_reduce(s, ev, src, stripe_res, q_out, agg_out, rows, cols, nbits, zt, tune);
+    }
+};
+
+
+template <>
+struct BatchAbi<float>
+{
+    typedef cntkq_quantize_item QItem;
+    typedef cntkq_unquantize_item UItem;
+    typedef cntkq_stripe_reduce_item SItem;
+    typedef QuantizeBatchEntry QEntry;
+    typedef UnquantizeBatchEntry UEntry;
+    typedef StripeBatchEntry SEntry;
+    static const char* suffix() { return ""; }
+    static unsigned word_bits() { return 32; }
+    static bool valid_nbits(size_t nbits) { return cntkq::valid_nbits(nbits); }
+    static bool aligned(const void* p) { return aligned4(p); }
+    static BatchTable& quantize_table(cntkq_quantizer* h) { return h->quantize_table; }
+    static BatchTable& unquantize_table(cntkq_quantizer* h) { return h->unquantize_table; }
+    static BatchTable& stripe_table(cntkq_quantizer* h) { return h->stripe_table; }
+
+    // Fills the geometry of a member of the quantize grid; false: the matrix gets a launch of its own.
+    static bool quantize_member(const QItem& it, size_t nbits, QEntry& e, size_t& lds, uint64_t& blocks)
+    {
+        const int path = quantize_auto_path(it.in, it.res_in, it.res_out, it.qbuf, it.rows, nbits);
+        if (path == kPathTile)
+        {
+            e.kind = 0;
+            e.t = make_tile_geom(it.rows, it.cols, nbits, 0, -1, 0);
+            lds = tile_lds_bytes(e.t, 0);
+            blocks = (e.t.cols + e.t.cols_per_tile - 1) / e.t.cols_per_tile;
+            return true;
+        }
+        // (a register-kernel matrix of modest size gives the same bytes as a member: a launch costs more than it gains)
+        if (path == kPathCol || (path == kPathReg && it.rows <= kTileMaxRows && it.rows * it.cols < kOwnLaunchElements))
+        {
+            e.kind = 1;
+            e.c = make_col_geom(it.rows, nbits, quantize_line_shift(it.in, it.res_in, it.res_out, it.rows));
+            lds = colg_lds_bytes_rt(e.c, nbits);
+            blocks = it.cols;
+            return true;
+        }
+        return false;
+    }
+    static hipError_t launch_quantize_members(hipStream_t s, LaunchEvents ev, const QEntry* de, const uint32_t* db, uint32_t members,
+                                              uint32_t blocks, size_t lds, size_t nbits, bool zt)
+    {
+        return launch_quantize_batch(s, ev, de, db, members, blocks, lds, nbits, zt);
+    }
+    static hipError_t launch_quantize_own(hipStream_t s, LaunchEvents ev, const QItem& it, size_t nbits, bool zt)
+    {
+        LaunchTuning autotune;
+        return launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune);
+    }
+
+    static int unquantize_one(cntkq_quantizer* h, const UItem& it, size_t nbits, int add)
+    {
+        return cntkq_unquantize_async(h, it.qbuf, qcol_bytes(nbits, it.rows) * it.cols, 0, it.out, it.rows, it.cols, nbits, add);
+    }
+    static bool unquantize_member(const UItem& it, size_t nbits, UEntry& e, size_t& lds, uint64_t& blocks)
+    {
+        LaunchTuning autotune;
+        const UnquantizePlan p = plan_unquantize(it.qbuf, it.out, it.rows, it.cols, nbits, autotune);
+        if (!p.ok)
+            return false;
+        e.kind = p.kind;
+        e.qw = p.qw;
+        e.seg = p.seg;
+        e.rowg = p.rowg;
+        e.tile = p.tile;
+        lds = p.lds;
+        blocks = p.blocks;
+        return true;
+    }
+    static hipError_t launch_unquantize_members(hipStream_t s, LaunchEvents ev, const UEntry* de, const uint32_t* db, uint32_t members,
+                                                uint32_t blocks, size_t nbits, bool add, size_t lds)
+    {
+        return launch_unquantize_batch(s, ev, de, db, members, blocks, nbits, add, lds);
+    }
+
+    static size_t stripe_max_rows(size_t nbits) { return stripe_reduce_max_rows(nbits); }
+    // taller stripes run 1024 threads per column: a launch of their own
+    static bool stripe_is_member(const SItem& it, size_t) { return it.rows <= kTileMaxRows; }
+    static int stripe_one(cntkq_quantizer* h, const SItem& it, size_t workers, size_t owner, size_t nbits, int zt)
+    {
+        return cntkq_stripe_reduce_async(h, it.stripes, workers, owner, it.rows, it.stripe_cols, nbits, it.stripe_res, it.q_out, it.agg_out, zt);
+    }
+    // the kernel family the plain call would take, so that both give the same bytes; false: does not fit the kernel
+    static bool stripe_member(const SItem& it, size_t workers, size_t nbits, SEntry& e, size_t& lds, uint64_t& blocks)
+    {
+        if (stripe_auto_col(it.rows))
+        {
+            e.kind = 1;
+            e.c = make_col_geom(it.rows, nbits, !columns_start_on_lines(it.stripe_res, it.rows));
+            lds = colg_lds_bytes_rt(e.c, nbits) + 2 * workers * sizeof(float);
+            blocks = it.stripe_cols;
+        }
+        else
+        {
+            e.kind = 0;
+            e.t = make_tile_geom(it.rows, it.stripe_cols, nbits, 0, -1, 0);
+            lds = tile_lds_bytes(e.t, (uint32_t) workers);
+            blocks = (e.t.cols + e.t.cols_per_tile - 1) / e.t.cols_per_tile;
+        }
+        return true;
+    }
+    static hipError_t launch_stripe_members(hipStream_t s, LaunchEvents ev, const SEntry* de, const uint32_t* db, uint32_t members,
+                                            uint32_t blocks, size_t lds, size_t nbits, bool zt)
+    {
+        return launch_stripe_reduce_batch(s, ev, de, db, members, blocks, lds, nbits, zt);
+    }
+};
+
+
+} // namespace cntkq_api
 
 namespace {
-
-thread_local char g_last_error[1024] = "";
-
-int fail(int code, const char* fmt, ...)
-{
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_last_error, sizeof g_last_error, fmt, ap);
-    va_end(ap);
-    return code;
-}
-
-#define HIP_TRY(call, what)                                                                                          \
-    do                                                                                                               \
-    {                                                                                                                \
-        hipError_t rc__ = (call);                                                                                    \
-        if (rc__ != hipSuccess)                                                                                      \
-            return fail(CNTKQ_RUNTIME_ERROR, "%s: %s (hip error %d)", what, hipGetErrorString(rc__), (int) rc__);    \
-    } while (0)
-
-// Process-wide streams per device, created on first use and never destroyed, like the reference's
-// static compute / fetch / assign streams (Source/Math/MatrixQuantizerGPU.cu:83-90, 197-206).
-constexpr int kMaxDevices = 64;
-struct DeviceStreams
-{
-    hipStream_t compute = nullptr;
-    hipStream_t fetch = nullptr;
-    hipStream_t assign = nullptr;
-};
-DeviceStreams g_streams[kMaxDevices];
-std::mutex g_streams_mutex;
 
 // ---- the argument table of cntkq_quantize_batch_noalloc ----------------------------------------------------------
 //
@@ -56,7 +154,6 @@ std::mutex g_streams_mutex;
 // until the process ends. Host code never uses the array's name as an address (in host code it is only a stand-in for
 // the symbol): scratch_for_device() asks the runtime for the copy's address on the current device, once per device, and
 // everything -- kernel arguments included -- goes through that pointer.
-constexpr size_t kNoAllocScratchBytes = 32 * 1024;
 static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 
 struct DeviceScratch
@@ -96,481 +193,6 @@ __global__ __launch_bounds__(256) void table_store_kernel(TableChunk chunk, uint
         dst[i] = chunk.w[i];
 }
 
-class DeviceGuard // PrepareDevice (Source/Math/MatrixQuantizerGPU.cu:186, 234): make the handle's device current
-{
-public:
-    explicit DeviceGuard(int device) : m_prev(-1), m_changed(false)
-    {
-        if (hipGetDevice(&m_prev) == hipSuccess && m_prev != device)
-            m_changed = (hipSetDevice(device) == hipSuccess);
-    }
-    ~DeviceGuard()
-    {
-        if (m_changed)
-            (void) hipSetDevice(m_prev);
-    }
-
-private:
-    int m_prev;
-    bool m_changed;
-};
-
-bool aligned4(const void* p)
-{
-    return (reinterpret_cast<uintptr_t>(p) & 3u) == 0;
-}
-
-// What differs between the two instantiations of the boundary (MatrixQuantizerImpl<float> / <double>).
-template <typename E>
-struct Elem;
-
-template <>
-struct Elem<float>
-{
-    static constexpr size_t kAlign = 4;
-    static constexpr size_t kWordBits = 32;
-    static size_t stripe_max_rows(size_t nbits) { return cntkq::stripe_reduce_max_rows(nbits); }
-    static bool valid_nbits(size_t nbits) { return cntkq::valid_nbits(nbits); }
-    static size_t qcol_bytes(size_t nbits, size_t rows) { return cntkq::qcol_bytes(nbits, rows); }
-    static hipError_t quantize(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, void* q, size_t rows,
-                               size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
-    {
-        return cntkq::launch_quantize(s, ev, g, r_in, r_out, q, rows, cols, nbits, zt, tune);
-    }
-    static hipError_t unquantize(hipStream_t s, LaunchEvents ev, const void* q, float* out, size_t rows, size_t cols, size_t nbits,
-                                 bool add, const LaunchTuning& tune)
-    {
-        return cntkq::launch_unquantize(s, ev, q, out, rows, cols, nbits, add, tune);
-    }
-    static hipError_t stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, void* q_out,
-                                    float* agg_out, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
-    {
-        return cntkq::launch_stripe_reduce(s, ev, src, stripe_res, q_out, agg_out, rows, cols, nbits, zt, tune);
-    }
-};
-
-template <>
-struct Elem<double>
-{
-    static constexpr size_t kAlign = 8;
-    static constexpr size_t kWordBits = 64;
-    static size_t stripe_max_rows(size_t nbits) { return cntkq::f64::stripe_reduce_max_rows(nbits); }
-    static bool valid_nbits(size_t nbits) { return cntkq::f64::valid_nbits(nbits); }
-    static size_t qcol_bytes(size_t nbits, size_t rows) { return cntkq::f64::qcol_bytes(nbits, rows); }
-    static hipError_t quantize(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, void* q, size_t rows,
-                               size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
-    {
-        return cntkq::f64::launch_quantize(s, ev, g, r_in, r_out, q, rows, cols, nbits, zt, tune);
-    }
-    static hipError_t unquantize(hipStream_t s, LaunchEvents ev, const void* q, double* out, size_t rows, size_t cols, size_t nbits,
-                                 bool add, const LaunchTuning& tune)
-    {
-        return cntkq::f64::launch_unquantize(s, ev, q, out, rows, cols, nbits, add, tune);
-    }
-    static hipError_t stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, double* stripe_res, void* q_out,
-                                    double* agg_out, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
-    {
-        return cntkq::f64::launch_stripe_reduce(s, ev, src, stripe_res, q_out, agg_out, rows, cols, nbits, zt, tune);
-    }
-};
-
-template <typename E>
-bool aligned_for(const void* p)
-{
-    return (reinterpret_cast<uintptr_t>(p) & (Elem<E>::kAlign - 1)) == 0;
-}
-
-} // namespace
-
-struct BatchTable
-{
-    std::vector<char> key;   // the item list and parameters the table was built for
-    char* host = nullptr;    // pinned
-    char* dev = nullptr;
-    size_t capacity = 0;
-    hipEvent_t event = nullptr; // set when the last kernel that reads the table has finished
-    bool in_flight = false;
-    // A launch that reads the table was recorded into a graph (stream capture): the graph may be replayed at any time
-    // from then on, so the buffers are never written again; a rebuild retires them (freed with the handle) and takes
-    // fresh ones.
-    bool captured = false;
-    std::vector<std::pair<char*, char*>> retired;
-    // launch parameters of the two LDS classes and the matrices that get a launch of their own
-    size_t members[2] = {0, 0};
-    uint32_t blocks[2] = {0, 0};
-    size_t lds[2] = {0, 0};
-    size_t first_entry[2] = {0, 0};
-    size_t first_begin[2] = {0, 0};
-    size_t entries_bytes = 0;
-    std::vector<size_t> own;
-};
-
-// Host-side state of cntkq_quantize_batch_noalloc: everything the call needs besides the device array, at fixed size,
-// so that the call itself touches no allocator (host or device).
-struct NoAllocState
-{
-    static constexpr size_t kMaxItems = CNTKQ_NOALLOC_MAX_ITEMS;
-    static constexpr size_t kTableWords = kNoAllocScratchBytes / sizeof(uint32_t);
-    // the table as uploaded: entries of the two LDS classes, then the first-workgroup lists (with sentinels)
-    alignas(16) uint32_t table[kTableWords];
-    size_t table_words = 0;
-    // launch parameters
-    size_t members[2] = {0, 0};
-    uint32_t blocks[2] = {0, 0};
-    size_t lds[2] = {0, 0};
-    size_t first_entry[2] = {0, 0};
-    size_t first_begin[2] = {0, 0};
-    size_t entries_bytes = 0;
-    size_t own[kMaxItems];
-    size_t own_count = 0;
-    // what the table was built for, and the upload of it that the device array last received from this handle
-    cntkq_quantize_item key_items[kMaxItems];
-    size_t key_count = 0, key_nbits = 0, key_zt = 0;
-    bool key_valid = false;
-    uint64_t uploaded_generation = 0;
-    hipStream_t uploaded_stream = nullptr; // later launches on another stream would not be ordered after that upload
-};
-
-struct cntkq_quantizer
-{
-    int device = 0;
-    bool dedicated = false;
-    hipStream_t main_stream = nullptr;
-    hipStream_t compute = nullptr; // == main_stream when !dedicated
-    hipStream_t fetch = nullptr;
-    hipStream_t assign = nullptr;
-    hipEvent_t ev_quantize = nullptr;
-    hipEvent_t ev_fetch = nullptr;
-    hipEvent_t ev_assign = nullptr;
-    hipEvent_t ev_unquantize = nullptr;
-    hipEvent_t ev_stripe = nullptr;
-    hipEvent_t ev_main = nullptr;
-    // the event each Wait call waits on: the handle's own, or one attached through the debug hook
-    hipEvent_t last_quantize = nullptr;
-    hipEvent_t last_unquantize = nullptr;
-    hipEvent_t last_stripe = nullptr;
-    hipEvent_t attach_start = nullptr; // one-shot: tied to the next kernel this handle launches
-    hipEvent_t attach_stop = nullptr;
-    bool quantize_included_fetch = false;
-    bool fetch_pending = false;   // a device-to-host copy out of the staging buffer may still be running
-    bool staging_read_pending = false; // a kernel reading the staging buffer may still be running
-    char* staging = nullptr;      // device buffer used when the packed matrix lives in host memory
-    size_t staging_bytes = 0;
-    // entry tables of the batched calls, one for quantize and one for unquantize. A gradient set is the same list of
-    // matrices step after step, so the table built for a list is kept (host key, pinned host copy, device copy, launch
-    // parameters) and a call with the same list only launches. A table is rebuilt only after the last kernel that
-    // reads it has finished (its event).
-    BatchTable quantize_table;
-    BatchTable unquantize_table;
-    BatchTable stripe_table;
-    BatchTable quantize_table64; // the same for the _f64 batched calls
-    BatchTable unquantize_table64;
-    BatchTable stripe_table64;
-    LaunchTuning tune;
-    struct NoAllocState* noalloc = nullptr; // fixed-size host state of cntkq_quantize_batch_noalloc (created with the handle)
-};
-
-namespace {
-
-hipStream_t work_stream(const cntkq_quantizer* h)
-{
-    return h->dedicated ? h->compute : h->main_stream;
-}
-
-// Completion is signalled by the kernel dispatch itself (no separate event record in the stream).
-LaunchEvents take_events(cntkq_quantizer* h, hipEvent_t own)
-{
-    LaunchEvents ev;
-    ev.start = h->attach_start;
-    ev.stop = h->attach_stop != nullptr ? h->attach_stop : own;
-    h->attach_start = nullptr;
-    h->attach_stop = nullptr;
-    return ev;
-}
-
-// Temp device buffer for a host-resident packed matrix (GetTempGPUQuantizedMatrix,
-// Source/Math/MatrixQuantizerGPU.cu:158-179). Grows only; waits for everything that may still use the old one.
-int ensure_staging(cntkq_quantizer* h, size_t bytes)
-{
-    if (h->staging_bytes >= bytes)
-        return CNTKQ_OK;
-    if (h->staging != nullptr)
-    {
-        HIP_TRY(hipStreamSynchronize(work_stream(h)), "hipStreamSynchronize failed");
-        HIP_TRY(hipStreamSynchronize(h->fetch), "hipStreamSynchronize failed");
-        HIP_TRY(hipStreamSynchronize(h->assign), "hipStreamSynchronize failed");
-        HIP_TRY(hipFree(h->staging), "hipFree failed");
-        h->staging = nullptr;
-        h->staging_bytes = 0;
-        h->fetch_pending = false;
-        h->staging_read_pending = false;
-    }
-    void* p = nullptr;
-    HIP_TRY(hipMalloc(&p, bytes), "hipMalloc of the packed staging buffer failed");
-    h->staging = static_cast<char*>(p);
-    h->staging_bytes = bytes;
-    return CNTKQ_OK;
-}
-
-// Whether work issued on `s` is being recorded into a graph instead of executed.
-bool stream_capturing(hipStream_t s)
-{
-    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &st) != hipSuccess)
-    {
-        (void) hipGetLastError();
-        return false;
-    }
-    return st == hipStreamCaptureStatusActive;
-}
-
-// True when `t` was built for exactly this item list and parameters.
-bool table_matches(const BatchTable& t, const void* items, size_t items_bytes, const size_t (&params)[3])
-{
-    if (t.key.size() != items_bytes + sizeof params)
-        return false;
-    return std::memcmp(t.key.data(), params, sizeof params) == 0 && std::memcmp(t.key.data() + sizeof params, items, items_bytes) == 0;
-}
-
-// Makes `t` writable with room for `bytes`: waits for the kernels that still read it, grows the buffers.
-int table_begin_rebuild(BatchTable& t, size_t bytes)
-{
-    t.key.clear();
-    if (t.event == nullptr)
-        HIP_TRY(hipEventCreateWithFlags(&t.event, hipEventDisableTiming), "hipEventCreateWithFlags failed");
-    if (t.captured)
-    {
-        t.retired.emplace_back(t.host, t.dev);
-        t.host = t.dev = nullptr;
-        t.capacity = 0;
-        t.captured = false;
-    }
-    if (t.in_flight)
-    {
-        HIP_TRY(hipEventSynchronize(t.event), "hipEventSynchronize failed");
-        t.in_flight = false;
-    }
-    if (bytes > t.capacity)
-    {
-        if (t.host != nullptr)
-            HIP_TRY(hipHostFree(t.host), "hipHostFree failed");
-        if (t.dev != nullptr)
-            HIP_TRY(hipFree(t.dev), "hipFree failed");
-        t.host = t.dev = nullptr;
-        t.capacity = 0;
-        const size_t cap = (bytes * 2 + 4095) & ~(size_t) 4095;
-        void* p = nullptr;
-        HIP_TRY(hipHostMalloc(&p, cap, hipHostMallocDefault), "hipHostMalloc of the batch table failed");
-        t.host = static_cast<char*>(p);
-        HIP_TRY(hipMalloc(&p, cap), "hipMalloc of the batch table failed");
-        t.dev = static_cast<char*>(p);
-        t.capacity = cap;
-    }
-    return CNTKQ_OK;
-}
-
-void table_set_key(BatchTable& t, const void* items, size_t items_bytes, const size_t (&params)[3])
-{
-    t.key.resize(items_bytes + sizeof params);
-    std::memcpy(t.key.data(), params, sizeof params);
-    std::memcpy(t.key.data() + sizeof params, items, items_bytes);
-}
-
-void table_destroy(BatchTable& t)
-{
-    if (t.event != nullptr)
-    {
-        if (t.in_flight)
-            (void) hipEventSynchronize(t.event);
-        (void) hipEventDestroy(t.event);
-    }
-    if (t.host != nullptr)
-        (void) hipHostFree(t.host);
-    if (t.dev != nullptr)
-        (void) hipFree(t.dev);
-    for (auto& r : t.retired)
-    {
-        (void) hipHostFree(r.first);
-        (void) hipFree(r.second);
-    }
-}
-
-int sync_event(hipEvent_t ev) // SyncEvent (Source/Math/MatrixQuantizerGPU.cu:68-80)
-{
-    hipError_t rc = hipEventQuery(ev);
-    if (rc == hipSuccess)
-        return CNTKQ_OK;
-    if (rc != hipErrorNotReady)
-        return fail(CNTKQ_RUNTIME_ERROR, "hipEventQuery failed: %s (hip error %d)", hipGetErrorString(rc), (int) rc);
-    HIP_TRY(hipEventSynchronize(ev), "hipEventSynchronize failed");
-    return CNTKQ_OK;
-}
-
-
-// ---- the three asynchronous calls, written once for both element types ----------------------------------
-
-template <typename E>
-int quantize_async_impl(cntkq_quantizer* h, const E* in, const E* res_in, size_t rows, size_t cols, void* qbuf, size_t qbuf_bytes,
-                        int qbuf_on_host, size_t nbits, E* res_out, int zero_threshold_for_1bit)
-{
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: null handle");
-    if (!Elem<E>::valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides %zu (got %zu)", Elem<E>::kWordBits, nbits);
-    if (rows >= (1ull << 31) || cols >= (1ull << 31))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: rows and cols must be below 2^31");
-    const size_t need = Elem<E>::qcol_bytes(nbits, rows) * cols;
-    if (qbuf_bytes != need)
-        return fail(CNTKQ_LOGIC_ERROR,
-                    "quantize: packed buffer of %zu bytes does not match %zu x %zu at %zu bits (%zu bytes)", qbuf_bytes,
-                    rows, cols, nbits, need);
-    h->quantize_included_fetch = false;
-    if (rows == 0 || cols == 0)
-        return CNTKQ_OK;
-    if (in == nullptr || res_in == nullptr || res_out == nullptr || qbuf == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: null matrix pointer");
-    if (!aligned_for<E>(in) || !aligned_for<E>(res_in) || !aligned_for<E>(res_out) || !aligned_for<E>(qbuf))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: pointers must be %zu-byte aligned", Elem<E>::kAlign);
-
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    char* qdev = static_cast<char*>(qbuf);
-    const bool capturing = stream_capturing(s);
-    if (capturing && qbuf_on_host)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_async: a host-resident packed matrix needs copies on other streams and cannot "
-                                            "be recorded into a graph");
-    if (qbuf_on_host)
-    {
-        int rc = ensure_staging(h, need);
-        if (rc != CNTKQ_OK)
-            return rc;
-        // a copy out of the staging buffer issued earlier must have drained before it is overwritten
-        if (h->fetch_pending)
-            HIP_TRY(hipStreamWaitEvent(s, h->ev_fetch, 0), "hipStreamWaitEvent failed");
-        qdev = h->staging;
-    }
-
-    LaunchEvents ev = take_events(h, h->ev_quantize);
-    if (capturing)
-        ev.stop = nullptr; // recorded, not executed: nothing to wait for
-    hipError_t lrc = Elem<E>::quantize(s, ev, in, res_in, res_out, qdev, rows, cols, nbits, zero_threshold_for_1bit != 0, h->tune);
-    if (lrc == hipErrorInvalidValue)
-        return fail(CNTKQ_INVALID_ARGUMENT, "quantize: the forced kernel path does not support %zu x %zu at %zu bits", rows, cols, nbits);
-    HIP_TRY(lrc, "quantize kernel launch failed");
-    h->last_quantize = ev.stop;
-
-    if (qbuf_on_host)
-    {
-        HIP_TRY(hipStreamWaitEvent(h->fetch, ev.stop, 0), "hipStreamWaitEvent failed");
-        HIP_TRY(hipMemcpyAsync(qbuf, qdev, need, hipMemcpyDeviceToHost, h->fetch), "hipMemcpyAsync failed");
-        HIP_TRY(hipEventRecord(h->ev_fetch, h->fetch), "hipEventRecord failed");
-        h->quantize_included_fetch = true;
-        h->fetch_pending = true;
-    }
-    return CNTKQ_OK;
-}
-
-template <typename E>
-int unquantize_async_impl(cntkq_quantizer* h, const void* qbuf, size_t qbuf_bytes, int qbuf_on_host, E* out, size_t rows, size_t cols,
-                          size_t nbits, int add)
-{
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: null handle");
-    if (!Elem<E>::valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides %zu (got %zu)", Elem<E>::kWordBits, nbits);
-    if (rows >= (1ull << 31) || cols >= (1ull << 31))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: rows and cols must be below 2^31");
-    const size_t need = Elem<E>::qcol_bytes(nbits, rows) * cols;
-    if (qbuf_bytes != need)
-        return fail(CNTKQ_LOGIC_ERROR,
-                    "unquantizestripe: dimension of patch to be unquantized does not match size of quantized data "
-                    "(%zu bytes given, %zu x %zu at %zu bits needs %zu)", qbuf_bytes, rows, cols, nbits, need);
-    if (qbuf_bytes == 0 || rows == 0 || cols == 0)
-        return CNTKQ_OK; // empty buffer: empty matrix, nothing to do
-    if (qbuf == nullptr || out == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: null matrix pointer");
-    if (!aligned_for<E>(qbuf) || !aligned_for<E>(out))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: pointers must be %zu-byte aligned", Elem<E>::kAlign);
-
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    const char* qdev = static_cast<const char*>(qbuf);
-    if (qbuf_on_host && stream_capturing(s))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_unquantize_async: a host-resident packed matrix needs copies on other streams and "
-                                            "cannot be recorded into a graph");
-    if (qbuf_on_host)
-    {
-        int rc = ensure_staging(h, need);
-        if (rc != CNTKQ_OK)
-            return rc;
-        // the staging buffer may still be read by an earlier kernel or copied out by an earlier fetch
-        HIP_TRY(hipEventRecord(h->ev_assign, s), "hipEventRecord failed");
-        HIP_TRY(hipStreamWaitEvent(h->assign, h->ev_assign, 0), "hipStreamWaitEvent failed");
-        if (h->fetch_pending)
-            HIP_TRY(hipStreamWaitEvent(h->assign, h->ev_fetch, 0), "hipStreamWaitEvent failed");
-        HIP_TRY(hipMemcpyAsync(h->staging, qbuf, need, hipMemcpyHostToDevice, h->assign), "hipMemcpyAsync failed");
-        HIP_TRY(hipEventRecord(h->ev_assign, h->assign), "hipEventRecord failed");
-        HIP_TRY(hipStreamWaitEvent(s, h->ev_assign, 0), "hipStreamWaitEvent failed");
-        qdev = h->staging;
-    }
-    LaunchEvents ev = take_events(h, h->ev_unquantize);
-    if (stream_capturing(s))
-        ev.stop = nullptr; // recorded, not executed: nothing to wait for
-    hipError_t lrc = Elem<E>::unquantize(s, ev, qdev, out, rows, cols, nbits, add != 0, h->tune);
-    if (lrc == hipErrorInvalidValue)
-        return fail(CNTKQ_INVALID_ARGUMENT, "unquantize: %zu x %zu at %zu bits is too large for one launch", rows, cols, nbits);
-    HIP_TRY(lrc, "unquantize kernel launch failed");
-    h->last_unquantize = ev.stop;
-    return CNTKQ_OK;
-}
-
-template <typename E>
-int stripe_reduce_async_impl(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows,
-                             size_t stripe_cols, size_t nbits, E* stripe_res, void* q_out, E* agg_out, int zero_threshold_for_1bit)
-{
-    if (h == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: null handle");
-    if (!Elem<E>::valid_nbits(nbits))
-        return fail(CNTKQ_LOGIC_ERROR, "Quantization: 'nbits' must be a power of two that divides %zu (got %zu)", Elem<E>::kWordBits, nbits);
-    if (workers == 0 || workers > CNTKQ_MAX_WORKERS || owner >= workers || stripes == nullptr)
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: need 1 <= workers <= %d and owner < workers",
-                    CNTKQ_MAX_WORKERS);
-    if (rows >= (1ull << 31) || stripe_cols >= (1ull << 31))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: rows and cols must be below 2^31");
-    if (rows == 0 || stripe_cols == 0)
-        return CNTKQ_OK;
-    if (rows > Elem<E>::stripe_max_rows(nbits))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: columns taller than %zu rows are not supported at %zu bits",
-                    Elem<E>::stripe_max_rows(nbits), nbits);
-    if (stripe_res == nullptr || q_out == nullptr || !aligned_for<E>(stripe_res) || !aligned_for<E>(q_out) || !aligned_for<E>(agg_out))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: null or misaligned matrix pointer");
-    StripeSources src;
-    std::memset(&src, 0, sizeof src);
-    for (size_t w = 0; w < workers; ++w)
-    {
-        if (stripes[w] == nullptr || !aligned_for<E>(stripes[w]))
-            return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: stripe %zu is null or misaligned", w);
-        src.q[w] = static_cast<const char*>(stripes[w]);
-    }
-    src.workers = (uint32_t) workers;
-    src.owner = (uint32_t) owner;
-
-    DeviceGuard guard(h->device);
-    hipStream_t s = work_stream(h);
-    LaunchEvents ev = take_events(h, h->ev_stripe);
-    if (stream_capturing(s))
-        ev.stop = nullptr; // recorded, not executed: nothing to wait for
-    hipError_t lrc = Elem<E>::stripe_reduce(s, ev, src, stripe_res, q_out, agg_out, rows, stripe_cols, nbits,
-                                            zero_threshold_for_1bit != 0, h->tune);
-    if (lrc == hipErrorInvalidValue)
-        return fail(CNTKQ_INVALID_ARGUMENT, "stripe reduction: %zu rows with %zu workers at %zu bits does not fit the kernel", rows, workers,
-                    nbits);
-    HIP_TRY(lrc, "stripe reduction kernel launch failed");
-    h->last_stripe = ev.stop;
-    return CNTKQ_OK;
-}
-
-#include "quantizer_api_batch.inc"
 
 // ---- the gradient-set quantize that allocates nothing -----------------------------------------------------------------
 //
@@ -785,30 +407,14 @@ size_t cntkq_qmatrix_bytes(size_t rows, size_t cols, size_t nbits)
     return valid_nbits(nbits) ? qcol_bytes(nbits, rows) * cols : 0;
 }
 
-size_t cntkq_qwords_per_col_f64(size_t rows, size_t nbits)
-{
-    return f64::valid_nbits(nbits) ? f64::qwords_per_col(rows, nbits) : 0;
-}
 
-size_t cntkq_qcol_bytes_f64(size_t nbits, size_t rows)
-{
-    return f64::valid_nbits(nbits) ? f64::qcol_bytes(nbits, rows) : 0;
-}
 
-size_t cntkq_qmatrix_bytes_f64(size_t rows, size_t cols, size_t nbits)
-{
-    return f64::valid_nbits(nbits) ? f64::qcol_bytes(nbits, rows) * cols : 0;
-}
 
 size_t cntkq_stripe_reduce_max_rows(size_t nbits)
 {
     return valid_nbits(nbits) ? Elem<float>::stripe_max_rows(nbits) : 0;
 }
 
-size_t cntkq_stripe_reduce_max_rows_f64(size_t nbits)
-{
-    return cntkq::f64::valid_nbits(nbits) ? Elem<double>::stripe_max_rows(nbits) : 0;
-}
 
 int cntkq_stripe_range(size_t cols, size_t rank, size_t workers, size_t* start_col, size_t* num_cols)
 {
@@ -976,11 +582,6 @@ int cntkq_quantize_async(cntkq_quantizer* h, const float* in, const float* res_i
     return quantize_async_impl<float>(h, in, res_in, rows, cols, qbuf, qbuf_bytes, qbuf_on_host, nbits, res_out, zero_threshold_for_1bit);
 }
 
-int cntkq_quantize_async_f64(cntkq_quantizer* h, const double* in, const double* res_in, size_t rows, size_t cols, void* qbuf,
-                             size_t qbuf_bytes, int qbuf_on_host, size_t nbits, double* res_out, int zero_threshold_for_1bit)
-{
-    return quantize_async_impl<double>(h, in, res_in, rows, cols, qbuf, qbuf_bytes, qbuf_on_host, nbits, res_out, zero_threshold_for_1bit);
-}
 
 int cntkq_wait_quantize_done(cntkq_quantizer* h)
 {
@@ -1003,11 +604,6 @@ int cntkq_unquantize_async(cntkq_quantizer* h, const void* qbuf, size_t qbuf_byt
     return unquantize_async_impl<float>(h, qbuf, qbuf_bytes, qbuf_on_host, out, rows, cols, nbits, add);
 }
 
-int cntkq_unquantize_async_f64(cntkq_quantizer* h, const void* qbuf, size_t qbuf_bytes, int qbuf_on_host, double* out,
-                               size_t rows, size_t cols, size_t nbits, int add)
-{
-    return unquantize_async_impl<double>(h, qbuf, qbuf_bytes, qbuf_on_host, out, rows, cols, nbits, add);
-}
 
 int cntkq_wait_unquantize_done(cntkq_quantizer* h)
 {
@@ -1042,13 +638,6 @@ int cntkq_stripe_reduce_async(cntkq_quantizer* h, const void* const* stripes, si
                                            zero_threshold_for_1bit);
 }
 
-int cntkq_stripe_reduce_async_f64(cntkq_quantizer* h, const void* const* stripes, size_t workers, size_t owner, size_t rows,
-                                  size_t stripe_cols, size_t nbits, double* stripe_res, void* q_out, double* agg_out,
-                                  int zero_threshold_for_1bit)
-{
-    return stripe_reduce_async_impl<double>(h, stripes, workers, owner, rows, stripe_cols, nbits, stripe_res, q_out, agg_out,
-                                            zero_threshold_for_1bit);
-}
 
 int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduce_item* items, size_t count, size_t workers,
                                     size_t owner, size_t nbits, int zero_threshold_for_1bit)
@@ -1064,24 +653,8 @@ int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h)
     return h->last_stripe != nullptr ? sync_event(h->last_stripe) : CNTKQ_OK;
 }
 
-// ---- the gradient-set calls on doubles (same implementation, see quantizer_api_batch.inc) ----------------------------
 
-int cntkq_quantize_batch_async_f64(cntkq_quantizer* h, const cntkq_quantize_item_f64* items, size_t count, size_t nbits,
-                                   int zero_threshold_for_1bit)
-{
-    return quantize_batch_impl<double>(h, items, count, nbits, zero_threshold_for_1bit);
-}
 
-int cntkq_unquantize_batch_async_f64(cntkq_quantizer* h, const cntkq_unquantize_item_f64* items, size_t count, size_t nbits, int add)
-{
-    return unquantize_batch_impl<double>(h, items, count, nbits, add);
-}
-
-int cntkq_stripe_reduce_batch_async_f64(cntkq_quantizer* h, const cntkq_stripe_reduce_item_f64* items, size_t count, size_t workers,
-                                        size_t owner, size_t nbits, int zero_threshold_for_1bit)
-{
-    return stripe_reduce_batch_impl<double>(h, items, count, workers, owner, nbits, zero_threshold_for_1bit);
-}
 
 // ---- hooks for tests and tuning runs (not part of the public header) --------------------------------
 
