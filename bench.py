@@ -111,7 +111,7 @@ def profiled_traffic():
 
     try:
         with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
-            m = re.search(r"^traffic_bytes_per_launch quantize = (\d+)", f.read(), re.M)
+            m = re.search(r"^\s*traffic_bytes_per_launch quantize = (\d+)", f.read(), re.M)
     except OSError:
         return None, None
     if not m:

@@ -119,7 +119,7 @@ struct BatchAbi<float>
     // the kernel family the plain call would take, so that both give the same bytes; false: does not fit the kernel
     static bool stripe_member(const SItem& it, size_t workers, size_t nbits, SEntry& e, size_t& lds, uint64_t& blocks)
     {
-        if (stripe_auto_col(it.rows))
+        if (stripe_auto_col(it.rows, it.stripe_res))
         {
             e.kind = 1;
             e.c = make_col_geom(it.rows, nbits, !columns_start_on_lines(it.stripe_res, it.rows));

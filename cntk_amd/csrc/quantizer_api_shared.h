@@ -101,6 +101,13 @@ struct BatchTable
     size_t capacity = 0;
     hipEvent_t event = nullptr; // set when the last kernel that reads the table has finished
     bool in_flight = false;
+    // The upload is an asynchronous copy on the stream of the call that built the table. A later call may run on another
+    // stream (the caller changed the handle's main stream): it is ordered after the upload, and after the kernels of
+    // the other stream that still read the table, by table_before_launch.
+    hipEvent_t upload_event = nullptr;
+    hipStream_t upload_stream = nullptr;
+    bool upload_known_done = true;
+    hipStream_t last_stream = nullptr; // stream of the last launch that read the table
     // A launch that reads the table was recorded into a graph (stream capture): the graph may be replayed at any time
     // from then on, so the buffers are never written again; a rebuild retires them (freed with the handle) and takes
     // fresh ones.
@@ -261,6 +268,12 @@ inline int table_begin_rebuild(BatchTable& t, size_t bytes)
         HIP_TRY(hipEventSynchronize(t.event), "hipEventSynchronize failed");
         t.in_flight = false;
     }
+    if (!t.upload_known_done)
+    {
+        // the copy out of the pinned host table may still be running (a table built and never read, or read on another stream)
+        HIP_TRY(hipEventSynchronize(t.upload_event), "hipEventSynchronize failed");
+        t.upload_known_done = true;
+    }
     if (bytes > t.capacity)
     {
         if (t.host != nullptr)
@@ -280,6 +293,53 @@ inline int table_begin_rebuild(BatchTable& t, size_t bytes)
     return CNTKQ_OK;
 }
 
+// After the upload of a freshly built table has been issued on `s`.
+inline int table_uploaded(BatchTable& t, hipStream_t s)
+{
+    if (t.upload_event == nullptr)
+        HIP_TRY(hipEventCreateWithFlags(&t.upload_event, hipEventDisableTiming), "hipEventCreateWithFlags failed");
+    HIP_TRY(hipEventRecord(t.upload_event, s), "hipEventRecord failed");
+    t.upload_stream = s;
+    t.upload_known_done = false;
+    t.last_stream = s;
+    return CNTKQ_OK;
+}
+
+// Before the launches of a call that reads `t` on stream `s`. The same stream as the upload and the last reader: nothing
+// to do (stream order). Another stream: the host waits once for the upload (a few microseconds, and legal while `s` is
+// being captured, since the event belongs to no capture), and `s` is made to wait for the last reader on the other
+// stream, so that the event of this call's last kernel again covers every reader.
+inline int table_before_launch(BatchTable& t, hipStream_t s, bool capturing)
+{
+    if (!t.upload_known_done && s != t.upload_stream)
+    {
+        HIP_TRY(hipEventSynchronize(t.upload_event), "hipEventSynchronize failed");
+        t.upload_known_done = true;
+    }
+    if (!capturing)
+    {
+        if (t.in_flight && t.last_stream != s)
+            HIP_TRY(hipStreamWaitEvent(s, t.event, 0), "hipStreamWaitEvent failed");
+        t.last_stream = s;
+    }
+    return CNTKQ_OK;
+}
+
+// A launch of a batched call failed after earlier ones of the same call were issued on `s`: the table's event is
+// recorded behind them, so that a rebuild and the Wait call still cover the work that was issued.
+inline hipEvent_t table_partial_failure(BatchTable& t, hipStream_t s, bool issued, bool capturing)
+{
+    if (!issued || capturing || t.event == nullptr)
+        return nullptr;
+    if (hipEventRecord(t.event, s) != hipSuccess)
+    {
+        (void) hipGetLastError();
+        return nullptr;
+    }
+    t.in_flight = true;
+    return t.event;
+}
+
 inline void table_set_key(BatchTable& t, const void* items, size_t items_bytes, const size_t (&params)[3])
 {
     t.key.resize(items_bytes + sizeof params);
@@ -294,6 +354,11 @@ inline void table_destroy(BatchTable& t)
         if (t.in_flight)
             (void) hipEventSynchronize(t.event);
         (void) hipEventDestroy(t.event);
+    }
+    if (t.upload_event != nullptr)
+    {
+        (void) hipEventSynchronize(t.upload_event);
+        (void) hipEventDestroy(t.upload_event);
     }
     if (t.host != nullptr)
         (void) hipHostFree(t.host);

@@ -567,7 +567,9 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
     for (uint32_t w = 0; w < src.workers; ++w)
         aligned8 = aligned8 && (reinterpret_cast<uintptr_t>(src.q[w]) & 7u) == 0;
     const bool col_forced = tune.quantize_path == kPathCol;
-    const bool col = (tune.quantize_path == kPathAuto || col_forced) && rows % 4 == 0 && (col_forced || rows >= kColMinRows);
+    // (a quantize call on a residual that is not 16-byte aligned takes the tile kernel, and so does the automatic choice here)
+    const bool col = (tune.quantize_path == kPathAuto || col_forced) && rows % 4 == 0 &&
+                     (col_forced || (rows >= kColMinRows && (reinterpret_cast<uintptr_t>(stripe_res) & 15u) == 0));
     // the summation order a quantize call on (aggregate, stripe residual) would use, given the residual's address
     const bool line_shift = !columns_start_on_lines(stripe_res, rows);
     if (col && (line_shift || !(aligned8 && col_unrolled(q_out, rows, nbits))))
@@ -849,9 +851,9 @@ inline hipError_t launch_stripe_reduce_batch(hipStream_t s, LaunchEvents ev, con
 }
 
 // which kernel family launch_stripe_reduce takes by itself for a stripe of this height: columns (true) or tiles
-inline bool stripe_auto_col(size_t rows)
+inline bool stripe_auto_col(size_t rows, const void* stripe_res)
 {
-    return rows % 4 == 0 && rows >= kColMinRows;
+    return rows % 4 == 0 && rows >= kColMinRows && (reinterpret_cast<uintptr_t>(stripe_res) & 15u) == 0;
 }
 
 // colg_lds_bytes for a bit width known only at run time

@@ -74,3 +74,21 @@ def zero_columns(a, seed, frac=0.9):
     mask = rng.random(a.shape[1]) < frac
     a[:, mask] = 0.0
     return mask
+
+
+def few_valued_stripe_sum(rows, cols, seed0=90000, seed1=95000):
+    """What the owner of a stripe requantizes at K = 2, 1 bit, zeroThresholdFor1Bit on: the sum of two workers'
+    reconstructions, i.e. columns that hold only four distinct values. The fp32 term-by-term sum of such a column
+    rounds the same way at every addition; at 6144 rows the bounds it gives are off by more than 1e-5 of the column
+    scale for many seeds (the recorded case: a 6144-row stripe of the two-worker aggregator run).
+    Returns (a, b, sum): the two gradients (exact bell-shaped values) and the fp32 sum of their reconstructions."""
+    import oracle
+
+    a = np.asfortranarray(np.concatenate([exact_bell(seed0 + j, rows, 1) for j in range(cols)], axis=1))
+    b = np.asfortranarray(np.concatenate([exact_bell(seed1 + j, rows, 1) for j in range(cols)], axis=1))
+    z = np.zeros_like(a, order="F")
+    qa, _ = oracle.quantize(a, z, 1, True, threads=4)
+    qb, _ = oracle.quantize(b, z, 1, True, threads=4)
+    s = oracle.unquantize(qa, rows, cols, 1, threads=4)
+    s = oracle.unquantize(qb, rows, cols, 1, out=s, add=True, threads=4)
+    return a, b, s

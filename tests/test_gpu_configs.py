@@ -98,9 +98,13 @@ def test_config1_512x512_single_step():
     parity.check_unquantize(Q.to_numpy(), rows, cols, 1, np_of(Out))
     assert Q.GetSize() == 36864
     say("config 1:", rep)
+    rep.assert_fallback_at_most(0)
 
 
 # ---- config 2 ----------------------------------------------------------------------------------------
+
+# columns (of 12 checked steps x 23,656) allowed to rest on the float64 bounds instead of the oracle's
+CONFIG2_FALLBACK_COLS = 0
 
 SPEECH_DNN = [(429, 2048)] + [(2048, 2048)] * 6 + [(2048, 9304)] + [(2048, 1)] * 7 + [(9304, 1)]
 
@@ -113,14 +117,14 @@ def test_config2_speech_dnn_100_steps(zt):
     gen.manual_seed(datagen.case_seed(2))
     chains = [Chain(r, c, 1, zt) for r, c in SPEECH_DNN]
     rep = parity.Report()
-    oracle_steps = {0, 1, 49, 99}
     for step in range(100):
         if step % 10 == 0:
             say("config 2 zeroThr", zt, "step", step)
         for ch in chains:
             G = device_student_t3(gen, ch.rows, ch.cols, 1e-3)
-            ch.step(G, step in oracle_steps, rep)
+            ch.step(G, step < 2 or step % 10 == 9, rep)  # the oracle sees steps 0, 1, 9, 19 ... 99
     say("config 2:", rep)
+    rep.assert_fallback_at_most(CONFIG2_FALLBACK_COLS)
 
 
 # ---- config 3 ----------------------------------------------------------------------------------------
@@ -155,6 +159,7 @@ def test_config3_resnet50_multibit(nbits):
         for ch in chains:
             ch.step(device_outliers(gen, ch.rows, ch.cols), True, rep)
     say("config 3:", rep)
+    rep.assert_fallback_at_most(0)
 
 
 # ---- config 4 ----------------------------------------------------------------------------------------
@@ -228,9 +233,13 @@ def test_config4_allreduce_full_shape():
             % (worst, ntaint, cols))
         assert ntaint <= cols // 100
     say("config 4:", rep)
+    rep.assert_fallback_at_most(0)
 
 
 # ---- config 5 ----------------------------------------------------------------------------------------
+
+# of 4 checked steps x 116,896 columns
+CONFIG5_FALLBACK_COLS = 8
 
 LSTM_LM = [(100000, 512, 0.9), (1024, 4096, 0.0), (1024, 4096, 0.0), (1024, 4096, 0.0), (1024, 4096, 0.0),
            (512, 100000, 0.0)]
@@ -251,8 +260,11 @@ def test_config5_lstm_lm_zero_threshold_20_steps():
                 # a different 90% of the columns is silent at every step
                 keep = (torch.rand(c, generator=gen, device="cuda:0") >= zero_frac).to(torch.float32)
                 G.data.view(c, r).mul_(keep[:, None])
-            ch.step(G, step in (0, 1, 19), rep)
+            ch.step(G, step < 2 or step % 10 == 9, rep)  # the oracle sees steps 0, 1, 9, 19
     say("config 5:", rep)
+    # only the 100000-row embedding columns that received a gradient (about 51 of 512 per step) are long enough for the
+    # oracle's own fp32 sum to use up the tolerance
+    rep.assert_fallback_at_most(CONFIG5_FALLBACK_COLS)
     # columns that never received a gradient keep lower = upper = 0 and all valid bits set
     z = Matrix(100000, 4)
     Qz = QuantizedMatrix(100000, 4, 1, 0)

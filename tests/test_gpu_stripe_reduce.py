@@ -107,6 +107,98 @@ def test_stripe_reduce(case):
     say("  ", rep)
 
 
+def test_stripe_reduce_of_few_valued_columns_6144_rows():
+    """The recorded miss of the 1e-5 bound tolerance: a 6144-row stripe at K = 2, 1 bit, zero threshold. The aggregate
+    holds four distinct values, the oracle's term-by-term fp32 sum of such a column is off by more than 1e-5 of the
+    column scale, the device's pairwise sums are not. The comparison accepts exactly those columns against the
+    float64 bounds and counts them."""
+    rows, cols, k = 6144, 32, 2
+    a, b, s = datagen.few_valued_stripe_sum(rows, cols)
+    zeros = np.zeros((rows, cols), np.float32, order="F")
+    qs = [oracle.quantize(g, zeros, 1, True, threads=8)[0] for g in (a, b)]
+    # one stripe of all columns: the second worker's packed matrix stands in for a stripe of the same width
+    qz = MatrixQuantizerImpl.Create(0, False)
+    Qs = []
+    for q in qs:
+        Q = QuantizedMatrix(rows, cols, 1, 0)
+        Q.from_numpy(q)
+        Qs.append(Q)
+    S, Agg = Matrix(rows, cols), Matrix(rows, cols)
+    qz.StripeReduceAsync(Qs, 0, S, Qs[0], True, agg_out=Agg)
+    qz.WaitStripeReduceDone()
+    torch.cuda.synchronize()
+    assert parity.bits_equal(Agg.to_numpy(), s)
+    rep = parity.check_quantize(s, zeros, Qs[0].to_numpy(), S.to_numpy(), 1, True, strict=True)
+    say("few-valued 6144-row stripe:", rep)
+    lo_g, hi_g = oracle.headers(Qs[0].to_numpy(), rows, cols, 1)
+    lo_x, hi_x = parity.exact_headers(s, zeros, 1, True)
+    assert np.max(np.maximum(np.abs(lo_g - lo_x), np.abs(hi_g - hi_x)) / (hi_x - lo_x)) < 1e-6
+    assert 3 <= rep.fallback_cols <= cols
+
+
+@pytest.mark.parametrize("rows,off", [(2048, 1), (1024, 3), (4096, 2), (9304, 1), (1028, 5), (20000, 1), (20001, 2)])
+@pytest.mark.parametrize("batched", [False, True], ids=["plain", "batched"])
+def test_stripe_residual_at_4_byte_offsets(rows, off, batched):
+    """A stripe residual that is only 4-byte aligned (a view `off` elements into an allocation): the fused reduction
+    must still give the bytes of the call sequence whose aggregate and residual sit at that same offset, i.e. pick the
+    kernel family a quantize call on such matrices picks. Also through the batched call, alone and beside a second item."""
+    from test_gpu_random_shapes import place
+
+    cols, k, nbits, zt = 6, 3, 1, False
+    qz = MatrixQuantizerImpl.Create(0, False)
+    gs = [datagen.normal(3100 + w + rows, rows, cols) for w in range(k)]
+    zeros = np.zeros((rows, cols), np.float32, order="F")
+    qs = [oracle.quantize(g, zeros, nbits, zt, threads=8)[0] for g in gs]
+    sres = datagen.normal(3200 + rows, rows, cols, 0.003)
+    Qs = []
+    for q in qs:
+        Q = QuantizedMatrix(rows, cols, nbits, 0)
+        Q.from_numpy(q)
+        Qs.append(Q)
+    S, _sbuf = place(sres, off, torch.float32)
+    Out = QuantizedMatrix(rows, cols, nbits, 0)
+    if batched:
+        # a second, ordinary item makes the call a real shared grid; then the item alone (the call falls back to the plain one)
+        g2 = [datagen.normal(3300 + w, 2048, 4) for w in range(k)]
+        Q2 = []
+        for g in g2:
+            Q = QuantizedMatrix(2048, 4, nbits, 0)
+            Q.from_numpy(oracle.quantize(g, np.zeros((2048, 4), np.float32, order="F"), nbits, zt)[0])
+            Q2.append(Q)
+        S2, Out2 = Matrix(2048, 4), QuantizedMatrix(2048, 4, nbits, 0)
+        qz.StripeReduceBatchAsync([(Qs, S, Out, None), (Q2, S2, Out2, None)], 0, zt)
+        qz.WaitStripeReduceDone()
+        torch.cuda.synchronize()
+        first = (Out.to_numpy().copy(), S.to_numpy().copy())
+        S, _sbuf = place(sres, off, torch.float32)
+        qz.StripeReduceBatchAsync([(Qs, S, Out, None)], 0, zt)
+    else:
+        first = None
+        qz.StripeReduceAsync(Qs, 0, S, Out, zt)
+    qz.WaitStripeReduceDone()
+    torch.cuda.synchronize()
+    q_new, s_new = Out.to_numpy(), S.to_numpy()
+    if first is not None:
+        assert np.array_equal(first[0], q_new) and parity.bits_equal(first[1], s_new), "batch member != item alone"
+    # the call sequence with aggregate and residual at the same offset
+    Agg, _abuf = place(zeros, off, torch.float32)
+    for w in range(k):
+        qz.UnquantizeAsync(Qs[w], Agg, add=(w > 0))
+    S2, _s2buf = place(sres, off, torch.float32)
+    Qo = QuantizedMatrix(rows, cols, nbits, 0)
+    qz.QuantizeAsync(Agg, S2, Qo, S2, zt)
+    qz.WaitQuantizeAsyncDone()
+    torch.cuda.synchronize()
+    assert np.array_equal(Qo.to_numpy(), q_new), "fused != call sequence (codes)"
+    assert parity.bits_equal(S2.to_numpy(), s_new), "fused != call sequence (residual)"
+    # (the packed matrices stand in for stripes of their full width: the aggregate is their decoded sum, worker 0 first)
+    agg_o = oracle.unquantize(qs[0], rows, cols, nbits, threads=8)
+    for w in range(1, k):
+        agg_o = oracle.unquantize(qs[w], rows, cols, nbits, out=agg_o, add=True, threads=8)
+    assert parity.bits_equal(agg_o, Agg.to_numpy())
+    parity.check_quantize(agg_o, sres, q_new, s_new, nbits, zt)
+
+
 def test_stripe_reduce_height_limit():
     """The tallest stripe the fused call takes depends on the bit width (its LDS holds the output QWords and one worker's
     record); taller ones are refused, and the limit can be asked for."""
