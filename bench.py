@@ -135,6 +135,11 @@ def main():
                     help="skip the two untimed passes that carry HIP events (GPU timeline, kernel durations)")
     ap.add_argument("--event-every", type=int, default=2,
                     help="kernel-duration pass: attach timing events to the kernels of every n-th step")
+    ap.add_argument("--config", type=int, default=0,
+                    help="instead of the headline, one of the gradient-set workloads as whole steps: 2 speech DNN set (1 bit), "
+                         "3 ResNet-50 set (2, 4, 8 bits: one line each), 4 simulated 8-worker all-reduce of 2048x9304, "
+                         "5 LSTM language-model set (1 bit, zero threshold); one JSON line per workload with the time of "
+                         "every call of a step and the roofline of the longest")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="instead of the benchmark, run plain device copies of one 2048x9304 fp32 matrix "
                          "(76,218,368 bytes read and as many written per copy), for scaling hardware counters")
@@ -142,6 +147,13 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU only (K workers are simulated in one GPU's memory); "
                  "--gpus %d is not supported" % args.gpus)
+
+    if args.config:
+        from cntk_amd import config_bench
+
+        # (the headline's defaults are 1000 steps of 52 us; a gradient-set step takes 0.1 - 0.7 ms)
+        config_bench.run(args.config, steps=min(args.steps, 200), warmup=min(args.warmup, 20))
+        return
 
     import torch
 

@@ -98,6 +98,9 @@ def lib():
         L.cntkq_quantize_batch_async_f64.argtypes = L.cntkq_quantize_batch_async.argtypes
         L.cntkq_unquantize_batch_async_f64.argtypes = L.cntkq_unquantize_batch_async.argtypes
         L.cntkq_stripe_reduce_batch_async_f64.argtypes = L.cntkq_stripe_reduce_batch_async.argtypes
+        L.cntkq_stripe_reduce_batch_owners_async.argtypes = [_vp, ctypes.POINTER(_StripeReduceItem), ctypes.POINTER(_sz), _sz, _sz, _sz,
+                                                             ctypes.c_int]
+        L.cntkq_stripe_reduce_batch_owners_async_f64.argtypes = L.cntkq_stripe_reduce_batch_owners_async.argtypes
         for name in ("cntkq_stripe_reduce_max_rows", "cntkq_stripe_reduce_max_rows_f64"):
             getattr(L, name).argtypes = [_sz]
             getattr(L, name).restype = _sz
@@ -490,7 +493,14 @@ class MatrixQuantizerImpl:
         if isinstance(items, PreparedBatch):
             if items.kind != "stripe_reduce":
                 raise QuantizerLogicError("StripeReduceBatchAsync: prepared for another call")
-            if items.count:
+            if items.count and isinstance(owner, (list, tuple)):
+                # an owner per item: the stripes of all the ranks of a cluster simulated on one GPU
+                if len(owner) != items.count:
+                    raise QuantizerLogicError("StripeReduceBatchAsync: one owner per item")
+                owners = (_sz * items.count)(*owner)
+                _check(_fn("cntkq_stripe_reduce_batch_owners_async", items.dtype)(self._h, items.array, owners, items.count, items.workers,
+                                                                                  items.nbits, int(bool(zero_threshold_for_1bit))))
+            elif items.count:
                 _check(_fn("cntkq_stripe_reduce_batch_async", items.dtype)(self._h, items.array, items.count, items.workers, owner,
                                                                            items.nbits, int(bool(zero_threshold_for_1bit))))
             return

@@ -31,6 +31,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cstdio>
+#include <deque>
 #include <future>
 #include <map>
 #include <tuple>
@@ -207,6 +208,11 @@ public:
     {
         bool useFusedStripeReduce = true; // one kernel for "unquantize all stripes, sum, requantize"
         bool useBatchedCalls = true;      // one launch for all gradients in steps 1 and 5
+        // InProcessCluster only: the K workers share one GPU and one stream, so the launches of all K workers in a step are
+        // issued as ONE call each (K workers' quantize items in one grid; all K owners' stripes in one grid with an owner
+        // per item; every worker's final unquantize in one grid). Same bytes as driving the workers one after another;
+        // needs useFusedStripeReduce and useBatchedCalls, and falls back when a stripe is too tall for the fused call.
+        bool useClusterBatching = true;
         // every syncStatsTrace-th aggregation is timed between two device synchronisations and reported on stderr as the
         // reference does ("Actual gradient aggregation time", Source/1BitSGD/AllReduceDistGradAggregator.h:153, 241-246,
         // 560-565); 0 = never
@@ -483,6 +489,134 @@ public:
         return headerCPU.numSamples != 0;
     }
 
+    // ---- the same three steps cut into "which items" and "bookkeeping", for InProcessCluster's one call per step --------
+    typedef MatrixQuantizerGPU<ElemType> GpuQuantizer;
+    struct ClusterLaunch
+    {
+        std::vector<typename GpuQuantizer::QuantizeItem> quantize;
+        std::vector<typename GpuQuantizer::StripeReduceItem> stripes;
+        std::vector<size_t> owners;
+        std::vector<typename GpuQuantizer::UnquantizeItem> unquantize;
+        // views the items point to (deques: addresses stay valid while they grow)
+        std::deque<QuantizedMatrix<ElemType>> packedViews;
+        std::deque<Matrix<ElemType>> matrixViews;
+    };
+
+    // whether every own stripe of this gradient set can go through the fused call (then the cluster may batch)
+    bool AllStripesFusable(const std::vector<Matrix<ElemType>*>& gradients) const
+    {
+        if (!(m_options.useFusedStripeReduce && m_useQuantizationForSelfStripe && m_options.useBatchedCalls && m_options.useClusterBatching))
+            return false;
+        const size_t fusedMaxRows = detail::Abi<ElemType>::StripeReduceMaxRows(m_numQuantizationBits);
+        for (auto* g : gradients)
+            if (g->GetNumRows() > fusedMaxRows)
+                return false;
+        return m_transport.StreamOrdered();
+    }
+
+    // step 1 without the launch (:250-266, 288-300)
+    void CollectQuantizeItems(const std::vector<Matrix<ElemType>*>& gradients, DistGradHeader& headerCPU, bool resetState, ClusterLaunch& launch)
+    {
+        ResetState(gradients, resetState);
+        if (headerCPU.numSamples == 0)
+            for (auto* g : gradients)
+                g->SetValue(0.0f);
+        for (size_t i = 0; i < gradients.size(); ++i)
+            launch.quantize.push_back({gradients[i], &m_preAggGradQuantizers[i]->GetResidualMatrix(), m_gradQuantized[i].get(),
+                                       const_cast<Matrix<ElemType>*>(&m_preAggGradQuantizers[i]->GetResidualMatrix())});
+    }
+    // step 2 on a stream-ordered transport
+    void PostQuantized(const std::vector<Matrix<ElemType>*>& gradients, DistGradHeader& headerCPU)
+    {
+        for (size_t i = 0; i < gradients.size(); ++i)
+            for (size_t j = 0; j < NumProc(); ++j)
+            {
+                const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), j, NumProc());
+                if (stripe.m_numCols != 0)
+                    m_transport.PostStripe(MyRank(), j, i, m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+            }
+        m_transport.PostHeader(MyRank(), headerCPU);
+    }
+    // step 3 without the launch (:365-436): one item per gradient with an own stripe
+    void CollectStripeItems(const std::vector<Matrix<ElemType>*>& gradients, ClusterLaunch& launch)
+    {
+        const size_t K = NumProc();
+        for (size_t i = 0; i < gradients.size(); ++i)
+        {
+            const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K);
+            if (stripe.m_numCols == 0)
+                continue;
+            launch.packedViews.push_back(m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+            typename GpuQuantizer::StripeReduceItem it;
+            for (size_t w = 0; w < K; ++w)
+                it.stripes.push_back(&m_transport.ReceivedStripe(MyRank(), w, i));
+            it.stripeResidual = &const_cast<Matrix<ElemType>&>(m_aggGradStripeQuantizers[i]->GetResidualMatrix());
+            it.outQStripe = &launch.packedViews.back();
+            it.aggregate = nullptr;
+            launch.stripes.push_back(std::move(it));
+            launch.owners.push_back(MyRank());
+        }
+    }
+    // step 4 on a stream-ordered transport
+    void PostReducedStripes(const std::vector<Matrix<ElemType>*>& gradients)
+    {
+        for (size_t i = 0; i < gradients.size(); ++i)
+        {
+            const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), NumProc());
+            if (stripe.m_numCols != 0)
+                m_transport.PostAggregatedStripe(MyRank(), i, m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+        }
+    }
+    // step 5 without the launch (:517-522): every stripe is decoded where its owner left it. False: some stripe cannot be
+    // read in place (nothing was appended then, and the caller takes FetchAndUnquantize).
+    bool CollectUnquantizeItems(const std::vector<Matrix<ElemType>*>& gradients, ClusterLaunch& launch)
+    {
+        const size_t K = NumProc();
+        for (size_t i = 0; i < gradients.size(); ++i)
+            for (size_t j = 0; j < K; ++j)
+                if (j != MyRank() && GetStripeForNode(gradients[i]->GetNumCols(), j, K).m_numCols > 0 &&
+                    m_transport.AggregatedStripeView(MyRank(), j, i) == nullptr)
+                    return false;
+        for (size_t i = 0; i < gradients.size(); ++i)
+            for (size_t j = 0; j < K; ++j)
+            {
+                const Stripe stripe = GetStripeForNode(gradients[i]->GetNumCols(), j, K);
+                if (stripe.m_numCols == 0)
+                    continue;
+                launch.matrixViews.push_back(gradients[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+                const QuantizedMatrix<ElemType>* packed = nullptr;
+                if (j == MyRank())
+                {
+                    launch.packedViews.push_back(m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+                    packed = &launch.packedViews.back();
+                }
+                else
+                    packed = m_transport.AggregatedStripeView(MyRank(), j, i);
+                launch.unquantize.push_back({packed, &launch.matrixViews.back()});
+            }
+        return true;
+    }
+    bool FinishHeader(DistGradHeader& headerCPU)
+    {
+        headerCPU.Aggregate(m_transport.AggregatedHeader(), false);
+        return headerCPU.numSamples != 0;
+    }
+    // the handles the cluster issues on (all quantizers of a cluster share one stream)
+    GpuQuantizer* GradientQuantizerGpu() { return m_preAggGradQuantizers.empty() ? nullptr : &Gpu(*m_preAggGradQuantizers[0]); }
+    GpuQuantizer* StripeQuantizerGpu()
+    {
+        for (auto& q : m_aggGradStripeQuantizers)
+            if (q)
+                return &Gpu(*q);
+        return nullptr;
+    }
+    void SyncGradientQuantizerWithMainStream()
+    {
+        if (m_useAsyncAggregation && !m_preAggGradQuantizers.empty())
+            SyncWithMainStream(*m_preAggGradQuantizers[0]);
+    }
+    bool ZeroThresholdFor1Bit() const { return m_zeroThresholdFor1Bit; }
+
     // Work this worker issues from now on starts only after `event` (a hipEvent_t recorded by the caller) has completed.
     // Needs the quantizers, i.e. a ResetState call before it.
     void WaitForEvent(void* event)
@@ -563,18 +697,74 @@ public:
             detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize"); // the gradients have been computed (:241-246)
             t0 = std::chrono::steady_clock::now();
         }
+        bool clusterBatching = true;
         for (size_t r = 0; r < K; ++r)
-            m_workers[r]->QuantizeAndPost(gradients[r], headers[r], resetState);
-        for (size_t r = 0; r < K; ++r)
-            m_workers[r]->ReduceOwnStripes(gradients[r]);
+            clusterBatching = clusterBatching && m_workers[r]->AllStripesFusable(gradients[r]);
         bool any = false;
-        for (size_t r = 0; r < (unquantizeOnAllWorkers ? K : 1); ++r)
-            any = m_workers[r]->FetchAndUnquantize(gradients[r], headers[r]) || any;
+        if (clusterBatching)
+            any = AggregateAsOneCallPerStep(gradients, headers, resetState, unquantizeOnAllWorkers ? K : 1);
+        else
+        {
+            for (size_t r = 0; r < K; ++r)
+                m_workers[r]->QuantizeAndPost(gradients[r], headers[r], resetState);
+            for (size_t r = 0; r < K; ++r)
+                m_workers[r]->ReduceOwnStripes(gradients[r]);
+            for (size_t r = 0; r < (unquantizeOnAllWorkers ? K : 1); ++r)
+                any = m_workers[r]->FetchAndUnquantize(gradients[r], headers[r]) || any;
+        }
         if (showSyncPerfStats)
         {
             detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize");
             const double seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
             std::fprintf(stderr, "Actual gradient aggregation time: %.6g\n", seconds);
+        }
+        return any;
+    }
+
+    // The K workers' steps with one call per step for the whole cluster (Options::useClusterBatching): the workers say which
+    // matrices, stripes and views their step covers, and the cluster issues them together on the stream they all share.
+    bool AggregateAsOneCallPerStep(const std::vector<std::vector<Matrix<ElemType>*>>& gradients, std::vector<DistGradHeader>& headers,
+                                   bool resetState, size_t unquantizingWorkers)
+    {
+        const size_t K = m_workers.size();
+        typename AllReduceDistGradAggregator<ElemType>::ClusterLaunch launch;
+        for (size_t r = 0; r < K; ++r)
+            m_workers[r]->CollectQuantizeItems(gradients[r], headers[r], resetState, launch);
+        auto* gradientGpu = m_workers[0]->GradientQuantizerGpu();
+        if (gradientGpu != nullptr)
+        {
+            m_workers[0]->SyncGradientQuantizerWithMainStream(); // the gradients were produced on the main stream
+            gradientGpu->QuantizeBatchAsync(launch.quantize, m_workers[0]->ZeroThresholdFor1Bit());
+        }
+        for (size_t r = 0; r < K; ++r)
+            m_workers[r]->PostQuantized(gradients[r], headers[r]);
+        typename AllReduceDistGradAggregator<ElemType>::GpuQuantizer* stripeGpu = nullptr;
+        for (size_t r = 0; r < K; ++r)
+        {
+            m_workers[r]->CollectStripeItems(gradients[r], launch);
+            if (stripeGpu == nullptr)
+                stripeGpu = m_workers[r]->StripeQuantizerGpu();
+        }
+        if (stripeGpu != nullptr && !launch.stripes.empty())
+            stripeGpu->StripeReduceBatchAsync(launch.stripes, launch.owners, m_workers[0]->ZeroThresholdFor1Bit());
+        for (size_t r = 0; r < K; ++r)
+            m_workers[r]->PostReducedStripes(gradients[r]);
+        bool any = false;
+        std::vector<size_t> viaFetch;
+        for (size_t r = 0; r < unquantizingWorkers; ++r)
+            if (!m_workers[r]->CollectUnquantizeItems(gradients[r], launch))
+                viaFetch.push_back(r);
+        if (gradientGpu != nullptr && !launch.unquantize.empty())
+        {
+            gradientGpu->UnquantizeBatchAsync(launch.unquantize, false);
+            gradientGpu->WaitUnquantizeAsyncDone();
+        }
+        for (size_t r = 0; r < unquantizingWorkers; ++r)
+        {
+            if (std::find(viaFetch.begin(), viaFetch.end(), r) != viaFetch.end())
+                any = m_workers[r]->FetchAndUnquantize(gradients[r], headers[r]) || any;
+            else
+                any = m_workers[r]->FinishHeader(headers[r]) || any;
         }
         return any;
     }

@@ -90,6 +90,11 @@ struct Abi<float>
     {
         return cntkq_stripe_reduce_batch_async(h, items, n, workers, owner, bits, zt);
     }
+    static int StripeReduceBatchOwners(cntkq_quantizer* h, const StripeReduceItem* items, const size_t* owners, size_t n, size_t workers,
+                                       size_t bits, int zt)
+    {
+        return cntkq_stripe_reduce_batch_owners_async(h, items, owners, n, workers, bits, zt);
+    }
 };
 
 template <>
@@ -127,6 +132,11 @@ struct Abi<double>
     static int StripeReduceBatch(cntkq_quantizer* h, const StripeReduceItem* items, size_t n, size_t workers, size_t owner, size_t bits, int zt)
     {
         return cntkq_stripe_reduce_batch_async_f64(h, items, n, workers, owner, bits, zt);
+    }
+    static int StripeReduceBatchOwners(cntkq_quantizer* h, const StripeReduceItem* items, const size_t* owners, size_t n, size_t workers,
+                                       size_t bits, int zt)
+    {
+        return cntkq_stripe_reduce_batch_owners_async_f64(h, items, owners, n, workers, bits, zt);
     }
 };
 } // namespace detail
@@ -516,6 +526,17 @@ public:
     };
     void StripeReduceBatchAsync(const std::vector<StripeReduceItem>& items, size_t owner, bool zeroThresholdFor1Bit)
     {
+        StripeReduceBatchAsync(items, owner, nullptr, zeroThresholdFor1Bit);
+    }
+    // owners[i]: the rank whose stripe item i is (all ranks of a cluster simulated on one GPU in one call)
+    void StripeReduceBatchAsync(const std::vector<StripeReduceItem>& items, const std::vector<size_t>& owners, bool zeroThresholdFor1Bit)
+    {
+        if (owners.size() != items.size())
+            throw std::invalid_argument("StripeReduceBatchAsync: one owner per item");
+        StripeReduceBatchAsync(items, 0, owners.data(), zeroThresholdFor1Bit);
+    }
+    void StripeReduceBatchAsync(const std::vector<StripeReduceItem>& items, size_t owner, const size_t* owners, bool zeroThresholdFor1Bit)
+    {
         if (items.empty())
             return;
         const size_t workers = items[0].stripes.size();
@@ -538,7 +559,11 @@ public:
                                                    it.aggregate ? it.aggregate->Data() : nullptr, it.outQStripe->GetNumRows(),
                                                    it.outQStripe->GetNumCols()});
         }
-        detail::Check(detail::Abi<ElemType>::StripeReduceBatch(m_handle, raw.data(), raw.size(), workers, owner, nbits, zeroThresholdFor1Bit ? 1 : 0));
+        if (owners != nullptr)
+            detail::Check(detail::Abi<ElemType>::StripeReduceBatchOwners(m_handle, raw.data(), owners, raw.size(), workers, nbits,
+                                                                         zeroThresholdFor1Bit ? 1 : 0));
+        else
+            detail::Check(detail::Abi<ElemType>::StripeReduceBatch(m_handle, raw.data(), raw.size(), workers, owner, nbits, zeroThresholdFor1Bit ? 1 : 0));
     }
     void WaitStripeReduceDone() { detail::Check(cntkq_wait_stripe_reduce_done(m_handle)); }
 

@@ -645,6 +645,14 @@ int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduc
     return stripe_reduce_batch_impl<float>(h, items, count, workers, owner, nbits, zero_threshold_for_1bit);
 }
 
+int cntkq_stripe_reduce_batch_owners_async(cntkq_quantizer* h, const cntkq_stripe_reduce_item* items, const size_t* owners, size_t count,
+                                           size_t workers, size_t nbits, int zero_threshold_for_1bit)
+{
+    if (owners == nullptr && count != 0)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_owners_async: null owner list");
+    return stripe_reduce_batch_impl<float>(h, items, count, workers, 0, nbits, zero_threshold_for_1bit, owners);
+}
+
 int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h)
 {
     if (h == nullptr)

@@ -183,4 +183,12 @@ int cntkq_stripe_reduce_batch_async_f64(cntkq_quantizer* h, const cntkq_stripe_r
     return stripe_reduce_batch_impl<double>(h, items, count, workers, owner, nbits, zero_threshold_for_1bit);
 }
 
+int cntkq_stripe_reduce_batch_owners_async_f64(cntkq_quantizer* h, const cntkq_stripe_reduce_item_f64* items, const size_t* owners,
+                                               size_t count, size_t workers, size_t nbits, int zero_threshold_for_1bit)
+{
+    if (owners == nullptr && count != 0)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_batch_owners_async_f64: null owner list");
+    return stripe_reduce_batch_impl<double>(h, items, count, workers, 0, nbits, zero_threshold_for_1bit, owners);
+}
+
 } // extern "C"

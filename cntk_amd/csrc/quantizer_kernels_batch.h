@@ -6,19 +6,28 @@
 
 namespace cntkq {
 
-// largest e with begins[e] <= b; b and everything derived from it is uniform over the workgroup
+// largest e with begins[e] <= b (begins ascending, begins[0] = 0); b and everything derived from it is uniform over the
+// workgroup. One round trip to the table instead of log2(count) dependent ones: the 64 lanes of a wavefront test one
+// entry each, and the number of entries <= b, minus one, is the answer; above 64 entries a first pass over every
+// stride-th entry narrows the range to at most 64 (4096 entries: two round trips). Every wavefront of the workgroup
+// does the same look-up. A workgroup of a batched launch lives a few microseconds, of which the dependent loads of a
+// binary search were a noticeable part (8 stripe views of 2048 x 1163 decoded in 15.8 us against 12.2 us for the
+// plain launch on the whole matrix).
 __device__ __forceinline__ uint32_t batch_find(const uint32_t* __restrict__ begins, uint32_t count, uint32_t b)
 {
-    uint32_t lo = 0, hi = count;
-    while (hi - lo > 1)
+    const uint32_t lane = threadIdx.x & 63u;
+    uint32_t first = 0, n = count;
+    while (n > 64)
     {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (begins[mid] <= b)
-            lo = mid;
-        else
-            hi = mid;
+        const uint32_t stride = (n + 63) / 64;
+        const uint32_t idx = lane * stride;
+        const uint32_t v = idx < n ? begins[first + idx] : 0xFFFFFFFFu;
+        const uint32_t cell = (uint32_t) __popcll(__ballot(v <= b)) - 1u;
+        first += cell * stride;
+        n = min(stride, n - cell * stride);
     }
-    return lo;
+    const uint32_t v = lane < n ? begins[first + lane] : 0xFFFFFFFFu;
+    return first + (uint32_t) __popcll(__ballot(v <= b)) - 1u;
 }
 
 // Many matrices in one launch: the workgroups of all matrices form one grid; `begins` (count + 1 entries, ascending)

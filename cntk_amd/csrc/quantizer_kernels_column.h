@@ -251,7 +251,7 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSo
 #pragma unroll
                 for (uint32_t kk = 0; kk < KS; ++kk)
                 {
-                    const float x = ((bits >> kk) & 1u) ? val1 : val0;
+                    const float x = pick_level(bits, kk, val0, val1);
                     // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
                     acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
                 }
@@ -611,12 +611,11 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
 #pragma unroll
                     for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
                     {
-                        const uint32_t code = (bits >> (kk * PS::SHIFT)) & PS::CODEMASK;
                         float x;
                         if constexpr (NBITS == 1)
-                            x = code ? b : a;
+                            x = pick_level(bits, kk, a, b);
                         else
-                            x = unquantize_value<NBITS>(a, b, code);
+                            x = unquantize_value<NBITS>(a, b, (bits >> (kk * PS::SHIFT)) & PS::CODEMASK);
                         // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
                         acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
                     }

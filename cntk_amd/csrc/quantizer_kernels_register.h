@@ -362,12 +362,11 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                 {
-                    const uint32_t code = (bits[ww] >> (kk * PS::SHIFT)) & PS::CODEMASK;
                     float x;
                     if constexpr (NBITS == 1)
-                        x = code ? val1 : val0;
+                        x = pick_level(bits[ww], kk, val0, val1);
                     else
-                        x = unquantize_value<NBITS>(uf, lo, code);
+                        x = unquantize_value<NBITS>(uf, lo, (bits[ww] >> (kk * PS::SHIFT)) & PS::CODEMASK);
                     // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
                     a[u][e] = (n == 0) ? x : x + a[u][e];
                     if (++ww == c.nq)

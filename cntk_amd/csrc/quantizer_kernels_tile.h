@@ -394,12 +394,11 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
 #pragma unroll
                     for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
                     {
-                        const uint32_t code = (bits >> (kk * PS::SHIFT)) & PS::CODEMASK;
                         float x;
                         if constexpr (NBITS == 1)
-                            x = code ? b : a;
+                            x = pick_level(bits, kk, a, b);
                         else
-                            x = unquantize_value<NBITS>(a, b, code);
+                            x = unquantize_value<NBITS>(a, b, (bits >> (kk * PS::SHIFT)) & PS::CODEMASK);
                         // the first term seeds the sum; afterwards: decoded value + running sum
                         acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
                     }

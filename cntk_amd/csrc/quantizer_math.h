@@ -122,6 +122,18 @@ __device__ __forceinline__ float unquantize_value(float uf, float lo, uint32_t q
     }
 }
 
+// 1-bit decoding of bit `pos` of a QWord: val1 where the bit is set, val0 elsewhere, as a bit-field extract (the bit
+// sign-extended to a mask) and a bitwise select, i.e. two instructions and no condition register. Written with compare
+// and conditional move the same choice takes three and a wait for the condition register each time; the stripe
+// reductions, which decode workers x elements values per column, are bound by instruction issue.
+__device__ __forceinline__ float pick_level(uint32_t bits, uint32_t pos, float val0, float val1)
+{
+    const int32_t mask = __builtin_amdgcn_sbfe((int32_t) bits, pos, 1u);
+    float x;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(x) : "v"(mask), "v"(val1), "v"(val0));
+    return x;
+}
+
 template <int NBITS>
 __device__ __forceinline__ float unquantize_value(const ValueQ& v, uint32_t q)
 {

@@ -221,6 +221,14 @@ typedef struct cntkq_stripe_reduce_item
 int cntkq_stripe_reduce_batch_async(cntkq_quantizer* h, const cntkq_stripe_reduce_item* items, size_t count, size_t workers,
                                     size_t owner, size_t nbits, int zero_threshold_for_1bit);
 
+/* The same with an owner per item: item i is reduced as rank owners[i] reduces its stripe, i.e. the loop of
+ * Source/1BitSGD/AllReduceDistGradAggregator.h:339-436 as EVERY rank runs it, in one call. For K workers simulated in
+ * one GPU's memory (all K ranks' stripes then form one grid instead of K launches that each fill a fraction of the chip);
+ * results identical to cntkq_stripe_reduce_async item by item with owner = owners[i]. owners: `count` entries, host
+ * memory, read during the call only. */
+int cntkq_stripe_reduce_batch_owners_async(cntkq_quantizer* h, const cntkq_stripe_reduce_item* items, const size_t* owners,
+                                           size_t count, size_t workers, size_t nbits, int zero_threshold_for_1bit);
+
 /* Blocks until the last stripe reduction of this handle has finished (the reference waits on the stripe
  * quantizer's WaitQuantizeAsyncDone, Source/1BitSGD/AllReduceDistGradAggregator.h:494). */
 int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h);
@@ -294,6 +302,8 @@ int cntkq_quantize_batch_async_f64(cntkq_quantizer* h, const cntkq_quantize_item
 int cntkq_unquantize_batch_async_f64(cntkq_quantizer* h, const cntkq_unquantize_item_f64* items, size_t count, size_t nbits, int add);
 int cntkq_stripe_reduce_batch_async_f64(cntkq_quantizer* h, const cntkq_stripe_reduce_item_f64* items, size_t count, size_t workers,
                                         size_t owner, size_t nbits, int zero_threshold_for_1bit);
+int cntkq_stripe_reduce_batch_owners_async_f64(cntkq_quantizer* h, const cntkq_stripe_reduce_item_f64* items, const size_t* owners,
+                                               size_t count, size_t workers, size_t nbits, int zero_threshold_for_1bit);
 
 #ifdef __cplusplus
 }

@@ -84,12 +84,13 @@ struct RunResult
 };
 
 static RunResult Run(const Shapes& shapes, size_t K, int nBits, bool zeroThr, bool selfStripeQuantized, bool useAsync, bool fused, bool batched,
-                     int steps, unsigned long seed, bool checkAllWorkersEqual)
+                     int steps, unsigned long seed, bool checkAllWorkersEqual, bool clusterBatching = true)
 {
     RunResult out;
     InProcessCluster<float>::Options opt;
     opt.useFusedStripeReduce = fused;
     opt.useBatchedCalls = batched;
+    opt.useClusterBatching = clusterBatching;
     out.cluster.reset(new InProcessCluster<float>(K, 0, nBits, zeroThr, selfStripeQuantized, useAsync, opt));
     for (int step = 0; step < steps; ++step)
     {
@@ -153,10 +154,12 @@ static void VariantsAreBitIdentical()
                 continue;
             // the reference's arrangement: per-matrix calls, unfused stripe reduction, main stream
             RunResult ref = Run(shapes, K, nBits, zeroThr, true, false, false, false, 3, 4242, true);
-            for (int variant = 1; variant < 8; ++variant)
+            // variants 6 and 7 (fused and batched) issue one call per step for the whole cluster; 8 and 9 are the same two
+            // with every worker issuing its own calls
+            for (int variant = 1; variant < 10; ++variant)
             {
-                const bool useAsync = variant & 1, fused = variant & 2, batched = variant & 4;
-                RunResult v = Run(shapes, K, nBits, zeroThr, true, useAsync, fused, batched, 3, 4242, false);
+                const bool useAsync = variant & 1, fused = (variant & 2) || variant >= 8, batched = (variant & 4) || variant >= 8;
+                RunResult v = Run(shapes, K, nBits, zeroThr, true, useAsync, fused, batched, 3, 4242, false, variant < 8);
                 for (size_t step = 0; step < ref.gradients.size(); ++step)
                     for (size_t i = 0; i < shapes.size(); ++i)
                         CHECK(ref.gradients[step][i].size() == v.gradients[step][i].size() &&

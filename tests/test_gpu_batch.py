@@ -131,6 +131,46 @@ def test_stripe_batch_equals_per_matrix_calls(nbits, zt, k):
     say("stripe batch", nbits, zt, k, "ok")
 
 
+@pytest.mark.parametrize("nbits,zt,k", [(1, False, 8), (1, True, 3), (4, False, 4)])
+def test_stripe_batch_with_an_owner_per_item(nbits, zt, k):
+    """All the ranks of a cluster simulated on one GPU in one call: item i reduced as rank owners[i] would, bytes of the
+    plain call with that owner."""
+    qz = MatrixQuantizerImpl.Create(0, False)
+    z = lambda r, c: np.zeros((r, c), np.float32, order="F")
+    sets = [(r, c) for r, c in STRIPE_SETS if r and c]
+    owners = [(3 * i + 1) % k for i in range(len(sets))]
+    packed = [[oracle.quantize(datagen.normal(60 * i + 7 * w + nbits, r, c), z(r, c), nbits, zt, threads=8)[0] for w in range(k)]
+              for i, (r, c) in enumerate(sets)]
+    sres = [datagen.normal(950 + i, r, c, 0.003) for i, (r, c) in enumerate(sets)]
+
+    def device_state():
+        Qs = []
+        for i, (r, c) in enumerate(sets):
+            row = []
+            for w in range(k):
+                Q = QuantizedMatrix(r, c, nbits, 0)
+                Q.from_numpy(packed[i][w])
+                row.append(Q)
+            Qs.append(row)
+        return Qs, [Matrix.from_numpy(s) for s in sres], [Matrix(r, c) for r, c in sets]
+
+    Q1, S1, A1 = device_state()
+    for i in range(len(sets)):
+        qz.StripeReduceAsync(Q1[i], owners[i], S1[i], Q1[i][owners[i]], zt, agg_out=A1[i])
+    qz.WaitStripeReduceDone()
+    Q2, S2, A2 = device_state()
+    qz.StripeReduceBatchAsync([(Q2[i], S2[i], Q2[i][owners[i]], A2[i]) for i in range(len(sets))], owners, zt)
+    qz.WaitStripeReduceDone()
+    torch.cuda.synchronize()
+    for i, (r, c) in enumerate(sets):
+        assert np.array_equal(Q1[i][owners[i]].to_numpy(), Q2[i][owners[i]].to_numpy()), ("packed", sets[i])
+        assert parity.bits_equal(S1[i].to_numpy(), S2[i].to_numpy()), ("stripe residual", sets[i])
+        assert parity.bits_equal(A1[i].to_numpy(), A2[i].to_numpy()), ("aggregate", sets[i])
+    with pytest.raises(cntk_amd.QuantizerLogicError):
+        qz.StripeReduceBatchAsync([(Q2[0], S2[0], Q2[0][0], None), (Q2[1], S2[1], Q2[1][0], None)], [0, k], zt)
+    say("stripe batch with owners", nbits, zt, k, "ok")
+
+
 def test_batch_argument_checks():
     qz = MatrixQuantizerImpl.Create(0, False)
     with pytest.raises(cntk_amd.QuantizerLogicError):
