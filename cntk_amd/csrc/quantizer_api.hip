@@ -65,10 +65,17 @@ struct BatchAbi<float>
         // (a register-kernel matrix of modest size gives the same bytes as a member: a launch costs more than it gains)
         if (path == kPathCol || (path == kPathReg && it.rows <= kTileMaxRows && it.rows * it.cols < kOwnLaunchElements))
         {
+            const bool line_shift = quantize_line_shift(it.in, it.res_in, it.res_out, it.rows);
             e.kind = 1;
-            e.c = make_col_geom(it.rows, nbits, quantize_line_shift(it.in, it.res_in, it.res_out, it.rows));
+            e.c = make_col_geom(it.rows, nbits, line_shift);
             lds = colg_lds_bytes_rt(e.c, nbits);
             blocks = it.cols;
+            // 1 bit, 1024 / 2048 / 4096 rows, columns on 128-byte lines, 8-byte aligned records: the unrolled body (same bytes)
+            if (!line_shift && col_unrolled(it.qbuf, it.rows, nbits))
+            {
+                e.kind = it.rows == 1024 ? 2 : (it.rows == 2048 ? 3 : 4);
+                lds = it.rows == 1024 ? col_lds_bytes<1>() : (it.rows == 2048 ? col_lds_bytes<2>() : col_lds_bytes<4>());
+            }
             return true;
         }
         return false;
@@ -121,10 +128,20 @@ struct BatchAbi<float>
     {
         if (stripe_auto_col(it.rows, it.stripe_res))
         {
+            const bool line_shift = !columns_start_on_lines(it.stripe_res, it.rows);
             e.kind = 1;
-            e.c = make_col_geom(it.rows, nbits, !columns_start_on_lines(it.stripe_res, it.rows));
+            e.c = make_col_geom(it.rows, nbits, line_shift);
             lds = colg_lds_bytes_rt(e.c, nbits) + 2 * workers * sizeof(float);
             blocks = it.stripe_cols;
+            // as launch_stripe_reduce chooses: the unrolled body where every packed stripe is 8-byte aligned
+            bool aligned = (reinterpret_cast<uintptr_t>(it.q_out) & 7u) == 0;
+            for (size_t w = 0; w < workers; ++w)
+                aligned = aligned && (reinterpret_cast<uintptr_t>(it.stripes[w]) & 7u) == 0;
+            if (!line_shift && aligned && it.rows <= 2048 && col_unrolled(it.q_out, it.rows, nbits))
+            {
+                e.kind = it.rows == 1024 ? 2 : 3;
+                lds = (it.rows == 1024 ? col_lds_bytes<1>() : col_lds_bytes<2>()) + 2 * kMaxWorkers * 4;
+            }
         }
         else
         {

@@ -40,7 +40,7 @@ struct QuantizeBatchEntry
     const float* r_in;
     float* r_out;
     char* q;
-    uint32_t kind; // 0: tiles (t), 1: columns (c)
+    uint32_t kind; // 0: tiles (t), 1: columns (c), 2 / 3 / 4: 1-bit columns of 1024 / 2048 / 4096 rows (the unrolled body; c.qcol)
     uint32_t pad;
     TileGeom t;
     ColGeom c;
@@ -59,10 +59,21 @@ __global__ __launch_bounds__(kTileThreads) void quantize_batch_kernel(const Quan
         const TileGeom t = entries[e].t;
         quantize_tile_body<NBITS, ZT>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, t, index);
     }
-    else
+    else if (NBITS != 1 || entries[e].kind == 1)
     {
         const ColGeom c = entries[e].c;
         quantize_colg_body<NBITS, ZT>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, c, index, smem_v4);
+    }
+    else if constexpr (NBITS == 1)
+    {
+        // the unrolled 1-bit column bodies: two thirds of the general body's instructions for the same bytes
+        const uint64_t qcol = entries[e].c.qcol;
+        if (entries[e].kind == 2)
+            quantize_col_body<ZT, 1>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, qcol, index, smem_v4);
+        else if (entries[e].kind == 3)
+            quantize_col_body<ZT, 2>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, qcol, index, smem_v4);
+        else
+            quantize_col_body<ZT, 4>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, qcol, index, smem_v4);
     }
 }
 
@@ -73,7 +84,7 @@ struct StripeBatchEntry
     float* stripe_res;
     char* q_out;
     float* agg_out;
-    uint32_t kind; // 0: tiles (t), 1: columns (c)
+    uint32_t kind; // 0: tiles (t), 1: columns (c), 2 / 3: 1-bit columns of 1024 / 2048 rows (the unrolled body; c.qcol)
     uint32_t pad;
     TileGeom t;
     ColGeom c;
@@ -92,10 +103,20 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_batch_kernel(const
         const TileGeom t = en.t;
         stripe_reduce_tile_body<NBITS, ZT>(en.src, en.stripe_res, en.q_out, en.agg_out, t, index);
     }
-    else
+    else if (NBITS != 1 || en.kind == 1)
     {
         const ColGeom c = en.c;
         stripe_reduce_colg_body<NBITS, ZT>(en.src, en.stripe_res, en.q_out, en.agg_out, c, index, smem_v4);
+    }
+    else if constexpr (NBITS == 1)
+    {
+        const uint64_t qcol = en.c.qcol;
+        // (4096 rows stay with the general body: unrolled they take 74 registers, which would cost every member of the
+        // launch two of its eight wavefronts per SIMD)
+        if (en.kind == 2)
+            stripe_reduce_col_body<ZT, 1>(en.src, en.stripe_res, en.q_out, en.agg_out, qcol, index, smem_v4);
+        else
+            stripe_reduce_col_body<ZT, 2>(en.src, en.stripe_res, en.q_out, en.agg_out, qcol, index, smem_v4);
     }
 }
 

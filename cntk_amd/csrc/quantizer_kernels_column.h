@@ -161,14 +161,13 @@ __device__ __forceinline__ void col_stats_pack(const ColLds& l, float csum, floa
 }
 
 template <bool ZT, int PER>
-__global__ __launch_bounds__(kColThreads) void quantize_col_kernel(const float* __restrict__ g, const float* r_in, float* r_out,
-                                                                   char* __restrict__ q, uint64_t qcol)
+__device__ __forceinline__ void quantize_col_body(const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q,
+                                                  uint64_t qcol, uint32_t column, f32x4* smem_v4)
 {
     constexpr uint32_t ROWS = 1024 * PER, T = kColThreads;
-    extern __shared__ f32x4 smem_v4[];
     const ColLds l = col_lds<PER>(smem_v4);
     const uint32_t tid = threadIdx.x;
-    const size_t base = (size_t) blockIdx.x * ROWS;
+    const size_t base = (size_t) column * ROWS;
     if (tid < 32 * PER)
         l.words[tid] = 0u;
     const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base);
@@ -188,22 +187,29 @@ __global__ __launch_bounds__(kColThreads) void quantize_col_kernel(const float* 
         t4[tid + T * u] = a[u];
     }
     // the whole column has been read before col_stats_pack's first barrier, so r_out may be r_in
-    col_stats_pack<ZT, PER>(l, col_thread_sum<PER>(a), r_out + base, q + (size_t) blockIdx.x * qcol);
+    col_stats_pack<ZT, PER>(l, col_thread_sum<PER>(a), r_out + base, q + (size_t) column * qcol);
+}
+
+template <bool ZT, int PER>
+__global__ __launch_bounds__(kColThreads) void quantize_col_kernel(const float* __restrict__ g, const float* r_in, float* r_out,
+                                                                   char* __restrict__ q, uint64_t qcol)
+{
+    extern __shared__ f32x4 smem_v4[];
+    quantize_col_body<ZT, PER>(g, r_in, r_out, q, qcol, blockIdx.x, smem_v4);
 }
 
 // Stripe reduction in the same shape: the work item that will pack (QWord p, chunk) first decodes those bit positions
 // from every worker's packed stripe, sums them (owner first, then ascending) and adds the stripe residual.
 template <bool ZT, int PER>
-__global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSources src, float* stripe_res, char* q_out,
-                                                                        float* agg_out, uint64_t qcol)
+__device__ __forceinline__ void stripe_reduce_col_body(const StripeSources& src, float* stripe_res, char* q_out, float* agg_out, uint64_t qcol,
+                                                       uint32_t column, f32x4* smem_v4)
 {
     constexpr uint32_t ROWS = 1024 * PER, NQ = 32 * PER, T = kColThreads, KS = 4 * PER, BATCH = 8;
-    extern __shared__ f32x4 smem_v4[];
     const ColLds l = col_lds<PER>(smem_v4);
     float* dec = reinterpret_cast<float*>(l.red_u + 4); // two reconstruction levels per worker, in summation order
     const uint32_t tid = threadIdx.x;
-    const size_t base = (size_t) blockIdx.x * ROWS;
-    const size_t rec = (size_t) blockIdx.x * qcol;
+    const size_t base = (size_t) column * ROWS;
+    const size_t rec = (size_t) column * qcol;
     const uint32_t K = src.workers;
     if (tid < NQ)
         l.words[tid] = 0u;
@@ -278,6 +284,14 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSo
         csum = col_thread_sum<PER>(v);
     }
     col_stats_pack<ZT, PER>(l, csum, stripe_res + base, q_out + rec);
+}
+
+template <bool ZT, int PER>
+__global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSources src, float* stripe_res, char* q_out,
+                                                                        float* agg_out, uint64_t qcol)
+{
+    extern __shared__ f32x4 smem_v4[];
+    stripe_reduce_col_body<ZT, PER>(src, stripe_res, q_out, agg_out, qcol, blockIdx.x, smem_v4);
 }
 
 // ---- the same decomposition for any bit width and any column height that is a multiple of 4 ----------------

@@ -280,20 +280,36 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
 }
 
 // Stripe reduction for tall columns (above the LDS kernels' 14336 rows), in the register kernel's shape: 1024 threads per
-// owned column, the running sum of the decoded stripes in registers. The workers are taken one at a time in the fixed
-// order (owner first, then ascending rank): the worker's packed record goes to LDS in one coalesced copy (every QWord
-// serves up to 32 rows), each thread decodes its slots' elements from it and adds them to its sums. Then the stripe
-// residual is added and reg_stats_pack requantizes, so that the result is, byte for byte, what the sequence
-// "unquantize own stripe, add the others, quantize_reg_kernel on (aggregate, stripe residual)" gives.
-// LDS: [48 reduction slots | nq output QWords | nq + 2 words of one worker's record].
-__host__ __device__ inline size_t stripe_reg_lds_bytes(const RegGeom& c)
+// owned column, the running sum of the decoded stripes in registers. The workers are taken in the fixed order (owner
+// first, then ascending rank), `group` of them at a time (as many as the CU's 160 KB of LDS hold; all 8 of a 100000-row
+// 1-bit stripe): their packed columns go to LDS in coalesced copies (every QWord serves up to 32 rows), and each thread
+// walks its slots once per group -- the position of a slot's elements (QWord, bit) is worked out once and serves every
+// worker of the group; a piece's four elements sit in four consecutive QWords at one bit position unless the piece
+// straddles the end of the QWord run, which takes an element-wise path. The kernel is bound by instruction issue, not by
+// memory: one worker at a time with every position recomputed per worker and element cost 11,500 vector instructions
+// per wavefront at 100000 rows and 8 workers, 14.7 per decoded value. Then the stripe residual is added and
+// reg_stats_pack requantizes, so that the result is, byte for byte, what the sequence "unquantize own stripe, add the
+// others, quantize_reg_kernel on (aggregate, stripe residual)" gives.
+// LDS: [48 reduction slots | nq output QWords | 2 decoding constants per worker of a group | group x nq QWords].
+__host__ __device__ inline size_t stripe_reg_lds_bytes(const RegGeom& c, uint32_t group)
 {
-    return ((size_t) kRegRedSlots + 2 * (size_t) c.nq + 2) * 4;
+    return ((size_t) kRegRedSlots + (size_t) c.nq + 2 * (size_t) group + (size_t) group * c.nq) * 4;
+}
+
+// how many workers' packed columns are decoded together: what fits the LDS of a CU beside the output QWords
+__host__ __device__ inline uint32_t stripe_reg_group(const RegGeom& c, uint32_t workers, size_t lds_limit = 160 * 1024)
+{
+    const size_t fixed = ((size_t) kRegRedSlots + c.nq) * 4;
+    const size_t per = ((size_t) c.nq + 2) * 4;
+    size_t g = lds_limit > fixed ? (lds_limit - fixed) / per : 0;
+    if (g < 1)
+        g = 1;
+    return (uint32_t) (g < workers ? g : workers);
 }
 
 template <int NBITS, bool ZT, int PER>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<1024, PER>(), reg_waves<1024, PER>()))) void stripe_reduce_reg_kernel(
-    StripeSources src, float* stripe_res, char* q_out, float* agg_out, RegGeom c)
+    StripeSources src, float* stripe_res, char* q_out, float* agg_out, RegGeom c, uint32_t group)
 {
     using PS = PackShape<NBITS>;
     static_assert(NBITS < 32, "32-bit codes are whole QWords: nothing to assemble");
@@ -302,7 +318,8 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<
     float* red = reinterpret_cast<float*>(smem_v4);
     uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
     uint32_t* words = reinterpret_cast<uint32_t*>(red + kRegRedSlots);
-    uint32_t* pw = words + c.nq; // one worker's record: lower, upper, QWords
+    float* dec = reinterpret_cast<float*>(words + c.nq); // per worker of the group: 1 bit -> the two levels, else (ufactor, lower)
+    uint32_t* pw = words + c.nq + 2 * group;             // the group's packed columns, nq QWords each
     const uint32_t tid = threadIdx.x;
     const size_t base = (size_t) blockIdx.x * c.rows;
     const size_t rec = (size_t) blockIdx.x * c.qcol;
@@ -316,63 +333,133 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<
     const bool has_edge = tid < head + tail;
     const uint32_t edge_at = tid < head ? tid : c.rows - tail + (tid - head);
     const uint32_t shift = column_shift(sres + head, c.line_shift);
-    const uint32_t ufirst = tid < shift ? 1u : 0u;
-    const uint32_t e0 = head + 4 * (tid + T * ufirst - shift);
-    const uint32_t k_first = e0 / c.nq;
-    const uint32_t w_first = e0 - k_first * c.nq;
-    const uint32_t edge_k = edge_at / c.nq;
-    const uint32_t edge_w = edge_at - edge_k * c.nq;
 
+    // -0 is the additive identity (x + -0 = x for every x, signed zeros included): the first worker's values seed the sums
+    // through the same addition as the others
     f32x4 a[PER];
-    float edge = 0.0f;
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+        a[u] = f32x4{-0.0f, -0.0f, -0.0f, -0.0f};
+    float edge = -0.0f;
     const uint32_t K = src.workers;
-    const uint32_t rec_words = c.nq + 2;
-    for (uint32_t n = 0; n < K; ++n)
+    for (uint32_t n0 = 0; n0 < K; n0 += group)
     {
-        const uint32_t* from = reinterpret_cast<const uint32_t*>(src.q[stripe_order(n, src.owner)] + rec);
-        if (n != 0)
-            __syncthreads(); // everyone has decoded the previous worker's record
-        for (uint32_t x = tid; x < rec_words; x += 8 * T)
+        const uint32_t G = min(group, K - n0);
+        if (n0 != 0)
+            __syncthreads(); // everyone has decoded the previous group
+        // decoding constants: one lane of a wavefront of its own per worker
+        for (uint32_t g = 0; g < G; ++g)
         {
-            uint32_t v[8];
+            if (tid == 64 * (g & 15u))
+            {
+                const float* h = reinterpret_cast<const float*>(src.q[stripe_order(n0 + g, src.owner)] + rec);
+                const float lo = h[0];
+                const float uf = make_ufactor<NBITS>(lo, h[1]);
+                if constexpr (NBITS == 1)
+                {
+                    dec[2 * g] = unquantize_value<NBITS>(uf, lo, 0u);
+                    dec[2 * g + 1] = unquantize_value<NBITS>(uf, lo, 1u);
+                }
+                else
+                {
+                    dec[2 * g] = uf;
+                    dec[2 * g + 1] = lo;
+                }
+            }
+        }
+        // the packed columns, four workers and four QWords per thread in flight together (one round trip for eight workers
+        // of a 100000-row column takes two passes, where a worker at a time took eight)
+        for (uint32_t g0 = 0; g0 < G; g0 += 4)
+        {
+            const uint32_t* from[4];
 #pragma unroll
-            for (uint32_t u = 0; u < 8; ++u)
-                v[u] = from[(x + T * u < rec_words) ? x + T * u : x];
+            for (uint32_t j = 0; j < 4; ++j)
+                from[j] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + min(g0 + j, G - 1), src.owner)] + rec) + 2;
+            for (uint32_t x = tid; x < c.nq; x += 4 * T)
+            {
+                uint32_t v[4][4];
 #pragma unroll
-            for (uint32_t u = 0; u < 8; ++u)
-                if (x + T * u < rec_words)
-                    pw[x + T * u] = v[u];
+                for (uint32_t j = 0; j < 4; ++j)
+#pragma unroll
+                    for (uint32_t u = 0; u < 4; ++u)
+                        v[j][u] = from[j][(x + T * u < c.nq) ? x + T * u : x];
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j)
+                    if (g0 + j < G)
+                    {
+                        uint32_t* to = pw + (size_t) (g0 + j) * c.nq;
+#pragma unroll
+                        for (uint32_t u = 0; u < 4; ++u)
+                            if (x + T * u < c.nq)
+                                to[x + T * u] = v[j][u];
+                    }
+            }
         }
         __syncthreads();
-        const float lo = __uint_as_float(pw[0]);
-        const float uf = make_ufactor<NBITS>(lo, __uint_as_float(pw[1]));
-        const float val0 = unquantize_value<NBITS>(uf, lo, 0u);
-        const float val1 = unquantize_value<NBITS>(uf, lo, 1u);
-        const uint32_t* bits = pw + 2;
-        // (opaque: the positions of all slots do not depend on the worker, and hoisted out of this loop they would be held
-        // in registers for its whole duration)
-        uint32_t k = opaque(k_first), w = opaque(w_first);
+        // (opaque: the positions of all slots do not depend on the group, and hoisted out of this loop they would be held
+        // in registers for its whole duration; the sums alone take 100 of a thread's 128 registers at 100000 rows)
         const uint32_t t = opaque(tid);
+        const uint32_t ufirst = t < shift ? 1u : 0u;
+        uint32_t k, w;
+        {
+            const uint32_t e0 = head + 4 * (t + T * ufirst - shift);
+            k = e0 / c.nq;
+            w = e0 - k * c.nq;
+        }
 #pragma unroll
         for (int u = 0; u < PER; ++u)
         {
             if (slot_valid(t + T * u, shift, pieces))
             {
-                uint32_t kk = k, ww = w;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
+                if (w + 3 < c.nq)
                 {
-                    float x;
-                    if constexpr (NBITS == 1)
-                        x = pick_level(bits[ww], kk, val0, val1);
-                    else
-                        x = unquantize_value<NBITS>(uf, lo, (bits[ww] >> (kk * PS::SHIFT)) & PS::CODEMASK);
-                    // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
-                    a[u][e] = (n == 0) ? x : x + a[u][e];
-                    if (++ww == c.nq)
+                    // the common case: four consecutive QWords, one bit position
+                    const uint32_t* bp = pw + w;
+                    const uint32_t sh = k * PS::SHIFT;
+                    for (uint32_t g = 0; g < G; ++g)
                     {
-                        ww = 0;
-                        ++kk;
+                        const uint32_t b0 = bp[0], b1 = bp[1], b2 = bp[2], b3 = bp[3];
+                        const float d0 = dec[2 * g], d1 = dec[2 * g + 1];
+                        bp += c.nq;
+                        if constexpr (NBITS == 1)
+                        {
+                            a[u].x = pick_level(b0, sh, d0, d1) + a[u].x;
+                            a[u].y = pick_level(b1, sh, d0, d1) + a[u].y;
+                            a[u].z = pick_level(b2, sh, d0, d1) + a[u].z;
+                            a[u].w = pick_level(b3, sh, d0, d1) + a[u].w;
+                        }
+                        else
+                        {
+                            a[u].x = unquantize_value<NBITS>(d0, d1, (b0 >> sh) & PS::CODEMASK) + a[u].x;
+                            a[u].y = unquantize_value<NBITS>(d0, d1, (b1 >> sh) & PS::CODEMASK) + a[u].y;
+                            a[u].z = unquantize_value<NBITS>(d0, d1, (b2 >> sh) & PS::CODEMASK) + a[u].z;
+                            a[u].w = unquantize_value<NBITS>(d0, d1, (b3 >> sh) & PS::CODEMASK) + a[u].w;
+                        }
+                    }
+                }
+                else
+                {
+                    // the piece runs past the last QWord: its later elements are the next bit position of the first QWords
+                    for (uint32_t g = 0; g < G; ++g)
+                    {
+                        const uint32_t* bits = pw + (size_t) g * c.nq;
+                        const float d0 = dec[2 * g], d1 = dec[2 * g + 1];
+                        uint32_t kk = k, ww = w;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            float x;
+                            if constexpr (NBITS == 1)
+                                x = pick_level(bits[ww], kk, d0, d1);
+                            else
+                                x = unquantize_value<NBITS>(d0, d1, (bits[ww] >> (kk * PS::SHIFT)) & PS::CODEMASK);
+                            a[u][e] = x + a[u][e];
+                            if (++ww == c.nq)
+                            {
+                                ww = 0;
+                                ++kk;
+                            }
+                        }
                     }
                 }
             }
@@ -389,13 +476,19 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<
         }
         if (has_edge)
         {
-            const uint32_t code = (bits[edge_w] >> (edge_k * PS::SHIFT)) & PS::CODEMASK;
-            float x;
-            if constexpr (NBITS == 1)
-                x = code ? val1 : val0;
-            else
-                x = unquantize_value<NBITS>(uf, lo, code);
-            edge = (n == 0) ? x : x + edge;
+            const uint32_t at = opaque(edge_at);
+            const uint32_t edge_k = at / c.nq;
+            const uint32_t edge_w = at - edge_k * c.nq;
+            for (uint32_t g = 0; g < G; ++g)
+            {
+                const uint32_t bits = pw[(size_t) g * c.nq + edge_w];
+                float x;
+                if constexpr (NBITS == 1)
+                    x = pick_level(bits, edge_k, dec[2 * g], dec[2 * g + 1]);
+                else
+                    x = unquantize_value<NBITS>(dec[2 * g], dec[2 * g + 1], (bits >> (edge_k * PS::SHIFT)) & PS::CODEMASK);
+                edge = x + edge;
+            }
         }
     }
     // aggregate out (optional), then the stripe residual in
@@ -427,6 +520,219 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<
         }
     }
     reg_stats_pack<NBITS, ZT, T, PER>(a, edge, has_edge, edge_at, head, pieces, shift, c, red, red_u, words, sres, q_out + rec);
+}
+
+// The 1-bit tall stripe reduction with up to eight workers decoded together from a worker-minor table in LDS. The kernel
+// above reads a piece's four QWords of one worker at a time (lanes 16 bytes apart, 4 bytes each: a quarter of the LDS
+// banks serve every access, and counters put the kernel at 122 us of LDS time for a 219 us run at 100000 x 512, K = 8).
+// Here QWord w of the group's worker g sits at dword (w / 4) * 36 + (w % 4) * 8 + g: the eight workers' copies of one QWord
+// are 32 consecutive bytes, fetched by two 16-byte reads, and the 4 padding dwords per row of 32 turn consecutive lanes
+// (QWords 4 apart) by 4 banks, so that every read and every fill of the table is free of bank conflicts. One worker's
+// level for a cleared bit is kept per thread, the level for a set bit per wavefront (scalar registers): a decoded value
+// costs a bit-field extract, a bitwise select and the addition.
+// LDS: [48 reduction slots | nq output QWords | 16 levels | padding to 16 bytes | ceil(nq / 4) rows of 36 dwords].
+constexpr uint32_t kStripe8Row = 36; // dwords; the decoder below spells 36 * 4 bytes out as shifts
+
+__host__ __device__ inline uint32_t stripe_reg8_table_offset(const RegGeom& c) // in dwords
+{
+    return (kRegRedSlots + c.nq + 16u + 3u) & ~3u;
+}
+
+__host__ __device__ inline size_t stripe_reg8_lds_bytes(const RegGeom& c)
+{
+    return ((size_t) stripe_reg8_table_offset(c) + (size_t) ((c.nq + 3) / 4) * kStripe8Row) * 4;
+}
+
+__device__ __forceinline__ float pick_level_s(uint32_t bits, uint32_t pos, float val0, float val1_uniform)
+{
+    const int32_t mask = __builtin_amdgcn_sbfe((int32_t) bits, pos, 1u);
+    float x;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(x) : "v"(mask), "s"(val1_uniform), "v"(val0));
+    return x;
+}
+
+template <bool ZT, int PER>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<1024, PER>(), reg_waves<1024, PER>()))) void stripe_reduce_reg8_kernel(
+    StripeSources src, float* stripe_res, char* q_out, float* agg_out, RegGeom c)
+{
+    constexpr uint32_t T = 1024, NW = T / 64, S = 8;
+    extern __shared__ f32x4 smem_v4[];
+    float* red = reinterpret_cast<float*>(smem_v4);
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
+    uint32_t* words = reinterpret_cast<uint32_t*>(red + kRegRedSlots);
+    float* dec = reinterpret_cast<float*>(words + c.nq); // [0, 8): level of a cleared bit per worker slot, [8, 16): of a set bit
+    uint32_t* tab = reinterpret_cast<uint32_t*>(red) + stripe_reg8_table_offset(c);
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * c.rows;
+    const size_t rec = (size_t) blockIdx.x * c.qcol;
+    for (uint32_t x = tid; x < c.nq; x += T)
+        words[x] = 0u;
+    float* sres = stripe_res + base;
+    const uint32_t head = (4u - (uint32_t) ((reinterpret_cast<uintptr_t>(sres) >> 2) & 3u)) & 3u;
+    const uint32_t pieces = (c.rows - head) >> 2;
+    const uint32_t tail = c.rows - head - 4 * pieces;
+    const bool has_edge = tid < head + tail;
+    const uint32_t edge_at = tid < head ? tid : c.rows - tail + (tid - head);
+    const uint32_t shift = column_shift(sres + head, c.line_shift);
+
+    // -0 is the additive identity (x + -0 = x for every x, signed zeros included)
+    f32x4 a[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+        a[u] = f32x4{-0.0f, -0.0f, -0.0f, -0.0f};
+    float edge = -0.0f;
+    const uint32_t K = src.workers;
+    for (uint32_t n0 = 0; n0 < K; n0 += S)
+    {
+        const uint32_t G = min(S, K - n0);
+        if (n0 != 0)
+            __syncthreads(); // everyone has decoded the previous group
+        for (uint32_t g = 0; g < S; ++g)
+        {
+            if (tid == 64 * g) // one lane of a wavefront of its own per worker slot; an empty slot decodes to -0
+            {
+                float v0 = -0.0f, v1 = -0.0f;
+                if (g < G)
+                {
+                    const float* h = reinterpret_cast<const float*>(src.q[stripe_order(n0 + g, src.owner)] + rec);
+                    const float lo = h[0];
+                    const float uf = make_ufactor<1>(lo, h[1]);
+                    v0 = unquantize_value<1>(uf, lo, 0u);
+                    v1 = unquantize_value<1>(uf, lo, 1u);
+                }
+                dec[g] = v0;
+                dec[S + g] = v1;
+            }
+        }
+        for (uint32_t g0 = 0; g0 < G; g0 += 4)
+        {
+            const uint32_t* from[4];
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                from[j] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + min(g0 + j, G - 1), src.owner)] + rec) + 2;
+            for (uint32_t x = tid; x < c.nq; x += 4 * T)
+            {
+                uint32_t v[4][4];
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j)
+#pragma unroll
+                    for (uint32_t u = 0; u < 4; ++u)
+                        v[j][u] = from[j][(x + T * u < c.nq) ? x + T * u : x];
+#pragma unroll
+                for (uint32_t u = 0; u < 4; ++u)
+                {
+                    const uint32_t w = x + T * u;
+                    if (w < c.nq)
+                    {
+                        uint32_t* to = tab + (w >> 2) * kStripe8Row + (w & 3u) * S + g0;
+#pragma unroll
+                        for (uint32_t j = 0; j < 4; ++j)
+                            if (g0 + j < G)
+                                to[j] = v[j][u];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        float val0[S], val1[S];
+#pragma unroll
+        for (uint32_t g = 0; g < S; ++g)
+        {
+            val0[g] = dec[g];
+            val1[g] = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(dec[S + g])));
+        }
+        // (opaque: the positions of all slots do not depend on the group, and hoisted out of this loop they would be held
+        // in registers for its whole duration; the sums alone take 100 of a thread's 128 registers at 100000 rows)
+        const uint32_t t = opaque(tid);
+        const uint32_t ufirst = t < shift ? 1u : 0u;
+        uint32_t k, w;
+        {
+            const uint32_t e0 = head + 4 * (t + T * ufirst - shift);
+            k = e0 / c.nq;
+            w = e0 - k * c.nq;
+        }
+        // With the last group the stripe residual is added piece by piece: a piece's residual is requested before its
+        // decoding and used after it, so that the memory latency runs under the arithmetic of this and the other
+        // wavefronts (one workgroup fills a CU: nothing else would overlap the two phases).
+        const bool last = n0 + S >= K;
+        const f32x4* r4 = reinterpret_cast<const f32x4*>(sres + head);
+        float* ag = agg_out != nullptr ? agg_out + base : nullptr;
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+        {
+            if (slot_valid(t + T * u, shift, pieces))
+            {
+                f32x4 rr = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                if (last)
+                    rr = __builtin_nontemporal_load(r4 + (t + T * u - shift));
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                {
+                    // element e of the piece: QWord w + e at bit k, or past the last QWord the next bit of the first ones
+                    uint32_t we = w + e, ke = k;
+                    if (we >= c.nq)
+                    {
+                        we -= c.nq;
+                        ++ke;
+                    }
+                    // byte offset of the eight workers' copies of QWord we: row (we / 4) of 144 bytes, 32 bytes per QWord
+                    const uint32_t row = we >> 2;
+                    const uint32_t off = (row << 7) + (row << 4) + ((we & 3u) << 5);
+                    const char* at = reinterpret_cast<const char*>(tab) + off;
+                    const u32x4 lo4 = *reinterpret_cast<const u32x4*>(at);
+                    const u32x4 hi4 = *reinterpret_cast<const u32x4*>(at + 16);
+                    // all eight slots, always: an empty slot's levels are both -0 and leave the sum as it is
+                    float acc = a[u][e];
+                    acc = pick_level_s(lo4.x, ke, val0[0], val1[0]) + acc;
+                    acc = pick_level_s(lo4.y, ke, val0[1], val1[1]) + acc;
+                    acc = pick_level_s(lo4.z, ke, val0[2], val1[2]) + acc;
+                    acc = pick_level_s(lo4.w, ke, val0[3], val1[3]) + acc;
+                    acc = pick_level_s(hi4.x, ke, val0[4], val1[4]) + acc;
+                    acc = pick_level_s(hi4.y, ke, val0[5], val1[5]) + acc;
+                    acc = pick_level_s(hi4.z, ke, val0[6], val1[6]) + acc;
+                    acc = pick_level_s(hi4.w, ke, val0[7], val1[7]) + acc;
+                    a[u][e] = acc;
+                }
+                if (last)
+                {
+                    if (ag != nullptr)
+                    {
+                        const uint32_t p = t + T * u - shift;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            ag[head + 4 * p + e] = a[u][e];
+                    }
+                    a[u] = a[u] + rr;
+                }
+            }
+            if ((uint32_t) u >= ufirst)
+            {
+                w += c.step_w;
+                k += c.step_k;
+                if (w >= c.nq)
+                {
+                    w -= c.nq;
+                    ++k;
+                }
+            }
+        }
+        if (has_edge)
+        {
+            const uint32_t at = opaque(edge_at);
+            const uint32_t edge_k = at / c.nq;
+            const uint32_t edge_w = at - edge_k * c.nq;
+            const uint32_t* p = tab + (edge_w >> 2) * kStripe8Row + (edge_w & 3u) * S;
+            for (uint32_t g = 0; g < G; ++g)
+                edge = pick_level(p[g], edge_k, dec[g], dec[S + g]) + edge;
+        }
+    }
+    if (has_edge)
+    {
+        if (agg_out != nullptr)
+            agg_out[base + edge_at] = edge;
+        edge = edge + sres[edge_at];
+    }
+    reg_stats_pack<1, ZT, T, PER>(a, edge, has_edge, edge_at, head, pieces, shift, c, red, red_u, words, sres, q_out + rec);
 }
 
 // ---- the same for tall columns of any height and alignment: elements instead of pieces ----------------------

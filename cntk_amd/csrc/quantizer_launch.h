@@ -513,8 +513,20 @@ template <int NBITS, bool ZT, int PER>
 inline hipError_t launch_stripe_reg_one(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
                                         uint32_t cols, const RegGeom& c)
 {
-    hipExtLaunchKernelGGL((stripe_reduce_reg_kernel<NBITS, ZT, PER>), dim3(cols), dim3(1024), stripe_reg_lds_bytes(c), s, ev.start, ev.stop, 0,
-                          src, stripe_res, q_out, agg_out, c);
+    if constexpr (NBITS == 1)
+    {
+        // 1 bit: eight workers at a time from the worker-minor table, where a CU's LDS holds it (always, up to 102400 rows)
+        // (it always decodes eight slots: with four workers or fewer the kernel below does less work)
+        if (src.workers > 4 && stripe_reg8_lds_bytes(c) <= 160 * 1024)
+        {
+            hipExtLaunchKernelGGL((stripe_reduce_reg8_kernel<ZT, PER>), dim3(cols), dim3(1024), stripe_reg8_lds_bytes(c), s, ev.start, ev.stop, 0,
+                                  src, stripe_res, q_out, agg_out, c);
+            return hipGetLastError();
+        }
+    }
+    const uint32_t group = stripe_reg_group(c, src.workers);
+    hipExtLaunchKernelGGL((stripe_reduce_reg_kernel<NBITS, ZT, PER>), dim3(cols), dim3(1024), stripe_reg_lds_bytes(c, group), s, ev.start,
+                          ev.stop, 0, src, stripe_res, q_out, agg_out, c, group);
     return hipGetLastError();
 }
 
