@@ -62,7 +62,7 @@ def build_library(verbose=False, only=None):
     return LIB_PATH
 
 
-CPP_TESTS = ["test_matrix_quantizer", "test_allreduce_aggregator", "test_distributed_learner", "bench_allreduce"]
+CPP_TESTS = ["test_matrix_quantizer", "test_allreduce_aggregator", "test_distributed_learner", "test_quantized_communicator", "bench_allreduce"]
 
 
 def build_cpp_tests(verbose=False):

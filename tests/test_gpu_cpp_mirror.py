@@ -49,6 +49,20 @@ def test_cpp_distributed_learner_suite():
 
 
 @pytest.mark.gpu
+def test_cpp_quantized_communicator_suite():
+    """The v2 communicator's call shape (cntk_amd/cpp/QuantizedDistributedCommunicator.h): out-of-place values and residues
+    against the aliased form, against the v1 aggregator, float and double by argument type."""
+    exe = os.path.join(ROOT, "tests", "cpp", "bin", "test_quantized_communicator")
+    assert os.path.exists(exe), "build it first: python -m cntk_amd.build"
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    print(res.stdout)
+    print(res.stderr[-4000:])
+    assert res.returncode == 0, "C++ communicator tests failed"
+    for name in ("OutOfPlaceEqualsAliasedFloat", "OutOfPlaceEqualsAliasedDouble", "EqualsAggregatorAndCallSequence", "TypesAndTrivialCases"):
+        assert "CommunicatorSuite/%s has passed" % name in res.stdout
+
+
+@pytest.mark.gpu
 def test_cpp_allreduce_timing_program_runs():
     """The all-reduce timing program runs through on a small shape and prints one line per arrangement."""
     exe = os.path.join(ROOT, "tests", "cpp", "bin", "bench_allreduce")
