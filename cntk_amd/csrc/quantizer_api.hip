@@ -70,6 +70,13 @@ struct BatchAbi<float>
             e.c = make_col_geom(it.rows, nbits, line_shift);
             lds = colg_lds_bytes_rt(e.c, nbits);
             blocks = it.cols;
+            // a few tall columns (a bias vector) do not get a launch with more LDS to themselves: they stage the column in
+            // the residual's memory and join the other members (same bytes)
+            if (lds > kBatchSmallLds && it.cols <= kStagedInResidualMaxCols)
+            {
+                e.kind = 5;
+                lds = ((nbits <= 2 ? e.c.nq : 0) + 12) * sizeof(float);
+            }
             // 1 bit, 1024 / 2048 / 4096 rows, columns on 128-byte lines, 8-byte aligned records: the unrolled body (same bytes)
             if (!line_shift && col_unrolled(it.qbuf, it.rows, nbits))
             {
@@ -80,6 +87,7 @@ struct BatchAbi<float>
         }
         return false;
     }
+    static bool first_in_grid(const QEntry& e) { return e.kind == 5; }
     static hipError_t launch_quantize_members(hipStream_t s, LaunchEvents ev, const QEntry* de, const uint32_t* db, uint32_t members,
                                               uint32_t blocks, size_t lds, size_t nbits, bool zt)
     {

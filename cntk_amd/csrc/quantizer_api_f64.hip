@@ -64,6 +64,7 @@ struct BatchAbi<double>
         blocks = (e.t.cols + e.t.cols_per_tile - 1) / e.t.cols_per_tile;
         return true;
     }
+    static bool first_in_grid(const QEntry&) { return false; }
     static hipError_t launch_quantize_members(hipStream_t s, LaunchEvents ev, const QEntry* de, const uint32_t* db, uint32_t members,
                                               uint32_t blocks, size_t lds, size_t nbits, bool zt)
     {

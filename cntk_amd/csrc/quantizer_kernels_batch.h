@@ -40,7 +40,9 @@ struct QuantizeBatchEntry
     const float* r_in;
     float* r_out;
     char* q;
-    uint32_t kind; // 0: tiles (t), 1: columns (c), 2 / 3 / 4: 1-bit columns of 1024 / 2048 / 4096 rows (the unrolled body; c.qcol)
+    // 0: tiles (t), 1: columns (c), 2 / 3 / 4: 1-bit columns of 1024 / 2048 / 4096 rows (the unrolled body; c.qcol),
+    // 5: columns staged in the residual's memory instead of LDS (c)
+    uint32_t kind;
     uint32_t pad;
     TileGeom t;
     ColGeom c;
@@ -58,6 +60,11 @@ __global__ __launch_bounds__(kTileThreads) void quantize_batch_kernel(const Quan
     {
         const TileGeom t = entries[e].t;
         quantize_tile_body<NBITS, ZT>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, t, index);
+    }
+    else if (entries[e].kind == 5)
+    {
+        const ColGeom c = entries[e].c;
+        quantize_colg_body<NBITS, ZT, true>(entries[e].g, entries[e].r_in, entries[e].r_out, entries[e].q, c, index, smem_v4);
     }
     else if (NBITS != 1 || entries[e].kind == 1)
     {

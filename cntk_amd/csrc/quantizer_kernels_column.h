@@ -471,17 +471,21 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
     }
 }
 
-template <int NBITS, bool ZT>
+// IN_RESIDUAL: the column v = g + r is staged in the residual output's own column in memory instead of LDS (every
+// element is then read back and replaced by its residual by the thread that coded it; all phases are separated by
+// workgroup barriers). Twice the traffic, served by L2 -- for the few tall columns of a gradient set (a 9304-row bias
+// vector) that would otherwise need a launch with more LDS per workgroup all to themselves: 12 us for one workgroup.
+template <int NBITS, bool ZT, bool IN_RESIDUAL = false>
 __device__ __forceinline__ void quantize_colg_body(const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q,
                                                    const ColGeom& c, uint32_t column, f32x4* smem)
 {
     using PS = PackShape<NBITS>;
     constexpr uint32_t T = kColThreads;
-    float* tile = reinterpret_cast<float*>(smem);
-    uint32_t* words = reinterpret_cast<uint32_t*>(tile + c.rows);
-    float* red = tile + c.rows + (PS::CHUNKS > 1 ? c.nq : 0);
     const uint32_t tid = threadIdx.x;
     const size_t base = (size_t) column * c.rows;
+    float* tile = IN_RESIDUAL ? r_out + base : reinterpret_cast<float*>(smem);
+    uint32_t* words = reinterpret_cast<uint32_t*>(smem) + (IN_RESIDUAL ? 0u : c.rows);
+    float* red = reinterpret_cast<float*>(words + (PS::CHUNKS > 1 ? c.nq : 0));
     if constexpr (PS::CHUNKS > 1)
         for (uint32_t x = tid; x < c.nq; x += T)
             words[x] = 0u;
