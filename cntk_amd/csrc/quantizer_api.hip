@@ -63,7 +63,8 @@ struct BatchAbi<float>
             return true;
         }
         // (a register-kernel matrix of modest size gives the same bytes as a member: a launch costs more than it gains)
-        if (path == kPathCol || (path == kPathReg && it.rows <= kTileMaxRows && it.rows * it.cols < kOwnLaunchElements))
+        if (path == kPathCol || (path == kPathReg && it.rows <= kTileMaxRows && it.rows * it.cols < kOwnLaunchElements &&
+                                 reg_applicable(it.in, it.res_in, it.res_out, it.qbuf, it.rows, nbits)))
         {
             const bool line_shift = quantize_line_shift(it.in, it.res_in, it.res_out, it.rows);
             e.kind = 1;
@@ -126,7 +127,7 @@ struct BatchAbi<float>
 
     static size_t stripe_max_rows(size_t nbits) { return stripe_reduce_max_rows(nbits); }
     // taller stripes run 1024 threads per column: a launch of their own
-    static bool stripe_is_member(const SItem& it, size_t) { return it.rows <= kTileMaxRows; }
+    static bool stripe_is_member(const SItem& it, size_t nbits) { return !stripe_uses_reg(it.rows, it.stripe_res, nbits); }
     static int stripe_one(cntkq_quantizer* h, const SItem& it, size_t workers, size_t owner, size_t nbits, int zt)
     {
         return cntkq_stripe_reduce_async(h, it.stripes, workers, owner, it.rows, it.stripe_cols, nbits, it.stripe_res, it.q_out, it.agg_out, zt);

@@ -371,6 +371,11 @@ inline bool reg_edge_applicable(const float* g, const float* r_in, const float* 
     return (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
 }
 
+// From this height on the 1024-thread register kernel with edge elements beats the tile kernel on matrices that are not
+// whole aligned pieces: 9305 x 2048 44 us against 57 us, 14335 x 1400 44 us against 82 us (4097 x 4652: 73 us against 48 us).
+// The fused stripe reduction follows with its own 1024-thread kernel, which sums in the same order.
+constexpr uint32_t kRegEdgeMinRows = 7168;
+
 constexpr uint32_t kRegsMaxRows = 1024 * 96;
 
 inline bool regs_applicable(size_t rows, size_t nbits)
@@ -419,12 +424,11 @@ inline int quantize_auto_path(const float* g, const float* r_in, const float* r_
                           !quantize_line_shift(g, r_in, r_out, rows);
     if (!unrolled && reg_applicable(g, r_in, r_out, q, rows, nbits))
         return kPathReg;
+    // not whole aligned pieces (odd heights, slices at a 4-byte offset): the register kernel with edge elements
+    if (rows > kRegEdgeMinRows && reg_edge_applicable(g, r_in, r_out, q, rows, nbits))
+        return kPathReg;
     if (rows > kTileMaxRows)
-    {
-        if (reg_edge_applicable(g, r_in, r_out, q, rows, nbits))
-            return kPathReg;
         return regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
-    }
     if (col_applicable(g, r_in, r_out, q, rows, nbits))
         return kPathCol;
     return kPathTile;
@@ -556,12 +560,23 @@ struct StripeRegLauncher
     }
 };
 
+// Whether the fused stripe reduction runs the 1024-thread register kernel: wherever a quantize call on (aggregate, stripe
+// residual) would run the 1024-thread register kernels, whose summation order it shares -- above the LDS kernels' heights,
+// and from kRegEdgeMinRows on for stripes that are not whole aligned pieces.
+inline bool stripe_uses_reg(size_t rows, const void* stripe_res, size_t nbits, int forced_path = kPathAuto)
+{
+    if (rows > kTileMaxRows)
+        return true;
+    const bool whole = rows % 4 == 0 && (reinterpret_cast<uintptr_t>(stripe_res) & 15u) == 0;
+    return forced_path == kPathAuto && rows > kRegEdgeMinRows && !whole && nbits < 32;
+}
+
 inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, void* q_out,
                                        float* agg_out, size_t rows, size_t cols, size_t nbits, bool zt,
                                        const LaunchTuning& tune)
 {
     zt = zt && (nbits == 1);
-    if (rows > kTileMaxRows)
+    if (stripe_uses_reg(rows, stripe_res, nbits, tune.quantize_path))
     {
         if (rows > stripe_reduce_max_rows(nbits) || (reinterpret_cast<uintptr_t>(q_out) & 3u) != 0)
             return hipErrorInvalidValue;
