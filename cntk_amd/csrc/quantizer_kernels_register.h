@@ -307,13 +307,13 @@ __host__ __device__ inline uint32_t stripe_reg_group(const RegGeom& c, uint32_t 
     return (uint32_t) (g < workers ? g : workers);
 }
 
-template <int NBITS, bool ZT, int PER>
-__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<1024, PER>(), reg_waves<1024, PER>()))) void stripe_reduce_reg_kernel(
+template <int NBITS, bool ZT, int PER, int TT = 1024>
+__global__ __launch_bounds__(TT) __attribute__((amdgpu_waves_per_eu(reg_waves<TT, PER>(), reg_waves<TT, PER>()))) void stripe_reduce_reg_kernel(
     StripeSources src, float* stripe_res, char* q_out, float* agg_out, RegGeom c, uint32_t group)
 {
     using PS = PackShape<NBITS>;
     static_assert(NBITS < 32, "32-bit codes are whole QWords: nothing to assemble");
-    constexpr uint32_t T = 1024, NW = T / 64;
+    constexpr uint32_t T = TT, NW = T / 64;
     extern __shared__ f32x4 smem_v4[];
     float* red = reinterpret_cast<float*>(smem_v4);
     uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<
         // decoding constants: one lane of a wavefront of its own per worker
         for (uint32_t g = 0; g < G; ++g)
         {
-            if (tid == 64 * (g & 15u))
+            if (tid == 64 * (g & (NW - 1u)))
             {
                 const float* h = reinterpret_cast<const float*>(src.q[stripe_order(n0 + g, src.owner)] + rec);
                 const float lo = h[0];

@@ -252,26 +252,36 @@ inline hipError_t launch_reg_one(hipStream_t s, LaunchEvents ev, const float* g,
     return hipGetLastError();
 }
 
-template <int NBITS, bool ZT, int PER>
+template <int NBITS, bool ZT, int PER, int T = 1024>
 inline hipError_t launch_reg_edge_one(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
                                       const RegGeom& c)
 {
-    hipExtLaunchKernelGGL((quantize_reg_kernel<NBITS, ZT, 1024, PER, true>), dim3(cols), dim3(1024), reg_lds_bytes(c), s, ev.start, ev.stop, 0,
+    hipExtLaunchKernelGGL((quantize_reg_kernel<NBITS, ZT, T, PER, true>), dim3(cols), dim3(T), reg_lds_bytes(c), s, ev.start, ev.stop, 0,
                           g, r_in, r_out, q, c);
     return hipGetLastError();
 }
 
-// The variant for columns that start anywhere and have any height (1024 threads only): c.pieces is an upper bound.
+// The variant for columns that start anywhere and have any height: c.pieces is an upper bound. 256 threads up to
+// kRegEdgeMinRows rows (2049 x 9304: the tile kernel's 57 us), 1024 above.
 template <int NBITS, bool ZT>
 struct RegEdgeLauncher
 {
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, RegGeom c)
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, RegGeom c,
+                          uint32_t threads)
     {
         if constexpr (NBITS >= 32)
             return hipErrorInvalidValue;
         else
         {
-            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + 1023u) / 1024u;
+            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + threads - 1) / threads;
+#define CNTKQ_REGE256(P) if (threads == 256 && per <= P) return launch_reg_edge_one<NBITS, ZT, P, 256>(s, ev, g, r_in, r_out, q, cols, c)
+            CNTKQ_REGE256(3);
+            CNTKQ_REGE256(4);
+            CNTKQ_REGE256(6);
+            CNTKQ_REGE256(8);
+#undef CNTKQ_REGE256
+            if (threads != 1024)
+                return hipErrorInvalidValue;
 #define CNTKQ_REGE(P) if (per <= P) return launch_reg_edge_one<NBITS, ZT, P>(s, ev, g, r_in, r_out, q, cols, c)
             CNTKQ_REGE(4);
             CNTKQ_REGE(6);
@@ -371,10 +381,23 @@ inline bool reg_edge_applicable(const float* g, const float* r_in, const float* 
     return (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
 }
 
-// From this height on the 1024-thread register kernel with edge elements beats the tile kernel on matrices that are not
-// whole aligned pieces: 9305 x 2048 44 us against 57 us, 14335 x 1400 44 us against 82 us (4097 x 4652: 73 us against 48 us).
-// The fused stripe reduction follows with its own 1024-thread kernel, which sums in the same order.
+// Matrices that are not whole aligned pieces (odd heights, slices at a 4-byte offset) above kRegEdge256MinRows rows: the
+// register kernels with edge elements. From this height on with 1024 threads per column (9305 x 2048 44 us against the tile kernel's
+// 57 us, 14335 x 1400 44 us against 82 us; at 4097 x 4652 the 1024 threads take 73 us against 48 us). The fused stripe
+// reduction follows with its register kernel of the same workgroup size, which sums in the same order.
 constexpr uint32_t kRegEdgeMinRows = 7168;
+
+// ... and below it the same kernels with 256 threads per column, down to 2049 rows: 2049 x 9304 38.5 us against the tile
+// kernel's 56 us, 4097 x 4652 40 us against 47 us, 6001 x 3000 38 us against 48 us. The stripe reduction that has to follow
+// is slower than the tile one at these heights (full width, K = 8: 90 us against 86 us, 84 against 74, 78 against 63), but
+// an all-reduce runs it on one K-th of the columns. At 1026 x 18000 the quantize kernels measure the same (49 us) and the
+// stripe reductions 126 us against 85 us: up to 2048 rows the tile kernels stay.
+constexpr uint32_t kRegEdge256MinRows = 2048;
+
+inline uint32_t reg_edge_threads(size_t rows)
+{
+    return rows <= kRegEdgeMinRows ? 256u : 1024u;
+}
 
 constexpr uint32_t kRegsMaxRows = 1024 * 96;
 
@@ -425,7 +448,7 @@ inline int quantize_auto_path(const float* g, const float* r_in, const float* r_
     if (!unrolled && reg_applicable(g, r_in, r_out, q, rows, nbits))
         return kPathReg;
     // not whole aligned pieces (odd heights, slices at a 4-byte offset): the register kernel with edge elements
-    if (rows > kRegEdgeMinRows && reg_edge_applicable(g, r_in, r_out, q, rows, nbits))
+    if (rows > kRegEdge256MinRows && reg_edge_applicable(g, r_in, r_out, q, rows, nbits))
         return kPathReg;
     if (rows > kTileMaxRows)
         return regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
@@ -452,8 +475,9 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
             // not whole aligned pieces: the variant with edge elements, where the three matrices allow it
             if (!reg_edge_applicable(g, r_in, r_out, q, rows, nbits))
                 return hipErrorInvalidValue;
-            RegGeom c = make_reg_geom(rows, nbits, 1024, true); // always dealt by the residual's lines
-            return dispatch_nbits<RegEdgeLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c);
+            const uint32_t threads = reg_edge_threads(rows);
+            RegGeom c = make_reg_geom(rows, nbits, threads, true); // always dealt by the residual's lines
+            return dispatch_nbits<RegEdgeLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, threads);
         }
         const uint32_t threads = reg_threads(rows);
         // up to 14336 rows the shift is part of the summation order all column kernels share; above, it is used where
@@ -513,11 +537,11 @@ inline size_t stripe_reduce_max_rows(size_t nbits)
     return tall > kTileMaxRows ? tall : kTileMaxRows;
 }
 
-template <int NBITS, bool ZT, int PER>
+template <int NBITS, bool ZT, int PER, int T = 1024>
 inline hipError_t launch_stripe_reg_one(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
                                         uint32_t cols, const RegGeom& c)
 {
-    if constexpr (NBITS == 1)
+    if constexpr (NBITS == 1 && T == 1024)
     {
         // 1 bit: eight workers at a time from the worker-minor table, where a CU's LDS holds it (always, up to 102400 rows)
         // (it always decodes eight slots: with four workers or fewer the kernel below does less work)
@@ -529,7 +553,7 @@ inline hipError_t launch_stripe_reg_one(hipStream_t s, LaunchEvents ev, const St
         }
     }
     const uint32_t group = stripe_reg_group(c, src.workers);
-    hipExtLaunchKernelGGL((stripe_reduce_reg_kernel<NBITS, ZT, PER>), dim3(cols), dim3(1024), stripe_reg_lds_bytes(c, group), s, ev.start,
+    hipExtLaunchKernelGGL((stripe_reduce_reg_kernel<NBITS, ZT, PER, T>), dim3(cols), dim3(T), stripe_reg_lds_bytes(c, group), s, ev.start,
                           ev.stop, 0, src, stripe_res, q_out, agg_out, c, group);
     return hipGetLastError();
 }
@@ -538,13 +562,21 @@ template <int NBITS, bool ZT>
 struct StripeRegLauncher
 {
     static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out, uint32_t cols,
-                          RegGeom c)
+                          RegGeom c, uint32_t threads)
     {
         if constexpr (NBITS >= 32)
             return hipErrorInvalidValue;
         else
         {
-            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + 1023u) / 1024u;
+            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + threads - 1) / threads;
+#define CNTKQ_SREG256(P) if (threads == 256 && per <= P) return launch_stripe_reg_one<NBITS, ZT, P, 256>(s, ev, src, stripe_res, q_out, agg_out, cols, c)
+            CNTKQ_SREG256(3);
+            CNTKQ_SREG256(4);
+            CNTKQ_SREG256(6);
+            CNTKQ_SREG256(8);
+#undef CNTKQ_SREG256
+            if (threads != 1024)
+                return hipErrorInvalidValue;
 #define CNTKQ_SREG(P) if (per <= P) return launch_stripe_reg_one<NBITS, ZT, P>(s, ev, src, stripe_res, q_out, agg_out, cols, c)
             CNTKQ_SREG(4);
             CNTKQ_SREG(6);
@@ -561,14 +593,14 @@ struct StripeRegLauncher
 };
 
 // Whether the fused stripe reduction runs the 1024-thread register kernel: wherever a quantize call on (aggregate, stripe
-// residual) would run the 1024-thread register kernels, whose summation order it shares -- above the LDS kernels' heights,
-// and from kRegEdgeMinRows on for stripes that are not whole aligned pieces.
+// residual) would run the register kernels with edge elements or with 1024 threads, whose summation order it shares -- above
+// the LDS kernels' heights, and from kRegEdge256MinRows + 1 rows on for stripes that are not whole aligned pieces.
 inline bool stripe_uses_reg(size_t rows, const void* stripe_res, size_t nbits, int forced_path = kPathAuto)
 {
     if (rows > kTileMaxRows)
         return true;
     const bool whole = rows % 4 == 0 && (reinterpret_cast<uintptr_t>(stripe_res) & 15u) == 0;
-    return forced_path == kPathAuto && rows > kRegEdgeMinRows && !whole && nbits < 32;
+    return forced_path == kPathAuto && rows > kRegEdge256MinRows && !whole && nbits < 32;
 }
 
 inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, void* q_out,
@@ -587,8 +619,11 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
         bool line_shift = whole ? !columns_start_on_lines(stripe_res, rows) : true;
         if (whole && rows / 4 + 7 > 1024 * (size_t) kRegMaxShiftPer)
             line_shift = false;
-        const RegGeom c = make_reg_geom(rows, nbits, 1024, line_shift);
-        return dispatch_nbits<StripeRegLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols, c);
+        // (only stripes that are not whole aligned pieces get here below the LDS kernels' limit: 256 threads up to 7168 rows)
+        const uint32_t threads = rows > kTileMaxRows ? 1024u : reg_edge_threads(rows);
+        const RegGeom c = make_reg_geom(rows, nbits, threads, line_shift);
+        return dispatch_nbits<StripeRegLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols, c,
+                                                 threads);
     }
     bool aligned8 = (reinterpret_cast<uintptr_t>(q_out) & 7u) == 0;
     for (uint32_t w = 0; w < src.workers; ++w)

@@ -57,7 +57,9 @@ CASES = [
     # above 14336 rows: the register kernel's shape (the running sum in registers, one worker's record at a time in LDS)
     (14340, 6, 4, 1, False), (14337, 3, 2, 2, False), (20000, 5, 3, 1, True), (32768, 4, 5, 4, False), (50257, 3, 8, 1, False),
     (100000, 2, 2, 1, False), (102365, 2, 3, 2, False), (16332, 2, 2, 16, False), (32668, 2, 2, 8, False),
-    # heights that are not a multiple of 4: the tile kernels up to 7168 rows, the 1024-thread register kernels above
+    # heights that are not a multiple of 4: the tile kernels up to 2048 rows, above them the register kernels with edge
+    # elements (256 threads per column up to 7168 rows, 1024 above)
+    (1023, 6, 3, 1, False), (1025, 6, 3, 1, False), (2049, 8, 8, 1, False), (2050, 5, 2, 1, True), (4097, 4, 3, 4, False), (6001, 3, 5, 2, False),
     (7167, 4, 3, 1, False), (7169, 3, 2, 4, False), (7170, 4, 3, 1, True), (8001, 4, 2, 2, False), (9305, 3, 3, 1, False),
     (14335, 2, 8, 1, False), (9305, 2, 2, 32, False),
 ]
