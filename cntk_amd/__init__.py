@@ -105,6 +105,7 @@ def lib():
             getattr(L, name).argtypes = [_sz]
             getattr(L, name).restype = _sz
         L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int]
+        L.cntkq_debug_set_strip_spin_limit.argtypes = [_vp, ctypes.c_uint]
         _lib = L
     return _lib
 
@@ -538,6 +539,9 @@ class MatrixQuantizerImpl:
 
     def _set_tuning(self, quantize_path=0, tile_gs=0, unq_slots=0, unq_mode=0, tile_stage=-1):
         _check(lib().cntkq_debug_set_tuning(self._h, quantize_path, tile_gs, unq_slots, unq_mode, tile_stage))
+
+    def _set_strip_spin_limit(self, limit):
+        _check(lib().cntkq_debug_set_strip_spin_limit(self._h, limit))
 
 
 class MatrixQuantizer:

@@ -94,9 +94,10 @@ struct BatchAbi<float>
     {
         return launch_quantize_batch(s, ev, de, db, members, blocks, lds, nbits, zt);
     }
-    static hipError_t launch_quantize_own(hipStream_t s, LaunchEvents ev, const QItem& it, size_t nbits, bool zt)
+    static hipError_t launch_quantize_own(cntkq_quantizer* h, hipStream_t s, LaunchEvents ev, const QItem& it, size_t nbits, bool zt)
     {
         LaunchTuning autotune;
+        autotune.strip = &h->strip_scratch;
         return launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune);
     }
 
@@ -402,7 +403,10 @@ int quantize_batch_noalloc_impl(cntkq_quantizer* h, const cntkq_quantize_item* i
         LaunchEvents ev;
         launches_left--;
         ev.stop = launches_left == 0 ? done : nullptr;
-        HIP_TRY(A::launch_quantize_own(s, ev, items[st.own[k]], nbits, zt), "quantize kernel launch failed");
+        // (without the strip kernels, whose scratch buffer is allocated on demand: this call allocates nothing)
+        const cntkq_quantize_item& it = items[st.own[k]];
+        LaunchTuning no_strip;
+        HIP_TRY(launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, no_strip), "quantize kernel launch failed");
     }
     h->last_quantize = done;
     h->quantize_included_fetch = false;
@@ -471,6 +475,7 @@ int cntkq_create(int device_id, int use_dedicated_stream, cntkq_quantizer** out)
         return fail(CNTKQ_RUNTIME_ERROR, "cntkq_create: out of host memory");
     h->device = device_id;
     h->dedicated = use_dedicated_stream != 0;
+    h->tune.strip = &h->strip_scratch;
     {
         std::lock_guard<std::mutex> lock(g_streams_mutex);
         DeviceStreams& ds = g_streams[device_id];
@@ -527,6 +532,13 @@ int cntkq_create(int device_id, int use_dedicated_stream, cntkq_quantizer** out)
             return fail(CNTKQ_RUNTIME_ERROR, "hipEventCreateWithFlags failed: %s", hipGetErrorString(rc));
         }
     }
+    {
+        // The strip kernels' scratch buffer at its starting size, so that a first call under graph capture (which cannot
+        // allocate) finds it. A failure here is not one of the handle: the first call that needs the buffer tries again.
+        StripScratch unused;
+        if (strip_scratch_for(h->strip_scratch, nullptr, 1, 2, unused) != hipSuccess || hipStreamSynchronize(nullptr) != hipSuccess)
+            (void) hipGetLastError();
+    }
     *out = h;
     return CNTKQ_OK;
 }
@@ -543,6 +555,10 @@ int cntkq_destroy(cntkq_quantizer* h)
     if (h->ev_stripe) (void) hipEventSynchronize(h->ev_stripe);
     if (h->staging != nullptr)
         (void) hipFree(h->staging);
+    if (h->strip_scratch.dev != nullptr)
+        (void) hipFree(h->strip_scratch.dev);
+    if (h->strip_scratch.error_host != nullptr)
+        (void) hipHostFree(h->strip_scratch.error_host);
     table_destroy(h->quantize_table);
     table_destroy(h->unquantize_table);
     table_destroy(h->stripe_table);
@@ -621,7 +637,8 @@ int cntkq_wait_quantize_done(cntkq_quantizer* h)
             h->fetch_pending = false;
         return rc;
     }
-    return h->last_quantize != nullptr ? sync_event(h->last_quantize) : CNTKQ_OK;
+    const int rc = h->last_quantize != nullptr ? sync_event(h->last_quantize) : CNTKQ_OK;
+    return rc != CNTKQ_OK ? rc : check_strip_error(h);
 }
 
 int cntkq_unquantize_async(cntkq_quantizer* h, const void* qbuf, size_t qbuf_bytes, int qbuf_on_host, float* out,
@@ -697,7 +714,7 @@ int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_
 {
     if (h == nullptr)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: null handle");
-    if (quantize_path < kPathAuto || quantize_path > kPathRegScalar)
+    if (quantize_path < kPathAuto || quantize_path > kPathStrip)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: unknown quantize path %d", quantize_path);
     if (tile_gs != 0 && (tile_gs < 8 || tile_gs > kTileThreads || (tile_gs & (tile_gs - 1)) != 0))
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: tile_gs must be a power of two in [8, 256]");
@@ -706,6 +723,16 @@ int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_
     h->tune.unq_slots = unq_slots;
     h->tune.unq_mode = unq_mode;
     h->tune.tile_stage = tile_stage;
+    return CNTKQ_OK;
+}
+
+// How often a lane of a strip kernel polls for another workgroup's partial sum before it gives up (tests of the error path
+// set it to zero: every kernel still runs to its end).
+int cntkq_debug_set_strip_spin_limit(cntkq_quantizer* h, unsigned limit)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_strip_spin_limit: null handle");
+    h->tune.strip_spin_limit = limit;
     return CNTKQ_OK;
 }
 

@@ -70,7 +70,7 @@ struct BatchAbi<double>
     {
         return f64::dispatch_nbits64<f64::QuantizeBatchLauncher64>(nbits, zt && nbits == 1, s, ev, de, db, members, blocks, lds);
     }
-    static hipError_t launch_quantize_own(hipStream_t s, LaunchEvents ev, const QItem& it, size_t nbits, bool zt)
+    static hipError_t launch_quantize_own(cntkq_quantizer*, hipStream_t s, LaunchEvents ev, const QItem& it, size_t nbits, bool zt)
     {
         LaunchTuning autotune;
         return f64::launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune);

@@ -185,6 +185,7 @@ struct cntkq_quantizer
     BatchTable unquantize_table64;
     BatchTable stripe_table64;
     cntkq::LaunchTuning tune;
+    cntkq::StripScratchOwner strip_scratch; // partial sums and launch count of the strip kernels (tune.strip points here)
     struct NoAllocState* noalloc = nullptr; // fixed-size host state of cntkq_quantize_batch_noalloc (created with the handle)
 };
 
@@ -369,6 +370,22 @@ inline void table_destroy(BatchTable& t)
         (void) hipHostFree(r.first);
         (void) hipFree(r.second);
     }
+}
+
+// After a wait: a strip kernel whose workgroups gave up waiting for one another has raised the error word (launches
+// replayed from a graph included, so the word is looked at whenever it exists).
+inline int check_strip_error(cntkq_quantizer* h)
+{
+    cntkq::StripScratchOwner& o = h->strip_scratch;
+    if (o.error_host == nullptr)
+        return CNTKQ_OK;
+    if (*static_cast<volatile uint32_t*>(o.error_host) != 0u)
+    {
+        *o.error_host = 0u;
+        return fail(CNTKQ_RUNTIME_ERROR,
+                    "quantize: the workgroups of a column gave up waiting for each other's partial sums; the result of the call is invalid");
+    }
+    return CNTKQ_OK;
 }
 
 inline int sync_event(hipEvent_t ev) // SyncEvent (Source/Math/MatrixQuantizerGPU.cu:68-80)

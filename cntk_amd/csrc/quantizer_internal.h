@@ -15,6 +15,8 @@ extern "C" {
  *                        three matrices at the same offset within 16 bytes),
  *                    5 = the same with one element per access: fp32 any alignment, up to 98304 rows; fp64 256 threads per
  *                        column, 1025 to 6144 rows, below 64 bits, the bytes of path 1
+ *                    6 = several workgroups per column, a strip of QWords each (fp32, 1 to 16 bits, any height whose
+ *                        strips number at most 64 per column, any alignment)
  *   tile_gs          0 = automatic, else threads per column in the tile statistics phase (power of two, 8..256)
  *   unq_slots        0 = automatic, else bit positions decoded per thread by the QWord-major unquantize
  *   unq_mode         0 = automatic, 1 = QWord-major decoder with one store per value, 2 = tile decoder wherever it can run,
@@ -22,6 +24,11 @@ extern "C" {
  *   tile_stage       -1 = automatic, 0 = tile kernels write the residual straight to memory, 1 = through LDS */
 int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_gs, unsigned unq_slots,
                            int unq_mode, int tile_stage);
+
+/* How often a lane of a strip kernel (path 6) polls for another workgroup's partial sum before it gives up and raises the
+ * error that the next cntkq_wait_quantize_done reports. Zero makes every exchange fail at once while every kernel still
+ * runs to its end: the way to test that error path. */
+int cntkq_debug_set_strip_spin_limit(cntkq_quantizer* h, unsigned limit);
 
 /* Ties caller-owned hipEvent_t objects (either may be NULL) to the NEXT kernel this handle launches: start_event is
  * set when that kernel begins, stop_event when it has finished, by the dispatch itself. Used to time single kernels

@@ -7,5 +7,6 @@
 #include "quantizer_kernels_column.h"
 #include "quantizer_kernels_register.h"
 #include "quantizer_kernels_tall.h"
+#include "quantizer_kernels_strip.h"
 #include "quantizer_kernels_unquantize.h"
 #include "quantizer_kernels_batch.h"

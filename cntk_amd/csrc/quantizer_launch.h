@@ -21,15 +21,28 @@ enum QuantizePath
     kPathTall = 2,    // one workgroup per column, global re-read (any rows)
     kPathCol = 3,     // one workgroup per column, column in LDS: rows a multiple of 4, matrices 16-byte aligned
     kPathReg = 4,     // one workgroup per column, column in registers: same conditions, 1 to 16 bits
-    kPathRegScalar = 5 // the same with one float per load and store: any height up to 98304 rows, any alignment, 1 to 16 bits
+    kPathRegScalar = 5, // the same with one float per load and store: any height up to 98304 rows, any alignment, 1 to 16 bits
+    kPathStrip = 6      // several workgroups per column, a strip of QWords with all its bit positions each: any height, any alignment, 1 to 16 bits
 };
 
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
 constexpr uint32_t kStripeWideItems = 768; // work items per column from which the stripe reduction uses 1024 threads
 constexpr uint32_t kColMinRows = 1024;   // shorter columns are better served several to a workgroup (tile kernels)
 
+// The scratch buffer of the strip kernels (partial sums of the columns' workgroups and the launch count), owned by a handle: one
+// launch stream at a time uses it. The error word lives in pinned host memory, where the host reads it without a copy.
+struct StripScratchOwner
+{
+    char* dev = nullptr;
+    size_t bytes = 0;        // header, finish counters, records
+    size_t groups_bytes = 0; // the part of it set aside for finish counters: 1/256 of the whole
+    uint32_t* error_host = nullptr;
+};
+
 struct LaunchTuning
 {
+    StripScratchOwner* strip = nullptr; // null: the strip kernels are not available to this launch
+    uint32_t strip_spin_limit = 1u << 20; // polls of a partial sum (a microsecond or so each) before a lane gives up
     int quantize_path = kPathAuto;
     uint32_t tile_gs = 0;   // 0 = pick from rows; else threads per column (power of two, 8..256)
     int tile_stage = -1;    // -1 = automatic; 0 / 1 = residual written straight to memory / staged through LDS
@@ -439,8 +452,121 @@ struct RegsLauncher
     }
 };
 
+// ---- strip kernels: any height, several workgroups per column ------------------------------------------------------
+
+
+// The workgroups of a column wait for each other and run on one die, so all of them must fit there at once: 64 of them is
+// half of what the 32 compute units of a die hold at four workgroups each (524288 rows at 1 to 4 bits, 262144 at 8,
+// 131072 at 16). Taller columns are left to the kernel that re-reads its column.
+constexpr uint32_t kStripMaxPerColumn = 64;
+
+inline bool strip_applicable(size_t rows, size_t nbits, const LaunchTuning& tune)
+{
+    return tune.strip != nullptr && nbits < 32 && rows >= 1 &&
+           (qwords_per_col(rows, nbits) + strip_words(nbits) - 1) / strip_words(nbits) <= kStripMaxPerColumn;
+}
+
+inline StripGeom make_strip_geom(size_t rows, size_t cols, size_t nbits, uint32_t spin_limit)
+{
+    StripGeom c;
+    c.rows = (uint32_t) rows;
+    c.cols = (uint32_t) cols;
+    c.nq = (uint32_t) qwords_per_col(rows, nbits);
+    c.strips = (c.nq + strip_words(nbits) - 1) / strip_words(nbits);
+    c.spin_limit = spin_limit;
+    c.inv_strips = 1.0 / (double) c.strips;
+    c.qcol = qcol_bytes(nbits, rows);
+    return c;
+}
+
+inline bool strip_scratch_fits(const StripScratchOwner& o, size_t cols, size_t strips)
+{
+    return o.dev != nullptr && strip_groups_bytes(cols, strips) <= o.groups_bytes &&
+           sizeof(StripHeader) + o.groups_bytes + strip_records_bytes(cols, strips) <= o.bytes;
+}
+
+// Makes the owner's buffer large enough for this launch (growing waits for the stream and clears the new buffer: the launch
+// count and every record's tag start at zero). Not possible while the stream is being captured.
+inline hipError_t strip_scratch_for(StripScratchOwner& o, hipStream_t s, size_t cols, size_t strips, StripScratch& out)
+{
+    if (o.error_host == nullptr)
+    {
+        void* p = nullptr;
+        hipError_t rc = hipHostMalloc(&p, 64, hipHostMallocDefault);
+        if (rc != hipSuccess)
+            return rc;
+        o.error_host = static_cast<uint32_t*>(p);
+        *o.error_host = 0u;
+    }
+    if (!strip_scratch_fits(o, cols, strips))
+    {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &st) == hipSuccess && st == hipStreamCaptureStatusActive)
+            return hipErrorStreamCaptureUnsupported;
+        hipError_t rc = hipStreamSynchronize(s);
+        if (rc != hipSuccess)
+            return rc;
+        if (o.dev != nullptr)
+            (void) hipFree(o.dev);
+        o.dev = nullptr;
+        o.bytes = 0;
+        const size_t need = sizeof(StripHeader) + strip_records_bytes(cols, strips);
+        const size_t cap = std::max<size_t>((need * 2 + 8191) & ~(size_t) 4095, (size_t) 1 << 20);
+        void* p = nullptr;
+        rc = hipMalloc(&p, cap);
+        if (rc != hipSuccess)
+            return rc;
+        rc = hipMemsetAsync(p, 0, cap, s);
+        if (rc != hipSuccess)
+        {
+            (void) hipFree(p);
+            return rc;
+        }
+        o.dev = static_cast<char*>(p);
+        o.bytes = cap;
+        o.groups_bytes = (cap / 256 + 63) & ~(size_t) 63; // counters need 1/512 of what the records need
+    }
+    out.error = o.error_host;
+    out.header = reinterpret_cast<StripHeader*>(o.dev);
+    out.groups = reinterpret_cast<uint32_t*>(o.dev + sizeof(StripHeader));
+    out.records = reinterpret_cast<uint64_t*>(o.dev + sizeof(StripHeader) + o.groups_bytes);
+    return hipSuccess;
+}
+
+// whether this launch finds its scratch buffer without allocating, or may allocate (the stream is not being captured)
+inline bool strip_scratch_ready(const StripScratchOwner& o, hipStream_t s, size_t cols, size_t strips)
+{
+    if (o.error_host != nullptr && strip_scratch_fits(o, cols, strips))
+        return true;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(s, &st) == hipSuccess && st == hipStreamCaptureStatusNone;
+}
+
+inline uint32_t strip_grid(size_t cols, size_t strips)
+{
+    return (uint32_t) ((cols + kStripDies - 1) / kStripDies * kStripDies * strips);
+}
+
+template <int NBITS, bool ZT>
+struct StripLauncher
+{
+    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, StripGeom c,
+                          StripScratch scratch)
+    {
+        if constexpr (NBITS >= 32)
+            return hipErrorInvalidValue;
+        else
+        {
+            hipExtLaunchKernelGGL((quantize_strip_kernel<NBITS, ZT>), dim3(strip_grid(cols, c.strips)), dim3(kStripThreads), strip_lds_bytes(NBITS), s,
+                                  ev.start, ev.stop, 0, g, r_in, r_out, q, c, scratch);
+            return hipGetLastError();
+        }
+    }
+};
+
 // which path launch_quantize takes for this matrix when nothing is forced
-inline int quantize_auto_path(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
+inline int quantize_auto_path(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits,
+                              bool strip_available = false)
 {
     // (2048 rows at 1 bit: the unrolled LDS kernel, where its conditions hold, is as fast)
     const bool unrolled = rows <= 2048 && col_applicable(g, r_in, r_out, q, rows, nbits) && col_unrolled(q, rows, nbits) &&
@@ -451,7 +577,14 @@ inline int quantize_auto_path(const float* g, const float* r_in, const float* r_
     if (rows > kRegEdge256MinRows && reg_edge_applicable(g, r_in, r_out, q, rows, nbits))
         return kPathReg;
     if (rows > kTileMaxRows)
-        return regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
+    {
+        // What no workgroup's registers hold in whole aligned pieces (the three matrices at different offsets within 16
+        // bytes): one element per access up to 98304 rows (as fast there as the strips, and faster below 50000 rows),
+        // then strips of the column on several workgroups, then -- above 64 strips -- the kernel that re-reads its column.
+        if (regs_applicable(rows, nbits))
+            return kPathRegScalar;
+        return strip_available ? kPathStrip : kPathTall;
+    }
     if (col_applicable(g, r_in, r_out, q, rows, nbits))
         return kPathCol;
     return kPathTile;
@@ -466,7 +599,14 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     int path = tune.quantize_path;
     if (path == kPathAuto)
     {
-        path = quantize_auto_path(g, r_in, r_out, q, rows, nbits);
+        path = quantize_auto_path(g, r_in, r_out, q, rows, nbits, strip_applicable(rows, nbits, tune));
+        if (path == kPathStrip)
+        {
+            // a stream under capture cannot wait for a larger scratch buffer: the kernels that need none take the matrix
+            const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit);
+            if ((uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull || !strip_scratch_ready(*tune.strip, s, cols, c.strips))
+                path = regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
+        }
     }
     if (path == kPathReg)
     {
@@ -485,6 +625,17 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
         const bool line_shift = quantize_line_shift(g, r_in, r_out, rows) && (threads == 256 || rows / 4 + 7 <= 1024 * (size_t) kRegMaxShiftPer);
         return dispatch_nbits<RegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols,
                                            make_reg_geom(rows, nbits, threads, line_shift), threads);
+    }
+    if (path == kPathStrip)
+    {
+        const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit);
+        if (!strip_applicable(rows, nbits, tune) || (uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull)
+            return hipErrorInvalidValue;
+        StripScratch scratch;
+        const hipError_t rc = strip_scratch_for(*tune.strip, s, cols, c.strips, scratch);
+        if (rc != hipSuccess)
+            return rc;
+        return dispatch_nbits<StripLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, scratch);
     }
     if (path == kPathRegScalar)
     {

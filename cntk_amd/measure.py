@@ -1,7 +1,7 @@
 """Kernel timing for one matrix shape: quantize, unquantize and (optionally) the fused stripe reduction.
 
     python -m cntk_amd.measure --rows 2048 --cols 9304 --nbits 1 [--dtype f64] [--workers 8] [--zero-threshold 1]
-                               [--steps 40] [--path 0|1|2|3]
+                               [--steps 40] [--path 0..6]
 
 Calls the C ABI directly. Every launch is timed with HIP events tied to the kernel dispatch (start when it begins,
 stop when it has finished) on the stream the handle launches on; buffer sets are rotated so that no launch finds its
@@ -33,7 +33,7 @@ def main():
     ap.add_argument("--steps", type=int, default=40)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--path", type=int, default=0, help="force a quantize kernel: 1 tile, 2 tall (re-reading), 3 column in LDS, 4 column in registers (16-byte accesses), "
-                    "5 column in registers (one element per access)")
+                    "5 column in registers (one element per access), 6 several workgroups per column (strips)")
     ap.add_argument("--unq-mode", type=int, default=0, help="decoder choice: 0 automatic, 1 QWord-major with one store per value, 2 tile decoder, 3 automatic without the tile "
                     "decoder, 4 row-major decoder")
     ap.add_argument("--budget-mb", type=int, default=1600, help="device memory for the rotating buffer sets")

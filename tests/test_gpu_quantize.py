@@ -21,7 +21,7 @@ from cntk_amd import Matrix, MatrixQuantizerImpl, QuantizedMatrix
 pytestmark = pytest.mark.gpu
 
 VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False)]
-PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG, PATH_REG_SCALAR = 0, 1, 2, 3, 4, 5
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG, PATH_REG_SCALAR, PATH_STRIP = 0, 1, 2, 3, 4, 5, 6
 
 
 def say(*a):
@@ -137,6 +137,11 @@ PATH_CASES = [
     # 14336 rows when the three matrices share their alignment)
     (9, 5, PATH_REG, 0), (37, 5, PATH_REG, 0), (1001, 3, PATH_REG, 0), (4099, 2, PATH_REG, 0), (14338, 3, PATH_REG, 0),
     (50257, 2, PATH_REG, 0), (102365, 1, PATH_REG, 0),
+    # several workgroups per column, a strip of QWords each: any height and alignment, one strip or many, full or ragged
+    (1, 3, PATH_STRIP, 0), (37, 5, PATH_STRIP, 0), (1000, 3, PATH_STRIP, 0), (8192, 3, PATH_STRIP, 0), (8193, 2, PATH_STRIP, 0),
+    (9304, 3, PATH_STRIP, 0), (16385, 2, PATH_STRIP, 0), (32768, 2, PATH_STRIP, 0), (50257, 3, PATH_STRIP, 0), (100000, 5, PATH_STRIP, 0),
+    (102401, 2, PATH_AUTO, 0), (200000, 3, PATH_AUTO, 0), (262147, 2, PATH_STRIP, 0), (524288, 9, PATH_STRIP, 0), (524289, 1, PATH_AUTO, 0),
+    (1000003, 1, PATH_AUTO, 0),
 ]
 
 
@@ -147,6 +152,12 @@ def test_kernel_paths(case):
     rep = parity.Report()
     for nbits, zt in VARIANTS:
         say("path case", case, "nbits", nbits, "zeroThr", zt)
+        if path == PATH_STRIP and (nbits == 32 or oracle.qwords_per_col(rows, nbits) > 64 * (256 if nbits == 1 else 512 if nbits == 2 else 1024)):
+            # whole-QWord codes need no assembling, and a column's strips must fit on one die of the device together
+            qz._set_tuning(quantize_path=path)
+            with pytest.raises(cntk_amd.QuantizerLogicError):
+                gpu_quantize(qz, datagen.normal(1, rows, cols), np.zeros((rows, cols), np.float32, order="F"), nbits, zt)
+            continue
         if path in (PATH_REG, PATH_REG_SCALAR) and (nbits == 32 or (48 + oracle.qwords_per_col(rows, nbits)) * 4 > 65536):
             # whole-QWord codes and columns whose QWords exceed 64 KB of LDS are not the register kernels' business
             qz._set_tuning(quantize_path=path)
@@ -516,3 +527,63 @@ def test_calls_replayed_from_a_hip_graph(rows, cols, nbits):
             assert torch.equal(getattr(graphed, name).data, getattr(eager, name).data), "replay %d: %s differs" % (step, name)
         assert torch.equal(graphed.Q.buffer, eager.Q.buffer), "replay %d: packed matrix differs" % step
         assert torch.equal(graphed.stripes[owner].buffer, eager.stripes[owner].buffer), "replay %d: reduced stripe differs" % step
+
+
+@pytest.mark.parametrize("rows,cols,nbits", [(150001, 3, 1), (120000, 2, 4)])
+def test_strip_kernel_replayed_from_a_hip_graph(rows, cols, nbits):
+    """Columns taller than any workgroup holds are cut into strips whose workgroups exchange partial sums through a
+    scratch buffer that carries a launch count from one launch to the next. A captured launch must find that state
+    right at every replay, with eager launches of the same and of another shape in between, and give the eager bytes."""
+    qz = MatrixQuantizerImpl.Create(0, False)
+    other_rows = 110000
+    graphed = (Matrix(rows, cols), Matrix(rows, cols), QuantizedMatrix(rows, cols, nbits, 0))
+    eager = (Matrix(rows, cols), Matrix(rows, cols), QuantizedMatrix(rows, cols, nbits, 0))
+    other = (Matrix(other_rows, 5), Matrix(other_rows, 5), QuantizedMatrix(other_rows, 5, nbits, 0))
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        qz.SetMainStream(torch.cuda.current_stream().cuda_stream)
+        qz.QuantizeAsync(graphed[0], graphed[1], graphed[2], graphed[1], False)
+    qz.SetMainStream(torch.cuda.current_stream().cuda_stream)
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(datagen.case_seed(81, nbits) + rows)
+    rep = parity.Report()
+    res = np.zeros((rows, cols), np.float32, order="F")
+    for step in range(4):
+        g = torch.randn(rows * cols, generator=gen, device="cuda:0") * 0.01
+        graphed[0].data.copy_(g)
+        eager[0].data.copy_(g)
+        qz.QuantizeAsync(eager[0], eager[1], eager[2], eager[1], False)
+        other[0].data.copy_(torch.randn(other_rows * 5, generator=gen, device="cuda:0"))
+        qz.QuantizeAsync(other[0], other[1], other[2], other[1], False)  # another geometry on the same scratch buffer
+        qz.WaitQuantizeAsyncDone()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        qz.WaitQuantizeAsyncDone()  # reports a strip kernel whose workgroups gave up on each other, replays included
+        assert torch.equal(graphed[1].data, eager[1].data), "replay %d: residual differs" % step
+        assert torch.equal(graphed[2].buffer, eager[2].buffer), "replay %d: packed matrix differs" % step
+        if step in (0, 3):
+            parity.check_quantize(np.asfortranarray(g.cpu().numpy().reshape((rows, cols), order="F")), res, graphed[2].to_numpy(),
+                                  graphed[1].to_numpy(), nbits, False, report=rep)
+        res = graphed[1].to_numpy().copy(order="F")
+    say("  ", rep)
+
+
+def test_strip_kernel_reports_workgroups_that_give_up():
+    """The workgroups of a column wait for each other's partial sums a bounded number of polls. With that number set to
+    zero from the host every wait gives up at once: the kernel still runs to its end, the next wait reports the call as
+    failed, and the handle goes on working afterwards."""
+    rows, cols = 130000, 4
+    qz = MatrixQuantizerImpl.Create(0, False)
+    g = datagen.normal(5, rows, cols)
+    G, R, Q = Matrix.from_numpy(g), Matrix(rows, cols), QuantizedMatrix(rows, cols, 1, 0)
+    qz._set_strip_spin_limit(0)
+    qz.QuantizeAsync(G, R, Q, R, False)
+    with pytest.raises(cntk_amd.QuantizerError):
+        qz.WaitQuantizeAsyncDone()
+    qz._set_strip_spin_limit(1 << 20)
+    R.data.zero_()
+    qz.QuantizeAsync(G, R, Q, R, False)
+    qz.WaitQuantizeAsyncDone()
+    parity.check_quantize(g, np.zeros_like(g, order="F"), Q.to_numpy(), R.to_numpy(), 1, False)
