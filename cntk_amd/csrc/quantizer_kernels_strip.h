@@ -30,9 +30,6 @@ namespace cntkq {
 constexpr uint32_t kStripThreads = 256;
 constexpr uint32_t kStripDies = 8; // accelerator dies that take the workgroups of a grid in turn
 
-typedef f32x4 f32x4_u __attribute__((aligned(4))); // a 16-byte access at any 4-byte alignment
-typedef u32x4 u32x4_u __attribute__((aligned(4)));
-
 template <int NBITS>
 struct StripShape
 {

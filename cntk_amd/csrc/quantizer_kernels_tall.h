@@ -38,7 +38,48 @@ __global__ __launch_bounds__(kTallThreads) void quantize_tall_kernel(const float
     const float* rp = r_in + base;
     float lo, hi;
 
-    if constexpr (NBITS == 1)
+    if constexpr (NBITS == 32)
+    {
+        // A 32-bit code is the value itself and its residual the value minus itself, whatever the range in the header: one
+        // pass computes the header's sum of squares while it writes both (four elements per access at any 4-byte alignment;
+        // a thread reads an element before it writes it and nobody else does either, so r_out may be r_in).
+        char* qc = q + (size_t) blockIdx.x * qcol;
+        uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
+        float* op = r_out + base;
+        const uint32_t quads = rows / 4;
+        float s = 0.0f;
+#pragma unroll 4
+        for (uint32_t x = tid; x < quads; x += kTallThreads)
+        {
+            const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(gp) + x) +
+                            __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(rp) + x);
+            s += v[0] * v[0];
+            s += v[1] * v[1];
+            s += v[2] * v[2];
+            s += v[3] * v[3];
+            const u32x4 code = {__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])};
+            __builtin_nontemporal_store(code, reinterpret_cast<u32x4_u*>(bits) + x);
+            __builtin_nontemporal_store(v - v, reinterpret_cast<f32x4_u*>(op) + x);
+        }
+        const uint32_t i = 4 * quads + tid;
+        if (i < rows)
+        {
+            const float v = gp[i] + rp[i];
+            s += v * v;
+            bits[i] = __float_as_uint(v);
+            op[i] = v - v;
+        }
+        s = tall_block_sum(s, scratch_f);
+        finish_stats_multibit(s, rows, lo, hi);
+        if (tid == 0)
+        {
+            float* gh = reinterpret_cast<float*>(qc);
+            gh[0] = lo;
+            gh[1] = hi;
+        }
+        return;
+    }
+    else if constexpr (NBITS == 1)
     {
         float mean = 0.0f;
         if constexpr (!ZT)
