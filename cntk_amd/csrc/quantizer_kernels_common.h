@@ -17,6 +17,8 @@
 
 #include "quantizer_math.h"
 
+#include <type_traits>
+
 namespace cntkq {
 
 constexpr uint32_t kTileThreads = 256;
@@ -30,16 +32,19 @@ constexpr uint32_t kTileMaxCols = 32;
 constexpr uint32_t kTilePrefixFloats = kTileScratchFloats + 2 * kTileMaxCols; // 76 floats = 304 B (16-B multiple)
 
 // A QWord is assembled from work items of at most 8 bit positions each, so that a tile with few QWords
-// still keeps every thread busy; the partial words meet in LDS (atomic OR).
-template <int NBITS>
-struct PackShape
+// still keeps every thread busy; the partial words meet in LDS (atomic OR). WORD_BITS: 32 for float columns, 64 for double.
+template <int NBITS, int WORD_BITS>
+struct PackShapeOf
 {
-    static constexpr uint32_t VPW = 32 / NBITS;              // values per QWord
+    typedef typename std::conditional<WORD_BITS == 64, uint64_t, uint32_t>::type Q;
+    static constexpr uint32_t VPW = WORD_BITS / NBITS;       // values per QWord
     static constexpr uint32_t SLOTS = VPW < 8 ? VPW : 8;     // bit positions per work item
-    static constexpr uint32_t CHUNKS = VPW / SLOTS;          // work items per QWord (4, 2, 1, 1, 1, 1)
-    static constexpr uint32_t SHIFT = NBITS & 31;
-    static constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
+    static constexpr uint32_t CHUNKS = VPW / SLOTS;          // work items per QWord (fp32: 4, 2, 1, 1, 1, 1; fp64: 8, 4, 2, 1, 1, 1, 1)
+    static constexpr uint32_t SHIFT = NBITS & (WORD_BITS - 1);
+    static constexpr Q CODEMASK = (NBITS >= WORD_BITS) ? ~(Q) 0 : (((Q) 1 << SHIFT) - (Q) 1);
 };
+template <int NBITS>
+using PackShape = PackShapeOf<NBITS, 32>;
 
 struct TileGeom
 {

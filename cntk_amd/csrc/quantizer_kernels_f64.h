@@ -17,133 +17,16 @@
 namespace cntkq {
 namespace f64 {
 
-typedef double f64x2 __attribute__((ext_vector_type(2)));
-
 constexpr uint32_t kThreads = 256;
 constexpr uint32_t kMaxTileCols = 32;
 // LDS prefix in 8-byte units: 8 double + 2 (four uint32) for the reductions of up to 4 wavefronts, then (lower, upper) per column
 constexpr uint32_t kPrefixWords = 10 + 2 * kMaxTileCols;
 
-// ---- per-value quantizer (Source/Math/ValueQuantizer.h:68-156 with ElemType = double) ----------------
-
-struct ValueQ
-{
-    double lo, hi, mid, qf, uf;
-};
-
+// The per-value quantizer, the header statistics and the pack shape are the element-type templates of quantizer_math.h
+// and quantizer_kernels_common.h, here on doubles and 64-bit QWords.
+typedef ValueQOf<double> ValueQ;
 template <int NBITS>
-__device__ __forceinline__ ValueQ make_vq(double lo, double hi)
-{
-    constexpr uint64_t rangeend = (NBITS >= 64) ? 0ull : (1ull << (NBITS & 63));
-    ValueQ v;
-    v.lo = lo;
-    v.hi = hi;
-    const double span = hi - lo;
-    // the reference compares with the float literal 1e-36f, converted to double
-    if ((span < (double) 1e-36f) || (rangeend == 0))
-    {
-        v.qf = 0.0;
-        v.uf = 0.0;
-    }
-    else
-    {
-        constexpr double used = (double) (rangeend - (NBITS > 1 ? 1ull : 0ull)); // exact: at most 2^32 - 1
-        v.qf = used / span;
-        v.uf = span / used;
-    }
-    v.mid = 0.5 * (hi + lo);
-    return v;
-}
-
-template <int NBITS, bool ZT>
-__device__ __forceinline__ uint64_t quantize_value(const ValueQ& v, double u)
-{
-    if constexpr (NBITS == 64)
-    {
-        return (uint64_t) __double_as_longlong(u);
-    }
-    else if constexpr (NBITS == 1)
-    {
-        return ZT ? (u >= 0.0 ? 1ull : 0ull) : (u >= v.mid ? 1ull : 0ull);
-    }
-    else
-    {
-        constexpr uint64_t top = (1ull << (NBITS & 63)) - 1ull;
-        if (u <= v.lo)
-            return 0ull;
-        if (u >= v.hi)
-            return top;
-        return (uint64_t) (int64_t) ((u - v.lo) * v.qf);
-    }
-}
-
-// (q + 0.5) * uf + lo, multiply and add rounded separately
-template <int NBITS>
-__device__ __forceinline__ double unquantize_value(double uf, double lo, uint64_t q)
-{
-    if constexpr (NBITS == 64)
-    {
-        return __longlong_as_double((long long) q);
-    }
-    else
-    {
-        // codes are below 2^32 here, so the conversion is exact whichever way it is done
-        double t = (double) (uint32_t) q + 0.5;
-        t = t * uf;
-        return t + lo;
-    }
-}
-
-// ---- column header from reduced sums (Source/Math/ColumnQuantizer.h:265-340) --------------------------
-
-template <bool ZT>
-__device__ __forceinline__ void finish_stats_1bit(double mean, double s0, double s1, uint32_t n0, uint32_t n1,
-                                                  uint32_t rows, double& lo, double& hi)
-{
-    double radius, centre;
-    if constexpr (!ZT)
-    {
-        const double dev0 = ((double) n0 * mean) - s0;
-        const double dev1 = s1 - ((double) n1 * mean);
-        const double dev = (dev0 + dev1) / (double) rows;
-        radius = 2.0 * dev;
-        centre = mean;
-    }
-    else
-    {
-        if (n0 == 0)
-            n0 = 1;
-        if (n1 == 0)
-            n1 = 1;
-        const double m0 = s0 / (double) n0;
-        const double m1 = s1 / (double) n1;
-        centre = 0.5 * (m0 + m1);
-        radius = 2.0 * (m1 - centre);
-    }
-    lo = centre - radius;
-    hi = centre + radius;
-}
-
-__device__ __forceinline__ void finish_stats_multibit(double sumsq, uint32_t rows, double& lo, double& hi)
-{
-    const double mean = 0.0;
-    const double sd = sqrt(sumsq / (double) rows);
-    const double half = 4.0 * sd;
-    lo = mean - half;
-    hi = mean + half;
-}
-
-// ---- geometry -------------------------------------------------------------------------------------------
-
-template <int NBITS>
-struct PackShape
-{
-    static constexpr uint32_t VPW = 64 / NBITS;          // values per QWord
-    static constexpr uint32_t SLOTS = VPW < 8 ? VPW : 8; // bit positions per work item
-    static constexpr uint32_t CHUNKS = VPW / SLOTS;      // work items per QWord (8, 4, 2, 1, 1, 1, 1)
-    static constexpr uint32_t SHIFT = NBITS & 63;
-    static constexpr uint64_t CODEMASK = (NBITS >= 64) ? ~0ull : ((1ull << SHIFT) - 1ull);
-};
+using PackShape = PackShapeOf<NBITS, 64>;
 
 struct TileGeom
 {
@@ -166,75 +49,7 @@ __host__ __device__ inline size_t tile_lds_bytes(const TileGeom& t, uint32_t wor
 
 // ---- statistics + packing of a tile in LDS (same contract as the fp32 tile_stats / tile_pack) ----------
 
-template <int NBITS, bool ZT>
-__device__ __forceinline__ void tile_stats(const double* tile, double* hdr, double* scratch_f, uint32_t* scratch_u,
-                                           const TileGeom& t, uint32_t nc, char* qtile)
-{
-    const uint32_t tid = threadIdx.x;
-    const uint32_t c = tid >> t.gs_log2;
-    const uint32_t lg = tid & (t.gs - 1);
-    const bool col_ok = c < nc;
-    const double* colv = tile + (size_t) c * t.rows;
-    double lo = 0.0, hi = 0.0;
-
-    if constexpr (NBITS == 1)
-    {
-        double mean = 0.0;
-        if constexpr (!ZT)
-        {
-            double s = 0.0;
-            if (col_ok)
-                for (uint32_t i = lg; i < t.rows; i += t.gs)
-                    s += colv[i];
-            s = group_sum(s, t.gs, scratch_f);
-            mean = s / (double) t.rows;
-        }
-        double s0 = 0.0, s1 = 0.0;
-        uint32_t n0 = 0;
-        if (col_ok)
-        {
-            for (uint32_t i = lg; i < t.rows; i += t.gs)
-            {
-                const double v = colv[i];
-                if (v < mean)
-                {
-                    s0 += v;
-                    n0++;
-                }
-                else
-                {
-                    s1 += v;
-                }
-            }
-        }
-        group_sum3(s0, s1, n0, t.gs, scratch_f, scratch_u);
-        finish_stats_1bit<ZT>(mean, s0, s1, n0, t.rows - n0, t.rows, lo, hi);
-    }
-    else
-    {
-        double s = 0.0;
-        if (col_ok)
-        {
-            for (uint32_t i = lg; i < t.rows; i += t.gs)
-            {
-                const double v = colv[i];
-                s += v * v;
-            }
-        }
-        s = group_sum(s, t.gs, scratch_f);
-        finish_stats_multibit(s, t.rows, lo, hi);
-    }
-
-    if (col_ok && lg == 0)
-    {
-        hdr[2 * c] = lo;
-        hdr[2 * c + 1] = hi;
-        double* gh = reinterpret_cast<double*>(qtile + (size_t) c * t.qcol);
-        gh[0] = lo;
-        gh[1] = hi;
-    }
-    __syncthreads();
-}
+// (tile_stats is the fp32 tile kernels' function, written over the element type)
 
 // Columns of fewer QWords than this hand their new residual back through the LDS tile.
 constexpr uint32_t kStagedResidualBelowQWords = 16;
@@ -539,101 +354,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(colreg
         bits[x] = words[x];
 }
 
-// one workgroup of 1024 threads per column, statistics and packing re-read global memory
-template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kTallThreads) void quantize_tall_kernel(const double* __restrict__ g, const double* r_in, double* r_out,
-                                                                     char* __restrict__ q, uint32_t rows, uint32_t nq, uint64_t qcol)
-{
-    using PS = PackShape<NBITS>;
-    __shared__ double scratch_f[kTallThreads / 64];
-    __shared__ uint32_t scratch_u[kTallThreads / 64];
-
-    const uint32_t tid = threadIdx.x;
-    const size_t base = (size_t) blockIdx.x * rows;
-    const double* gp = g + base;
-    const double* rp = r_in + base;
-    double lo, hi;
-
-    if constexpr (NBITS == 1)
-    {
-        double mean = 0.0;
-        if constexpr (!ZT)
-        {
-            double s = 0.0;
-            for (uint32_t i = tid; i < rows; i += kTallThreads)
-                s += gp[i] + rp[i];
-            s = tall_block_sum(s, scratch_f);
-            mean = s / (double) rows;
-        }
-        double s0 = 0.0, s1 = 0.0;
-        uint32_t n0 = 0, n1 = 0;
-        for (uint32_t i = tid; i < rows; i += kTallThreads)
-        {
-            const double v = gp[i] + rp[i];
-            if (v < mean)
-            {
-                s0 += v;
-                n0++;
-            }
-            else
-            {
-                s1 += v;
-                n1++;
-            }
-        }
-        s0 = tall_block_sum(s0, scratch_f);
-        s1 = tall_block_sum(s1, scratch_f);
-        n0 = tall_block_sum(n0, scratch_u);
-        n1 = tall_block_sum(n1, scratch_u);
-        finish_stats_1bit<ZT>(mean, s0, s1, n0, n1, rows, lo, hi);
-    }
-    else
-    {
-        double s = 0.0;
-        for (uint32_t i = tid; i < rows; i += kTallThreads)
-        {
-            const double v = gp[i] + rp[i];
-            s += v * v;
-        }
-        s = tall_block_sum(s, scratch_f);
-        finish_stats_multibit(s, rows, lo, hi);
-    }
-    // every thread has passed the last barrier of tall_block_sum: all statistics reads of r_in are done
-    // before any residual is written (r_out may be r_in)
-
-    char* qc = q + (size_t) blockIdx.x * qcol;
-    if (tid == 0)
-    {
-        double* gh = reinterpret_cast<double*>(qc);
-        gh[0] = lo;
-        gh[1] = hi;
-    }
-    const ValueQ vq = make_vq<NBITS>(lo, hi);
-    const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
-    const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
-    double* op = r_out + base;
-    uint64_t* bits = reinterpret_cast<uint64_t*>(qc + 16);
-    for (uint32_t w = tid; w < nq; w += kTallThreads)
-    {
-        uint64_t word = 0;
-        for (uint32_t k = 0; k < PS::VPW; ++k)
-        {
-            const uint32_t i = w + k * nq;
-            if (i >= rows)
-                break;
-            const double v = gp[i] + rp[i];
-            const uint64_t code = quantize_value<NBITS, ZT>(vq, v);
-            double back;
-            if constexpr (NBITS == 1)
-                back = code ? val1 : val0;
-            else
-                back = unquantize_value<NBITS>(vq.uf, vq.lo, code);
-            op[i] = v - back;
-            word |= code << (k * PS::SHIFT);
-        }
-        bits[w] = word;
-    }
-}
+// (columns too tall for these take quantize_tall_kernel of quantizer_kernels_tall.h, written over the element type)
 
 // ---- stripe reduction: K packed stripes -> fp64 sum (owner first, then ascending) -> requantize ------------
 

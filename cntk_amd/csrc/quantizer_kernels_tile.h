@@ -12,36 +12,35 @@ namespace cntkq {
 // in global memory and in hdr[], codes are in global memory and the new residual v - unquantize(code) has
 // been written to res_out (dense, column-major, tile-relative).
 
-template <int NBITS, bool ZT>
-__device__ __forceinline__ void tile_stats(const float* tile, float* hdr, float* scratch_f, uint32_t* scratch_u,
-                                           const TileGeom& t, uint32_t nc, char* qtile)
+template <int NBITS, bool ZT, typename E, typename Geom>
+__device__ __forceinline__ void tile_stats(const E* tile, E* hdr, E* scratch_f, uint32_t* scratch_u, const Geom& t, uint32_t nc, char* qtile)
 {
     const uint32_t tid = threadIdx.x;
     const uint32_t c = tid >> t.gs_log2;
     const uint32_t lg = tid & (t.gs - 1);
     const bool col_ok = c < nc;
-    const float* colv = tile + (size_t) c * t.rows;
-    float lo = 0.0f, hi = 0.0f;
+    const E* colv = tile + (size_t) c * t.rows;
+    E lo = (E) 0, hi = (E) 0;
 
     if constexpr (NBITS == 1)
     {
-        float mean = 0.0f;
+        E mean = (E) 0;
         if constexpr (!ZT)
         {
-            float s = 0.0f;
+            E s = (E) 0;
             if (col_ok)
                 for (uint32_t i = lg; i < t.rows; i += t.gs)
                     s += colv[i];
             s = group_sum(s, t.gs, scratch_f);
-            mean = s / (float) t.rows;
+            mean = s / (E) t.rows;
         }
-        float s0 = 0.0f, s1 = 0.0f;
+        E s0 = (E) 0, s1 = (E) 0;
         uint32_t n0 = 0;
         if (col_ok)
         {
             for (uint32_t i = lg; i < t.rows; i += t.gs)
             {
-                const float v = colv[i];
+                const E v = colv[i];
                 if (v < mean)
                 {
                     s0 += v;
@@ -58,12 +57,12 @@ __device__ __forceinline__ void tile_stats(const float* tile, float* hdr, float*
     }
     else
     {
-        float s = 0.0f;
+        E s = (E) 0;
         if (col_ok)
         {
             for (uint32_t i = lg; i < t.rows; i += t.gs)
             {
-                const float v = colv[i];
+                const E v = colv[i];
                 s += v * v;
             }
         }
@@ -75,8 +74,8 @@ __device__ __forceinline__ void tile_stats(const float* tile, float* hdr, float*
     {
         hdr[2 * c] = lo;
         hdr[2 * c + 1] = hi;
-        // a record is only 4-byte aligned when the column has an odd number of QWords
-        float* gh = reinterpret_cast<float*>(qtile + (size_t) c * t.qcol);
+        // (a float record is only 4-byte aligned when the column has an odd number of QWords)
+        E* gh = reinterpret_cast<E*>(qtile + (size_t) c * t.qcol);
         gh[0] = lo;
         gh[1] = hi;
     }

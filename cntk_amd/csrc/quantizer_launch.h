@@ -141,7 +141,7 @@ struct TallLauncher
     static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t rows,
                           uint32_t cols, uint32_t nq, uint64_t qcol)
     {
-        hipExtLaunchKernelGGL((quantize_tall_kernel<NBITS, ZT>), dim3(cols), dim3(kTallThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, q, rows,
+        hipExtLaunchKernelGGL((quantize_tall_kernel<NBITS, ZT, float>), dim3(cols), dim3(kTallThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, q, rows,
                            nq, qcol);
         return hipGetLastError();
     }

@@ -90,7 +90,7 @@ struct TallLauncher
     static hipError_t run(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, char* q, uint32_t rows,
                           uint32_t cols, uint32_t nq, uint64_t qcol)
     {
-        hipExtLaunchKernelGGL((quantize_tall_kernel<NBITS, ZT>), dim3(cols), dim3(kTallThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out,
+        hipExtLaunchKernelGGL((quantize_tall_kernel<NBITS, ZT, double>), dim3(cols), dim3(kTallThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out,
                               q, rows, nq, qcol);
         return hipGetLastError();
     }

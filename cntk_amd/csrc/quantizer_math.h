@@ -1,6 +1,6 @@
 // Device-side arithmetic of the per-column quantizer for gfx950.
 //
-// Every floating-point operation here is a separately rounded IEEE fp32 operation; the file must be
+// Every floating-point operation here is a separately rounded IEEE operation in the element type; the file must be
 // compiled with -ffp-contract=off (no fused multiply-add) and without fast-math so that, given the
 // same column header, codes and residuals are bit-identical to the reference CPU quantizer
 // (Source/Math/ValueQuantizer.h, Source/Math/ColumnQuantizer.h).
@@ -20,48 +20,88 @@ typedef u32x4 u32x4_u __attribute__((aligned(4)));
 
 constexpr int kWave = 64;
 
-// ---- per-value quantizer (Source/Math/ValueQuantizer.h:68-97) ------------------------------------
+// ---- element types and their QWords (Source/Math/ValueQuantizer.h:48-57) -------------------------
 
-struct ValueQ
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+
+// What differs between MatrixQuantizerImpl<float> and <double>: the QWord a column is packed into (as wide as the element),
+// its signed twin for the float -> code conversion, the raw bits of a value (the "code" when NBITS is the QWord's width) and
+// the square root of the header statistics. Everything below is written once over this.
+template <typename E>
+struct Word;
+template <>
+struct Word<float>
 {
-    float lo, hi; // reconstruction range as stored in the column header
-    float mid;    // 1-bit decision threshold derived from the STORED header, not from the column mean
-    float qf, uf; // value -> code and code -> value scale factors
+    typedef uint32_t Q;
+    typedef int32_t S;
+    static constexpr int kBits = 32;
+    static __device__ __forceinline__ Q bits_of(float x) { return __float_as_uint(x); }
+    static __device__ __forceinline__ float value_of(Q q) { return __uint_as_float(q); }
+    static __device__ __forceinline__ float root(float x) { return sqrtf(x); }
+};
+template <>
+struct Word<double>
+{
+    typedef uint64_t Q;
+    typedef int64_t S;
+    static constexpr int kBits = 64;
+    static __device__ __forceinline__ Q bits_of(double x) { return (Q) __double_as_longlong(x); }
+    static __device__ __forceinline__ double value_of(Q q) { return __longlong_as_double((long long) q); }
+    static __device__ __forceinline__ double root(double x) { return sqrt(x); }
 };
 
-template <int NBITS>
-__device__ __forceinline__ ValueQ make_vq(float lo, float hi)
+// ---- per-value quantizer (Source/Math/ValueQuantizer.h:68-97) ------------------------------------
+
+template <typename E>
+struct ValueQOf
 {
-    constexpr uint32_t rangeend = (NBITS >= 32) ? 0u : (1u << (NBITS & 31));
-    ValueQ v;
+    E lo, hi; // reconstruction range as stored in the column header
+    E mid;    // 1-bit decision threshold derived from the STORED header, not from the column mean
+    E qf, uf; // value -> code and code -> value scale factors
+};
+typedef ValueQOf<float> ValueQ;
+
+// the number of codes that span the range: one fewer than 2^NBITS when NBITS > 1, which leaves a code for 0; 0 when a code
+// is the value itself (exact in either element type: at most 2^32 - 1 where it is used)
+template <int NBITS, typename E>
+__device__ __forceinline__ constexpr uint64_t codes_in_range()
+{
+    return NBITS >= Word<E>::kBits ? 0ull : (1ull << (NBITS & 63)) - (NBITS > 1 ? 1ull : 0ull);
+}
+
+template <int NBITS, typename E>
+__device__ __forceinline__ ValueQOf<E> make_vq(E lo, E hi)
+{
+    constexpr uint64_t codes = codes_in_range<NBITS, E>();
+    ValueQOf<E> v;
     v.lo = lo;
     v.hi = hi;
-    const float span = hi - lo;
-    if ((span < 1e-36f) || (rangeend == 0))
+    const E span = hi - lo;
+    // the reference compares with the float literal 1e-36f in either precision
+    if ((span < (E) 1e-36f) || (codes == 0))
     {
-        v.qf = 0.0f;
-        v.uf = 0.0f;
+        v.qf = (E) 0;
+        v.uf = (E) 0;
     }
     else
     {
-        // one code fewer than 2^NBITS spans the range when NBITS > 1, which leaves a code for 0
-        constexpr float used = (float) (rangeend - (NBITS > 1 ? 1u : 0u));
+        constexpr E used = (E) codes;
         v.qf = used / span;
         v.uf = span / used;
     }
-    v.mid = 0.5f * (hi + lo);
+    v.mid = (E) 0.5 * (hi + lo);
     return v;
 }
 
 // Only what decoding needs: the code -> value step of the same quantizer state (identical arithmetic to make_vq).
-template <int NBITS>
-__device__ __forceinline__ float make_ufactor(float lo, float hi)
+template <int NBITS, typename E>
+__device__ __forceinline__ E make_ufactor(E lo, E hi)
 {
-    constexpr uint32_t rangeend = (NBITS >= 32) ? 0u : (1u << (NBITS & 31));
-    const float span = hi - lo;
-    if ((span < 1e-36f) || (rangeend == 0))
-        return 0.0f;
-    constexpr float used = (float) (rangeend - (NBITS > 1 ? 1u : 0u));
+    constexpr uint64_t codes = codes_in_range<NBITS, E>();
+    const E span = hi - lo;
+    if ((span < (E) 1e-36f) || (codes == 0))
+        return (E) 0;
+    constexpr E used = (E) codes;
     return span / used;
 }
 
@@ -86,39 +126,41 @@ __device__ __forceinline__ void divmod_u32(uint32_t x, uint32_t d, double inv_d,
 }
 
 // Source/Math/ValueQuantizer.h:101-128, 144-156
-template <int NBITS, bool ZT>
-__device__ __forceinline__ uint32_t quantize_value(const ValueQ& v, float u)
+template <int NBITS, bool ZT, typename E>
+__device__ __forceinline__ typename Word<E>::Q quantize_value(const ValueQOf<E>& v, E u)
 {
-    if constexpr (NBITS == 32)
+    typedef typename Word<E>::Q Q;
+    if constexpr (NBITS == Word<E>::kBits)
     {
-        return __float_as_uint(u);
+        return Word<E>::bits_of(u);
     }
     else if constexpr (NBITS == 1)
     {
-        return ZT ? (u >= 0.0f ? 1u : 0u) : (u >= v.mid ? 1u : 0u);
+        return ZT ? (u >= (E) 0 ? (Q) 1 : (Q) 0) : (u >= v.mid ? (Q) 1 : (Q) 0);
     }
     else
     {
-        constexpr uint32_t top = (1u << (NBITS & 31)) - 1u;
+        constexpr Q top = ((Q) 1 << (NBITS & 63)) - (Q) 1;
         if (u <= v.lo)
-            return 0u;
+            return (Q) 0;
         if (u >= v.hi)
             return top;
-        return (uint32_t) (int32_t) ((u - v.lo) * v.qf);
+        return (Q) (typename Word<E>::S)((u - v.lo) * v.qf);
     }
 }
 
 // Source/Math/ValueQuantizer.h:131-141.  (q + 0.5) * uf + lo, multiply and add rounded separately.
-template <int NBITS>
-__device__ __forceinline__ float unquantize_value(float uf, float lo, uint32_t q)
+template <int NBITS, typename E>
+__device__ __forceinline__ E unquantize_value(E uf, E lo, typename Word<E>::Q q)
 {
-    if constexpr (NBITS == 32)
+    if constexpr (NBITS == Word<E>::kBits)
     {
-        return __uint_as_float(q);
+        return Word<E>::value_of(q);
     }
     else
     {
-        float t = (float) q + 0.5f;
+        // codes are below 2^32 here, so the conversion is exact whichever way it is done
+        E t = (E) (uint32_t) q + (E) 0.5;
         t = t * uf;
         return t + lo;
     }
@@ -136,8 +178,8 @@ __device__ __forceinline__ float pick_level(uint32_t bits, uint32_t pos, float v
     return x;
 }
 
-template <int NBITS>
-__device__ __forceinline__ float unquantize_value(const ValueQ& v, uint32_t q)
+template <int NBITS, typename E>
+__device__ __forceinline__ E unquantize_value(const ValueQOf<E>& v, typename Word<E>::Q q)
 {
     return unquantize_value<NBITS>(v.uf, v.lo, q);
 }
@@ -145,17 +187,16 @@ __device__ __forceinline__ float unquantize_value(const ValueQ& v, uint32_t q)
 // ---- column header from reduced sums (Source/Math/ColumnQuantizer.h:265-340) ---------------------
 
 // 1 bit: the two reconstruction levels are  centre -/+ radius/2;  the header stores centre -/+ radius.
-template <bool ZT>
-__device__ __forceinline__ void finish_stats_1bit(float mean, float s0, float s1, uint32_t n0, uint32_t n1,
-                                                  uint32_t rows, float& lo, float& hi)
+template <bool ZT, typename E>
+__device__ __forceinline__ void finish_stats_1bit(E mean, E s0, E s1, uint32_t n0, uint32_t n1, uint32_t rows, E& lo, E& hi)
 {
-    float radius, centre;
+    E radius, centre;
     if constexpr (!ZT)
     {
-        const float dev0 = ((float) n0 * mean) - s0;
-        const float dev1 = s1 - ((float) n1 * mean);
-        const float dev = (dev0 + dev1) / (float) rows;
-        radius = 2.0f * dev;
+        const E dev0 = ((E) n0 * mean) - s0;
+        const E dev1 = s1 - ((E) n1 * mean);
+        const E dev = (dev0 + dev1) / (E) rows;
+        radius = (E) 2 * dev;
         centre = mean;
     }
     else
@@ -164,21 +205,22 @@ __device__ __forceinline__ void finish_stats_1bit(float mean, float s0, float s1
             n0 = 1;
         if (n1 == 0)
             n1 = 1;
-        const float m0 = s0 / (float) n0;
-        const float m1 = s1 / (float) n1;
-        centre = 0.5f * (m0 + m1);
-        radius = 2.0f * (m1 - centre);
+        const E m0 = s0 / (E) n0;
+        const E m1 = s1 / (E) n1;
+        centre = (E) 0.5 * (m0 + m1);
+        radius = (E) 2 * (m1 - centre);
     }
     lo = centre - radius;
     hi = centre + radius;
 }
 
 // more than 1 bit: +/- 4 standard deviations around a mean that is taken to be 0
-__device__ __forceinline__ void finish_stats_multibit(float sumsq, uint32_t rows, float& lo, float& hi)
+template <typename E>
+__device__ __forceinline__ void finish_stats_multibit(E sumsq, uint32_t rows, E& lo, E& hi)
 {
-    const float mean = 0.0f;
-    const float sd = sqrtf(sumsq / (float) rows);
-    const float half = 4.0f * sd;
+    const E mean = (E) 0;
+    const E sd = Word<E>::root(sumsq / (E) rows);
+    const E half = (E) 4 * sd;
     lo = mean - half;
     hi = mean + half;
 }
