@@ -39,11 +39,11 @@ class QuantizerLogicError(ValueError):
 
 
 class _QuantizeItem(ctypes.Structure):
-    _fields_ = [("in_", _vp), ("res_in", _vp), ("res_out", _vp), ("qbuf", _vp), ("rows", _sz), ("cols", _sz)]
+    _fields_ = [("in_", _vp), ("res_in", _vp), ("res_out", _vp), ("qbuf", _vp), ("rows", _sz), ("cols", _sz), ("qbuf_bytes", _sz)]
 
 
 class _UnquantizeItem(ctypes.Structure):
-    _fields_ = [("qbuf", _vp), ("out", _vp), ("rows", _sz), ("cols", _sz)]
+    _fields_ = [("qbuf", _vp), ("out", _vp), ("rows", _sz), ("cols", _sz), ("qbuf_bytes", _sz)]
 
 
 class _StripeReduceItem(ctypes.Structure):
@@ -438,7 +438,7 @@ class MatrixQuantizerImpl:
                 raise QuantizerLogicError("QuantizeBatchAsync: packed matrices must share one bit width and live on the device")
             if any(m.dtype != items[0][0].dtype for m in (g, r_in, r_out, q)):
                 raise QuantizerLogicError("QuantizeBatchAsync: all matrices of a call must have one element type")
-            arr[k] = _QuantizeItem(g.Data(), r_in.Data(), r_out.Data(), q.Buffer(), rows, cols)
+            arr[k] = _QuantizeItem(g.Data(), r_in.Data(), r_out.Data(), q.Buffer(), rows, cols, q.GetSize())
         return PreparedBatch("quantize", arr, len(items), nbits, (), dtype=items[0][0].dtype)
 
     def UnquantizeBatchAsync(self, items, add=False):
@@ -466,7 +466,7 @@ class MatrixQuantizerImpl:
                 raise QuantizerLogicError("UnquantizeBatchAsync: packed matrices must share one bit width and live on the device")
             if q.dtype != items[0][1].dtype or out.dtype != items[0][1].dtype:
                 raise QuantizerLogicError("UnquantizeBatchAsync: all matrices of a call must have one element type")
-            arr[k] = _UnquantizeItem(q.Buffer(), out.Data(), out.GetNumRows(), out.GetNumCols())
+            arr[k] = _UnquantizeItem(q.Buffer(), out.Data(), out.GetNumRows(), out.GetNumCols(), q.GetSize())
         return PreparedBatch("unquantize", arr, len(items), nbits, (), dtype=items[0][1].dtype)
 
     def StripeReduceAsync(self, stripes, owner, stripe_residual, out_qstripe, zero_threshold_for_1bit, agg_out=None):

@@ -472,7 +472,7 @@ public:
                 throw std::invalid_argument("QuantizeBatchAsync: matrix dimensions do not match");
             if (it.outQMatrix->GetNumBits() != nbits || it.outQMatrix->GetDeviceId() < 0)
                 throw std::invalid_argument("QuantizeBatchAsync: packed matrices must share one bit width and live on the device");
-            raw.push_back(typename detail::Abi<ElemType>::QuantizeItem{it.inMatrix->Data(), it.inResidual->Data(), it.outResidual->Data(), it.outQMatrix->Buffer(), rows, cols});
+            raw.push_back(typename detail::Abi<ElemType>::QuantizeItem{it.inMatrix->Data(), it.inResidual->Data(), it.outResidual->Data(), it.outQMatrix->Buffer(), rows, cols, it.outQMatrix->GetSize()});
         }
         detail::Check(detail::Abi<ElemType>::QuantizeBatch(m_handle, raw.data(), raw.size(), nbits, zeroThresholdFor1Bit ? 1 : 0));
     }
@@ -493,7 +493,7 @@ public:
                 throw std::invalid_argument("UnquantizeBatchAsync: matrix dimensions do not match");
             if (it.inQMatrix->GetNumBits() != nbits || it.inQMatrix->GetDeviceId() < 0)
                 throw std::invalid_argument("UnquantizeBatchAsync: packed matrices must share one bit width and live on the device");
-            raw.push_back(typename detail::Abi<ElemType>::UnquantizeItem{it.inQMatrix->Buffer(), it.outMatrix->Data(), it.outMatrix->GetNumRows(), it.outMatrix->GetNumCols()});
+            raw.push_back(typename detail::Abi<ElemType>::UnquantizeItem{it.inQMatrix->Buffer(), it.outMatrix->Data(), it.outMatrix->GetNumRows(), it.outMatrix->GetNumCols(), it.inQMatrix->GetSize()});
         }
         detail::Check(detail::Abi<ElemType>::UnquantizeBatch(m_handle, raw.data(), raw.size(), nbits, add ? 1 : 0));
     }

@@ -252,6 +252,9 @@ int quantize_batch_noalloc_impl(cntkq_quantizer* h, const cntkq_quantize_item* i
         if (it.in == nullptr || it.res_in == nullptr || it.res_out == nullptr || it.qbuf == nullptr || !aligned4(it.in) || !aligned4(it.res_in) ||
             !aligned4(it.res_out) || !aligned4(it.qbuf))
             return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_quantize_batch_noalloc: item %zu: null or misaligned pointer", i);
+        if (it.qbuf_bytes != qcol_bytes(nbits, it.rows) * it.cols)
+            return fail(CNTKQ_LOGIC_ERROR, "cntkq_quantize_batch_noalloc: item %zu: packed buffer of %zu bytes does not match %zu x %zu at %zu bits (%zu bytes)",
+                        i, it.qbuf_bytes, it.rows, it.cols, nbits, qcol_bytes(nbits, it.rows) * it.cols);
     }
     const bool zt = zero_threshold_for_1bit != 0;
     DeviceGuard guard(h->device);

@@ -54,74 +54,20 @@ __host__ __device__ inline size_t tile_lds_bytes(const TileGeom& t, uint32_t wor
 // Columns of fewer QWords than this hand their new residual back through the LDS tile.
 constexpr uint32_t kStagedResidualBelowQWords = 16;
 
-// words[] (LDS, nc * nq entries) must be zero on entry when PackShape<NBITS>::CHUNKS > 1.
-// For a fixed bit position consecutive threads hold consecutive rows of a column, nq of them: where that run is at least a
-// 128-byte line the new residual goes straight to global memory; shorter runs (a 147-row column at 1 bit: 3 doubles) would
-// reach memory as fragments, so there the residual replaces the value in the tile (every value is read by exactly one work
-// item) and the tile leaves in consecutive stores.
-template <int NBITS, bool ZT>
-__device__ __forceinline__ void tile_pack(double* tile, const double* hdr, unsigned long long* words, const TileGeom& t,
-                                          uint32_t nc, char* qtile, double* res_out)
+// (tile_pack is the fp32 tile kernels' function too.) For a fixed bit position consecutive threads hold consecutive rows of a
+// column, nq of them: where that run is at least a 128-byte line the new residual goes straight to global memory; shorter
+// runs (a 147-row column at 1 bit: 3 doubles) would reach memory as fragments, so there the residual replaces the value in
+// the tile and the tile leaves in consecutive stores.
+__device__ __forceinline__ bool tile_residual_staged(const TileGeom& t)
 {
-    using PS = PackShape<NBITS>;
-    const uint32_t nwords = nc * t.nq;
-    const uint32_t items = nwords * PS::CHUNKS;
-    const bool staged = t.nq < kStagedResidualBelowQWords;
-    for (uint32_t it = threadIdx.x; it < items; it += kThreads)
-    {
-        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
-        const uint32_t qi = it - chunk * nwords;
-        const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
-        const uint32_t w = qi - c * t.nq;
-        const ValueQ vq = make_vq<NBITS>(hdr[2 * c], hdr[2 * c + 1]);
-        const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
-        const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
-        double* colv = tile + (size_t) c * t.rows;
-        double* ro = res_out + (size_t) c * t.rows;
-        uint64_t word = 0;
-#pragma unroll
-        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
-        {
-            const uint32_t k = chunk * PS::SLOTS + kk;
-            const uint32_t i = w + k * t.nq;
-            if (i < t.rows)
-            {
-                const double v = colv[i];
-                const uint64_t code = quantize_value<NBITS, ZT>(vq, v);
-                double back;
-                if constexpr (NBITS == 1)
-                    back = code ? val1 : val0;
-                else
-                    back = unquantize_value<NBITS>(vq.uf, vq.lo, code);
-                if (staged)
-                    colv[i] = v - back;
-                else
-                    __builtin_nontemporal_store(v - back, ro + i);
-                word |= code << (k * PS::SHIFT);
-            }
-        }
-        if constexpr (PS::CHUNKS == 1)
-            reinterpret_cast<uint64_t*>(qtile + (size_t) c * t.qcol + 16)[w] = word;
-        else
-            atomicOr(&words[qi], (unsigned long long) word);
-    }
-    if (PS::CHUNKS > 1 || staged) // uniform over the workgroup
-        __syncthreads();
-    if constexpr (PS::CHUNKS > 1)
-    {
-        for (uint32_t qi = threadIdx.x; qi < nwords; qi += kThreads)
-        {
-            const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
-            const uint32_t w = qi - c * t.nq;
-            reinterpret_cast<uint64_t*>(qtile + (size_t) c * t.qcol + 16)[w] = words[qi];
-        }
-    }
-    if (staged)
-    {
-        const uint32_t total = nc * t.rows;
-        for (uint32_t e = threadIdx.x; e < total; e += kThreads)
-            __builtin_nontemporal_store(tile[e], res_out + e);
-    }
+    return t.nq < kStagedResidualBelowQWords;
+}
+
+// after tile_pack with a staged residual: the tile to global memory
+__device__ __forceinline__ void tile_store(const double* tile, double* res_out, uint32_t total)
+{
+    for (uint32_t e = threadIdx.x; e < total; e += kThreads)
+        __builtin_nontemporal_store(tile[e], res_out + e);
 }
 
 struct TileLds
@@ -130,7 +76,7 @@ struct TileLds
     uint32_t* scratch_u;
     double* hdr;
     double* tile;
-    unsigned long long* words;
+    uint64_t* words;
     double* dec;
 };
 
@@ -141,7 +87,7 @@ __device__ __forceinline__ TileLds tile_lds(double* smem, const TileGeom& t)
     l.scratch_u = reinterpret_cast<uint32_t*>(smem + 8);
     l.hdr = smem + 10;
     l.tile = smem + kPrefixWords;
-    l.words = reinterpret_cast<unsigned long long*>(smem + kPrefixWords + t.tile_words);
+    l.words = reinterpret_cast<uint64_t*>(smem + kPrefixWords + t.tile_words);
     l.dec = smem + kPrefixWords + t.tile_words + t.words_words;
     return l;
 }
@@ -193,7 +139,10 @@ __device__ __forceinline__ void quantize_tile_body(const double* __restrict__ g,
 
     char* qtile = q + (size_t) j0 * t.qcol;
     tile_stats<NBITS, ZT>(l.tile, l.hdr, l.scratch_f, l.scratch_u, t, nc, qtile);
-    tile_pack<NBITS, ZT>(l.tile, l.hdr, l.words, t, nc, qtile, r_out + base);
+    const bool staged = tile_residual_staged(t);
+    tile_pack<NBITS, ZT>(l.tile, l.hdr, l.words, t, staged, nc, qtile, r_out + base);
+    if (staged)
+        tile_store(l.tile, r_out + base, nc * t.rows);
 }
 
 template <int NBITS, bool ZT>
@@ -379,7 +328,7 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
             l.words[x] = 0ull;
 
     // short columns: the stripe residual comes in as one consecutive run (see tile_pack), not as runs of nq rows
-    const bool staged = t.nq < kStagedResidualBelowQWords;
+    const bool staged = tile_residual_staged(t);
     if (staged)
         for (uint32_t e = tid; e < nc * t.rows; e += kThreads)
             l.tile[e] = __builtin_nontemporal_load(sp + e);
@@ -463,7 +412,9 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
 
     char* qtile = q_out + (size_t) j0 * t.qcol;
     tile_stats<NBITS, ZT>(l.tile, l.hdr, l.scratch_f, l.scratch_u, t, nc, qtile);
-    tile_pack<NBITS, ZT>(l.tile, l.hdr, l.words, t, nc, qtile, sp);
+    tile_pack<NBITS, ZT>(l.tile, l.hdr, l.words, t, staged, nc, qtile, sp);
+    if (staged)
+        tile_store(l.tile, sp, nc * t.rows);
 }
 
 template <int NBITS, bool ZT>

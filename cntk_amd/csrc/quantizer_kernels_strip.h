@@ -423,7 +423,7 @@ template <int NBITS>
 __device__ __forceinline__ uint32_t strip_valid_mask(const StripGeom& c, uint32_t w, uint32_t k0)
 {
     using SS = StripShape<NBITS>;
-    uint32_t valid = SS::SLOTS < 8 ? ~((1u << (4 * SS::SLOTS)) - 1u) : 0u; // bits beyond the thread's values count as present
+    uint32_t valid = ~(uint32_t) ((1ull << (4 * SS::SLOTS)) - 1ull); // bits beyond the thread's values count as present
 #pragma unroll
     for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
 #pragma unroll

@@ -82,28 +82,35 @@ __device__ __forceinline__ void tile_stats(const E* tile, E* hdr, E* scratch_f, 
     __syncthreads();
 }
 
-// words[] (LDS, nc * nq entries) must be zero on entry when PackShape<NBITS>::CHUNKS > 1.
-template <int NBITS, bool ZT>
-__device__ __forceinline__ void tile_pack(float* tile, const float* hdr, uint32_t* words, const TileGeom& t,
-                                          uint32_t nc, char* qtile, float* res_out)
+__device__ __forceinline__ void lds_or(uint32_t* p, uint32_t v) { atomicOr(p, v); }
+__device__ __forceinline__ void lds_or(uint64_t* p, uint64_t v) { atomicOr(reinterpret_cast<unsigned long long*>(p), (unsigned long long) v); }
+
+// words[] (LDS, nc * nq entries) must be zero on entry when a QWord has several work items (PackShape CHUNKS > 1).
+// stage: the new residual replaces the value in the tile (every value is read by exactly one work item) and the caller
+// writes the tile out afterwards; otherwise it goes straight to res_out. Written over the element type (E, its QWord) and
+// the tile geometry of either precision; the workgroup's size is blockDim.x.
+template <int NBITS, bool ZT, typename E, typename Geom>
+__device__ __forceinline__ void tile_pack(E* tile, const E* hdr, typename Word<E>::Q* words, const Geom& t, bool stage, uint32_t nc, char* qtile,
+                                          E* res_out)
 {
-    using PS = PackShape<NBITS>;
+    typedef typename Word<E>::Q QWord;
+    using PS = PackShapeOf<NBITS, Word<E>::kBits>;
+    const uint32_t threads = blockDim.x;
     const uint32_t nwords = nc * t.nq;
     const uint32_t items = nwords * PS::CHUNKS;
-    const bool stage = t.stage_residual != 0;
-    for (uint32_t it = threadIdx.x; it < items; it += t.threads)
+    for (uint32_t it = threadIdx.x; it < items; it += threads)
     {
         // chunk-major: consecutive threads take consecutive QWords, hence consecutive rows
         const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
         const uint32_t qi = it - chunk * nwords;
         const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
         const uint32_t w = qi - c * t.nq;
-        const ValueQ vq = make_vq<NBITS>(hdr[2 * c], hdr[2 * c + 1]);
-        const float val0 = unquantize_value<NBITS>(vq, 0u);
-        const float val1 = unquantize_value<NBITS>(vq, 1u);
-        float* colv = tile + (size_t) c * t.rows;
-        float* ro = res_out + (size_t) c * t.rows;
-        uint32_t word = 0;
+        const ValueQOf<E> vq = make_vq<NBITS>(hdr[2 * c], hdr[2 * c + 1]);
+        const E val0 = unquantize_value<NBITS>(vq, 0u);
+        const E val1 = unquantize_value<NBITS>(vq, 1u);
+        E* colv = tile + (size_t) c * t.rows;
+        E* ro = res_out + (size_t) c * t.rows;
+        QWord word = 0;
 #pragma unroll
         for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
         {
@@ -111,14 +118,14 @@ __device__ __forceinline__ void tile_pack(float* tile, const float* hdr, uint32_
             const uint32_t i = w + k * t.nq;
             if (i < t.rows)
             {
-                const float v = colv[i];
-                const uint32_t code = quantize_value<NBITS, ZT>(vq, v);
-                float back;
+                const E v = colv[i];
+                const QWord code = quantize_value<NBITS, ZT>(vq, v);
+                E back;
                 if constexpr (NBITS == 1)
                     back = code ? val1 : val0;
                 else
                     back = unquantize_value<NBITS>(vq, code);
-                const float res = v - back;
+                const E res = v - back;
                 if (stage)
                     colv[i] = res; // this element belongs to this work item alone
                 else
@@ -127,18 +134,18 @@ __device__ __forceinline__ void tile_pack(float* tile, const float* hdr, uint32_
             }
         }
         if constexpr (PS::CHUNKS == 1)
-            reinterpret_cast<uint32_t*>(qtile + (size_t) c * t.qcol + 8)[w] = word;
+            reinterpret_cast<QWord*>(qtile + (size_t) c * t.qcol + 2 * sizeof(E))[w] = word;
         else
-            atomicOr(&words[qi], word);
+            lds_or(&words[qi], word);
     }
     if constexpr (PS::CHUNKS > 1)
     {
         __syncthreads();
-        for (uint32_t qi = threadIdx.x; qi < nwords; qi += t.threads)
+        for (uint32_t qi = threadIdx.x; qi < nwords; qi += threads)
         {
             const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
             const uint32_t w = qi - c * t.nq;
-            reinterpret_cast<uint32_t*>(qtile + (size_t) c * t.qcol + 8)[w] = words[qi];
+            reinterpret_cast<QWord*>(qtile + (size_t) c * t.qcol + 2 * sizeof(E))[w] = words[qi];
         }
     }
     else if (stage)
@@ -280,7 +287,7 @@ __device__ __forceinline__ void quantize_tile_body(const float* __restrict__ g, 
 
     char* qtile = q + (size_t) j0 * t.qcol;
     tile_stats<NBITS, ZT>(tile, hdr, scratch_f, scratch_u, t, nc, qtile);
-    tile_pack<NBITS, ZT>(tile, hdr, words, t, nc, qtile, r_out + base);
+    tile_pack<NBITS, ZT>(tile, hdr, words, t, t.stage_residual != 0, nc, qtile, r_out + base);
     if (t.stage_residual)
         tile_store(tile, mis_g, r_out + base, total, t);
 }
@@ -422,7 +429,7 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
 
     char* qtile = q_out + (size_t) j0 * t.qcol;
     tile_stats<NBITS, ZT>(tile, hdr, scratch_f, scratch_u, t, nc, qtile);
-    tile_pack<NBITS, ZT>(tile, hdr, words, t, nc, qtile, sp);
+    tile_pack<NBITS, ZT>(tile, hdr, words, t, t.stage_residual != 0, nc, qtile, sp);
     if (t.stage_residual)
         tile_store(tile, mis_s, sp, total, t);
 }

@@ -148,17 +148,19 @@ typedef struct cntkq_quantize_item
     const float* in;
     const float* res_in;
     float* res_out;
-    void* qbuf; /* cntkq_qmatrix_bytes(rows, cols, nbits) bytes */
+    void* qbuf;
     size_t rows;
     size_t cols;
+    size_t qbuf_bytes; /* must be cntkq_qmatrix_bytes(rows, cols, nbits): the packed-size LogicError of the plain call */
 } cntkq_quantize_item;
 
 typedef struct cntkq_unquantize_item
 {
-    const void* qbuf; /* cntkq_qmatrix_bytes(rows, cols, nbits) bytes */
+    const void* qbuf;
     float* out;
     size_t rows;
     size_t cols;
+    size_t qbuf_bytes; /* must be cntkq_qmatrix_bytes(rows, cols, nbits) */
 } cntkq_unquantize_item;
 
 int cntkq_quantize_batch_async(cntkq_quantizer* h, const cntkq_quantize_item* items, size_t count, size_t nbits,
@@ -274,9 +276,10 @@ typedef struct cntkq_quantize_item_f64
     const double* in;
     const double* res_in;
     double* res_out; /* may be res_in */
-    void* qbuf;      /* device memory, cols * cntkq_qcol_bytes_f64(nbits, rows) bytes */
+    void* qbuf;      /* device memory */
     size_t rows;
     size_t cols;
+    size_t qbuf_bytes; /* must be cols * cntkq_qcol_bytes_f64(nbits, rows) */
 } cntkq_quantize_item_f64;
 
 typedef struct cntkq_unquantize_item_f64
@@ -285,6 +288,7 @@ typedef struct cntkq_unquantize_item_f64
     double* out;
     size_t rows;
     size_t cols;
+    size_t qbuf_bytes; /* must be cols * cntkq_qcol_bytes_f64(nbits, rows) */
 } cntkq_unquantize_item_f64;
 
 typedef struct cntkq_stripe_reduce_item_f64

@@ -182,6 +182,17 @@ def test_batch_argument_checks():
         qz.UnquantizeBatchAsync([(QuantizedMatrix(8, 4, 1, cntk_amd.CPUDEVICE), Matrix(8, 4))])
     qz.QuantizeBatchAsync([], False)
     qz.UnquantizeBatchAsync([])
+    # the packed-size check of the plain calls (Source/Math/MatrixQuantizer_kernel.cu:216-222, 280-289) holds per item, in either precision
+    for tdt in (torch.float32, torch.float64):
+        G, R, Q, Out = Matrix(64, 4, dtype=tdt), Matrix(64, 4, dtype=tdt), QuantizedMatrix(64, 4, 2, 0, dtype=tdt), Matrix(64, 4, dtype=tdt)
+        prepared = MatrixQuantizerImpl.PrepareQuantizeBatch([(G, R, Q, R), (G, R, Q, R)])
+        prepared.array[1].qbuf_bytes -= 4
+        with pytest.raises(cntk_amd.QuantizerLogicError, match="item 1: packed buffer"):
+            qz.QuantizeBatchAsync(prepared, False)
+        prepared = MatrixQuantizerImpl.PrepareUnquantizeBatch([(Q, Out), (Q, Out)])
+        prepared.array[0].qbuf_bytes += 8
+        with pytest.raises(cntk_amd.QuantizerLogicError, match="item 0: packed buffer"):
+            qz.UnquantizeBatchAsync(prepared)
 
 
 @pytest.mark.filterwarnings("ignore:The CUDA Graph is empty")  # the refused capture below leaves one
