@@ -562,6 +562,8 @@ int cntkq_destroy(cntkq_quantizer* h)
         (void) hipFree(h->strip_scratch.dev);
     if (h->strip_scratch.error_host != nullptr)
         (void) hipHostFree(h->strip_scratch.error_host);
+    if (h->strip_scratch.order_event != nullptr)
+        (void) hipEventDestroy(h->strip_scratch.order_event);
     table_destroy(h->quantize_table);
     table_destroy(h->unquantize_table);
     table_destroy(h->stripe_table);

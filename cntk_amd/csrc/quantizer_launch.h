@@ -37,6 +37,11 @@ struct StripScratchOwner
     size_t bytes = 0;        // header, finish counters, records
     size_t groups_bytes = 0; // the part of it set aside for finish counters: 1/256 of the whole
     uint32_t* error_host = nullptr;
+    // Launches that share the buffer must not overlap. One stream orders them by itself; when the handle's stream changes,
+    // the new stream first waits for the last launch on the old one (an event recorded after every launch).
+    hipEvent_t order_event = nullptr;
+    hipStream_t last_stream = nullptr;
+    bool launched = false;
 };
 
 struct LaunchTuning
@@ -517,6 +522,8 @@ inline hipError_t strip_scratch_for(StripScratchOwner& o, hipStream_t s, size_t 
         if (rc != hipSuccess)
             return rc;
         rc = hipMemsetAsync(p, 0, cap, s);
+        if (rc == hipSuccess)
+            rc = hipStreamSynchronize(s); // whichever stream launches next finds the buffer cleared
         if (rc != hipSuccess)
         {
             (void) hipFree(p);
@@ -631,11 +638,28 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
         const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit);
         if (!strip_applicable(rows, nbits, tune) || (uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull)
             return hipErrorInvalidValue;
+        StripScratchOwner& o = *tune.strip;
         StripScratch scratch;
-        const hipError_t rc = strip_scratch_for(*tune.strip, s, cols, c.strips, scratch);
+        hipError_t rc = strip_scratch_for(o, s, cols, c.strips, scratch);
         if (rc != hipSuccess)
             return rc;
-        return dispatch_nbits<StripLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, scratch);
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        const bool capturing = hipStreamIsCapturing(s, &st) != hipSuccess || st != hipStreamCaptureStatusNone;
+        if (!capturing)
+        {
+            if (o.order_event == nullptr && (rc = hipEventCreateWithFlags(&o.order_event, hipEventDisableTiming)) != hipSuccess)
+                return rc;
+            if (o.launched && o.last_stream != s && (rc = hipStreamWaitEvent(s, o.order_event, 0)) != hipSuccess)
+                return rc;
+        }
+        rc = dispatch_nbits<StripLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, scratch);
+        if (rc == hipSuccess && !capturing)
+        {
+            rc = hipEventRecord(o.order_event, s);
+            o.last_stream = s;
+            o.launched = true;
+        }
+        return rc;
     }
     if (path == kPathRegScalar)
     {

@@ -587,3 +587,27 @@ def test_strip_kernel_reports_workgroups_that_give_up():
     qz.QuantizeAsync(G, R, Q, R, False)
     qz.WaitQuantizeAsyncDone()
     parity.check_quantize(g, np.zeros_like(g, order="F"), Q.to_numpy(), R.to_numpy(), 1, False)
+
+
+def test_strip_kernel_across_a_stream_change():
+    """Strip launches of one handle share its scratch buffer, so a launch on a new main stream must wait for the last one
+    on the old stream: two tall matrices quantized back to back on two streams, several times over, both right."""
+    rows, cols = 140000, 24
+    qz = MatrixQuantizerImpl.Create(0, False)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    gs = [datagen.normal(7 + i, rows, cols) for i in range(2)]
+    G = [Matrix.from_numpy(g) for g in gs]
+    R = [Matrix(rows, cols) for _ in range(2)]
+    Q = [QuantizedMatrix(rows, cols, 1, 0) for _ in range(2)]
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for i in range(2):
+            R[i].data.zero_()
+        torch.cuda.synchronize()
+        for i in range(2):
+            qz.SetMainStream(streams[i].cuda_stream)
+            qz.QuantizeAsync(G[i], R[i], Q[i], R[i], False)
+        torch.cuda.synchronize()
+        qz.WaitQuantizeAsyncDone()
+        for i in range(2):
+            parity.check_quantize(gs[i], np.zeros_like(gs[i], order="F"), Q[i].to_numpy(), R[i].to_numpy(), 1, False)
