@@ -150,7 +150,7 @@ struct BatchAbi<float>
             if (!line_shift && aligned && it.rows <= 2048 && col_unrolled(it.q_out, it.rows, nbits))
             {
                 e.kind = it.rows == 1024 ? 2 : 3;
-                lds = (it.rows == 1024 ? col_lds_bytes<1>() : col_lds_bytes<2>()) + 2 * kMaxWorkers * 4;
+                lds = (it.rows == 1024 ? col_lds_bytes<1>() : col_lds_bytes<2>()) + kStripeColExtraLds;
             }
         }
         else

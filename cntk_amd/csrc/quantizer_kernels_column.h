@@ -42,6 +42,10 @@ constexpr size_t col_lds_bytes()
     return (size_t) (1024 * PER + 32 * PER + 8 + 4) * 4;
 }
 
+// LDS of the stripe reduction beyond col_lds_bytes: two levels per worker (up to kMaxWorkers), or, with up to eight
+// workers, their sixteen levels and the 256 sums they can add up to
+constexpr size_t kStripeColExtraLds = (2 * 8 + 256) * 4 > 2 * kMaxWorkers * 4 ? (2 * 8 + 256) * 4 : 2 * kMaxWorkers * 4;
+
 // The 1-bit split sums of one 16-byte piece (x y z w in order): values below the mean go to s0 / n0, the others to s1.
 // Like the column sum, the split sums are taken piece by piece by every column kernel, whether it keeps the column in
 // LDS or in registers, so that all of them give the same header for the same column.
@@ -238,6 +242,40 @@ __device__ __forceinline__ void stripe_reduce_col_body(const StripeSources& src,
     __syncthreads();
 
     float acc[KS];
+    if (K <= BATCH)
+    {
+        // Up to eight workers: the sum of an element is one of 256 values, picked by the workers' bits of the element. The
+        // workgroup's 256 threads build one entry each (the additions of the loop below, in its order, seeded with -0:
+        // x + -0 = x for every x), the thread turns its eight QWords into one byte per bit position (bit g = worker g of
+        // the order) and looks the sums up: a bit-field extract and an LDS read per element instead of three instructions
+        // per worker and element.
+        float* lut = dec + 2 * BATCH;
+        {
+            float a = -0.0f;
+#pragma unroll
+            for (uint32_t u = 0; u < BATCH; ++u)
+                if (u < K)
+                    a = ((tid >> u) & 1u ? dec[2 * u + 1] : dec[2 * u]) + a;
+            lut[tid] = a;
+        }
+        __syncthreads();
+#pragma unroll
+        for (uint32_t b = 0; b < (KS + 7) / 8; ++b)
+        {
+            uint32_t row[BATCH];
+#pragma unroll
+            for (uint32_t u = 0; u < BATCH; ++u)
+                row[u] = u < K ? word[u] >> (sh0 + 8 * b) : 0u;
+            // byte 0 of the second operand, byte 0 of the first, zeros
+            uint32_t lo = __builtin_amdgcn_perm(row[1], row[0], 0x0C0C0400u) | (__builtin_amdgcn_perm(row[3], row[2], 0x0C0C0400u) << 16);
+            uint32_t hi = __builtin_amdgcn_perm(row[5], row[4], 0x0C0C0400u) | (__builtin_amdgcn_perm(row[7], row[6], 0x0C0C0400u) << 16);
+            transpose_bits_8x8(lo, hi);
+#pragma unroll
+            for (uint32_t r = 0; r < 8 && 8 * b + r < KS; ++r)
+                acc[8 * b + r] = lut[((r < 4 ? lo : hi) >> (8 * (r & 3u))) & 255u];
+        }
+    }
+    else
     for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
     {
         if (n0 != 0)

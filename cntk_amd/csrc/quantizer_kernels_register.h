@@ -735,6 +735,165 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<
     reg_stats_pack<1, ZT, T, PER>(a, edge, has_edge, edge_at, head, pieces, shift, c, red, red_u, words, sres, q_out + rec);
 }
 
+// ---- 1 bit, up to eight workers: the sum of a row looked up, not added up ----------------------------------------------
+//
+// With K <= 8 workers the aggregate of an element is one of 256 values: the levels of the K columns' headers added up in
+// the summation order (owner first), picked by the K bits of the element. A workgroup builds that table once per column
+// (256 entries, each with the additions of the decoding loop in their order, hence the same bits) and turns the workers'
+// QWords into one byte per element: bit g of the byte = the element's bit in the stripe of the g-th worker of the order.
+// The bytes lie in element order (QWord w of bit position k holds element k * nq + w), so the four elements of a piece are
+// one aligned dword (the table is shifted by the column's `head`) and need no position arithmetic at all. Decoding an
+// element is a bit-field extract, an address and an LDS read where the kernels above spend three instructions per worker;
+// the transposition costs about five per element (8 x 8 bit blocks, three exchange steps each).
+// LDS: [48 reduction slots | nq output QWords | 256 sums | rows + 8 bytes].
+
+__host__ __device__ inline uint32_t stripe_lut_bytes_offset(const RegGeom& c) // in dwords
+{
+    return (kRegRedSlots + c.nq + 256u + 3u) & ~3u;
+}
+
+__host__ __device__ inline size_t stripe_lut_lds_bytes(const RegGeom& c)
+{
+    return (size_t) stripe_lut_bytes_offset(c) * 4 + (((size_t) c.rows + 8 + 15) & ~(size_t) 15);
+}
+
+template <bool ZT, int PER>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<1024, PER>(), reg_waves<1024, PER>()))) void stripe_reduce_lut_kernel(
+    StripeSources src, float* stripe_res, char* q_out, float* agg_out, RegGeom c)
+{
+    constexpr uint32_t T = 1024, NW = T / 64, S = 8;
+    extern __shared__ f32x4 smem_v4[];
+    float* red = reinterpret_cast<float*>(smem_v4);
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
+    uint32_t* words = reinterpret_cast<uint32_t*>(red + kRegRedSlots);
+    float* lut = reinterpret_cast<float*>(words + c.nq);
+    uint8_t* pat = reinterpret_cast<uint8_t*>(reinterpret_cast<uint32_t*>(red) + stripe_lut_bytes_offset(c));
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) blockIdx.x * c.rows;
+    const size_t rec = (size_t) blockIdx.x * c.qcol;
+    for (uint32_t x = tid; x < c.nq; x += T)
+        words[x] = 0u;
+    float* sres = stripe_res + base;
+    const uint32_t head = (4u - (uint32_t) ((reinterpret_cast<uintptr_t>(sres) >> 2) & 3u)) & 3u;
+    const uint32_t pieces = (c.rows - head) >> 2;
+    const uint32_t tail = c.rows - head - 4 * pieces;
+    const bool has_edge = tid < head + tail;
+    const uint32_t edge_at = tid < head ? tid : c.rows - tail + (tid - head);
+    const uint32_t shift = column_shift(sres + head, c.line_shift);
+    const uint32_t K = src.workers; // at most 8
+    // element i has its byte at pat[i + lead]: piece p (elements head + 4 p ...) is the aligned dword 4 p + lead + head
+    const uint32_t lead = (4u - head) & 3u;
+
+    // The stripe residual is requested first: its latency runs under the table building below (one workgroup fills a CU,
+    // nothing else would overlap the two), and a sum plus its residual is the same bits in either order. The tallest
+    // columns, whose residual would leave the table building no registers, request it piece by piece at the look-ups.
+    constexpr bool EARLY = PER <= 20;
+    f32x4 a[PER];
+    const f32x4* r4 = reinterpret_cast<const f32x4*>(sres + head);
+    if constexpr (EARLY)
+    {
+        const uint32_t t = opaque(tid);
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+        {
+            a[u] = f32x4{-0.0f, -0.0f, -0.0f, -0.0f};
+            if (slot_valid(t + T * u, shift, pieces))
+                a[u] = __builtin_nontemporal_load(r4 + (t + T * u - shift));
+        }
+    }
+
+    // the 256 sums: entry x adds, in the order of the summation, the level each worker's header gives for its bit of x,
+    // starting from -0 (x + -0 = x for every x, signed zeros included), as unquantize ... unquantize-and-add would
+    if (tid < 256)
+    {
+        float acc = -0.0f;
+        for (uint32_t g = 0; g < K; ++g)
+        {
+            const float* h = reinterpret_cast<const float*>(src.q[stripe_order(g, src.owner)] + rec);
+            const float lo = h[0];
+            const float uf = make_ufactor<1>(lo, h[1]);
+            acc = unquantize_value<1>(uf, lo, (tid >> g) & 1u) + acc;
+        }
+        lut[tid] = acc;
+    }
+    // the workers' QWords, transposed into one byte per element
+    {
+        const uint32_t* from[S];
+#pragma unroll
+        for (uint32_t g = 0; g < S; ++g)
+            from[g] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(min(g, K - 1), src.owner)] + rec) + 2;
+        for (uint32_t x = tid; x < c.nq; x += T)
+        {
+            uint32_t d[S];
+#pragma unroll
+            for (uint32_t g = 0; g < S; ++g)
+                d[g] = from[g][x];
+#pragma unroll
+            for (uint32_t g = 0; g < S; ++g)
+                d[g] = g < K ? d[g] : 0u;
+            uint8_t* to = pat + lead + x;
+#pragma unroll 1 // (one block at a time: most registers are taken by the residual by now)
+            for (uint32_t j = 0; j < 4; ++j)
+            {
+                // byte j of every worker's QWord: an 8 x 8 block of (worker, bit position 8 j ...)
+                const uint32_t sel = 0x0C0C0000u | ((4u + j) << 8) | j; // byte 0: byte j of the second operand, byte 1: of the first
+                uint32_t lo = __builtin_amdgcn_perm(d[1], d[0], sel) | (__builtin_amdgcn_perm(d[3], d[2], sel) << 16);
+                uint32_t hi = __builtin_amdgcn_perm(d[5], d[4], sel) | (__builtin_amdgcn_perm(d[7], d[6], sel) << 16);
+                transpose_bits_8x8(lo, hi);
+#pragma unroll
+                for (uint32_t r = 0; r < 8; ++r)
+                {
+                    const uint32_t k = 8 * j + r;
+                    const uint32_t i = k * c.nq + x;
+                    if (i < c.rows)
+                        to[k * c.nq] = (uint8_t) ((r < 4 ? lo : hi) >> (8 * (r & 3u)));
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    float edge = -0.0f;
+    {
+        const uint32_t t = opaque(tid);
+        const uint32_t* pat4 = reinterpret_cast<const uint32_t*>(pat + lead + head);
+        float* ag = agg_out != nullptr ? agg_out + base : nullptr;
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+        {
+            if constexpr (!EARLY)
+                a[u] = f32x4{-0.0f, -0.0f, -0.0f, -0.0f};
+            if (slot_valid(t + T * u, shift, pieces))
+            {
+                const uint32_t p = t + T * u - shift;
+                if constexpr (!EARLY)
+                    a[u] = __builtin_nontemporal_load(r4 + p); // requested before the look-ups, used after them
+                const uint32_t four = pat4[p];
+                f32x4 v;
+                v[0] = lut[four & 255u];
+                v[1] = lut[(four >> 8) & 255u];
+                v[2] = lut[(four >> 16) & 255u];
+                v[3] = lut[four >> 24];
+                if (ag != nullptr)
+                {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        ag[head + 4 * p + e] = v[e];
+                }
+                a[u] = v + a[u];
+            }
+        }
+        if (has_edge)
+        {
+            edge = lut[pat[lead + edge_at]];
+            if (agg_out != nullptr)
+                agg_out[base + edge_at] = edge;
+            edge = edge + sres[edge_at];
+        }
+    }
+    reg_stats_pack<1, ZT, T, PER>(a, edge, has_edge, edge_at, head, pieces, shift, c, red, red_u, words, sres, q_out + rec);
+}
+
 // ---- the same for tall columns of any height and alignment: elements instead of pieces ----------------------
 //
 // Thread tid of 1024 keeps elements tid, tid + 1024, ... (at most EPT) of the column in registers, loaded and stored one

@@ -361,7 +361,7 @@ template <bool ZT, int PER>
 inline void launch_stripe_col(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
                               uint32_t cols, uint64_t qcol)
 {
-    hipExtLaunchKernelGGL((stripe_reduce_col_kernel<ZT, PER>), dim3(cols), dim3(kColThreads), col_lds_bytes<PER>() + 2 * kMaxWorkers * 4, s,
+    hipExtLaunchKernelGGL((stripe_reduce_col_kernel<ZT, PER>), dim3(cols), dim3(kColThreads), col_lds_bytes<PER>() + kStripeColExtraLds, s,
                           ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, qcol);
 }
 
@@ -720,6 +720,13 @@ inline hipError_t launch_stripe_reg_one(hipStream_t s, LaunchEvents ev, const St
     {
         // 1 bit: eight workers at a time from the worker-minor table, where a CU's LDS holds it (always, up to 102400 rows)
         // (it always decodes eight slots: with four workers or fewer the kernel below does less work)
+        // up to eight workers: the row sums looked up in a table of 256 (the same additions, made once per column)
+        if (src.workers <= 8 && stripe_lut_lds_bytes(c) <= 160 * 1024)
+        {
+            hipExtLaunchKernelGGL((stripe_reduce_lut_kernel<ZT, PER>), dim3(cols), dim3(1024), stripe_lut_lds_bytes(c), s, ev.start, ev.stop, 0,
+                                  src, stripe_res, q_out, agg_out, c);
+            return hipGetLastError();
+        }
         if (src.workers > 4 && stripe_reg8_lds_bytes(c) <= 160 * 1024)
         {
             hipExtLaunchKernelGGL((stripe_reduce_reg8_kernel<ZT, PER>), dim3(cols), dim3(1024), stripe_reg8_lds_bytes(c), s, ev.start, ev.stop, 0,

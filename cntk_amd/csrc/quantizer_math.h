@@ -225,6 +225,29 @@ __device__ __forceinline__ void finish_stats_multibit(E sumsq, uint32_t rows, E&
     hi = mean + half;
 }
 
+// ---- bit matrices -------------------------------------------------------------------------------
+
+// Transposes an 8 x 8 bit matrix held as two dwords (row r = byte r, lo holds rows 0-3): three rounds of swapping
+// off-diagonal blocks. After it byte r has, as bit g, bit r of the former byte g.
+__device__ __forceinline__ void transpose_bits_8x8(uint32_t& lo, uint32_t& hi)
+{
+    uint32_t t;
+    // 1 x 1 blocks within 2 x 2: bit c of row r <-> bit r of row c for neighbours (rows 8 bits apart: shift 7)
+    t = (lo ^ (lo >> 7)) & 0x00AA00AAu;
+    lo = lo ^ t ^ (t << 7);
+    t = (hi ^ (hi >> 7)) & 0x00AA00AAu;
+    hi = hi ^ t ^ (t << 7);
+    // 2 x 2 blocks within 4 x 4 (rows 16 bits apart: shift 14)
+    t = (lo ^ (lo >> 14)) & 0x0000CCCCu;
+    lo = lo ^ t ^ (t << 14);
+    t = (hi ^ (hi >> 14)) & 0x0000CCCCu;
+    hi = hi ^ t ^ (t << 14);
+    // 4 x 4 blocks: the high nibbles of rows 0-3 <-> the low nibbles of rows 4-7
+    t = ((lo >> 4) ^ hi) & 0x0F0F0F0Fu;
+    hi = hi ^ t;
+    lo = lo ^ (t << 4);
+}
+
 // ---- cross-lane sums ----------------------------------------------------------------------------
 
 // Sum over aligned groups of `width` lanes (power of two, <= 64); every lane of a group gets the
