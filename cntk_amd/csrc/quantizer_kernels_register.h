@@ -757,11 +757,12 @@ __host__ __device__ inline size_t stripe_lut_lds_bytes(const RegGeom& c)
     return (size_t) stripe_lut_bytes_offset(c) * 4 + (((size_t) c.rows + 8 + 15) & ~(size_t) 15);
 }
 
-template <bool ZT, int PER>
-__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<1024, PER>(), reg_waves<1024, PER>()))) void stripe_reduce_lut_kernel(
+template <bool ZT, int PER, int TT = 1024>
+__global__ __launch_bounds__(TT) __attribute__((amdgpu_waves_per_eu(reg_waves<TT, PER>(), reg_waves<TT, PER>()))) void stripe_reduce_lut_kernel(
     StripeSources src, float* stripe_res, char* q_out, float* agg_out, RegGeom c)
 {
-    constexpr uint32_t T = 1024, NW = T / 64, S = 8;
+    constexpr uint32_t T = TT, NW = T / 64, S = 8;
+    static_assert(T >= 256, "one thread per table entry");
     extern __shared__ f32x4 smem_v4[];
     float* red = reinterpret_cast<float*>(smem_v4);
     uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);

@@ -716,17 +716,20 @@ template <int NBITS, bool ZT, int PER, int T = 1024>
 inline hipError_t launch_stripe_reg_one(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
                                         uint32_t cols, const RegGeom& c)
 {
+    if constexpr (NBITS == 1)
+    {
+        // up to eight workers: the row sums looked up in a table of 256 (the same additions, made once per column)
+        if (src.workers <= 8 && stripe_lut_lds_bytes(c) <= 160 * 1024)
+        {
+            hipExtLaunchKernelGGL((stripe_reduce_lut_kernel<ZT, PER, T>), dim3(cols), dim3(T), stripe_lut_lds_bytes(c), s, ev.start, ev.stop, 0, src,
+                                  stripe_res, q_out, agg_out, c);
+            return hipGetLastError();
+        }
+    }
     if constexpr (NBITS == 1 && T == 1024)
     {
         // 1 bit: eight workers at a time from the worker-minor table, where a CU's LDS holds it (always, up to 102400 rows)
         // (it always decodes eight slots: with four workers or fewer the kernel below does less work)
-        // up to eight workers: the row sums looked up in a table of 256 (the same additions, made once per column)
-        if (src.workers <= 8 && stripe_lut_lds_bytes(c) <= 160 * 1024)
-        {
-            hipExtLaunchKernelGGL((stripe_reduce_lut_kernel<ZT, PER>), dim3(cols), dim3(1024), stripe_lut_lds_bytes(c), s, ev.start, ev.stop, 0,
-                                  src, stripe_res, q_out, agg_out, c);
-            return hipGetLastError();
-        }
         if (src.workers > 4 && stripe_reg8_lds_bytes(c) <= 160 * 1024)
         {
             hipExtLaunchKernelGGL((stripe_reduce_reg8_kernel<ZT, PER>), dim3(cols), dim3(1024), stripe_reg8_lds_bytes(c), s, ev.start, ev.stop, 0,
