@@ -803,32 +803,46 @@ __global__ __launch_bounds__(TT) __attribute__((amdgpu_waves_per_eu(reg_waves<TT
         }
     }
 
+    // this thread's first QWords are requested before the table of sums is built, so that headers and QWords cost one round
+    // trip to memory, not two
+    const uint32_t* from[S];
+#pragma unroll
+    for (uint32_t g = 0; g < S; ++g)
+        from[g] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(min(g, K - 1), src.owner)] + rec) + 2;
+    uint32_t first[S];
+#pragma unroll
+    for (uint32_t g = 0; g < S; ++g)
+        first[g] = from[g][min(tid, c.nq - 1)];
+
     // the 256 sums: entry x adds, in the order of the summation, the level each worker's header gives for its bit of x,
     // starting from -0 (x + -0 = x for every x, signed zeros included), as unquantize ... unquantize-and-add would
     if (tid < 256)
     {
+        // (all headers requested together: a loop over the K workers would wait for each in turn)
+        f32x2 h[S];
+#pragma unroll
+        for (uint32_t g = 0; g < S; ++g)
+            h[g] = *reinterpret_cast<const f32x2_u*>(src.q[stripe_order(min(g, K - 1), src.owner)] + rec);
         float acc = -0.0f;
-        for (uint32_t g = 0; g < K; ++g)
+#pragma unroll
+        for (uint32_t g = 0; g < S; ++g)
         {
-            const float* h = reinterpret_cast<const float*>(src.q[stripe_order(g, src.owner)] + rec);
-            const float lo = h[0];
-            const float uf = make_ufactor<1>(lo, h[1]);
-            acc = unquantize_value<1>(uf, lo, (tid >> g) & 1u) + acc;
+            if (g < K)
+            {
+                const float uf = make_ufactor<1>(h[g].x, h[g].y);
+                acc = unquantize_value<1>(uf, h[g].x, (tid >> g) & 1u) + acc;
+            }
         }
         lut[tid] = acc;
     }
     // the workers' QWords, transposed into one byte per element
     {
-        const uint32_t* from[S];
-#pragma unroll
-        for (uint32_t g = 0; g < S; ++g)
-            from[g] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(min(g, K - 1), src.owner)] + rec) + 2;
         for (uint32_t x = tid; x < c.nq; x += T)
         {
             uint32_t d[S];
 #pragma unroll
             for (uint32_t g = 0; g < S; ++g)
-                d[g] = from[g][x];
+                d[g] = x == tid ? first[g] : from[g][x];
 #pragma unroll
             for (uint32_t g = 0; g < S; ++g)
                 d[g] = g < K ? d[g] : 0u;

@@ -17,6 +17,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef f32x4 f32x4_u __attribute__((aligned(4))); // a 16-byte access at any 4-byte alignment
 typedef u32x4 u32x4_u __attribute__((aligned(4)));
+typedef f32x2 f32x2_u __attribute__((aligned(4)));
 
 constexpr int kWave = 64;
 
