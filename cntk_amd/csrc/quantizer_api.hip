@@ -538,8 +538,9 @@ int cntkq_create(int device_id, int use_dedicated_stream, cntkq_quantizer** out)
     {
         // The strip kernels' scratch buffer at its starting size, so that a first call under graph capture (which cannot
         // allocate) finds it. A failure here is not one of the handle: the first call that needs the buffer tries again.
+        // (cleared on one of the handle's own streams and waited for there: the legacy default stream stays out of it)
         StripScratch unused;
-        if (strip_scratch_for(h->strip_scratch, nullptr, 1, 2, unused) != hipSuccess || hipStreamSynchronize(nullptr) != hipSuccess)
+        if (strip_scratch_for(h->strip_scratch, h->fetch, 1, 2, unused) != hipSuccess)
             (void) hipGetLastError();
     }
     *out = h;
