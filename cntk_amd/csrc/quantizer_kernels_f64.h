@@ -426,98 +426,9 @@ __global__ __launch_bounds__(kThreads) void stripe_reduce_tile_kernel(StripeSour
 }
 
 // ---- unquantize ----------------------------------------------------------------------------------------------
-// One thread decodes WV consecutive QWords of a column (WV = 2: 16-byte stores; WV = 1: any shape) for a chunk of
-// `slots` consecutive bit positions; for a fixed bit position consecutive QWords are consecutive rows.
-
-struct UnqGeom
-{
-    uint32_t rows;
-    uint32_t cols;
-    uint32_t nq;
-    uint32_t groups;  // ceil(nq / WV)
-    uint32_t chunks;  // ceil(VPW / slots)
-    uint32_t slots;
-    uint32_t per_col; // groups * chunks
-    uint32_t items;   // per_col * cols
-    uint32_t swz_members; // > 1: workgroups regrouped by XCD (unq_xcd_block)
-    uint32_t swz_gw;
-    uint64_t qcol;
-};
-
-template <int NBITS, int WV>
-__device__ __forceinline__ void unquantize_body(const char* __restrict__ q, double* out, const UnqGeom& t, int add, uint32_t block_in)
-{
-    using PS = PackShape<NBITS>;
-    const uint32_t block = t.swz_members > 1 ? unq_xcd_block(block_in, t.items / 256, t.swz_members, t.swz_gw) : block_in;
-    const uint64_t id64 = (uint64_t) block * 256 + threadIdx.x;
-    if (id64 >= t.items)
-        return;
-    const uint32_t id = (uint32_t) id64;
-    const uint32_t c = id / t.per_col;
-    const uint32_t rem = id - c * t.per_col;
-    const uint32_t chunk = rem / t.groups;
-    const uint32_t grp = rem - chunk * t.groups;
-    const uint32_t w0 = grp * WV;
-
-    const char* qc = q + (size_t) c * t.qcol;
-    const double* gh = reinterpret_cast<const double*>(qc);
-    const ValueQ vq = make_vq<NBITS>(gh[0], gh[1]);
-    const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
-    const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
-    const uint64_t* bits = reinterpret_cast<const uint64_t*>(qc + 16);
-    double* oc = out + (size_t) c * t.rows;
-
-    uint64_t word[WV];
-#pragma unroll
-    for (int u = 0; u < WV; ++u)
-        word[u] = bits[w0 + u]; // WV == 2 only when nq is even
-
-    const uint32_t k0 = chunk * t.slots;
-    const uint32_t k1 = min(k0 + t.slots, PS::VPW);
-    for (uint32_t k = k0; k < k1; ++k)
-    {
-        const uint32_t i = w0 + k * t.nq;
-        if (i >= t.rows)
-            break; // rows only grow with k
-        const uint32_t sh = k * PS::SHIFT;
-        if constexpr (WV == 2)
-        {
-            // rows and nq even, i even: both rows are inside the column and the store is 16-byte aligned
-            f64x2 x;
-            if constexpr (NBITS == 1)
-            {
-                x.x = ((word[0] >> sh) & 1ull) ? val1 : val0;
-                x.y = ((word[1] >> sh) & 1ull) ? val1 : val0;
-            }
-            else
-            {
-                x.x = unquantize_value<NBITS>(vq.uf, vq.lo, (word[0] >> sh) & PS::CODEMASK);
-                x.y = unquantize_value<NBITS>(vq.uf, vq.lo, (word[1] >> sh) & PS::CODEMASK);
-            }
-            f64x2* dst = reinterpret_cast<f64x2*>(oc + i);
-            if (add)
-                x = x + *dst; // unquantized value + previous content
-            __builtin_nontemporal_store(x, dst);
-        }
-        else
-        {
-            double x;
-            if constexpr (NBITS == 1)
-                x = ((word[0] >> sh) & 1ull) ? val1 : val0;
-            else
-                x = unquantize_value<NBITS>(vq.uf, vq.lo, (word[0] >> sh) & PS::CODEMASK);
-            if (add)
-                x = x + oc[i];
-            oc[i] = x;
-        }
-    }
-}
-
-template <int NBITS, int WV>
-__global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, double* out, UnqGeom t, int add)
-{
-    unquantize_body<NBITS, WV>(q, out, t, add, blockIdx.x);
-}
+//
+// The QWord-major decoder (UnqGeom, unquantize_body, unquantize_kernel) is the fp32 source, written over the element type:
+// two QWords and two rows per thread and bit position where rows and QWords per column are even, else one.
 
 // ---- row-major and tile decoders (the fp32 unquantize_rows_kernel / unquantize_tile_kernel on doubles) ---------
 //

@@ -55,12 +55,15 @@ __device__ __forceinline__ uint32_t unq_xcd_block(uint32_t b, uint32_t blocks, u
     return (c * members + m) * gw + g;
 }
 
-template <int NBITS, int WV>
-__device__ __forceinline__ void unquantize_body(const char* __restrict__ q, float* out, const UnqGeom& t, int add, uint32_t block)
+// Written over the element type: E = float with 32-bit QWords (WV = 4 QWords and rows per thread and bit position, one
+// 16-byte store) or double with 64-bit QWords (WV = 2); WV = 1 stores one element at a time, whatever the alignment.
+template <int NBITS, int WV, typename E>
+__device__ __forceinline__ void unquantize_body(const char* __restrict__ q, E* out, const UnqGeom& t, int add, uint32_t block)
 {
-    constexpr uint32_t VPW = 32 / NBITS;
-    constexpr uint32_t MASKBITS = NBITS & 31;
-    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << MASKBITS) - 1u);
+    typedef typename Word<E>::Q QWord;
+    using PS = PackShapeOf<NBITS, Word<E>::kBits>;
+    typedef E Vec __attribute__((ext_vector_type(WV == 1 ? 2 : WV))); // (unused when WV == 1)
+    static_assert(WV == 1 || WV * sizeof(E) == 16, "one 16-byte store per bit position");
 
     if (t.swz_members > 1)
         block = unq_xcd_block(block, t.items / 256, t.swz_members, t.swz_gw);
@@ -75,17 +78,17 @@ __device__ __forceinline__ void unquantize_body(const char* __restrict__ q, floa
     const uint32_t w0 = grp * WV;
 
     const char* qc = q + (size_t) c * t.qcol;
-    const float* gh = reinterpret_cast<const float*>(qc);
-    ValueQ vq; // decoding needs only the code -> value factor and the lower bound
+    const E* gh = reinterpret_cast<const E*>(qc);
+    ValueQOf<E> vq; // decoding needs only the code -> value factor and the lower bound
     vq.lo = gh[0];
     vq.uf = make_ufactor<NBITS>(gh[0], gh[1]);
-    const float val0 = unquantize_value<NBITS>(vq, 0u);
-    const float val1 = unquantize_value<NBITS>(vq, 1u);
-    const uint32_t* bits = reinterpret_cast<const uint32_t*>(qc + 8);
-    float* oc = out + (size_t) c * t.rows;
+    const E val0 = unquantize_value<NBITS>(vq, 0u);
+    const E val1 = unquantize_value<NBITS>(vq, 1u);
+    const QWord* bits = reinterpret_cast<const QWord*>(qc + 2 * sizeof(E));
+    E* oc = out + (size_t) c * t.rows;
 
-    uint32_t word[WV];
-    if constexpr (WV == 4)
+    QWord word[WV];
+    if constexpr (WV == 4 && sizeof(QWord) == 4)
     {
         // the word group starts 8 bytes past a 16-byte boundary or on one: two 8-byte loads are always aligned
         const u32x2 a = *reinterpret_cast<const u32x2*>(bits + w0);
@@ -97,47 +100,43 @@ __device__ __forceinline__ void unquantize_body(const char* __restrict__ q, floa
     }
     else
     {
-        word[0] = bits[w0];
+#pragma unroll
+        for (int u = 0; u < WV; ++u)
+            word[u] = bits[w0 + u]; // (double: WV == 2 only when nq is even)
     }
 
     const uint32_t k0 = chunk * t.slots;
-    const uint32_t k1 = min(k0 + t.slots, VPW);
+    const uint32_t k1 = min(k0 + t.slots, PS::VPW);
     for (uint32_t k = k0; k < k1; ++k)
     {
         const uint32_t i = w0 + k * t.nq;
         if (i >= t.rows)
             break; // rows only grow with k
-        const uint32_t sh = k * MASKBITS;
-        if constexpr (WV == 4)
+        const uint32_t sh = k * PS::SHIFT;
+        if constexpr (WV > 1)
         {
-            // rows % 4 == 0 and i % 4 == 0: the four rows are all inside the column
-            f32x4 x;
-            if constexpr (NBITS == 1)
+            // rows, nq and i are multiples of WV: the WV rows are all inside the column and the store is 16-byte aligned
+            Vec x;
+#pragma unroll
+            for (int u = 0; u < WV; ++u)
             {
-                x.x = ((word[0] >> sh) & 1u) ? val1 : val0;
-                x.y = ((word[1] >> sh) & 1u) ? val1 : val0;
-                x.z = ((word[2] >> sh) & 1u) ? val1 : val0;
-                x.w = ((word[3] >> sh) & 1u) ? val1 : val0;
+                if constexpr (NBITS == 1)
+                    x[u] = ((word[u] >> sh) & 1u) ? val1 : val0;
+                else
+                    x[u] = unquantize_value<NBITS>(vq, (word[u] >> sh) & PS::CODEMASK);
             }
-            else
-            {
-                x.x = unquantize_value<NBITS>(vq, (word[0] >> sh) & CODEMASK);
-                x.y = unquantize_value<NBITS>(vq, (word[1] >> sh) & CODEMASK);
-                x.z = unquantize_value<NBITS>(vq, (word[2] >> sh) & CODEMASK);
-                x.w = unquantize_value<NBITS>(vq, (word[3] >> sh) & CODEMASK);
-            }
-            f32x4* dst = reinterpret_cast<f32x4*>(oc + i);
+            Vec* dst = reinterpret_cast<Vec*>(oc + i);
             if (add)
                 x = x + *dst; // unquantized value + previous content
             __builtin_nontemporal_store(x, dst);
         }
         else
         {
-            float x;
+            E x;
             if constexpr (NBITS == 1)
                 x = ((word[0] >> sh) & 1u) ? val1 : val0;
             else
-                x = unquantize_value<NBITS>(vq, (word[0] >> sh) & CODEMASK);
+                x = unquantize_value<NBITS>(vq, (word[0] >> sh) & PS::CODEMASK);
             if (add)
                 x = x + oc[i];
             oc[i] = x;
@@ -145,8 +144,8 @@ __device__ __forceinline__ void unquantize_body(const char* __restrict__ q, floa
     }
 }
 
-template <int NBITS, int WV>
-__global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, float* out, UnqGeom t, int add)
+template <int NBITS, int WV, typename E>
+__global__ __launch_bounds__(256) void unquantize_kernel(const char* __restrict__ q, E* out, UnqGeom t, int add)
 {
     unquantize_body<NBITS, WV>(q, out, t, add, blockIdx.x);
 }

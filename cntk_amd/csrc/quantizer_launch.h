@@ -1028,9 +1028,9 @@ inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const c
     else if (p.kind == kUnqSegment)
         hipExtLaunchKernelGGL((unquantize_segment_kernel<NBITS>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.seg, add);
     else if (p.kind == kUnqVec4)
-        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 4>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.qw, add);
+        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 4, float>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.qw, add);
     else
-        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 1>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.qw, add);
+        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 1, float>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.qw, add);
     return hipGetLastError();
 }
 

@@ -349,9 +349,9 @@ inline hipError_t launch_unquantize_n(hipStream_t s, LaunchEvents ev, const char
 {
     const uint32_t blocks = (uint32_t) (((uint64_t) t.items + 255) / 256);
     if (vec)
-        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 2>), dim3(blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, t, add);
+        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 2, double>), dim3(blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, t, add);
     else
-        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 1>), dim3(blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, t, add);
+        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 1, double>), dim3(blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, t, add);
     return hipGetLastError();
 }
 
