@@ -434,105 +434,7 @@ __global__ __launch_bounds__(kThreads) void stripe_reduce_tile_kernel(StripeSour
 //
 // A 16-byte store holds two doubles; QWords are 64-bit; a packed record is nq + 2 QWords (lower, upper, bits).
 
-template <int NBITS>
-__device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q, double* out, const UnqRowGeom& t, int add, uint32_t block,
-                                                     uint64_t* words)
-{
-    using PS = PackShape<NBITS>;
-    const uint32_t tid = threadIdx.x;
-    uint32_t c, ch;
-    unq_rows_block_to_chunk(block, t.chunks, t.blocks, c, ch);
-    const char* qc = q + (size_t) c * t.qcol;
-    const double* gh = reinterpret_cast<const double*>(qc);
-    const ValueQ vq = make_vq<NBITS>(gh[0], gh[1]);
-    const uint64_t* bits = reinterpret_cast<const uint64_t*>(qc + 16);
-    for (uint32_t w = tid; w < t.nq; w += 4 * 256)
-    {
-        uint64_t v[4];
-#pragma unroll
-        for (uint32_t u = 0; u < 4; ++u)
-            v[u] = bits[(w + 256 * u < t.nq) ? w + 256 * u : w];
-#pragma unroll
-        for (uint32_t u = 0; u < 4; ++u)
-            if (w + 256 * u < t.nq)
-                words[w + 256 * u] = v[u];
-    }
-    __syncthreads();
-    // any height, any (8-byte) alignment: one row may lie before the column's first aligned pair and one after its last;
-    // the first chunk's workgroup writes the former, the last one's the latter
-    double* oc = out + (size_t) c * t.rows;
-    const uint32_t head = (uint32_t) ((reinterpret_cast<uintptr_t>(oc) >> 3) & 1u);
-    const uint32_t body = (t.rows - head) & ~1u;
-    const uint32_t tail = t.rows - head - body;
-    const uint32_t r0 = ch * t.chunk;
-    const uint32_t pieces = ((ch + 1 == t.chunks ? body : r0 + t.chunk) - r0) >> 1; // the last chunk runs to the end
-    f64x2* o2 = reinterpret_cast<f64x2*>(oc + head + r0);
-    const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
-    const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
-    {
-        uint32_t row = t.rows; // none
-        if (ch == 0 && tid < head)
-            row = 0;
-        else if (ch + 1 == t.chunks && tid == 1 && tail != 0)
-            row = t.rows - 1;
-        if (row < t.rows)
-        {
-            const uint32_t k = row / t.nq;
-            const uint64_t code = (words[row - k * t.nq] >> (k * PS::SHIFT)) & PS::CODEMASK;
-            double x;
-            if constexpr (NBITS == 1)
-                x = code ? val1 : val0;
-            else
-                x = unquantize_value<NBITS>(vq.uf, vq.lo, code);
-            oc[row] = add ? x + oc[row] : x;
-        }
-    }
-    // slots dealt by 128-byte lines, as in the fp32 decoder
-    const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o2) >> 4) & 7u);
-    const uint32_t vfirst = tid < shift ? tid + 256 : tid;
-    // row i sits in QWord i % nq at bit position i / nq; a thread's pieces are 512 rows apart
-    const uint32_t i0 = head + r0 + 2 * (vfirst - shift);
-    uint32_t k0 = i0 / t.nq;
-    uint32_t w0 = i0 - k0 * t.nq;
-    const uint32_t dk = 512u / t.nq;
-    const uint32_t dw = 512u - dk * t.nq;
-    for (uint32_t p = vfirst - shift; p < pieces; p += 256)
-    {
-        uint32_t k = k0, w = w0;
-        f64x2 x;
-#pragma unroll
-        for (int e = 0; e < 2; ++e)
-        {
-            const uint64_t code = (words[w] >> (k * PS::SHIFT)) & PS::CODEMASK;
-            if constexpr (NBITS == 1)
-                x[e] = code ? val1 : val0;
-            else
-                x[e] = unquantize_value<NBITS>(vq.uf, vq.lo, code);
-            if (++w == t.nq)
-            {
-                w = 0;
-                ++k;
-            }
-        }
-        if (add)
-            x = x + o2[p]; // unquantized value + previous content
-        __builtin_nontemporal_store(x, o2 + p);
-        k0 += dk;
-        w0 += dw;
-        if (w0 >= t.nq)
-        {
-            w0 -= t.nq;
-            ++k0;
-        }
-    }
-}
-
-template <int NBITS>
-__global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __restrict__ q, double* out, UnqRowGeom t, int add)
-{
-    extern __shared__ f32x4 smem_v4[];
-    unquantize_rows_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint64_t*>(smem_v4));
-}
+// (the row-major decoder, unquantize_rows_body / unquantize_rows_kernel, is the fp32 source, written over the element type)
 
 template <int NBITS>
 __device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q, double* out, const UnqTileGeom& t, int add, uint32_t block,

@@ -264,20 +264,23 @@ __device__ __forceinline__ void unq_rows_block_to_chunk(uint32_t block, uint32_t
     }
 }
 
-template <int NBITS>
-__device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q, float* out, const UnqRowGeom& t, int add, uint32_t block,
-                                                     uint32_t* words)
+// Written over the element type: N = 4 floats or 2 doubles per 16-byte store; `words` holds the column's QWords.
+template <int NBITS, typename E>
+__device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q, E* out, const UnqRowGeom& t, int add, uint32_t block,
+                                                     typename Word<E>::Q* words)
 {
-    constexpr uint32_t SHIFT = NBITS & 31;
-    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
+    typedef typename Word<E>::Q QWord;
+    using PS = PackShapeOf<NBITS, Word<E>::kBits>;
+    constexpr uint32_t N = 16 / sizeof(E);
+    typedef E Vec __attribute__((ext_vector_type(N)));
     const uint32_t tid = threadIdx.x;
     uint32_t c, ch;
     unq_rows_block_to_chunk(block, t.chunks, t.blocks, c, ch);
     const char* qc = q + (size_t) c * t.qcol;
-    const float* gh = reinterpret_cast<const float*>(qc);
-    const float lo = gh[0];
-    const float uf = make_ufactor<NBITS>(lo, gh[1]);
-    const uint32_t* bits = reinterpret_cast<const uint32_t*>(qc + 8);
+    const E* gh = reinterpret_cast<const E*>(qc);
+    const E lo = gh[0];
+    const E uf = make_ufactor<NBITS>(lo, gh[1]);
+    const QWord* bits = reinterpret_cast<const QWord*>(qc + 2 * sizeof(E));
     if (t.nq <= 1024)
     {
         for (uint32_t w = tid; w < t.nq; w += 256)
@@ -289,7 +292,7 @@ __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q,
         // them would cost more than the decoding
         for (uint32_t w = tid; w < t.nq; w += 8 * 256)
         {
-            uint32_t v[8];
+            QWord v[8];
 #pragma unroll
             for (uint32_t u = 0; u < 8; ++u)
                 v[u] = bits[(w + 256 * u < t.nq) ? w + 256 * u : w];
@@ -300,29 +303,29 @@ __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q,
         }
     }
     __syncthreads();
-    // The column need not start on a 16-byte boundary nor hold a multiple of 4 rows: `head` rows (0..3) lie before its
-    // first aligned group of four and `tail` rows (0..3) after the last; chunks are counted from the first aligned row,
+    // The column need not start on a 16-byte boundary nor hold a multiple of N rows: `head` rows (0..N-1) lie before its
+    // first aligned group of N and `tail` rows (0..N-1) after the last; chunks are counted from the first aligned row,
     // the first chunk's workgroup also writes the head rows, the last one's the tail rows, one row per thread.
-    float* oc = out + (size_t) c * t.rows;
-    const uint32_t head = (4u - (uint32_t) ((reinterpret_cast<uintptr_t>(oc) >> 2) & 3u)) & 3u;
-    const uint32_t body = (t.rows - head) & ~3u; // rows in aligned groups of four
+    E* oc = out + (size_t) c * t.rows;
+    const uint32_t head = (N - (uint32_t) ((reinterpret_cast<uintptr_t>(oc) / sizeof(E)) & (N - 1))) & (N - 1);
+    const uint32_t body = (t.rows - head) & ~(N - 1); // rows in aligned groups of N
     const uint32_t tail = t.rows - head - body;
     const uint32_t r0 = ch * t.chunk;
-    const uint32_t pieces = ((ch + 1 == t.chunks ? body : r0 + t.chunk) - r0) >> 2; // the last chunk runs to the end
-    f32x4* o4 = reinterpret_cast<f32x4*>(oc + head + r0);
-    const float val0 = unquantize_value<NBITS>(uf, lo, 0u);
-    const float val1 = unquantize_value<NBITS>(uf, lo, 1u);
+    const uint32_t pieces = ((ch + 1 == t.chunks ? body : r0 + t.chunk) - r0) / N; // the last chunk runs to the end
+    Vec* o4 = reinterpret_cast<Vec*>(oc + head + r0);
+    const E val0 = unquantize_value<NBITS>(uf, lo, 0u);
+    const E val1 = unquantize_value<NBITS>(uf, lo, 1u);
     {
         uint32_t row = t.rows; // none
         if (ch == 0 && tid < head)
             row = tid;
-        else if (ch + 1 == t.chunks && tid >= 4 && tid < 4 + tail)
-            row = head + body + (tid - 4);
+        else if (ch + 1 == t.chunks && tid >= N && tid < N + tail)
+            row = head + body + (tid - N);
         if (row < t.rows)
         {
             const uint32_t k = row / t.nq;
-            const uint32_t code = (words[row - k * t.nq] >> (k * SHIFT)) & CODEMASK;
-            float x;
+            const QWord code = (words[row - k * t.nq] >> (k * PS::SHIFT)) & PS::CODEMASK;
+            E x;
             if constexpr (NBITS == 1)
                 x = code ? val1 : val0;
             else
@@ -334,20 +337,20 @@ __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q,
     // that every wavefront's 64 stores cover whole lines also where columns do not start on one (9304 rows).
     const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o4) >> 4) & 7u);
     const uint32_t vfirst = tid < shift ? tid + 256 : tid;
-    // row i sits in QWord i % nq at bit position i / nq; a thread's pieces are 1024 rows apart
-    const uint32_t i0 = head + r0 + 4 * (vfirst - shift);
+    // row i sits in QWord i % nq at bit position i / nq; a thread's pieces are 256 * N rows apart
+    const uint32_t i0 = head + r0 + N * (vfirst - shift);
     uint32_t k0 = i0 / t.nq;
     uint32_t w0 = i0 - k0 * t.nq;
-    const uint32_t dk = 1024u / t.nq;
-    const uint32_t dw = 1024u - dk * t.nq;
+    const uint32_t dk = (256u * N) / t.nq;
+    const uint32_t dw = 256u * N - dk * t.nq;
     for (uint32_t p = vfirst - shift; p < pieces; p += 256)
     {
         uint32_t k = k0, w = w0;
-        f32x4 x;
+        Vec x;
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
+        for (uint32_t e = 0; e < N; ++e)
         {
-            const uint32_t code = (words[w] >> (k * SHIFT)) & CODEMASK;
+            const QWord code = (words[w] >> (k * PS::SHIFT)) & PS::CODEMASK;
             if constexpr (NBITS == 1)
                 x[e] = code ? val1 : val0;
             else
@@ -371,11 +374,11 @@ __device__ __forceinline__ void unquantize_rows_body(const char* __restrict__ q,
     }
 }
 
-template <int NBITS>
-__global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __restrict__ q, float* out, UnqRowGeom t, int add)
+template <int NBITS, typename E>
+__global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __restrict__ q, E* out, UnqRowGeom t, int add)
 {
     extern __shared__ f32x4 smem_v4[];
-    unquantize_rows_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint32_t*>(smem_v4));
+    unquantize_rows_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<typename Word<E>::Q*>(smem_v4));
 }
 
 // Tile decoder for short columns. Consecutive columns are adjacent in the packed matrix and in the output, so a

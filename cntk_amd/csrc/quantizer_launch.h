@@ -1024,7 +1024,7 @@ inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const c
     if (p.kind == kUnqTile)
         hipExtLaunchKernelGGL((unquantize_tile_kernel<NBITS>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.tile, add);
     else if (p.kind == kUnqRows)
-        hipExtLaunchKernelGGL((unquantize_rows_kernel<NBITS>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.rowg, add);
+        hipExtLaunchKernelGGL((unquantize_rows_kernel<NBITS, float>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.rowg, add);
     else if (p.kind == kUnqSegment)
         hipExtLaunchKernelGGL((unquantize_segment_kernel<NBITS>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.seg, add);
     else if (p.kind == kUnqVec4)

@@ -362,7 +362,7 @@ constexpr size_t kUnqTileElems64 = 2048;   // values per workgroup the tile deco
 template <int NBITS>
 inline hipError_t launch_unquantize_rows(hipStream_t s, LaunchEvents ev, const char* q, double* out, const UnqRowGeom& t, int add)
 {
-    hipExtLaunchKernelGGL((unquantize_rows_kernel<NBITS>), dim3(t.blocks), dim3(256), (size_t) t.nq * 8, s, ev.start, ev.stop, 0, q, out, t, add);
+    hipExtLaunchKernelGGL((unquantize_rows_kernel<NBITS, double>), dim3(t.blocks), dim3(256), (size_t) t.nq * 8, s, ev.start, ev.stop, 0, q, out, t, add);
     return hipGetLastError();
 }
 
