@@ -430,100 +430,9 @@ __global__ __launch_bounds__(kThreads) void stripe_reduce_tile_kernel(StripeSour
 // The QWord-major decoder (UnqGeom, unquantize_body, unquantize_kernel) is the fp32 source, written over the element type:
 // two QWords and two rows per thread and bit position where rows and QWords per column are even, else one.
 
-// ---- row-major and tile decoders (the fp32 unquantize_rows_kernel / unquantize_tile_kernel on doubles) ---------
-//
-// A 16-byte store holds two doubles; QWords are 64-bit; a packed record is nq + 2 QWords (lower, upper, bits).
+// The row-major decoder (unquantize_rows_kernel) and the tile decoder (unquantize_tile_kernel) are the fp32 sources too: a
+// 16-byte store holds two doubles, QWords are 64-bit, a packed record is nq + 2 QWords (lower, upper, bits).
 
-// (the row-major decoder, unquantize_rows_body / unquantize_rows_kernel, is the fp32 source, written over the element type)
-
-template <int NBITS>
-__device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q, double* out, const UnqTileGeom& t, int add, uint32_t block,
-                                                     uint64_t* words)
-{
-    using PS = PackShape<NBITS>;
-    double* dec = reinterpret_cast<double*>(words + t.cpt * t.rec_words); // per column: the two levels (1 bit) or (ufactor, lower)
-    const uint32_t tid = threadIdx.x;
-    const uint32_t col0 = block * t.cpt;
-    const uint32_t ncols = (t.cols - col0 < t.cpt) ? t.cols - col0 : t.cpt;
-    const uint64_t* src = reinterpret_cast<const uint64_t*>(q + (size_t) col0 * t.rec_words * 8);
-    const uint32_t total_words = ncols * t.rec_words;
-    for (uint32_t x = tid; x < total_words; x += 256)
-        words[x] = __builtin_nontemporal_load(src + x);
-    __syncthreads();
-    for (uint32_t c = tid; c < ncols; c += 256)
-    {
-        const double lo = __longlong_as_double((long long) words[c * t.rec_words]);
-        const double hi = __longlong_as_double((long long) words[c * t.rec_words + 1]);
-        const ValueQ vq = make_vq<NBITS>(lo, hi);
-        if constexpr (NBITS == 1)
-        {
-            dec[2 * c] = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
-            dec[2 * c + 1] = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
-        }
-        else
-        {
-            dec[2 * c] = vq.uf;
-            dec[2 * c + 1] = vq.lo;
-        }
-    }
-    __syncthreads();
-    const uint32_t elems = ncols * t.rows;
-    double* o = out + (size_t) col0 * t.rows;
-    // slots dealt by 128-byte lines, as in the fp32 decoder
-    const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o) >> 4) & 7u);
-    for (uint32_t i = 2 * ((tid < shift ? tid + 256 : tid) - shift); i < elems; i += 512)
-    {
-        uint32_t c = small_div(i, t.rows, t.rows_magic);
-        uint32_t r = i - c * t.rows;
-        uint32_t k = small_div(r, t.nq, t.nq_magic);
-        uint32_t w = r - k * t.nq;
-        const uint64_t* cw = words + c * t.rec_words + 2;
-        double d0 = dec[2 * c], d1 = dec[2 * c + 1];
-        f64x2 x;
-#pragma unroll
-        for (int e = 0; e < 2; ++e)
-        {
-            // (past the end of the matrix the reads stay inside the LDS block and the value is not stored)
-            const uint64_t code = (cw[w] >> (k * PS::SHIFT)) & PS::CODEMASK;
-            if constexpr (NBITS == 1)
-                x[e] = code ? d1 : d0;
-            else
-                x[e] = unquantize_value<NBITS>(d0, d1, code);
-            ++r;
-            if (++w == t.nq)
-            {
-                w = 0;
-                ++k;
-            }
-            if (r == t.rows)
-            {
-                r = 0;
-                k = 0;
-                w = 0;
-                c = (c + 1 < t.cpt) ? c + 1 : c;
-                cw = words + c * t.rec_words + 2;
-                d0 = dec[2 * c];
-                d1 = dec[2 * c + 1];
-            }
-        }
-        if (i + 2 <= elems)
-        {
-            f64x2* o2 = reinterpret_cast<f64x2*>(o + i);
-            if (add)
-                x = x + *o2; // unquantized value + previous content
-            __builtin_nontemporal_store(x, o2);
-        }
-        else
-            o[i] = add ? x[0] + o[i] : x[0];
-    }
-}
-
-template <int NBITS>
-__global__ __launch_bounds__(256) void unquantize_tile_kernel(const char* __restrict__ q, double* out, UnqTileGeom t, int add)
-{
-    extern __shared__ f32x4 smem_v4[];
-    unquantize_tile_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint64_t*>(smem_v4));
-}
 
 // ---- one workgroup per column, the column in registers (the fp32 quantize_reg_kernel on doubles) ------------
 //

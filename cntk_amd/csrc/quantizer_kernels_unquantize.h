@@ -392,7 +392,7 @@ struct UnqTileGeom
     uint32_t cols;
     uint32_t nq;
     uint32_t cpt;        // columns per workgroup
-    uint32_t rec_words;  // nq + 2: 32-bit words per packed record
+    uint32_t rec_words;  // nq + 2: QWords per packed record (lower, upper, bits)
     uint32_t rows_magic; // ceil(2^32 / rows) (unused when rows == 1)
     uint32_t nq_magic;   // ceil(2^32 / nq) (unused when nq == 1)
     uint32_t blocks;
@@ -409,27 +409,31 @@ __device__ __forceinline__ uint32_t small_div(uint32_t x, uint32_t d, uint32_t m
     return d == 1 ? x : __umulhi(x, magic);
 }
 
-template <int NBITS>
-__device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q, float* out, const UnqTileGeom& t, int add, uint32_t block,
-                                                     uint32_t* smem)
+// Written over the element type: N = 4 floats or 2 doubles per 16-byte store; a packed record is rec_words QWords
+// (lower, upper, bits), and smem holds cpt records and two decode constants per column.
+template <int NBITS, typename E>
+__device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q, E* out, const UnqTileGeom& t, int add, uint32_t block,
+                                                     typename Word<E>::Q* smem)
 {
-    constexpr uint32_t SHIFT = NBITS & 31;
-    constexpr uint32_t CODEMASK = (NBITS >= 32) ? 0xFFFFFFFFu : ((1u << SHIFT) - 1u);
+    typedef typename Word<E>::Q QWord;
+    using PS = PackShapeOf<NBITS, Word<E>::kBits>;
+    constexpr uint32_t N = 16 / sizeof(E);
+    typedef E Vec __attribute__((ext_vector_type(N)));
     const uint32_t tid = threadIdx.x;
     const uint32_t col0 = block * t.cpt;
     const uint32_t ncols = (t.cols - col0 < t.cpt) ? t.cols - col0 : t.cpt;
-    uint32_t* words = smem;                                          // ncols packed records
-    float* dec = reinterpret_cast<float*>(smem + t.cpt * t.rec_words); // per column: the two levels (1 bit) or (ufactor, lower)
-    const uint32_t* src = reinterpret_cast<const uint32_t*>(q + (size_t) col0 * t.rec_words * 4);
+    QWord* words = smem;                                        // ncols packed records
+    E* dec = reinterpret_cast<E*>(smem + t.cpt * t.rec_words); // per column: the two levels (1 bit) or (ufactor, lower)
+    const QWord* src = reinterpret_cast<const QWord*>(q + (size_t) col0 * t.rec_words * sizeof(QWord));
     const uint32_t total_words = ncols * t.rec_words;
     for (uint32_t x = tid; x < total_words; x += 256)
         words[x] = __builtin_nontemporal_load(src + x);
     __syncthreads();
     for (uint32_t c = tid; c < ncols; c += 256)
     {
-        const float lo = __uint_as_float(words[c * t.rec_words]);
-        const float hi = __uint_as_float(words[c * t.rec_words + 1]);
-        const float uf = make_ufactor<NBITS>(lo, hi);
+        const E lo = Word<E>::value_of(words[c * t.rec_words]);
+        const E hi = Word<E>::value_of(words[c * t.rec_words + 1]);
+        const E uf = make_ufactor<NBITS>(lo, hi);
         if constexpr (NBITS == 1)
         {
             dec[2 * c] = unquantize_value<NBITS>(uf, lo, 0u);
@@ -443,24 +447,24 @@ __device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q,
     }
     __syncthreads();
     const uint32_t elems = ncols * t.rows;
-    float* o = out + (size_t) col0 * t.rows;
-    // slots dealt by 128-byte lines: slot v = tid, tid + 256, ... holds the group of four that starts at element
-    // 4 * (v - shift), shift = the tile's offset into its line in 16-byte pieces
+    E* o = out + (size_t) col0 * t.rows;
+    // slots dealt by 128-byte lines: slot v = tid, tid + 256, ... holds the group of N that starts at element
+    // N * (v - shift), shift = the tile's offset into its line in 16-byte pieces
     const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o) >> 4) & 7u);
-    for (uint32_t i = 4 * ((tid < shift ? tid + 256 : tid) - shift); i < elems; i += 1024)
+    for (uint32_t i = N * ((tid < shift ? tid + 256 : tid) - shift); i < elems; i += 256 * N)
     {
         uint32_t c = small_div(i, t.rows, t.rows_magic);
         uint32_t r = i - c * t.rows;
         uint32_t k = small_div(r, t.nq, t.nq_magic);
         uint32_t w = r - k * t.nq;
-        const uint32_t* cw = words + c * t.rec_words + 2;
-        float d0 = dec[2 * c], d1 = dec[2 * c + 1];
-        f32x4 x;
+        const QWord* cw = words + c * t.rec_words + 2;
+        E d0 = dec[2 * c], d1 = dec[2 * c + 1];
+        Vec x;
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
+        for (uint32_t e = 0; e < N; ++e)
         {
             // (past the end of the matrix c == ncols: the reads stay inside the LDS block and the value is not stored)
-            const uint32_t code = (cw[w] >> (k * SHIFT)) & CODEMASK;
+            const QWord code = (cw[w] >> (k * PS::SHIFT)) & PS::CODEMASK;
             if constexpr (NBITS == 1)
                 x[e] = code ? d1 : d0;
             else
@@ -482,9 +486,9 @@ __device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q,
                 d1 = dec[2 * c + 1];
             }
         }
-        if (i + 4 <= elems)
+        if (i + N <= elems)
         {
-            f32x4* o4 = reinterpret_cast<f32x4*>(o + i);
+            Vec* o4 = reinterpret_cast<Vec*>(o + i);
             if (add)
                 x = x + *o4; // unquantized value + previous content
             __builtin_nontemporal_store(x, o4);
@@ -497,11 +501,11 @@ __device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q,
     }
 }
 
-template <int NBITS>
-__global__ __launch_bounds__(256) void unquantize_tile_kernel(const char* __restrict__ q, float* out, UnqTileGeom t, int add)
+template <int NBITS, typename E>
+__global__ __launch_bounds__(256) void unquantize_tile_kernel(const char* __restrict__ q, E* out, UnqTileGeom t, int add)
 {
     extern __shared__ f32x4 smem_v4[];
-    unquantize_tile_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<uint32_t*>(smem_v4));
+    unquantize_tile_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<typename Word<E>::Q*>(smem_v4));
 }
 
 } // namespace cntkq

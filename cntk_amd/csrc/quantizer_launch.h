@@ -1022,7 +1022,7 @@ template <int NBITS>
 inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const char* q, float* out, const UnquantizePlan& p, int add)
 {
     if (p.kind == kUnqTile)
-        hipExtLaunchKernelGGL((unquantize_tile_kernel<NBITS>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.tile, add);
+        hipExtLaunchKernelGGL((unquantize_tile_kernel<NBITS, float>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.tile, add);
     else if (p.kind == kUnqRows)
         hipExtLaunchKernelGGL((unquantize_rows_kernel<NBITS, float>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.rowg, add);
     else if (p.kind == kUnqSegment)

@@ -369,7 +369,7 @@ inline hipError_t launch_unquantize_rows(hipStream_t s, LaunchEvents ev, const c
 template <int NBITS>
 inline hipError_t launch_unquantize_tile(hipStream_t s, LaunchEvents ev, const char* q, double* out, const UnqTileGeom& t, int add)
 {
-    hipExtLaunchKernelGGL((unquantize_tile_kernel<NBITS>), dim3(t.blocks), dim3(256), (size_t) t.cpt * (t.rec_words + 2) * 8, s, ev.start,
+    hipExtLaunchKernelGGL((unquantize_tile_kernel<NBITS, double>), dim3(t.blocks), dim3(256), (size_t) t.cpt * (t.rec_words + 2) * 8, s, ev.start,
                           ev.stop, 0, q, out, t, add);
     return hipGetLastError();
 }
