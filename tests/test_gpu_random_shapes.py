@@ -24,9 +24,16 @@ def say(*a):
     sys.stdout.flush()
 
 
-def draw_case(rng, is64):
+TALL = [102401, 110000, 131072, 131073, 147456, 200000, 262144, 262145, 300001, 524288, 524289, 600000]
+
+
+def draw_case(rng, is64, tall=False):
     r = rng.random()
-    if r < 0.5:
+    if tall:
+        # above what one workgroup holds: strips of a column on several workgroups (up to 64 of them), then the kernel that
+        # re-reads its column
+        rows = int(rng.choice(TALL)) if r < 0.6 else int(rng.integers(102401, 540000))
+    elif r < 0.5:
         rows = int(rng.choice(BOUNDARIES))
     elif r < 0.8:
         rows = int(rng.integers(1, 3000))
@@ -53,15 +60,16 @@ def place(a, off, tdt):
     return Matrix(a.shape[0], a.shape[1], 0, buf[off:off + n], dtype=tdt), buf
 
 
-@pytest.mark.parametrize("dtype,seed,count", [("f32", 11, 150), ("f32", 12, 150), ("f64", 13, 120), ("f64", 14, 120)])
-def test_random_shapes(dtype, seed, count):
+@pytest.mark.parametrize("dtype,seed,count,tall", [("f32", 11, 150, False), ("f32", 12, 150, False), ("f64", 13, 120, False), ("f64", 14, 120, False),
+                                                   ("f32", 15, 40, True), ("f64", 16, 12, True)])
+def test_random_shapes(dtype, seed, count, tall):
     is64 = dtype == "f64"
     ndt, tdt = (np.float64, torch.float64) if is64 else (np.float32, torch.float32)
     rng = np.random.default_rng(seed)
     qz = MatrixQuantizerImpl.Create(0, False)
     rep = parity.Report()
     for n in range(count):
-        rows, cols, nbits, zt, offs, in_place = draw_case(rng, is64)
+        rows, cols, nbits, zt, offs, in_place = draw_case(rng, is64, tall)
         say("random case", dtype, seed, n, "rows", rows, "cols", cols, "nbits", nbits, "zeroThr", zt, "offsets", offs, "in place", in_place)
         g = datagen.normal_with_outliers(seed * 1000 + n, rows, cols, 0.01, dtype=ndt)
         r = datagen.normal(seed * 2000 + n, rows, cols, 0.002, dtype=ndt)
