@@ -4,23 +4,25 @@
 // of W consecutive QWords with ALL their bit positions: 32 / NBITS runs of W consecutive elements, nq elements apart. One
 // 256-thread workgroup owns one strip: a thread holds four consecutive QWords' elements at up to eight bit positions (32
 // values: eight 16-byte loads of gradient and residual, at any 4-byte alignment), builds its part of the four QWords and
-// writes the residual back from registers; the parts of a QWord meet in LDS. Gradient and residual are read once and the
-// strip needs 1 KB of LDS and 64 registers whatever the height, so eight workgroups share a CU and their load, statistics
-// and store phases interleave -- what the one-workgroup-per-column kernels lose above 14336 rows, where a column fills a CU
-// by itself (100000 x 512: 67 % of peak), and what columns above 102400 rows, which no workgroup's registers hold, could
-// only have by reading their inputs two or three times.
+// writes the residual back from registers; the parts of a QWord meet in LDS. Gradient and residual are read once whatever
+// the height, which columns above 102400 rows -- more than any workgroup's registers hold -- could otherwise only have by
+// reading their inputs two or three times. A strip needs 1 to 4 KB of LDS and, at 1 to 4 bits, some 100 registers (its 32
+// values, their addresses, the masks of the ragged last strip), so five workgroups share a CU; it is the exchange
+// described next, not memory, that bounds the kernel (about 3 TB/s), and below 102400 rows the kernels with one workgroup
+// per column are faster.
 //
 // The column statistics span the strips of a column. Every workgroup publishes its partial sums in a scratch buffer, one
 // 8-byte record per sum: the value and the tag of the launch, written by one atomic store, so that whoever reads the tag
 // of this launch has the value with it and no second word needs ordering against the first. Then the first wavefront of
-// every workgroup of the column polls the S records (a lane per record) until all carry the tag, and adds them in strip
-// order -- one fixed order, the same bytes in every workgroup. One exchange for the sum of squares (more than 1 bit) or
+// every workgroup of the column polls the S records (a lane per record) until all carry the tag, and adds them up, lanes
+// meeting by butterfly -- one fixed order, the same bytes in every workgroup. One exchange for the sum of squares (more than 1 bit) or
 // the split sums (1 bit against 0), two for 1 bit against the mean (mean, then split sums). The tag is a launch count
 // kept in the scratch buffer itself: every workgroup reads it when it starts, and the last workgroup to finish (a second
-// counter tells) raises it, so that replays of a recorded graph see fresh tags like any other launch. The workgroups of a
-// column are adjacent in the grid, hence dispatched together; a workgroup only ever waits for workgroups of lower or
-// adjacent index, which are running or next in line. The wait is bounded all the same: after `spin_limit` polls a lane
-// gives up, raises the error word and goes on with whatever the record holds, so that the grid always drains.
+// counter tells) raises it, so that replays of a recorded graph see fresh tags like any other launch. The strips of a
+// column take workgroup indices 8 apart: the device's eight dies take the workgroups of a grid in turn, so a column's
+// strips run on one die, next to each other in its queue, and start together (at most 64 of them: all must be resident
+// at once). The wait is bounded all the same: after `spin_limit` polls a lane gives up, raises the error word and goes on
+// with whatever the record holds, so that the grid always drains.
 #pragma once
 
 #include "quantizer_kernels_common.h"
@@ -38,7 +40,8 @@ struct StripShape
     static constexpr uint32_t CHUNKS = PS::CHUNKS;                // threads per QWord quad
     static constexpr uint32_t QUADS = kStripThreads / CHUNKS;     // quads of four QWords per strip
     static constexpr uint32_t WORDS = 4 * QUADS;                  // QWords per strip: 256, 512, 1024, 1024, 1024 at 1, 2, 4, 8, 16 bits
-    // wavefronts per SIMD the kernels are compiled for (the registers that leaves them: 80 at 6, 64 at 8), without spills
+    // wavefronts per SIMD the kernels are compiled for (the registers that leaves them: 96 at 5, 64 at 8); with more at 1 to 4
+    // bits the ragged last strip spills, and every strip of its column waits for it
     static constexpr uint32_t WAVES = NBITS <= 4 ? 5 : 8;
 };
 
@@ -59,8 +62,9 @@ struct StripGeom
     uint64_t qcol;
 };
 
-// Scratch of one launch stream: a header, the finish counters, then four records per (column, strip): the statistic, then the two split sums
-// and the count below the threshold. The buffer starts zeroed; tags start at 1.
+// Scratch of one launch stream: a header, the finish counters, then four records per (column, strip): the statistic, then
+// the two split sums and the count below the threshold. The buffer starts zeroed; tags start at 1.
+//
 // Reads of one address take their turns like atomic operations on it (a few nanoseconds each, but thousands of workgroups
 // start within microseconds), so the launch count is kept in 256 copies, 256 bytes apart, and a wavefront reads the copy
 // its index selects.
@@ -170,8 +174,8 @@ __device__ __forceinline__ uint32_t strip_block_sum(uint32_t v, uint32_t* red)
     return t;
 }
 
-// The column's statistic from the strip's: every workgroup of the column publishes its own and adds all of them in strip
-// order. red: the workgroup's reduction slots. Every thread returns the same bits, in every workgroup of the column.
+// The column's statistic from the strip's: every workgroup of the column publishes its own and adds all of them in the
+// order of strip_collect. red: the workgroup's reduction slots. Every thread returns the same bits, in every workgroup of the column.
 __device__ __forceinline__ float strip_exchange_stat(float stat, uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
                                                      const StripScratch& scratch, float* red)
 {
