@@ -84,6 +84,19 @@ struct BatchAbi<float>
                 e.kind = it.rows == 1024 ? 2 : (it.rows == 2048 ? 3 : 4);
                 lds = it.rows == 1024 ? col_lds_bytes<1>() : (it.rows == 2048 ? col_lds_bytes<2>() : col_lds_bytes<4>());
             }
+            else if (path == kPathReg && e.kind == 1)
+            {
+                // what the plain call runs for this matrix, where a thread holds at most 6 pieces (6144 rows): the column in
+                // registers, with the slots dealt as the plain call deals them (same bytes as the LDS body either way)
+                const RegGeom r = make_reg_geom(it.rows, nbits, kTileThreads, line_shift);
+                const uint32_t per = (r.pieces + (r.line_shift ? 7u : 0u) + kTileThreads - 1) / kTileThreads;
+                if (per <= 6)
+                {
+                    e.kind = per <= 3 ? 6 : 7;
+                    e.r = r;
+                    lds = reg_lds_bytes(r);
+                }
+            }
             return true;
         }
         return false;

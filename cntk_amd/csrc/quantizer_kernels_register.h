@@ -222,18 +222,17 @@ __device__ __forceinline__ void reg_stats_pack(f32x4 (&a)[PER], float edge, bool
 // first aligned piece and up to 3 after the last are held, one each, by threads 0..5 and take part in every phase after
 // the thread's pieces. (c.pieces then only bounds the pieces; the count is taken from the column's address.)
 template <int NBITS, bool ZT, int T, int PER, bool EDGE = false>
-__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, PER>(), reg_waves<T, PER>()))) void quantize_reg_kernel(
-    const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q, RegGeom c)
+__device__ __forceinline__ void quantize_reg_body(const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q, const RegGeom& c,
+                                                  uint32_t column, f32x4* smem_v4)
 {
     static_assert(NBITS < 32, "32-bit codes are whole QWords: nothing to assemble");
     constexpr uint32_t NW = T / 64;
-    extern __shared__ f32x4 smem_v4[];
     float* red = reinterpret_cast<float*>(smem_v4);
     uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
     uint32_t* words = reinterpret_cast<uint32_t*>(red + kRegRedSlots);
     const uint32_t tid = threadIdx.x;
-    const size_t base = (size_t) blockIdx.x * c.rows;
-    char* qc = q + (size_t) blockIdx.x * c.qcol;
+    const size_t base = (size_t) column * c.rows;
+    char* qc = q + (size_t) column * c.qcol;
     for (uint32_t x = tid; x < c.nq; x += T)
         words[x] = 0u;
     uint32_t head = 0, tail = 0, pieces = c.pieces;
@@ -277,6 +276,14 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
             a[u] = a[u] + b[u - u0];
     }
     reg_stats_pack<NBITS, ZT, T, PER>(a, edge, has_edge, edge_at, head, pieces, shift, c, red, red_u, words, r_out + base, qc);
+}
+
+template <int NBITS, bool ZT, int T, int PER, bool EDGE = false>
+__global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, PER>(), reg_waves<T, PER>()))) void quantize_reg_kernel(
+    const float* __restrict__ g, const float* r_in, float* r_out, char* __restrict__ q, RegGeom c)
+{
+    extern __shared__ f32x4 smem_v4[];
+    quantize_reg_body<NBITS, ZT, T, PER, EDGE>(g, r_in, r_out, q, c, blockIdx.x, smem_v4);
 }
 
 // Stripe reduction for tall columns (above the LDS kernels' 14336 rows), in the register kernel's shape: 1024 threads per
