@@ -22,7 +22,10 @@ def say(*a):
 
 MIXED = [(147, 64), (64, 64), (576, 64), (64, 256), (1, 5), (5, 1), (429, 37), (2048, 33), (2304, 5), (4608, 3), (9304, 1),
          (2048, 1), (0, 4), (1000, 1), (1152, 128), (4096, 6), (20000, 2), (512, 100), (33, 67), (14336, 1), (2048, 1100),
-         (1028, 9), (12000, 2)]
+         (1028, 9), (12000, 2),
+         # columns held in registers inside the shared launch, some starting inside a 128-byte line, up to the last height
+         # that fits six pieces per thread and just past it
+         (4100, 7), (5000, 3), (6116, 2), (6144, 2), (6148, 2), (3072, 4)]
 
 
 @pytest.mark.parametrize("nbits,zt", [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False)])
