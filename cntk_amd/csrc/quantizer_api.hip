@@ -141,7 +141,16 @@ struct BatchAbi<float>
 
     static size_t stripe_max_rows(size_t nbits) { return stripe_reduce_max_rows(nbits); }
     // taller stripes run 1024 threads per column: a launch of their own
-    static bool stripe_is_member(const SItem& it, size_t nbits) { return !stripe_uses_reg(it.rows, it.stripe_res, nbits); }
+    // (so do stripes that the table-driven register kernel takes with more than six pieces per thread: the shared launch is
+    // compiled for what its largest member needs)
+    static bool stripe_is_member(const SItem& it, size_t workers, size_t nbits)
+    {
+        if (stripe_uses_reg(it.rows, it.stripe_res, nbits))
+            return false;
+        if (stripe_auto_col(it.rows, it.stripe_res) && stripe_looks_up(it.rows, nbits, workers))
+            return stripe_lookup_per(it.rows, !columns_start_on_lines(it.stripe_res, it.rows)) <= 6;
+        return true;
+    }
     static int stripe_one(cntkq_quantizer* h, const SItem& it, size_t workers, size_t owner, size_t nbits, int zt)
     {
         return cntkq_stripe_reduce_async(h, it.stripes, workers, owner, it.rows, it.stripe_cols, nbits, it.stripe_res, it.q_out, it.agg_out, zt);
@@ -165,6 +174,13 @@ struct BatchAbi<float>
                 e.kind = it.rows == 1024 ? 2 : 3;
                 lds = (it.rows == 1024 ? col_lds_bytes<1>() : col_lds_bytes<2>()) + kStripeColExtraLds;
             }
+            else if (stripe_looks_up(it.rows, nbits, workers))
+            {
+                // as launch_stripe_reduce chooses (stripe_is_member has left those with more than six pieces per thread out)
+                e.r = make_reg_geom(it.rows, nbits, 256, line_shift);
+                e.kind = stripe_lookup_per(it.rows, line_shift) <= 3 ? 4 : 5;
+                lds = stripe_lut_lds_bytes(e.r);
+            }
         }
         else
         {
@@ -175,10 +191,13 @@ struct BatchAbi<float>
         }
         return true;
     }
+    // members that look their sums up need 76 registers where the others need 44: a launch without them keeps eight
+    // wavefronts per SIMD
+    static bool stripe_entry_wide(const SEntry& e) { return e.kind >= 4; }
     static hipError_t launch_stripe_members(hipStream_t s, LaunchEvents ev, const SEntry* de, const uint32_t* db, uint32_t members,
-                                            uint32_t blocks, size_t lds, size_t nbits, bool zt)
+                                            uint32_t blocks, size_t lds, size_t nbits, bool zt, bool wide)
     {
-        return launch_stripe_reduce_batch(s, ev, de, db, members, blocks, lds, nbits, zt);
+        return launch_stripe_reduce_batch(s, ev, de, db, members, blocks, lds, nbits, zt, wide);
     }
 };
 

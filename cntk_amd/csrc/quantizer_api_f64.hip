@@ -102,7 +102,7 @@ struct BatchAbi<double>
 
     static size_t stripe_max_rows(size_t nbits) { return f64::stripe_reduce_max_rows(nbits); }
     // stripes of the register kernel's heights run 1024 threads per column: a launch of their own
-    static bool stripe_is_member(const SItem& it, size_t nbits) { return !f64::stripe_uses_reg(it.rows, nbits); }
+    static bool stripe_is_member(const SItem& it, size_t, size_t nbits) { return !f64::stripe_uses_reg(it.rows, nbits); }
     static int stripe_one(cntkq_quantizer* h, const SItem& it, size_t workers, size_t owner, size_t nbits, int zt)
     {
         return cntkq_stripe_reduce_async_f64(h, it.stripes, workers, owner, it.rows, it.stripe_cols, nbits, it.stripe_res, it.q_out, it.agg_out,
@@ -115,8 +115,9 @@ struct BatchAbi<double>
         blocks = (e.t.cols + e.t.cols_per_tile - 1) / e.t.cols_per_tile;
         return lds <= f64::kMaxLdsBytes;
     }
+    static bool stripe_entry_wide(const SEntry&) { return false; }
     static hipError_t launch_stripe_members(hipStream_t s, LaunchEvents ev, const SEntry* de, const uint32_t* db, uint32_t members,
-                                            uint32_t blocks, size_t lds, size_t nbits, bool zt)
+                                            uint32_t blocks, size_t lds, size_t nbits, bool zt, bool)
     {
         return f64::dispatch_nbits64<f64::StripeBatchLauncher64>(nbits, zt && nbits == 1, s, ev, de, db, members, blocks, lds);
     }

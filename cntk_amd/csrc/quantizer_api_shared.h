@@ -117,6 +117,7 @@ struct BatchTable
     size_t members[2] = {0, 0};
     uint32_t blocks[2] = {0, 0};
     size_t lds[2] = {0, 0};
+    bool wide[2] = {false, false}; // a member of the class needs the kernel variant compiled for more registers
     size_t first_entry[2] = {0, 0};
     size_t first_begin[2] = {0, 0};
     size_t entries_bytes = 0;
@@ -136,6 +137,7 @@ struct NoAllocState
     size_t members[2] = {0, 0};
     uint32_t blocks[2] = {0, 0};
     size_t lds[2] = {0, 0};
+    bool wide[2] = {false, false}; // a member of the class needs the kernel variant compiled for more registers
     size_t first_entry[2] = {0, 0};
     size_t first_begin[2] = {0, 0};
     size_t entries_bytes = 0;

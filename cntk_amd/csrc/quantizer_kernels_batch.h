@@ -109,13 +109,18 @@ struct StripeBatchEntry
     float* stripe_res;
     char* q_out;
     float* agg_out;
-    uint32_t kind; // 0: tiles (t), 1: columns (c), 2 / 3: 1-bit columns of 1024 / 2048 rows (the unrolled body; c.qcol)
+    // 0: tiles (t), 1: columns (c), 2 / 3: 1-bit columns of 1024 / 2048 rows (the unrolled body; c.qcol),
+    // 4 / 5: 1-bit columns of up to eight workers, sums looked up, up to 3 / 6 pieces per thread (r)
+    uint32_t kind;
     uint32_t pad;
     TileGeom t;
     ColGeom c;
+    RegGeom r;
 };
 
-template <int NBITS, bool ZT>
+// LOOKUP: the variant that also runs members of kinds 4 and 5 (76 registers instead of 44: a launch without such members
+// takes the other one and keeps eight wavefronts per SIMD)
+template <int NBITS, bool ZT, bool LOOKUP>
 __global__ __launch_bounds__(kTileThreads) void stripe_reduce_batch_kernel(const StripeBatchEntry* __restrict__ entries,
                                                                            const uint32_t* __restrict__ begins, uint32_t count)
 {
@@ -132,6 +137,18 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_batch_kernel(const
     {
         const ColGeom c = en.c;
         stripe_reduce_colg_body<NBITS, ZT>(en.src, en.stripe_res, en.q_out, en.agg_out, c, index, smem_v4);
+    }
+    else if (LOOKUP && NBITS == 1 && en.kind >= 4)
+    {
+        // the plain call's kernel for these stripes: the bytes of the general column body, up to twice as fast
+        if constexpr (LOOKUP && NBITS == 1)
+        {
+            const RegGeom c = en.r;
+            if (en.kind == 4)
+                stripe_reduce_lut_body<ZT, 3, kTileThreads>(en.src, en.stripe_res, en.q_out, en.agg_out, c, index, smem_v4);
+            else
+                stripe_reduce_lut_body<ZT, 6, kTileThreads>(en.src, en.stripe_res, en.q_out, en.agg_out, c, index, smem_v4);
+        }
     }
     else if constexpr (NBITS == 1)
     {

@@ -765,20 +765,19 @@ __host__ __device__ inline size_t stripe_lut_lds_bytes(const RegGeom& c)
 }
 
 template <bool ZT, int PER, int TT = 1024>
-__global__ __launch_bounds__(TT) __attribute__((amdgpu_waves_per_eu(reg_waves<TT, PER>(), reg_waves<TT, PER>()))) void stripe_reduce_lut_kernel(
-    StripeSources src, float* stripe_res, char* q_out, float* agg_out, RegGeom c)
+__device__ __forceinline__ void stripe_reduce_lut_body(const StripeSources& src, float* stripe_res, char* q_out, float* agg_out, const RegGeom& c,
+                                                       uint32_t column, f32x4* smem_v4)
 {
     constexpr uint32_t T = TT, NW = T / 64, S = 8;
     static_assert(T >= 256, "one thread per table entry");
-    extern __shared__ f32x4 smem_v4[];
     float* red = reinterpret_cast<float*>(smem_v4);
     uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 2 * NW);
     uint32_t* words = reinterpret_cast<uint32_t*>(red + kRegRedSlots);
     float* lut = reinterpret_cast<float*>(words + c.nq);
     uint8_t* pat = reinterpret_cast<uint8_t*>(reinterpret_cast<uint32_t*>(red) + stripe_lut_bytes_offset(c));
     const uint32_t tid = threadIdx.x;
-    const size_t base = (size_t) blockIdx.x * c.rows;
-    const size_t rec = (size_t) blockIdx.x * c.qcol;
+    const size_t base = (size_t) column * c.rows;
+    const size_t rec = (size_t) column * c.qcol;
     for (uint32_t x = tid; x < c.nq; x += T)
         words[x] = 0u;
     float* sres = stripe_res + base;
@@ -914,6 +913,14 @@ __global__ __launch_bounds__(TT) __attribute__((amdgpu_waves_per_eu(reg_waves<TT
         }
     }
     reg_stats_pack<1, ZT, T, PER>(a, edge, has_edge, edge_at, head, pieces, shift, c, red, red_u, words, sres, q_out + rec);
+}
+
+template <bool ZT, int PER, int TT = 1024>
+__global__ __launch_bounds__(TT) __attribute__((amdgpu_waves_per_eu(reg_waves<TT, PER>(), reg_waves<TT, PER>()))) void stripe_reduce_lut_kernel(
+    StripeSources src, float* stripe_res, char* q_out, float* agg_out, RegGeom c)
+{
+    extern __shared__ f32x4 smem_v4[];
+    stripe_reduce_lut_body<ZT, PER, TT>(src, stripe_res, q_out, agg_out, c, blockIdx.x, smem_v4);
 }
 
 // ---- the same for tall columns of any height and alignment: elements instead of pieces ----------------------

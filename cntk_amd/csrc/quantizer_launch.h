@@ -759,6 +759,10 @@ struct StripeRegLauncher
             CNTKQ_SREG256(4);
             CNTKQ_SREG256(6);
             CNTKQ_SREG256(8);
+            CNTKQ_SREG256(10);
+            CNTKQ_SREG256(12);
+            CNTKQ_SREG256(14);
+            CNTKQ_SREG256(16);
 #undef CNTKQ_SREG256
             if (threads != 1024)
                 return hipErrorInvalidValue;
@@ -776,6 +780,17 @@ struct StripeRegLauncher
         }
     }
 };
+
+// Whether a stripe whose height and alignment would let the LDS column kernels take it goes to the table-driven register
+// kernel with 256 threads instead (1 bit, up to eight workers, above 2048 rows), and how many pieces a thread holds there.
+inline bool stripe_looks_up(size_t rows, size_t nbits, size_t workers)
+{
+    return nbits == 1 && workers >= 1 && workers <= 8 && rows > 2048;
+}
+inline uint32_t stripe_lookup_per(size_t rows, bool line_shift)
+{
+    return (uint32_t) ((rows / 4 + (line_shift ? 7 : 0) + 255) / 256);
+}
 
 // Whether the fused stripe reduction runs the 1024-thread register kernel: wherever a quantize call on (aggregate, stripe
 // residual) would run the register kernels with edge elements or with 1024 threads, whose summation order it shares -- above
@@ -820,8 +835,19 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
     // the summation order a quantize call on (aggregate, stripe residual) would use, given the residual's address
     const bool line_shift = !columns_start_on_lines(stripe_res, rows);
     if (col && (line_shift || !(aligned8 && col_unrolled(q_out, rows, nbits))))
+    {
+        // 1 bit, up to eight workers, above 2048 rows: the table-driven register kernel with 256 threads, which sums the
+        // statistics in the LDS column kernels' order (same bytes) and is faster (6144 x 3101, K = 8: 36 against 69 us;
+        // at 1152 rows there is nothing in it)
+        if (tune.quantize_path == kPathAuto && stripe_looks_up(rows, nbits, src.workers))
+        {
+            const RegGeom c = make_reg_geom(rows, nbits, 256, line_shift);
+            return dispatch_nbits<StripeRegLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols, c,
+                                                     256u);
+        }
         return dispatch_nbits<StripeColLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols,
                                                  make_col_geom(rows, nbits, line_shift));
+    }
     if (col)
     {
         // same column statistics, in the same order, as quantize_col_kernel
@@ -1082,19 +1108,23 @@ template <int NBITS, bool ZT>
 struct StripeBatchLauncher
 {
     static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeBatchEntry* entries, const uint32_t* begins, uint32_t count,
-                          uint32_t total_blocks, size_t lds)
+                          uint32_t total_blocks, size_t lds, bool wide)
     {
-        hipExtLaunchKernelGGL((stripe_reduce_batch_kernel<NBITS, ZT>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start, ev.stop, 0,
-                              entries, begins, count);
+        if (wide && NBITS == 1)
+            hipExtLaunchKernelGGL((stripe_reduce_batch_kernel<NBITS, ZT, NBITS == 1>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start,
+                                  ev.stop, 0, entries, begins, count);
+        else
+            hipExtLaunchKernelGGL((stripe_reduce_batch_kernel<NBITS, ZT, false>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start,
+                                  ev.stop, 0, entries, begins, count);
         return hipGetLastError();
     }
 };
 
 inline hipError_t launch_stripe_reduce_batch(hipStream_t s, LaunchEvents ev, const StripeBatchEntry* entries, const uint32_t* begins,
-                                             uint32_t count, uint32_t total_blocks, size_t lds, size_t nbits, bool zt)
+                                             uint32_t count, uint32_t total_blocks, size_t lds, size_t nbits, bool zt, bool wide)
 {
     zt = zt && (nbits == 1);
-    return dispatch_nbits<StripeBatchLauncher>(nbits, zt, s, ev, entries, begins, count, total_blocks, lds);
+    return dispatch_nbits<StripeBatchLauncher>(nbits, zt, s, ev, entries, begins, count, total_blocks, lds, wide);
 }
 
 // which kernel family launch_stripe_reduce takes by itself for a stripe of this height: columns (true) or tiles
