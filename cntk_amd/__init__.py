@@ -106,6 +106,7 @@ def lib():
             getattr(L, name).restype = _sz
         L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int]
         L.cntkq_debug_set_strip_spin_limit.argtypes = [_vp, ctypes.c_uint]
+        L.cntkq_set_force_sync.argtypes = [_vp, ctypes.c_int]
         _lib = L
     return _lib
 
@@ -329,7 +330,7 @@ class PreparedBatch:
 class MatrixQuantizerImpl:
     """The quantizer object (Source/Math/MatrixQuantizerImpl.h:19-49) for one GPU."""
 
-    def __init__(self, device_id, use_async):
+    def __init__(self, device_id, use_async, force_sync=False):
         if device_id < 0:
             # the reference returns its CPU quantizer here; this library has none
             raise QuantizerError("MatrixQuantizerImpl.Create: no CPU quantizer in this library (device %d)" % device_id)
@@ -337,6 +338,9 @@ class MatrixQuantizerImpl:
         _check(lib().cntkq_create(device_id, int(bool(use_async)), ctypes.byref(h)))
         self._h = h
         self._device_id = device_id
+        if force_sync:
+            # MatrixQuantizerGPU(deviceId, useDedicatedComputeStream, forceSync) (Source/Math/MatrixQuantizerGPU.h:20)
+            _check(lib().cntkq_set_force_sync(h, 1))
 
     @staticmethod
     def Create(device_id, use_async):

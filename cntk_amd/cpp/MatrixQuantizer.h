@@ -419,9 +419,12 @@ template <class ElemType>
 class MatrixQuantizerGPU final : public MatrixQuantizerImpl<ElemType>
 {
 public:
-    MatrixQuantizerGPU(int deviceId, bool useDedicatedComputeStream) : MatrixQuantizerImpl<ElemType>(deviceId)
+    // forceSync: every call waits for its own work (Source/Math/MatrixQuantizerGPU.h:20), for time measurements
+    MatrixQuantizerGPU(int deviceId, bool useDedicatedComputeStream, bool forceSync = false) : MatrixQuantizerImpl<ElemType>(deviceId)
     {
         detail::Check(cntkq_create(deviceId, useDedicatedComputeStream ? 1 : 0, &m_handle));
+        if (forceSync)
+            detail::Check(cntkq_set_force_sync(m_handle, 1));
     }
     ~MatrixQuantizerGPU() override { (void) cntkq_destroy(m_handle); }
 

@@ -635,6 +635,14 @@ int cntkq_set_main_stream(cntkq_quantizer* h, void* hip_stream)
     return CNTKQ_OK;
 }
 
+int cntkq_set_force_sync(cntkq_quantizer* h, int force_sync)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_set_force_sync: null handle");
+    h->force_sync = force_sync != 0;
+    return CNTKQ_OK;
+}
+
 int cntkq_sync_with_main_stream(cntkq_quantizer* h)
 {
     if (h == nullptr)

@@ -187,6 +187,7 @@ struct cntkq_quantizer
     BatchTable unquantize_table64;
     BatchTable stripe_table64;
     cntkq::LaunchTuning tune;
+    bool force_sync = false; // the host waits after every step of a call (the reference's m_forceSync, for time measurements)
     cntkq::StripScratchOwner strip_scratch; // partial sums and launch count of the strip kernels (tune.strip points here)
     struct NoAllocState* noalloc = nullptr; // fixed-size host state of cntkq_quantize_batch_noalloc (created with the handle)
 };
@@ -445,6 +446,11 @@ int quantize_async_impl(cntkq_quantizer* h, const E* in, const E* res_in, size_t
         qdev = h->staging;
     }
 
+    // serialised mode (Source/Math/MatrixQuantizerGPU.cu:237-240, 118-122, 137-141): the device is idle before the kernel
+    // starts, and the host waits for the kernel and for the copy
+    const bool force_sync = h->force_sync && !capturing;
+    if (force_sync)
+        HIP_TRY(hipDeviceSynchronize(), "hipDeviceSynchronize failed");
     LaunchEvents ev = take_events(h, h->ev_quantize);
     if (capturing)
         ev.stop = nullptr; // recorded, not executed: nothing to wait for
@@ -453,6 +459,8 @@ int quantize_async_impl(cntkq_quantizer* h, const E* in, const E* res_in, size_t
         return fail(CNTKQ_INVALID_ARGUMENT, "quantize: the forced kernel path does not support %zu x %zu at %zu bits", rows, cols, nbits);
     HIP_TRY(lrc, "quantize kernel launch failed");
     h->last_quantize = ev.stop;
+    if (force_sync)
+        HIP_TRY(hipStreamSynchronize(s), "hipStreamSynchronize failed");
 
     if (qbuf_on_host)
     {
@@ -461,6 +469,8 @@ int quantize_async_impl(cntkq_quantizer* h, const E* in, const E* res_in, size_t
         HIP_TRY(hipEventRecord(h->ev_fetch, h->fetch), "hipEventRecord failed");
         h->quantize_included_fetch = true;
         h->fetch_pending = true;
+        if (force_sync)
+            HIP_TRY(hipStreamSynchronize(h->fetch), "hipStreamSynchronize failed");
     }
     return CNTKQ_OK;
 }
@@ -505,6 +515,8 @@ int unquantize_async_impl(cntkq_quantizer* h, const void* qbuf, size_t qbuf_byte
             HIP_TRY(hipStreamWaitEvent(h->assign, h->ev_fetch, 0), "hipStreamWaitEvent failed");
         HIP_TRY(hipMemcpyAsync(h->staging, qbuf, need, hipMemcpyHostToDevice, h->assign), "hipMemcpyAsync failed");
         HIP_TRY(hipEventRecord(h->ev_assign, h->assign), "hipEventRecord failed");
+        if (h->force_sync) // Source/Math/MatrixQuantizerGPU.cu:318-321
+            HIP_TRY(hipStreamSynchronize(h->assign), "hipStreamSynchronize failed");
         HIP_TRY(hipStreamWaitEvent(s, h->ev_assign, 0), "hipStreamWaitEvent failed");
         qdev = h->staging;
     }

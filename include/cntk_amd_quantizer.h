@@ -96,6 +96,13 @@ void* cntkq_stream(const cntkq_quantizer* h);
  * main stream is not ordered against work issued on the new one: that is the caller's to arrange. */
 int cntkq_set_main_stream(cntkq_quantizer* h, void* hip_stream);
 
+/* The forceSync argument of the reference's constructor (Source/Math/MatrixQuantizerGPU.h:20,
+ * Source/Math/MatrixQuantizerGPU.cu:118-122, 137-141, 237-240, 318-321): when set, cntkq_quantize_async and
+ * cntkq_unquantize_async run serialised, for time measurements -- the device is synchronised before a quantization starts,
+ * and the host waits for the kernel and for the copy to or from a host-resident packed matrix before the call returns.
+ * Off by default. Calls recorded into a graph ignore it. */
+int cntkq_set_force_sync(cntkq_quantizer* h, int force_sync);
+
 /* MatrixComputeStreamEvent::Create + SynchronizeQuantizationComputeStreamWithEvent
  * (Source/Math/MatrixQuantizerImpl.h:53-72, Source/Math/MatrixQuantizerGPU.cu:347-371): work issued on the
  * handle's stream after this call starts only after everything already issued on the main stream. */
