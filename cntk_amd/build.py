@@ -62,7 +62,8 @@ def build_library(verbose=False, only=None):
     return LIB_PATH
 
 
-CPP_TESTS = ["test_matrix_quantizer", "test_allreduce_aggregator", "test_distributed_learner", "test_quantized_communicator", "bench_allreduce"]
+CPP_TESTS = ["test_matrix_quantizer", "test_allreduce_aggregator", "test_distributed_learner", "test_quantized_communicator", "test_v2_aggregator",
+             "bench_allreduce"]
 
 
 def build_cpp_tests(verbose=False):

@@ -50,6 +50,9 @@ public:
         else
             m_double = std::make_shared<Matrix<double>>(numRows, numCols, deviceId);
     }
+    // over a matrix that exists (possibly a view of the caller's memory)
+    explicit NDArrayView(std::shared_ptr<Matrix<float>> m) : m_type(DataType::Float), m_float(std::move(m)) {}
+    explicit NDArrayView(std::shared_ptr<Matrix<double>> m) : m_type(DataType::Double), m_double(std::move(m)) {}
     DataType GetDataType() const { return m_type; }
     size_t GetNumRows() const { return m_float ? m_float->GetNumRows() : m_double->GetNumRows(); }
     size_t GetNumCols() const { return m_float ? m_float->GetNumCols() : m_double->GetNumCols(); }
@@ -389,6 +392,24 @@ public:
             m_workers[r]->ReduceOwnStripes(calls[r]);
         for (size_t r = 0; r < K; ++r)
             m_workers[r]->FetchAndUnquantize(calls[r]);
+    }
+
+    // The plain sum of host values over the workers, each worker's buffer replaced by the sum
+    // (MPICommunicatorImpl::AggregateInPlace, Source/CNTKv2LibraryDll/DistributedCommunicator.cpp:304-309, for CPU values;
+    // the workers are added in ascending rank order).
+    void AggregateInPlace(std::vector<std::vector<double>>& values)
+    {
+        if (values.size() != m_workers.size())
+            throw std::invalid_argument("InProcessCommunicators: one argument list per worker");
+        for (const auto& v : values)
+            if (v.size() != values[0].size())
+                throw std::logic_error("InProcessCommunicators: the workers' values differ in size");
+        std::vector<double> sum = values[0];
+        for (size_t r = 1; r < values.size(); ++r)
+            for (size_t i = 0; i < sum.size(); ++i)
+                sum[i] += values[r][i];
+        for (auto& v : values)
+            v = sum;
     }
 
     // (:51-62)

@@ -63,6 +63,21 @@ def test_cpp_quantized_communicator_suite():
 
 
 @pytest.mark.gpu
+def test_cpp_v2_aggregator_suite():
+    """The aggregator over the v2 communicator (cntk_amd/cpp/V2AllReduceDistGradAggregator.h): the v1 aggregator's bytes and
+    header, the header sent as doubles, workers without samples, reset, double buffering."""
+    exe = os.path.join(ROOT, "tests", "cpp", "bin", "test_v2_aggregator")
+    assert os.path.exists(exe), "build it first: python -m cntk_amd.build"
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    print(res.stdout)
+    print(res.stderr[-4000:])
+    assert res.returncode == 0, "C++ v2 aggregator tests failed"
+    for name in ("EqualsV1AggregatorFloat", "EqualsV1AggregatorDouble", "HeaderAsDoubles", "WorkerWithoutSamples", "ResetClearsResidues",
+                 "DoubleBuffered"):
+        assert "V2AggregatorSuite/%s has passed" % name in res.stdout
+
+
+@pytest.mark.gpu
 def test_cpp_allreduce_timing_program_runs():
     """The all-reduce timing program runs through on a small shape and prints one line per arrangement."""
     exe = os.path.join(ROOT, "tests", "cpp", "bin", "bench_allreduce")
