@@ -26,7 +26,9 @@ enum QuantizePath
 };
 
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
-constexpr uint32_t kStripeWideItems = 768; // work items per column from which the stripe reduction uses 1024 threads
+constexpr uint32_t kStripeWideItems = 768;   // work items per column from which the stripe reduction may use more than 256 threads
+constexpr uint32_t kStripeWideMaxCols = 256; // ... 1024 threads up to this many columns
+constexpr uint32_t kStripeMidMinRows = 6144; // ... 512 threads above this height
 constexpr uint32_t kColMinRows = 1024;   // shorter columns are better served several to a workgroup (tile kernels)
 
 // The scratch buffer of the strip kernels (partial sums of the columns' workgroups and the launch count), owned by a handle: one
@@ -236,10 +238,20 @@ struct StripeColLauncher
     static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
                           uint32_t cols, ColGeom c)
     {
-        // columns with many work items (QWords x chunks of bit positions) get 1024 threads: each item is a chain of
-        // dependent loads, and few columns of a tall stripe would leave a CU with four wavefronts
+        // Every work item (a QWord, or a chunk of its bit positions) is a chain of dependent loads, and the column's LDS
+        // limits how many workgroups a CU holds: from 24 KB per column on (6 workgroups or fewer per CU) 512 threads keep
+        // the CU's wavefront slots filled, and where the stripe has no more columns than the device has CUs, 1024 do.
+        // Measured at 8 workers, 256 / 512 / 1024 threads: 9304 x 2048 at 2 bits 62 / 58 / 84 us, 14336 x 1328 at 4 bits
+        // 91 / 68 / 80, 4096 x 4652 at 8 bits 67 / 75 / 114, 6144 x 3101 at 2 bits 55 / 59 / 99, 14336 x 256 at 2 bits
+        // 28 / 19 / 15, 8192 x 300 at 8 bits 23 / 16 / 20.
+        uint32_t wg = 256u;
         if (c.nq * PackShape<NBITS>::CHUNKS >= kStripeWideItems)
+            wg = cols <= kStripeWideMaxCols ? 1024u : (c.rows > kStripeMidMinRows ? 512u : 256u);
+        if (wg == 1024)
             hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, 1024>), dim3(cols), dim3(1024), colg_lds_bytes<NBITS>(c, src.workers),
+                                  s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
+        else if (wg == 512)
+            hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, 512>), dim3(cols), dim3(512), colg_lds_bytes<NBITS>(c, src.workers),
                                   s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
         else
             hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, kColThreads>), dim3(cols), dim3(kColThreads),

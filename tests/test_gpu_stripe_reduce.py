@@ -62,6 +62,8 @@ CASES = [
     (1023, 6, 3, 1, False), (1025, 6, 3, 1, False), (2049, 8, 8, 1, False), (2050, 5, 2, 1, True), (4097, 4, 3, 4, False), (6001, 3, 5, 2, False),
     (7167, 4, 3, 1, False), (7169, 3, 2, 4, False), (7170, 4, 3, 1, True), (8001, 4, 2, 2, False), (9305, 3, 3, 1, False),
     (14335, 2, 8, 1, False), (9305, 2, 2, 32, False),
+    # stripes of more than 256 columns above 6144 rows: 512 threads per column in the LDS column kernel
+    (6400, 600, 2, 2, False), (8192, 540, 2, 8, False), (6148, 2320, 9, 1, False),
 ]
 
 
