@@ -371,7 +371,7 @@ struct ColGeom
 template <int NBITS>
 __host__ __device__ inline size_t colg_lds_bytes(const ColGeom& c, uint32_t workers)
 {
-    return ((size_t) c.rows + (PackShape<NBITS>::CHUNKS > 1 ? c.nq : 0) + 12 + (size_t) 2 * workers) * sizeof(float);
+    return ((size_t) c.rows + (PackShape<NBITS>::CHUNKS > 1 ? c.nq : 0) + 12 + (size_t) stripe_dec_floats(NBITS) * workers) * sizeof(float);
 }
 
 template <int NBITS>
@@ -595,6 +595,13 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
     // headers, QWords and stripe residual instead of three (see stripe_reduce_col_kernel)
     const float* sp = stripe_res + base;
     const uint32_t items = c.nq * PS::CHUNKS;
+    // the QWords of this column in the first BATCH workers' records, in summation order (beyond the last worker: the last
+    // one's again, fetched and not used). Looked up once: inside the loop over the work items every worker's pointer
+    // would be fetched from the kernel's arguments again, one after the other, before the loads that need it go out.
+    const uint32_t* first[BATCH];
+#pragma unroll
+    for (uint32_t u = 0; u < BATCH; ++u)
+        first[u] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(min(u, K - 1u), src.owner)] + rec + 8);
     uint32_t word[BATCH];
     float resid[PS::SLOTS];
     if (tid < items)
@@ -603,17 +610,23 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
         const uint32_t w = tid - chunk * c.nq;
 #pragma unroll
         for (uint32_t u = 0; u < BATCH; ++u)
-            if (u < K)
-                word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(u, src.owner)] + rec + 8 + (size_t) w * 4);
+            word[u] = first[u][w];
+        // (a row beyond the column reads the last row instead, and is not used: no branch around any of the loads)
 #pragma unroll
         for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+            resid[kk] = __builtin_nontemporal_load(sp + min(w + (chunk * PS::SLOTS + kk) * c.nq, c.rows - 1u));
+    }
+    constexpr uint32_t DEC = stripe_dec_floats(NBITS);
+    constexpr bool LEVELS = DEC > 2; // every level of every worker in LDS
+    if constexpr (LEVELS)
+    {
+        for (uint32_t x = tid; x < K * DEC; x += WG)
         {
-            const uint32_t i = w + (chunk * PS::SLOTS + kk) * c.nq;
-            if (i < c.rows)
-                resid[kk] = __builtin_nontemporal_load(sp + i);
+            const float* h = reinterpret_cast<const float*>(src.q[stripe_order(x / DEC, src.owner)] + rec);
+            dec[x] = unquantize_value<NBITS>(make_vq<NBITS>(h[0], h[1]), x % DEC);
         }
     }
-    if (tid < K)
+    else if (tid < K)
     {
         const float* h = reinterpret_cast<const float*>(src.q[stripe_order(tid, src.owner)] + rec);
         const ValueQ vq = make_vq<NBITS>(h[0], h[1]);
@@ -640,40 +653,55 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
         {
 #pragma unroll
             for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
-            {
-                const uint32_t i = w + (chunk * PS::SLOTS + kk) * c.nq;
-                if (i < c.rows)
-                    resid[kk] = __builtin_nontemporal_load(sp + i);
-            }
+                resid[kk] = __builtin_nontemporal_load(sp + min(w + (chunk * PS::SLOTS + kk) * c.nq, c.rows - 1u));
         }
         float acc[PS::SLOTS];
         for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
         {
-            if (it != tid || n0 != 0)
+            if (n0 != 0)
             {
 #pragma unroll
                 for (uint32_t u = 0; u < BATCH; ++u)
                     if (n0 + u < K)
                         word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + word_off);
             }
+            else if (it != tid)
+            {
+#pragma unroll
+                for (uint32_t u = 0; u < BATCH; ++u)
+                    word[u] = first[u][w];
+            }
 #pragma unroll
             for (uint32_t u = 0; u < BATCH; ++u)
             {
                 if (n0 + u < K)
                 {
-                    const float a = dec[2 * (n0 + u)];
-                    const float b = dec[2 * (n0 + u) + 1];
                     const uint32_t bits = word[u] >> sh0;
-#pragma unroll
-                    for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+                    if constexpr (LEVELS)
                     {
-                        float x;
-                        if constexpr (NBITS == 1)
-                            x = pick_level(bits, kk, a, b);
-                        else
-                            x = unquantize_value<NBITS>(a, b, (bits >> (kk * PS::SHIFT)) & PS::CODEMASK);
-                        // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
-                        acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
+                        const float* lev = dec + (n0 + u) * DEC;
+#pragma unroll
+                        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+                        {
+                            const float x = lev[(bits >> (kk * PS::SHIFT)) & PS::CODEMASK];
+                            acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
+                        }
+                    }
+                    else
+                    {
+                        const float a = dec[2 * (n0 + u)];
+                        const float b = dec[2 * (n0 + u) + 1];
+#pragma unroll
+                        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+                        {
+                            float x;
+                            if constexpr (NBITS == 1)
+                                x = pick_level(bits, kk, a, b);
+                            else
+                                x = unquantize_value<NBITS>(a, b, (bits >> (kk * PS::SHIFT)) & PS::CODEMASK);
+                            // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
+                            acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
+                        }
                     }
                 }
             }

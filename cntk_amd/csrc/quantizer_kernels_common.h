@@ -46,6 +46,14 @@ struct PackShapeOf
 template <int NBITS>
 using PackShape = PackShapeOf<NBITS, 32>;
 
+// What a stripe reduction keeps in LDS per worker and column to decode that worker's codes: at 2 and 4 bits every level
+// of the column (a decoded value is then one LDS read at the code's offset: three vector instructions per value and
+// worker instead of six), at 1 bit the two levels, else (ufactor, lower).
+__host__ __device__ constexpr uint32_t stripe_dec_floats(size_t nbits)
+{
+    return (nbits == 2 || nbits == 4) ? (1u << nbits) : 2u;
+}
+
 struct TileGeom
 {
     uint32_t rows;
