@@ -58,6 +58,8 @@ struct StripGeom
     uint32_t nq;
     uint32_t strips;     // workgroups per column: ceil(nq / WORDS)
     uint32_t spin_limit; // polls of a record before a lane gives up
+    uint32_t poll_pause; // pauses of 64 cycles between two polls of a record
+    uint32_t poll_first; // ... and before the first poll
     double inv_strips;   // for workgroup index -> (column, strip)
     uint64_t qcol;
 };
@@ -108,18 +110,26 @@ __device__ __forceinline__ void strip_publish(uint64_t* rec, uint32_t value_bits
 
 // One wavefront collects the S records of a field: lane l polls records l, l + 64, ... until they carry the tag, adds
 // their values in ascending order, and the lanes meet by butterfly. Every lane returns the same bits.
+// Polls are loads at device scope, and a thousand resident workgroups polling as fast as they can took half of the L2's
+// request rate from the loads and stores that the records wait for: a lane pauses poll_pause x 64 cycles between two polls
+// (200000 x 256 at 1 bit over 1 / 16 / 64 / 128 / 256: 214 / 208 / 200 / 198 / 208 us), and first_pause x 64 cycles
+// before the first one of an exchange, which with many strips per column practically never finds the record there
+// (262144 x 200, 32 strips: 174 -> 154 us with 64; 24576 x 2048, 3 strips: 116 -> 132 us, so only from 16 strips on).
 template <typename T>
-__device__ __forceinline__ T strip_collect(const uint64_t* recs, uint32_t strips, uint32_t tag, uint32_t spin_limit, uint32_t* error)
+__device__ __forceinline__ T strip_collect(const uint64_t* recs, uint32_t strips, uint32_t tag, const StripGeom& c, uint32_t first_pause, uint32_t* error)
 {
     T t = 0;
     for (uint32_t s = threadIdx.x & 63u; s < strips; s += 64)
     {
         uint32_t polls = 0;
+        for (uint32_t z = 0; z < first_pause; ++z)
+            __builtin_amdgcn_s_sleep(1);
         uint64_t x;
         while ((uint32_t) ((x = __hip_atomic_load(recs + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) != tag)
         {
-            __builtin_amdgcn_s_sleep(1);
-            if (++polls >= spin_limit)
+            for (uint32_t z = 0; z < c.poll_pause; ++z)
+                __builtin_amdgcn_s_sleep(1);
+            if (++polls >= c.spin_limit)
             {
                 __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                 break;
@@ -186,7 +196,7 @@ __device__ __forceinline__ float strip_exchange_stat(float stat, uint32_t column
         strip_publish(recs + strip, __float_as_uint(stat), tag);
     if (threadIdx.x < 64)
     {
-        const float t = strip_collect<float>(recs, c.strips, tag, c.spin_limit, scratch.error);
+        const float t = strip_collect<float>(recs, c.strips, tag, c, c.poll_first, scratch.error);
         if (threadIdx.x == 0)
             red[0] = t;
     }
@@ -211,9 +221,9 @@ __device__ __forceinline__ void strip_exchange_split(float& s0, float& s1, uint3
     }
     if (threadIdx.x < 64)
     {
-        const float t0 = strip_collect<float>(recs + 1 * c.strips, c.strips, tag, c.spin_limit, scratch.error);
-        const float t1 = strip_collect<float>(recs + 2 * c.strips, c.strips, tag, c.spin_limit, scratch.error);
-        const uint32_t tn = strip_collect<uint32_t>(recs + 3 * c.strips, c.strips, tag, c.spin_limit, scratch.error);
+        const float t0 = strip_collect<float>(recs + 1 * c.strips, c.strips, tag, c, c.poll_first, scratch.error);
+        const float t1 = strip_collect<float>(recs + 2 * c.strips, c.strips, tag, c, 0u, scratch.error);
+        const uint32_t tn = strip_collect<uint32_t>(recs + 3 * c.strips, c.strips, tag, c, 0u, scratch.error);
         if (threadIdx.x == 0)
         {
             red[0] = t0;

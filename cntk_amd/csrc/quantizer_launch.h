@@ -26,6 +26,8 @@ enum QuantizePath
 };
 
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
+constexpr uint32_t kStripPollPause = 64;           // strip kernel: 64-cycle pauses between two polls of a partial sum
+constexpr uint32_t kStripFirstPauseMinStrips = 16; // ... strips per column from which a pause of 2 x strips precedes the first poll
 constexpr uint32_t kStripeWideItems = 768;   // work items per column from which the stripe reduction may use more than 256 threads
 constexpr uint32_t kStripeWideMaxCols = 256; // ... 1024 threads up to this many columns
 constexpr uint32_t kStripeMidMinRows = 6144; // ... 512 threads above this height
@@ -49,7 +51,7 @@ struct StripScratchOwner
 struct LaunchTuning
 {
     StripScratchOwner* strip = nullptr; // null: the strip kernels are not available to this launch
-    uint32_t strip_spin_limit = 1u << 20; // polls of a partial sum (a microsecond or so each) before a lane gives up
+    uint32_t strip_spin_limit = 1u << 17; // polls of a partial sum (two microseconds or so each) before a lane gives up
     int quantize_path = kPathAuto;
     uint32_t tile_gs = 0;   // 0 = pick from rows; else threads per column (power of two, 8..256)
     int tile_stage = -1;    // -1 = automatic; 0 / 1 = residual written straight to memory / staged through LDS
@@ -491,6 +493,8 @@ inline StripGeom make_strip_geom(size_t rows, size_t cols, size_t nbits, uint32_
     c.nq = (uint32_t) qwords_per_col(rows, nbits);
     c.strips = (c.nq + strip_words(nbits) - 1) / strip_words(nbits);
     c.spin_limit = spin_limit;
+    c.poll_pause = kStripPollPause;
+    c.poll_first = c.strips >= kStripFirstPauseMinStrips ? 2u * c.strips : 0u;
     c.inv_strips = 1.0 / (double) c.strips;
     c.qcol = qcol_bytes(nbits, rows);
     return c;

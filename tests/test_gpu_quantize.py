@@ -582,7 +582,7 @@ def test_strip_kernel_reports_workgroups_that_give_up():
     qz.QuantizeAsync(G, R, Q, R, False)
     with pytest.raises(cntk_amd.QuantizerError):
         qz.WaitQuantizeAsyncDone()
-    qz._set_strip_spin_limit(1 << 20)
+    qz._set_strip_spin_limit(1 << 17)
     R.data.zero_()
     qz.QuantizeAsync(G, R, Q, R, False)
     qz.WaitQuantizeAsyncDone()
