@@ -25,6 +25,36 @@ HIPCC_FLAGS = [
 SOURCES = ["quantizer_api.hip", "quantizer_api_f64.hip"]
 
 
+def resource_report_path(source):
+    """Where build_library leaves the compiler's per-kernel resource figures of a source file: one line per kernel,
+    `name=<mangled> VGPRs=.. ScratchSize=.. Occupancy=.. VGPRsSpill=.. SGPRsSpill=..` (scratch in bytes per lane)."""
+    return os.path.join(HERE, "csrc", "build", os.path.splitext(source)[0] + ".resources.txt")
+
+
+def split_resource_remarks(stderr):
+    """Separates hipcc's kernel-resource-usage remarks from the rest of its output; returns ([{field: value} per kernel],
+    [other lines])."""
+    fields = {"TotalSGPRs": "SGPRs", "VGPRs": "VGPRs", "ScratchSize [bytes/lane]": "ScratchSize", "Occupancy [waves/SIMD]": "Occupancy",
+              "SGPRs Spill": "SGPRsSpill", "VGPRs Spill": "VGPRsSpill", "LDS Size [bytes/block]": "LDS"}
+    kernels, rest, skip = [], [], 0
+    for line in stderr.splitlines():
+        if "[-Rpass-analysis=kernel-resource-usage]" in line:
+            body = line.split("remark:", 1)[1].rsplit("[-Rpass-analysis", 1)[0].strip()
+            key, _, value = body.partition(":")
+            if key.strip() == "Function Name":
+                kernels.append({"name": value.strip()})
+            elif kernels and key.strip() in fields:
+                kernels[-1][fields[key.strip()]] = value.strip()
+            skip = 2  # the source line and the caret that follow a remark
+        elif skip > 0 and (line.lstrip().startswith("|") or line.lstrip()[:1].isdigit() or line.startswith("In file included")):
+            skip -= 1
+        elif line.startswith("In file included from"):
+            continue
+        else:
+            rest.append(line)
+    return kernels, rest
+
+
 def build_library(verbose=False, only=None):
     """Compiles the sources (or, with `only`, just the named ones, keeping the other object files) and links the
     library."""
@@ -38,18 +68,24 @@ def build_library(verbose=False, only=None):
         objs.append(obj)
         if only is not None and name not in only and os.path.exists(obj):
             continue
-        cmd = [hipcc] + HIPCC_FLAGS + ["-c", "-o", obj, os.path.join(HERE, "csrc", name)]
+        # the compiler reports every kernel's registers, scratch memory and occupancy: kept beside the object file
+        cmd = [hipcc] + HIPCC_FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c", "-o", obj, os.path.join(HERE, "csrc", name)]
         if verbose:
             print(" ".join(cmd), flush=True)
-        procs.append((name, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
+        procs.append((name, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
     errors = []
-    for name, proc in procs:
+    for name, obj, proc in procs:
         _, stderr = proc.communicate()
+        remarks, rest = split_resource_remarks(stderr)
         # the host pass does not know the packed-fp32 feature and says so; that warning is harmless
-        err = "\n".join(l for l in stderr.splitlines() if "packed-fp32-ops" not in l)
+        err = "\n".join(l for l in rest if "packed-fp32-ops" not in l)
         if proc.returncode != 0:
             errors.append("%s:\n%s" % (name, err))
-        elif verbose and err.strip():
+            continue
+        with open(resource_report_path(name), "w") as f:
+            for kernel in remarks:
+                f.write(" ".join("%s=%s" % kv for kv in kernel.items()) + "\n")
+        if verbose and err.strip():
             print(err, file=sys.stderr)
     if errors:
         raise RuntimeError("hipcc failed:\n" + "\n".join(errors))

@@ -558,8 +558,16 @@ __device__ __forceinline__ float pick_level_s(uint32_t bits, uint32_t pos, float
     return x;
 }
 
+// (six pieces per thread do not fit the 64 registers that two workgroups per CU leave: one workgroup without spills does
+// 20000 x 1024, K = 12, in 93 us, two with 50 spilled registers in 108 us)
+template <int PER>
+constexpr int reg8_waves()
+{
+    return PER == 6 ? 4 : reg_waves<1024, PER>();
+}
+
 template <bool ZT, int PER>
-__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg_waves<1024, PER>(), reg_waves<1024, PER>()))) void stripe_reduce_reg8_kernel(
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(reg8_waves<PER>(), reg8_waves<PER>()))) void stripe_reduce_reg8_kernel(
     StripeSources src, float* stripe_res, char* q_out, float* agg_out, RegGeom c)
 {
     constexpr uint32_t T = 1024, NW = T / 64, S = 8;
@@ -793,8 +801,9 @@ __device__ __forceinline__ void stripe_reduce_lut_body(const StripeSources& src,
 
     // The stripe residual is requested first: its latency runs under the table building below (one workgroup fills a CU,
     // nothing else would overlap the two), and a sum plus its residual is the same bits in either order. The tallest
-    // columns, whose residual would leave the table building no registers, request it piece by piece at the look-ups.
-    constexpr bool EARLY = PER <= 20;
+    // columns, whose residual would leave the table building no registers, request it piece by piece at the look-ups,
+    // and so does the one shape that has two workgroups per CU only within 64 registers.
+    constexpr bool EARLY = PER <= 20 && !(PER == 6 && TT == 1024);
     f32x4 a[PER];
     const f32x4* r4 = reinterpret_cast<const f32x4*>(sres + head);
     if constexpr (EARLY)
@@ -915,8 +924,18 @@ __device__ __forceinline__ void stripe_reduce_lut_body(const StripeSources& src,
     reg_stats_pack<1, ZT, T, PER>(a, edge, has_edge, edge_at, head, pieces, shift, c, red, red_u, words, sres, q_out + rec);
 }
 
+// The register budget of the look-up kernel: that of the other register kernels, except at six pieces per thread, where
+// their eight wavefronts per SIMD (64 registers) made it spill 512 registers' worth (6144 x 3101, K = 8: 548 us instead of
+// 39 us). With 256 threads it gets the 74 it needs (six wavefronts); with 1024 threads it keeps eight -- two workgroups per
+// CU -- and fits by requesting the residual at the look-ups (20000 x 2048, K = 8: 83 us; 113 us with one workgroup per CU).
+template <int T, int PER>
+constexpr int lut_waves()
+{
+    return PER == 6 && T != 1024 ? 6 : reg_waves<T, PER>();
+}
+
 template <bool ZT, int PER, int TT = 1024>
-__global__ __launch_bounds__(TT) __attribute__((amdgpu_waves_per_eu(reg_waves<TT, PER>(), reg_waves<TT, PER>()))) void stripe_reduce_lut_kernel(
+__global__ __launch_bounds__(TT) __attribute__((amdgpu_waves_per_eu(lut_waves<TT, PER>(), lut_waves<TT, PER>()))) void stripe_reduce_lut_kernel(
     StripeSources src, float* stripe_res, char* q_out, float* agg_out, RegGeom c)
 {
     extern __shared__ f32x4 smem_v4[];

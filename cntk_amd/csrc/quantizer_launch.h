@@ -853,7 +853,7 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
     if (col && (line_shift || !(aligned8 && col_unrolled(q_out, rows, nbits))))
     {
         // 1 bit, up to eight workers, above 2048 rows: the table-driven register kernel with 256 threads, which sums the
-        // statistics in the LDS column kernels' order (same bytes) and is faster (6144 x 3101, K = 8: 36 against 69 us;
+        // statistics in the LDS column kernels' order (same bytes) and is faster (6144 x 3101, K = 8: 39 against 69 us;
         // at 1152 rows there is nothing in it)
         if (tune.quantize_path == kPathAuto && stripe_looks_up(rows, nbits, src.workers))
         {

@@ -1,0 +1,51 @@
+"""The compiler's own figures for every kernel of the library (registers, scratch memory per lane, occupancy), as
+`python -m cntk_amd.build` leaves them beside the object files: no kernel may spill more than a few registers' worth.
+
+A kernel whose register budget (`amdgpu_waves_per_eu`) is a little too small still compiles and still gives the right
+bytes, only many times slower -- the table-driven stripe reduction at six pieces per thread once ran 6144-row stripes in
+548 us instead of 39 us on 388 bytes of scratch per lane -- so the bound is checked where it costs nothing."""
+import os
+
+import pytest
+
+from cntk_amd import build
+
+# the largest scratch of a kernel today: the tall stripe reductions at 25 pieces per thread (80001 to 102400 rows), which
+# have the SIMD's registers to themselves and still keep 79 values too many
+MAX_SCRATCH_BYTES_PER_LANE = 160
+
+
+def read_report(source):
+    path = build.resource_report_path(source)
+    if not os.path.exists(path):
+        pytest.skip("no resource report at %s: build the library first (python -m cntk_amd.build)" % path)
+    kernels = []
+    with open(path) as f:
+        for line in f:
+            kernels.append(dict(kv.split("=", 1) for kv in line.split()))
+    return kernels
+
+
+@pytest.mark.parametrize("source", build.SOURCES)
+def test_no_kernel_lives_on_scratch_memory(source):
+    kernels = read_report(source)
+    assert len(kernels) > 100, "the report of %s lists %d kernels only" % (source, len(kernels))
+    worst = sorted(kernels, key=lambda k: -int(k["ScratchSize"]))[:5]
+    print([(k["name"][:70], k["ScratchSize"], k["VGPRs"]) for k in worst])
+    for k in kernels:
+        assert int(k["ScratchSize"]) <= MAX_SCRATCH_BYTES_PER_LANE, \
+            "%s: %s bytes of scratch per lane (%s registers spilled at %s registers, %s wavefronts per SIMD)" % (
+                k["name"], k["ScratchSize"], k["VGPRsSpill"], k["VGPRs"], k["Occupancy"])
+
+
+def test_headline_kernels_spill_nothing():
+    """The kernels of the headline benchmark and of the batched launches: no scratch at all."""
+    kernels = read_report("quantizer_api.hip")
+    seen = 0
+    for k in kernels:
+        n = k["name"]
+        if any(s in n for s in ("quantize_col_kernel", "quantize_batch_kernel", "stripe_reduce_col_kernel", "stripe_reduce_batch_kernel",
+                                "unquantize_kernel", "unquantize_batch_kernel", "stripe_reduce_lut_kernelILb0ELi6E", "stripe_reduce_lut_kernelILb1ELi6E")):
+            seen += 1
+            assert int(k["ScratchSize"]) == 0, "%s uses %s bytes of scratch per lane" % (n, k["ScratchSize"])
+    assert seen >= 20
