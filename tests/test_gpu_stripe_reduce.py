@@ -64,6 +64,10 @@ CASES = [
     (14335, 2, 8, 1, False), (9305, 2, 2, 32, False),
     # stripes of more than 256 columns above 6144 rows: 512 threads per column in the LDS column kernel
     (6400, 600, 2, 2, False), (8192, 540, 2, 8, False), (6148, 2320, 9, 1, False),
+    # more than eight workers at 2 and 4 bits: the second batch of workers reads its levels from the table too
+    (2048, 26, 13, 2, False), (4096, 20, 10, 4, False), (1152, 22, 11, 4, False),
+    # six pieces per thread in the table-driven kernels (256 threads: 4100 to 6144 rows, 1024 threads: 16388 to 24576)
+    (6144, 16, 8, 1, False), (5000, 16, 8, 1, True), (24576, 8, 8, 1, False), (20000, 6, 12, 1, False),
 ]
 
 
