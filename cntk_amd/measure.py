@@ -49,6 +49,12 @@ def main():
     qz._set_tuning(quantize_path=args.path, unq_mode=args.unq_mode)
     h = qz._h
 
+    # no fused stripe reduction above this height: the other two calls are still measured
+    stripe_limit = getattr(L, "cntkq_stripe_reduce_max_rows" + sfx)(nbits)
+    stripe_skipped = bool(args.workers) and rows > stripe_limit
+    if stripe_skipped:
+        args.workers = 0
+
     elems = rows * cols
     qbytes = QuantizedMatrix(rows, cols, nbits, 0, dtype=tdt).GetSize()
     per_set = elems * eb * 3 + qbytes * (1 + max(args.workers - 1, 0))
@@ -126,6 +132,8 @@ def main():
         "quantize": {"us": round(q_ms * 1e3, 2), "algorithmic_bytes": q_bytes, "GBps": round(q_bytes / q_ms / 1e6, 1)},
         "unquantize": {"us": round(u_ms * 1e3, 2), "algorithmic_bytes": u_bytes, "GBps": round(u_bytes / u_ms / 1e6, 1)},
     }
+    if stripe_skipped:
+        out["stripe_reduce"] = {"skipped": "columns of %d rows: the fused stripe reduction takes at most %d at %d bits" % (rows, stripe_limit, nbits)}
     if args.workers:
         s_ms = avg_ms(4, 5)
         s_bytes = (args.workers + 1) * qbytes + 2 * elems * eb
