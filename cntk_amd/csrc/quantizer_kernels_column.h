@@ -583,7 +583,7 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
     float* tile = reinterpret_cast<float*>(smem);
     uint32_t* words = reinterpret_cast<uint32_t*>(tile + c.rows);
     float* red = tile + c.rows + (PS::CHUNKS > 1 ? c.nq : 0);
-    float* dec = red + 12; // per worker, in summation order: 1 bit -> the two levels, else (ufactor, lower)
+    float* dec = red + 12; // per worker, in summation order: 1 bit -> the two levels, 2 and 4 bits -> every level, else (ufactor, lower)
     const uint32_t tid = threadIdx.x;
     const size_t base = (size_t) column * c.rows;
     const size_t rec = (size_t) column * c.qcol;

@@ -8,13 +8,13 @@
 // the height, which columns above 102400 rows -- more than any workgroup's registers hold -- could otherwise only have by
 // reading their inputs two or three times. A strip needs 1 to 4 KB of LDS and, at 1 to 4 bits, some 100 registers (its 32
 // values, their addresses, the masks of the ragged last strip), so five workgroups share a CU; it is the exchange
-// described next, not memory, that bounds the kernel (about 3 TB/s), and below 102400 rows the kernels with one workgroup
+// described next, not memory, that bounds the kernel (3.3 to 4.4 TB/s), and below 102400 rows the kernels with one workgroup
 // per column are faster.
 //
 // The column statistics span the strips of a column. Every workgroup publishes its partial sums in a scratch buffer, one
 // 8-byte record per sum: the value and the tag of the launch, written by one atomic store, so that whoever reads the tag
 // of this launch has the value with it and no second word needs ordering against the first. Then the first wavefront of
-// every workgroup of the column polls the S records (a lane per record) until all carry the tag, and adds them up, lanes
+// every workgroup of the column polls the S records (a lane per record, with pauses) until all carry the tag, and adds them up, lanes
 // meeting by butterfly -- one fixed order, the same bytes in every workgroup. One exchange for the sum of squares (more than 1 bit) or
 // the split sums (1 bit against 0), two for 1 bit against the mean (mean, then split sums). The tag is a launch count
 // kept in the scratch buffer itself: every workgroup reads it when it starts, and the last workgroup to finish (a second
