@@ -14,10 +14,16 @@ finds its inputs in the 256 MB Infinity Cache. Prints ONE JSON line.
             are part of it (a 20-step run is about 1 ms long). gpu_timeline_ms_per_step, from a second pass of the
             same K steps, is first kernel start -> last kernel end by dispatch-attached events.
   roofline  the dominant kernel (quantize): algorithmic bytes per launch (12 + nbits/8 per element + 8 per column
-            = 231,116,664) over its average duration measured with HIP events on the launch stream in a third,
+            = 231,111,360) over its average duration measured with HIP events on the launch stream in a third,
             untimed pass of the same steps, against 8 TB/s of HBM
-  cpu_baseline  the CPU oracle (a port of the reference's MatrixQuantizerCPU) timed on this host, single thread
-            like the reference, on the same matrix
+  cpu_baseline  the reference's own CPU quantizer (its headers, compiled under oracle/_ref) where that build is present,
+            else the CPU oracle (a port of it), timed on this host, single thread like the reference, on the same
+            matrix; the compiler flags of both CPU libraries are stated in the line
+  configs   after the headline's timed region and event passes (so `value` is untouched), the other workloads of this
+            path as whole steps through the gradient-set calls: speech DNN set (1 bit), ResNet-50 set (2, 4, 8 bits),
+            the simulated 8-worker all-reduce of 2048 x 9304, the LSTM language-model set (1 bit, zero threshold); for
+            each: step time, % of HBM peak, every call of a step timed between two stream events, and the roofline
+            of the longest call (`--no-configs` leaves them out; `--config N` runs one of them alone)
 """
 import argparse
 import json
@@ -85,11 +91,13 @@ def cpu_baseline(budget_s=12.0):
         pass
     tn, pn = run(cores, budget_s / 3)
     tb = tr if have_ref else t1
+    flags = oracle.build_flags()
     return {
         "value": round((qb + ub) / tb / 1e9, 4),
         "unit": "GB/s",
         "cores": 1,
         "kind": "reference" if have_ref else "port",
+        "compiler_flags": {"reference": flags.get("CXXFLAGS"), "port": flags.get("CFLAGS"), "compilers": "g++ / gcc"},
         "port": {"cores": 1, "value": round((qb + ub) / t1 / 1e9, 4), "ms_per_step": round(t1 * 1e3, 2), "passes": p1},
         "cpu_model": cpu_model,
         "host_cpus": os.cpu_count(),
@@ -140,6 +148,8 @@ def main():
                          "3 ResNet-50 set (2, 4, 8 bits: one line each), 4 simulated 8-worker all-reduce of 2048x9304, "
                          "5 LSTM language-model set (1 bit, zero threshold); one JSON line per workload with the time of "
                          "every call of a step and the roofline of the longest")
+    ap.add_argument("--no-configs", action="store_true", help="headline only: skip the other four workloads that follow it")
+    ap.add_argument("--config-steps", type=int, default=100, help="timed steps of each of the workloads that follow the headline")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="instead of the benchmark, run plain device copies of one 2048x9304 fp32 matrix "
                          "(76,218,368 bytes read and as many written per copy), for scaling hardware counters")
@@ -331,6 +341,19 @@ def main():
             "traffic_source": traffic_source,
         },
     }
+    if not args.no_configs:
+        # the other workloads, after everything of the headline has been measured; the headline's buffers go first
+        from cntk_amd import config_bench
+
+        del sets, ptrs
+        torch.cuda.empty_cache()
+        configs = {}
+        for cfg in (2, 3, 4, 5):
+            for line in config_bench.run(cfg, steps=args.config_steps, warmup=10, emit=False):
+                key = "%d_%dbit" % (cfg, line["workload"]["nbits"]) if cfg == 3 else str(cfg)
+                configs[key] = {k: line[k] for k in ("value", "unit", "pct_hbm_peak", "steps", "warmup", "ms_per_step",
+                                                     "gpu_timeline_ms_per_step", "workload", "calls", "calls_timed", "roofline")}
+        result["configs"] = configs
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result), flush=True)

@@ -2,6 +2,7 @@
 import os
 import subprocess
 import sys
+import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libcntk_amd_quantizer.so")
@@ -20,9 +21,14 @@ HIPCC_FLAGS = [
 ]
 
 
-# The library's two source files (float matrices + everything independent of the element type; double matrices) share
-# no device code and are compiled side by side.
-SOURCES = ["quantizer_api.hip", "quantizer_api_f64.hip"]
+# The library's source files share no device code and are compiled side by side: the C ABI (float matrices and everything
+# independent of the element type), one file per kernel family of the float instantiation, and the double instantiation.
+SOURCES = ["quantizer_api.hip", "quantizer_family_tile.hip", "quantizer_family_column.hip", "quantizer_family_register_256.hip",
+           "quantizer_family_register_1024.hip", "quantizer_family_register_edge.hip", "quantizer_family_strip.hip",
+           "quantizer_family_stripe_register_256.hip", "quantizer_family_stripe_register_1024.hip", "quantizer_family_unquantize.hip",
+           "quantizer_family_batch_quantize.hip", "quantizer_family_batch_stripe.hip", "quantizer_api_f64.hip"]
+# compilers running at once (a source file takes up to 3 GB while it is compiled)
+JOBS = max(1, min(16, os.cpu_count() or 1, int(os.environ.get("MAX_JOBS", "16"))))
 
 
 def resource_report_path(source):
@@ -61,32 +67,45 @@ def build_library(verbose=False, only=None):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     obj_dir = os.path.join(HERE, "csrc", "build")
     os.makedirs(obj_dir, exist_ok=True)
-    procs = []
     objs = []
+    todo = []
     for name in SOURCES:
         obj = os.path.join(obj_dir, os.path.splitext(name)[0] + ".o")
         objs.append(obj)
         if only is not None and name not in only and os.path.exists(obj):
             continue
         # the compiler reports every kernel's registers, scratch memory and occupancy: kept beside the object file
-        cmd = [hipcc] + HIPCC_FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c", "-o", obj, os.path.join(HERE, "csrc", name)]
-        if verbose:
-            print(" ".join(cmd), flush=True)
-        procs.append((name, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
+        todo.append((name, [hipcc] + HIPCC_FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c", "-o", obj, os.path.join(HERE, "csrc", name)]))
     errors = []
-    for name, obj, proc in procs:
-        _, stderr = proc.communicate()
+    running = []
+
+    def reap(proc_entry):
+        name, proc, log = proc_entry
+        proc.wait()
+        log.seek(0)
+        stderr = log.read()
+        log.close()
         remarks, rest = split_resource_remarks(stderr)
         # the host pass does not know the packed-fp32 feature and says so; that warning is harmless
         err = "\n".join(l for l in rest if "packed-fp32-ops" not in l)
         if proc.returncode != 0:
             errors.append("%s:\n%s" % (name, err))
-            continue
+            return
         with open(resource_report_path(name), "w") as f:
             for kernel in remarks:
                 f.write(" ".join("%s=%s" % kv for kv in kernel.items()) + "\n")
         if verbose and err.strip():
             print(err, file=sys.stderr)
+
+    for name, cmd in todo:
+        while len(running) >= JOBS:
+            reap(running.pop(0))
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        log = tempfile.TemporaryFile(mode="w+")  # (not a pipe: hundreds of remarks would fill it while the compiler waits its turn to be read)
+        running.append((name, subprocess.Popen(cmd, stdout=subprocess.DEVNULL, stderr=log, text=True), log))
+    for entry in running:
+        reap(entry)
     if errors:
         raise RuntimeError("hipcc failed:\n" + "\n".join(errors))
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs

@@ -161,7 +161,8 @@ def _allreduce_steps(torch, rows, cols, k, nbits, zt, sets_wanted):
     return steps, names, nbytes, keep
 
 
-def run(config, steps=200, warmup=20, nbits_list=None):
+def run(config, steps=200, warmup=20, nbits_list=None, emit=True):
+    """Measures workload `config`; returns its JSON lines (one per bit width for workload 3) and, with `emit`, prints them."""
     import torch
 
     assert torch.cuda.is_available(), "bench.py needs the GPU"
@@ -257,7 +258,8 @@ def run(config, steps=200, warmup=20, nbits_list=None):
             "roofline": {"bound": "hbm", "kernel": names[dom], "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(achieved / HBM_PEAK_GBS, 4), "algorithmic_bytes_per_launch": nbytes[dom], "traffic": None},
         }
-        print(json.dumps(line), flush=True)
+        if emit:
+            print(json.dumps(line), flush=True)
         lines.append(line)
         del sets, keep
         torch.cuda.empty_cache()

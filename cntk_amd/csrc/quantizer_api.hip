@@ -220,6 +220,9 @@ struct DeviceScratch
     unsigned char* ptr = nullptr;        // address of `scratch` on this device
     const void* writer = nullptr;        // the handle whose table the array holds (host-side bookkeeping)
     uint64_t generation = 0;             // bumped on every upload
+    // A call recorded into a graph (stream capture) writes the array whenever the graph is replayed, which no host-side
+    // bookkeeping sees: once there is such a call on the device, every call uploads its table.
+    bool recorded_call = false;
 };
 DeviceScratch g_scratch[kMaxDevices];
 
@@ -391,17 +394,22 @@ int quantize_batch_noalloc_impl(cntkq_quantizer* h, const cntkq_quantize_item* i
     }
 
     // The device array is shared by every handle on this GPU and keeps the last call's contents: upload unless this very
-    // table is what it received last. (A recorded call always uploads: a replay must not depend on what ran before it.)
+    // table is what it received last. A recorded call always uploads (a replay must not depend on what ran before it) and
+    // is never taken for an upload that has happened: nothing ran yet, and from then on replays rewrite the array at times
+    // the host does not know of.
     bool upload = st.table_words != 0;
     {
         std::lock_guard<std::mutex> lock(g_streams_mutex);
-        if (upload && !capturing && ds.writer == h && st.uploaded_generation != 0 && ds.generation == st.uploaded_generation &&
-            st.uploaded_stream == s)
+        if (capturing)
+            ds.recorded_call = true;
+        if (upload && !capturing && !ds.recorded_call && ds.writer == h && st.uploaded_generation != 0 &&
+            ds.generation == st.uploaded_generation && st.uploaded_stream == s)
             upload = false;
         if (upload)
         {
-            ds.writer = h;
-            st.uploaded_generation = ++ds.generation;
+            ++ds.generation;
+            ds.writer = capturing ? nullptr : h;
+            st.uploaded_generation = capturing ? 0 : ds.generation;
             st.uploaded_stream = s;
         }
     }
@@ -438,10 +446,14 @@ int quantize_batch_noalloc_impl(cntkq_quantizer* h, const cntkq_quantize_item* i
         LaunchEvents ev;
         launches_left--;
         ev.stop = launches_left == 0 ? done : nullptr;
-        // (without the strip kernels, whose scratch buffer is allocated on demand: this call allocates nothing)
+        // (the strip kernels only where the handle's scratch buffer, made when the handle was created, holds the matrix
+        // as it stands: this call allocates nothing. A taller or wider matrix runs the kernel that re-reads its columns,
+        // whose sums are added in another order: its column bounds may differ from the batched call's in their last bits.)
         const cntkq_quantize_item& it = items[st.own[k]];
-        LaunchTuning no_strip;
-        HIP_TRY(launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, no_strip), "quantize kernel launch failed");
+        LaunchTuning fixed;
+        fixed.strip = h->strip_scratch.order_event != nullptr ? &h->strip_scratch : nullptr;
+        fixed.strip_may_allocate = false;
+        HIP_TRY(launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, fixed), "quantize kernel launch failed");
     }
     h->last_quantize = done;
     h->quantize_included_fetch = false;
@@ -572,7 +584,8 @@ int cntkq_create(int device_id, int use_dedicated_stream, cntkq_quantizer** out)
         // allocate) finds it. A failure here is not one of the handle: the first call that needs the buffer tries again.
         // (cleared on one of the handle's own streams and waited for there: the legacy default stream stays out of it)
         StripScratch unused;
-        if (strip_scratch_for(h->strip_scratch, h->fetch, 1, 2, unused) != hipSuccess)
+        if (strip_scratch_for(h->strip_scratch, h->fetch, 1, 2, unused) != hipSuccess ||
+            hipEventCreateWithFlags(&h->strip_scratch.order_event, hipEventDisableTiming) != hipSuccess)
             (void) hipGetLastError();
     }
     *out = h;
@@ -593,6 +606,8 @@ int cntkq_destroy(cntkq_quantizer* h)
         (void) hipFree(h->staging);
     if (h->strip_scratch.dev != nullptr)
         (void) hipFree(h->strip_scratch.dev);
+    for (char* p : h->strip_scratch.retired)
+        (void) hipFree(p);
     if (h->strip_scratch.error_host != nullptr)
         (void) hipHostFree(h->strip_scratch.error_host);
     if (h->strip_scratch.order_event != nullptr)
@@ -681,7 +696,8 @@ int cntkq_wait_quantize_done(cntkq_quantizer* h)
         int rc = sync_event(h->ev_fetch);
         if (rc == CNTKQ_OK)
             h->fetch_pending = false;
-        return rc;
+        // (the copy ran after the kernel: whatever the kernel reported is there by now)
+        return rc != CNTKQ_OK ? rc : check_strip_error(h);
     }
     const int rc = h->last_quantize != nullptr ? sync_event(h->last_quantize) : CNTKQ_OK;
     return rc != CNTKQ_OK ? rc : check_strip_error(h);

@@ -12,6 +12,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
+#include <cstddef>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -385,8 +386,20 @@ inline int check_strip_error(cntkq_quantizer* h)
     if (*static_cast<volatile uint32_t*>(o.error_host) != 0u)
     {
         *o.error_host = 0u;
+        // how many columns: the buffer's count only ever goes up, so the difference to what was seen last is this call's
+        // (a launch replayed on a retired buffer counted there: then the figure is a lower bound)
+        uint32_t now = o.abandoned_seen;
+        // (copied on one of the handle's own streams: the legacy default stream stays out of it)
+        if (o.dev != nullptr &&
+            (hipMemcpyAsync(&now, o.dev + offsetof(cntkq::StripHeader, abandoned), sizeof now, hipMemcpyDeviceToHost, h->fetch) != hipSuccess ||
+             hipStreamSynchronize(h->fetch) != hipSuccess))
+            (void) hipGetLastError();
+        const uint32_t columns = now - o.abandoned_seen;
+        o.abandoned_seen = now;
         return fail(CNTKQ_RUNTIME_ERROR,
-                    "quantize: the workgroups of a column gave up waiting for each other's partial sums; the result of the call is invalid");
+                    "quantize: the workgroups of %s%u column(s) gave up waiting for each other's partial sums; those columns were left as "
+                    "they were (no header, no codes, residual not updated) and the result of the call is invalid",
+                    columns == 0 ? "at least " : "", columns == 0 ? 1u : columns);
     }
     return CNTKQ_OK;
 }
@@ -528,6 +541,10 @@ int unquantize_async_impl(cntkq_quantizer* h, const void* qbuf, size_t qbuf_byte
         return fail(CNTKQ_INVALID_ARGUMENT, "unquantize: %zu x %zu at %zu bits is too large for one launch", rows, cols, nbits);
     HIP_TRY(lrc, "unquantize kernel launch failed");
     h->last_unquantize = ev.stop;
+    // serialised mode: the host waits for the kernel before the call returns (RecordQuantizeCompleteEvent,
+    // Source/Math/MatrixQuantizerGPU.cu:118-122, called at the end of UnquantizeAsync, :338)
+    if (h->force_sync && !stream_capturing(s))
+        HIP_TRY(hipStreamSynchronize(s), "hipStreamSynchronize failed");
     return CNTKQ_OK;
 }
 

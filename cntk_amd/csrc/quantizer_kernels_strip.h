@@ -21,8 +21,15 @@
 // counter tells) raises it, so that replays of a recorded graph see fresh tags like any other launch. The strips of a
 // column take workgroup indices 8 apart: the device's eight dies take the workgroups of a grid in turn, so a column's
 // strips run on one die, next to each other in its queue, and start together (at most 64 of them: all must be resident
-// at once). The wait is bounded all the same: after `spin_limit` polls a lane gives up, raises the error word and goes on
-// with whatever the record holds, so that the grid always drains.
+// at once). That placement is what the hardware does, not what any specification promises, so the wait is bounded: after
+// `spin_limit` polls a lane gives up. A workgroup that gave up raises the error word, marks its own records as abandoned
+// (the launch's tag with the top bit set) and stores nothing: no header, no codes, no residual. A workgroup of the same
+// column that finds an abandoned record abandons its strip in the same way, without waiting. A column whose strips did
+// not all become resident in time is therefore left as it was -- with the residual updated in place, the error feedback
+// of that column survives and the call can be repeated -- and the grid always drains. (What remains open is a strip that
+// is resident, has published its first sum and then stalls for the whole bounded wait before its second exchange: its
+// neighbours abandon the column while it may still complete its own part.) Strip 0 of an abandoned column counts the
+// column in the scratch header.
 #pragma once
 
 #include "quantizer_kernels_common.h"
@@ -80,7 +87,10 @@ struct StripHeader
     } copy[kStripTagCopies];
     uint32_t finished; // groups of workgroups of the running launch that are done; back to zero when the last one is
     uint32_t pad[63];
+    uint32_t abandoned; // columns left untouched because their strips gave up waiting for each other; only ever counted up
+    uint32_t pad2[63];
 };
+constexpr uint32_t kStripAbandoned = 0x80000000u; // top bit of a record's tag: the strip's workgroup gave up; tags proper have 31 bits
 constexpr uint32_t kStripRecords = 4;
 constexpr uint32_t kStripFinishGroup = 64;
 struct StripScratch
@@ -116,31 +126,50 @@ __device__ __forceinline__ void strip_publish(uint64_t* rec, uint32_t value_bits
 // before the first one of an exchange, which with many strips per column practically never finds the record there
 // (262144 x 200, 32 strips: 174 -> 154 us with 64; 24576 x 2048, 3 strips: 116 -> 132 us, so only from 16 strips on).
 template <typename T>
-__device__ __forceinline__ T strip_collect(const uint64_t* recs, uint32_t strips, uint32_t tag, const StripGeom& c, uint32_t first_pause, uint32_t* error)
+__device__ __forceinline__ T strip_collect(const uint64_t* recs, uint32_t strips, uint32_t tag, const StripGeom& c, uint32_t first_pause, bool& gave_up)
 {
     T t = 0;
+    bool bad = false;
     for (uint32_t s = threadIdx.x & 63u; s < strips; s += 64)
     {
         uint32_t polls = 0;
         for (uint32_t z = 0; z < first_pause; ++z)
             __builtin_amdgcn_s_sleep(1);
         uint64_t x;
-        while ((uint32_t) ((x = __hip_atomic_load(recs + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) >> 32) != tag)
+        for (;;)
         {
-            for (uint32_t z = 0; z < c.poll_pause; ++z)
-                __builtin_amdgcn_s_sleep(1);
-            if (++polls >= c.spin_limit)
+            x = __hip_atomic_load(recs + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint32_t got = (uint32_t) (x >> 32);
+            if (got == tag)
+                break;
+            // abandoned by its workgroup, or not there after the bounded wait
+            if (got == (tag | kStripAbandoned) || polls >= c.spin_limit)
             {
-                __hip_atomic_store(error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                bad = true;
                 break;
             }
+            ++polls;
+            for (uint32_t z = 0; z < c.poll_pause; ++z)
+                __builtin_amdgcn_s_sleep(1);
         }
         T val;
         const uint32_t lo = (uint32_t) x;
         __builtin_memcpy(&val, &lo, 4);
         t += val;
     }
+    gave_up = gave_up || __ballot(bad) != 0ull; // the same in every lane of the wavefront
     return wave_sum(t);
+}
+
+// The workgroup abandons its strip: every record of it says so (whichever exchange a neighbour is in, it meets the mark),
+// the host learns of it through the error word, and strip 0 counts the column.
+__device__ __forceinline__ void strip_abandon(uint64_t* recs, uint32_t strip, uint32_t tag, const StripGeom& c, const StripScratch& scratch)
+{
+    for (uint32_t f = 0; f < kStripRecords; ++f)
+        strip_publish(recs + f * c.strips + strip, 0u, tag | kStripAbandoned);
+    __hip_atomic_store(scratch.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (strip == 0)
+        __hip_atomic_fetch_add(&scratch.header->abandoned, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // A workgroup is done with the scratch buffer: the last one of the launch readies the header for the next launch. Atomic
@@ -187,7 +216,7 @@ __device__ __forceinline__ uint32_t strip_block_sum(uint32_t v, uint32_t* red)
 // The column's statistic from the strip's: every workgroup of the column publishes its own and adds all of them in the
 // order of strip_collect. red: the workgroup's reduction slots. Every thread returns the same bits, in every workgroup of the column.
 __device__ __forceinline__ float strip_exchange_stat(float stat, uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
-                                                     const StripScratch& scratch, float* red)
+                                                     const StripScratch& scratch, float* red, bool& ok)
 {
     if (c.strips == 1)
         return stat;
@@ -196,19 +225,26 @@ __device__ __forceinline__ float strip_exchange_stat(float stat, uint32_t column
         strip_publish(recs + strip, __float_as_uint(stat), tag);
     if (threadIdx.x < 64)
     {
-        const float t = strip_collect<float>(recs, c.strips, tag, c, c.poll_first, scratch.error);
+        bool gave_up = false;
+        const float t = strip_collect<float>(recs, c.strips, tag, c, c.poll_first, gave_up);
         if (threadIdx.x == 0)
+        {
             red[0] = t;
+            red[3] = gave_up ? 1.0f : 0.0f;
+            if (gave_up)
+                strip_abandon(recs, strip, tag, c, scratch);
+        }
     }
     __syncthreads();
     const float total = red[0];
+    ok = red[3] == 0.0f;
     __syncthreads();
     return total;
 }
 
 // the same for the sums on either side of the 1-bit threshold and the count below it
 __device__ __forceinline__ void strip_exchange_split(float& s0, float& s1, uint32_t& n0, uint32_t column, uint32_t strip, uint32_t tag,
-                                                     const StripGeom& c, const StripScratch& scratch, float* red)
+                                                     const StripGeom& c, const StripScratch& scratch, float* red, bool& ok)
 {
     if (c.strips == 1)
         return;
@@ -221,52 +257,64 @@ __device__ __forceinline__ void strip_exchange_split(float& s0, float& s1, uint3
     }
     if (threadIdx.x < 64)
     {
-        const float t0 = strip_collect<float>(recs + 1 * c.strips, c.strips, tag, c, c.poll_first, scratch.error);
-        const float t1 = strip_collect<float>(recs + 2 * c.strips, c.strips, tag, c, 0u, scratch.error);
-        const uint32_t tn = strip_collect<uint32_t>(recs + 3 * c.strips, c.strips, tag, c, 0u, scratch.error);
+        bool gave_up = false;
+        const float t0 = strip_collect<float>(recs + 1 * c.strips, c.strips, tag, c, c.poll_first, gave_up);
+        const float t1 = strip_collect<float>(recs + 2 * c.strips, c.strips, tag, c, 0u, gave_up);
+        const uint32_t tn = strip_collect<uint32_t>(recs + 3 * c.strips, c.strips, tag, c, 0u, gave_up);
         if (threadIdx.x == 0)
         {
             red[0] = t0;
             red[1] = t1;
             red[2] = __uint_as_float(tn);
+            red[3] = gave_up ? 1.0f : 0.0f;
+            if (gave_up)
+                strip_abandon(recs, strip, tag, c, scratch);
         }
     }
     __syncthreads();
     s0 = red[0];
     s1 = red[1];
     n0 = __float_as_uint(red[2]);
+    ok = red[3] == 0.0f;
     __syncthreads();
 }
 
 // From the strip's sums to the column's header: the exchanges, the header (written by strip 0) and the release of the
 // scratch buffer. `sums(mean, s0, s1, n0)` gives the strip's split sums (1 bit only), in the same bits in every thread.
+// False (in every thread of the workgroup alike): the column was abandoned and nothing of it may be stored.
 template <int NBITS, bool ZT, typename SplitSums>
-__device__ __forceinline__ void strip_column_range(float stat, SplitSums sums, uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
+__device__ __forceinline__ bool strip_column_range(float stat, SplitSums sums, uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
                                                    const StripScratch& scratch, float* red, char* qc, float& lo, float& hi)
 {
     constexpr bool need_stat = (NBITS != 1) || !ZT;
     float total = 0.0f;
+    bool ok = true;
     if constexpr (need_stat)
-        total = strip_exchange_stat(stat, column, strip, tag, c, scratch, red);
+        total = strip_exchange_stat(stat, column, strip, tag, c, scratch, red, ok);
     if constexpr (NBITS == 1)
     {
-        const float mean = ZT ? 0.0f : total / (float) c.rows;
-        float s0, s1;
-        uint32_t n0;
-        sums(mean, s0, s1, n0);
-        strip_exchange_split(s0, s1, n0, column, strip, tag, c, scratch, red);
-        finish_stats_1bit<ZT>(mean, s0, s1, n0, c.rows - n0, c.rows, lo, hi);
+        // (an abandoned strip takes no part in the second exchange: its records already say so)
+        if (ok)
+        {
+            const float mean = ZT ? 0.0f : total / (float) c.rows;
+            float s0, s1;
+            uint32_t n0;
+            sums(mean, s0, s1, n0);
+            strip_exchange_split(s0, s1, n0, column, strip, tag, c, scratch, red, ok);
+            finish_stats_1bit<ZT>(mean, s0, s1, n0, c.rows - n0, c.rows, lo, hi);
+        }
     }
     else
         finish_stats_multibit(total, c.rows, lo, hi);
     if (c.strips > 1 && threadIdx.x == 0)
         strip_finish(scratch, tag);
-    if (strip == 0 && threadIdx.x == 0)
+    if (ok && strip == 0 && threadIdx.x == 0)
     {
         float* gh = reinterpret_cast<float*>(qc);
         gh[0] = lo;
         gh[1] = hi;
     }
+    return ok;
 }
 
 // A strip with its values in registers: v[kk] = the four values of QWords w ... w + 3 at bit position k0 + kk. FULL: every
@@ -304,8 +352,8 @@ __device__ __forceinline__ void strip_stats_pack(f32x4 (&v)[StripShape<NBITS>::S
             }
         stat = strip_block_sum(stat, red);
     }
-    float lo, hi;
-    strip_column_range<NBITS, ZT>(
+    float lo = 0.0f, hi = 0.0f;
+    const bool column_ok = strip_column_range<NBITS, ZT>(
         stat,
         [&](float mean, float& s0, float& s1, uint32_t& n0) {
             s0 = 0.0f, s1 = 0.0f, n0 = 0;
@@ -327,6 +375,8 @@ __device__ __forceinline__ void strip_stats_pack(f32x4 (&v)[StripShape<NBITS>::S
             n0 = strip_block_sum(n0, red_u);
         },
         column, strip, tag, c, scratch, red, qc, lo, hi);
+    if (!column_ok)
+        return; // abandoned column: codes and residual stay as they were
     const ValueQ vq = make_vq<NBITS>(lo, hi);
     const float val0 = unquantize_value<NBITS>(vq, 0u);
     const float val1 = unquantize_value<NBITS>(vq, 1u);
@@ -424,7 +474,7 @@ __device__ __forceinline__ bool strip_assignment(const StripGeom& c, const Strip
     strip = c.strips - 1 - strip; // the strip at the ragged end of the column, which takes longest, starts first
     // the same tag in every workgroup: the count moves when all of them are done
     const uint32_t copy = (blockIdx.x * (kStripThreads / kWave) + threadIdx.x / kWave) % kStripTagCopies;
-    tag = c.strips > 1 ? __hip_atomic_load(&scratch.header->copy[copy].launches, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u : 0u;
+    tag = c.strips > 1 ? (__hip_atomic_load(&scratch.header->copy[copy].launches, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) % 0x7FFFFFFFu) + 1u : 0u;
     if (column < c.cols)
         return true;
     if (c.strips > 1 && threadIdx.x == 0)

@@ -10,6 +10,7 @@
 #include <stdint.h>
 #include <string.h>
 #include <cstring>
+#include <vector>
 
 namespace cntkq {
 
@@ -46,12 +47,19 @@ struct StripScratchOwner
     hipEvent_t order_event = nullptr;
     hipStream_t last_stream = nullptr;
     bool launched = false;
+    // A launch recorded into a graph (stream capture) has the buffer's addresses in its kernel node and may be replayed at
+    // any time from then on: such a buffer is never freed while the handle lives. When a later launch needs a larger one,
+    // the old buffer is retired (freed with the handle) instead. Graphs must not outlive the handle.
+    bool captured = false;
+    std::vector<char*> retired;
+    uint32_t abandoned_seen = 0; // what the buffer's count of abandoned columns read when the host last looked
 };
 
 struct LaunchTuning
 {
     StripScratchOwner* strip = nullptr; // null: the strip kernels are not available to this launch
     uint32_t strip_spin_limit = 1u << 17; // polls of a partial sum (two microseconds or so each) before a lane gives up
+    bool strip_may_allocate = true; // false: the strip kernels only where the scratch buffer as it stands holds the launch
     int quantize_path = kPathAuto;
     uint32_t tile_gs = 0;   // 0 = pick from rows; else threads per column (power of two, 8..256)
     int tile_stage = -1;    // -1 = automatic; 0 / 1 = residual written straight to memory / staged through LDS
@@ -132,43 +140,46 @@ inline hipError_t dispatch_nbits(size_t nbits, bool zt, Args... args)
     }
 }
 
-template <int NBITS, bool ZT>
-struct TileLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, TileGeom t)
-    {
-        const uint32_t tiles = (t.cols + t.cols_per_tile - 1) / t.cols_per_tile;
-        const size_t lds = tile_lds_bytes(t, 0);
-        hipExtLaunchKernelGGL((quantize_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(t.threads), lds, s, ev.start, ev.stop, 0, g, r_in, r_out, q, t);
-        return hipGetLastError();
-    }
-};
-
-template <int NBITS, bool ZT>
-struct TallLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t rows,
-                          uint32_t cols, uint32_t nq, uint64_t qcol)
-    {
-        hipExtLaunchKernelGGL((quantize_tall_kernel<NBITS, ZT, float>), dim3(cols), dim3(kTallThreads), 0, s, ev.start, ev.stop, 0, g, r_in, r_out, q, rows,
-                           nq, qcol);
-        return hipGetLastError();
-    }
-};
-
-template <int NBITS, bool ZT>
-struct StripeLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
-                          TileGeom t)
-    {
-        const uint32_t tiles = (t.cols + t.cols_per_tile - 1) / t.cols_per_tile;
-        const size_t lds = tile_lds_bytes(t, src.workers);
-        hipExtLaunchKernelGGL((stripe_reduce_tile_kernel<NBITS, ZT>), dim3(tiles), dim3(t.threads), lds, s, ev.start, ev.stop, 0, src, stripe_res,
-                           q_out, agg_out, t);
-        return hipGetLastError();
-    }
-};
+// ---- the kernel families ----------------------------------------------------------------------------------------------
+// Each family of kernels is instantiated in a source file of its own (quantizer_family_*.hip), so that the families
+// compile side by side and a source file that only plans launches (the C ABI, the double-precision instantiation) carries
+// no copy of them. nbits is 1, 2, 4, 8, 16 or 32; zt only matters at 1 bit. hipErrorInvalidValue: the family has no
+// kernel for the arguments.
+struct UnquantizePlan;
+hipError_t family_tile_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, TileGeom t);
+hipError_t family_tile_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out,
+                              float* agg_out, TileGeom t);
+hipError_t family_tall_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q,
+                                uint32_t rows, uint32_t cols, uint32_t nq, uint64_t qcol);
+hipError_t family_col_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q,
+                               uint32_t cols, ColGeom c);
+// per: 1, 2 or 4 pieces per thread (1024, 2048, 4096 rows at 1 bit)
+hipError_t family_col_quantize_unrolled(bool zt, int per, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q,
+                                        uint32_t cols, uint64_t qcol);
+hipError_t family_col_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out,
+                             float* agg_out, uint32_t cols, ColGeom c);
+hipError_t family_col_stripe_unrolled(bool zt, int per, hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out,
+                                      float* agg_out, uint32_t cols, uint64_t qcol);
+// threads: 256 or 1024 per column
+hipError_t family_reg_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q,
+                               uint32_t cols, RegGeom c, uint32_t threads);
+hipError_t family_reg_edge_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q,
+                                    uint32_t cols, RegGeom c, uint32_t threads);
+hipError_t family_regs_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q,
+                                uint32_t cols, RegGeom c);
+hipError_t family_reg_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out,
+                             float* agg_out, uint32_t cols, RegGeom c, uint32_t threads);
+hipError_t family_strip_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q,
+                                 uint32_t cols, StripGeom c, StripScratch scratch);
+// workgroups of the strip kernel that the runtime says a compute unit holds at once
+hipError_t family_strip_occupancy(size_t nbits, bool zt, int* per_cu);
+hipError_t family_unquantize(size_t nbits, hipStream_t s, LaunchEvents ev, const char* q, float* out, const UnquantizePlan& p, int add);
+hipError_t family_batch_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const QuantizeBatchEntry* entries, const uint32_t* begins,
+                                 uint32_t count, uint32_t total_blocks, size_t lds);
+hipError_t family_batch_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const StripeBatchEntry* entries, const uint32_t* begins,
+                               uint32_t count, uint32_t total_blocks, size_t lds, bool wide);
+hipError_t launch_unquantize_batch(hipStream_t s, LaunchEvents ev, const UnquantizeBatchEntry* entries, const uint32_t* begins, uint32_t count,
+                                   uint32_t total_blocks, size_t nbits, bool add, size_t lds);
 
 // forced = the caller insists on the column kernels: any height they can handle; otherwise only where they pay
 inline bool col_applicable(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits,
@@ -223,45 +234,6 @@ inline ColGeom make_col_geom(size_t rows, size_t nbits, bool line_shift)
     return c;
 }
 
-template <int NBITS, bool ZT>
-struct ColLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, ColGeom c)
-    {
-        hipExtLaunchKernelGGL((quantize_colg_kernel<NBITS, ZT>), dim3(cols), dim3(kColThreads), colg_lds_bytes<NBITS>(c, 0), s, ev.start,
-                              ev.stop, 0, g, r_in, r_out, q, c);
-        return hipGetLastError();
-    }
-};
-
-template <int NBITS, bool ZT>
-struct StripeColLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
-                          uint32_t cols, ColGeom c)
-    {
-        // Every work item (a QWord, or a chunk of its bit positions) is a chain of dependent loads, and the column's LDS
-        // limits how many workgroups a CU holds: from 24 KB per column on (6 workgroups or fewer per CU) 512 threads keep
-        // the CU's wavefront slots filled, and where the stripe has no more columns than the device has CUs, 1024 do.
-        // Measured at 8 workers, 256 / 512 / 1024 threads: 9304 x 2048 at 2 bits 62 / 58 / 84 us, 14336 x 1328 at 4 bits
-        // 91 / 68 / 80, 4096 x 4652 at 8 bits 67 / 75 / 114, 6144 x 3101 at 2 bits 55 / 59 / 99, 14336 x 256 at 2 bits
-        // 28 / 19 / 15, 8192 x 300 at 8 bits 23 / 16 / 20.
-        uint32_t wg = 256u;
-        if (c.nq * PackShape<NBITS>::CHUNKS >= kStripeWideItems)
-            wg = cols <= kStripeWideMaxCols ? 1024u : (c.rows > kStripeMidMinRows ? 512u : 256u);
-        if (wg == 1024)
-            hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, 1024>), dim3(cols), dim3(1024), colg_lds_bytes<NBITS>(c, src.workers),
-                                  s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
-        else if (wg == 512)
-            hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, 512>), dim3(cols), dim3(512), colg_lds_bytes<NBITS>(c, src.workers),
-                                  s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
-        else
-            hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, kColThreads>), dim3(cols), dim3(kColThreads),
-                                  colg_lds_bytes<NBITS>(c, src.workers), s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
-        return hipGetLastError();
-    }
-};
-
 inline RegGeom make_reg_geom(size_t rows, size_t nbits, uint32_t threads, bool line_shift)
 {
     RegGeom c;
@@ -273,110 +245,6 @@ inline RegGeom make_reg_geom(size_t rows, size_t nbits, uint32_t threads, bool l
     c.line_shift = line_shift ? 1u : 0u;
     c.qcol = qcol_bytes(nbits, rows);
     return c;
-}
-
-template <int NBITS, bool ZT, int T, int PER>
-inline hipError_t launch_reg_one(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
-                                 const RegGeom& c)
-{
-    hipExtLaunchKernelGGL((quantize_reg_kernel<NBITS, ZT, T, PER>), dim3(cols), dim3(T), reg_lds_bytes(c), s, ev.start, ev.stop, 0, g, r_in,
-                          r_out, q, c);
-    return hipGetLastError();
-}
-
-template <int NBITS, bool ZT, int PER, int T = 1024>
-inline hipError_t launch_reg_edge_one(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
-                                      const RegGeom& c)
-{
-    hipExtLaunchKernelGGL((quantize_reg_kernel<NBITS, ZT, T, PER, true>), dim3(cols), dim3(T), reg_lds_bytes(c), s, ev.start, ev.stop, 0,
-                          g, r_in, r_out, q, c);
-    return hipGetLastError();
-}
-
-// The variant for columns that start anywhere and have any height: c.pieces is an upper bound. 256 threads up to
-// kRegEdgeMinRows rows (2049 x 9304: the tile kernel's 57 us), 1024 above.
-template <int NBITS, bool ZT>
-struct RegEdgeLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, RegGeom c,
-                          uint32_t threads)
-    {
-        if constexpr (NBITS >= 32)
-            return hipErrorInvalidValue;
-        else
-        {
-            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + threads - 1) / threads;
-#define CNTKQ_REGE256(P) if (threads == 256 && per <= P) return launch_reg_edge_one<NBITS, ZT, P, 256>(s, ev, g, r_in, r_out, q, cols, c)
-            CNTKQ_REGE256(3);
-            CNTKQ_REGE256(4);
-            CNTKQ_REGE256(6);
-            CNTKQ_REGE256(8);
-#undef CNTKQ_REGE256
-            if (threads != 1024)
-                return hipErrorInvalidValue;
-#define CNTKQ_REGE(P) if (per <= P) return launch_reg_edge_one<NBITS, ZT, P>(s, ev, g, r_in, r_out, q, cols, c)
-            CNTKQ_REGE(4);
-            CNTKQ_REGE(6);
-            CNTKQ_REGE(8);
-            CNTKQ_REGE(10);
-            CNTKQ_REGE(13);
-            CNTKQ_REGE(16);
-            CNTKQ_REGE(20);
-            CNTKQ_REGE(25);
-#undef CNTKQ_REGE
-            return hipErrorInvalidValue;
-        }
-    }
-};
-
-template <int NBITS, bool ZT>
-struct RegLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, RegGeom c,
-                          uint32_t threads)
-    {
-        if constexpr (NBITS >= 32)
-            return hipErrorInvalidValue;
-        else
-        {
-            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + threads - 1) / threads; // up to 7 slots lie before the column
-#define CNTKQ_REG(T, P) if (threads == T && per <= P) return launch_reg_one<NBITS, ZT, T, P>(s, ev, g, r_in, r_out, q, cols, c)
-            CNTKQ_REG(256, 3);
-            CNTKQ_REG(256, 4);
-            CNTKQ_REG(256, 6);
-            CNTKQ_REG(256, 8);
-            CNTKQ_REG(256, 10);
-            CNTKQ_REG(256, 12);
-            CNTKQ_REG(256, 14);
-            CNTKQ_REG(256, 16);
-            CNTKQ_REG(1024, 4);
-            CNTKQ_REG(1024, 6);
-            CNTKQ_REG(1024, 8);
-            CNTKQ_REG(1024, 10);
-            CNTKQ_REG(1024, 13);
-            CNTKQ_REG(1024, 16);
-            CNTKQ_REG(1024, 20);
-            CNTKQ_REG(1024, 25);
-#undef CNTKQ_REG
-            return hipErrorInvalidValue;
-        }
-    }
-};
-
-template <bool ZT, int PER>
-inline void launch_quantize_col(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
-                                uint64_t qcol)
-{
-    hipExtLaunchKernelGGL((quantize_col_kernel<ZT, PER>), dim3(cols), dim3(kColThreads), col_lds_bytes<PER>(), s, ev.start, ev.stop, 0, g,
-                          r_in, r_out, q, qcol);
-}
-
-template <bool ZT, int PER>
-inline void launch_stripe_col(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
-                              uint32_t cols, uint64_t qcol)
-{
-    hipExtLaunchKernelGGL((stripe_reduce_col_kernel<ZT, PER>), dim3(cols), dim3(kColThreads), col_lds_bytes<PER>() + kStripeColExtraLds, s,
-                          ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, qcol);
 }
 
 // The register kernels: above 1024 rows (unless forced; 37.7 M elements at 1152 / 1536 / 2000 rows: 95 / 76 / 72 us against
@@ -438,39 +306,6 @@ inline bool regs_applicable(size_t rows, size_t nbits)
     return rows >= 1 && rows <= kRegsMaxRows && nbits < 32 && (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
 }
 
-template <int NBITS, bool ZT, int EPT>
-inline hipError_t launch_regs_one(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols,
-                                  const RegGeom& c)
-{
-    hipExtLaunchKernelGGL((quantize_regs_kernel<NBITS, ZT, EPT>), dim3(cols), dim3(kRegsThreads), reg_lds_bytes(c), s, ev.start, ev.stop, 0, g,
-                          r_in, r_out, q, c);
-    return hipGetLastError();
-}
-
-template <int NBITS, bool ZT>
-struct RegsLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, RegGeom c)
-    {
-        if constexpr (NBITS >= 32)
-            return hipErrorInvalidValue;
-        else
-        {
-            const uint32_t ept = (c.rows + kRegsThreads - 1) / kRegsThreads;
-#define CNTKQ_REGS(E) if (ept <= E) return launch_regs_one<NBITS, ZT, E>(s, ev, g, r_in, r_out, q, cols, c)
-            CNTKQ_REGS(16);
-            CNTKQ_REGS(24);
-            CNTKQ_REGS(32);
-            CNTKQ_REGS(48);
-            CNTKQ_REGS(64);
-            CNTKQ_REGS(80);
-            CNTKQ_REGS(96);
-#undef CNTKQ_REGS
-            return hipErrorInvalidValue;
-        }
-    }
-};
-
 // ---- strip kernels: any height, several workgroups per column ------------------------------------------------------
 
 
@@ -528,9 +363,16 @@ inline hipError_t strip_scratch_for(StripScratchOwner& o, hipStream_t s, size_t 
         if (rc != hipSuccess)
             return rc;
         if (o.dev != nullptr)
-            (void) hipFree(o.dev);
+        {
+            if (o.captured)
+                o.retired.push_back(o.dev); // a recorded launch may still be replayed on it
+            else
+                (void) hipFree(o.dev);
+        }
         o.dev = nullptr;
         o.bytes = 0;
+        o.captured = false;
+        o.abandoned_seen = 0;
         const size_t need = sizeof(StripHeader) + strip_records_bytes(cols, strips);
         const size_t cap = std::max<size_t>((need * 2 + 8191) & ~(size_t) 4095, (size_t) 1 << 20);
         void* p = nullptr;
@@ -556,11 +398,14 @@ inline hipError_t strip_scratch_for(StripScratchOwner& o, hipStream_t s, size_t 
     return hipSuccess;
 }
 
-// whether this launch finds its scratch buffer without allocating, or may allocate (the stream is not being captured)
-inline bool strip_scratch_ready(const StripScratchOwner& o, hipStream_t s, size_t cols, size_t strips)
+// whether this launch finds its scratch buffer without allocating, or may allocate (the caller permits it and the stream
+// is not being captured)
+inline bool strip_scratch_ready(const StripScratchOwner& o, hipStream_t s, size_t cols, size_t strips, bool may_allocate = true)
 {
     if (o.error_host != nullptr && strip_scratch_fits(o, cols, strips))
         return true;
+    if (!may_allocate)
+        return false;
     hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
     return hipStreamIsCapturing(s, &st) == hipSuccess && st == hipStreamCaptureStatusNone;
 }
@@ -570,22 +415,30 @@ inline uint32_t strip_grid(size_t cols, size_t strips)
     return (uint32_t) ((cols + kStripDies - 1) / kStripDies * kStripDies * strips);
 }
 
-template <int NBITS, bool ZT>
-struct StripLauncher
+// How many strips a column may have for the automatic choice to take the strip kernels: the strips of a column wait for
+// each other on one die, so all of them must be resident there together, next to the strips of the columns around them.
+// Half of what the die holds by the runtime's own occupancy figure for the kernel (workgroups per compute unit x compute
+// units of the device / 8 dies); 0 where the runtime cannot say. Asked once per kernel variant and device.
+inline uint32_t strip_resident_limit(size_t nbits, bool zt)
 {
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, StripGeom c,
-                          StripScratch scratch)
+    static int cache[64][6][2]; // 0: not asked yet; -1: unknown
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return 0;
+    const int b = nbits == 1 ? 0 : nbits == 2 ? 1 : nbits == 4 ? 2 : nbits == 8 ? 3 : 4;
+    int& slot = cache[dev][b][zt ? 1 : 0];
+    if (slot == 0)
     {
-        if constexpr (NBITS >= 32)
-            return hipErrorInvalidValue;
-        else
-        {
-            hipExtLaunchKernelGGL((quantize_strip_kernel<NBITS, ZT>), dim3(strip_grid(cols, c.strips)), dim3(kStripThreads), strip_lds_bytes(NBITS), s,
-                                  ev.start, ev.stop, 0, g, r_in, r_out, q, c, scratch);
-            return hipGetLastError();
-        }
+        int per_cu = 0, cus = 0;
+        hipError_t rc = family_strip_occupancy(nbits, zt, &per_cu);
+        if (rc == hipSuccess)
+            rc = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (rc != hipSuccess)
+            (void) hipGetLastError();
+        slot = (rc == hipSuccess && per_cu > 0 && cus >= (int) kStripDies) ? per_cu * (cus / (int) kStripDies) / 2 : -1;
     }
-};
+    return slot > 0 ? (uint32_t) slot : 0u;
+}
 
 // which path launch_quantize takes for this matrix when nothing is forced
 inline int quantize_auto_path(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits,
@@ -627,7 +480,8 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
         {
             // a stream under capture cannot wait for a larger scratch buffer: the kernels that need none take the matrix
             const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit);
-            if ((uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull || !strip_scratch_ready(*tune.strip, s, cols, c.strips))
+            if ((uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull ||
+                !strip_scratch_ready(*tune.strip, s, cols, c.strips, tune.strip_may_allocate) || c.strips > strip_resident_limit(nbits, zt))
                 path = regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
         }
     }
@@ -640,13 +494,13 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
                 return hipErrorInvalidValue;
             const uint32_t threads = reg_edge_threads(rows);
             RegGeom c = make_reg_geom(rows, nbits, threads, true); // always dealt by the residual's lines
-            return dispatch_nbits<RegEdgeLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, threads);
+            return family_reg_edge_quantize(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, threads);
         }
         const uint32_t threads = reg_threads(rows);
         // up to 14336 rows the shift is part of the summation order all column kernels share; above, it is used where
         // the registers allow
         const bool line_shift = quantize_line_shift(g, r_in, r_out, rows) && (threads == 256 || rows / 4 + 7 <= 1024 * (size_t) kRegMaxShiftPer);
-        return dispatch_nbits<RegLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols,
+        return family_reg_quantize(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols,
                                            make_reg_geom(rows, nbits, threads, line_shift), threads);
     }
     if (path == kPathStrip)
@@ -661,6 +515,8 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
             return rc;
         hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
         const bool capturing = hipStreamIsCapturing(s, &st) != hipSuccess || st != hipStreamCaptureStatusNone;
+        if (capturing)
+            o.captured = true;
         if (!capturing)
         {
             if (o.order_event == nullptr && (rc = hipEventCreateWithFlags(&o.order_event, hipEventDisableTiming)) != hipSuccess)
@@ -668,7 +524,7 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
             if (o.launched && o.last_stream != s && (rc = hipStreamWaitEvent(s, o.order_event, 0)) != hipSuccess)
                 return rc;
         }
-        rc = dispatch_nbits<StripLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, scratch);
+        rc = family_strip_quantize(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, scratch);
         if (rc == hipSuccess && !capturing)
         {
             rc = hipEventRecord(o.order_event, s);
@@ -684,7 +540,7 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
         RegGeom c = make_reg_geom(rows, nbits, kRegsThreads, false);
         c.step_k = kRegsThreads / c.nq; // a thread's next element lies 1024 elements further on
         c.step_w = kRegsThreads % c.nq;
-        return dispatch_nbits<RegsLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c);
+        return family_regs_quantize(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c);
     }
     if (path == kPathCol)
     {
@@ -693,25 +549,19 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
         // (the unrolled kernels deal pieces without a shift: only for columns that start on lines)
         const bool line_shift = quantize_line_shift(g, r_in, r_out, rows);
         if (line_shift || !col_unrolled(q, rows, nbits))
-            return dispatch_nbits<ColLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, make_col_geom(rows, nbits, line_shift));
+            return family_col_quantize(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, make_col_geom(rows, nbits, line_shift));
         const uint64_t qcol = qcol_bytes(nbits, rows);
         const uint32_t c = (uint32_t) cols;
-        if (rows == 1024)
-            zt ? launch_quantize_col<true, 1>(s, ev, g, r_in, r_out, qc, c, qcol) : launch_quantize_col<false, 1>(s, ev, g, r_in, r_out, qc, c, qcol);
-        else if (rows == 2048)
-            zt ? launch_quantize_col<true, 2>(s, ev, g, r_in, r_out, qc, c, qcol) : launch_quantize_col<false, 2>(s, ev, g, r_in, r_out, qc, c, qcol);
-        else
-            zt ? launch_quantize_col<true, 4>(s, ev, g, r_in, r_out, qc, c, qcol) : launch_quantize_col<false, 4>(s, ev, g, r_in, r_out, qc, c, qcol);
-        return hipGetLastError();
+        return family_col_quantize_unrolled(zt, rows == 1024 ? 1 : (rows == 2048 ? 2 : 4), s, ev, g, r_in, r_out, qc, c, qcol);
     }
     if (path == kPathTile)
     {
         if (rows > kTileMaxRows)
             return hipErrorInvalidValue;
         const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs, tune.tile_stage, tune.tile_threads);
-        return dispatch_nbits<TileLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, t);
+        return family_tile_quantize(nbits, zt, s, ev, g, r_in, r_out, qc, t);
     }
-    return dispatch_nbits<TallLauncher>(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) rows, (uint32_t) cols,
+    return family_tall_quantize(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) rows, (uint32_t) cols,
                                         (uint32_t) qwords_per_col(rows, nbits), (uint64_t) qcol_bytes(nbits, rows));
 }
 
@@ -727,75 +577,6 @@ inline size_t stripe_reduce_max_rows(size_t nbits)
     const size_t tall = by_lds < by_regs ? by_lds : by_regs;
     return tall > kTileMaxRows ? tall : kTileMaxRows;
 }
-
-template <int NBITS, bool ZT, int PER, int T = 1024>
-inline hipError_t launch_stripe_reg_one(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
-                                        uint32_t cols, const RegGeom& c)
-{
-    if constexpr (NBITS == 1)
-    {
-        // up to eight workers: the row sums looked up in a table of 256 (the same additions, made once per column)
-        if (src.workers <= 8 && stripe_lut_lds_bytes(c) <= 160 * 1024)
-        {
-            hipExtLaunchKernelGGL((stripe_reduce_lut_kernel<ZT, PER, T>), dim3(cols), dim3(T), stripe_lut_lds_bytes(c), s, ev.start, ev.stop, 0, src,
-                                  stripe_res, q_out, agg_out, c);
-            return hipGetLastError();
-        }
-    }
-    if constexpr (NBITS == 1 && T == 1024)
-    {
-        // 1 bit: eight workers at a time from the worker-minor table, where a CU's LDS holds it (always, up to 102400 rows)
-        // (it always decodes eight slots: with four workers or fewer the kernel below does less work)
-        if (src.workers > 4 && stripe_reg8_lds_bytes(c) <= 160 * 1024)
-        {
-            hipExtLaunchKernelGGL((stripe_reduce_reg8_kernel<ZT, PER>), dim3(cols), dim3(1024), stripe_reg8_lds_bytes(c), s, ev.start, ev.stop, 0,
-                                  src, stripe_res, q_out, agg_out, c);
-            return hipGetLastError();
-        }
-    }
-    const uint32_t group = stripe_reg_group(c, src.workers);
-    hipExtLaunchKernelGGL((stripe_reduce_reg_kernel<NBITS, ZT, PER, T>), dim3(cols), dim3(T), stripe_reg_lds_bytes(c, group), s, ev.start,
-                          ev.stop, 0, src, stripe_res, q_out, agg_out, c, group);
-    return hipGetLastError();
-}
-
-template <int NBITS, bool ZT>
-struct StripeRegLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out, uint32_t cols,
-                          RegGeom c, uint32_t threads)
-    {
-        if constexpr (NBITS >= 32)
-            return hipErrorInvalidValue;
-        else
-        {
-            const uint32_t per = (c.pieces + (c.line_shift ? 7u : 0u) + threads - 1) / threads;
-#define CNTKQ_SREG256(P) if (threads == 256 && per <= P) return launch_stripe_reg_one<NBITS, ZT, P, 256>(s, ev, src, stripe_res, q_out, agg_out, cols, c)
-            CNTKQ_SREG256(3);
-            CNTKQ_SREG256(4);
-            CNTKQ_SREG256(6);
-            CNTKQ_SREG256(8);
-            CNTKQ_SREG256(10);
-            CNTKQ_SREG256(12);
-            CNTKQ_SREG256(14);
-            CNTKQ_SREG256(16);
-#undef CNTKQ_SREG256
-            if (threads != 1024)
-                return hipErrorInvalidValue;
-#define CNTKQ_SREG(P) if (per <= P) return launch_stripe_reg_one<NBITS, ZT, P>(s, ev, src, stripe_res, q_out, agg_out, cols, c)
-            CNTKQ_SREG(4);
-            CNTKQ_SREG(6);
-            CNTKQ_SREG(8);
-            CNTKQ_SREG(10);
-            CNTKQ_SREG(13);
-            CNTKQ_SREG(16);
-            CNTKQ_SREG(20);
-            CNTKQ_SREG(25);
-#undef CNTKQ_SREG
-            return hipErrorInvalidValue;
-        }
-    }
-};
 
 // Whether a stripe whose height and alignment would let the LDS column kernels take it goes to the table-driven register
 // kernel with 256 threads instead (1 bit, up to eight workers, above 2048 rows), and how many pieces a thread holds there.
@@ -838,7 +619,7 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
         // (only stripes that are not whole aligned pieces get here below the LDS kernels' limit: 256 threads up to 7168 rows)
         const uint32_t threads = rows > kTileMaxRows ? 1024u : reg_edge_threads(rows);
         const RegGeom c = make_reg_geom(rows, nbits, threads, line_shift);
-        return dispatch_nbits<StripeRegLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols, c,
+        return family_reg_stripe(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols, c,
                                                  threads);
     }
     bool aligned8 = (reinterpret_cast<uintptr_t>(q_out) & 7u) == 0;
@@ -858,10 +639,10 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
         if (tune.quantize_path == kPathAuto && stripe_looks_up(rows, nbits, src.workers))
         {
             const RegGeom c = make_reg_geom(rows, nbits, 256, line_shift);
-            return dispatch_nbits<StripeRegLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols, c,
+            return family_reg_stripe(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols, c,
                                                      256u);
         }
-        return dispatch_nbits<StripeColLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols,
+        return family_col_stripe(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols,
                                                  make_col_geom(rows, nbits, line_shift));
     }
     if (col)
@@ -870,18 +651,12 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
         const uint64_t qcol = qcol_bytes(nbits, rows);
         const uint32_t c = (uint32_t) cols;
         char* qo = static_cast<char*>(q_out);
-        if (rows == 1024)
-            zt ? launch_stripe_col<true, 1>(s, ev, src, stripe_res, qo, agg_out, c, qcol) : launch_stripe_col<false, 1>(s, ev, src, stripe_res, qo, agg_out, c, qcol);
-        else if (rows == 2048)
-            zt ? launch_stripe_col<true, 2>(s, ev, src, stripe_res, qo, agg_out, c, qcol) : launch_stripe_col<false, 2>(s, ev, src, stripe_res, qo, agg_out, c, qcol);
-        else
-            zt ? launch_stripe_col<true, 4>(s, ev, src, stripe_res, qo, agg_out, c, qcol) : launch_stripe_col<false, 4>(s, ev, src, stripe_res, qo, agg_out, c, qcol);
-        return hipGetLastError();
+        return family_col_stripe_unrolled(zt, rows == 1024 ? 1 : (rows == 2048 ? 2 : 4), s, ev, src, stripe_res, qo, agg_out, c, qcol);
     }
     // Same tile geometry as launch_quantize would use for a matrix of this height, so that the statistics are summed in
     // the same order and the fused call gives the bytes of the reference's unquantize ... quantize call sequence.
     const TileGeom t = make_tile_geom(rows, cols, nbits, tune.tile_gs, tune.tile_stage, tune.tile_threads);
-    return dispatch_nbits<StripeLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, t);
+    return family_tile_stripe(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, t);
 }
 
 // ---- unquantize: which decoder, with which geometry ---------------------------------------------------
@@ -1060,87 +835,31 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
     return p;
 }
 
-template <int NBITS>
-inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const char* q, float* out, const UnquantizePlan& p, int add)
-{
-    if (p.kind == kUnqTile)
-        hipExtLaunchKernelGGL((unquantize_tile_kernel<NBITS, float>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.tile, add);
-    else if (p.kind == kUnqRows)
-        hipExtLaunchKernelGGL((unquantize_rows_kernel<NBITS, float>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.rowg, add);
-    else if (p.kind == kUnqSegment)
-        hipExtLaunchKernelGGL((unquantize_segment_kernel<NBITS>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.seg, add);
-    else if (p.kind == kUnqVec4)
-        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 4, float>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.qw, add);
-    else
-        hipExtLaunchKernelGGL((unquantize_kernel<NBITS, 1, float>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.qw, add);
-    return hipGetLastError();
-}
-
 inline hipError_t launch_unquantize(hipStream_t s, LaunchEvents ev, const void* q, float* out, size_t rows, size_t cols, size_t nbits,
                                     bool add, const LaunchTuning& tune)
 {
     const UnquantizePlan p = plan_unquantize(q, out, rows, cols, nbits, tune);
     if (!p.ok)
         return hipErrorInvalidValue;
-    const char* qc = static_cast<const char*>(q);
-    const int a = add ? 1 : 0;
-    switch (nbits)
-    {
-    case 1: return launch_unquantize_plan<1>(s, ev, qc, out, p, a);
-    case 2: return launch_unquantize_plan<2>(s, ev, qc, out, p, a);
-    case 4: return launch_unquantize_plan<4>(s, ev, qc, out, p, a);
-    case 8: return launch_unquantize_plan<8>(s, ev, qc, out, p, a);
-    case 16: return launch_unquantize_plan<16>(s, ev, qc, out, p, a);
-    case 32: return launch_unquantize_plan<32>(s, ev, qc, out, p, a);
-    default: return hipErrorInvalidValue;
-    }
+    return family_unquantize(nbits, s, ev, static_cast<const char*>(q), out, p, add ? 1 : 0);
 }
 
 // ---- many matrices per launch -----------------------------------------------------------------------
 // The entry tables live in device memory; the caller (the C-ABI layer) owns them and keeps them alive until the
 // kernel has finished.
 
-template <int NBITS, bool ZT>
-struct BatchLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const QuantizeBatchEntry* entries, const uint32_t* begins, uint32_t count,
-                          uint32_t total_blocks, size_t lds)
-    {
-        static_assert(kTileThreads == kColThreads, "tiles and columns share one workgroup size in a batch");
-        hipExtLaunchKernelGGL((quantize_batch_kernel<NBITS, ZT>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start, ev.stop, 0,
-                              entries, begins, count);
-        return hipGetLastError();
-    }
-};
-
 inline hipError_t launch_quantize_batch(hipStream_t s, LaunchEvents ev, const QuantizeBatchEntry* entries, const uint32_t* begins,
                                         uint32_t count, uint32_t total_blocks, size_t lds, size_t nbits, bool zt)
 {
     zt = zt && (nbits == 1);
-    return dispatch_nbits<BatchLauncher>(nbits, zt, s, ev, entries, begins, count, total_blocks, lds);
+    return family_batch_quantize(nbits, zt, s, ev, entries, begins, count, total_blocks, lds);
 }
-
-template <int NBITS, bool ZT>
-struct StripeBatchLauncher
-{
-    static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeBatchEntry* entries, const uint32_t* begins, uint32_t count,
-                          uint32_t total_blocks, size_t lds, bool wide)
-    {
-        if (wide && NBITS == 1)
-            hipExtLaunchKernelGGL((stripe_reduce_batch_kernel<NBITS, ZT, NBITS == 1>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start,
-                                  ev.stop, 0, entries, begins, count);
-        else
-            hipExtLaunchKernelGGL((stripe_reduce_batch_kernel<NBITS, ZT, false>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start,
-                                  ev.stop, 0, entries, begins, count);
-        return hipGetLastError();
-    }
-};
 
 inline hipError_t launch_stripe_reduce_batch(hipStream_t s, LaunchEvents ev, const StripeBatchEntry* entries, const uint32_t* begins,
                                              uint32_t count, uint32_t total_blocks, size_t lds, size_t nbits, bool zt, bool wide)
 {
     zt = zt && (nbits == 1);
-    return dispatch_nbits<StripeBatchLauncher>(nbits, zt, s, ev, entries, begins, count, total_blocks, lds, wide);
+    return family_batch_stripe(nbits, zt, s, ev, entries, begins, count, total_blocks, lds, wide);
 }
 
 // which kernel family launch_stripe_reduce takes by itself for a stripe of this height: columns (true) or tiles
@@ -1153,23 +872,6 @@ inline bool stripe_auto_col(size_t rows, const void* stripe_res)
 inline size_t colg_lds_bytes_rt(const ColGeom& c, size_t nbits)
 {
     return ((size_t) c.rows + (nbits <= 2 ? c.nq : 0) + 12) * sizeof(float);
-}
-
-inline hipError_t launch_unquantize_batch(hipStream_t s, LaunchEvents ev, const UnquantizeBatchEntry* entries, const uint32_t* begins,
-                                          uint32_t count, uint32_t total_blocks, size_t nbits, bool add, size_t lds)
-{
-    const int a = add ? 1 : 0;
-    switch (nbits)
-    {
-    case 1: hipExtLaunchKernelGGL((unquantize_batch_kernel<1>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    case 2: hipExtLaunchKernelGGL((unquantize_batch_kernel<2>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    case 4: hipExtLaunchKernelGGL((unquantize_batch_kernel<4>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    case 8: hipExtLaunchKernelGGL((unquantize_batch_kernel<8>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    case 16: hipExtLaunchKernelGGL((unquantize_batch_kernel<16>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    case 32: hipExtLaunchKernelGGL((unquantize_batch_kernel<32>), dim3(total_blocks), dim3(256), lds, s, ev.start, ev.stop, 0, entries, begins, count, a); break;
-    default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
 }
 
 

@@ -29,8 +29,11 @@
  * matching cntkq_wait_* call then has nothing to wait for and returns at once: order against a replay with the graph's
  * own launch stream. A batched call must have run once outside the capture with the same item list (its argument
  * table is built and uploaded then); after a capture that table is never written again -- a later call with another
- * list builds a new one -- so graphs stay valid until the handle is destroyed. Packed matrices in host memory
- * (qbuf_on_host) are refused during capture.
+ * list builds a new one -- so graphs stay valid until the handle is destroyed. The same holds for the scratch buffer of
+ * the kernels that cut very tall columns into strips: once a launch on it has been recorded, the buffer is kept until the
+ * handle is destroyed, and a later launch that needs a larger one takes a new buffer. A graph must not be replayed after
+ * the handle it was recorded from has been destroyed. Packed matrices in host memory (qbuf_on_host) are refused during
+ * capture.
  */
 #ifndef CNTK_AMD_QUANTIZER_H
 #define CNTK_AMD_QUANTIZER_H
@@ -127,7 +130,11 @@ int cntkq_quantize_async(cntkq_quantizer* h, const float* in, const float* res_i
                          int zero_threshold_for_1bit);
 
 /* MatrixQuantizerImpl::WaitQuantizeAsyncDone (Source/Math/MatrixQuantizerGPU.cu:271-284): blocks the host
- * until the last quantize of this handle (including its copy to the host, if any) has finished. */
+ * until the last quantize of this handle (including its copy to the host, if any) has finished.
+ * CNTKQ_RUNTIME_ERROR here can also mean that a launch on columns of more than 102400 rows did not complete: the
+ * workgroups that share such a column wait for each other a bounded time, and a column whose workgroups gave up is left
+ * as it was -- no header, no codes, residual not updated, also when res_out == res_in -- so the call may be repeated.
+ * The error text says how many columns. The other columns of the call are complete and right. */
 int cntkq_wait_quantize_done(cntkq_quantizer* h);
 
 /* MatrixQuantizerImpl::UnquantizeAsync (Source/Math/MatrixQuantizerImpl.h:33, Source/Math/MatrixQuantizerGPU.cu:286-334).
@@ -176,7 +183,7 @@ int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item
 
 /* cntkq_quantize_batch_async for callers that cannot allocate. It has no counterpart in the reference; it is for code
  * under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc. Same arguments, same kernels and the
- * same bytes as cntkq_quantize_batch_async, but the call touches no allocator, device or host: the argument table that
+ * same bytes as cntkq_quantize_batch_async (one exception below), but the call touches no allocator, device or host: the argument table that
  * the batched kernels read (the only memory of that call beyond its inputs and outputs) lives in a fixed array in the
  * library's device image -- 32 KB, held by every GPU the library runs on until the process ends -- and reaches it as
  * kernel arguments of a small store kernel, not through a copy.
@@ -185,7 +192,13 @@ int cntkq_unquantize_batch_async(cntkq_quantizer* h, const cntkq_unquantize_item
  *   CNTKQ_INVALID_ARGUMENT and does nothing.
  *   The array is shared by every call on that GPU and keeps the last call's contents. Calls on one stream are ordered
  *   like any other stream work; calls that can overlap on one GPU (other streams, other handles on other streams) race
- *   for the array and must be ordered by the caller.
+ *   for the array and must be ordered by the caller. A call recorded into a graph writes the array at every replay; from
+ *   the first such call on a GPU every call on that GPU uploads its table (a few small launches) instead of trusting
+ *   what the array held last.
+ *   Columns above 102400 rows: the batched call cuts them into strips whose workgroups meet in a scratch buffer that it
+ *   grows on demand. This call uses that buffer only as it stands (created with the handle: enough for about 30000
+ *   column-strips, e.g. 150000 x 1500 at 1 bit); a matrix beyond that runs the kernel that re-reads its columns, whose
+ *   sums are added in another order, so its column bounds may differ from the batched call's in their last bits.
  *   cntkq_wait_quantize_done waits for the whole batch. */
 #define CNTKQ_NOALLOC_MAX_ITEMS 256
 #define CNTKQ_NOALLOC_ENTRY_BYTES 112

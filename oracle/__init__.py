@@ -34,6 +34,17 @@ def build(ref=False):
     subprocess.run(["make", "-C", _HERE, "-B"] + targets, check=True, capture_output=True)
 
 
+def build_flags():
+    """The compiler flags the two CPU libraries are built with, as the Makefile states them ({"CFLAGS": ..., "CXXFLAGS": ...})."""
+    out = {}
+    with open(os.path.join(_HERE, "Makefile")) as f:
+        for line in f:
+            name, eq, value = line.partition("=")
+            if eq and name.strip() in ("CFLAGS", "CXXFLAGS"):
+                out[name.strip()] = value.strip()
+    return out
+
+
 def lib():
     global _LIB
     if _LIB is None:

@@ -570,23 +570,139 @@ def test_strip_kernel_replayed_from_a_hip_graph(rows, cols, nbits):
     say("  ", rep)
 
 
-def test_strip_kernel_reports_workgroups_that_give_up():
+def columns_untouched_or_right(g, r_in, q_before, q_after, r_after, nbits, zt):
+    """What a strip launch may leave behind when some of its workgroups gave up: every column is either as it was (packed
+    column and residual untouched) or quantized right. Returns the number of untouched columns."""
+    rows, cols = g.shape
+    qcol = q_after.size // cols
+    untouched = 0
+    for j in range(cols):
+        qa, qb = q_after[j * qcol:(j + 1) * qcol], q_before[j * qcol:(j + 1) * qcol]
+        if np.array_equal(qa, qb) and parity.bits_equal(r_after[:, j], r_in[:, j]):
+            untouched += 1
+            continue
+        parity.check_quantize(np.asfortranarray(g[:, j:j + 1]), np.asfortranarray(r_in[:, j:j + 1]), qa.copy(),
+                              np.asfortranarray(r_after[:, j:j + 1]), nbits, zt)
+    return untouched
+
+
+@pytest.mark.parametrize("host_q", [False, True], ids=["device_q", "host_q"])
+def test_strip_kernel_reports_workgroups_that_give_up(host_q):
     """The workgroups of a column wait for each other's partial sums a bounded number of polls. With that number set to
-    zero from the host every wait gives up at once: the kernel still runs to its end, the next wait reports the call as
-    failed, and the handle goes on working afterwards."""
+    zero from the host every wait that does not find its record at the first look gives up: the kernel still runs to its
+    end, the column is left as it was (packed column and in-place residual untouched, so the error feedback survives),
+    the next wait reports the call as failed -- also where the packed matrix lives in host memory and the wait is for
+    the copy -- and the handle goes on working afterwards."""
     rows, cols = 130000, 4
     qz = MatrixQuantizerImpl.Create(0, False)
     g = datagen.normal(5, rows, cols)
-    G, R, Q = Matrix.from_numpy(g), Matrix(rows, cols), QuantizedMatrix(rows, cols, 1, 0)
+    r0 = datagen.normal(6, rows, cols, 0.002)
+    G, R = Matrix.from_numpy(g), Matrix.from_numpy(r0)
+    Q = QuantizedMatrix(rows, cols, 1, cntk_amd.CPUDEVICE if host_q else 0)
+    Q.buffer.fill_(0xA5)
+    q_before = Q.to_numpy()
+    torch.cuda.synchronize()
     qz._set_strip_spin_limit(0)
     qz.QuantizeAsync(G, R, Q, R, False)
-    with pytest.raises(cntk_amd.QuantizerError):
+    with pytest.raises(cntk_amd.QuantizerError, match="left as they were"):
         qz.WaitQuantizeAsyncDone()
+    torch.cuda.synchronize()
+    if not host_q:  # (the copy to the host takes the staging buffer's bytes, which nothing preset)
+        n = columns_untouched_or_right(g, r0, q_before, Q.to_numpy(), R.to_numpy(), 1, False)
+        say("   columns left untouched: %d of %d" % (n, cols))
+        assert n >= 1
+    else:
+        r_after = R.to_numpy()
+        assert any(parity.bits_equal(r_after[:, j], r0[:, j]) for j in range(cols))
     qz._set_strip_spin_limit(1 << 17)
     R.data.zero_()
     qz.QuantizeAsync(G, R, Q, R, False)
     qz.WaitQuantizeAsyncDone()
     parity.check_quantize(g, np.zeros_like(g, order="F"), Q.to_numpy(), R.to_numpy(), 1, False)
+
+
+def test_strip_kernel_beside_other_work_on_the_device():
+    """The strips of a column wait for each other, which needs all of them resident together. Here the device is kept busy
+    by long fill and copy kernels on another stream while tall matrices are quantized on the quantizer's dedicated stream:
+    whatever the scheduler does, every kernel ends (the wait is bounded), and the outcome is the right bytes or a reported
+    error with every column either untouched or right -- never silently wrong."""
+    rows, cols, nbits = 200000, 96, 1
+    qz = MatrixQuantizerImpl.Create(0, True)
+    g = datagen.normal(9, rows, cols)
+    r0 = datagen.normal(10, rows, cols, 0.002)
+    G = Matrix.from_numpy(g)
+    side = torch.cuda.Stream()
+    big = torch.empty(1 << 30, dtype=torch.float32, device="cuda:0")  # 4 GB: a fill takes about a millisecond
+    big2 = torch.empty_like(big)
+    reported = 0
+    for rep in range(3):
+        R = Matrix.from_numpy(r0)
+        Q = QuantizedMatrix(rows, cols, nbits, 0)
+        Q.buffer.fill_(0xA5)
+        q_before = Q.to_numpy()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            for i in range(6):
+                big.fill_(float(i))
+                big2.copy_(big)
+        qz.QuantizeAsync(G, R, Q, R, False)
+        try:
+            qz.WaitQuantizeAsyncDone()
+            failed = False
+        except cntk_amd.QuantizerError:
+            failed = True
+            reported += 1
+        torch.cuda.synchronize()
+        if failed:
+            columns_untouched_or_right(g, r0, q_before, Q.to_numpy(), R.to_numpy(), nbits, False)
+        else:
+            parity.check_quantize(g, r0, Q.to_numpy(), R.to_numpy(), nbits, False)
+    say("   launches that reported strips giving up: %d of 3" % reported)
+
+
+def test_strip_scratch_outgrown_after_a_recorded_launch():
+    """A recorded strip launch has the scratch buffer's addresses in its graph node. A later, larger launch makes the handle
+    take a larger buffer; the old one must stay alive for the replays (it is freed with the handle): replays after the
+    growth still give the eager bytes."""
+    rows, cols, nbits = 150001, 3, 1
+    wide_rows, wide_cols = 110000, 2400  # 14 strips x 2400 columns: more records than the starting buffer holds
+    qz = MatrixQuantizerImpl.Create(0, False)
+    graphed = (Matrix(rows, cols), Matrix(rows, cols), QuantizedMatrix(rows, cols, nbits, 0))
+    eager = (Matrix(rows, cols), Matrix(rows, cols), QuantizedMatrix(rows, cols, nbits, 0))
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        qz.SetMainStream(torch.cuda.current_stream().cuda_stream)
+        qz.QuantizeAsync(graphed[0], graphed[1], graphed[2], graphed[1], False)
+    qz.SetMainStream(torch.cuda.current_stream().cuda_stream)
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(4711)
+    wide = (Matrix(wide_rows, wide_cols), Matrix(wide_rows, wide_cols), QuantizedMatrix(wide_rows, wide_cols, nbits, 0))
+    wide[0].data.copy_(torch.randn(wide_rows * wide_cols, generator=gen, device="cuda:0") * 0.01)
+    for step in range(3):
+        g = torch.randn(rows * cols, generator=gen, device="cuda:0") * 0.01
+        graphed[0].data.copy_(g)
+        eager[0].data.copy_(g)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        if step == 0:
+            say("   the wide launch that outgrows the buffer")
+            qz.QuantizeAsync(wide[0], wide[1], wide[2], wide[1], False)
+            qz.WaitQuantizeAsyncDone()
+            torch.cuda.synchronize()
+            # the conservation law on the wide matrix: g + r_in (zero) == unquantize(q) + r_out
+            back = Matrix(wide_rows, wide_cols)
+            qz.UnquantizeAsync(wide[2], back)
+            qz.WaitUnquantizeAsyncDone()
+            torch.cuda.synchronize()
+            assert torch.equal(back.data + wide[1].data, wide[0].data) or \
+                float((back.data + wide[1].data - wide[0].data).abs().max()) <= 1e-6
+        qz.QuantizeAsync(eager[0], eager[1], eager[2], eager[1], False)
+        qz.WaitQuantizeAsyncDone()
+        torch.cuda.synchronize()
+        assert torch.equal(graphed[1].data, eager[1].data), "replay %d: residual differs" % step
+        assert torch.equal(graphed[2].buffer, eager[2].buffer), "replay %d: packed matrix differs" % step
 
 
 def test_strip_kernel_across_a_stream_change():
@@ -634,5 +750,8 @@ def test_force_sync_mode_waits_inside_the_calls():
         assert np.array_equal(q_now, Qhost.to_numpy())
         Out = Matrix(rows, cols)
         qz.UnquantizeAsync(Qhost, Out)
+        # the call has waited for its kernel too (RecordQuantizeCompleteEvent at the end of UnquantizeAsync)
+        assert stream.query(), "the work stream still has work after UnquantizeAsync in forceSync mode"
+        out_now = Out.to_numpy().copy()
         qz.WaitUnquantizeAsyncDone()
-        parity.check_unquantize(q_now, rows, cols, 1, Out.to_numpy())
+        parity.check_unquantize(q_now, rows, cols, 1, out_now)

@@ -26,10 +26,17 @@ def read_report(source):
     return kernels
 
 
-@pytest.mark.parametrize("source", build.SOURCES)
-def test_no_kernel_lives_on_scratch_memory(source):
-    kernels = read_report(source)
-    assert len(kernels) > 100, "the report of %s lists %d kernels only" % (source, len(kernels))
+def all_kernels(sources):
+    return [k for source in sources for k in read_report(source)]
+
+
+FLOAT_SOURCES = [s for s in build.SOURCES if not s.endswith("_f64.hip")]
+
+
+@pytest.mark.parametrize("sources", [FLOAT_SOURCES, ["quantizer_api_f64.hip"]], ids=["float", "double"])
+def test_no_kernel_lives_on_scratch_memory(sources):
+    kernels = all_kernels(sources)
+    assert len(kernels) > 100, "the reports of %s list %d kernels only" % (sources, len(kernels))
     worst = sorted(kernels, key=lambda k: -int(k["ScratchSize"]))[:5]
     print([(k["name"][:70], k["ScratchSize"], k["VGPRs"]) for k in worst])
     for k in kernels:
@@ -40,7 +47,7 @@ def test_no_kernel_lives_on_scratch_memory(source):
 
 def test_headline_kernels_spill_nothing():
     """The kernels of the headline benchmark and of the batched launches: no scratch at all."""
-    kernels = read_report("quantizer_api.hip")
+    kernels = all_kernels(FLOAT_SOURCES)
     seen = 0
     for k in kernels:
         n = k["name"]

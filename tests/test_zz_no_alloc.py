@@ -3,7 +3,7 @@ array in the library's device image) gives exactly the bytes of cntkq_quantize_b
 
 Two calls in a row on one handle, the second with a smaller item list, so that the fixed array is reused while it
 still holds the first call's table; then the first list again (its table must be uploaded anew), a second handle in
-between (the array is shared by all handles of a GPU), and the limits."""
+between (the array is shared by all handles of a GPU), a call recorded into a graph mixed with eager calls, and the limits."""
 import sys
 
 import numpy as np
@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 
 LARGE = [(147, 64), (64, 64), (576, 64), (64, 256), (1, 5), (5, 1), (429, 37), (2048, 33), (2304, 5), (4608, 3), (9304, 1),
          (2048, 1), (0, 4), (1000, 1), (1152, 128), (4096, 6), (20000, 2), (512, 100), (33, 67), (14336, 1), (2048, 1100),
-         (1028, 9), (12000, 2)]
+         (1028, 9), (12000, 2), (150001, 3)]
 SMALL = [(429, 37), (64, 256), (2048, 7), (33, 67), (1152, 16)]
 
 
@@ -94,6 +94,77 @@ def test_noalloc_same_list_twice_skips_nothing_visible():
         for i in range(len(shapes)):
             assert np.array_equal(Q1[i].to_numpy(), Q2[i].to_numpy()), ("packed", shapes[i], step)
             assert parity.bits_equal(R1[i].to_numpy(), R2[i].to_numpy()), ("residual", shapes[i], step)
+
+
+class _Pair:
+    """One gradient set twice: for the no-alloc entry point and for the batched call it must equal."""
+
+    def __init__(self, shapes, nbits, seed):
+        self.shapes, self.nbits = shapes, nbits
+        self.gen = torch.Generator(device="cuda:0")
+        self.gen.manual_seed(seed)
+        self.G = [Matrix(r, c) for r, c in shapes]
+        self.R = [[Matrix(r, c) for r, c in shapes] for _ in range(2)]
+        self.Q = [[QuantizedMatrix(r, c, nbits, 0) for r, c in shapes] for _ in range(2)]
+        self.items = [MatrixQuantizerImpl.PrepareQuantizeBatch([(g, r, q, r) for g, r, q in zip(self.G, self.R[k], self.Q[k])])
+                      for k in range(2)]
+
+    def new_gradients(self):
+        for g in self.G:
+            g.data.copy_(torch.randn(g.data.numel(), generator=self.gen, device="cuda:0") * 0.01)
+        for q in self.Q[0]:
+            q.buffer.fill_(0xA5)
+        torch.cuda.synchronize()
+
+    def check(self, what):
+        torch.cuda.synchronize()
+        for i, shape in enumerate(self.shapes):
+            assert torch.equal(self.Q[0][i].buffer, self.Q[1][i].buffer), (what, "packed", shape)
+            assert torch.equal(self.R[0][i].data.view(torch.int32), self.R[1][i].data.view(torch.int32)), (what, "residual", shape)
+
+
+def test_noalloc_recorded_call_among_eager_calls():
+    """A recorded call has not run when the recording ends, and its replays rewrite the shared array at times the
+    library does not see: an eager call may never take its table for uploaded because of either. List A is recorded;
+    then: eager A before the first replay, replay, eager B, replay, eager B again -- every result equal to the batched
+    call's on the same inputs, residuals carried."""
+    nbits = 1
+    new, ref = MatrixQuantizerImpl.Create(0, False), MatrixQuantizerImpl.Create(0, False)
+    a = _Pair([(429, 37), (64, 256), (2048, 7), (33, 67), (1152, 16)], nbits, 901)
+    b = _Pair([(147, 64), (2048, 33), (576, 64), (4608, 3)], nbits, 902)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    a.new_gradients()
+    with torch.cuda.graph(graph, stream=side):
+        new.SetMainStream(torch.cuda.current_stream().cuda_stream)
+        new.QuantizeBatchNoAlloc(a.items[0], False)
+    new.SetMainStream(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+
+    def eager(pair, what):
+        say("no-alloc:", what)
+        pair.new_gradients()
+        new.QuantizeBatchNoAlloc(pair.items[0], False)
+        ref.QuantizeBatchAsync(pair.items[1], False)
+        new.WaitQuantizeAsyncDone()
+        ref.WaitQuantizeAsyncDone()
+        pair.check(what)
+
+    def replay(what):
+        say("no-alloc:", what)
+        a.new_gradients()
+        graph.replay()
+        ref.QuantizeBatchAsync(a.items[1], False)
+        ref.WaitQuantizeAsyncDone()
+        a.check(what)
+
+    eager(a, "eager call with the recorded list before the first replay")
+    replay("first replay")
+    eager(b, "eager call with another list")
+    replay("second replay")
+    eager(b, "the other list again, right after a replay")
+    replay("third replay")
+    eager(a, "the recorded list, eager, after the replays")
 
 
 def test_noalloc_limits():
