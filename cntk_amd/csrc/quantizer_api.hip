@@ -76,7 +76,7 @@ struct BatchAbi<float>
             if (lds > kBatchSmallLds && it.cols <= kStagedInResidualMaxCols)
             {
                 e.kind = 5;
-                lds = ((nbits <= 2 ? e.c.nq : 0) + 12) * sizeof(float);
+                lds = ((nbits <= 2 ? e.c.nq : 0) + kColgRedSlots) * sizeof(float);
             }
             // 1 bit, 1024 / 2048 / 4096 rows, columns on 128-byte lines, 8-byte aligned records: the unrolled body (same bytes)
             if (!line_shift && col_unrolled(it.qbuf, it.rows, nbits))
@@ -194,9 +194,35 @@ struct BatchAbi<float>
     // members that look their sums up need 76 registers where the others need 44: a launch without them keeps eight
     // wavefronts per SIMD
     static bool stripe_entry_wide(const SEntry& e) { return e.kind >= 4; }
-    static hipError_t launch_stripe_members(hipStream_t s, LaunchEvents ev, const SEntry* de, const uint32_t* db, uint32_t members,
-                                            uint32_t blocks, size_t lds, size_t nbits, bool zt, bool wide)
+    // he / hb: the host's copy of the entries and first workgroups that de / db hold on the device
+    static hipError_t launch_stripe_members(hipStream_t s, LaunchEvents ev, const SEntry* de, const uint32_t* db, const SEntry* he,
+                                            const uint32_t* hb, uint32_t members, uint32_t blocks, size_t lds, size_t nbits, bool zt, bool wide)
     {
+        // a few stripes of one shape that all run the unrolled 1-bit column body with up to eight workers (the ranks of a
+        // small cluster simulated on one GPU): described in the kernel's arguments instead of the table in device memory
+        bool as_set = members <= kStripeSetMax && nbits == 1 && (he[0].kind == 2 || he[0].kind == 3) && he[0].src.workers <= kStripeSetMax;
+        for (uint32_t i = 1; i < members && as_set; ++i)
+            as_set = he[i].kind == he[0].kind && he[i].src.workers == he[0].src.workers;
+        if (as_set)
+        {
+            StripeColSet set;
+            std::memset(&set, 0, sizeof set);
+            for (uint32_t i = 0; i <= kStripeSetMax; ++i)
+                set.begin[i] = i <= members ? hb[i] : 0xFFFFFFFFu;
+            for (uint32_t i = 0; i < members; ++i)
+            {
+                for (uint32_t w = 0; w < he[i].src.workers; ++w)
+                    set.q[i][w] = he[i].src.q[w];
+                set.stripe_res[i] = he[i].stripe_res;
+                set.q_out[i] = he[i].q_out;
+                set.agg_out[i] = he[i].agg_out;
+                set.owner[i] = he[i].src.owner;
+            }
+            set.count = members;
+            set.workers = he[0].src.workers;
+            set.qcol = he[0].c.qcol;
+            return family_col_stripe_set(zt && nbits == 1, he[0].kind == 2 ? 1 : 2, s, ev, set);
+        }
         return launch_stripe_reduce_batch(s, ev, de, db, members, blocks, lds, nbits, zt, wide);
     }
 };

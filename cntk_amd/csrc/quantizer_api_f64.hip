@@ -116,8 +116,8 @@ struct BatchAbi<double>
         return lds <= f64::kMaxLdsBytes;
     }
     static bool stripe_entry_wide(const SEntry&) { return false; }
-    static hipError_t launch_stripe_members(hipStream_t s, LaunchEvents ev, const SEntry* de, const uint32_t* db, uint32_t members,
-                                            uint32_t blocks, size_t lds, size_t nbits, bool zt, bool)
+    static hipError_t launch_stripe_members(hipStream_t s, LaunchEvents ev, const SEntry* de, const uint32_t* db, const SEntry*, const uint32_t*,
+                                            uint32_t members, uint32_t blocks, size_t lds, size_t nbits, bool zt, bool)
     {
         return f64::dispatch_nbits64<f64::StripeBatchLauncher64>(nbits, zt && nbits == 1, s, ev, de, db, members, blocks, lds);
     }

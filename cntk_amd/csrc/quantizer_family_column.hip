@@ -98,4 +98,26 @@ hipError_t family_col_stripe_unrolled(bool zt, int per, hipStream_t s, LaunchEve
     return hipGetLastError();
 }
 
+hipError_t family_col_stripe_set(bool zt, int per, hipStream_t s, LaunchEvents ev, const StripeColSet& set)
+{
+    const uint32_t grid = set.begin[set.count];
+    if (per == 1)
+    {
+        if (zt)
+            hipExtLaunchKernelGGL((stripe_reduce_col_set_kernel<true, 1>), dim3(grid), dim3(kColThreads), col_lds_bytes<1>() + kStripeColExtraLds, s, ev.start, ev.stop, 0, set);
+        else
+            hipExtLaunchKernelGGL((stripe_reduce_col_set_kernel<false, 1>), dim3(grid), dim3(kColThreads), col_lds_bytes<1>() + kStripeColExtraLds, s, ev.start, ev.stop, 0, set);
+    }
+    else if (per == 2)
+    {
+        if (zt)
+            hipExtLaunchKernelGGL((stripe_reduce_col_set_kernel<true, 2>), dim3(grid), dim3(kColThreads), col_lds_bytes<2>() + kStripeColExtraLds, s, ev.start, ev.stop, 0, set);
+        else
+            hipExtLaunchKernelGGL((stripe_reduce_col_set_kernel<false, 2>), dim3(grid), dim3(kColThreads), col_lds_bytes<2>() + kStripeColExtraLds, s, ev.start, ev.stop, 0, set);
+    }
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
 } // namespace cntkq

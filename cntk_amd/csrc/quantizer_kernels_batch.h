@@ -153,12 +153,14 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_batch_kernel(const
     else if constexpr (NBITS == 1)
     {
         const uint64_t qcol = en.c.qcol;
+        // (workgroups with the same index modulo 8 run on one die wherever the member starts in the grid)
+        const uint32_t column = column_of_workgroup(index, begins[e + 1] - begins[e]);
         // (4096 rows stay with the general body: unrolled they take 74 registers, which would cost every member of the
         // launch two of its eight wavefronts per SIMD)
         if (en.kind == 2)
-            stripe_reduce_col_body<ZT, 1>(en.src, en.stripe_res, en.q_out, en.agg_out, qcol, index, smem_v4);
+            stripe_reduce_col_body<ZT, 1>(en.src, en.stripe_res, en.q_out, en.agg_out, qcol, column, smem_v4);
         else
-            stripe_reduce_col_body<ZT, 2>(en.src, en.stripe_res, en.q_out, en.agg_out, qcol, index, smem_v4);
+            stripe_reduce_col_body<ZT, 2>(en.src, en.stripe_res, en.q_out, en.agg_out, qcol, column, smem_v4);
     }
 }
 

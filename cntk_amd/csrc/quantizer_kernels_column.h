@@ -21,8 +21,9 @@ struct ColLds
 {
     float* tile;      // 1024 * PER floats, 16-byte aligned
     uint32_t* words;  // 32 * PER partial QWords
-    float* red_f;     // 2 * 4 floats
-    uint32_t* red_u;  // 4
+    float* red_f;     // 2 * 4 floats: the split sums of the four wavefronts
+    uint32_t* red_u;  // 4: their counts
+    float* red_m;     // 4: the wavefronts' sums for the mean (slots of their own: no barrier between reading these and writing the others)
 };
 
 template <int PER>
@@ -33,13 +34,14 @@ __device__ __forceinline__ ColLds col_lds(f32x4* smem)
     l.words = reinterpret_cast<uint32_t*>(l.tile + 1024 * PER);
     l.red_f = reinterpret_cast<float*>(l.words + 32 * PER);
     l.red_u = reinterpret_cast<uint32_t*>(l.red_f + 8);
+    l.red_m = reinterpret_cast<float*>(l.red_u + 4);
     return l;
 }
 
 template <int PER>
 constexpr size_t col_lds_bytes()
 {
-    return (size_t) (1024 * PER + 32 * PER + 8 + 4) * 4;
+    return (size_t) (1024 * PER + 32 * PER + 8 + 4 + 4) * 4;
 }
 
 // LDS of the stripe reduction beyond col_lds_bytes: two levels per worker (up to kMaxWorkers), or, with up to eight
@@ -93,15 +95,15 @@ __device__ __forceinline__ void col_stats_pack(const ColLds& l, float csum, floa
     {
         const float s = wave_sum(csum);
         if (lane == 0)
-            l.red_f[wave] = s;
+            l.red_m[wave] = s;
     }
     __syncthreads(); // the column and the wave sums are visible
     if constexpr (!ZT)
     {
-        float s = l.red_f[0];
+        float s = l.red_m[0];
 #pragma unroll
         for (uint32_t x = 1; x < NW; ++x)
-            s += l.red_f[x];
+            s += l.red_m[x];
         mean = s / (float) ROWS;
     }
     float s0 = 0.0f, s1 = 0.0f;
@@ -115,7 +117,6 @@ __device__ __forceinline__ void col_stats_pack(const ColLds& l, float csum, floa
     s0 = wave_sum(s0);
     s1 = wave_sum(s1);
     n0 = wave_sum(n0);
-    __syncthreads(); // everyone has read the wave sums of the mean
     if (lane == 0)
     {
         l.red_f[wave] = s0;
@@ -202,31 +203,154 @@ __global__ __launch_bounds__(kColThreads) void quantize_col_kernel(const float* 
     quantize_col_body<ZT, PER>(g, r_in, r_out, q, qcol, blockIdx.x, smem_v4);
 }
 
-// Stripe reduction in the same shape: the work item that will pack (QWord p, chunk) first decodes those bit positions
-// from every worker's packed stripe, sums them (owner first, then ascending) and adds the stripe residual.
+// Consecutive workgroups go to the device's eight dies in turn, each die with an L2 of its own. A packed column record is
+// not a whole number of 128-byte lines (264 bytes at 2048 rows), so neighbouring columns share lines, and neighbours on
+// different dies fetch such a line into two L2s (2048 x 9304, eight workers: 29 MB read for 19.6 MB of packed stripes).
+// Runs of 16 consecutive columns therefore go to one die; the eight dies still walk through memory side by side, a
+// megabyte of residual at a time. Maps workgroup b of n to its column (the last n % 128 keep their index).
+__device__ __forceinline__ uint32_t column_of_workgroup(uint32_t b, uint32_t n)
+{
+    constexpr uint32_t RUN = 16, DIES = 8;
+    const uint32_t whole = n - n % (RUN * DIES);
+    if (b >= whole)
+        return b;
+    const uint32_t die = b % DIES, slot = b / DIES;
+    return ((slot / RUN) * DIES + die) * RUN + slot % RUN;
+}
+
+// Stripe reduction in the same shape, up to eight workers: the sum of an element is one of 256 values, picked by the
+// workers' bits of the element. The work item that will pack (QWord p, chunk) turns that QWord of every worker into one
+// byte per bit position (bit u = worker u) by an 8 x 8 bit transposition and looks the sums up in a table that the
+// workgroup's 256 threads build, one entry each, by the additions of the plain decoding loop in its order (owner first,
+// then ascending rank; seeded with -0, and -0 for a worker that is skipped: x + -0 = x for every x): a bit-field extract
+// and an LDS read per element instead of three instructions per worker and element.
+// A stripe can be one GPU's share of a matrix, a single round of workgroups whose time is the length of one workgroup's
+// chain of dependent steps, so everything a thread needs from memory is requested at once, before the first barrier, and
+// nothing in those requests depends on anything but the kernel's arguments: the workers' records are read in worker
+// order (whoever the owner is; the order of the additions is the table's business), so that their addresses come from
+// one scalar load instead of eight dependent ones, and the lane that decodes worker u's header picks that worker's
+// address out of registers instead of loading it.
+template <bool ZT, int PER>
+__device__ __forceinline__ void stripe_reduce_col_lookup(const StripeSources& src, float* stripe_res, char* q_out, float* agg_out, uint64_t qcol,
+                                                         uint32_t column, f32x4* smem_v4)
+{
+    constexpr uint32_t ROWS = 1024 * PER, NQ = 32 * PER, T = kColThreads, KS = 4 * PER, W = 8;
+    const ColLds l = col_lds<PER>(smem_v4);
+    float* dec = l.red_m + 4; // two reconstruction levels per worker, in worker order
+    float* lut = dec + 2 * W;
+    const uint32_t tid = threadIdx.x;
+    const size_t base = (size_t) column * ROWS;
+    const size_t rec = (size_t) column * qcol;
+    const uint32_t K = src.workers, owner = src.owner;
+    if (tid < NQ)
+        l.words[tid] = 0u;
+    const uint32_t p = tid % NQ, chunk = tid / NQ;
+    const uint32_t sh0 = chunk * KS;
+    // (beyond the last worker: worker 0's record, fetched and not used)
+    const char* record[W];
+#pragma unroll
+    for (uint32_t u = 0; u < W; ++u)
+        record[u] = (u < K ? src.q[u] : src.q[0]) + rec;
+    uint32_t word[W];
+#pragma unroll
+    for (uint32_t u = 0; u < W; ++u)
+        word[u] = reinterpret_cast<const uint32_t*>(record[u] + 8)[p];
+    const float* sp = stripe_res + base;
+    float resid[KS];
+#pragma unroll
+    for (uint32_t kk = 0; kk < KS; ++kk)
+        resid[kk] = __builtin_nontemporal_load(sp + p + NQ * (sh0 + kk));
+    if (tid < K)
+    {
+        const char* mine = record[0];
+#pragma unroll
+        for (uint32_t u = 1; u < W; ++u)
+            mine = tid == u ? record[u] : mine;
+        const float* h = reinterpret_cast<const float*>(mine);
+        const ValueQ vq = make_vq<1>(h[0], h[1]);
+        dec[2 * tid] = unquantize_value<1>(vq, 0u);
+        dec[2 * tid + 1] = unquantize_value<1>(vq, 1u);
+    }
+    __syncthreads();
+    {
+        float a = dec[2 * owner + ((tid >> owner) & 1u)] + -0.0f;
+#pragma unroll
+        for (uint32_t u = 0; u < W; ++u)
+        {
+            const float x = dec[2 * u + ((tid >> u) & 1u)];
+            a = ((u < K && u != owner) ? x : -0.0f) + a;
+        }
+        lut[tid] = a;
+    }
+    // the bytes that index the table do not need it yet
+    uint32_t index[(KS + 7) / 8][2];
+#pragma unroll
+    for (uint32_t b = 0; b < (KS + 7) / 8; ++b)
+    {
+        uint32_t row[W];
+#pragma unroll
+        for (uint32_t u = 0; u < W; ++u)
+            row[u] = word[u] >> (sh0 + 8 * b);
+        // byte 0 of the second operand, byte 0 of the first, zeros
+        uint32_t lo = __builtin_amdgcn_perm(row[1], row[0], 0x0C0C0400u) | (__builtin_amdgcn_perm(row[3], row[2], 0x0C0C0400u) << 16);
+        uint32_t hi = __builtin_amdgcn_perm(row[5], row[4], 0x0C0C0400u) | (__builtin_amdgcn_perm(row[7], row[6], 0x0C0C0400u) << 16);
+        transpose_bits_8x8(lo, hi);
+        index[b][0] = lo;
+        index[b][1] = hi;
+    }
+    __syncthreads();
+    float acc[KS];
+#pragma unroll
+    for (uint32_t kk = 0; kk < KS; ++kk)
+        acc[kk] = lut[(index[kk / 8][(kk & 7u) < 4 ? 0 : 1] >> (8 * (kk & 3u))) & 255u];
+#pragma unroll
+    for (uint32_t kk = 0; kk < KS; ++kk)
+    {
+        const uint32_t i = p + NQ * (sh0 + kk);
+        if (agg_out != nullptr)
+            agg_out[base + i] = acc[kk];
+        l.tile[i] = acc[kk] + resid[kk];
+    }
+    float csum = 0.0f;
+    if constexpr (!ZT)
+    {
+        __syncthreads();
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(l.tile);
+        f32x4 v[PER];
+#pragma unroll
+        for (int u = 0; u < PER; ++u)
+            v[u] = t4[tid + T * u];
+        csum = col_thread_sum<PER>(v);
+    }
+    col_stats_pack<ZT, PER>(l, csum, stripe_res + base, q_out + rec);
+}
+
+// More than eight workers: the work item that will pack (QWord p, chunk) decodes those bit positions from every worker's
+// packed stripe, eight workers at a time, sums them (owner first, then ascending) and adds the stripe residual.
 template <bool ZT, int PER>
 __device__ __forceinline__ void stripe_reduce_col_body(const StripeSources& src, float* stripe_res, char* q_out, float* agg_out, uint64_t qcol,
                                                        uint32_t column, f32x4* smem_v4)
 {
     constexpr uint32_t ROWS = 1024 * PER, NQ = 32 * PER, T = kColThreads, KS = 4 * PER, BATCH = 8;
+    const uint32_t K = src.workers;
+    if (K <= BATCH)
+    {
+        stripe_reduce_col_lookup<ZT, PER>(src, stripe_res, q_out, agg_out, qcol, column, smem_v4);
+        return;
+    }
     const ColLds l = col_lds<PER>(smem_v4);
-    float* dec = reinterpret_cast<float*>(l.red_u + 4); // two reconstruction levels per worker, in summation order
+    float* dec = l.red_m + 4; // two reconstruction levels per worker, in summation order
     const uint32_t tid = threadIdx.x;
     const size_t base = (size_t) column * ROWS;
     const size_t rec = (size_t) column * qcol;
-    const uint32_t K = src.workers;
     if (tid < NQ)
         l.words[tid] = 0u;
-    // Everything this thread will need from memory is requested before the first barrier, so that the headers, the
-    // first eight workers' QWords and the stripe residual cost one round trip, not three: a stripe is one GPU's share
-    // of a matrix, a single round of workgroups, and its time is the length of this dependent chain.
     const uint32_t p = tid % NQ, chunk = tid / NQ;
     const uint32_t sh0 = chunk * KS;
     uint32_t word[BATCH];
 #pragma unroll
     for (uint32_t u = 0; u < BATCH; ++u)
-        if (u < K)
-            word[u] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(u, src.owner)] + rec + 8)[p];
+        word[u] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(u, src.owner)] + rec + 8)[p];
     const float* sp = stripe_res + base;
     float resid[KS];
 #pragma unroll
@@ -242,40 +366,6 @@ __device__ __forceinline__ void stripe_reduce_col_body(const StripeSources& src,
     __syncthreads();
 
     float acc[KS];
-    if (K <= BATCH)
-    {
-        // Up to eight workers: the sum of an element is one of 256 values, picked by the workers' bits of the element. The
-        // workgroup's 256 threads build one entry each (the additions of the loop below, in its order, seeded with -0:
-        // x + -0 = x for every x), the thread turns its eight QWords into one byte per bit position (bit g = worker g of
-        // the order) and looks the sums up: a bit-field extract and an LDS read per element instead of three instructions
-        // per worker and element.
-        float* lut = dec + 2 * BATCH;
-        {
-            float a = -0.0f;
-#pragma unroll
-            for (uint32_t u = 0; u < BATCH; ++u)
-                if (u < K)
-                    a = ((tid >> u) & 1u ? dec[2 * u + 1] : dec[2 * u]) + a;
-            lut[tid] = a;
-        }
-        __syncthreads();
-#pragma unroll
-        for (uint32_t b = 0; b < (KS + 7) / 8; ++b)
-        {
-            uint32_t row[BATCH];
-#pragma unroll
-            for (uint32_t u = 0; u < BATCH; ++u)
-                row[u] = u < K ? word[u] >> (sh0 + 8 * b) : 0u;
-            // byte 0 of the second operand, byte 0 of the first, zeros
-            uint32_t lo = __builtin_amdgcn_perm(row[1], row[0], 0x0C0C0400u) | (__builtin_amdgcn_perm(row[3], row[2], 0x0C0C0400u) << 16);
-            uint32_t hi = __builtin_amdgcn_perm(row[5], row[4], 0x0C0C0400u) | (__builtin_amdgcn_perm(row[7], row[6], 0x0C0C0400u) << 16);
-            transpose_bits_8x8(lo, hi);
-#pragma unroll
-            for (uint32_t r = 0; r < 8 && 8 * b + r < KS; ++r)
-                acc[8 * b + r] = lut[((r < 4 ? lo : hi) >> (8 * (r & 3u))) & 255u];
-        }
-    }
-    else
     for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
     {
         if (n0 != 0)
@@ -329,7 +419,44 @@ __global__ __launch_bounds__(kColThreads) void stripe_reduce_col_kernel(StripeSo
                                                                         float* agg_out, uint64_t qcol)
 {
     extern __shared__ f32x4 smem_v4[];
-    stripe_reduce_col_body<ZT, PER>(src, stripe_res, q_out, agg_out, qcol, blockIdx.x, smem_v4);
+    stripe_reduce_col_body<ZT, PER>(src, stripe_res, q_out, agg_out, qcol, column_of_workgroup(blockIdx.x, gridDim.x), smem_v4);
+}
+
+// A few stripes of one shape in one grid, everything a workgroup needs to find its column in the kernel's arguments: the
+// stripes of all the ranks of a small cluster simulated in one GPU's memory. The table-driven launch for whole gradient
+// sets (stripe_reduce_batch_kernel) finds a workgroup's stripe by two dependent reads of device memory before the first
+// load of data goes out, which a workgroup that lives a few microseconds notices (8 x 1163 columns of 2048 rows: 38 us
+// against 32 us for the same columns as one stripe).
+constexpr uint32_t kStripeSetMax = 8; // stripes per launch, and workers per stripe
+struct StripeColSet
+{
+    const char* q[kStripeSetMax][kStripeSetMax]; // [stripe][worker]; beyond the last worker: null
+    float* stripe_res[kStripeSetMax];
+    char* q_out[kStripeSetMax];
+    float* agg_out[kStripeSetMax];
+    uint32_t begin[kStripeSetMax + 1]; // first workgroup of every stripe; begin[count] = the grid; beyond: 0xFFFFFFFF
+    uint32_t owner[kStripeSetMax];
+    uint32_t count;
+    uint32_t workers;
+    uint64_t qcol;
+};
+
+template <bool ZT, int PER>
+__global__ __launch_bounds__(kColThreads) void stripe_reduce_col_set_kernel(StripeColSet set)
+{
+    extern __shared__ f32x4 smem_v4[];
+    uint32_t e = 0;
+#pragma unroll
+    for (uint32_t i = 1; i < kStripeSetMax; ++i)
+        e += blockIdx.x >= set.begin[i] ? 1u : 0u;
+    StripeSources src;
+#pragma unroll
+    for (uint32_t u = 0; u < kStripeSetMax; ++u)
+        src.q[u] = set.q[e][u];
+    src.workers = set.workers;
+    src.owner = set.owner[e];
+    const uint32_t column = column_of_workgroup(blockIdx.x - set.begin[e], set.begin[e + 1] - set.begin[e]);
+    stripe_reduce_col_lookup<ZT, PER>(src, set.stripe_res[e], set.q_out[e], set.agg_out[e], set.qcol, column, smem_v4);
 }
 
 // ---- the same decomposition for any bit width and any column height that is a multiple of 4 ----------------
@@ -367,11 +494,12 @@ struct ColGeom
     uint64_t qcol;
 };
 
-// LDS in floats: [column | partial QWords (nq when a QWord has several work items) | 12 reduction slots | decode constants]
+// LDS in floats: [column | partial QWords (nq when a QWord has several work items) | kColgRedSlots reduction slots | decode constants]
+constexpr uint32_t kColgRedSlots = 16; // 4 + 4 split sums, 4 counts, 4 sums for the mean or the sum of squares
 template <int NBITS>
 __host__ __device__ inline size_t colg_lds_bytes(const ColGeom& c, uint32_t workers)
 {
-    return ((size_t) c.rows + (PackShape<NBITS>::CHUNKS > 1 ? c.nq : 0) + 12 + (size_t) stripe_dec_floats(NBITS) * workers) * sizeof(float);
+    return ((size_t) c.rows + (PackShape<NBITS>::CHUNKS > 1 ? c.nq : 0) + kColgRedSlots + (size_t) stripe_dec_floats(NBITS) * workers) * sizeof(float);
 }
 
 template <int NBITS>
@@ -395,7 +523,7 @@ __device__ __forceinline__ float colg_add_piece(float s, const f32x4& v)
 }
 
 // stat: this thread's running statistic over its pieces (unused for 1 bit with ZT). tile = the column, words = zeroed
-// partial QWords, red = 12 reduction slots. No barrier is needed between writing the column and calling this.
+// partial QWords, red = kColgRedSlots reduction slots. No barrier is needed between writing the column and calling this.
 // WG: threads in the workgroup. The sums are always taken by the first 256 threads (their order is part of the result);
 // coding and packing use all of them.
 template <int NBITS, bool ZT, int WG = kColThreads>
@@ -411,17 +539,18 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
     float total = 0.0f;
     if constexpr (need_stat)
     {
+        // (slots of their own: the split sums below are written without a barrier after these have been read)
         const float s = wave_sum(stat);
         if (lane == 0 && wave < NW)
-            red[wave] = s;
+            red[12 + wave] = s;
     }
     __syncthreads(); // the column and the wave sums are visible
     if constexpr (need_stat)
     {
-        total = red[0];
+        total = red[12];
 #pragma unroll
         for (uint32_t x = 1; x < NW; ++x)
-            total += red[x];
+            total += red[12 + x];
     }
     float lo, hi;
     if constexpr (NBITS == 1)
@@ -437,7 +566,6 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
         s0 = wave_sum(s0);
         s1 = wave_sum(s1);
         n0 = wave_sum(n0);
-        __syncthreads(); // everyone has read the wave sums of the mean
         if (lane == 0 && wave < NW)
         {
             red[wave] = s0;
@@ -583,7 +711,7 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
     float* tile = reinterpret_cast<float*>(smem);
     uint32_t* words = reinterpret_cast<uint32_t*>(tile + c.rows);
     float* red = tile + c.rows + (PS::CHUNKS > 1 ? c.nq : 0);
-    float* dec = red + 12; // per worker, in summation order: 1 bit -> the two levels, 2 and 4 bits -> every level, else (ufactor, lower)
+    float* dec = red + kColgRedSlots; // per worker, in summation order: 1 bit -> the two levels, 2 and 4 bits -> every level, else (ufactor, lower)
     const uint32_t tid = threadIdx.x;
     const size_t base = (size_t) column * c.rows;
     const size_t rec = (size_t) column * c.qcol;

@@ -160,6 +160,8 @@ hipError_t family_col_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents 
                              float* agg_out, uint32_t cols, ColGeom c);
 hipError_t family_col_stripe_unrolled(bool zt, int per, hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out,
                                       float* agg_out, uint32_t cols, uint64_t qcol);
+// up to kStripeSetMax stripes of 1024 (per = 1) or 2048 (per = 2) rows at 1 bit with up to eight workers each, described in the arguments
+hipError_t family_col_stripe_set(bool zt, int per, hipStream_t s, LaunchEvents ev, const StripeColSet& set);
 // threads: 256 or 1024 per column
 hipError_t family_reg_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q,
                                uint32_t cols, RegGeom c, uint32_t threads);
@@ -871,7 +873,7 @@ inline bool stripe_auto_col(size_t rows, const void* stripe_res)
 // colg_lds_bytes for a bit width known only at run time
 inline size_t colg_lds_bytes_rt(const ColGeom& c, size_t nbits)
 {
-    return ((size_t) c.rows + (nbits <= 2 ? c.nq : 0) + 12) * sizeof(float);
+    return ((size_t) c.rows + (nbits <= 2 ? c.nq : 0) + kColgRedSlots) * sizeof(float);
 }
 
 

@@ -250,23 +250,93 @@ __device__ __forceinline__ void transpose_bits_8x8(uint32_t& lo, uint32_t& hi)
 }
 
 // ---- cross-lane sums ----------------------------------------------------------------------------
+//
+// A butterfly over the lanes of a wavefront, nearest partners first: lane ^ 1, ^ 2, ^ 4, ^ 8, then the rows of 16 lanes in
+// pairs, then the pairs. Each step adds the same two operands on both partner lanes, so all lanes of a group hold the same
+// bits after it, and the tree -- which decides the last bits of a column's bounds -- is the same in every kernel. The
+// steps are data-parallel-primitive modifiers of the addition itself (a permutation within four lanes; the mirror image
+// of a half row and of a row, which is the partner's value once groups of four and eight lanes agree; the last lane of
+// the row before, and lane 31, broadcast to the rows that follow): no trip through the LDS crossbar, which costs an
+// index computation and some hundred cycles of latency per step, six steps per sum and four sums per column.
 
-// Sum over aligned groups of `width` lanes (power of two, <= 64); every lane of a group gets the
-// same bits because each butterfly step adds the same two operands on both partner lanes.
-template <typename T>
-__device__ __forceinline__ T lanes_sum(T v, uint32_t width)
+constexpr int kDppXor1 = 0xB1;       // quad_perm [1, 0, 3, 2]
+constexpr int kDppXor2 = 0x4E;       // quad_perm [2, 3, 0, 1]
+constexpr int kDppHalfMirror = 0x141; // lane 7 - i of each half row
+constexpr int kDppMirror = 0x140;     // lane 15 - i of each row
+constexpr int kDppBcast15 = 0x142;    // lane 15 of a row to every lane of the next row
+constexpr int kDppBcast31 = 0x143;    // lane 31 to every lane of rows 2 and 3
+
+// the value another lane holds, chosen by a DPP control (a lane without a source reads zero bits; written so that the
+// compiler folds the move into the addition that follows)
+template <int CTRL, typename T>
+__device__ __forceinline__ T dpp_lane(T v)
 {
-    for (uint32_t off = width >> 1; off > 0; off >>= 1)
-        v += __shfl_xor(v, (int) off, kWave);
-    return v;
+    static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- and 64-bit values");
+    int w[sizeof(T) / 4];
+    __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(T) / 4; ++i)
+        w[i] = __builtin_amdgcn_update_dpp(0, w[i], CTRL, 0xF, 0xF, true);
+    T r;
+    __builtin_memcpy(&r, w, sizeof(T));
+    return r;
 }
 
+// the value lane `lane` (the same for the whole wavefront) holds
+template <typename T>
+__device__ __forceinline__ T read_lane(T v, int lane)
+{
+    static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- and 64-bit values");
+    int w[sizeof(T) / 4];
+    __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(T) / 4; ++i)
+        w[i] = __builtin_amdgcn_readlane(w[i], lane);
+    T r;
+    __builtin_memcpy(&r, w, sizeof(T));
+    return r;
+}
+
+// Sum over the 64 lanes of a wavefront (all of them active); every lane gets the same bits.
 template <typename T>
 __device__ __forceinline__ T wave_sum(T v)
 {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1)
-        v += __shfl_xor(v, off, kWave);
+    v += dpp_lane<kDppXor1>(v);
+    v += dpp_lane<kDppXor2>(v);
+    v += dpp_lane<kDppHalfMirror>(v);
+    v += dpp_lane<kDppMirror>(v);  // every lane: the sum of its row
+    v += dpp_lane<kDppBcast15>(v); // rows 1 and 3: rows 0 + 1 and 2 + 3 (rows 0 and 2 hold nothing of use from here on)
+    v += dpp_lane<kDppBcast31>(v); // row 3: (2 + 3) + (0 + 1)
+    return read_lane(v, 63);
+}
+
+// Sum over aligned groups of `width` lanes (power of two, <= 64; the same for the whole wavefront, all lanes active);
+// every lane of a group gets the same bits. lanes_sum(v, 64) and wave_sum(v) are the same tree.
+template <typename T>
+__device__ __forceinline__ T lanes_sum(T v, uint32_t width)
+{
+    if (width >= 2)
+        v += dpp_lane<kDppXor1>(v);
+    if (width >= 4)
+        v += dpp_lane<kDppXor2>(v);
+    if (width >= 8)
+        v += dpp_lane<kDppHalfMirror>(v);
+    if (width >= 16)
+        v += dpp_lane<kDppMirror>(v);
+    if (width >= 32)
+    {
+        T t = v + dpp_lane<kDppBcast15>(v);
+        if (width == 32)
+        {
+            const T first = read_lane(t, 31), second = read_lane(t, 63);
+            v = (threadIdx.x & 32u) ? second : first;
+        }
+        else
+        {
+            t += dpp_lane<kDppBcast31>(t);
+            v = read_lane(t, 63);
+        }
+    }
     return v;
 }
 
