@@ -217,7 +217,13 @@ public:
         // reference does ("Actual gradient aggregation time", Source/1BitSGD/AllReduceDistGradAggregator.h:153, 241-246,
         // 560-565); 0 = never
         int syncStatsTrace = 0;
+        // from kDebugOutputTraceLevel on: the 3 x 3 corner of every gradient before it is quantized, of every packed stripe
+        // that is sent, of every stripe that was received and of every aggregated gradient goes to stderr
+        // (m_traceLevel >= DEBUG_OUTPUT_TRACE_LEVEL, Source/1BitSGD/AllReduceDistGradAggregator.h:37, 292-297, 351-361, 409-416,
+        // 533-538); each peek waits for the device, so the steps no longer overlap
+        int traceLevel = 0;
     };
+    static const int kDebugOutputTraceLevel = 3;
 
     AllReduceDistGradAggregator(StripeTransportT<ElemType>& transport, size_t myRank, int deviceId, int nBits, bool zeroThresholdFor1Bit,
                                 bool useQuantizationForSelfStripe, bool useAsyncAggregation, Options options = Options())
@@ -281,6 +287,9 @@ public:
         if (headerCPU.numSamples == 0)
             for (auto* g : gradients)
                 g->SetValue(0.0f);
+        if (m_options.traceLevel >= kDebugOutputTraceLevel)
+            for (size_t i = 0; i < numGradMatrices; ++i)
+                PrintMatrix(Label("Original Gradient Matrix No. %d", i).c_str(), gradients[i]);
         // the gradients were produced on the main stream
         if (m_useAsyncAggregation && numGradMatrices > 0)
             SyncWithMainStream(*m_preAggGradQuantizers[0]);
@@ -314,6 +323,9 @@ public:
                     continue;
                 // the owner's own stripe travels the same way: the fused reduction reads it like any other
                 m_transport.PostStripe(MyRank(), j, i, m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
+                if (m_options.traceLevel >= kDebugOutputTraceLevel && j != MyRank())
+                    PeekQuantized(Label("Sending Gradient Matrix No. %d slice", i).c_str(),
+                                  m_gradQuantized[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols));
             }
         }
         m_transport.PostHeader(MyRank(), headerCPU);
@@ -327,6 +339,11 @@ public:
         // stripes too tall for the fused call keep the reference's sequence of calls
         const size_t fusedMaxRows = detail::Abi<ElemType>::StripeReduceMaxRows(m_numQuantizationBits);
         auto fusable = [&](size_t i) { return fused && gradients[i]->GetNumRows() <= fusedMaxRows; };
+        if (m_options.traceLevel >= kDebugOutputTraceLevel)
+            for (size_t i = 0; i < gradients.size(); ++i)
+                for (size_t w = 0; w < K; ++w)
+                    if (w != MyRank() && GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K).m_numCols != 0)
+                        PeekQuantized(Label("Received Gradient Matrix No. %d slice", i).c_str(), m_transport.ReceivedStripe(MyRank(), w, i));
         // every matrix's stripe in one call: the stripe quantizers share one stream, so any of their handles will do
         const bool batched = fused && m_options.useBatchedCalls && gradients.size() > 1;
         if (batched)
@@ -485,8 +502,39 @@ public:
             for (size_t i = 0; i < gradients.size(); ++i)
                 m_preAggGradQuantizers[i]->WaitUnquantizeAsyncDone();                                   // (:531)
         }
+        if (m_options.traceLevel >= kDebugOutputTraceLevel)
+            for (size_t i = 0; i < gradients.size(); ++i)
+                PrintMatrix(Label("Aggregated Gradient Matrix No. %d", i).c_str(), gradients[i]);
         headerCPU.Aggregate(m_transport.AggregatedHeader(), false);
         return headerCPU.numSamples != 0;
+    }
+
+    // Debug helper: the 3 x 3 corner of a matrix (PrintMatrix with peek, Source/1BitSGD/AllReduceDistGradAggregator.h:568-587)
+    static void PrintMatrix(const char* printHeader, const Matrix<ElemType>* matrixToPrint, FILE* out = stderr)
+    {
+        const size_t numRowsToPrint = (std::min)((size_t) 3, matrixToPrint->GetNumRows());
+        const size_t numColsToPrint = (std::min)((size_t) 3, matrixToPrint->GetNumCols());
+        if (numRowsToPrint != 0 && numColsToPrint != 0)
+            matrixToPrint->Print(printHeader, 0, numRowsToPrint - 1, 0, numColsToPrint - 1, out);
+        std::fflush(out);
+    }
+    // ... and of a packed matrix (:351-361)
+    static void PeekQuantized(const char* printHeader, const QuantizedMatrix<ElemType>& q, FILE* out = stderr)
+    {
+        const size_t numRowsToPrint = (std::min)((size_t) 3, q.GetNumRows());
+        const size_t numColsToPrint = (std::min)((size_t) 3, q.GetNumCols());
+        if (numRowsToPrint != 0 && numColsToPrint != 0)
+        {
+            detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize");
+            q.Print(printHeader, 0, numRowsToPrint - 1, 0, numColsToPrint - 1, out);
+        }
+        std::fflush(out);
+    }
+    std::string Label(const char* what, size_t matrixIdx) const
+    {
+        char buf[256];
+        std::snprintf(buf, sizeof buf, (std::string("MPI Rank: %d, ") + what).c_str(), (int) MyRank(), (int) matrixIdx);
+        return buf;
     }
 
     // ---- the same three steps cut into "which items" and "bookkeeping", for InProcessCluster's one call per step --------
@@ -507,6 +555,8 @@ public:
     {
         if (!(m_options.useFusedStripeReduce && m_useQuantizationForSelfStripe && m_options.useBatchedCalls && m_options.useClusterBatching))
             return false;
+        if (m_options.traceLevel >= kDebugOutputTraceLevel)
+            return false; // the debug peeks sit in the per-worker steps
         const size_t fusedMaxRows = detail::Abi<ElemType>::StripeReduceMaxRows(m_numQuantizationBits);
         for (auto* g : gradients)
             if (g->GetNumRows() > fusedMaxRows)

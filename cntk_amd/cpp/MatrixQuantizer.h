@@ -207,6 +207,45 @@ public:
         if (GetNumElements() != 0)
             detail::HipCheck(hipMemcpy(m_data, hostColumnMajor, GetNumElements() * sizeof(ElemType), hipMemcpyHostToDevice), "hipMemcpy");
     }
+    // Matrix::Print of an inclusive range (Source/Math/CPUMatrixImpl.h:4097-4149, the form the aggregator's debug peeks
+    // use: a corner that starts at the first row and column): name and shape, the range where it is not the whole matrix,
+    // then the values row by row with "..." where rows or columns are left out. Reads the range back from the device.
+    void Print(const char* matrixName, size_t rowFirst, size_t rowLast, size_t colFirst, size_t colLast, FILE* out = stderr) const
+    {
+        std::fprintf(out, "\n###### ");
+        if (matrixName != nullptr)
+            std::fprintf(out, "%s ", matrixName);
+        std::fprintf(out, "(%lu, %lu)", (unsigned long) m_rows, (unsigned long) m_cols);
+        if (rowFirst != 0 || colFirst != 0 || rowLast + 1 != m_rows || colLast + 1 != m_cols)
+            std::fprintf(out, " [%ld:%ld, %ld:%ld]", (long) rowFirst, (long) rowLast, (long) colFirst, (long) colLast);
+        std::fprintf(out, " ######\n\n");
+        if (GetNumElements() == 0 || rowFirst > rowLast || colFirst > colLast || rowLast >= m_rows || colLast >= m_cols)
+        {
+            std::fprintf(out, "(empty)\n");
+            return;
+        }
+        const size_t nr = rowLast - rowFirst + 1, nc = colLast - colFirst + 1;
+        std::vector<ElemType> host(nr * nc);
+        detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize");
+        for (size_t j = 0; j < nc; ++j)
+            detail::HipCheck(hipMemcpy(host.data() + j * nr, m_data + (colFirst + j) * m_rows + rowFirst, nr * sizeof(ElemType), hipMemcpyDeviceToHost),
+                             "hipMemcpy");
+        if (rowFirst > 0)
+            std::fprintf(out, "...\n");
+        for (size_t i = 0; i < nr; ++i)
+        {
+            if (colFirst > 0)
+                std::fprintf(out, "...\t");
+            for (size_t j = 0; j < nc; ++j)
+                std::fprintf(out, "%.10f\t", (double) host[j * nr + i]);
+            if (colLast + 1 < m_cols)
+                std::fprintf(out, "...");
+            std::fprintf(out, "\n");
+        }
+        if (rowLast + 1 < m_rows)
+            std::fprintf(out, "...\n");
+    }
+
     // host copy in column-major order (Matrix::CopyToArray)
     std::unique_ptr<ElemType[]> CopyToArray() const
     {

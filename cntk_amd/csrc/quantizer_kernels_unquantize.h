@@ -451,6 +451,51 @@ __device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q,
     // slots dealt by 128-byte lines: slot v = tid, tid + 256, ... holds the group of N that starts at element
     // N * (v - shift), shift = the tile's offset into its line in 16-byte pieces
     const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o) >> 4) & 7u);
+    if (t.rows % N == 0 && t.nq % N == 0)
+    {
+        // Heights and QWord counts that are multiples of N (64, 128, 256, 512, 576, 1152 rows at 2 to 8 bits; 512 rows at
+        // 1 bit): a group of N consecutive elements lies in one column at one bit position of N consecutive QWords, so
+        // column, bit position and QWord are worked out once per group and nothing wraps inside it (the general loop below
+        // checks both wraps after every element: some 19 vector instructions per element against 6 here).
+        for (uint32_t i = N * ((tid < shift ? tid + 256 : tid) - shift); i < elems; i += 256 * N)
+        {
+            const uint32_t c = small_div(i, t.rows, t.rows_magic);
+            const uint32_t r = i - c * t.rows;
+            const uint32_t k = small_div(r, t.nq, t.nq_magic);
+            const QWord* cw = words + c * t.rec_words + 2 + (r - k * t.nq);
+            const E d0 = dec[2 * c], d1 = dec[2 * c + 1];
+            const uint32_t sh = k * PS::SHIFT;
+            QWord packed[N];
+            if constexpr (N == 4)
+            {
+                // (records are an even number of QWords long here and start on one: pairs of QWords are 8-byte aligned)
+                typedef QWord Pair __attribute__((ext_vector_type(2)));
+                const Pair a = *reinterpret_cast<const Pair*>(cw), b = *reinterpret_cast<const Pair*>(cw + 2);
+                packed[0] = a.x, packed[1] = a.y, packed[2] = b.x, packed[3] = b.y;
+            }
+            else
+            {
+#pragma unroll
+                for (uint32_t e = 0; e < N; ++e)
+                    packed[e] = cw[e];
+            }
+            Vec x;
+#pragma unroll
+            for (uint32_t e = 0; e < N; ++e)
+            {
+                const QWord code = (packed[e] >> sh) & PS::CODEMASK;
+                if constexpr (NBITS == 1)
+                    x[e] = code ? d1 : d0;
+                else
+                    x[e] = unquantize_value<NBITS>(d0, d1, code);
+            }
+            Vec* o4 = reinterpret_cast<Vec*>(o + i);
+            if (add)
+                x = x + *o4; // unquantized value + previous content
+            __builtin_nontemporal_store(x, o4);
+        }
+        return;
+    }
     for (uint32_t i = N * ((tid < shift ? tid + 256 : tid) - shift); i < elems; i += 256 * N)
     {
         uint32_t c = small_div(i, t.rows, t.rows_magic);

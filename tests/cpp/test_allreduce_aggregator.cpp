@@ -466,6 +466,74 @@ static void SyncStatsTrace()
     CHECK(lines == 3, "aggregations 0, 2 and 4 are reported, got %d lines", lines);
 }
 
+// traceLevel = 3: the 3 x 3 corners of the original gradients, of the packed stripes sent and received and of the aggregated
+// gradients go to stderr, in the reference's wording; the aggregation itself gives the bytes it gives without them.
+static void DebugPeeks()
+{
+    const size_t K = 2;
+    std::vector<std::vector<float>> results[2];
+    std::string text;
+    for (int traced = 0; traced < 2; ++traced)
+    {
+        InProcessCluster<float>::Options opt;
+        opt.traceLevel = traced ? 3 : 0;
+        InProcessCluster<float> cluster(K, 0, 1, false, true, false, opt);
+        FILE* saved = stderr;
+        FILE* f = std::tmpfile();
+        CHECK(f != nullptr, "tmpfile");
+        if (f == nullptr)
+            return;
+        stderr = f;
+        std::vector<std::unique_ptr<Matrix<float>>> owned;
+        std::vector<std::vector<Matrix<float>*>> grads(K);
+        std::vector<DistGradHeader> headers;
+        for (size_t r = 0; r < K; ++r)
+        {
+            for (size_t i = 0; i < 2; ++i)
+            {
+                const size_t rows = i == 0 ? 64 : 2, cols = i == 0 ? 8 : 5;
+                owned.emplace_back(new Matrix<float>(rows, cols, 0));
+                owned.back()->SetValue(Gaussian(rows * cols, 0.01f, 77 + 10 * r + i).data());
+                grads[r].push_back(owned.back().get());
+            }
+            headers.emplace_back(1);
+            headers.back().numSamples = 4;
+        }
+        cluster.AggregateGradients(grads, headers, true, true);
+        detail::HipCheck(hipDeviceSynchronize(), "hipDeviceSynchronize");
+        stderr = saved;
+        std::rewind(f);
+        char buf[512];
+        while (std::fgets(buf, sizeof buf, f) != nullptr)
+            if (traced)
+                text += buf;
+            else
+                CHECK(false, "output without tracing: %s", buf);
+        std::fclose(f);
+        for (auto* g : grads[0])
+        {
+            auto a = g->CopyToArray();
+            results[traced].emplace_back(a.get(), a.get() + g->GetNumElements());
+        }
+    }
+    for (size_t i = 0; i < results[0].size(); ++i)
+        CHECK(results[0][i].size() == results[1][i].size() &&
+                  std::memcmp(results[0][i].data(), results[1][i].data(), results[0][i].size() * sizeof(float)) == 0,
+              "matrix %zu: the traced aggregation gives other bytes", i);
+    auto count = [&](const char* what) {
+        int n = 0;
+        for (size_t at = text.find(what); at != std::string::npos; at = text.find(what, at + 1))
+            n++;
+        return n;
+    };
+    CHECK(count("MPI Rank: 0, Original Gradient Matrix No. 0 (64, 8) [0:2, 0:2] ######") == 1, "original gradient of rank 0");
+    CHECK(count("MPI Rank: 1, Original Gradient Matrix No. 1 (2, 5) [0:1, 0:2] ######") == 1, "a matrix of two rows is peeked at two rows");
+    CHECK(count("Sending Gradient Matrix No.") == 4, "every rank sends one slice of every matrix to the other: %d", count("Sending Gradient Matrix No."));
+    CHECK(count("Received Gradient Matrix No.") == 4, "and receives one: %d", count("Received Gradient Matrix No."));
+    CHECK(count("Aggregated Gradient Matrix No.") == 4, "aggregated gradients: %d", count("Aggregated Gradient Matrix No."));
+    CHECK(count("Lower=") >= 8 && count("------ Print Range (0:2, 0:2) ------") >= 1, "packed stripes are printed with their column bounds");
+}
+
 int main()
 {
     try
@@ -475,7 +543,7 @@ int main()
                            {"QuantizedAllReduceUnquantizedSelfStripe", UnquantizedSelfStripe}, {"QuantizedAllReduceEmptyMinibatchAndReset", EmptyMinibatchAndReset},
                            {"QuantizedAllReduceBufferedAggregation", BufferedAggregation},
                            {"QuantizedAllReduceDoublePrecision", DoublePrecisionVariantsAreBitIdentical},
-                           {"QuantizedAllReduceSyncStatsTrace", SyncStatsTrace}};
+                           {"QuantizedAllReduceSyncStatsTrace", SyncStatsTrace}, {"QuantizedAllReduceDebugPeeks", DebugPeeks}};
         for (const T& t : tests)
         {
             const int before = g_failures;
