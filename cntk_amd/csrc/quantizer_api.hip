@@ -163,7 +163,7 @@ struct BatchAbi<float>
             const bool line_shift = !columns_start_on_lines(it.stripe_res, it.rows);
             e.kind = 1;
             e.c = make_col_geom(it.rows, nbits, line_shift);
-            lds = colg_lds_bytes_rt(e.c, nbits) + stripe_dec_floats(nbits) * workers * sizeof(float);
+            lds = colg_lds_bytes_rt(e.c, nbits) + stripe_dec_bytes(nbits, workers);
             blocks = it.stripe_cols;
             // as launch_stripe_reduce chooses: the unrolled body where every packed stripe is 8-byte aligned
             bool aligned = (reinterpret_cast<uintptr_t>(it.q_out) & 7u) == 0;

@@ -11,12 +11,17 @@ struct StripeBatchLauncher
     static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeBatchEntry* entries, const uint32_t* begins, uint32_t count,
                           uint32_t total_blocks, size_t lds, bool wide)
     {
-        if (wide && NBITS == 1)
-            hipExtLaunchKernelGGL((stripe_reduce_batch_kernel<NBITS, ZT, NBITS == 1>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start,
-                                  ev.stop, 0, entries, begins, count);
-        else
-            hipExtLaunchKernelGGL((stripe_reduce_batch_kernel<NBITS, ZT, false>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start,
-                                  ev.stop, 0, entries, begins, count);
+        if constexpr (NBITS == 1)
+        {
+            if (wide)
+            {
+                hipExtLaunchKernelGGL((stripe_reduce_batch_lookup_kernel<ZT>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start, ev.stop,
+                                      0, entries, begins, count);
+                return hipGetLastError();
+            }
+        }
+        hipExtLaunchKernelGGL((stripe_reduce_batch_kernel<NBITS, ZT>), dim3(total_blocks), dim3(kTileThreads), lds, s, ev.start, ev.stop, 0,
+                              entries, begins, count);
         return hipGetLastError();
     }
 };

@@ -3,6 +3,8 @@
 // between the families.
 #include "quantizer_launch.h"
 
+#include <algorithm>
+
 namespace cntkq {
 
 template <int NBITS, bool ZT>
@@ -22,24 +24,43 @@ struct StripeColLauncher
     static hipError_t run(hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
                           uint32_t cols, ColGeom c)
     {
-        // Every work item (a QWord, or a chunk of its bit positions) is a chain of dependent loads, and the column's LDS
-        // limits how many workgroups a CU holds: from 24 KB per column on (6 workgroups or fewer per CU) 512 threads keep
-        // the CU's wavefront slots filled, and where the stripe has no more columns than the device has CUs, 1024 do.
-        // Measured at 8 workers, 256 / 512 / 1024 threads: 9304 x 2048 at 2 bits 62 / 58 / 84 us, 14336 x 1328 at 4 bits
-        // 91 / 68 / 80, 4096 x 4652 at 8 bits 67 / 75 / 114, 6144 x 3101 at 2 bits 55 / 59 / 99, 14336 x 256 at 2 bits
-        // 28 / 19 / 15, 8192 x 300 at 8 bits 23 / 16 / 20.
+        // How many threads a column gets. The work items of a column (a QWord, or a chunk of its bit positions) are dealt to
+        // the threads in rounds, each a chain of dependent loads; the column's LDS limits how many workgroups a compute unit
+        // holds, and a workgroup's sums are taken by its first 256 threads whatever its size (their order is part of the
+        // result), so larger workgroups pay for idle threads in those phases. The size is the one of 256, 512 and 768 (whole
+        // wavefronts on every SIMD: 576 and 640 threads measure a third slower than 512) with the most busy threads per
+        // compute unit: resident workgroups x threads x the fill of the last round of items, times 0.8 for 512 and 0.75 for
+        // 768 threads. Measured at 8 workers over 256 / 512 / 768 / 1024 threads: 9304 x 2048 at 2 bits 54 / 49 / 52 / 74 us,
+        // at 8 bits 77 / 69 / 69 / 83; 14336 x 1328 at 2 bits 70 / 53 / 49 / 66, at 8 bits 93 / 70 / 68 / 80; 6144 x 3101 at 2
+        // bits 44 / 50 / 51 / 82, at 8 bits 66 / 63 / 66 / 97; 4096 x 4652 at 2 bits 41 / 48 / 59 / 97. Where the stripe has no
+        // more columns than the device has compute units, 1024 threads (14336 x 256 at 2 bits: 28 / 19 / - / 15 us).
+        const uint32_t items = c.nq * PackShape<NBITS>::CHUNKS;
         uint32_t wg = 256u;
-        if (c.nq * PackShape<NBITS>::CHUNKS >= kStripeWideItems)
-            wg = cols <= kStripeWideMaxCols ? 1024u : (c.rows > kStripeMidMinRows ? 512u : 256u);
-        if (wg == 1024)
-            hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, 1024>), dim3(cols), dim3(1024), colg_lds_bytes<NBITS>(c, src.workers),
-                                  s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
-        else if (wg == 512)
-            hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, 512>), dim3(cols), dim3(512), colg_lds_bytes<NBITS>(c, src.workers),
-                                  s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
-        else
+        if (items >= kStripeWideItems && cols <= kStripeWideMaxCols)
+            wg = 1024u;
+        else if (items >= kStripeWideItems)
+        {
+            const size_t lds = colg_lds_bytes<NBITS>(c, src.workers);
+            double best = 0.0;
+            for (uint32_t t = 256; t <= 768; t += 256)
+            {
+                const uint32_t resident = (uint32_t) std::max<size_t>(1, std::min<size_t>(2048 / t, (160 * 1024) / lds));
+                const uint32_t rounds = (items + t - 1) / t;
+                const double busy = (double) std::min(2048u, resident * t) * ((double) items / (double) (rounds * t)) *
+                                    (t == 256 ? 1.0 : (t == 512 ? 0.8 : 0.75));
+                if (busy > best)
+                {
+                    best = busy;
+                    wg = t;
+                }
+            }
+        }
+        if (wg == kColThreads)
             hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, kColThreads>), dim3(cols), dim3(kColThreads),
                                   colg_lds_bytes<NBITS>(c, src.workers), s, ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
+        else
+            hipExtLaunchKernelGGL((stripe_reduce_colg_kernel<NBITS, ZT, 0>), dim3(cols), dim3(wg), colg_lds_bytes<NBITS>(c, src.workers), s,
+                                  ev.start, ev.stop, 0, src, stripe_res, q_out, agg_out, c);
         return hipGetLastError();
     }
 };

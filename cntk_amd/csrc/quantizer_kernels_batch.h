@@ -121,8 +121,8 @@ struct StripeBatchEntry
 // LOOKUP: the variant that also runs members of kinds 4 and 5 (76 registers instead of 44: a launch without such members
 // takes the other one and keeps eight wavefronts per SIMD)
 template <int NBITS, bool ZT, bool LOOKUP>
-__global__ __launch_bounds__(kTileThreads) void stripe_reduce_batch_kernel(const StripeBatchEntry* __restrict__ entries,
-                                                                           const uint32_t* __restrict__ begins, uint32_t count)
+__device__ __forceinline__ void stripe_reduce_batch_body(const StripeBatchEntry* __restrict__ entries, const uint32_t* __restrict__ begins,
+                                                         uint32_t count)
 {
     extern __shared__ f32x4 smem_v4[];
     const uint32_t e = batch_find(begins, count, blockIdx.x);
@@ -162,6 +162,21 @@ __global__ __launch_bounds__(kTileThreads) void stripe_reduce_batch_kernel(const
         else
             stripe_reduce_col_body<ZT, 2>(en.src, en.stripe_res, en.q_out, en.agg_out, qcol, column, smem_v4);
     }
+}
+
+template <int NBITS, bool ZT>
+__global__ __launch_bounds__(kTileThreads) CNTKQ_SGPRS_FOR_8_WAVES void stripe_reduce_batch_kernel(const StripeBatchEntry* __restrict__ entries,
+                                                                                                   const uint32_t* __restrict__ begins, uint32_t count)
+{
+    stripe_reduce_batch_body<NBITS, ZT, false>(entries, begins, count);
+}
+
+// (six wavefronts per SIMD by its vector registers: as many scalar registers as the compiler likes)
+template <bool ZT>
+__global__ __launch_bounds__(kTileThreads) void stripe_reduce_batch_lookup_kernel(const StripeBatchEntry* __restrict__ entries,
+                                                                                  const uint32_t* __restrict__ begins, uint32_t count)
+{
+    stripe_reduce_batch_body<1, ZT, true>(entries, begins, count);
 }
 
 

@@ -494,12 +494,13 @@ struct ColGeom
     uint64_t qcol;
 };
 
-// LDS in floats: [column | partial QWords (nq when a QWord has several work items) | kColgRedSlots reduction slots | decode constants]
+// LDS: [stripe reductions: the first workers' decoding tables | column | partial QWords (nq when a QWord has several work
+// items) | kColgRedSlots reduction slots | stripe reductions: further workers' tables]; workers = 0: a quantize kernel
 constexpr uint32_t kColgRedSlots = 16; // 4 + 4 split sums, 4 counts, 4 sums for the mean or the sum of squares
 template <int NBITS>
 __host__ __device__ inline size_t colg_lds_bytes(const ColGeom& c, uint32_t workers)
 {
-    return ((size_t) c.rows + (PackShape<NBITS>::CHUNKS > 1 ? c.nq : 0) + kColgRedSlots + (size_t) stripe_dec_floats(NBITS) * workers) * sizeof(float);
+    return ((size_t) c.rows + (PackShape<NBITS>::CHUNKS > 1 ? c.nq : 0) + kColgRedSlots) * sizeof(float) + (workers != 0 ? stripe_dec_bytes(NBITS, workers) : 0);
 }
 
 template <int NBITS>
@@ -522,17 +523,33 @@ __device__ __forceinline__ float colg_add_piece(float s, const f32x4& v)
     return s;
 }
 
+// which chunk of bit positions work item `it` of a column of nq QWords belongs to (chunk-major numbering), without a division
+template <uint32_t CHUNKS>
+__device__ __forceinline__ uint32_t chunk_of_item(uint32_t it, uint32_t nq)
+{
+    static_assert(CHUNKS <= 4, "up to four chunks per QWord");
+    uint32_t chunk = 0;
+    if constexpr (CHUNKS > 1)
+        chunk += it >= nq ? 1u : 0u;
+    if constexpr (CHUNKS > 2)
+        chunk += it >= 2 * nq ? 1u : 0u;
+    if constexpr (CHUNKS > 3)
+        chunk += it >= 3 * nq ? 1u : 0u;
+    return chunk;
+}
+
 // stat: this thread's running statistic over its pieces (unused for 1 bit with ZT). tile = the column, words = zeroed
 // partial QWords, red = kColgRedSlots reduction slots. No barrier is needed between writing the column and calling this.
-// WG: threads in the workgroup. The sums are always taken by the first 256 threads (their order is part of the result);
+// WGT: threads in the workgroup, or 0 for "as launched" (any multiple of 64 from 256 on). The sums are always taken by the first 256 threads (their order is part of the result);
 // coding and packing use all of them.
-template <int NBITS, bool ZT, int WG = kColThreads>
+template <int NBITS, bool ZT, int WGT = kColThreads>
 __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, float* red, const ColGeom& c, float stat,
                                                 uint32_t shift, float* res_col, char* qc)
 {
     using PS = PackShape<NBITS>;
     constexpr uint32_t T = kColThreads, NW = T / 64;
-    static_assert(WG >= (int) T && WG % 64 == 0, "workgroup size");
+    static_assert(WGT == 0 || (WGT >= (int) T && WGT % 64 == 0), "workgroup size");
+    const uint32_t WG = WGT == 0 ? blockDim.x : (uint32_t) WGT;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     uint32_t* red_u = reinterpret_cast<uint32_t*>(red + 8);
     constexpr bool need_stat = (NBITS != 1) || !ZT;
@@ -559,7 +576,7 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
         float s0 = 0.0f, s1 = 0.0f;
         uint32_t n0 = 0;
         const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
-        if (WG == T || tid < T)
+        if (WGT == (int) T || tid < T)
             for (uint32_t v = tid; v < c.pieces + shift; v += T)
                 if (v >= shift)
                     split_add_piece(t4[v - shift], mean, s0, s1, n0);
@@ -600,30 +617,44 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
     const float val1 = unquantize_value<NBITS>(vq, 1u);
     uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
     const uint32_t items = c.nq * PS::CHUNKS;
-    for (uint32_t it = tid; it < items; it += WG)
-    {
-        // chunk-major: consecutive threads take consecutive QWords, hence consecutive rows
-        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / c.nq;
-        const uint32_t w = it - chunk * c.nq;
+    // A QWord's bit positions are nq elements apart; element i lies 4 * i bytes into the column, in LDS as in memory, so
+    // one byte offset serves the read and the store (the column's address is the same for all threads and stays in scalar
+    // registers). In a column of more than VPW * VPW rows only a QWord's last bit position can lie beyond the end: a work
+    // item with all of its elements inside runs without a branch per element.
+    const uint32_t step = c.nq * 4u, end = c.rows * 4u;
+    auto pack_item = [&](uint32_t off, auto guard) {
         uint32_t word = 0;
 #pragma unroll
         for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
         {
-            const uint32_t k = chunk * PS::SLOTS + kk;
-            const uint32_t i = w + k * c.nq;
-            if (i < c.rows)
+            if (!decltype(guard)::value || off < end)
             {
-                const float v = tile[i];
+                const float v = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(tile) + off);
                 const uint32_t code = quantize_value<NBITS, ZT>(vq, v);
                 float back;
                 if constexpr (NBITS == 1)
                     back = code ? val1 : val0;
                 else
                     back = unquantize_value<NBITS>(vq, code);
-                __builtin_nontemporal_store(v - back, res_col + i);
-                word |= code << (k * PS::SHIFT);
+                __builtin_nontemporal_store(v - back, reinterpret_cast<float*>(reinterpret_cast<char*>(res_col) + off));
+                word |= code << (kk * PS::SHIFT);
             }
+            off += step;
         }
+        return word;
+    };
+    for (uint32_t it = tid; it < items; it += WG)
+    {
+        // chunk-major: consecutive threads take consecutive QWords, hence consecutive rows
+        const uint32_t chunk = chunk_of_item<PS::CHUNKS>(it, c.nq);
+        const uint32_t w = it - chunk * c.nq;
+        const uint32_t off = (w + chunk * PS::SLOTS * c.nq) * 4u;
+        uint32_t word;
+        if (off + (PS::SLOTS - 1u) * step < end)
+            word = pack_item(off, std::false_type());
+        else
+            word = pack_item(off, std::true_type());
+        word <<= chunk * PS::SLOTS * PS::SHIFT;
         if constexpr (PS::CHUNKS == 1)
             bits[w] = word;
         else
@@ -699,19 +730,116 @@ __global__ __launch_bounds__(kColThreads) void quantize_colg_kernel(const float*
     quantize_colg_body<NBITS, ZT>(g, r_in, r_out, q, c, blockIdx.x, smem_v4);
 }
 
-// WG: threads in the workgroup (256, or 1024 for tall columns, whose many work items would otherwise be a long chain of
-// dependent loads for each of few threads)
-template <int NBITS, bool ZT, int WG = kColThreads>
+// One group of up to eight workers (n0 ... n0 + 7 of the summation order) added to the running sums of a work item's SLOTS
+// elements. word[u]: worker n0 + u's QWord; dec: the group's decoding tables. FIRST: the group that holds the owner, whose
+// value seeds the sum, and whose tables start at LDS address 0 (see lds_read). FULL: count is 8 (nothing to branch around,
+// and the look-ups of all eight workers can be in flight together).
+template <int NBITS, bool FIRST, bool FULL>
+__device__ __forceinline__ void stripe_add_group(float (&acc)[PackShape<NBITS>::SLOTS], const uint32_t (&word)[8], uint32_t sh0, uint32_t count,
+                                                 const float* dec)
+{
+    using PS = PackShape<NBITS>;
+    constexpr uint32_t DEC = stripe_dec_floats(NBITS);
+#pragma unroll
+    for (uint32_t u = 0; u < 8; ++u)
+    {
+        if (FULL || u < count)
+        {
+            const uint32_t bits = word[u] >> sh0;
+            const float* lev = dec + u * DEC;
+            if constexpr (NBITS == 2)
+            {
+                // two codes at a time: their four bits, times 8 bytes, are the offset of the pair of levels
+                static_assert(PS::SLOTS % 2 == 0, "pairs of bit positions");
+#pragma unroll
+                for (uint32_t j = 0; j < PS::SLOTS / 2; ++j)
+                {
+                    const uint32_t off = j == 0 ? (bits << 3) & 0x78u : (bits >> (4 * j - 3)) & 0x78u;
+                    f32x2 x;
+                    if constexpr (FIRST)
+                        x = lds_read<f32x2>(off + u * DEC * 4u);
+                    else
+                        x = *reinterpret_cast<const f32x2*>(reinterpret_cast<const char*>(lev) + off);
+                    acc[2 * j] = (FIRST && u == 0) ? x.x : x.x + acc[2 * j];
+                    acc[2 * j + 1] = (FIRST && u == 0) ? x.y : x.y + acc[2 * j + 1];
+                }
+            }
+            else if constexpr (NBITS == 4)
+            {
+#pragma unroll
+                for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+                {
+                    const uint32_t off = kk == 0 ? (bits << 2) & 0x3Cu : (bits >> (4 * kk - 2)) & 0x3Cu;
+                    float x;
+                    if constexpr (FIRST)
+                        x = lds_read<float>(off + u * DEC * 4u);
+                    else
+                        x = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(lev) + off);
+                    acc[kk] = (FIRST && u == 0) ? x : x + acc[kk];
+                }
+            }
+            else
+            {
+                const float a = lev[0];
+                const float b = lev[1];
+#pragma unroll
+                for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
+                {
+                    float x;
+                    if constexpr (NBITS == 1)
+                        x = pick_level(bits, kk, a, b);
+                    else
+                        x = unquantize_value<NBITS>(a, b, (bits >> (kk * PS::SHIFT)) & PS::CODEMASK);
+                    // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
+                    acc[kk] = (FIRST && u == 0) ? x : x + acc[kk];
+                }
+            }
+        }
+    }
+}
+
+// The sums' results for one work item: SLOTS elements, nq apart, from byte offset off0 of the column on; the aggregate
+// (when asked for) to memory, aggregate plus stripe residual to the column in LDS (which starts at LDS address tile_at, see
+// lds_write). GUARD: some may lie beyond the column.
+template <int NBITS, bool GUARD>
+__device__ __forceinline__ void stripe_store_item(const float (&acc)[PackShape<NBITS>::SLOTS], const float (&resid)[PackShape<NBITS>::SLOTS],
+                                                  uint32_t tile_at, float* agg_col, uint32_t off0, uint32_t step, uint32_t end)
+{
+    uint32_t off = off0;
+#pragma unroll
+    for (uint32_t kk = 0; kk < PackShape<NBITS>::SLOTS; ++kk)
+    {
+        if (!GUARD || off < end)
+        {
+            if (agg_col != nullptr)
+                *reinterpret_cast<float*>(reinterpret_cast<char*>(agg_col) + off) = acc[kk];
+            lds_write<float>(tile_at + off, acc[kk] + resid[kk]);
+        }
+        off += step;
+    }
+}
+
+// WGT: threads in the workgroup, or 0 for what the launch says (tall columns: many work items would otherwise be a long
+// chain of dependent loads for each of few threads).
+// LDS: the decoding tables of the first eight workers of the summation order (at offsets the compiler knows, which the
+// look-ups then carry in the instruction), the column, its QWords under assembly (when a QWord's bit positions are
+// dealt to several work items), the sums' slots, the tables of any further workers.
+template <int NBITS, bool ZT, int WGT = kColThreads>
 __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src, float* stripe_res, char* q_out, float* agg_out,
                                                         const ColGeom& c, uint32_t column, f32x4* smem)
 {
     using PS = PackShape<NBITS>;
-    constexpr uint32_t T = kColThreads, BATCH = 8;
-    static_assert(WG >= (int) T, "workgroup size");
-    float* tile = reinterpret_cast<float*>(smem);
+    constexpr uint32_t T = kColThreads, BATCH = kStripeDecGroup;
+    constexpr uint32_t DEC = stripe_dec_floats(NBITS);
+    static_assert(WGT == 0 || WGT >= (int) T, "workgroup size");
+    static_assert(BATCH * DEC % 4 == 0, "the column starts on a 16-byte boundary");
+    const uint32_t WG = WGT == 0 ? blockDim.x : (uint32_t) WGT;
+    float* dec = reinterpret_cast<float*>(smem);
+    float* tile = dec + BATCH * DEC;
     uint32_t* words = reinterpret_cast<uint32_t*>(tile + c.rows);
     float* red = tile + c.rows + (PS::CHUNKS > 1 ? c.nq : 0);
-    float* dec = red + kColgRedSlots; // per worker, in summation order: 1 bit -> the two levels, 2 and 4 bits -> every level, else (ufactor, lower)
+    // from an 8-byte boundary on
+    float* dec_more = red + kColgRedSlots + ((c.rows + (PS::CHUNKS > 1 ? c.nq : 0)) & 1u);
     const uint32_t tid = threadIdx.x;
     const size_t base = (size_t) column * c.rows;
     const size_t rec = (size_t) column * c.qcol;
@@ -722,129 +850,111 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
     // what this thread's first work item needs from memory is requested before the first barrier: one round trip for
     // headers, QWords and stripe residual instead of three (see stripe_reduce_col_kernel)
     const float* sp = stripe_res + base;
+    float* agg_col = agg_out != nullptr ? agg_out + base : nullptr;
     const uint32_t items = c.nq * PS::CHUNKS;
+    // A QWord's bit positions are nq elements apart; element i lies 4 * i bytes into the column, in memory as in LDS, and
+    // all of a column's addresses are a base that every thread shares plus a 32-bit offset.
+    const uint32_t step = c.nq * 4u, end = c.rows * 4u;
     // the QWords of this column in the first BATCH workers' records, in summation order (beyond the last worker: the last
     // one's again, fetched and not used). Looked up once: inside the loop over the work items every worker's pointer
     // would be fetched from the kernel's arguments again, one after the other, before the loads that need it go out.
-    const uint32_t* first[BATCH];
+    const char* first[BATCH];
 #pragma unroll
     for (uint32_t u = 0; u < BATCH; ++u)
-        first[u] = reinterpret_cast<const uint32_t*>(src.q[stripe_order(min(u, K - 1u), src.owner)] + rec + 8);
-    uint32_t word[BATCH];
-    float resid[PS::SLOTS];
-    if (tid < items)
-    {
-        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : tid / c.nq;
-        const uint32_t w = tid - chunk * c.nq;
+        first[u] = src.q[stripe_order(min(u, K - 1u), src.owner)] + rec + 8;
+    uint32_t word[BATCH], word_next[BATCH];
+    float resid[PS::SLOTS], resid_next[PS::SLOTS];
+    // (a row beyond the column reads the last row instead, and is not used: no branch around any of the loads)
+    auto fetch = [&](uint32_t it, uint32_t (&wd)[BATCH], float (&rs)[PS::SLOTS]) {
+        const uint32_t chunk = chunk_of_item<PS::CHUNKS>(it, c.nq);
+        const uint32_t w = it - chunk * c.nq;
 #pragma unroll
         for (uint32_t u = 0; u < BATCH; ++u)
-            word[u] = first[u][w];
-        // (a row beyond the column reads the last row instead, and is not used: no branch around any of the loads)
+            wd[u] = *reinterpret_cast<const uint32_t*>(first[u] + w * 4u);
+        uint32_t off = (w + chunk * PS::SLOTS * c.nq) * 4u;
 #pragma unroll
         for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
-            resid[kk] = __builtin_nontemporal_load(sp + min(w + (chunk * PS::SLOTS + kk) * c.nq, c.rows - 1u));
+        {
+            rs[kk] = __builtin_nontemporal_load(reinterpret_cast<const float*>(reinterpret_cast<const char*>(sp) + min(off, end - 4u)));
+            off += step;
+        }
+    };
+    if (tid < items)
+        fetch(tid, word, resid);
+    auto table_of = [&](uint32_t n) { return n < BATCH ? dec + n * DEC : dec_more + (n - BATCH) * DEC; };
+    if constexpr (NBITS == 2)
+    {
+        // entry x of a worker: the levels of codes x & 3 and x >> 2, side by side
+        for (uint32_t x = tid; x < K * 16u; x += WG)
+        {
+            const uint32_t n = x / 16u, e = x % 16u;
+            const float* h = reinterpret_cast<const float*>(src.q[stripe_order(n, src.owner)] + rec);
+            const ValueQ vq = make_vq<NBITS>(h[0], h[1]);
+            float* t = table_of(n);
+            t[2 * e] = unquantize_value<NBITS>(vq, e & 3u);
+            t[2 * e + 1] = unquantize_value<NBITS>(vq, e >> 2);
+        }
     }
-    constexpr uint32_t DEC = stripe_dec_floats(NBITS);
-    constexpr bool LEVELS = DEC > 2; // every level of every worker in LDS
-    if constexpr (LEVELS)
+    else if constexpr (NBITS == 4)
     {
         for (uint32_t x = tid; x < K * DEC; x += WG)
         {
-            const float* h = reinterpret_cast<const float*>(src.q[stripe_order(x / DEC, src.owner)] + rec);
-            dec[x] = unquantize_value<NBITS>(make_vq<NBITS>(h[0], h[1]), x % DEC);
+            const uint32_t n = x / DEC, e = x % DEC;
+            const float* h = reinterpret_cast<const float*>(src.q[stripe_order(n, src.owner)] + rec);
+            table_of(n)[e] = unquantize_value<NBITS>(make_vq<NBITS>(h[0], h[1]), e);
         }
     }
     else if (tid < K)
     {
         const float* h = reinterpret_cast<const float*>(src.q[stripe_order(tid, src.owner)] + rec);
         const ValueQ vq = make_vq<NBITS>(h[0], h[1]);
+        float* t = table_of(tid);
         if constexpr (NBITS == 1)
         {
-            dec[2 * tid] = unquantize_value<NBITS>(vq, 0u);
-            dec[2 * tid + 1] = unquantize_value<NBITS>(vq, 1u);
+            t[0] = unquantize_value<NBITS>(vq, 0u);
+            t[1] = unquantize_value<NBITS>(vq, 1u);
         }
         else
         {
-            dec[2 * tid] = vq.uf;
-            dec[2 * tid + 1] = vq.lo;
+            t[0] = vq.uf;
+            t[1] = vq.lo;
         }
     }
     __syncthreads();
 
     for (uint32_t it = tid; it < items; it += WG)
     {
-        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / c.nq;
+        const uint32_t chunk = chunk_of_item<PS::CHUNKS>(it, c.nq);
         const uint32_t w = it - chunk * c.nq;
-        const size_t word_off = rec + 8 + (size_t) w * 4;
+        const uint32_t off0 = (w + chunk * PS::SLOTS * c.nq) * 4u;
         const uint32_t sh0 = chunk * PS::SLOTS * PS::SHIFT;
-        if (it != tid)
-        {
-#pragma unroll
-            for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
-                resid[kk] = __builtin_nontemporal_load(sp + min(w + (chunk * PS::SLOTS + kk) * c.nq, c.rows - 1u));
-        }
+        // the next work item's inputs are on their way while this one's are summed
+        if (it + WG < items)
+            fetch(it + WG, word_next, resid_next);
         float acc[PS::SLOTS];
-        for (uint32_t n0 = 0; n0 < K; n0 += BATCH)
+        // up to eight workers (the tables at offsets the compiler knows), then the others eight at a time
+        if (K >= BATCH)
+            stripe_add_group<NBITS, true, true>(acc, word, sh0, BATCH, dec);
+        else
+            stripe_add_group<NBITS, true, false>(acc, word, sh0, K, dec);
+        for (uint32_t n0 = BATCH; n0 < K; n0 += BATCH)
         {
-            if (n0 != 0)
-            {
-#pragma unroll
-                for (uint32_t u = 0; u < BATCH; ++u)
-                    if (n0 + u < K)
-                        word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(n0 + u, src.owner)] + word_off);
-            }
-            else if (it != tid)
-            {
-#pragma unroll
-                for (uint32_t u = 0; u < BATCH; ++u)
-                    word[u] = first[u][w];
-            }
 #pragma unroll
             for (uint32_t u = 0; u < BATCH; ++u)
-            {
-                if (n0 + u < K)
-                {
-                    const uint32_t bits = word[u] >> sh0;
-                    if constexpr (LEVELS)
-                    {
-                        const float* lev = dec + (n0 + u) * DEC;
-#pragma unroll
-                        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
-                        {
-                            const float x = lev[(bits >> (kk * PS::SHIFT)) & PS::CODEMASK];
-                            acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
-                        }
-                    }
-                    else
-                    {
-                        const float a = dec[2 * (n0 + u)];
-                        const float b = dec[2 * (n0 + u) + 1];
-#pragma unroll
-                        for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
-                        {
-                            float x;
-                            if constexpr (NBITS == 1)
-                                x = pick_level(bits, kk, a, b);
-                            else
-                                x = unquantize_value<NBITS>(a, b, (bits >> (kk * PS::SHIFT)) & PS::CODEMASK);
-                            // the first term (the owner's) seeds the sum; afterwards: decoded value + running sum
-                            acc[kk] = (n0 + u == 0) ? x : x + acc[kk];
-                        }
-                    }
-                }
-            }
+                word[u] = *reinterpret_cast<const uint32_t*>(src.q[stripe_order(min(n0 + u, K - 1u), src.owner)] + rec + 8 + w * 4u);
+            stripe_add_group<NBITS, false, false>(acc, word, sh0, min(K - n0, BATCH), dec_more + (n0 - BATCH) * DEC);
         }
+        // only the last of a QWord's bit positions can lie beyond the end of a column of more than VPW * VPW rows
+        if (off0 + (PS::SLOTS - 1u) * step < end)
+            stripe_store_item<NBITS, false>(acc, resid, BATCH * DEC * 4u, agg_col, off0, step, end);
+        else
+            stripe_store_item<NBITS, true>(acc, resid, BATCH * DEC * 4u, agg_col, off0, step, end);
+#pragma unroll
+        for (uint32_t u = 0; u < BATCH; ++u)
+            word[u] = word_next[u];
 #pragma unroll
         for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
-        {
-            const uint32_t i = w + (chunk * PS::SLOTS + kk) * c.nq;
-            if (i < c.rows)
-            {
-                if (agg_out != nullptr)
-                    agg_out[base + i] = acc[kk];
-                tile[i] = acc[kk] + resid[kk];
-            }
-        }
+            resid[kk] = resid_next[kk];
     }
     float stat = 0.0f;
     // the quantize kernels' summation order for a residual at this address
@@ -853,20 +963,21 @@ __device__ __forceinline__ void stripe_reduce_colg_body(const StripeSources& src
     {
         __syncthreads();
         const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
-        if (WG == T || tid < T)
+        if (WGT == (int) T || tid < T)
             for (uint32_t v = tid; v < c.pieces + shift; v += T)
                 if (v >= shift)
                     stat = colg_add_piece<NBITS>(stat, t4[v - shift]);
     }
-    colg_stats_pack<NBITS, ZT, WG>(tile, words, red, c, stat, shift, stripe_res + base, q_out + rec);
+    colg_stats_pack<NBITS, ZT, WGT>(tile, words, red, c, stat, shift, stripe_res + base, q_out + rec);
 }
 
-template <int NBITS, bool ZT, int WG>
-__global__ __launch_bounds__(WG) void stripe_reduce_colg_kernel(StripeSources src, float* stripe_res, char* q_out, float* agg_out,
-                                                                ColGeom c)
+// WGT: the workgroup's size, or 0 for any multiple of 64 from 256 to 1024 (the launch says)
+template <int NBITS, bool ZT, int WGT>
+__global__ __launch_bounds__(WGT == 0 ? 1024 : WGT) CNTKQ_SGPRS_FOR_8_WAVES void stripe_reduce_colg_kernel(StripeSources src, float* stripe_res, char* q_out, float* agg_out,
+                                                                                   ColGeom c)
 {
     extern __shared__ f32x4 smem_v4[];
-    stripe_reduce_colg_body<NBITS, ZT, WG>(src, stripe_res, q_out, agg_out, c, blockIdx.x, smem_v4);
+    stripe_reduce_colg_body<NBITS, ZT, WGT>(src, stripe_res, q_out, agg_out, c, blockIdx.x, smem_v4);
 }
 
 } // namespace cntkq

@@ -46,12 +46,22 @@ struct PackShapeOf
 template <int NBITS>
 using PackShape = PackShapeOf<NBITS, 32>;
 
-// What a stripe reduction keeps in LDS per worker and column to decode that worker's codes: at 2 and 4 bits every level
-// of the column (a decoded value is then one LDS read at the code's offset: three vector instructions per value and
-// worker instead of six), at 1 bit the two levels, else (ufactor, lower).
+// What a stripe reduction keeps in LDS per worker and column to decode that worker's codes: at 4 bits every level of the
+// column (a decoded value is then one LDS read at the code's offset: three vector instructions per value and worker instead
+// of six); at 2 bits the levels of two neighbouring codes side by side, for each of their 16 combinations (one 8-byte
+// LDS read at the offset that the four bits make decodes two values); at 1 bit the two levels; else (ufactor, lower).
 __host__ __device__ constexpr uint32_t stripe_dec_floats(size_t nbits)
 {
-    return (nbits == 2 || nbits == 4) ? (1u << nbits) : 2u;
+    return nbits == 2 ? 32u : (nbits == 4 ? 16u : 2u);
+}
+
+// The workers whose tables sit at the front of LDS (room for them is always there), at offsets the compiler knows
+constexpr uint32_t kStripeDecGroup = 8;
+
+// ... in bytes for `workers` workers, with room to start the later workers' tables on an 8-byte boundary
+__host__ __device__ constexpr size_t stripe_dec_bytes(size_t nbits, size_t workers)
+{
+    return (size_t) stripe_dec_floats(nbits) * (workers < kStripeDecGroup ? kStripeDecGroup : workers) * sizeof(float) + 8;
 }
 
 struct TileGeom

@@ -418,7 +418,7 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
 }
 
 template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kThreads) void stripe_reduce_tile_kernel(StripeSources src, double* stripe_res, char* q_out,
+__global__ __launch_bounds__(kThreads) CNTKQ_SGPRS_FOR_8_WAVES void stripe_reduce_tile_kernel(StripeSources src, double* stripe_res, char* q_out,
                                                                       double* agg_out, TileGeom t)
 {
     extern __shared__ f64x2 smem_f64[];
@@ -867,7 +867,7 @@ struct StripeBatchEntry64
 };
 
 template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kThreads) void stripe_reduce_batch_kernel64(const StripeBatchEntry64* __restrict__ entries,
+__global__ __launch_bounds__(kThreads) CNTKQ_SGPRS_FOR_8_WAVES void stripe_reduce_batch_kernel64(const StripeBatchEntry64* __restrict__ entries,
                                                                          const uint32_t* __restrict__ begins, uint32_t count)
 {
     extern __shared__ f64x2 smem_f64[];

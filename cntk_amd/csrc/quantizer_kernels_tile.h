@@ -435,7 +435,7 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
 }
 
 template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kTileThreads) void stripe_reduce_tile_kernel(StripeSources src, float* stripe_res,
+__global__ __launch_bounds__(kTileThreads) CNTKQ_SGPRS_FOR_8_WAVES void stripe_reduce_tile_kernel(StripeSources src, float* stripe_res,
                                                                           char* q_out, float* agg_out, TileGeom t)
 {
     stripe_reduce_tile_body<NBITS, ZT>(src, stripe_res, q_out, agg_out, t, blockIdx.x);

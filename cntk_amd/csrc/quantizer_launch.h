@@ -31,7 +31,6 @@ constexpr uint32_t kStripPollPause = 64;           // strip kernel: 64-cycle pau
 constexpr uint32_t kStripFirstPauseMinStrips = 16; // ... strips per column from which a pause of 2 x strips precedes the first poll
 constexpr uint32_t kStripeWideItems = 768;   // work items per column from which the stripe reduction may use more than 256 threads
 constexpr uint32_t kStripeWideMaxCols = 256; // ... 1024 threads up to this many columns
-constexpr uint32_t kStripeMidMinRows = 6144; // ... 512 threads above this height
 constexpr uint32_t kColMinRows = 1024;   // shorter columns are better served several to a workgroup (tile kernels)
 
 // The scratch buffer of the strip kernels (partial sums of the columns' workgroups and the launch count), owned by a handle: one

@@ -16,6 +16,26 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef f32x4 f32x4_u __attribute__((aligned(4))); // a 16-byte access at any 4-byte alignment
+
+// For kernels meant to run eight wavefronts per SIMD. A SIMD's 800 scalar registers are dealt in blocks of 16, and every
+// wavefront gets 16 more than its kernel asks for (measured with a kernel that does nothing but hold registers: up to 80
+// scalar registers eight wavefronts per SIMD are resident, up to 96 seven, beyond that six); the compiler counts without
+// those 16 and would take up to 96. The kernels that get a set of stripes by value are the ones that reach that many.
+#define CNTKQ_SGPRS_FOR_8_WAVES __attribute__((amdgpu_num_sgpr(80)))
+
+// LDS by byte address, for kernels that declare no LDS of their own and get all of theirs from the launch (theirs starts
+// at address 0). Through an `extern __shared__` array that start reaches the compiler too late to be folded into the
+// instructions: every access at a computed offset then carries an addition of zero, which these do not.
+template <typename T>
+__device__ __forceinline__ T lds_read(uint32_t byte_address)
+{
+    return *(const __attribute__((address_space(3))) T*) byte_address;
+}
+template <typename T>
+__device__ __forceinline__ void lds_write(uint32_t byte_address, T v)
+{
+    *(__attribute__((address_space(3))) T*) byte_address = v;
+}
 typedef u32x4 u32x4_u __attribute__((aligned(4)));
 typedef f32x2 f32x2_u __attribute__((aligned(4)));
 
@@ -141,12 +161,12 @@ __device__ __forceinline__ typename Word<E>::Q quantize_value(const ValueQOf<E>&
     }
     else
     {
+        // (written as selects: with early returns the compiler branches around the conversion for every value, and the
+        // kernels that code many values per thread spend more on the branches than on the arithmetic; a value outside the
+        // range converts to something that is not used)
         constexpr Q top = ((Q) 1 << (NBITS & 63)) - (Q) 1;
-        if (u <= v.lo)
-            return (Q) 0;
-        if (u >= v.hi)
-            return top;
-        return (Q) (typename Word<E>::S)((u - v.lo) * v.qf);
+        const Q inside = (Q) (typename Word<E>::S)((u - v.lo) * v.qf);
+        return u <= v.lo ? (Q) 0 : (u >= v.hi ? top : inside);
     }
 }
 

@@ -56,3 +56,26 @@ def test_headline_kernels_spill_nothing():
             seen += 1
             assert int(k["ScratchSize"]) == 0, "%s uses %s bytes of scratch per lane" % (n, k["ScratchSize"])
     assert seen >= 20
+
+
+def wavefronts_by_scalar_registers(sgprs):
+    """Resident wavefronts per SIMD that a kernel's scalar registers allow on the MI355X as it runs here: every wavefront
+    is given 16 scalar registers beyond its kernel's own, in blocks of 16, out of 800 per SIMD (measured with a kernel that
+    only holds registers: up to 80 -> 8 wavefronts, up to 96 -> 7, beyond -> 6). The compiler's occupancy figure does not
+    count those 16."""
+    return min(8, 800 // ((sgprs + 15) // 16 * 16 + 16))
+
+
+@pytest.mark.parametrize("sources", [FLOAT_SOURCES, ["quantizer_api_f64.hip"]], ids=["float", "double"])
+def test_scalar_registers_cost_the_stripe_kernels_no_wavefront(sources):
+    """The kernels that take a set of stripes by value are the ones that reach 80 scalar registers; they are built with a
+    cap, so the wavefronts that their vector registers allow are the ones that run."""
+    seen = 0
+    for k in all_kernels(sources):
+        n = k["name"]
+        if any(s in n for s in ("stripe_reduce_colg_kernel", "stripe_reduce_batch_kernel", "stripe_reduce_tile_kernel")):
+            seen += 1
+            assert wavefronts_by_scalar_registers(int(k["SGPRs"])) >= int(k["Occupancy"]), \
+                "%s: %s scalar registers allow %d wavefronts per SIMD, its vector registers %s" % (
+                    n, k["SGPRs"], wavefronts_by_scalar_registers(int(k["SGPRs"])), k["Occupancy"])
+    assert seen >= 8
