@@ -98,12 +98,14 @@ __device__ __forceinline__ void tile_pack(E* tile, const E* hdr, typename Word<E
     const uint32_t threads = blockDim.x;
     const uint32_t nwords = nc * t.nq;
     const uint32_t items = nwords * PS::CHUNKS;
+    // (a tile lives in LDS, so its item numbers are far below the 2^20 that small_div takes)
+    const float inv_nwords = small_divisor(nwords), inv_nq = small_divisor(t.nq);
     for (uint32_t it = threadIdx.x; it < items; it += threads)
     {
         // chunk-major: consecutive threads take consecutive QWords, hence consecutive rows
-        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
+        const uint32_t chunk = (PS::CHUNKS == 1 || nc == 1) ? (PS::CHUNKS == 1 ? 0u : it / nwords) : small_div(it, inv_nwords);
         const uint32_t qi = it - chunk * nwords;
-        const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
+        const uint32_t c = (nc == 1) ? 0u : small_div(qi, inv_nq);
         const uint32_t w = qi - c * t.nq;
         const ValueQOf<E> vq = make_vq<NBITS>(hdr[2 * c], hdr[2 * c + 1]);
         const E val0 = unquantize_value<NBITS>(vq, 0u);
@@ -143,7 +145,7 @@ __device__ __forceinline__ void tile_pack(E* tile, const E* hdr, typename Word<E
         __syncthreads();
         for (uint32_t qi = threadIdx.x; qi < nwords; qi += threads)
         {
-            const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
+            const uint32_t c = (nc == 1) ? 0u : small_div(qi, inv_nq);
             const uint32_t w = qi - c * t.nq;
             reinterpret_cast<QWord*>(qtile + (size_t) c * t.qcol + 2 * sizeof(E))[w] = words[qi];
         }
@@ -352,9 +354,10 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
 
     // decode constants from every worker's column header, stored in summation order:
     // 1 bit -> the two levels, else (ufactor, lower)
+    const float inv_k = small_divisor(K);
     for (uint32_t x = tid; x < nc * K; x += t.threads)
     {
-        const uint32_t c = x / K;
+        const uint32_t c = small_div(x, inv_k);
         const uint32_t n = x - c * K;
         const float* h = reinterpret_cast<const float*>(src.q[stripe_order(n, src.owner)] + (size_t) (j0 + c) * t.qcol);
         const ValueQ vq = make_vq<NBITS>(h[0], h[1]);
@@ -372,11 +375,12 @@ __device__ __forceinline__ void stripe_reduce_tile_body(const StripeSources& src
     __syncthreads();
 
     const uint32_t items = nwords * PS::CHUNKS;
+    const float inv_nwords = small_divisor(nwords), inv_nq = small_divisor(t.nq);
     for (uint32_t it = tid; it < items; it += t.threads)
     {
-        const uint32_t chunk = (PS::CHUNKS == 1) ? 0u : it / nwords;
+        const uint32_t chunk = (PS::CHUNKS == 1 || nc == 1) ? (PS::CHUNKS == 1 ? 0u : it / nwords) : small_div(it, inv_nwords);
         const uint32_t qi = it - chunk * nwords;
-        const uint32_t c = (nc == 1) ? 0u : qi / t.nq;
+        const uint32_t c = (nc == 1) ? 0u : small_div(qi, inv_nq);
         const uint32_t w = qi - c * t.nq;
         const size_t word_off = (size_t) (j0 + c) * t.qcol + 8 + (size_t) w * 4;
         const uint32_t sh0 = chunk * PS::SLOTS * PS::SHIFT;

@@ -27,6 +27,7 @@ enum QuantizePath
 };
 
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
+constexpr size_t kTileMaxFloats = 5120;   // ... and 20 KB for a tile of several columns
 constexpr uint32_t kStripPollPause = 64;           // strip kernel: 64-cycle pauses between two polls of a partial sum
 constexpr uint32_t kStripFirstPauseMinStrips = 16; // ... strips per column from which a pause of 2 x strips precedes the first poll
 constexpr uint32_t kStripeWideItems = 768;   // work items per column from which the stripe reduction may use more than 256 threads
@@ -107,9 +108,12 @@ inline TileGeom make_tile_geom(size_t rows, size_t cols, size_t nbits, uint32_t 
             gs <<= 1;
     if (gs > threads)
         gs = threads;
-    // a tile may not exceed 4096 floats (16 KB) unless it is a single column: small tiles keep many
-    // workgroups resident per CU, which is what hides the barrier-separated phases of each of them
-    while (gs < threads && (size_t) (threads / gs) * rows > 4096)
+    // a tile may not exceed 5120 floats (20 KB) unless it is a single column: eight workgroups, all that a compute unit's
+    // wavefront slots take, then still find room in its LDS, and it is the number of resident workgroups that hides the
+    // barrier-separated phases of each of them. (Measured over limits of 2048 / 4096 / 5120 / 8192 floats, quantize and
+    // stripe reduction over 4 workers: 147 x 100000 37 / 34 / 34 / 34 and 58 / 49 / 45 / 45 us, 576 x 30000 46 / 37 / 37 / 38
+    // and 70 / 57 / 49 / 49 us, 1000 x 18000 - / 39 / 39 / 47 and - / 49 / 48 / 72 us.)
+    while (gs < threads && (size_t) (threads / gs) * rows > kTileMaxFloats)
         gs <<= 1;
     t.threads = threads;
     t.gs = gs;

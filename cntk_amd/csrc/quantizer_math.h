@@ -17,6 +17,18 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef f32x4 f32x4_u __attribute__((aligned(4))); // a 16-byte access at any 4-byte alignment
 
+// floor(a / d) for a below 2^20, given inv = small_divisor(d): four instructions where the integer division takes thirty.
+// (a + 0.5) / d lies at least 0.5 / d away from every integer, the reciprocal and the product are off by less than
+// 2^-22 of the quotient together, and (a + 0.5) * 2^-21 stays below 1.
+__device__ __forceinline__ float small_divisor(uint32_t d)
+{
+    return __builtin_amdgcn_rcpf((float) d);
+}
+__device__ __forceinline__ uint32_t small_div(uint32_t a, float inv)
+{
+    return (uint32_t) (((float) a + 0.5f) * inv);
+}
+
 // For kernels meant to run eight wavefronts per SIMD. A SIMD's 800 scalar registers are dealt in blocks of 16, and every
 // wavefront gets 16 more than its kernel asks for (measured with a kernel that does nothing but hold registers: up to 80
 // scalar registers eight wavefronts per SIMD are resident, up to 96 seven, beyond that six); the compiler counts without

@@ -36,6 +36,7 @@ def main():
                     "5 column in registers (one element per access), 6 several workgroups per column (strips)")
     ap.add_argument("--unq-mode", type=int, default=0, help="decoder choice: 0 automatic, 1 QWord-major with one store per value, 2 tile decoder, 3 automatic without the tile "
                     "decoder, 4 row-major decoder")
+    ap.add_argument("--tile-gs", type=int, default=0, help="threads per column of the tile kernels' statistics phase (0: the library's choice)")
     ap.add_argument("--budget-mb", type=int, default=1600, help="device memory for the rotating buffer sets")
     args = ap.parse_args()
 
@@ -46,7 +47,7 @@ def main():
     sfx = "_f64" if args.dtype == "f64" else ""
     L = cntk_amd.lib()
     qz = MatrixQuantizerImpl.Create(0, False)
-    qz._set_tuning(quantize_path=args.path, unq_mode=args.unq_mode)
+    qz._set_tuning(quantize_path=args.path, unq_mode=args.unq_mode, tile_gs=args.tile_gs)
     h = qz._h
 
     # no fused stripe reduction above this height: the other two calls are still measured
