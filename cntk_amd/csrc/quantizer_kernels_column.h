@@ -496,6 +496,11 @@ struct ColGeom
 
 // LDS: [stripe reductions: the first workers' decoding tables | column | partial QWords (nq when a QWord has several work
 // items) | kColgRedSlots reduction slots | stripe reductions: further workers' tables]; workers = 0: a quantize kernel
+// Columns from this height on hand their residual back through LDS where a bit position's runs do not start on 128-byte
+// lines (stripe reduction over 8 workers, staged against direct: 1152 x 16384 at 1 bit 63 against 60 us, 1536 x 12288 52
+// against 48, 2304 x 8192 at 2 bits 48 against 46, 3000 x 6300 45.5 against 45.2, 4100 x 4600 at 4 bits 52 against 55,
+// 5000 x 3800 46 against 48, 7000 x 2700 48 against 50, 9304 x 2048 at 2 bits 42 against 45)
+constexpr uint32_t kColStageMinRows = 3073;
 constexpr uint32_t kColgRedSlots = 16; // 4 + 4 split sums, 4 counts, 4 sums for the mean or the sum of squares
 template <int NBITS>
 __host__ __device__ inline size_t colg_lds_bytes(const ColGeom& c, uint32_t workers)
@@ -622,21 +627,33 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
     // registers). In a column of more than VPW * VPW rows only a QWord's last bit position can lie beyond the end: a work
     // item with all of its elements inside runs without a branch per element.
     const uint32_t step = c.nq * 4u, end = c.rows * 4u;
-    auto pack_item = [&](uint32_t off, auto guard) {
+    // A wavefront's store of one bit position is a run of 256 bytes; where the runs of a column do not all start on 128-byte
+    // lines (the column starts inside a line, or its QWords are not a multiple of 32) they end in partial lines, which the
+    // memory writes by reading the line first: 9304 x 2048 then moves 24 MB more than its 195 MB. There the residual goes
+    // back into the LDS column instead (an element is read by the one thread that replaces it) and leaves afterwards in
+    // whole lines -- from kColStageMinRows rows on: shorter columns lose more by the barrier and the second pass than
+    // they gain. (A column staged in memory is its own residual: nothing to stage.)
+    const bool staged = c.rows >= kColStageMinRows && reinterpret_cast<const void*>(tile) != reinterpret_cast<const void*>(res_col) &&
+                        ((c.nq & 31u) != 0 || (reinterpret_cast<uintptr_t>(res_col) & 127u) != 0);
+    auto pack_item = [&](uint32_t off, auto guard, auto to_lds) {
         uint32_t word = 0;
 #pragma unroll
         for (uint32_t kk = 0; kk < PS::SLOTS; ++kk)
         {
             if (!decltype(guard)::value || off < end)
             {
-                const float v = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(tile) + off);
+                float* at = reinterpret_cast<float*>(reinterpret_cast<char*>(tile) + off);
+                const float v = *at;
                 const uint32_t code = quantize_value<NBITS, ZT>(vq, v);
                 float back;
                 if constexpr (NBITS == 1)
                     back = code ? val1 : val0;
                 else
                     back = unquantize_value<NBITS>(vq, code);
-                __builtin_nontemporal_store(v - back, reinterpret_cast<float*>(reinterpret_cast<char*>(res_col) + off));
+                if constexpr (decltype(to_lds)::value)
+                    *at = v - back;
+                else
+                    __builtin_nontemporal_store(v - back, reinterpret_cast<float*>(reinterpret_cast<char*>(res_col) + off));
                 word |= code << (kk * PS::SHIFT);
             }
             off += step;
@@ -650,21 +667,32 @@ __device__ __forceinline__ void colg_stats_pack(float* tile, uint32_t* words, fl
         const uint32_t w = it - chunk * c.nq;
         const uint32_t off = (w + chunk * PS::SLOTS * c.nq) * 4u;
         uint32_t word;
-        if (off + (PS::SLOTS - 1u) * step < end)
-            word = pack_item(off, std::false_type());
+        const bool whole = off + (PS::SLOTS - 1u) * step < end;
+        if (staged)
+            word = whole ? pack_item(off, std::false_type(), std::true_type()) : pack_item(off, std::true_type(), std::true_type());
         else
-            word = pack_item(off, std::true_type());
+            word = whole ? pack_item(off, std::false_type(), std::false_type()) : pack_item(off, std::true_type(), std::false_type());
         word <<= chunk * PS::SLOTS * PS::SHIFT;
         if constexpr (PS::CHUNKS == 1)
             bits[w] = word;
         else
             atomicOr(&words[w], word);
     }
+    if (PS::CHUNKS > 1 || staged)
+        __syncthreads();
     if constexpr (PS::CHUNKS > 1)
     {
-        __syncthreads();
         for (uint32_t w = tid; w < c.nq; w += WG)
             bits[w] = words[w];
+    }
+    if (staged)
+    {
+        // slot v holds piece v - shift: wavefronts cover whole lines (see column_shift)
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(tile);
+        f32x4* r4 = reinterpret_cast<f32x4*>(res_col);
+        for (uint32_t v = tid; v < c.pieces + shift; v += WG)
+            if (v >= shift)
+                __builtin_nontemporal_store(t4[v - shift], r4 + (v - shift));
     }
 }
 
