@@ -106,6 +106,8 @@ def lib():
             getattr(L, name).restype = _sz
         L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int]
         L.cntkq_debug_set_strip_spin_limit.argtypes = [_vp, ctypes.c_uint]
+        L.cntkq_debug_strip_max_strips.argtypes = [_vp, _sz, ctypes.c_int]
+        L.cntkq_debug_strip_max_strips.restype = ctypes.c_uint
         L.cntkq_set_force_sync.argtypes = [_vp, ctypes.c_int]
         _lib = L
     return _lib
@@ -546,6 +548,10 @@ class MatrixQuantizerImpl:
 
     def _set_strip_spin_limit(self, limit):
         _check(lib().cntkq_debug_set_strip_spin_limit(self._h, limit))
+
+    def _strip_max_strips(self, nbits, zero_threshold_for_1bit=False):
+        """Most strips per column that the strip kernels take on this device at this bit width (0: none)."""
+        return int(lib().cntkq_debug_strip_max_strips(self._h, nbits, 1 if zero_threshold_for_1bit else 0))
 
 
 class MatrixQuantizer:

@@ -824,6 +824,15 @@ int cntkq_debug_set_strip_spin_limit(cntkq_quantizer* h, unsigned limit)
     return CNTKQ_OK;
 }
 
+unsigned cntkq_debug_strip_max_strips(cntkq_quantizer* h, size_t nbits, int zero_threshold_for_1bit)
+{
+    if (h == nullptr || !valid_nbits(nbits) || nbits >= 32)
+        return 0;
+    DeviceGuard guard(h->device);
+    const uint32_t resident = strip_resident_limit(nbits, zero_threshold_for_1bit != 0 && nbits == 1);
+    return resident < kStripMaxPerColumn ? resident : kStripMaxPerColumn;
+}
+
 int cntkq_debug_attach_events(cntkq_quantizer* h, void* start_event, void* stop_event)
 {
     if (h == nullptr)

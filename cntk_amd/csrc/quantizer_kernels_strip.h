@@ -20,7 +20,7 @@
 // kept in the scratch buffer itself: every workgroup reads it when it starts, and the last workgroup to finish (a second
 // counter tells) raises it, so that replays of a recorded graph see fresh tags like any other launch. The strips of a
 // column take workgroup indices 8 apart: the device's eight dies take the workgroups of a grid in turn, so a column's
-// strips run on one die, next to each other in its queue, and start together (at most 64 of them: all must be resident
+// strips run on one die, next to each other in its queue, and start together (at most half of what the die holds: all must be resident
 // at once). That placement is what the hardware does, not what any specification promises, so the wait is bounded: after
 // `spin_limit` polls a lane gives up. A workgroup that gave up raises the error word, marks its own records as abandoned
 // (the launch's tag with the top bit set) and stores nothing: no header, no codes, no residual. A workgroup of the same

@@ -314,10 +314,11 @@ inline bool regs_applicable(size_t rows, size_t nbits)
 // ---- strip kernels: any height, several workgroups per column ------------------------------------------------------
 
 
-// The workgroups of a column wait for each other and run on one die, so all of them must fit there at once: 64 of them is
-// half of what the 32 compute units of a die hold at four workgroups each (524288 rows at 1 to 4 bits, 262144 at 8,
-// 131072 at 16). Taller columns are left to the kernel that re-reads its column.
-constexpr uint32_t kStripMaxPerColumn = 64;
+// The workgroups of a column wait for each other and run on one die, so all of them must fit there at once: a launch
+// takes at most half of what the die holds of the kernel (strip_resident_limit, asked from the runtime: 80 strips at 1
+// to 4 bits, i.e. 655360 rows, on a die of 32 compute units at five workgroups each), and never more than this many.
+// Taller columns are left to the kernel that re-reads its column.
+constexpr uint32_t kStripMaxPerColumn = 128;
 
 inline bool strip_applicable(size_t rows, size_t nbits, const LaunchTuning& tune)
 {
@@ -461,7 +462,7 @@ inline int quantize_auto_path(const float* g, const float* r_in, const float* r_
     {
         // What no workgroup's registers hold in whole aligned pieces (the three matrices at different offsets within 16
         // bytes): one element per access up to 98304 rows (as fast there as the strips, and faster below 50000 rows),
-        // then strips of the column on several workgroups, then -- above 64 strips -- the kernel that re-reads its column.
+        // then strips of the column on several workgroups, then -- above what a die holds of them -- the kernel that re-reads its column.
         if (regs_applicable(rows, nbits))
             return kPathRegScalar;
         return strip_available ? kPathStrip : kPathTall;
@@ -511,7 +512,8 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     if (path == kPathStrip)
     {
         const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit);
-        if (!strip_applicable(rows, nbits, tune) || (uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull)
+        if (!strip_applicable(rows, nbits, tune) || (uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull ||
+            c.strips > strip_resident_limit(nbits, zt))
             return hipErrorInvalidValue;
         StripScratchOwner& o = *tune.strip;
         StripScratch scratch;

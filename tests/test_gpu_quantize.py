@@ -141,7 +141,7 @@ PATH_CASES = [
     (1, 3, PATH_STRIP, 0), (37, 5, PATH_STRIP, 0), (1000, 3, PATH_STRIP, 0), (8192, 3, PATH_STRIP, 0), (8193, 2, PATH_STRIP, 0),
     (9304, 3, PATH_STRIP, 0), (16385, 2, PATH_STRIP, 0), (32768, 2, PATH_STRIP, 0), (50257, 3, PATH_STRIP, 0), (100000, 5, PATH_STRIP, 0),
     (102401, 2, PATH_AUTO, 0), (200000, 3, PATH_AUTO, 0), (262147, 2, PATH_STRIP, 0), (524288, 9, PATH_STRIP, 0), (524289, 1, PATH_AUTO, 0),
-    (1000003, 1, PATH_AUTO, 0),
+    (600000, 9, PATH_STRIP, 0), (655361, 1, PATH_AUTO, 0), (1000003, 1, PATH_AUTO, 0),
 ]
 
 
@@ -152,7 +152,8 @@ def test_kernel_paths(case):
     rep = parity.Report()
     for nbits, zt in VARIANTS:
         say("path case", case, "nbits", nbits, "zeroThr", zt)
-        if path == PATH_STRIP and (nbits == 32 or oracle.qwords_per_col(rows, nbits) > 64 * (256 if nbits == 1 else 512 if nbits == 2 else 1024)):
+        if path == PATH_STRIP and (nbits == 32 or oracle.qwords_per_col(rows, nbits) >
+                                   qz._strip_max_strips(nbits, zt) * (256 if nbits == 1 else 512 if nbits == 2 else 1024)):
             # whole-QWord codes need no assembling, and a column's strips must fit on one die of the device together
             qz._set_tuning(quantize_path=path)
             with pytest.raises(cntk_amd.QuantizerLogicError):
