@@ -153,7 +153,8 @@ __device__ __forceinline__ void reg_stats_pack(f32x4 (&a)[PER], float edge, bool
     const ValueQ vq = make_vq<NBITS>(lo, hi);
     const float val0 = unquantize_value<NBITS>(vq, 0u);
     const float val1 = unquantize_value<NBITS>(vq, 1u);
-    f32x4* o4 = reinterpret_cast<f32x4*>(r_out_col + head);
+    // (with edge elements the residual output may lie at another offset within 16 bytes than the input that the pieces follow)
+    f32x4_u* o4 = reinterpret_cast<f32x4_u*>(r_out_col + head);
     // the first element of this thread's first slot inside the column is bit position k of QWord w; the elements after it
     // are the following QWords, the slots after it lie 4 * T elements further on
     const uint32_t ufirst = tid < shift ? 1u : 0u;
@@ -218,7 +219,8 @@ __device__ __forceinline__ void reg_stats_pack(f32x4 (&a)[PER], float edge, bool
         bits[x] = words[x];
 }
 
-// EDGE: the column need not start on a 16-byte boundary nor hold a multiple of 4 elements: up to 3 elements before the
+// EDGE: the column need not start on a 16-byte boundary nor hold a multiple of 4 elements, and the three matrices need
+// not share their offset within 16 bytes (the aligned pieces are the residual input's): up to 3 elements before the
 // first aligned piece and up to 3 after the last are held, one each, by threads 0..5 and take part in every phase after
 // the thread's pieces. (c.pieces then only bounds the pieces; the count is taken from the column's address.)
 template <int NBITS, bool ZT, int T, int PER, bool EDGE = false>
@@ -242,7 +244,9 @@ __device__ __forceinline__ void quantize_reg_body(const float* __restrict__ g, c
         pieces = (c.rows - head) >> 2;
         tail = c.rows - head - 4 * pieces;
     }
-    const f32x4* g4 = reinterpret_cast<const f32x4*>(g + base + head);
+    // (the pieces follow the residual input; with edge elements the gradient may lie at another offset within 16 bytes)
+    using GradientPiece = typename std::conditional<EDGE, f32x4_u, f32x4>::type;
+    const GradientPiece* g4 = reinterpret_cast<const GradientPiece*>(g + base + head);
     const f32x4* r4 = reinterpret_cast<const f32x4*>(r_in + base + head);
     // the edge element of this thread, if it has one
     const bool has_edge = EDGE && tid < head + tail;

@@ -181,8 +181,22 @@ __device__ __forceinline__ void tile_store(const float* tile, uint32_t mis, floa
     }
     else
     {
-        for (uint32_t e = tid; e < total; e += t.threads)
-            __builtin_nontemporal_store(tile[e], dst + e);
+        // the destination at another phase: 16-byte stores all the same, at the 4-byte alignment that leaves them (a
+        // store per element costs four times the instructions; quantize + unquantize of 2048 x 9304 with the gradient one
+        // float off the residual: 73 -> 58 us, 512 x 37216: 71 -> 58 us)
+        uint32_t head = (4u - mis) & 3u;
+        if (head > total)
+            head = total;
+        const uint32_t nvec = (total - head) >> 2;
+        const uint32_t tail0 = head + (nvec << 2);
+        if (tid < head)
+            dst[tid] = tile[tid];
+        const f32x4* t4 = reinterpret_cast<const f32x4*>(tile + head);
+        f32x4_u* d4 = reinterpret_cast<f32x4_u*>(dst + head);
+        for (uint32_t e = tid; e < nvec; e += t.threads)
+            __builtin_nontemporal_store(t4[e], d4 + e);
+        for (uint32_t e = tail0 + tid; e < total; e += t.threads)
+            dst[e] = tile[e];
     }
 }
 
@@ -282,8 +296,41 @@ __device__ __forceinline__ void quantize_tile_body(const float* __restrict__ g, 
     }
     else
     {
-        for (uint32_t e = tid; e < total; e += t.threads)
-            tile[e] = __builtin_nontemporal_load(gp + e) + __builtin_nontemporal_load(rp + e);
+        // the residual at another phase than the gradient: the gradient in aligned pieces, the residual in 16-byte loads at
+        // the 4-byte alignment that leaves them
+        uint32_t head = (4u - mis_g) & 3u;
+        if (head > total)
+            head = total;
+        const uint32_t nvec = (total - head) >> 2;
+        const uint32_t tail0 = head + (nvec << 2);
+        if (tid < head)
+            tile[tid] = gp[tid] + rp[tid];
+        const f32x4* g4 = reinterpret_cast<const f32x4*>(gp + head);
+        const f32x4_u* r4 = reinterpret_cast<const f32x4_u*>(rp + head);
+        f32x4* t4 = reinterpret_cast<f32x4*>(tile + head);
+        for (uint32_t e0 = tid; e0 < nvec; e0 += 4 * t.threads)
+        {
+            f32x4 a[4], b[4];
+#pragma unroll
+            for (uint32_t u = 0; u < 4; ++u)
+            {
+                const uint32_t e = e0 + u * t.threads;
+                if (e < nvec)
+                {
+                    a[u] = __builtin_nontemporal_load(g4 + e);
+                    b[u] = __builtin_nontemporal_load(r4 + e);
+                }
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 4; ++u)
+            {
+                const uint32_t e = e0 + u * t.threads;
+                if (e < nvec)
+                    t4[e] = a[u] + b[u];
+            }
+        }
+        for (uint32_t e = tail0 + tid; e < total; e += t.threads)
+            tile[e] = gp[e] + rp[e];
     }
     __syncthreads();
 

@@ -419,6 +419,8 @@ __device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q,
     using PS = PackShapeOf<NBITS, Word<E>::kBits>;
     constexpr uint32_t N = 16 / sizeof(E);
     typedef E Vec __attribute__((ext_vector_type(N)));
+    // (the output may start on any element boundary: the 16-byte accesses are then at that alignment)
+    typedef Vec VecAt4 __attribute__((aligned(sizeof(E))));
     const uint32_t tid = threadIdx.x;
     const uint32_t col0 = block * t.cpt;
     const uint32_t ncols = (t.cols - col0 < t.cpt) ? t.cols - col0 : t.cpt;
@@ -489,7 +491,7 @@ __device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q,
                 else
                     x[e] = unquantize_value<NBITS>(d0, d1, code);
             }
-            Vec* o4 = reinterpret_cast<Vec*>(o + i);
+            VecAt4* o4 = reinterpret_cast<VecAt4*>(o + i);
             if (add)
                 x = x + *o4; // unquantized value + previous content
             __builtin_nontemporal_store(x, o4);
@@ -533,7 +535,7 @@ __device__ __forceinline__ void unquantize_tile_body(const char* __restrict__ q,
         }
         if (i + N <= elems)
         {
-            Vec* o4 = reinterpret_cast<Vec*>(o + i);
+            VecAt4* o4 = reinterpret_cast<VecAt4*>(o + i);
             if (add)
                 x = x + *o4; // unquantized value + previous content
             __builtin_nontemporal_store(x, o4);

@@ -275,13 +275,17 @@ inline bool reg_applicable(const float* g, const float* r_in, const float* r_out
     return (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
 }
 
-// The piece-wise register kernel with edge elements: matrices only 4-byte aligned but at the same offset within 16
-// bytes (then every column of all three starts at the same offset), any height from 8 rows on.
+// The piece-wise register kernel with edge elements: matrices only 4-byte aligned, any height from 8 rows on. The aligned
+// pieces are those of the residual input; a gradient or residual output at another offset within 16 bytes is read and
+// written in 16-byte accesses at the 4-byte alignment that leaves them (quantize + unquantize of 50257 x 512 with the three
+// matrices at three offsets: 81 us like the matrices at one offset, against 118 us one element per access; 9304 x 2048:
+// 56.5 against 90 us).
 inline bool reg_edge_applicable(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits)
 {
-    const uintptr_t a = reinterpret_cast<uintptr_t>(g) & 15u, b = reinterpret_cast<uintptr_t>(r_in) & 15u,
-                    c = reinterpret_cast<uintptr_t>(r_out) & 15u;
-    if (a != b || b != c || rows < 8 || rows > kRegMaxRows - 32 || nbits >= 32 || (reinterpret_cast<uintptr_t>(q) & 3u) != 0)
+    (void) g;
+    (void) r_in;
+    (void) r_out;
+    if (rows < 8 || rows > kRegMaxRows - 32 || nbits >= 32 || (reinterpret_cast<uintptr_t>(q) & 3u) != 0)
         return false;
     return (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
 }
@@ -705,7 +709,7 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
     const bool vec_can = (nq % 4 == 0) && (rows % 4 == 0) && out16 && (reinterpret_cast<uintptr_t>(q) & 7u) == 0;
     const bool vec_ideal = vec_can && nq % 32 == 0 && rows % 32 == 0 && rows * nbits == nq * 32;
     const bool rows_can = slots_free && rows >= 16 && nq >= 32 && nq * 4 <= kUnqRowsMaxLds; // any height, any (4-byte) alignment
-    const bool tile_can = slots_free && out16 && rows <= kUnqTileMaxRows;
+    const bool tile_can = slots_free && rows <= kUnqTileMaxRows; // (any 4-byte alignment of the output)
     bool vec = false, rowmajor = false, tile = false, seg_allowed = true;
     if (mode == 1)
         seg_allowed = false; // QWord-major, 4-byte stores

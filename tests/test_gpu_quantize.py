@@ -756,3 +756,52 @@ def test_force_sync_mode_waits_inside_the_calls():
         out_now = Out.to_numpy().copy()
         qz.WaitUnquantizeAsyncDone()
         parity.check_unquantize(q_now, rows, cols, 1, out_now)
+
+
+OFFSET_SHAPES = [(147, 300), (512, 200), (1000, 90), (2048, 40), (2049, 37), (4100, 24), (9304, 16), (20001, 9), (50257, 5)]
+
+
+@pytest.mark.parametrize("shape", OFFSET_SHAPES, ids=["%dx%d" % s for s in OFFSET_SHAPES])
+def test_matrices_at_different_offsets_within_16_bytes(shape):
+    """Gradient, residual and residual output that start at different 4-byte offsets within 16 bytes (slices of larger
+    buffers, the gradient views of a flat communication bucket beside separately allocated residuals): the kernels read and
+    write such matrices in 16-byte accesses at whatever alignment that leaves them -- the tile kernels up to 2048 rows, the
+    register kernels with edge elements above (their aligned pieces are the residual input's) -- and the tile decoder
+    writes to an output at any offset. Checked against the oracle; nothing may be written outside the matrices."""
+    rows, cols = shape
+    qz = MatrixQuantizerImpl.Create(0, False)
+    rep = parity.Report()
+
+    def place(a, off):
+        buf = torch.zeros(a.size + 64, dtype=torch.float32, device="cuda:0")
+        buf[off:off + a.size] = torch.from_numpy(a.reshape(-1, order="F").copy()).cuda()
+        return Matrix(a.shape[0], a.shape[1], 0, buf[off:off + a.size]), buf
+
+    n = 0
+    for offs in ((1, 0, 0), (0, 2, 0), (1, 2, 3), (3, 3, 1), (5, 7, 6)):
+        for nbits, zt in ((1, False), (1, True), (4, False)):
+            n += 1
+            say("offsets", shape, offs, "nbits", nbits, "zeroThr", zt)
+            g = datagen.normal_with_outliers(100 * rows + n, rows, cols, 0.01)
+            r = datagen.normal(200 * rows + n, rows, cols, 0.002)
+            G, _gbuf = place(g, offs[0])
+            R, rbuf = place(r, offs[1])
+            in_place = n % 2 == 0
+            Rout, obuf = (R, rbuf) if in_place else place(np.zeros_like(g, order="F"), offs[2])
+            Q = QuantizedMatrix(rows, cols, nbits, 0)
+            qz.QuantizeAsync(G, R, Q, Rout, zt)
+            qz.WaitQuantizeAsyncDone()
+            torch.cuda.synchronize()
+            q_gpu = Q.to_numpy()
+            parity.check_quantize(g, r, q_gpu, Rout.to_numpy(), nbits, zt, report=rep)
+            off_o = offs[1] if in_place else offs[2]
+            assert float(obuf[:off_o].abs().sum()) == 0.0 and float(obuf[off_o + rows * cols:].abs().sum()) == 0.0
+            prev = datagen.normal(300 * rows + n, rows, cols, 1.0)
+            add = n % 3 == 0
+            Out, outbuf = place(prev, offs[2])
+            qz.UnquantizeAsync(Q, Out, add=add)
+            qz.WaitUnquantizeAsyncDone()
+            torch.cuda.synchronize()
+            parity.check_unquantize(q_gpu, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
+            assert float(outbuf[:offs[2]].abs().sum()) == 0.0 and float(outbuf[offs[2] + rows * cols:].abs().sum()) == 0.0
+    say("  ", rep)
