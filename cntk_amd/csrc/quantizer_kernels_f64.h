@@ -567,7 +567,8 @@ __device__ __forceinline__ void reg_stats_pack(f64x2 (&a)[PER], double edge, boo
     const ValueQ vq = make_vq<NBITS>(lo, hi);
     const double val0 = unquantize_value<NBITS>(vq.uf, vq.lo, 0ull);
     const double val1 = unquantize_value<NBITS>(vq.uf, vq.lo, 1ull);
-    f64x2* o2 = reinterpret_cast<f64x2*>(r_out_col + head);
+    // (the residual output may lie 8 bytes off the residual input that the pieces follow)
+    f64x2_u* o2 = reinterpret_cast<f64x2_u*>(r_out_col + head);
     // the first element of this thread's first slot inside the column is bit position k of QWord w; the element after it
     // is the following QWord, the slots after it lie 2 * T elements further on (step_k, step_w)
     const uint32_t ufirst = tid < shift ? 1u : 0u;
@@ -652,7 +653,8 @@ __global__ __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(reg_waves<T, 
     const uint32_t head = (uint32_t) ((reinterpret_cast<uintptr_t>(r_in + base) >> 3) & 1u);
     const uint32_t pieces = (c.rows - head) >> 1;
     const uint32_t tail = c.rows - head - 2 * pieces;
-    const f64x2* g2 = reinterpret_cast<const f64x2*>(g + base + head);
+    // (the aligned pairs are the residual input's; the gradient may lie 8 bytes off them)
+    const f64x2_u* g2 = reinterpret_cast<const f64x2_u*>(g + base + head);
     const f64x2* r2 = reinterpret_cast<const f64x2*>(r_in + base + head);
     const bool has_edge = (tid == 0 && head != 0) || (tid == 1 && tail != 0);
     const uint32_t edge_at = tid == 0 ? 0u : c.rows - 1;

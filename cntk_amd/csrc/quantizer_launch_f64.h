@@ -117,10 +117,12 @@ constexpr size_t kRegMinRows = 6145; // up to 6144 rows the element-wise registe
 
 inline bool reg_applicable(const double* g, const double* r_in, const double* r_out, size_t rows, size_t nbits)
 {
-    // any height from 4 rows on; the three matrices at the same offset within 16 bytes (then so are all their columns)
-    const uintptr_t a = reinterpret_cast<uintptr_t>(g) & 15u, b = reinterpret_cast<uintptr_t>(r_in) & 15u,
-                    c = reinterpret_cast<uintptr_t>(r_out) & 15u;
-    if (a != b || b != c || rows < 4 || rows > kRegMaxRows - 16 || nbits >= 64)
+    // any height from 4 rows on, any 8-byte alignment: the aligned pairs are the residual input's, gradient and residual
+    // output are read and written in 16-byte accesses wherever they lie
+    (void) g;
+    (void) r_in;
+    (void) r_out;
+    if (rows < 4 || rows > kRegMaxRows - 16 || nbits >= 64)
         return false;
     return (kRegRedSlots + qwords_per_col(rows, nbits)) * 8 <= kMaxLdsBytes;
 }

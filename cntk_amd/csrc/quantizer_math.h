@@ -56,6 +56,7 @@ constexpr int kWave = 64;
 // ---- element types and their QWords (Source/Math/ValueQuantizer.h:48-57) -------------------------
 
 typedef double f64x2 __attribute__((ext_vector_type(2)));
+typedef f64x2 f64x2_u __attribute__((aligned(8))); // a 16-byte access at any 8-byte alignment
 
 // What differs between MatrixQuantizerImpl<float> and <double>: the QWord a column is packed into (as wide as the element),
 // its signed twin for the float -> code conversion, the raw bits of a value (the "code" when NBITS is the QWord's width) and

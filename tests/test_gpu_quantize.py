@@ -805,3 +805,44 @@ def test_matrices_at_different_offsets_within_16_bytes(shape):
             parity.check_unquantize(q_gpu, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
             assert float(outbuf[:offs[2]].abs().sum()) == 0.0 and float(outbuf[offs[2] + rows * cols:].abs().sum()) == 0.0
     say("  ", rep)
+
+
+@pytest.mark.parametrize("shape", [(1000, 60), (4100, 24), (9304, 16), (20001, 9)], ids=lambda s: "%dx%d" % s)
+def test_double_matrices_at_different_offsets_within_16_bytes(shape):
+    """The same for doubles: gradient, residual and residual output 8 bytes apart in their 16-byte phase."""
+    rows, cols = shape
+    qz = MatrixQuantizerImpl.Create(0, False)
+    rep = parity.Report()
+
+    def place(a, off):
+        buf = torch.zeros(a.size + 64, dtype=torch.float64, device="cuda:0")
+        buf[off:off + a.size] = torch.from_numpy(a.reshape(-1, order="F").copy()).cuda()
+        return Matrix(a.shape[0], a.shape[1], 0, buf[off:off + a.size], dtype=torch.float64), buf
+
+    n = 0
+    for offs in ((1, 0, 0), (0, 1, 0), (1, 0, 1), (3, 2, 5)):
+        for nbits, zt in ((1, False), (4, False)):
+            n += 1
+            say("double offsets", shape, offs, "nbits", nbits, "zeroThr", zt)
+            g = datagen.normal_with_outliers(100 * rows + n, rows, cols, 0.01, dtype=np.float64)
+            r = datagen.normal(200 * rows + n, rows, cols, 0.002, dtype=np.float64)
+            G, _gbuf = place(g, offs[0])
+            R, rbuf = place(r, offs[1])
+            in_place = n % 2 == 0
+            Rout, obuf = (R, rbuf) if in_place else place(np.zeros_like(g, order="F"), offs[2])
+            Q = QuantizedMatrix(rows, cols, nbits, 0, dtype=torch.float64)
+            qz.QuantizeAsync(G, R, Q, Rout, zt)
+            qz.WaitQuantizeAsyncDone()
+            torch.cuda.synchronize()
+            q_gpu = Q.to_numpy()
+            parity.check_quantize(g, r, q_gpu, Rout.to_numpy(), nbits, zt, report=rep)
+            off_o = offs[1] if in_place else offs[2]
+            assert float(obuf[:off_o].abs().sum()) == 0.0 and float(obuf[off_o + rows * cols:].abs().sum()) == 0.0
+            prev = datagen.normal(300 * rows + n, rows, cols, 1.0, dtype=np.float64)
+            Out, outbuf = place(prev, offs[2])
+            qz.UnquantizeAsync(Q, Out, add=False)
+            qz.WaitUnquantizeAsyncDone()
+            torch.cuda.synchronize()
+            parity.check_unquantize(q_gpu, rows, cols, nbits, Out.to_numpy())
+            assert float(outbuf[:offs[2]].abs().sum()) == 0.0 and float(outbuf[offs[2] + rows * cols:].abs().sum()) == 0.0
+    say("  ", rep)
