@@ -829,8 +829,7 @@ unsigned cntkq_debug_strip_max_strips(cntkq_quantizer* h, size_t nbits, int zero
     if (h == nullptr || !valid_nbits(nbits) || nbits >= 32)
         return 0;
     DeviceGuard guard(h->device);
-    const uint32_t resident = strip_resident_limit(nbits, zero_threshold_for_1bit != 0 && nbits == 1);
-    return resident < kStripMaxPerColumn ? resident : kStripMaxPerColumn;
+    return strip_max_strips(nbits, zero_threshold_for_1bit != 0 && nbits == 1);
 }
 
 int cntkq_debug_attach_events(cntkq_quantizer* h, void* start_event, void* stop_event)

@@ -15,7 +15,7 @@ struct StripLauncher
             return hipErrorInvalidValue;
         else
         {
-            hipExtLaunchKernelGGL((quantize_strip_kernel<NBITS, ZT>), dim3(strip_grid(cols, c.strips)), dim3(kStripThreads), strip_lds_bytes(NBITS), s,
+            hipExtLaunchKernelGGL((quantize_strip_kernel<NBITS, ZT>), dim3(strip_grid(cols, c)), dim3(kStripThreads), strip_lds_bytes(NBITS), s,
                                   ev.start, ev.stop, 0, g, r_in, r_out, q, c, scratch);
             return hipGetLastError();
         }

@@ -16,7 +16,7 @@ extern "C" {
  *                    5 = the same with one element per access: fp32 any alignment, up to 98304 rows; fp64 256 threads per
  *                        column, 1025 to 6144 rows, below 64 bits, the bytes of path 1
  *                    6 = several workgroups per column, a strip of QWords each (fp32, 1 to 16 bits, any height whose
- *                        strips number at most half of what a die holds of the kernel, any alignment)
+ *                        strips number at most half of what the device holds of the kernel, any alignment)
  *   tile_gs          0 = automatic, else threads per column in the tile statistics phase (power of two, 8..256)
  *   unq_slots        0 = automatic, else bit positions decoded per thread by the QWord-major unquantize
  *   unq_mode         0 = automatic, 1 = QWord-major decoder with one store per value, 2 = tile decoder wherever it can run,
@@ -31,8 +31,9 @@ int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_
 int cntkq_debug_set_strip_spin_limit(cntkq_quantizer* h, unsigned limit);
 
 /* The most strips per column that the strip kernels (path 6) take on the handle's device at this bit width: half of what
- * one die holds of the kernel, as the runtime's occupancy query tells, and never more than 128 (0: unknown, or no strip
- * kernel for the bit width). A strip is 256 / 512 / 1024 QWords at 1 / 2 / 4 and more bits. */
+ * the device holds of the kernel, as the runtime's occupancy query tells (a column of more strips than half a die holds
+ * has them on all eight dies), never more than 8 x 128 (0: unknown, or no strip kernel for the bit width). A strip is
+ * 256 / 512 / 1024 QWords at 1 / 2 / 4 and more bits. */
 unsigned cntkq_debug_strip_max_strips(cntkq_quantizer* h, size_t nbits, int zero_threshold_for_1bit);
 
 /* Ties caller-owned hipEvent_t objects (either may be NULL) to the NEXT kernel this handle launches: start_event is

@@ -21,7 +21,7 @@
 // counter tells) raises it, so that replays of a recorded graph see fresh tags like any other launch. The strips of a
 // column take workgroup indices 8 apart: the device's eight dies take the workgroups of a grid in turn, so a column's
 // strips run on one die, next to each other in its queue, and start together (at most half of what the die holds: all must be resident
-// at once). That placement is what the hardware does, not what any specification promises, so the wait is bounded: after
+// at once; a column of more strips has them side by side in the grid instead, on all dies, up to half of what the device holds). That placement is what the hardware does, not what any specification promises, so the wait is bounded: after
 // `spin_limit` polls a lane gives up. A workgroup that gave up raises the error word, marks its own records as abandoned
 // (the launch's tag with the top bit set) and stores nothing: no header, no codes, no residual. A workgroup of the same
 // column that finds an abandoned record abandons its strip in the same way, without waiting. A column whose strips did
@@ -68,6 +68,8 @@ struct StripGeom
     uint32_t poll_pause; // pauses of 64 cycles between two polls of a record
     uint32_t poll_first; // ... and before the first poll
     double inv_strips;   // for workgroup index -> (column, strip)
+    uint32_t spread;     // non-zero: a column's strips take consecutive workgroup indices, i.e. all dies (columns of more strips than one die holds)
+    uint32_t pad;
     uint64_t qcol;
 };
 
@@ -469,8 +471,17 @@ __device__ __forceinline__ void strip_thread_slots(uint32_t strip, uint32_t& w, 
 // the launch, or false for a workgroup beyond the last column (the grid is rounded up to eight columns).
 __device__ __forceinline__ bool strip_assignment(const StripGeom& c, const StripScratch& scratch, uint32_t& column, uint32_t& strip, uint32_t& tag)
 {
-    divmod_u32(blockIdx.x / kStripDies, c.strips, c.inv_strips, column, strip);
-    column = column * kStripDies + blockIdx.x % kStripDies;
+    if (c.spread)
+    {
+        // a column of more strips than one die holds: its strips side by side in the grid, on all dies, which start them in
+        // order like everything else (the partial sums then meet in memory instead of one die's L2)
+        divmod_u32(blockIdx.x, c.strips, c.inv_strips, column, strip);
+    }
+    else
+    {
+        divmod_u32(blockIdx.x / kStripDies, c.strips, c.inv_strips, column, strip);
+        column = column * kStripDies + blockIdx.x % kStripDies;
+    }
     strip = c.strips - 1 - strip; // the strip at the ragged end of the column, which takes longest, starts first
     // the same tag in every workgroup: the count moves when all of them are done
     const uint32_t copy = (blockIdx.x * (kStripThreads / kWave) + threadIdx.x / kWave) % kStripTagCopies;

@@ -318,19 +318,22 @@ inline bool regs_applicable(size_t rows, size_t nbits)
 // ---- strip kernels: any height, several workgroups per column ------------------------------------------------------
 
 
-// The workgroups of a column wait for each other and run on one die, so all of them must fit there at once: a launch
-// takes at most half of what the die holds of the kernel (strip_resident_limit, asked from the runtime: 80 strips at 1
-// to 4 bits, i.e. 655360 rows, on a die of 32 compute units at five workgroups each), and never more than this many.
-// Taller columns are left to the kernel that re-reads its column.
+// The workgroups of a column wait for each other, so all of them must be resident at once: on one die at most half of
+// what the die holds of the kernel (strip_resident_limit, asked from the runtime: 80 strips at 1 to 4 bits, i.e. 655360
+// rows, on a die of 32 compute units at five workgroups each) and never more than this many; a column of more strips has
+// them on all eight dies, up to eight times as many (5.2 M rows at 1 to 4 bits). Taller columns are left to the kernel
+// that re-reads its column.
 constexpr uint32_t kStripMaxPerColumn = 128;
 
 inline bool strip_applicable(size_t rows, size_t nbits, const LaunchTuning& tune)
 {
     return tune.strip != nullptr && nbits < 32 && rows >= 1 &&
-           (qwords_per_col(rows, nbits) + strip_words(nbits) - 1) / strip_words(nbits) <= kStripMaxPerColumn;
+           (qwords_per_col(rows, nbits) + strip_words(nbits) - 1) / strip_words(nbits) <= kStripMaxPerColumn * kStripDies;
 }
 
-inline StripGeom make_strip_geom(size_t rows, size_t cols, size_t nbits, uint32_t spin_limit)
+// per_die: the most strips of a column that one die takes (strip_resident_limit); a column of more has its strips on all
+// dies (StripGeom::spread), up to kStripDies times as many
+inline StripGeom make_strip_geom(size_t rows, size_t cols, size_t nbits, uint32_t spin_limit, uint32_t per_die)
 {
     StripGeom c;
     c.rows = (uint32_t) rows;
@@ -339,11 +342,14 @@ inline StripGeom make_strip_geom(size_t rows, size_t cols, size_t nbits, uint32_
     c.strips = (c.nq + strip_words(nbits) - 1) / strip_words(nbits);
     c.spin_limit = spin_limit;
     c.poll_pause = kStripPollPause;
-    c.poll_first = c.strips >= kStripFirstPauseMinStrips ? 2u * c.strips : 0u;
+    c.poll_first = c.strips >= kStripFirstPauseMinStrips ? 2u * std::min(c.strips, kStripMaxPerColumn) : 0u;
     c.inv_strips = 1.0 / (double) c.strips;
+    c.spread = c.strips > per_die ? 1u : 0u;
+    c.pad = 0;
     c.qcol = qcol_bytes(nbits, rows);
     return c;
 }
+
 
 inline bool strip_scratch_fits(const StripScratchOwner& o, size_t cols, size_t strips)
 {
@@ -420,9 +426,9 @@ inline bool strip_scratch_ready(const StripScratchOwner& o, hipStream_t s, size_
     return hipStreamIsCapturing(s, &st) == hipSuccess && st == hipStreamCaptureStatusNone;
 }
 
-inline uint32_t strip_grid(size_t cols, size_t strips)
+inline uint32_t strip_grid(size_t cols, const StripGeom& c)
 {
-    return (uint32_t) ((cols + kStripDies - 1) / kStripDies * kStripDies * strips);
+    return (uint32_t) (c.spread ? cols * c.strips : (cols + kStripDies - 1) / kStripDies * kStripDies * c.strips);
 }
 
 // How many strips a column may have for the automatic choice to take the strip kernels: the strips of a column wait for
@@ -448,6 +454,18 @@ inline uint32_t strip_resident_limit(size_t nbits, bool zt)
         slot = (rc == hipSuccess && per_cu > 0 && cus >= (int) kStripDies) ? per_cu * (cus / (int) kStripDies) / 2 : -1;
     }
     return slot > 0 ? (uint32_t) slot : 0u;
+}
+
+// ... the same, never more than kStripMaxPerColumn
+inline uint32_t strip_per_die(size_t nbits, bool zt)
+{
+    return std::min(strip_resident_limit(nbits, zt), kStripMaxPerColumn);
+}
+
+// the most strips per column that the strip kernels take on the current device, spread over all dies
+inline uint32_t strip_max_strips(size_t nbits, bool zt)
+{
+    return strip_per_die(nbits, zt) * kStripDies;
 }
 
 // which path launch_quantize takes for this matrix when nothing is forced
@@ -489,9 +507,9 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
         if (path == kPathStrip)
         {
             // a stream under capture cannot wait for a larger scratch buffer: the kernels that need none take the matrix
-            const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit);
+            const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit, strip_per_die(nbits, zt));
             if ((uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull ||
-                !strip_scratch_ready(*tune.strip, s, cols, c.strips, tune.strip_may_allocate) || c.strips > strip_resident_limit(nbits, zt))
+                !strip_scratch_ready(*tune.strip, s, cols, c.strips, tune.strip_may_allocate) || c.strips > strip_max_strips(nbits, zt))
                 path = regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
         }
     }
@@ -515,9 +533,9 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     }
     if (path == kPathStrip)
     {
-        const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit);
+        const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit, strip_per_die(nbits, zt));
         if (!strip_applicable(rows, nbits, tune) || (uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull ||
-            c.strips > strip_resident_limit(nbits, zt))
+            c.strips > strip_max_strips(nbits, zt))
             return hipErrorInvalidValue;
         StripScratchOwner& o = *tune.strip;
         StripScratch scratch;

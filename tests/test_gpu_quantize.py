@@ -141,7 +141,7 @@ PATH_CASES = [
     (1, 3, PATH_STRIP, 0), (37, 5, PATH_STRIP, 0), (1000, 3, PATH_STRIP, 0), (8192, 3, PATH_STRIP, 0), (8193, 2, PATH_STRIP, 0),
     (9304, 3, PATH_STRIP, 0), (16385, 2, PATH_STRIP, 0), (32768, 2, PATH_STRIP, 0), (50257, 3, PATH_STRIP, 0), (100000, 5, PATH_STRIP, 0),
     (102401, 2, PATH_AUTO, 0), (200000, 3, PATH_AUTO, 0), (262147, 2, PATH_STRIP, 0), (524288, 9, PATH_STRIP, 0), (524289, 1, PATH_AUTO, 0),
-    (600000, 9, PATH_STRIP, 0), (655361, 1, PATH_AUTO, 0), (1000003, 1, PATH_AUTO, 0),
+    (600000, 9, PATH_STRIP, 0), (655361, 1, PATH_AUTO, 0), (1000003, 1, PATH_AUTO, 0), (1500001, 2, PATH_STRIP, 0),
 ]
 
 
