@@ -79,3 +79,16 @@ def test_scalar_registers_cost_the_stripe_kernels_no_wavefront(sources):
                 "%s: %s scalar registers allow %d wavefronts per SIMD, its vector registers %s" % (
                     n, k["SGPRs"], wavefronts_by_scalar_registers(int(k["SGPRs"])), k["Occupancy"])
     assert seen >= 8
+
+
+def test_kernels_that_address_lds_by_number_declare_none_of_their_own():
+    """The multi-bit column stripe reduction reads its decoding tables and writes its column at LDS addresses counted from 0
+    (`lds_read` / `lds_write`), which is where a kernel's LDS from the launch starts only if the kernel declares none
+    itself: the compiler's figure for declared LDS must be 0 for every kernel that contains that body."""
+    seen = 0
+    for k in all_kernels(FLOAT_SOURCES):
+        n = k["name"]
+        if "stripe_reduce_colg_kernel" in n or "stripe_reduce_batch" in n:
+            seen += 1
+            assert int(k["LDS"]) == 0, "%s declares %s bytes of LDS of its own" % (n, k["LDS"])
+    assert seen >= 10
