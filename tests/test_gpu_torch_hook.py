@@ -101,6 +101,7 @@ def test_in_process_workers_against_the_oracle(K, nbits, zt):
             for w in range(K):
                 parity.check_quantize(gs[w][i], res_in[w][i], q1[w][i], res_out[w][i], nbits, zt, threads=8, report=rep, strict=rows <= 16384)
                 tainted |= rep.last_mismatch_cols
+            aggs_g = [None] * K
             for s in range(K):
                 start, n = oracle.stripe_range(cols, s, K)
                 if n == 0:
@@ -108,12 +109,13 @@ def test_in_process_workers_against_the_oracle(K, nbits, zt):
                 q_copy = [q[i].copy() for q in q1]
                 s_copy = sres_in[s][i].copy(order="F")
                 agg = oracle.stripe_reduce(q_copy, s, rows, cols, nbits, s_copy, zt, threads=8)
+                aggs_g[s] = agg
                 parity.check_quantize(agg, sres_in[s][i], qagg_g[start * qcol:(start + n) * qcol], sres_out[s], nbits, zt,
                                       threads=8, report=rep, strict=rows <= 16384)
                 tainted[start:start + n] |= rep.last_mismatch_cols
             parity.check_unquantize(qagg_g, rows, cols, nbits, outs[0], threads=8)
             parity.check_end_to_end(aggs_o, [sres_in[s][i] for s in range(K)], qagg_g, sres_out, outs[0], qagg_o, out_o, rows, cols,
-                                    nbits, zt, tainted, threads=8, report=rep)
+                                    nbits, zt, tainted, threads=8, report=rep, aggs_gpu=aggs_g)
             if rows <= 16384:  # (a column of 100000 elements is likelier than not to hold one element at a threshold)
                 assert tainted.sum() <= max(1, cols // 50)
     say("torch hook K=%d nbits=%d:" % (K, nbits), rep)

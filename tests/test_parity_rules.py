@@ -88,3 +88,37 @@ def test_no_fallback_on_ordinary_data():
     q, r_out = oracle.quantize(g, r, 1, False, threads=4)
     rep = parity.check_quantize(g, r, q, r_out, 1, False, threads=4, strict=True)
     assert rep.fallback_cols == 0 and rep.fallback_elements == 0 and rep.cols == 24
+
+
+def test_inputs_that_all_moved_one_way_explain_as_much_on_the_bounds():
+    """A second-stage quantization whose inputs (the aggregates) are themselves equal only within a tolerance: a shift
+    of every input moves the bounds by as much, and is allowed only when the caller states it."""
+    g = datagen.normal(13, 2048, 8)
+    r = datagen.normal(14, 2048, 8, 0.002)
+    shift = np.float32(4e-7)  # about 2e-5 of the column scale of 0.02
+    q, r_out = oracle.quantize(np.asfortranarray(g + shift), r, 1, False, threads=4)
+    with pytest.raises(AssertionError, match="column bounds off"):
+        parity.check_quantize(g, r, q, r_out, 1, False, threads=4, exact=False)
+    parity.check_quantize(g, r, q, r_out, 1, False, threads=4, exact=False, input_dev=np.full(8, float(shift)))
+
+
+def test_an_element_on_the_other_side_of_zero_leaves_its_column_out_of_the_whole_run():
+    """With the zero threshold the bounds are the means of the two sides: one element at -2e-8 here and 0.0 there moves
+    both by mean / count (1e-4 of the scale at 2000 rows). The whole-run comparison leaves such a column out, and counts
+    it, when it is given the aggregates of both sides; without them it must refuse."""
+    rows, cols = 2000, 6
+    a = datagen.normal(15, rows, cols)
+    a[7, 2] = np.float32(-2e-8)
+    b = a.copy(order="F")
+    b[7, 2] = np.float32(0.0)
+    z = np.zeros_like(a, order="F")
+    q_or, _ = oracle.quantize(a, z, 1, True, threads=4)
+    q_gpu, s_gpu = oracle.quantize(b, z, 1, True, threads=4)
+    out_or = oracle.unquantize(q_or, rows, cols, 1, threads=4)
+    out_gpu = oracle.unquantize(q_gpu, rows, cols, 1, threads=4)
+    none = np.zeros(cols, dtype=bool)
+    with pytest.raises(AssertionError, match="column bounds off"):
+        parity.check_end_to_end([a], [z], q_gpu, [s_gpu], out_gpu, q_or, out_or, rows, cols, 1, True, none, threads=4)
+    _, left_out = parity.check_end_to_end([a], [z], q_gpu, [s_gpu], out_gpu, q_or, out_or, rows, cols, 1, True, none, threads=4,
+                                          aggs_gpu=[b])
+    assert left_out == 1 and not none.any()
