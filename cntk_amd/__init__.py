@@ -104,10 +104,14 @@ def lib():
         for name in ("cntkq_stripe_reduce_max_rows", "cntkq_stripe_reduce_max_rows_f64"):
             getattr(L, name).argtypes = [_sz]
             getattr(L, name).restype = _sz
+        for name in ("cntkq_stripe_reduce_takes", "cntkq_stripe_reduce_takes_f64"):
+            getattr(L, name).argtypes = [_vp, _sz, _sz, _sz, ctypes.c_int]
         L.cntkq_debug_set_tuning.argtypes = [_vp, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int]
         L.cntkq_debug_set_strip_spin_limit.argtypes = [_vp, ctypes.c_uint]
         L.cntkq_debug_strip_max_strips.argtypes = [_vp, _sz, ctypes.c_int]
         L.cntkq_debug_strip_max_strips.restype = ctypes.c_uint
+        L.cntkq_debug_strip_max_strips_f64.argtypes = [_vp, _sz, ctypes.c_int]
+        L.cntkq_debug_strip_max_strips_f64.restype = ctypes.c_uint
         L.cntkq_set_force_sync.argtypes = [_vp, ctypes.c_int]
         _lib = L
     return _lib
@@ -494,6 +498,11 @@ class MatrixQuantizerImpl:
                                                out_qstripe.Buffer(), agg_out.Data() if agg_out is not None else None,
                                                int(bool(zero_threshold_for_1bit))))
 
+    def StripeReduceTakes(self, rows, cols, nbits, zero_threshold_for_1bit=False, dtype=torch.float32):
+        """Whether StripeReduceAsync takes stripes of this shape; where not, the caller runs the reference's sequence of
+        UnquantizeAsync ... QuantizeAsync calls (Source/1BitSGD/AllReduceDistGradAggregator.h:365-436)."""
+        return bool(_fn("cntkq_stripe_reduce_takes", dtype)(self._h, rows, cols, nbits, int(bool(zero_threshold_for_1bit))))
+
     def StripeReduceBatchAsync(self, items, owner, zero_threshold_for_1bit):
         """The owner's stripe reductions of a whole gradient set as one call. items: sequence of
         (stripes, stripe_residual, out_qstripe, agg_out or None), one per gradient matrix, one element type."""
@@ -549,9 +558,10 @@ class MatrixQuantizerImpl:
     def _set_strip_spin_limit(self, limit):
         _check(lib().cntkq_debug_set_strip_spin_limit(self._h, limit))
 
-    def _strip_max_strips(self, nbits, zero_threshold_for_1bit=False):
+    def _strip_max_strips(self, nbits, zero_threshold_for_1bit=False, dtype=torch.float32):
         """Most strips per column that the strip kernels take on this device at this bit width (0: none)."""
-        return int(lib().cntkq_debug_strip_max_strips(self._h, nbits, 1 if zero_threshold_for_1bit else 0))
+        f = lib().cntkq_debug_strip_max_strips_f64 if dtype == torch.float64 else lib().cntkq_debug_strip_max_strips
+        return int(f(self._h, nbits, 1 if zero_threshold_for_1bit else 0))
 
 
 class MatrixQuantizer:

@@ -13,6 +13,10 @@ struct Elem<float>
     static constexpr size_t kAlign = 4;
     static constexpr size_t kWordBits = 32;
     static size_t stripe_max_rows(size_t nbits) { return cntkq::stripe_reduce_max_rows(nbits); }
+    static bool stripe_takes_strips(hipStream_t s, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+    {
+        return cntkq::stripe_takes_strips(s, rows, cols, nbits, zt, tune);
+    }
     static bool valid_nbits(size_t nbits) { return cntkq::valid_nbits(nbits); }
     static size_t qcol_bytes(size_t nbits, size_t rows) { return cntkq::qcol_bytes(nbits, rows); }
     static hipError_t quantize(hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, void* q, size_t rows,
@@ -140,7 +144,12 @@ struct BatchAbi<float>
     }
 
     static size_t stripe_max_rows(size_t nbits) { return stripe_reduce_max_rows(nbits); }
-    // taller stripes run 1024 threads per column: a launch of their own
+    static bool stripe_takes_strips(cntkq_quantizer* h, size_t rows, size_t cols, size_t nbits, bool zt)
+    {
+        DeviceGuard guard(h->device);
+        return cntkq::stripe_takes_strips(work_stream(h), rows, cols, nbits, zt, h->tune);
+    }
+    // taller stripes run 1024 threads per column, or on strips: a launch of their own
     // (so do stripes that the table-driven register kernel takes with more than six pieces per thread: the shared launch is
     // compiled for what its largest member needs)
     static bool stripe_is_member(const SItem& it, size_t workers, size_t nbits)
@@ -610,7 +619,7 @@ int cntkq_create(int device_id, int use_dedicated_stream, cntkq_quantizer** out)
         // allocate) finds it. A failure here is not one of the handle: the first call that needs the buffer tries again.
         // (cleared on one of the handle's own streams and waited for there: the legacy default stream stays out of it)
         StripScratch unused;
-        if (strip_scratch_for(h->strip_scratch, h->fetch, 1, 2, unused) != hipSuccess ||
+        if (strip_scratch_for(h->strip_scratch, h->fetch, 1, 2, strip_records<double>(), unused) != hipSuccess ||
             hipEventCreateWithFlags(&h->strip_scratch.order_event, hipEventDisableTiming) != hipSuccess)
             (void) hipGetLastError();
     }
@@ -789,7 +798,19 @@ int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h)
     if (h == nullptr)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_wait_stripe_reduce_done: null handle");
     DeviceGuard guard(h->device);
-    return h->last_stripe != nullptr ? sync_event(h->last_stripe) : CNTKQ_OK;
+    const int rc = h->last_stripe != nullptr ? sync_event(h->last_stripe) : CNTKQ_OK;
+    // (a reduction on strips reports workgroups that gave up on each other like a quantize call on strips)
+    return rc != CNTKQ_OK ? rc : check_strip_error(h);
+}
+
+int cntkq_stripe_reduce_takes(cntkq_quantizer* h, size_t rows, size_t stripe_cols, size_t nbits, int zero_threshold_for_1bit)
+{
+    if (h == nullptr || !valid_nbits(nbits) || rows == 0 || stripe_cols == 0 || rows >= (1ull << 31) || stripe_cols >= (1ull << 31))
+        return 0;
+    if (rows <= Elem<float>::stripe_max_rows(nbits))
+        return 1;
+    DeviceGuard guard(h->device);
+    return cntkq::stripe_takes_strips(work_stream(h), rows, stripe_cols, nbits, zero_threshold_for_1bit != 0, h->tune) ? 1 : 0;
 }
 
 
@@ -829,7 +850,15 @@ unsigned cntkq_debug_strip_max_strips(cntkq_quantizer* h, size_t nbits, int zero
     if (h == nullptr || !valid_nbits(nbits) || nbits >= 32)
         return 0;
     DeviceGuard guard(h->device);
-    return strip_max_strips(nbits, zero_threshold_for_1bit != 0 && nbits == 1);
+    return strip_max_strips<float>(nbits, zero_threshold_for_1bit != 0 && nbits == 1);
+}
+
+unsigned cntkq_debug_strip_max_strips_f64(cntkq_quantizer* h, size_t nbits, int zero_threshold_for_1bit)
+{
+    if (h == nullptr || nbits == 0 || nbits >= 64 || (nbits & (nbits - 1)) != 0)
+        return 0;
+    DeviceGuard guard(h->device);
+    return strip_max_strips<double>(nbits, zero_threshold_for_1bit != 0 && nbits == 1);
 }
 
 int cntkq_debug_attach_events(cntkq_quantizer* h, void* start_event, void* stop_event)

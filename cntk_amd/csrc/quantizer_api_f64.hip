@@ -14,6 +14,10 @@ struct Elem<double>
     static constexpr size_t kAlign = 8;
     static constexpr size_t kWordBits = 64;
     static size_t stripe_max_rows(size_t nbits) { return cntkq::f64::stripe_reduce_max_rows(nbits); }
+    static bool stripe_takes_strips(hipStream_t s, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+    {
+        return cntkq::f64::stripe_takes_strips(s, rows, cols, nbits, zt, tune);
+    }
     static bool valid_nbits(size_t nbits) { return cntkq::f64::valid_nbits(nbits); }
     static size_t qcol_bytes(size_t nbits, size_t rows) { return cntkq::f64::qcol_bytes(nbits, rows); }
     static hipError_t quantize(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, void* q, size_t rows,
@@ -70,9 +74,10 @@ struct BatchAbi<double>
     {
         return f64::dispatch_nbits64<f64::QuantizeBatchLauncher64>(nbits, zt && nbits == 1, s, ev, de, db, members, blocks, lds);
     }
-    static hipError_t launch_quantize_own(cntkq_quantizer*, hipStream_t s, LaunchEvents ev, const QItem& it, size_t nbits, bool zt)
+    static hipError_t launch_quantize_own(cntkq_quantizer* h, hipStream_t s, LaunchEvents ev, const QItem& it, size_t nbits, bool zt)
     {
         LaunchTuning autotune;
+        autotune.strip = &h->strip_scratch;
         return f64::launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune);
     }
 
@@ -101,8 +106,16 @@ struct BatchAbi<double>
     }
 
     static size_t stripe_max_rows(size_t nbits) { return f64::stripe_reduce_max_rows(nbits); }
-    // stripes of the register kernel's heights run 1024 threads per column: a launch of their own
-    static bool stripe_is_member(const SItem& it, size_t, size_t nbits) { return !f64::stripe_uses_reg(it.rows, nbits); }
+    static bool stripe_takes_strips(cntkq_quantizer* h, size_t rows, size_t cols, size_t nbits, bool zt)
+    {
+        DeviceGuard guard(h->device);
+        return f64::stripe_takes_strips(work_stream(h), rows, cols, nbits, zt, h->tune);
+    }
+    // stripes of the register kernel's heights run 1024 threads per column, taller ones on strips: a launch of their own
+    static bool stripe_is_member(const SItem& it, size_t, size_t nbits)
+    {
+        return it.rows <= f64::stripe_reduce_max_rows(nbits) && !f64::stripe_uses_reg(it.rows, nbits);
+    }
     static int stripe_one(cntkq_quantizer* h, const SItem& it, size_t workers, size_t owner, size_t nbits, int zt)
     {
         return cntkq_stripe_reduce_async_f64(h, it.stripes, workers, owner, it.rows, it.stripe_cols, nbits, it.stripe_res, it.q_out, it.agg_out,
@@ -146,6 +159,16 @@ size_t cntkq_qmatrix_bytes_f64(size_t rows, size_t cols, size_t nbits)
 size_t cntkq_stripe_reduce_max_rows_f64(size_t nbits)
 {
     return cntkq::f64::valid_nbits(nbits) ? Elem<double>::stripe_max_rows(nbits) : 0;
+}
+
+int cntkq_stripe_reduce_takes_f64(cntkq_quantizer* h, size_t rows, size_t stripe_cols, size_t nbits, int zero_threshold_for_1bit)
+{
+    if (h == nullptr || !cntkq::f64::valid_nbits(nbits) || rows == 0 || stripe_cols == 0 || rows >= (1ull << 31) || stripe_cols >= (1ull << 31))
+        return 0;
+    if (rows <= Elem<double>::stripe_max_rows(nbits))
+        return 1;
+    DeviceGuard guard(h->device);
+    return cntkq::f64::stripe_takes_strips(work_stream(h), rows, stripe_cols, nbits, zero_threshold_for_1bit != 0, h->tune) ? 1 : 0;
 }
 
 int cntkq_quantize_async_f64(cntkq_quantizer* h, const double* in, const double* res_in, size_t rows, size_t cols, void* qbuf,

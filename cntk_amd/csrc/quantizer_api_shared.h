@@ -564,8 +564,15 @@ int stripe_reduce_async_impl(cntkq_quantizer* h, const void* const* stripes, siz
     if (rows == 0 || stripe_cols == 0)
         return CNTKQ_OK;
     if (rows > Elem<E>::stripe_max_rows(nbits))
-        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: columns taller than %zu rows are not supported at %zu bits",
-                    Elem<E>::stripe_max_rows(nbits), nbits);
+    {
+        // taller stripes run on strips where the device holds a column's strips at once (cntkq_stripe_reduce_takes)
+        DeviceGuard guard(h->device);
+        if (!Elem<E>::stripe_takes_strips(work_stream(h), rows, stripe_cols, nbits, zero_threshold_for_1bit != 0, h->tune))
+            return fail(CNTKQ_INVALID_ARGUMENT,
+                        "cntkq_stripe_reduce_async: columns of %zu rows are not supported at %zu bits (up to %zu rows, and on strips the "
+                        "heights that cntkq_stripe_reduce_takes reports)",
+                        rows, nbits, Elem<E>::stripe_max_rows(nbits));
+    }
     if (stripe_res == nullptr || q_out == nullptr || !aligned_for<E>(stripe_res) || !aligned_for<E>(q_out) || !aligned_for<E>(agg_out))
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_stripe_reduce_async: null or misaligned matrix pointer");
     StripeSources src;

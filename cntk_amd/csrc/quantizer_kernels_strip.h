@@ -2,9 +2,10 @@
 //
 // A column of `rows` elements is packed into nq QWords, element i in QWord i % nq at bit position i / nq. A strip is a run
 // of W consecutive QWords with ALL their bit positions: 32 / NBITS runs of W consecutive elements, nq elements apart. One
-// 256-thread workgroup owns one strip: a thread holds four consecutive QWords' elements at up to eight bit positions (32
-// values: eight 16-byte loads of gradient and residual, at any 4-byte alignment), builds its part of the four QWords and
-// writes the residual back from registers; the parts of a QWord meet in LDS. Gradient and residual are read once whatever
+// 256-thread workgroup owns one strip: a thread holds the elements of 16 bytes' worth of consecutive QWords (four of a
+// float column, two of a double column) at up to eight bit positions (eight 16-byte loads of gradient and residual, at
+// any alignment the element type allows), builds its part of those QWords and writes the residual back from registers;
+// the parts of a QWord meet in LDS. The kernels are written once over the element type. Gradient and residual are read once whatever
 // the height, which columns above 102400 rows -- more than any workgroup's registers hold -- could otherwise only have by
 // reading their inputs two or three times. A strip needs 1 to 4 KB of LDS and, at 1 to 4 bits, some 100 registers (its 32
 // values, their addresses, the masks of the ragged last strip), so five workgroups share a CU; it is the exchange
@@ -12,8 +13,8 @@
 // per column are faster.
 //
 // The column statistics span the strips of a column. Every workgroup publishes its partial sums in a scratch buffer, one
-// 8-byte record per sum: the value and the tag of the launch, written by one atomic store, so that whoever reads the tag
-// of this launch has the value with it and no second word needs ordering against the first. Then the first wavefront of
+// 8-byte record per 32 bits of a sum (a double takes two): the bits and the tag of the launch, written by one atomic store,
+// so that whoever reads the tag of this launch has the bits with it and no second word needs ordering against the first. Then the first wavefront of
 // every workgroup of the column polls the S records (a lane per record, with pauses) until all carry the tag, and adds them up, lanes
 // meeting by butterfly -- one fixed order, the same bytes in every workgroup. One exchange for the sum of squares (more than 1 bit) or
 // the split sums (1 bit against 0), two for 1 bit against the mean (mean, then split sums). The tag is a launch count
@@ -32,30 +33,67 @@
 // column in the scratch header.
 #pragma once
 
-#include "quantizer_kernels_common.h"
+#include <type_traits>
+
+#include "quantizer_kernels_tile.h" // StripeSources, stripe_order
 
 namespace cntkq {
 
 constexpr uint32_t kStripThreads = 256;
 constexpr uint32_t kStripDies = 8; // accelerator dies that take the workgroups of a grid in turn
 
-template <int NBITS>
-struct StripShape
+typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+typedef u64x2 u64x2_u __attribute__((aligned(8)));
+
+// The 16-byte accesses of either element type: PER consecutive elements, or QWords, at the alignment of one.
+template <typename E>
+struct StripElem;
+template <>
+struct StripElem<float>
 {
-    using PS = PackShape<NBITS>;
-    static constexpr uint32_t SLOTS = PS::SLOTS;                  // bit positions per thread
-    static constexpr uint32_t CHUNKS = PS::CHUNKS;                // threads per QWord quad
-    static constexpr uint32_t QUADS = kStripThreads / CHUNKS;     // quads of four QWords per strip
-    static constexpr uint32_t WORDS = 4 * QUADS;                  // QWords per strip: 256, 512, 1024, 1024, 1024 at 1, 2, 4, 8, 16 bits
-    // wavefronts per SIMD the kernels are compiled for (the registers that leaves them: 96 at 5, 64 at 8); with more at 1 to 4
-    // bits the ragged last strip spills, and every strip of its column waits for it
-    static constexpr uint32_t WAVES = NBITS <= 4 ? 5 : 8;
+    typedef f32x4 V;
+    typedef f32x4_u VU;
+    typedef u32x4 QV;
+    typedef u32x4_u QVU;
+    static constexpr uint32_t PER = 4;
+    static __device__ __forceinline__ QV words(const uint32_t* w) { return QV{w[0], w[1], w[2], w[3]}; }
+};
+template <>
+struct StripElem<double>
+{
+    typedef f64x2 V;
+    typedef f64x2_u VU;
+    typedef u64x2 QV;
+    typedef u64x2_u QVU;
+    static constexpr uint32_t PER = 2;
+    static __device__ __forceinline__ QV words(const uint64_t* w) { return QV{w[0], w[1]}; }
 };
 
-// how many QWords a strip holds at this bit width (host side)
+template <typename E>
+using StripVec = typename StripElem<E>::V;
+
+template <int NBITS, typename E>
+struct StripShape
+{
+    using PS = PackShapeOf<NBITS, Word<E>::kBits>;
+    static constexpr uint32_t PER = StripElem<E>::PER;            // consecutive QWords per thread
+    static constexpr uint32_t SLOTS = PS::SLOTS;                  // bit positions per thread
+    static constexpr uint32_t CHUNKS = PS::CHUNKS;                // threads per run of PER QWords
+    static constexpr uint32_t RUNS = kStripThreads / CHUNKS;      // runs of PER QWords per strip
+    // QWords per strip: float 256, 512, 1024, 1024, 1024 at 1, 2, 4, 8, 16 bits; double 64, 128, 256, 512, 512, 512 at 1 ... 32 bits
+    static constexpr uint32_t WORDS = PER * RUNS;
+    // wavefronts per SIMD the kernels are compiled for (the registers that leaves them: 96 at 5, 64 at 8); with more where a
+    // thread holds eight bit positions the ragged last strip spills, and every strip of its column waits for it
+    static constexpr uint32_t WAVES = SLOTS == 8 ? 5 : 8;
+};
+
+// how many QWords a strip holds at this bit width (host side; the same arithmetic as StripShape)
+template <typename E>
 __host__ __device__ inline uint32_t strip_words(size_t nbits)
 {
-    return nbits == 1 ? StripShape<1>::WORDS : nbits == 2 ? StripShape<2>::WORDS : StripShape<4>::WORDS;
+    const uint32_t vpw = (uint32_t) (Word<E>::kBits / nbits);
+    const uint32_t slots = vpw < 8 ? vpw : 8;
+    return (uint32_t) (16 / sizeof(E)) * (kStripThreads / (vpw / slots));
 }
 
 struct StripGeom
@@ -73,8 +111,9 @@ struct StripGeom
     uint64_t qcol;
 };
 
-// Scratch of one launch stream: a header, the finish counters, then four records per (column, strip): the statistic, then
-// the two split sums and the count below the threshold. The buffer starts zeroed; tags start at 1.
+// Scratch of one launch stream: a header, the finish counters, then the records of every (column, strip): the statistic,
+// then the two split sums (each one record for floats, two for doubles) and the count below the threshold. The buffer
+// starts zeroed; tags start at 1.
 //
 // Reads of one address take their turns like atomic operations on it (a few nanoseconds each, but thousands of workgroups
 // start within microseconds), so the launch count is kept in 256 copies, 256 bytes apart, and a wavefront reads the copy
@@ -93,14 +132,19 @@ struct StripHeader
     uint32_t pad2[63];
 };
 constexpr uint32_t kStripAbandoned = 0x80000000u; // top bit of a record's tag: the strip's workgroup gave up; tags proper have 31 bits
-constexpr uint32_t kStripRecords = 4;
+// records per (column, strip): three sums of the element type and a count (doubles: one record stays unused)
+template <typename E>
+constexpr uint32_t strip_records()
+{
+    return 4u * (uint32_t) (sizeof(E) / 4);
+}
 constexpr uint32_t kStripFinishGroup = 64;
 struct StripScratch
 {
     uint32_t* error;      // pinned host memory
     StripHeader* header;
     uint32_t* groups;     // workgroups done per group of kStripFinishGroup; zero between launches
-    uint64_t* records;    // [column][field][strip]: value in the low half, tag in the high half
+    uint64_t* records;    // [column][record][strip]: 32 bits of a value in the low half, tag in the high half
 };
 
 // Bytes of finish counters and of records that a launch of this geometry uses. The two live in regions of the buffer
@@ -110,9 +154,9 @@ inline size_t strip_groups_bytes(size_t cols, size_t strips)
     const size_t grid = (cols + kStripDies - 1) / kStripDies * kStripDies * strips;
     return (grid + kStripFinishGroup - 1) / kStripFinishGroup * sizeof(uint32_t);
 }
-inline size_t strip_records_bytes(size_t cols, size_t strips)
+inline size_t strip_records_bytes(size_t cols, size_t strips, size_t records_each)
 {
-    return cols * strips * kStripRecords * sizeof(uint64_t);
+    return cols * strips * records_each * sizeof(uint64_t);
 }
 
 __device__ __forceinline__ void strip_publish(uint64_t* rec, uint32_t value_bits, uint32_t tag)
@@ -120,8 +164,43 @@ __device__ __forceinline__ void strip_publish(uint64_t* rec, uint32_t value_bits
     __hip_atomic_store(rec, ((uint64_t) tag << 32) | value_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// One wavefront collects the S records of a field: lane l polls records l, l + 64, ... until they carry the tag, adds
-// their values in ascending order, and the lanes meet by butterfly. Every lane returns the same bits.
+// a value of 4 or 8 bytes: records `rec`, and `rec + strips` for the upper half
+template <typename T>
+__device__ __forceinline__ void strip_publish_value(uint64_t* rec, uint32_t strips, T value, uint32_t tag)
+{
+    uint32_t w[sizeof(T) / 4];
+    __builtin_memcpy(w, &value, sizeof(T));
+#pragma unroll
+    for (uint32_t h = 0; h < sizeof(T) / 4; ++h)
+        strip_publish(rec + h * strips, w[h], tag);
+}
+
+// Waits for one record to carry the tag and returns its 32 bits. `bad`: its workgroup abandoned it, or it was not there
+// after the bounded wait.
+__device__ __forceinline__ uint32_t strip_poll(const uint64_t* rec, uint32_t tag, const StripGeom& c, bool& bad)
+{
+    uint32_t polls = 0;
+    uint64_t x;
+    for (;;)
+    {
+        x = __hip_atomic_load(rec, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t got = (uint32_t) (x >> 32);
+        if (got == tag)
+            break;
+        if (got == (tag | kStripAbandoned) || polls >= c.spin_limit)
+        {
+            bad = true;
+            break;
+        }
+        ++polls;
+        for (uint32_t z = 0; z < c.poll_pause; ++z)
+            __builtin_amdgcn_s_sleep(1);
+    }
+    return (uint32_t) x;
+}
+
+// One wavefront collects the S values of a sum: lane l polls the records of strips l, l + 64, ... until they carry the tag,
+// adds their values in ascending order, and the lanes meet by butterfly. Every lane returns the same bits.
 // Polls are loads at device scope, and a thousand resident workgroups polling as fast as they can took half of the L2's
 // request rate from the loads and stores that the records wait for: a lane pauses poll_pause x 64 cycles between two polls
 // (200000 x 256 at 1 bit over 1 / 16 / 64 / 128 / 256: 214 / 208 / 200 / 198 / 208 us), and first_pause x 64 cycles
@@ -134,29 +213,14 @@ __device__ __forceinline__ T strip_collect(const uint64_t* recs, uint32_t strips
     bool bad = false;
     for (uint32_t s = threadIdx.x & 63u; s < strips; s += 64)
     {
-        uint32_t polls = 0;
         for (uint32_t z = 0; z < first_pause; ++z)
             __builtin_amdgcn_s_sleep(1);
-        uint64_t x;
-        for (;;)
-        {
-            x = __hip_atomic_load(recs + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const uint32_t got = (uint32_t) (x >> 32);
-            if (got == tag)
-                break;
-            // abandoned by its workgroup, or not there after the bounded wait
-            if (got == (tag | kStripAbandoned) || polls >= c.spin_limit)
-            {
-                bad = true;
-                break;
-            }
-            ++polls;
-            for (uint32_t z = 0; z < c.poll_pause; ++z)
-                __builtin_amdgcn_s_sleep(1);
-        }
+        uint32_t w[sizeof(T) / 4];
+#pragma unroll
+        for (uint32_t h = 0; h < sizeof(T) / 4; ++h)
+            w[h] = bad ? 0u : strip_poll(recs + h * strips + s, tag, c, bad);
         T val;
-        const uint32_t lo = (uint32_t) x;
-        __builtin_memcpy(&val, &lo, 4);
+        __builtin_memcpy(&val, w, sizeof(T));
         t += val;
     }
     gave_up = gave_up || __ballot(bad) != 0ull; // the same in every lane of the wavefront
@@ -165,9 +229,10 @@ __device__ __forceinline__ T strip_collect(const uint64_t* recs, uint32_t strips
 
 // The workgroup abandons its strip: every record of it says so (whichever exchange a neighbour is in, it meets the mark),
 // the host learns of it through the error word, and strip 0 counts the column.
-__device__ __forceinline__ void strip_abandon(uint64_t* recs, uint32_t strip, uint32_t tag, const StripGeom& c, const StripScratch& scratch)
+__device__ __forceinline__ void strip_abandon(uint64_t* recs, uint32_t records_each, uint32_t strip, uint32_t tag, const StripGeom& c,
+                                              const StripScratch& scratch)
 {
-    for (uint32_t f = 0; f < kStripRecords; ++f)
+    for (uint32_t f = 0; f < records_each; ++f)
         strip_publish(recs + f * c.strips + strip, 0u, tag | kStripAbandoned);
     __hip_atomic_store(scratch.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     if (strip == 0)
@@ -193,116 +258,111 @@ __device__ __forceinline__ void strip_finish(const StripScratch& sc, uint32_t ta
 
 // Sum of a value over the workgroup in a fixed order (lanes by butterfly, then the four wavefronts in ascending order),
 // the same bits in every thread. red: 4 slots; two barriers.
-__device__ __forceinline__ float strip_block_sum(float v, float* red)
+template <typename T>
+__device__ __forceinline__ T strip_block_sum(T v, T* red)
 {
     v = wave_sum(v);
     if ((threadIdx.x & 63u) == 0)
         red[threadIdx.x >> 6] = v;
     __syncthreads();
-    const float t = ((red[0] + red[1]) + red[2]) + red[3];
-    __syncthreads();
-    return t;
-}
-
-__device__ __forceinline__ uint32_t strip_block_sum(uint32_t v, uint32_t* red)
-{
-    v = wave_sum(v);
-    if ((threadIdx.x & 63u) == 0)
-        red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    const uint32_t t = red[0] + red[1] + red[2] + red[3];
+    const T t = ((red[0] + red[1]) + red[2]) + red[3];
     __syncthreads();
     return t;
 }
 
 // The column's statistic from the strip's: every workgroup of the column publishes its own and adds all of them in the
-// order of strip_collect. red: the workgroup's reduction slots. Every thread returns the same bits, in every workgroup of the column.
-__device__ __forceinline__ float strip_exchange_stat(float stat, uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
-                                                     const StripScratch& scratch, float* red, bool& ok)
+// order of strip_collect. red, red_u: the workgroup's reduction slots (four each). Every thread returns the same bits, in
+// every workgroup of the column.
+template <typename E>
+__device__ __forceinline__ E strip_exchange_stat(E stat, uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
+                                                 const StripScratch& scratch, E* red, uint32_t* red_u, bool& ok)
 {
     if (c.strips == 1)
         return stat;
-    uint64_t* recs = scratch.records + (size_t) column * kStripRecords * c.strips; // [field][strip]
+    constexpr uint32_t H = sizeof(E) / 4; // records per sum
+    uint64_t* recs = scratch.records + (size_t) column * strip_records<E>() * c.strips; // [record][strip]
     if (threadIdx.x == 0)
-        strip_publish(recs + strip, __float_as_uint(stat), tag);
+        strip_publish_value(recs + strip, c.strips, stat, tag);
     if (threadIdx.x < 64)
     {
         bool gave_up = false;
-        const float t = strip_collect<float>(recs, c.strips, tag, c, c.poll_first, gave_up);
+        const E t = strip_collect<E>(recs, c.strips, tag, c, c.poll_first, gave_up);
         if (threadIdx.x == 0)
         {
             red[0] = t;
-            red[3] = gave_up ? 1.0f : 0.0f;
+            red_u[3] = gave_up ? 1u : 0u;
             if (gave_up)
-                strip_abandon(recs, strip, tag, c, scratch);
+                strip_abandon(recs, H * 4, strip, tag, c, scratch);
         }
     }
     __syncthreads();
-    const float total = red[0];
-    ok = red[3] == 0.0f;
+    const E total = red[0];
+    ok = red_u[3] == 0u;
     __syncthreads();
     return total;
 }
 
 // the same for the sums on either side of the 1-bit threshold and the count below it
-__device__ __forceinline__ void strip_exchange_split(float& s0, float& s1, uint32_t& n0, uint32_t column, uint32_t strip, uint32_t tag,
-                                                     const StripGeom& c, const StripScratch& scratch, float* red, bool& ok)
+template <typename E>
+__device__ __forceinline__ void strip_exchange_split(E& s0, E& s1, uint32_t& n0, uint32_t column, uint32_t strip, uint32_t tag,
+                                                     const StripGeom& c, const StripScratch& scratch, E* red, uint32_t* red_u, bool& ok)
 {
     if (c.strips == 1)
         return;
-    uint64_t* recs = scratch.records + (size_t) column * kStripRecords * c.strips;
+    constexpr uint32_t H = sizeof(E) / 4;
+    uint64_t* recs = scratch.records + (size_t) column * strip_records<E>() * c.strips;
     if (threadIdx.x == 0)
     {
-        strip_publish(recs + 1 * c.strips + strip, __float_as_uint(s0), tag);
-        strip_publish(recs + 2 * c.strips + strip, __float_as_uint(s1), tag);
-        strip_publish(recs + 3 * c.strips + strip, n0, tag);
+        strip_publish_value(recs + 1 * H * c.strips + strip, c.strips, s0, tag);
+        strip_publish_value(recs + 2 * H * c.strips + strip, c.strips, s1, tag);
+        strip_publish_value(recs + 3 * H * c.strips + strip, c.strips, n0, tag);
     }
     if (threadIdx.x < 64)
     {
         bool gave_up = false;
-        const float t0 = strip_collect<float>(recs + 1 * c.strips, c.strips, tag, c, c.poll_first, gave_up);
-        const float t1 = strip_collect<float>(recs + 2 * c.strips, c.strips, tag, c, 0u, gave_up);
-        const uint32_t tn = strip_collect<uint32_t>(recs + 3 * c.strips, c.strips, tag, c, 0u, gave_up);
+        const E t0 = strip_collect<E>(recs + 1 * H * c.strips, c.strips, tag, c, c.poll_first, gave_up);
+        const E t1 = strip_collect<E>(recs + 2 * H * c.strips, c.strips, tag, c, 0u, gave_up);
+        const uint32_t tn = strip_collect<uint32_t>(recs + 3 * H * c.strips, c.strips, tag, c, 0u, gave_up);
         if (threadIdx.x == 0)
         {
             red[0] = t0;
             red[1] = t1;
-            red[2] = __uint_as_float(tn);
-            red[3] = gave_up ? 1.0f : 0.0f;
+            red_u[2] = tn;
+            red_u[3] = gave_up ? 1u : 0u;
             if (gave_up)
-                strip_abandon(recs, strip, tag, c, scratch);
+                strip_abandon(recs, H * 4, strip, tag, c, scratch);
         }
     }
     __syncthreads();
     s0 = red[0];
     s1 = red[1];
-    n0 = __float_as_uint(red[2]);
-    ok = red[3] == 0.0f;
+    n0 = red_u[2];
+    ok = red_u[3] == 0u;
     __syncthreads();
 }
 
 // From the strip's sums to the column's header: the exchanges, the header (written by strip 0) and the release of the
 // scratch buffer. `sums(mean, s0, s1, n0)` gives the strip's split sums (1 bit only), in the same bits in every thread.
 // False (in every thread of the workgroup alike): the column was abandoned and nothing of it may be stored.
-template <int NBITS, bool ZT, typename SplitSums>
-__device__ __forceinline__ bool strip_column_range(float stat, SplitSums sums, uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
-                                                   const StripScratch& scratch, float* red, char* qc, float& lo, float& hi)
+template <int NBITS, bool ZT, typename E, typename SplitSums>
+__device__ __forceinline__ bool strip_column_range(E stat, SplitSums sums, uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
+                                                   const StripScratch& scratch, E* red, uint32_t* red_u, char* qc, E& lo, E& hi)
 {
     constexpr bool need_stat = (NBITS != 1) || !ZT;
-    float total = 0.0f;
+    E total = 0;
     bool ok = true;
     if constexpr (need_stat)
-        total = strip_exchange_stat(stat, column, strip, tag, c, scratch, red, ok);
+        total = strip_exchange_stat(stat, column, strip, tag, c, scratch, red, red_u, ok);
     if constexpr (NBITS == 1)
     {
         // (an abandoned strip takes no part in the second exchange: its records already say so)
         if (ok)
         {
-            const float mean = ZT ? 0.0f : total / (float) c.rows;
-            float s0, s1;
+            const E mean = ZT ? (E) 0 : total / (E) c.rows;
+            E s0, s1;
             uint32_t n0;
             sums(mean, s0, s1, n0);
-            strip_exchange_split(s0, s1, n0, column, strip, tag, c, scratch, red, ok);
+            strip_exchange_split(s0, s1, n0, column, strip, tag, c, scratch, red, red_u, ok);
             finish_stats_1bit<ZT>(mean, s0, s1, n0, c.rows - n0, c.rows, lo, hi);
         }
     }
@@ -312,118 +372,129 @@ __device__ __forceinline__ bool strip_column_range(float stat, SplitSums sums, u
         strip_finish(scratch, tag);
     if (ok && strip == 0 && threadIdx.x == 0)
     {
-        float* gh = reinterpret_cast<float*>(qc);
+        E* gh = reinterpret_cast<E*>(qc);
         gh[0] = lo;
         gh[1] = hi;
     }
     return ok;
 }
 
-// A strip with its values in registers: v[kk] = the four values of QWords w ... w + 3 at bit position k0 + kk. FULL: every
-// QWord of the strip exists and has an element at every bit position; otherwise `valid` has bit 4 * kk + e set for the
-// values that exist, and the others are zero (which no sum notices; the count below the threshold is corrected, the codes
-// are masked and nothing is stored for them). Statistics across the strips of the column,
-// header, codes, residual and packed QWords. smem: 8 reduction slots, then WORDS partial QWords when a QWord has several
-// threads. Used by the quantize and the stripe-reduction kernel, which therefore give the same bytes for the same column.
-template <int NBITS, bool ZT, bool FULL>
-__device__ __forceinline__ void strip_stats_pack(f32x4 (&v)[StripShape<NBITS>::SLOTS], uint32_t valid, uint32_t w, uint32_t k0, uint32_t column,
-                                                 uint32_t strip, uint32_t tag, const StripGeom& c, const StripScratch& scratch, float* smem,
-                                                 float* res_col, char* qc)
+// A strip with its values in registers: v[kk] (kk below SLOTS) = the PER values of QWords w ... w + PER - 1 at bit position k0 + kk. FULL:
+// every QWord of the strip exists and has an element at every bit position; otherwise `valid` has bit PER * kk + e set for
+// the values that exist, and the others are zero (which no sum notices; the count below the threshold is corrected, the
+// codes are masked and nothing is stored for them). Statistics across the strips of the column, header, codes, residual
+// and packed QWords. smem: four reduction slots of the element type, four of 32 bits, then WORDS partial QWords when a QWord
+// has several threads. Used by the quantize and the stripe-reduction kernel, which therefore give the same bytes for the
+// same column.
+template <typename E>
+constexpr uint32_t kStripRedBytes = 4 * sizeof(E) + 16;
+
+template <int NBITS, bool ZT, bool FULL, typename E>
+__device__ __forceinline__ void strip_stats_pack(StripVec<E>* v, uint32_t valid, uint32_t w, uint32_t k0,
+                                                 uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c, const StripScratch& scratch,
+                                                 char* smem, E* res_col, char* qc)
 {
-    using SS = StripShape<NBITS>;
-    using PS = PackShape<NBITS>;
+    using SS = StripShape<NBITS, E>;
+    using PS = typename SS::PS;
+    using SE = StripElem<E>;
+    using Q = typename Word<E>::Q;
+    constexpr uint32_t PER = SS::PER;
     const uint32_t tid = threadIdx.x;
-    float* red = smem;
-    uint32_t* red_u = reinterpret_cast<uint32_t*>(smem + 4);
-    uint32_t* words = reinterpret_cast<uint32_t*>(smem + 8);
+    E* red = reinterpret_cast<E*>(smem);
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(smem + 4 * sizeof(E));
+    Q* words = reinterpret_cast<Q*>(smem + kStripRedBytes<E>);
     if constexpr (SS::CHUNKS > 1)
     {
         for (uint32_t x = tid; x < SS::WORDS; x += kStripThreads)
             words[x] = 0u;
     }
-    float stat = 0.0f;
+    E stat = 0;
     if constexpr ((NBITS != 1) || !ZT)
     {
 #pragma unroll
         for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
 #pragma unroll
-            for (uint32_t e = 0; e < 4; ++e)
+            for (uint32_t e = 0; e < PER; ++e)
             {
-                const float x = v[kk][e];
+                const E x = v[kk][e];
                 stat += NBITS == 1 ? x : x * x;
             }
         stat = strip_block_sum(stat, red);
     }
-    float lo = 0.0f, hi = 0.0f;
-    const bool column_ok = strip_column_range<NBITS, ZT>(
+    E lo = 0, hi = 0;
+    const bool column_ok = strip_column_range<NBITS, ZT, E>(
         stat,
-        [&](float mean, float& s0, float& s1, uint32_t& n0) {
-            s0 = 0.0f, s1 = 0.0f, n0 = 0;
+        [&](E mean, E& s0, E& s1, uint32_t& n0) {
+            s0 = 0, s1 = 0, n0 = 0;
 #pragma unroll
             for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
 #pragma unroll
-                for (uint32_t e = 0; e < 4; ++e)
+                for (uint32_t e = 0; e < PER; ++e)
                 {
-                    const float x = v[kk][e];
+                    const E x = v[kk][e];
                     const bool below = x < mean;
-                    s0 += below ? x : 0.0f;
-                    s1 += below ? 0.0f : x;
+                    s0 += below ? x : (E) 0;
+                    s1 += below ? (E) 0 : x;
                     n0 += below ? 1u : 0u;
                 }
             if constexpr (!FULL)
-                n0 -= 0.0f < mean ? (uint32_t) __popc(~valid) : 0u; // the zeros that stand in for elements that do not exist
+                n0 -= (E) 0 < mean ? (uint32_t) __popc(~valid) : 0u; // the zeros that stand in for elements that do not exist
             s0 = strip_block_sum(s0, red);
             s1 = strip_block_sum(s1, red);
             n0 = strip_block_sum(n0, red_u);
         },
-        column, strip, tag, c, scratch, red, qc, lo, hi);
+        column, strip, tag, c, scratch, red, red_u, qc, lo, hi);
     if (!column_ok)
         return; // abandoned column: codes and residual stay as they were
-    const ValueQ vq = make_vq<NBITS>(lo, hi);
-    const float val0 = unquantize_value<NBITS>(vq, 0u);
-    const float val1 = unquantize_value<NBITS>(vq, 1u);
-    uint32_t word[4] = {0u, 0u, 0u, 0u};
-    float* res = res_col + (size_t) k0 * c.nq; // k0 is the same in a wavefront: a scalar base, one offset per lane
+    const ValueQOf<E> vq = make_vq<NBITS, E>(lo, hi);
+    const E val0 = unquantize_value<NBITS, E>(vq, (Q) 0);
+    const E val1 = unquantize_value<NBITS, E>(vq, (Q) 1);
+    Q word[PER];
+#pragma unroll
+    for (uint32_t e = 0; e < PER; ++e)
+        word[e] = 0;
+    E* res = res_col + (size_t) k0 * c.nq; // (where k0 is the same in a wavefront: a scalar base, one offset per lane)
 #pragma unroll
     for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
     {
-        f32x4 r;
+        typename SE::V r;
 #pragma unroll
-        for (uint32_t e = 0; e < 4; ++e)
+        for (uint32_t e = 0; e < PER; ++e)
         {
-            const float x = v[kk][e];
-            uint32_t code = quantize_value<NBITS, ZT>(vq, x);
-            float back;
+            const E x = v[kk][e];
+            Q code = quantize_value<NBITS, ZT, E>(vq, x);
+            E back;
             if constexpr (NBITS == 1)
                 back = code ? val1 : val0;
             else
-                back = unquantize_value<NBITS>(vq, code);
+                back = unquantize_value<NBITS, E>(vq, code);
             r[e] = x - back;
             if constexpr (!FULL)
-                code &= 0u - ((valid >> (4 * kk + e)) & 1u);
+                code &= (Q) 0 - (Q) ((valid >> (PER * kk + e)) & 1u);
             word[e] |= code << ((k0 + kk) * PS::SHIFT);
         }
-        float* dst = res + (size_t) kk * c.nq + w;
-        const uint32_t ok = FULL ? 15u : (valid >> (4 * kk)) & 15u;
-        if (ok == 15u)
-            __builtin_nontemporal_store(r, reinterpret_cast<f32x4_u*>(dst));
+        E* dst = res + (size_t) kk * c.nq + w;
+        constexpr uint32_t ALL = (1u << PER) - 1u;
+        const uint32_t ok = FULL ? ALL : (valid >> (PER * kk)) & ALL;
+        if (ok == ALL)
+            __builtin_nontemporal_store(r, reinterpret_cast<typename SE::VU*>(dst));
         else if (ok != 0u)
         {
 #pragma unroll
-            for (uint32_t e = 0; e < 4; ++e)
+            for (uint32_t e = 0; e < PER; ++e)
                 if ((ok >> e) & 1u)
                     dst[e] = r[e];
         }
     }
-    uint32_t* bits = reinterpret_cast<uint32_t*>(qc + 8);
+    Q* bits = reinterpret_cast<Q*>(qc + 2 * sizeof(E));
     if constexpr (SS::CHUNKS == 1)
     {
-        if (FULL || w + 4 <= c.nq)
-            *reinterpret_cast<u32x4_u*>(bits + w) = u32x4{word[0], word[1], word[2], word[3]};
+        if (FULL || w + PER <= c.nq)
+            *reinterpret_cast<typename SE::QVU*>(bits + w) = SE::words(word);
         else
         {
 #pragma unroll
-            for (uint32_t e = 0; e < 4; ++e)
+            for (uint32_t e = 0; e < PER; ++e)
                 if (w + e < c.nq)
                     bits[w + e] = word[e];
         }
@@ -432,8 +503,13 @@ __device__ __forceinline__ void strip_stats_pack(f32x4 (&v)[StripShape<NBITS>::S
     {
         const uint32_t local = w - strip * SS::WORDS;
 #pragma unroll
-        for (uint32_t e = 0; e < 4; ++e)
-            atomicOr(&words[local + e], word[e]);
+        for (uint32_t e = 0; e < PER; ++e)
+        {
+            if constexpr (sizeof(Q) == 8)
+                atomicOr(reinterpret_cast<unsigned long long*>(&words[local + e]), (unsigned long long) word[e]);
+            else
+                atomicOr(&words[local + e], word[e]);
+        }
         __syncthreads();
         for (uint32_t x = tid; x < SS::WORDS; x += kStripThreads)
             if (FULL || strip * SS::WORDS + x < c.nq)
@@ -441,29 +517,34 @@ __device__ __forceinline__ void strip_stats_pack(f32x4 (&v)[StripShape<NBITS>::S
     }
 }
 
+template <typename E>
 __host__ __device__ inline size_t strip_lds_bytes(size_t nbits)
 {
-    return (8 + (nbits <= 2 ? (size_t) strip_words(nbits) : 0)) * 4;
+    const size_t vpw = Word<E>::kBits / nbits;
+    return kStripRedBytes<E> + (vpw > 8 ? (size_t) strip_words<E>(nbits) * sizeof(E) : 0);
 }
 
 // whether every QWord of the strip exists and has an element at every bit position (only the last bit position can be
 // short of elements, and only in the last QWords of the column)
-template <int NBITS>
+template <int NBITS, typename E>
 __device__ __forceinline__ bool strip_is_full(const StripGeom& c, uint32_t strip)
 {
-    const uint32_t end = (strip + 1) * StripShape<NBITS>::WORDS;
-    return end <= c.nq && (uint64_t) (PackShape<NBITS>::VPW - 1) * c.nq + end <= c.rows;
+    using SS = StripShape<NBITS, E>;
+    const uint32_t end = (strip + 1) * SS::WORDS;
+    return end <= c.nq && (uint64_t) (SS::PS::VPW - 1) * c.nq + end <= c.rows;
 }
 
-// which QWords and bit positions a thread holds of a full strip: four QWords from w, SLOTS bit positions from k0 (the
-// same in a wavefront, so returned as a scalar)
-template <int NBITS>
+// which QWords and bit positions a thread holds of a strip: PER QWords from w, SLOTS bit positions from k0. Where a
+// wavefront holds one range of bit positions k0 is a scalar.
+template <int NBITS, typename E>
 __device__ __forceinline__ void strip_thread_slots(uint32_t strip, uint32_t& w, uint32_t& k0)
 {
-    using SS = StripShape<NBITS>;
-    static_assert(SS::QUADS % kWave == 0, "a wavefront holds one range of bit positions");
-    w = strip * SS::WORDS + 4 * (threadIdx.x % SS::QUADS);
-    k0 = __builtin_amdgcn_readfirstlane(threadIdx.x / SS::QUADS) * SS::SLOTS;
+    using SS = StripShape<NBITS, E>;
+    w = strip * SS::WORDS + SS::PER * (threadIdx.x % SS::RUNS);
+    if constexpr (SS::RUNS % kWave == 0)
+        k0 = __builtin_amdgcn_readfirstlane(threadIdx.x / SS::RUNS) * SS::SLOTS;
+    else
+        k0 = threadIdx.x / SS::RUNS * SS::SLOTS;
 }
 
 // Workgroups go to the eight dies of the device in turn, each die starting its share in order. The strips of a column
@@ -493,42 +574,48 @@ __device__ __forceinline__ bool strip_assignment(const StripGeom& c, const Strip
     return false;
 }
 
-// which of a thread's 4 * SLOTS values exist in a strip at the ragged end of its column
-template <int NBITS>
+// which of a thread's PER * SLOTS values exist in a strip at the ragged end of its column
+template <int NBITS, typename E>
 __device__ __forceinline__ uint32_t strip_valid_mask(const StripGeom& c, uint32_t w, uint32_t k0)
 {
-    using SS = StripShape<NBITS>;
-    uint32_t valid = ~(uint32_t) ((1ull << (4 * SS::SLOTS)) - 1ull); // bits beyond the thread's values count as present
+    using SS = StripShape<NBITS, E>;
+    uint32_t valid = ~(uint32_t) ((1ull << (SS::PER * SS::SLOTS)) - 1ull); // bits beyond the thread's values count as present
 #pragma unroll
     for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
 #pragma unroll
-        for (uint32_t e = 0; e < 4; ++e)
+        for (uint32_t e = 0; e < SS::PER; ++e)
         {
             const uint64_t i = (uint64_t) (w + e) + (uint64_t) (k0 + kk) * c.nq;
-            valid |= (w + e < c.nq && i < c.rows) ? (1u << (4 * kk + e)) : 0u;
+            valid |= (w + e < c.nq && i < c.rows) ? (1u << (SS::PER * kk + e)) : 0u;
         }
     return valid;
 }
 
-// Four consecutive values of a column from element i on, at any 4-byte alignment. FULL: all exist. Otherwise bit e of `ok`
-// says whether value e does, the others read as zero; the 16-byte load never leaves the column (it moves back to the
-// column's last four elements when it would), and the few lanes with some but not all of their values fetch them one by one.
-template <bool FULL>
-__device__ __forceinline__ f32x4 strip_load4(const float* col, uint32_t i, uint32_t rows, uint32_t ok)
+// The PER consecutive values of a column from element i on (16 bytes at the alignment of an element). FULL: all exist.
+// Otherwise bit e of `ok` says whether value e does, the others read as zero; the 16-byte load never leaves the column (it
+// moves back to the column's last PER elements when it would), and the few lanes with some but not all of their values
+// fetch them one by one.
+template <bool FULL, typename E>
+__device__ __forceinline__ StripVec<E> strip_load(const E* col, uint32_t i, uint32_t rows, uint32_t ok)
 {
+    using SE = StripElem<E>;
+    constexpr uint32_t PER = SE::PER;
     if constexpr (FULL)
-        return __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(col + i));
+        return __builtin_nontemporal_load(reinterpret_cast<const typename SE::VU*>(col + i));
     else
     {
-        const uint32_t at = (rows >= 4 && i + 4 > rows) ? rows - 4 : i;
-        f32x4 x = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (rows >= 4)
-            x = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(col + at));
-        if (ok != 15u)
+        const uint32_t at = (rows >= PER && i + PER > rows) ? rows - PER : i;
+        typename SE::V x;
+#pragma unroll
+        for (uint32_t e = 0; e < PER; ++e)
+            x[e] = 0;
+        if (rows >= PER)
+            x = __builtin_nontemporal_load(reinterpret_cast<const typename SE::VU*>(col + at));
+        if (ok != (1u << PER) - 1u)
         {
 #pragma unroll
-            for (uint32_t e = 0; e < 4; ++e)
-                x[e] = ((ok >> e) & 1u) ? col[i + e] : 0.0f;
+            for (uint32_t e = 0; e < PER; ++e)
+                x[e] = ((ok >> e) & 1u) ? col[i + e] : (E) 0;
         }
         return x;
     }
@@ -536,51 +623,175 @@ __device__ __forceinline__ f32x4 strip_load4(const float* col, uint32_t i, uint3
 
 // The gradient goes straight into the registers that will hold the sums, the residual joins it four loads at a time. Every
 // value of the strip is in registers before anything is stored, so r_out may be r_in.
-template <int NBITS, bool ZT, bool FULL>
-__device__ __forceinline__ void quantize_strip_body(const float* g_col, const float* r_col, float* res_col, char* qc, uint32_t column, uint32_t strip,
-                                                    uint32_t tag, const StripGeom& c, const StripScratch& scratch, float* smem)
+template <int NBITS, bool ZT, bool FULL, typename E>
+__device__ __forceinline__ void quantize_strip_body(const E* g_col, const E* r_col, E* res_col, char* qc, uint32_t column, uint32_t strip,
+                                                    uint32_t tag, const StripGeom& c, const StripScratch& scratch, char* smem)
 {
-    using SS = StripShape<NBITS>;
+    using SS = StripShape<NBITS, E>;
+    constexpr uint32_t PER = SS::PER, ALL = (1u << PER) - 1u;
     uint32_t w, k0;
-    strip_thread_slots<NBITS>(strip, w, k0);
-    const uint32_t valid = FULL ? 0xFFFFFFFFu : strip_valid_mask<NBITS>(c, w, k0);
+    strip_thread_slots<NBITS, E>(strip, w, k0);
+    const uint32_t valid = FULL ? 0xFFFFFFFFu : strip_valid_mask<NBITS, E>(c, w, k0);
     const uint32_t i0 = k0 * c.nq + w;
-    f32x4 v[SS::SLOTS];
+    StripVec<E> v[SS::SLOTS];
 #pragma unroll
     for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
-        v[kk] = strip_load4<FULL>(g_col, i0 + kk * c.nq, c.rows, (valid >> (4 * kk)) & 15u);
+        v[kk] = strip_load<FULL, E>(g_col, i0 + kk * c.nq, c.rows, (valid >> (PER * kk)) & ALL);
     constexpr uint32_t BATCH = SS::SLOTS < 4 ? SS::SLOTS : 4;
 #pragma unroll
     for (uint32_t k1 = 0; k1 < SS::SLOTS; k1 += BATCH)
     {
-        f32x4 b[BATCH];
+        StripVec<E> b[BATCH];
 #pragma unroll
         for (uint32_t kk = 0; kk < BATCH; ++kk)
-            b[kk] = strip_load4<FULL>(r_col, i0 + (k1 + kk) * c.nq, c.rows, (valid >> (4 * (k1 + kk))) & 15u);
+            b[kk] = strip_load<FULL, E>(r_col, i0 + (k1 + kk) * c.nq, c.rows, (valid >> (PER * (k1 + kk))) & ALL);
 #pragma unroll
         for (uint32_t kk = 0; kk < BATCH; ++kk)
             v[k1 + kk] = v[k1 + kk] + b[kk];
     }
-    strip_stats_pack<NBITS, ZT, FULL>(v, valid, w, k0, column, strip, tag, c, scratch, smem, res_col, qc);
+    strip_stats_pack<NBITS, ZT, FULL, E>(v, valid, w, k0, column, strip, tag, c, scratch, smem, res_col, qc);
 }
 
-template <int NBITS, bool ZT>
-__global__ __launch_bounds__(kStripThreads, StripShape<NBITS>::WAVES) void quantize_strip_kernel(const float* __restrict__ g, const float* r_in,
-                                                                                                 float* r_out, char* __restrict__ q, StripGeom c,
-                                                                                                 StripScratch scratch)
+template <int NBITS, bool ZT, typename E>
+__global__ __launch_bounds__(kStripThreads, (StripShape<NBITS, E>::WAVES)) void quantize_strip_kernel(const E* __restrict__ g, const E* r_in, E* r_out,
+                                                                                                    char* __restrict__ q, StripGeom c,
+                                                                                                    StripScratch scratch)
 {
-    static_assert(NBITS < 32, "32-bit codes are whole QWords: nothing to assemble");
+    static_assert(NBITS < Word<E>::kBits, "codes as wide as a QWord are whole QWords: nothing to assemble");
     extern __shared__ f32x4 smem_v4[];
-    float* smem = reinterpret_cast<float*>(smem_v4);
+    char* smem = reinterpret_cast<char*>(smem_v4);
     uint32_t column, strip, tag;
     if (!strip_assignment(c, scratch, column, strip, tag))
         return;
     const size_t base = (size_t) column * c.rows;
     char* qc = q + (size_t) column * c.qcol;
-    if (strip_is_full<NBITS>(c, strip))
-        quantize_strip_body<NBITS, ZT, true>(g + base, r_in + base, r_out + base, qc, column, strip, tag, c, scratch, smem);
+    if (strip_is_full<NBITS, E>(c, strip))
+        quantize_strip_body<NBITS, ZT, true, E>(g + base, r_in + base, r_out + base, qc, column, strip, tag, c, scratch, smem);
     else
-        quantize_strip_body<NBITS, ZT, false>(g + base, r_in + base, r_out + base, qc, column, strip, tag, c, scratch, smem);
+        quantize_strip_body<NBITS, ZT, false, E>(g + base, r_in + base, r_out + base, qc, column, strip, tag, c, scratch, smem);
+}
+
+// ---- the stripe reduction of the quantized all-reduce on strips: K packed stripes -> sum -> requantize with the stripe
+// residual (Source/1BitSGD/AllReduceDistGradAggregator.h:385-436: unquantize the owner's stripe, add the other workers' in
+// ascending order, quantize the sum with the stripe residual). A thread decodes its QWords of every worker at its bit
+// positions into the registers that strip_stats_pack then takes, so the call gives the bytes of that call sequence with the
+// strip kernel as its quantize step. Every worker's column header is read before the strip publishes its first partial
+// sum, and strip 0 writes the new header only after it has every strip's: q_out may be the owner's own stripe.
+template <int NBITS, bool ZT, bool FULL, typename E>
+__device__ __forceinline__ void stripe_reduce_strip_body(const StripeSources& src, size_t col_off, E* res_col, char* qc_out, E* agg_col,
+                                                         uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
+                                                         const StripScratch& scratch, char* smem)
+{
+    using SS = StripShape<NBITS, E>;
+    using PS = typename SS::PS;
+    using SE = StripElem<E>;
+    using Q = typename Word<E>::Q;
+    constexpr uint32_t PER = SS::PER, ALL = (1u << PER) - 1u;
+    uint32_t w, k0;
+    strip_thread_slots<NBITS, E>(strip, w, k0);
+    const uint32_t valid = FULL ? 0xFFFFFFFFu : strip_valid_mask<NBITS, E>(c, w, k0);
+    StripVec<E> v[SS::SLOTS];
+    auto add_worker = [&](uint32_t n, auto first) {
+        const char* qc = src.q[stripe_order(n, src.owner)] + col_off;
+        const E* h = reinterpret_cast<const E*>(qc);
+        const ValueQOf<E> vq = make_vq<NBITS, E>(h[0], h[1]);
+        const Q* bits = reinterpret_cast<const Q*>(qc + 2 * sizeof(E));
+        Q word[PER];
+        if (FULL || w + PER <= c.nq)
+        {
+            const typename SE::QV x = *reinterpret_cast<const typename SE::QVU*>(bits + w);
+#pragma unroll
+            for (uint32_t e = 0; e < PER; ++e)
+                word[e] = x[e];
+        }
+        else
+        {
+#pragma unroll
+            for (uint32_t e = 0; e < PER; ++e)
+                word[e] = w + e < c.nq ? bits[w + e] : (Q) 0;
+        }
+        const E val0 = unquantize_value<NBITS, E>(vq, (Q) 0);
+        const E val1 = unquantize_value<NBITS, E>(vq, (Q) 1);
+#pragma unroll
+        for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
+#pragma unroll
+            for (uint32_t e = 0; e < PER; ++e)
+            {
+                const Q code = (word[e] >> ((k0 + kk) * PS::SHIFT)) & PS::CODEMASK;
+                E x;
+                if constexpr (NBITS == 1)
+                    x = code ? val1 : val0;
+                else
+                    x = unquantize_value<NBITS, E>(vq, code);
+                // the first term seeds the sum; afterwards: decoded value + running sum
+                if constexpr (decltype(first)::value)
+                    v[kk][e] = x;
+                else
+                    v[kk][e] = x + v[kk][e];
+            }
+    };
+    add_worker(0u, std::true_type());
+    for (uint32_t n = 1; n < src.workers; ++n)
+        add_worker(n, std::false_type());
+    if constexpr (!FULL)
+    {
+        // (a QWord's bits beyond the column's last element are zero and decode to the lowest level: those values do not exist)
+#pragma unroll
+        for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
+#pragma unroll
+            for (uint32_t e = 0; e < PER; ++e)
+                v[kk][e] = ((valid >> (PER * kk + e)) & 1u) ? v[kk][e] : (E) 0;
+    }
+    const uint32_t i0 = k0 * c.nq + w;
+    if (agg_col != nullptr)
+    {
+#pragma unroll
+        for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
+        {
+            E* dst = agg_col + i0 + kk * c.nq;
+            const uint32_t ok = FULL ? ALL : (valid >> (PER * kk)) & ALL;
+            if (ok == ALL)
+                __builtin_nontemporal_store(v[kk], reinterpret_cast<typename SE::VU*>(dst));
+            else if (ok != 0u)
+            {
+#pragma unroll
+                for (uint32_t e = 0; e < PER; ++e)
+                    if ((ok >> e) & 1u)
+                        dst[e] = v[kk][e];
+            }
+        }
+    }
+    constexpr uint32_t BATCH = SS::SLOTS < 4 ? SS::SLOTS : 4;
+#pragma unroll
+    for (uint32_t k1 = 0; k1 < SS::SLOTS; k1 += BATCH)
+    {
+        StripVec<E> b[BATCH];
+#pragma unroll
+        for (uint32_t kk = 0; kk < BATCH; ++kk)
+            b[kk] = strip_load<FULL, E>(res_col, i0 + (k1 + kk) * c.nq, c.rows, (valid >> (PER * (k1 + kk))) & ALL);
+#pragma unroll
+        for (uint32_t kk = 0; kk < BATCH; ++kk)
+            v[k1 + kk] = v[k1 + kk] + b[kk];
+    }
+    strip_stats_pack<NBITS, ZT, FULL, E>(v, valid, w, k0, column, strip, tag, c, scratch, smem, res_col, qc_out);
+}
+
+template <int NBITS, bool ZT, typename E>
+__global__ __launch_bounds__(kStripThreads, (StripShape<NBITS, E>::WAVES)) void stripe_reduce_strip_kernel(StripeSources src, E* stripe_res, char* q_out,
+                                                                                                           E* agg_out, StripGeom c, StripScratch scratch)
+{
+    static_assert(NBITS < Word<E>::kBits, "codes as wide as a QWord are whole QWords: nothing to assemble");
+    extern __shared__ f32x4 smem_v4[];
+    char* smem = reinterpret_cast<char*>(smem_v4);
+    uint32_t column, strip, tag;
+    if (!strip_assignment(c, scratch, column, strip, tag))
+        return;
+    const size_t base = (size_t) column * c.rows, col_off = (size_t) column * c.qcol;
+    E* agg_col = agg_out != nullptr ? agg_out + base : nullptr;
+    if (strip_is_full<NBITS, E>(c, strip))
+        stripe_reduce_strip_body<NBITS, ZT, true, E>(src, col_off, stripe_res + base, q_out + col_off, agg_col, column, strip, tag, c, scratch, smem);
+    else
+        stripe_reduce_strip_body<NBITS, ZT, false, E>(src, col_off, stripe_res + base, q_out + col_off, agg_col, column, strip, tag, c, scratch, smem);
 }
 
 } // namespace cntkq

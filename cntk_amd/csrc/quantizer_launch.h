@@ -174,10 +174,18 @@ hipError_t family_regs_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEven
                                 uint32_t cols, RegGeom c);
 hipError_t family_reg_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out,
                              float* agg_out, uint32_t cols, RegGeom c, uint32_t threads);
+hipError_t family_strip_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, char* q,
+                                 uint32_t cols, StripGeom c, StripScratch scratch);
 hipError_t family_strip_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q,
                                  uint32_t cols, StripGeom c, StripScratch scratch);
 // workgroups of the strip kernel that the runtime says a compute unit holds at once
-hipError_t family_strip_occupancy(size_t nbits, bool zt, int* per_cu);
+hipError_t family_strip_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out,
+                               float* agg_out, uint32_t cols, StripGeom c, StripScratch scratch);
+hipError_t family_strip_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const StripeSources& src, double* stripe_res, char* q_out,
+                               double* agg_out, uint32_t cols, StripGeom c, StripScratch scratch);
+// (stripe: of the stripe-reduction kernel instead of the quantize kernel; the last argument only names the element type)
+hipError_t family_strip_occupancy(size_t nbits, bool zt, bool stripe, int* per_cu, const float*);
+hipError_t family_strip_occupancy(size_t nbits, bool zt, bool stripe, int* per_cu, const double*);
 hipError_t family_unquantize(size_t nbits, hipStream_t s, LaunchEvents ev, const char* q, float* out, const UnquantizePlan& p, int add);
 hipError_t family_batch_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const QuantizeBatchEntry* entries, const uint32_t* begins,
                                  uint32_t count, uint32_t total_blocks, size_t lds);
@@ -325,41 +333,51 @@ inline bool regs_applicable(size_t rows, size_t nbits)
 // that re-reads its column.
 constexpr uint32_t kStripMaxPerColumn = 128;
 
+// (written over the element type: E's QWord has Word<E>::kBits bits)
+template <typename E>
+inline size_t strip_qwords_per_col(size_t rows, size_t nbits)
+{
+    const size_t vpw = Word<E>::kBits / nbits;
+    return (rows + vpw - 1) / vpw;
+}
+
+template <typename E>
 inline bool strip_applicable(size_t rows, size_t nbits, const LaunchTuning& tune)
 {
-    return tune.strip != nullptr && nbits < 32 && rows >= 1 &&
-           (qwords_per_col(rows, nbits) + strip_words(nbits) - 1) / strip_words(nbits) <= kStripMaxPerColumn * kStripDies;
+    return tune.strip != nullptr && nbits < (size_t) Word<E>::kBits && rows >= 1 &&
+           (strip_qwords_per_col<E>(rows, nbits) + strip_words<E>(nbits) - 1) / strip_words<E>(nbits) <= kStripMaxPerColumn * kStripDies;
 }
 
 // per_die: the most strips of a column that one die takes (strip_resident_limit); a column of more has its strips on all
 // dies (StripGeom::spread), up to kStripDies times as many
+template <typename E>
 inline StripGeom make_strip_geom(size_t rows, size_t cols, size_t nbits, uint32_t spin_limit, uint32_t per_die)
 {
     StripGeom c;
     c.rows = (uint32_t) rows;
     c.cols = (uint32_t) cols;
-    c.nq = (uint32_t) qwords_per_col(rows, nbits);
-    c.strips = (c.nq + strip_words(nbits) - 1) / strip_words(nbits);
+    c.nq = (uint32_t) strip_qwords_per_col<E>(rows, nbits);
+    c.strips = (c.nq + strip_words<E>(nbits) - 1) / strip_words<E>(nbits);
     c.spin_limit = spin_limit;
     c.poll_pause = kStripPollPause;
     c.poll_first = c.strips >= kStripFirstPauseMinStrips ? 2u * std::min(c.strips, kStripMaxPerColumn) : 0u;
     c.inv_strips = 1.0 / (double) c.strips;
     c.spread = c.strips > per_die ? 1u : 0u;
     c.pad = 0;
-    c.qcol = qcol_bytes(nbits, rows);
+    c.qcol = (uint64_t) (2 + c.nq) * sizeof(E); // the header's two bounds, then the QWords
     return c;
 }
 
-
-inline bool strip_scratch_fits(const StripScratchOwner& o, size_t cols, size_t strips)
+// records_each: records per (column, strip) of the element type (strip_records<E>())
+inline bool strip_scratch_fits(const StripScratchOwner& o, size_t cols, size_t strips, size_t records_each)
 {
     return o.dev != nullptr && strip_groups_bytes(cols, strips) <= o.groups_bytes &&
-           sizeof(StripHeader) + o.groups_bytes + strip_records_bytes(cols, strips) <= o.bytes;
+           sizeof(StripHeader) + o.groups_bytes + strip_records_bytes(cols, strips, records_each) <= o.bytes;
 }
 
 // Makes the owner's buffer large enough for this launch (growing waits for the stream and clears the new buffer: the launch
 // count and every record's tag start at zero). Not possible while the stream is being captured.
-inline hipError_t strip_scratch_for(StripScratchOwner& o, hipStream_t s, size_t cols, size_t strips, StripScratch& out)
+inline hipError_t strip_scratch_for(StripScratchOwner& o, hipStream_t s, size_t cols, size_t strips, size_t records_each, StripScratch& out)
 {
     if (o.error_host == nullptr)
     {
@@ -370,7 +388,7 @@ inline hipError_t strip_scratch_for(StripScratchOwner& o, hipStream_t s, size_t 
         o.error_host = static_cast<uint32_t*>(p);
         *o.error_host = 0u;
     }
-    if (!strip_scratch_fits(o, cols, strips))
+    if (!strip_scratch_fits(o, cols, strips, records_each))
     {
         hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(s, &st) == hipSuccess && st == hipStreamCaptureStatusActive)
@@ -389,7 +407,7 @@ inline hipError_t strip_scratch_for(StripScratchOwner& o, hipStream_t s, size_t 
         o.bytes = 0;
         o.captured = false;
         o.abandoned_seen = 0;
-        const size_t need = sizeof(StripHeader) + strip_records_bytes(cols, strips);
+        const size_t need = sizeof(StripHeader) + strip_records_bytes(cols, strips, records_each);
         const size_t cap = std::max<size_t>((need * 2 + 8191) & ~(size_t) 4095, (size_t) 1 << 20);
         void* p = nullptr;
         rc = hipMalloc(&p, cap);
@@ -416,9 +434,9 @@ inline hipError_t strip_scratch_for(StripScratchOwner& o, hipStream_t s, size_t 
 
 // whether this launch finds its scratch buffer without allocating, or may allocate (the caller permits it and the stream
 // is not being captured)
-inline bool strip_scratch_ready(const StripScratchOwner& o, hipStream_t s, size_t cols, size_t strips, bool may_allocate = true)
+inline bool strip_scratch_ready(const StripScratchOwner& o, hipStream_t s, size_t cols, size_t strips, size_t records_each, bool may_allocate = true)
 {
-    if (o.error_host != nullptr && strip_scratch_fits(o, cols, strips))
+    if (o.error_host != nullptr && strip_scratch_fits(o, cols, strips, records_each))
         return true;
     if (!may_allocate)
         return false;
@@ -435,18 +453,19 @@ inline uint32_t strip_grid(size_t cols, const StripGeom& c)
 // each other on one die, so all of them must be resident there together, next to the strips of the columns around them.
 // Half of what the die holds by the runtime's own occupancy figure for the kernel (workgroups per compute unit x compute
 // units of the device / 8 dies); 0 where the runtime cannot say. Asked once per kernel variant and device.
-inline uint32_t strip_resident_limit(size_t nbits, bool zt)
+template <typename E>
+inline uint32_t strip_resident_limit(size_t nbits, bool zt, bool stripe = false)
 {
-    static int cache[64][6][2]; // 0: not asked yet; -1: unknown
+    static int cache[64][6][2][2]; // 0: not asked yet; -1: unknown (one table per element type)
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
         return 0;
-    const int b = nbits == 1 ? 0 : nbits == 2 ? 1 : nbits == 4 ? 2 : nbits == 8 ? 3 : 4;
-    int& slot = cache[dev][b][zt ? 1 : 0];
+    const int b = nbits == 1 ? 0 : nbits == 2 ? 1 : nbits == 4 ? 2 : nbits == 8 ? 3 : nbits == 16 ? 4 : 5;
+    int& slot = cache[dev][b][zt ? 1 : 0][stripe ? 1 : 0];
     if (slot == 0)
     {
         int per_cu = 0, cus = 0;
-        hipError_t rc = family_strip_occupancy(nbits, zt, &per_cu);
+        hipError_t rc = family_strip_occupancy(nbits, zt, stripe, &per_cu, (const E*) nullptr);
         if (rc == hipSuccess)
             rc = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         if (rc != hipSuccess)
@@ -457,15 +476,85 @@ inline uint32_t strip_resident_limit(size_t nbits, bool zt)
 }
 
 // ... the same, never more than kStripMaxPerColumn
-inline uint32_t strip_per_die(size_t nbits, bool zt)
+template <typename E>
+inline uint32_t strip_per_die(size_t nbits, bool zt, bool stripe = false)
 {
-    return std::min(strip_resident_limit(nbits, zt), kStripMaxPerColumn);
+    return std::min(strip_resident_limit<E>(nbits, zt, stripe), kStripMaxPerColumn);
 }
 
 // the most strips per column that the strip kernels take on the current device, spread over all dies
-inline uint32_t strip_max_strips(size_t nbits, bool zt)
+template <typename E>
+inline uint32_t strip_max_strips(size_t nbits, bool zt, bool stripe = false)
 {
-    return strip_per_die(nbits, zt) * kStripDies;
+    return strip_per_die<E>(nbits, zt, stripe) * kStripDies;
+}
+
+// Whether the automatic choice may hand this matrix to the strip kernels right now: a column within what the device holds
+// of strips, and a scratch buffer that is there or may be made (a stream under capture cannot wait for a larger one).
+template <typename E>
+inline bool strip_ready(hipStream_t s, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune, bool stripe = false)
+{
+    if (!strip_applicable<E>(rows, nbits, tune))
+        return false;
+    const StripGeom c = make_strip_geom<E>(rows, cols, nbits, tune.strip_spin_limit, strip_per_die<E>(nbits, zt, stripe));
+    return (uint64_t) (cols + kStripDies) * c.strips <= 0x7FFFFFFFull && c.strips <= strip_max_strips<E>(nbits, zt, stripe) &&
+           strip_scratch_ready(*tune.strip, s, cols, c.strips, strip_records<E>(), tune.strip_may_allocate);
+}
+
+// A strip kernel on one matrix of either element type: the scratch buffer (grown if need be), the order against the last
+// launch that used it on another stream, then `launch(geometry, scratch)`.
+template <typename E, typename Launch>
+inline hipError_t launch_on_strips(hipStream_t s, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune, bool stripe,
+                                   Launch launch)
+{
+    const StripGeom c = make_strip_geom<E>(rows, cols, nbits, tune.strip_spin_limit, strip_per_die<E>(nbits, zt, stripe));
+    if (!strip_applicable<E>(rows, nbits, tune) || (uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull ||
+        c.strips > strip_max_strips<E>(nbits, zt, stripe))
+        return hipErrorInvalidValue;
+    StripScratchOwner& o = *tune.strip;
+    StripScratch scratch;
+    hipError_t rc = strip_scratch_for(o, s, cols, c.strips, strip_records<E>(), scratch);
+    if (rc != hipSuccess)
+        return rc;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(s, &st) != hipSuccess || st != hipStreamCaptureStatusNone;
+    if (capturing)
+        o.captured = true;
+    if (!capturing)
+    {
+        if (o.order_event == nullptr && (rc = hipEventCreateWithFlags(&o.order_event, hipEventDisableTiming)) != hipSuccess)
+            return rc;
+        if (o.launched && o.last_stream != s && (rc = hipStreamWaitEvent(s, o.order_event, 0)) != hipSuccess)
+            return rc;
+    }
+    rc = launch(c, scratch);
+    if (rc == hipSuccess && !capturing)
+    {
+        rc = hipEventRecord(o.order_event, s);
+        o.last_stream = s;
+        o.launched = true;
+    }
+    return rc;
+}
+
+template <typename E>
+inline hipError_t launch_strip_quantize(hipStream_t s, LaunchEvents ev, const E* g, const E* r_in, E* r_out, char* qc, size_t rows, size_t cols,
+                                        size_t nbits, bool zt, const LaunchTuning& tune)
+{
+    return launch_on_strips<E>(s, rows, cols, nbits, zt, tune, false, [&](const StripGeom& c, const StripScratch& scratch) {
+        return family_strip_quantize(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, scratch);
+    });
+}
+
+// The fused stripe reduction on strips: for stripes taller than the kernels with a workgroup per column take, where a
+// quantize call on (aggregate, stripe residual) takes the strip kernel too, so that both give the same bytes.
+template <typename E>
+inline hipError_t launch_strip_stripe(hipStream_t s, LaunchEvents ev, const StripeSources& src, E* stripe_res, char* q_out, E* agg_out, size_t rows,
+                                      size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+{
+    return launch_on_strips<E>(s, rows, cols, nbits, zt, tune, true, [&](const StripGeom& c, const StripScratch& scratch) {
+        return family_strip_stripe(nbits, zt, s, ev, src, stripe_res, q_out, agg_out, (uint32_t) cols, c, scratch);
+    });
 }
 
 // which path launch_quantize takes for this matrix when nothing is forced
@@ -503,15 +592,10 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     int path = tune.quantize_path;
     if (path == kPathAuto)
     {
-        path = quantize_auto_path(g, r_in, r_out, q, rows, nbits, strip_applicable(rows, nbits, tune));
-        if (path == kPathStrip)
-        {
-            // a stream under capture cannot wait for a larger scratch buffer: the kernels that need none take the matrix
-            const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit, strip_per_die(nbits, zt));
-            if ((uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull ||
-                !strip_scratch_ready(*tune.strip, s, cols, c.strips, tune.strip_may_allocate) || c.strips > strip_max_strips(nbits, zt))
-                path = regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
-        }
+        path = quantize_auto_path(g, r_in, r_out, q, rows, nbits, strip_applicable<float>(rows, nbits, tune));
+        // (a stream under capture cannot wait for a larger scratch buffer: the kernels that need none take the matrix)
+        if (path == kPathStrip && !strip_ready<float>(s, rows, cols, nbits, zt, tune))
+            path = regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
     }
     if (path == kPathReg)
     {
@@ -532,36 +616,7 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
                                            make_reg_geom(rows, nbits, threads, line_shift), threads);
     }
     if (path == kPathStrip)
-    {
-        const StripGeom c = make_strip_geom(rows, cols, nbits, tune.strip_spin_limit, strip_per_die(nbits, zt));
-        if (!strip_applicable(rows, nbits, tune) || (uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull ||
-            c.strips > strip_max_strips(nbits, zt))
-            return hipErrorInvalidValue;
-        StripScratchOwner& o = *tune.strip;
-        StripScratch scratch;
-        hipError_t rc = strip_scratch_for(o, s, cols, c.strips, scratch);
-        if (rc != hipSuccess)
-            return rc;
-        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-        const bool capturing = hipStreamIsCapturing(s, &st) != hipSuccess || st != hipStreamCaptureStatusNone;
-        if (capturing)
-            o.captured = true;
-        if (!capturing)
-        {
-            if (o.order_event == nullptr && (rc = hipEventCreateWithFlags(&o.order_event, hipEventDisableTiming)) != hipSuccess)
-                return rc;
-            if (o.launched && o.last_stream != s && (rc = hipStreamWaitEvent(s, o.order_event, 0)) != hipSuccess)
-                return rc;
-        }
-        rc = family_strip_quantize(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, scratch);
-        if (rc == hipSuccess && !capturing)
-        {
-            rc = hipEventRecord(o.order_event, s);
-            o.last_stream = s;
-            o.launched = true;
-        }
-        return rc;
-    }
+        return launch_strip_quantize<float>(s, ev, g, r_in, r_out, qc, rows, cols, nbits, zt, tune);
     if (path == kPathRegScalar)
     {
         if (!regs_applicable(rows, nbits))
@@ -607,6 +662,22 @@ inline size_t stripe_reduce_max_rows(size_t nbits)
     return tall > kTileMaxRows ? tall : kTileMaxRows;
 }
 
+// Heights at which no kernel with one workgroup per column takes a matrix whatever its alignment, so that the automatic
+// choice of a quantize call is the strip kernels (or, without them, the kernel that re-reads its columns).
+inline bool strip_only_height(size_t rows, size_t nbits)
+{
+    return nbits < 32 && rows > kTileMaxRows && (rows > kRegMaxRows || (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 > 64 * 1024);
+}
+
+// Whether the fused stripe reduction takes a stripe taller than stripe_reduce_max_rows: on strips, where a quantize call
+// on (aggregate, stripe residual) would run on strips as well (same bytes), with the scratch buffer there or obtainable.
+inline bool stripe_takes_strips(hipStream_t s, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+{
+    zt = zt && nbits == 1;
+    return strip_only_height(rows, nbits) && strip_ready<float>(s, rows, cols, nbits, zt, tune, false) &&
+           strip_ready<float>(s, rows, cols, nbits, zt, tune, true);
+}
+
 // Whether a stripe whose height and alignment would let the LDS column kernels take it goes to the table-driven register
 // kernel with 256 threads instead (1 bit, up to eight workers, above 2048 rows), and how many pieces a thread holds there.
 inline bool stripe_looks_up(size_t rows, size_t nbits, size_t workers)
@@ -634,6 +705,12 @@ inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const Str
                                        const LaunchTuning& tune)
 {
     zt = zt && (nbits == 1);
+    if (rows > stripe_reduce_max_rows(nbits))
+    {
+        if (!stripe_takes_strips(s, rows, cols, nbits, zt, tune) || (reinterpret_cast<uintptr_t>(q_out) & 3u) != 0)
+            return hipErrorInvalidValue;
+        return launch_strip_stripe<float>(s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, rows, cols, nbits, zt, tune);
+    }
     if (stripe_uses_reg(rows, stripe_res, nbits, tune.quantize_path))
     {
         if (rows > stripe_reduce_max_rows(nbits) || (reinterpret_cast<uintptr_t>(q_out) & 3u) != 0)

@@ -234,7 +234,7 @@ inline int quantize_auto_path(const double* g, const double* r_in, const double*
     return rows <= kTileMaxRows ? kPathTile : kPathTall;
 }
 
-// rows, cols > 0; pointers 8-byte aligned (checked by the caller). tune.quantize_path may force the tile or tall kernel.
+// rows, cols > 0; pointers 8-byte aligned (checked by the caller). tune.quantize_path may force a kernel family.
 inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, void* q, size_t rows,
                                   size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
 {
@@ -242,7 +242,15 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* 
     char* qc = static_cast<char*>(q);
     int path = tune.quantize_path;
     if (path == kPathAuto)
+    {
         path = quantize_auto_path(g, r_in, r_out, rows, nbits);
+        // columns that no workgroup's registers hold: strips of the column on several workgroups, which read their inputs
+        // once, where the device holds all strips of a column at once and the scratch buffer is there or may be made
+        if (path == kPathTall && nbits < 64 && strip_ready<double>(s, rows, cols, nbits, zt, tune))
+            path = kPathStrip;
+    }
+    if (path == kPathStrip)
+        return launch_strip_quantize<double>(s, ev, g, r_in, r_out, qc, rows, cols, nbits, zt, tune);
     if (path == kPathReg)
     {
         if (!reg_applicable(g, r_in, r_out, rows, nbits))
@@ -331,10 +339,32 @@ inline size_t stripe_reduce_max_rows(size_t nbits)
 // The kernel family, and within it the geometry, that a quantize call on (aggregate, stripe residual) would take, so that the
 // fused call gives the bytes of the unquantize ... quantize call sequence (the sequence's aggregate must sit at the stripe
 // residual's offset within 16 bytes for that, as whole allocations do).
+// Heights at which the automatic choice of a quantize call is the strip kernels (or, without them, the kernel that re-reads
+// its columns): what no workgroup's registers hold.
+inline bool strip_only_height(size_t rows, size_t nbits)
+{
+    return nbits < 64 && rows > kTileMaxRows && quantize_auto_path(nullptr, nullptr, nullptr, rows, nbits) == kPathTall;
+}
+
+// Whether the fused stripe reduction takes a stripe taller than stripe_reduce_max_rows: on strips, where a quantize call
+// on (aggregate, stripe residual) would run on strips as well (same bytes), with the scratch buffer there or obtainable.
+inline bool stripe_takes_strips(hipStream_t s, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+{
+    zt = zt && nbits == 1;
+    return strip_only_height(rows, nbits) && strip_ready<double>(s, rows, cols, nbits, zt, tune, false) &&
+           strip_ready<double>(s, rows, cols, nbits, zt, tune, true);
+}
+
 inline hipError_t launch_stripe_reduce(hipStream_t s, LaunchEvents ev, const StripeSources& src, double* stripe_res, void* q_out,
                                        double* agg_out, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
 {
     zt = zt && (nbits == 1);
+    if (rows > stripe_reduce_max_rows(nbits))
+    {
+        if (!f64::stripe_takes_strips(s, rows, cols, nbits, zt, tune))
+            return hipErrorInvalidValue;
+        return launch_strip_stripe<double>(s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, rows, cols, nbits, zt, tune);
+    }
     if (stripe_uses_reg(rows, nbits))
         return dispatch_nbits64<StripeRegLauncher>(nbits, zt, s, ev, src, stripe_res, static_cast<char*>(q_out), agg_out, (uint32_t) cols,
                                                    make_reg_geom(rows, nbits, reg_line_shift(stripe_res, rows)));

@@ -52,7 +52,7 @@ def main():
 
     # no fused stripe reduction above this height: the other two calls are still measured
     stripe_limit = getattr(L, "cntkq_stripe_reduce_max_rows" + sfx)(nbits)
-    stripe_skipped = bool(args.workers) and rows > stripe_limit
+    stripe_skipped = bool(args.workers) and not qz.StripeReduceTakes(rows, cols, nbits, zt, tdt)
     if stripe_skipped:
         args.workers = 0
 
@@ -134,7 +134,8 @@ def main():
         "unquantize": {"us": round(u_ms * 1e3, 2), "algorithmic_bytes": u_bytes, "GBps": round(u_bytes / u_ms / 1e6, 1)},
     }
     if stripe_skipped:
-        out["stripe_reduce"] = {"skipped": "columns of %d rows: the fused stripe reduction takes at most %d at %d bits" % (rows, stripe_limit, nbits)}
+        out["stripe_reduce"] = {"skipped": "columns of %d rows: the fused stripe reduction does not take them at %d bits (at most %d, and taller ones "
+                                            "where the strip kernels do)" % (rows, nbits, stripe_limit)}
     if args.workers:
         s_ms = avg_ms(4, 5)
         s_bytes = (args.workers + 1) * qbytes + 2 * elems * eb

@@ -209,8 +209,6 @@ class QuantizedGradientAggregator:
         """The owner's stripe reductions: they touch the aggregator's own buffers only, so they are laid out once."""
         W, me = self.transport.world_size, self.transport.rank
         arrived = self._send if W == 1 else self._recv
-        max32 = _fn("cntkq_stripe_reduce_max_rows", torch.float32)(self.nbits)
-        max64 = _fn("cntkq_stripe_reduce_max_rows", torch.float64)(self.nbits)
         fused, fused64, tall = [], [], []
         for i, (rows, _, dt, _) in enumerate(self._shapes):
             n = self._stripe[me][i][1]
@@ -220,7 +218,7 @@ class QuantizedGradientAggregator:
             stripes = [self._packed(self._send, me, me, i) if r == me else self._packed(arrived, r, me, i) for r in range(W)]
             sres = Matrix(rows, n, self._send.device.index, self._stripe_residual[i])
             item = (stripes, sres, self._packed(self._mine, 0, me, i), None)
-            if rows > (max32 if dt == torch.float32 else max64):
+            if not self._impl.StripeReduceTakes(rows, n, self.nbits, self.zt, dt):
                 tall.append(item)
             elif dt == torch.float32:
                 fused.append(item)
@@ -253,7 +251,7 @@ class QuantizedGradientAggregator:
         for prepared in self._s_fused:
             self._impl.StripeReduceBatchAsync(prepared, me, self.zt)
         for stripes, sres, out, _ in self._s_tall:
-            # columns too tall for the fused kernel: the reference's own sequence of calls
+            # shapes the fused kernels do not take: the reference's own sequence of calls
             agg = Matrix(sres.rows, sres.cols, sres.device_id, dtype=sres.dtype)
             self._impl.UnquantizeAsync(stripes[me], agg, add=False)
             for r in range(W):

@@ -73,8 +73,9 @@ size_t cntkq_qmatrix_bytes(size_t rows, size_t cols, size_t nbits);
 int cntkq_stripe_range(size_t cols, size_t rank, size_t workers, size_t* start_col, size_t* num_cols);
 
 /* Tallest column the fused stripe reduction (cntkq_stripe_reduce_async / _batch_async, an optional fast path without a
- * counterpart in the reference) accepts at this bit width (0 for an invalid width); for taller stripes the caller keeps the reference's sequence of
- * UnquantizeAsync ... QuantizeAsync calls (Source/1BitSGD/AllReduceDistGradAggregator.h:365-436). */
+ * counterpart in the reference) accepts on any device at this bit width (0 for an invalid width). Taller stripes: ask
+ * cntkq_stripe_reduce_takes; where it says no, the caller keeps the reference's sequence of UnquantizeAsync ...
+ * QuantizeAsync calls (Source/1BitSGD/AllReduceDistGradAggregator.h:365-436). */
 size_t cntkq_stripe_reduce_max_rows(size_t nbits);
 
 /* ---- the quantizer object -------------------------------------------------------------------- */
@@ -252,8 +253,19 @@ int cntkq_stripe_reduce_batch_owners_async(cntkq_quantizer* h, const cntkq_strip
                                            size_t count, size_t workers, size_t nbits, int zero_threshold_for_1bit);
 
 /* Blocks until the last stripe reduction of this handle has finished (the reference waits on the stripe
- * quantizer's WaitQuantizeAsyncDone, Source/1BitSGD/AllReduceDistGradAggregator.h:494). */
+ * quantizer's WaitQuantizeAsyncDone, Source/1BitSGD/AllReduceDistGradAggregator.h:494). A reduction that ran on strips
+ * (see cntkq_stripe_reduce_takes) reports here, as CNTKQ_RUNTIME_ERROR, columns whose workgroups gave up waiting for one
+ * another; those columns are left as they were. */
 int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h);
+
+/* Whether the fused stripe reduction of this handle takes stripes of this shape (1) or the caller keeps the reference's
+ * sequence of UnquantizeAsync ... QuantizeAsync calls for them (0). No counterpart in the reference: the fused call is
+ * an optional fast path. Always 1 up to cntkq_stripe_reduce_max_rows(nbits). Taller stripes run with several workgroups per
+ * column where a QuantizeAsync call on the same shape does too (heights that no single workgroup holds: above 102400
+ * rows, or fewer at 8 and 16 bits) and the device holds all of a column's workgroups at once: 1 to 16 bits, up to some 5
+ * million rows at 1 to 4 bits on an MI355X. The answer holds for the handle's current stream; under stream capture it is
+ * 0 where the call would have to allocate. */
+int cntkq_stripe_reduce_takes(cntkq_quantizer* h, size_t rows, size_t stripe_cols, size_t nbits, int zero_threshold_for_1bit);
 
 /* ---- the double instantiation: MatrixQuantizerImpl<double> -----------------------------------------------
  *
@@ -265,7 +277,7 @@ int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h);
  *   - packed matrix: cols records { double lower; double upper; uint64_t bits[nq]; }, nq = ceil(rows / (64 / nbits)),
  *     element i in bits[i % nq] at bit (i / nq) * nbits; the buffer must be 8-byte aligned;
  *   - nbits one of 1, 2, 4, 8, 16, 32, 64 (64 = pass-through; 32 is a real quantizer with 2^32 - 1 steps);
- *   - stripe reduction: rows <= cntkq_stripe_reduce_max_rows_f64(nbits).
+ *   - stripe reduction: rows <= cntkq_stripe_reduce_max_rows_f64(nbits), or a shape cntkq_stripe_reduce_takes_f64 accepts.
  * The gradient-set (batch) calls have their _f64 forms further down. */
 
 /* ColumnQuantizer<double>::QWordsPerCol, QuantizedColumn<double>::QuantizedColumnSize, QuantizedMatrix<double>::GetSize. */
@@ -287,6 +299,8 @@ int cntkq_stripe_reduce_async_f64(cntkq_quantizer* h, const void* const* stripes
                                   size_t rows, size_t stripe_cols, size_t nbits, double* stripe_res, void* q_out,
                                   double* agg_out, int zero_threshold_for_1bit);
 size_t cntkq_stripe_reduce_max_rows_f64(size_t nbits);
+/* cntkq_stripe_reduce_takes for double stripes (taller than cntkq_stripe_reduce_max_rows_f64: from 51185 rows, 1 to 32 bits). */
+int cntkq_stripe_reduce_takes_f64(cntkq_quantizer* h, size_t rows, size_t stripe_cols, size_t nbits, int zero_threshold_for_1bit);
 
 /* The gradient-set calls (cntkq_quantize_batch_async, cntkq_unquantize_batch_async, cntkq_stripe_reduce_batch_async) for
  * double matrices: the same loops of the aggregator (Source/1BitSGD/AllReduceDistGradAggregator.h:288-300, 339-436,
@@ -317,7 +331,7 @@ typedef struct cntkq_stripe_reduce_item_f64
     double* stripe_res;         /* rows x stripe_cols, updated in place */
     void* q_out;                /* packed stripe receiving the requantized aggregate; may be stripes[owner] */
     double* agg_out;            /* optional (may be NULL) */
-    size_t rows;                /* at most cntkq_stripe_reduce_max_rows_f64(nbits) */
+    size_t rows;                /* a height cntkq_stripe_reduce_takes_f64 accepts */
     size_t stripe_cols;
 } cntkq_stripe_reduce_item_f64;
 

@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 
 F64 = np.float64
 VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False), (64, False)]
-PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG, PATH_REGS = 0, 1, 2, 3, 4, 5
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG, PATH_REGS, PATH_STRIP = 0, 1, 2, 3, 4, 5, 6
 
 
 def say(*a):
@@ -143,7 +143,17 @@ PATH_CASES = [
     (1025, 3, PATH_REGS, 0), (2048, 5, PATH_REGS, 0), (2049, 3, PATH_AUTO, 0), (3073, 3, PATH_REGS, 0), (4096, 3, PATH_AUTO, 0),
     (4991, 2, PATH_AUTO, 0), (5120, 2, PATH_REGS, 0), (4099, 2, PATH_REGS, 0), (6144, 2, PATH_AUTO, 0), (6143, 2, PATH_AUTO, 0),
     (6146, 2, PATH_AUTO, 0),
+    # several workgroups per column, a strip of QWords each: any height, one strip or many, full or ragged; the automatic
+    # choice above what one workgroup's registers hold (51184 rows), on one die or, from 81 strips on, on all of them
+    (1, 3, PATH_STRIP, 0), (37, 5, PATH_STRIP, 0), (1000, 3, PATH_STRIP, 0), (4096, 3, PATH_STRIP, 0), (4097, 2, PATH_STRIP, 0),
+    (9304, 3, PATH_STRIP, 0), (16385, 2, PATH_STRIP, 0), (50257, 3, PATH_STRIP, 0), (51201, 2, PATH_AUTO, 0), (102401, 2, PATH_AUTO, 0),
+    (200000, 3, PATH_AUTO, 0), (262147, 2, PATH_STRIP, 0), (330001, 1, PATH_AUTO, 0), (400000, 9, PATH_STRIP, 0),
 ]
+
+
+def strip_words_f64(nbits):
+    """QWords of a double column that one strip holds."""
+    return {1: 64, 2: 128, 4: 256}.get(nbits, 512)
 
 
 @pytest.mark.parametrize("case", PATH_CASES, ids=["%dx%d_p%d_g%d" % c for c in PATH_CASES])
@@ -155,8 +165,11 @@ def test_kernel_paths_f64(case):
     for nbits, zt in VARIANTS:
         say("f64 path case", case, "nbits", nbits, "zeroThr", zt)
         if (path == PATH_REGS and nbits == 64) or \
-                (path == PATH_REG and (nbits == 64 or (48 + oracle.qwords_per_col(rows, nbits, F64)) * 8 > 65536)):
-            # whole-QWord codes and columns whose QWords exceed 64 KB of LDS are refused when forced
+                (path == PATH_REG and (nbits == 64 or (48 + oracle.qwords_per_col(rows, nbits, F64)) * 8 > 65536)) or \
+                (path == PATH_STRIP and (nbits == 64 or oracle.qwords_per_col(rows, nbits, F64) >
+                                         qz._strip_max_strips(nbits, zt, torch.float64) * strip_words_f64(nbits))):
+            # whole-QWord codes, columns whose QWords exceed 64 KB of LDS and columns of more strips than the device holds at
+            # once are refused when forced
             with pytest.raises(cntk_amd.QuantizerLogicError):
                 gpu_quantize(qz, datagen.normal(1, rows, cols, dtype=F64), zeros(rows, cols), nbits, zt)
             continue
@@ -348,10 +361,13 @@ def stripe_max_rows_f64(nbits):
 
 
 @pytest.mark.parametrize("rows,n,k", [(70, 9, 3), (429, 12, 4), (2048, 20, 8), (4096, 3, 2), (4988, 3, 3), (4992, 3, 3), (5003, 2, 2),
-                                      (6144, 2, 3), (6145, 2, 2), (6148, 3, 3), (7168, 2, 5), (64, 40, 64), (8000, 2, 3), (20001, 2, 2), (51184, 1, 2)])
+                                      (6144, 2, 3), (6145, 2, 2), (6148, 3, 3), (7168, 2, 5), (64, 40, 64), (8000, 2, 3), (20001, 2, 2), (51184, 1, 2),
+                                      # on strips: the heights that no single workgroup holds
+                                      (51201, 2, 2), (102401, 2, 3), (330001, 1, 2)])
 def test_stripe_reduce_f64(quantizer, rows, n, k):
     for nbits, zt in VARIANTS:
-        if rows > stripe_max_rows_f64(nbits):
+        if not quantizer.StripeReduceTakes(rows, n, nbits, zt, torch.float64):
+            assert rows > stripe_max_rows_f64(nbits)
             continue
         say("f64 stripe reduce", rows, n, k, nbits, zt)
         stripes = [oracle.quantize(datagen.normal(31 * w + rows + nbits, rows, n, dtype=F64), zeros(rows, n), nbits, zt, threads=8)[0]
@@ -510,5 +526,8 @@ def test_stripe_reduce_height_limit_f64(quantizer):
     rows, n, k = 16286, 2, 2
     Qs = [QuantizedMatrix(rows, n, 16, 0, dtype=torch.float64) for _ in range(k)]
     S = Matrix(rows, n, dtype=torch.float64)
-    with pytest.raises(cntk_amd.QuantizerLogicError, match="taller than 16284 rows"):
+    with pytest.raises(cntk_amd.QuantizerLogicError, match="up to 16284 rows"):
         quantizer.StripeReduceAsync(Qs, 0, S, Qs[0], False)
+    takes = lambda rows, nbits: quantizer.StripeReduceTakes(rows, 2, nbits, False, torch.float64)
+    assert takes(16284, 16) and not takes(16286, 16) and takes(40000, 16)  # (up to 32576 rows the register kernel quantizes)
+    assert takes(51184, 1) and takes(51185, 1) and takes(400000, 4) and not takes(20000, 64) and not takes(50000000, 1)

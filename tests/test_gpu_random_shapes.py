@@ -99,7 +99,7 @@ def test_random_shapes(dtype, seed, count, tall):
     say("  ", rep)
 
 
-@pytest.mark.parametrize("seed,count,tall", [(21, 60, False), (22, 60, False), (23, 40, True)])
+@pytest.mark.parametrize("seed,count,tall", [(21, 60, False), (22, 60, False), (23, 40, True), (24, 24, 2)])
 def test_random_stripe_reductions(seed, count, tall):
     """Random stripes through the fused reduction: the fp32 aggregate bit-exact against the oracle (owner first, then
     ascending rank), the requantized stripe like any quantize result, and the bytes of the reference's call sequence
@@ -112,7 +112,17 @@ def test_random_stripe_reductions(seed, count, tall):
     heights = [h for h in BOUNDARIES if h <= 14336]
     for n in range(count):
         nbits = int(rng.choice([1, 1, 1, 2, 4, 8, 16, 32]))
-        if tall:
+        if tall == 2:
+            # what no single workgroup holds: the reduction on strips, on one die and (above some 655360 rows) on all
+            nbits = int(rng.choice([1, 1, 2, 4, 8, 16]))
+            least = {1: 102401, 2: 102401, 4: 102401, 8: 65345, 16: 32673}[nbits]
+            most = {1: 1000000, 2: 800000, 4: 500000, 8: 300000, 16: 150000}[nbits]
+            rows = int(rng.choice([least, least + 3, 131072, 200000, 262147, int(rng.integers(least, most))]))
+            rows = max(least, min(most, rows))
+            k = int(rng.choice([1, 2, 3, 5, 8]))
+            cols = int(rng.integers(1, 4))
+            assert qz.StripeReduceTakes(rows, 1, nbits)
+        elif tall:
             # above the LDS kernels' heights: the register kernel of the stripe reduction, up to its limit per bit width
             nbits = int(rng.choice([1, 1, 2, 4, 8, 16]))
             limit = {1: 102368, 2: 102368, 4: 65336, 8: 32668, 16: 16334}[nbits]

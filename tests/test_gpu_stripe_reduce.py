@@ -68,6 +68,10 @@ CASES = [
     (2048, 26, 13, 2, False), (4096, 20, 10, 4, False), (1152, 22, 11, 4, False),
     # six pieces per thread in the table-driven kernels (256 threads: 4100 to 6144 rows, 1024 threads: 16388 to 24576)
     (6144, 16, 8, 1, False), (5000, 16, 8, 1, True), (24576, 8, 8, 1, False), (20000, 6, 12, 1, False),
+    # taller than any workgroup holds: the reduction on strips, several workgroups per column (on one die, and -- the last
+    # case -- on all of them), wherever the call sequence's quantize step runs on strips too
+    (102401, 4, 2, 1, False), (110000, 3, 3, 1, True), (150001, 4, 4, 2, False), (131072, 2, 2, 4, False), (70000, 2, 2, 8, False),
+    (40000, 2, 2, 16, False), (262147, 2, 8, 1, False), (700000, 2, 2, 1, False),
 ]
 
 
@@ -225,6 +229,12 @@ def test_stripe_reduce_height_limit():
     qs = [oracle.quantize(datagen.normal(5 + w, rows, cols), zeros, 16, False)[0] for w in range(k)]
     with pytest.raises(cntk_amd.QuantizerLogicError):
         gpu_stripe_reduce(qz, qs, 0, rows, cols, 16, np.zeros((rows, 1), np.float32, order="F"), False)
+    # Taller stripes are taken where a quantize call on the same shape runs on strips (what no single workgroup holds): the
+    # library says which. Between the two ranges the caller keeps the reference's call sequence.
+    assert qz.StripeReduceTakes(16334, 1, 16) and not qz.StripeReduceTakes(16336, 1, 16) and qz.StripeReduceTakes(40000, 1, 16)
+    assert qz.StripeReduceTakes(102368, 5, 1) and qz.StripeReduceTakes(102401, 5, 1, True) and qz.StripeReduceTakes(1000000, 5, 2)
+    assert not qz.StripeReduceTakes(102369, 5, 1)  # (a height the register kernels still take)
+    assert not qz.StripeReduceTakes(20000, 5, 32) and not qz.StripeReduceTakes(50000000, 1, 1) and not qz.StripeReduceTakes(0, 1, 1)
 
 
 def test_stripe_reduce_32bit_equals_plain_sum():
@@ -361,3 +371,57 @@ def test_config4_shape_one_stripe():
     assert parity.bits_equal(agg, agg_o)
     rep = parity.check_quantize(agg_o, sres, q_new, s_new, nbits, False)
     say("  ", rep)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["f32", "f64"])
+def test_stripe_reduce_on_strips_reports_workgroups_that_give_up(dtype):
+    """A stripe taller than any workgroup holds is reduced by several workgroups per column that wait for each other's
+    partial sums a bounded number of polls. With that number set to zero from the host every wait that does not find its
+    record at the first look gives up: the kernel still runs to its end, such a column is left as it was (output stripe
+    and stripe residual untouched), the wait reports the call as failed, and the handle goes on working afterwards."""
+    # (fewer than 16 strips per column: the first look at the other strips' records then follows a strip's own sum at once)
+    rows, n, k, nbits = (110000 if dtype == torch.float32 else 60000), 3, 2, 1
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    qz = MatrixQuantizerImpl.Create(0, False)
+    assert qz.StripeReduceTakes(rows, n, nbits, False, dtype)
+    zeros = np.zeros((rows, n), npdt, order="F")
+    stripes = [oracle.quantize(datagen.normal(50 + w, rows, n, dtype=npdt), zeros, nbits, False, threads=8)[0] for w in range(k)]
+    sres = datagen.normal(60, rows, n, 0.002, dtype=npdt)
+    agg_o = oracle.unquantize(stripes[0], rows, n, nbits, dtype=npdt, threads=8)
+    oracle.unquantize(stripes[1], rows, n, nbits, out=agg_o, add=True, threads=8)
+    qcol = oracle.qcol_bytes(nbits, rows, npdt)
+
+    def run():
+        Qs = []
+        for w in range(k):
+            Q = QuantizedMatrix(rows, n, nbits, 0, dtype=dtype)
+            Q.from_numpy(stripes[w])
+            Qs.append(Q)
+        S = Matrix.from_numpy(sres)
+        Out = QuantizedMatrix(rows, n, nbits, 0, dtype=dtype)
+        Out.buffer.fill_(0xA5)
+        before = Out.to_numpy()
+        torch.cuda.synchronize()
+        qz.StripeReduceAsync(Qs, 0, S, Out, False)
+        return before, Out, S
+
+    qz._set_strip_spin_limit(0)
+    before, Out, S = run()
+    with pytest.raises(cntk_amd.QuantizerError, match="left as they were"):
+        qz.WaitStripeReduceDone()
+    torch.cuda.synchronize()
+    q_after, s_after = Out.to_numpy(), S.to_numpy()
+    untouched = 0
+    for j in range(n):
+        qa = q_after[j * qcol:(j + 1) * qcol]
+        if np.array_equal(qa, before[j * qcol:(j + 1) * qcol]) and parity.bits_equal(s_after[:, j], sres[:, j]):
+            untouched += 1
+            continue
+        parity.check_quantize(np.asfortranarray(agg_o[:, j:j + 1]), np.asfortranarray(sres[:, j:j + 1]), qa.copy(),
+                              np.asfortranarray(s_after[:, j:j + 1]), nbits, False)
+    say("   columns left untouched: %d of %d" % (untouched, n))
+    assert untouched >= 1
+    qz._set_strip_spin_limit(1 << 17)
+    _, Out, S = run()
+    qz.WaitStripeReduceDone()
+    parity.check_quantize(agg_o, sres, Out.to_numpy(), S.to_numpy(), nbits, False)
