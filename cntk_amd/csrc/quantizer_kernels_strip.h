@@ -107,6 +107,8 @@ struct StripGeom
     uint32_t poll_first; // ... and before the first poll
     double inv_strips;   // for workgroup index -> (column, strip)
     uint32_t spread;     // non-zero: a column's strips take consecutive workgroup indices, i.e. all dies (columns of more strips than one die holds)
+    uint32_t whole_positions; // rows / nq: bit positions at which every QWord of a column has an element
+    uint32_t last_words;      // rows % nq: QWords with an element at bit position whole_positions (none beyond it)
     uint32_t pad;
     uint64_t qcol;
 };
@@ -574,29 +576,36 @@ __device__ __forceinline__ bool strip_assignment(const StripGeom& c, const Strip
     return false;
 }
 
-// which of a thread's PER * SLOTS values exist in a strip at the ragged end of its column
+// which of a thread's PER * SLOTS values exist in a strip at the ragged end of its column: element (QWord q, bit position
+// k) is q + k * nq, so up to bit position whole_positions all of an existing QWord's do, at that one those of the first
+// last_words QWords, beyond it none
 template <int NBITS, typename E>
 __device__ __forceinline__ uint32_t strip_valid_mask(const StripGeom& c, uint32_t w, uint32_t k0)
 {
     using SS = StripShape<NBITS, E>;
-    uint32_t valid = ~(uint32_t) ((1ull << (SS::PER * SS::SLOTS)) - 1ull); // bits beyond the thread's values count as present
+    constexpr uint32_t PER = SS::PER;
+    uint32_t words = 0u, last = 0u;
+#pragma unroll
+    for (uint32_t e = 0; e < PER; ++e)
+    {
+        words |= (w + e < c.nq) ? (1u << e) : 0u;
+        last |= (w + e < c.last_words) ? (1u << e) : 0u;
+    }
+    uint32_t valid = ~(uint32_t) ((1ull << (PER * SS::SLOTS)) - 1ull); // bits beyond the thread's values count as present
 #pragma unroll
     for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
-#pragma unroll
-        for (uint32_t e = 0; e < SS::PER; ++e)
-        {
-            const uint64_t i = (uint64_t) (w + e) + (uint64_t) (k0 + kk) * c.nq;
-            valid |= (w + e < c.nq && i < c.rows) ? (1u << (SS::PER * kk + e)) : 0u;
-        }
+    {
+        const uint32_t k = k0 + kk;
+        valid |= (k < c.whole_positions ? words : (k == c.whole_positions ? last : 0u)) << (PER * kk);
+    }
     return valid;
 }
 
 // The PER consecutive values of a column from element i on (16 bytes at the alignment of an element). FULL: all exist.
-// Otherwise bit e of `ok` says whether value e does, the others read as zero; the 16-byte load never leaves the column (it
-// moves back to the column's last PER elements when it would), and the few lanes with some but not all of their values
-// fetch them one by one.
+// Otherwise bit e of `ok` says whether value e does and the others read as zero: a lane with all of them loads 16 bytes, the
+// few lanes with some fetch them one by one, a lane with none loads nothing.
 template <bool FULL, typename E>
-__device__ __forceinline__ StripVec<E> strip_load(const E* col, uint32_t i, uint32_t rows, uint32_t ok)
+__device__ __forceinline__ StripVec<E> strip_load(const E* col, uint32_t i, uint32_t ok)
 {
     using SE = StripElem<E>;
     constexpr uint32_t PER = SE::PER;
@@ -604,14 +613,13 @@ __device__ __forceinline__ StripVec<E> strip_load(const E* col, uint32_t i, uint
         return __builtin_nontemporal_load(reinterpret_cast<const typename SE::VU*>(col + i));
     else
     {
-        const uint32_t at = (rows >= PER && i + PER > rows) ? rows - PER : i;
         typename SE::V x;
 #pragma unroll
         for (uint32_t e = 0; e < PER; ++e)
             x[e] = 0;
-        if (rows >= PER)
-            x = __builtin_nontemporal_load(reinterpret_cast<const typename SE::VU*>(col + at));
-        if (ok != (1u << PER) - 1u)
+        if (ok == (1u << PER) - 1u)
+            x = __builtin_nontemporal_load(reinterpret_cast<const typename SE::VU*>(col + i));
+        else if (ok != 0u)
         {
 #pragma unroll
             for (uint32_t e = 0; e < PER; ++e)
@@ -636,7 +644,7 @@ __device__ __forceinline__ void quantize_strip_body(const E* g_col, const E* r_c
     StripVec<E> v[SS::SLOTS];
 #pragma unroll
     for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
-        v[kk] = strip_load<FULL, E>(g_col, i0 + kk * c.nq, c.rows, (valid >> (PER * kk)) & ALL);
+        v[kk] = strip_load<FULL, E>(g_col, i0 + kk * c.nq, (valid >> (PER * kk)) & ALL);
     constexpr uint32_t BATCH = SS::SLOTS < 4 ? SS::SLOTS : 4;
 #pragma unroll
     for (uint32_t k1 = 0; k1 < SS::SLOTS; k1 += BATCH)
@@ -644,7 +652,7 @@ __device__ __forceinline__ void quantize_strip_body(const E* g_col, const E* r_c
         StripVec<E> b[BATCH];
 #pragma unroll
         for (uint32_t kk = 0; kk < BATCH; ++kk)
-            b[kk] = strip_load<FULL, E>(r_col, i0 + (k1 + kk) * c.nq, c.rows, (valid >> (PER * (k1 + kk))) & ALL);
+            b[kk] = strip_load<FULL, E>(r_col, i0 + (k1 + kk) * c.nq, (valid >> (PER * (k1 + kk))) & ALL);
 #pragma unroll
         for (uint32_t kk = 0; kk < BATCH; ++kk)
             v[k1 + kk] = v[k1 + kk] + b[kk];
@@ -768,7 +776,7 @@ __device__ __forceinline__ void stripe_reduce_strip_body(const StripeSources& sr
         StripVec<E> b[BATCH];
 #pragma unroll
         for (uint32_t kk = 0; kk < BATCH; ++kk)
-            b[kk] = strip_load<FULL, E>(res_col, i0 + (k1 + kk) * c.nq, c.rows, (valid >> (PER * (k1 + kk))) & ALL);
+            b[kk] = strip_load<FULL, E>(res_col, i0 + (k1 + kk) * c.nq, (valid >> (PER * (k1 + kk))) & ALL);
 #pragma unroll
         for (uint32_t kk = 0; kk < BATCH; ++kk)
             v[k1 + kk] = v[k1 + kk] + b[kk];

@@ -363,6 +363,8 @@ inline StripGeom make_strip_geom(size_t rows, size_t cols, size_t nbits, uint32_
     c.poll_first = c.strips >= kStripFirstPauseMinStrips ? 2u * std::min(c.strips, kStripMaxPerColumn) : 0u;
     c.inv_strips = 1.0 / (double) c.strips;
     c.spread = c.strips > per_die ? 1u : 0u;
+    c.whole_positions = (uint32_t) (rows / c.nq);
+    c.last_words = (uint32_t) (rows % c.nq);
     c.pad = 0;
     c.qcol = (uint64_t) (2 + c.nq) * sizeof(E); // the header's two bounds, then the QWords
     return c;
