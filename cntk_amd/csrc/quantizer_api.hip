@@ -823,7 +823,7 @@ int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_
 {
     if (h == nullptr)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: null handle");
-    if (quantize_path < kPathAuto || quantize_path > kPathStrip)
+    if (quantize_path < kPathAuto || quantize_path > kPathStripPasses)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: unknown quantize path %d", quantize_path);
     if (tile_gs != 0 && (tile_gs < 8 || tile_gs > kTileThreads || (tile_gs & (tile_gs - 1)) != 0))
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_debug_set_tuning: tile_gs must be a power of two in [8, 256]");

@@ -25,6 +25,45 @@ struct StripFor
         }
     };
 
+    // the quantization cut into launches that follow each other on the stream (columns of more strips than the device holds)
+    template <int NBITS, bool ZT>
+    struct PassLauncher
+    {
+        template <int PASS>
+        static hipError_t one(hipStream_t s, hipEvent_t start, hipEvent_t stop, const E* g, const E* r_in, E* r_out, char* q, uint32_t cols,
+                              const StripGeom& c, const StripScratch& scratch)
+        {
+            hipExtLaunchKernelGGL((quantize_strip_kernel<NBITS, ZT, E, PASS>), dim3(strip_grid(cols, c)), dim3(kStripThreads),
+                                  strip_lds_bytes<E>(NBITS), s, start, stop, 0, g, r_in, r_out, q, c, scratch);
+            return hipGetLastError();
+        }
+        static hipError_t run(hipStream_t s, LaunchEvents ev, const E* g, const E* r_in, E* r_out, char* q, uint32_t cols, StripGeom c,
+                              StripScratch scratch)
+        {
+            if constexpr (NBITS >= Word<E>::kBits)
+                return hipErrorInvalidValue;
+            else
+            {
+                hipError_t rc = hipSuccess;
+                hipEvent_t start = ev.start;
+                if constexpr (NBITS != 1 || !ZT)
+                {
+                    rc = one<kStripPassStat>(s, start, nullptr, g, r_in, r_out, q, cols, c, scratch);
+                    start = nullptr;
+                }
+                if constexpr (NBITS == 1)
+                {
+                    if (rc == hipSuccess)
+                        rc = one<kStripPassSplit>(s, start, nullptr, g, r_in, r_out, q, cols, c, scratch);
+                    start = nullptr;
+                }
+                if (rc == hipSuccess)
+                    rc = one<kStripPassPack>(s, start, ev.stop, g, r_in, r_out, q, cols, c, scratch);
+                return rc;
+            }
+        }
+    };
+
     template <int NBITS, bool ZT>
     struct StripeLauncher
     {
@@ -67,6 +106,16 @@ hipError_t family_strip_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEve
 hipError_t family_strip_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, char* q, uint32_t cols, StripGeom c, StripScratch scratch)
 {
     return dispatch_nbits<StripFor<double>::Launcher>(nbits, zt, s, ev, g, r_in, r_out, q, cols, c, scratch);
+}
+
+hipError_t family_strip_quantize_passes(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q, uint32_t cols, StripGeom c, StripScratch scratch)
+{
+    return dispatch_nbits<StripFor<float>::PassLauncher>(nbits, zt, s, ev, g, r_in, r_out, q, cols, c, scratch);
+}
+
+hipError_t family_strip_quantize_passes(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out, char* q, uint32_t cols, StripGeom c, StripScratch scratch)
+{
+    return dispatch_nbits<StripFor<double>::PassLauncher>(nbits, zt, s, ev, g, r_in, r_out, q, cols, c, scratch);
 }
 
 hipError_t family_strip_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out, float* agg_out, uint32_t cols, StripGeom c, StripScratch scratch)

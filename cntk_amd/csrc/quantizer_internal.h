@@ -15,8 +15,10 @@ extern "C" {
  *                        three matrices at the same offset within 16 bytes),
  *                    5 = the same with one element per access: fp32 any alignment, up to 98304 rows; fp64 256 threads per
  *                        column, 1025 to 6144 rows, below 64 bits, the bytes of path 1
- *                    6 = several workgroups per column, a strip of QWords each (fp32, 1 to 16 bits, any height whose
+ *                    6 = several workgroups per column, a strip of QWords each (below 32 (fp64: 64) bits, any height whose
  *                        strips number at most half of what the device holds of the kernel, any alignment)
+ *                    7 = the same in two or three launches, each reading the matrix: any height of two strips or more (the
+ *                        bytes of path 6)
  *   tile_gs          0 = automatic, else threads per column in the tile statistics phase (power of two, 8..256)
  *   unq_slots        0 = automatic, else bit positions decoded per thread by the QWord-major unquantize
  *   unq_mode         0 = automatic, 1 = QWord-major decoder with one store per value, 2 = tile decoder wherever it can run,

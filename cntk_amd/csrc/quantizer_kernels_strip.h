@@ -275,16 +275,26 @@ __device__ __forceinline__ T strip_block_sum(T v, T* red)
 // The column's statistic from the strip's: every workgroup of the column publishes its own and adds all of them in the
 // order of strip_collect. red, red_u: the workgroup's reduction slots (four each). Every thread returns the same bits, in
 // every workgroup of the column.
-template <typename E>
+//
+// PASS: 0 = one kernel does everything and its workgroups wait for each other. Otherwise the work is cut where they would
+// wait, into kernels that run one after the other on a stream (kStripPassStat: publish the statistic and stop;
+// kStripPassSplit: collect the statistics, publish the split sums and stop; kStripPassPack: collect and go on), each
+// loading the strip's values anew: nothing waits, so no workgroup need be resident beside another, and the sums are the
+// same bits as the single kernel's.
+constexpr int kStripPassStat = 1, kStripPassSplit = 2, kStripPassPack = 3;
+
+template <int PASS, typename E>
 __device__ __forceinline__ E strip_exchange_stat(E stat, uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
                                                  const StripScratch& scratch, E* red, uint32_t* red_u, bool& ok)
 {
-    if (c.strips == 1)
+    if (PASS == 0 && c.strips == 1)
         return stat;
     constexpr uint32_t H = sizeof(E) / 4; // records per sum
     uint64_t* recs = scratch.records + (size_t) column * strip_records<E>() * c.strips; // [record][strip]
-    if (threadIdx.x == 0)
+    if (threadIdx.x == 0 && PASS <= kStripPassStat)
         strip_publish_value(recs + strip, c.strips, stat, tag);
+    if constexpr (PASS == kStripPassStat)
+        return stat;
     if (threadIdx.x < 64)
     {
         bool gave_up = false;
@@ -305,20 +315,22 @@ __device__ __forceinline__ E strip_exchange_stat(E stat, uint32_t column, uint32
 }
 
 // the same for the sums on either side of the 1-bit threshold and the count below it
-template <typename E>
+template <int PASS, typename E>
 __device__ __forceinline__ void strip_exchange_split(E& s0, E& s1, uint32_t& n0, uint32_t column, uint32_t strip, uint32_t tag,
                                                      const StripGeom& c, const StripScratch& scratch, E* red, uint32_t* red_u, bool& ok)
 {
-    if (c.strips == 1)
+    if (PASS == 0 && c.strips == 1)
         return;
     constexpr uint32_t H = sizeof(E) / 4;
     uint64_t* recs = scratch.records + (size_t) column * strip_records<E>() * c.strips;
-    if (threadIdx.x == 0)
+    if (threadIdx.x == 0 && PASS != kStripPassPack)
     {
         strip_publish_value(recs + 1 * H * c.strips + strip, c.strips, s0, tag);
         strip_publish_value(recs + 2 * H * c.strips + strip, c.strips, s1, tag);
         strip_publish_value(recs + 3 * H * c.strips + strip, c.strips, n0, tag);
     }
+    if constexpr (PASS == kStripPassSplit)
+        return;
     if (threadIdx.x < 64)
     {
         bool gave_up = false;
@@ -345,32 +357,42 @@ __device__ __forceinline__ void strip_exchange_split(E& s0, E& s1, uint32_t& n0,
 
 // From the strip's sums to the column's header: the exchanges, the header (written by strip 0) and the release of the
 // scratch buffer. `sums(mean, s0, s1, n0)` gives the strip's split sums (1 bit only), in the same bits in every thread.
-// False (in every thread of the workgroup alike): the column was abandoned and nothing of it may be stored.
-template <int NBITS, bool ZT, typename E, typename SplitSums>
+// False (in every thread of the workgroup alike): nothing of the column may be stored, because it was abandoned or because
+// this pass ends with its sums.
+template <int NBITS, bool ZT, int PASS, typename E, typename SplitSums>
 __device__ __forceinline__ bool strip_column_range(E stat, SplitSums sums, uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c,
                                                    const StripScratch& scratch, E* red, uint32_t* red_u, char* qc, E& lo, E& hi)
 {
     constexpr bool need_stat = (NBITS != 1) || !ZT;
+    static_assert(PASS != kStripPassStat || need_stat, "no statistic before the split sums against zero");
+    static_assert(PASS != kStripPassSplit || NBITS == 1, "split sums at 1 bit only");
     E total = 0;
     bool ok = true;
     if constexpr (need_stat)
-        total = strip_exchange_stat(stat, column, strip, tag, c, scratch, red, red_u, ok);
+        total = strip_exchange_stat<PASS>(stat, column, strip, tag, c, scratch, red, red_u, ok);
+    if constexpr (PASS == kStripPassStat)
+        return false;
     if constexpr (NBITS == 1)
     {
         // (an abandoned strip takes no part in the second exchange: its records already say so)
         if (ok)
         {
             const E mean = ZT ? (E) 0 : total / (E) c.rows;
-            E s0, s1;
-            uint32_t n0;
-            sums(mean, s0, s1, n0);
-            strip_exchange_split(s0, s1, n0, column, strip, tag, c, scratch, red, red_u, ok);
+            E s0 = 0, s1 = 0;
+            uint32_t n0 = 0;
+            if constexpr (PASS != kStripPassPack)
+                sums(mean, s0, s1, n0);
+            strip_exchange_split<PASS>(s0, s1, n0, column, strip, tag, c, scratch, red, red_u, ok);
+            if constexpr (PASS == kStripPassSplit)
+                return false;
             finish_stats_1bit<ZT>(mean, s0, s1, n0, c.rows - n0, c.rows, lo, hi);
         }
+        else if (PASS == kStripPassSplit)
+            return false;
     }
     else
         finish_stats_multibit(total, c.rows, lo, hi);
-    if (c.strips > 1 && threadIdx.x == 0)
+    if ((PASS != 0 || c.strips > 1) && threadIdx.x == 0)
         strip_finish(scratch, tag);
     if (ok && strip == 0 && threadIdx.x == 0)
     {
@@ -391,7 +413,7 @@ __device__ __forceinline__ bool strip_column_range(E stat, SplitSums sums, uint3
 template <typename E>
 constexpr uint32_t kStripRedBytes = 4 * sizeof(E) + 16;
 
-template <int NBITS, bool ZT, bool FULL, typename E>
+template <int NBITS, bool ZT, bool FULL, typename E, int PASS = 0>
 __device__ __forceinline__ void strip_stats_pack(StripVec<E>* v, uint32_t valid, uint32_t w, uint32_t k0,
                                                  uint32_t column, uint32_t strip, uint32_t tag, const StripGeom& c, const StripScratch& scratch,
                                                  char* smem, E* res_col, char* qc)
@@ -411,7 +433,7 @@ __device__ __forceinline__ void strip_stats_pack(StripVec<E>* v, uint32_t valid,
             words[x] = 0u;
     }
     E stat = 0;
-    if constexpr ((NBITS != 1) || !ZT)
+    if constexpr (((NBITS != 1) || !ZT) && PASS <= kStripPassStat)
     {
 #pragma unroll
         for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
@@ -424,7 +446,7 @@ __device__ __forceinline__ void strip_stats_pack(StripVec<E>* v, uint32_t valid,
         stat = strip_block_sum(stat, red);
     }
     E lo = 0, hi = 0;
-    const bool column_ok = strip_column_range<NBITS, ZT, E>(
+    const bool column_ok = strip_column_range<NBITS, ZT, PASS, E>(
         stat,
         [&](E mean, E& s0, E& s1, uint32_t& n0) {
             s0 = 0, s1 = 0, n0 = 0;
@@ -447,7 +469,7 @@ __device__ __forceinline__ void strip_stats_pack(StripVec<E>* v, uint32_t valid,
         },
         column, strip, tag, c, scratch, red, red_u, qc, lo, hi);
     if (!column_ok)
-        return; // abandoned column: codes and residual stay as they were
+        return; // abandoned column: codes and residual stay as they were (or a pass that ends with its sums)
     const ValueQOf<E> vq = make_vq<NBITS, E>(lo, hi);
     const E val0 = unquantize_value<NBITS, E>(vq, (Q) 0);
     const E val1 = unquantize_value<NBITS, E>(vq, (Q) 1);
@@ -631,7 +653,7 @@ __device__ __forceinline__ StripVec<E> strip_load(const E* col, uint32_t i, uint
 
 // The gradient goes straight into the registers that will hold the sums, the residual joins it four loads at a time. Every
 // value of the strip is in registers before anything is stored, so r_out may be r_in.
-template <int NBITS, bool ZT, bool FULL, typename E>
+template <int NBITS, bool ZT, bool FULL, typename E, int PASS>
 __device__ __forceinline__ void quantize_strip_body(const E* g_col, const E* r_col, E* res_col, char* qc, uint32_t column, uint32_t strip,
                                                     uint32_t tag, const StripGeom& c, const StripScratch& scratch, char* smem)
 {
@@ -657,10 +679,13 @@ __device__ __forceinline__ void quantize_strip_body(const E* g_col, const E* r_c
         for (uint32_t kk = 0; kk < BATCH; ++kk)
             v[k1 + kk] = v[k1 + kk] + b[kk];
     }
-    strip_stats_pack<NBITS, ZT, FULL, E>(v, valid, w, k0, column, strip, tag, c, scratch, smem, res_col, qc);
+    strip_stats_pack<NBITS, ZT, FULL, E, PASS>(v, valid, w, k0, column, strip, tag, c, scratch, smem, res_col, qc);
 }
 
-template <int NBITS, bool ZT, typename E>
+// PASS 0: the whole quantization in one launch. Otherwise one of the launches it is cut into (kStripPassStat, where the
+// bit width has a statistic; kStripPassSplit, at 1 bit; kStripPassPack), issued in that order on one stream with
+// geometry.spread set: for columns of more strips than the device holds at once.
+template <int NBITS, bool ZT, typename E, int PASS = 0>
 __global__ __launch_bounds__(kStripThreads, (StripShape<NBITS, E>::WAVES)) void quantize_strip_kernel(const E* __restrict__ g, const E* r_in, E* r_out,
                                                                                                     char* __restrict__ q, StripGeom c,
                                                                                                     StripScratch scratch)
@@ -674,9 +699,9 @@ __global__ __launch_bounds__(kStripThreads, (StripShape<NBITS, E>::WAVES)) void 
     const size_t base = (size_t) column * c.rows;
     char* qc = q + (size_t) column * c.qcol;
     if (strip_is_full<NBITS, E>(c, strip))
-        quantize_strip_body<NBITS, ZT, true, E>(g + base, r_in + base, r_out + base, qc, column, strip, tag, c, scratch, smem);
+        quantize_strip_body<NBITS, ZT, true, E, PASS>(g + base, r_in + base, r_out + base, qc, column, strip, tag, c, scratch, smem);
     else
-        quantize_strip_body<NBITS, ZT, false, E>(g + base, r_in + base, r_out + base, qc, column, strip, tag, c, scratch, smem);
+        quantize_strip_body<NBITS, ZT, false, E, PASS>(g + base, r_in + base, r_out + base, qc, column, strip, tag, c, scratch, smem);
 }
 
 // ---- the stripe reduction of the quantized all-reduce on strips: K packed stripes -> sum -> requantize with the stripe

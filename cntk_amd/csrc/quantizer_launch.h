@@ -23,7 +23,8 @@ enum QuantizePath
     kPathCol = 3,     // one workgroup per column, column in LDS: rows a multiple of 4, matrices 16-byte aligned
     kPathReg = 4,     // one workgroup per column, column in registers: same conditions, 1 to 16 bits
     kPathRegScalar = 5, // the same with one float per load and store: any height up to 98304 rows, any alignment, 1 to 16 bits
-    kPathStrip = 6      // several workgroups per column, a strip of QWords with all its bit positions each: any height, any alignment, 1 to 16 bits
+    kPathStrip = 6,     // several workgroups per column, a strip of QWords with all its bit positions each: any height, any alignment, 1 to 16 bits
+    kPathStripPasses = 7 // the same cut into two or three launches that read the matrix once each: columns of more strips than the device holds at once
 };
 
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
@@ -179,6 +180,10 @@ hipError_t family_strip_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEve
 hipError_t family_strip_quantize(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out, char* q,
                                  uint32_t cols, StripGeom c, StripScratch scratch);
 // workgroups of the strip kernel that the runtime says a compute unit holds at once
+hipError_t family_strip_quantize_passes(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const float* g, const float* r_in, float* r_out,
+                                        char* q, uint32_t cols, StripGeom c, StripScratch scratch);
+hipError_t family_strip_quantize_passes(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const double* g, const double* r_in, double* r_out,
+                                        char* q, uint32_t cols, StripGeom c, StripScratch scratch);
 hipError_t family_strip_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const StripeSources& src, float* stripe_res, char* q_out,
                                float* agg_out, uint32_t cols, StripGeom c, StripScratch scratch);
 hipError_t family_strip_stripe(size_t nbits, bool zt, hipStream_t s, LaunchEvents ev, const StripeSources& src, double* stripe_res, char* q_out,
@@ -493,6 +498,18 @@ inline uint32_t strip_max_strips(size_t nbits, bool zt, bool stripe = false)
 
 // Whether the automatic choice may hand this matrix to the strip kernels right now: a column within what the device holds
 // of strips, and a scratch buffer that is there or may be made (a stream under capture cannot wait for a larger one).
+// Whether the strip kernels cut into passes may take this matrix right now: any number of strips (nothing waits, so nothing
+// need be resident together), at least two, a grid the launch can express, and the scratch buffer there or obtainable.
+template <typename E>
+inline bool strip_passes_ready(hipStream_t s, size_t rows, size_t cols, size_t nbits, const LaunchTuning& tune)
+{
+    if (tune.strip == nullptr || nbits >= (size_t) Word<E>::kBits || rows < 1)
+        return false;
+    const size_t strips = (strip_qwords_per_col<E>(rows, nbits) + strip_words<E>(nbits) - 1) / strip_words<E>(nbits);
+    return strips >= 2 && (uint64_t) (cols + kStripDies) * strips <= 0x7FFFFFFFull &&
+           strip_scratch_ready(*tune.strip, s, cols, strips, strip_records<E>(), tune.strip_may_allocate);
+}
+
 template <typename E>
 inline bool strip_ready(hipStream_t s, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune, bool stripe = false)
 {
@@ -507,11 +524,18 @@ inline bool strip_ready(hipStream_t s, size_t rows, size_t cols, size_t nbits, b
 // launch that used it on another stream, then `launch(geometry, scratch)`.
 template <typename E, typename Launch>
 inline hipError_t launch_on_strips(hipStream_t s, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune, bool stripe,
-                                   Launch launch)
+                                   Launch launch, bool passes = false)
 {
-    const StripGeom c = make_strip_geom<E>(rows, cols, nbits, tune.strip_spin_limit, strip_per_die<E>(nbits, zt, stripe));
-    if (!strip_applicable<E>(rows, nbits, tune) || (uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull ||
-        c.strips > strip_max_strips<E>(nbits, zt, stripe))
+    // (in passes: strips side by side in the grid whatever their number, and no pause before a first look that finds everything)
+    StripGeom c = make_strip_geom<E>(rows, cols, nbits, tune.strip_spin_limit, passes ? 0u : strip_per_die<E>(nbits, zt, stripe));
+    if (passes)
+    {
+        c.poll_first = 0;
+        if (tune.strip == nullptr || nbits >= (size_t) Word<E>::kBits || c.strips < 2 || (uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull)
+            return hipErrorInvalidValue;
+    }
+    else if (!strip_applicable<E>(rows, nbits, tune) || (uint64_t) (cols + kStripDies) * c.strips > 0x7FFFFFFFull ||
+             c.strips > strip_max_strips<E>(nbits, zt, stripe))
         return hipErrorInvalidValue;
     StripScratchOwner& o = *tune.strip;
     StripScratch scratch;
@@ -546,6 +570,19 @@ inline hipError_t launch_strip_quantize(hipStream_t s, LaunchEvents ev, const E*
     return launch_on_strips<E>(s, rows, cols, nbits, zt, tune, false, [&](const StripGeom& c, const StripScratch& scratch) {
         return family_strip_quantize(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, scratch);
     });
+}
+
+// ... cut into two or three launches: for columns of more strips than the device holds at once (same bytes)
+template <typename E>
+inline hipError_t launch_strip_quantize_passes(hipStream_t s, LaunchEvents ev, const E* g, const E* r_in, E* r_out, char* qc, size_t rows,
+                                               size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
+{
+    return launch_on_strips<E>(
+        s, rows, cols, nbits, zt, tune, false,
+        [&](const StripGeom& c, const StripScratch& scratch) {
+            return family_strip_quantize_passes(nbits, zt, s, ev, g, r_in, r_out, qc, (uint32_t) cols, c, scratch);
+        },
+        true);
 }
 
 // The fused stripe reduction on strips: for stripes taller than the kernels with a workgroup per column take, where a
@@ -598,6 +635,10 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
         // (a stream under capture cannot wait for a larger scratch buffer: the kernels that need none take the matrix)
         if (path == kPathStrip && !strip_ready<float>(s, rows, cols, nbits, zt, tune))
             path = regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
+        // columns of more strips than the device holds at once: the strips in passes, which read the matrix two or three
+        // times like the kernel with one workgroup per column, but on the whole device
+        if (path == kPathTall && nbits < 32 && strip_passes_ready<float>(s, rows, cols, nbits, tune))
+            path = kPathStripPasses;
     }
     if (path == kPathReg)
     {
@@ -619,6 +660,8 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     }
     if (path == kPathStrip)
         return launch_strip_quantize<float>(s, ev, g, r_in, r_out, qc, rows, cols, nbits, zt, tune);
+    if (path == kPathStripPasses)
+        return launch_strip_quantize_passes<float>(s, ev, g, r_in, r_out, qc, rows, cols, nbits, zt, tune);
     if (path == kPathRegScalar)
     {
         if (!regs_applicable(rows, nbits))

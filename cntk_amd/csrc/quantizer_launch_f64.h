@@ -248,9 +248,14 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* 
         // once, where the device holds all strips of a column at once and the scratch buffer is there or may be made
         if (path == kPathTall && nbits < 64 && strip_ready<double>(s, rows, cols, nbits, zt, tune))
             path = kPathStrip;
+        // ... and of more strips than that: the strips in passes (two or three reads, on the whole device)
+        if (path == kPathTall && nbits < 64 && strip_passes_ready<double>(s, rows, cols, nbits, tune))
+            path = kPathStripPasses;
     }
     if (path == kPathStrip)
         return launch_strip_quantize<double>(s, ev, g, r_in, r_out, qc, rows, cols, nbits, zt, tune);
+    if (path == kPathStripPasses)
+        return launch_strip_quantize_passes<double>(s, ev, g, r_in, r_out, qc, rows, cols, nbits, zt, tune);
     if (path == kPathReg)
     {
         if (!reg_applicable(g, r_in, r_out, rows, nbits))

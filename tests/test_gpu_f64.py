@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 
 F64 = np.float64
 VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False), (64, False)]
-PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG, PATH_REGS, PATH_STRIP = 0, 1, 2, 3, 4, 5, 6
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG, PATH_REGS, PATH_STRIP, PATH_STRIP_PASSES = 0, 1, 2, 3, 4, 5, 6, 7
 
 
 def say(*a):
@@ -148,6 +148,8 @@ PATH_CASES = [
     (1, 3, PATH_STRIP, 0), (37, 5, PATH_STRIP, 0), (1000, 3, PATH_STRIP, 0), (4096, 3, PATH_STRIP, 0), (4097, 2, PATH_STRIP, 0),
     (9304, 3, PATH_STRIP, 0), (16385, 2, PATH_STRIP, 0), (50257, 3, PATH_STRIP, 0), (51201, 2, PATH_AUTO, 0), (102401, 2, PATH_AUTO, 0),
     (200000, 3, PATH_AUTO, 0), (262147, 2, PATH_STRIP, 0), (330001, 1, PATH_AUTO, 0), (400000, 9, PATH_STRIP, 0),
+    # the strips in two or three launches: any height of two strips or more; the automatic choice above what the device holds
+    (9304, 3, PATH_STRIP_PASSES, 0), (51201, 2, PATH_STRIP_PASSES, 0), (3000001, 1, PATH_AUTO, 0),
 ]
 
 
@@ -167,7 +169,8 @@ def test_kernel_paths_f64(case):
         if (path == PATH_REGS and nbits == 64) or \
                 (path == PATH_REG and (nbits == 64 or (48 + oracle.qwords_per_col(rows, nbits, F64)) * 8 > 65536)) or \
                 (path == PATH_STRIP and (nbits == 64 or oracle.qwords_per_col(rows, nbits, F64) >
-                                         qz._strip_max_strips(nbits, zt, torch.float64) * strip_words_f64(nbits))):
+                                         qz._strip_max_strips(nbits, zt, torch.float64) * strip_words_f64(nbits))) or \
+                (path == PATH_STRIP_PASSES and (nbits == 64 or oracle.qwords_per_col(rows, nbits, F64) <= strip_words_f64(nbits))):
             # whole-QWord codes, columns whose QWords exceed 64 KB of LDS and columns of more strips than the device holds at
             # once are refused when forced
             with pytest.raises(cntk_amd.QuantizerLogicError):

@@ -21,7 +21,7 @@ from cntk_amd import Matrix, MatrixQuantizerImpl, QuantizedMatrix
 pytestmark = pytest.mark.gpu
 
 VARIANTS = [(1, False), (1, True), (2, False), (4, False), (8, False), (16, False), (32, False)]
-PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG, PATH_REG_SCALAR, PATH_STRIP = 0, 1, 2, 3, 4, 5, 6
+PATH_AUTO, PATH_TILE, PATH_TALL, PATH_COL, PATH_REG, PATH_REG_SCALAR, PATH_STRIP, PATH_STRIP_PASSES = 0, 1, 2, 3, 4, 5, 6, 7
 
 
 def say(*a):
@@ -142,7 +142,16 @@ PATH_CASES = [
     (9304, 3, PATH_STRIP, 0), (16385, 2, PATH_STRIP, 0), (32768, 2, PATH_STRIP, 0), (50257, 3, PATH_STRIP, 0), (100000, 5, PATH_STRIP, 0),
     (102401, 2, PATH_AUTO, 0), (200000, 3, PATH_AUTO, 0), (262147, 2, PATH_STRIP, 0), (524288, 9, PATH_STRIP, 0), (524289, 1, PATH_AUTO, 0),
     (600000, 9, PATH_STRIP, 0), (655361, 1, PATH_AUTO, 0), (1000003, 1, PATH_AUTO, 0), (1500001, 2, PATH_STRIP, 0),
+    # the strips in two or three launches (nothing waits, nothing need be resident together): any height of two strips or
+    # more, and the automatic choice for columns of more strips than the device holds at once
+    (9304, 3, PATH_STRIP_PASSES, 0), (16385, 2, PATH_STRIP_PASSES, 0), (50257, 3, PATH_STRIP_PASSES, 0), (102401, 2, PATH_STRIP_PASSES, 0),
+    (262147, 2, PATH_STRIP_PASSES, 0), (6000001, 1, PATH_AUTO, 0),
 ]
+
+
+def strip_words(nbits):
+    """QWords of a float column that one strip holds."""
+    return 256 if nbits == 1 else 512 if nbits == 2 else 1024
 
 
 @pytest.mark.parametrize("case", PATH_CASES, ids=["%dx%d_p%d_g%d" % c for c in PATH_CASES])
@@ -152,9 +161,10 @@ def test_kernel_paths(case):
     rep = parity.Report()
     for nbits, zt in VARIANTS:
         say("path case", case, "nbits", nbits, "zeroThr", zt)
-        if path == PATH_STRIP and (nbits == 32 or oracle.qwords_per_col(rows, nbits) >
-                                   qz._strip_max_strips(nbits, zt) * (256 if nbits == 1 else 512 if nbits == 2 else 1024)):
-            # whole-QWord codes need no assembling, and a column's strips must fit on one die of the device together
+        if (path == PATH_STRIP and (nbits == 32 or oracle.qwords_per_col(rows, nbits) > qz._strip_max_strips(nbits, zt) * strip_words(nbits))) or \
+                (path == PATH_STRIP_PASSES and (nbits == 32 or oracle.qwords_per_col(rows, nbits) <= strip_words(nbits))):
+            # whole-QWord codes need no assembling, a column's strips must be resident on the device together, and a single
+            # strip has nothing to cut into passes
             qz._set_tuning(quantize_path=path)
             with pytest.raises(cntk_amd.QuantizerLogicError):
                 gpu_quantize(qz, datagen.normal(1, rows, cols), np.zeros((rows, cols), np.float32, order="F"), nbits, zt)
@@ -176,6 +186,32 @@ def test_kernel_paths(case):
             return a
         run_chain(qz, rows, cols, nbits, zt, make, 2, rep)
     say("  ", rep)
+
+
+@pytest.mark.parametrize("rows,cols", [(9000, 7), (150001, 5), (262144, 3)])
+def test_strips_in_passes_give_the_strip_kernels_bytes(rows, cols):
+    """The strip kernel cut into launches at the points where its workgroups would wait for each other adds the same
+    partial sums in the same order: packed bytes and residuals are identical, for floats and doubles."""
+    qz = MatrixQuantizerImpl.Create(0, False)
+    for dtype, npdt in ((torch.float32, np.float32), (torch.float64, np.float64)):
+        g, r = datagen.normal_with_outliers(rows, rows, cols, 0.01, dtype=npdt), datagen.normal(rows + 1, rows, cols, 0.002, dtype=npdt)
+        for nbits, zt in VARIANTS:
+            per_strip = (64 // nbits if npdt == np.float64 else 32 // nbits) * (strip_words(nbits) if npdt == np.float32 else
+                                                                                 {1: 64, 2: 128, 4: 256}.get(nbits, 512))
+            if nbits == 32 or rows <= per_strip:
+                continue
+            say("strips in one launch and in passes", rows, cols, npdt.__name__, nbits, zt)
+            outs = []
+            for path in (PATH_STRIP, PATH_STRIP_PASSES):
+                qz._set_tuning(quantize_path=path)
+                G, R = Matrix.from_numpy(g), Matrix.from_numpy(r)
+                Q = QuantizedMatrix(rows, cols, nbits, 0, dtype=dtype)
+                qz.QuantizeAsync(G, R, Q, R, zt)
+                qz.WaitQuantizeAsyncDone()
+                torch.cuda.synchronize()
+                outs.append((Q.to_numpy(), R.to_numpy()))
+            assert np.array_equal(outs[0][0], outs[1][0]) and parity.bits_equal(outs[0][1], outs[1][1])
+        qz._set_tuning(quantize_path=PATH_AUTO)
 
 
 @pytest.mark.parametrize("rows", [2048, 4100, 9304, 14336])
