@@ -103,7 +103,7 @@ def test_config1_512x512_single_step():
 
 # ---- config 2 ----------------------------------------------------------------------------------------
 
-# columns (of 12 checked steps x 23,656) allowed to rest on the float64 bounds instead of the oracle's
+# columns (of 27 checked steps x 23,656) allowed to rest on the float64 bounds instead of the oracle's
 CONFIG2_FALLBACK_COLS = 0
 
 SPEECH_DNN = [(429, 2048)] + [(2048, 2048)] * 6 + [(2048, 9304)] + [(2048, 1)] * 7 + [(9304, 1)]
@@ -122,7 +122,7 @@ def test_config2_speech_dnn_100_steps(zt):
             say("config 2 zeroThr", zt, "step", step)
         for ch in chains:
             G = device_student_t3(gen, ch.rows, ch.cols, 1e-3)
-            ch.step(G, step < 2 or step % 10 == 9, rep)  # the oracle sees steps 0, 1, 9, 19 ... 99
+            ch.step(G, step < 2 or step % 4 == 3, rep)  # the oracle sees steps 0, 1, 3, 7, 11 ... 99
     say("config 2:", rep)
     rep.assert_fallback_at_most(CONFIG2_FALLBACK_COLS)
 
@@ -238,7 +238,7 @@ def test_config4_allreduce_full_shape():
 
 # ---- config 5 ----------------------------------------------------------------------------------------
 
-# of 4 checked steps x 116,896 columns
+# of 11 checked steps x 116,896 columns
 CONFIG5_FALLBACK_COLS = 8
 
 LSTM_LM = [(100000, 512, 0.9), (1024, 4096, 0.0), (1024, 4096, 0.0), (1024, 4096, 0.0), (1024, 4096, 0.0),
@@ -260,7 +260,7 @@ def test_config5_lstm_lm_zero_threshold_20_steps():
                 # a different 90% of the columns is silent at every step
                 keep = (torch.rand(c, generator=gen, device="cuda:0") >= zero_frac).to(torch.float32)
                 G.data.view(c, r).mul_(keep[:, None])
-            ch.step(G, step < 2 or step % 10 == 9, rep)  # the oracle sees steps 0, 1, 9, 19
+            ch.step(G, step < 2 or step % 2 == 1, rep)  # the oracle sees steps 0, 1, 3, 5 ... 19
     say("config 5:", rep)
     # only the 100000-row embedding columns that received a gradient (about 51 of 512 per step) are long enough for the
     # oracle's own fp32 sum to use up the tolerance
