@@ -336,9 +336,12 @@ public:
     {
         const size_t K = NumProc();
         const bool fused = m_options.useFusedStripeReduce && m_useQuantizationForSelfStripe;
-        // stripes too tall for the fused call keep the reference's sequence of calls
-        const size_t fusedMaxRows = detail::Abi<ElemType>::StripeReduceMaxRows(m_numQuantizationBits);
-        auto fusable = [&](size_t i) { return fused && gradients[i]->GetNumRows() <= fusedMaxRows; };
+        // stripes that the fused call does not take keep the reference's sequence of calls
+        auto fusable = [&](size_t i) {
+            const size_t stripeCols = GetStripeForNode(gradients[i]->GetNumCols(), MyRank(), K).m_numCols;
+            return fused && stripeCols != 0 &&
+                   Gpu(*m_aggGradStripeQuantizers[i]).StripeReduceTakes(gradients[i]->GetNumRows(), stripeCols, m_numQuantizationBits, m_zeroThresholdFor1Bit);
+        };
         if (m_options.traceLevel >= kDebugOutputTraceLevel)
             for (size_t i = 0; i < gradients.size(); ++i)
                 for (size_t w = 0; w < K; ++w)

@@ -61,6 +61,10 @@ struct Abi<float>
     typedef uint32_t QWord;
     static size_t QColBytes(size_t bits, size_t rows) { return cntkq_qcol_bytes(bits, rows); }
     static size_t StripeReduceMaxRows(size_t bits) { return cntkq_stripe_reduce_max_rows(bits); }
+    static bool StripeReduceTakes(cntkq_quantizer* h, size_t rows, size_t cols, size_t bits, int zt)
+    {
+        return cntkq_stripe_reduce_takes(h, rows, cols, bits, zt) != 0;
+    }
     static int Quantize(cntkq_quantizer* h, const float* in, const float* resIn, size_t rows, size_t cols, void* q, size_t qBytes, int onHost,
                         size_t bits, float* resOut, int zt)
     {
@@ -103,6 +107,10 @@ struct Abi<double>
     typedef uint64_t QWord;
     static size_t QColBytes(size_t bits, size_t rows) { return cntkq_qcol_bytes_f64(bits, rows); }
     static size_t StripeReduceMaxRows(size_t bits) { return cntkq_stripe_reduce_max_rows_f64(bits); }
+    static bool StripeReduceTakes(cntkq_quantizer* h, size_t rows, size_t cols, size_t bits, int zt)
+    {
+        return cntkq_stripe_reduce_takes_f64(h, rows, cols, bits, zt) != 0;
+    }
     static int Quantize(cntkq_quantizer* h, const double* in, const double* resIn, size_t rows, size_t cols, void* q, size_t qBytes,
                         int onHost, size_t bits, double* resOut, int zt)
     {
@@ -538,6 +546,13 @@ public:
             raw.push_back(typename detail::Abi<ElemType>::UnquantizeItem{it.inQMatrix->Buffer(), it.outMatrix->Data(), it.outMatrix->GetNumRows(), it.outMatrix->GetNumCols(), it.inQMatrix->GetSize()});
         }
         detail::Check(detail::Abi<ElemType>::UnquantizeBatch(m_handle, raw.data(), raw.size(), nbits, add ? 1 : 0));
+    }
+
+    // Whether StripeReduceAsync takes stripes of this shape on this quantizer; where not, the caller keeps the reference's
+    // sequence of UnquantizeAsync ... QuantizeAsync calls (Source/1BitSGD/AllReduceDistGradAggregator.h:365-436).
+    bool StripeReduceTakes(size_t numRows, size_t numStripeCols, size_t nbits, bool zeroThresholdFor1Bit) const
+    {
+        return detail::Abi<ElemType>::StripeReduceTakes(m_handle, numRows, numStripeCols, nbits, zeroThresholdFor1Bit ? 1 : 0);
     }
 
     // Fused stripe reduction of the quantized all-reduce (dataflow of Source/1BitSGD/AllReduceDistGradAggregator.h:365-436):

@@ -281,7 +281,6 @@ private:
     void ReduceOwnStripesT(Call& call, StripeTransportT<ElemType>& transport, State<ElemType>& st)
     {
         const size_t K = NumWorkers();
-        const size_t fusedMaxRows = detail::Abi<ElemType>::StripeReduceMaxRows(m_numQuantizationBits);
         for (size_t i = 0; i < call.inValues.size(); ++i)
         {
             const auto stripe = AllReduceDistGradAggregator<ElemType>::GetStripeForNode(call.inValues[i]->GetNumCols(), m_rank, K);
@@ -291,7 +290,9 @@ private:
             QuantizedMatrix<ElemType> ownSlice = st.quantizedGradients[i]->ColumnSlice(stripe.m_startCol, stripe.m_numCols);
             Matrix<ElemType>& inStripeResidue = *call.stripeResidues[i]->template GetWritableMatrix<ElemType>();
             Matrix<ElemType>& outStripeResidue = *call.newStripeResidues[i]->template GetWritableMatrix<ElemType>();
-            const bool fused = m_options.useFusedStripeReduce && m_useQuantizationForSelfStripe && call.inValues[i]->GetNumRows() <= fusedMaxRows;
+            const bool fused = m_options.useFusedStripeReduce && m_useQuantizationForSelfStripe &&
+                               Gpu(stripeQuantizer).StripeReduceTakes(call.inValues[i]->GetNumRows(), stripe.m_numCols, m_numQuantizationBits,
+                                                                      m_zeroThresholdFor1Bit);
             if (fused)
             {
                 // the fused call updates one residue in place: distinct buffers get the input's contents first

@@ -144,8 +144,10 @@ static RunResult Run(const Shapes& shapes, size_t K, int nBits, bool zeroThr, bo
 
 static void VariantsAreBitIdentical()
 {
-    // (14340 rows: too tall for the fused stripe reduction, which then keeps the reference's call sequence for that matrix)
-    const Shapes shapes = {{2048, 40}, {429, 37}, {64, 5}, {576, 24}, {1, 9}, {33, 3}, {14340, 6}};
+    // (14340 rows: the stripe reduction's register kernel; 110000 rows: taller than any workgroup holds, quantized and reduced
+    // by several workgroups per column -- fused where the library says it takes the stripe, else by the reference's call
+    // sequence, and a cluster with such a matrix issues its calls worker by worker)
+    const Shapes shapes = {{2048, 40}, {429, 37}, {64, 5}, {576, 24}, {1, 9}, {33, 3}, {14340, 6}, {110000, 5}};
     const size_t K = 4;
     for (int nBits : {1, 4})
         for (bool zeroThr : {false, true})
