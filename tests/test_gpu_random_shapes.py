@@ -24,14 +24,15 @@ def say(*a):
     sys.stdout.flush()
 
 
-TALL = [102401, 110000, 131072, 131073, 147456, 200000, 262144, 262145, 300001, 524288, 524289, 600000, 655361, 700001, 1048577]
+TALL = [102401, 110000, 131072, 131073, 147456, 200000, 262144, 262145, 300001, 524288, 524289, 600000, 655361, 700001, 1048577, 2800001,
+        6000001]
 
 
 def draw_case(rng, is64, tall=False):
     r = rng.random()
     if tall:
         # above what one workgroup holds: strips of a column on several workgroups (on one die, or on all), then the
-        # kernel that re-reads its column
+        # same strips in several launches
         rows = int(rng.choice(TALL)) if r < 0.6 else int(rng.integers(102401, 540000))
     elif r < 0.5:
         rows = int(rng.choice(BOUNDARIES))
