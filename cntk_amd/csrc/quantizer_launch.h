@@ -267,7 +267,7 @@ inline RegGeom make_reg_geom(size_t rows, size_t nbits, uint32_t threads, bool l
 
 // The register kernels: above 1024 rows (unless forced; 37.7 M elements at 1152 / 1536 / 2000 rows: 95 / 76 / 72 us against
 // 102 / 81 / 80 us with the LDS column kernels, the same bytes), up to 25 pieces for each of
-// 1024 threads, the column's QWords within 64 KB of LDS. 256 threads up to the height the stripe reduction handles (whose
+// 1024 threads, the column's QWords in LDS (reg_lds_fits). 256 threads up to the height the stripe reduction handles (whose
 // LDS kernels then sum in the same order), 1024 above.
 constexpr uint32_t kRegMinRows = 1024;
 constexpr uint32_t kRegMaxRows = 4 * 1024 * 25;
@@ -275,6 +275,16 @@ constexpr uint32_t kRegMaxRows = 4 * 1024 * 25;
 inline uint32_t reg_threads(size_t rows)
 {
     return rows <= kTileMaxRows ? 256u : 1024u;
+}
+
+// LDS of the register kernels: a workgroup may have all 160 KB of its compute unit. The quantize kernels keep the column's
+// QWords there, the fused stripe reduction the output QWords and at least one worker's packed record: both families take
+// the heights at which the latter fits, so that every stripe whose quantize step runs in registers can be reduced in
+// registers too.
+constexpr size_t kRegMaxLdsBytes = 160 * 1024;
+inline bool reg_lds_fits(size_t rows, size_t nbits)
+{
+    return ((size_t) kRegRedSlots + 2 * qwords_per_col(rows, nbits) + 2) * 4 <= kRegMaxLdsBytes;
 }
 
 inline bool reg_applicable(const float* g, const float* r_in, const float* r_out, const void* q, size_t rows, size_t nbits,
@@ -285,7 +295,7 @@ inline bool reg_applicable(const float* g, const float* r_in, const float* r_out
         return false;
     if (!forced && rows <= kRegMinRows)
         return false;
-    return (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
+    return reg_lds_fits(rows, nbits);
 }
 
 // The piece-wise register kernel with edge elements: matrices only 4-byte aligned, any height from 8 rows on. The aligned
@@ -300,7 +310,7 @@ inline bool reg_edge_applicable(const float* g, const float* r_in, const float* 
     (void) r_out;
     if (rows < 8 || rows > kRegMaxRows - 32 || nbits >= 32 || (reinterpret_cast<uintptr_t>(q) & 3u) != 0)
         return false;
-    return (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
+    return reg_lds_fits(rows, nbits);
 }
 
 // Matrices that are not whole aligned pieces (odd heights, slices at a 4-byte offset) above kRegEdge256MinRows rows: the
@@ -325,7 +335,7 @@ constexpr uint32_t kRegsMaxRows = 1024 * 96;
 
 inline bool regs_applicable(size_t rows, size_t nbits)
 {
-    return rows >= 1 && rows <= kRegsMaxRows && nbits < 32 && (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 <= 64 * 1024;
+    return rows >= 1 && rows <= kRegsMaxRows && nbits < 32 && reg_lds_fits(rows, nbits);
 }
 
 // ---- strip kernels: any height, several workgroups per column ------------------------------------------------------
@@ -700,7 +710,7 @@ inline size_t stripe_reduce_max_rows(size_t nbits)
 {
     if (nbits >= 32)
         return kTileMaxRows;
-    const size_t max_nq = (64 * 1024 / 4 - kRegRedSlots - 2) / 2;
+    const size_t max_nq = (kRegMaxLdsBytes / 4 - kRegRedSlots - 2) / 2;
     const size_t by_lds = max_nq * (32 / nbits);
     const size_t by_regs = kRegMaxRows - 32;
     const size_t tall = by_lds < by_regs ? by_lds : by_regs;
@@ -711,7 +721,7 @@ inline size_t stripe_reduce_max_rows(size_t nbits)
 // choice of a quantize call is the strip kernels (or, without them, the kernel that re-reads its columns).
 inline bool strip_only_height(size_t rows, size_t nbits)
 {
-    return nbits < 32 && rows > kTileMaxRows && (rows > kRegMaxRows || (kRegRedSlots + qwords_per_col(rows, nbits)) * 4 > 64 * 1024);
+    return nbits < 32 && rows > kTileMaxRows && (rows > kRegMaxRows || !reg_lds_fits(rows, nbits));
 }
 
 // Whether the fused stripe reduction takes a stripe taller than stripe_reduce_max_rows: on strips, where a quantize call

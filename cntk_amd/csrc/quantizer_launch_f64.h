@@ -9,6 +9,9 @@ namespace f64 {
 
 constexpr uint32_t kTileMaxRows = 7168; // 56 KB of LDS for a one-column tile of doubles
 constexpr size_t kMaxLdsBytes = 64 * 1024;
+// the register kernels may have all of a compute unit's LDS; quantize and fused stripe reduction take the same heights (see
+// reg_lds_fits of the float kernels)
+constexpr size_t kRegMaxLdsBytes = 160 * 1024;
 
 inline bool valid_nbits(size_t nbits)
 {
@@ -124,7 +127,7 @@ inline bool reg_applicable(const double* g, const double* r_in, const double* r_
     (void) r_out;
     if (rows < 4 || rows > kRegMaxRows - 16 || nbits >= 64)
         return false;
-    return (kRegRedSlots + qwords_per_col(rows, nbits)) * 8 <= kMaxLdsBytes;
+    return ((size_t) kRegRedSlots + 2 * qwords_per_col(rows, nbits) + 2) * 8 <= kRegMaxLdsBytes;
 }
 
 // Slots are dealt by 128-byte lines where some column of the residual starts inside one and the registers allow it. Only
@@ -326,7 +329,7 @@ inline bool stripe_uses_reg(size_t rows, size_t nbits)
 {
     if (rows < kRegMinRows || rows > kRegMaxRows - 16 || nbits >= 64)
         return false;
-    return ((size_t) kRegRedSlots + 2 * qwords_per_col(rows, nbits) + 2) * 8 <= kMaxLdsBytes;
+    return ((size_t) kRegRedSlots + 2 * qwords_per_col(rows, nbits) + 2) * 8 <= kRegMaxLdsBytes;
 }
 
 // Tallest column the fused stripe reduction takes at this bit width.
@@ -334,7 +337,7 @@ inline size_t stripe_reduce_max_rows(size_t nbits)
 {
     if (nbits >= 64)
         return kTileMaxRows;
-    const size_t max_nq = (kMaxLdsBytes / 8 - kRegRedSlots - 2) / 2;
+    const size_t max_nq = (kRegMaxLdsBytes / 8 - kRegRedSlots - 2) / 2;
     const size_t by_lds = max_nq * (64 / nbits);
     const size_t by_regs = kRegMaxRows - 16;
     const size_t tall = by_lds < by_regs ? by_lds : by_regs;

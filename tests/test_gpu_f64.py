@@ -167,12 +167,12 @@ def test_kernel_paths_f64(case):
     for nbits, zt in VARIANTS:
         say("f64 path case", case, "nbits", nbits, "zeroThr", zt)
         if (path == PATH_REGS and nbits == 64) or \
-                (path == PATH_REG and (nbits == 64 or (48 + oracle.qwords_per_col(rows, nbits, F64)) * 8 > 65536)) or \
+                (path == PATH_REG and (nbits == 64 or (50 + 2 * oracle.qwords_per_col(rows, nbits, F64)) * 8 > 163840)) or \
                 (path == PATH_STRIP and (nbits == 64 or oracle.qwords_per_col(rows, nbits, F64) >
                                          qz._strip_max_strips(nbits, zt, torch.float64) * strip_words_f64(nbits))) or \
                 (path == PATH_STRIP_PASSES and (nbits == 64 or oracle.qwords_per_col(rows, nbits, F64) <= strip_words_f64(nbits))):
-            # whole-QWord codes, columns whose QWords exceed 64 KB of LDS and columns of more strips than the device holds at
-            # once are refused when forced
+            # whole-QWord codes, columns whose QWords (twice, as the stripe reduction keeps them) exceed the LDS of a compute unit
+            # and columns of more strips than the device holds at once are refused when forced
             with pytest.raises(cntk_amd.QuantizerLogicError):
                 gpu_quantize(qz, datagen.normal(1, rows, cols, dtype=F64), zeros(rows, cols), nbits, zt)
             continue
@@ -366,7 +366,9 @@ def stripe_max_rows_f64(nbits):
 @pytest.mark.parametrize("rows,n,k", [(70, 9, 3), (429, 12, 4), (2048, 20, 8), (4096, 3, 2), (4988, 3, 3), (4992, 3, 3), (5003, 2, 2),
                                       (6144, 2, 3), (6145, 2, 2), (6148, 3, 3), (7168, 2, 5), (64, 40, 64), (8000, 2, 3), (20001, 2, 2), (51184, 1, 2),
                                       # on strips: the heights that no single workgroup holds
-                                      (51201, 2, 2), (102401, 2, 3), (330001, 1, 2)])
+                                      (51201, 2, 2), (102401, 2, 3), (330001, 1, 2),
+                                      # the register kernel's tallest stripes at 16 and 32 bits (all of a compute unit's LDS)
+                                      (40860, 2, 2), (20430, 2, 3)])
 def test_stripe_reduce_f64(quantizer, rows, n, k):
     for nbits, zt in VARIANTS:
         if not quantizer.StripeReduceTakes(rows, n, nbits, zt, torch.float64):
@@ -525,12 +527,13 @@ def test_stripe_batch_equals_per_matrix_calls_f64(quantizer, nbits, zt, k):
 def test_stripe_reduce_height_limit_f64(quantizer):
     """The limit the library reports per bit width is the tallest column the fused call takes."""
     assert stripe_max_rows_f64(64) == 7168 and stripe_max_rows_f64(1) == 51184 and stripe_max_rows_f64(3) == 0
-    assert stripe_max_rows_f64(16) == 16284 and stripe_max_rows_f64(32) == 8142 and stripe_max_rows_f64(8) == 32568
-    rows, n, k = 16286, 2, 2
-    Qs = [QuantizedMatrix(rows, n, 16, 0, dtype=torch.float64) for _ in range(k)]
+    assert stripe_max_rows_f64(16) == 40860 and stripe_max_rows_f64(32) == 20430 and stripe_max_rows_f64(8) == 51184
+    rows, n, k = 7170, 2, 2  # (codes as wide as a QWord: the tile kernels' heights only)
+    Qs = [QuantizedMatrix(rows, n, 64, 0, dtype=torch.float64) for _ in range(k)]
     S = Matrix(rows, n, dtype=torch.float64)
-    with pytest.raises(cntk_amd.QuantizerLogicError, match="up to 16284 rows"):
+    with pytest.raises(cntk_amd.QuantizerLogicError, match="up to 7168 rows"):
         quantizer.StripeReduceAsync(Qs, 0, S, Qs[0], False)
     takes = lambda rows, nbits: quantizer.StripeReduceTakes(rows, 2, nbits, False, torch.float64)
-    assert takes(16284, 16) and not takes(16286, 16) and takes(40000, 16)  # (up to 32576 rows the register kernel quantizes)
+    # (the register kernels quantize and reduce the same heights; whatever is taller goes to the strips, both of them)
+    assert takes(40860, 16) and takes(40862, 16) and takes(20430, 32) and takes(20432, 32)
     assert takes(51184, 1) and takes(51185, 1) and takes(400000, 4) and not takes(20000, 64) and not takes(50000000, 1)

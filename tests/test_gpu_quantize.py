@@ -169,8 +169,9 @@ def test_kernel_paths(case):
             with pytest.raises(cntk_amd.QuantizerLogicError):
                 gpu_quantize(qz, datagen.normal(1, rows, cols), np.zeros((rows, cols), np.float32, order="F"), nbits, zt)
             continue
-        if path in (PATH_REG, PATH_REG_SCALAR) and (nbits == 32 or (48 + oracle.qwords_per_col(rows, nbits)) * 4 > 65536):
-            # whole-QWord codes and columns whose QWords exceed 64 KB of LDS are not the register kernels' business
+        if path in (PATH_REG, PATH_REG_SCALAR) and (nbits == 32 or (50 + 2 * oracle.qwords_per_col(rows, nbits)) * 4 > 163840):
+            # whole-QWord codes and columns whose QWords (twice, as the stripe reduction keeps them) exceed the LDS of a compute
+            # unit are not the register kernels' business
             qz._set_tuning(quantize_path=path)
             with pytest.raises(cntk_amd.QuantizerLogicError):
                 gpu_quantize(qz, datagen.normal(1, rows, cols), np.zeros((rows, cols), np.float32, order="F"), nbits, zt)

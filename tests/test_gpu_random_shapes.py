@@ -116,7 +116,7 @@ def test_random_stripe_reductions(seed, count, tall):
         if tall == 2:
             # what no single workgroup holds: the reduction on strips, on one die and (above some 655360 rows) on all
             nbits = int(rng.choice([1, 1, 2, 4, 8, 16]))
-            least = {1: 102401, 2: 102401, 4: 102401, 8: 65345, 16: 32673}[nbits]
+            least = {1: 102401, 2: 102401, 4: 102401, 8: 81821, 16: 40911}[nbits]
             most = {1: 1000000, 2: 800000, 4: 500000, 8: 300000, 16: 150000}[nbits]
             rows = int(rng.choice([least, least + 3, 131072, 200000, 262147, int(rng.integers(least, most))]))
             rows = max(least, min(most, rows))
@@ -126,8 +126,8 @@ def test_random_stripe_reductions(seed, count, tall):
         elif tall:
             # above the LDS kernels' heights: the register kernel of the stripe reduction, up to its limit per bit width
             nbits = int(rng.choice([1, 1, 2, 4, 8, 16]))
-            limit = {1: 102368, 2: 102368, 4: 65336, 8: 32668, 16: 16334}[nbits]
-            rows = int(rng.choice([14337, 14340, 16334, 20000, 32668, 50257, 65536, 102368, int(rng.integers(14337, 102369))]))
+            limit = {1: 102368, 2: 102368, 4: 102368, 8: 81820, 16: 40910}[nbits]
+            rows = int(rng.choice([14337, 14340, 16334, 20000, 32668, 40910, 50257, 65536, 81820, 102368, int(rng.integers(14337, 102369))]))
             rows = max(14337, min(limit, rows + int(rng.choice([0, 0, -1, 1, 2]))))
             k = int(rng.choice([1, 2, 3, 5, 8]))
             cols = int(rng.integers(1, max(2, min(8, 240000 // rows)) + 1))

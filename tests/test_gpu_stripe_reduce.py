@@ -56,7 +56,8 @@ CASES = [
     (9304, 6, 4, 1, False), (8192, 4, 3, 4, False), (12000, 4, 5, 2, False), (14336, 2, 2, 8, False),
     # above 14336 rows: the register kernel's shape (the running sum in registers, one worker's record at a time in LDS)
     (14340, 6, 4, 1, False), (14337, 3, 2, 2, False), (20000, 5, 3, 1, True), (32768, 4, 5, 4, False), (50257, 3, 8, 1, False),
-    (100000, 2, 2, 1, False), (102365, 2, 3, 2, False), (16332, 2, 2, 16, False), (32668, 2, 2, 8, False),
+    (100000, 2, 2, 1, False), (102365, 2, 3, 2, False), (16332, 2, 2, 16, False), (32668, 2, 2, 8, False), (40910, 2, 2, 16, False),
+    (81820, 2, 3, 8, False), (100000, 2, 2, 4, False),
     # heights that are not a multiple of 4: the tile kernels up to 2048 rows, above them the register kernels with edge
     # elements (256 threads per column up to 7168 rows, 1024 above)
     (1023, 6, 3, 1, False), (1025, 6, 3, 1, False), (2049, 8, 8, 1, False), (2050, 5, 2, 1, True), (4097, 4, 3, 4, False), (6001, 3, 5, 2, False),
@@ -70,8 +71,8 @@ CASES = [
     (6144, 16, 8, 1, False), (5000, 16, 8, 1, True), (24576, 8, 8, 1, False), (20000, 6, 12, 1, False),
     # taller than any workgroup holds: the reduction on strips, several workgroups per column (on one die, and -- the last
     # case -- on all of them), wherever the call sequence's quantize step runs on strips too
-    (102401, 4, 2, 1, False), (110000, 3, 3, 1, True), (150001, 4, 4, 2, False), (131072, 2, 2, 4, False), (70000, 2, 2, 8, False),
-    (40000, 2, 2, 16, False), (262147, 2, 8, 1, False), (700000, 2, 2, 1, False),
+    (102401, 4, 2, 1, False), (110000, 3, 3, 1, True), (150001, 4, 4, 2, False), (131072, 2, 2, 4, False), (81822, 2, 2, 8, False),
+    (40912, 2, 2, 16, False), (90000, 2, 2, 16, False), (262147, 2, 8, 1, False), (700000, 2, 2, 1, False),
 ]
 
 
@@ -215,23 +216,23 @@ def test_stripe_residual_at_4_byte_offsets(rows, off, batched):
 
 
 def test_stripe_reduce_height_limit():
-    """The tallest stripe the fused call takes depends on the bit width (its LDS holds the output QWords and one worker's
-    record); taller ones are refused, and the limit can be asked for."""
+    """The tallest stripe the fused call takes with one workgroup per column depends on the bit width (its LDS holds the
+    output QWords and one worker's record); the limit can be asked for, and so can whether a taller stripe is taken."""
     L = cntk_amd.lib()
     L.cntkq_stripe_reduce_max_rows.restype = ctypes.c_size_t
     L.cntkq_stripe_reduce_max_rows.argtypes = [ctypes.c_size_t]
     assert L.cntkq_stripe_reduce_max_rows(1) == 102368 and L.cntkq_stripe_reduce_max_rows(32) == 14336
-    assert L.cntkq_stripe_reduce_max_rows(16) == 16334 and L.cntkq_stripe_reduce_max_rows(8) == 32668 and L.cntkq_stripe_reduce_max_rows(3) == 0
-    assert L.cntkq_stripe_reduce_max_rows(4) == 65336 and L.cntkq_stripe_reduce_max_rows(2) == 102368
+    assert L.cntkq_stripe_reduce_max_rows(16) == 40910 and L.cntkq_stripe_reduce_max_rows(8) == 81820 and L.cntkq_stripe_reduce_max_rows(3) == 0
+    assert L.cntkq_stripe_reduce_max_rows(4) == 102368 and L.cntkq_stripe_reduce_max_rows(2) == 102368
     qz = MatrixQuantizerImpl.Create(0, False)
-    rows, cols, k = 16336, 2, 2
+    rows, cols, k = 14340, 2, 2  # (codes as wide as a QWord: the LDS kernels' heights only)
     zeros = np.zeros((rows, cols), np.float32, order="F")
-    qs = [oracle.quantize(datagen.normal(5 + w, rows, cols), zeros, 16, False)[0] for w in range(k)]
+    qs = [oracle.quantize(datagen.normal(5 + w, rows, cols), zeros, 32, False)[0] for w in range(k)]
     with pytest.raises(cntk_amd.QuantizerLogicError):
-        gpu_stripe_reduce(qz, qs, 0, rows, cols, 16, np.zeros((rows, 1), np.float32, order="F"), False)
+        gpu_stripe_reduce(qz, qs, 0, rows, cols, 32, np.zeros((rows, 1), np.float32, order="F"), False)
     # Taller stripes are taken where a quantize call on the same shape runs on strips (what no single workgroup holds): the
-    # library says which. Between the two ranges the caller keeps the reference's call sequence.
-    assert qz.StripeReduceTakes(16334, 1, 16) and not qz.StripeReduceTakes(16336, 1, 16) and qz.StripeReduceTakes(40000, 1, 16)
+    # library says which. (Between 102369 and 102400 rows a quantize call still runs in registers: the call sequence.)
+    assert qz.StripeReduceTakes(40910, 1, 16) and qz.StripeReduceTakes(40912, 1, 16) and qz.StripeReduceTakes(81822, 1, 8)
     assert qz.StripeReduceTakes(102368, 5, 1) and qz.StripeReduceTakes(102401, 5, 1, True) and qz.StripeReduceTakes(1000000, 5, 2)
     assert not qz.StripeReduceTakes(102369, 5, 1)  # (a height the register kernels still take)
     assert not qz.StripeReduceTakes(20000, 5, 32) and not qz.StripeReduceTakes(50000000, 1, 1) and not qz.StripeReduceTakes(0, 1, 1)
