@@ -96,14 +96,16 @@ def test_stripe_batch_equals_per_matrix_calls(nbits, zt, k):
     """One call for the stripe reductions of a whole gradient set gives the bytes of one call per matrix."""
     qz = MatrixQuantizerImpl.Create(0, False)
     owner = k // 2
+    # (and a stripe that no single workgroup holds: a launch of its own, on strips)
+    sets = STRIPE_SETS + ([(110000, 2)] if nbits < 32 else [])
     z = lambda r, c: np.zeros((r, c), np.float32, order="F")
     packed = [[oracle.quantize(datagen.normal(50 * i + 7 * w + nbits, r, c), z(r, c), nbits, zt, threads=8)[0] if r and c else
-               np.zeros(0, np.uint8) for w in range(k)] for i, (r, c) in enumerate(STRIPE_SETS)]
-    sres = [datagen.normal(900 + i, r, c, 0.003) for i, (r, c) in enumerate(STRIPE_SETS)]
+               np.zeros(0, np.uint8) for w in range(k)] for i, (r, c) in enumerate(sets)]
+    sres = [datagen.normal(900 + i, r, c, 0.003) for i, (r, c) in enumerate(sets)]
 
     def device_state():
         Qs = []
-        for i, (r, c) in enumerate(STRIPE_SETS):
+        for i, (r, c) in enumerate(sets):
             row = []
             for w in range(k):
                 Q = QuantizedMatrix(r, c, nbits, 0)
@@ -111,26 +113,26 @@ def test_stripe_batch_equals_per_matrix_calls(nbits, zt, k):
                     Q.from_numpy(packed[i][w])
                 row.append(Q)
             Qs.append(row)
-        return Qs, [Matrix.from_numpy(s) for s in sres], [Matrix(r, c) for r, c in STRIPE_SETS]
+        return Qs, [Matrix.from_numpy(s) for s in sres], [Matrix(r, c) for r, c in sets]
 
     for step in range(2):  # the second step finds the cached table only if the buffers are the same: build fresh ones once
         Q1, S1, A1 = device_state()
-        for i in range(len(STRIPE_SETS)):
+        for i in range(len(sets)):
             qz.StripeReduceAsync(Q1[i], owner, S1[i], Q1[i][owner], zt, agg_out=A1[i])
         qz.WaitStripeReduceDone()
         Q2, S2, A2 = device_state()
-        items = [(Q2[i], S2[i], Q2[i][owner], A2[i]) for i in range(len(STRIPE_SETS))]
+        items = [(Q2[i], S2[i], Q2[i][owner], A2[i]) for i in range(len(sets))]
         qz.StripeReduceBatchAsync(items, owner, zt)
         qz.StripeReduceBatchAsync(items, owner, zt)  # again on its own output: same table, new stripe residuals
         qz.WaitStripeReduceDone()
-        for i in range(len(STRIPE_SETS)):
+        for i in range(len(sets)):
             qz.StripeReduceAsync(Q1[i], owner, S1[i], Q1[i][owner], zt, agg_out=A1[i])
         qz.WaitStripeReduceDone()
         torch.cuda.synchronize()
-        for i, (r, c) in enumerate(STRIPE_SETS):
-            assert np.array_equal(Q1[i][owner].to_numpy(), Q2[i][owner].to_numpy()), ("packed", STRIPE_SETS[i])
-            assert parity.bits_equal(S1[i].to_numpy(), S2[i].to_numpy()), ("stripe residual", STRIPE_SETS[i])
-            assert parity.bits_equal(A1[i].to_numpy(), A2[i].to_numpy()), ("aggregate", STRIPE_SETS[i])
+        for i, (r, c) in enumerate(sets):
+            assert np.array_equal(Q1[i][owner].to_numpy(), Q2[i][owner].to_numpy()), ("packed", sets[i])
+            assert parity.bits_equal(S1[i].to_numpy(), S2[i].to_numpy()), ("stripe residual", sets[i])
+            assert parity.bits_equal(A1[i].to_numpy(), A2[i].to_numpy()), ("aggregate", sets[i])
     say("stripe batch", nbits, zt, k, "ok")
 
 

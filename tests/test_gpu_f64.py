@@ -485,13 +485,15 @@ STRIPE_SETS64 = [(147, 8), (64, 16), (576, 9), (1, 5), (429, 7), (2048, 12), (46
 def test_stripe_batch_equals_per_matrix_calls_f64(quantizer, nbits, zt, k):
     qz = quantizer
     owner = k // 2
+    # (and a stripe that no single workgroup holds: a launch of its own, on strips)
+    sets = STRIPE_SETS64 + ([(60000, 2)] if nbits < 64 else [])
     packed = [[oracle.quantize(datagen.normal(50 * i + 7 * w + nbits, r, c, dtype=F64), zeros(r, c), nbits, zt, threads=8)[0] if r and c
-               else np.zeros(0, np.uint8) for w in range(k)] for i, (r, c) in enumerate(STRIPE_SETS64)]
-    sres = [datagen.normal(900 + i, r, c, 0.003, dtype=F64) for i, (r, c) in enumerate(STRIPE_SETS64)]
+               else np.zeros(0, np.uint8) for w in range(k)] for i, (r, c) in enumerate(sets)]
+    sres = [datagen.normal(900 + i, r, c, 0.003, dtype=F64) for i, (r, c) in enumerate(sets)]
 
     def device_state():
         Qs = []
-        for i, (r, c) in enumerate(STRIPE_SETS64):
+        for i, (r, c) in enumerate(sets):
             row = []
             for w in range(k):
                 Q = QuantizedMatrix(r, c, nbits, 0, dtype=torch.float64)
@@ -499,29 +501,29 @@ def test_stripe_batch_equals_per_matrix_calls_f64(quantizer, nbits, zt, k):
                     Q.from_numpy(packed[i][w])
                 row.append(Q)
             Qs.append(row)
-        return Qs, [Matrix.from_numpy(s) for s in sres], [Matrix(r, c, dtype=torch.float64) for r, c in STRIPE_SETS64]
+        return Qs, [Matrix.from_numpy(s) for s in sres], [Matrix(r, c, dtype=torch.float64) for r, c in sets]
 
     Q1, S1, A1 = device_state()
-    for i in range(len(STRIPE_SETS64)):
-        if STRIPE_SETS64[i][0]:
+    for i in range(len(sets)):
+        if sets[i][0]:
             qz.StripeReduceAsync(Q1[i], owner, S1[i], Q1[i][owner], zt, agg_out=A1[i])
     qz.WaitStripeReduceDone()
     Q2, S2, A2 = device_state()
     for rep in range(2):  # the second call finds the cached table
         if rep == 1:
-            for i, (r, c) in enumerate(STRIPE_SETS64):
+            for i, (r, c) in enumerate(sets):
                 S2[i].data.copy_(Matrix.from_numpy(sres[i]).data)
                 if r and c:
                     Q2[i][owner].from_numpy(packed[i][owner])
-        qz.StripeReduceBatchAsync([(Q2[i], S2[i], Q2[i][owner], A2[i]) for i in range(len(STRIPE_SETS64))], owner, zt)
+        qz.StripeReduceBatchAsync([(Q2[i], S2[i], Q2[i][owner], A2[i]) for i in range(len(sets))], owner, zt)
         qz.WaitStripeReduceDone()
         torch.cuda.synchronize()
-        for i, (r, c) in enumerate(STRIPE_SETS64):
+        for i, (r, c) in enumerate(sets):
             if r == 0:
                 continue
-            assert np.array_equal(Q1[i][owner].to_numpy(), Q2[i][owner].to_numpy()), ("packed", STRIPE_SETS64[i])
-            assert parity.bits_equal(S1[i].to_numpy(), S2[i].to_numpy()), ("stripe residual", STRIPE_SETS64[i])
-            assert parity.bits_equal(A1[i].to_numpy(), A2[i].to_numpy()), ("aggregate", STRIPE_SETS64[i])
+            assert np.array_equal(Q1[i][owner].to_numpy(), Q2[i][owner].to_numpy()), ("packed", sets[i])
+            assert parity.bits_equal(S1[i].to_numpy(), S2[i].to_numpy()), ("stripe residual", sets[i])
+            assert parity.bits_equal(A1[i].to_numpy(), A2[i].to_numpy()), ("aggregate", sets[i])
 
 
 def test_stripe_reduce_height_limit_f64(quantizer):
