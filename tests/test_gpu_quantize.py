@@ -567,11 +567,12 @@ def test_calls_replayed_from_a_hip_graph(rows, cols, nbits):
         assert torch.equal(graphed.stripes[owner].buffer, eager.stripes[owner].buffer), "replay %d: reduced stripe differs" % step
 
 
-@pytest.mark.parametrize("rows,cols,nbits", [(150001, 3, 1), (120000, 2, 4)])
+@pytest.mark.parametrize("rows,cols,nbits", [(150001, 3, 1), (120000, 2, 4), (6000001, 1, 1)])
 def test_strip_kernel_replayed_from_a_hip_graph(rows, cols, nbits):
     """Columns taller than any workgroup holds are cut into strips whose workgroups exchange partial sums through a
     scratch buffer that carries a launch count from one launch to the next. A captured launch must find that state
-    right at every replay, with eager launches of the same and of another shape in between, and give the eager bytes."""
+    right at every replay, with eager launches of the same and of another shape in between, and give the eager bytes.
+    (The tallest case has more strips than the device holds at once: three launches, recorded as three kernel nodes.)"""
     qz = MatrixQuantizerImpl.Create(0, False)
     other_rows = 110000
     graphed = (Matrix(rows, cols), Matrix(rows, cols), QuantizedMatrix(rows, cols, nbits, 0))
