@@ -113,6 +113,7 @@ def lib():
         L.cntkq_debug_strip_max_strips_f64.argtypes = [_vp, _sz, ctypes.c_int]
         L.cntkq_debug_strip_max_strips_f64.restype = ctypes.c_uint
         L.cntkq_set_force_sync.argtypes = [_vp, ctypes.c_int]
+        L.cntkq_set_tall_columns_never_wait.argtypes = [_vp, ctypes.c_int]
         _lib = L
     return _lib
 
@@ -497,6 +498,11 @@ class MatrixQuantizerImpl:
         _check(_fn("cntkq_stripe_reduce_async", out_qstripe.dtype)(self._h, arr, k, owner, rows, cols, nbits, stripe_residual.Data(),
                                                out_qstripe.Buffer(), agg_out.Data() if agg_out is not None else None,
                                                int(bool(zero_threshold_for_1bit))))
+
+    def SetTallColumnsNeverWait(self, never_wait):
+        """Columns taller than one workgroup holds: several launches whose workgroups never wait for each other instead of one
+        launch whose workgroups do (for handles whose stream shares the device with other work)."""
+        _check(lib().cntkq_set_tall_columns_never_wait(self._h, int(bool(never_wait))))
 
     def StripeReduceTakes(self, rows, cols, nbits, zero_threshold_for_1bit=False, dtype=torch.float32):
         """Whether StripeReduceAsync takes stripes of this shape; where not, the caller runs the reference's sequence of

@@ -475,6 +475,10 @@ public:
     }
     ~MatrixQuantizerGPU() override { (void) cntkq_destroy(m_handle); }
 
+    // No counterpart in the reference: columns taller than one workgroup holds as several launches whose workgroups never wait
+    // for one another, instead of one launch whose workgroups do (for quantizers whose stream shares the device with other work).
+    void SetTallColumnsNeverWait(bool neverWait) { detail::Check(cntkq_set_tall_columns_never_wait(m_handle, neverWait ? 1 : 0)); }
+
     void QuantizeAsync(const Matrix<ElemType>& inMatrix, const Matrix<ElemType>& inResidual, QuantizedMatrix<ElemType>& outQMatrix,
                        Matrix<ElemType>& outResidual, bool zeroThresholdFor1Bit) override
     {

@@ -115,6 +115,7 @@ struct BatchAbi<float>
     {
         LaunchTuning autotune;
         autotune.strip = &h->strip_scratch;
+        autotune.strip_never_waits = h->tune.strip_never_waits;
         return launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune);
     }
 
@@ -488,6 +489,7 @@ int quantize_batch_noalloc_impl(cntkq_quantizer* h, const cntkq_quantize_item* i
         LaunchTuning fixed;
         fixed.strip = h->strip_scratch.order_event != nullptr ? &h->strip_scratch : nullptr;
         fixed.strip_may_allocate = false;
+        fixed.strip_never_waits = h->tune.strip_never_waits;
         HIP_TRY(launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, fixed), "quantize kernel launch failed");
     }
     h->last_quantize = done;
@@ -690,6 +692,14 @@ int cntkq_set_force_sync(cntkq_quantizer* h, int force_sync)
     if (h == nullptr)
         return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_set_force_sync: null handle");
     h->force_sync = force_sync != 0;
+    return CNTKQ_OK;
+}
+
+int cntkq_set_tall_columns_never_wait(cntkq_quantizer* h, int never_wait)
+{
+    if (h == nullptr)
+        return fail(CNTKQ_INVALID_ARGUMENT, "cntkq_set_tall_columns_never_wait: null handle");
+    h->tune.strip_never_waits = never_wait != 0;
     return CNTKQ_OK;
 }
 

@@ -78,6 +78,7 @@ struct BatchAbi<double>
     {
         LaunchTuning autotune;
         autotune.strip = &h->strip_scratch;
+        autotune.strip_never_waits = h->tune.strip_never_waits;
         return f64::launch_quantize(s, ev, it.in, it.res_in, it.res_out, it.qbuf, it.rows, it.cols, nbits, zt, autotune);
     }
 

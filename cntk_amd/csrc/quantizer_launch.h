@@ -61,6 +61,7 @@ struct LaunchTuning
     StripScratchOwner* strip = nullptr; // null: the strip kernels are not available to this launch
     uint32_t strip_spin_limit = 1u << 17; // polls of a partial sum (two microseconds or so each) before a lane gives up
     bool strip_may_allocate = true; // false: the strip kernels only where the scratch buffer as it stands holds the launch
+    bool strip_never_waits = false; // true: tall columns take the strips in passes, whose workgroups never wait for one another
     int quantize_path = kPathAuto;
     uint32_t tile_gs = 0;   // 0 = pick from rows; else threads per column (power of two, 8..256)
     int tile_stage = -1;    // -1 = automatic; 0 / 1 = residual written straight to memory / staged through LDS
@@ -643,7 +644,7 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const float* g
     {
         path = quantize_auto_path(g, r_in, r_out, q, rows, nbits, strip_applicable<float>(rows, nbits, tune));
         // (a stream under capture cannot wait for a larger scratch buffer: the kernels that need none take the matrix)
-        if (path == kPathStrip && !strip_ready<float>(s, rows, cols, nbits, zt, tune))
+        if (path == kPathStrip && (tune.strip_never_waits || !strip_ready<float>(s, rows, cols, nbits, zt, tune)))
             path = regs_applicable(rows, nbits) ? kPathRegScalar : kPathTall;
         // columns of more strips than the device holds at once: the strips in passes, which read the matrix two or three
         // times like the kernel with one workgroup per column, but on the whole device
@@ -729,7 +730,7 @@ inline bool strip_only_height(size_t rows, size_t nbits)
 inline bool stripe_takes_strips(hipStream_t s, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
 {
     zt = zt && nbits == 1;
-    return strip_only_height(rows, nbits) && strip_ready<float>(s, rows, cols, nbits, zt, tune, false) &&
+    return !tune.strip_never_waits && strip_only_height(rows, nbits) && strip_ready<float>(s, rows, cols, nbits, zt, tune, false) &&
            strip_ready<float>(s, rows, cols, nbits, zt, tune, true);
 }
 

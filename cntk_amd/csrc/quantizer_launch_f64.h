@@ -249,7 +249,7 @@ inline hipError_t launch_quantize(hipStream_t s, LaunchEvents ev, const double* 
         path = quantize_auto_path(g, r_in, r_out, rows, nbits);
         // columns that no workgroup's registers hold: strips of the column on several workgroups, which read their inputs
         // once, where the device holds all strips of a column at once and the scratch buffer is there or may be made
-        if (path == kPathTall && nbits < 64 && strip_ready<double>(s, rows, cols, nbits, zt, tune))
+        if (path == kPathTall && nbits < 64 && !tune.strip_never_waits && strip_ready<double>(s, rows, cols, nbits, zt, tune))
             path = kPathStrip;
         // ... and of more strips than that: the strips in passes (two or three reads, on the whole device)
         if (path == kPathTall && nbits < 64 && strip_passes_ready<double>(s, rows, cols, nbits, tune))
@@ -359,7 +359,7 @@ inline bool strip_only_height(size_t rows, size_t nbits)
 inline bool stripe_takes_strips(hipStream_t s, size_t rows, size_t cols, size_t nbits, bool zt, const LaunchTuning& tune)
 {
     zt = zt && nbits == 1;
-    return strip_only_height(rows, nbits) && strip_ready<double>(s, rows, cols, nbits, zt, tune, false) &&
+    return !tune.strip_never_waits && strip_only_height(rows, nbits) && strip_ready<double>(s, rows, cols, nbits, zt, tune, false) &&
            strip_ready<double>(s, rows, cols, nbits, zt, tune, true);
 }
 

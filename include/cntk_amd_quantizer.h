@@ -107,6 +107,16 @@ int cntkq_set_main_stream(cntkq_quantizer* h, void* hip_stream);
  * Off by default. Calls recorded into a graph ignore it. */
 int cntkq_set_force_sync(cntkq_quantizer* h, int force_sync);
 
+/* No counterpart in the reference. Columns taller than one workgroup holds (above 102400 rows; doubles 51184) are cut into
+ * strips on several workgroups, which by default run as ONE launch whose workgroups wait for each other's partial sums:
+ * gradient and residual are read once, but all strips of a column must be running on the device together, which other work
+ * on the device at the same time (a training step's kernels on another stream) can prevent -- such a column is then left
+ * untouched and the next wait reports it. With never_wait set, the handle runs the strips as two or three launches that
+ * read the matrix once each instead: about 1.6 times the time, the same bytes, and no workgroup ever waits for another;
+ * cntkq_stripe_reduce_takes then answers 0 for such heights (the caller's sequence of calls, whose QuantizeAsync step runs in
+ * those launches). Off by default. */
+int cntkq_set_tall_columns_never_wait(cntkq_quantizer* h, int never_wait);
+
 /* MatrixComputeStreamEvent::Create + SynchronizeQuantizationComputeStreamWithEvent
  * (Source/Math/MatrixQuantizerImpl.h:53-72, Source/Math/MatrixQuantizerGPU.cu:347-371): work issued on the
  * handle's stream after this call starts only after everything already issued on the main stream. */

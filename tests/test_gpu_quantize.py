@@ -215,6 +215,43 @@ def test_strips_in_passes_give_the_strip_kernels_bytes(rows, cols):
         qz._set_tuning(quantize_path=PATH_AUTO)
 
 
+def test_tall_columns_that_never_wait():
+    """A handle told that its tall columns must never wait runs them as the strips in passes (the bytes of the single launch),
+    keeps doing so for the tall member of a batched call, and no longer offers the fused reduction of tall stripes."""
+    rows, cols = 150001, 4
+    a, b = MatrixQuantizerImpl.Create(0, False), MatrixQuantizerImpl.Create(0, False)
+    b.SetTallColumnsNeverWait(True)
+    assert a.StripeReduceTakes(rows, cols, 1) and not b.StripeReduceTakes(rows, cols, 1) and b.StripeReduceTakes(9304, cols, 1)
+    g, r = datagen.normal_with_outliers(3, rows, cols, 0.01), datagen.normal(4, rows, cols, 0.002)
+    small = datagen.normal(5, 2048, 6)
+    outs = []
+    for qz in (a, b):
+        G, R, Q = Matrix.from_numpy(g), Matrix.from_numpy(r), QuantizedMatrix(rows, cols, 1, 0)
+        qz.QuantizeAsync(G, R, Q, R, False)
+        qz.WaitQuantizeAsyncDone()
+        G2, R2, Q2 = Matrix.from_numpy(g), Matrix.from_numpy(r), QuantizedMatrix(rows, cols, 1, 0)
+        S, RS, QS = Matrix.from_numpy(small), Matrix(2048, 6), QuantizedMatrix(2048, 6, 1, 0)
+        S3, RS3, QS3 = Matrix.from_numpy(small), Matrix(2048, 6), QuantizedMatrix(2048, 6, 1, 0)
+        qz.QuantizeBatchAsync([(G2, R2, Q2, R2), (S, RS, QS, RS), (S3, RS3, QS3, RS3)], False)
+        qz.WaitQuantizeAsyncDone()
+        torch.cuda.synchronize()
+        assert np.array_equal(Q.to_numpy(), Q2.to_numpy()) and parity.bits_equal(R.to_numpy(), R2.to_numpy())
+        outs.append((Q.to_numpy(), R.to_numpy()))
+    assert np.array_equal(outs[0][0], outs[1][0]) and parity.bits_equal(outs[0][1], outs[1][1])
+    parity.check_quantize(g, r, outs[1][0], outs[1][1], 1, False)
+    # with no patience at all for another workgroup's partial sum (every wait that does not find its record at the first
+    # look gives up) the launches that never wait still give the right bytes
+    b._set_strip_spin_limit(0)
+    G, R, Q = Matrix.from_numpy(g), Matrix.from_numpy(r), QuantizedMatrix(rows, cols, 1, 0)
+    b.QuantizeAsync(G, R, Q, R, False)
+    b.WaitQuantizeAsyncDone()
+    torch.cuda.synchronize()
+    assert np.array_equal(Q.to_numpy(), outs[0][0]) and parity.bits_equal(R.to_numpy(), outs[0][1])
+    b._set_strip_spin_limit(1 << 17)
+    b.SetTallColumnsNeverWait(False)
+    assert b.StripeReduceTakes(rows, cols, 1)
+
+
 @pytest.mark.parametrize("rows", [2048, 4100, 9304, 14336])
 def test_register_and_lds_column_kernels_give_the_same_bytes(rows):
     """Up to 14336 rows the register kernels sum the column statistics in the order of the LDS kernels (which the
