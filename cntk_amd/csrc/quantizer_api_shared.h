@@ -211,6 +211,26 @@ inline LaunchEvents take_events(cntkq_quantizer* h, hipEvent_t own)
     return ev;
 }
 
+// The same for a call of several launches (the gradient-set calls): the first launch starts the one event, the last ends
+// the other. Nothing is attached to launches that are only recorded into a graph.
+struct AttachedEvents
+{
+    hipEvent_t start = nullptr;
+    hipEvent_t stop = nullptr;
+};
+inline AttachedEvents take_attached(cntkq_quantizer* h, bool capturing)
+{
+    AttachedEvents a;
+    if (!capturing)
+    {
+        a.start = h->attach_start;
+        a.stop = h->attach_stop;
+    }
+    h->attach_start = nullptr;
+    h->attach_stop = nullptr;
+    return a;
+}
+
 // Temp device buffer for a host-resident packed matrix (GetTempGPUQuantizedMatrix,
 // Source/Math/MatrixQuantizerGPU.cu:158-179). Grows only; waits for everything that may still use the old one.
 inline int ensure_staging(cntkq_quantizer* h, size_t bytes)

@@ -42,7 +42,8 @@ unsigned cntkq_debug_strip_max_strips_f64(cntkq_quantizer* h, size_t nbits, int 
 /* Ties caller-owned hipEvent_t objects (either may be NULL) to the NEXT kernel this handle launches: start_event is
  * set when that kernel begins, stop_event when it has finished, by the dispatch itself. Used to time single kernels
  * without putting extra commands into the stream. The stop event also becomes what the matching Wait call waits on,
- * so it must stay alive until then. */
+ * so it must stay alive until then. With a gradient-set call next: start_event at its first launch, stop_event at its
+ * last, and the call's own completion event recorded on the stream behind that. */
 int cntkq_debug_attach_events(cntkq_quantizer* h, void* start_event, void* stop_event);
 
 #ifdef __cplusplus
