@@ -669,7 +669,9 @@ def test_strip_kernel_reports_workgroups_that_give_up(host_q):
     end, the column is left as it was (packed column and in-place residual untouched, so the error feedback survives),
     the next wait reports the call as failed -- also where the packed matrix lives in host memory and the wait is for
     the copy -- and the handle goes on working afterwards."""
-    rows, cols = 130000, 4
+    # (14 strips per column: below 16 a strip looks for the others' records the moment it has published its own, and the
+    # first one of a column to do so cannot find them)
+    rows, cols = 110000, 4
     qz = MatrixQuantizerImpl.Create(0, False)
     g = datagen.normal(5, rows, cols)
     r0 = datagen.normal(6, rows, cols, 0.002)
@@ -734,6 +736,20 @@ def test_strip_kernel_beside_other_work_on_the_device():
         else:
             parity.check_quantize(g, r0, Q.to_numpy(), R.to_numpy(), nbits, False)
     say("   launches that reported strips giving up: %d of 3" % reported)
+    # told that its tall columns must never wait, the same handle beside the same work cannot fail that way
+    qz.SetTallColumnsNeverWait(True)
+    for rep in range(2):
+        R = Matrix.from_numpy(r0)
+        Q = QuantizedMatrix(rows, cols, nbits, 0)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            for i in range(6):
+                big.fill_(float(i))
+                big2.copy_(big)
+        qz.QuantizeAsync(G, R, Q, R, False)
+        qz.WaitQuantizeAsyncDone()
+        torch.cuda.synchronize()
+        parity.check_quantize(g, r0, Q.to_numpy(), R.to_numpy(), nbits, False)
 
 
 def test_strip_scratch_outgrown_after_a_recorded_launch():
