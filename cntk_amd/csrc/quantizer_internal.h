@@ -35,7 +35,7 @@ int cntkq_debug_set_strip_spin_limit(cntkq_quantizer* h, unsigned limit);
 /* The most strips per column that the strip kernels (path 6) take on the handle's device at this bit width: half of what
  * the device holds of the kernel, as the runtime's occupancy query tells (a column of more strips than half a die holds
  * has them on all eight dies), never more than 8 x 128 (0: unknown, or no strip kernel for the bit width). A strip is
- * 256 / 512 / 1024 QWords at 1 / 2 / 4 and more bits; of a double matrix 64 / 128 / 256 / 512 at 1 / 2 / 4 / 8 and more. */
+ * 512 / 1024 / 2048 QWords at 1 / 2 / 4 and more bits; of a double matrix 128 / 256 / 512 / 1024 at 1 / 2 / 4 / 8 and more. */
 unsigned cntkq_debug_strip_max_strips(cntkq_quantizer* h, size_t nbits, int zero_threshold_for_1bit);
 unsigned cntkq_debug_strip_max_strips_f64(cntkq_quantizer* h, size_t nbits, int zero_threshold_for_1bit);
 

@@ -2,15 +2,17 @@
 //
 // A column of `rows` elements is packed into nq QWords, element i in QWord i % nq at bit position i / nq. A strip is a run
 // of W consecutive QWords with ALL their bit positions: 32 / NBITS runs of W consecutive elements, nq elements apart. One
-// 256-thread workgroup owns one strip: a thread holds the elements of 16 bytes' worth of consecutive QWords (four of a
+// 512-thread workgroup owns one strip: a thread holds the elements of 16 bytes' worth of consecutive QWords (four of a
 // float column, two of a double column) at up to eight bit positions (eight 16-byte loads of gradient and residual, at
 // any alignment the element type allows), builds its part of those QWords and writes the residual back from registers;
 // the parts of a QWord meet in LDS. The kernels are written once over the element type. Gradient and residual are read once whatever
 // the height, which columns above 102400 rows -- more than any workgroup's registers hold -- could otherwise only have by
-// reading their inputs two or three times. A strip needs 1 to 4 KB of LDS and, at 1 to 4 bits, some 100 registers (its 32
-// values, their addresses, the masks of the ragged last strip), so five workgroups share a CU; it is the exchange
-// described next, not memory, that bounds the kernel (3.3 to 4.4 TB/s), and below 102400 rows the kernels with one workgroup
-// per column are faster.
+// reading their inputs two or three times. A strip needs 2 to 8 KB of LDS and, at 1 to 4 bits, some 100 registers (its 32
+// values, their addresses, the masks of the ragged last strip), so two workgroups share a CU; it is the exchange
+// described next, not memory, that bounds the kernel (3.7 to 4.8 TB/s), and below 102400 rows the kernels with one workgroup
+// per column are faster. (Strips of 256 threads, five to a CU, were 7 to 25 % slower, strips of 1024 threads about as fast
+// as these at a few shapes and slower at most: the fewer workgroups a column's sums must cross, the better, until too few
+// bytes are in flight.)
 //
 // The column statistics span the strips of a column. Every workgroup publishes its partial sums in a scratch buffer, one
 // 8-byte record per 32 bits of a sum (a double takes two): the bits and the tag of the launch, written by one atomic store,
@@ -39,7 +41,8 @@
 
 namespace cntkq {
 
-constexpr uint32_t kStripThreads = 256;
+constexpr uint32_t kStripThreads = 512;
+constexpr uint32_t kStripWaves = kStripThreads / 64;
 constexpr uint32_t kStripDies = 8; // accelerator dies that take the workgroups of a grid in turn
 
 typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
@@ -80,11 +83,12 @@ struct StripShape
     static constexpr uint32_t SLOTS = PS::SLOTS;                  // bit positions per thread
     static constexpr uint32_t CHUNKS = PS::CHUNKS;                // threads per run of PER QWords
     static constexpr uint32_t RUNS = kStripThreads / CHUNKS;      // runs of PER QWords per strip
-    // QWords per strip: float 256, 512, 1024, 1024, 1024 at 1, 2, 4, 8, 16 bits; double 64, 128, 256, 512, 512, 512 at 1 ... 32 bits
+    // QWords per strip: float 512, 1024, 2048, 2048, 2048 at 1, 2, 4, 8, 16 bits; double 128, 256, 512, 1024, 1024, 1024 at 1 ... 32 bits
     static constexpr uint32_t WORDS = PER * RUNS;
-    // wavefronts per SIMD the kernels are compiled for (the registers that leaves them: 96 at 5, 64 at 8); with more where a
-    // thread holds eight bit positions the ragged last strip spills, and every strip of its column waits for it
-    static constexpr uint32_t WAVES = SLOTS == 8 ? 5 : 8;
+    // wavefronts per SIMD the kernels are compiled for (the registers that leaves them: 128 at 4, 64 at 8): two workgroups of
+    // eight wavefronts are what a compute unit holds where a thread has eight bit positions, and with fewer registers the
+    // ragged last strip spills, and every strip of its column waits for it
+    static constexpr uint32_t WAVES = SLOTS == 8 ? 4 : 8;
 };
 
 // how many QWords a strip holds at this bit width (host side; the same arithmetic as StripShape)
@@ -267,7 +271,10 @@ __device__ __forceinline__ T strip_block_sum(T v, T* red)
     if ((threadIdx.x & 63u) == 0)
         red[threadIdx.x >> 6] = v;
     __syncthreads();
-    const T t = ((red[0] + red[1]) + red[2]) + red[3];
+    T t = red[0];
+#pragma unroll
+    for (uint32_t i = 1; i < kStripWaves; ++i)
+        t = t + red[i];
     __syncthreads();
     return t;
 }
@@ -411,7 +418,7 @@ __device__ __forceinline__ bool strip_column_range(E stat, SplitSums sums, uint3
 // has several threads. Used by the quantize and the stripe-reduction kernel, which therefore give the same bytes for the
 // same column.
 template <typename E>
-constexpr uint32_t kStripRedBytes = 4 * sizeof(E) + 16;
+constexpr uint32_t kStripRedBytes = kStripWaves * sizeof(E) + 4 * kStripWaves;
 
 template <int NBITS, bool ZT, bool FULL, typename E, int PASS = 0>
 __device__ __forceinline__ void strip_stats_pack(StripVec<E>* v, uint32_t valid, uint32_t w, uint32_t k0,
@@ -425,7 +432,7 @@ __device__ __forceinline__ void strip_stats_pack(StripVec<E>* v, uint32_t valid,
     constexpr uint32_t PER = SS::PER;
     const uint32_t tid = threadIdx.x;
     E* red = reinterpret_cast<E*>(smem);
-    uint32_t* red_u = reinterpret_cast<uint32_t*>(smem + 4 * sizeof(E));
+    uint32_t* red_u = reinterpret_cast<uint32_t*>(smem + kStripWaves * sizeof(E));
     Q* words = reinterpret_cast<Q*>(smem + kStripRedBytes<E>);
     if constexpr (SS::CHUNKS > 1)
     {

@@ -343,10 +343,10 @@ inline bool regs_applicable(size_t rows, size_t nbits)
 
 
 // The workgroups of a column wait for each other, so all of them must be resident at once: on one die at most half of
-// what the die holds of the kernel (strip_resident_limit, asked from the runtime: 80 strips at 1 to 4 bits, i.e. 655360
-// rows, on a die of 32 compute units at five workgroups each) and never more than this many; a column of more strips has
-// them on all eight dies, up to eight times as many (5.2 M rows at 1 to 4 bits). Taller columns are left to the kernel
-// that re-reads its column.
+// what the die holds of the kernel (strip_resident_limit, asked from the runtime: 32 strips at 1 to 4 bits, i.e. 524288
+// rows, on a die of 32 compute units at two workgroups each) and never more than this many; a column of more strips has
+// them on all eight dies, up to eight times as many (4.2 M rows at 1 to 8 bits). Taller columns run the same strips in
+// several launches.
 constexpr uint32_t kStripMaxPerColumn = 128;
 
 // (written over the element type: E's QWord has Word<E>::kBits bits)

@@ -272,7 +272,7 @@ int cntkq_wait_stripe_reduce_done(cntkq_quantizer* h);
  * sequence of UnquantizeAsync ... QuantizeAsync calls for them (0). No counterpart in the reference: the fused call is
  * an optional fast path. Always 1 up to cntkq_stripe_reduce_max_rows(nbits). Taller stripes run with several workgroups per
  * column where a QuantizeAsync call on the same shape does too (heights that no single workgroup holds: above 102400
- * rows, 81820 at 8 bits, 40910 at 16) and the device holds all of a column's workgroups at once: 1 to 16 bits, up to some 5
+ * rows, 81820 at 8 bits, 40910 at 16) and the device holds all of a column's workgroups at once: 1 to 16 bits, up to some 4
  * million rows at 1 to 4 bits on an MI355X. The answer holds for the handle's current stream; under stream capture it is
  * 0 where the call would have to allocate. */
 int cntkq_stripe_reduce_takes(cntkq_quantizer* h, size_t rows, size_t stripe_cols, size_t nbits, int zero_threshold_for_1bit);

@@ -144,7 +144,7 @@ PATH_CASES = [
     (4991, 2, PATH_AUTO, 0), (5120, 2, PATH_REGS, 0), (4099, 2, PATH_REGS, 0), (6144, 2, PATH_AUTO, 0), (6143, 2, PATH_AUTO, 0),
     (6146, 2, PATH_AUTO, 0),
     # several workgroups per column, a strip of QWords each: any height, one strip or many, full or ragged; the automatic
-    # choice above what one workgroup's registers hold (51184 rows), on one die or, from 81 strips on, on all of them
+    # choice above what one workgroup's registers hold (51184 rows), on one die or, from 33 strips on, on all of them
     (1, 3, PATH_STRIP, 0), (37, 5, PATH_STRIP, 0), (1000, 3, PATH_STRIP, 0), (4096, 3, PATH_STRIP, 0), (4097, 2, PATH_STRIP, 0),
     (9304, 3, PATH_STRIP, 0), (16385, 2, PATH_STRIP, 0), (50257, 3, PATH_STRIP, 0), (51201, 2, PATH_AUTO, 0), (102401, 2, PATH_AUTO, 0),
     (200000, 3, PATH_AUTO, 0), (262147, 2, PATH_STRIP, 0), (330001, 1, PATH_AUTO, 0), (400000, 9, PATH_STRIP, 0),
@@ -155,7 +155,7 @@ PATH_CASES = [
 
 def strip_words_f64(nbits):
     """QWords of a double column that one strip holds."""
-    return {1: 64, 2: 128, 4: 256}.get(nbits, 512)
+    return {1: 128, 2: 256, 4: 512}.get(nbits, 1024)
 
 
 @pytest.mark.parametrize("case", PATH_CASES, ids=["%dx%d_p%d_g%d" % c for c in PATH_CASES])

@@ -139,6 +139,7 @@ PATH_CASES = [
     (50257, 2, PATH_REG, 0), (102365, 1, PATH_REG, 0),
     # several workgroups per column, a strip of QWords each: any height and alignment, one strip or many, full or ragged
     (1, 3, PATH_STRIP, 0), (37, 5, PATH_STRIP, 0), (1000, 3, PATH_STRIP, 0), (8192, 3, PATH_STRIP, 0), (8193, 2, PATH_STRIP, 0),
+    (16384, 2, PATH_STRIP, 0),
     (9304, 3, PATH_STRIP, 0), (16385, 2, PATH_STRIP, 0), (32768, 2, PATH_STRIP, 0), (50257, 3, PATH_STRIP, 0), (100000, 5, PATH_STRIP, 0),
     (102401, 2, PATH_AUTO, 0), (200000, 3, PATH_AUTO, 0), (262147, 2, PATH_STRIP, 0), (524288, 9, PATH_STRIP, 0), (524289, 1, PATH_AUTO, 0),
     (600000, 9, PATH_STRIP, 0), (655361, 1, PATH_AUTO, 0), (1000003, 1, PATH_AUTO, 0), (1500001, 2, PATH_STRIP, 0),
@@ -151,7 +152,7 @@ PATH_CASES = [
 
 def strip_words(nbits):
     """QWords of a float column that one strip holds."""
-    return 256 if nbits == 1 else 512 if nbits == 2 else 1024
+    return 512 if nbits == 1 else 1024 if nbits == 2 else 2048
 
 
 @pytest.mark.parametrize("case", PATH_CASES, ids=["%dx%d_p%d_g%d" % c for c in PATH_CASES])
@@ -189,7 +190,7 @@ def test_kernel_paths(case):
     say("  ", rep)
 
 
-@pytest.mark.parametrize("rows,cols", [(9000, 7), (150001, 5), (262144, 3)])
+@pytest.mark.parametrize("rows,cols", [(9000, 7), (40000, 5), (150001, 5), (262144, 3)])
 def test_strips_in_passes_give_the_strip_kernels_bytes(rows, cols):
     """The strip kernel cut into launches at the points where its workgroups would wait for each other adds the same
     partial sums in the same order: packed bytes and residuals are identical, for floats and doubles."""
@@ -198,7 +199,7 @@ def test_strips_in_passes_give_the_strip_kernels_bytes(rows, cols):
         g, r = datagen.normal_with_outliers(rows, rows, cols, 0.01, dtype=npdt), datagen.normal(rows + 1, rows, cols, 0.002, dtype=npdt)
         for nbits, zt in VARIANTS:
             per_strip = (64 // nbits if npdt == np.float64 else 32 // nbits) * (strip_words(nbits) if npdt == np.float32 else
-                                                                                 {1: 64, 2: 128, 4: 256}.get(nbits, 512))
+                                                                                 {1: 128, 2: 256, 4: 512}.get(nbits, 1024))
             if nbits == 32 or rows <= per_strip:
                 continue
             say("strips in one launch and in passes", rows, cols, npdt.__name__, nbits, zt)
@@ -669,7 +670,7 @@ def test_strip_kernel_reports_workgroups_that_give_up(host_q):
     end, the column is left as it was (packed column and in-place residual untouched, so the error feedback survives),
     the next wait reports the call as failed -- also where the packed matrix lives in host memory and the wait is for
     the copy -- and the handle goes on working afterwards."""
-    # (14 strips per column: below 16 a strip looks for the others' records the moment it has published its own, and the
+    # (7 strips per column: below 16 a strip looks for the others' records the moment it has published its own, and the
     # first one of a column to do so cannot find them)
     rows, cols = 110000, 4
     qz = MatrixQuantizerImpl.Create(0, False)

@@ -114,7 +114,7 @@ def test_random_stripe_reductions(seed, count, tall):
     for n in range(count):
         nbits = int(rng.choice([1, 1, 1, 2, 4, 8, 16, 32]))
         if tall == 2:
-            # what no single workgroup holds: the reduction on strips, on one die and (above some 655360 rows) on all
+            # what no single workgroup holds: the reduction on strips, on one die and (above some 524288 rows) on all
             nbits = int(rng.choice([1, 1, 2, 4, 8, 16]))
             least = {1: 102401, 2: 102401, 4: 102401, 8: 81821, 16: 40911}[nbits]
             most = {1: 1000000, 2: 800000, 4: 500000, 8: 300000, 16: 150000}[nbits]
