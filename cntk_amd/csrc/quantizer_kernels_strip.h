@@ -211,7 +211,8 @@ __device__ __forceinline__ uint32_t strip_poll(const uint64_t* rec, uint32_t tag
 // request rate from the loads and stores that the records wait for: a lane pauses poll_pause x 64 cycles between two polls
 // (200000 x 256 at 1 bit over 1 / 16 / 64 / 128 / 256: 214 / 208 / 200 / 198 / 208 us), and first_pause x 64 cycles
 // before the first one of an exchange, which with many strips per column practically never finds the record there
-// (262144 x 200, 32 strips: 174 -> 154 us with 64; 24576 x 2048, 3 strips: 116 -> 132 us, so only from 16 strips on).
+// (with strips of 256 threads: 262144 x 200, 32 strips: 174 -> 154 us with 64; 24576 x 2048, 3 strips: 116 -> 132 us; with
+// strips of 512 threads: 204800 x 256, 13 strips: 140 -> 135 us; 102401 x 512, 7 strips: 173 -> 175 us: from 8 strips on).
 template <typename T>
 __device__ __forceinline__ T strip_collect(const uint64_t* recs, uint32_t strips, uint32_t tag, const StripGeom& c, uint32_t first_pause, bool& gave_up)
 {

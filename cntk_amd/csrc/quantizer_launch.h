@@ -30,7 +30,7 @@ enum QuantizePath
 constexpr uint32_t kTileMaxRows = 14336; // 56 KB of LDS for a one-column tile
 constexpr size_t kTileMaxFloats = 5120;   // ... and 20 KB for a tile of several columns
 constexpr uint32_t kStripPollPause = 64;           // strip kernel: 64-cycle pauses between two polls of a partial sum
-constexpr uint32_t kStripFirstPauseMinStrips = 16; // ... strips per column from which a pause of 2 x strips precedes the first poll
+constexpr uint32_t kStripFirstPauseMinStrips = 8; // ... strips per column from which a pause of 2 x strips precedes the first poll
 constexpr uint32_t kStripeWideItems = 768;   // work items per column from which the stripe reduction may use more than 256 threads
 constexpr uint32_t kStripeWideMaxCols = 256; // ... 1024 threads up to this many columns
 constexpr uint32_t kColMinRows = 1024;   // shorter columns are better served several to a workgroup (tile kernels)

@@ -670,7 +670,7 @@ def test_strip_kernel_reports_workgroups_that_give_up(host_q):
     end, the column is left as it was (packed column and in-place residual untouched, so the error feedback survives),
     the next wait reports the call as failed -- also where the packed matrix lives in host memory and the wait is for
     the copy -- and the handle goes on working afterwards."""
-    # (7 strips per column: below 16 a strip looks for the others' records the moment it has published its own, and the
+    # (7 strips per column: below 8 a strip looks for the others' records the moment it has published its own, and the
     # first one of a column to do so cannot find them)
     rows, cols = 110000, 4
     qz = MatrixQuantizerImpl.Create(0, False)

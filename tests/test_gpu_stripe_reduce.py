@@ -380,8 +380,8 @@ def test_stripe_reduce_on_strips_reports_workgroups_that_give_up(dtype):
     partial sums a bounded number of polls. With that number set to zero from the host every wait that does not find its
     record at the first look gives up: the kernel still runs to its end, such a column is left as it was (output stripe
     and stripe residual untouched), the wait reports the call as failed, and the handle goes on working afterwards."""
-    # (fewer than 16 strips per column: the first look at the other strips' records then follows a strip's own sum at once)
-    rows, n, k, nbits = (110000 if dtype == torch.float32 else 60000), 3, 2, 1
+    # (seven strips per column, fewer than 8: the first look at the other strips' records then follows a strip's own sum at once)
+    rows, n, k, nbits = (110000 if dtype == torch.float32 else 57000), 3, 2, 1
     npdt = np.float32 if dtype == torch.float32 else np.float64
     qz = MatrixQuantizerImpl.Create(0, False)
     assert qz.StripeReduceTakes(rows, n, nbits, False, dtype)
