@@ -631,31 +631,71 @@ __device__ __forceinline__ uint32_t strip_valid_mask(const StripGeom& c, uint32_
     return valid;
 }
 
-// The PER consecutive values of a column from element i on (16 bytes at the alignment of an element). FULL: all exist.
-// Otherwise bit e of `ok` says whether value e does and the others read as zero: a lane with all of them loads 16 bytes, the
-// few lanes with some fetch them one by one, a lane with none loads nothing.
-template <bool FULL, typename E>
-__device__ __forceinline__ StripVec<E> strip_load(const E* col, uint32_t i, uint32_t ok)
+// N pieces of a column, the PER consecutive values from element i0 + n * stride on each (16 bytes at the alignment of an
+// element), all requested before any is used. FULL: all values exist. Otherwise bit PER * n + e of `valid` says whether
+// value e of piece n does, and the others read as zero. Every lane loads 16 bytes from inside its column whatever it
+// holds (its own piece where that ends inside the column, the column's first elements otherwise), so that no branch
+// stands between the loads; what does not exist is then cleared, and the few values of a piece that runs over the
+// column's end (fewer than PER per column) are fetched one by one.
+template <bool FULL, uint32_t N, typename E>
+__device__ __forceinline__ void strip_load_pieces(const E* col, uint32_t i0, uint32_t stride, uint32_t rows, uint32_t valid, StripVec<E>* out)
 {
     using SE = StripElem<E>;
-    constexpr uint32_t PER = SE::PER;
+    constexpr uint32_t PER = SE::PER, ALL = (1u << PER) - 1u;
     if constexpr (FULL)
-        return __builtin_nontemporal_load(reinterpret_cast<const typename SE::VU*>(col + i));
+    {
+#pragma unroll
+        for (uint32_t n = 0; n < N; ++n)
+            out[n] = __builtin_nontemporal_load(reinterpret_cast<const typename SE::VU*>(col + i0 + n * stride));
+    }
     else
     {
-        typename SE::V x;
-#pragma unroll
-        for (uint32_t e = 0; e < PER; ++e)
-            x[e] = 0;
-        if (ok == (1u << PER) - 1u)
-            x = __builtin_nontemporal_load(reinterpret_cast<const typename SE::VU*>(col + i));
-        else if (ok != 0u)
+        uint32_t over = 0; // pieces with values that run over the column's end
+        if (rows >= PER)
         {
 #pragma unroll
-            for (uint32_t e = 0; e < PER; ++e)
-                x[e] = ((ok >> e) & 1u) ? col[i + e] : (E) 0;
+            for (uint32_t n = 0; n < N; ++n)
+            {
+                const uint32_t i = i0 + n * stride;
+                out[n] = __builtin_nontemporal_load(reinterpret_cast<const typename SE::VU*>(col + (i + PER <= rows ? i : 0u)));
+            }
+#pragma unroll
+            for (uint32_t n = 0; n < N; ++n)
+            {
+                const uint32_t i = i0 + n * stride, ok = (valid >> (PER * n)) & ALL;
+                const bool inside = i + PER <= rows;
+                over |= (!inside && ok != 0u) ? (1u << n) : 0u;
+#pragma unroll
+                for (uint32_t e = 0; e < PER; ++e)
+                    out[n][e] = (inside && ((ok >> e) & 1u)) ? out[n][e] : (E) 0;
+            }
         }
-        return x;
+        else
+        {
+#pragma unroll
+            for (uint32_t n = 0; n < N; ++n)
+            {
+#pragma unroll
+                for (uint32_t e = 0; e < PER; ++e)
+                    out[n][e] = 0;
+                over |= ((valid >> (PER * n)) & ALL) != 0u ? (1u << n) : 0u;
+            }
+        }
+        if (over != 0u)
+        {
+#pragma unroll
+            for (uint32_t n = 0; n < N; ++n)
+            {
+                const uint32_t i = i0 + n * stride, ok = (valid >> (PER * n)) & ALL;
+                if ((over >> n) & 1u)
+                {
+#pragma unroll
+                    for (uint32_t e = 0; e < PER; ++e)
+                        if ((ok >> e) & 1u)
+                            out[n][e] = col[i + e];
+                }
+            }
+        }
     }
 }
 
@@ -666,23 +706,19 @@ __device__ __forceinline__ void quantize_strip_body(const E* g_col, const E* r_c
                                                     uint32_t tag, const StripGeom& c, const StripScratch& scratch, char* smem)
 {
     using SS = StripShape<NBITS, E>;
-    constexpr uint32_t PER = SS::PER, ALL = (1u << PER) - 1u;
+    constexpr uint32_t PER = SS::PER;
     uint32_t w, k0;
     strip_thread_slots<NBITS, E>(strip, w, k0);
     const uint32_t valid = FULL ? 0xFFFFFFFFu : strip_valid_mask<NBITS, E>(c, w, k0);
     const uint32_t i0 = k0 * c.nq + w;
     StripVec<E> v[SS::SLOTS];
-#pragma unroll
-    for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
-        v[kk] = strip_load<FULL, E>(g_col, i0 + kk * c.nq, (valid >> (PER * kk)) & ALL);
+    strip_load_pieces<FULL, SS::SLOTS, E>(g_col, i0, c.nq, c.rows, valid, v);
     constexpr uint32_t BATCH = SS::SLOTS < 4 ? SS::SLOTS : 4;
 #pragma unroll
     for (uint32_t k1 = 0; k1 < SS::SLOTS; k1 += BATCH)
     {
         StripVec<E> b[BATCH];
-#pragma unroll
-        for (uint32_t kk = 0; kk < BATCH; ++kk)
-            b[kk] = strip_load<FULL, E>(r_col, i0 + (k1 + kk) * c.nq, (valid >> (PER * (k1 + kk))) & ALL);
+        strip_load_pieces<FULL, BATCH, E>(r_col, i0 + k1 * c.nq, c.nq, c.rows, valid >> (PER * k1), b);
 #pragma unroll
         for (uint32_t kk = 0; kk < BATCH; ++kk)
             v[k1 + kk] = v[k1 + kk] + b[kk];
@@ -807,9 +843,7 @@ __device__ __forceinline__ void stripe_reduce_strip_body(const StripeSources& sr
     for (uint32_t k1 = 0; k1 < SS::SLOTS; k1 += BATCH)
     {
         StripVec<E> b[BATCH];
-#pragma unroll
-        for (uint32_t kk = 0; kk < BATCH; ++kk)
-            b[kk] = strip_load<FULL, E>(res_col, i0 + (k1 + kk) * c.nq, (valid >> (PER * (k1 + kk))) & ALL);
+        strip_load_pieces<FULL, BATCH, E>(res_col, i0 + k1 * c.nq, c.nq, c.rows, valid >> (PER * k1), b);
 #pragma unroll
         for (uint32_t kk = 0; kk < BATCH; ++kk)
             v[k1 + kk] = v[k1 + kk] + b[kk];
