@@ -9,7 +9,7 @@
 // the height, which columns above 102400 rows -- more than any workgroup's registers hold -- could otherwise only have by
 // reading their inputs two or three times. A strip needs 2 to 8 KB of LDS and, at 1 to 4 bits, some 100 registers (its 32
 // values, their addresses, the masks of the ragged last strip), so two workgroups share a CU; it is the exchange
-// described next, not memory, that bounds the kernel (3.7 to 4.8 TB/s), and below 102400 rows the kernels with one workgroup
+// described next, not memory, that bounds the kernel (4.0 to 5.0 TB/s), and below 102400 rows the kernels with one workgroup
 // per column are faster. (Strips of 256 threads, five to a CU, were 7 to 25 % slower, strips of 1024 threads about as fast
 // as these at a few shapes and slower at most: the fewer workgroups a column's sums must cross, the better, until too few
 // bytes are in flight.)
@@ -768,48 +768,66 @@ __device__ __forceinline__ void stripe_reduce_strip_body(const StripeSources& sr
     strip_thread_slots<NBITS, E>(strip, w, k0);
     const uint32_t valid = FULL ? 0xFFFFFFFFu : strip_valid_mask<NBITS, E>(c, w, k0);
     StripVec<E> v[SS::SLOTS];
-    auto add_worker = [&](uint32_t n, auto first) {
-        const char* qc = src.q[stripe_order(n, src.owner)] + col_off;
-        const E* h = reinterpret_cast<const E*>(qc);
-        const ValueQOf<E> vq = make_vq<NBITS, E>(h[0], h[1]);
-        const Q* bits = reinterpret_cast<const Q*>(qc + 2 * sizeof(E));
-        Q word[PER];
-        if (FULL || w + PER <= c.nq)
+    // The workers' QWords are requested four workers at a time, before any of them is decoded (a worker beyond the last
+    // repeats the last one's addresses and is left out of the sum): one memory round trip per four workers.
+    constexpr uint32_t GROUP = 4;
+    auto add_group = [&](uint32_t n0, auto first_group) {
+        Q word[GROUP][PER];
+        E lo[GROUP], hi[GROUP];
+#pragma unroll
+        for (uint32_t u = 0; u < GROUP; ++u)
         {
-            const typename SE::QV x = *reinterpret_cast<const typename SE::QVU*>(bits + w);
-#pragma unroll
-            for (uint32_t e = 0; e < PER; ++e)
-                word[e] = x[e];
-        }
-        else
-        {
-#pragma unroll
-            for (uint32_t e = 0; e < PER; ++e)
-                word[e] = w + e < c.nq ? bits[w + e] : (Q) 0;
-        }
-        const E val0 = unquantize_value<NBITS, E>(vq, (Q) 0);
-        const E val1 = unquantize_value<NBITS, E>(vq, (Q) 1);
-#pragma unroll
-        for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
-#pragma unroll
-            for (uint32_t e = 0; e < PER; ++e)
+            const uint32_t n = n0 + u < src.workers ? n0 + u : src.workers - 1;
+            const char* qc = src.q[stripe_order(n, src.owner)] + col_off;
+            const E* h = reinterpret_cast<const E*>(qc);
+            lo[u] = h[0];
+            hi[u] = h[1];
+            const Q* bits = reinterpret_cast<const Q*>(qc + 2 * sizeof(E));
+            if constexpr (FULL)
             {
-                const Q code = (word[e] >> ((k0 + kk) * PS::SHIFT)) & PS::CODEMASK;
-                E x;
-                if constexpr (NBITS == 1)
-                    x = code ? val1 : val0;
-                else
-                    x = unquantize_value<NBITS, E>(vq, code);
-                // the first term seeds the sum; afterwards: decoded value + running sum
-                if constexpr (decltype(first)::value)
-                    v[kk][e] = x;
-                else
-                    v[kk][e] = x + v[kk][e];
+                const typename SE::QV x = *reinterpret_cast<const typename SE::QVU*>(bits + w);
+#pragma unroll
+                for (uint32_t e = 0; e < PER; ++e)
+                    word[u][e] = x[e];
             }
+            else
+            {
+                // (QWord by QWord, from inside the column whatever the lane holds: no branch between the loads)
+#pragma unroll
+                for (uint32_t e = 0; e < PER; ++e)
+                    word[u][e] = bits[w + e < c.nq ? w + e : c.nq - 1];
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < GROUP; ++u)
+        {
+            if (n0 + u >= src.workers)
+                break;
+            const ValueQOf<E> vq = make_vq<NBITS, E>(lo[u], hi[u]);
+            const E val0 = unquantize_value<NBITS, E>(vq, (Q) 0);
+            const E val1 = unquantize_value<NBITS, E>(vq, (Q) 1);
+#pragma unroll
+            for (uint32_t kk = 0; kk < SS::SLOTS; ++kk)
+#pragma unroll
+                for (uint32_t e = 0; e < PER; ++e)
+                {
+                    const Q code = (word[u][e] >> ((k0 + kk) * PS::SHIFT)) & PS::CODEMASK;
+                    E x;
+                    if constexpr (NBITS == 1)
+                        x = code ? val1 : val0;
+                    else
+                        x = unquantize_value<NBITS, E>(vq, code);
+                    // the first term seeds the sum; afterwards: decoded value + running sum
+                    if (decltype(first_group)::value && u == 0)
+                        v[kk][e] = x;
+                    else
+                        v[kk][e] = x + v[kk][e];
+                }
+        }
     };
-    add_worker(0u, std::true_type());
-    for (uint32_t n = 1; n < src.workers; ++n)
-        add_worker(n, std::false_type());
+    add_group(0u, std::true_type());
+    for (uint32_t n0 = GROUP; n0 < src.workers; n0 += GROUP)
+        add_group(n0, std::false_type());
     if constexpr (!FULL)
     {
         // (a QWord's bits beyond the column's last element are zero and decode to the lowest level: those values do not exist)
