@@ -118,10 +118,11 @@ def test_random_stripe_reductions(seed, count, tall):
             nbits = int(rng.choice([1, 1, 2, 4, 8, 16]))
             least = {1: 102401, 2: 102401, 4: 102401, 8: 81821, 16: 40911}[nbits]
             most = {1: 1000000, 2: 800000, 4: 500000, 8: 300000, 16: 150000}[nbits]
+            k = int(rng.choice([1, 2, 3, 5, 6, 8, 11]))
+            cols = int(rng.integers(1, 4)) + k - 1  # every owner has a column
+            most = max(least + 4, min(most, 16000000 // (cols * k)))  # bounds what the oracle quantizes per case
             rows = int(rng.choice([least, least + 3, 131072, 200000, 262147, int(rng.integers(least, most))]))
             rows = max(least, min(most, rows))
-            k = int(rng.choice([1, 2, 3, 5, 8]))
-            cols = int(rng.integers(1, 4))
             assert qz.StripeReduceTakes(rows, 1, nbits)
         elif tall:
             # above the LDS kernels' heights: the register kernel of the stripe reduction, up to its limit per bit width

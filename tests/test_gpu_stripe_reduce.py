@@ -73,6 +73,8 @@ CASES = [
     # case -- on all of them), wherever the call sequence's quantize step runs on strips too
     (102401, 4, 2, 1, False), (110000, 3, 3, 1, True), (150001, 4, 4, 2, False), (131072, 2, 2, 4, False), (81822, 2, 2, 8, False),
     (40912, 2, 2, 16, False), (90000, 2, 2, 16, False), (262147, 2, 8, 1, False), (700000, 2, 2, 1, False),
+    # worker counts that are no multiple of the four workers whose QWords a strip requests together, up to the most workers
+    (120001, 5, 5, 1, False), (102403, 13, 13, 2, False), (110000, 3, 64, 1, True), (131075, 2, 7, 4, False),
 ]
 
 
