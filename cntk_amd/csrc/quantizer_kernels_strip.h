@@ -1,38 +1,40 @@
 // gfx950 kernels of the per-column gradient quantizer: columns of any height cut into strips of QWords.
 //
-// A column of `rows` elements is packed into nq QWords, element i in QWord i % nq at bit position i / nq. A strip is a run
-// of W consecutive QWords with ALL their bit positions: 32 / NBITS runs of W consecutive elements, nq elements apart. One
-// 512-thread workgroup owns one strip: a thread holds the elements of 16 bytes' worth of consecutive QWords (four of a
-// float column, two of a double column) at up to eight bit positions (eight 16-byte loads of gradient and residual, at
-// any alignment the element type allows), builds its part of those QWords and writes the residual back from registers;
-// the parts of a QWord meet in LDS. The kernels are written once over the element type. Gradient and residual are read once whatever
-// the height, which columns above 102400 rows -- more than any workgroup's registers hold -- could otherwise only have by
-// reading their inputs two or three times. A strip needs 2 to 8 KB of LDS and, at 1 to 4 bits, some 100 registers (its 32
-// values, their addresses, the masks of the ragged last strip), so two workgroups share a CU; it is the exchange
-// described next, not memory, that bounds the kernel (4.0 to 5.0 TB/s), and below 102400 rows the kernels with one workgroup
-// per column are faster. (Strips of 256 threads, five to a CU, were 7 to 25 % slower, strips of 1024 threads about as fast
-// as these at a few shapes and slower at most: the fewer workgroups a column's sums must cross, the better, until too few
-// bytes are in flight.)
+// A column of `rows` elements is packed into nq QWords, element i in QWord i % nq at bit position i / nq. A strip is a
+// run of W consecutive QWords with ALL their bit positions: 32 / NBITS runs of W consecutive elements, nq elements
+// apart. One 512-thread workgroup owns one strip: a thread holds the elements of 16 bytes' worth of consecutive QWords
+// (four of a float column, two of a double column) at up to eight bit positions (eight 16-byte loads of gradient and
+// residual, at any alignment the element type allows), builds its part of those QWords and writes the residual back
+// from registers; the parts of a QWord meet in LDS. The kernels are written once over the element type. Gradient and
+// residual are read once whatever the height, which columns above 102400 rows -- more than any workgroup's registers
+// hold -- could otherwise only have by reading their inputs two or three times. A strip needs 2 to 8 KB of LDS and, at
+// 1 to 4 bits, some 100 registers (its 32 values, their addresses, the masks of the ragged last strip), so two
+// workgroups share a CU; it is the exchange described next, not memory, that bounds the kernel (4.0 to 5.0 TB/s), and
+// below 102400 rows the kernels with one workgroup per column are faster. (Strips of 256 threads, five to a CU, were 7
+// to 25 % slower, strips of 1024 threads about as fast as these at a few shapes and slower at most: the fewer
+// workgroups a column's sums must cross, the better, until too few bytes are in flight.)
 //
-// The column statistics span the strips of a column. Every workgroup publishes its partial sums in a scratch buffer, one
-// 8-byte record per 32 bits of a sum (a double takes two): the bits and the tag of the launch, written by one atomic store,
-// so that whoever reads the tag of this launch has the bits with it and no second word needs ordering against the first. Then the first wavefront of
-// every workgroup of the column polls the S records (a lane per record, with pauses) until all carry the tag, and adds them up, lanes
-// meeting by butterfly -- one fixed order, the same bytes in every workgroup. One exchange for the sum of squares (more than 1 bit) or
-// the split sums (1 bit against 0), two for 1 bit against the mean (mean, then split sums). The tag is a launch count
-// kept in the scratch buffer itself: every workgroup reads it when it starts, and the last workgroup to finish (a second
-// counter tells) raises it, so that replays of a recorded graph see fresh tags like any other launch. The strips of a
-// column take workgroup indices 8 apart: the device's eight dies take the workgroups of a grid in turn, so a column's
-// strips run on one die, next to each other in its queue, and start together (at most half of what the die holds: all must be resident
-// at once; a column of more strips has them side by side in the grid instead, on all dies, up to half of what the device holds). That placement is what the hardware does, not what any specification promises, so the wait is bounded: after
-// `spin_limit` polls a lane gives up. A workgroup that gave up raises the error word, marks its own records as abandoned
-// (the launch's tag with the top bit set) and stores nothing: no header, no codes, no residual. A workgroup of the same
-// column that finds an abandoned record abandons its strip in the same way, without waiting. A column whose strips did
-// not all become resident in time is therefore left as it was -- with the residual updated in place, the error feedback
-// of that column survives and the call can be repeated -- and the grid always drains. (What remains open is a strip that
-// is resident, has published its first sum and then stalls for the whole bounded wait before its second exchange: its
-// neighbours abandon the column while it may still complete its own part.) Strip 0 of an abandoned column counts the
-// column in the scratch header.
+// The column statistics span the strips of a column. Every workgroup publishes its partial sums in a scratch buffer,
+// one 8-byte record per 32 bits of a sum (a double takes two): the bits and the tag of the launch, written by one
+// atomic store, so that whoever reads the tag of this launch has the bits with it and no second word needs ordering
+// against the first. Then the first wavefront of every workgroup of the column polls the S records (a lane per record,
+// with pauses) until all carry the tag, and adds them up, lanes meeting by butterfly -- one fixed order, the same bytes
+// in every workgroup. One exchange for the sum of squares (more than 1 bit) or the split sums (1 bit against 0), two
+// for 1 bit against the mean (mean, then split sums). The tag is a launch count kept in the scratch buffer itself:
+// every workgroup reads it when it starts, and the last workgroup to finish (a second counter tells) raises it, so that
+// replays of a recorded graph see fresh tags like any other launch. The strips of a column take workgroup indices 8
+// apart: the device's eight dies take the workgroups of a grid in turn, so a column's strips run on one die, next to
+// each other in its queue, and start together (at most half of what the die holds: all must be resident at once; a
+// column of more strips has them side by side in the grid instead, on all dies, up to half of what the device holds).
+// That placement is what the hardware does, not what any specification promises, so the wait is bounded: after
+// `spin_limit` polls a lane gives up. A workgroup that gave up raises the error word, marks its own records as
+// abandoned (the launch's tag with the top bit set) and stores nothing: no header, no codes, no residual. A workgroup
+// of the same column that finds an abandoned record abandons its strip in the same way, without waiting. A column whose
+// strips did not all become resident in time is therefore left as it was -- with the residual updated in place, the
+// error feedback of that column survives and the call can be repeated -- and the grid always drains. (What remains open
+// is a strip that is resident, has published its first sum and then stalls for the whole bounded wait before its second
+// exchange: its neighbours abandon the column while it may still complete its own part.) Strip 0 of an abandoned column
+// counts the column in the scratch header.
 #pragma once
 
 #include <type_traits>
