@@ -126,6 +126,7 @@ struct BatchAbi<float>
     static bool unquantize_member(const UItem& it, size_t nbits, UEntry& e, size_t& lds, uint64_t& blocks)
     {
         LaunchTuning autotune;
+        autotune.unq_member = true;
         const UnquantizePlan p = plan_unquantize(it.qbuf, it.out, it.rows, it.cols, nbits, autotune);
         if (!p.ok)
             return false;

@@ -22,7 +22,8 @@ extern "C" {
  *   tile_gs          0 = automatic, else threads per column in the tile statistics phase (power of two, 8..256)
  *   unq_slots        0 = automatic, else bit positions decoded per thread by the QWord-major unquantize
  *   unq_mode         0 = automatic, 1 = QWord-major decoder with one store per value, 2 = tile decoder wherever it can run,
- *                    3 = automatic without the tile decoder, 4 = row-major decoder wherever it can run
+ *                    3 = automatic without the tile decoder, 4 = row-major decoder (packed column in LDS) wherever it can
+ *                    run, 5 = row-major decoder that fetches its QWords itself wherever it can run
  *   tile_stage       -1 = automatic, 0 = tile kernels write the residual straight to memory, 1 = through LDS */
 int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_gs, unsigned unq_slots,
                            int unq_mode, int tile_stage);

@@ -187,7 +187,8 @@ enum UnqKind : uint32_t
     kUnqScalar = 1,  // QWord-major, 4-byte stores
     kUnqSegment = 2, // segment decoder
     kUnqRows = 3,    // row-major decoder, packed column in LDS
-    kUnqTile = 4     // several short columns per workgroup, packed records in LDS
+    kUnqTile = 4,    // several short columns per workgroup, packed records in LDS
+    kUnqDirect = 5   // row-major decoder, QWords fetched by the threads that decode them (geometry in rowg)
 };
 
 struct UnquantizeBatchEntry
@@ -198,7 +199,7 @@ struct UnquantizeBatchEntry
     uint32_t pad;
     UnqGeom qw;      // valid for kUnqVec4 / kUnqScalar
     UnqSegGeom seg;  // valid for kUnqSegment
-    UnqRowGeom rowg; // valid for kUnqRows
+    UnqRowGeom rowg; // valid for kUnqRows / kUnqDirect
     UnqTileGeom tile; // valid for kUnqTile
 };
 
@@ -220,6 +221,11 @@ __global__ __launch_bounds__(256) void unquantize_batch_kernel(const UnquantizeB
     {
         const UnqRowGeom t = en.rowg; // by value: the loop below stores between its uses
         unquantize_rows_body<NBITS>(en.q, en.out, t, add, block, reinterpret_cast<uint32_t*>(smem_v4));
+    }
+    else if (en.kind == kUnqDirect)
+    {
+        const UnqRowGeom t = en.rowg;
+        unquantize_direct_body<NBITS>(en.q, en.out, t, add, block);
     }
     else
     {

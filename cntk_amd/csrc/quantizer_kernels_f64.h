@@ -884,7 +884,7 @@ struct UnquantizeBatchEntry64
 {
     const char* q;
     double* out;
-    uint32_t kind; // kUnqVec4 (here: 16-byte stores of two doubles), kUnqScalar, kUnqRows or kUnqTile
+    uint32_t kind; // kUnqVec4 (here: 16-byte stores of two doubles), kUnqScalar, kUnqRows, kUnqDirect or kUnqTile
     uint32_t pad;
     UnqGeom qw;
     UnqRowGeom rowg;
@@ -907,6 +907,11 @@ __global__ __launch_bounds__(256) void unquantize_batch_kernel64(const Unquantiz
     {
         const UnqRowGeom t = en.rowg; // by value: the loop below stores between its uses
         unquantize_rows_body<NBITS>(en.q, en.out, t, add, block, reinterpret_cast<uint64_t*>(smem_v4));
+    }
+    else if (en.kind == kUnqDirect)
+    {
+        const UnqRowGeom t = en.rowg;
+        unquantize_direct_body<NBITS>(en.q, en.out, t, add, block);
     }
     else
     {

@@ -381,6 +381,141 @@ __global__ __launch_bounds__(256) void unquantize_rows_kernel(const char* __rest
     unquantize_rows_body<NBITS>(q, out, t, add, blockIdx.x, reinterpret_cast<typename Word<E>::Q*>(smem_v4));
 }
 
+// Row-major decoder that keeps nothing in LDS: the geometry of the one above (chunks of consecutive rows of a column, its
+// head and tail rows, slots dealt by 128-byte lines), but a thread fetches the QWords of its groups of N consecutive rows
+// itself -- N consecutive QWords at one bit position, one 16-byte load at the alignment of a QWord -- all kUnqDirectPieces
+// of them before it decodes the first. Every QWord is fetched once per bit position, from the L2 that the column's other
+// chunks go through as well (their workgroups are 8 apart). No copy of the packed column per workgroup, no barrier, any
+// QWord count: the choice for columns whose packed record is large against a chunk of rows.
+constexpr uint32_t kUnqDirectPieces = 2;
+
+template <int NBITS, typename E>
+__device__ __forceinline__ void unquantize_direct_body(const char* __restrict__ q, E* out, const UnqRowGeom& t, int add, uint32_t block)
+{
+    typedef typename Word<E>::Q QWord;
+    using PS = PackShapeOf<NBITS, Word<E>::kBits>;
+    constexpr uint32_t N = 16 / sizeof(E);
+    constexpr uint32_t P = kUnqDirectPieces;
+    typedef E Vec __attribute__((ext_vector_type(N)));
+    typedef QWord QVec __attribute__((ext_vector_type(N)));
+    typedef QVec QVecAtWord __attribute__((aligned(sizeof(QWord))));
+    const uint32_t tid = threadIdx.x;
+    uint32_t c, ch;
+    unq_rows_block_to_chunk(block, t.chunks, t.blocks, c, ch);
+    const char* qc = q + (size_t) c * t.qcol;
+    const E* gh = reinterpret_cast<const E*>(qc);
+    const E lo = gh[0];
+    const E uf = make_ufactor<NBITS>(lo, gh[1]);
+    const QWord* bits = reinterpret_cast<const QWord*>(qc + 2 * sizeof(E));
+    // head, body and tail rows of the column as in the decoder above; here every chunk is t.chunk rows at most
+    E* oc = out + (size_t) c * t.rows;
+    const uint32_t head = (N - (uint32_t) ((reinterpret_cast<uintptr_t>(oc) / sizeof(E)) & (N - 1))) & (N - 1);
+    const uint32_t body = (t.rows - head) & ~(N - 1);
+    const uint32_t tail = t.rows - head - body;
+    const uint32_t r0 = ch * t.chunk;
+    const uint32_t end = body < r0 + t.chunk ? body : r0 + t.chunk;
+    const uint32_t pieces = end > r0 ? (end - r0) / N : 0u;
+    Vec* o4 = reinterpret_cast<Vec*>(oc + head + r0);
+    const E val0 = unquantize_value<NBITS>(uf, lo, 0u);
+    const E val1 = unquantize_value<NBITS>(uf, lo, 1u);
+    {
+        uint32_t row = t.rows; // none
+        if (ch == 0 && tid < head)
+            row = tid;
+        else if (ch + 1 == t.chunks && tid >= N && tid < N + tail)
+            row = head + body + (tid - N);
+        if (row < t.rows)
+        {
+            const uint32_t k = row / t.nq;
+            const QWord code = (bits[row - k * t.nq] >> (k * PS::SHIFT)) & PS::CODEMASK;
+            E x;
+            if constexpr (NBITS == 1)
+                x = code ? val1 : val0;
+            else
+                x = unquantize_value<NBITS>(uf, lo, code);
+            oc[row] = add ? x + oc[row] : x;
+        }
+    }
+    const uint32_t shift = (uint32_t) ((reinterpret_cast<uintptr_t>(o4) >> 4) & 7u);
+    const uint32_t p0 = (tid < shift ? tid + 256 : tid) - shift;
+    const uint32_t i0 = head + r0 + N * p0;
+    const uint32_t k0 = i0 / t.nq;
+    const uint32_t w0 = i0 - k0 * t.nq;
+    const uint32_t dk = (256u * N) / t.nq;
+    const uint32_t dw = 256u * N - dk * t.nq;
+    QVec qv[P];
+    Vec prev[P];
+    uint32_t ks[P], ws[P];
+    {
+        uint32_t k = k0, w = w0;
+#pragma unroll
+        for (uint32_t u = 0; u < P; ++u)
+        {
+            const uint32_t p = p0 + 256 * u;
+            ks[u] = k;
+            ws[u] = w;
+            // (a group that wraps to the next bit position inside is fetched QWord by QWord below; a piece beyond the
+            // chunk fetches the column's first QWords and uses nothing)
+            const uint32_t from = p < pieces ? (w + N <= t.nq ? w : t.nq - N) : 0u;
+            qv[u] = *reinterpret_cast<const QVecAtWord*>(bits + from);
+            if (add)
+                prev[u] = o4[p < pieces ? p : 0u];
+            k += dk;
+            w += dw;
+            if (w >= t.nq)
+            {
+                w -= t.nq;
+                ++k;
+            }
+        }
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < P; ++u)
+    {
+        const uint32_t p = p0 + 256 * u;
+        if (p < pieces)
+        {
+            QWord wd[N];
+            uint32_t sh[N];
+#pragma unroll
+            for (uint32_t e = 0; e < N; ++e)
+            {
+                wd[e] = qv[u][e];
+                sh[e] = ks[u] * PS::SHIFT;
+            }
+            if (ws[u] + N > t.nq)
+            {
+#pragma unroll
+                for (uint32_t e = 0; e < N; ++e)
+                {
+                    const bool wraps = ws[u] + e >= t.nq;
+                    wd[e] = bits[wraps ? ws[u] + e - t.nq : ws[u] + e];
+                    sh[e] = (wraps ? ks[u] + 1 : ks[u]) * PS::SHIFT;
+                }
+            }
+            Vec x;
+#pragma unroll
+            for (uint32_t e = 0; e < N; ++e)
+            {
+                const QWord code = (wd[e] >> sh[e]) & PS::CODEMASK;
+                if constexpr (NBITS == 1)
+                    x[e] = code ? val1 : val0;
+                else
+                    x[e] = unquantize_value<NBITS>(uf, lo, code);
+            }
+            if (add)
+                x = x + prev[u]; // unquantized value + previous content
+            __builtin_nontemporal_store(x, o4 + p);
+        }
+    }
+}
+
+template <int NBITS, typename E>
+__global__ __launch_bounds__(256) void unquantize_direct_kernel(const char* __restrict__ q, E* out, UnqRowGeom t, int add)
+{
+    unquantize_direct_body<NBITS>(q, out, t, add, blockIdx.x);
+}
+
 // Tile decoder for short columns. Consecutive columns are adjacent in the packed matrix and in the output, so a
 // workgroup takes `cpt` columns at once: their packed records (one contiguous run) go to LDS in coalesced loads, each
 // column's decoding constants are computed once, and the cpt * rows values (one contiguous run) leave in aligned

@@ -67,7 +67,8 @@ struct LaunchTuning
     int tile_stage = -1;    // -1 = automatic; 0 / 1 = residual written straight to memory / staged through LDS
     uint32_t tile_threads = 0; // 0 = automatic; else workgroup size of the tile kernels (64, 128, 256)
     uint32_t unq_slots = 0; // 0 = default; else bit positions per thread in unquantize
-    int unq_mode = 0; // 0 automatic, 1 QWord-major with 4-byte stores, 2 / 4 tile / row-major decoder wherever it can run, 3 automatic without the tile decoder
+    int unq_mode = 0; // 0 automatic, 1 QWord-major with 4-byte stores, 2 / 4 / 5 tile / row-major / LDS-free row-major decoder wherever it can run, 3 automatic without the tile decoder
+    bool unq_member = false; // the matrix is decoded as a member of a gradient-set launch
 };
 
 // Events tied to the kernel dispatch itself (its completion signal), not recorded as separate stream
@@ -842,6 +843,25 @@ constexpr size_t kUnqTileElems = 4096;    // values per workgroup the tile decod
 constexpr size_t kUnqRowsMinRows = 1664;  // from this height on a column per workgroup (row-major decoder) beats several columns per
                                           // workgroup (tile decoder): 1152 x 8192 7.5 us against 9.8 us, 1792 x 5266 8.5 us against 7.6 us
 
+// The geometry of the row-major decoder that fetches its QWords itself: chunks of 256 threads x kUnqDirectPieces 16-byte
+// stores (per16 elements each). False if the grid would not fit.
+inline bool make_unq_direct_geom(UnqRowGeom& t, size_t rows, size_t cols, size_t nq, uint64_t qcol, size_t per16)
+{
+    const size_t chunk = 256 * kUnqDirectPieces * per16;
+    const uint64_t chunks = (rows + chunk - 1) / chunk;
+    const uint64_t blocks = (uint64_t) cols * chunks;
+    if (blocks > 0x7FFFFFFFull)
+        return false;
+    t.rows = (uint32_t) rows;
+    t.nq = (uint32_t) nq;
+    t.chunk = (uint32_t) chunk;
+    t.chunks = (uint32_t) chunks;
+    t.blocks = (uint32_t) blocks;
+    t.pad = 0;
+    t.qcol = qcol;
+    return true;
+}
+
 inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t rows, size_t cols, size_t nbits,
                                       const LaunchTuning& tune)
 {
@@ -861,8 +881,21 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
     const bool vec_ideal = vec_can && nq % 32 == 0 && rows % 32 == 0 && rows * nbits == nq * 32;
     const bool rows_can = slots_free && rows >= 16 && nq >= 32 && nq * 4 <= kUnqRowsMaxLds; // any height, any (4-byte) alignment
     const bool tile_can = slots_free && rows <= kUnqTileMaxRows; // (any 4-byte alignment of the output)
-    bool vec = false, rowmajor = false, tile = false, seg_allowed = true;
-    if (mode == 1)
+    const bool direct_can = slots_free && rows >= 16 && nq >= 32; // any height, any (4-byte) alignment
+    // Where the row-major decoder that fetches its QWords itself is the automatic choice (measured against the others):
+    // from 16384 rows on; from 8192 rows at 2 bits and more where the QWord-major stores would not be whole lines, unless
+    // the last chunk of a column would be mostly empty; and the 1- and 2-bit columns of exactly one to four chunks
+    // (2048 ... 8192 rows), by 2 to 3 % -- in a launch of their own: as members of a gradient-set launch they measured slower.
+    const size_t direct_chunk = 256 * kUnqDirectPieces * 4;
+    const bool direct_full = (((rows + direct_chunk - 1) / direct_chunk) * direct_chunk - rows) * 8 <= rows;
+    const bool direct_auto = direct_can && (rows >= 16384 || (!vec_ideal && nbits >= 2 && rows >= 8192 && direct_full) ||
+                                            (vec_ideal && nbits <= 2 && rows % direct_chunk == 0 && rows <= 8192 && !tune.unq_member));
+    bool vec = false, rowmajor = false, tile = false, seg_allowed = true, direct = false;
+    if (mode == 5 && direct_can)
+        direct = true;
+    else if (mode == 0 && direct_auto)
+        direct = true;
+    else if (mode == 1)
         seg_allowed = false; // QWord-major, 4-byte stores
     else if (mode == 2 && tile_can)
         tile = true;
@@ -908,6 +941,13 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
             return p;
         }
         vec = vec_can;
+    }
+    if (direct && make_unq_direct_geom(p.rowg, rows, cols, nq, qcol_bytes(nbits, rows), 4))
+    {
+        p.kind = kUnqDirect;
+        p.blocks = p.rowg.blocks;
+        p.ok = true;
+        return p;
     }
     if (rowmajor)
     {

@@ -454,8 +454,25 @@ inline UnquantizePlan64 plan_unquantize(const double* out, size_t rows, size_t c
     const bool vec_ideal = nq % 16 == 0 && rows % 16 == 0 && rows * nbits == nq * 64 && out16;
     const bool rows_can = tune.unq_slots == 0 && rows >= 16 && nq >= 16 && nq * 8 <= 48 * 1024; // any height, any alignment
     const bool tile_can = tune.unq_slots == 0 && out16 && rows <= kUnqTileMaxRows64;
+    const bool direct_can = tune.unq_slots == 0 && rows >= 16 && nq >= 16; // any height, any alignment
+    // (the automatic choice from 16384 rows on, for 1- and 2-bit columns of whole chunks of 1024 rows, and from 8192 rows
+    // at 2 bits and more where the QWord-major stores would not be whole lines and the last chunk is not mostly empty)
+    const size_t direct_chunk = 256 * kUnqDirectPieces * 2;
+    const bool direct_full = (((rows + direct_chunk - 1) / direct_chunk) * direct_chunk - rows) * 8 <= rows;
+    const bool direct_auto = direct_can && (rows >= 16384 || (nbits <= 2 && rows % direct_chunk == 0) ||
+                                            (!vec_ideal && nbits >= 2 && rows >= 8192 && direct_full));
     bool use_rows = false, use_tile = false;
-    if (mode == 2 && tile_can)
+    if ((mode == 5 && direct_can) || (mode == 0 && direct_auto))
+    {
+        if (make_unq_direct_geom(p.rowg, rows, cols, nq, qcol_bytes(nbits, rows), 2))
+        {
+            p.kind = kUnqDirect;
+            p.blocks = p.rowg.blocks;
+            p.ok = true;
+            return p;
+        }
+    }
+    else if (mode == 2 && tile_can)
         use_tile = true;
     else if (mode == 4 && rows_can)
         use_rows = true;
@@ -561,6 +578,11 @@ inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const c
 {
     if (p.kind == kUnqRows)
         return launch_unquantize_rows<NBITS>(s, ev, q, out, p.rowg, add);
+    if (p.kind == kUnqDirect)
+    {
+        hipExtLaunchKernelGGL((unquantize_direct_kernel<NBITS, double>), dim3(p.rowg.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.rowg, add);
+        return hipGetLastError();
+    }
     if (p.kind == kUnqTile)
         return launch_unquantize_tile<NBITS>(s, ev, q, out, p.tile, add);
     return launch_unquantize_n<NBITS>(s, ev, q, out, p.qw, p.kind == kUnqVec4, add);

@@ -260,13 +260,14 @@ DECODER_SHAPES_F64 = [(1, 1), (1, 9), (3, 5), (31, 13), (64, 100), (147, 64), (4
 @pytest.mark.parametrize("shape", DECODER_SHAPES_F64, ids=["%dx%d" % s for s in DECODER_SHAPES_F64])
 def test_tile_and_row_major_decoders_f64(shape):
     """The decoders for columns whose QWord-major stores would not be whole lines: several short columns per workgroup
-    (mode 2), row-major with the packed column in LDS (mode 4), and the automatic choice; add and overwrite; bit-exact."""
+    (mode 2), row-major with the packed column in LDS (mode 4), row-major with every thread fetching its own QWords
+    (mode 5), and the automatic choice; add and overwrite; bit-exact."""
     rows, cols = shape
     for nbits, zt in VARIANTS:
         g = datagen.normal_with_outliers(rows * 11 + nbits, rows, cols, 0.01, dtype=F64)
         q, _ = oracle.quantize(g, zeros(rows, cols), nbits, zt)
         prev = datagen.normal(rows * 13 + nbits, rows, cols, 1.0, dtype=F64)
-        for mode in (2, 4, 0):
+        for mode in (2, 4, 5, 0):
             say("f64 decoder", rows, cols, nbits, "mode", mode)
             qz = MatrixQuantizerImpl.Create(0, False)
             qz._set_tuning(unq_mode=mode)

@@ -377,7 +377,7 @@ def test_tile_decoder(shape):
         g = datagen.normal_with_outliers(rows * 11 + nbits, rows, cols, 0.01)
         q, _ = oracle.quantize(g, np.zeros_like(g, order="F"), nbits, zt)
         prev = datagen.normal(rows * 13 + nbits, rows, cols, 1.0)
-        for mode in (2, 0, 3):
+        for mode in (2, 0, 3, 5):
             say("tile decoder", rows, cols, nbits, "mode", mode)
             qz = MatrixQuantizerImpl.Create(0, False)
             qz._set_tuning(unq_mode=mode)
@@ -395,6 +395,37 @@ def test_tile_decoder(shape):
         qz.WaitUnquantizeAsyncDone()
         parity.check_unquantize(q, rows, cols, nbits, Out.to_numpy())
         assert float(big[0]) == 0.0 and float(big[-1]) == 0.0 and float(big[-2]) == 0.0 and float(big[-3]) == 0.0
+
+
+DIRECT_DECODER_SHAPES = [(2048, 5), (2049, 3), (4096, 3), (6143, 2), (8192, 3), (9304, 3), (16384, 2), (20001, 2), (32770, 2), (100000, 2),
+                         (150001, 2), (600000, 1)]
+
+
+@pytest.mark.parametrize("shape", DIRECT_DECODER_SHAPES, ids=["%dx%d" % s for s in DIRECT_DECODER_SHAPES])
+def test_row_major_decoder_that_fetches_its_qwords(shape):
+    """The row-major decoder without a copy of the packed column in LDS, forced (mode 5) and as the automatic choice:
+    one chunk and many per column, a last chunk of a few rows, groups of four that wrap to the next bit position,
+    outputs at every offset within 16 bytes; add and overwrite; bit-exact, and nothing written outside the matrix."""
+    rows, cols = shape
+    for nbits, zt in VARIANTS:
+        g = datagen.normal_with_outliers(rows * 17 + nbits, rows, cols, 0.01)
+        q, _ = oracle.quantize(g, np.zeros_like(g, order="F"), nbits, zt, threads=8)
+        prev = datagen.normal(rows * 19 + nbits, rows, cols, 1.0)
+        Q = QuantizedMatrix(rows, cols, nbits, 0)
+        Q.from_numpy(q)
+        for mode in (5, 0):
+            qz = MatrixQuantizerImpl.Create(0, False)
+            qz._set_tuning(unq_mode=mode)
+            for offset in (0, 1, 2, 3):
+                say("decoder without LDS", rows, cols, nbits, "mode", mode, "offset", offset)
+                for add in (False, True):
+                    big = torch.full((rows * cols + 8,), 7.0, dtype=torch.float32, device="cuda:0")
+                    big[offset:offset + rows * cols] = torch.from_numpy(np.ascontiguousarray(prev.reshape(-1, order="F"))).cuda()
+                    Out = Matrix(rows, cols, 0, big[offset:offset + rows * cols])
+                    qz.UnquantizeAsync(Q, Out, add=add)
+                    qz.WaitUnquantizeAsyncDone()
+                    parity.check_unquantize(q, rows, cols, nbits, Out.to_numpy(), prev_out=prev if add else None)
+                    assert bool((big[:offset] == 7.0).all()) and bool((big[offset + rows * cols:] == 7.0).all())
 
 
 # ---- boundary behaviour ------------------------------------------------------------------------------
