@@ -89,6 +89,7 @@ struct BatchAbi<double>
     static bool unquantize_member(const UItem& it, size_t nbits, UEntry& e, size_t& lds, uint64_t& blocks)
     {
         LaunchTuning autotune;
+        autotune.unq_member = true;
         const f64::UnquantizePlan64 p = f64::plan_unquantize(it.out, it.rows, it.cols, nbits, autotune);
         if (!p.ok)
             return false;

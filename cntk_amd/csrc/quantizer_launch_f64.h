@@ -455,11 +455,12 @@ inline UnquantizePlan64 plan_unquantize(const double* out, size_t rows, size_t c
     const bool rows_can = tune.unq_slots == 0 && rows >= 16 && nq >= 16 && nq * 8 <= 48 * 1024; // any height, any alignment
     const bool tile_can = tune.unq_slots == 0 && out16 && rows <= kUnqTileMaxRows64;
     const bool direct_can = tune.unq_slots == 0 && rows >= 16 && nq >= 16; // any height, any alignment
-    // (the automatic choice from 16384 rows on, for 1- and 2-bit columns of whole chunks of 1024 rows, and from 8192 rows
+    // (the automatic choice from 16384 rows on, for 1- and 2-bit columns of whole chunks of 1024 rows in a launch of their
+    // own -- as members of a gradient-set launch they measured slower than with the QWord-major decoder --, and from 8192 rows
     // at 2 bits and more where the QWord-major stores would not be whole lines and the last chunk is not mostly empty)
     const size_t direct_chunk = 256 * kUnqDirectPieces * 2;
     const bool direct_full = (((rows + direct_chunk - 1) / direct_chunk) * direct_chunk - rows) * 8 <= rows;
-    const bool direct_auto = direct_can && (rows >= 16384 || (nbits <= 2 && rows % direct_chunk == 0) ||
+    const bool direct_auto = direct_can && (rows >= 16384 || (nbits <= 2 && rows % direct_chunk == 0 && !tune.unq_member) ||
                                             (!vec_ideal && nbits >= 2 && rows >= 8192 && direct_full));
     bool use_rows = false, use_tile = false;
     if ((mode == 5 && direct_can) || (mode == 0 && direct_auto))
