@@ -134,6 +134,7 @@ struct BatchAbi<float>
         e.qw = p.qw;
         e.seg = p.seg;
         e.rowg = p.rowg;
+        e.flat = p.flat;
         e.tile = p.tile;
         lds = p.lds;
         blocks = p.blocks;

@@ -96,6 +96,7 @@ struct BatchAbi<double>
         e.kind = p.kind;
         e.qw = p.qw;
         e.rowg = p.rowg;
+        e.flat = p.flat;
         e.tile = p.tile;
         lds = p.lds;
         blocks = p.blocks;

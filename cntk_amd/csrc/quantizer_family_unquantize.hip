@@ -14,6 +14,8 @@ inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const c
         hipExtLaunchKernelGGL((unquantize_rows_kernel<NBITS, float>), dim3(p.blocks), dim3(256), p.lds, s, ev.start, ev.stop, 0, q, out, p.rowg, add);
     else if (p.kind == kUnqDirect)
         hipExtLaunchKernelGGL((unquantize_direct_kernel<NBITS, float>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.rowg, add);
+    else if (p.kind == kUnqFlat)
+        hipExtLaunchKernelGGL((unquantize_flat_kernel<NBITS, float>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.flat, add);
     else if (p.kind == kUnqSegment)
         hipExtLaunchKernelGGL((unquantize_segment_kernel<NBITS>), dim3(p.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.seg, add);
     else if (p.kind == kUnqVec4)

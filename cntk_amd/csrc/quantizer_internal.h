@@ -23,7 +23,8 @@ extern "C" {
  *   unq_slots        0 = automatic, else bit positions decoded per thread by the QWord-major unquantize
  *   unq_mode         0 = automatic, 1 = QWord-major decoder with one store per value, 2 = tile decoder wherever it can run,
  *                    3 = automatic without the tile decoder, 4 = row-major decoder (packed column in LDS) wherever it can
- *                    run, 5 = row-major decoder that fetches its QWords itself wherever it can run
+ *                    run, 5 = row-major decoder that fetches its QWords itself wherever it can run, 6 = the same for short
+ *                    columns (the matrix as one run of 16-byte groups) wherever it can run
  *   tile_stage       -1 = automatic, 0 = tile kernels write the residual straight to memory, 1 = through LDS */
 int cntkq_debug_set_tuning(cntkq_quantizer* h, int quantize_path, unsigned tile_gs, unsigned unq_slots,
                            int unq_mode, int tile_stage);

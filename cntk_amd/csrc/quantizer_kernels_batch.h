@@ -188,7 +188,8 @@ enum UnqKind : uint32_t
     kUnqSegment = 2, // segment decoder
     kUnqRows = 3,    // row-major decoder, packed column in LDS
     kUnqTile = 4,    // several short columns per workgroup, packed records in LDS
-    kUnqDirect = 5   // row-major decoder, QWords fetched by the threads that decode them (geometry in rowg)
+    kUnqDirect = 5,  // row-major decoder, QWords fetched by the threads that decode them (geometry in rowg)
+    kUnqFlat = 6     // the same for short columns: the matrix as one run of groups of consecutive elements
 };
 
 struct UnquantizeBatchEntry
@@ -201,6 +202,7 @@ struct UnquantizeBatchEntry
     UnqSegGeom seg;  // valid for kUnqSegment
     UnqRowGeom rowg; // valid for kUnqRows / kUnqDirect
     UnqTileGeom tile; // valid for kUnqTile
+    UnqFlatGeom flat; // valid for kUnqFlat
 };
 
 template <int NBITS>
@@ -226,6 +228,11 @@ __global__ __launch_bounds__(256) void unquantize_batch_kernel(const UnquantizeB
     {
         const UnqRowGeom t = en.rowg;
         unquantize_direct_body<NBITS>(en.q, en.out, t, add, block);
+    }
+    else if (en.kind == kUnqFlat)
+    {
+        const UnqFlatGeom t = en.flat;
+        unquantize_flat_body<NBITS>(en.q, en.out, t, add, block);
     }
     else
     {

@@ -884,11 +884,12 @@ struct UnquantizeBatchEntry64
 {
     const char* q;
     double* out;
-    uint32_t kind; // kUnqVec4 (here: 16-byte stores of two doubles), kUnqScalar, kUnqRows, kUnqDirect or kUnqTile
+    uint32_t kind; // kUnqVec4 (here: 16-byte stores of two doubles), kUnqScalar, kUnqRows, kUnqDirect, kUnqFlat or kUnqTile
     uint32_t pad;
     UnqGeom qw;
     UnqRowGeom rowg;
     UnqTileGeom tile;
+    UnqFlatGeom flat;
 };
 
 template <int NBITS>
@@ -912,6 +913,11 @@ __global__ __launch_bounds__(256) void unquantize_batch_kernel64(const Unquantiz
     {
         const UnqRowGeom t = en.rowg;
         unquantize_direct_body<NBITS>(en.q, en.out, t, add, block);
+    }
+    else if (en.kind == kUnqFlat)
+    {
+        const UnqFlatGeom t = en.flat;
+        unquantize_flat_body<NBITS>(en.q, en.out, t, add, block);
     }
     else
     {

@@ -516,6 +516,87 @@ __global__ __launch_bounds__(256) void unquantize_direct_kernel(const char* __re
     unquantize_direct_body<NBITS>(q, out, t, add, blockIdx.x);
 }
 
+// The same without LDS for short columns whose heights and QWord counts are multiples of N (the elements of 16 bytes):
+// consecutive columns are adjacent in the output, so the matrix is one run of groups of N consecutive elements, each group
+// inside one column at one bit position of N consecutive QWords. A thread takes kUnqDirectPieces groups, 256 groups apart,
+// finds column, bit position and QWord of each, requests the column's header and the N QWords of every group and then
+// decodes. The output is 16-byte aligned and the matrix has fewer than 2^32 elements (checked by the host).
+struct UnqFlatGeom
+{
+    uint32_t rows;
+    uint32_t nq;
+    uint32_t groups; // rows * cols / N
+    uint32_t blocks;
+    double inv_rows;
+    double inv_nq;
+    uint64_t qcol;
+};
+
+template <int NBITS, typename E>
+__device__ __forceinline__ void unquantize_flat_body(const char* __restrict__ q, E* out, const UnqFlatGeom& t, int add, uint32_t block)
+{
+    typedef typename Word<E>::Q QWord;
+    using PS = PackShapeOf<NBITS, Word<E>::kBits>;
+    constexpr uint32_t N = 16 / sizeof(E);
+    constexpr uint32_t P = kUnqDirectPieces;
+    typedef E Vec __attribute__((ext_vector_type(N)));
+    typedef E Pair __attribute__((ext_vector_type(2)));
+    typedef Pair PairAtElem __attribute__((aligned(sizeof(E))));
+    typedef QWord QVec __attribute__((ext_vector_type(N)));
+    typedef QVec QVecAtWord __attribute__((aligned(sizeof(QWord))));
+    Vec* o4 = reinterpret_cast<Vec*>(out);
+    QVec qv[P];
+    Pair hd[P];
+    Vec prev[P];
+    uint32_t sh[P];
+#pragma unroll
+    for (uint32_t u = 0; u < P; ++u)
+    {
+        const uint32_t g = block * (256u * P) + 256u * u + threadIdx.x;
+        const uint32_t gg = g < t.groups ? g : 0u; // a group beyond the matrix fetches the first one's and uses nothing
+        uint32_t c, r, k, w;
+        divmod_u32(gg * N, t.rows, t.inv_rows, c, r);
+        divmod_u32(r, t.nq, t.inv_nq, k, w);
+        const char* qc = q + (size_t) c * t.qcol;
+        hd[u] = *reinterpret_cast<const PairAtElem*>(qc);
+        qv[u] = *reinterpret_cast<const QVecAtWord*>(qc + 2 * sizeof(E) + (size_t) w * sizeof(QWord));
+        sh[u] = k * PS::SHIFT;
+        if (add)
+            prev[u] = o4[gg];
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < P; ++u)
+    {
+        const uint32_t g = block * (256u * P) + 256u * u + threadIdx.x;
+        if (g < t.groups)
+        {
+            const E lo = hd[u][0];
+            const E uf = make_ufactor<NBITS>(lo, hd[u][1]);
+            const E val0 = unquantize_value<NBITS>(uf, lo, 0u);
+            const E val1 = unquantize_value<NBITS>(uf, lo, 1u);
+            Vec x;
+#pragma unroll
+            for (uint32_t e = 0; e < N; ++e)
+            {
+                const QWord code = (qv[u][e] >> sh[u]) & PS::CODEMASK;
+                if constexpr (NBITS == 1)
+                    x[e] = code ? val1 : val0;
+                else
+                    x[e] = unquantize_value<NBITS>(uf, lo, code);
+            }
+            if (add)
+                x = x + prev[u];
+            __builtin_nontemporal_store(x, o4 + g);
+        }
+    }
+}
+
+template <int NBITS, typename E>
+__global__ __launch_bounds__(256) void unquantize_flat_kernel(const char* __restrict__ q, E* out, UnqFlatGeom t, int add)
+{
+    unquantize_flat_body<NBITS>(q, out, t, add, blockIdx.x);
+}
+
 // Tile decoder for short columns. Consecutive columns are adjacent in the packed matrix and in the output, so a
 // workgroup takes `cpt` columns at once: their packed records (one contiguous run) go to LDS in coalesced loads, each
 // column's decoding constants are computed once, and the cpt * rows values (one contiguous run) leave in aligned

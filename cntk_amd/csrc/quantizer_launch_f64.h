@@ -434,6 +434,7 @@ struct UnquantizePlan64
     UnqGeom qw;
     UnqRowGeom rowg;
     UnqTileGeom tile;
+    UnqFlatGeom flat;
     uint32_t blocks = 0; // 256-thread blocks
     size_t lds = 0;      // dynamic LDS (kUnqRows, kUnqTile)
     bool ok = false;
@@ -445,6 +446,7 @@ inline UnquantizePlan64 plan_unquantize(const double* out, size_t rows, size_t c
     std::memset(&p.qw, 0, sizeof p.qw);
     std::memset(&p.rowg, 0, sizeof p.rowg);
     std::memset(&p.tile, 0, sizeof p.tile);
+    std::memset(&p.flat, 0, sizeof p.flat);
     const size_t vpw = 64 / nbits;
     const size_t nq = qwords_per_col(rows, nbits);
     const bool out16 = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
@@ -462,6 +464,18 @@ inline UnquantizePlan64 plan_unquantize(const double* out, size_t rows, size_t c
     const bool direct_full = (((rows + direct_chunk - 1) / direct_chunk) * direct_chunk - rows) * 8 <= rows;
     const bool direct_auto = direct_can && (rows >= 16384 || (nbits <= 2 && rows % direct_chunk == 0 && !tune.unq_member) ||
                                             (!vec_ideal && nbits >= 2 && rows >= 8192 && direct_full));
+    // (the LDS-free decoder for short columns: the rule of the float side, up to 2048 rows -- 512 x 50000 38.0 -> 32.4 us,
+    // 576 x 16384 at 2 bits 15.6 -> 12.8 us, 1536 x 6144 13.7 -> 12.0 us, even at 2048 x 4652 at 4 bits; 4608 x 2048 at 4 bits
+    // is 13 % slower with it than with the packed column in LDS)
+    const bool flat_auto = mode == 0 && !direct_auto && rows <= 2048 &&
+                           (!tune.unq_member || (!vec_ideal && (uint64_t) rows * cols >= ((uint64_t) 1 << 22)));
+    if ((mode == 6 || flat_auto) && tune.unq_slots == 0 && out16 && make_unq_flat_geom(p.flat, rows, cols, nq, qcol_bytes(nbits, rows), 2))
+    {
+        p.kind = kUnqFlat;
+        p.blocks = p.flat.blocks;
+        p.ok = true;
+        return p;
+    }
     bool use_rows = false, use_tile = false;
     if ((mode == 5 && direct_can) || (mode == 0 && direct_auto))
     {
@@ -582,6 +596,11 @@ inline hipError_t launch_unquantize_plan(hipStream_t s, LaunchEvents ev, const c
     if (p.kind == kUnqDirect)
     {
         hipExtLaunchKernelGGL((unquantize_direct_kernel<NBITS, double>), dim3(p.rowg.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.rowg, add);
+        return hipGetLastError();
+    }
+    if (p.kind == kUnqFlat)
+    {
+        hipExtLaunchKernelGGL((unquantize_flat_kernel<NBITS, double>), dim3(p.flat.blocks), dim3(256), 0, s, ev.start, ev.stop, 0, q, out, p.flat, add);
         return hipGetLastError();
     }
     if (p.kind == kUnqTile)

@@ -35,7 +35,7 @@ def main():
     ap.add_argument("--path", type=int, default=0, help="force a quantize kernel: 1 tile, 2 tall (re-reading), 3 column in LDS, 4 column in registers (16-byte accesses), "
                     "5 column in registers (one element per access), 6 several workgroups per column (strips)")
     ap.add_argument("--unq-mode", type=int, default=0, help="decoder choice: 0 automatic, 1 QWord-major with one store per value, 2 tile decoder, 3 automatic without the tile "
-                    "decoder, 4 row-major decoder with the packed column in LDS, 5 row-major decoder that fetches its QWords itself")
+                    "decoder, 4 row-major decoder with the packed column in LDS, 5 row-major decoder that fetches its QWords itself, 6 the same over short columns")
     ap.add_argument("--tile-gs", type=int, default=0, help="threads per column of the tile kernels' statistics phase (0: the library's choice)")
     ap.add_argument("--budget-mb", type=int, default=1600, help="device memory for the rotating buffer sets")
     args = ap.parse_args()

@@ -254,7 +254,8 @@ def test_unquantize_variants_f64(quantizer):
 
 
 DECODER_SHAPES_F64 = [(1, 1), (1, 9), (3, 5), (31, 13), (64, 100), (147, 64), (429, 37), (512, 24), (1000, 9), (1001, 5), (2048, 7),
-                      (4095, 3), (4096, 2), (4097, 3), (9304, 3), (9305, 2), (16383, 2), (20000, 2), (20001, 3), (50257, 2), (100000, 2)]
+                      (4095, 3), (4096, 2), (4097, 3), (9304, 3), (9305, 2), (16383, 2), (20000, 2), (20001, 3), (50257, 2), (100000, 2),
+                      (2, 3), (128, 4099), (576, 50), (1152, 33), (1536, 9)]
 
 
 @pytest.mark.parametrize("shape", DECODER_SHAPES_F64, ids=["%dx%d" % s for s in DECODER_SHAPES_F64])
@@ -267,7 +268,7 @@ def test_tile_and_row_major_decoders_f64(shape):
         g = datagen.normal_with_outliers(rows * 11 + nbits, rows, cols, 0.01, dtype=F64)
         q, _ = oracle.quantize(g, zeros(rows, cols), nbits, zt)
         prev = datagen.normal(rows * 13 + nbits, rows, cols, 1.0, dtype=F64)
-        for mode in (2, 4, 5, 0):
+        for mode in (2, 4, 5, 6, 0):
             say("f64 decoder", rows, cols, nbits, "mode", mode)
             qz = MatrixQuantizerImpl.Create(0, False)
             qz._set_tuning(unq_mode=mode)

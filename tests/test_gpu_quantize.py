@@ -364,7 +364,9 @@ def test_unquantize_variants(quantizer):
 
 
 TILE_DECODER_SHAPES = [(1, 1), (1, 9), (2, 7), (3, 5), (5, 3), (31, 13), (32, 8), (33, 41), (64, 100), (147, 64), (256, 1031),
-                       (429, 37), (512, 24), (1000, 9), (1001, 5), (1024, 3), (2047, 2), (2048, 7), (4096, 5), (4095, 3), (4097, 3), (9305, 2), (16383, 2), (16385, 2), (1025, 7), (1026, 5), (1027, 3), (50257, 2), (100001, 2)]
+                       (429, 37), (512, 24), (1000, 9), (1001, 5), (1024, 3), (2047, 2), (2048, 7), (4096, 5), (4095, 3), (4097, 3), (9305, 2), (16383, 2), (16385, 2), (1025, 7), (1026, 5), (1027, 3), (50257, 2), (100001, 2),
+                       # heights and QWord counts in whole 16-byte groups: the decoder that treats the matrix as one run of such groups
+                       (4, 3), (12, 50), (128, 4099), (576, 50), (1152, 33), (4608, 3)]
 
 
 @pytest.mark.parametrize("shape", TILE_DECODER_SHAPES, ids=["%dx%d" % s for s in TILE_DECODER_SHAPES])
@@ -377,7 +379,7 @@ def test_tile_decoder(shape):
         g = datagen.normal_with_outliers(rows * 11 + nbits, rows, cols, 0.01)
         q, _ = oracle.quantize(g, np.zeros_like(g, order="F"), nbits, zt)
         prev = datagen.normal(rows * 13 + nbits, rows, cols, 1.0)
-        for mode in (2, 0, 3, 5):
+        for mode in (2, 0, 3, 5, 6):
             say("tile decoder", rows, cols, nbits, "mode", mode)
             qz = MatrixQuantizerImpl.Create(0, False)
             qz._set_tuning(unq_mode=mode)
