@@ -913,11 +913,11 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
     // The LDS-free decoder for short columns, wherever it can run up to 4608 rows: in a launch of its
     // own it measured 4 to 24 % faster than the tile, row-major and QWord-major decoders it replaces (512 x 100000: 38.3 ->
     // 33.7 us, 576 x 16384 at 2 bits 9.1 -> 7.0 us, 64 x 400000 at 8 bits 22.9 -> 19.4 us, 1536 x 12288 13.4 -> 12.1 us;
-    // even at 512 x 40000 and 2304 x 4096 at 4 bits). As a member of a gradient-set launch only a large matrix gains (the
-    // 512 x 100000 member of the LSTM set: the set's decode 80.6 -> 68.8 us); ResNet-50's 161 members and the 2048-row
-    // stripes of the all-reduce measured 5 to 7 % slower with it and keep their decoders.
+    // even at 512 x 40000 and 2304 x 4096 at 4 bits). As a member of a gradient-set launch only a large matrix (4 M elements)
+    // gains (the LSTM set's decode with its 512 x 100000 and 1024 x 4096 members: 80.6 -> 69.4 us); ResNet-50's 161 members
+    // and the 2048 x 1163 stripes of the all-reduce measured 5 to 7 % slower with it and keep their decoders.
     const bool flat_auto = mode == 0 && !direct_auto && rows <= 4608 && // (the tallest measured)
-                           (!tune.unq_member || (!vec_ideal && (uint64_t) rows * cols >= ((uint64_t) 1 << 23)));
+                           (!tune.unq_member || (uint64_t) rows * cols >= ((uint64_t) 1 << 22));
     if ((mode == 6 || flat_auto) && slots_free && out16 && make_unq_flat_geom(p.flat, rows, cols, nq, qcol_bytes(nbits, rows), 4))
     {
         p.kind = kUnqFlat;

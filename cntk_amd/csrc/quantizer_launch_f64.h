@@ -468,7 +468,7 @@ inline UnquantizePlan64 plan_unquantize(const double* out, size_t rows, size_t c
     // 576 x 16384 at 2 bits 15.6 -> 12.8 us, 1536 x 6144 13.7 -> 12.0 us, even at 2048 x 4652 at 4 bits; 4608 x 2048 at 4 bits
     // is 13 % slower with it than with the packed column in LDS)
     const bool flat_auto = mode == 0 && !direct_auto && rows <= 2048 &&
-                           (!tune.unq_member || (!vec_ideal && (uint64_t) rows * cols >= ((uint64_t) 1 << 22)));
+                           (!tune.unq_member || (uint64_t) rows * cols >= ((uint64_t) 1 << 22));
     if ((mode == 6 || flat_auto) && tune.unq_slots == 0 && out16 && make_unq_flat_geom(p.flat, rows, cols, nq, qcol_bytes(nbits, rows), 2))
     {
         p.kind = kUnqFlat;
