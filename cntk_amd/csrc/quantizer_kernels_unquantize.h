@@ -516,9 +516,9 @@ __global__ __launch_bounds__(256) void unquantize_direct_kernel(const char* __re
     unquantize_direct_body<NBITS>(q, out, t, add, blockIdx.x);
 }
 
-// The same without LDS for short columns whose heights and QWord counts are multiples of N (the elements of 16 bytes):
+// The same without LDS for short columns whose heights are multiples of N (the elements of 16 bytes), with N QWords or more:
 // consecutive columns are adjacent in the output, so the matrix is one run of groups of N consecutive elements, each group
-// inside one column at one bit position of N consecutive QWords. A thread takes kUnqDirectPieces groups, 256 groups apart,
+// inside one column and, where the QWord count is a multiple of N too, at one bit position of N consecutive QWords. A thread takes kUnqDirectPieces groups, 256 groups apart,
 // finds column, bit position and QWord of each, requests the column's header and the N QWords of every group and then
 // decodes. The output is 16-byte aligned and the matrix has fewer than 2^32 elements (checked by the host).
 struct UnqFlatGeom
@@ -548,7 +548,7 @@ __device__ __forceinline__ void unquantize_flat_body(const char* __restrict__ q,
     QVec qv[P];
     Pair hd[P];
     Vec prev[P];
-    uint32_t sh[P];
+    uint32_t sh[P], ws[P], cs[P];
 #pragma unroll
     for (uint32_t u = 0; u < P; ++u)
     {
@@ -559,8 +559,12 @@ __device__ __forceinline__ void unquantize_flat_body(const char* __restrict__ q,
         divmod_u32(r, t.nq, t.inv_nq, k, w);
         const char* qc = q + (size_t) c * t.qcol;
         hd[u] = *reinterpret_cast<const PairAtElem*>(qc);
-        qv[u] = *reinterpret_cast<const QVecAtWord*>(qc + 2 * sizeof(E) + (size_t) w * sizeof(QWord));
+        // (a group that wraps to the next bit position inside -- QWord counts that are no multiple of N -- is fetched QWord by
+        // QWord below)
+        qv[u] = *reinterpret_cast<const QVecAtWord*>(qc + 2 * sizeof(E) + (size_t) (w + N <= t.nq ? w : t.nq - N) * sizeof(QWord));
         sh[u] = k * PS::SHIFT;
+        ws[u] = w;
+        cs[u] = c;
         if (add)
             prev[u] = o4[gg];
     }
@@ -574,11 +578,30 @@ __device__ __forceinline__ void unquantize_flat_body(const char* __restrict__ q,
             const E uf = make_ufactor<NBITS>(lo, hd[u][1]);
             const E val0 = unquantize_value<NBITS>(uf, lo, 0u);
             const E val1 = unquantize_value<NBITS>(uf, lo, 1u);
+            QWord wd[N];
+            uint32_t she[N];
+#pragma unroll
+            for (uint32_t e = 0; e < N; ++e)
+            {
+                wd[e] = qv[u][e];
+                she[e] = sh[u];
+            }
+            if (ws[u] + N > t.nq)
+            {
+                const QWord* bits = reinterpret_cast<const QWord*>(q + (size_t) cs[u] * t.qcol + 2 * sizeof(E));
+#pragma unroll
+                for (uint32_t e = 0; e < N; ++e)
+                {
+                    const bool wraps = ws[u] + e >= t.nq;
+                    wd[e] = bits[wraps ? ws[u] + e - t.nq : ws[u] + e];
+                    she[e] = wraps ? sh[u] + PS::SHIFT : sh[u];
+                }
+            }
             Vec x;
 #pragma unroll
             for (uint32_t e = 0; e < N; ++e)
             {
-                const QWord code = (qv[u][e] >> sh[u]) & PS::CODEMASK;
+                const QWord code = (wd[e] >> she[e]) & PS::CODEMASK;
                 if constexpr (NBITS == 1)
                     x[e] = code ? val1 : val0;
                 else

@@ -837,12 +837,12 @@ struct UnquantizePlan
     bool ok = false;
 };
 
-// The geometry of the LDS-free decoder for short columns (per16 elements in 16 bytes): heights and QWord counts that are
-// multiples of per16, fewer than 2^32 elements. False where it cannot run.
+// The geometry of the LDS-free decoder for short columns (per16 elements in 16 bytes): heights that are multiples of per16,
+// per16 QWords or more, fewer than 2^32 elements. False where it cannot run.
 inline bool make_unq_flat_geom(UnqFlatGeom& t, size_t rows, size_t cols, size_t nq, uint64_t qcol, size_t per16)
 {
     const uint64_t elems = (uint64_t) rows * cols;
-    if (rows == 0 || rows % per16 != 0 || nq % per16 != 0 || elems == 0 || elems > 0xFFFFFFFFull)
+    if (rows == 0 || rows % per16 != 0 || nq < per16 || elems == 0 || elems > 0xFFFFFFFFull)
         return false;
     t.rows = (uint32_t) rows;
     t.nq = (uint32_t) nq;
@@ -910,13 +910,14 @@ inline UnquantizePlan plan_unquantize(const void* q, const float* out, size_t ro
     const bool direct_auto = direct_can && (rows >= 16384 || (!vec_ideal && nbits >= 2 && rows >= 8192 && direct_full) ||
                                             (vec_ideal && nbits <= 2 && rows % direct_chunk == 0 && rows <= 8192 && !tune.unq_member));
     bool vec = false, rowmajor = false, tile = false, seg_allowed = true, direct = false;
-    // The LDS-free decoder for short columns, wherever it can run up to 4608 rows: in a launch of its
+    // The LDS-free decoder for short columns, wherever it can run below 10000 rows: in a launch of its
     // own it measured 4 to 24 % faster than the tile, row-major and QWord-major decoders it replaces (512 x 100000: 38.3 ->
-    // 33.7 us, 576 x 16384 at 2 bits 9.1 -> 7.0 us, 64 x 400000 at 8 bits 22.9 -> 19.4 us, 1536 x 12288 13.4 -> 12.1 us;
+    // 33.7 us, 576 x 16384 at 2 bits 9.1 -> 7.0 us, 64 x 400000 at 8 bits 22.9 -> 19.4 us, 1536 x 12288 13.4 -> 12.1 us,
+    // 1000 x 20000 at 1 / 8 bits 16.3 / 21.5 -> 12.9 / 17.1 us;
     // even at 512 x 40000 and 2304 x 4096 at 4 bits). As a member of a gradient-set launch only a large matrix (4 M elements)
     // gains (the LSTM set's decode with its 512 x 100000 and 1024 x 4096 members: 80.6 -> 69.4 us); ResNet-50's 161 members
     // and the 2048 x 1163 stripes of the all-reduce measured 5 to 7 % slower with it and keep their decoders.
-    const bool flat_auto = mode == 0 && !direct_auto && rows <= 4608 && // (the tallest measured)
+    const bool flat_auto = mode == 0 && !direct_auto && rows < 10000 && // (9304 x 2048: 14.4 -> 13.7 us; even from 10000 rows on)
                            (!tune.unq_member || (uint64_t) rows * cols >= ((uint64_t) 1 << 22));
     if ((mode == 6 || flat_auto) && slots_free && out16 && make_unq_flat_geom(p.flat, rows, cols, nq, qcol_bytes(nbits, rows), 4))
     {

@@ -467,7 +467,9 @@ inline UnquantizePlan64 plan_unquantize(const double* out, size_t rows, size_t c
     // (the LDS-free decoder for short columns: the rule of the float side, up to 2048 rows -- 512 x 50000 38.0 -> 32.4 us,
     // 576 x 16384 at 2 bits 15.6 -> 12.8 us, 1536 x 6144 13.7 -> 12.0 us, even at 2048 x 4652 at 4 bits; 4608 x 2048 at 4 bits
     // is 13 % slower with it than with the packed column in LDS)
-    const bool flat_auto = mode == 0 && !direct_auto && rows <= 2048 &&
+    // (QWord counts that are odd stay with the tile and row-major decoders here: 1000 x 10000 at 8 bits and 200 x 100000 at 2
+    // bits were 11 % slower with it, 576 x 16384 at 1 bit 10 % faster)
+    const bool flat_auto = mode == 0 && !direct_auto && rows <= 2048 && nq % 2 == 0 &&
                            (!tune.unq_member || (uint64_t) rows * cols >= ((uint64_t) 1 << 22));
     if ((mode == 6 || flat_auto) && tune.unq_slots == 0 && out16 && make_unq_flat_geom(p.flat, rows, cols, nq, qcol_bytes(nbits, rows), 2))
     {
