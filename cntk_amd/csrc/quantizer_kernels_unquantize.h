@@ -518,15 +518,16 @@ __global__ __launch_bounds__(256) void unquantize_direct_kernel(const char* __re
 
 // The same without LDS for short columns whose heights are multiples of N (the elements of 16 bytes), with N QWords or more:
 // consecutive columns are adjacent in the output, so the matrix is one run of groups of N consecutive elements, each group
-// inside one column and, where the QWord count is a multiple of N too, at one bit position of N consecutive QWords. A thread takes kUnqDirectPieces groups, 256 groups apart,
-// finds column, bit position and QWord of each, requests the column's header and the N QWords of every group and then
-// decodes. The output is 16-byte aligned and the matrix has fewer than 2^32 elements (checked by the host).
+// inside one column and, where the QWord count is a multiple of N too, at one bit position of N consecutive QWords. A
+// thread takes kUnqDirectPieces groups, 256 groups apart, finds column, bit position and QWord of each, requests the
+// column's header and the N QWords of every group and then decodes. The output is 16-byte aligned and the matrix has
+// fewer than 2^32 elements (checked by the host).
 struct UnqFlatGeom
 {
     uint32_t rows;
     uint32_t nq;
     uint32_t groups; // rows * cols / N
-    uint32_t blocks;
+    uint32_t blocks; // workgroups: 256 * kUnqDirectPieces groups each
     double inv_rows;
     double inv_nq;
     uint64_t qcol;
