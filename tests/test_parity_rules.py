@@ -102,6 +102,23 @@ def test_inputs_that_all_moved_one_way_explain_as_much_on_the_bounds():
     parity.check_quantize(g, r, q, r_out, 1, False, threads=4, exact=False, input_dev=np.full(8, float(shift)))
 
 
+def test_a_column_without_spread_whose_inputs_moved_a_little():
+    """The whole-run comparison on a column that is all zero on the oracle's side (bounds 0, 0) and off by the inputs'
+    difference on the other: exact agreement is asked for only where the inputs are the same."""
+    g = np.zeros((64, 3), np.float32, order="F")
+    r = np.zeros((64, 3), np.float32, order="F")
+    moved = g.copy(order="F")
+    moved[:, 1] = np.float32(3e-9)
+    for nbits in (1, 2):
+        q, r_out = oracle.quantize(moved, r, nbits, False, threads=2)
+        with pytest.raises(AssertionError):
+            parity.check_quantize(g, r, q, r_out, nbits, False, threads=2, exact=False)
+        dev = np.array([0.0, 3e-9, 0.0])
+        parity.check_quantize(g, r, q, r_out, nbits, False, threads=2, exact=False, input_dev=dev)
+        with pytest.raises(AssertionError, match="without spread"):
+            parity.check_quantize(g, r, q, r_out, nbits, False, threads=2, exact=False, input_dev=dev * 1e-3)
+
+
 def test_an_element_on_the_other_side_of_zero_leaves_its_column_out_of_the_whole_run():
     """With the zero threshold the bounds are the means of the two sides: one element at -2e-8 here and 0.0 there moves
     both by mean / count (1e-4 of the scale at 2000 rows). The whole-run comparison leaves such a column out, and counts
